@@ -1,0 +1,526 @@
+// CPU oracle: f32 restatement of the reference's host path.  TEST INFRASTRUCTURE ONLY - see pyre_oracle.h.
+// Every function cites the reference lines it follows (paths relative to the reference tree).
+// Build: g++ -O2 -std=c++17 -mavx2 -mfma -ffp-contract=off -fPIC -shared -pthread (see oracle/Makefile).
+#include "pyre_oracle.h"
+#include "iq_codebooks.h"
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <thread>
+#include <vector>
+
+namespace {
+
+// ---------- small scalar helpers -------------------------------------------------------------
+// IEEE binary16 -> binary32 (the `half` crate's f16::to_f32, used by h2f at gguf_q.rs:60).
+inline float h2f(const uint8_t* b) {
+  uint32_t h = (uint32_t)b[0] | ((uint32_t)b[1] << 8);
+  uint32_t s = (h & 0x8000u) << 16, e = (h >> 10) & 0x1F, m = h & 0x3FF, u;
+  if (e == 0) {
+    if (m == 0) u = s;
+    else { int sh = 0; while (!(m & 0x400)) { m <<= 1; ++sh; } m &= 0x3FF; u = s | ((uint32_t)(113 - sh) << 23) | (m << 13); }
+  } else if (e == 31) u = s | 0x7F800000u | (m << 13);
+  else u = s | ((e + 112) << 23) | (m << 13);
+  float f; memcpy(&f, &u, 4); return f;
+}
+
+struct Tables { uint32_t iq3s[512]; uint64_t iq2xs[512]; uint8_t ksigns[128]; };
+const Tables& tables() {
+  static Tables t = [] {
+    Tables t{};
+    static const uint8_t tri[3] = {8, 25, 43};
+    for (int e = 0; e < 512; ++e) {
+      uint32_t v = 0; for (int j = 0; j < 4; ++j) v |= (uint32_t)(2 * ((kIq3sCode[e] >> (3 * j)) & 7) + 1) << (8 * j);
+      t.iq3s[e] = v;
+      uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(kIq2xsCode[e] >> (2 * j)) & 3] << (8 * j);
+      t.iq2xs[e] = w;
+    }
+    for (int i = 0; i < 128; ++i) t.ksigns[i] = (uint8_t)(i | ((__builtin_popcount(i) & 1) << 7));
+    return t;
+  }();
+  return t;
+}
+
+// put8, gguf_q.rs:58: y[j] = d * g[j] * s[j], evaluated left to right.
+inline void put8(float* y, float d, const float* g, uint8_t signs) {
+  for (int j = 0; j < 8; ++j) { float s = (signs >> j) & 1 ? -1.0f : 1.0f; y[j] = d * g[j] * s; }
+}
+
+// scale_min_k4, gguf_q.rs:62-64
+inline void scale_min_k4(int j, const uint8_t* q, uint8_t* s, uint8_t* m) {
+  if (j < 4) { *s = q[j] & 63; *m = q[j + 4] & 63; }
+  else { *s = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4)); *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4)); }
+}
+
+bool geom(uint32_t ty, int* el, int* by) {
+  switch (ty) {  // QType::geom, gguf_q.rs:33-41
+    case ORC_F32: *el = 1; *by = 4; return true;
+    case ORC_F16: case ORC_BF16: *el = 1; *by = 2; return true;
+    case ORC_Q8_0: *el = 32; *by = 34; return true;
+    case ORC_Q4_K: *el = 256; *by = 144; return true;
+    case ORC_IQ2_XS: *el = 256; *by = 74; return true;
+    case ORC_IQ3_S: *el = 256; *by = 110; return true;
+  }
+  return false;
+}
+
+// dequant, gguf_q.rs:67-166 (arms F32 :71, F16 :72, BF16 :73, Q8_0 :79, Q4K :103-107, IQ2XS :126-129, IQ3S :141-151)
+bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
+  int qk, bs; if (!geom(ty, &qk, &bs)) return false;
+  size_t nb = n / qk;
+  const Tables& T = tables();
+  switch (ty) {
+    case ORC_F32: memcpy(y, x, 4 * n); break;
+    case ORC_F16: for (size_t i = 0; i < n; ++i) y[i] = h2f(x + 2 * i); break;
+    case ORC_BF16: for (size_t i = 0; i < n; ++i) { uint32_t u = ((uint32_t)x[2 * i] | ((uint32_t)x[2 * i + 1] << 8)) << 16; memcpy(&y[i], &u, 4); } break;
+    case ORC_Q8_0:
+      for (size_t i = 0; i < nb; ++i) { const uint8_t* b = x + i * bs; float d = h2f(b); for (int j = 0; j < 32; ++j) y[i * 32 + j] = (float)(int8_t)b[2 + j] * d; }
+      break;
+    case ORC_Q4_K:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b), mn = h2f(b + 2); const uint8_t* sc = b + 4; const uint8_t* q = b + 16; float* yy = y + i * 256;
+        for (int j = 0; j < 4; ++j) {
+          uint8_t s1, m1, s2, m2; scale_min_k4(2 * j, sc, &s1, &m1); scale_min_k4(2 * j + 1, sc, &s2, &m2);
+          float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
+          for (int l = 0; l < 32; ++l) { yy[l] = d1 * (float)(q[l] & 0xF) - M1; yy[l + 32] = d2 * (float)(q[l] >> 4) - M2; }
+          yy += 64; q += 32;
+        }
+      }
+      break;
+    case ORC_IQ2_XS:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); const uint8_t* qs = b + 2; const uint8_t* sc = b + 66; float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          float db[2] = { d * (0.5f + (float)(sc[ib] & 0xF)) * 0.25f, d * (0.5f + (float)(sc[ib] >> 4)) * 0.25f };
+          for (int l = 0; l < 4; ++l) {
+            uint32_t q = (uint32_t)qs[2 * (4 * ib + l)] | ((uint32_t)qs[2 * (4 * ib + l) + 1] << 8);
+            uint64_t gv = T.iq2xs[q & 511]; float g[8]; for (int j = 0; j < 8; ++j) g[j] = (float)((gv >> (8 * j)) & 0xFF);
+            put8(yy, db[l / 2], g, T.ksigns[q >> 9]); yy += 8;
+          }
+        }
+      }
+      break;
+    case ORC_IQ3_S:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); const uint8_t* qs = b + 2; const uint8_t* qh = b + 66; const uint8_t* signs = b + 74; const uint8_t* sc = b + 106;
+        float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ib += 2) {
+          for (int half = 0; half < 2; ++half) {
+            uint8_t s = sc[ib / 2]; float db = d * (float)(1 + 2 * (half == 0 ? (s & 0xF) : (s >> 4)));
+            for (int l = 0; l < 4; ++l) {
+              uint32_t g1 = T.iq3s[qs[2 * l] | (((uint32_t)qh[half] << (8 - 2 * l)) & 256)];
+              uint32_t g2 = T.iq3s[qs[2 * l + 1] | (((uint32_t)qh[half] << (7 - 2 * l)) & 256)];
+              float g[8]; for (int j = 0; j < 4; ++j) { g[j] = (float)((g1 >> (8 * j)) & 0xFF); g[4 + j] = (float)((g2 >> (8 * j)) & 0xFF); }
+              put8(yy, db, g, signs[l]); yy += 8;
+            }
+            qs += 8; signs += 4;
+          }
+          qh += 2;
+        }
+      }
+      break;
+    default: return false;
+  }
+  return true;
+}
+
+// dot_avx2, gguf_q.rs:175-197: four 8-lane FMA accumulators over strides of 32, an 8-wide tail into the first,
+// (s0+s1)+(s2+s3), the 8 lanes summed in order, then a scalar tail (mul then add, not fused: `r += a[i] * b[i]`).
+float dot(const float* a, const float* b, size_t n) {
+  float s[4][8] = {};
+  size_t i = 0;
+  for (; i + 32 <= n; i += 32)
+    for (int k = 0; k < 4; ++k)
+      for (int j = 0; j < 8; ++j) s[k][j] = __builtin_fmaf(a[i + 8 * k + j], b[i + 8 * k + j], s[k][j]);
+  for (; i + 8 <= n; i += 8) for (int j = 0; j < 8; ++j) s[0][j] = __builtin_fmaf(a[i + j], b[i + j], s[0][j]);
+  float t[8]; for (int j = 0; j < 8; ++j) t[j] = (s[0][j] + s[1][j]) + (s[2][j] + s[3][j]);
+  float r = 0.0f; for (int j = 0; j < 8; ++j) r += t[j];
+  for (; i < n; ++i) r += a[i] * b[i];
+  return r;
+}
+
+void parallel_for(size_t n, int threads, const std::function<void(size_t, size_t)>& f) {
+  if (threads <= 1 || n < 2) { f(0, n); return; }
+  size_t nt = std::min<size_t>(threads, n);
+  std::vector<std::thread> th; th.reserve(nt);
+  std::atomic<size_t> next{0};
+  size_t chunk = std::max<size_t>(1, n / (nt * 8));
+  for (size_t k = 0; k < nt; ++k) th.emplace_back([&] { for (;;) { size_t a = next.fetch_add(chunk); if (a >= n) break; f(a, std::min(n, a + chunk)); } });
+  for (auto& t : th) t.join();
+}
+
+// QMat::matmul for t < 16, gguf_q.rs:233-241: each row dequantized once, dotted against every token.
+// y[ti*rows + r] = sum_c W[r,c] * x[ti*cols + c]   (gguf_q.rs:216)
+bool matmul(uint32_t ty, const uint8_t* w, size_t rows, size_t cols, const float* x, int t, float* y, int threads) {
+  int qk, bs; if (!geom(ty, &qk, &bs) || cols % qk) return false;
+  size_t rb = cols / qk * bs;
+  int th = (rows * cols < (1u << 18)) ? 1 : threads;
+  parallel_for(rows, th, [&](size_t r0, size_t r1) {
+    std::vector<float> buf(cols);
+    for (size_t r = r0; r < r1; ++r) { dequant(ty, w + r * rb, cols, buf.data()); for (int ti = 0; ti < t; ++ti) y[(size_t)ti * rows + r] = dot(buf.data(), x + (size_t)ti * cols, cols); }
+  });
+  return true;
+}
+inline bool mm(const OrcTensor* m, const float* x, int t, float* y, int threads) { return matmul(m->ty, (const uint8_t*)m->data, m->rows, m->cols, x, t, y, threads); }
+
+inline float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }               // qwen4exp_gguf.rs:457
+inline float silu(float x) { return x * sigm(x); }                             // :458
+inline float softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }     // :459
+
+// rms, qwen4exp_gguf.rs:209: y = x * s * w ;  rms_inplace, :210: x *= s * w  (different association)
+inline float rms_scale(const float* x, size_t n, float eps) { float ss = 0.0f; for (size_t i = 0; i < n; ++i) ss += x[i] * x[i]; return 1.0f / sqrtf(ss / (float)n + eps); }
+void rms(const float* x, const float* w, float eps, float* y, size_t n) { float s = rms_scale(x, n, eps); for (size_t i = 0; i < n; ++i) y[i] = x[i] * s * w[i]; }
+void rms_inplace(float* x, const float* w, float eps, size_t n) { float s = rms_scale(x, n, eps); for (size_t i = 0; i < n; ++i) x[i] *= s * w[i]; }
+
+// kv4::pack, kv4.rs:12-31 (Rust f32::round = half away from zero = roundf)
+void kv4_pack(const float* x, size_t n, uint32_t* w, float* sc) {
+  for (size_t b = 0; b < n / 32; ++b) {
+    const float* p = x + 32 * b; float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(p[i]));
+    float s = (m > 0.0f && std::isfinite(m)) ? m / 7.0f : 0.0f; sc[b] = s;
+    for (int c = 0; c < 4; ++c) {
+      uint32_t u = 0;
+      for (int j = 0; j < 8; ++j) { int q = s > 0.0f ? (int)fminf(fmaxf(roundf(p[8 * c + j] / s), -7.0f), 7.0f) : 0; u |= ((uint32_t)(uint8_t)(int8_t)q & 0xF) << (4 * j); }
+      w[4 * b + c] = u;
+    }
+  }
+}
+inline float kv4_get(const uint32_t* w, const float* sc, size_t i) {  // kv4.rs:35-39
+  uint32_t nib = (w[i / 8] >> (4 * (i % 8))) & 0xF; int q = (int)nib - (nib >= 8 ? 16 : 0); return (float)q * sc[i / 32];
+}
+// kvq_roundtrip, qwen4exp_gguf.rs:3313-3317
+void kvq_roundtrip(float* x, size_t n, int bits) {
+  float q = (float)((1 << (bits - 1)) - 1);
+  for (size_t b = 0; b < n / 32; ++b) { float* p = x + 32 * b; float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(p[i]));
+    if (m == 0.0f || !std::isfinite(m)) continue; float s = m / q; for (int i = 0; i < 32; ++i) p[i] = fminf(fmaxf(roundf(p[i] / s), -q), q) * s; }
+}
+// Packed region of the cache for a query that sees n positions: [0, ((n - recent)/64)*64), the split of
+// kv_push's packed branch (qwen4exp_gguf.rs:1519-1520: `cl > dense + recent + 64`, `q8n = ((cl - recent)/64)*64`),
+// applied at every step instead of only when the device buffer is reallocated.
+size_t packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 4 || n <= (size_t)recent + 64) return 0; return ((n - recent) / 64) * 64; }
+
+// top_k + soft_top, qwen4exp_gguf.rs:3121-3139.  The reference's host selection leaves the order among the k chosen
+// unspecified (select_nth_unstable); its device router ranks with lower-index-wins ties and lists the chosen experts
+// in ascending id (qn_cube.rs:5225-5237).  This statement fixes: ties -> lower index, order -> ascending id,
+// max / exp / sum / divide over that order.  NaN logits -> -inf, all non-finite max -> uniform (:3121-3129).
+bool top_k(const float* r0, int n, int k, int32_t* idx, float* w) {
+  if (k > n || k <= 0) return false;
+  std::vector<float> r(r0, r0 + n);
+  for (auto& v : r) if (std::isnan(v)) v = -INFINITY;
+  int c = 0;
+  for (int e = 0; e < n; ++e) { int rank = 0; for (int j = 0; j < n; ++j) if (r[j] > r[e] || (r[j] == r[e] && j < e)) ++rank; if (rank < k) idx[c++] = e; }
+  float mx = -INFINITY; for (int i = 0; i < k; ++i) mx = fmaxf(mx, r[idx[i]]);
+  if (!std::isfinite(mx)) { for (int i = 0; i < k; ++i) w[i] = 1.0f / (float)k; return true; }
+  float sum = 0.0f; for (int i = 0; i < k; ++i) { w[i] = expf(r[idx[i]] - mx); sum += w[i]; }
+  for (int i = 0; i < k; ++i) w[i] = w[i] / sum;
+  return true;
+}
+
+// linear_core, qwen4exp_gguf.rs:1624-1673 (the t == 1 loop form, :1642-1647, applied per token)
+void gdn_core(int nk, int nv, int dk, int dv, int kk, float eps, const float* a, const float* dt, const float* conv, const float* norm,
+              const float* m, const float* zz, const float* bb, const float* aa, int t, float* cs, float* s, float* o_all) {
+  int ch = 2 * nk * dk + nv * dv; int w = nv * dv;
+  std::vector<float> co(ch), mem(dv), delta(dv);
+  for (int ti = 0; ti < t; ++ti) {
+    const float* cur = m + (size_t)ti * ch;
+    for (int cc = 0; cc < ch; ++cc) { float o = conv[cc * kk + kk - 1] * cur[cc]; for (int k = 0; k < kk - 1; ++k) o += conv[cc * kk + k] * cs[(size_t)k * ch + cc]; co[cc] = silu(o); }
+    memmove(cs, cs + ch, sizeof(float) * (size_t)(kk - 2) * ch); memcpy(cs + (size_t)(kk - 2) * ch, cur, sizeof(float) * ch);
+    for (int h = 0; h < nk; ++h) {  // :1649-1651
+      float* qp = co.data() + h * dk; float* kp = co.data() + nk * dk + h * dk;
+      float sq = 0.0f; for (int i = 0; i < dk; ++i) sq += qp[i] * qp[i]; float nq = (1.0f / sqrtf(sq + 1e-6f)) * (1.0f / sqrtf((float)dk)); for (int i = 0; i < dk; ++i) qp[i] *= nq;
+      float sk = 0.0f; for (int i = 0; i < dk; ++i) sk += kp[i] * kp[i]; float nkk = (1.0f / sqrtf(sk + 1e-6f)) * 1.0f; for (int i = 0; i < dk; ++i) kp[i] *= nkk;
+    }
+    for (int h = 0; h < nv; ++h) {  // :1654-1670
+      int kh = h % nk; float* sh = s + (size_t)h * dk * dv;
+      const float* qv = co.data() + kh * dk; const float* kv = co.data() + nk * dk + kh * dk; const float* vv = co.data() + 2 * nk * dk + h * dv;
+      float g = expf(softplus(aa[ti * nv + h] + dt[h]) * a[h]); float b = sigm(bb[ti * nv + h]);
+      for (int i = 0; i < dk * dv; ++i) sh[i] *= g;
+      for (int j = 0; j < dv; ++j) mem[j] = 0.0f;
+      for (int i = 0; i < dk; ++i) { float ki = kv[i]; const float* row = sh + (size_t)i * dv; for (int j = 0; j < dv; ++j) mem[j] += row[j] * ki; }
+      for (int j = 0; j < dv; ++j) delta[j] = (vv[j] - mem[j]) * b;
+      float* oh = o_all + (size_t)ti * w + h * dv; for (int j = 0; j < dv; ++j) oh[j] = 0.0f;
+      for (int i = 0; i < dk; ++i) { float ki = kv[i], qi = qv[i]; float* row = sh + (size_t)i * dv; for (int j = 0; j < dv; ++j) { row[j] += ki * delta[j]; oh[j] += row[j] * qi; } }
+      rms_inplace(oh, norm, eps, dv); const float* zh = zz + (size_t)ti * w + h * dv; for (int j = 0; j < dv; ++j) oh[j] *= sigm(zh[j]);
+    }
+  }
+}
+
+// rope, qwen4exp_gguf.rs:1436-1439 with rope_cs :529-533 (mscale == 1): angle = pos as f32 * inv[i]
+void rope(float* v, int pos, int n_rot, const float* inv) {
+  int half = n_rot / 2;
+  for (int i = 0; i < half; ++i) { float a = (float)pos * inv[i]; float s = sinf(a), c = cosf(a); float x0 = v[i], x1 = v[i + half]; v[i] = x0 * c - x1 * s; v[i + half] = x1 * c + x0 * s; }
+}
+
+// attn_core, qwen4exp_gguf.rs:1558-1615, dense branch (no indexer).  Cache rows below the packed boundary are read
+// through the 4-bit round trip (kvq_roundtrip semantics, :1535), the cache itself keeps f32.
+void attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, const float* qn, const float* kn,
+               const float* qf, const float* kf_in, const float* vf, int start, int t, int kv_bits, int recent, float* kc, float* vc, float* att) {
+  size_t row = (size_t)nkv * hd;
+  std::vector<float> kf(kf_in, kf_in + (size_t)t * row);
+  for (int ti = 0; ti < t; ++ti) for (int h = 0; h < nkv; ++h) { float* kh = kf.data() + ti * row + (size_t)h * hd; rms_inplace(kh, kn, eps, hd); rope(kh, start + ti, n_rot, inv); }
+  memcpy(kc + start * row, kf.data(), sizeof(float) * t * row); memcpy(vc + start * row, vf, sizeof(float) * t * row);
+  float scale = 1.0f / sqrtf((float)hd); int grp = nh / nkv;
+  std::vector<float> qh(hd), krt(row), vrt(row);
+  for (int ti = 0; ti < t; ++ti) {
+    int n = start + ti + 1; size_t pb = packed_boundary(n, kv_bits, recent);
+    for (int h = 0; h < nh; ++h) {
+      size_t base = (size_t)ti * nh * 2 * hd + (size_t)h * 2 * hd;
+      memcpy(qh.data(), qf + base, sizeof(float) * hd); rms_inplace(qh.data(), qn, eps, hd); rope(qh.data(), start + ti, n_rot, inv);
+      int kvh = h / grp; float* out = att + ((size_t)ti * nh + h) * hd; for (int i = 0; i < hd; ++i) out[i] = 0.0f;
+      std::vector<float> sc(n);
+      for (int p = 0; p < n; ++p) {
+        const float* kr = kc + p * row + (size_t)kvh * hd;
+        if ((size_t)p < pb) { memcpy(krt.data(), kr, sizeof(float) * hd); kvq_roundtrip(krt.data(), hd, 4); kr = krt.data(); }
+        sc[p] = dot(qh.data(), kr, hd) * scale;
+      }
+      float mx = -INFINITY; for (int p = 0; p < n; ++p) mx = fmaxf(mx, sc[p]);
+      float sum = 0.0f; for (int p = 0; p < n; ++p) { sc[p] = expf(sc[p] - mx); sum += sc[p]; }
+      float iv = 1.0f / sum;
+      for (int p = 0; p < n; ++p) {
+        float wgt = sc[p] * iv; const float* vr = vc + p * row + (size_t)kvh * hd;
+        if ((size_t)p < pb) { memcpy(vrt.data(), vr, sizeof(float) * hd); kvq_roundtrip(vrt.data(), hd, 4); vr = vrt.data(); }
+        for (int i = 0; i < hd; ++i) out[i] += wgt * vr[i];
+      }
+      const float* gate = qf + base + hd; for (int i = 0; i < hd; ++i) out[i] *= sigm(gate[i]);
+    }
+  }
+}
+
+// ffn + routed (f32 branch), qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793.
+bool moe_ffn(int d, int n_exp, int k, int ff, const OrcTensor* router, const OrcTensor* gate_e, const OrcTensor* up_e, const OrcTensor* down_e,
+             const float* sh_gate_inp, const OrcTensor* sh_gate, const OrcTensor* sh_up, const OrcTensor* sh_down,
+             const float* x, int t, float* y, int32_t* sel_idx, float* sel_w, int threads) {
+  size_t sf = sh_gate->rows;
+  std::vector<float> lg((size_t)t * n_exp), g((size_t)t * sf), u((size_t)t * sf);
+  if (!mm(router, x, t, lg.data(), threads) || !mm(sh_gate, x, t, g.data(), threads) || !mm(sh_up, x, t, u.data(), threads)) return false;
+  for (size_t i = 0; i < g.size(); ++i) g[i] = silu(g[i]) * u[i];
+  if (!mm(sh_down, g.data(), t, y, threads)) return false;
+  for (int ti = 0; ti < t; ++ti) { float sg = sigm(dot(sh_gate_inp, x + (size_t)ti * d, d)); for (int i = 0; i < d; ++i) y[(size_t)ti * d + i] *= sg; }
+  std::vector<std::vector<std::pair<int, float>>> by_exp(n_exp);
+  std::vector<int32_t> idx(k); std::vector<float> w(k);
+  for (int ti = 0; ti < t; ++ti) {
+    if (!top_k(lg.data() + (size_t)ti * n_exp, n_exp, k, idx.data(), w.data())) return false;
+    for (int i = 0; i < k; ++i) { by_exp[idx[i]].push_back({ti, w[i]}); if (sel_idx) sel_idx[ti * k + i] = idx[i]; if (sel_w) sel_w[ti * k + i] = w[i]; }
+  }
+  int qk, bs; geom(gate_e->ty, &qk, &bs); size_t rb_g = (size_t)d / qk * bs; geom(up_e->ty, &qk, &bs); size_t rb_u = (size_t)d / qk * bs; geom(down_e->ty, &qk, &bs); size_t rb_d = (size_t)ff / qk * bs;
+  std::vector<int> work; for (int e = 0; e < n_exp; ++e) if (!by_exp[e].empty()) work.push_back(e);
+  // hidden rows per expert: h[r] = silu(gate_e[r].x) * (up_e[r].x)   (:1773-1776)
+  std::vector<std::vector<float>> hid(n_exp);
+  for (int e : work) hid[e].assign(by_exp[e].size() * (size_t)ff, 0.0f);
+  parallel_for(work.size() * (size_t)ff, threads, [&](size_t a, size_t b) {
+    std::vector<float> buf(d);
+    for (size_t q = a; q < b; ++q) {
+      int e = work[q / ff]; size_t r = q % ff;
+      dequant(gate_e->ty, (const uint8_t*)gate_e->data + ((size_t)e * ff + r) * rb_g, d, buf.data());
+      std::vector<float> gv(by_exp[e].size()); for (size_t j = 0; j < by_exp[e].size(); ++j) gv[j] = dot(buf.data(), x + (size_t)by_exp[e][j].first * d, d);
+      dequant(up_e->ty, (const uint8_t*)up_e->data + ((size_t)e * ff + r) * rb_u, d, buf.data());
+      for (size_t j = 0; j < by_exp[e].size(); ++j) hid[e][j * ff + r] = silu(gv[j]) * dot(buf.data(), x + (size_t)by_exp[e][j].first * d, d);
+    }
+  });
+  // o[ti][r] += w * (down_e[e*d + r] . hid), experts in ascending id from 0, then y += o   (:1786-1793)
+  std::vector<float> o((size_t)t * d, 0.0f);
+  parallel_for(d, threads, [&](size_t r0, size_t r1) {
+    std::vector<float> buf(ff);
+    for (size_t r = r0; r < r1; ++r) for (int e : work) {
+      dequant(down_e->ty, (const uint8_t*)down_e->data + ((size_t)e * d + r) * rb_d, ff, buf.data());
+      for (size_t j = 0; j < by_exp[e].size(); ++j) { int ti = by_exp[e][j].first; o[(size_t)ti * d + r] += by_exp[e][j].second * dot(buf.data(), hid[e].data() + j * ff, ff); }
+    }
+  });
+  for (size_t i = 0; i < o.size(); ++i) y[i] += o[i];
+  return true;
+}
+
+// hc_mix, qwen4exp_gguf.rs:1357-1382 (f32 branch :1373-1381); hc_combine :1384-1388
+bool hc_mix(int d, int hc, float eps, const float* norm, const OrcTensor* down, const OrcTensor* inject, const OrcTensor* up,
+            const float* x, int t, float* mixed, float* inj, int threads) {
+  size_t w = (size_t)hc * d; size_t lr = down->rows;
+  std::vector<float> xn(t * w), lo((size_t)t * lr), gate(t * w);
+  for (size_t i = 0; i < (size_t)t * hc; ++i) { size_t s = i % hc; rms(x + i * d, norm + s * d, eps, xn.data() + i * d, d); }
+  if (!mm(down, xn.data(), t, lo.data(), threads)) return false;
+  for (auto& v : lo) v = silu(v / (float)hc);
+  if (inject) { if (!mm(inject, xn.data(), t, inj, threads)) return false; for (int i = 0; i < t * hc; ++i) inj[i] /= (float)hc; }
+  else for (int i = 0; i < t * hc; ++i) inj[i] = 0.0f;
+  if (!mm(up, lo.data(), t, gate.data(), threads)) return false;
+  for (int ti = 0; ti < t; ++ti) {
+    float* mr = mixed + (size_t)ti * d; for (int i = 0; i < d; ++i) mr[i] = 0.0f;
+    for (int s = 0; s < hc; ++s) for (int i = 0; i < d; ++i) { size_t k = ti * w + (size_t)s * d + i; mr[i] += xn[k] * sigm(gate[k]); }
+    for (int i = 0; i < d; ++i) mr[i] /= (float)hc;
+  }
+  return true;
+}
+void hc_combine(int d, int hc, float* x, const float* out, const float* inj, int t) {
+  for (int ti = 0; ti < t; ++ti) for (int s = 0; s < hc; ++s) { float w = 2.0f * sigm(inj[ti * hc + s]); float* r = x + ((size_t)ti * hc + s) * d; for (int i = 0; i < d; ++i) r[i] += out[(size_t)ti * d + i] * w; }
+}
+
+}  // namespace
+
+// ---------- model ------------------------------------------------------------------------------
+struct OrcModel {
+  OrcCfg c; std::vector<OrcTensor> lt; OrcTensor g[ORC_GLOBAL_SLOTS]; int threads;
+  std::vector<float> rope_inv;
+  std::vector<std::vector<float>> vec;  // dequantized small tensors, indexed like lt (empty when unused)
+  std::vector<float> head_norm;
+  const OrcTensor& T(int il, int slot) const { return lt[(size_t)il * ORC_LAYER_SLOTS + slot]; }
+  const float* V(int il, int slot) const { return vec[(size_t)il * ORC_LAYER_SLOTS + slot].data(); }
+  bool full(int il) const { return (il + 1) % c.full_every == 0; }
+};
+struct OrcCkpt { std::vector<std::vector<float>> conv, ssm; };
+struct OrcState {
+  std::vector<uint32_t> tokens;
+  std::vector<std::vector<float>> conv, ssm, k, v;
+  std::vector<OrcCkpt> ck;  // state after each token of the last forward_multi
+};
+
+static bool to_vec(const OrcTensor& t, std::vector<float>& out) {
+  if (!t.data) return true; out.resize(t.rows * t.cols); int qk, bs; if (!geom(t.ty, &qk, &bs)) return false;
+  return dequant(t.ty, (const uint8_t*)t.data, t.rows * t.cols, out.data());
+}
+
+extern "C" {
+
+int orc_type_geom(uint32_t ty, int* e, int* b) { return geom(ty, e, b) ? 0 : -1; }
+int orc_dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) { int qk, bs; if (!geom(ty, &qk, &bs) || n % qk) return -1; return dequant(ty, x, n, y) ? 0 : -1; }
+float orc_dot(const float* a, const float* b, size_t n) { return dot(a, b, n); }
+int orc_matmul(uint32_t ty, const uint8_t* w, size_t rows, size_t cols, const float* x, int t, float* y, int threads) { return matmul(ty, w, rows, cols, x, t, y, threads) ? 0 : -1; }
+void orc_expand_iq3s(uint32_t* o) { memcpy(o, tables().iq3s, sizeof(uint32_t) * 512); }
+void orc_expand_iq2xs(uint64_t* o) { memcpy(o, tables().iq2xs, sizeof(uint64_t) * 512); }
+uint8_t orc_ksigns(int i) { return tables().ksigns[i & 127]; }
+
+void orc_kv4_pack(const float* x, size_t n, uint32_t* w, float* sc) { kv4_pack(x, n, w, sc); }
+float orc_kv4_get(const uint32_t* w, const float* sc, size_t i) { return kv4_get(w, sc, i); }
+void orc_kvq_roundtrip(float* x, size_t n, int bits) { kvq_roundtrip(x, n, bits); }
+size_t orc_kv_packed_boundary(size_t n, int kv_bits, int recent) { return packed_boundary(n, kv_bits, recent); }
+
+// rope_inv, qn_ctx.rs:164-170 (unscaled branch): inv[i] = base.powf(-(2 i) / n_rot)
+void orc_rope_inv(int n_rot, float base, float* inv) { for (int i = 0; i < n_rot / 2; ++i) inv[i] = powf(base, -(2.0f * (float)i) / (float)n_rot); }
+// sampler::argmax, sampler.rs:142-148: first index of the maximum (strict >)
+uint32_t orc_argmax(const float* l, size_t n) { size_t best = 0; for (size_t i = 1; i < n; ++i) if (l[i] > l[best]) best = i; return (uint32_t)best; }
+int orc_top_k(const float* r, int n, int k, int32_t* idx, float* w) { return top_k(r, n, k, idx, w) ? 0 : -1; }
+void orc_rms(const float* x, const float* w, float eps, float* y, size_t n) { rms(x, w, eps, y, n); }
+void orc_rms_inplace(float* x, const float* w, float eps, size_t n) { rms_inplace(x, w, eps, n); }
+float orc_sigm(float x) { return sigm(x); }
+float orc_silu(float x) { return silu(x); }
+float orc_softplus(float x) { return softplus(x); }
+
+void orc_gdn_core(int nk, int nv, int dk, int dv, int conv_k, float eps, const float* a, const float* dt, const float* conv_w, const float* norm_w,
+                  const float* qkv, const float* z, const float* beta, const float* alpha, int t, float* conv_state, float* ssm, float* out) {
+  gdn_core(nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w, qkv, z, beta, alpha, t, conv_state, ssm, out);
+}
+void orc_attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, const float* qn, const float* kn, const float* q, const float* k, const float* v,
+                   int start, int t, int kv_bits, int kv_recent, float* kc, float* vc, float* out) {
+  attn_core(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, start, t, kv_bits, kv_recent, kc, vc, out);
+}
+int orc_moe_ffn(int d, int n_exp, int top_k_, int ff, const OrcTensor* router, const OrcTensor* gate_e, const OrcTensor* up_e, const OrcTensor* down_e,
+                const float* sh_gate_inp, const OrcTensor* sh_gate, const OrcTensor* sh_up, const OrcTensor* sh_down,
+                const float* x, int t, float* y, int32_t* sel_idx, float* sel_w, int threads) {
+  return moe_ffn(d, n_exp, top_k_, ff, router, gate_e, up_e, down_e, sh_gate_inp, sh_gate, sh_up, sh_down, x, t, y, sel_idx, sel_w, threads) ? 0 : -1;
+}
+int orc_hc_mix(int d, int hc, float eps, const float* norm, const OrcTensor* down, const OrcTensor* inject, const OrcTensor* up,
+               const float* x, int t, float* mixed, float* inj, int threads) { return hc_mix(d, hc, eps, norm, down, inject, up, x, t, mixed, inj, threads) ? 0 : -1; }
+void orc_hc_combine(int d, int hc, float* x, const float* out, const float* inj, int t) { hc_combine(d, hc, x, out, inj, t); }
+
+OrcModel* orc_model_create(const OrcCfg* cfg, const OrcTensor* lt, const OrcTensor* globals, int threads) {
+  OrcModel* m = new OrcModel(); m->c = *cfg; m->threads = threads;
+  m->lt.assign(lt, lt + (size_t)cfg->n_layers * ORC_LAYER_SLOTS); for (int i = 0; i < ORC_GLOBAL_SLOTS; ++i) m->g[i] = globals[i];
+  m->vec.resize(m->lt.size());
+  static const int vs[] = {ORC_HCA_NORM, ORC_HCF_NORM, ORC_ATTN_QN, ORC_ATTN_KN, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_SH_GATE_INP};
+  for (int il = 0; il < cfg->n_layers; ++il) for (int s : vs) if (!to_vec(m->T(il, s), m->vec[(size_t)il * ORC_LAYER_SLOTS + s])) { delete m; return nullptr; }
+  if (!to_vec(m->g[ORC_G_HEAD_NORM], m->head_norm)) { delete m; return nullptr; }
+  m->rope_inv.resize(cfg->n_rot / 2); orc_rope_inv(cfg->n_rot, cfg->rope_base, m->rope_inv.data());
+  return m;
+}
+void orc_model_destroy(OrcModel* m) { delete m; }
+
+OrcState* orc_state_create(const OrcModel* m) {  // new_state, qwen4exp_gguf.rs:1345-1353
+  OrcState* s = new OrcState(); const OrcCfg& c = m->c; int ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv;
+  for (int il = 0; il < c.n_layers; ++il) {
+    if (m->full(il)) { s->k.emplace_back(); s->v.emplace_back(); }
+    else { s->conv.emplace_back((size_t)(c.conv_k - 1) * ch, 0.0f); s->ssm.emplace_back((size_t)c.lin_nv * c.lin_dk * c.lin_dv, 0.0f); }
+  }
+  return s;
+}
+void orc_state_destroy(OrcState* s) { delete s; }
+int orc_state_len(const OrcState* s) { return (int)s->tokens.size(); }
+float* orc_state_conv(OrcState* s, int li) { return s->conv[li].data(); }
+float* orc_state_ssm(OrcState* s, int li) { return s->ssm[li].data(); }
+float* orc_state_k(OrcState* s, int ai) { return s->k[ai].data(); }
+float* orc_state_v(OrcState* s, int ai) { return s->v[ai].data(); }
+
+// forward_inner, qwen4exp_gguf.rs:2087-2157 (host branch :2134-2142, head :2150-2153)
+int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, float* logits) {
+  const OrcCfg& c = m->c; int d = c.d, hc = c.hc; int start = (int)st->tokens.size(); int th = m->threads;
+  for (int i = 0; i < t; ++i) if (ids[i] >= (uint32_t)c.vocab) return -1;
+  st->tokens.insert(st->tokens.end(), ids, ids + t);
+  std::vector<float> x((size_t)t * hc * d), e(d);
+  const OrcTensor& embd = m->g[ORC_G_EMBD]; int qk, bs; if (!geom(embd.ty, &qk, &bs)) return -1; size_t erb = (size_t)d / qk * bs;
+  for (int ti = 0; ti < t; ++ti) { dequant(embd.ty, (const uint8_t*)embd.data + ids[ti] * erb, d, e.data()); for (int s = 0; s < hc; ++s) memcpy(&x[((size_t)ti * hc + s) * d], e.data(), sizeof(float) * d); }
+  int li = 0, ai = 0;
+  std::vector<float> mixed((size_t)t * d), inj((size_t)t * hc), o((size_t)t * d);
+  for (int il = 0; il < c.n_layers; ++il) {
+    if (hc_mix(d, hc, c.eps, m->V(il, ORC_HCA_NORM), &m->T(il, ORC_HCA_DOWN), &m->T(il, ORC_HCA_INJECT), &m->T(il, ORC_HCA_UP), x.data(), t, mixed.data(), inj.data(), th) == false) return -2;
+    if (m->full(il)) {  // attn, :1441-1446
+      int nh = c.n_head, nkv = c.n_kv, hd = c.hd; size_t row = (size_t)nkv * hd;
+      std::vector<float> q((size_t)t * nh * 2 * hd), k(t * row), v(t * row), att((size_t)t * nh * hd);
+      if (!mm(&m->T(il, ORC_ATTN_Q), mixed.data(), t, q.data(), th) || !mm(&m->T(il, ORC_ATTN_K), mixed.data(), t, k.data(), th) || !mm(&m->T(il, ORC_ATTN_V), mixed.data(), t, v.data(), th)) return -3;
+      st->k[ai].resize((size_t)(start + t) * row); st->v[ai].resize((size_t)(start + t) * row);
+      attn_core(nh, nkv, hd, c.n_rot, c.eps, m->rope_inv.data(), m->V(il, ORC_ATTN_QN), m->V(il, ORC_ATTN_KN), q.data(), k.data(), v.data(), start, t, c.kv_bits, c.kv_recent, st->k[ai].data(), st->v[ai].data(), att.data());
+      if (!mm(&m->T(il, ORC_ATTN_O), att.data(), t, o.data(), th)) return -3;
+      ++ai;
+    } else {  // linear, :1617-1621
+      int nk = c.lin_nk, nv = c.lin_nv, dk = c.lin_dk, dv = c.lin_dv; int ch = 2 * nk * dk + nv * dv;
+      std::vector<float> qkv((size_t)t * ch), z((size_t)t * nv * dv), be((size_t)t * nv), al((size_t)t * nv), oa((size_t)t * nv * dv);
+      if (!mm(&m->T(il, ORC_LIN_QKV), mixed.data(), t, qkv.data(), th) || !mm(&m->T(il, ORC_LIN_Z), mixed.data(), t, z.data(), th) || !mm(&m->T(il, ORC_LIN_BETA), mixed.data(), t, be.data(), th) || !mm(&m->T(il, ORC_LIN_ALPHA), mixed.data(), t, al.data(), th)) return -4;
+      gdn_core(nk, nv, dk, dv, c.conv_k, c.eps, m->V(il, ORC_LIN_A), m->V(il, ORC_LIN_DT), m->V(il, ORC_LIN_CONV), m->V(il, ORC_LIN_NORM), qkv.data(), z.data(), be.data(), al.data(), t, st->conv[li].data(), st->ssm[li].data(), oa.data());
+      if (!mm(&m->T(il, ORC_LIN_OUT), oa.data(), t, o.data(), th)) return -4;
+      ++li;
+    }
+    hc_combine(d, hc, x.data(), o.data(), inj.data(), t);
+    if (!hc_mix(d, hc, c.eps, m->V(il, ORC_HCF_NORM), &m->T(il, ORC_HCF_DOWN), &m->T(il, ORC_HCF_INJECT), &m->T(il, ORC_HCF_UP), x.data(), t, mixed.data(), inj.data(), th)) return -5;
+    if (!moe_ffn(d, c.n_exp, c.top_k, c.ff_exp, &m->T(il, ORC_ROUTER), &m->T(il, ORC_GATE_E), &m->T(il, ORC_UP_E), &m->T(il, ORC_DOWN_E), m->V(il, ORC_SH_GATE_INP),
+                 &m->T(il, ORC_SH_GATE), &m->T(il, ORC_SH_UP), &m->T(il, ORC_SH_DOWN), mixed.data(), t, o.data(), nullptr, nullptr, th)) return -6;
+    hc_combine(d, hc, x.data(), o.data(), inj.data(), t);
+  }
+  std::vector<float> h(d), dummy(hc);
+  if (!hc_mix(d, hc, c.eps, m->head_norm.data(), &m->g[ORC_G_HEAD_DOWN], nullptr, &m->g[ORC_G_HEAD_UP], x.data() + (size_t)(t - 1) * hc * d, 1, h.data(), dummy.data(), th)) return -7;
+  if (!mm(&m->g[ORC_G_OUT], h.data(), 1, logits, th)) return -8;  // head_logits, :2361-2364
+  return 0;
+}
+
+// forward_multi, qwen4exp_gguf.rs:2365-2480: logits after each token, every token's arithmetic equal to one-token
+// decode (:2357-2360), recurrent-state checkpoints after each token for spec_keep.
+int orc_forward_multi(const OrcModel* m, OrcState* st, const uint32_t* ids, int n, float* logits) {
+  st->ck.clear();
+  for (int i = 0; i < n; ++i) { int rc = orc_forward(m, st, ids + i, 1, logits + (size_t)i * m->c.vocab); if (rc) return rc; st->ck.push_back({st->conv, st->ssm}); }
+  return 0;
+}
+// spec_keep, qwen4exp_gguf.rs:2495-2515
+int orc_spec_keep(const OrcModel* m, OrcState* st, int t, int keep) {
+  if (keep >= t || t < 2) return 0; if (keep < 1) keep = 1; if ((int)st->ck.size() < t) return -1;
+  size_t n = st->tokens.size() - t + keep; st->tokens.resize(n);
+  st->conv = st->ck[keep - 1].conv; st->ssm = st->ck[keep - 1].ssm;
+  size_t row = (size_t)m->c.n_kv * m->c.hd; for (auto& k : st->k) k.resize(n * row); for (auto& v : st->v) v.resize(n * row);
+  return 0;
+}
+// spec::generate, greedy branch (spec.rs:156-267; accept loop :229-238, keep :249), drafts from a fixed stream:
+// the round that starts with `produced` tokens emitted proposes draft_stream[produced .. produced+kk).
+int orc_generate_greedy(const OrcModel* m, OrcState* st, const float* first_logits, int n_out, uint32_t* out, int n_draft, const uint32_t* draft_stream) {
+  size_t V = m->c.vocab; std::vector<float> lg(first_logits, first_logits + V), ls; int produced = 0, rounds = 0;
+  uint32_t pending = orc_argmax(lg.data(), V);
+  for (;;) {
+    out[produced++] = pending; if (produced >= n_out) break;
+    int left = n_out - produced; int kk = std::min(std::min(n_draft, left - 1), 8); if (!draft_stream) kk = 0;
+    if (kk <= 0) { if (orc_forward(m, st, &pending, 1, lg.data())) return -1; pending = orc_argmax(lg.data(), V); continue; }
+    std::vector<uint32_t> toks{pending}; for (int j = 0; j < kk; ++j) toks.push_back(draft_stream[produced + j]);
+    ls.resize(toks.size() * V); if (orc_forward_multi(m, st, toks.data(), (int)toks.size(), ls.data())) return -1;
+    int acc = 0; bool have = false; uint32_t nx = 0;
+    for (int i = 0; i < kk; ++i) { uint32_t tk = orc_argmax(ls.data() + (size_t)i * V, V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = orc_argmax(ls.data() + (size_t)kk * V, V);
+    orc_spec_keep(m, st, (int)toks.size(), acc + 1); ++rounds;
+    bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
+    if (stop) break; pending = nx;
+  }
+  return rounds;
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+/* CPU oracle for the Qwen-Next (qwen4exp) decode token loop.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is a from-scratch f32 restatement of the reference's host
+ * path (src/model/gguf_q.rs, src/model/kv4.rs, src/model/qwen4exp_gguf.rs, src/qn_ctx.rs,
+ * src/sampler.rs, src/spec.rs of the reference tree), used as the checker by tests/, by
+ * __graft_entry__.smoke() and by bench.py's cpu_baseline leg.  Nothing in the shipped HIP
+ * library links, loads or calls it.
+ *
+ * Pinning status (what fixes each function besides transcription):
+ *   orc_dequant            known-answer blocks derived from the format definition, the
+ *                          codebook digests, an independent numpy statement (tests/), sign and
+ *                          scale single-bit perturbation tests
+ *   orc_dot / orc_matmul   f64-accumulated dot of the dequantized rows
+ *   orc_kv4_*              the reference's own test inputs and asserted properties
+ *                          (kv4.rs:52-104), brute-force numpy statement
+ *   orc_rope_inv           closed form base^(-2i/n_rot), qn_ctx.rs:406-411
+ *   orc_argmax             sampler.rs:154-159 vector
+ *   orc_top_k              brute force on distinct logits + explicit ties
+ *   orc_gdn_core           closed forms (zero state, delta-rule overwrite property, pure decay,
+ *                          one-hot conv = delay) + an independent numpy statement
+ *   orc_attn_core          single position, uniform keys, rope at pos 0, numpy statement
+ *   orc_moe_ffn            numpy statement built from orc_dequant'd dense weights
+ *   orc_forward            numpy statement of the whole token step on a tiny model
+ * Parity unpinned (only running the reference could pin): the last-ulp behaviour of
+ * expf/log1pf/powf/sincosf on the reference's own target libm.
+ */
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids, gguf_q.rs:25-28 */
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_IQ2_XS = 17, ORC_IQ3_S = 21, ORC_BF16 = 30 };
+
+typedef struct { uint32_t ty; uint64_t rows, cols; const void* data; } OrcTensor;
+
+/* per-layer tensor slots (GGUF tensor names in comments, qwen4exp_gguf.rs:494-512) */
+enum {
+  ORC_HCA_NORM = 0, ORC_HCA_DOWN, ORC_HCA_INJECT, ORC_HCA_UP,       /* blk.N.hc_attn_{norm,down,inject,up} */
+  ORC_HCF_NORM, ORC_HCF_DOWN, ORC_HCF_INJECT, ORC_HCF_UP,           /* blk.N.hc_ffn_* */
+  ORC_ATTN_Q, ORC_ATTN_K, ORC_ATTN_V, ORC_ATTN_O, ORC_ATTN_QN, ORC_ATTN_KN,
+  ORC_LIN_QKV, ORC_LIN_Z, ORC_LIN_BETA, ORC_LIN_ALPHA, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_LIN_OUT,
+  ORC_ROUTER, ORC_GATE_E, ORC_UP_E, ORC_DOWN_E, ORC_SH_GATE_INP, ORC_SH_GATE, ORC_SH_UP, ORC_SH_DOWN,
+  ORC_LAYER_SLOTS
+};
+enum { ORC_G_EMBD = 0, ORC_G_HEAD_NORM, ORC_G_HEAD_DOWN, ORC_G_HEAD_UP, ORC_G_OUT, ORC_GLOBAL_SLOTS };
+
+typedef struct {
+  int32_t n_layers, d, hc, hc_lr, n_head, n_kv, hd, n_rot;
+  float rope_base, eps;
+  int32_t n_exp, top_k, ff_exp;
+  int32_t lin_nk, lin_nv, lin_dk, lin_dv, conv_k, full_every;
+  int32_t vocab;
+  int32_t kv_bits;    /* 0 = f32 cache everywhere, 4 = positions below the packed boundary are read through kv4 */
+  int32_t kv_recent;  /* f32 window kept at the tail (reference default 1024) */
+} OrcCfg;
+
+int    orc_type_geom(uint32_t ty, int* elems, int* bytes);
+int    orc_dequant(uint32_t ty, const uint8_t* x, size_t n_elems, float* y);
+float  orc_dot(const float* a, const float* b, size_t n);
+int    orc_matmul(uint32_t ty, const uint8_t* w, size_t rows, size_t cols, const float* x, int t, float* y, int threads);
+void   orc_expand_iq3s(uint32_t* out512);
+void   orc_expand_iq2xs(uint64_t* out512);
+uint8_t orc_ksigns(int i);
+
+void   orc_kv4_pack(const float* x, size_t n, uint32_t* w, float* sc);
+float  orc_kv4_get(const uint32_t* w, const float* sc, size_t i);
+void   orc_kvq_roundtrip(float* x, size_t n, int bits);
+size_t orc_kv_packed_boundary(size_t n_visible, int kv_bits, int recent);
+
+void   orc_rope_inv(int n_rot, float base, float* inv);
+uint32_t orc_argmax(const float* logits, size_t n);
+int    orc_top_k(const float* r, int n, int k, int32_t* idx, float* w);
+void   orc_rms(const float* x, const float* w, float eps, float* y, size_t n);
+void   orc_rms_inplace(float* x, const float* w, float eps, size_t n);
+float  orc_sigm(float x);
+float  orc_silu(float x);
+float  orc_softplus(float x);
+
+/* Gated DeltaNet after its projections (linear_core).  proj = qkv [t][ch], z [t][nv*dv], beta [t][nv], alpha [t][nv].
+ * conv_state [(k-1)][ch] oldest first, ssm [nv][dk][dv]; both updated in place.  out [t][nv*dv]. */
+void   orc_gdn_core(int nk, int nv, int dk, int dv, int conv_k, float eps,
+                    const float* a, const float* dt, const float* conv_w, const float* norm_w,
+                    const float* qkv, const float* z, const float* beta, const float* alpha, int t,
+                    float* conv_state, float* ssm, float* out);
+
+/* Gated attention core (attn_core, dense branch).  q [t][nh][2*hd], k,v [t][nkv*hd] (raw projections).
+ * kc/vc: caller-owned caches with room for start+t rows of nkv*hd floats; rows [0,start) valid on entry. */
+void   orc_attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* rope_inv,
+                     const float* qn, const float* kn, const float* q, const float* k, const float* v,
+                     int start, int t, int kv_bits, int kv_recent, float* kc, float* vc, float* out);
+
+/* MoE FFN (ffn + routed f32 branch).  x [t][d] -> y [t][d]. sel_idx/sel_w (optional) receive [t][k]. */
+int    orc_moe_ffn(int d, int n_exp, int top_k, int ff, const OrcTensor* router, const OrcTensor* gate_e,
+                   const OrcTensor* up_e, const OrcTensor* down_e, const float* sh_gate_inp,
+                   const OrcTensor* sh_gate, const OrcTensor* sh_up, const OrcTensor* sh_down,
+                   const float* x, int t, float* y, int32_t* sel_idx, float* sel_w, int threads);
+
+/* Hyper-connection mix / combine (hc_mix, hc_combine).  inject may be NULL (head mixer). */
+int    orc_hc_mix(int d, int hc, float eps, const float* norm, const OrcTensor* down, const OrcTensor* inject,
+                  const OrcTensor* up, const float* x, int t, float* mixed, float* inj, int threads);
+void   orc_hc_combine(int d, int hc, float* x, const float* out, const float* inj, int t);
+
+typedef struct OrcModel OrcModel;
+typedef struct OrcState OrcState;
+OrcModel* orc_model_create(const OrcCfg* cfg, const OrcTensor* layer_tensors /*[n_layers][ORC_LAYER_SLOTS]*/,
+                           const OrcTensor* globals /*[ORC_GLOBAL_SLOTS]*/, int threads);
+void      orc_model_destroy(OrcModel*);
+OrcState* orc_state_create(const OrcModel*);
+void      orc_state_destroy(OrcState*);
+int       orc_state_len(const OrcState*);
+/* direct access for tests: li-th GDN layer's conv / ssm, ai-th attention layer's k / v cache */
+float*    orc_state_conv(OrcState*, int li);
+float*    orc_state_ssm(OrcState*, int li);
+float*    orc_state_k(OrcState*, int ai);
+float*    orc_state_v(OrcState*, int ai);
+/* Model::forward: append ids, return logits of the last token in logits[vocab]. */
+int       orc_forward(const OrcModel*, OrcState*, const uint32_t* ids, int n, float* logits);
+/* forward_multi semantics = n sequential steps; logits [n][vocab]; keeps per-token checkpoints. */
+int       orc_forward_multi(const OrcModel*, OrcState*, const uint32_t* ids, int n, float* logits);
+/* spec_keep(t, keep): roll the state back so that only the first `keep` of the last t tokens remain. */
+int       orc_spec_keep(const OrcModel*, OrcState*, int t, int keep);
+/* spec::generate, greedy branch, with an optional fixed draft source: drafts[i] (n_draft per round) are proposed
+ * after each pending token; out receives n_out tokens.  Returns the number of verify rounds used. */
+int       orc_generate_greedy(const OrcModel*, OrcState*, const float* first_logits, int n_out, uint32_t* out,
+                              int n_draft, const uint32_t* draft_stream);
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,280 @@
+"""Independent numpy statements used to pin the C++ oracle (and, through it, the HIP library).
+
+Nothing here shares code with oracle/pyre_oracle.cpp: the codebooks are re-expanded from the header text,
+the dequantizers are vectorised over blocks, and the block-level math (DeltaNet, attention, MoE, hyper-connections,
+token step) is written in float64 from the format / architecture definitions.
+"""
+import hashlib
+import os
+import re
+
+import numpy as np
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# sha256 of the expanded little-endian tables, computed from the reference's iq_tables.rs by oracle/make_codebooks.py
+IQ3S_SHA256 = "bd1af4945a1717c65610b0284e4628b9a1ba3b306fae3a06f6e5f597356e349f"
+IQ2XS_SHA256 = "06e47aaca60b4dc1d9b5a3f34540437058a6b142b4d7a59d5ded769b4d1bf1de"
+KSIGNS_SHA256 = "a76742a603f8beca5212ecce0f1f02f11a4887fd2f7c8b15aca0ea3eb3380c31"
+
+
+def _codes(path, name):
+    txt = open(path).read()
+    m = re.search(r"%s\[(\d+)\] = \{(.*?)\};" % name, txt, re.S)
+    v = np.array([int(s) for s in re.findall(r"\d+", m.group(2))], dtype=np.uint32)
+    assert v.size == int(m.group(1))
+    return v
+
+
+def codebooks(header=None):
+    """(iq3s_grid u8[512,4], iq2xs_grid u8[512,8], ksigns u8[128]) expanded from a codebook header."""
+    header = header or os.path.join(_ROOT, "oracle", "iq_codebooks.h")
+    c3 = _codes(header, "kIq3sCode")
+    c2 = _codes(header, "kIq2xsCode")
+    g3 = np.stack([2 * ((c3 >> (3 * j)) & 7) + 1 for j in range(4)], axis=1).astype(np.uint8)
+    tri = np.array([8, 25, 43], dtype=np.uint8)
+    g2 = np.stack([tri[(c2 >> (2 * j)) & 3] for j in range(8)], axis=1).astype(np.uint8)
+    i = np.arange(128, dtype=np.uint32)
+    par = np.zeros(128, dtype=np.uint32)
+    for b in range(7):
+        par ^= (i >> b) & 1
+    ks = (i | (par << 7)).astype(np.uint8)
+    return g3, g2, ks
+
+
+def codebook_digests(header=None):
+    g3, g2, ks = codebooks(header)
+    return (hashlib.sha256(g3.tobytes()).hexdigest(), hashlib.sha256(g2.tobytes()).hexdigest(), hashlib.sha256(ks.tobytes()).hexdigest())
+
+
+def f16_to_f32(b):
+    return np.ascontiguousarray(b).view(np.float16).astype(np.float32)
+
+
+def _signs(s):
+    """sign byte array [...] -> [..., 8] of +-1 float32 (bit j set = negative)."""
+    return np.where((s[..., None] >> np.arange(8, dtype=np.uint8)) & 1, np.float32(-1), np.float32(1)).astype(np.float32)
+
+
+def dequant(ty, raw, n):
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    g3, g2, ks = codebooks()
+    if ty == 0:
+        return raw[:4 * n].view(np.float32).copy()
+    if ty == 1:
+        return f16_to_f32(raw[:2 * n])
+    if ty == 30:
+        return (raw[:2 * n].view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+    if ty == 8:
+        b = raw[:n // 32 * 34].reshape(-1, 34)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        return (b[:, 2:].view(np.int8).astype(np.float32) * d).reshape(-1)
+    if ty == 12:
+        b = raw[:n // 256 * 144].reshape(-1, 144)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1)
+        mn = f16_to_f32(b[:, 2:4].copy()).reshape(-1)
+        sc = b[:, 4:16].astype(np.uint32)
+        s = np.empty((b.shape[0], 8), dtype=np.uint32); m = np.empty_like(s)
+        for j in range(8):
+            if j < 4:
+                s[:, j] = sc[:, j] & 63; m[:, j] = sc[:, j + 4] & 63
+            else:
+                s[:, j] = (sc[:, j + 4] & 0xF) | ((sc[:, j - 4] >> 6) << 4)
+                m[:, j] = (sc[:, j + 4] >> 4) | ((sc[:, j] >> 6) << 4)
+        q = b[:, 16:].reshape(-1, 4, 32)
+        out = np.empty((b.shape[0], 4, 2, 32), dtype=np.float32)
+        for g in range(4):
+            d1 = (d * s[:, 2 * g].astype(np.float32)).astype(np.float32)[:, None]
+            m1 = (mn * m[:, 2 * g].astype(np.float32)).astype(np.float32)[:, None]
+            d2 = (d * s[:, 2 * g + 1].astype(np.float32)).astype(np.float32)[:, None]
+            m2 = (mn * m[:, 2 * g + 1].astype(np.float32)).astype(np.float32)[:, None]
+            out[:, g, 0] = (d1 * (q[:, g] & 0xF).astype(np.float32)).astype(np.float32) - m1
+            out[:, g, 1] = (d2 * (q[:, g] >> 4).astype(np.float32)).astype(np.float32) - m2
+        return out.reshape(-1)
+    if ty == 17:
+        b = raw[:n // 256 * 74].reshape(-1, 74)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qs = b[:, 2:66].copy().view(np.uint16).reshape(-1, 8, 4).astype(np.uint32)
+        sc = b[:, 66:74]
+        lo = ((d * (np.float32(0.5) + (sc & 0xF).astype(np.float32))).astype(np.float32) * np.float32(0.25)).astype(np.float32)
+        hi = ((d * (np.float32(0.5) + (sc >> 4).astype(np.float32))).astype(np.float32) * np.float32(0.25)).astype(np.float32)
+        db = np.stack([lo, lo, hi, hi], axis=2)                       # [nb, 8, 4]
+        grid = g2[qs & 511].astype(np.float32)                        # [nb, 8, 4, 8]
+        sg = _signs(ks[qs >> 9])
+        return ((db[..., None] * grid).astype(np.float32) * sg).astype(np.float32).reshape(-1)
+    if ty == 21:
+        b = raw[:n // 256 * 110].reshape(-1, 110)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qs = b[:, 2:66].reshape(-1, 8, 8).astype(np.uint32)           # [nb, sub-block, 8 index bytes]
+        qh = b[:, 66:74].astype(np.uint32)                            # one byte per sub-block
+        sg = b[:, 74:106].reshape(-1, 8, 4)
+        sc = b[:, 106:110]
+        nib = np.stack([sc & 0xF, sc >> 4], axis=2).reshape(-1, 8).astype(np.float32)
+        db = (d * (np.float32(1) + np.float32(2) * nib)).astype(np.float32)   # d * (1 + 2 nib) -- integer valued, exact
+        hbit = (qh[:, :, None] >> np.arange(8, dtype=np.uint32)) & 1   # bit k of qh goes with index byte k
+        idx = qs | (hbit << 8)
+        grid = g3[idx].astype(np.float32).reshape(-1, 8, 4, 8)         # two 4-byte entries per group of 8 values
+        s = _signs(sg)
+        return ((db[:, :, None, None] * grid).astype(np.float32) * s).astype(np.float32).reshape(-1)
+    raise ValueError(ty)
+
+
+# ---- hand packers for known-answer blocks -----------------------------------------------------------------------
+def f16_bytes(v):
+    return np.array([v], dtype=np.float16).view(np.uint8)
+
+
+def pack_iq3s(d, qs, qh, signs, scales):
+    b = np.zeros(110, dtype=np.uint8)
+    b[0:2] = f16_bytes(d); b[2:66] = qs; b[66:74] = qh; b[74:106] = signs; b[106:110] = scales
+    return b
+
+
+def pack_iq2xs(d, qs16, scales):
+    b = np.zeros(74, dtype=np.uint8)
+    b[0:2] = f16_bytes(d); b[2:66] = np.asarray(qs16, dtype=np.uint16).view(np.uint8); b[66:74] = scales
+    return b
+
+
+def pack_q4k(d, dmin, s, m, q):
+    """s, m: 8 six-bit scale / min values; q: 256 four-bit values in element order."""
+    b = np.zeros(144, dtype=np.uint8)
+    b[0:2] = f16_bytes(d); b[2:4] = f16_bytes(dmin)
+    s = np.asarray(s, dtype=np.uint8); m = np.asarray(m, dtype=np.uint8)
+    sc = np.zeros(12, dtype=np.uint8)
+    for j in range(4):
+        sc[j] = (s[j] & 63) | ((s[j + 4] >> 4) << 6)
+        sc[j + 4] = (m[j] & 63) | ((m[j + 4] >> 4) << 6)
+        sc[j + 8] = (s[j + 4] & 0xF) | ((m[j + 4] & 0xF) << 4)
+    b[4:16] = sc
+    q = np.asarray(q, dtype=np.uint8).reshape(4, 2, 32)
+    b[16:] = (q[:, 0] | (q[:, 1] << 4)).reshape(-1)
+    return b
+
+
+def pack_q8_0(d, q):
+    b = np.zeros(34, dtype=np.uint8)
+    b[0:2] = f16_bytes(d); b[2:] = np.asarray(q, dtype=np.int8).view(np.uint8)
+    return b
+
+
+# ---- float64 block math -----------------------------------------------------------------------------------------
+def sigm(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def silu(x):
+    return x * sigm(x)
+
+
+def softplus(x):
+    return np.where(x > 20.0, x, np.log1p(np.exp(np.minimum(x, 20.0))))
+
+
+def rms(x, w, eps):
+    return x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * w
+
+
+def kv4_roundtrip(x):
+    x = np.asarray(x, dtype=np.float32).reshape(-1, 32)
+    m = np.abs(x).max(axis=1, keepdims=True)
+    s = np.where((m > 0) & np.isfinite(m), (m / np.float32(7)).astype(np.float32), np.float32(0))
+    with np.errstate(divide="ignore", invalid="ignore"):
+        r = (x / s).astype(np.float32)
+    q = np.where(s > 0, np.clip(np.sign(r) * np.floor(np.abs(r) + np.float32(0.5)), -7, 7), 0).astype(np.int32).astype(np.float32)  # integer code: no -0
+    return (q * s).astype(np.float32).reshape(-1), q.astype(np.int32).reshape(-1), s.reshape(-1)
+
+
+def gdn_step(nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w, qkv, z, beta, alpha, conv_state, S):
+    """One token, float64.  conv_state [(k-1), ch] oldest first, S [nv, dk, dv]. Returns (out, conv_state', S')."""
+    ch = 2 * nk * dk + nv * dv
+    conv_w = np.asarray(conv_w, dtype=np.float64).reshape(ch, conv_k)
+    win = np.concatenate([np.asarray(conv_state, dtype=np.float64).reshape(conv_k - 1, ch), np.asarray(qkv, dtype=np.float64)[None]], axis=0)
+    co = silu((win * conv_w.T).sum(axis=0))
+    q = co[:nk * dk].reshape(nk, dk); k = co[nk * dk:2 * nk * dk].reshape(nk, dk); v = co[2 * nk * dk:].reshape(nv, dv)
+    q = q / np.sqrt((q * q).sum(-1, keepdims=True) + 1e-6) / np.sqrt(dk)
+    k = k / np.sqrt((k * k).sum(-1, keepdims=True) + 1e-6)
+    S = np.asarray(S, dtype=np.float64).reshape(nv, dk, dv).copy()
+    out = np.empty((nv, dv))
+    for h in range(nv):
+        kh = h % nk
+        g = np.exp(softplus(float(alpha[h]) + float(dt[h])) * float(a[h])); b = sigm(float(beta[h]))
+        S[h] *= g
+        mem = S[h].T @ k[kh]
+        delta = (v[h] - mem) * b
+        S[h] += np.outer(k[kh], delta)
+        o = S[h].T @ q[kh]
+        out[h] = rms(o, np.asarray(norm_w, dtype=np.float64), eps) * sigm(np.asarray(z, dtype=np.float64)[h * dv:(h + 1) * dv])
+    return out.reshape(-1), win[1:], S
+
+
+def rope(v, pos, n_rot, inv):
+    v = np.array(v, dtype=np.float64); half = n_rot // 2
+    ang = np.float64(np.float32(pos)) * np.asarray(inv, dtype=np.float64)
+    c, s = np.cos(ang), np.sin(ang)
+    x0, x1 = v[..., :half].copy(), v[..., half:n_rot].copy()
+    v[..., :half] = x0 * c - x1 * s
+    v[..., half:n_rot] = x1 * c + x0 * s
+    return v
+
+
+def attn_step(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, pos, K, V, packed_below=0):
+    """One token at position pos, float64. K,V [pos, nkv*hd] caches (f32 content). Returns (out, k_row, v_row)."""
+    k = rope(rms(np.asarray(k, dtype=np.float64).reshape(nkv, hd), np.asarray(kn, dtype=np.float64), eps), pos, n_rot, inv)
+    Kf = np.concatenate([np.asarray(K, dtype=np.float64).reshape(pos, nkv * hd), k.reshape(1, -1)], axis=0)
+    Vf = np.concatenate([np.asarray(V, dtype=np.float64).reshape(pos, nkv * hd), np.asarray(v, dtype=np.float64).reshape(1, -1)], axis=0)
+    Ke, Ve = Kf.copy(), Vf.copy()
+    if packed_below:
+        Ke[:packed_below] = kv4_roundtrip(Kf[:packed_below].astype(np.float32))[0].reshape(packed_below, -1)
+        Ve[:packed_below] = kv4_roundtrip(Vf[:packed_below].astype(np.float32))[0].reshape(packed_below, -1)
+    q = np.asarray(q, dtype=np.float64).reshape(nh, 2 * hd)
+    out = np.empty((nh, hd)); grp = nh // nkv
+    for h in range(nh):
+        qh = rope(rms(q[h, :hd], np.asarray(qn, dtype=np.float64), eps), pos, n_rot, inv)
+        kvh = h // grp
+        sc = Ke[:, kvh * hd:(kvh + 1) * hd] @ qh / np.sqrt(hd)
+        w = np.exp(sc - sc.max()); w /= w.sum()
+        out[h] = (w[:, None] * Ve[:, kvh * hd:(kvh + 1) * hd]).sum(0) * sigm(q[h, hd:])
+    return out.reshape(-1), Kf[-1].astype(np.float32), Vf[-1].astype(np.float32)
+
+
+def top_k(r, k):
+    r = np.asarray(r, dtype=np.float64).copy(); r[np.isnan(r)] = -np.inf
+    order = sorted(range(r.size), key=lambda e: (-r[e], e))[:k]
+    idx = np.array(sorted(order))
+    mx = r[idx].max()
+    if not np.isfinite(mx):
+        return idx, np.full(k, 1.0 / k)
+    w = np.exp(r[idx] - mx)
+    return idx, w / w.sum()
+
+
+def moe_ffn(d, n_exp, k, ff, W, x):
+    """W: dict of dense float64 matrices router [E,d], gate_e [E,ff,d], up_e [E,ff,d], down_e [E,d,ff], sh_gate_inp [d],
+    sh_gate [sf,d], sh_up [sf,d], sh_down [d,sf].  x [d]."""
+    x = np.asarray(x, dtype=np.float64)
+    lg = W["router"] @ x
+    y = W["sh_down"] @ (silu(W["sh_gate"] @ x) * (W["sh_up"] @ x))
+    y = y * sigm(W["sh_gate_inp"] @ x)
+    idx, w = top_k(lg, k)
+    for e, we in zip(idx, w):
+        h = silu(W["gate_e"][e] @ x) * (W["up_e"][e] @ x)
+        y = y + we * (W["down_e"][e] @ h)
+    return y, idx, w
+
+
+def hc_mix(d, hc, eps, norm, down, inject, up, x):
+    x = np.asarray(x, dtype=np.float64).reshape(hc, d)
+    xn = np.stack([rms(x[s], np.asarray(norm, dtype=np.float64)[s * d:(s + 1) * d], eps) for s in range(hc)]).reshape(-1)
+    lo = silu((down @ xn) / hc)
+    inj = (inject @ xn) / hc if inject is not None else np.zeros(hc)
+    gate = up @ lo
+    mixed = (xn * sigm(gate)).reshape(hc, d).sum(0) / hc
+    return mixed, inj
+
+
+def hc_combine(d, hc, x, out, inj):
+    x = np.asarray(x, dtype=np.float64).reshape(hc, d).copy()
+    for s in range(hc):
+        x[s] += out * (2.0 * sigm(inj[s]))
+    return x.reshape(-1)

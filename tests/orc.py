@@ -1,0 +1,267 @@
+"""ctypes binding of the CPU oracle (oracle/liborc.so).  Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+_SO = os.path.join(_DIR, "liborc.so")
+
+F32, F16, Q8_0, Q4_K, IQ2_XS, IQ3_S, BF16 = 0, 1, 8, 12, 17, 21, 30
+(HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
+ ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, LAYER_SLOTS) = range(32)
+G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
+
+
+class Tensor(C.Structure):
+    _fields_ = [("ty", C.c_uint32), ("rows", C.c_uint64), ("cols", C.c_uint64), ("data", C.c_void_p)]
+
+
+class Cfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
+               [("rope_base", C.c_float), ("eps", C.c_float)] + \
+               [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
+                                         "full_every", "vocab", "kv_bits", "kv_recent")]
+
+
+def build():
+    subprocess.check_call(["make", "-s", "-C", _DIR])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        L.orc_dot.restype = C.c_float
+        L.orc_kv4_get.restype = C.c_float
+        L.orc_kv_packed_boundary.restype = C.c_size_t
+        L.orc_kv_packed_boundary.argtypes = [C.c_size_t, C.c_int, C.c_int]
+        L.orc_argmax.restype = C.c_uint32
+        L.orc_ksigns.restype = C.c_uint8
+        for n in ("orc_sigm", "orc_silu", "orc_softplus"):
+            getattr(L, n).restype = C.c_float
+            getattr(L, n).argtypes = [C.c_float]
+        L.orc_model_create.restype = C.c_void_p
+        L.orc_state_create.restype = C.c_void_p
+        for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v"):
+            getattr(L, n).restype = C.POINTER(C.c_float)
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def dequant(ty, raw, n):
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    y = np.empty(n, dtype=np.float32)
+    rc = lib().orc_dequant(C.c_uint32(ty), _p(raw), C.c_size_t(n), _p(y))
+    assert rc == 0
+    return y
+
+
+def dot(a, b):
+    a, b = f32(a), f32(b)
+    return float(lib().orc_dot(_p(a), _p(b), C.c_size_t(a.size)))
+
+
+def matmul(ty, raw, rows, cols, x, threads=4):
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    x = f32(x).reshape(-1, cols)
+    t = x.shape[0]
+    y = np.empty((t, rows), dtype=np.float32)
+    rc = lib().orc_matmul(C.c_uint32(ty), _p(raw), C.c_size_t(rows), C.c_size_t(cols), _p(x), C.c_int(t), _p(y), C.c_int(threads))
+    assert rc == 0
+    return y
+
+
+def kv4_pack(x):
+    x = f32(x).reshape(-1)
+    w = np.empty(x.size // 8, dtype=np.uint32)
+    sc = np.empty(x.size // 32, dtype=np.float32)
+    lib().orc_kv4_pack(_p(x), C.c_size_t(x.size), _p(w), _p(sc))
+    return w, sc
+
+
+def kv4_unpack(w, sc, n):
+    return np.array([lib().orc_kv4_get(_p(w), _p(sc), C.c_size_t(i)) for i in range(n)], dtype=np.float32)
+
+
+def kvq_roundtrip(x, bits):
+    y = f32(x).reshape(-1).copy()
+    lib().orc_kvq_roundtrip(_p(y), C.c_size_t(y.size), C.c_int(bits))
+    return y.reshape(np.shape(x))
+
+
+def packed_boundary(n, kv_bits=4, recent=1024):
+    return int(lib().orc_kv_packed_boundary(n, kv_bits, recent))
+
+
+def rope_inv(n_rot, base):
+    inv = np.empty(n_rot // 2, dtype=np.float32)
+    lib().orc_rope_inv(C.c_int(n_rot), C.c_float(base), _p(inv))
+    return inv
+
+
+def argmax(l):
+    l = f32(l)
+    return int(lib().orc_argmax(_p(l), C.c_size_t(l.size)))
+
+
+def top_k(r, k):
+    r = f32(r)
+    idx = np.empty(k, dtype=np.int32)
+    w = np.empty(k, dtype=np.float32)
+    rc = lib().orc_top_k(_p(r), C.c_int(r.size), C.c_int(k), _p(idx), _p(w))
+    assert rc == 0
+    return idx, w
+
+
+def tensor(ty, rows, cols, arr):
+    """arr: numpy array holding the raw bytes (kept alive by the caller)."""
+    return Tensor(ty, rows, cols, arr.ctypes.data if arr is not None else None)
+
+
+def vec_tensor(arr):
+    return Tensor(F32, 1, arr.size, arr.ctypes.data)
+
+
+def gdn_core(nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w, qkv, z, beta, alpha, conv_state, ssm):
+    """Runs t tokens; conv_state and ssm (float32 arrays) are updated in place. Returns out [t][nv*dv]."""
+    qkv = f32(qkv); t = qkv.shape[0]
+    z, beta, alpha = f32(z), f32(beta), f32(alpha)
+    a, dt, conv_w, norm_w = f32(a), f32(dt), f32(conv_w), f32(norm_w)
+    out = np.empty((t, nv * dv), dtype=np.float32)
+    lib().orc_gdn_core(nk, nv, dk, dv, conv_k, C.c_float(eps), _p(a), _p(dt), _p(conv_w), _p(norm_w), _p(qkv), _p(z), _p(beta), _p(alpha),
+                       C.c_int(t), _p(conv_state), _p(ssm), _p(out))
+    return out
+
+
+def attn_core(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, start, kv_bits, kv_recent, kc, vc):
+    q = f32(q); t = q.shape[0]
+    k, v, qn, kn, inv = f32(k), f32(v), f32(qn), f32(kn), f32(inv)
+    out = np.empty((t, nh * hd), dtype=np.float32)
+    lib().orc_attn_core(nh, nkv, hd, n_rot, C.c_float(eps), _p(inv), _p(qn), _p(kn), _p(q), _p(k), _p(v), C.c_int(start), C.c_int(t),
+                        C.c_int(kv_bits), C.c_int(kv_recent), _p(kc), _p(vc), _p(out))
+    return out
+
+
+def moe_ffn(d, n_exp, k, ff, router, gate_e, up_e, down_e, sh_gate_inp, sh_gate, sh_up, sh_down, x, threads=4):
+    x = f32(x).reshape(-1, d); t = x.shape[0]
+    y = np.empty((t, d), dtype=np.float32)
+    idx = np.empty((t, k), dtype=np.int32); w = np.empty((t, k), dtype=np.float32)
+    sgi = f32(sh_gate_inp)
+    rc = lib().orc_moe_ffn(d, n_exp, k, ff, C.byref(router), C.byref(gate_e), C.byref(up_e), C.byref(down_e), _p(sgi),
+                           C.byref(sh_gate), C.byref(sh_up), C.byref(sh_down), _p(x), C.c_int(t), _p(y), _p(idx), _p(w), C.c_int(threads))
+    assert rc == 0
+    return y, idx, w
+
+
+def hc_mix(d, hc, eps, norm, down, inject, up, x, threads=4):
+    x = f32(x).reshape(-1, hc * d); t = x.shape[0]
+    norm = f32(norm)
+    mixed = np.empty((t, d), dtype=np.float32); inj = np.empty((t, hc), dtype=np.float32)
+    rc = lib().orc_hc_mix(d, hc, C.c_float(eps), _p(norm), C.byref(down), C.byref(inject) if inject is not None else None, C.byref(up),
+                          _p(x), C.c_int(t), _p(mixed), _p(inj), C.c_int(threads))
+    assert rc == 0
+    return mixed, inj
+
+
+def hc_combine(d, hc, x, out, inj):
+    x = f32(x).copy(); out = f32(out); inj = f32(inj)
+    t = x.size // (hc * d)
+    lib().orc_hc_combine(d, hc, _p(x), _p(out), _p(inj), C.c_int(t))
+    return x
+
+
+class Model:
+    """Oracle model over a weight set (see tests/modelgen.py for the container)."""
+
+    def __init__(self, cfg, layer_tensors, globals_, threads=4, keep=()):
+        self.cfg = cfg
+        self._keep = keep
+        n = cfg.n_layers * LAYER_SLOTS
+        self._lt = (Tensor * n)(*layer_tensors)
+        self._g = (Tensor * GLOBAL_SLOTS)(*globals_)
+        self.h = C.c_void_p(lib().orc_model_create(C.byref(cfg), self._lt, self._g, C.c_int(threads)))
+        assert self.h
+
+    def new_state(self):
+        return State(self)
+
+    def forward(self, ids, st):
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        lg = np.empty(self.cfg.vocab, dtype=np.float32)
+        rc = lib().orc_forward(self.h, st.h, _p(ids), C.c_int(ids.size), _p(lg))
+        assert rc == 0, rc
+        return lg
+
+    def forward_multi(self, ids, st):
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        lg = np.empty((ids.size, self.cfg.vocab), dtype=np.float32)
+        rc = lib().orc_forward_multi(self.h, st.h, _p(ids), C.c_int(ids.size), _p(lg))
+        assert rc == 0, rc
+        return lg
+
+    def spec_keep(self, st, t, keep):
+        assert lib().orc_spec_keep(self.h, st.h, C.c_int(t), C.c_int(keep)) == 0
+
+    def generate_greedy(self, st, first_logits, n_out, n_draft=0, draft_stream=None):
+        out = np.empty(n_out, dtype=np.uint32)
+        fl = f32(first_logits)
+        ds = None
+        if draft_stream is not None:
+            ds = np.ascontiguousarray(draft_stream, dtype=np.uint32)
+            assert ds.size >= n_out + 8
+        rounds = lib().orc_generate_greedy(self.h, st.h, _p(fl), C.c_int(n_out), _p(out), C.c_int(n_draft), _p(ds) if ds is not None else None)
+        assert rounds >= 0
+        return out, rounds
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_model_destroy(self.h)
+            self.h = None
+
+
+class State:
+    def __init__(self, model):
+        self.m = model
+        self.h = C.c_void_p(lib().orc_state_create(model.h))
+
+    def __len__(self):
+        return lib().orc_state_len(self.h)
+
+    def ssm(self, li):
+        c = self.m.cfg
+        n = c.lin_nv * c.lin_dk * c.lin_dv
+        return np.ctypeslib.as_array(lib().orc_state_ssm(self.h, li), shape=(n,))
+
+    def conv(self, li):
+        c = self.m.cfg
+        ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv
+        return np.ctypeslib.as_array(lib().orc_state_conv(self.h, li), shape=((c.conv_k - 1) * ch,))
+
+    def kcache(self, ai):
+        c = self.m.cfg
+        return np.ctypeslib.as_array(lib().orc_state_k(self.h, ai), shape=(len(self) * c.n_kv * c.hd,))
+
+    def vcache(self, ai):
+        c = self.m.cfg
+        return np.ctypeslib.as_array(lib().orc_state_v(self.h, ai), shape=(len(self) * c.n_kv * c.hd,))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_state_destroy(self.h)
+            self.h = None
