@@ -1,0 +1,153 @@
+"""Synthetic qwen4exp weight sets (host side) for tests, smoke and the benchmark.
+
+Tensor slots follow the GGUF tensor names the reference loads (qwen4exp_gguf.rs:494-512); the slot numbering is the
+one include/pyre_hip.h declares.  Every tensor is (ggml type id, rows, cols, raw bytes) with rows = prod(shape[1:]),
+cols = shape[0] as Gguf::mat lays them out (gguf_q.rs:326-331).
+"""
+from dataclasses import dataclass, field
+
+import numpy as np
+
+from . import synth
+
+(HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
+ ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, LAYER_SLOTS) = range(32)
+G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
+
+CFG_FIELDS = ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot", "rope_base", "eps", "n_exp", "top_k",
+              "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k", "full_every", "vocab", "kv_bits", "kv_recent")
+
+
+@dataclass
+class Config:
+    n_layers: int = 4
+    d: int = 256
+    hc: int = 2
+    hc_lr: int = 32
+    n_head: int = 4
+    n_kv: int = 2
+    hd: int = 256
+    n_rot: int = 64
+    rope_base: float = 1e7
+    eps: float = 1e-6
+    n_exp: int = 8
+    top_k: int = 2
+    ff_exp: int = 256
+    lin_nk: int = 2
+    lin_nv: int = 4
+    lin_dk: int = 128
+    lin_dv: int = 128
+    conv_k: int = 4
+    full_every: int = 4
+    vocab: int = 512
+    kv_bits: int = 4
+    kv_recent: int = 1024
+    # generation knobs (not part of the model contract)
+    qtype: int = synth.IQ3_S          # type of every projection / expert / embedding / head matrix
+    hc_type: int = synth.BF16         # type of the hyper-connection matrices (BF16 in real files)
+    ff_sh: int = 0                    # shared-expert width (0 = ff_exp)
+    d_lo: float = 1e-3
+    d_hi: float = 2e-2
+
+    @property
+    def ch(self):
+        return 2 * self.lin_nk * self.lin_dk + self.lin_nv * self.lin_dv
+
+    def full(self, il):
+        return (il + 1) % self.full_every == 0
+
+
+def a3b_config(**kw):
+    """The Qwen-Next-style A3B hybrid of the benchmark: 48 layers (3 Gated DeltaNet + 1 gated attention per group),
+    512 routed experts top-10 + 1 shared, d 2048, expert ff 512, vocab 151936, 4 hyper-connection streams."""
+    c = Config(n_layers=48, d=2048, hc=4, hc_lr=256, n_head=16, n_kv=2, hd=256, n_rot=64, rope_base=1e7, eps=1e-6,
+               n_exp=512, top_k=10, ff_exp=512, lin_nk=16, lin_nv=32, lin_dk=128, lin_dv=128, conv_k=4, full_every=4,
+               vocab=151936, kv_bits=4, kv_recent=1024, qtype=synth.IQ3_S, hc_type=synth.IQ3_S)
+    for k, v in kw.items():
+        setattr(c, k, v)
+    return c
+
+
+def tensor_specs(c: Config):
+    """[(layer or -1, slot, kind, ty, rows, cols)] for every tensor of the model; kind in {'q','vec:<name>'}."""
+    sf = c.ff_sh or c.ff_exp
+    w = c.hc * c.d
+    out = []
+    for il in range(c.n_layers):
+        for base in (HCA_NORM, HCF_NORM):
+            out += [(il, base, "vec:norm1", synth.F32, 1, w), (il, base + 1, "q", c.hc_type, c.hc_lr, w),
+                    (il, base + 2, "q", c.hc_type, c.hc, w),
+                    (il, base + 3, "q", c.hc_type, w, c.hc_lr)]
+        if c.full(il):
+            out += [(il, ATTN_Q, "q", c.qtype, c.n_head * 2 * c.hd, c.d), (il, ATTN_K, "q", c.qtype, c.n_kv * c.hd, c.d),
+                    (il, ATTN_V, "q", c.qtype, c.n_kv * c.hd, c.d), (il, ATTN_O, "q", c.qtype, c.d, c.n_head * c.hd),
+                    (il, ATTN_QN, "vec:norm1", synth.F32, 1, c.hd), (il, ATTN_KN, "vec:norm1", synth.F32, 1, c.hd)]
+        else:
+            out += [(il, LIN_QKV, "q", c.qtype, c.ch, c.d), (il, LIN_Z, "q", c.qtype, c.lin_nv * c.lin_dv, c.d),
+                    (il, LIN_BETA, "q", c.qtype, c.lin_nv, c.d), (il, LIN_ALPHA, "q", c.qtype, c.lin_nv, c.d),
+                    (il, LIN_A, "vec:a", synth.F32, 1, c.lin_nv), (il, LIN_DT, "vec:dt", synth.F32, 1, c.lin_nv),
+                    (il, LIN_CONV, "vec:conv", synth.F32, 1, c.ch * c.conv_k), (il, LIN_NORM, "vec:norm1", synth.F32, 1, c.lin_dv),
+                    (il, LIN_OUT, "q", c.qtype, c.d, c.lin_nv * c.lin_dv)]
+        out += [(il, ROUTER, "router", synth.BF16, c.n_exp, c.d), (il, GATE_E, "q", c.qtype, c.n_exp * c.ff_exp, c.d),
+                (il, UP_E, "q", c.qtype, c.n_exp * c.ff_exp, c.d), (il, DOWN_E, "q", c.qtype, c.n_exp * c.d, c.ff_exp),
+                (il, SH_GATE_INP, "vec:small", synth.F32, 1, c.d), (il, SH_GATE, "q", c.qtype, sf, c.d),
+                (il, SH_UP, "q", c.qtype, sf, c.d), (il, SH_DOWN, "q", c.qtype, c.d, sf)]
+    out += [(-1, G_EMBD, "q", c.qtype, c.vocab, c.d), (-1, G_HEAD_NORM, "vec:norm1", synth.F32, 1, w),
+            (-1, G_HEAD_DOWN, "q", c.hc_type, c.hc_lr, w), (-1, G_HEAD_UP, "q", c.hc_type, w, c.hc_lr),
+            (-1, G_OUT, "q", c.qtype, c.vocab, c.d)]
+    return out
+
+
+def tensor_seed(seed, il, slot):
+    return (seed * 1000003 + (il + 1) * 64 + slot) & 0x7FFFFFFFFFFFFFFF
+
+
+def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
+    s = tensor_seed(seed, il, slot)
+    if kind == "q":
+        if ty in (synth.F32, synth.F16, synth.BF16):
+            std = 1.0 / np.sqrt(cols)
+            if ty == synth.BF16:
+                return synth.bf16_normal(rows, cols, s, std)
+            x = synth.normal((rows, cols), s, std)
+            return (x if ty == synth.F32 else x.astype(np.float16)).view(np.uint8).reshape(-1).copy()
+        return synth.matrix(ty, rows, cols, s, c.d_lo, c.d_hi)
+    if kind == "router":
+        return synth.bf16_normal(rows, cols, s, 0.02)
+    name = kind.split(":")[1]
+    if name == "norm1":
+        v = synth.normal((cols,), s, 0.1, 1.0)
+    elif name == "a":
+        v = -np.exp(synth.uniform((cols,), s, 0.0, float(np.log(16.0))))      # ssm_a = -exp(A_log), A_log ~ U(0, ln 16)
+    elif name == "dt":
+        v = np.zeros(cols, dtype=np.float32)
+    elif name == "conv":
+        v = synth.normal((cols,), s, 0.5)
+    elif name == "small":
+        v = synth.normal((cols,), s, 0.02)
+    else:
+        raise ValueError(kind)
+    return v.astype(np.float32).view(np.uint8).reshape(-1).copy()
+
+
+@dataclass
+class HostWeights:
+    cfg: Config
+    seed: int
+    layers: list = field(default_factory=list)     # per layer: dict slot -> (ty, rows, cols, bytes)
+    globals_: dict = field(default_factory=dict)
+
+    def f32(self, il, slot):
+        ty, rows, cols, b = (self.layers[il] if il >= 0 else self.globals_)[slot]
+        assert ty == synth.F32
+        return b.view(np.float32)
+
+
+def build_host(c: Config, seed=1):
+    """All tensors as numpy byte arrays (only sensible for small configurations)."""
+    hw = HostWeights(c, seed, [dict() for _ in range(c.n_layers)], {})
+    for il, slot, kind, ty, rows, cols in tensor_specs(c):
+        b = host_tensor(c, seed, il, slot, kind, ty, rows, cols)
+        (hw.layers[il] if il >= 0 else hw.globals_)[slot] = (ty, rows, cols, b)
+    return hw

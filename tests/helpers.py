@@ -1,0 +1,82 @@
+"""Shared test helpers: oracle tensors / models from pyre_amd.modelgen weight sets, dense float64 views."""
+import numpy as np
+
+import np_ref
+import orc
+from pyre_amd import modelgen as mg
+
+
+def relerr(a, b):
+    a = np.asarray(a, dtype=np.float64).reshape(-1); b = np.asarray(b, dtype=np.float64).reshape(-1)
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def orc_tensor(entry):
+    ty, rows, cols, b = entry
+    return orc.tensor(ty, rows, cols, b)
+
+
+def orc_cfg(c):
+    cfg = orc.Cfg()
+    for f in mg.CFG_FIELDS:
+        setattr(cfg, f, getattr(c, f))
+    return cfg
+
+
+def orc_model(hw, threads=4):
+    c = hw.cfg
+    lt = []
+    for il in range(c.n_layers):
+        for slot in range(mg.LAYER_SLOTS):
+            e = hw.layers[il].get(slot)
+            lt.append(orc_tensor(e) if e is not None else orc.Tensor(0, 0, 0, None))
+    g = [orc_tensor(hw.globals_[s]) for s in range(mg.GLOBAL_SLOTS)]
+    return orc.Model(orc_cfg(c), lt, g, threads=threads, keep=(hw,))
+
+
+def dense(entry):
+    ty, rows, cols, b = entry
+    return np_ref.dequant(ty, b, rows * cols).reshape(rows, cols).astype(np.float64)
+
+
+def np_forward_tokens(hw, ids):
+    """float64 numpy statement of the token loop (one token at a time); returns logits after each token."""
+    c = hw.cfg; d, hc = c.d, c.hc
+    inv = (np.float64(np.float32(c.rope_base)) ** (-2.0 * np.arange(c.n_rot // 2) / c.n_rot))
+    L = [{s: (dense(e) if e[0] != 0 or e[1] > 1 else e[3].view(np.float32).astype(np.float64)) for s, e in lay.items()} for lay in hw.layers]
+    G = {s: (dense(e) if e[1] > 1 else e[3].view(np.float32).astype(np.float64)) for s, e in hw.globals_.items()}
+    conv = {}; S = {}; K = {}; V = {}
+    for il in range(c.n_layers):
+        if c.full(il):
+            K[il] = np.zeros((0, c.n_kv * c.hd), np.float32); V[il] = np.zeros((0, c.n_kv * c.hd), np.float32)
+        else:
+            conv[il] = np.zeros((c.conv_k - 1, c.ch)); S[il] = np.zeros((c.lin_nv, c.lin_dk, c.lin_dv))
+    out = []
+    for pos, tok in enumerate(ids):
+        x = np.tile(G[mg.G_EMBD][tok], hc)
+        for il in range(c.n_layers):
+            W = L[il]
+            m, inj = np_ref.hc_mix(d, hc, c.eps, W[mg.HCA_NORM], W[mg.HCA_DOWN], W[mg.HCA_INJECT], W[mg.HCA_UP], x)
+            if c.full(il):
+                n = pos + 1
+                pb = orc.packed_boundary(n, c.kv_bits, c.kv_recent)
+                o, kr, vr = np_ref.attn_step(c.n_head, c.n_kv, c.hd, c.n_rot, c.eps, inv, W[mg.ATTN_QN], W[mg.ATTN_KN],
+                                             W[mg.ATTN_Q] @ m, W[mg.ATTN_K] @ m, W[mg.ATTN_V] @ m, pos, K[il], V[il], pb)
+                K[il] = np.concatenate([K[il], kr[None]]); V[il] = np.concatenate([V[il], vr[None]])
+                o = W[mg.ATTN_O] @ o
+            else:
+                o, conv[il], S[il] = np_ref.gdn_step(c.lin_nk, c.lin_nv, c.lin_dk, c.lin_dv, c.conv_k, c.eps, W[mg.LIN_A], W[mg.LIN_DT],
+                                                     W[mg.LIN_CONV], W[mg.LIN_NORM], W[mg.LIN_QKV] @ m, W[mg.LIN_Z] @ m,
+                                                     W[mg.LIN_BETA] @ m, W[mg.LIN_ALPHA] @ m, conv[il], S[il])
+                o = W[mg.LIN_OUT] @ o
+            x = np_ref.hc_combine(d, hc, x, o, inj)
+            m, inj = np_ref.hc_mix(d, hc, c.eps, W[mg.HCF_NORM], W[mg.HCF_DOWN], W[mg.HCF_INJECT], W[mg.HCF_UP], x)
+            sf = W[mg.SH_GATE].shape[0]
+            Wm = {"router": W[mg.ROUTER], "gate_e": W[mg.GATE_E].reshape(c.n_exp, c.ff_exp, d), "up_e": W[mg.UP_E].reshape(c.n_exp, c.ff_exp, d),
+                  "down_e": W[mg.DOWN_E].reshape(c.n_exp, d, c.ff_exp), "sh_gate_inp": W[mg.SH_GATE_INP], "sh_gate": W[mg.SH_GATE],
+                  "sh_up": W[mg.SH_UP], "sh_down": W[mg.SH_DOWN]}
+            o, _, _ = np_ref.moe_ffn(d, c.n_exp, c.top_k, c.ff_exp, Wm, m)
+            x = np_ref.hc_combine(d, hc, x, o, inj)
+        h, _ = np_ref.hc_mix(d, hc, c.eps, G[mg.G_HEAD_NORM], G[mg.G_HEAD_DOWN], None, G[mg.G_HEAD_UP], x)
+        out.append(G[mg.G_OUT] @ h)
+    return np.array(out)

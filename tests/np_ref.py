@@ -210,7 +210,7 @@ def gdn_step(nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w, qkv, z, beta, a
 
 def rope(v, pos, n_rot, inv):
     v = np.array(v, dtype=np.float64); half = n_rot // 2
-    ang = np.float64(np.float32(pos)) * np.asarray(inv, dtype=np.float64)
+    ang = (np.float32(pos) * np.asarray(inv, dtype=np.float32)).astype(np.float64)   # the angle itself is an f32 product (qwen4exp_gguf.rs:530)
     c, s = np.cos(ang), np.sin(ang)
     x0, x1 = v[..., :half].copy(), v[..., half:n_rot].copy()
     v[..., :half] = x0 * c - x1 * s
