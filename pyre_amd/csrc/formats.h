@@ -1,0 +1,213 @@
+// GGUF block formats on the device: plane geometry, bit-exact element decode, and the factored per-unit
+// dot products the GEMV kernels use.  Format definitions: src/model/gguf_q.rs:67-166 of the reference.
+#pragma once
+#include "common.h"
+
+enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_COUNT = 7 };
+
+struct FmtGeom { int el, bytes; int V; int e1, e2, e3, eb; };   // GGUF block (elements, bytes); plane entry sizes
+__host__ __device__ inline FmtGeom fmt_geom(int fmt) {
+  switch (fmt) {
+    case FMT_F32:    return {1, 4, 16, 0, 0, 0, 0};
+    case FMT_F16:    return {1, 2, 8, 0, 0, 0, 0};
+    case FMT_BF16:   return {1, 2, 8, 0, 0, 0, 0};
+    case FMT_Q8_0:   return {32, 34, 4, 4, 0, 0, 0};     // p1: the two f16 scales of the unit's two blocks
+    case FMT_Q4_K:   return {256, 144, 2, 0, 0, 0, 16};  // pb: d, dmin, scales[12]
+    case FMT_IQ2_XS: return {256, 74, 1, 2, 0, 0, 2};    // p1: two scale bytes; pb: d
+    default:         return {256, 110, 1, 8, 2, 1, 2};   // IQ3_S  p1: signs, p2: qh pair, p3: scale byte; pb: d
+  }
+}
+inline int fmt_from_ggml(uint32_t ty) {
+  switch (ty) { case PYRE_F32: return FMT_F32; case PYRE_F16: return FMT_F16; case PYRE_BF16: return FMT_BF16; case PYRE_Q8_0: return FMT_Q8_0;
+    case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S; }
+  return -1;
+}
+
+// ---- plane accessors ------------------------------------------------------------------------------------------------
+template <int V> __device__ __forceinline__ uint4 ld_vec(const QMatDev& m, int tile, int ku, int chunk, int lane) {
+  return ((const uint4*)m.p0)[(((size_t)tile * m.U + ku) * V + chunk) * 64 + lane];
+}
+template <typename E> __device__ __forceinline__ E ld_small(const uint8_t* p, const QMatDev& m, int tile, int ku, int lane) {
+  return ((const E*)p)[((size_t)tile * m.U + ku) * 64 + lane];
+}
+template <typename E> __device__ __forceinline__ E ld_block(const QMatDev& m, int tile, int ku, int lane) {
+  return ((const E*)m.pb)[((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane];
+}
+
+__device__ __forceinline__ float h2f_bits(uint32_t h) { return __half2float(__ushort_as_half((unsigned short)(h & 0xFFFF))); }
+__device__ __forceinline__ float flip(float v, uint32_t neg) { return __uint_as_float(__float_as_uint(v) ^ (neg << 31)); }
+__device__ __forceinline__ uint32_t ksigns(uint32_t i) { return i | ((__popc(i) & 1u) << 7); }   // KSIGNS_IQ2XS closed form
+// byte i (0..11) of the Q4_K scales field held in three dwords (selects, so the words stay in registers)
+__device__ __forceinline__ uint32_t k4_byte(uint32_t a, uint32_t b, uint32_t c, int i) { uint32_t w = i < 4 ? a : (i < 8 ? b : c); return (w >> (8 * (i & 3))) & 0xFF; }
+__device__ __forceinline__ void scale_min_k4(int j, uint32_t a, uint32_t b, uint32_t c, uint32_t& s, uint32_t& m) {    // gguf_q.rs:62-64
+  if (j < 4) { s = k4_byte(a, b, c, j) & 63; m = k4_byte(a, b, c, j + 4) & 63; }
+  else { s = (k4_byte(a, b, c, j + 4) & 0xF) | ((k4_byte(a, b, c, j - 4) >> 6) << 4); m = (k4_byte(a, b, c, j + 4) >> 4) | ((k4_byte(a, b, c, j) >> 6) << 4); }
+}
+
+// ---- bit-exact decode of one unit (64 consecutive values of one row) -----------------------------------------------
+// Same operations in the same order as gguf_q::dequant; compiled with -ffp-contract=off so nothing is fused.
+template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const uint32_t* g3, const uint64_t* g2, int tile, int ku, int lane, float* y) {
+  if constexpr (FMT == FMT_F32) {
+    for (int c = 0; c < 16; ++c) { uint4 v = ld_vec<16>(m, tile, ku, c, lane); y[4 * c] = __uint_as_float(v.x); y[4 * c + 1] = __uint_as_float(v.y); y[4 * c + 2] = __uint_as_float(v.z); y[4 * c + 3] = __uint_as_float(v.w); }
+  } else if constexpr (FMT == FMT_F16 || FMT == FMT_BF16) {
+    for (int c = 0; c < 8; ++c) {
+      uint4 v = ld_vec<8>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int k = 0; k < 4; ++k) for (int hh = 0; hh < 2; ++hh) { uint32_t u = (w[k] >> (16 * hh)) & 0xFFFF; y[8 * c + 2 * k + hh] = FMT == FMT_F16 ? h2f_bits(u) : __uint_as_float(u << 16); }
+    }
+  } else if constexpr (FMT == FMT_Q8_0) {          // gguf_q.rs:79
+    uint32_t dd = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
+    for (int c = 0; c < 4; ++c) {
+      float d = h2f_bits(dd >> (16 * (c >> 1)));
+      uint4 v = ld_vec<4>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int k = 0; k < 16; ++k) y[16 * c + k] = (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3))) * d;
+    }
+  } else if constexpr (FMT == FMT_Q4_K) {          // gguf_q.rs:103-107
+    uint4 hb = ld_block<uint4>(m, tile, ku, lane);
+    float d = h2f_bits(hb.x), mn = h2f_bits(hb.x >> 16);
+    int j = ku & 3; uint32_t s1, m1, s2, m2; scale_min_k4(2 * j, hb.y, hb.z, hb.w, s1, m1); scale_min_k4(2 * j + 1, hb.y, hb.z, hb.w, s2, m2);
+    float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
+    for (int c = 0; c < 2; ++c) {
+      uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int k = 0; k < 16; ++k) { uint32_t b = (w[k >> 2] >> (8 * (k & 3))) & 0xFF; y[16 * c + k] = d1 * (float)(b & 0xF) - M1; y[32 + 16 * c + k] = d2 * (float)(b >> 4) - M2; }
+    }
+  } else if constexpr (FMT == FMT_IQ2_XS) {        // gguf_q.rs:126-129
+    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
+    uint32_t sc = ld_small<uint16_t>(m.p1, m, tile, ku, lane);
+    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int ib = 0; ib < 2; ++ib) {
+      uint32_t s = (sc >> (8 * ib)) & 0xFF;
+      float db0 = d * (0.5f + (float)(s & 0xF)) * 0.25f, db1 = d * (0.5f + (float)(s >> 4)) * 0.25f;
+      for (int l = 0; l < 4; ++l) {
+        uint32_t q = (w[2 * ib + (l >> 1)] >> (16 * (l & 1))) & 0xFFFF;
+        uint64_t g = g2[q & 511]; uint32_t sg = ksigns(q >> 9); float db = l < 2 ? db0 : db1;
+        for (int jj = 0; jj < 8; ++jj) y[32 * ib + 8 * l + jj] = flip(db * (float)(uint32_t)((g >> (8 * jj)) & 0xFF), (sg >> jj) & 1);
+      }
+    }
+  } else {                                         // IQ3_S, gguf_q.rs:141-151
+    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
+    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t q[4] = {v.x, v.y, v.z, v.w};
+    uint2 sv = ld_small<uint2>(m.p1, m, tile, ku, lane); uint32_t sg[2] = {sv.x, sv.y};
+    uint32_t qh = ld_small<uint16_t>(m.p2, m, tile, ku, lane), sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
+    for (int sb = 0; sb < 2; ++sb) {
+      float db = d * (float)(1 + 2 * ((sc >> (4 * sb)) & 0xF)); uint32_t h = (qh >> (8 * sb)) & 0xFF;
+      for (int l = 0; l < 4; ++l) {
+        uint32_t qq = q[2 * sb + (l >> 1)] >> (16 * (l & 1));
+        uint32_t gA = g3[(qq & 0xFF) | ((h << (8 - 2 * l)) & 256)], gB = g3[((qq >> 8) & 0xFF) | ((h << (7 - 2 * l)) & 256)];
+        uint32_t s = (sg[sb] >> (8 * l)) & 0xFF;
+        for (int jj = 0; jj < 4; ++jj) { y[32 * sb + 8 * l + jj] = flip(db * (float)((gA >> (8 * jj)) & 0xFF), (s >> jj) & 1); y[32 * sb + 8 * l + 4 + jj] = flip(db * (float)((gB >> (8 * jj)) & 0xFF), (s >> (4 + jj)) & 1); }
+      }
+    }
+  }
+}
+
+// ---- factored per-unit dot products for the GEMV ------------------------------------------------------------------
+// xs points at the unit's 64 activations of token 0 (wave-uniform address -> scalar loads); token t is xs + t*xstride.
+// acc[t] += sum_j W[row, 64*ku + j] * x[t][64*ku + j].  The operation sequence per token does not depend on T.
+template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint32_t* lds3, const uint2* lds2, int tile, int ku, int lane,
+                                                                   const float* __restrict__ xs, int xstride, float (&acc)[T]) {
+  if constexpr (FMT == FMT_F32) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) { uint4 v = ld_vec<16>(m, tile, ku, c, lane); float w[4] = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[t] = fmaf(w[k], xs[t * xstride + 4 * c + k], acc[t]); }
+  } else if constexpr (FMT == FMT_F16 || FMT == FMT_BF16) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      uint4 v = ld_vec<8>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float lo = FMT == FMT_F16 ? h2f_bits(w[k]) : __uint_as_float(w[k] << 16), hi = FMT == FMT_F16 ? h2f_bits(w[k] >> 16) : __uint_as_float(w[k] & 0xFFFF0000u);
+#pragma unroll
+        for (int t = 0; t < T; ++t) { acc[t] = fmaf(lo, xs[t * xstride + 8 * c + 2 * k], acc[t]); acc[t] = fmaf(hi, xs[t * xstride + 8 * c + 2 * k + 1], acc[t]); }
+      }
+    }
+  } else if constexpr (FMT == FMT_Q8_0) {
+    uint32_t dd = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        uint4 v = ld_vec<4>(m, tile, ku, 2 * b + c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 16; ++k) { float f = (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3)));
+#pragma unroll
+          for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 32 * b + 16 * c + k], part[t]); }
+      }
+      float d = h2f_bits(dd >> (16 * b));
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(d, part[t], acc[t]);
+    }
+  } else if constexpr (FMT == FMT_Q4_K) {
+    uint4 hb = ld_block<uint4>(m, tile, ku, lane);
+    float d = h2f_bits(hb.x), mn = h2f_bits(hb.x >> 16);
+    int j = ku & 3; uint32_t s1, m1, s2, m2; scale_min_k4(2 * j, hb.y, hb.z, hb.w, s1, m1); scale_min_k4(2 * j + 1, hb.y, hb.z, hb.w, s2, m2);
+    float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        uint32_t b = (w[k >> 2] >> (8 * (k & 3))) & 0xFF;
+        float lo = fmaf(d1, (float)(b & 0xF), -M1), hi = fmaf(d2, (float)(b >> 4), -M2);
+#pragma unroll
+        for (int t = 0; t < T; ++t) { acc[t] = fmaf(lo, xs[t * xstride + 16 * c + k], acc[t]); acc[t] = fmaf(hi, xs[t * xstride + 32 + 16 * c + k], acc[t]); }
+      }
+    }
+  } else if constexpr (FMT == FMT_IQ2_XS) {
+    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
+    uint32_t sc = ld_small<uint16_t>(m.p1, m, tile, ku, lane);
+    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int ib = 0; ib < 2; ++ib) {
+      uint32_t s = (sc >> (8 * ib)) & 0xFF;
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+#pragma unroll
+        for (int l2 = 0; l2 < 2; ++l2) {
+          int l = 2 * hf + l2;
+          uint32_t q = (w[2 * ib + (l >> 1)] >> (16 * (l & 1))) & 0xFFFF;
+          uint2 g = lds2[q & 511]; uint32_t sg = ksigns(q >> 9);
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            uint32_t gw = jj < 4 ? g.x : g.y;
+            float f = __uint_as_float(__float_as_uint((float)((gw >> (8 * (jj & 3))) & 0xFF)) | ((sg << (31 - jj)) & 0x80000000u));
+#pragma unroll
+            for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 32 * ib + 8 * l + jj], part[t]);
+          }
+        }
+        float db = d * (0.5f + (float)((s >> (4 * hf)) & 0xF)) * 0.25f;
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
+      }
+    }
+  } else {   // IQ3_S
+    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
+    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t q[4] = {v.x, v.y, v.z, v.w};
+    uint2 sv = ld_small<uint2>(m.p1, m, tile, ku, lane); uint32_t sg[2] = {sv.x, sv.y};
+    uint32_t qh = ld_small<uint16_t>(m.p2, m, tile, ku, lane), sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      uint32_t h = (qh >> (8 * sb)) & 0xFF;
+      float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+#pragma unroll
+      for (int l = 0; l < 4; ++l) {
+        uint32_t qq = q[2 * sb + (l >> 1)] >> (16 * (l & 1));
+        uint32_t gA = lds3[(qq & 0xFF) | ((h << (8 - 2 * l)) & 256)], gB = lds3[((qq >> 8) & 0xFF) | ((h << (7 - 2 * l)) & 256)];
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+          uint32_t gw = jj < 4 ? gA : gB; int bit = 8 * l + jj;
+          float f = __uint_as_float(__float_as_uint((float)((gw >> (8 * (jj & 3))) & 0xFF)) | ((sg[sb] << (31 - bit)) & 0x80000000u));
+#pragma unroll
+          for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 32 * sb + 8 * l + jj], part[t]);
+        }
+      }
+      float db = d * (float)(1 + 2 * ((sc >> (4 * sb)) & 0xF));
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
+    }
+  }
+}

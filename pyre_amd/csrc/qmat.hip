@@ -1,0 +1,249 @@
+// Quantized matrix operator: GGUF blocks -> lane=row planes (repack), bit-exact dequant export, dequant-GEMV.
+// Drop-in for QMat / QMat::matmul of the reference (src/model/gguf_q.rs:201-247).
+#include "formats.h"
+#include <stdlib.h>
+
+// ---- repack: raw GGUF rows -> planes --------------------------------------------------------------------------------
+// One thread per (padded row, unit).  Rows beyond m.rows are written as zeros (they decode to 0 and are never stored).
+__global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_bytes, uint8_t* p0, uint8_t* p1, uint8_t* p2, uint8_t* p3, uint8_t* pb) {
+  size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t total = (size_t)m.tiles * 64 * m.U;
+  if (gid >= total) return;
+  int ku = (int)(gid % m.U); size_t r = gid / m.U; int tile = (int)(r / 64), lane = (int)(r % 64);
+  bool live = r < (size_t)m.rows;
+  const uint8_t* row = raw + r * row_bytes;
+  FmtGeom g = fmt_geom(m.fmt);
+  size_t e = ((size_t)tile * m.U + ku) * 64 + lane;              // entry index in per-unit planes
+  uint8_t* v = p0 + ((size_t)tile * m.U + ku) * g.V * 64 * 16;     // chunk c of this lane at v + (c*64 + lane)*16
+  auto put_vec = [&](int chunk, const uint8_t* src) { uint8_t* d = v + ((size_t)chunk * 64 + lane) * 16; for (int i = 0; i < 16; ++i) d[i] = live ? src[i] : 0; };
+  switch (m.fmt) {
+    case FMT_F32: for (int c = 0; c < 16; ++c) put_vec(c, row + (size_t)ku * 256 + 16 * c); break;
+    case FMT_F16: case FMT_BF16: for (int c = 0; c < 8; ++c) put_vec(c, row + (size_t)ku * 128 + 16 * c); break;
+    case FMT_Q8_0: {
+      const uint8_t* b0 = row + (size_t)(2 * ku) * 34; const uint8_t* b1 = b0 + 34;
+      put_vec(0, b0 + 2); put_vec(1, b0 + 18); put_vec(2, b1 + 2); put_vec(3, b1 + 18);
+      uint8_t* d = p1 + e * 4; d[0] = live ? b0[0] : 0; d[1] = live ? b0[1] : 0; d[2] = live ? b1[0] : 0; d[3] = live ? b1[1] : 0;
+    } break;
+    case FMT_Q4_K: {
+      const uint8_t* b = row + (size_t)(ku >> 2) * 144; int j = ku & 3;
+      put_vec(0, b + 16 + 32 * j); put_vec(1, b + 32 + 32 * j);
+      if (j == 0) { uint8_t* d = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 16; for (int i = 0; i < 16; ++i) d[i] = live ? b[i] : 0; }
+    } break;
+    case FMT_IQ2_XS: {
+      const uint8_t* b = row + (size_t)(ku >> 2) * 74; int j = ku & 3;
+      put_vec(0, b + 2 + 16 * j);
+      uint8_t* d = p1 + e * 2; d[0] = live ? b[66 + 2 * j] : 0; d[1] = live ? b[67 + 2 * j] : 0;
+      if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
+    } break;
+    default: {   // IQ3_S
+      const uint8_t* b = row + (size_t)(ku >> 2) * 110; int j = ku & 3;
+      put_vec(0, b + 2 + 16 * j);
+      uint8_t* s = p1 + e * 8; for (int i = 0; i < 8; ++i) s[i] = live ? b[74 + 8 * j + i] : 0;
+      uint8_t* h = p2 + e * 2; h[0] = live ? b[66 + 2 * j] : 0; h[1] = live ? b[67 + 2 * j] : 0;
+      p3[e] = live ? b[106 + j] : 0;
+      if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
+    }
+  }
+}
+
+// ---- bit-exact dequant export -----------------------------------------------------------------------------------------
+// grid (U, tiles), 64 threads: lane l decodes unit ku of row tile*64+l, the tile is transposed through LDS so that
+// each row's 64 values leave as one contiguous 256-byte store.
+template <int FMT> __global__ __launch_bounds__(64) void k_dequant(QMatDev m, const uint32_t* g3, const uint64_t* g2, float* __restrict__ out) {
+  __shared__ float tile_buf[64][65];
+  int ku = blockIdx.x, tile = blockIdx.y, lane = threadIdx.x;
+  float y[64];
+  decode_exact<FMT>(m, g3, g2, tile, ku, lane, y);
+  for (int i = 0; i < 64; ++i) tile_buf[lane][i] = y[i];
+  __syncthreads();
+  for (int r = 0; r < 64; ++r) { size_t row = (size_t)tile * 64 + r; if (row < (size_t)m.rows) out[row * m.cols + (size_t)ku * 64 + lane] = tile_buf[r][lane]; }
+}
+
+// rows by index (embedding lookup, QMat::row): grid (ceil(U/64), n), 64 threads, thread = unit
+template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const uint32_t* g3, const uint64_t* g2, const uint32_t* __restrict__ idx, float* __restrict__ out, int out_stride) {
+  int ku = blockIdx.x * 64 + threadIdx.x; if (ku >= m.U) return;
+  uint32_t r = idx[blockIdx.y]; if (r >= (uint32_t)m.rows) return;
+  float y[64];
+  decode_exact<FMT>(m, g3, g2, (int)(r >> 6), ku, (int)(r & 63), y);
+  float* o = out + (size_t)blockIdx.y * out_stride + (size_t)ku * 64;
+  for (int i = 0; i < 64; ++i) o[i] = y[i];
+}
+
+// ---- dequant-GEMV -----------------------------------------------------------------------------------------------------
+// grid (tiles, ksplit), NW waves.  Wave w of K-slice ks walks units [(ks*NW+w)*upw, +upw).  Lane l owns row tile*64+l:
+// weights come from coalesced per-lane loads, activations from wave-uniform (scalar) loads, so there is no cross-lane
+// reduction at all; the NW partial sums meet in LDS, and when the row's K range is split over several workgroups the
+// last one to finish (ticket counter) adds the slices in slice order - a fixed order, so results are reproducible.
+template <int FMT, int T, int NW>
+__global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int ksplit, int upw,
+                                                  float* partial, uint32_t* ticket, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  __shared__ float red[NW][T][64];
+  __shared__ uint32_t is_last;
+  const int tile = blockIdx.x, ks = blockIdx.y;
+  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
+  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int k0 = (ks * NW + wave) * upw; const int k1 = min(m.U, k0 + upw);
+  float acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+  for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds3, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
+#pragma unroll
+  for (int t = 0; t < T; ++t) red[wave][t][lane] = acc[t];
+  __syncthreads();
+  const size_t r64 = (size_t)m.tiles * 64;
+  for (int i = threadIdx.x; i < T * 64; i += NW * 64) {
+    int t = i >> 6, l = i & 63; float s = red[0][t][l];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) s += red[w][t][l];
+    size_t row = (size_t)tile * 64 + l;
+    if (ksplit == 1) { if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s; }
+    else partial[((size_t)ks * T + t) * r64 + row] = s;
+  }
+  if (ksplit == 1) return;
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) { uint32_t old = atomicAdd(&ticket[tile], 1u); is_last = (old == (uint32_t)(ksplit - 1)); }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  for (int i = threadIdx.x; i < T * 64; i += NW * 64) {
+    int t = i >> 6, l = i & 63; size_t row = (size_t)tile * 64 + l;
+    float s = partial[(size_t)t * r64 + row];
+    for (int k = 1; k < ksplit; ++k) s += partial[((size_t)k * T + t) * r64 + row];
+    if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s;
+  }
+  if (threadIdx.x == 0) ticket[tile] = 0;   // ready for the next launch on this stream
+}
+
+namespace {
+constexpr int kNW = 4;
+int env_int(const char* n, int dflt) { const char* v = getenv(n); return v && *v ? atoi(v) : dflt; }
+
+template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y) {
+  static const int target_waves = env_int("PYRE_GEMV_WAVES", 4096), max_upw = env_int("PYRE_GEMV_MAX_UPW", 8);
+  long total = (long)m.tiles * m.U;
+  int upw = (int)((total + target_waves - 1) / target_waves); if (upw < 1) upw = 1; if (upw > max_upw) upw = max_upw; if (upw > m.U) upw = m.U;
+  int wpt = (m.U + upw - 1) / upw; int ksplit = (wpt + kNW - 1) / kNW;
+  if (ksplit > 1) { int rc = pyre_workspace(ctx, (size_t)ksplit * T * m.tiles * 64 * sizeof(float), (size_t)m.tiles); if (rc) return rc; }
+  hipLaunchKernelGGL((k_gemv<FMT, T, kNW>), dim3(m.tiles, ksplit), dim3(kNW * 64), 0, ctx->stream, m, x, y, ksplit, upw, ctx->ws_partial, ctx->ws_ticket,
+                     (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
+  switch (t) { case 1: return gemv_t<FMT, 1>(ctx, m, x, y); case 2: return gemv_t<FMT, 2>(ctx, m, x, y); case 3: return gemv_t<FMT, 3>(ctx, m, x, y); case 4: return gemv_t<FMT, 4>(ctx, m, x, y);
+    case 5: return gemv_t<FMT, 5>(ctx, m, x, y); case 6: return gemv_t<FMT, 6>(ctx, m, x, y); case 7: return gemv_t<FMT, 7>(ctx, m, x, y); case 8: return gemv_t<FMT, 8>(ctx, m, x, y); }
+  return pyre_fail(ctx, PYRE_E_ARG, "qmatmul: t = %d outside 1..8", t);
+}
+#define FMT_DISPATCH(fmt, CALL) \
+  switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; CALL; } break; case FMT_F16: { constexpr int F = FMT_F16; CALL; } break; case FMT_BF16: { constexpr int F = FMT_BF16; CALL; } break; \
+    case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
+    default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
+}  // namespace
+
+int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
+  int rc = PYRE_OK;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y));
+  return rc;
+}
+
+int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* idx, int n, float* out, int out_stride) {
+  if (n <= 0) return PYRE_OK;
+  dim3 grid((m.U + 63) / 64, n);
+  FMT_DISPATCH(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+
+static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, pyre_qmat** out) {
+  if (!ctx || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: null argument");
+  *out = nullptr;
+  int fmt = fmt_from_ggml(ty); if (fmt < 0) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmat_create: unsupported ggml type %u", ty);
+  FmtGeom g = fmt_geom(fmt);
+  if (rows == 0 || cols == 0 || cols % PYRE_UNIT != 0 || cols % g.el != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu: cols must be a non-zero multiple of 64 and of the block size %d", rows, cols, g.el);
+  if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
+  size_t row_bytes = cols / g.el * g.bytes;
+  if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
+  PYRE_HIP(ctx, hipSetDevice(ctx->device));
+  pyre_qmat* m = new pyre_qmat(); m->ctx = ctx; m->ty = ty; m->rows = rows; m->cols = cols; m->gguf_bytes = nbytes;
+  int U = (int)(cols / PYRE_UNIT), tiles = (int)((rows + 63) / 64);
+  size_t ent = (size_t)tiles * U * 64;
+  auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  size_t s0 = al(ent * g.V * 16), s1 = al(ent * g.e1), s2 = al(ent * g.e2), s3 = al(ent * g.e3), sb = al(ent / 4 * g.eb + 256);
+  m->dev_bytes = s0 + s1 + s2 + s3 + sb;
+  hipError_t e = hipMalloc(&m->base, m->dev_bytes);
+  if (e != hipSuccess) { delete m; return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", s0 + s1 + s2 + s3 + sb, hipGetErrorString(e)); }
+  uint8_t* b = (uint8_t*)m->base;
+  m->dv = QMatDev{b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (int)rows, (int)cols, U, tiles, fmt};
+  const uint8_t* src = (const uint8_t*)blocks; void* tmp = nullptr;
+  if (!on_device) {
+    e = hipMalloc(&tmp, nbytes);
+    if (e == hipSuccess) e = hipMemcpyAsync(tmp, blocks, nbytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); (void)hipFree(m->base); delete m; return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: upload failed: %s", hipGetErrorString(e)); }
+    src = (const uint8_t*)tmp;
+  }
+  size_t total = ent * 1; unsigned nblk = (unsigned)((total + 255) / 256);
+  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3);
+  e = hipGetLastError();
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (tmp) (void)hipFree(tmp);
+  if (e != hipSuccess) { (void)hipFree(m->base); delete m; return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: repack failed: %s", hipGetErrorString(e)); }
+  *out = m; return PYRE_OK;
+}
+
+extern "C" {
+
+int pyre_qmat_create(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* host_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, host_blocks, false, nbytes, out); }
+int pyre_qmat_create_dev(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* dev_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, dev_blocks, true, nbytes, out); }
+void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); (void)hipFree(m->base); delete m; }
+size_t pyre_qmat_rows(const pyre_qmat* m) { return m ? m->rows : 0; }
+size_t pyre_qmat_cols(const pyre_qmat* m) { return m ? m->cols : 0; }
+size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; }
+
+int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
+  if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");
+  dim3 grid(m->dv.U, m->dv.tiles);
+  FMT_DISPATCH(m->dv.fmt, hipLaunchKernelGGL((k_dequant<F>), grid, dim3(64), 0, ctx->stream, m->dv, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out_dev));
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+int pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host) {
+  if (!ctx || !m || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");
+  size_t n = m->rows * m->cols * sizeof(float); void* tmp = nullptr;
+  PYRE_HIP(ctx, hipMalloc(&tmp, n));
+  int rc = pyre_qmat_dequant_dev(ctx, m, (float*)tmp);
+  hipError_t e = hipSuccess;
+  if (!rc) { e = hipMemcpyAsync(out_host, tmp, n, hipMemcpyDeviceToHost, ctx->stream); if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream); }
+  (void)hipFree(tmp);
+  if (rc) return rc; if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_dequant: %s", hipGetErrorString(e));
+  return PYRE_OK;
+}
+int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host) {
+  if (!ctx || !m || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_row: null argument");
+  if (row >= m->rows) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_row: row %zu of %zu", row, m->rows);
+  void* st; int rc = pyre_stage(ctx, m->cols * sizeof(float) + 256, &st); if (rc) return rc;
+  uint32_t r = (uint32_t)row; uint32_t* idx = (uint32_t*)((uint8_t*)st + m->cols * sizeof(float));
+  PYRE_HIP(ctx, hipMemcpyAsync(idx, &r, 4, hipMemcpyHostToDevice, ctx->stream));
+  rc = pyre_row_launch(ctx, m->dv, idx, 1, (float*)st, (int)m->cols); if (rc) return rc;
+  PYRE_HIP(ctx, hipMemcpyAsync(out_host, st, m->cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+int pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
+  if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
+  return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
+}
+int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) {
+  if (!ctx || !m || !x_host || !y_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
+  size_t xb = (size_t)t * m->cols * sizeof(float), yb = (size_t)t * m->rows * sizeof(float), xo = (xb + 255) & ~(size_t)255;
+  void* st; int rc = pyre_stage(ctx, xo + yb, &st); if (rc) return rc;
+  float* xd = (float*)st; float* yd = (float*)((uint8_t*)st + xo);
+  PYRE_HIP(ctx, hipMemcpyAsync(xd, x_host, xb, hipMemcpyHostToDevice, ctx->stream));
+  rc = pyre_gemv_launch(ctx, m->dv, xd, t, yd); if (rc) return rc;
+  PYRE_HIP(ctx, hipMemcpyAsync(y_host, yd, yb, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+}  // extern "C"

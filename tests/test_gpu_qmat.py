@@ -1,0 +1,156 @@
+"""GPU parity of the quantized-matrix operator through the C ABI: dequant bit-exact with the oracle, GEMV within
+1e-5 of the f64-accumulated truth (max|dy| / max|y|, the reference's own normalisation, kquant.rs:203-206)."""
+import numpy as np
+import pytest
+
+import np_ref
+import orc
+from helpers import relerr
+from pyre_amd import lib, synth
+
+pytestmark = pytest.mark.gpu
+FMTS = [lib.Q8_0, lib.Q4_K, lib.IQ2_XS, lib.IQ3_S]
+ALL = FMTS + [lib.BF16, lib.F16, lib.F32]
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def raw_matrix(ty, rows, cols, seed):
+    if ty == lib.BF16:
+        return synth.bf16_normal(rows, cols, seed, 0.02)
+    if ty == lib.F16:
+        return synth.normal((rows, cols), seed, 0.05).astype(np.float16).view(np.uint8).reshape(-1)
+    if ty == lib.F32:
+        return synth.normal((rows, cols), seed, 0.05).view(np.uint8).reshape(-1)
+    return synth.matrix(ty, rows, cols, seed)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("ty", ALL)
+@pytest.mark.parametrize("rows,cols", [(64, 256), (100, 512), (513, 2048)])
+def test_dequant_bit_exact(ctx, ty, rows, cols):
+    raw = raw_matrix(ty, rows, cols, 11 + ty)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
+    got = m.to_f32()
+    exp = orc.dequant(ty, raw, rows * cols).reshape(rows, cols)
+    assert np.array_equal(bits(got), bits(exp))
+    for r in (0, rows // 2, rows - 1):
+        assert np.array_equal(bits(m.row(r)), bits(exp[r]))
+    assert m.gguf_bytes == raw.nbytes
+
+
+@pytest.mark.parametrize("ty", FMTS)
+def test_dequant_bit_exact_on_arbitrary_bytes_and_known_answers(ctx, ty):
+    el, bs, _ = synth.GEOM[ty]
+    rows, cols = 96, 512
+    raw = np.random.Generator(np.random.PCG64(99 + ty)).integers(0, 256, rows * cols // el * bs, dtype=np.uint8)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
+    with np.errstate(all="ignore"):
+        got = m.to_f32(); exp = orc.dequant(ty, raw, rows * cols).reshape(rows, cols)
+    ok = (bits(got) == bits(exp)) | (np.isnan(got) & np.isnan(exp))
+    assert ok.all()
+
+
+def test_known_answer_blocks_on_device(ctx):
+    z = np_ref.pack_iq3s(1.0, np.zeros(64, np.uint8), np.zeros(8, np.uint8), np.zeros(32, np.uint8), np.zeros(4, np.uint8))
+    m = lib.QMat(ctx, lib.IQ3_S, 1, 256, z)
+    assert np.array_equal(m.to_f32(), np.ones((1, 256), np.float32))
+    z2 = np_ref.pack_iq2xs(2.0, np.zeros(32, np.uint16), np.zeros(8, np.uint8))
+    assert np.array_equal(lib.QMat(ctx, lib.IQ2_XS, 1, 256, z2).to_f32(), np.full((1, 256), 2.0, np.float32))
+
+
+@pytest.mark.parametrize("ty", ALL)
+@pytest.mark.parametrize("t", [1, 2, 3, 4, 5, 8])
+def test_gemv_matches_truth_and_oracle(ctx, ty, t):
+    rows, cols = 320, 2048
+    raw = raw_matrix(ty, rows, cols, 21 + ty)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
+    x = synth.normal((t, cols), 31 + t)
+    y = m.matmul(x)
+    W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    truth = x.astype(np.float64) @ W.T
+    assert relerr(y, truth) <= TOL
+    assert relerr(orc.matmul(ty, raw, rows, cols, x), truth) <= TOL
+
+
+# the shapes of the benchmark sweep: rows <- cols
+SHAPES = [(4096, 2048), (2048, 4096), (512, 2048), (2048, 512)]
+
+
+@pytest.mark.parametrize("ty", FMTS)
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_gemv_sweep_shapes(ctx, ty, rows, cols):
+    raw = synth.matrix(ty, rows, cols, 41 + ty)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
+    W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    for t in (1, 4, 8):
+        x = synth.normal((t, cols), 51 + t)
+        assert relerr(m.matmul(x), x.astype(np.float64) @ W.T) <= TOL, t
+
+
+@pytest.mark.parametrize("ty", FMTS)
+def test_result_for_a_token_does_not_depend_on_batch_width(ctx, ty):
+    rows, cols = 1024, 2048
+    m = lib.QMat(ctx, ty, rows, cols, synth.matrix(ty, rows, cols, 61 + ty))
+    x = synth.normal((8, cols), 71)
+    y8 = m.matmul(x)
+    for t in (1, 2, 4):
+        yt = m.matmul(x[:t])
+        assert np.array_equal(bits(yt), bits(y8[:t])), t
+    assert np.array_equal(bits(m.matmul(x[3:4])), bits(y8[3:4]))
+    # and it is reproducible run to run (split-K partials are added in a fixed order)
+    assert np.array_equal(bits(m.matmul(x)), bits(y8))
+
+
+def test_linearity_and_zero_input(ctx):
+    rows, cols = 2048, 2048
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, synth.matrix(lib.IQ3_S, rows, cols, 81))
+    a = synth.normal((1, cols), 82); b = synth.normal((1, cols), 83)
+    ya, yb, yab = m.matmul(a), m.matmul(b), m.matmul(2 * a - b)
+    assert relerr(yab, 2 * ya.astype(np.float64) - yb) <= 1e-5
+    assert not m.matmul(np.zeros((1, cols), np.float32)).any()
+
+
+def test_vocab_head_shape_against_sampled_rows(ctx):
+    rows, cols = 151936, 2048
+    ty = lib.IQ3_S
+    el, bs, _ = synth.GEOM[ty]
+    nb = rows * cols // el
+    dev = ctx.alloc(nb * bs)
+    ctx.synth_blocks(ty, nb, 4242, dev_out=dev)
+    m = lib.QMat(ctx, ty, rows, cols, dev_blocks=dev, nbytes=nb * bs)
+    ctx.free(dev)
+    raw = synth.matrix(ty, rows, cols, 4242)
+    x = synth.normal((2, cols), 91)
+    y = m.matmul(x)
+    sel = np.r_[0:64, 75000:75064, rows - 64:rows]
+    rb = cols // el * bs
+    Wsel = np.stack([orc.dequant(ty, raw[r * rb:(r + 1) * rb], cols) for r in sel]).astype(np.float64)
+    truth = x.astype(np.float64) @ Wsel.T
+    assert np.abs(y[:, sel] - truth).max() / np.abs(truth).max() <= TOL
+    # device generator == host generator, through the bit-exact dequant of a few rows
+    for r in (0, 12345, rows - 1):
+        assert np.array_equal(bits(m.row(r)), bits(orc.dequant(ty, raw[r * rb:(r + 1) * rb], cols)))
+
+
+def test_argument_errors_are_reported(ctx):
+    with pytest.raises(lib.PyreError):
+        lib.QMat(ctx, 99, 64, 256, np.zeros(16, np.uint8))               # unknown type
+    with pytest.raises(lib.PyreError):
+        lib.QMat(ctx, lib.IQ3_S, 64, 200, np.zeros(16, np.uint8))        # cols not a block multiple
+    with pytest.raises(lib.PyreError):
+        lib.QMat(ctx, lib.IQ3_S, 64, 256, np.zeros(16, np.uint8))        # wrong byte count
+    m = lib.QMat(ctx, lib.Q8_0, 64, 256, synth.matrix(lib.Q8_0, 64, 256, 1))
+    with pytest.raises(lib.PyreError):
+        m.matmul(np.zeros((9, 256), np.float32))                         # t outside 1..8
+    with pytest.raises(lib.PyreError):
+        m.row(64)
