@@ -73,6 +73,116 @@ int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, i
  * uniformly from [d_lo, d_hi].  Bit-identical to pyre_amd/synth.py:blocks(). */
 int    pyre_synth_blocks(pyre_ctx* ctx, uint32_t ggml_type, size_t n_blocks, uint64_t seed, float d_lo, float d_hi, void* dev_out);
 
+
+/* ---- MoE FFN block ---------------------------------------------------------------------------------------------
+ * ffn + routed, f32 branch (src/model/qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793) with the router of
+ * top_k / soft_top / nan_clean (:3121-3139): softmax over the top-k logits, ties to the lower expert id, the chosen
+ * experts listed and summed in ascending id (the order the reference's device router uses, qn_cube.rs:5225-5237).
+ * Expert tensors are the fused GGUF matrices: gate/up [n_exp*ff x d], down [n_exp*d x ff], expert e = rows e*ff.. /
+ * e*d.. (QMat::slice_rows, gguf_q.rs:215).  The qmats are borrowed and must outlive the block. */
+typedef struct pyre_moe pyre_moe;
+int  pyre_moe_create(pyre_ctx* ctx, int top_k, const pyre_qmat* router, const pyre_qmat* gate_exps, const pyre_qmat* up_exps, const pyre_qmat* down_exps,
+                     const float* sh_gate_inp_host /*[d]*/, const pyre_qmat* sh_gate, const pyre_qmat* sh_up, const pyre_qmat* sh_down, pyre_moe** out);
+void pyre_moe_destroy(pyre_moe* m);
+/* x [t][d] -> y [t][d], t in 1..8; sel_idx / sel_w (optional) receive the routing [t][top_k]. */
+int  pyre_moe_ffn(pyre_ctx* ctx, pyre_moe* m, const float* x_host, int t, float* y_host, int32_t* sel_idx_host, float* sel_w_host);
+int  pyre_moe_ffn_dev(pyre_ctx* ctx, pyre_moe* m, const float* x_dev, int t, float* y_dev);
+
+/* ---- Gated DeltaNet layer core ---------------------------------------------------------------------------------
+ * linear_core (qwen4exp_gguf.rs:1624-1673): causal depthwise conv (kernel conv_k, weight [ch][conv_k], newest tap
+ * last) + SiLU, L2-normalised q/k, per value head h (key head h % nk) the gated delta rule on the f32 state
+ * S [nv][dk][dv], gated RMSNorm.  The block owns its recurrent state (conv [(conv_k-1)][ch] oldest first, S), which
+ * stays resident in HBM across calls; a, dt [nv], conv_w [ch*conv_k], norm_w [dv] are host f32. dk = dv = 128. */
+typedef struct pyre_gdn pyre_gdn;
+int  pyre_gdn_create(pyre_ctx* ctx, int nk, int nv, int dk, int dv, int conv_k, float eps, const float* a, const float* dt, const float* conv_w, const float* norm_w, pyre_gdn** out);
+void pyre_gdn_destroy(pyre_gdn* g);
+int  pyre_gdn_set_state(pyre_ctx* ctx, pyre_gdn* g, const float* conv_host /*NULL = zeros*/, const float* ssm_host /*NULL = zeros*/);
+int  pyre_gdn_get_state(pyre_ctx* ctx, pyre_gdn* g, float* conv_host, float* ssm_host);
+/* proj [t][ch + nv*dv + 2*nv] = per token [qkv | z | beta | alpha] -> out [t][nv*dv]; tokens run in time order. */
+int  pyre_gdn_step(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int t, float* out_host);
+
+/* ---- gated attention layer core over a 4-bit KV cache --------------------------------------------------------------
+ * attn_core, dense branch (qwen4exp_gguf.rs:1558-1615): k RMSNorm + RoPE, append; per head q RMSNorm + RoPE,
+ * softmax(q.K/sqrt(hd)) V, * sigmoid(gate); q and gate interleaved per head [h][2*hd]; kv head = h / (nh/nkv);
+ * partial RoPE over the first n_rot dims, pairs (i, i + n_rot/2), inv[i] = base^(-2i/n_rot) (src/qn_ctx.rs:168).
+ * Cache positions below ((n - kv_recent)/64)*64 (n = positions visible to the query, only when n > kv_recent + 64)
+ * are read from the 4-bit cache of src/model/kv4.rs:12-42; the rest from f32 (split of kv_push, :1519-1520).
+ * kv_bits = 0 keeps everything f32.  hd = 256. */
+typedef struct pyre_attn pyre_attn;
+int  pyre_attn_create(pyre_ctx* ctx, int nh, int nkv, int hd, int n_rot, float rope_base, float eps, const float* qn /*[hd]*/, const float* kn /*[hd]*/,
+                      int kv_bits, int kv_recent, int max_ctx, pyre_attn** out);
+void pyre_attn_destroy(pyre_attn* a);
+int  pyre_attn_len(const pyre_attn* a);
+int  pyre_attn_truncate(pyre_ctx* ctx, pyre_attn* a, int len);
+/* qkv [t][nh*2*hd + 2*nkv*hd] raw projections [q,gate per head | k | v] for the next t positions -> out [t][nh*hd]. */
+int  pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, int t, float* out_host);
+/* Harness access: install n positions of (already normalised + rotated) keys and values [n][nkv*hd]; read them back. */
+int  pyre_attn_load_cache(pyre_ctx* ctx, pyre_attn* a, const float* k_host, const float* v_host, int n);
+int  pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_host);
+
+/* ---- model: the layer API engine_qn drives ------------------------------------------------------------------------
+ * Model::{load, new_state, forward, forward_multi, spec_keep} (qwen4exp_gguf.rs:462, 1345, 2050, 2365, 2495) as
+ * consumed through QnTarget: spec::Target (src/engine_qn.rs:245-253). */
+typedef struct {
+  uint32_t ggml_type;   /* PYRE_* */
+  uint32_t on_device;   /* 0: data is host memory, 1: data is device memory on the context's device */
+  uint64_t rows, cols;  /* Gguf::mat view: rows = prod(shape[1..]), cols = shape[0]; vectors have rows = 1 */
+  const void* data;     /* raw GGUF bytes; NULL for a slot the layer does not have */
+} pyre_tensor;
+
+/* per-layer tensor slots, named after the GGUF tensors Model::load reads (qwen4exp_gguf.rs:489-512) */
+enum {
+  PYRE_T_HC_ATTN_NORM = 0, PYRE_T_HC_ATTN_DOWN, PYRE_T_HC_ATTN_INJECT, PYRE_T_HC_ATTN_UP,     /* blk.N.hc_attn_{norm,down,inject,up}.weight */
+  PYRE_T_HC_FFN_NORM, PYRE_T_HC_FFN_DOWN, PYRE_T_HC_FFN_INJECT, PYRE_T_HC_FFN_UP,             /* blk.N.hc_ffn_* */
+  PYRE_T_ATTN_Q, PYRE_T_ATTN_K, PYRE_T_ATTN_V, PYRE_T_ATTN_OUTPUT, PYRE_T_ATTN_Q_NORM, PYRE_T_ATTN_K_NORM,
+  PYRE_T_ATTN_QKV, PYRE_T_ATTN_GATE, PYRE_T_SSM_BETA, PYRE_T_SSM_ALPHA, PYRE_T_SSM_A, PYRE_T_SSM_DT_BIAS, PYRE_T_SSM_CONV1D, PYRE_T_SSM_NORM, PYRE_T_SSM_OUT,
+  PYRE_T_FFN_GATE_INP, PYRE_T_FFN_GATE_EXPS, PYRE_T_FFN_UP_EXPS, PYRE_T_FFN_DOWN_EXPS, PYRE_T_FFN_GATE_INP_SHEXP, PYRE_T_FFN_GATE_SHEXP, PYRE_T_FFN_UP_SHEXP, PYRE_T_FFN_DOWN_SHEXP,
+  PYRE_LAYER_SLOTS
+};
+enum { PYRE_G_TOKEN_EMBD = 0, PYRE_G_OUTPUT_HC_NORM, PYRE_G_OUTPUT_HC_DOWN, PYRE_G_OUTPUT_HC_UP, PYRE_G_OUTPUT, PYRE_GLOBAL_SLOTS };
+
+/* Cfg (qwen4exp_gguf.rs:18-26), the fields the decode loop uses. */
+typedef struct {
+  int32_t n_layers, d, hc, hc_lr, n_head, n_kv, hd, n_rot;
+  float rope_base, eps;
+  int32_t n_exp, top_k, ff_exp;
+  int32_t lin_nk, lin_nv, lin_dk, lin_dv, conv_k, full_every;
+  int32_t vocab;
+  int32_t kv_bits;    /* 4 (PYRE_QN_KV_BITS default) or 0 */
+  int32_t kv_recent;  /* PYRE_QN_KV8_RECENT default 1024 */
+} pyre_model_cfg;
+
+/* Copies (and re-lays-out) every tensor into device memory; the caller's buffers are free afterwards. */
+int   pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* layer_tensors /*[n_layers][PYRE_LAYER_SLOTS]*/,
+                        const pyre_tensor* globals /*[PYRE_GLOBAL_SLOTS]*/, pyre_model** out);
+void  pyre_model_destroy(pyre_model* m);
+/* GGUF bytes of the weights one decode step reads (dense matrices, router, top_k + 1 experts, head, one embedding row). */
+size_t pyre_model_weight_bytes_per_token(const pyre_model* m);
+/* new_state: empty token list, zero recurrent state, KV room for max_ctx positions. */
+int   pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_state** out);
+void  pyre_state_destroy(pyre_state* s);
+int   pyre_state_reset(pyre_ctx* ctx, pyre_state* s);
+int   pyre_state_len(const pyre_state* s);
+/* Test access to the recurrent state: li-th DeltaNet layer's S [nv][dk][dv] and conv [(k-1)][ch]; ai-th attention layer's f32 K / V rows [len][nkv*hd]. */
+int   pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, float* ssm_host);
+int   pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, float* v_host);
+/* forward: append n tokens (any n >= 1; processed in windows of up to 8), logits of the last one -> logits_host[vocab]. */
+int   pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host);
+/* forward_multi: n in 1..8 tokens, logits after each -> logits_host [n][vocab]; arms spec_keep for this window. */
+int   pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host);
+/* spec_keep(t, keep): keep the first `keep` of the last t tokens fed by forward_multi (recurrent state rolled back, caches truncated). */
+int   pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int keep);
+/* spec::generate, greedy branch (src/spec.rs:156-267, accept loop :229-238; argmax = first maximum, src/sampler.rs:142-148).
+ * first_logits_host: logits after the prompt.  n_draft = 0: plain decode, the whole loop runs on the device without
+ * host round trips.  n_draft in 1..7 with draft_stream [n_out + 8]: the round that starts with `produced` tokens
+ * emitted verifies draft_stream[produced .. produced + n_draft) and keeps the accepted prefix.
+ * out [n_out] tokens; *rounds (optional) = verify rounds used. */
+int   pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
+                           int n_draft, const uint32_t* draft_stream, int* rounds);
+/* The decode loop as the benchmark times it: n_steps greedy steps starting from token `first`, everything on the device;
+ * tokens (optional, host) receives the n_steps generated ids after the call. */
+int   pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host);
+
 #ifdef __cplusplus
 }
 #endif

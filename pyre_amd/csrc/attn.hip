@@ -1,0 +1,320 @@
+// Gated full attention at decode: q/k RMSNorm + partial RoPE + KV append, softmax(q K^T / sqrt(hd)) V * sigmoid(gate)
+// over a cache whose old positions are 4-bit (absmax per 32, kv4) and whose recent window is f32.
+// Follows attn_core (dense branch), src/model/qwen4exp_gguf.rs:1558-1615, rope :1436-1439 / :529-533,
+// kv4::pack / get, src/model/kv4.rs:12-42, and the packed/recent split of kv_push, qwen4exp_gguf.rs:1519-1520.
+#include "formats.h"
+
+__device__ __forceinline__ float a_sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+size_t pyre_packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 4 || n <= (size_t)recent + 64) return 0; return ((n - recent) / 64) * 64; }
+
+// grid (nkv + nh, t), hd threads.  Blocks 0..nkv-1: key head -> rms_inplace(kn) -> rope -> cache (and the raw value row);
+// blocks nkv..: query head h -> rms_inplace(qn) -> rope -> q scratch.
+template <int HD>
+__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, float* __restrict__ qout) {
+  __shared__ float buf[HD]; __shared__ float red[HD / 64];
+  const int b = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, pos = start + ti;
+  const bool is_k = b < a.nkv; const int h = is_k ? b : b - a.nkv;
+  const float* row = qkv + (size_t)ti * stride;
+  const float* src = is_k ? row + (size_t)a.nh * 2 * HD + (size_t)h * HD : row + (size_t)h * 2 * HD;
+  float v = src[tid];
+  float ss = v * v;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  float tot = 0.0f;
+#pragma unroll
+  for (int i = 0; i < HD / 64; ++i) tot += red[i];
+  const float sc = 1.0f / sqrtf(tot / (float)HD + a.eps);
+  v = v * (sc * (is_k ? a.kn[tid] : a.qn[tid]));            // rms_inplace: x *= s * w
+  buf[tid] = v;
+  __syncthreads();
+  const int half = a.n_rot / 2;
+  if (tid < a.n_rot) {
+    int i = tid < half ? tid : tid - half;
+    float ang = (float)pos * a.rope_inv[i];
+    float sn = sinf(ang), cs = cosf(ang);
+    float x0 = buf[i], x1 = buf[i + half];
+    v = tid < half ? x0 * cs - x1 * sn : x1 * cs + x0 * sn;
+  }
+  if (is_k) {
+    kv.kf[((size_t)h * HD + tid) * kv.cap + pos] = v;
+    kv.vf[(size_t)pos * a.nkv * HD + (size_t)h * HD + tid] = row[(size_t)a.nh * 2 * HD + (size_t)a.nkv * HD + (size_t)h * HD + tid];
+  } else qout[((size_t)ti * a.nh + h) * HD + tid] = v;
+}
+
+// kv4::pack for positions [p0, p1): one thread per (position, 32-value block, K or V).
+template <int HD>
+__global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1) {
+  const int bpr = a.nkv * HD / 32;                 // blocks per cache row
+  size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t per = (size_t)(p1 - p0) * bpr;
+  if (gid >= 2 * per) return;
+  const bool is_v = gid >= per; if (is_v) gid -= per;
+  const int pos = p0 + (int)(gid / bpr), blk = (int)(gid % bpr), kvh = blk / (HD / 32), bb = blk % (HD / 32);
+  float x[32];
+  for (int i = 0; i < 32; ++i) x[i] = is_v ? kv.vf[(size_t)pos * a.nkv * HD + (size_t)blk * 32 + i] : kv.kf[((size_t)kvh * HD + bb * 32 + i) * kv.cap + pos];
+  float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(x[i]));
+  const float s = (m > 0.0f && isfinite(m)) ? m / 7.0f : 0.0f;
+  for (int w = 0; w < 4; ++w) {
+    uint32_t u = 0;
+    for (int j = 0; j < 8; ++j) { int q = s > 0.0f ? (int)fminf(fmaxf(roundf(x[8 * w + j] / s), -7.0f), 7.0f) : 0; u |= ((uint32_t)q & 0xFu) << (4 * j); }
+    if (is_v) kv.vq[(size_t)pos * (a.nkv * HD / 8) + (size_t)blk * 4 + w] = u;
+    else kv.kq[((size_t)kvh * (HD / 8) + bb * 4 + w) * kv.cap + pos] = u;
+  }
+  if (is_v) kv.vs[(size_t)pos * bpr + blk] = s; else kv.ks[((size_t)kvh * (HD / 32) + bb) * kv.cap + pos] = s;
+}
+
+__device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((int)(w << (28 - 4 * i))) >> 28); }   // sign-extended nibble i
+
+// grid (chunks of 256 positions, nkv, t), 256 threads.  One workgroup serves the G query heads that share a KV head.
+//  phase 1: lane = position, scores for the G heads (cache read once per group, coalesced along positions)
+//  phase 2: chunk-local max / exp / sum per head
+//  phase 3: lane = value dims, unnormalised sum_p e_p V[p]; waves and half-waves are added in a fixed order
+template <int HD, int G>
+__global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+  __shared__ float qs[G][HD];
+  __shared__ float sc[256][G];
+  __shared__ float part[4][G][HD];
+  __shared__ float wred[4][G], cm[G];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = start + ti + 1;
+  if (chunk * 256 >= n) return;
+  const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
+  const size_t cap = kv.cap;
+  for (int i = tid; i < G * HD; i += 256) qs[i / HD][i % HD] = qbuf[((size_t)ti * a.nh + (size_t)kvh * G + i / HD) * HD + i % HD];
+  __syncthreads();
+  const int wbase = chunk * 256 + wave * 64, p = wbase + lane;
+  const bool valid = p < n, packed = wbase < pb;
+  const float scale = 1.0f / sqrtf((float)HD);
+  float s[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) s[g] = 0.0f;
+  if (wbase < n) {
+    const int pp = valid ? p : n - 1;
+    if (packed) {
+      for (int b = 0; b < HD / 32; ++b) {
+        float bp[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) bp[g] = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          uint32_t u = kv.kq[((size_t)kvh * (HD / 8) + b * 4 + w) * cap + pp];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) { float kvl = nib_val(u, i);
+#pragma unroll
+            for (int g = 0; g < G; ++g) bp[g] = fmaf(kvl, qs[g][b * 32 + w * 8 + i], bp[g]); }
+        }
+        float ksc = kv.ks[((size_t)kvh * (HD / 32) + b) * cap + pp];
+#pragma unroll
+        for (int g = 0; g < G; ++g) s[g] = fmaf(ksc, bp[g], s[g]);
+      }
+    } else {
+      for (int dd = 0; dd < HD; ++dd) { float kvl = kv.kf[((size_t)kvh * HD + dd) * cap + pp];
+#pragma unroll
+        for (int g = 0; g < G; ++g) s[g] = fmaf(kvl, qs[g][dd], s[g]); }
+    }
+  }
+  // phase 2
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    s[g] = valid ? s[g] * scale : -INFINITY;
+    float m = s[g];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (lane == 0) wred[wave][g] = m;
+  }
+  __syncthreads();
+  if (tid < G) cm[tid] = fmaxf(fmaxf(wred[0][tid], wred[1][tid]), fmaxf(wred[2][tid], wred[3][tid]));
+  __syncthreads();
+  float e[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) { e[g] = valid ? expf(s[g] - cm[g]) : 0.0f; sc[tid][g] = e[g]; }
+  __syncthreads();   // all maxima read, scores of every wave visible
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float l = e[g];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    if (lane == 0) wred[wave][g] = l;
+  }
+  // phase 3
+  const int row = a.nkv * HD;
+  if (packed) {
+    float acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+    const int w32 = lane & 31, hf = lane >> 5;
+    if (wbase < n) for (int it = 0; it < 32; ++it) {
+      int pl = 2 * it + hf, pg = wbase + pl; if (pg >= n) continue;
+      uint32_t u = kv.vq[(size_t)pg * (row / 8) + (size_t)kvh * (HD / 8) + w32];
+      float vsc = kv.vs[(size_t)pg * (row / 32) + (size_t)kvh * (HD / 32) + (w32 >> 2)];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { float vv = nib_val(u, i) * vsc;
+#pragma unroll
+        for (int g = 0; g < G; ++g) acc[g][i] = fmaf(sc[wave * 64 + pl][g], vv, acc[g][i]); }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { float o = acc[g][i] + __shfl_xor(acc[g][i], 32); if (hf == 0) part[wave][g][w32 * 8 + i] = o; }
+  } else {
+    float acc[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[g][i] = 0.0f;
+    if (wbase < n) for (int pl = 0; pl < 64; ++pl) {
+      int pg = wbase + pl; if (pg >= n) break;
+      float4 vv = *(const float4*)(kv.vf + (size_t)pg * row + (size_t)kvh * HD + 4 * lane);
+#pragma unroll
+      for (int g = 0; g < G; ++g) { float wgt = sc[wave * 64 + pl][g]; acc[g][0] = fmaf(wgt, vv.x, acc[g][0]); acc[g][1] = fmaf(wgt, vv.y, acc[g][1]); acc[g][2] = fmaf(wgt, vv.z, acc[g][2]); acc[g][3] = fmaf(wgt, vv.w, acc[g][3]); }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave][g][4 * lane + i] = acc[g][i];
+  }
+  __syncthreads();
+  for (int i = tid; i < G * HD; i += 256) {
+    int g = i / HD, dd = i % HD;
+    float o = ((part[0][g][dd] + part[1][g][dd]) + part[2][g][dd]) + part[3][g][dd];
+    part_o[(((size_t)ti * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
+  }
+  if (tid < G) {
+    float l = ((wred[0][tid] + wred[1][tid]) + wred[2][tid]) + wred[3][tid];
+    float* ml = part_ml + (((size_t)ti * a.nh + (size_t)kvh * G + tid) * max_chunks + chunk) * 2;
+    ml[0] = cm[tid]; ml[1] = l;
+  }
+}
+
+// grid (nh, t), HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
+template <int HD>
+__global__ __launch_bounds__(HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                     int max_chunks, float* __restrict__ out) {
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, n = start + ti + 1, nc = (n + 255) / 256;
+  const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
+  const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
+  float M = -INFINITY; for (int c = 0; c < nc; ++c) M = fmaxf(M, ml[2 * c]);
+  float L = 0.0f, o = 0.0f;
+  for (int c = 0; c < nc; ++c) { float f = expf(ml[2 * c] - M); L = fmaf(ml[2 * c + 1], f, L); o = fmaf(po[(size_t)c * HD + tid], f, o); }
+  float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + tid];
+  out[((size_t)ti * a.nh + h) * HD + tid] = (o / L) * a_sigm(gate);
+}
+
+size_t pyre_kv_bytes(const AttnDev& a, int cap) {
+  size_t row = (size_t)a.nkv * a.hd, c = cap;
+  return 6 * 256 + c * row * 4 * 2 + c * row / 8 * 4 * 2 + c * row / 32 * 4 * 2;
+}
+void pyre_kv_carve(const AttnDev& a, int cap, void* base, KvDev* kv) {
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
+  size_t row = (size_t)a.nkv * a.hd, c = cap;
+  kv->kf = (float*)take(c * row * 4); kv->vf = (float*)take(c * row * 4); kv->kq = (uint32_t*)take(c * row / 8 * 4); kv->ks = (float*)take(c * row / 32 * 4);
+  kv->vq = (uint32_t*)take(c * row / 8 * 4); kv->vs = (float*)take(c * row / 32 * 4); kv->cap = cap;
+}
+size_t pyre_attn_work_bytes(const AttnDev& a, int cap) {
+  size_t mc = ((size_t)cap + 255) / 256;
+  return 3 * 256 + 4 * (8 * (size_t)a.nh * a.hd + 8 * (size_t)a.nh * mc * a.hd + 8 * (size_t)a.nh * mc * 2);
+}
+void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
+  size_t mc = ((size_t)cap + 255) / 256;
+  w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
+}
+
+template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t) {
+  int n = start + t, chunks = (n + 255) / 256;
+  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256), 0, ctx->stream, a, kv, w.q, start, w.part_o, w.part_ml, w.max_chunks);
+}
+
+int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out) {
+  if (a.hd != 256) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: head dim %d unsupported (256 only)", a.hd);
+  if (a.nkv < 1 || a.nh % a.nkv) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: %d query heads over %d kv heads", a.nh, a.nkv);
+  int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
+  if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
+  if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
+  hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, w.q); PYRE_CHECK_LAUNCH(ctx);
+  // pack the positions that fall below the boundary of the longest view of this call
+  int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
+  if (pbn > *packed_done) {
+    size_t thr = (size_t)(pbn - *packed_done) * (a.nkv * a.hd / 32) * 2;
+    hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn); PYRE_CHECK_LAUNCH(ctx);
+    *packed_done = pbn;
+  }
+  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t); break; default: launch_decode<8>(ctx, a, kv, w, start, t); }
+  PYRE_CHECK_LAUNCH(ctx);
+  hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, w.part_o, w.part_ml, w.max_chunks, out); PYRE_CHECK_LAUNCH(ctx);
+  return PYRE_OK;
+}
+
+// ---- C ABI: standalone attention layer core for the block harness -----------------------------------------------------
+struct pyre_attn { pyre_ctx* ctx; AttnDev dv; KvDev kv; AttnWork w; float* params; void* kvmem; void* wmem; float* io; int len, packed, cap; };
+
+extern "C" {
+
+int pyre_attn_create(pyre_ctx* ctx, int nh, int nkv, int hd, int n_rot, float rope_base, float eps, const float* qn, const float* kn, int kv_bits, int kv_recent, int max_ctx, pyre_attn** out) {
+  if (!ctx || !out || !qn || !kn) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_create: null argument");
+  *out = nullptr;
+  if (hd != 256 || nkv < 1 || nh % nkv || n_rot > hd || (n_rot & 1) || max_ctx < 1 || (kv_bits != 0 && kv_bits != 4) || kv_recent < 64) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_attn_create: unsupported geometry");
+  pyre_attn* a = new pyre_attn(); a->ctx = ctx; a->len = 0; a->packed = 0; a->cap = (max_ctx + 255) / 256 * 256;
+  std::vector<float> hp(2 * (size_t)hd + n_rot / 2); memcpy(hp.data(), qn, 4 * hd); memcpy(hp.data() + hd, kn, 4 * hd);
+  for (int i = 0; i < n_rot / 2; ++i) hp[2 * hd + i] = powf(rope_base, -(2.0f * (float)i) / (float)n_rot);    // rope_inv, src/qn_ctx.rs:168
+  a->dv = AttnDev{nullptr, nullptr, nullptr, nh, nkv, hd, n_rot, kv_bits, kv_recent, eps};
+  size_t qw = (size_t)nh * 2 * hd + 2 * (size_t)nkv * hd;
+  hipError_t e = hipMalloc((void**)&a->params, hp.size() * 4);
+  if (e == hipSuccess) e = hipMemcpy(a->params, hp.data(), hp.size() * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMalloc(&a->kvmem, pyre_kv_bytes(a->dv, a->cap));
+  if (e == hipSuccess) e = hipMalloc(&a->wmem, pyre_attn_work_bytes(a->dv, a->cap));
+  if (e == hipSuccess) e = hipMalloc((void**)&a->io, 8 * (qw + (size_t)nh * hd) * 4);
+  if (e != hipSuccess) { int rc = pyre_fail(ctx, PYRE_E_HIP, "pyre_attn_create: %s", hipGetErrorString(e)); delete a; return rc; }
+  a->dv.qn = a->params; a->dv.kn = a->params + hd; a->dv.rope_inv = a->params + 2 * hd;
+  pyre_kv_carve(a->dv, a->cap, a->kvmem, &a->kv); pyre_attn_work_carve(a->dv, a->cap, a->wmem, &a->w);
+  *out = a; return PYRE_OK;
+}
+void pyre_attn_destroy(pyre_attn* a) { if (!a) return; (void)hipStreamSynchronize(a->ctx->stream); (void)hipFree(a->params); (void)hipFree(a->kvmem); (void)hipFree(a->wmem); (void)hipFree(a->io); delete a; }
+int pyre_attn_len(const pyre_attn* a) { return a ? a->len : 0; }
+int pyre_attn_truncate(pyre_ctx* ctx, pyre_attn* a, int len) { if (!a || len < 0 || len > a->len) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_truncate: bad length"); a->len = len; return PYRE_OK; }
+
+// Decode / verify step of one attention layer over its own cache: qkv [t][nh*2*hd + 2*nkv*hd] raw projections for the
+// next t positions -> out [t][nh*hd]; the positions are appended to the cache.
+int pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, int t, float* out_host) {
+  if (!ctx || !a || !qkv_host || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_decode_kv4: null argument");
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_decode_kv4: t = %d outside 1..8", t);
+  size_t qw = (size_t)a->dv.nh * 2 * a->dv.hd + 2 * (size_t)a->dv.nkv * a->dv.hd, ow = (size_t)a->dv.nh * a->dv.hd;
+  float* qd = a->io; float* od = a->io + 8 * qw;
+  PYRE_HIP(ctx, hipMemcpyAsync(qd, qkv_host, (size_t)t * qw * 4, hipMemcpyHostToDevice, ctx->stream));
+  int rc = pyre_attn_launch(ctx, a->dv, a->kv, a->w, qd, (int)qw, a->len, t, &a->packed, od); if (rc) return rc;
+  a->len += t;
+  PYRE_HIP(ctx, hipMemcpyAsync(out_host, od, (size_t)t * ow * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+// Test / harness access: load n positions of already-normalised keys and values (row-major [n][nkv*hd]) as the cache
+// content, and read the f32 rows back.
+int pyre_attn_load_cache(pyre_ctx* ctx, pyre_attn* a, const float* k_host, const float* v_host, int n) {
+  if (!ctx || !a || !k_host || !v_host || n < 0 || n > a->cap) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_load_cache: bad argument");
+  size_t row = (size_t)a->dv.nkv * a->dv.hd; std::vector<float> kt(row * a->cap, 0.0f);
+  for (int p = 0; p < n; ++p) for (size_t c = 0; c < row; ++c) kt[c * a->cap + p] = k_host[(size_t)p * row + c];
+  PYRE_HIP(ctx, hipMemcpyAsync(a->kv.kf, kt.data(), kt.size() * 4, hipMemcpyHostToDevice, ctx->stream));
+  PYRE_HIP(ctx, hipMemcpyAsync(a->kv.vf, v_host, (size_t)n * row * 4, hipMemcpyHostToDevice, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  a->len = n; a->packed = 0;
+  int pbn = (int)pyre_packed_boundary((size_t)n, a->dv.kv_bits, a->dv.kv_recent);
+  if (pbn > 0) { size_t thr = (size_t)pbn * (row / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a->dv, a->kv, 0, pbn); PYRE_CHECK_LAUNCH(ctx); a->packed = pbn; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+  return PYRE_OK;
+}
+int pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_host) {
+  if (!ctx || !a || !k_host || !v_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_read_cache: null argument");
+  size_t row = (size_t)a->dv.nkv * a->dv.hd; std::vector<float> kt(row * a->cap);
+  PYRE_HIP(ctx, hipMemcpyAsync(kt.data(), a->kv.kf, kt.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipMemcpyAsync(v_host, a->kv.vf, (size_t)a->len * row * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  for (int p = 0; p < a->len; ++p) for (size_t c = 0; c < row; ++c) k_host[(size_t)p * row + c] = kt[c * a->cap + p];
+  return PYRE_OK;
+}
+// kv4 pack / unpack of a flat f32 array through the device kernels' arithmetic is covered by load_cache + decode; this
+// export packs n values (multiple of 32) exactly like kv4::pack and returns words and scales.
+}  // extern "C"

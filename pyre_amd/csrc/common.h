@@ -54,3 +54,62 @@ struct pyre_qmat {
 // launchers implemented in qmat.hip, used by the block / model code
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev, int n, float* out_dev, int out_stride);
+
+// ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
+struct MoeDev {
+  QMatDev router, gate_e, up_e, down_e, sh_gate, sh_up, sh_down;
+  const float* sh_gate_inp;
+  int d, n_exp, top_k, ff, sf;
+};
+struct MoeWork {            // scratch for up to 8 tokens, owned by whoever launches the block
+  float* logits;            // [8][n_exp]
+  int32_t* sel_idx;         // [8][top_k] ascending expert id
+  float* sel_w;             // [8][top_k]
+  float* sg;                // [8] sigmoid(sh_gate_inp . x)
+  float* h;                 // [8*(top_k+1)][max(ff, sf)]
+  float* partial;           // [8*(top_k+1)][d]
+};
+size_t pyre_moe_work_bytes(const MoeDev& m);
+void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
+// y[t][d] = ffn(x[t][d]).  If comb_x != nullptr the result is also folded into the residual streams:
+// comb_x[ti][s][i] += y[ti][i] * 2*sigmoid(comb_inj[ti][s])   (hc_combine)
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev);
+
+// ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
+struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
+struct HcWork { float* xn; float* o; float* lo; float* gate; };     // [8][hc*d], [8][lr+hc], [8][lr], [8][hc*d]
+size_t pyre_hc_work_bytes(const HcDev& h);
+void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
+// optional combine first (x[ti][s][:] += comb_out[ti][:] * 2*sigmoid(comb_inj[ti][s])), then mixed/inj = hc_mix(x)
+int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, float* x_dev, int t, const float* comb_out, const float* comb_inj,
+                       float eps, float* mixed_dev, float* inj_dev);
+int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, const float* out_dev, const float* inj_dev);
+
+// ---- Gated DeltaNet (gdn.hip) -----------------------------------------------------------------------------------------
+struct GdnDev { const float* a; const float* dt; const float* conv_w; const float* norm_w; int nk, nv, dk, dv, conv_k; float eps; };
+// proj [t][ch + nv*dv + 2*nv] = [qkv | z | beta | alpha] per token (row stride = proj_stride floats).
+// conv_in/conv_out [(k-1)][ch], ssm_in/ssm_out [nv][dk][dv] (in != out).  co_scratch [8][ch].  out [t][nv*dv].
+int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev);
+
+// ---- gated attention over the KV cache (attn.hip) -----------------------------------------------------------------------
+struct AttnDev { const float* qn; const float* kn; const float* rope_inv; int nh, nkv, hd, n_rot, kv_bits, kv_recent; float eps; };
+struct KvDev {
+  float* kf;        // [nkv][hd][cap]      f32 keys, position-minor (lane = position reads are coalesced)
+  float* vf;        // [cap][nkv*hd]       f32 values, row-major
+  uint32_t* kq;     // [nkv][hd/8][cap]    4-bit keys: word w of position p holds dims 8w..8w+7
+  float* ks;        // [nkv][hd/32][cap]   key scales
+  uint32_t* vq;     // [cap][nkv*hd/8]     4-bit values
+  float* vs;        // [cap][nkv*hd/32]    value scales
+  int cap;
+};
+struct AttnWork { float* q; float* part_o; float* part_ml; int max_chunks; };   // q [8][nh][hd]; partials per (token, head, chunk)
+size_t pyre_kv_bytes(const AttnDev& a, int cap);
+void   pyre_kv_carve(const AttnDev& a, int cap, void* base, KvDev* kv);
+size_t pyre_attn_work_bytes(const AttnDev& a, int cap);
+void   pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w);
+// qkv [t][nh*2*hd + 2*nkv*hd] = [q (with interleaved gate) | k | v] raw projections; positions start..start+t-1 are
+// appended; packed_done = number of leading positions already packed (updated by the call). out [t][nh*hd].
+int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
+                     int* packed_done, float* out_dev);
+size_t pyre_packed_boundary(size_t n_visible, int kv_bits, int recent);

@@ -1,0 +1,165 @@
+// Gated DeltaNet recurrent step: causal depthwise conv1d + SiLU, L2-normalised q/k, gated delta rule on the fp32
+// state kept resident in HBM, gated RMSNorm.  Follows linear_core, src/model/qwen4exp_gguf.rs:1624-1673.
+#include "formats.h"
+
+__device__ __forceinline__ float g_sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float g_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+
+// grid ceil(ch/256): channel c runs its t tokens in order (:1643-1647): o = w[k-1]*cur + sum_j w[j]*state[j], co = silu(o),
+// then the window slides.  State rows are oldest first.
+__global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj, int stride, int t, int ch, int kk, const float* __restrict__ conv_w,
+                                                  const float* __restrict__ conv_in, float* __restrict__ conv_out, float* __restrict__ co) {
+  int c = blockIdx.x * 256 + threadIdx.x; if (c >= ch) return;
+  float w[8], hist[8];
+  for (int k = 0; k < kk; ++k) w[k] = conv_w[(size_t)c * kk + k];
+  for (int k = 0; k < kk - 1; ++k) hist[k] = conv_in[(size_t)k * ch + c];
+  for (int ti = 0; ti < t; ++ti) {
+    float cur = proj[(size_t)ti * stride + c];
+    float o = w[kk - 1] * cur;
+    for (int k = 0; k < kk - 1; ++k) o += w[k] * hist[k];
+    co[(size_t)ti * ch + c] = o * g_sigm(o);
+    for (int k = 0; k + 1 < kk - 1; ++k) hist[k] = hist[k + 1];
+    hist[kk - 2] = cur;
+  }
+  for (int k = 0; k < kk - 1; ++k) conv_out[(size_t)k * ch + c] = hist[k];
+}
+
+// grid nv, 512 threads.  Thread (grp = tid/128, j = tid%128) keeps rows 32*grp..32*grp+31 of column j of the head's
+// 128x128 state in registers across the whole token window, so the state is read once and written once per launch.
+template <int DK, int DV>
+__global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
+                                                   const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out) {
+  static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
+  constexpr int G = 4, R = DK / G;
+  __shared__ float qs[DK], ks[DK], pm[G][DV], po[G][DV], red[8];
+  const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7;
+  const int ch = 2 * p.nk * DK + p.nv * DV, w = p.nv * DV;
+  const float* sin_ = ssm_in + (size_t)h * DK * DV; float* sout = ssm_out + (size_t)h * DK * DV;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) S[r] = sin_[(size_t)(grp * R + r) * DV + j];
+  const float a = p.a[h], dtb = p.dt[h];
+  for (int ti = 0; ti < t; ++ti) {
+    const float* co = co_all + (size_t)ti * ch;
+    const float* pr = proj + (size_t)ti * stride;
+    // L2 norms of q (threads 0..127) and k (threads 128..255) of key head kh (:1649-1651)
+    float v = 0.0f;
+    if (tid < DK) v = co[kh * DK + tid]; else if (tid < 2 * DK) v = co[p.nk * DK + kh * DK + (tid - DK)];
+    float sq = v * v;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+    if ((tid & 63) == 0) red[tid >> 6] = sq;
+    __syncthreads();
+    if (tid < DK) qs[tid] = v * ((1.0f / sqrtf(red[0] + red[1] + 1e-6f)) * (1.0f / sqrtf((float)DK)));
+    else if (tid < 2 * DK) ks[tid - DK] = v * ((1.0f / sqrtf(red[2] + red[3] + 1e-6f)) * 1.0f);
+    const float g = expf(g_softplus(pr[ch + w + p.nv + h] + dtb) * a);      // alpha at [ch + nv*dv + nv + h]
+    const float b = g_sigm(pr[ch + w + h]);                                 // beta  at [ch + nv*dv + h]
+    __syncthreads();
+    float pmv = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[grp * R + r]; }
+    pm[grp][j] = pmv;
+    __syncthreads();
+    const float mem = ((pm[0][j] + pm[1][j]) + pm[2][j]) + pm[3][j];
+    const float delta = (co[2 * p.nk * DK + h * DV + j] - mem) * b;
+    float pov = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) { S[r] += ks[grp * R + r] * delta; pov += S[r] * qs[grp * R + r]; }
+    po[grp][j] = pov;
+    __syncthreads();
+    if (tid < DV) {
+      float o = ((po[0][j] + po[1][j]) + po[2][j]) + po[3][j];
+      float ss = o * o;
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) ss += __shfl_xor(ss, d);
+      if ((tid & 63) == 0) red[4 + (tid >> 6)] = ss;
+      pm[0][j] = o;                       // pm is free again: keep o across the barrier below
+    }
+    __syncthreads();
+    if (tid < DV) {
+      float sc = 1.0f / sqrtf((red[4] + red[5]) / (float)DV + p.eps);
+      float o = pm[0][j] * (sc * p.norm_w[j]);                              // rms_inplace: x *= s * w  (:210)
+      out[(size_t)ti * w + h * DV + j] = o * g_sigm(pr[ch + h * DV + j]);   // z at [ch + h*dv + j]
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) sout[(size_t)(grp * R + r) * DV + j] = S[r];
+}
+
+int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
+                    const float* ssm_in, float* ssm_out, float* co, float* out) {
+  if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
+  if (g.conv_k < 2 || g.conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: conv kernel %d outside 2..8", g.conv_k);
+  if (t < 1) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d", t);
+  int ch = 2 * g.nk * g.dk + g.nv * g.dv;
+  hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); PYRE_CHECK_LAUNCH(ctx);
+  hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out); PYRE_CHECK_LAUNCH(ctx);
+  return PYRE_OK;
+}
+
+// ---- C ABI: standalone layer core for the block harness ---------------------------------------------------------------
+struct pyre_gdn {
+  pyre_ctx* ctx; GdnDev dv; float* params; int ch, pw;      // pw = projection width per token
+  float* conv[2]; float* ssm[2]; int cur; float* co; float* io; size_t io_tokens;
+};
+
+extern "C" {
+
+int pyre_gdn_create(pyre_ctx* ctx, int nk, int nv, int dk, int dv, int conv_k, float eps, const float* a, const float* dt, const float* conv_w, const float* norm_w, pyre_gdn** out) {
+  if (!ctx || !out || !a || !dt || !conv_w || !norm_w) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_create: null argument");
+  *out = nullptr;
+  if (dk != 128 || dv != 128 || nk < 1 || nv < 1 || nv % nk || conv_k < 2 || conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_gdn_create: unsupported geometry nk %d nv %d dk %d dv %d conv %d", nk, nv, dk, dv, conv_k);
+  pyre_gdn* g = new pyre_gdn(); g->ctx = ctx; g->ch = 2 * nk * dk + nv * dv; g->pw = g->ch + nv * dv + 2 * nv; g->cur = 0; g->io = nullptr; g->io_tokens = 0;
+  size_t np = (size_t)2 * nv + (size_t)g->ch * conv_k + dv;
+  std::vector<float> hp(np); memcpy(hp.data(), a, 4 * nv); memcpy(hp.data() + nv, dt, 4 * nv); memcpy(hp.data() + 2 * nv, conv_w, 4 * (size_t)g->ch * conv_k); memcpy(hp.data() + 2 * nv + (size_t)g->ch * conv_k, norm_w, 4 * dv);
+  size_t cs = (size_t)(conv_k - 1) * g->ch, ss = (size_t)nv * dk * dv;
+  hipError_t e = hipMalloc((void**)&g->params, np * 4);
+  if (e == hipSuccess) e = hipMemcpy(g->params, hp.data(), np * 4, hipMemcpyHostToDevice);
+  for (int i = 0; i < 2 && e == hipSuccess; ++i) { e = hipMalloc((void**)&g->conv[i], cs * 4); if (e == hipSuccess) e = hipMalloc((void**)&g->ssm[i], ss * 4);
+    if (e == hipSuccess) e = hipMemset(g->conv[i], 0, cs * 4); if (e == hipSuccess) e = hipMemset(g->ssm[i], 0, ss * 4); }
+  if (e == hipSuccess) e = hipMalloc((void**)&g->co, (size_t)8 * g->ch * 4);
+  if (e != hipSuccess) { int rc = pyre_fail(ctx, PYRE_E_HIP, "pyre_gdn_create: %s", hipGetErrorString(e)); delete g; return rc; }
+  g->dv = GdnDev{g->params, g->params + nv, g->params + 2 * nv, g->params + 2 * nv + (size_t)g->ch * conv_k, nk, nv, dk, dv, conv_k, eps};
+  *out = g; return PYRE_OK;
+}
+void pyre_gdn_destroy(pyre_gdn* g) { if (!g) return; (void)hipStreamSynchronize(g->ctx->stream); (void)hipFree(g->params); for (int i = 0; i < 2; ++i) { (void)hipFree(g->conv[i]); (void)hipFree(g->ssm[i]); } (void)hipFree(g->co); if (g->io) (void)hipFree(g->io); delete g; }
+
+int pyre_gdn_set_state(pyre_ctx* ctx, pyre_gdn* g, const float* conv_host, const float* ssm_host) {
+  if (!ctx || !g) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_set_state: null argument");
+  size_t cs = (size_t)(g->dv.conv_k - 1) * g->ch * 4, ss = (size_t)g->dv.nv * g->dv.dk * g->dv.dv * 4;
+  if (conv_host) PYRE_HIP(ctx, hipMemcpyAsync(g->conv[g->cur], conv_host, cs, hipMemcpyHostToDevice, ctx->stream)); else PYRE_HIP(ctx, hipMemsetAsync(g->conv[g->cur], 0, cs, ctx->stream));
+  if (ssm_host) PYRE_HIP(ctx, hipMemcpyAsync(g->ssm[g->cur], ssm_host, ss, hipMemcpyHostToDevice, ctx->stream)); else PYRE_HIP(ctx, hipMemsetAsync(g->ssm[g->cur], 0, ss, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+int pyre_gdn_get_state(pyre_ctx* ctx, pyre_gdn* g, float* conv_host, float* ssm_host) {
+  if (!ctx || !g) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_get_state: null argument");
+  size_t cs = (size_t)(g->dv.conv_k - 1) * g->ch * 4, ss = (size_t)g->dv.nv * g->dv.dk * g->dv.dv * 4;
+  if (conv_host) PYRE_HIP(ctx, hipMemcpyAsync(conv_host, g->conv[g->cur], cs, hipMemcpyDeviceToHost, ctx->stream));
+  if (ssm_host) PYRE_HIP(ctx, hipMemcpyAsync(ssm_host, g->ssm[g->cur], ss, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+static int gdn_io(pyre_ctx* ctx, pyre_gdn* g, size_t tokens) {
+  if (tokens <= g->io_tokens) return PYRE_OK;
+  if (g->io) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(g->io)); g->io = nullptr; g->io_tokens = 0; }
+  PYRE_HIP(ctx, hipMalloc((void**)&g->io, tokens * ((size_t)g->pw + (size_t)g->dv.nv * g->dv.dv) * 4)); g->io_tokens = tokens; return PYRE_OK;
+}
+
+// The recurrent decode / verify step over t tokens (sequential in time): proj [t][ch + nv*dv + 2*nv] -> out [t][nv*dv].
+int pyre_gdn_step(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int t, float* out_host) {
+  if (!ctx || !g || !proj_host || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_step: null argument");
+  if (t < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_step: t = %d", t);
+  int rc = gdn_io(ctx, g, t); if (rc) return rc;
+  float* pd = g->io; float* od = g->io + (size_t)t * g->pw; size_t ow = (size_t)g->dv.nv * g->dv.dv;
+  PYRE_HIP(ctx, hipMemcpyAsync(pd, proj_host, (size_t)t * g->pw * 4, hipMemcpyHostToDevice, ctx->stream));
+  for (int t0 = 0; t0 < t; t0 += 8) {          // the conv scratch holds 8 tokens
+    int n = t - t0 < 8 ? t - t0 : 8; int nx = g->cur ^ 1;
+    rc = pyre_gdn_launch(ctx, g->dv, pd + (size_t)t0 * g->pw, g->pw, n, g->conv[g->cur], g->conv[nx], g->ssm[g->cur], g->ssm[nx], g->co, od + (size_t)t0 * ow); if (rc) return rc;
+    g->cur = nx;
+  }
+  PYRE_HIP(ctx, hipMemcpyAsync(out_host, od, (size_t)t * ow * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+}  // extern "C"

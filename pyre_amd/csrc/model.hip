@@ -1,0 +1,391 @@
+// The qwen4exp token step on the device: embed -> per layer { hc_mix -> Gated DeltaNet | gated attention -> hc_combine
+// -> hc_mix -> MoE FFN -> hc_combine } -> head hc_mix -> logits, plus the multi-token verify window, rollback and the
+// greedy loop.  Follows Model::forward_inner / forward_multi / spec_keep (src/model/qwen4exp_gguf.rs:2087-2157,
+// 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
+#include "formats.h"
+#include <memory>
+
+namespace {
+
+struct Layer {
+  bool full = false;
+  HcDev hca{}, hcf{};
+  QMatDev proj{};            // attention: [q ; k ; v]   DeltaNet: [qkv ; z ; beta ; alpha]
+  QMatDev outp{};            // attn_output / ssm_out
+  AttnDev attn{}; GdnDev gdn{}; MoeDev moe{};
+  int mix_index = 0;         // index among the attention or among the DeltaNet layers
+};
+
+}  // namespace
+
+struct pyre_model {
+  pyre_ctx* ctx = nullptr; pyre_model_cfg c{};
+  std::vector<Layer> layers; HcDev head{}; QMatDev embd{}, out{};
+  std::vector<pyre_qmat*> owned; std::vector<void*> bufs;
+  float* rope_inv = nullptr; int n_attn = 0, n_lin = 0, ch = 0, pw_lin = 0, pw_attn = 0;
+  size_t token_weight_bytes = 0;
+  // activations for a window of up to 8 tokens
+  void* work = nullptr; HcWork hw{}; MoeWork mw{};
+  float *x = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
+  uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0;
+};
+
+struct pyre_state {
+  pyre_ctx* ctx = nullptr; const pyre_model* m = nullptr; int cap = 0, len = 0;
+  void* mem = nullptr;
+  std::vector<float*> conv[2], ssm[2]; std::vector<int> cur;     // DeltaNet double buffers
+  std::vector<float*> proj_saved;                                // per DeltaNet layer [8][pw_lin]: inputs of the last window
+  std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
+  int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
+};
+
+namespace {
+
+__global__ void k_replicate(const float* __restrict__ e, int d, int hc, float* __restrict__ x) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x, s = blockIdx.y, ti = blockIdx.z; if (i >= d) return;
+  x[((size_t)ti * hc + s) * d + i] = e[(size_t)ti * d + i];
+}
+// first index of the maximum (sampler::argmax, strict >); one block, result -> out[0] (and mirror, if given)
+__global__ __launch_bounds__(1024) void k_argmax(const float* __restrict__ lg, int n, uint32_t* out, uint32_t* mirror) {
+  __shared__ float bv[1024]; __shared__ int bi[1024];
+  int tid = threadIdx.x; float best = -INFINITY; int idx = n;
+  for (int i = tid; i < n; i += 1024) { float v = lg[i]; if (idx == n || v > best) { best = v; idx = i; } }
+  bv[tid] = best; bi[tid] = idx; __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if (tid < s) { float v2 = bv[tid + s]; int i2 = bi[tid + s]; if (i2 < n && (bi[tid] >= n || v2 > bv[tid] || (v2 == bv[tid] && i2 < bi[tid]))) { bv[tid] = v2; bi[tid] = i2; } }
+    __syncthreads();
+  }
+  if (tid == 0) { uint32_t r = (uint32_t)(bi[0] < n ? bi[0] : 0); out[0] = r; if (mirror) mirror[0] = r; }
+}
+
+struct Builder {
+  pyre_ctx* ctx; pyre_model* m;
+  int fail(int code, const char* what) { return pyre_fail(ctx, code, "pyre_model_create: %s", what); }
+
+  // one matrix out of `n` row-concatenated tensors of one type and width
+  int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes) {
+    uint32_t ty = ts[0]->ggml_type; uint64_t cols = ts[0]->cols; uint32_t dev = ts[0]->on_device; uint64_t rows = 0; size_t total = 0;
+    int fmt = fmt_from_ggml(ty); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported tensor type");
+    FmtGeom g = fmt_geom(fmt);
+    for (int i = 0; i < n; ++i) {
+      if (!ts[i]->data) return fail(PYRE_E_ARG, "missing tensor");
+      if (ts[i]->ggml_type != ty || ts[i]->cols != cols || ts[i]->on_device != dev) return fail(PYRE_E_TYPE, "tensors of one projection group differ in type, width or location");
+      rows += ts[i]->rows; total += ts[i]->rows * (cols / g.el * g.bytes);
+    }
+    pyre_qmat* q = nullptr; int rc;
+    if (n == 1) rc = dev ? pyre_qmat_create_dev(ctx, ty, rows, cols, ts[0]->data, total, &q) : pyre_qmat_create(ctx, ty, rows, cols, ts[0]->data, total, &q);
+    else {
+      void* tmp = nullptr; PYRE_HIP(ctx, hipMalloc(&tmp, total)); size_t off = 0;
+      for (int i = 0; i < n; ++i) { size_t nb = ts[i]->rows * (cols / g.el * g.bytes);
+        hipError_t e = hipMemcpy((uint8_t*)tmp + off, ts[i]->data, nb, dev ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
+        if (e != hipSuccess) { (void)hipFree(tmp); return pyre_fail(ctx, PYRE_E_HIP, "pyre_model_create: copy: %s", hipGetErrorString(e)); } off += nb; }
+      rc = pyre_qmat_create_dev(ctx, ty, rows, cols, tmp, total, &q); (void)hipFree(tmp);
+    }
+    if (rc) return rc;
+    m->owned.push_back(q); *out = q->dv; if (gguf_bytes) *gguf_bytes += total; return PYRE_OK;
+  }
+  int one(const pyre_tensor& t, QMatDev* out, size_t* gguf_bytes) { const pyre_tensor* p = &t; return cat(&p, 1, out, gguf_bytes); }
+
+  // Gguf::vec: a small tensor fully dequantized to f32 on the device
+  int vec(const pyre_tensor& t, size_t expect, const float** out) {
+    if (!t.data) return fail(PYRE_E_ARG, "missing vector tensor");
+    size_t n = t.rows * t.cols; if (n != expect) return fail(PYRE_E_SHAPE, "vector tensor has the wrong length");
+    float* d = nullptr; PYRE_HIP(ctx, hipMalloc((void**)&d, n * 4)); m->bufs.push_back(d);
+    if (t.ggml_type == PYRE_F32) { PYRE_HIP(ctx, hipMemcpy(d, t.data, n * 4, t.on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice)); }
+    else {
+      pyre_qmat* q = nullptr; int fmt = fmt_from_ggml(t.ggml_type); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported vector type"); FmtGeom g = fmt_geom(fmt);
+      size_t nb = n / g.el * g.bytes;
+      int rc = t.on_device ? pyre_qmat_create_dev(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q) : pyre_qmat_create(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q); if (rc) return rc;
+      rc = pyre_qmat_dequant_dev(ctx, q, d); if (!rc) rc = pyre_ctx_sync(ctx); pyre_qmat_destroy(q); if (rc) return rc;
+    }
+    *out = d; return PYRE_OK;
+  }
+  int hc(const pyre_tensor& norm, const pyre_tensor& down, const pyre_tensor* inject, const pyre_tensor& up, HcDev* h, size_t* bytes) {
+    const pyre_model_cfg& c = m->c; size_t w = (size_t)c.hc * c.d;
+    if (down.rows != (uint64_t)c.hc_lr || down.cols != w || up.rows != w || up.cols != (uint64_t)c.hc_lr) return fail(PYRE_E_SHAPE, "hyper-connection matrix shapes");
+    if (inject && (inject->rows != (uint64_t)c.hc || inject->cols != w)) return fail(PYRE_E_SHAPE, "hyper-connection inject shape");
+    const pyre_tensor* grp[2] = {&down, inject}; int rc = cat(grp, inject ? 2 : 1, &h->di, bytes); if (rc) return rc;
+    rc = one(up, &h->up, bytes); if (rc) return rc;
+    rc = vec(norm, w, &h->norm); if (rc) return rc;
+    h->d = c.d; h->hc = c.hc; h->lr = c.hc_lr; h->has_inject = inject != nullptr; return PYRE_OK;
+  }
+};
+
+size_t al256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* lt, const pyre_tensor* gl, pyre_model** out) {
+  if (!ctx || !cfg || !lt || !gl || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_create: null argument");
+  *out = nullptr;
+  const pyre_model_cfg& c = *cfg;
+  if (c.n_layers < 1 || c.d < 64 || c.d % 64 || c.hc < 1 || c.hc > 8 || c.hc_lr < 64 || c.hc_lr % 64 || c.full_every < 1 || c.vocab < 1 || c.top_k < 1 || c.n_exp < c.top_k)
+    return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_create: unsupported configuration (d and hc_lr must be multiples of 64, hc <= 8)");
+  PYRE_HIP(ctx, hipSetDevice(ctx->device));
+  std::unique_ptr<pyre_model> M(new pyre_model()); pyre_model* m = M.get(); m->ctx = ctx; m->c = c;
+  struct Guard { pyre_model* m; bool armed = true; ~Guard() { if (armed && m) { for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); } } } guard{m};
+  Builder B{ctx, m};
+  m->ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv; m->pw_lin = m->ch + c.lin_nv * c.lin_dv + 2 * c.lin_nv; m->pw_attn = c.n_head * 2 * c.hd + 2 * c.n_kv * c.hd;
+  std::vector<float> inv(c.n_rot / 2); for (int i = 0; i < c.n_rot / 2; ++i) inv[i] = powf(c.rope_base, -(2.0f * (float)i) / (float)c.n_rot);   // qn_ctx.rs:168
+  PYRE_HIP(ctx, hipMalloc((void**)&m->rope_inv, (inv.size() + 1) * 4)); m->bufs.push_back(m->rope_inv);
+  PYRE_HIP(ctx, hipMemcpy(m->rope_inv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice));
+  size_t tok_bytes = 0; int rc;
+  m->layers.resize(c.n_layers);
+  for (int il = 0; il < c.n_layers; ++il) {
+    const pyre_tensor* T = lt + (size_t)il * PYRE_LAYER_SLOTS; Layer& L = m->layers[il];
+    L.full = (il + 1) % c.full_every == 0;
+    if ((rc = B.hc(T[PYRE_T_HC_ATTN_NORM], T[PYRE_T_HC_ATTN_DOWN], &T[PYRE_T_HC_ATTN_INJECT], T[PYRE_T_HC_ATTN_UP], &L.hca, &tok_bytes))) return rc;
+    if ((rc = B.hc(T[PYRE_T_HC_FFN_NORM], T[PYRE_T_HC_FFN_DOWN], &T[PYRE_T_HC_FFN_INJECT], T[PYRE_T_HC_FFN_UP], &L.hcf, &tok_bytes))) return rc;
+    if (L.full) {
+      L.mix_index = m->n_attn++;
+      const pyre_tensor* grp[3] = {&T[PYRE_T_ATTN_Q], &T[PYRE_T_ATTN_K], &T[PYRE_T_ATTN_V]};
+      if (grp[0]->rows != (uint64_t)c.n_head * 2 * c.hd || grp[1]->rows != (uint64_t)c.n_kv * c.hd || grp[2]->rows != (uint64_t)c.n_kv * c.hd || grp[0]->cols != (uint64_t)c.d)
+        return B.fail(PYRE_E_SHAPE, "attention projection shapes");
+      if ((rc = B.cat(grp, 3, &L.proj, &tok_bytes))) return rc;
+      if (T[PYRE_T_ATTN_OUTPUT].rows != (uint64_t)c.d || T[PYRE_T_ATTN_OUTPUT].cols != (uint64_t)c.n_head * c.hd) return B.fail(PYRE_E_SHAPE, "attn_output shape");
+      if ((rc = B.one(T[PYRE_T_ATTN_OUTPUT], &L.outp, &tok_bytes))) return rc;
+      L.attn = AttnDev{nullptr, nullptr, m->rope_inv, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
+      if ((rc = B.vec(T[PYRE_T_ATTN_Q_NORM], c.hd, &L.attn.qn)) || (rc = B.vec(T[PYRE_T_ATTN_K_NORM], c.hd, &L.attn.kn))) return rc;
+    } else {
+      L.mix_index = m->n_lin++;
+      const pyre_tensor* grp[4] = {&T[PYRE_T_ATTN_QKV], &T[PYRE_T_ATTN_GATE], &T[PYRE_T_SSM_BETA], &T[PYRE_T_SSM_ALPHA]};
+      if (grp[0]->rows != (uint64_t)m->ch || grp[1]->rows != (uint64_t)c.lin_nv * c.lin_dv || grp[2]->rows != (uint64_t)c.lin_nv || grp[3]->rows != (uint64_t)c.lin_nv || grp[0]->cols != (uint64_t)c.d)
+        return B.fail(PYRE_E_SHAPE, "DeltaNet projection shapes");
+      if ((rc = B.cat(grp, 4, &L.proj, &tok_bytes))) return rc;
+      if (T[PYRE_T_SSM_OUT].rows != (uint64_t)c.d || T[PYRE_T_SSM_OUT].cols != (uint64_t)c.lin_nv * c.lin_dv) return B.fail(PYRE_E_SHAPE, "ssm_out shape");
+      if ((rc = B.one(T[PYRE_T_SSM_OUT], &L.outp, &tok_bytes))) return rc;
+      L.gdn = GdnDev{nullptr, nullptr, nullptr, nullptr, c.lin_nk, c.lin_nv, c.lin_dk, c.lin_dv, c.conv_k, c.eps};
+      if ((rc = B.vec(T[PYRE_T_SSM_A], c.lin_nv, &L.gdn.a)) || (rc = B.vec(T[PYRE_T_SSM_DT_BIAS], c.lin_nv, &L.gdn.dt)) ||
+          (rc = B.vec(T[PYRE_T_SSM_CONV1D], (size_t)m->ch * c.conv_k, &L.gdn.conv_w)) || (rc = B.vec(T[PYRE_T_SSM_NORM], c.lin_dv, &L.gdn.norm_w))) return rc;
+    }
+    MoeDev& mo = L.moe; size_t router_b = 0, ge = 0, ue = 0, de = 0, sh = 0;
+    if ((rc = B.one(T[PYRE_T_FFN_GATE_INP], &mo.router, &router_b)) || (rc = B.one(T[PYRE_T_FFN_GATE_EXPS], &mo.gate_e, &ge)) || (rc = B.one(T[PYRE_T_FFN_UP_EXPS], &mo.up_e, &ue)) ||
+        (rc = B.one(T[PYRE_T_FFN_DOWN_EXPS], &mo.down_e, &de)) || (rc = B.one(T[PYRE_T_FFN_GATE_SHEXP], &mo.sh_gate, &sh)) || (rc = B.one(T[PYRE_T_FFN_UP_SHEXP], &mo.sh_up, &sh)) ||
+        (rc = B.one(T[PYRE_T_FFN_DOWN_SHEXP], &mo.sh_down, &sh))) return rc;
+    mo.d = c.d; mo.n_exp = c.n_exp; mo.top_k = c.top_k; mo.ff = c.ff_exp; mo.sf = mo.sh_gate.rows;
+    if (mo.router.rows != c.n_exp || mo.router.cols != c.d || mo.gate_e.rows != c.n_exp * c.ff_exp || mo.up_e.rows != c.n_exp * c.ff_exp || mo.gate_e.cols != c.d || mo.up_e.cols != c.d ||
+        (size_t)mo.down_e.rows != (size_t)c.n_exp * c.d || mo.down_e.cols != c.ff_exp || mo.sh_up.rows != mo.sf || mo.sh_down.rows != c.d || mo.sh_down.cols != mo.sf || c.ff_exp % 64 || mo.sf % 64)
+      return B.fail(PYRE_E_SHAPE, "expert tensor shapes");
+    if (mo.gate_e.fmt != mo.up_e.fmt || mo.sh_gate.fmt != mo.gate_e.fmt || mo.sh_up.fmt != mo.gate_e.fmt || mo.sh_down.fmt != mo.down_e.fmt) return B.fail(PYRE_E_TYPE, "gate/up (and shared) expert types must agree");
+    if ((rc = B.vec(T[PYRE_T_FFN_GATE_INP_SHEXP], c.d, &mo.sh_gate_inp))) return rc;
+    tok_bytes += router_b + sh + (ge + ue + de) / c.n_exp * c.top_k;
+  }
+  if ((rc = B.one(gl[PYRE_G_TOKEN_EMBD], &m->embd, nullptr))) return rc;
+  if (m->embd.rows != c.vocab || m->embd.cols != c.d) return B.fail(PYRE_E_SHAPE, "token_embd shape");
+  if ((rc = B.hc(gl[PYRE_G_OUTPUT_HC_NORM], gl[PYRE_G_OUTPUT_HC_DOWN], nullptr, gl[PYRE_G_OUTPUT_HC_UP], &m->head, &tok_bytes))) return rc;
+  if ((rc = B.one(gl[PYRE_G_OUTPUT], &m->out, &tok_bytes))) return rc;
+  if (m->out.rows != c.vocab || m->out.cols != c.d) return B.fail(PYRE_E_SHAPE, "output shape");
+  { FmtGeom g = fmt_geom(m->embd.fmt); tok_bytes += (size_t)c.d / g.el * g.bytes; }
+  m->token_weight_bytes = tok_bytes;
+  // window workspace
+  const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
+  HcDev hmax = m->head; hmax.lr = c.hc_lr;
+  MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
+  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + 4096;
+  PYRE_HIP(ctx, hipMalloc(&m->work, total));
+  uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
+  pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
+  m->x = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
+  m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
+  m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
+  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16);
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  guard.armed = false; *out = M.release(); return PYRE_OK;
+}
+
+void pyre_model_destroy(pyre_model* m) {
+  if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
+  for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); if (m->toks) (void)hipFree(m->toks); delete m;
+}
+size_t pyre_model_weight_bytes_per_token(const pyre_model* m) { return m ? m->token_weight_bytes : 0; }
+
+int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_state** out) {
+  if (!ctx || !m || !out || max_ctx < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_create: bad argument");
+  *out = nullptr; const pyre_model_cfg& c = m->c;
+  std::unique_ptr<pyre_state> S(new pyre_state()); pyre_state* s = S.get(); s->ctx = ctx; s->m = m; s->cap = (max_ctx + 8 + 255) / 256 * 256;
+  size_t cs = al256((size_t)(c.conv_k - 1) * m->ch * 4), ss = al256((size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4), ps = al256((size_t)8 * m->pw_lin * 4);
+  AttnDev a0{nullptr, nullptr, nullptr, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
+  size_t kvb = al256(pyre_kv_bytes(a0, s->cap)), awb = al256(pyre_attn_work_bytes(a0, s->cap));
+  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * kvb + awb + 4096;
+  hipError_t e = hipMalloc(&s->mem, total);
+  if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_create: hipMalloc(%zu): %s", total, hipGetErrorString(e));
+  uint8_t* p = (uint8_t*)s->mem; auto take = [&](size_t n) { void* r = p; p += n; return r; };
+  for (int li = 0; li < m->n_lin; ++li) { for (int b = 0; b < 2; ++b) { s->conv[b].push_back((float*)take(cs)); s->ssm[b].push_back((float*)take(ss)); } s->proj_saved.push_back((float*)take(ps)); s->cur.push_back(0); }
+  for (int ai = 0; ai < m->n_attn; ++ai) { KvDev kv; pyre_kv_carve(a0, s->cap, take(kvb), &kv); s->kv.push_back(kv); s->packed.push_back(0); }
+  pyre_attn_work_carve(a0, s->cap, take(awb), &s->aw);
+  int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
+  *out = S.release(); return PYRE_OK;
+}
+void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); (void)hipFree(s->mem); delete s; }
+int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
+  if (!ctx || !s) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_reset: null argument");
+  const pyre_model_cfg& c = s->m->c; size_t cs = (size_t)(c.conv_k - 1) * s->m->ch * 4, ss = (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4;
+  for (size_t li = 0; li < s->cur.size(); ++li) { s->cur[li] = 0; PYRE_HIP(ctx, hipMemsetAsync(s->conv[0][li], 0, cs, ctx->stream)); PYRE_HIP(ctx, hipMemsetAsync(s->ssm[0][li], 0, ss, ctx->stream)); }
+  for (auto& pk : s->packed) pk = 0;
+  s->len = 0; s->last_window = 0; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+int pyre_state_len(const pyre_state* s) { return s ? s->len : 0; }
+int pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, float* ssm_host) {
+  if (!ctx || !s || li < 0 || li >= (int)s->cur.size()) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_read_gdn: bad layer");
+  const pyre_model_cfg& c = s->m->c; int b = s->cur[li];
+  if (conv_host) PYRE_HIP(ctx, hipMemcpyAsync(conv_host, s->conv[b][li], (size_t)(c.conv_k - 1) * s->m->ch * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (ssm_host) PYRE_HIP(ctx, hipMemcpyAsync(ssm_host, s->ssm[b][li], (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, float* v_host) {
+  if (!ctx || !s || ai < 0 || ai >= (int)s->kv.size() || !k_host || !v_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_read_kv: bad argument");
+  const pyre_model_cfg& c = s->m->c; size_t row = (size_t)c.n_kv * c.hd; std::vector<float> kt(row * s->cap);
+  PYRE_HIP(ctx, hipMemcpyAsync(kt.data(), s->kv[ai].kf, kt.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipMemcpyAsync(v_host, s->kv[ai].vf, (size_t)s->len * row * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  for (int p = 0; p < s->len; ++p) for (size_t cc = 0; cc < row; ++cc) k_host[(size_t)p * row + cc] = kt[cc * s->cap + p];
+  return PYRE_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+// One window of t <= 8 tokens whose ids already sit in m->ids.  head_tokens: 0 = no logits, 1 = last token only,
+// t = every token (logits rows 0..t-1 of m->logits).
+int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int head_tokens) {
+  const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len;
+  if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
+  int rc = pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  hipLaunchKernelGGL(k_replicate, dim3((d + 255) / 256, hc, t), dim3(256), 0, ctx->stream, m->emb, d, hc, m->x); PYRE_CHECK_LAUNCH(ctx);
+  const float* comb_out = nullptr; const float* comb_inj = nullptr;
+  for (int il = 0; il < c.n_layers; ++il) {
+    const Layer& L = m->layers[il];
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
+    if (L.full) {
+      int ai = L.mix_index;
+      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
+      if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core))) return rc;
+    } else {
+      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li];
+      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, pj))) return rc;
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[b ^ 1][li], s->ssm[b][li], s->ssm[b ^ 1][li], m->co, m->core))) return rc;
+      s->cur[li] = b ^ 1;
+    }
+    if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, m->x, t, m->o, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
+    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, m->y))) return rc;
+    comb_out = m->y; comb_inj = m->inj_f;
+  }
+  s->len = start + t;
+  if (head_tokens == 0) {   // the pending ffn output still has to reach the residual streams of ... nobody: the window's x is dropped
+    return PYRE_OK;
+  }
+  if (head_tokens >= t) {
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
+    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
+  }
+  // last token only: fold the pending ffn output into its streams, then the head
+  float* xl = m->x + (size_t)(t - 1) * hc * d;
+  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xl, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
+  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
+}
+
+int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
+  for (int i = 0; i < n; ++i) if (ids[i] >= (uint32_t)m->c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "forward: token id %u outside the vocabulary (%d)", ids[i], m->c.vocab);
+  return PYRE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host) {
+  if (!ctx || !m || !s || !ids || n < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward: bad argument");
+  if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: state belongs to another model");
+  if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: %d + %d tokens exceed the state's capacity %d", s->len, n, s->cap);
+  int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
+  s->last_window = 0;
+  for (int i = 0; i < n; i += 8) {
+    int t = n - i < 8 ? n - i : 8; bool last = i + t >= n;
+    PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
+    if ((rc = run_window(ctx, m, s, t, last && logits_host ? 1 : 0))) return rc;
+  }
+  if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host) {
+  if (!ctx || !m || !s || !ids || !logits_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward_multi: null argument");
+  if (n < 1 || n > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward_multi: window of %d tokens outside 1..8", n);
+  if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: state belongs to another model");
+  if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: context exceeds the state's capacity %d", s->cap);
+  int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
+  PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+  if ((rc = run_window(ctx, m, s, n, n))) return rc;
+  s->last_window = n;
+  PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)n * m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+// The DeltaNet layers kept the window's inputs and their pre-window state (the other half of the double buffer): the
+// first `keep` tokens are run again from there, which reproduces the checkpoint after token `keep` bit for bit.
+int pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int keep) {
+  if (!ctx || !m || !s) return pyre_fail(ctx, PYRE_E_ARG, "pyre_spec_keep: null argument");
+  if (keep >= t || t < 2) return PYRE_OK;
+  if (keep < 1) keep = 1;
+  if (s->last_window != t) return pyre_fail(ctx, PYRE_E_STATE, "pyre_spec_keep: the last forward_multi window had %d tokens, not %d", s->last_window, t);
+  for (const Layer& L : m->layers) if (!L.full) {
+    int li = L.mix_index, after = s->cur[li], before = after ^ 1;
+    int rc = pyre_gdn_launch(ctx, L.gdn, s->proj_saved[li], m->pw_lin, keep, s->conv[before][li], s->conv[after][li], s->ssm[before][li], s->ssm[after][li], m->co, m->core); if (rc) return rc;
+  }
+  s->len -= t - keep; s->last_window = 0;
+  return PYRE_OK;
+}
+
+int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host) {
+  pyre_model* m = const_cast<pyre_model*>(mc);
+  if (!ctx || !m || !s || n_steps < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_decode_greedy_dev: bad argument");
+  if (s->len + n_steps > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_decode_greedy_dev: context exceeds the state's capacity %d", s->cap);
+  int rc = check_ids(ctx, m, &first, 1); if (rc) return rc;
+  if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }
+  s->last_window = 0;
+  PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
+  for (int i = 0; i < n_steps; ++i) {
+    if ((rc = run_window(ctx, m, s, 1, 1))) return rc;
+    hipLaunchKernelGGL(k_argmax, dim3(1), dim3(1024), 0, ctx->stream, m->logits, m->c.vocab, m->ids, m->toks + i); PYRE_CHECK_LAUNCH(ctx);
+  }
+  if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+  return PYRE_OK;
+}
+
+static uint32_t host_argmax(const float* l, size_t n) { size_t b = 0; for (size_t i = 1; i < n; ++i) if (l[i] > l[b]) b = i; return (uint32_t)b; }
+
+int pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int n_draft, const uint32_t* draft_stream, int* rounds_out) {
+  if (!ctx || !m || !s || !first_logits || !out || n_out < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy: bad argument");
+  if (n_draft < 0 || n_draft > 7) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy: n_draft %d outside 0..7", n_draft);
+  const size_t V = m->c.vocab; int produced = 0, rounds = 0;
+  uint32_t pending = host_argmax(first_logits, V);
+  if (n_draft == 0 || !draft_stream) {
+    out[produced++] = pending;
+    if (produced < n_out) { int rc = pyre_decode_greedy_dev(ctx, m, s, pending, n_out - 1, out + 1); if (rc) return rc; }
+    if (rounds_out) *rounds_out = 0; return PYRE_OK;
+  }
+  std::vector<float> ls((size_t)8 * V);
+  for (;;) {
+    out[produced++] = pending; if (produced >= n_out) break;
+    int left = n_out - produced; int kk = n_draft < left - 1 ? n_draft : left - 1;
+    if (kk <= 0) { int rc = pyre_forward(ctx, m, s, &pending, 1, ls.data()); if (rc) return rc; pending = host_argmax(ls.data(), V); continue; }
+    uint32_t toks[8]; toks[0] = pending; for (int j = 0; j < kk; ++j) toks[j + 1] = draft_stream[produced + j];
+    int rc = pyre_forward_multi(ctx, m, s, toks, kk + 1, ls.data()); if (rc) return rc;
+    int acc = 0; bool have = false; uint32_t nx = 0;
+    for (int i = 0; i < kk; ++i) { uint32_t tk = host_argmax(ls.data() + (size_t)i * V, V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = host_argmax(ls.data() + (size_t)kk * V, V);
+    if ((rc = pyre_spec_keep(ctx, m, s, kk + 1, acc + 1))) return rc; ++rounds;
+    bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
+    if (stop) break;
+    pending = nx;
+  }
+  if (rounds_out) *rounds_out = rounds;
+  return PYRE_OK;
+}
+
+}  // extern "C"

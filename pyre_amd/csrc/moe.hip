@@ -1,0 +1,184 @@
+// MoE FFN block: router logits -> softmax top-k (one kernel) -> grouped expert GEMV over only the selected experts.
+// Follows ffn / routed (f32 branch) of the reference, src/model/qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793,
+// and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
+#include "formats.h"
+
+// ---- router: top-k by rank counting (ties -> lower index), softmax over the chosen k in ascending expert id, and the
+// shared-expert gate sigmoid(sh_gate_inp . x).  grid = tokens, 256 threads.
+__global__ __launch_bounds__(256) void k_router_topk(const float* __restrict__ logits, int n_exp, int k, const float* __restrict__ sh_gate_inp,
+                                                     const float* __restrict__ x, int d, int32_t* sel_idx, float* sel_w, float* sg) {
+  extern __shared__ float sm[];                 // n_exp logits, then n_exp flags (as uint32)
+  float* lg = sm; uint32_t* flag = (uint32_t*)(sm + n_exp);
+  __shared__ float red[256];
+  __shared__ int32_t s_idx[64]; __shared__ float s_w[64];
+  const int ti = blockIdx.x, tid = threadIdx.x;
+  for (int e = tid; e < n_exp; e += 256) { float v = logits[(size_t)ti * n_exp + e]; lg[e] = isnan(v) ? -INFINITY : v; }   // nan_clean
+  __syncthreads();
+  for (int e = tid; e < n_exp; e += 256) {
+    float v = lg[e]; int rank = 0;
+    for (int j = 0; j < n_exp; ++j) { float u = lg[j]; rank += (u > v || (u == v && j < e)) ? 1 : 0; }
+    flag[e] = rank < k ? 1u : 0u;
+  }
+  __syncthreads();
+  for (int e = tid; e < n_exp; e += 256) if (flag[e]) { int pos = 0; for (int j = 0; j < e; ++j) pos += flag[j]; s_idx[pos] = e; }
+  // shared-expert gate
+  float p = 0.0f; for (int i = tid; i < d; i += 256) p = fmaf(sh_gate_inp[i], x[(size_t)ti * d + i], p);
+  red[tid] = p; __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) { if (tid < s) red[tid] += red[tid + s]; __syncthreads(); }
+  if (tid == 0) {
+    sg[ti] = 1.0f / (1.0f + expf(-red[0]));
+    float mx = -INFINITY; for (int i = 0; i < k; ++i) mx = fmaxf(mx, lg[s_idx[i]]);
+    if (!isfinite(mx)) { for (int i = 0; i < k; ++i) s_w[i] = 1.0f / (float)k; }
+    else { float sum = 0.0f; for (int i = 0; i < k; ++i) { s_w[i] = expf(lg[s_idx[i]] - mx); sum += s_w[i]; } for (int i = 0; i < k; ++i) s_w[i] = s_w[i] / sum; }
+  }
+  __syncthreads();
+  if (tid < k) { sel_idx[ti * k + tid] = s_idx[tid]; sel_w[ti * k + tid] = s_w[tid]; }
+}
+
+// ---- expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) ----------------------------------------------------
+// grid (row tiles, entries); entry = ti*(k+1) + j, j < k: routed expert sel_idx[ti][j], j == k: the shared expert.
+template <int FMT, int NW>
+__global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ x, float* __restrict__ h, int hstride,
+                                                   const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  __shared__ float red[2][NW][64];
+  const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
+  const bool shared = j == m.top_k;
+  const int nrows = shared ? m.sf : m.ff;
+  if ((int)blockIdx.x * 64 >= nrows) return;
+  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
+  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
+  const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
+  const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.ff >> 6)) + blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
+  const float* xs = x + (size_t)ti * m.d;
+  float ag[1] = {0.0f}, au[1] = {0.0f};
+  for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(G, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, au); }
+  red[0][wave][lane] = ag[0]; red[1][wave][lane] = au[0];
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    float g = red[0][0][lane], u = red[1][0][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) { g += red[0][w][lane]; u += red[1][w][lane]; }
+    float s = 1.0f / (1.0f + expf(-g));
+    h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+  }
+}
+
+// ---- expert down: partial[entry][r] = down[r] . h[entry] ---------------------------------------------------------------
+template <int FMT, int NW>
+__global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
+                                                     const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  __shared__ float red[NW][64];
+  const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
+  const bool shared = j == m.top_k;
+  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
+  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
+  const QMatDev& D = shared ? m.sh_down : m.down_e;
+  const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.d >> 6)) + blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int upw = (D.U + NW - 1) / NW, k0 = wave * upw, kend = min(D.U, k0 + upw);
+  const float* xs = h + (size_t)entry * hstride;
+  float acc[1] = {0.0f};
+  for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
+  red[wave][lane] = acc[0];
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    float s = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) s += red[w][lane];
+    partial[(size_t)entry * m.d + blockIdx.x * 64 + lane] = s;
+  }
+}
+
+// y[ti][r] = shared[ti][r] * sg[ti] + (sum over the token's experts, ascending id, from zero, of w * partial)
+__global__ void k_moe_sum(const float* __restrict__ partial, const float* __restrict__ sel_w, const float* __restrict__ sg, int d, int k, float* __restrict__ y) {
+  int r = blockIdx.x * blockDim.x + threadIdx.x, ti = blockIdx.y; if (r >= d) return;
+  const float* p = partial + (size_t)ti * (k + 1) * d;
+  float o = 0.0f; for (int j = 0; j < k; ++j) o += sel_w[ti * k + j] * p[(size_t)j * d + r];
+  float yv = p[(size_t)k * d + r] * sg[ti];
+  y[(size_t)ti * d + r] = yv + o;
+}
+
+size_t pyre_moe_work_bytes(const MoeDev& m) {
+  size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
+  return 256 * 8 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs + 8 * k1 * (size_t)m.d);
+}
+void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
+  size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
+  w->logits = (float*)take(4 * 8 * (size_t)m.n_exp); w->sel_idx = (int32_t*)take(4 * 8 * (size_t)m.top_k); w->sel_w = (float*)take(4 * 8 * (size_t)m.top_k);
+  w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
+}
+
+#define MOE_FMT_DISPATCH(fmt, CALL) \
+  switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; CALL; } break; case FMT_F16: { constexpr int F = FMT_F16; CALL; } break; case FMT_BF16: { constexpr int F = FMT_BF16; CALL; } break; \
+    case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
+    default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
+
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y) {
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
+  int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc;
+  hipLaunchKernelGGL(k_router_topk, dim3(t), dim3(256), 2 * sizeof(float) * m.n_exp, ctx->stream, w.logits, m.n_exp, m.top_k, m.sh_gate_inp, x, m.d, w.sel_idx, w.sel_w, w.sg);
+  PYRE_CHECK_LAUNCH(ctx);
+  const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
+  const uint32_t* g3 = ctx->d_iq3s; const uint2* g2 = (const uint2*)ctx->d_iq2xs;
+  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g3, g2));
+  PYRE_CHECK_LAUNCH(ctx);
+  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g3, g2));
+  PYRE_CHECK_LAUNCH(ctx);
+  hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y);
+  PYRE_CHECK_LAUNCH(ctx);
+  return PYRE_OK;
+}
+
+// ---- C ABI -------------------------------------------------------------------------------------------------------------
+struct pyre_moe { pyre_ctx* ctx; MoeDev dv; MoeWork w; void* work; float* gate_inp; float* xy; };
+
+extern "C" {
+
+int pyre_moe_create(pyre_ctx* ctx, int top_k, const pyre_qmat* router, const pyre_qmat* gate_e, const pyre_qmat* up_e, const pyre_qmat* down_e,
+                    const float* sh_gate_inp_host, const pyre_qmat* sh_gate, const pyre_qmat* sh_up, const pyre_qmat* sh_down, pyre_moe** out) {
+  if (!ctx || !out || !router || !gate_e || !up_e || !down_e || !sh_gate_inp_host || !sh_gate || !sh_up || !sh_down) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_create: null argument");
+  *out = nullptr;
+  size_t d = router->cols, E = router->rows; if (E == 0 || gate_e->rows % E) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_moe_create: gate_exps rows %zu not a multiple of %zu experts", gate_e->rows, E);
+  size_t ff = gate_e->rows / E, sf = sh_gate->rows;
+  if (gate_e->cols != d || up_e->cols != d || up_e->rows != E * ff || down_e->rows != E * d || down_e->cols != ff || sh_gate->cols != d || sh_up->cols != d || sh_up->rows != sf ||
+      sh_down->rows != d || sh_down->cols != sf) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_moe_create: inconsistent expert tensor shapes");
+  if (ff % 64 || sf % 64 || d % 64) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_moe_create: d, expert and shared widths must be multiples of 64");
+  if (top_k < 1 || top_k > 32 || (size_t)top_k > E || E > 4096) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_create: top_k %d / experts %zu unsupported", top_k, E);
+  if (gate_e->dv.fmt != up_e->dv.fmt || sh_gate->dv.fmt != gate_e->dv.fmt || sh_up->dv.fmt != gate_e->dv.fmt || sh_down->dv.fmt != down_e->dv.fmt)
+    return pyre_fail(ctx, PYRE_E_TYPE, "pyre_moe_create: gate/up (and shared gate/up) must share one type, down and shared down another");
+  pyre_moe* m = new pyre_moe(); m->ctx = ctx;
+  m->dv = MoeDev{router->dv, gate_e->dv, up_e->dv, down_e->dv, sh_gate->dv, sh_up->dv, sh_down->dv, nullptr, (int)d, (int)E, top_k, (int)ff, (int)sf};
+  hipError_t e = hipMalloc((void**)&m->gate_inp, d * 4);
+  if (e == hipSuccess) e = hipMemcpy(m->gate_inp, sh_gate_inp_host, d * 4, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = hipMalloc(&m->work, pyre_moe_work_bytes(m->dv));
+  if (e == hipSuccess) e = hipMalloc((void**)&m->xy, 2 * 8 * d * 4);
+  if (e != hipSuccess) { int rc = pyre_fail(ctx, PYRE_E_HIP, "pyre_moe_create: %s", hipGetErrorString(e)); delete m; return rc; }
+  m->dv.sh_gate_inp = m->gate_inp; pyre_moe_work_carve(m->dv, m->work, &m->w);
+  *out = m; return PYRE_OK;
+}
+void pyre_moe_destroy(pyre_moe* m) { if (!m) return; (void)hipStreamSynchronize(m->ctx->stream); (void)hipFree(m->gate_inp); (void)hipFree(m->work); (void)hipFree(m->xy); delete m; }
+
+int pyre_moe_ffn_dev(pyre_ctx* ctx, pyre_moe* m, const float* x_dev, int t, float* y_dev) {
+  if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_ffn: null argument");
+  return pyre_moe_launch(ctx, m->dv, m->w, x_dev, t, y_dev);
+}
+int pyre_moe_ffn(pyre_ctx* ctx, pyre_moe* m, const float* x_host, int t, float* y_host, int32_t* sel_idx_host, float* sel_w_host) {
+  if (!ctx || !m || !x_host || !y_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_ffn: null argument");
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_ffn: t = %d outside 1..8", t);
+  size_t n = (size_t)t * m->dv.d * 4; float* xd = m->xy; float* yd = m->xy + 8 * (size_t)m->dv.d;
+  PYRE_HIP(ctx, hipMemcpyAsync(xd, x_host, n, hipMemcpyHostToDevice, ctx->stream));
+  int rc = pyre_moe_launch(ctx, m->dv, m->w, xd, t, yd); if (rc) return rc;
+  PYRE_HIP(ctx, hipMemcpyAsync(y_host, yd, n, hipMemcpyDeviceToHost, ctx->stream));
+  if (sel_idx_host) PYRE_HIP(ctx, hipMemcpyAsync(sel_idx_host, m->w.sel_idx, (size_t)t * m->dv.top_k * 4, hipMemcpyDeviceToHost, ctx->stream));
+  if (sel_w_host) PYRE_HIP(ctx, hipMemcpyAsync(sel_w_host, m->w.sel_w, (size_t)t * m->dv.top_k * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+}  // extern "C"

@@ -41,6 +41,36 @@ def _declare(L):
         "pyre_qmatmul": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_synth_blocks": (i32, [vp, u32, sz, u64, f32, f32, vp]),
+        "pyre_moe_create": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, C.POINTER(vp)]),
+        "pyre_moe_destroy": (None, [vp]),
+        "pyre_moe_ffn": (i32, [vp, vp, vp, i32, vp, vp, vp]),
+        "pyre_moe_ffn_dev": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_gdn_create": (i32, [vp, i32, i32, i32, i32, i32, f32, vp, vp, vp, vp, C.POINTER(vp)]),
+        "pyre_gdn_destroy": (None, [vp]),
+        "pyre_gdn_set_state": (i32, [vp, vp, vp, vp]),
+        "pyre_gdn_get_state": (i32, [vp, vp, vp, vp]),
+        "pyre_gdn_step": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_attn_create": (i32, [vp, i32, i32, i32, i32, f32, f32, vp, vp, i32, i32, i32, C.POINTER(vp)]),
+        "pyre_attn_destroy": (None, [vp]),
+        "pyre_attn_len": (i32, [vp]),
+        "pyre_attn_truncate": (i32, [vp, vp, i32]),
+        "pyre_attn_decode_kv4": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_attn_load_cache": (i32, [vp, vp, vp, vp, i32]),
+        "pyre_attn_read_cache": (i32, [vp, vp, vp, vp]),
+        "pyre_model_create": (i32, [vp, vp, vp, vp, C.POINTER(vp)]),
+        "pyre_model_destroy": (None, [vp]),
+        "pyre_model_weight_bytes_per_token": (sz, [vp]),
+        "pyre_state_create": (i32, [vp, vp, i32, C.POINTER(vp)]),
+        "pyre_state_destroy": (None, [vp]),
+        "pyre_state_reset": (i32, [vp, vp]),
+        "pyre_state_len": (i32, [vp]),
+        "pyre_state_read_gdn": (i32, [vp, vp, i32, vp, vp]),
+        "pyre_state_read_kv": (i32, [vp, vp, i32, vp, vp]),
+        "pyre_forward": (i32, [vp, vp, vp, vp, i32, vp]),
+        "pyre_forward_multi": (i32, [vp, vp, vp, vp, i32, vp]),
+        "pyre_spec_keep": (i32, [vp, vp, vp, i32, i32]),
+        "pyre_generate_greedy": (i32, [vp, vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32)]),
+        "pyre_decode_greedy_dev": (i32, [vp, vp, vp, u32, i32, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -176,6 +206,264 @@ class QMat:
     def close(self):
         if getattr(self, "h", None) and getattr(self.ctx, "h", None):
             self.ctx.L.pyre_qmat_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Moe:
+    """MoE FFN block over borrowed QMats (ffn / routed of the reference, qwen4exp_gguf.rs:1675-1795)."""
+
+    def __init__(self, ctx, top_k, router, gate_e, up_e, down_e, sh_gate_inp, sh_gate, sh_up, sh_down):
+        self.ctx = ctx
+        self._keep = (router, gate_e, up_e, down_e, sh_gate, sh_up, sh_down)
+        self.d, self.top_k = router.cols, top_k
+        sgi = np.ascontiguousarray(sh_gate_inp, dtype=np.float32)
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_moe_create(ctx.h, top_k, router.h, gate_e.h, up_e.h, down_e.h, _ptr(sgi), sh_gate.h, sh_up.h, sh_down.h, C.byref(h)), "moe_create")
+        self.h = h
+
+    def ffn(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.d)
+        t = x.shape[0]
+        y = np.empty((t, self.d), dtype=np.float32)
+        idx = np.empty((t, self.top_k), dtype=np.int32)
+        w = np.empty((t, self.top_k), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_moe_ffn(self.ctx.h, self.h, _ptr(x), t, _ptr(y), _ptr(idx), _ptr(w)), "moe_ffn")
+        return y, idx, w
+
+    def ffn_dev(self, x_dev, t, y_dev):
+        self.ctx.check(self.ctx.L.pyre_moe_ffn_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "moe_ffn_dev")
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_moe_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Gdn:
+    """Gated DeltaNet layer core with its resident recurrent state (linear_core, qwen4exp_gguf.rs:1624-1673)."""
+
+    def __init__(self, ctx, nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w):
+        self.ctx = ctx
+        self.nk, self.nv, self.dk, self.dv, self.conv_k = nk, nv, dk, dv, conv_k
+        self.ch = 2 * nk * dk + nv * dv
+        self.pw = self.ch + nv * dv + 2 * nv
+        f = lambda v: np.ascontiguousarray(v, dtype=np.float32)
+        a, dt, conv_w, norm_w = f(a), f(dt), f(conv_w), f(norm_w)
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_gdn_create(ctx.h, nk, nv, dk, dv, conv_k, eps, _ptr(a), _ptr(dt), _ptr(conv_w), _ptr(norm_w), C.byref(h)), "gdn_create")
+        self.h = h
+
+    def set_state(self, conv=None, ssm=None):
+        f = lambda v: None if v is None else np.ascontiguousarray(v, dtype=np.float32)
+        conv, ssm = f(conv), f(ssm)
+        self.ctx.check(self.ctx.L.pyre_gdn_set_state(self.ctx.h, self.h, _ptr(conv), _ptr(ssm)), "gdn_set_state")
+
+    def get_state(self):
+        conv = np.empty(((self.conv_k - 1), self.ch), dtype=np.float32)
+        ssm = np.empty((self.nv, self.dk, self.dv), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_gdn_get_state(self.ctx.h, self.h, _ptr(conv), _ptr(ssm)), "gdn_get_state")
+        return conv, ssm
+
+    def step(self, qkv, z, beta, alpha):
+        proj = np.ascontiguousarray(np.concatenate([qkv, z, beta, alpha], axis=1), dtype=np.float32)
+        t = proj.shape[0]
+        assert proj.shape[1] == self.pw
+        out = np.empty((t, self.nv * self.dv), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_gdn_step(self.ctx.h, self.h, _ptr(proj), t, _ptr(out)), "gdn_step")
+        return out
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_gdn_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Attn:
+    """Gated attention layer core over its own KV cache (attn_core dense branch, qwen4exp_gguf.rs:1558-1615)."""
+
+    def __init__(self, ctx, nh, nkv, hd, n_rot, rope_base, eps, qn, kn, kv_bits, kv_recent, max_ctx):
+        self.ctx = ctx
+        self.nh, self.nkv, self.hd = nh, nkv, hd
+        qn = np.ascontiguousarray(qn, dtype=np.float32); kn = np.ascontiguousarray(kn, dtype=np.float32)
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_attn_create(ctx.h, nh, nkv, hd, n_rot, rope_base, eps, _ptr(qn), _ptr(kn), kv_bits, kv_recent, max_ctx, C.byref(h)), "attn_create")
+        self.h = h
+
+    def __len__(self):
+        return self.ctx.L.pyre_attn_len(self.h)
+
+    def truncate(self, n):
+        self.ctx.check(self.ctx.L.pyre_attn_truncate(self.ctx.h, self.h, n), "attn_truncate")
+
+    def load_cache(self, k, v):
+        k = np.ascontiguousarray(k, dtype=np.float32); v = np.ascontiguousarray(v, dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_attn_load_cache(self.ctx.h, self.h, _ptr(k), _ptr(v), k.shape[0]), "attn_load_cache")
+
+    def read_cache(self):
+        n = len(self)
+        k = np.empty((n, self.nkv * self.hd), dtype=np.float32); v = np.empty_like(k)
+        self.ctx.check(self.ctx.L.pyre_attn_read_cache(self.ctx.h, self.h, _ptr(k), _ptr(v)), "attn_read_cache")
+        return k, v
+
+    def decode(self, q, k, v):
+        qkv = np.ascontiguousarray(np.concatenate([q, k, v], axis=1), dtype=np.float32)
+        t = qkv.shape[0]
+        out = np.empty((t, self.nh * self.hd), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_attn_decode_kv4(self.ctx.h, self.h, _ptr(qkv), t, _ptr(out)), "attn_decode_kv4")
+        return out
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_attn_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class TensorDesc(C.Structure):
+    _fields_ = [("ggml_type", C.c_uint32), ("on_device", C.c_uint32), ("rows", C.c_uint64), ("cols", C.c_uint64), ("data", C.c_void_p)]
+
+
+class ModelCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
+               [("rope_base", C.c_float), ("eps", C.c_float)] + \
+               [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
+                                         "full_every", "vocab", "kv_bits", "kv_recent")]
+
+
+LAYER_SLOTS, GLOBAL_SLOTS = 31, 5
+
+
+class Model:
+    """Model::{load, new_state, forward, forward_multi, spec_keep} of the reference over device-resident weights."""
+
+    def __init__(self, ctx, cfg, layer_tensors, globals_):
+        """cfg: object with the ModelCfg field names; layer_tensors: per layer dict slot -> (ty, rows, cols, data) where
+        data is a numpy uint8 array (host) or an int device pointer; globals_: dict slot -> the same."""
+        self.ctx = ctx
+        self.cfg = ModelCfg()
+        for name, _ in ModelCfg._fields_:
+            setattr(self.cfg, name, getattr(cfg, name))
+        keep = []
+
+        def desc(e):
+            if e is None:
+                return TensorDesc(0, 0, 0, 0, None)
+            ty, rows, cols, data = e
+            if isinstance(data, np.ndarray):
+                data = np.ascontiguousarray(data); keep.append(data)
+                return TensorDesc(ty, 0, rows, cols, data.ctypes.data)
+            return TensorDesc(ty, 1, rows, cols, int(data))
+        lt = (TensorDesc * (self.cfg.n_layers * LAYER_SLOTS))(*[desc(layer_tensors[il].get(s)) for il in range(self.cfg.n_layers) for s in range(LAYER_SLOTS)])
+        gl = (TensorDesc * GLOBAL_SLOTS)(*[desc(globals_.get(s)) for s in range(GLOBAL_SLOTS)])
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_model_create(ctx.h, C.byref(self.cfg), lt, gl, C.byref(h)), "model_create")
+        self.h = h
+        self.vocab = self.cfg.vocab
+
+    @property
+    def weight_bytes_per_token(self):
+        return self.ctx.L.pyre_model_weight_bytes_per_token(self.h)
+
+    def new_state(self, max_ctx):
+        return State(self, max_ctx)
+
+    def forward(self, ids, st, want_logits=True):
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        lg = np.empty(self.vocab, dtype=np.float32) if want_logits else None
+        self.ctx.check(self.ctx.L.pyre_forward(self.ctx.h, self.h, st.h, _ptr(ids), ids.size, _ptr(lg)), "forward")
+        return lg
+
+    def forward_multi(self, ids, st):
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        lg = np.empty((ids.size, self.vocab), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_forward_multi(self.ctx.h, self.h, st.h, _ptr(ids), ids.size, _ptr(lg)), "forward_multi")
+        return lg
+
+    def spec_keep(self, st, t, keep):
+        self.ctx.check(self.ctx.L.pyre_spec_keep(self.ctx.h, self.h, st.h, t, keep), "spec_keep")
+
+    def generate_greedy(self, st, first_logits, n_out, n_draft=0, draft_stream=None):
+        fl = np.ascontiguousarray(first_logits, dtype=np.float32)
+        out = np.empty(n_out, dtype=np.uint32)
+        ds = None
+        if draft_stream is not None:
+            ds = np.ascontiguousarray(draft_stream, dtype=np.uint32)
+            assert ds.size >= n_out + 8
+        rounds = C.c_int(0)
+        self.ctx.check(self.ctx.L.pyre_generate_greedy(self.ctx.h, self.h, st.h, _ptr(fl), n_out, _ptr(out), n_draft, _ptr(ds), C.byref(rounds)), "generate_greedy")
+        return out, rounds.value
+
+    def decode_greedy_dev(self, st, first, n_steps, fetch=True):
+        out = np.empty(n_steps, dtype=np.uint32) if fetch else None
+        self.ctx.check(self.ctx.L.pyre_decode_greedy_dev(self.ctx.h, self.h, st.h, int(first), n_steps, _ptr(out)), "decode_greedy_dev")
+        return out
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_model_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class State:
+    def __init__(self, model, max_ctx):
+        self.m = model
+        h = C.c_void_p()
+        model.ctx.check(model.ctx.L.pyre_state_create(model.ctx.h, model.h, max_ctx, C.byref(h)), "state_create")
+        self.h = h
+
+    def __len__(self):
+        return self.m.ctx.L.pyre_state_len(self.h)
+
+    def reset(self):
+        self.m.ctx.check(self.m.ctx.L.pyre_state_reset(self.m.ctx.h, self.h), "state_reset")
+
+    def gdn(self, li):
+        c = self.m.cfg
+        ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv
+        conv = np.empty(((c.conv_k - 1) * ch,), dtype=np.float32)
+        ssm = np.empty((c.lin_nv * c.lin_dk * c.lin_dv,), dtype=np.float32)
+        self.m.ctx.check(self.m.ctx.L.pyre_state_read_gdn(self.m.ctx.h, self.h, li, _ptr(conv), _ptr(ssm)), "state_read_gdn")
+        return conv, ssm
+
+    def kv(self, ai):
+        c = self.m.cfg
+        n = len(self)
+        k = np.empty((n, c.n_kv * c.hd), dtype=np.float32); v = np.empty_like(k)
+        self.m.ctx.check(self.m.ctx.L.pyre_state_read_kv(self.m.ctx.h, self.h, ai, _ptr(k), _ptr(v)), "state_read_kv")
+        return k, v
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.m, "h", None):
+            self.m.ctx.L.pyre_state_destroy(self.h)
         self.h = None
 
     def __del__(self):

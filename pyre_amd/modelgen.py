@@ -49,6 +49,10 @@ class Config:
     ff_sh: int = 0                    # shared-expert width (0 = ff_exp)
     d_lo: float = 1e-3
     d_hi: float = 2e-2
+    # quantized hyper-connection matrices use a smaller scale range: with d in [1e-3, 2e-2] their gate pre-activations
+    # reach the hundreds, every sigmoid saturates and the network becomes chaotic in f32 (f32 and f64 evaluations of
+    # the same weights then differ by percents), which would make any parity statement meaningless
+    hc_d_div: float = 64.0
 
     @property
     def ch(self):
@@ -103,6 +107,15 @@ def tensor_seed(seed, il, slot):
     return (seed * 1000003 + (il + 1) * 64 + slot) & 0x7FFFFFFFFFFFFFFF
 
 
+HC_SLOTS_LAYER = (HCA_DOWN, HCA_INJECT, HCA_UP, HCF_DOWN, HCF_INJECT, HCF_UP)
+HC_SLOTS_GLOBAL = (G_HEAD_DOWN, G_HEAD_UP)
+
+
+def scale_range(c: Config, il, slot):
+    hc = slot in (HC_SLOTS_LAYER if il >= 0 else HC_SLOTS_GLOBAL)
+    return (c.d_lo / c.hc_d_div, c.d_hi / c.hc_d_div) if hc else (c.d_lo, c.d_hi)
+
+
 def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
     s = tensor_seed(seed, il, slot)
     if kind == "q":
@@ -112,7 +125,7 @@ def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
                 return synth.bf16_normal(rows, cols, s, std)
             x = synth.normal((rows, cols), s, std)
             return (x if ty == synth.F32 else x.astype(np.float16)).view(np.uint8).reshape(-1).copy()
-        return synth.matrix(ty, rows, cols, s, c.d_lo, c.d_hi)
+        return synth.matrix(ty, rows, cols, s, *scale_range(c, il, slot))
     if kind == "router":
         return synth.bf16_normal(rows, cols, s, 0.02)
     name = kind.split(":")[1]

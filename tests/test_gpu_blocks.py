@@ -1,0 +1,194 @@
+"""GPU parity of the block-level entry points (MoE FFN, Gated DeltaNet step, gated attention over the 4-bit cache)
+against the CPU oracle, through the C ABI.  Tolerance 1e-5 on max|d| / max|ref| unless stated."""
+import numpy as np
+import pytest
+
+import orc
+from helpers import orc_tensor, relerr
+from pyre_amd import lib, synth
+from pyre_amd import modelgen as mg
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+# ---- MoE --------------------------------------------------------------------------------------------------------------
+def moe_pair(ctx, c, seed):
+    hw = mg.build_host(c, seed=seed); L = hw.layers[0]
+    qm = {s: lib.QMat(ctx, L[s][0], L[s][1], L[s][2], L[s][3]) for s in (mg.ROUTER, mg.GATE_E, mg.UP_E, mg.DOWN_E, mg.SH_GATE, mg.SH_UP, mg.SH_DOWN)}
+    moe = lib.Moe(ctx, c.top_k, qm[mg.ROUTER], qm[mg.GATE_E], qm[mg.UP_E], qm[mg.DOWN_E], hw.f32(0, mg.SH_GATE_INP), qm[mg.SH_GATE], qm[mg.SH_UP], qm[mg.SH_DOWN])
+
+    def oracle(x):
+        return orc.moe_ffn(c.d, c.n_exp, c.top_k, c.ff_exp, *(orc_tensor(L[s]) for s in (mg.ROUTER, mg.GATE_E, mg.UP_E, mg.DOWN_E)),
+                           hw.f32(0, mg.SH_GATE_INP), *(orc_tensor(L[s]) for s in (mg.SH_GATE, mg.SH_UP, mg.SH_DOWN)), x)
+    return moe, oracle, hw
+
+
+@pytest.mark.parametrize("qtype", [synth.IQ3_S, synth.IQ2_XS, synth.Q4_K, synth.Q8_0])
+@pytest.mark.parametrize("t", [1, 4])
+def test_moe_ffn_small(ctx, qtype, t):
+    c = mg.Config(n_layers=1, full_every=4, d=512, n_exp=16, top_k=4, ff_exp=256, qtype=qtype)
+    moe, oracle, _ = moe_pair(ctx, c, 7)
+    x = synth.normal((t, c.d), 100 + t)
+    y, idx, w = moe.ffn(x)
+    yo, io, wo = oracle(x)
+    assert np.array_equal(idx, io) and np.abs(w - wo).max() < 1e-6
+    assert relerr(y, yo) <= TOL
+
+
+@pytest.mark.parametrize("t", [1, 4])
+def test_moe_ffn_benchmark_geometry(ctx, t):
+    # 512 routed experts + 1 shared, d 2048, expert ff 512, top-10, IQ3_S (reduced to 64 resident experts' worth of
+    # distinct routing by the seed; all 512 experts exist)
+    c = mg.Config(n_layers=1, full_every=4, d=2048, n_exp=512, top_k=10, ff_exp=512, qtype=synth.IQ3_S)
+    moe, oracle, _ = moe_pair(ctx, c, 9)
+    x = synth.normal((t, c.d), 200 + t)
+    y, idx, w = moe.ffn(x)
+    yo, io, wo = oracle(x)
+    assert np.array_equal(idx, io) and np.abs(w - wo).max() < 1e-6 and (np.diff(idx, axis=1) > 0).all()
+    assert relerr(y, yo) <= TOL
+    # each token's result does not depend on its companions in the window
+    y1, _, _ = moe.ffn(x[:1])
+    assert np.array_equal(y1.view(np.uint32), y[:1].view(np.uint32))
+
+
+def test_router_ties_and_nan(ctx):
+    c = mg.Config(n_layers=1, full_every=4, d=256, n_exp=8, top_k=3, ff_exp=256, qtype=synth.Q8_0)
+    moe, oracle, hw = moe_pair(ctx, c, 11)
+    # x = 0 -> all router logits equal (0): ties resolve to the lowest expert ids, uniform weights
+    y, idx, w = moe.ffn(np.zeros((1, c.d), np.float32))
+    assert list(idx[0]) == [0, 1, 2] and np.allclose(w, 1 / 3) and not y.any()
+    xn = synth.normal((1, c.d), 5); xn[0, 3] = np.nan
+    y, idx, w = moe.ffn(xn)          # every logit NaN -> -inf -> lowest ids, uniform weights (nan_clean / soft_top)
+    assert list(idx[0]) == [0, 1, 2] and np.allclose(w, 1 / 3)
+
+
+# ---- Gated DeltaNet ------------------------------------------------------------------------------------------------------
+def gdn_params(nk, nv, seed, conv_k=4):
+    ch = 2 * nk * 128 + nv * 128
+    a = -np.exp(synth.uniform((nv,), seed + 1, 0.0, np.log(16.0)))
+    return dict(a=a, dt=synth.normal((nv,), seed + 8, 0.1), conv_w=synth.normal((ch * conv_k,), seed + 2, 0.5), norm_w=1 + synth.normal((128,), seed + 3, 0.1)), ch
+
+
+def gdn_inputs(nv, ch, t, seed):
+    return synth.normal((t, ch), seed + 4), synth.normal((t, nv * 128), seed + 5), synth.normal((t, nv), seed + 6), synth.normal((t, nv), seed + 7)
+
+
+@pytest.mark.parametrize("nk,nv", [(2, 4), (16, 32)])
+def test_gdn_step_matches_oracle(ctx, nk, nv):
+    p, ch = gdn_params(nk, nv, 300 + nv)
+    g = lib.Gdn(ctx, nk, nv, 128, 128, 4, 1e-6, p["a"], p["dt"], p["conv_w"], p["norm_w"])
+    S0 = synth.normal((nv, 128, 128), 77, 0.01); cs0 = synth.normal((3, ch), 78, 0.3)
+    g.set_state(cs0, S0)
+    so, co = S0.copy().reshape(-1), cs0.copy().reshape(-1)
+    for rnd, t in enumerate((1, 1, 5, 8, 13)):
+        qkv, z, beta, alpha = gdn_inputs(nv, ch, t, 1000 * rnd)
+        out = g.step(qkv, z, beta, alpha)
+        ref = orc.gdn_core(nk, nv, 128, 128, 4, 1e-6, p["a"], p["dt"], p["conv_w"], p["norm_w"], qkv, z, beta, alpha, co, so)
+        assert relerr(out, ref) <= TOL, (rnd, t)
+    conv, ssm = g.get_state()
+    assert relerr(ssm, so) <= TOL and np.array_equal(conv.reshape(-1), co)
+
+
+def test_gdn_benchmark_config_state_and_closed_forms(ctx):
+    # 16 QK heads, 32 V heads, head dim 128, conv 4, state N(0, 0.01), A_log ~ U(0, ln 16), dt_bias 0
+    nk, nv = 16, 32
+    p, ch = gdn_params(nk, nv, 400); p["dt"] = np.zeros(nv, np.float32)
+    g = lib.Gdn(ctx, nk, nv, 128, 128, 4, 1e-6, p["a"], p["dt"], p["conv_w"], p["norm_w"])
+    S0 = synth.normal((nv, 128, 128), 79, 0.01)
+    g.set_state(None, S0)
+    qkv, z, beta, alpha = gdn_inputs(nv, ch, 1, 5000)
+    # delta-rule property: g = 1, beta = 1 -> afterwards S^T k = v
+    alpha[:] = -40.0; beta[:] = 40.0
+    g.step(qkv, z, beta, alpha)
+    _, S = g.get_state()
+    w = p["conv_w"].reshape(ch, 4).astype(np.float64)
+    o = w[:, 3] * qkv[0]; co = o / (1 + np.exp(-o))
+    k = co[nk * 128:2 * nk * 128].reshape(nk, 128); k = k / np.sqrt((k * k).sum(-1, keepdims=True) + 1e-6); v = co[2 * nk * 128:].reshape(nv, 128)
+    for h in (0, 7, 31):
+        assert relerr(S[h].astype(np.float64).T @ k[h % nk], v[h]) < 1e-5
+    # pure decay: beta = 0 -> S' = g S
+    g.set_state(None, S0); beta[:] = -200.0; alpha = synth.normal((1, nv), 9)
+    g.step(qkv, z, beta, alpha)
+    _, S = g.get_state()
+    for h in (0, 13, 31):
+        gg = np.exp(np.log1p(np.exp(float(alpha[0, h]))) * float(p["a"][h]))
+        assert relerr(S[h], gg * S0[h].astype(np.float64)) < 1e-6
+
+
+def test_gdn_window_equals_single_steps(ctx):
+    nk, nv = 2, 4
+    p, ch = gdn_params(nk, nv, 500)
+    g1 = lib.Gdn(ctx, nk, nv, 128, 128, 4, 1e-6, p["a"], p["dt"], p["conv_w"], p["norm_w"])
+    g2 = lib.Gdn(ctx, nk, nv, 128, 128, 4, 1e-6, p["a"], p["dt"], p["conv_w"], p["norm_w"])
+    qkv, z, beta, alpha = gdn_inputs(nv, ch, 6, 6000)
+    a = g1.step(qkv, z, beta, alpha)
+    b = np.concatenate([g2.step(qkv[i:i + 1], z[i:i + 1], beta[i:i + 1], alpha[i:i + 1]) for i in range(6)])
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(g1.get_state()[1].view(np.uint32), g2.get_state()[1].view(np.uint32))
+
+
+# ---- attention -------------------------------------------------------------------------------------------------------------
+def attn_inputs(nh, nkv, seed, t):
+    g = lambda s, shape, std=1.0: synth.normal(shape, seed * 100 + s, std)
+    return dict(q=g(1, (t, nh * 2 * 256)), k=g(2, (t, nkv * 256)), v=g(3, (t, nkv * 256)), qn=1 + g(4, (256,), 0.1), kn=1 + g(5, (256,), 0.1))
+
+
+@pytest.mark.parametrize("nh,nkv", [(4, 2), (16, 2)])
+@pytest.mark.parametrize("kv_bits,recent,start", [(0, 1024, 0), (0, 1024, 300), (4, 64, 200), (4, 64, 700), (4, 1024, 1500)])
+def test_attention_matches_oracle(ctx, nh, nkv, kv_bits, recent, start):
+    t = 3
+    p = attn_inputs(nh, nkv, 3 + start, t)
+    row = nkv * 256
+    kc = synth.normal((start, row), 6); vc = synth.normal((start, row), 7)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], kv_bits, recent, start + 16)
+    att.load_cache(kc, vc)
+    out = att.decode(p["q"], p["k"], p["v"])
+    K = np.zeros((start + t, row), np.float32); V = np.zeros_like(K); K[:start] = kc; V[:start] = vc
+    ref = orc.attn_core(nh, nkv, 256, 64, 1e-6, orc.rope_inv(64, 1e7), p["qn"], p["kn"], p["q"], p["k"], p["v"], start, kv_bits, recent, K, V)
+    assert relerr(out, ref) <= 2e-5
+    k2, v2 = att.read_cache()
+    assert len(att) == start + t and relerr(k2, K) <= 1e-6 and np.array_equal(v2, V)
+
+
+def test_attention_token_by_token_growth_crosses_the_packing_boundary(ctx):
+    nh, nkv, recent = 4, 2, 64
+    row = nkv * 256
+    p = attn_inputs(nh, nkv, 9, 200)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, recent, 256)
+    K = np.zeros((200, row), np.float32); V = np.zeros_like(K)
+    inv = orc.rope_inv(64, 1e7)
+    worst = 0.0
+    i = 0
+    for t in [1] * 130 + [8] * 8 + [3, 3]:
+        out = att.decode(p["q"][i:i + t], p["k"][i:i + t], p["v"][i:i + t])
+        ref = orc.attn_core(nh, nkv, 256, 64, 1e-6, inv, p["qn"], p["kn"], p["q"][i:i + t], p["k"][i:i + t], p["v"][i:i + t], i, 4, recent, K, V)
+        worst = max(worst, relerr(out, ref)); i += t
+    assert i == 200 and orc.packed_boundary(200, 4, recent) == 128 and worst <= 2e-5
+
+
+def test_attention_closed_forms(ctx):
+    nh, nkv = 16, 2
+    p = attn_inputs(nh, nkv, 11, 1)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, 1024, 64)
+    out = att.decode(p["q"], p["k"], p["v"])       # a single position: out = v * sigmoid(gate)
+    for h in range(nh):
+        gate = p["q"][0].reshape(nh, 512)[h, 256:].astype(np.float64)
+        assert relerr(out[0].reshape(nh, 256)[h], p["v"][0].reshape(nkv, 256)[h // 8] / (1 + np.exp(-gate))) < 1e-6
+    # all keys zero -> uniform softmax -> mean of the values
+    att2 = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 0, 1024, 64)
+    n = 9; vc = synth.normal((n, nkv * 256), 5)
+    att2.load_cache(np.zeros((n, nkv * 256), np.float32), vc)
+    p["k"][:] = 0
+    out = att2.decode(p["q"], p["k"], p["v"])
+    allv = np.concatenate([vc, p["v"]]).astype(np.float64).reshape(n + 1, nkv, 256).mean(0)
+    for h in (0, 9, 15):
+        gate = p["q"][0].reshape(nh, 512)[h, 256:].astype(np.float64)
+        assert relerr(out[0].reshape(nh, 256)[h], allv[h // 8] / (1 + np.exp(-gate))) < 1e-5

@@ -1,0 +1,125 @@
+"""GPU parity of the layer API (forward / forward_multi / spec_keep / greedy generation) against the CPU oracle on
+small configurations the oracle finishes in seconds.  Logits: max|d| / max|logit| <= 1e-3 (in practice ~1e-6),
+greedy token streams identical."""
+import numpy as np
+import pytest
+
+import orc
+from helpers import orc_model, relerr
+from pyre_amd import lib, synth
+from pyre_amd import modelgen as mg
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def small_cfg(**kw):
+    c = mg.Config(n_layers=4, d=256, hc=2, hc_lr=64, n_exp=8, top_k=2, ff_exp=256, vocab=512, kv_recent=64)
+    for k, v in kw.items():
+        setattr(c, k, v)
+    return c
+
+
+def pair(ctx, c, seed, max_ctx=512):
+    hw = mg.build_host(c, seed=seed)
+    gm = lib.Model(ctx, c, hw.layers, hw.globals_)
+    om = orc_model(hw)
+    return hw, gm, om
+
+
+@pytest.mark.parametrize("qtype,hc_type", [(synth.IQ3_S, synth.BF16), (synth.IQ3_S, synth.IQ3_S), (synth.Q4_K, synth.F32), (synth.IQ2_XS, synth.F16), (synth.Q8_0, synth.BF16)])
+def test_forward_logits_and_state_match_oracle(ctx, qtype, hc_type):
+    c = small_cfg(qtype=qtype, hc_type=hc_type, hc_lr=256 if hc_type == synth.IQ3_S else 64)
+    hw, gm, om = pair(ctx, c, 5)
+    ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88], dtype=np.uint32)
+    gs, os_ = gm.new_state(64), om.new_state()
+    lg = gm.forward(ids, gs); lo = om.forward(ids, os_)            # prefill of 11 tokens (windows of 8 + 3)
+    assert relerr(lg, lo) <= 1e-3 and relerr(lg, lo) <= 1e-4
+    assert orc.argmax(lg) == orc.argmax(lo) and len(gs) == len(os_) == 11
+    for i in range(4):                                              # then token by token
+        tok = np.array([orc.argmax(lo)], dtype=np.uint32)
+        lg = gm.forward(tok, gs); lo = om.forward(tok, os_)
+        assert relerr(lg, lo) <= 1e-4, i
+    conv, ssm = gs.gdn(0)
+    assert relerr(ssm, os_.ssm(0)) <= 1e-4 and relerr(conv, os_.conv(0)) <= 1e-5
+    k, v = gs.kv(0)
+    assert relerr(k.reshape(-1), os_.kcache(0)) <= 1e-4 and relerr(v.reshape(-1), os_.vcache(0)) <= 1e-4
+
+
+def test_greedy_stream_identical_to_oracle_across_the_packing_boundary(ctx):
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 6)
+    prompt = (np.arange(100, dtype=np.uint32) * 37 + 11) % c.vocab
+    gs, os_ = gm.new_state(300), om.new_state()
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-4
+    n = 96                                                            # context grows to 195 > recent + 64: packed region active
+    out_g, _ = gm.generate_greedy(gs, lg, n)
+    out_o, _ = om.generate_greedy(os_, lo, n)
+    # report the oracle's top-2 margins if the streams ever split
+    assert np.array_equal(out_g, out_o), "first split at %d" % int(np.argmax(out_g != out_o))
+    assert len(gs) == len(os_) == 100 + n - 1 and orc.packed_boundary(len(os_), 4, 64) == 128
+
+
+def test_verify_window_equals_single_steps_and_rollback(ctx):
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 7)
+    prompt = np.array([5, 6, 7, 8, 9, 10, 11, 12, 13, 14], dtype=np.uint32)
+    sa, sb = gm.new_state(64), gm.new_state(64)
+    gm.forward(prompt, sa); gm.forward(prompt, sb)
+    toks = np.array([9, 100, 11, 212, 13], dtype=np.uint32)
+    lv = gm.forward_multi(toks, sa)
+    singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(5)])
+    assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32))       # every token's arithmetic = one-token decode
+    so = om.new_state(); om.forward(prompt, so); lo = om.forward_multi(toks, so)
+    assert relerr(lv, lo) <= 1e-4
+    # keep 2 of 5, continue: identical to a state that only ever saw those 2
+    gm.spec_keep(sa, 5, 2)
+    sc = gm.new_state(64); gm.forward(prompt, sc); gm.forward(toks[0:1], sc); gm.forward(toks[1:2], sc)
+    assert len(sa) == len(sc) == 12
+    nxt = np.array([40], dtype=np.uint32)
+    assert np.array_equal(gm.forward(nxt, sa).view(np.uint32), gm.forward(nxt, sc).view(np.uint32))
+    assert np.array_equal(sa.gdn(1)[1].view(np.uint32), sc.gdn(1)[1].view(np.uint32))
+    with pytest.raises(lib.PyreError):
+        gm.spec_keep(sa, 5, 2)                                        # not armed any more
+
+
+def test_drafted_generation_identical_to_plain_and_to_oracle(ctx):
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 8)
+    prompt = np.array([5, 6, 7, 8], dtype=np.uint32)
+    s0 = gm.new_state(128); f0 = gm.forward(prompt, s0)
+    plain, _ = gm.generate_greedy(s0, f0, 24)
+    so = om.new_state(); fo = om.forward(prompt, so)
+    assert np.array_equal(plain, om.generate_greedy(so, fo, 24)[0])
+    for corrupt in (False, True):
+        ds = np.concatenate([plain, np.zeros(8, np.uint32)]).astype(np.uint32)
+        if corrupt:
+            ds[3::4] = (ds[3::4] + 1) % c.vocab
+        s1 = gm.new_state(128); f1 = gm.forward(prompt, s1)
+        out, rounds = gm.generate_greedy(s1, f1, 24, n_draft=4, draft_stream=ds)
+        assert np.array_equal(out, plain) and rounds > 0
+        so = om.new_state(); fo = om.forward(prompt, so)
+        oo, orounds = om.generate_greedy(so, fo, 24, n_draft=4, draft_stream=ds)
+        assert np.array_equal(oo, plain) and orounds == rounds
+
+
+def test_errors(ctx):
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 9)
+    st = gm.new_state(16)
+    with pytest.raises(lib.PyreError):
+        gm.forward(np.array([c.vocab], dtype=np.uint32), st)                 # id outside the vocabulary
+    with pytest.raises(lib.PyreError):
+        gm.forward_multi(np.arange(9, dtype=np.uint32), st)                  # window > 8
+    with pytest.raises(lib.PyreError):
+        gm.forward(np.zeros(400, dtype=np.uint32), st)                       # beyond the state's capacity
+    bad = [dict(l) for l in hw.layers]; bad[0].pop(mg.ROUTER)
+    with pytest.raises(lib.PyreError):
+        lib.Model(ctx, c, bad, hw.globals_)                                  # missing tensor
