@@ -1,10 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark driver.  `python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.
 
-Workloads (all synthetic, inputs resident in HBM before the timed region):
+Workloads (synthetic weights and inputs, resident in HBM before the timed region):
+  decode  (default) batch-1 greedy decode of the Qwen-Next-style A3B hybrid of BASELINE.json configs[4]: 48 layers
+          (3 Gated DeltaNet + 1 gated attention per group), 512 routed experts top-10 + 1 shared per layer, vocab
+          151936, everything IQ3_S except the bf16 router, 4-bit KV cache behind a --ctx token prompt of random ids.
+          One step = one generated token; the whole loop runs on the device without host round trips.
   gemv    one IQ3_S dequant-GEMV of the vocabulary-head shape (151936 x 2048, t = 1) per step, rotating over enough
           distinct weight buffers (> 512 MB) that nothing is served from the 256 MB Infinity Cache.
-The timed region is bracketed by HIP events recorded on the library's own stream.
+Timed regions are bracketed by HIP events recorded on the library's own stream; per-kernel-class durations come from
+the library's event-pair profiler in a second, separately timed pass.
 """
 import argparse
 import ctypes as C
@@ -47,8 +52,13 @@ class HipEvents:
         return float(ms.value)
 
 
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+# ---------------------------------------------------------------------------------------------------------------- gemv
 def cpu_baseline_gemv(ty, rows, cols, seed, budget_s=12.0):
-    """The oracle's QMat::matmul restatement (row dequant + f32 dot, rows over all host threads) on a bounded row
+    """The oracle's QMat::matmul restatement (row dequant + f32 dot, rows over the host threads) on a bounded row
     sample of the same matrix."""
     import orc
     from pyre_amd import synth
@@ -64,8 +74,7 @@ def cpu_baseline_gemv(ty, rows, cols, seed, budget_s=12.0):
         dt = time.perf_counter() - t0
         if dt > budget_s or n >= 200:
             break
-    rows_per_s = n * sample_rows / dt
-    gb_s = rows_per_s * (cols // el * bs) / 1e9
+    gb_s = n * sample_rows / dt * (cols // el * bs) / 1e9
     return {"value": round(gb_s, 3), "unit": "GB/s of GGUF weight bytes", "cores": threads, "kind": "port",
             "sample": "%d launches of the oracle matmul over the first %d rows x %d cols (IQ3_S), t=1" % (n, sample_rows, cols)}
 
@@ -90,15 +99,11 @@ def bench_gemv(args):
         mats[i % nbuf].matmul_dev(x, 1, y)
     ctx.sync()
     e0, e1 = ev.event(), ev.event()
-    t0 = time.perf_counter()
     ev.record(e0, ctx.stream)
     for i in range(args.steps):
         mats[i % nbuf].matmul_dev(x, 1, y)
     ev.record(e1, ctx.stream)
-    ms = ev.elapsed_ms(e0, e1)
-    ctx.sync()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    per = ms / args.steps
+    per = ev.elapsed_ms(e0, e1) / args.steps
     alg_bytes = mats[0].gguf_bytes + 4 * cols + 4 * rows
     gbs = alg_bytes / (per * 1e-3) / 1e9
     out = {
@@ -108,25 +113,157 @@ def bench_gemv(args):
         "config": {"workload": "configs[1]: IQ3_S GEMV 2048->151936, batch 1, rotating over %d weight buffers (%.0f MB)" % (nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": "k_gemv<IQ3_S,1>", "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(per * 1e3, 3)},
-        "wall_ms_per_step": round(wall_ms / args.steps, 5),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemv(ty, rows, cols, 9000)
     return out
 
 
+# -------------------------------------------------------------------------------------------------------------- decode
+def cpu_baseline_decode(cfg, seed, budget_s=20.0):
+    """The oracle's token step (the reference's host f32 path restated in C++) on a bounded sample: ONE group of four
+    layers (3 Gated DeltaNet + 1 attention, all 512 experts resident) plus the head of the same configuration, decoded
+    at a short context; tok/s of the 48-layer model follows from time(4 layers) * 12 + time(head)."""
+    import copy
+    import orc
+    from helpers import orc_model
+    from pyre_amd import modelgen as mg
+    threads = min(os.cpu_count() or 1, 16)
+    c4 = copy.copy(cfg); c4.n_layers = 4
+    t0 = time.perf_counter()
+    hw = mg.build_host(c4, seed=seed)
+    om = orc_model(hw, threads=threads)
+    log("cpu baseline: 4-layer host weights in %.1f s" % (time.perf_counter() - t0))
+    st = om.new_state()
+    g = np.random.Generator(np.random.PCG64(11))
+    prompt = g.integers(0, cfg.vocab, 16, dtype=np.uint32)
+    lg = om.forward(prompt, st)
+    # time the head separately: logits of a 0-layer model are not available, so time full steps and the head GEMV alone
+    n = 0; t0 = time.perf_counter(); tok = np.array([orc.argmax(lg)], dtype=np.uint32)
+    while True:
+        lg = om.forward(tok, st); tok = np.array([orc.argmax(lg)], dtype=np.uint32); n += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or n >= 64:
+            break
+    step4 = dt / n
+    ty, rows, cols, raw = hw.globals_[mg.G_OUT]
+    x = np.ones((1, cols), np.float32)
+    orc.matmul(ty, raw, rows, cols, x, threads=threads)
+    t0 = time.perf_counter(); k = 0
+    while k < 5:
+        orc.matmul(ty, raw, rows, cols, x, threads=threads); k += 1
+    head = (time.perf_counter() - t0) / k
+    full = (step4 - head) * (cfg.n_layers / 4.0) + head
+    return {"value": round(1.0 / full, 3), "unit": "tok/s", "cores": threads, "kind": "port",
+            "sample": "oracle (C++ restatement of the reference's host f32 path, not the pyre executable): %d greedy steps of a 4-layer slice "
+                      "(3 DeltaNet + 1 attention, 512 experts each) at context %d took %.3f s/step incl. the %.3f s vocabulary head; "
+                      "scaled to %d layers: (step - head) * %d + head" % (n, len(st), step4, head, cfg.n_layers, cfg.n_layers // 4)}
+
+
+def kv_bytes_per_token(cfg, n):
+    """Bytes of KV cache one decode step reads at context n (packed region 0.625 B/value incl. scales, f32 recent)."""
+    pb = ((n - cfg.kv_recent) // 64) * 64 if (cfg.kv_bits == 4 and n > cfg.kv_recent + 64) else 0
+    per_layer = 2 * cfg.n_kv * cfg.hd * (pb * 0.625 + (n - pb) * 4.0)
+    n_attn = cfg.n_layers // cfg.full_every
+    return per_layer * n_attn
+
+
+def bench_decode(args):
+    from pyre_amd import lib, synth
+    from pyre_amd import modelgen as mg
+    ev = HipEvents()
+    ctx = lib.Context(0)
+    cfg = mg.a3b_config()
+    if args.layers:
+        cfg.n_layers = args.layers
+    t0 = time.perf_counter()
+    layers, globals_, raw = mg.build_device(ctx, cfg, seed=args.seed)
+    ctx.sync()
+    log("synthetic tensors on the device in %.1f s" % (time.perf_counter() - t0)); t0 = time.perf_counter()
+    model = lib.Model(ctx, cfg, layers, globals_)
+    for p in raw:
+        ctx.free(p)
+    log("model resident (re-laid-out) in %.1f s; weight bytes per token %.1f MB" % (time.perf_counter() - t0, model.weight_bytes_per_token / 1e6))
+    n_ctx = args.ctx
+    st = model.new_state(n_ctx + args.steps + args.warmup + 64)
+    g = np.random.Generator(np.random.PCG64(args.seed + 1))
+    prompt = g.integers(0, cfg.vocab, n_ctx, dtype=np.uint32)
+    t0 = time.perf_counter()
+    done = 0
+    while done < n_ctx:                      # prefill in pieces so a long prompt keeps printing progress
+        piece = prompt[done:done + 2048]
+        last = done + piece.size >= n_ctx
+        lg = model.forward(piece, st, want_logits=last)
+        done += piece.size
+        if done % 8192 == 0 or last:
+            log("prefill %d / %d tokens (%.1f s)" % (done, n_ctx, time.perf_counter() - t0))
+    first = int(np.argmax(lg))
+    toks = model.decode_greedy_dev(st, first, args.warmup) if args.warmup else np.array([first], dtype=np.uint32)
+    nxt = int(toks[-1])
+    ctx.sync()
+    e0, e1 = ev.event(), ev.event()
+    n0 = len(st)
+    ev.record(e0, ctx.stream)
+    model.decode_greedy_dev(st, nxt, args.steps, fetch=False)
+    ev.record(e1, ctx.stream)
+    ms = ev.elapsed_ms(e0, e1)
+    ctx.sync()
+    per = ms / args.steps
+    tok_s = 1e3 / per
+    wbytes = model.weight_bytes_per_token
+    n_mid = n0 + args.steps // 2
+    kvb = kv_bytes_per_token(cfg, n_mid)
+    n_lin = cfg.n_layers - cfg.n_layers // cfg.full_every
+    state_b = n_lin * (2 * cfg.lin_nv * cfg.lin_dk * cfg.lin_dv * 4 + 2 * (cfg.conv_k - 1) * cfg.ch * 4)
+    all_b = wbytes + kvb + state_b
+    # second pass: per-kernel-class durations from event pairs around every launch
+    ctx.prof_reset(); ctx.prof_enable(True)
+    pn = min(16, args.steps)
+    model.decode_greedy_dev(st, nxt, pn, fetch=False)
+    prof = ctx.prof_report(); ctx.prof_enable(False)
+    classes = sorted(prof.items(), key=lambda kv: -kv[1][1])
+    tot_ms = sum(v[1] for v in prof.values())
+    breakdown = [{"kernel": k, "launches_per_token": round(v[0] / pn, 2), "us_per_token": round(v[1] / pn * 1e3, 2),
+                  "avg_launch_us": round(v[1] / v[0] * 1e3, 3), "GBps": round(v[2] / (v[1] * 1e-3) / 1e9, 1) if v[1] > 0 else None} for k, v in classes]
+    dom_k, dom = classes[0]
+    dom_gbs = dom[2] / (dom[1] * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s batch-1 (A3B hybrid IQ3_S)", "value": round(tok_s, 2), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[4]: Qwen-Next-style A3B hybrid, %d layers (3 Gated DeltaNet + 1 gated attention per group), 512 experts top-10 + shared, "
+                               "IQ3_S weights (bf16 router), 4 hyper-connection streams, 4-bit KV, greedy decode after a %d-token random prompt" % (cfg.n_layers, n_ctx),
+                   "context": n_ctx, "layers": cfg.n_layers},
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": dom_k, "algorithmic_bytes_per_launch": round(dom[2] / dom[0]), "avg_launch_us": round(dom[1] / dom[0] * 1e3, 3),
+                     "share_of_kernel_time": round(dom[1] / tot_ms, 3)},
+        "token_roofline": {"weight_bytes_per_token": wbytes, "kv_bytes_per_token": round(kvb), "state_bytes_per_token": state_b,
+                           "weights_only": {"GBps": round(wbytes / (per * 1e-3) / 1e9, 1), "frac": round(wbytes / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+                           "all_bytes": {"GBps": round(all_b / (per * 1e-3) / 1e9, 1), "frac": round(all_b / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+                           "kernel_time_us_per_token": round(tot_ms / pn * 1e3, 1)},
+        "kernels": breakdown,
+    }
+    if not args.no_cpu:
+        del model, st
+        out["cpu_baseline"] = cpu_baseline_decode(cfg, args.seed)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gemv")
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv"])
+    ap.add_argument("--ctx", type=int, default=32768, help="prompt length for the decode workload")
+    ap.add_argument("--layers", type=int, default=0, help="debug: fewer layers than the 48 of the configuration")
+    ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the reference path is single-GPU, single-process); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    out = {"gemv": bench_gemv}[args.workload](args)
+    out = {"gemv": bench_gemv, "decode": bench_decode}[args.workload](args)
     print(json.dumps(out))
 
 

@@ -43,6 +43,13 @@ int         pyre_dev_free(pyre_ctx* ctx, void* dev);
 int         pyre_dev_upload(pyre_ctx* ctx, void* dst_dev, const void* src_host, size_t nbytes);
 int         pyre_dev_download(pyre_ctx* ctx, void* dst_host, const void* src_dev, size_t nbytes);
 
+/* Per-kernel-class timing (the reference's PYRE_QN_PROFILE counters, qwen4exp_gguf.rs:2107,2155, measure phases on
+ * the host; here a HIP event pair brackets every launch on the context's stream).  pyre_prof_report returns lines
+ * "<kernel class> <launches> <total ms> <algorithmic bytes>" valid until the next call. */
+int         pyre_prof_enable(pyre_ctx* ctx, int on);
+int         pyre_prof_reset(pyre_ctx* ctx);
+const char* pyre_prof_report(pyre_ctx* ctx);
+
 /* ---- quantized matrix operator --------------------------------------------------------------------------------
  * The drop-in for pyre's quantized-matmul operator: QMat { ty, rows, cols, bytes } + QMat::matmul
  * (src/model/gguf_q.rs:201-242), which is also what the burn-gguf call sites reduce to

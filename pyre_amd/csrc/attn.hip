@@ -94,6 +94,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const 
   if (wbase < n) {
     const int pp = valid ? p : n - 1;
     if (packed) {
+#pragma unroll 2
       for (int b = 0; b < HD / 32; ++b) {
         float bp[G];
 #pragma unroll
@@ -111,6 +112,7 @@ __global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const 
         for (int g = 0; g < G; ++g) s[g] = fmaf(ksc, bp[g], s[g]);
       }
     } else {
+#pragma unroll 16
       for (int dd = 0; dd < HD; ++dd) { float kvl = kv.kf[((size_t)kvh * HD + dd) * cap + pp];
 #pragma unroll
         for (int g = 0; g < G; ++g) s[g] = fmaf(kvl, qs[g][dd], s[g]); }
@@ -148,7 +150,9 @@ __global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const 
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
     const int w32 = lane & 31, hf = lane >> 5;
-    if (wbase < n) for (int it = 0; it < 32; ++it) {
+    if (wbase < n)
+#pragma unroll 4
+    for (int it = 0; it < 32; ++it) {
       int pl = 2 * it + hf, pg = wbase + pl; if (pg >= n) continue;
       uint32_t u = kv.vq[(size_t)pg * (row / 8) + (size_t)kvh * (HD / 8) + w32];
       float vsc = kv.vs[(size_t)pg * (row / 32) + (size_t)kvh * (HD / 32) + (w32 >> 2)];
@@ -167,7 +171,9 @@ __global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const 
     for (int g = 0; g < G; ++g)
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[g][i] = 0.0f;
-    if (wbase < n) for (int pl = 0; pl < 64; ++pl) {
+    if (wbase < n)
+#pragma unroll 4
+    for (int pl = 0; pl < 64; ++pl) {
       int pg = wbase + pl; if (pg >= n) break;
       float4 vv = *(const float4*)(kv.vf + (size_t)pg * row + (size_t)kvh * HD + 4 * lane);
 #pragma unroll
@@ -237,17 +243,19 @@ int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const Att
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
-  hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, w.q); PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, w.q); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
   int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
   if (pbn > *packed_done) {
     size_t thr = (size_t)(pbn - *packed_done) * (a.nkv * a.hd / 32) * 2;
-    hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn); PYRE_CHECK_LAUNCH(ctx);
+    { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn); } PYRE_CHECK_LAUNCH(ctx);
     *packed_done = pbn;
   }
-  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t); break; default: launch_decode<8>(ctx, a, kv, w, start, t); }
+  double kvb = 0; for (int ti = 0; ti < t; ++ti) { double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent); kvb += 2.0 * a.nkv * a.hd * (pb * 0.625 + (n - pb) * 4.0); }
+  { ProfScope ps(ctx, "attn_decode", kvb);
+  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t); break; default: launch_decode<8>(ctx, a, kv, w, start, t); } }
   PYRE_CHECK_LAUNCH(ctx);
-  hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, w.part_o, w.part_ml, w.max_chunks, out); PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

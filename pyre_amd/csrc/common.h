@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <map>
 #include <string>
 #include <vector>
 #include "../../include/pyre_hip.h"
@@ -16,13 +17,26 @@ struct pyre_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   std::string err;
-  // split-K workspace: partial sums [ksplit][t][rows64] and one self-resetting ticket counter per row tile
-  float* ws_partial = nullptr; size_t ws_partial_bytes = 0;
-  uint32_t* ws_ticket = nullptr; size_t ws_ticket_n = 0;
   // staging for host-pointer entry points
   void* stage = nullptr; size_t stage_bytes = 0;
   // expanded codebooks in device memory: iq3s u32[512], iq2xs u64[512]
   uint32_t* d_iq3s = nullptr; uint64_t* d_iq2xs = nullptr;
+  // optional per-kernel-class timing: an event pair around every launch, resolved at pyre_prof_report
+  struct ProfPending { const char* name; double bytes; hipEvent_t a, b; };
+  struct ProfAcc { long count = 0; double ms = 0, bytes = 0; };
+  bool prof_on = false; std::vector<ProfPending> prof_pending; std::map<std::string, ProfAcc> prof_acc; std::vector<hipEvent_t> prof_pool;
+  std::string prof_text;
+};
+
+// Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
+struct ProfScope {
+  pyre_ctx* ctx; hipEvent_t a = nullptr, b = nullptr; const char* name; double bytes;
+  ProfScope(pyre_ctx* c, const char* n, double by) : ctx(c), name(n), bytes(by) {
+    if (!ctx->prof_on) return;
+    auto get = [&]() { hipEvent_t e = nullptr; if (!ctx->prof_pool.empty()) { e = ctx->prof_pool.back(); ctx->prof_pool.pop_back(); } else (void)hipEventCreate(&e); return e; };
+    a = get(); b = get(); (void)hipEventRecord(a, ctx->stream);
+  }
+  ~ProfScope() { if (!a) return; (void)hipEventRecord(b, ctx->stream); ctx->prof_pending.push_back({name, bytes, a, b}); }
 };
 
 extern thread_local std::string g_pyre_create_err;
@@ -32,7 +46,6 @@ int pyre_fail(pyre_ctx* ctx, int code, const char* fmt, ...);
 #define PYRE_CHECK_LAUNCH(ctx) PYRE_HIP(ctx, hipGetLastError())
 
 int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out);          // grow-only device staging buffer
-int pyre_workspace(pyre_ctx* ctx, size_t partial_bytes, size_t tickets);
 
 // ---- device-side matrix view --------------------------------------------------------------------------------------
 // Weights live in "lane = row" planes: rows are grouped in tiles of 64, and for every (tile, unit) the 64 rows'
@@ -53,7 +66,15 @@ struct pyre_qmat {
 
 // launchers implemented in qmat.hip, used by the block / model code
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+// K range split over `ksplit` workgroups per row tile; partial[(ks*t_count + t)*tiles*64 + row] holds the slice sums and
+// the consumer adds them in slice order.
+int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit);
+// t = 1 GEMV that also leaves, per row tile, (bits of the maximum, first row holding it) in best[2*tile], best[2*tile+1].
+int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev);
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev, int n, float* out_dev, int out_stride);
+// Greedy pick from per-tile maxima (first maximum overall) -> id_out[0] (and mirror[0] if given); when m is given the
+// chosen row is dequantized into out_dev in the same launch (the next token's embedding).
+int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev);
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {
@@ -77,7 +98,7 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
-struct HcWork { float* xn; float* o; float* lo; float* gate; };     // [8][hc*d], [8][lr+hc], [8][lr], [8][hc*d]
+struct HcWork { float* xn; float* o; float* lo; float* gate; int ksplit; };     // [8][hc*d], [ksplit][8][tiles*64] slice sums of [down;inject], [8][lr], [8][hc*d]
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // optional combine first (x[ti][s][:] += comb_out[ti][:] * 2*sigmoid(comb_inj[ti][s])), then mixed/inj = hc_mix(x)

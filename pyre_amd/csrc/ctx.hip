@@ -21,20 +21,6 @@ int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out) {
   *out = ctx->stage; return PYRE_OK;
 }
 
-int pyre_workspace(pyre_ctx* ctx, size_t partial_bytes, size_t tickets) {
-  if (partial_bytes > ctx->ws_partial_bytes) {
-    if (ctx->ws_partial) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(ctx->ws_partial)); ctx->ws_partial = nullptr; ctx->ws_partial_bytes = 0; }
-    PYRE_HIP(ctx, hipMalloc((void**)&ctx->ws_partial, partial_bytes)); ctx->ws_partial_bytes = partial_bytes;
-  }
-  if (tickets > ctx->ws_ticket_n) {
-    if (ctx->ws_ticket) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(ctx->ws_ticket)); ctx->ws_ticket = nullptr; ctx->ws_ticket_n = 0; }
-    size_t n = tickets < 4096 ? 4096 : tickets;
-    PYRE_HIP(ctx, hipMalloc((void**)&ctx->ws_ticket, n * sizeof(uint32_t)));
-    PYRE_HIP(ctx, hipMemset(ctx->ws_ticket, 0, n * sizeof(uint32_t))); ctx->ws_ticket_n = n;   // tickets reset themselves after every launch
-  }
-  return PYRE_OK;
-}
-
 // ---- synthetic blocks: pyre_amd/synth.py:blocks() on the device -----------------------------------------------------
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull; z ^= z >> 27; z *= 0x94D049BB133111EBull; z ^= z >> 31; return z;
@@ -87,11 +73,11 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-  if (ctx->ws_partial) (void)hipFree(ctx->ws_partial);
-  if (ctx->ws_ticket) (void)hipFree(ctx->ws_ticket);
   if (ctx->stage) (void)hipFree(ctx->stage);
   if (ctx->d_iq3s) (void)hipFree(ctx->d_iq3s);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
+  for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+  for (auto e : ctx->prof_pool) (void)hipEventDestroy(e);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
 }
@@ -112,6 +98,22 @@ int pyre_dev_upload(pyre_ctx* ctx, void* dst, const void* src, size_t n) {
 int pyre_dev_download(pyre_ctx* ctx, void* dst, const void* src, size_t n) {
   if (!ctx || (!dst && n) || (!src && n)) return pyre_fail(ctx, PYRE_E_ARG, "pyre_dev_download: null pointer");
   PYRE_HIP(ctx, hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
+int pyre_prof_enable(pyre_ctx* ctx, int on) { if (!ctx) return PYRE_E_ARG; ctx->prof_on = on != 0; return PYRE_OK; }
+int pyre_prof_reset(pyre_ctx* ctx) {
+  if (!ctx) return PYRE_E_ARG; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  for (auto& p : ctx->prof_pending) { ctx->prof_pool.push_back(p.a); ctx->prof_pool.push_back(p.b); }
+  ctx->prof_pending.clear(); ctx->prof_acc.clear(); return PYRE_OK;
+}
+const char* pyre_prof_report(pyre_ctx* ctx) {
+  if (!ctx) return "";
+  (void)hipStreamSynchronize(ctx->stream);
+  for (auto& p : ctx->prof_pending) { float ms = 0; if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) { auto& a = ctx->prof_acc[p.name]; a.count++; a.ms += ms; a.bytes += p.bytes; } ctx->prof_pool.push_back(p.a); ctx->prof_pool.push_back(p.b); }
+  ctx->prof_pending.clear();
+  ctx->prof_text.clear(); char line[256];
+  for (auto& kv : ctx->prof_acc) { snprintf(line, sizeof line, "%s %ld %.6f %.0f\n", kv.first.c_str(), kv.second.count, kv.second.ms, kv.second.bytes); ctx->prof_text += line; }
+  return ctx->prof_text.c_str();
 }
 
 int pyre_synth_blocks(pyre_ctx* ctx, uint32_t ty, size_t n_blocks, uint64_t seed, float d_lo, float d_hi, void* dev_out) {

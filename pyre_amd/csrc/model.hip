@@ -27,7 +27,7 @@ struct pyre_model {
   // activations for a window of up to 8 tokens
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
   float *x = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
-  uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0;
+  uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
 };
 
 struct pyre_state {
@@ -45,19 +45,6 @@ __global__ void k_replicate(const float* __restrict__ e, int d, int hc, float* _
   int i = blockIdx.x * blockDim.x + threadIdx.x, s = blockIdx.y, ti = blockIdx.z; if (i >= d) return;
   x[((size_t)ti * hc + s) * d + i] = e[(size_t)ti * d + i];
 }
-// first index of the maximum (sampler::argmax, strict >); one block, result -> out[0] (and mirror, if given)
-__global__ __launch_bounds__(1024) void k_argmax(const float* __restrict__ lg, int n, uint32_t* out, uint32_t* mirror) {
-  __shared__ float bv[1024]; __shared__ int bi[1024];
-  int tid = threadIdx.x; float best = -INFINITY; int idx = n;
-  for (int i = tid; i < n; i += 1024) { float v = lg[i]; if (idx == n || v > best) { best = v; idx = i; } }
-  bv[tid] = best; bi[tid] = idx; __syncthreads();
-  for (int s = 512; s > 0; s >>= 1) {
-    if (tid < s) { float v2 = bv[tid + s]; int i2 = bi[tid + s]; if (i2 < n && (bi[tid] >= n || v2 > bv[tid] || (v2 == bv[tid] && i2 < bi[tid]))) { bv[tid] = v2; bi[tid] = i2; } }
-    __syncthreads();
-  }
-  if (tid == 0) { uint32_t r = (uint32_t)(bi[0] < n ? bi[0] : 0); out[0] = r; if (mirror) mirror[0] = r; }
-}
-
 struct Builder {
   pyre_ctx* ctx; pyre_model* m;
   int fail(int code, const char* what) { return pyre_fail(ctx, code, "pyre_model_create: %s", what); }
@@ -121,7 +108,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   if (!ctx || !cfg || !lt || !gl || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_create: null argument");
   *out = nullptr;
   const pyre_model_cfg& c = *cfg;
-  if (c.n_layers < 1 || c.d < 64 || c.d % 64 || c.hc < 1 || c.hc > 8 || c.hc_lr < 64 || c.hc_lr % 64 || c.full_every < 1 || c.vocab < 1 || c.top_k < 1 || c.n_exp < c.top_k)
+  if (c.n_layers < 1 || c.d < 64 || c.d % 64 || c.hc < 1 || c.hc > 8 || c.hc_lr < 64 || c.hc_lr % 64 || c.full_every < 1 || c.vocab < 1 || c.top_k < 1 || c.top_k > 32 || c.n_exp < c.top_k || c.n_exp > 1024)
     return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_create: unsupported configuration (d and hc_lr must be multiples of 64, hc <= 8)");
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
   std::unique_ptr<pyre_model> M(new pyre_model()); pyre_model* m = M.get(); m->ctx = ctx; m->c = c;
@@ -184,14 +171,14 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
   MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
   m->x = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
-  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16);
+  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   guard.armed = false; *out = M.release(); return PYRE_OK;
 }
@@ -250,12 +237,14 @@ int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, floa
 namespace {
 
 // One window of t <= 8 tokens whose ids already sit in m->ids.  head_tokens: 0 = no logits, 1 = last token only,
-// t = every token (logits rows 0..t-1 of m->logits).
-int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int head_tokens) {
+// t = every token (logits rows 0..t-1 of m->logits).  greedy (t == 1 only): the head GEMV also leaves per-tile maxima in
+// m->best; with from_best the token itself is picked from the previous step's maxima inside the embedding launch and
+// stored to toks_out[0].
+int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int head_tokens, bool greedy = false, bool from_best = false, uint32_t* toks_out = nullptr) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  int rc = pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
-  hipLaunchKernelGGL(k_replicate, dim3((d + 255) / 256, hc, t), dim3(256), 0, ctx->stream, m->emb, d, hc, m->x); PYRE_CHECK_LAUNCH(ctx);
+  int rc = from_best ? pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, toks_out, &m->embd, m->emb) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  { ProfScope ps(ctx, "replicate", 4.0 * t * d * (hc + 1)); hipLaunchKernelGGL(k_replicate, dim3((d + 255) / 256, hc, t), dim3(256), 0, ctx->stream, m->emb, d, hc, m->x); } PYRE_CHECK_LAUNCH(ctx);
   const float* comb_out = nullptr; const float* comb_inj = nullptr;
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
@@ -281,11 +270,13 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int hea
   }
   if (head_tokens >= t) {
     if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
+    if (greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
     return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
   }
   // last token only: fold the pending ffn output into its streams, then the head
   float* xl = m->x + (size_t)(t - 1) * hc * d;
   if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xl, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
+  if (greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }
 
@@ -349,10 +340,8 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
   if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }
   s->last_window = 0;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
-  for (int i = 0; i < n_steps; ++i) {
-    if ((rc = run_window(ctx, m, s, 1, 1))) return rc;
-    hipLaunchKernelGGL(k_argmax, dim3(1), dim3(1024), 0, ctx->stream, m->logits, m->c.vocab, m->ids, m->toks + i); PYRE_CHECK_LAUNCH(ctx);
-  }
+  for (int i = 0; i < n_steps; ++i) if ((rc = run_window(ctx, m, s, 1, 1, true, i > 0, i > 0 ? m->toks + i - 1 : nullptr))) return rc;
+  if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr))) return rc;
   if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
   return PYRE_OK;
 }

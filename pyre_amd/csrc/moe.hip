@@ -4,35 +4,46 @@
 #include "formats.h"
 
 // ---- router: top-k by rank counting (ties -> lower index), softmax over the chosen k in ascending expert id, and the
-// shared-expert gate sigmoid(sh_gate_inp . x).  grid = tokens, 256 threads.
-__global__ __launch_bounds__(256) void k_router_topk(const float* __restrict__ logits, int n_exp, int k, const float* __restrict__ sh_gate_inp,
-                                                     const float* __restrict__ x, int d, int32_t* sel_idx, float* sel_w, float* sg) {
-  extern __shared__ float sm[];                 // n_exp logits, then n_exp flags (as uint32)
-  float* lg = sm; uint32_t* flag = (uint32_t*)(sm + n_exp);
-  __shared__ float red[256];
+// shared-expert gate sigmoid(sh_gate_inp . x).  grid = tokens; one thread per expert (block = n_exp rounded up to 64).
+__global__ __launch_bounds__(1024) void k_router_topk(const float* __restrict__ logits, int n_exp, int k, const float* __restrict__ sh_gate_inp,
+                                                      const float* __restrict__ x, int d, int32_t* sel_idx, float* sel_w, float* sg) {
+  __shared__ float4 lg4[256];                    // up to 1024 logits, padded with -inf
+  __shared__ int wcount[16]; __shared__ float wsum[16];
   __shared__ int32_t s_idx[64]; __shared__ float s_w[64];
-  const int ti = blockIdx.x, tid = threadIdx.x;
-  for (int e = tid; e < n_exp; e += 256) { float v = logits[(size_t)ti * n_exp + e]; lg[e] = isnan(v) ? -INFINITY : v; }   // nan_clean
+  float* lg = (float*)lg4;
+  const int ti = blockIdx.x, e = threadIdx.x, lane = e & 63, wave = e >> 6, nw = blockDim.x >> 6;
+  float v = -INFINITY;
+  if (e < n_exp) { v = logits[(size_t)ti * n_exp + e]; if (isnan(v)) v = -INFINITY; }      // nan_clean
+  lg[e] = v;
+  for (int i = blockDim.x + e; i < 1024; i += blockDim.x) lg[i] = -INFINITY;
   __syncthreads();
-  for (int e = tid; e < n_exp; e += 256) {
-    float v = lg[e]; int rank = 0;
-    for (int j = 0; j < n_exp; ++j) { float u = lg[j]; rank += (u > v || (u == v && j < e)) ? 1 : 0; }
-    flag[e] = rank < k ? 1u : 0u;
+  int rank = 0; const int n4 = (n_exp + 3) >> 2;
+#pragma unroll 8
+  for (int j4 = 0; j4 < n4; ++j4) {
+    float4 u = lg4[j4]; int j = 4 * j4;
+    rank += (u.x > v || (u.x == v && j < e)) ? 1 : 0; rank += (u.y > v || (u.y == v && j + 1 < e)) ? 1 : 0;
+    rank += (u.z > v || (u.z == v && j + 2 < e)) ? 1 : 0; rank += (u.w > v || (u.w == v && j + 3 < e)) ? 1 : 0;
   }
+  const bool sel = e < n_exp && rank < k;
+  const unsigned long long mask = __ballot(sel);
+  if (lane == 0) wcount[wave] = __popcll(mask);
+  // shared-expert gate: all threads stride over d
+  float p = 0.0f; for (int i = e; i < d; i += blockDim.x) p = fmaf(sh_gate_inp[i], x[(size_t)ti * d + i], p);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
+  if (lane == 0) wsum[wave] = p;
   __syncthreads();
-  for (int e = tid; e < n_exp; e += 256) if (flag[e]) { int pos = 0; for (int j = 0; j < e; ++j) pos += flag[j]; s_idx[pos] = e; }
-  // shared-expert gate
-  float p = 0.0f; for (int i = tid; i < d; i += 256) p = fmaf(sh_gate_inp[i], x[(size_t)ti * d + i], p);
-  red[tid] = p; __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) { if (tid < s) red[tid] += red[tid + s]; __syncthreads(); }
-  if (tid == 0) {
-    sg[ti] = 1.0f / (1.0f + expf(-red[0]));
+  if (sel) { int pos = __popcll(mask & ((1ull << lane) - 1ull)); for (int w = 0; w < wave; ++w) pos += wcount[w]; s_idx[pos] = e; }
+  __syncthreads();
+  if (e == 0) {
+    float tot = 0.0f; for (int w = 0; w < nw; ++w) tot += wsum[w];
+    sg[ti] = 1.0f / (1.0f + expf(-tot));
     float mx = -INFINITY; for (int i = 0; i < k; ++i) mx = fmaxf(mx, lg[s_idx[i]]);
     if (!isfinite(mx)) { for (int i = 0; i < k; ++i) s_w[i] = 1.0f / (float)k; }
     else { float sum = 0.0f; for (int i = 0; i < k; ++i) { s_w[i] = expf(lg[s_idx[i]] - mx); sum += s_w[i]; } for (int i = 0; i < k; ++i) s_w[i] = s_w[i] / sum; }
   }
   __syncthreads();
-  if (tid < k) { sel_idx[ti * k + tid] = s_idx[tid]; sel_w[ti * k + tid] = s_w[tid]; }
+  if (e < k) { sel_idx[ti * k + e] = s_idx[e]; sel_w[ti * k + e] = s_w[e]; }
 }
 
 // ---- expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) ----------------------------------------------------
@@ -123,15 +134,20 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc;
-  hipLaunchKernelGGL(k_router_topk, dim3(t), dim3(256), 2 * sizeof(float) * m.n_exp, ctx->stream, w.logits, m.n_exp, m.top_k, m.sh_gate_inp, x, m.d, w.sel_idx, w.sel_w, w.sg);
+  auto mat_bytes = [](const QMatDev& q, double rows) { FmtGeom g = fmt_geom(q.fmt); return rows * (q.cols / g.el) * g.bytes; };
+  { ProfScope ps(ctx, "router_topk", 4.0 * t * (m.n_exp + m.d) + 4.0 * m.d);
+  hipLaunchKernelGGL(k_router_topk, dim3(t), dim3((m.n_exp + 63) / 64 * 64), 0, ctx->stream, w.logits, m.n_exp, m.top_k, m.sh_gate_inp, x, m.d, w.sel_idx, w.sel_w, w.sg); }
   PYRE_CHECK_LAUNCH(ctx);
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint32_t* g3 = ctx->d_iq3s; const uint2* g2 = (const uint2*)ctx->d_iq2xs;
-  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g3, g2));
+  { ProfScope ps(ctx, "moe_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)));
+  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g3, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
-  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g3, g2));
+  { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
+  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g3, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
-  hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y);
+  { ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
+  hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y); }
   PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
@@ -150,7 +166,7 @@ int pyre_moe_create(pyre_ctx* ctx, int top_k, const pyre_qmat* router, const pyr
   if (gate_e->cols != d || up_e->cols != d || up_e->rows != E * ff || down_e->rows != E * d || down_e->cols != ff || sh_gate->cols != d || sh_up->cols != d || sh_up->rows != sf ||
       sh_down->rows != d || sh_down->cols != sf) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_moe_create: inconsistent expert tensor shapes");
   if (ff % 64 || sf % 64 || d % 64) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_moe_create: d, expert and shared widths must be multiples of 64");
-  if (top_k < 1 || top_k > 32 || (size_t)top_k > E || E > 4096) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_create: top_k %d / experts %zu unsupported", top_k, E);
+  if (top_k < 1 || top_k > 32 || (size_t)top_k > E || E > 1024) return pyre_fail(ctx, PYRE_E_ARG, "pyre_moe_create: top_k %d / experts %zu unsupported", top_k, E);
   if (gate_e->dv.fmt != up_e->dv.fmt || sh_gate->dv.fmt != gate_e->dv.fmt || sh_up->dv.fmt != gate_e->dv.fmt || sh_down->dv.fmt != down_e->dv.fmt)
     return pyre_fail(ctx, PYRE_E_TYPE, "pyre_moe_create: gate/up (and shared gate/up) must share one type, down and shared down another");
   pyre_moe* m = new pyre_moe(); m->ctx = ctx;

@@ -72,16 +72,19 @@ template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const
 // ---- dequant-GEMV -----------------------------------------------------------------------------------------------------
 // grid (tiles, ksplit), NW waves.  Wave w of K-slice ks walks units [(ks*NW+w)*upw, +upw).  Lane l owns row tile*64+l:
 // weights come from coalesced per-lane loads, activations from wave-uniform (scalar) loads, so there is no cross-lane
-// reduction at all; the NW partial sums meet in LDS, and when the row's K range is split over several workgroups the
-// last one to finish (ticket counter) adds the slices in slice order - a fixed order, so results are reproducible.
+// reduction at all; the NW partial sums meet in LDS and are added in wave order.
+//   ksplit == 1: y[t*rows + row] = sum.
+//   ksplit  > 1: y is a partial buffer, y[(ks*T + t)*tiles*64 + row] = slice sum; the consumer kernel adds the slices in
+//                slice order (no in-kernel cross-workgroup reduction: a device-scope fence per workgroup costs about a
+//                microsecond of serialized L2 write-back per XCD on this part).
+//   best != nullptr (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 template <int FMT, int T, int NW>
-__global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int ksplit, int upw,
-                                                  float* partial, uint32_t* ticket, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+__global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int upw,
+                                                  uint32_t* __restrict__ best, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
   __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[NW][T][64];
-  __shared__ uint32_t is_last;
-  const int tile = blockIdx.x, ks = blockIdx.y;
+  const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -100,41 +103,45 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
     for (int w = 1; w < NW; ++w) s += red[w][t][l];
     size_t row = (size_t)tile * 64 + l;
     if (ksplit == 1) { if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s; }
-    else partial[((size_t)ks * T + t) * r64 + row] = s;
+    else y[((size_t)ks * T + t) * r64 + row] = s;
+    if (T == 1 && best != nullptr) {       // threads 0..63 = wave 0: first maximum of the tile (sampler::argmax order)
+      float bv = row < (size_t)m.rows ? s : -INFINITY; uint32_t bi = (uint32_t)row;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; } }
+      if (l == 0) { best[2 * tile] = __float_as_uint(bv); best[2 * tile + 1] = bi; }
+    }
   }
-  if (ksplit == 1) return;
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) { uint32_t old = atomicAdd(&ticket[tile], 1u); is_last = (old == (uint32_t)(ksplit - 1)); }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  for (int i = threadIdx.x; i < T * 64; i += NW * 64) {
-    int t = i >> 6, l = i & 63; size_t row = (size_t)tile * 64 + l;
-    float s = partial[(size_t)t * r64 + row];
-    for (int k = 1; k < ksplit; ++k) s += partial[((size_t)k * T + t) * r64 + row];
-    if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s;
-  }
-  if (threadIdx.x == 0) ticket[tile] = 0;   // ready for the next launch on this stream
 }
 
 namespace {
-constexpr int kNW = 4;
 int env_int(const char* n, int dflt) { const char* v = getenv(n); return v && *v ? atoi(v) : dflt; }
 
-template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y) {
-  static const int target_waves = env_int("PYRE_GEMV_WAVES", 4096), max_upw = env_int("PYRE_GEMV_MAX_UPW", 8);
-  long total = (long)m.tiles * m.U;
-  int upw = (int)((total + target_waves - 1) / target_waves); if (upw < 1) upw = 1; if (upw > max_upw) upw = max_upw; if (upw > m.U) upw = m.U;
-  int wpt = (m.U + upw - 1) / upw; int ksplit = (wpt + kNW - 1) / kNW;
-  if (ksplit > 1) { int rc = pyre_workspace(ctx, (size_t)ksplit * T * m.tiles * 64 * sizeof(float), (size_t)m.tiles); if (rc) return rc; }
-  hipLaunchKernelGGL((k_gemv<FMT, T, kNW>), dim3(m.tiles, ksplit), dim3(kNW * 64), 0, ctx->stream, m, x, y, ksplit, upw, ctx->ws_partial, ctx->ws_ticket,
-                     (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, uint32_t* best) {
+  int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
+  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s"};
+  static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
+  FmtGeom g = fmt_geom(FMT);
+  ProfScope ps(ctx, name.c_str(), (double)m.rows * (m.cols / g.el) * g.bytes + 4.0 * T * ((double)m.cols + m.rows));
+  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, best, (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
-template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
-  switch (t) { case 1: return gemv_t<FMT, 1>(ctx, m, x, y); case 2: return gemv_t<FMT, 2>(ctx, m, x, y); case 3: return gemv_t<FMT, 3>(ctx, m, x, y); case 4: return gemv_t<FMT, 4>(ctx, m, x, y);
-    case 5: return gemv_t<FMT, 5>(ctx, m, x, y); case 6: return gemv_t<FMT, 6>(ctx, m, x, y); case 7: return gemv_t<FMT, 7>(ctx, m, x, y); case 8: return gemv_t<FMT, 8>(ctx, m, x, y); }
+// Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
+// fewer when there are so many tiles that the chip is full anyway.
+template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, uint32_t* best) {
+  static const int force = env_int("PYRE_GEMV_NW", 0);
+  int per_wg = (m.U + ksplit - 1) / ksplit;
+  int nw = m.tiles >= 1024 ? 4 : (m.tiles >= 256 ? 8 : 16);
+  while (nw > 1 && nw / 2 >= per_wg) nw /= 2;          // no idle waves
+  if (nw < 4) nw = 4;
+  if (force == 4 || force == 8 || force == 16) nw = force;
+  if (nw == 4) return gemv_launch_nw<FMT, T, 4>(ctx, m, x, y, ksplit, best);
+  if (nw == 8) return gemv_launch_nw<FMT, T, 8>(ctx, m, x, y, ksplit, best);
+  return gemv_launch_nw<FMT, T, 16>(ctx, m, x, y, ksplit, best);
+}
+template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, uint32_t* best) {
+  switch (t) { case 1: return gemv_t<FMT, 1>(ctx, m, x, y, ksplit, best); case 2: return gemv_t<FMT, 2>(ctx, m, x, y, ksplit, best); case 3: return gemv_t<FMT, 3>(ctx, m, x, y, ksplit, best);
+    case 4: return gemv_t<FMT, 4>(ctx, m, x, y, ksplit, best); case 5: return gemv_t<FMT, 5>(ctx, m, x, y, ksplit, best); case 6: return gemv_t<FMT, 6>(ctx, m, x, y, ksplit, best);
+    case 7: return gemv_t<FMT, 7>(ctx, m, x, y, ksplit, best); case 8: return gemv_t<FMT, 8>(ctx, m, x, y, ksplit, best); }
   return pyre_fail(ctx, PYRE_E_ARG, "qmatmul: t = %d outside 1..8", t);
 }
 #define FMT_DISPATCH(fmt, CALL) \
@@ -145,13 +152,51 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
 
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
   int rc = PYRE_OK;
-  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y));
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, nullptr));
   return rc;
+}
+int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* partial, int ksplit) {
+  int rc = PYRE_OK;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, partial, ksplit, nullptr));
+  return rc;
+}
+int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best) {
+  int rc = PYRE_OK;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, 1, y, 1, best));
+  return rc;
+}
+
+// 64 threads per block: every block redoes the (tiny) scan of the per-tile maxima, block 0 publishes the id, and when a
+// matrix is given thread u of block b then dequantizes unit 64*b+u of the chosen row.
+template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* __restrict__ best, int n_tiles, uint32_t* id_out, uint32_t* mirror, QMatDev m, int have_m,
+                                                               const uint32_t* g3, const uint64_t* g2, float* __restrict__ out) {
+  const int tid = threadIdx.x;
+  float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
+  for (int i = tid; i < n_tiles; i += 64) { float v = __uint_as_float(best[2 * i]); uint32_t r = best[2 * i + 1]; if (bi == 0xFFFFFFFFu || v > bv || (v == bv && r < bi)) { bv = v; bi = r; } }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; } }
+  if (bi == 0xFFFFFFFFu) bi = 0;
+  if (blockIdx.x == 0 && tid == 0) { id_out[0] = bi; if (mirror) mirror[0] = bi; }
+  if (!have_m) return;
+  int ku = blockIdx.x * 64 + tid; if (ku >= m.U || bi >= (uint32_t)m.rows) return;
+  float y[64];
+  decode_exact<FMT>(m, g3, g2, (int)(bi >> 6), ku, (int)(bi & 63), y);
+  float* o = out + (size_t)ku * 64;
+  for (int i = 0; i < 64; ++i) o[i] = y[i];
+}
+
+int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out) {
+  ProfScope ps(ctx, "pick_embed", 8.0 * n_tiles);
+  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out); }
+  else { dim3 grid((m->U + 63) / 64);
+    FMT_DISPATCH(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out)); }
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* idx, int n, float* out, int out_stride) {
   if (n <= 0) return PYRE_OK;
   dim3 grid((m.U + 63) / 64, n);
+  ProfScope ps(ctx, "embed_rows", 0.0);
   FMT_DISPATCH(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }

@@ -25,6 +25,9 @@ def _declare(L):
         "pyre_last_error": (C.c_char_p, [vp]),
         "pyre_ctx_sync": (i32, [vp]),
         "pyre_ctx_stream": (vp, [vp]),
+        "pyre_prof_enable": (i32, [vp, i32]),
+        "pyre_prof_reset": (i32, [vp]),
+        "pyre_prof_report": (C.c_char_p, [vp]),
         "pyre_dev_alloc": (i32, [vp, sz, C.POINTER(vp)]),
         "pyre_dev_free": (i32, [vp, vp]),
         "pyre_dev_upload": (i32, [vp, vp, vp, sz]),
@@ -150,6 +153,20 @@ class Context:
 
     def synth_blocks(self, ty, n_blocks, seed, d_lo=1e-3, d_hi=2e-2, dev_out=None):
         self.check(self.L.pyre_synth_blocks(self.h, ty, n_blocks, seed, d_lo, d_hi, C.c_void_p(dev_out)), "synth_blocks")
+
+    def prof_enable(self, on=True):
+        self.check(self.L.pyre_prof_enable(self.h, 1 if on else 0), "prof_enable")
+
+    def prof_reset(self):
+        self.check(self.L.pyre_prof_reset(self.h), "prof_reset")
+
+    def prof_report(self):
+        """{kernel class: (launches, total_ms, algorithmic_bytes)}"""
+        out = {}
+        for line in self.L.pyre_prof_report(self.h).decode().splitlines():
+            name, n, ms, by = line.split()
+            out[name] = (int(n), float(ms), float(by))
+        return out
 
     def close(self):
         if getattr(self, "h", None):

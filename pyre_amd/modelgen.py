@@ -164,3 +164,25 @@ def build_host(c: Config, seed=1):
         b = host_tensor(c, seed, il, slot, kind, ty, rows, cols)
         (hw.layers[il] if il >= 0 else hw.globals_)[slot] = (ty, rows, cols, b)
     return hw
+
+
+def build_device(ctx, c: Config, seed=1):
+    """The same tensors as build_host, with every quantized matrix generated on the device (pyre_synth_blocks is
+    bit-identical to synth.blocks).  Returns (layers, globals, raw_device_buffers); the raw buffers can be freed once
+    the model has been created."""
+    layers = [dict() for _ in range(c.n_layers)]
+    globals_ = {}
+    raw = []
+    for il, slot, kind, ty, rows, cols in tensor_specs(c):
+        if kind == "q" and ty in (synth.Q8_0, synth.Q4_K, synth.IQ2_XS, synth.IQ3_S):
+            el, bs, _ = synth.GEOM[ty]
+            nb = rows * (cols // el)
+            dev = ctx.alloc(nb * bs)
+            lo, hi = scale_range(c, il, slot)
+            ctx.synth_blocks(ty, nb, tensor_seed(seed, il, slot), lo, hi, dev_out=dev)
+            raw.append(dev)
+            entry = (ty, rows, cols, dev)
+        else:
+            entry = (ty, rows, cols, host_tensor(c, seed, il, slot, kind, ty, rows, cols))
+        (layers[il] if il >= 0 else globals_)[slot] = entry
+    return layers, globals_, raw
