@@ -11,8 +11,9 @@ size_t pyre_packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 
 // grid (nkv + nh, t), hd threads.  Blocks 0..nkv-1: key head -> rms_inplace(kn) -> rope -> cache (and the raw value row);
 // blocks nkv..: query head h -> rms_inplace(qn) -> rope -> q scratch.
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, float* __restrict__ qout) {
+__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout) {
   __shared__ float buf[HD]; __shared__ float red[HD / 64];
+  if (posp) start = *posp;
   const int b = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, pos = start + ti;
   const bool is_k = b < a.nkv; const int h = is_k ? b : b - a.nkv;
   const float* row = qkv + (size_t)ti * stride;
@@ -45,8 +46,16 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
 }
 
 // kv4::pack for positions [p0, p1): one thread per (position, 32-value block, K or V).
+// With posp the range is decided on the device: the positions that fall below the packed boundary when the context
+// grows from *posp to *posp + 1 positions (nothing on most steps).
 template <int HD>
-__global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1) {
+__global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1, const int* __restrict__ posp) {
+  if (posp) {
+    int n = *posp + 1;
+    p1 = (a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0;
+    p0 = (a.kv_bits == 4 && n - 1 > a.kv_recent + 64) ? ((n - 1 - a.kv_recent) / 64) * 64 : 0;
+    if (p1 <= p0) return;
+  }
   const int bpr = a.nkv * HD / 32;                 // blocks per cache row
   size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t per = (size_t)(p1 - p0) * bpr;
@@ -73,12 +82,13 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 //  phase 2: chunk-local max / exp / sum per head
 //  phase 3: lane = value dims, unnormalised sum_p e_p V[p]; waves and half-waves are added in a fixed order
 template <int HD, int G>
-__global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+__global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
   __shared__ float qs[G][HD];
   __shared__ float sc[256][G];
   __shared__ float part[4][G][HD];
   __shared__ float wred[4][G], cm[G];
   const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (posp) start = *posp;
   const int n = start + ti + 1;
   if (chunk * 256 >= n) return;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
@@ -199,8 +209,9 @@ __global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const 
 
 // grid (nh, t), HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+__global__ __launch_bounds__(HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                      int max_chunks, float* __restrict__ out) {
+  if (posp) start = *posp;
   const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, n = start + ti + 1, nc = (n + 255) / 256;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
@@ -231,31 +242,33 @@ void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
   w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
 }
 
-template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t) {
-  int n = start + t, chunks = (n + 255) / 256;
-  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256), 0, ctx->stream, a, kv, w.q, start, w.part_o, w.part_ml, w.max_chunks);
+template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp) {
+  int n = start + t, chunks = posp ? w.max_chunks : (n + 255) / 256;      // device-side position: cover the whole cache, surplus workgroups leave at once
+  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
 }
 
-int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out) {
+int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
   if (a.hd != 256) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: head dim %d unsupported (256 only)", a.hd);
   if (a.nkv < 1 || a.nh % a.nkv) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: %d query heads over %d kv heads", a.nh, a.nkv);
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, w.q); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
   int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
-  if (pbn > *packed_done) {
+  if (posp) {   // one 64-position packing step at most; the kernel decides from the device-side position
+    if (a.kv_bits == 4) { size_t thr = (size_t)64 * (a.nkv * a.hd / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, 0, 0, posp); PYRE_CHECK_LAUNCH(ctx); }
+  } else if (pbn > *packed_done) {
     size_t thr = (size_t)(pbn - *packed_done) * (a.nkv * a.hd / 32) * 2;
-    { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn); } PYRE_CHECK_LAUNCH(ctx);
+    { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn, (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
     *packed_done = pbn;
   }
   double kvb = 0; for (int ti = 0; ti < t; ++ti) { double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent); kvb += 2.0 * a.nkv * a.hd * (pb * 0.625 + (n - pb) * 4.0); }
   { ProfScope ps(ctx, "attn_decode", kvb);
-  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t); break; default: launch_decode<8>(ctx, a, kv, w, start, t); } }
+  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp); break; default: launch_decode<8>(ctx, a, kv, w, start, t, posp); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 
@@ -295,7 +308,7 @@ int pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, int
   size_t qw = (size_t)a->dv.nh * 2 * a->dv.hd + 2 * (size_t)a->dv.nkv * a->dv.hd, ow = (size_t)a->dv.nh * a->dv.hd;
   float* qd = a->io; float* od = a->io + 8 * qw;
   PYRE_HIP(ctx, hipMemcpyAsync(qd, qkv_host, (size_t)t * qw * 4, hipMemcpyHostToDevice, ctx->stream));
-  int rc = pyre_attn_launch(ctx, a->dv, a->kv, a->w, qd, (int)qw, a->len, t, &a->packed, od); if (rc) return rc;
+  int rc = pyre_attn_launch(ctx, a->dv, a->kv, a->w, qd, (int)qw, a->len, t, &a->packed, od, nullptr); if (rc) return rc;
   a->len += t;
   PYRE_HIP(ctx, hipMemcpyAsync(out_host, od, (size_t)t * ow * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
@@ -311,7 +324,7 @@ int pyre_attn_load_cache(pyre_ctx* ctx, pyre_attn* a, const float* k_host, const
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   a->len = n; a->packed = 0;
   int pbn = (int)pyre_packed_boundary((size_t)n, a->dv.kv_bits, a->dv.kv_recent);
-  if (pbn > 0) { size_t thr = (size_t)pbn * (row / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a->dv, a->kv, 0, pbn); PYRE_CHECK_LAUNCH(ctx); a->packed = pbn; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+  if (pbn > 0) { size_t thr = (size_t)pbn * (row / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a->dv, a->kv, 0, pbn, (const int*)nullptr); PYRE_CHECK_LAUNCH(ctx); a->packed = pbn; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
   return PYRE_OK;
 }
 int pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_host) {

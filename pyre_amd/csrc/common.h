@@ -74,7 +74,9 @@ int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev,
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev, int n, float* out_dev, int out_stride);
 // Greedy pick from per-tile maxima (first maximum overall) -> id_out[0] (and mirror[0] if given); when m is given the
 // chosen row is dequantized into out_dev in the same launch (the next token's embedding).
-int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev);
+// step_dev (optional, device int[2]): step_dev[0] is incremented first (the position of the token being started) and the
+// id goes to mirror[step_dev[0] - step_dev[1]] instead of mirror[0].
+int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev, int* step_dev);
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {
@@ -131,6 +133,8 @@ size_t pyre_attn_work_bytes(const AttnDev& a, int cap);
 void   pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w);
 // qkv [t][nh*2*hd + 2*nkv*hd] = [q (with interleaved gate) | k | v] raw projections; positions start..start+t-1 are
 // appended; packed_done = number of leading positions already packed (updated by the call). out [t][nh*hd].
+// posp != nullptr: the kernels take the window's first position from *posp (device memory) instead of `start`, so the
+// launch sequence can be replayed from a captured graph; packed_done is then left to the caller.
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
-                     int* packed_done, float* out_dev);
+                     int* packed_done, float* out_dev, const int* posp);
 size_t pyre_packed_boundary(size_t n_visible, int kv_bits, int recent);

@@ -4,6 +4,7 @@
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
 #include <memory>
+#include <stdlib.h>
 
 namespace {
 
@@ -37,6 +38,7 @@ struct pyre_state {
   std::vector<float*> proj_saved;                                // per DeltaNet layer [8][pw_lin]: inputs of the last window
   std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
+  int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
 };
 
 namespace {
@@ -196,17 +198,18 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   size_t cs = al256((size_t)(c.conv_k - 1) * m->ch * 4), ss = al256((size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4), ps = al256((size_t)8 * m->pw_lin * 4);
   AttnDev a0{nullptr, nullptr, nullptr, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
   size_t kvb = al256(pyre_kv_bytes(a0, s->cap)), awb = al256(pyre_attn_work_bytes(a0, s->cap));
-  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * kvb + awb + 4096;
+  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * kvb + awb + 4096 + 256;
   hipError_t e = hipMalloc(&s->mem, total);
   if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_create: hipMalloc(%zu): %s", total, hipGetErrorString(e));
   uint8_t* p = (uint8_t*)s->mem; auto take = [&](size_t n) { void* r = p; p += n; return r; };
   for (int li = 0; li < m->n_lin; ++li) { for (int b = 0; b < 2; ++b) { s->conv[b].push_back((float*)take(cs)); s->ssm[b].push_back((float*)take(ss)); } s->proj_saved.push_back((float*)take(ps)); s->cur.push_back(0); }
   for (int ai = 0; ai < m->n_attn; ++ai) { KvDev kv; pyre_kv_carve(a0, s->cap, take(kvb), &kv); s->kv.push_back(kv); s->packed.push_back(0); }
   pyre_attn_work_carve(a0, s->cap, take(awb), &s->aw);
+  s->step_dev = (int*)take(256);
   int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
   *out = S.release(); return PYRE_OK;
 }
-void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); (void)hipFree(s->mem); delete s; }
+void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec); (void)hipFree(s->mem); delete s; }
 int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
   if (!ctx || !s) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_reset: null argument");
   const pyre_model_cfg& c = s->m->c; size_t cs = (size_t)(c.conv_k - 1) * s->m->ch * 4, ss = (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4;
@@ -236,14 +239,20 @@ int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, floa
 
 namespace {
 
-// One window of t <= 8 tokens whose ids already sit in m->ids.  head_tokens: 0 = no logits, 1 = last token only,
-// t = every token (logits rows 0..t-1 of m->logits).  greedy (t == 1 only): the head GEMV also leaves per-tile maxima in
-// m->best; with from_best the token itself is picked from the previous step's maxima inside the embedding launch and
-// stored to toks_out[0].
-int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int head_tokens, bool greedy = false, bool from_best = false, uint32_t* toks_out = nullptr) {
-  const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len;
+struct WinOpt {
+  int head_tokens = 1;          // 0 = no logits, 1 = last token only, t = every token (rows 0..t-1 of m->logits)
+  bool greedy = false;          // t == 1: the head GEMV also leaves per-tile maxima in m->best
+  bool from_best = false;       // the token is picked from the previous step's maxima inside the embedding launch
+  uint32_t* toks_out = nullptr; // where the picked id is mirrored
+  int* step_dev = nullptr;      // replayable form: position and output slot live in device memory (see pyre_pick_launch);
+                                // recurrent state is updated in place and no host-side bookkeeping is touched
+};
+
+// One window of t <= 8 tokens (ids in m->ids unless from_best).
+int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
+  const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  int rc = from_best ? pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, toks_out, &m->embd, m->emb) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, o.toks_out, &m->embd, m->emb, o.step_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
   { ProfScope ps(ctx, "replicate", 4.0 * t * d * (hc + 1)); hipLaunchKernelGGL(k_replicate, dim3((d + 255) / 256, hc, t), dim3(256), 0, ctx->stream, m->emb, d, hc, m->x); } PYRE_CHECK_LAUNCH(ctx);
   const float* comb_out = nullptr; const float* comb_inj = nullptr;
   for (int il = 0; il < c.n_layers; ++il) {
@@ -252,31 +261,29 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int hea
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
-      if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core))) return rc;
+      if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev))) return rc;
     } else {
-      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li];
+      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = replay ? b : b ^ 1;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, pj))) return rc;
-      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[b ^ 1][li], s->ssm[b][li], s->ssm[b ^ 1][li], m->co, m->core))) return rc;
-      s->cur[li] = b ^ 1;
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core))) return rc;
+      s->cur[li] = nb;
     }
     if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, m->x, t, m->o, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
     if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, m->y))) return rc;
     comb_out = m->y; comb_inj = m->inj_f;
   }
-  s->len = start + t;
-  if (head_tokens == 0) {   // the pending ffn output still has to reach the residual streams of ... nobody: the window's x is dropped
-    return PYRE_OK;
-  }
-  if (head_tokens >= t) {
+  if (!replay) s->len = start + t;
+  if (o.head_tokens == 0) return PYRE_OK;       // prompt window whose logits nobody reads
+  if (o.head_tokens >= t) {
     if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
-    if (greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
+    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
     return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
   }
   // last token only: fold the pending ffn output into its streams, then the head
   float* xl = m->x + (size_t)(t - 1) * hc * d;
   if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xl, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
-  if (greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
+  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }
 
@@ -298,7 +305,8 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
   for (int i = 0; i < n; i += 8) {
     int t = n - i < 8 ? n - i : 8; bool last = i + t >= n;
     PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
-    if ((rc = run_window(ctx, m, s, t, last && logits_host ? 1 : 0))) return rc;
+    WinOpt o; o.head_tokens = last && logits_host ? 1 : 0;
+    if ((rc = run_window(ctx, m, s, t, o))) return rc;
   }
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
@@ -311,7 +319,7 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
-  if ((rc = run_window(ctx, m, s, n, n))) return rc;
+  { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
   s->last_window = n;
   PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)n * m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
@@ -332,16 +340,45 @@ int pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int
   return PYRE_OK;
 }
 
+// The greedy loop on the device.  Step 0 runs eagerly from the host-supplied token; every further step is the same
+// launch sequence with its position and output slot in device memory, captured once per state into a HIP graph and
+// replayed (PYRE_NO_GRAPH=1, or profiling switched on, replays it eagerly instead).
 int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host) {
   pyre_model* m = const_cast<pyre_model*>(mc);
   if (!ctx || !m || !s || n_steps < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_decode_greedy_dev: bad argument");
+  if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_decode_greedy_dev: state belongs to another model");
   if (s->len + n_steps > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_decode_greedy_dev: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, &first, 1); if (rc) return rc;
   if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }
   s->last_window = 0;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
-  for (int i = 0; i < n_steps; ++i) if ((rc = run_window(ctx, m, s, 1, 1, true, i > 0, i > 0 ? m->toks + i - 1 : nullptr))) return rc;
-  if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr))) return rc;
+  { WinOpt o; o.greedy = true; if ((rc = run_window(ctx, m, s, 1, o))) return rc; }
+  if (n_steps > 1) {
+    static const bool no_graph = getenv("PYRE_NO_GRAPH") && atoi(getenv("PYRE_NO_GRAPH")) != 0;
+    int step_host[2] = {s->len - 1, s->len};      // the pick increments [0] to the position it starts; slot = [0] - [1]
+    PYRE_HIP(ctx, hipMemcpyAsync(s->step_dev, step_host, 8, hipMemcpyHostToDevice, ctx->stream));
+    WinOpt o; o.greedy = true; o.from_best = true; o.toks_out = m->toks; o.step_dev = s->step_dev;
+    if (no_graph || ctx->prof_on) {
+      for (int i = 1; i < n_steps; ++i) if ((rc = run_window(ctx, m, s, 1, o))) return rc;
+    } else {
+      if (!s->graph_exec || s->graph_toks != m->toks) {
+        if (s->graph_exec) { (void)hipGraphExecDestroy(s->graph_exec); s->graph_exec = nullptr; }
+        hipGraph_t g = nullptr;
+        PYRE_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+        rc = run_window(ctx, m, s, 1, o);
+        hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+        if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+        if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: stream capture failed: %s", hipGetErrorString(e));
+        e = hipGraphInstantiate(&s->graph_exec, g, nullptr, nullptr, 0); (void)hipGraphDestroy(g);
+        if (e != hipSuccess) { s->graph_exec = nullptr; return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: graph instantiate failed: %s", hipGetErrorString(e)); }
+        s->graph_toks = m->toks;
+      }
+      for (int i = 1; i < n_steps; ++i) PYRE_HIP(ctx, hipGraphLaunch(s->graph_exec, ctx->stream));
+    }
+    s->len += n_steps - 1;
+    for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
+  }
+  if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr, nullptr))) return rc;
   if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
   return PYRE_OK;
 }
