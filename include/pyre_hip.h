@@ -107,6 +107,10 @@ int  pyre_gdn_set_state(pyre_ctx* ctx, pyre_gdn* g, const float* conv_host /*NUL
 int  pyre_gdn_get_state(pyre_ctx* ctx, pyre_gdn* g, float* conv_host, float* ssm_host);
 /* proj [t][ch + nv*dv + 2*nv] = per token [qkv | z | beta | alpha] -> out [t][nv*dv]; tokens run in time order. */
 int  pyre_gdn_step(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int t, float* out_host);
+/* The same recurrence for a prompt of T tokens in chunked form (chunk = 64) on the fp32 matrix cores; the reference has
+ * only the sequential form (linear_core above), which is therefore the oracle.  A remainder T % 64 runs through the
+ * step kernels. */
+int  pyre_gdn_prefill_chunked(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int T, int chunk, float* out_host);
 
 /* ---- gated attention layer core over a 4-bit KV cache --------------------------------------------------------------
  * attn_core, dense branch (qwen4exp_gguf.rs:1558-1615): k RMSNorm + RoPE, append; per head q RMSNorm + RoPE,

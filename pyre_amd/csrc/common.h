@@ -115,6 +115,11 @@ struct GdnDev { const float* a; const float* dt; const float* conv_w; const floa
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
                     const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev);
 
+// Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
+// scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].
+int pyre_gdn_prefill_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int T, const float* conv_in, float* conv_out,
+                            const float* ssm_in, float* ssm_out, float* co, float* logg, float* beta, float* oraw, float* out_dev);
+
 // ---- gated attention over the KV cache (attn.hip) -----------------------------------------------------------------------
 struct AttnDev { const float* qn; const float* kn; const float* rope_inv; int nh, nkv, hd, n_rot, kv_bits, kv_recent; float eps; };
 struct KvDev {

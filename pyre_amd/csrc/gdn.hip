@@ -162,4 +162,31 @@ int pyre_gdn_step(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int t, flo
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
+// Prefill of T tokens: whole chunks of 64 go through the matrix-core chunked form, the remainder through the step kernels.
+int pyre_gdn_prefill_chunked(pyre_ctx* ctx, pyre_gdn* g, const float* proj_host, int T, int chunk, float* out_host) {
+  if (!ctx || !g || !proj_host || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_prefill_chunked: null argument");
+  if (T < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_prefill_chunked: T = %d", T);
+  if (chunk != 64) return pyre_fail(ctx, PYRE_E_ARG, "pyre_gdn_prefill_chunked: chunk size %d unsupported (64 only)", chunk);
+  int rc = gdn_io(ctx, g, T); if (rc) return rc;
+  float* pd = g->io; float* od = g->io + (size_t)T * g->pw; size_t ow = (size_t)g->dv.nv * g->dv.dv;
+  PYRE_HIP(ctx, hipMemcpyAsync(pd, proj_host, (size_t)T * g->pw * 4, hipMemcpyHostToDevice, ctx->stream));
+  int Tc = T / 64 * 64;
+  if (Tc) {
+    float* scr = nullptr; size_t n = (size_t)Tc * ((size_t)g->ch + 2 * g->dv.nv + ow);
+    PYRE_HIP(ctx, hipMalloc((void**)&scr, n * 4));
+    float* co = scr; float* lg = co + (size_t)Tc * g->ch; float* be = lg + (size_t)Tc * g->dv.nv; float* oraw = be + (size_t)Tc * g->dv.nv; int nx = g->cur ^ 1;
+    rc = pyre_gdn_prefill_launch(ctx, g->dv, pd, g->pw, Tc, g->conv[g->cur], g->conv[nx], g->ssm[g->cur], g->ssm[nx], co, lg, be, oraw, od);
+    hipError_t e = hipStreamSynchronize(ctx->stream); (void)hipFree(scr);
+    if (rc) return rc; if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "pyre_gdn_prefill_chunked: %s", hipGetErrorString(e));
+    g->cur = nx;
+  }
+  for (int t0 = Tc; t0 < T; t0 += 8) {
+    int n = T - t0 < 8 ? T - t0 : 8; int nx = g->cur ^ 1;
+    rc = pyre_gdn_launch(ctx, g->dv, pd + (size_t)t0 * g->pw, g->pw, n, g->conv[g->cur], g->conv[nx], g->ssm[g->cur], g->ssm[nx], g->co, od + (size_t)t0 * ow); if (rc) return rc;
+    g->cur = nx;
+  }
+  PYRE_HIP(ctx, hipMemcpyAsync(out_host, od, (size_t)T * ow * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+
 }  // extern "C"

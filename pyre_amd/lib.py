@@ -53,6 +53,7 @@ def _declare(L):
         "pyre_gdn_set_state": (i32, [vp, vp, vp, vp]),
         "pyre_gdn_get_state": (i32, [vp, vp, vp, vp]),
         "pyre_gdn_step": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_gdn_prefill_chunked": (i32, [vp, vp, vp, i32, i32, vp]),
         "pyre_attn_create": (i32, [vp, i32, i32, i32, i32, f32, f32, vp, vp, i32, i32, i32, C.POINTER(vp)]),
         "pyre_attn_destroy": (None, [vp]),
         "pyre_attn_len": (i32, [vp]),
@@ -299,6 +300,13 @@ class Gdn:
         assert proj.shape[1] == self.pw
         out = np.empty((t, self.nv * self.dv), dtype=np.float32)
         self.ctx.check(self.ctx.L.pyre_gdn_step(self.ctx.h, self.h, _ptr(proj), t, _ptr(out)), "gdn_step")
+        return out
+
+    def prefill_chunked(self, qkv, z, beta, alpha, chunk=64):
+        proj = np.ascontiguousarray(np.concatenate([qkv, z, beta, alpha], axis=1), dtype=np.float32)
+        t = proj.shape[0]
+        out = np.empty((t, self.nv * self.dv), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_gdn_prefill_chunked(self.ctx.h, self.h, _ptr(proj), t, chunk, _ptr(out)), "gdn_prefill_chunked")
         return out
 
     def close(self):
