@@ -100,11 +100,14 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
-struct HcWork { float* xn; float* o; float* lo; float* gate; int ksplit; };     // [8][hc*d], [ksplit][8][tiles*64] slice sums of [down;inject], [8][lr], [8][hc*d]
+struct HcWork { float* xn; float* o; };     // [8][hc*d] normalized streams, [<=32][8][tiles*64] slice sums of [down ; inject]
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
-// optional combine first (x[ti][s][:] += comb_out[ti][:] * 2*sigmoid(comb_inj[ti][s])), then mixed/inj = hc_mix(x)
-int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, float* x_dev, int t, const float* comb_out, const float* comb_inj,
+// Streams are read from x_in (element i of stream s of token ti at x_in[ti*in_ts + s*in_ss + i]; in_ss = 0 replicates one
+// row over the streams), the pending residual update is applied first when comb_out is given
+// (x[ti][s][:] += comb_out[ti][:] * 2*sigmoid(comb_inj[ti][s])), and the updated streams go to x_out [t][hc][d], which
+// must not overlap x_in.  mixed [t][d] and inj [t][hc] = hc_mix(updated streams).
+int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj,
                        float eps, float* mixed_dev, float* inj_dev);
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, const float* out_dev, const float* inj_dev);
 

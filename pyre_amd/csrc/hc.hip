@@ -1,49 +1,129 @@
 // Hyper-connection mix / combine around every block: grouped RMSNorm over the hc residual streams, low-rank sigmoid
 // gate, stream mean; residual update.  Follows hc_mix / hc_combine, src/model/qwen4exp_gguf.rs:1357-1388 (f32 branch).
+//
+// One mix is two launches.  k_hc_norm_down folds the pending residual update, the grouped RMSNorm and the
+// [down ; inject] GEMV (K cut into slices, one slice per workgroup); k_hc_up_mix adds the slice sums, applies silu,
+// runs the up GEMV from shared memory and reduces the gated streams to their mean.
 #include "formats.h"
 
 __device__ __forceinline__ float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-__device__ __forceinline__ float block_sum_256(float v, float* red) {
-  int tid = threadIdx.x; red[tid] = v; __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) { if (tid < s) red[tid] += red[tid + s]; __syncthreads(); }
-  float r = red[0]; __syncthreads(); return r;
+// Stream element i of token ti with the pending residual update applied: x + out * w  (:1384-1387), w = 2*sigm(inj).
+__device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, float w, int d, int ti, int s, int i) {
+  float v = x_in[(size_t)ti * in_ts + (size_t)s * in_ss + i];
+  if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
+  return v;
 }
 
-// grid (hc, t), 256 threads: optional residual update x[ti][s][:] += out[ti][:] * 2*sigm(inj[ti][s]), then
-// xn[ti][s][:] = x * rsqrt(mean(x^2) + eps) * norm[s][:]     (rms, :209: (x * s) * w)
-__global__ __launch_bounds__(256) void k_hc_rms(float* __restrict__ x, const float* __restrict__ comb_out, const float* __restrict__ comb_inj, const float* __restrict__ norm,
-                                                int d, int hc, float eps, float* __restrict__ xn) {
-  __shared__ float red[256];
-  const int s = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x;
-  float* xs = x + ((size_t)ti * hc + s) * d;
-  float ss = 0.0f;
-  if (comb_out) {
-    float w = 2.0f * sigm(comb_inj[ti * hc + s]);
-    for (int i = tid; i < d; i += 256) { float v = xs[i] + comb_out[(size_t)ti * d + i] * w; xs[i] = v; ss += v * v; }
-  } else for (int i = tid; i < d; i += 256) { float v = xs[i]; ss += v * v; }
-  float tot = block_sum_256(ss, red);
-  float sc = 1.0f / sqrtf(tot / (float)d + eps);
-  for (int i = tid; i < d; i += 256) xn[((size_t)ti * hc + s) * d + i] = xs[i] * sc * norm[(size_t)s * d + i];
+// grid (row tiles of [down ; inject], K slices), nw waves.  A workgroup owns L = nw*upw*64 columns of one stream s:
+//   1. every workgroup recomputes sum(x_new^2) over the whole stream (d elements per token, tiny) -> scale
+//   2. its L columns of xn = (x_new * scale) * norm go to shared memory; the tile-0 workgroup of the slice also
+//      publishes them (xn) and the updated stream (x_out, never the buffer x_in points into)
+//   3. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
+template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
+    const float* __restrict__ comb_out, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
+    float* __restrict__ part, int upw, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  extern __shared__ __align__(16) float sm[];
+  const int nthr = blockDim.x, nw = nthr >> 6, tid = threadIdx.x, L = nw * upw * 64;
+  float* xs = sm;                         // [T][L]
+  float* red = sm + (size_t)T * L;        // [nw][T][64]
+  float* wsum = red + (size_t)nw * T * 64;   // [nw][T]
+  const int tile = blockIdx.x, ks = blockIdx.y;
+  if constexpr (FMT == FMT_IQ3_S) for (int i = tid; i < 512; i += nthr) lds3[i] = g3[i];
+  if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
+  float w[T], ss[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) { w[t] = comb_out ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
+  for (int i = tid; i < d; i += nthr) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, w[t], d, t, s, i); ss[t] += v * v; }
+  }
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss[t] += __shfl_xor(ss[t], o);
+    if (lane == 0) wsum[wave * T + t] = ss[t];
+  }
+  __syncthreads();
+  float sc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) { float tot = wsum[t]; for (int q = 1; q < nw; ++q) tot += wsum[q * T + t]; sc[t] = 1.0f / sqrtf(tot / (float)d + eps); }
+  for (int j = tid; j < L; j += nthr) {
+    const float nv = norm[(size_t)s * d + i0 + j];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, w[t], d, t, s, i0 + j);
+      float o = v * sc[t] * nv;                                   // rms, :209: (x * s) * w
+      xs[(size_t)t * L + j] = o;
+      if (tile == 0) { size_t k = ((size_t)t * hc + s) * d + i0 + j; xn[k] = o; x_out[k] = v; }
+    }
+  }
+  __syncthreads();
+  float acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; unit_dot<FMT, T>(m, lds3, lds2, tile, ks * nw * upw + lu, lane, xs + lu * 64, L, acc); }
+#pragma unroll
+  for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
+  __syncthreads();
+  const size_t r64 = (size_t)m.tiles * 64;
+  for (int i = tid; i < T * 64; i += nthr) {
+    int t = i >> 6, l = i & 63; float a = red[(size_t)t * 64 + l];
+    for (int q = 1; q < nw; ++q) a += red[((size_t)q * T + t) * 64 + l];
+    part[((size_t)ks * T + t) * r64 + (size_t)tile * 64 + l] = a;
+  }
 }
 
-// o = slice sums of the [down ; inject] GEMV, part[(ks*t + ti)*r64 + i], added in slice order;
-// lo[ti][i] = silu(o[i] / hc) for i < lr ; inj[ti][s] = o[lr + s] / hc (zeros without inject)   (:1376-1378)
-__global__ void k_hc_lo(const float* __restrict__ part, int ksplit, int r64, int lr, int hc, int has_inject, float* __restrict__ lo, float* __restrict__ inj) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x, ti = blockIdx.y, t = gridDim.y;
-  if (i >= lr + hc) return;
-  float o = 0.0f;
-  if (i < lr || has_inject) { o = part[(size_t)ti * r64 + i]; for (int ks = 1; ks < ksplit; ++ks) o += part[((size_t)ks * t + ti) * r64 + i]; }
-  float v = o / (float)hc;
-  if (i < lr) lo[(size_t)ti * lr + i] = v * sigm(v); else inj[ti * hc + (i - lr)] = has_inject ? v : 0.0f;
-}
-
-// mixed[ti][i] = (sum_s xn[ti][s][i] * sigm(gate[ti][s][i])) / hc, s ascending from zero   (:1380)
-__global__ void k_hc_mixed(const float* __restrict__ xn, const float* __restrict__ gate, int d, int hc, float* __restrict__ mixed) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x, ti = blockIdx.y; if (i >= d) return;
-  float m = 0.0f;
-  for (int s = 0; s < hc; ++s) { size_t k = ((size_t)ti * hc + s) * d + i; m += xn[k] * sigm(gate[k]); }
-  mixed[(size_t)ti * d + i] = m / (float)hc;
+// grid (d / 64), hc*U waves (U = lr / 64 units of the up matrix).  Prologue: o = slice sums of [down ; inject] added in
+// slice order; lo = silu(o / hc) for the first lr rows -> shared memory, inj = o[lr + s] / hc (zeros without inject)
+// (:1376-1378).  Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is
+// the sum of its waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc, s ascending from zero (:1380).
+template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, int ksplit, int r64, int lr, int hc, int has_inject,
+    const float* __restrict__ xn, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
+  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  extern __shared__ __align__(16) float sm[];
+  const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6;
+  float* lo = sm;                         // [T][lr]
+  float* red = sm + (size_t)T * lr;       // [nw][T][64]
+  if constexpr (FMT == FMT_IQ3_S) for (int i = tid; i < 512; i += nthr) lds3[i] = g3[i];
+  if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
+  const int n_o = lr + hc;
+  for (int idx = tid; idx < T * n_o; idx += nthr) {
+    int t = idx / n_o, i = idx - t * n_o;
+    float o = 0.0f;
+    if (i < lr || has_inject) {
+      o = part[(size_t)t * r64 + i];
+#pragma unroll 4
+      for (int ks = 1; ks < ksplit; ++ks) o += part[((size_t)ks * T + t) * r64 + i];
+    }
+    float v = o / (float)hc;
+    if (i < lr) lo[t * lr + i] = v * sigm(v);
+    else if (blockIdx.x == 0) inj[t * hc + (i - lr)] = has_inject ? v : 0.0f;
+  }
+  __syncthreads();
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int s = wave / U, ku = wave - s * U;
+  float acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+  unit_dot<FMT, T>(up, lds3, lds2, s * (d >> 6) + blockIdx.x, ku, lane, lo + ku * 64, lr, acc);
+#pragma unroll
+  for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
+  __syncthreads();
+  for (int i = tid; i < T * 64; i += nthr) {
+    int t = i >> 6, l = i & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
+    for (int q = 0; q < hc; ++q) {
+      float g = red[((size_t)(q * U) * T + t) * 64 + l];
+      for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t) * 64 + l];
+      mx += xn[((size_t)t * hc + q) * d + col] * sigm(g);
+    }
+    mixed[(size_t)t * d + col] = mx / (float)hc;
+  }
 }
 
 __global__ void k_hc_combine(float* __restrict__ x, const float* __restrict__ out, const float* __restrict__ inj, int d, int hc) {
@@ -52,24 +132,64 @@ __global__ void k_hc_combine(float* __restrict__ x, const float* __restrict__ ou
   x[((size_t)ti * hc + s) * d + i] += out[(size_t)ti * d + i] * w;
 }
 
-// the [down ; inject] matrix has few rows and a long K: its K range is cut into slices so that about 96 workgroups run
-static int hc_ksplit(const HcDev& h) { int ks = 96 / h.di.tiles; if (ks < 1) ks = 1; if (ks > h.di.U / 4) ks = h.di.U / 4; if (ks < 1) ks = 1; if (ks > 32) ks = 32; return ks; }
-size_t pyre_hc_work_bytes(const HcDev& h) { size_t w = (size_t)h.hc * h.d; return 256 * 4 + 4 * 8 * (2 * w + (size_t)h.lr) + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
-void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
-  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
-  size_t wd = (size_t)h.hc * h.d;
-  w->xn = (float*)take(4 * 8 * wd); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64)); w->lo = (float*)take(4 * 8 * (size_t)h.lr); w->gate = (float*)take(4 * 8 * wd); w->ksplit = 0;
+namespace {
+// Waves per workgroup and units per wave of k_hc_norm_down: a workgroup's columns must lie inside one stream, and at
+// most 32 K slices fit the slice-sum buffer.
+struct DownPlan { int nw, upw, ksplit; };
+DownPlan down_plan(const HcDev& h) {
+  int ud = h.d / 64, nw = 8; while (nw > 1 && ud % nw) nw >>= 1;
+  int upw = 1; while ((h.di.U / (nw * upw)) > 32 && (ud / nw) % (2 * upw) == 0) upw *= 2;
+  return DownPlan{nw, upw, h.di.U / (nw * upw)};
 }
 
-int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, float* x, int t, const float* comb_out, const float* comb_inj, float eps, float* mixed, float* inj) {
+template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out,
+                                               const float* comb_out, const float* comb_inj, float eps) {
+  const int L = p.nw * p.upw * 64; size_t lds = 4 * ((size_t)T * L + (size_t)p.nw * T * 64 + (size_t)p.nw * T);
+  FmtGeom g = fmt_geom(FMT);
+  ProfScope ps(ctx, "hc_norm_down", (double)h.di.rows * (h.di.cols / g.el) * g.bytes + 4.0 * T * h.hc * h.d * 4);
+  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, comb_inj, h.norm, h.d, h.hc, eps,
+                     w.xn, w.o, p.upw, (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, float* mixed, float* inj) {
+  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64);
+  FmtGeom g = fmt_geom(FMT);
+  ProfScope ps(ctx, "hc_up_mix", (double)h.up.rows * (h.up.cols / g.el) * g.bytes + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
+  hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, w.xn, h.d, mixed, inj,
+                     (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+#define HC_T_SWITCH(F, FN, ...) \
+  switch (t) { case 1: return FN<F, 1>(__VA_ARGS__); case 2: return FN<F, 2>(__VA_ARGS__); case 3: return FN<F, 3>(__VA_ARGS__); case 4: return FN<F, 4>(__VA_ARGS__); \
+    case 5: return FN<F, 5>(__VA_ARGS__); case 6: return FN<F, 6>(__VA_ARGS__); case 7: return FN<F, 7>(__VA_ARGS__); default: return FN<F, 8>(__VA_ARGS__); }
+#define HC_FMT_SWITCH(fmt, BODY) \
+  switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; BODY } case FMT_F16: { constexpr int F = FMT_F16; BODY } case FMT_BF16: { constexpr int F = FMT_BF16; BODY } \
+    case FMT_Q8_0: { constexpr int F = FMT_Q8_0; BODY } case FMT_Q4_K: { constexpr int F = FMT_Q4_K; BODY } case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; BODY } \
+    default: { constexpr int F = FMT_IQ3_S; BODY } }
+int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj, float eps) {
+  HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, comb_inj, eps))
+}
+int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, float* mixed, float* inj) {
+  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, mixed, inj))
+}
+}  // namespace
+
+size_t pyre_hc_work_bytes(const HcDev& h) { size_t w = (size_t)h.hc * h.d; return 256 * 3 + 4 * 8 * w + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
+void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
+  w->xn = (float*)take(4 * 8 * (size_t)h.hc * h.d); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
+}
+
+int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj,
+                       float eps, float* mixed, float* inj) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
-  { ProfScope ps(ctx, "hc_rms", 4.0 * t * h.hc * h.d * 3); hipLaunchKernelGGL(k_hc_rms, dim3(h.hc, t), dim3(256), 0, ctx->stream, x, comb_out, comb_inj, h.norm, h.d, h.hc, eps, w.xn); } PYRE_CHECK_LAUNCH(ctx);
-  const int ks = hc_ksplit(h), r64 = ks == 1 ? h.di.rows : h.di.tiles * 64;
-  int rc = pyre_gemv_split_launch(ctx, h.di, w.xn, t, w.o, ks); if (rc) return rc;
-  { ProfScope ps(ctx, "hc_lo", 4.0 * t * (h.lr + h.hc) * (ks + 1)); hipLaunchKernelGGL(k_hc_lo, dim3((h.lr + h.hc + 255) / 256, t), dim3(256), 0, ctx->stream, w.o, ks, r64, h.lr, h.hc, h.has_inject ? 1 : 0, w.lo, inj); } PYRE_CHECK_LAUNCH(ctx);
-  rc = pyre_gemv_launch(ctx, h.up, w.lo, t, w.gate); if (rc) return rc;
-  { ProfScope ps(ctx, "hc_mixed", 4.0 * t * h.d * (2 * h.hc + 1)); hipLaunchKernelGGL(k_hc_mixed, dim3((h.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.xn, w.gate, h.d, h.hc, mixed); } PYRE_CHECK_LAUNCH(ctx);
-  return PYRE_OK;
+  if (x_in == x_out) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: the updated streams must go to another buffer");
+  if (h.d % 64 || h.lr % 64 || h.hc * h.up.U > 16 || h.up.tiles != h.hc * (h.d / 64) || h.di.U != h.hc * (h.d / 64))
+    return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: needs d and the low rank in multiples of 64 and hc * (low rank / 64) <= 16 (d %d, low rank %d, hc %d)", h.d, h.lr, h.hc);
+  DownPlan p = down_plan(h);
+  if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
+  int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_inj, eps); if (rc) return rc;
+  return up_mix(ctx, h, w, p.ksplit, t, mixed, inj);
 }
 
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x, int t, const float* out, const float* inj) {

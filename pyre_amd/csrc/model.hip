@@ -27,7 +27,7 @@ struct pyre_model {
   size_t token_weight_bytes = 0;
   // activations for a window of up to 8 tokens
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
-  float *x = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
+  float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
 };
 
@@ -43,10 +43,6 @@ struct pyre_state {
 
 namespace {
 
-__global__ void k_replicate(const float* __restrict__ e, int d, int hc, float* __restrict__ x) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x, s = blockIdx.y, ti = blockIdx.z; if (i >= d) return;
-  x[((size_t)ti * hc + s) * d + i] = e[(size_t)ti * d + i];
-}
 struct Builder {
   pyre_ctx* ctx; pyre_model* m;
   int fail(int code, const char* what) { return pyre_fail(ctx, code, "pyre_model_create: %s", what); }
@@ -172,12 +168,12 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
   MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
-  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
+  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
                  al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
-  m->x = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
+  m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
@@ -253,11 +249,15 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
   int rc = o.from_best ? pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, o.toks_out, &m->embd, m->emb, o.step_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
-  { ProfScope ps(ctx, "replicate", 4.0 * t * d * (hc + 1)); hipLaunchKernelGGL(k_replicate, dim3((d + 255) / 256, hc, t), dim3(256), 0, ctx->stream, m->emb, d, hc, m->x); } PYRE_CHECK_LAUNCH(ctx);
+  // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
+  // leaves the updated streams in the other
+  const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
+  auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
   const float* comb_out = nullptr; const float* comb_inj = nullptr;
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
+    advance();
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
@@ -269,20 +269,21 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       s->cur[li] = nb;
     }
     if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
-    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, m->x, t, m->o, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
+    advance();
     if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, m->y))) return rc;
     comb_out = m->y; comb_inj = m->inj_f;
   }
   if (!replay) s->len = start + t;
   if (o.head_tokens == 0) return PYRE_OK;       // prompt window whose logits nobody reads
   if (o.head_tokens >= t) {
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, m->x, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
     if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
     return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
   }
   // last token only: fold the pending ffn output into its streams, then the head
-  float* xl = m->x + (size_t)(t - 1) * hc * d;
-  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xl, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
+  const size_t last = (size_t)(t - 1) * hc * d;
+  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
   if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }
