@@ -77,149 +77,216 @@ __global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1, const int* __rest
 
 __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((int)(w << (28 - 4 * i))) >> 28); }   // sign-extended nibble i
 
-// grid (chunks of 256 positions, nkv, t), 256 threads.  One workgroup serves the G query heads that share a KV head.
-//  phase 1: lane = position, scores for the G heads (cache read once per group, coalesced along positions)
-//  phase 2: chunk-local max / exp / sum per head
-//  phase 3: lane = value dims, unnormalised sum_p e_p V[p]; waves and half-waves are added in a fixed order
+// grid (chunks of 256 positions, nkv, t), 1024 threads.  One workgroup serves the G query heads that share a KV head.
+// Wave (pw, dq) owns the 64 positions pw*64.. of the chunk and the 64 head dims dq*64.., so every cache element is read
+// once per workgroup and each wave has all of its loads in flight at once (the step is bound by memory latency, not
+// bandwidth, at decode sizes).
+//  phase 1: lane = position; partial scores over the wave's dims for the G heads (q comes from scalar loads);
+//           the four dim quarters are added in order
+//  phase 2: chunk-local max / exp / sum per head (thread = position x head group)
+//  phase 3: unnormalised sum_p e_p V[p] over the wave's positions for the wave's dims; f32 rows: lane = dim;
+//           4-bit rows: lane = (position mod 8, word), folded over the 8 position groups by a fixed shuffle tree;
+//           the four position quarters are added in order
 template <int HD, int G>
-__global__ __launch_bounds__(256) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
-  __shared__ float qs[G][HD];
+__global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+  static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
+  __shared__ float red[4 * 256 * G];          // phase 1: [dq][position][g];  phase 3: [pw][g][dim]
   __shared__ float sc[256][G];
-  __shared__ float part[4][G][HD];
-  __shared__ float wred[4][G], cm[G];
-  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ float wmax[4][G], wsum[4][G], cm[G];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave & 3, dq = wave >> 2;
   if (posp) start = *posp;
   const int n = start + ti + 1;
   if (chunk * 256 >= n) return;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
   const size_t cap = kv.cap;
-  for (int i = tid; i < G * HD; i += 256) qs[i / HD][i % HD] = qbuf[((size_t)ti * a.nh + (size_t)kvh * G + i / HD) * HD + i % HD];
-  __syncthreads();
-  const int wbase = chunk * 256 + wave * 64, p = wbase + lane;
-  const bool valid = p < n, packed = wbase < pb;
+  const float* __restrict__ qg = qbuf + ((size_t)ti * a.nh + (size_t)kvh * G) * HD + dq * 64;     // wave-uniform reads -> scalar loads
+  const int wbase = chunk * 256 + pw * 64, p = wbase + lane;
+  const bool valid = p < n, packed = wbase < pb, active = wbase < n;
   const float scale = 1.0f / sqrtf((float)HD);
+  constexpr int QB = G >= 8 ? 4 : 8;
   float s[G];
 #pragma unroll
   for (int g = 0; g < G; ++g) s[g] = 0.0f;
-  if (wbase < n) {
+  if (active) {
     const int pp = valid ? p : n - 1;
     if (packed) {
-#pragma unroll 2
-      for (int b = 0; b < HD / 32; ++b) {
+      uint32_t kw[8]; float ksc[2];
+#pragma unroll
+      for (int w = 0; w < 8; ++w) kw[w] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + w) * cap + pp];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) ksc[b] = kv.ks[((size_t)kvh * (HD / 32) + dq * 2 + b) * cap + pp];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
         float bp[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) bp[g] = 0.0f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          uint32_t u = kv.kq[((size_t)kvh * (HD / 8) + b * 4 + w) * cap + pp];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) { float kvl = nib_val(u, i);
+          for (int i = 0; i < 8; ++i) { float kvl = nib_val(kw[b * 4 + w], i);
+            if (i % QB == 0) __builtin_amdgcn_sched_barrier(0);      // q scalars of QB dims at a time
 #pragma unroll
-            for (int g = 0; g < G; ++g) bp[g] = fmaf(kvl, qs[g][b * 32 + w * 8 + i], bp[g]); }
+            for (int g = 0; g < G; ++g) bp[g] = fmaf(kvl, qg[g * HD + b * 32 + w * 8 + i], bp[g]); }
         }
-        float ksc = kv.ks[((size_t)kvh * (HD / 32) + b) * cap + pp];
 #pragma unroll
-        for (int g = 0; g < G; ++g) s[g] = fmaf(ksc, bp[g], s[g]);
+        for (int g = 0; g < G; ++g) s[g] = fmaf(ksc[b], bp[g], s[g]);
       }
+      __builtin_amdgcn_sched_barrier(0);
     } else {
-#pragma unroll 16
-      for (int dd = 0; dd < HD; ++dd) { float kvl = kv.kf[((size_t)kvh * HD + dd) * cap + pp];
+      float kreg[64];
 #pragma unroll
-        for (int g = 0; g < G; ++g) s[g] = fmaf(kvl, qs[g][dd], s[g]); }
+      for (int dd = 0; dd < 64; ++dd) kreg[dd] = kv.kf[((size_t)kvh * HD + dq * 64 + dd) * cap + pp];
+#pragma unroll
+      for (int d8 = 0; d8 < 64; d8 += QB) {     // q scalars of QB dims at a time: the fences keep the scalar loads from piling up
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int dd = d8; dd < d8 + QB; ++dd)
+#pragma unroll
+          for (int g = 0; g < G; ++g) s[g] = fmaf(kreg[dd], qg[g * HD + dd], s[g]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
-  // phase 2
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    s[g] = valid ? s[g] * scale : -INFINITY;
-    float m = s[g];
+  for (int g = 0; g < G; ++g) red[((size_t)dq * 256 + pw * 64 + lane) * G + g] = s[g];
+  __syncthreads();
+  // phase 2: this thread's position is pw*64 + lane, its heads are dq, dq + 4, ...
+  constexpr int GH = (G + 3) / 4;
+  const int pos = pw * 64 + lane;
+  float sv[GH];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if (lane == 0) wred[wave][g] = m;
+  for (int gi = 0; gi < GH; ++gi) {
+    const int g = dq + 4 * gi; sv[gi] = -INFINITY;
+    if (g < G) {
+      float v = ((red[((size_t)0 * 256 + pos) * G + g] + red[((size_t)1 * 256 + pos) * G + g]) + red[((size_t)2 * 256 + pos) * G + g]) + red[((size_t)3 * 256 + pos) * G + g];
+      sv[gi] = valid ? v * scale : -INFINITY;
+      float m = sv[gi];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      if (lane == 0) wmax[pw][g] = m;
+    }
   }
   __syncthreads();
-  if (tid < G) cm[tid] = fmaxf(fmaxf(wred[0][tid], wred[1][tid]), fmaxf(wred[2][tid], wred[3][tid]));
+  if (tid < G) cm[tid] = fmaxf(fmaxf(wmax[0][tid], wmax[1][tid]), fmaxf(wmax[2][tid], wmax[3][tid]));
   __syncthreads();
-  float e[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) { e[g] = valid ? expf(s[g] - cm[g]) : 0.0f; sc[tid][g] = e[g]; }
-  __syncthreads();   // all maxima read, scores of every wave visible
+  for (int gi = 0; gi < GH; ++gi) {
+    const int g = dq + 4 * gi;
+    if (g < G) {
+      float e = valid ? expf(sv[gi] - cm[g]) : 0.0f; sc[pos][g] = e;
+      float l = e;
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float l = e[g];
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
-    if (lane == 0) wred[wave][g] = l;
+      for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+      if (lane == 0) wsum[pw][g] = l;
+    }
   }
+  __syncthreads();   // weights of every position visible; the score partials in `red` are dead
   // phase 3
   const int row = a.nkv * HD;
   if (packed) {
-    float acc[G][8];
+    const int psub = lane >> 3, w8 = lane & 7;
+    uint32_t vw[8]; float vsc[8];              // packed positions lie below the boundary, hence inside the view
 #pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
-    const int w32 = lane & 31, hf = lane >> 5;
-    if (wbase < n)
-#pragma unroll 4
-    for (int it = 0; it < 32; ++it) {
-      int pl = 2 * it + hf, pg = wbase + pl; if (pg >= n) continue;
-      uint32_t u = kv.vq[(size_t)pg * (row / 8) + (size_t)kvh * (HD / 8) + w32];
-      float vsc = kv.vs[(size_t)pg * (row / 32) + (size_t)kvh * (HD / 32) + (w32 >> 2)];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) { float vv = nib_val(u, i) * vsc;
-#pragma unroll
-        for (int g = 0; g < G; ++g) acc[g][i] = fmaf(sc[wave * 64 + pl][g], vv, acc[g][i]); }
+    for (int it = 0; it < 8; ++it) {
+      const size_t pg = (size_t)wbase + it * 8 + psub;
+      vw[it] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + w8];
+      vsc[it] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (w8 >> 2)];
     }
+    constexpr int HG = G > 4 ? 4 : G;          // heads per pass (bounds the accumulator registers)
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g0 = 0; g0 < G; g0 += HG) {
+      float acc[HG][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) { float o = acc[g][i] + __shfl_xor(acc[g][i], 32); if (hf == 0) part[wave][g][w32 * 8 + i] = o; }
+      for (int g = 0; g < HG; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        __builtin_amdgcn_sched_barrier(0);
+        const int pl = it * 8 + psub;
+        float wg[HG];
+#pragma unroll
+        for (int g = 0; g < HG; ++g) wg[g] = sc[pw * 64 + pl][g0 + g];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { float vv = nib_val(vw[it], i) * vsc[it];
+#pragma unroll
+          for (int g = 0; g < HG; ++g) acc[g][i] = fmaf(wg[g], vv, acc[g][i]); }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int g = 0; g < HG; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float o = acc[g][i]; o += __shfl_xor(o, 8); o += __shfl_xor(o, 16); o += __shfl_xor(o, 32);
+          if (psub == 0) red[((size_t)pw * G + g0 + g) * HD + dq * 64 + w8 * 8 + i] = o;
+        }
+    }
   } else {
-    float acc[G][4];
+    float acc[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) acc[g] = 0.0f;
+    if (active) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[g][i] = 0.0f;
-    if (wbase < n)
-#pragma unroll 4
-    for (int pl = 0; pl < 64; ++pl) {
-      int pg = wbase + pl; if (pg >= n) break;
-      float4 vv = *(const float4*)(kv.vf + (size_t)pg * row + (size_t)kvh * HD + 4 * lane);
+      for (int hf = 0; hf < 2; ++hf) {          // positions past the view carry weight zero; their address is clamped
+        float vreg[32];
 #pragma unroll
-      for (int g = 0; g < G; ++g) { float wgt = sc[wave * 64 + pl][g]; acc[g][0] = fmaf(wgt, vv.x, acc[g][0]); acc[g][1] = fmaf(wgt, vv.y, acc[g][1]); acc[g][2] = fmaf(wgt, vv.z, acc[g][2]); acc[g][3] = fmaf(wgt, vv.w, acc[g][3]); }
+        for (int j = 0; j < 32; ++j) { const int pg = min(wbase + hf * 32 + j, n - 1); vreg[j] = kv.vf[(size_t)pg * row + (size_t)kvh * HD + dq * 64 + lane]; }
+#pragma unroll
+        for (int j8 = 0; j8 < 32; j8 += 8) {
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = j8; j < j8 + 8; ++j)
+#pragma unroll
+            for (int g = 0; g < G; ++g) acc[g] = fmaf(sc[pw * 64 + hf * 32 + j][g], vreg[j], acc[g]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 #pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) part[wave][g][4 * lane + i] = acc[g][i];
+    for (int g = 0; g < G; ++g) red[((size_t)pw * G + g) * HD + dq * 64 + lane] = acc[g];
   }
   __syncthreads();
-  for (int i = tid; i < G * HD; i += 256) {
+  for (int i = tid; i < G * HD; i += 1024) {
     int g = i / HD, dd = i % HD;
-    float o = ((part[0][g][dd] + part[1][g][dd]) + part[2][g][dd]) + part[3][g][dd];
+    float o = ((red[((size_t)0 * G + g) * HD + dd] + red[((size_t)1 * G + g) * HD + dd]) + red[((size_t)2 * G + g) * HD + dd]) + red[((size_t)3 * G + g) * HD + dd];
     part_o[(((size_t)ti * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
   }
   if (tid < G) {
-    float l = ((wred[0][tid] + wred[1][tid]) + wred[2][tid]) + wred[3][tid];
+    float l = ((wsum[0][tid] + wsum[1][tid]) + wsum[2][tid]) + wsum[3][tid];
     float* ml = part_ml + (((size_t)ti * a.nh + (size_t)kvh * G + tid) * max_chunks + chunk) * 2;
     ml[0] = cm[tid]; ml[1] = l;
   }
 }
 
-// grid (nh, t), HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
+// grid (nh, t), 4*HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
+// Thread (grp, dim) adds the chunks grp, grp+4, ... in ascending order; the four groups are then added in order.
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                     int max_chunks, float* __restrict__ out) {
+__global__ __launch_bounds__(4 * HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                         int max_chunks, float* __restrict__ out) {
+  __shared__ float wmax[4 * HD / 64]; __shared__ float so[4][HD]; __shared__ float sl[4];
   if (posp) start = *posp;
-  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, n = start + ti + 1, nc = (n + 255) / 256;
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD, n = start + ti + 1, nc = (n + 255) / 256;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
-  float M = -INFINITY; for (int c = 0; c < nc; ++c) M = fmaxf(M, ml[2 * c]);
+  float M = -INFINITY; for (int c = tid; c < nc; c += 4 * HD) M = fmaxf(M, ml[2 * c]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  if ((tid & 63) == 0) wmax[tid >> 6] = M;
+  __syncthreads();
+  M = wmax[0];
+#pragma unroll
+  for (int i = 1; i < 4 * HD / 64; ++i) M = fmaxf(M, wmax[i]);
   float L = 0.0f, o = 0.0f;
-  for (int c = 0; c < nc; ++c) { float f = expf(ml[2 * c] - M); L = fmaf(ml[2 * c + 1], f, L); o = fmaf(po[(size_t)c * HD + tid], f, o); }
-  float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + tid];
-  out[((size_t)ti * a.nh + h) * HD + tid] = (o / L) * a_sigm(gate);
+#pragma unroll 4
+  for (int c = grp; c < nc; c += 4) { float f = expf(ml[2 * c] - M); L = fmaf(ml[2 * c + 1], f, L); o = fmaf(po[(size_t)c * HD + dd], f, o); }
+  so[grp][dd] = o; if (dd == 0) sl[grp] = L;
+  __syncthreads();
+  if (grp == 0) {
+    o = ((so[0][dd] + so[1][dd]) + so[2][dd]) + so[3][dd]; L = ((sl[0] + sl[1]) + sl[2]) + sl[3];
+    float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd];
+    out[((size_t)ti * a.nh + h) * HD + dd] = (o / L) * a_sigm(gate);
+  }
 }
 
 size_t pyre_kv_bytes(const AttnDev& a, int cap) {
@@ -244,7 +311,7 @@ void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
 
 template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp) {
   int n = start + t, chunks = posp ? w.max_chunks : (n + 255) / 256;      // device-side position: cover the whole cache, surplus workgroups leave at once
-  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
+  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(1024), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
 }
 
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
@@ -268,7 +335,7 @@ int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const Att
   { ProfScope ps(ctx, "attn_decode", kvb);
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp); break; default: launch_decode<8>(ctx, a, kv, w, start, t, posp); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

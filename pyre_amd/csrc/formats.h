@@ -14,7 +14,7 @@ __host__ __device__ inline FmtGeom fmt_geom(int fmt) {
     case FMT_Q8_0:   return {32, 34, 4, 4, 0, 0, 0};     // p1: the two f16 scales of the unit's two blocks
     case FMT_Q4_K:   return {256, 144, 2, 0, 0, 0, 16};  // pb: d, dmin, scales[12]
     case FMT_IQ2_XS: return {256, 74, 1, 2, 0, 0, 2};    // p1: two scale bytes; pb: d
-    default:         return {256, 110, 1, 8, 2, 1, 2};   // IQ3_S  p1: signs, p2: qh pair, p3: scale byte; pb: d
+    default:         return {256, 110, 2, 0, 0, 1, 2};   // IQ3_S, re-coded at load: p0: 64 four-bit codes, p3: scale byte; pb: d
   }
 }
 inline int fmt_from_ggml(uint32_t ty) {
@@ -44,9 +44,14 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t a, uint32_t b, uint
   else { s = (k4_byte(a, b, c, j + 4) & 0xF) | ((k4_byte(a, b, c, j - 4) >> 6) << 4); m = (k4_byte(a, b, c, j + 4) >> 4) | ((k4_byte(a, b, c, j) >> 6) << 4); }
 }
 
+// IQ3_S values are sign * grid with grid in {1, 3, .., 15}: sixteen odd integers -15..15.  At load each value w is
+// re-coded as the 4-bit number (w + 15) / 2 (code c of value j of a unit sits in bits 4*(j%8).. of word j/8), which
+// decodes without the codebook: w = 2c - 15.
+__host__ __device__ inline uint32_t iq3s_code(uint32_t grid_byte, uint32_t neg) { int w = neg ? -(int)grid_byte : (int)grid_byte; return (uint32_t)((w + 15) >> 1); }
+
 // ---- bit-exact decode of one unit (64 consecutive values of one row) -----------------------------------------------
 // Same operations in the same order as gguf_q::dequant; compiled with -ffp-contract=off so nothing is fused.
-template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const uint32_t* g3, const uint64_t* g2, int tile, int ku, int lane, float* y) {
+template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const uint64_t* g2, int tile, int ku, int lane, float* y) {
   if constexpr (FMT == FMT_F32) {
     for (int c = 0; c < 16; ++c) { uint4 v = ld_vec<16>(m, tile, ku, c, lane); y[4 * c] = __uint_as_float(v.x); y[4 * c + 1] = __uint_as_float(v.y); y[4 * c + 2] = __uint_as_float(v.z); y[4 * c + 3] = __uint_as_float(v.w); }
   } else if constexpr (FMT == FMT_F16 || FMT == FMT_BF16) {
@@ -83,19 +88,13 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
         for (int jj = 0; jj < 8; ++jj) y[32 * ib + 8 * l + jj] = flip(db * (float)(uint32_t)((g >> (8 * jj)) & 0xFF), (sg >> jj) & 1);
       }
     }
-  } else {                                         // IQ3_S, gguf_q.rs:141-151
+  } else {                                         // IQ3_S, gguf_q.rs:141-151, from the 4-bit codes (see iq3s_code)
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
-    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t q[4] = {v.x, v.y, v.z, v.w};
-    uint2 sv = ld_small<uint2>(m.p1, m, tile, ku, lane); uint32_t sg[2] = {sv.x, sv.y};
-    uint32_t qh = ld_small<uint16_t>(m.p2, m, tile, ku, lane), sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
-    for (int sb = 0; sb < 2; ++sb) {
-      float db = d * (float)(1 + 2 * ((sc >> (4 * sb)) & 0xF)); uint32_t h = (qh >> (8 * sb)) & 0xFF;
-      for (int l = 0; l < 4; ++l) {
-        uint32_t qq = q[2 * sb + (l >> 1)] >> (16 * (l & 1));
-        uint32_t gA = g3[(qq & 0xFF) | ((h << (8 - 2 * l)) & 256)], gB = g3[((qq >> 8) & 0xFF) | ((h << (7 - 2 * l)) & 256)];
-        uint32_t s = (sg[sb] >> (8 * l)) & 0xFF;
-        for (int jj = 0; jj < 4; ++jj) { y[32 * sb + 8 * l + jj] = flip(db * (float)((gA >> (8 * jj)) & 0xFF), (s >> jj) & 1); y[32 * sb + 8 * l + 4 + jj] = flip(db * (float)((gB >> (8 * jj)) & 0xFF), (s >> (4 + jj)) & 1); }
-      }
+    uint32_t sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
+    for (int c = 0; c < 2; ++c) {
+      float db = d * (float)(1 + 2 * ((sc >> (4 * c)) & 0xF));
+      uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int j = 0; j < 32; ++j) { int sv = 2 * (int)((w[j >> 3] >> (4 * (j & 7))) & 0xF) - 15; y[32 * c + j] = flip(db * (float)(sv < 0 ? -sv : sv), sv < 0 ? 1u : 0u); }
     }
   }
 }
@@ -103,7 +102,7 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
 // ---- factored per-unit dot products for the GEMV ------------------------------------------------------------------
 // xs points at the unit's 64 activations of token 0 (wave-uniform address -> scalar loads); token t is xs + t*xstride.
 // acc[t] += sum_j W[row, 64*ku + j] * x[t][64*ku + j].  The operation sequence per token does not depend on T.
-template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint32_t* lds3, const uint2* lds2, int tile, int ku, int lane,
+template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint2* lds2, int tile, int ku, int lane,
                                                                    const float* __restrict__ xs, int xstride, float (&acc)[T]) {
   if constexpr (FMT == FMT_F32) {
 #pragma unroll
@@ -184,30 +183,35 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
         for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
       }
     }
-  } else {   // IQ3_S
+  } else {   // IQ3_S from 4-bit codes c = (w + 15) / 2: sum w x = 2 sum c x - 15 sum x per 32-value sub-block
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
-    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t q[4] = {v.x, v.y, v.z, v.w};
-    uint2 sv = ld_small<uint2>(m.p1, m, tile, ku, lane); uint32_t sg[2] = {sv.x, sv.y};
-    uint32_t qh = ld_small<uint16_t>(m.p2, m, tile, ku, lane), sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
+    uint32_t sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
+    uint4 v0 = ld_vec<2>(m, tile, ku, 0, lane), v1 = ld_vec<2>(m, tile, ku, 1, lane);
+    uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+    float sx[T][2];            // sub-block sums of the activations: lane j holds x[j], folded inside each half of the wave
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float xv = xs[t * xstride + lane];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) xv += __shfl_xor(xv, o);
+      sx[t][0] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), 0)); sx[t][1] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), 32));
+    }
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
-      uint32_t h = (qh >> (8 * sb)) & 0xFF;
       float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
-      for (int l = 0; l < 4; ++l) {
-        uint32_t qq = q[2 * sb + (l >> 1)] >> (16 * (l & 1));
-        uint32_t gA = lds3[(qq & 0xFF) | ((h << (8 - 2 * l)) & 256)], gB = lds3[((qq >> 8) & 0xFF) | ((h << (7 - 2 * l)) & 256)];
+      for (int k = 0; k < 4; ++k) {
+        uint32_t u = w[4 * sb + k], lo = u & 0x0F0F0F0Fu, hi = (u >> 4) & 0x0F0F0F0Fu;
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-          uint32_t gw = jj < 4 ? gA : gB; int bit = 8 * l + jj;
-          float f = __uint_as_float(__float_as_uint((float)((gw >> (8 * (jj & 3))) & 0xFF)) | ((sg[sb] << (31 - bit)) & 0x80000000u));
+        for (int b = 0; b < 4; ++b) {
+          float fl = (float)((lo >> (8 * b)) & 0xFF), fh = (float)((hi >> (8 * b)) & 0xFF);
 #pragma unroll
-          for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 32 * sb + 8 * l + jj], part[t]);
+          for (int t = 0; t < T; ++t) { part[t] = fmaf(fl, xs[t * xstride + 32 * sb + 8 * k + 2 * b], part[t]); part[t] = fmaf(fh, xs[t * xstride + 32 * sb + 8 * k + 2 * b + 1], part[t]); }
         }
       }
       float db = d * (float)(1 + 2 * ((sc >> (4 * sb)) & 0xF));
 #pragma unroll
-      for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(db, fmaf(-15.0f, sx[t][sb], 2.0f * part[t]), acc[t]);
     }
   }
 }

@@ -22,8 +22,7 @@ __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in
 //   3. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
 template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
     const float* __restrict__ comb_out, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
-    float* __restrict__ part, int upw, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
-  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+    float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, nw = nthr >> 6, tid = threadIdx.x, L = nw * upw * 64;
@@ -31,7 +30,6 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   float* red = sm + (size_t)T * L;        // [nw][T][64]
   float* wsum = red + (size_t)nw * T * 64;   // [nw][T]
   const int tile = blockIdx.x, ks = blockIdx.y;
-  if constexpr (FMT == FMT_IQ3_S) for (int i = tid; i < 512; i += nthr) lds3[i] = g3[i];
   if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
@@ -66,7 +64,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; unit_dot<FMT, T>(m, lds3, lds2, tile, ks * nw * upw + lu, lane, xs + lu * 64, L, acc); }
+  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; unit_dot<FMT, T>(m, lds2, tile, ks * nw * upw + lu, lane, xs + lu * 64, L, acc); }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
@@ -83,14 +81,12 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 // (:1376-1378).  Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is
 // the sum of its waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc, s ascending from zero (:1380).
 template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, int ksplit, int r64, int lr, int hc, int has_inject,
-    const float* __restrict__ xn, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
-  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+    const float* __restrict__ xn, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6;
   float* lo = sm;                         // [T][lr]
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
-  if constexpr (FMT == FMT_IQ3_S) for (int i = tid; i < 512; i += nthr) lds3[i] = g3[i];
   if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int n_o = lr + hc;
   for (int idx = tid; idx < T * n_o; idx += nthr) {
@@ -111,7 +107,7 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  unit_dot<FMT, T>(up, lds3, lds2, s * (d >> 6) + blockIdx.x, ku, lane, lo + ku * 64, lr, acc);
+  unit_dot<FMT, T>(up, lds2, s * (d >> 6) + blockIdx.x, ku, lane, lo + ku * 64, lr, acc);
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
@@ -148,7 +144,7 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
   FmtGeom g = fmt_geom(FMT);
   ProfScope ps(ctx, "hc_norm_down", (double)h.di.rows * (h.di.cols / g.el) * g.bytes + 4.0 * T * h.hc * h.d * 4);
   hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, comb_inj, h.norm, h.d, h.hc, eps,
-                     w.xn, w.o, p.upw, (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+                     w.xn, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, float* mixed, float* inj) {
@@ -156,7 +152,7 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
   FmtGeom g = fmt_geom(FMT);
   ProfScope ps(ctx, "hc_up_mix", (double)h.up.rows * (h.up.cols / g.el) * g.bytes + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
   hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, w.xn, h.d, mixed, inj,
-                     (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+                     (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 #define HC_T_SWITCH(F, FN, ...) \

@@ -3,62 +3,63 @@
 // and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
 #include "formats.h"
 
-// ---- router: top-k by rank counting (ties -> lower index), softmax over the chosen k in ascending expert id, and the
-// shared-expert gate sigmoid(sh_gate_inp . x).  grid = tokens; one thread per expert (block = n_exp rounded up to 64).
+// ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id, and the shared-expert
+// gate sigmoid(sh_gate_inp . x).  grid = tokens; one thread per expert (block = n_exp rounded up to 64).
+// Two-level selection: every wave ranks its own 64 logits through lane broadcasts and keeps its best k as candidates
+// (an expert outside its wave's best k cannot be in the global best k); the nw*k candidates are then ranked against
+// each other from shared memory.
 __global__ __launch_bounds__(1024) void k_router_topk(const float* __restrict__ logits, int n_exp, int k, const float* __restrict__ sh_gate_inp,
                                                       const float* __restrict__ x, int d, int32_t* sel_idx, float* sel_w, float* sg) {
-  __shared__ float4 lg4[256];                    // up to 1024 logits, padded with -inf
-  __shared__ int wcount[16]; __shared__ float wsum[16];
-  __shared__ int32_t s_idx[64]; __shared__ float s_w[64];
-  float* lg = (float*)lg4;
+  __shared__ float c_val[16 * 32]; __shared__ int c_idx[16 * 32];     // candidates [wave][local rank]
+  __shared__ float r_val[32]; __shared__ int r_idx[32];               // the k winners by value rank
+  __shared__ float s_val[32]; __shared__ int s_idx[32]; __shared__ float s_w[32];   // ... by ascending expert id
+  __shared__ float wsum[16];
   const int ti = blockIdx.x, e = threadIdx.x, lane = e & 63, wave = e >> 6, nw = blockDim.x >> 6;
   float v = -INFINITY;
   if (e < n_exp) { v = logits[(size_t)ti * n_exp + e]; if (isnan(v)) v = -INFINITY; }      // nan_clean
-  lg[e] = v;
-  for (int i = blockDim.x + e; i < 1024; i += blockDim.x) lg[i] = -INFINITY;
-  __syncthreads();
-  int rank = 0; const int n4 = (n_exp + 3) >> 2;
-#pragma unroll 8
-  for (int j4 = 0; j4 < n4; ++j4) {
-    float4 u = lg4[j4]; int j = 4 * j4;
-    rank += (u.x > v || (u.x == v && j < e)) ? 1 : 0; rank += (u.y > v || (u.y == v && j + 1 < e)) ? 1 : 0;
-    rank += (u.z > v || (u.z == v && j + 2 < e)) ? 1 : 0; rank += (u.w > v || (u.w == v && j + 3 < e)) ? 1 : 0;
-  }
-  const bool sel = e < n_exp && rank < k;
-  const unsigned long long mask = __ballot(sel);
-  if (lane == 0) wcount[wave] = __popcll(mask);
+  int lr = 0;
+#pragma unroll
+  for (int j = 0; j < 64; ++j) { float u = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); lr += (u > v || (u == v && j < lane)) ? 1 : 0; }
+  if (lr < k) { c_val[wave * k + lr] = v; c_idx[wave * k + lr] = e; }
   // shared-expert gate: all threads stride over d
   float p = 0.0f; for (int i = e; i < d; i += blockDim.x) p = fmaf(sh_gate_inp[i], x[(size_t)ti * d + i], p);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
   if (lane == 0) wsum[wave] = p;
   __syncthreads();
-  if (sel) { int pos = __popcll(mask & ((1ull << lane) - 1ull)); for (int w = 0; w < wave; ++w) pos += wcount[w]; s_idx[pos] = e; }
-  __syncthreads();
-  if (e == 0) {
-    float tot = 0.0f; for (int w = 0; w < nw; ++w) tot += wsum[w];
-    sg[ti] = 1.0f / (1.0f + expf(-tot));
-    float mx = -INFINITY; for (int i = 0; i < k; ++i) mx = fmaxf(mx, lg[s_idx[i]]);
-    if (!isfinite(mx)) { for (int i = 0; i < k; ++i) s_w[i] = 1.0f / (float)k; }
-    else { float sum = 0.0f; for (int i = 0; i < k; ++i) { s_w[i] = expf(lg[s_idx[i]] - mx); sum += s_w[i]; } for (int i = 0; i < k; ++i) s_w[i] = s_w[i] / sum; }
+  const int nc = nw * k;
+  if (e < nc) {
+    float cv = c_val[e]; int ci = c_idx[e], rank = 0;
+#pragma unroll 16
+    for (int j = 0; j < nc; ++j) { float u = c_val[j]; int ui = c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
+    if (rank < k) { r_val[rank] = cv; r_idx[rank] = ci; }
   }
   __syncthreads();
-  if (e < k) { sel_idx[ti * k + e] = s_idx[e]; sel_w[ti * k + e] = s_w[e]; }
+  if (e < k) { int me = r_idx[e], pos = 0; for (int j = 0; j < k; ++j) pos += r_idx[j] < me ? 1 : 0; s_idx[pos] = me; s_val[pos] = r_val[e]; }
+  __syncthreads();
+  float mx = -INFINITY;
+  if (e < k) { for (int i = 0; i < k; ++i) mx = fmaxf(mx, s_val[i]); s_w[e] = isfinite(mx) ? expf(s_val[e] - mx) : 1.0f; }
+  __syncthreads();
+  if (e < k) {
+    float w;
+    if (!isfinite(mx)) w = 1.0f / (float)k;
+    else { float sum = 0.0f; for (int i = 0; i < k; ++i) sum += s_w[i]; w = s_w[e] / sum; }
+    sel_idx[ti * k + e] = s_idx[e]; sel_w[ti * k + e] = w;
+  }
+  if (e == 0) { float tot = 0.0f; for (int w = 0; w < nw; ++w) tot += wsum[w]; sg[ti] = 1.0f / (1.0f + expf(-tot)); }
 }
 
 // ---- expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) ----------------------------------------------------
 // grid (row tiles, entries); entry = ti*(k+1) + j, j < k: routed expert sel_idx[ti][j], j == k: the shared expert.
 template <int FMT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ x, float* __restrict__ h, int hstride,
-                                                   const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
-  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+                                                   const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[2][NW][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
   const int nrows = shared ? m.sf : m.ff;
   if ((int)blockIdx.x * 64 >= nrows) return;
-  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
   const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.ff >> 6)) + blockIdx.x;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __r
   const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
   const float* xs = x + (size_t)ti * m.d;
   float ag[1] = {0.0f}, au[1] = {0.0f};
-  for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(G, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, au); }
+  for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(G, lds2, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, lds2, tile, ku, lane, xs + ku * 64, 0, au); }
   red[0][wave][lane] = ag[0]; red[1][wave][lane] = au[0];
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -81,13 +82,11 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __r
 // ---- expert down: partial[entry][r] = down[r] . h[entry] ---------------------------------------------------------------
 template <int FMT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
-                                                     const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
-  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+                                                     const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[NW][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
-  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const QMatDev& D = shared ? m.sh_down : m.down_e;
   const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.d >> 6)) + blockIdx.x;
@@ -95,7 +94,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
   const int upw = (D.U + NW - 1) / NW, k0 = wave * upw, kend = min(D.U, k0 + upw);
   const float* xs = h + (size_t)entry * hstride;
   float acc[1] = {0.0f};
-  for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds3, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
+  for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
   red[wave][lane] = acc[0];
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -139,12 +138,12 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   hipLaunchKernelGGL(k_router_topk, dim3(t), dim3((m.n_exp + 63) / 64 * 64), 0, ctx->stream, w.logits, m.n_exp, m.top_k, m.sh_gate_inp, x, m.d, w.sel_idx, w.sel_w, w.sg); }
   PYRE_CHECK_LAUNCH(ctx);
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
-  const uint32_t* g3 = ctx->d_iq3s; const uint2* g2 = (const uint2*)ctx->d_iq2xs;
+  const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   { ProfScope ps(ctx, "moe_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)));
-  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g3, g2)); }
+  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
-  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g3, g2)); }
+  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
   hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y); }

@@ -5,7 +5,7 @@
 
 // ---- repack: raw GGUF rows -> planes --------------------------------------------------------------------------------
 // One thread per (padded row, unit).  Rows beyond m.rows are written as zeros (they decode to 0 and are never stored).
-__global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_bytes, uint8_t* p0, uint8_t* p1, uint8_t* p2, uint8_t* p3, uint8_t* pb) {
+__global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_bytes, uint8_t* p0, uint8_t* p1, uint8_t* p2, uint8_t* p3, uint8_t* pb, const uint32_t* __restrict__ g3) {
   size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t total = (size_t)m.tiles * 64 * m.U;
   if (gid >= total) return;
@@ -35,11 +35,18 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
       uint8_t* d = p1 + e * 2; d[0] = live ? b[66 + 2 * j] : 0; d[1] = live ? b[67 + 2 * j] : 0;
       if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
     } break;
-    default: {   // IQ3_S
+    default: {   // IQ3_S: codebook lookups and signs are resolved here, once (gguf_q.rs:141-151), into 4-bit codes
       const uint8_t* b = row + (size_t)(ku >> 2) * 110; int j = ku & 3;
-      put_vec(0, b + 2 + 16 * j);
-      uint8_t* s = p1 + e * 8; for (int i = 0; i < 8; ++i) s[i] = live ? b[74 + 8 * j + i] : 0;
-      uint8_t* h = p2 + e * 2; h[0] = live ? b[66 + 2 * j] : 0; h[1] = live ? b[67 + 2 * j] : 0;
+      for (int c = 0; c < 2; ++c) {              // chunk c = sub-block 2j + c of the super-block: 32 values
+        int ib = 2 * j + c; uint32_t words[4] = {0, 0, 0, 0}; uint32_t h = live ? b[66 + ib] : 0;
+        for (int l = 0; live && l < 4; ++l) {      // padding rows lie past the end of the raw buffer: never read them
+          uint32_t gA = g3[b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256)], gB = g3[b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256)];
+          uint32_t sg = b[74 + 4 * ib + l], wd = 0;
+          for (int jj = 0; jj < 4; ++jj) { wd |= iq3s_code((gA >> (8 * jj)) & 0xFF, (sg >> jj) & 1) << (4 * jj); wd |= iq3s_code((gB >> (8 * jj)) & 0xFF, (sg >> (4 + jj)) & 1) << (16 + 4 * jj); }
+          words[l] = wd;
+        }
+        uint32_t* dst = (uint32_t*)(v + ((size_t)c * 64 + lane) * 16); for (int i = 0; i < 4; ++i) dst[i] = words[i];
+      }
       p3[e] = live ? b[106 + j] : 0;
       if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
     }
@@ -49,22 +56,22 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
 // ---- bit-exact dequant export -----------------------------------------------------------------------------------------
 // grid (U, tiles), 64 threads: lane l decodes unit ku of row tile*64+l, the tile is transposed through LDS so that
 // each row's 64 values leave as one contiguous 256-byte store.
-template <int FMT> __global__ __launch_bounds__(64) void k_dequant(QMatDev m, const uint32_t* g3, const uint64_t* g2, float* __restrict__ out) {
+template <int FMT> __global__ __launch_bounds__(64) void k_dequant(QMatDev m, const uint64_t* g2, float* __restrict__ out) {
   __shared__ float tile_buf[64][65];
   int ku = blockIdx.x, tile = blockIdx.y, lane = threadIdx.x;
   float y[64];
-  decode_exact<FMT>(m, g3, g2, tile, ku, lane, y);
+  decode_exact<FMT>(m, g2, tile, ku, lane, y);
   for (int i = 0; i < 64; ++i) tile_buf[lane][i] = y[i];
   __syncthreads();
   for (int r = 0; r < 64; ++r) { size_t row = (size_t)tile * 64 + r; if (row < (size_t)m.rows) out[row * m.cols + (size_t)ku * 64 + lane] = tile_buf[r][lane]; }
 }
 
 // rows by index (embedding lookup, QMat::row): grid (ceil(U/64), n), 64 threads, thread = unit
-template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const uint32_t* g3, const uint64_t* g2, const uint32_t* __restrict__ idx, float* __restrict__ out, int out_stride) {
+template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const uint64_t* g2, const uint32_t* __restrict__ idx, float* __restrict__ out, int out_stride) {
   int ku = blockIdx.x * 64 + threadIdx.x; if (ku >= m.U) return;
   uint32_t r = idx[blockIdx.y]; if (r >= (uint32_t)m.rows) return;
   float y[64];
-  decode_exact<FMT>(m, g3, g2, (int)(r >> 6), ku, (int)(r & 63), y);
+  decode_exact<FMT>(m, g2, (int)(r >> 6), ku, (int)(r & 63), y);
   float* o = out + (size_t)blockIdx.y * out_stride + (size_t)ku * 64;
   for (int i = 0; i < 64; ++i) o[i] = y[i];
 }
@@ -80,19 +87,17 @@ template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const
 //   best != nullptr (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 template <int FMT, int T, int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int upw,
-                                                  uint32_t* __restrict__ best, const uint32_t* __restrict__ g3, const uint2* __restrict__ g2) {
-  __shared__ uint32_t lds3[FMT == FMT_IQ3_S ? 512 : 1];
+                                                  uint32_t* __restrict__ best, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[NW][T][64];
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
-  if constexpr (FMT == FMT_IQ3_S) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds3[i] = g3[i]; __syncthreads(); }
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int k0 = (ks * NW + wave) * upw; const int k1 = min(m.U, k0 + upw);
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds3, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
+  for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
 #pragma unroll
   for (int t = 0; t < T; ++t) red[wave][t][lane] = acc[t];
   __syncthreads();
@@ -122,7 +127,7 @@ template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDe
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   FmtGeom g = fmt_geom(FMT);
   ProfScope ps(ctx, name.c_str(), (double)m.rows * (m.cols / g.el) * g.bytes + 4.0 * T * ((double)m.cols + m.rows));
-  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, best, (const uint32_t*)ctx->d_iq3s, (const uint2*)ctx->d_iq2xs);
+  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, best, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 // Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
@@ -169,7 +174,7 @@ int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, flo
 // 64 threads per block: every block redoes the (tiny) scan of the per-tile maxima, block 0 publishes the id, and when a
 // matrix is given thread u of block b then dequantizes unit 64*b+u of the chosen row.
 template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* __restrict__ best, int n_tiles, uint32_t* id_out, uint32_t* mirror, QMatDev m, int have_m,
-                                                               const uint32_t* g3, const uint64_t* g2, float* __restrict__ out, int* step) {
+                                                               const uint64_t* g2, float* __restrict__ out, int* step) {
   const int tid = threadIdx.x;
   float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
   const uint2* b2 = (const uint2*)best;
@@ -182,16 +187,16 @@ template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* 
   if (!have_m) return;
   int ku = blockIdx.x * 64 + tid; if (ku >= m.U || bi >= (uint32_t)m.rows) return;
   float y[64];
-  decode_exact<FMT>(m, g3, g2, (int)(bi >> 6), ku, (int)(bi & 63), y);
+  decode_exact<FMT>(m, g2, (int)(bi >> 6), ku, (int)(bi & 63), y);
   float* o = out + (size_t)ku * 64;
   for (int i = 0; i < 64; ++i) o[i] = y[i];
 }
 
 int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out, int* step) {
   ProfScope ps(ctx, "pick_embed", 8.0 * n_tiles);
-  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out, step); }
+  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step); }
   else { dim3 grid((m->U + 63) / 64);
-    FMT_DISPATCH(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out, step)); }
+    FMT_DISPATCH(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step)); }
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
@@ -199,7 +204,7 @@ int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* idx, int n,
   if (n <= 0) return PYRE_OK;
   dim3 grid((m.U + 63) / 64, n);
   ProfScope ps(ctx, "embed_rows", 0.0);
-  FMT_DISPATCH(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
+  FMT_DISPATCH(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
@@ -231,7 +236,7 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
     src = (const uint8_t*)tmp;
   }
   size_t total = ent * 1; unsigned nblk = (unsigned)((total + 255) / 256);
-  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3);
+  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (const uint32_t*)ctx->d_iq3s);
   e = hipGetLastError();
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (tmp) (void)hipFree(tmp);
@@ -251,7 +256,7 @@ size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; 
 int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
   if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");
   dim3 grid(m->dv.U, m->dv.tiles);
-  FMT_DISPATCH(m->dv.fmt, hipLaunchKernelGGL((k_dequant<F>), grid, dim3(64), 0, ctx->stream, m->dv, (const uint32_t*)ctx->d_iq3s, (const uint64_t*)ctx->d_iq2xs, out_dev));
+  FMT_DISPATCH(m->dv.fmt, hipLaunchKernelGGL((k_dequant<F>), grid, dim3(64), 0, ctx->stream, m->dv, (const uint64_t*)ctx->d_iq2xs, out_dev));
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 int pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host) {
