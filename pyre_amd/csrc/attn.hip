@@ -79,14 +79,18 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 
 // grid (chunks of 256 positions, nkv, t), 1024 threads.  One workgroup serves the G query heads that share a KV head.
 // Wave (pw, dq) owns the 64 positions pw*64.. of the chunk and the 64 head dims dq*64.., so every cache element is read
-// once per workgroup and each wave has all of its loads in flight at once (the step is bound by memory latency, not
-// bandwidth, at decode sizes).
-//  phase 1: lane = position; partial scores over the wave's dims for the G heads (q comes from scalar loads);
-//           the four dim quarters are added in order
+// once per workgroup and each wave has all of its loads in flight at once (at decode sizes the step is bound by memory
+// latency, not bandwidth).  Both products run on the fp32 matrix cores as 16x16x4 tiles with the G heads as the
+// (zero-padded) 16 columns: the query and the softmax weights are then ordinary per-lane operands instead of
+// wave-uniform values that would have to come through scalar loads or shared-memory broadcasts.
+//   v_mfma_f32_16x16x4f32: lane l supplies A[i = l%16][k = l/16] and B[k = l/16][j = l%16], and holds
+//   D[i = 4*(l/16) + r][j = l%16] in register r.
+//  phase 1: D[position][head] += K[position][dim] q[head][dim]; step s of lane group kg stands for dim 16*kg + s, so a
+//           lane's 16 dims are 4 float4 of q and 2 words of 4-bit keys.  The four dim quarters are added in order.
 //  phase 2: chunk-local max / exp / sum per head (thread = position x head group)
-//  phase 3: unnormalised sum_p e_p V[p] over the wave's positions for the wave's dims; f32 rows: lane = dim;
-//           4-bit rows: lane = (position mod 8, word), folded over the 8 position groups by a fixed shuffle tree;
-//           the four position quarters are added in order
+//  phase 3: D[dim][head] += V[position][dim] e[position][head]; row i of tile dt stands for dim 4*i + dt, so a lane's
+//           4 tiles are one float4 (or 4 nibbles of one word) per position.  The four position quarters are added in order.
+typedef float f4v __attribute__((ext_vector_type(4)));
 template <int HD, int G>
 __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
   static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
@@ -100,58 +104,61 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
   if (chunk * 256 >= n) return;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
   const size_t cap = kv.cap;
-  const float* __restrict__ qg = qbuf + ((size_t)ti * a.nh + (size_t)kvh * G) * HD + dq * 64;     // wave-uniform reads -> scalar loads
   const int wbase = chunk * 256 + pw * 64, p = wbase + lane;
   const bool valid = p < n, packed = wbase < pb, active = wbase < n;
   const float scale = 1.0f / sqrtf((float)HD);
-  constexpr int QB = G >= 8 ? 4 : 8;
-  float s[G];
+  const int li = lane & 15, lg = lane >> 4;
+  const int row = a.nkv * HD;
+  // ---- phase 1
+  {
+    f4v D[4];
 #pragma unroll
-  for (int g = 0; g < G; ++g) s[g] = 0.0f;
-  if (active) {
-    const int pp = valid ? p : n - 1;
-    if (packed) {
-      uint32_t kw[8]; float ksc[2];
+    for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) {
+      float B[16];
+      if (li < G) {
+        const float4* q4 = (const float4*)(qbuf + ((size_t)ti * a.nh + (size_t)kvh * G + li) * HD + dq * 64 + 16 * lg);
 #pragma unroll
-      for (int w = 0; w < 8; ++w) kw[w] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + w) * cap + pp];
+        for (int j = 0; j < 4; ++j) { float4 v = q4[j]; B[4 * j] = v.x; B[4 * j + 1] = v.y; B[4 * j + 2] = v.z; B[4 * j + 3] = v.w; }
+      } else {
 #pragma unroll
-      for (int b = 0; b < 2; ++b) ksc[b] = kv.ks[((size_t)kvh * (HD / 32) + dq * 2 + b) * cap + pp];
+        for (int s = 0; s < 16; ++s) B[s] = 0.0f;
+      }
+      float A[4][16];
+      if (packed) {
+        uint32_t kw[4][2]; float ksc[4];
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        float bp[G];
-#pragma unroll
-        for (int g = 0; g < G; ++g) bp[g] = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) { float kvl = nib_val(kw[b * 4 + w], i);
-            if (i % QB == 0) __builtin_amdgcn_sched_barrier(0);      // q scalars of QB dims at a time
-#pragma unroll
-            for (int g = 0; g < G; ++g) bp[g] = fmaf(kvl, qg[g * HD + b * 32 + w * 8 + i], bp[g]); }
+        for (int pt = 0; pt < 4; ++pt) {
+          const size_t pp = (size_t)wbase + 16 * pt + li;
+          kw[pt][0] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg) * cap + pp]; kw[pt][1] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1) * cap + pp];
+          ksc[pt] = kv.ks[((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1)) * cap + pp];
         }
 #pragma unroll
-        for (int g = 0; g < G; ++g) s[g] = fmaf(ksc[b], bp[g], s[g]);
+        for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(kw[pt][s >> 3], s & 7) * ksc[pt];
+      } else {
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt) {
+          const size_t pp = (size_t)min(wbase + 16 * pt + li, n - 1);
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[((size_t)kvh * HD + dq * 64 + 16 * lg + s) * cap + pp];
+        }
       }
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
-      float kreg[64];
 #pragma unroll
-      for (int dd = 0; dd < 64; ++dd) kreg[dd] = kv.kf[((size_t)kvh * HD + dq * 64 + dd) * cap + pp];
+      for (int s = 0; s < 16; ++s)
 #pragma unroll
-      for (int d8 = 0; d8 < 64; d8 += QB) {     // q scalars of QB dims at a time: the fences keep the scalar loads from piling up
-        __builtin_amdgcn_sched_barrier(0);
+        for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
+    }
+    if (li < G) {
 #pragma unroll
-        for (int dd = d8; dd < d8 + QB; ++dd)
+      for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-          for (int g = 0; g < G; ++g) s[g] = fmaf(kreg[dd], qg[g * HD + dd], s[g]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+        for (int r = 0; r < 4; ++r) red[((size_t)dq * 256 + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
     }
   }
-#pragma unroll
-  for (int g = 0; g < G; ++g) red[((size_t)dq * 256 + pw * 64 + lane) * G + g] = s[g];
   __syncthreads();
-  // phase 2: this thread's position is pw*64 + lane, its heads are dq, dq + 4, ...
+  // ---- phase 2: this thread's position is pw*64 + lane, its heads are dq, dq + 4, ...
   constexpr int GH = (G + 3) / 4;
   const int pos = pw * 64 + lane;
   float sv[GH];
@@ -182,69 +189,49 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
     }
   }
   __syncthreads();   // weights of every position visible; the score partials in `red` are dead
-  // phase 3
-  const int row = a.nkv * HD;
-  if (packed) {
-    const int psub = lane >> 3, w8 = lane & 7;
-    uint32_t vw[8]; float vsc[8];              // packed positions lie below the boundary, hence inside the view
+  // ---- phase 3
+  {
+    f4v D[4];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const size_t pg = (size_t)wbase + it * 8 + psub;
-      vw[it] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + w8];
-      vsc[it] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (w8 >> 2)];
-    }
-    constexpr int HG = G > 4 ? 4 : G;          // heads per pass (bounds the accumulator registers)
-#pragma unroll
-    for (int g0 = 0; g0 < G; g0 += HG) {
-      float acc[HG][8];
-#pragma unroll
-      for (int g = 0; g < HG; ++g)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        __builtin_amdgcn_sched_barrier(0);
-        const int pl = it * 8 + psub;
-        float wg[HG];
-#pragma unroll
-        for (int g = 0; g < HG; ++g) wg[g] = sc[pw * 64 + pl][g0 + g];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { float vv = nib_val(vw[it], i) * vsc[it];
-#pragma unroll
-          for (int g = 0; g < HG; ++g) acc[g][i] = fmaf(wg[g], vv, acc[g][i]); }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int g = 0; g < HG; ++g)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          float o = acc[g][i]; o += __shfl_xor(o, 8); o += __shfl_xor(o, 16); o += __shfl_xor(o, 32);
-          if (psub == 0) red[((size_t)pw * G + g0 + g) * HD + dq * 64 + w8 * 8 + i] = o;
-        }
-    }
-  } else {
-    float acc[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) acc[g] = 0.0f;
+    for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     if (active) {
+      float A[4][16];
+      if (packed) {             // packed positions lie below the boundary, hence inside the view
+        uint32_t vw[16]; float vsc[16];
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {          // positions past the view carry weight zero; their address is clamped
-        float vreg[32];
-#pragma unroll
-        for (int j = 0; j < 32; ++j) { const int pg = min(wbase + hf * 32 + j, n - 1); vreg[j] = kv.vf[(size_t)pg * row + (size_t)kvh * HD + dq * 64 + lane]; }
-#pragma unroll
-        for (int j8 = 0; j8 < 32; j8 += 8) {
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int j = j8; j < j8 + 8; ++j)
-#pragma unroll
-            for (int g = 0; g < G; ++g) acc[g] = fmaf(sc[pw * 64 + hf * 32 + j][g], vreg[j], acc[g]);
+        for (int s = 0; s < 16; ++s) {
+          const size_t pg = (size_t)wbase + 4 * s + lg;
+          vw[s] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
+          vsc[s] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
         }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
 #pragma unroll
-    for (int g = 0; g < G; ++g) red[((size_t)pw * G + g) * HD + dq * 64 + lane] = acc[g];
+        for (int s = 0; s < 16; ++s) {
+          const uint32_t hw = vw[s] >> (16 * (li & 1));      // the lane's four nibbles
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc[s];
+        }
+      } else {                  // positions past the view carry weight zero; their address is clamped
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+          const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);
+          float4 v = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+          A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
+        }
+      }
+      float B[16];
+#pragma unroll
+      for (int s = 0; s < 16; ++s) B[s] = li < G ? sc[pw * 64 + 4 * s + lg][li < G ? li : 0] : 0.0f;
+#pragma unroll
+      for (int s = 0; s < 16; ++s)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
+    }
+    if (li < G) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((size_t)pw * G + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
+    }
   }
   __syncthreads();
   for (int i = tid; i < G * HD; i += 1024) {
