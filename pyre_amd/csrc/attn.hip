@@ -40,7 +40,7 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
     v = tid < half ? x0 * cs - x1 * sn : x1 * cs + x0 * sn;
   }
   if (is_k) {
-    kv.kf[((size_t)h * HD + tid) * kv.cap + pos] = v;
+    kv.kf[kv_blk((size_t)h * HD + tid, (size_t)a.nkv * HD, pos)] = v;
     kv.vf[(size_t)pos * a.nkv * HD + (size_t)h * HD + tid] = row[(size_t)a.nh * 2 * HD + (size_t)a.nkv * HD + (size_t)h * HD + tid];
   } else qout[((size_t)ti * a.nh + h) * HD + tid] = v;
 }
@@ -63,16 +63,16 @@ __global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1, const int* __rest
   const bool is_v = gid >= per; if (is_v) gid -= per;
   const int pos = p0 + (int)(gid / bpr), blk = (int)(gid % bpr), kvh = blk / (HD / 32), bb = blk % (HD / 32);
   float x[32];
-  for (int i = 0; i < 32; ++i) x[i] = is_v ? kv.vf[(size_t)pos * a.nkv * HD + (size_t)blk * 32 + i] : kv.kf[((size_t)kvh * HD + bb * 32 + i) * kv.cap + pos];
+  for (int i = 0; i < 32; ++i) x[i] = is_v ? kv.vf[(size_t)pos * a.nkv * HD + (size_t)blk * 32 + i] : kv.kf[kv_blk((size_t)kvh * HD + bb * 32 + i, (size_t)a.nkv * HD, pos)];
   float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(x[i]));
   const float s = (m > 0.0f && isfinite(m)) ? m / 7.0f : 0.0f;
   for (int w = 0; w < 4; ++w) {
     uint32_t u = 0;
     for (int j = 0; j < 8; ++j) { int q = s > 0.0f ? (int)fminf(fmaxf(roundf(x[8 * w + j] / s), -7.0f), 7.0f) : 0; u |= ((uint32_t)q & 0xFu) << (4 * j); }
     if (is_v) kv.vq[(size_t)pos * (a.nkv * HD / 8) + (size_t)blk * 4 + w] = u;
-    else kv.kq[((size_t)kvh * (HD / 8) + bb * 4 + w) * kv.cap + pos] = u;
+    else kv.kq[kv_blk((size_t)kvh * (HD / 8) + bb * 4 + w, (size_t)a.nkv * (HD / 8), pos)] = u;
   }
-  if (is_v) kv.vs[(size_t)pos * bpr + blk] = s; else kv.ks[((size_t)kvh * (HD / 32) + bb) * kv.cap + pos] = s;
+  if (is_v) kv.vs[(size_t)pos * bpr + blk] = s; else kv.ks[kv_blk((size_t)kvh * (HD / 32) + bb, (size_t)a.nkv * (HD / 32), pos)] = s;
 }
 
 __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((int)(w << (28 - 4 * i))) >> 28); }   // sign-extended nibble i
@@ -103,7 +103,6 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
   const int n = start + ti + 1;
   if (chunk * 256 >= n) return;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
-  const size_t cap = kv.cap;
   const int wbase = chunk * 256 + pw * 64, p = wbase + lane;
   const bool valid = p < n, packed = wbase < pb, active = wbase < n;
   const float scale = 1.0f / sqrtf((float)HD);
@@ -130,8 +129,8 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) {
           const size_t pp = (size_t)wbase + 16 * pt + li;
-          kw[pt][0] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg) * cap + pp]; kw[pt][1] = kv.kq[((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1) * cap + pp];
-          ksc[pt] = kv.ks[((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1)) * cap + pp];
+          kw[pt][0] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp)]; kw[pt][1] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp)];
+          ksc[pt] = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp)];
         }
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt)
@@ -142,7 +141,7 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
         for (int pt = 0; pt < 4; ++pt) {
           const size_t pp = (size_t)min(wbase + 16 * pt + li, n - 1);
 #pragma unroll
-          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[((size_t)kvh * HD + dq * 64 + 16 * lg + s) * cap + pp];
+          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp)];
         }
       }
 #pragma unroll
@@ -372,7 +371,7 @@ int pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, int
 int pyre_attn_load_cache(pyre_ctx* ctx, pyre_attn* a, const float* k_host, const float* v_host, int n) {
   if (!ctx || !a || !k_host || !v_host || n < 0 || n > a->cap) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_load_cache: bad argument");
   size_t row = (size_t)a->dv.nkv * a->dv.hd; std::vector<float> kt(row * a->cap, 0.0f);
-  for (int p = 0; p < n; ++p) for (size_t c = 0; c < row; ++c) kt[c * a->cap + p] = k_host[(size_t)p * row + c];
+  for (int p = 0; p < n; ++p) for (size_t c = 0; c < row; ++c) kt[kv_blk(c, row, p)] = k_host[(size_t)p * row + c];
   PYRE_HIP(ctx, hipMemcpyAsync(a->kv.kf, kt.data(), kt.size() * 4, hipMemcpyHostToDevice, ctx->stream));
   PYRE_HIP(ctx, hipMemcpyAsync(a->kv.vf, v_host, (size_t)n * row * 4, hipMemcpyHostToDevice, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -387,7 +386,7 @@ int pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_ho
   PYRE_HIP(ctx, hipMemcpyAsync(kt.data(), a->kv.kf, kt.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipMemcpyAsync(v_host, a->kv.vf, (size_t)a->len * row * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  for (int p = 0; p < a->len; ++p) for (size_t c = 0; c < row; ++c) k_host[(size_t)p * row + c] = kt[c * a->cap + p];
+  for (int p = 0; p < a->len; ++p) for (size_t c = 0; c < row; ++c) k_host[(size_t)p * row + c] = kt[kv_blk(c, row, p)];
   return PYRE_OK;
 }
 // kv4 pack / unpack of a flat f32 array through the device kernels' arithmetic is covered by load_cache + decode; this

@@ -92,10 +92,31 @@ struct MoeWork {            // scratch for up to 8 tokens, owned by whoever laun
   float* h;                 // [8*(top_k+1)][max(ff, sf)]
   float* partial;           // [8*(top_k+1)][d]
 };
+// The FFN output of a window, left unreduced for the consumer to fold:
+//   y[ti][r] = partial[ti*(k+1)+k][r] * sg[ti] + (sum_j sel_w[ti*k+j] * partial[ti*(k+1)+j][r], j ascending, from zero)
+struct MoeOut { const float* partial; const float* sel_w; const float* sg; int d, k; };
+#define PYRE_MOE_KMAX 16      // moe_out_value keeps up to this many expert terms in registers
+#ifdef __HIPCC__
+// All loads are issued before the first add, so the value costs one memory round trip, not k + 1.
+__device__ __forceinline__ float moe_out_value(const MoeOut& mo, int ti, int r) {
+  const float* p = mo.partial + (size_t)ti * (mo.k + 1) * mo.d + r; const float* w = mo.sel_w + ti * mo.k;
+  float pv[PYRE_MOE_KMAX], wv[PYRE_MOE_KMAX];
+#pragma unroll
+  for (int j = 0; j < PYRE_MOE_KMAX; ++j) { pv[j] = j < mo.k ? p[(size_t)j * mo.d] : 0.0f; wv[j] = j < mo.k ? w[j] : 0.0f; }
+  float sh = p[(size_t)mo.k * mo.d], g = mo.sg[ti];
+  float o = 0.0f;
+#pragma unroll
+  for (int j = 0; j < PYRE_MOE_KMAX; ++j) if (j < mo.k) o += wv[j] * pv[j];
+  return sh * g + o;
+}
+#endif
+inline MoeOut pyre_moe_out(const MoeDev& m, const MoeWork& w, int first_token) {
+  return MoeOut{w.partial + (size_t)first_token * (m.top_k + 1) * m.d, w.sel_w + (size_t)first_token * m.top_k, w.sg + first_token, m.d, m.top_k};
+}
 size_t pyre_moe_work_bytes(const MoeDev& m);
 void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
-// y[t][d] = ffn(x[t][d]).  If comb_x != nullptr the result is also folded into the residual streams:
-// comb_x[ti][s][i] += y[ti][i] * 2*sigmoid(comb_inj[ti][s])   (hc_combine)
+// y[t][d] = ffn(x[t][d]).  With y == nullptr (top_k <= PYRE_MOE_KMAX) the output stays unreduced in the work buffers
+// (pyre_moe_out) for a consumer that evaluates moe_out_value itself.
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev);
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
@@ -104,10 +125,10 @@ struct HcWork { float* xn; float* o; };     // [8][hc*d] normalized streams, [<=
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // Streams are read from x_in (element i of stream s of token ti at x_in[ti*in_ts + s*in_ss + i]; in_ss = 0 replicates one
-// row over the streams), the pending residual update is applied first when comb_out is given
-// (x[ti][s][:] += comb_out[ti][:] * 2*sigmoid(comb_inj[ti][s])), and the updated streams go to x_out [t][hc][d], which
+// row over the streams), the pending residual update is applied first when comb_out (a [t][d] vector) or comb_moe (the
+// unreduced FFN output) is given (x[ti][s][:] += out[ti][:] * 2*sigmoid(comb_inj[ti][s])), and the updated streams go to x_out [t][hc][d], which
 // must not overlap x_in.  mixed [t][d] and inj [t][hc] = hc_mix(updated streams).
-int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj,
+int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
                        float eps, float* mixed_dev, float* inj_dev);
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, const float* out_dev, const float* inj_dev);
 
@@ -126,14 +147,17 @@ int pyre_gdn_prefill_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, i
 // ---- gated attention over the KV cache (attn.hip) -----------------------------------------------------------------------
 struct AttnDev { const float* qn; const float* kn; const float* rope_inv; int nh, nkv, hd, n_rot, kv_bits, kv_recent; float eps; };
 struct KvDev {
-  float* kf;        // [nkv][hd][cap]      f32 keys, position-minor (lane = position reads are coalesced)
+  // key planes are blocked by 64 positions: row r of R rows at position p sits at kv_blk(r, R, p), so the rows a wave
+  // reads for its 64 positions are one contiguous range (lane = position reads stay coalesced)
+  float* kf;        // [cap/64][nkv*hd][64]      f32 keys
   float* vf;        // [cap][nkv*hd]       f32 values, row-major
-  uint32_t* kq;     // [nkv][hd/8][cap]    4-bit keys: word w of position p holds dims 8w..8w+7
-  float* ks;        // [nkv][hd/32][cap]   key scales
+  uint32_t* kq;     // [cap/64][nkv*hd/8][64]    4-bit keys: word w of position p holds dims 8w..8w+7
+  float* ks;        // [cap/64][nkv*hd/32][64]   key scales
   uint32_t* vq;     // [cap][nkv*hd/8]     4-bit values
   float* vs;        // [cap][nkv*hd/32]    value scales
   int cap;
 };
+__host__ __device__ inline size_t kv_blk(size_t r, size_t R, size_t p) { return ((p >> 6) * R + r) * 64 + (p & 63); }
 struct AttnWork { float* q; float* part_o; float* part_ml; int max_chunks; };   // q [8][nh][hd]; partials per (token, head, chunk)
 size_t pyre_kv_bytes(const AttnDev& a, int cap);
 void   pyre_kv_carve(const AttnDev& a, int cap, void* base, KvDev* kv);

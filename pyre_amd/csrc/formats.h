@@ -126,7 +126,9 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
     uint32_t dd = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+      float part[T];
+_Pragma("unroll")
+      for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         uint4 v = ld_vec<4>(m, tile, ku, 2 * b + c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -164,7 +166,9 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
       uint32_t s = (sc >> (8 * ib)) & 0xFF;
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
-        float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+        float part[T];
+_Pragma("unroll")
+      for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
         for (int l2 = 0; l2 < 2; ++l2) {
           int l = 2 * hf + l2;
@@ -198,7 +202,9 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
     }
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
-      float part[T]; for (int t = 0; t < T; ++t) part[t] = 0.0f;
+      float part[T];
+_Pragma("unroll")
+      for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         uint32_t u = w[4 * sb + k], lo = u & 0x0F0F0F0Fu, hi = (u >> 4) & 0x0F0F0F0Fu;

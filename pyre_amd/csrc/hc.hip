@@ -9,9 +9,11 @@
 __device__ __forceinline__ float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // Stream element i of token ti with the pending residual update applied: x + out * w  (:1384-1387), w = 2*sigm(inj).
-__device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, float w, int d, int ti, int s, int i) {
+// `out` is a plain [t][d] vector (comb_out) or the unreduced FFN output (mo.partial != nullptr).
+__device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, const MoeOut& mo, float w, int d, int ti, int s, int i) {
   float v = x_in[(size_t)ti * in_ts + (size_t)s * in_ss + i];
-  if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
+  if (mo.partial) v = v + moe_out_value(mo, ti, i) * w;
+  else if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
   return v;
 }
 
@@ -21,7 +23,7 @@ __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in
 //      publishes them (xn) and the updated stream (x_out, never the buffer x_in points into)
 //   3. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
 template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
-    const float* __restrict__ comb_out, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
+    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   extern __shared__ __align__(16) float sm[];
@@ -35,10 +37,10 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
   float w[T], ss[T];
 #pragma unroll
-  for (int t = 0; t < T; ++t) { w[t] = comb_out ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
+  for (int t = 0; t < T; ++t) { w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
   for (int i = tid; i < d; i += nthr) {
 #pragma unroll
-    for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, w[t], d, t, s, i); ss[t] += v * v; }
+    for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i); ss[t] += v * v; }
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -54,7 +56,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
     const float nv = norm[(size_t)s * d + i0 + j];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, w[t], d, t, s, i0 + j);
+      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
       float o = v * sc[t] * nv;                                   // rms, :209: (x * s) * w
       xs[(size_t)t * L + j] = o;
       if (tile == 0) { size_t k = ((size_t)t * hc + s) * d + i0 + j; xn[k] = o; x_out[k] = v; }
@@ -139,11 +141,11 @@ DownPlan down_plan(const HcDev& h) {
 }
 
 template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out,
-                                               const float* comb_out, const float* comb_inj, float eps) {
+                                               const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   const int L = p.nw * p.upw * 64; size_t lds = 4 * ((size_t)T * L + (size_t)p.nw * T * 64 + (size_t)p.nw * T);
   FmtGeom g = fmt_geom(FMT);
   ProfScope ps(ctx, "hc_norm_down", (double)h.di.rows * (h.di.cols / g.el) * g.bytes + 4.0 * T * h.hc * h.d * 4);
-  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, comb_inj, h.norm, h.d, h.hc, eps,
+  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, eps,
                      w.xn, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
@@ -162,8 +164,8 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
   switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; BODY } case FMT_F16: { constexpr int F = FMT_F16; BODY } case FMT_BF16: { constexpr int F = FMT_BF16; BODY } \
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; BODY } case FMT_Q4_K: { constexpr int F = FMT_Q4_K; BODY } case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; BODY } \
     default: { constexpr int F = FMT_IQ3_S; BODY } }
-int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj, float eps) {
-  HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, comb_inj, eps))
+int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
+  HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, eps))
 }
 int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, float* mixed, float* inj) {
   HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, mixed, inj))
@@ -176,7 +178,7 @@ void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
   w->xn = (float*)take(4 * 8 * (size_t)h.hc * h.d); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
 }
 
-int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const float* comb_inj,
+int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
                        float eps, float* mixed, float* inj) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
   if (x_in == x_out) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: the updated streams must go to another buffer");
@@ -184,7 +186,9 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: needs d and the low rank in multiples of 64 and hc * (low rank / 64) <= 16 (d %d, low rank %d, hc %d)", h.d, h.lr, h.hc);
   DownPlan p = down_plan(h);
   if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
-  int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_inj, eps); if (rc) return rc;
+  MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
+  if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);
+  int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, mo, comb_inj, eps); if (rc) return rc;
   return up_mix(ctx, h, w, p.ksplit, t, mixed, inj);
 }
 

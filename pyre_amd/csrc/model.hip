@@ -227,7 +227,7 @@ int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, floa
   PYRE_HIP(ctx, hipMemcpyAsync(kt.data(), s->kv[ai].kf, kt.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipMemcpyAsync(v_host, s->kv[ai].vf, (size_t)s->len * row * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  for (int p = 0; p < s->len; ++p) for (size_t cc = 0; cc < row; ++cc) k_host[(size_t)p * row + cc] = kt[cc * s->cap + p];
+  for (int p = 0; p < s->len; ++p) for (size_t cc = 0; cc < row; ++cc) k_host[(size_t)p * row + cc] = kt[kv_blk(cc, row, p)];
   return PYRE_OK;
 }
 
@@ -253,10 +253,11 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   // leaves the updated streams in the other
   const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
   auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
-  const float* comb_out = nullptr; const float* comb_inj = nullptr;
+  const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself
+  MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
     advance();
     if (L.full) {
       int ai = L.mix_index;
@@ -269,21 +270,23 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       s->cur[li] = nb;
     }
     if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
-    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
     advance();
-    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, m->y))) return rc;
-    comb_out = m->y; comb_inj = m->inj_f;
+    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y))) return rc;
+    if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
+    comb_inj = m->inj_f;
   }
   if (!replay) s->len = start + t;
   if (o.head_tokens == 0) return PYRE_OK;       // prompt window whose logits nobody reads
   if (o.head_tokens >= t) {
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
     if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
     return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
   }
   // last token only: fold the pending ffn output into its streams, then the head
   const size_t last = (size_t)(t - 1) * hc * d;
-  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out + (size_t)(t - 1) * d, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
+  MoeOut mol{}; if (comb_moe) mol = pyre_moe_out(m->layers.back().moe, m->mw, t - 1);
+  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
   if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }

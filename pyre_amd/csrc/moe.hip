@@ -1,71 +1,82 @@
-// MoE FFN block: router logits -> softmax top-k (one kernel) -> grouped expert GEMV over only the selected experts.
+// MoE FFN block: router logits -> softmax top-k (inside the gate/up launch) -> grouped expert GEMV over only the
+// selected experts.
 // Follows ffn / routed (f32 branch) of the reference, src/model/qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793,
 // and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
 #include "formats.h"
 
-// ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id, and the shared-expert
-// gate sigmoid(sh_gate_inp . x).  grid = tokens; one thread per expert (block = n_exp rounded up to 64).
-// Two-level selection: every wave ranks its own 64 logits through lane broadcasts and keeps its best k as candidates
-// (an expert outside its wave's best k cannot be in the global best k); the nw*k candidates are then ranked against
-// each other from shared memory.
-__global__ __launch_bounds__(1024) void k_router_topk(const float* __restrict__ logits, int n_exp, int k, const float* __restrict__ sh_gate_inp,
-                                                      const float* __restrict__ x, int d, int32_t* sel_idx, float* sel_w, float* sg) {
-  __shared__ float c_val[16 * 32]; __shared__ int c_idx[16 * 32];     // candidates [wave][local rank]
-  __shared__ float r_val[32]; __shared__ int r_idx[32];               // the k winners by value rank
-  __shared__ float s_val[32]; __shared__ int s_idx[32]; __shared__ float s_w[32];   // ... by ascending expert id
-  __shared__ float wsum[16];
-  const int ti = blockIdx.x, e = threadIdx.x, lane = e & 63, wave = e >> 6, nw = blockDim.x >> 6;
-  float v = -INFINITY;
-  if (e < n_exp) { v = logits[(size_t)ti * n_exp + e]; if (isnan(v)) v = -INFINITY; }      // nan_clean
-  int lr = 0;
+// ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id -----------------------------
+// Runs inside every gate/up workgroup of a routed entry (all of them need the expert id before they can touch a
+// weight, and a separate launch would cost more than redoing this small selection everywhere).
+// Two-level selection: wave w < ceil(n_exp/64) ranks its own 64 logits through lane broadcasts and keeps its best k as
+// candidates (an expert outside its wave's best k cannot be in the global best k); the candidates are then ranked
+// against each other from shared memory.  Leaves ids (ascending) in s_idx[0..k) and weights in s_w[0..k).
+struct RouteLds { float c_val[16 * 32]; int c_idx[16 * 32]; float r_val[32]; int r_idx[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
+__device__ __forceinline__ void route_topk(const float* __restrict__ logits, int n_exp, int k, RouteLds& L) {
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6, nwa = (n_exp + 63) >> 6;
+  if (wave < nwa) {
+    float v = -INFINITY;
+    if (e < n_exp) { v = logits[e]; if (isnan(v)) v = -INFINITY; }      // nan_clean
+    int lr = 0;
 #pragma unroll
-  for (int j = 0; j < 64; ++j) { float u = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); lr += (u > v || (u == v && j < lane)) ? 1 : 0; }
-  if (lr < k) { c_val[wave * k + lr] = v; c_idx[wave * k + lr] = e; }
-  // shared-expert gate: all threads stride over d
-  float p = 0.0f; for (int i = e; i < d; i += blockDim.x) p = fmaf(sh_gate_inp[i], x[(size_t)ti * d + i], p);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
-  if (lane == 0) wsum[wave] = p;
-  __syncthreads();
-  const int nc = nw * k;
-  if (e < nc) {
-    float cv = c_val[e]; int ci = c_idx[e], rank = 0;
-#pragma unroll 16
-    for (int j = 0; j < nc; ++j) { float u = c_val[j]; int ui = c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
-    if (rank < k) { r_val[rank] = cv; r_idx[rank] = ci; }
+    for (int j = 0; j < 64; ++j) { float u = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); lr += (u > v || (u == v && j < lane)) ? 1 : 0; }
+    if (lr < k) { L.c_val[wave * k + lr] = v; L.c_idx[wave * k + lr] = e; }
   }
   __syncthreads();
-  if (e < k) { int me = r_idx[e], pos = 0; for (int j = 0; j < k; ++j) pos += r_idx[j] < me ? 1 : 0; s_idx[pos] = me; s_val[pos] = r_val[e]; }
+  const int nc = nwa * k;
+  if (e < nc) {
+    float cv = L.c_val[e]; int ci = L.c_idx[e], rank = 0;
+#pragma unroll 16
+    for (int j = 0; j < nc; ++j) { float u = L.c_val[j]; int ui = L.c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
+    if (rank < k) { L.r_val[rank] = cv; L.r_idx[rank] = ci; }
+  }
   __syncthreads();
-  float mx = -INFINITY;
-  if (e < k) { for (int i = 0; i < k; ++i) mx = fmaxf(mx, s_val[i]); s_w[e] = isfinite(mx) ? expf(s_val[e] - mx) : 1.0f; }
+  if (e < k) { int me = L.r_idx[e], pos = 0; for (int j = 0; j < k; ++j) pos += L.r_idx[j] < me ? 1 : 0; L.s_idx[pos] = me; L.s_val[pos] = L.r_val[e]; }
+  __syncthreads();
+  float mx = -INFINITY, ex = 1.0f;
+  if (e < k) { for (int i = 0; i < k; ++i) mx = fmaxf(mx, L.s_val[i]); ex = isfinite(mx) ? expf(L.s_val[e] - mx) : 1.0f; L.r_val[e] = ex; }
   __syncthreads();
   if (e < k) {
     float w;
     if (!isfinite(mx)) w = 1.0f / (float)k;
-    else { float sum = 0.0f; for (int i = 0; i < k; ++i) sum += s_w[i]; w = s_w[e] / sum; }
-    sel_idx[ti * k + e] = s_idx[e]; sel_w[ti * k + e] = w;
+    else { float sum = 0.0f; for (int i = 0; i < k; ++i) sum += L.r_val[i]; w = ex / sum; }
+    L.s_w[e] = w;
   }
-  if (e == 0) { float tot = 0.0f; for (int w = 0; w < nw; ++w) tot += wsum[w]; sg[ti] = 1.0f / (1.0f + expf(-tot)); }
+  __syncthreads();
 }
 
-// ---- expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) ----------------------------------------------------
-// grid (row tiles, entries); entry = ti*(k+1) + j, j < k: routed expert sel_idx[ti][j], j == k: the shared expert.
+// ---- routing + expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) -------------------------------------------
+// grid (row tiles, entries), 16 waves; entry = ti*(k+1) + j, j < k: the j-th chosen expert of token ti (ascending id),
+// j == k: the shared expert.  Tile 0 of entry (ti, 0) publishes the token's expert ids and weights, tile 0 of the shared
+// entry publishes the shared-expert gate sigmoid(sh_gate_inp . x).
 template <int FMT, int NW>
-__global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ x, float* __restrict__ h, int hstride,
-                                                   const uint2* __restrict__ g2) {
+__global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
+                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[2][NW][64];
+  __shared__ RouteLds rl;
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
   const int nrows = shared ? m.sf : m.ff;
   if ((int)blockIdx.x * 64 >= nrows) return;
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
-  const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
-  const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.ff >> 6)) + blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
   const float* xs = x + (size_t)ti * m.d;
+  int expert = 0;
+  if (!shared) {
+    route_topk(logits + (size_t)ti * m.n_exp, m.n_exp, m.top_k, rl);
+    expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]);
+  } else if (blockIdx.x == 0) {
+    float p = 0.0f; for (int i = threadIdx.x; i < m.d; i += NW * 64) p = fmaf(m.sh_gate_inp[i], xs[i], p);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
+    if (lane == 0) red[0][wave][0] = p;
+    __syncthreads();
+    if (threadIdx.x == 0) { float tot = 0.0f; for (int w = 0; w < NW; ++w) tot += red[0][w][0]; rl.s_w[0] = 1.0f / (1.0f + expf(-tot)); }
+    __syncthreads();
+  }
+  const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
+  const int tile = (shared ? 0 : expert * (m.ff >> 6)) + blockIdx.x;
+  const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
   float ag[1] = {0.0f}, au[1] = {0.0f};
   for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(G, lds2, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, lds2, tile, ku, lane, xs + ku * 64, 0, au); }
   red[0][wave][lane] = ag[0]; red[1][wave][lane] = au[0];
@@ -76,6 +87,12 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const int32_t* __r
     for (int w = 1; w < NW; ++w) { g += red[0][w][lane]; u += red[1][w][lane]; }
     float s = 1.0f / (1.0f + expf(-g));
     h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+  }
+  // Publishing comes last: a global store ahead of the dot products would stop the compiler from keeping the
+  // activations in scalar registers (it could no longer prove them unmodified).
+  if (blockIdx.x == 0) {
+    if (shared) { if (threadIdx.x == 0) sg[ti] = rl.s_w[0]; }
+    else if (j == 0 && threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
   }
 }
 
@@ -132,22 +149,22 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
 
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
+  if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
   int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc;
   auto mat_bytes = [](const QMatDev& q, double rows) { FmtGeom g = fmt_geom(q.fmt); return rows * (q.cols / g.el) * g.bytes; };
-  { ProfScope ps(ctx, "router_topk", 4.0 * t * (m.n_exp + m.d) + 4.0 * m.d);
-  hipLaunchKernelGGL(k_router_topk, dim3(t), dim3((m.n_exp + 63) / 64 * 64), 0, ctx->stream, w.logits, m.n_exp, m.top_k, m.sh_gate_inp, x, m.d, w.sel_idx, w.sel_w, w.sg); }
-  PYRE_CHECK_LAUNCH(ctx);
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
-  { ProfScope ps(ctx, "moe_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)));
-  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.sel_idx, x, w.h, hs, g2)); }
+  { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
+  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.logits, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
   MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
-  hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y); }
-  PYRE_CHECK_LAUNCH(ctx);
+  if (y) {
+    ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
+    hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y);
+    PYRE_CHECK_LAUNCH(ctx);
+  }
   return PYRE_OK;
 }
 
