@@ -64,6 +64,12 @@ struct pyre_qmat {
   void* base; size_t dev_bytes; QMatDev dv;
 };
 
+// Optional work folded into the end of a GEMV launch (qmat.hip):
+//   best: t = 1, per row tile (bits of the maximum, first row holding it) -> best[2*tile], best[2*tile+1]
+//   co:   rows < ch are the channels of a causal depthwise conv1d (kernel kk, weights conv_w[ch][kk]); the lane that
+//         owns a row runs the window's tokens in order, o = w[kk-1]*cur + sum_j w[j]*state[j], co[t][row] = silu(o),
+//         and slides the row's state conv_in -> conv_out ([kk-1][ch], oldest first; in == out is fine).
+struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; };
 // launchers implemented in qmat.hip, used by the block / model code
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 // K range split over `ksplit` workgroups per row tile; partial[(ks*t_count + t)*tiles*64 + row] holds the slice sums and
@@ -71,6 +77,8 @@ int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t,
 int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit);
 // t = 1 GEMV that also leaves, per row tile, (bits of the maximum, first row holding it) in best[2*tile], best[2*tile+1].
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev);
+// y as pyre_gemv_launch (raw projections), plus the conv epilogue described at GemvEpi (best ignored).
+int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, const GemvEpi& conv);
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev, int n, float* out_dev, int out_stride);
 // Greedy pick from per-tile maxima (first maximum overall) -> id_out[0] (and mirror[0] if given); when m is given the
 // chosen row is dequantized into out_dev in the same launch (the next token's embedding).
@@ -136,8 +144,9 @@ int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, co
 struct GdnDev { const float* a; const float* dt; const float* conv_w; const float* norm_w; int nk, nv, dk, dv, conv_k; float eps; };
 // proj [t][ch + nv*dv + 2*nv] = [qkv | z | beta | alpha] per token (row stride = proj_stride floats).
 // conv_in/conv_out [(k-1)][ch], ssm_in/ssm_out [nv][dk][dv] (in != out).  co_scratch [8][ch].  out [t][nv*dv].
+// conv_done: co_scratch already holds silu(conv) of the window and the conv state has been advanced (GemvEpi).
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev);
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false);
 
 // Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
 // scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].

@@ -88,12 +88,12 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co, float* out) {
+                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done) {
   if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
   if (g.conv_k < 2 || g.conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: conv kernel %d outside 2..8", g.conv_k);
   if (t < 1) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d", t);
   int ch = 2 * g.nk * g.dk + g.nv * g.dv;
-  { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
+  if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }

@@ -265,8 +265,9 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = replay ? b : b ^ 1;
-      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, pj))) return rc;
-      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core))) return rc;
+      GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
+      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv))) return rc;
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true))) return rc;
       s->cur[li] = nb;
     }
     if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;

@@ -9,7 +9,7 @@
 // weight, and a separate launch would cost more than redoing this small selection everywhere).
 // Two-level selection: wave w < ceil(n_exp/64) ranks its own 64 logits through lane broadcasts and keeps its best k as
 // candidates (an expert outside its wave's best k cannot be in the global best k); the candidates are then ranked
-// against each other from shared memory.  Leaves ids (ascending) in s_idx[0..k) and weights in s_w[0..k).
+// against each other from shared memory.  Leaves the chosen ids (ascending) in s_idx[0..k) and their logits in s_val[0..k).
 struct RouteLds { float c_val[16 * 32]; int c_idx[16 * 32]; float r_val[32]; int r_idx[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
 __device__ __forceinline__ void route_topk(const float* __restrict__ logits, int n_exp, int k, RouteLds& L) {
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6, nwa = (n_exp + 63) >> 6;
@@ -22,16 +22,27 @@ __device__ __forceinline__ void route_topk(const float* __restrict__ logits, int
     if (lr < k) { L.c_val[wave * k + lr] = v; L.c_idx[wave * k + lr] = e; }
   }
   __syncthreads();
-  const int nc = nwa * k;
-  if (e < nc) {
-    float cv = L.c_val[e]; int ci = L.c_idx[e], rank = 0;
-#pragma unroll 16
-    for (int j = 0; j < nc; ++j) { float u = L.c_val[j]; int ui = L.c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
-    if (rank < k) { L.r_val[rank] = cv; L.r_idx[rank] = ci; }
+  // candidate c is ranked by SP threads, each against a slice of the candidates; the SP counts meet through shuffles
+  const int nc = nwa * k; int SP = 8; while (SP > 1 && nc * SP > (int)blockDim.x) SP >>= 1;
+  {
+    const int c = e / SP, part = e % SP, per = (nc + SP - 1) / SP; int rank = 0;
+    float cv = 0.0f; int ci = 0;
+    if (c < nc) {
+      cv = L.c_val[c]; ci = L.c_idx[c];
+      const int j1 = min(nc, (part + 1) * per);
+#pragma unroll 4
+      for (int j = part * per; j < j1; ++j) { float u = L.c_val[j]; int ui = L.c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
+    }
+    for (int o = 1; o < SP; o <<= 1) rank += __shfl_xor(rank, o);
+    if (c < nc && part == 0 && rank < k) { L.r_val[rank] = cv; L.r_idx[rank] = ci; }
   }
   __syncthreads();
   if (e < k) { int me = L.r_idx[e], pos = 0; for (int j = 0; j < k; ++j) pos += L.r_idx[j] < me ? 1 : 0; L.s_idx[pos] = me; L.s_val[pos] = L.r_val[e]; }
   __syncthreads();
+}
+// softmax over the chosen logits in ascending expert id (soft_top); called by the whole workgroup after route_topk
+__device__ __forceinline__ void route_weights(int k, RouteLds& L) {
+  const int e = threadIdx.x;
   float mx = -INFINITY, ex = 1.0f;
   if (e < k) { for (int i = 0; i < k; ++i) mx = fmaxf(mx, L.s_val[i]); ex = isfinite(mx) ? expf(L.s_val[e] - mx) : 1.0f; L.r_val[e] = ex; }
   __syncthreads();
@@ -41,7 +52,6 @@ __device__ __forceinline__ void route_topk(const float* __restrict__ logits, int
     else { float sum = 0.0f; for (int i = 0; i < k; ++i) sum += L.r_val[i]; w = ex / sum; }
     L.s_w[e] = w;
   }
-  __syncthreads();
 }
 
 // ---- routing + expert gate/up: h[entry][r] = silu(gate[r] . x) * (up[r] . x) -------------------------------------------
@@ -92,7 +102,10 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   // activations in scalar registers (it could no longer prove them unmodified).
   if (blockIdx.x == 0) {
     if (shared) { if (threadIdx.x == 0) sg[ti] = rl.s_w[0]; }
-    else if (j == 0 && threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
+    else if (j == 0) {
+      route_weights(m.top_k, rl);       // thread e < k writes and then reads its own s_w entry
+      if (threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
+    }
   }
 }
 

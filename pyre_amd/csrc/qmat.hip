@@ -87,12 +87,19 @@ template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const
 //   best != nullptr (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 template <int FMT, int T, int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int upw,
-                                                  uint32_t* __restrict__ best, const uint2* __restrict__ g2) {
+                                                  GemvEpi ep, const uint2* __restrict__ g2) {
   __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
   __shared__ float red[NW][T][64];
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  // conv epilogue: wave 0 fetches its rows' taps and state first, so the loads overlap the dot products
+  float cw[8], chist[8]; const bool conv_row = ep.co != nullptr && wave == 0 && tile * 64 + lane < ep.ch;
+  if (conv_row) {
+    const size_t row = (size_t)tile * 64 + lane;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { cw[k] = k < ep.kk ? ep.conv_w[row * ep.kk + k] : 0.0f; chist[k] = k < ep.kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
+  }
   const int k0 = (ks * NW + wave) * upw; const int k1 = min(m.U, k0 + upw);
   float acc[T];
 #pragma unroll
@@ -109,44 +116,65 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
     size_t row = (size_t)tile * 64 + l;
     if (ksplit == 1) { if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s; }
     else y[((size_t)ks * T + t) * r64 + row] = s;
-    if (T == 1 && best != nullptr) {       // threads 0..63 = wave 0: first maximum of the tile (sampler::argmax order)
+    if (T == 1 && ep.best != nullptr) {       // threads 0..63 = wave 0: first maximum of the tile (sampler::argmax order)
       float bv = row < (size_t)m.rows ? s : -INFINITY; uint32_t bi = (uint32_t)row;
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; } }
-      if (l == 0) { best[2 * tile] = __float_as_uint(bv); best[2 * tile + 1] = bi; }
+      if (l == 0) { ep.best[2 * tile] = __float_as_uint(bv); ep.best[2 * tile + 1] = bi; }
     }
+  }
+  if (conv_row) {      // linear_core's conv1d + SiLU for this row, tokens in order (qwen4exp_gguf.rs:1643-1647)
+    const size_t row = (size_t)tile * 64 + lane;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float cur = red[0][t][lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) cur += red[w][t][lane];
+      float o = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) if (k == ep.kk - 1) o = cw[k] * cur;
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) o += cw[k] * chist[k];
+      ep.co[(size_t)t * ep.ch + row] = o * (1.0f / (1.0f + expf(-o)));
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k + 1 < ep.kk - 1) chist[k] = chist[k + 1];
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k == ep.kk - 2) chist[k] = cur;
+    }
+#pragma unroll
+    for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
   }
 }
 
 namespace {
 int env_int(const char* n, int dflt) { const char* v = getenv(n); return v && *v ? atoi(v) : dflt; }
 
-template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, uint32_t* best) {
+template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
   static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   FmtGeom g = fmt_geom(FMT);
   ProfScope ps(ctx, name.c_str(), (double)m.rows * (m.cols / g.el) * g.bytes + 4.0 * T * ((double)m.cols + m.rows));
-  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, best, (const uint2*)ctx->d_iq2xs);
+  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 // Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
 // fewer when there are so many tiles that the chip is full anyway.
-template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, uint32_t* best) {
+template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   static const int force = env_int("PYRE_GEMV_NW", 0);
   int per_wg = (m.U + ksplit - 1) / ksplit;
   int nw = m.tiles >= 1024 ? 4 : (m.tiles >= 256 ? 8 : 16);
   while (nw > 1 && nw / 2 >= per_wg) nw /= 2;          // no idle waves
   if (nw < 4) nw = 4;
   if (force == 4 || force == 8 || force == 16) nw = force;
-  if (nw == 4) return gemv_launch_nw<FMT, T, 4>(ctx, m, x, y, ksplit, best);
-  if (nw == 8) return gemv_launch_nw<FMT, T, 8>(ctx, m, x, y, ksplit, best);
-  return gemv_launch_nw<FMT, T, 16>(ctx, m, x, y, ksplit, best);
+  if (nw == 4) return gemv_launch_nw<FMT, T, 4>(ctx, m, x, y, ksplit, ep);
+  if (nw == 8) return gemv_launch_nw<FMT, T, 8>(ctx, m, x, y, ksplit, ep);
+  return gemv_launch_nw<FMT, T, 16>(ctx, m, x, y, ksplit, ep);
 }
-template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, uint32_t* best) {
-  switch (t) { case 1: return gemv_t<FMT, 1>(ctx, m, x, y, ksplit, best); case 2: return gemv_t<FMT, 2>(ctx, m, x, y, ksplit, best); case 3: return gemv_t<FMT, 3>(ctx, m, x, y, ksplit, best);
-    case 4: return gemv_t<FMT, 4>(ctx, m, x, y, ksplit, best); case 5: return gemv_t<FMT, 5>(ctx, m, x, y, ksplit, best); case 6: return gemv_t<FMT, 6>(ctx, m, x, y, ksplit, best);
-    case 7: return gemv_t<FMT, 7>(ctx, m, x, y, ksplit, best); case 8: return gemv_t<FMT, 8>(ctx, m, x, y, ksplit, best); }
+template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, const GemvEpi& ep) {
+  switch (t) { case 1: return gemv_t<FMT, 1>(ctx, m, x, y, ksplit, ep); case 2: return gemv_t<FMT, 2>(ctx, m, x, y, ksplit, ep); case 3: return gemv_t<FMT, 3>(ctx, m, x, y, ksplit, ep);
+    case 4: return gemv_t<FMT, 4>(ctx, m, x, y, ksplit, ep); case 5: return gemv_t<FMT, 5>(ctx, m, x, y, ksplit, ep); case 6: return gemv_t<FMT, 6>(ctx, m, x, y, ksplit, ep);
+    case 7: return gemv_t<FMT, 7>(ctx, m, x, y, ksplit, ep); case 8: return gemv_t<FMT, 8>(ctx, m, x, y, ksplit, ep); }
   return pyre_fail(ctx, PYRE_E_ARG, "qmatmul: t = %d outside 1..8", t);
 }
 #define FMT_DISPATCH(fmt, CALL) \
@@ -157,17 +185,24 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
 
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
   int rc = PYRE_OK;
-  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, nullptr));
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, GemvEpi{}));
   return rc;
 }
 int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* partial, int ksplit) {
   int rc = PYRE_OK;
-  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, partial, ksplit, nullptr));
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, partial, ksplit, GemvEpi{}));
   return rc;
 }
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best) {
   int rc = PYRE_OK;
-  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, 1, y, 1, best));
+  GemvEpi ep{}; ep.best = best;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, 1, y, 1, ep));
+  return rc;
+}
+int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, const GemvEpi& conv) {
+  if (!conv.co || !conv.conv_w || !conv.conv_in || !conv.conv_out || conv.kk < 2 || conv.kk > 8 || conv.ch < 1 || conv.ch > m.rows) return pyre_fail(ctx, PYRE_E_ARG, "gemv: bad conv epilogue (kernel %d, %d channels of %d rows)", conv.kk, conv.ch, m.rows);
+  GemvEpi ep = conv; ep.best = nullptr; int rc = PYRE_OK;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, ep));
   return rc;
 }
 
