@@ -100,13 +100,27 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
 }
 
 // ---- factored per-unit dot products for the GEMV ------------------------------------------------------------------
+// A unit's packed data is fetched first (unit_load) and consumed later (unit_fma), so a kernel can issue the weight
+// loads ahead of a barrier or of the previous unit's arithmetic; unit_dot does both at once.
+template <int FMT> struct UnitRaw { uint4 v[FMT == FMT_F32 ? 16 : (FMT == FMT_F16 || FMT == FMT_BF16) ? 8 : FMT == FMT_Q8_0 ? 4 : (FMT == FMT_Q4_K || FMT == FMT_IQ3_S) ? 2 : 1]; uint4 hb; uint32_t s0, s1; };
+template <int FMT> __device__ __forceinline__ UnitRaw<FMT> unit_load(const QMatDev& m, int tile, int ku, int lane) {
+  UnitRaw<FMT> r; r.hb = uint4{0, 0, 0, 0}; r.s0 = 0; r.s1 = 0;
+  constexpr int V = sizeof(r.v) / sizeof(uint4);
+#pragma unroll
+  for (int c = 0; c < V; ++c) r.v[c] = ld_vec<V>(m, tile, ku, c, lane);
+  if constexpr (FMT == FMT_Q8_0) r.s0 = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
+  if constexpr (FMT == FMT_Q4_K) r.hb = ld_block<uint4>(m, tile, ku, lane);
+  if constexpr (FMT == FMT_IQ2_XS) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint16_t>(m.p1, m, tile, ku, lane); }
+  if constexpr (FMT == FMT_IQ3_S) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint8_t>(m.p3, m, tile, ku, lane); }
+  return r;
+}
 // xs points at the unit's 64 activations of token 0 (wave-uniform address -> scalar loads); token t is xs + t*xstride.
 // acc[t] += sum_j W[row, 64*ku + j] * x[t][64*ku + j].  The operation sequence per token does not depend on T.
-template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint2* lds2, int tile, int ku, int lane,
+template <int FMT, int T> __device__ __forceinline__ void unit_fma(const UnitRaw<FMT>& r, int ku, const uint2* lds2, int lane,
                                                                    const float* __restrict__ xs, int xstride, float (&acc)[T]) {
   if constexpr (FMT == FMT_F32) {
 #pragma unroll
-    for (int c = 0; c < 16; ++c) { uint4 v = ld_vec<16>(m, tile, ku, c, lane); float w[4] = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+    for (int c = 0; c < 16; ++c) { uint4 v = r.v[c]; float w[4] = {__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
 #pragma unroll
       for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -114,7 +128,7 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
   } else if constexpr (FMT == FMT_F16 || FMT == FMT_BF16) {
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      uint4 v = ld_vec<8>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint4 v = r.v[c]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         float lo = FMT == FMT_F16 ? h2f_bits(w[k]) : __uint_as_float(w[k] << 16), hi = FMT == FMT_F16 ? h2f_bits(w[k] >> 16) : __uint_as_float(w[k] & 0xFFFF0000u);
@@ -123,7 +137,7 @@ template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev
       }
     }
   } else if constexpr (FMT == FMT_Q8_0) {
-    uint32_t dd = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
+    uint32_t dd = r.s0;
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       float part[T];
@@ -131,7 +145,7 @@ _Pragma("unroll")
       for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
-        uint4 v = ld_vec<4>(m, tile, ku, 2 * b + c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint4 v = r.v[2 * b + c]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int k = 0; k < 16; ++k) { float f = (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3)));
 #pragma unroll
@@ -142,13 +156,13 @@ _Pragma("unroll")
       for (int t = 0; t < T; ++t) acc[t] = fmaf(d, part[t], acc[t]);
     }
   } else if constexpr (FMT == FMT_Q4_K) {
-    uint4 hb = ld_block<uint4>(m, tile, ku, lane);
+    uint4 hb = r.hb;
     float d = h2f_bits(hb.x), mn = h2f_bits(hb.x >> 16);
     int j = ku & 3; uint32_t s1, m1, s2, m2; scale_min_k4(2 * j, hb.y, hb.z, hb.w, s1, m1); scale_min_k4(2 * j + 1, hb.y, hb.z, hb.w, s2, m2);
     float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
-      uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      uint4 v = r.v[c]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
       for (int k = 0; k < 16; ++k) {
         uint32_t b = (w[k >> 2] >> (8 * (k & 3))) & 0xFF;
@@ -158,9 +172,9 @@ _Pragma("unroll")
       }
     }
   } else if constexpr (FMT == FMT_IQ2_XS) {
-    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
-    uint32_t sc = ld_small<uint16_t>(m.p1, m, tile, ku, lane);
-    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float d = h2f_bits(r.s0);
+    uint32_t sc = r.s1;
+    uint4 v = r.v[0]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib) {
       uint32_t s = (sc >> (8 * ib)) & 0xFF;
@@ -188,9 +202,9 @@ _Pragma("unroll")
       }
     }
   } else {   // IQ3_S from 4-bit codes c = (w + 15) / 2: sum w x = 2 sum c x - 15 sum x per 32-value sub-block
-    float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
-    uint32_t sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
-    uint4 v0 = ld_vec<2>(m, tile, ku, 0, lane), v1 = ld_vec<2>(m, tile, ku, 1, lane);
+    float d = h2f_bits(r.s0);
+    uint32_t sc = r.s1;
+    uint4 v0 = r.v[0], v1 = r.v[1];
     uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
     float sx[T][2];            // sub-block sums of the activations: lane j holds x[j], folded inside each half of the wave
 #pragma unroll
@@ -220,4 +234,9 @@ _Pragma("unroll")
       for (int t = 0; t < T; ++t) acc[t] = fmaf(db, fmaf(-15.0f, sx[t][sb], 2.0f * part[t]), acc[t]);
     }
   }
+}
+template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint2* lds2, int tile, int ku, int lane,
+                                                                   const float* __restrict__ xs, int xstride, float (&acc)[T]) {
+  UnitRaw<FMT> r = unit_load<FMT>(m, tile, ku, lane);
+  unit_fma<FMT, T>(r, ku, lds2, lane, xs, xstride, acc);
 }

@@ -35,9 +35,13 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
+  UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);     // in flight across both barriers
   float w[T], ss[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) { w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
+  float mine[T];        // upw == 1: the slice element this thread normalizes later, fetched with the others
+#pragma unroll
+  for (int t = 0; t < T; ++t) mine[t] = upw == 1 ? hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid) : 0.0f;
   for (int i = tid; i < d; i += nthr) {
 #pragma unroll
     for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i); ss[t] += v * v; }
@@ -56,7 +60,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
     const float nv = norm[(size_t)s * d + i0 + j];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
+      float v = upw == 1 ? mine[t] : hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
       float o = v * sc[t] * nv;                                   // rms, :209: (x * s) * w
       xs[(size_t)t * L + j] = o;
       if (tile == 0) { size_t k = ((size_t)t * hc + s) * d + i0 + j; xn[k] = o; x_out[k] = v; }
@@ -66,7 +70,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; unit_dot<FMT, T>(m, lds2, tile, ks * nw * upw + lu, lane, xs + lu * 64, L, acc); }
+  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, T>(raw, ks * nw * upw + lu, lds2, lane, xs + lu * 64, L, acc); }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
@@ -91,25 +95,29 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
   if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int n_o = lr + hc;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int s = wave / U, ku = wave - s * U;
+  UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);        // in flight across the prologue
   for (int idx = tid; idx < T * n_o; idx += nthr) {
     int t = idx / n_o, i = idx - t * n_o;
     float o = 0.0f;
     if (i < lr || has_inject) {
-      o = part[(size_t)t * r64 + i];
-#pragma unroll 4
-      for (int ks = 1; ks < ksplit; ++ks) o += part[((size_t)ks * T + t) * r64 + i];
+      float pv[32];                 // every slice is fetched before the first add: one round trip
+#pragma unroll
+      for (int ks = 0; ks < 32; ++ks) pv[ks] = ks < ksplit ? part[((size_t)ks * T + t) * r64 + i] : 0.0f;
+      o = pv[0];
+#pragma unroll
+      for (int ks = 1; ks < 32; ++ks) if (ks < ksplit) o += pv[ks];
     }
     float v = o / (float)hc;
     if (i < lr) lo[t * lr + i] = v * sigm(v);
     else if (blockIdx.x == 0) inj[t * hc + (i - lr)] = has_inject ? v : 0.0f;
   }
   __syncthreads();
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int s = wave / U, ku = wave - s * U;
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  unit_dot<FMT, T>(up, lds2, s * (d >> 6) + blockIdx.x, ku, lane, lo + ku * 64, lr, acc);
+  unit_fma<FMT, T>(raw, ku, lds2, lane, lo + ku * 64, lr, acc);
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
