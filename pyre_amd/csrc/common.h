@@ -72,6 +72,8 @@ struct pyre_qmat {
 struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; };
 // launchers implemented in qmat.hip, used by the block / model code
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+// waves per workgroup and units per wave the (unsplit) GEMV uses for this matrix
+void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw);
 // K range split over `ksplit` workgroups per row tile; partial[(ks*t_count + t)*tiles*64 + row] holds the slice sums and
 // the consumer adds them in slice order.
 int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit);
@@ -138,6 +140,8 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // must not overlap x_in.  mixed [t][d] and inj [t][hc] = hc_mix(updated streams).
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
                        float eps, float* mixed_dev, float* inj_dev);
+// waves per workgroup, units per wave and K slices of the norm + [down ; inject] kernel; false if the shape is unsupported
+bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit);
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, const float* out_dev, const float* inj_dev);
 
 // ---- Gated DeltaNet (gdn.hip) -----------------------------------------------------------------------------------------

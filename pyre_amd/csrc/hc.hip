@@ -180,6 +180,11 @@ int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, fl
 }
 }  // namespace
 
+bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit) {
+  if (h.d % 64 || h.lr % 64 || h.hc * h.up.U > 16 || h.up.tiles != h.hc * (h.d / 64) || h.di.U != h.hc * (h.d / 64)) return false;
+  DownPlan p = down_plan(h); *nw = p.nw; *upw = p.upw; *ksplit = p.ksplit;
+  return p.ksplit >= 1 && p.ksplit <= 32 && p.ksplit * p.nw * p.upw == h.di.U;
+}
 size_t pyre_hc_work_bytes(const HcDev& h) { size_t w = (size_t)h.hc * h.d; return 256 * 3 + 4 * 8 * w + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
 void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };

@@ -3,6 +3,7 @@
 // greedy loop.  Follows Model::forward_inner / forward_multi / spec_keep (src/model/qwen4exp_gguf.rs:2087-2157,
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
+#include "mega.h"
 #include <memory>
 #include <stdlib.h>
 
@@ -29,6 +30,8 @@ struct pyre_model {
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
   float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
+  int mega_ok = -1;               // persistent-kernel decode: -1 not probed, 0 unsupported shape/types, 1 usable
+  std::vector<mega::Layer> mega_layers; mega::Args mega_args{}; mega::Layer* mega_dev = nullptr; unsigned* mega_ctl = nullptr; int mega_wgs = 0;
 };
 
 struct pyre_state {
@@ -183,7 +186,8 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
 
 void pyre_model_destroy(pyre_model* m) {
   if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
-  for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); if (m->toks) (void)hipFree(m->toks); delete m;
+  for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); if (m->toks) (void)hipFree(m->toks);
+  if (m->mega_dev) (void)hipFree(m->mega_dev); if (m->mega_ctl) (void)hipFree(m->mega_ctl); delete m;
 }
 size_t pyre_model_weight_bytes_per_token(const pyre_model* m) { return m ? m->token_weight_bytes : 0; }
 
@@ -292,6 +296,82 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }
 
+// ---- persistent-kernel decode (mega.h) ------------------------------------------------------------------------------------
+// Usable when every matrix but the router is IQ3_S, the router is bf16, and the shapes fit the kernel's stages; anything
+// else keeps the launch-per-stage path.
+bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
+  if (m->mega_ok >= 0) return m->mega_ok == 1;
+  m->mega_ok = 0;
+  const pyre_model_cfg& c = m->c;
+  auto w_ok = [](const QMatDev& q) { return q.fmt == FMT_IQ3_S; };
+  auto hc_ok = [&](const HcDev& h, mega::HcPlan* p) { return w_ok(h.di) && w_ok(h.up) && pyre_hc_plan(h, &p->nw, &p->upw, &p->ksplit); };
+  if (c.top_k > PYRE_MOE_KMAX || c.hd != 256 || c.lin_dk != 128 || c.lin_dv != 128 || c.conv_k < 2 || c.conv_k > 8 || c.n_exp > 1024) return false;
+  if (!w_ok(m->embd) || !w_ok(m->out)) return false;
+  mega::Args& a = m->mega_args; a = mega::Args{};
+  if (!hc_ok(m->head, &a.ph)) return false;
+  m->mega_layers.assign(c.n_layers, mega::Layer{});
+  for (int il = 0; il < c.n_layers; ++il) {
+    const Layer& L = m->layers[il]; mega::Layer& M = m->mega_layers[il];
+    if (!hc_ok(L.hca, &M.pa) || !hc_ok(L.hcf, &M.pf) || !w_ok(L.proj) || !w_ok(L.outp)) return false;
+    const MoeDev& mo = L.moe;
+    if (mo.router.fmt != FMT_BF16 || !w_ok(mo.gate_e) || !w_ok(mo.up_e) || !w_ok(mo.down_e) || !w_ok(mo.sh_gate) || !w_ok(mo.sh_up) || !w_ok(mo.sh_down)) return false;
+    if (L.full) { int G = L.attn.nh / L.attn.nkv; if (L.attn.nh % L.attn.nkv || (G != 1 && G != 2 && G != 4 && G != 8)) return false; }
+    else if (L.gdn.nv % L.gdn.nk) return false;
+    if ((size_t)L.proj.cols * 4 + 4096 > mega::LDS_BYTES || (size_t)L.outp.cols * 4 + 4096 > mega::LDS_BYTES) return false;
+    M.hca = L.hca; M.hcf = L.hcf; M.proj = L.proj; M.outp = L.outp; M.moe = L.moe; M.attn = L.attn; M.gdn = L.gdn; M.full = L.full ? 1 : 0;
+    pyre_gemv_plan(L.proj, &M.gp.nw, &M.gp.upw); pyre_gemv_plan(L.outp, &M.go.nw, &M.go.upw); pyre_gemv_plan(mo.router, &M.gr.nw, &M.gr.upw);
+  }
+  if ((size_t)c.d * 4 + 8192 + sizeof(mega::RouteLds) > mega::LDS_BYTES) return false;
+  hipDeviceProp_t prop; if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return false;
+  int wgs = prop.multiProcessorCount; if (wgs > 256) wgs = 256; if (wgs < 32) return false;
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)mega::k_decode<FMT_IQ3_S, FMT_BF16>, mega::WGT, mega::LDS_BYTES) != hipSuccess || per_cu < 1) return false;
+  if (hipMalloc((void**)&m->mega_dev, sizeof(mega::Layer) * c.n_layers) != hipSuccess) return false;
+  if (hipMalloc((void**)&m->mega_ctl, 4096) != hipSuccess) return false;
+  m->mega_wgs = wgs;
+  a.n_layers = c.n_layers; a.head = m->head; a.embd = m->embd; a.out = m->out; pyre_gemv_plan(m->out, &a.gh.nw, &a.gh.upw);
+  a.d = c.d; a.hc = c.hc; a.ch = m->ch; a.pw_lin = m->pw_lin; a.pw_attn = m->pw_attn; a.conv_k = c.conv_k; a.eps = c.eps;
+  a.emb = m->emb; a.xa = m->x; a.xb = m->x2; a.xn = m->hw.xn; a.part = m->hw.o; a.mixed = m->mixed; a.inj_a = m->inj_a; a.inj_f = m->inj_f; a.proj = m->proj; a.co = m->co; a.core = m->core;
+  a.o = m->o; a.hbuf = m->hbuf; a.vlogits = m->logits; a.best = m->best; a.mw = m->mw; a.ctl = m->mega_ctl; a.limit = 4000000u;
+  m->mega_ok = 1; return true;
+}
+
+int mega_decode(pyre_ctx* ctx, pyre_model* m, pyre_state* s, uint32_t first, int n_steps) {
+  // per-state pointers: recurrent state in place in the current buffers, KV caches, raw-projection rows
+  int li = 0, ai = 0;
+  for (int il = 0; il < m->c.n_layers; ++il) {
+    mega::Layer& M = m->mega_layers[il];
+    if (M.full) { M.kv = s->kv[ai]; ++ai; }
+    else { M.conv = s->conv[s->cur[li]][li]; M.ssm = s->ssm[s->cur[li]][li]; M.proj_saved = s->proj_saved[li]; ++li; }
+  }
+  PYRE_HIP(ctx, hipMemcpyAsync(m->mega_dev, m->mega_layers.data(), sizeof(mega::Layer) * m->mega_layers.size(), hipMemcpyHostToDevice, ctx->stream));
+  const int chunk = 256;                       // tokens per launch
+  for (int done = 0; done < n_steps; done += chunk) {
+    int n = n_steps - done < chunk ? n_steps - done : chunk;
+    mega::Args a = m->mega_args; a.layers = m->mega_dev; a.aw = s->aw; a.toks = m->toks + done; a.n_steps = n; a.start_pos = s->len + done;
+    a.first = first;
+    if (done > 0) {   // continue from the previous launch's last pick
+      PYRE_HIP(ctx, hipMemcpyAsync(&a.first, m->toks + done - 1, 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    PYRE_HIP(ctx, hipMemsetAsync(m->mega_ctl, 0, 4096, ctx->stream));
+    { const char* e = getenv("PYRE_MEGA_TIMES"); a.stage_ticks = e && atoi(e) ? (unsigned long long*)(m->mega_ctl + 512) : nullptr; }
+    void* args[] = {&a};
+    { ProfScope ps(ctx, "decode_persistent", 0.0);
+      PYRE_HIP(ctx, hipLaunchCooperativeKernel((const void*)mega::k_decode<FMT_IQ3_S, FMT_BF16>, dim3(m->mega_wgs), dim3(mega::WGT), args, mega::LDS_BYTES, ctx->stream)); }
+    unsigned flags[32];
+    PYRE_HIP(ctx, hipMemcpyAsync(flags, m->mega_ctl, sizeof(flags), hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (a.stage_ticks) {
+      unsigned long long tk[16]; PYRE_HIP(ctx, hipMemcpy(tk, a.stage_ticks, sizeof(tk), hipMemcpyDeviceToHost));
+      static const char* nm[13] = {"pick_embed", "hc_norm_down", "hc_up_mix", "proj_gemv", "attn_prep", "attn_decode", "attn_combine", "gdn_delta", "out_gemv", "router_gemv", "route_gate_up", "moe_down", "head_gemv"};
+      fprintf(stderr, "[pyre] persistent decode, %d tokens, us per token by stage class (incl. the barrier after it):\n", n);
+      double tot = 0; for (int i = 0; i < 13; ++i) { double us = tk[i] * 0.01 / n; tot += us; fprintf(stderr, "[pyre]   %-14s %9.1f\n", nm[i], us); }
+      fprintf(stderr, "[pyre]   %-14s %9.1f\n", "total", tot);
+    }
+    if (flags[16]) return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: the persistent kernel gave up waiting at barrier round %u", flags[0]);
+  }
+  return PYRE_OK;
+}
+
 int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
   for (int i = 0; i < n; ++i) if (ids[i] >= (uint32_t)m->c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "forward: token id %u outside the vocabulary (%d)", ids[i], m->c.vocab);
   return PYRE_OK;
@@ -356,6 +436,15 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
   int rc = check_ids(ctx, m, &first, 1); if (rc) return rc;
   if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }
   s->last_window = 0;
+  { const char* e = getenv("PYRE_MEGA"); const int want = e && *e ? atoi(e) : 0;      // 1: use it when the model qualifies, 2: fail if it does not
+    if (want == 2 && !mega_probe(ctx, m)) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_decode_greedy_dev: the persistent decode kernel does not support this model (types or shapes)");
+    if (want && !ctx->prof_on && mega_probe(ctx, m)) {
+      if ((rc = mega_decode(ctx, m, s, first, n_steps))) return rc;
+      s->len += n_steps;
+      for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
+      if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+      return PYRE_OK;
+    } }
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
   { WinOpt o; o.greedy = true; if ((rc = run_window(ctx, m, s, 1, o))) return rc; }
   if (n_steps > 1) {

@@ -149,6 +149,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
 namespace {
 int env_int(const char* n, int dflt) { const char* v = getenv(n); return v && *v ? atoi(v) : dflt; }
 
+int gemv_nw(const QMatDev& m, int ksplit) {
+  static const int force = env_int("PYRE_GEMV_NW", 0);
+  int per_wg = (m.U + ksplit - 1) / ksplit;
+  int nw = m.tiles >= 1024 ? 4 : (m.tiles >= 256 ? 8 : 16);
+  while (nw > 1 && nw / 2 >= per_wg) nw /= 2;          // no idle waves
+  if (nw < 4) nw = 4;
+  if (force == 4 || force == 8 || force == 16) nw = force;
+  return nw;
+}
 template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
   static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s"};
@@ -161,12 +170,7 @@ template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDe
 // Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
 // fewer when there are so many tiles that the chip is full anyway.
 template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
-  static const int force = env_int("PYRE_GEMV_NW", 0);
-  int per_wg = (m.U + ksplit - 1) / ksplit;
-  int nw = m.tiles >= 1024 ? 4 : (m.tiles >= 256 ? 8 : 16);
-  while (nw > 1 && nw / 2 >= per_wg) nw /= 2;          // no idle waves
-  if (nw < 4) nw = 4;
-  if (force == 4 || force == 8 || force == 16) nw = force;
+  int nw = gemv_nw(m, ksplit);
   if (nw == 4) return gemv_launch_nw<FMT, T, 4>(ctx, m, x, y, ksplit, ep);
   if (nw == 8) return gemv_launch_nw<FMT, T, 8>(ctx, m, x, y, ksplit, ep);
   return gemv_launch_nw<FMT, T, 16>(ctx, m, x, y, ksplit, ep);
@@ -183,6 +187,7 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
 }  // namespace
 
+void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw) { *nw = gemv_nw(m, 1); *upw = (m.U + *nw - 1) / *nw; if (*upw < 1) *upw = 1; }
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
   int rc = PYRE_OK;
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, GemvEpi{}));
