@@ -19,6 +19,10 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
   const float* row = qkv + (size_t)ti * stride;
   const float* src = is_k ? row + (size_t)a.nh * 2 * HD + (size_t)h * HD : row + (size_t)h * 2 * HD;
   float v = src[tid];
+  // the norm weight, the rotation frequency and the value element are fetched now, ahead of the barriers
+  const int half = a.n_rot / 2, ri = tid < half ? tid : tid - half;
+  const float nwt = is_k ? a.kn[tid] : a.qn[tid], rinv = tid < a.n_rot ? a.rope_inv[ri] : 0.0f;
+  const float vrow = is_k ? row[(size_t)a.nh * 2 * HD + (size_t)a.nkv * HD + (size_t)h * HD + tid] : 0.0f;
   float ss = v * v;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
@@ -28,20 +32,19 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) tot += red[i];
   const float sc = 1.0f / sqrtf(tot / (float)HD + a.eps);
-  v = v * (sc * (is_k ? a.kn[tid] : a.qn[tid]));            // rms_inplace: x *= s * w
+  v = v * (sc * nwt);            // rms_inplace: x *= s * w
   buf[tid] = v;
   __syncthreads();
-  const int half = a.n_rot / 2;
   if (tid < a.n_rot) {
-    int i = tid < half ? tid : tid - half;
-    float ang = (float)pos * a.rope_inv[i];
+    int i = ri;
+    float ang = (float)pos * rinv;
     float sn = sinf(ang), cs = cosf(ang);
     float x0 = buf[i], x1 = buf[i + half];
     v = tid < half ? x0 * cs - x1 * sn : x1 * cs + x0 * sn;
   }
   if (is_k) {
     kv.kf[kv_blk((size_t)h * HD + tid, (size_t)a.nkv * HD, pos)] = v;
-    kv.vf[(size_t)pos * a.nkv * HD + (size_t)h * HD + tid] = row[(size_t)a.nh * 2 * HD + (size_t)a.nkv * HD + (size_t)h * HD + tid];
+    kv.vf[(size_t)pos * a.nkv * HD + (size_t)h * HD + tid] = vrow;
   } else qout[((size_t)ti * a.nh + h) * HD + tid] = v;
 }
 

@@ -45,6 +45,9 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     // L2 norms of q (threads 0..127) and k (threads 128..255) of key head kh (:1649-1651)
     float v = 0.0f;
     if (tid < DK) v = co[kh * DK + tid]; else if (tid < 2 * DK) v = co[p.nk * DK + kh * DK + (tid - DK)];
+    // everything else this token needs from memory is fetched now, ahead of the barriers
+    const float alpha_raw = pr[ch + w + p.nv + h], beta_raw = pr[ch + w + h], v_j = co[2 * p.nk * DK + h * DV + j];
+    const float z_j = tid < DV ? pr[ch + h * DV + j] : 0.0f, nw_j = tid < DV ? p.norm_w[j] : 0.0f;
     float sq = v * v;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
@@ -52,8 +55,8 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     __syncthreads();
     if (tid < DK) qs[tid] = v * ((1.0f / sqrtf(red[0] + red[1] + 1e-6f)) * (1.0f / sqrtf((float)DK)));
     else if (tid < 2 * DK) ks[tid - DK] = v * ((1.0f / sqrtf(red[2] + red[3] + 1e-6f)) * 1.0f);
-    const float g = expf(g_softplus(pr[ch + w + p.nv + h] + dtb) * a);      // alpha at [ch + nv*dv + nv + h]
-    const float b = g_sigm(pr[ch + w + h]);                                 // beta  at [ch + nv*dv + h]
+    const float g = expf(g_softplus(alpha_raw + dtb) * a);      // alpha at [ch + nv*dv + nv + h]
+    const float b = g_sigm(beta_raw);                                 // beta  at [ch + nv*dv + h]
     __syncthreads();
     float pmv = 0.0f;
 #pragma unroll
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     pm[grp][j] = pmv;
     __syncthreads();
     const float mem = ((pm[0][j] + pm[1][j]) + pm[2][j]) + pm[3][j];
-    const float delta = (co[2 * p.nk * DK + h * DV + j] - mem) * b;
+    const float delta = (v_j - mem) * b;
     float pov = 0.0f;
 #pragma unroll
     for (int r = 0; r < R; ++r) { S[r] += ks[grp * R + r] * delta; pov += S[r] * qs[grp * R + r]; }
@@ -78,8 +81,8 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     __syncthreads();
     if (tid < DV) {
       float sc = 1.0f / sqrtf((red[4] + red[5]) / (float)DV + p.eps);
-      float o = pm[0][j] * (sc * p.norm_w[j]);                              // rms_inplace: x *= s * w  (:210)
-      out[(size_t)ti * w + h * DV + j] = o * g_sigm(pr[ch + h * DV + j]);   // z at [ch + h*dv + j]
+      float o = pm[0][j] * (sc * nw_j);                              // rms_inplace: x *= s * w  (:210)
+      out[(size_t)ti * w + h * DV + j] = o * g_sigm(z_j);   // z at [ch + h*dv + j]
     }
     __syncthreads();
   }

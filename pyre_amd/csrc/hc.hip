@@ -39,9 +39,10 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   float w[T], ss[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) { w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
-  float mine[T];        // upw == 1: the slice element this thread normalizes later, fetched with the others
+  float mine[T];        // upw == 1: the slice element this thread normalizes later (and its norm weight), fetched with the others
 #pragma unroll
   for (int t = 0; t < T; ++t) mine[t] = upw == 1 ? hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid) : 0.0f;
+  const float mine_nv = upw == 1 ? norm[(size_t)s * d + i0 + tid] : 0.0f;
   for (int i = tid; i < d; i += nthr) {
 #pragma unroll
     for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i); ss[t] += v * v; }
@@ -57,7 +58,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 #pragma unroll
   for (int t = 0; t < T; ++t) { float tot = wsum[t]; for (int q = 1; q < nw; ++q) tot += wsum[q * T + t]; sc[t] = 1.0f / sqrtf(tot / (float)d + eps); }
   for (int j = tid; j < L; j += nthr) {
-    const float nv = norm[(size_t)s * d + i0 + j];
+    const float nv = upw == 1 ? mine_nv : norm[(size_t)s * d + i0 + j];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       float v = upw == 1 ? mine[t] : hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
@@ -98,6 +99,9 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave / U, ku = wave - s * U;
   UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);        // in flight across the prologue
+  float xpre[8];                  // the epilogue's normalized-stream values of this thread's first output, fetched now
+#pragma unroll
+  for (int q = 0; q < 8; ++q) xpre[q] = (tid < T * 64 && q < hc) ? xn[((size_t)(tid >> 6) * hc + q) * d + blockIdx.x * 64 + (tid & 63)] : 0.0f;
   for (int idx = tid; idx < T * n_o; idx += nthr) {
     int t = idx / n_o, i = idx - t * n_o;
     float o = 0.0f;
@@ -123,10 +127,12 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   __syncthreads();
   for (int i = tid; i < T * 64; i += nthr) {
     int t = i >> 6, l = i & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
-    for (int q = 0; q < hc; ++q) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) if (q < hc) {
       float g = red[((size_t)(q * U) * T + t) * 64 + l];
       for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t) * 64 + l];
-      mx += xn[((size_t)t * hc + q) * d + col] * sigm(g);
+      const float xv = i == tid ? xpre[q] : xn[((size_t)t * hc + q) * d + col];
+      mx += xv * sigm(g);
     }
     mixed[(size_t)t * d + col] = mx / (float)hc;
   }
