@@ -95,13 +95,17 @@ def bench_gemv(args):
         ctx.free(dev)
     x = ctx.upload(synth.normal((1, cols), 3))
     y = ctx.alloc(rows * 4)
+    t = args.t
+    if t > 1:
+        x = ctx.upload(synth.normal((t, cols), 3)); y = ctx.alloc(t * rows * 4)
+    run = (lambda m: m.matmul_mfma_dev(x, t, y)) if args.mfma else (lambda m: m.matmul_dev(x, t, y))
     for i in range(args.warmup):
-        mats[i % nbuf].matmul_dev(x, 1, y)
+        run(mats[i % nbuf])
     ctx.sync()
     e0, e1 = ev.event(), ev.event()
     ev.record(e0, ctx.stream)
     for i in range(args.steps):
-        mats[i % nbuf].matmul_dev(x, 1, y)
+        run(mats[i % nbuf])
     ev.record(e1, ctx.stream)
     per = ev.elapsed_ms(e0, e1) / args.steps
     if args.calib_copy:
@@ -113,22 +117,22 @@ def bench_gemv(args):
             dst.copy_(src)
         torch.cuda.synchronize()
         log("calibration: 4 device copies of %d MiB (each reads and writes that many bytes)" % args.calib_copy)
-    alg_bytes = mats[0].gguf_bytes + 4 * cols + 4 * rows
+    alg_bytes = mats[0].gguf_bytes + 4 * t * cols + 4 * t * rows
     traffic = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary, when present
     try:
         for line in open(os.path.join(ROOT, "profiles", "gemv_iq3s_vocab_head_kernel_stats.txt")):
-            if line.startswith("traffic_bytes_per_launch:"):
+            if t == 1 and line.startswith("traffic_bytes_per_launch:"):
                 traffic = int(line.split(":")[1])
     except OSError:
         pass
     gbs = alg_bytes / (per * 1e-3) / 1e9
     out = {
-        "metric": "IQ3_S dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=1)", "value": round(gbs, 1), "unit": "GB/s",
+        "metric": "IQ3_S dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=%d%s)" % (t, ", matrix cores" if args.mfma else ""), "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[1]: IQ3_S GEMV 2048->151936, batch 1, rotating over %d weight buffers (%.0f MB)" % (nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
+        "config": {"workload": "configs[1]: IQ3_S GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "k_gemv<IQ3_S,1>", "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(per * 1e3, 3)},
+                     "kernel": "k_gemm_mfma_iq3s (+ k_xsplit)" if args.mfma else "k_gemv<IQ3_S,%d>" % t, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(per * 1e3, 3)},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemv(ty, rows, cols, 9000)
@@ -275,6 +279,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="debug: fewer layers than the 48 of the configuration")
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
+    ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MiB", help="gemv workload: also run 4 plain device copies of this size (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:

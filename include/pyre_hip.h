@@ -73,6 +73,11 @@ int    pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_h
  * multi-token verify pass equal one-token decode (qwen4exp_gguf.rs:2357-2360). */
 int    pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
+/* The batch 2..8 speculative-verify GEMM on the matrix cores (the reference's verify kernels, src/model/qn_cube.rs:17,6454,
+ * and lcm_dense, qwen4exp_gguf.rs:2641-2737): IQ3_S matrices, t in 2..8.  Same contract as pyre_qmatmul; the result
+ * agrees with it to about 1e-7 of max|y| but not bit for bit (f16 two-term split of the activations, f32 accumulation). */
+int    pyre_qmatmul_mfma(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
+int    pyre_qmatmul_mfma_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
 
 /* ---- synthetic tensors (no counterpart in the reference's API; its micro-benchmarks build the same kind of data
  * inline, src/model/qdot.rs:823-859, src/model/qn_cube.rs:7216-7249) ---------------------------------------------

@@ -26,6 +26,7 @@ struct pyre_ctx {
   struct ProfAcc { long count = 0; double ms = 0, bytes = 0; };
   bool prof_on = false; std::vector<ProfPending> prof_pending; std::map<std::string, ProfAcc> prof_acc; std::vector<hipEvent_t> prof_pool;
   std::string prof_text;
+  void* mfma_buf = nullptr; size_t mfma_bytes = 0;     // split activations of the matrix-core verify GEMM (grow-only)
 };
 
 // Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
@@ -87,6 +88,11 @@ int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev
 // step_dev (optional, device int[2]): step_dev[0] is incremented first (the position of the token being started) and the
 // id goes to mirror[step_dev[0] - step_dev[1]] instead of mirror[0].
 int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev, int* step_dev);
+
+// Verify GEMM on the matrix cores (verify_mfma.hip): IQ3_S, 2 <= t <= 8; y[t][rows] as pyre_gemv_launch, equal to it to
+// ~1e-7 relative (not bit for bit).
+bool pyre_gemm_mfma_ok(const QMatDev& m, int t);
+int pyre_gemm_mfma_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {

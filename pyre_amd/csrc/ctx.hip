@@ -75,6 +75,7 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   if (ctx->stage) (void)hipFree(ctx->stage);
   if (ctx->d_iq3s) (void)hipFree(ctx->d_iq3s);
+  if (ctx->mfma_buf) (void)hipFree(ctx->mfma_buf);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
   for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto e : ctx->prof_pool) (void)hipEventDestroy(e);

@@ -43,6 +43,8 @@ def _declare(L):
         "pyre_qmat_row": (i32, [vp, vp, sz, vp]),
         "pyre_qmatmul": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_dev": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmatmul_mfma_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_synth_blocks": (i32, [vp, u32, sz, u64, f32, f32, vp]),
         "pyre_moe_create": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, C.POINTER(vp)]),
         "pyre_moe_destroy": (None, [vp]),
@@ -217,6 +219,16 @@ class QMat:
         y = np.empty((t, self.rows), dtype=np.float32)
         self.ctx.check(self.ctx.L.pyre_qmatmul(self.ctx.h, self.h, _ptr(x), t, _ptr(y)), "qmatmul")
         return y
+
+    def matmul_mfma(self, x):
+        """The matrix-core verify GEMM (IQ3_S, 2..8 tokens): same contract as matmul, ~1e-7 of max|y| from it."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
+        y = np.empty((x.shape[0], self.rows), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_qmatmul_mfma(self.ctx.h, self.h, _ptr(x), x.shape[0], _ptr(y)), "qmatmul_mfma")
+        return y
+
+    def matmul_mfma_dev(self, x_dev, t, y_dev):
+        self.ctx.check(self.ctx.L.pyre_qmatmul_mfma_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_mfma_dev")
 
     def matmul_dev(self, x_dev, t, y_dev):
         self.ctx.check(self.ctx.L.pyre_qmatmul_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_dev")

@@ -154,3 +154,29 @@ def test_argument_errors_are_reported(ctx):
         m.matmul(np.zeros((9, 256), np.float32))                         # t outside 1..8
     with pytest.raises(lib.PyreError):
         m.row(64)
+
+
+# ---- the batch 2..8 verify GEMM on the matrix cores (IQ3_S) -----------------------------------------------------------
+@pytest.mark.parametrize("t", [2, 3, 4, 5, 8])
+@pytest.mark.parametrize("rows,cols", [(320, 2048), (4096, 2048), (2048, 4096), (2048, 512), (100, 256)])
+def test_verify_gemm_on_matrix_cores_matches_truth(ctx, rows, cols, t):
+    raw = synth.matrix(lib.IQ3_S, rows, cols, 61 + t)
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
+    W = orc.dequant(lib.IQ3_S, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    x = synth.normal((t, cols), 71 + t)
+    x[0] *= 3000.0                                   # a token far outside the half range: the exact power-of-two rescaling
+    x[-1] *= 1e-6
+    truth = x.astype(np.float64) @ W.T
+    y = m.matmul_mfma(x)
+    for i in range(t):                               # per token: the tokens differ by nine orders of magnitude
+        assert relerr(y[i], truth[i]) <= TOL, i
+    assert relerr(y, m.matmul(x)) <= 2e-6
+
+
+def test_verify_gemm_on_matrix_cores_rejects_other_types_and_widths(ctx):
+    m = lib.QMat(ctx, lib.Q8_0, 64, 256, synth.matrix(lib.Q8_0, 64, 256, 3))
+    with pytest.raises(lib.PyreError):
+        m.matmul_mfma(synth.normal((2, 256), 1))
+    m3 = lib.QMat(ctx, lib.IQ3_S, 64, 256, synth.matrix(lib.IQ3_S, 64, 256, 3))
+    with pytest.raises(lib.PyreError):
+        m3.matmul_mfma(synth.normal((1, 256), 1))
