@@ -205,7 +205,7 @@ def bench_decode(args):
         ctx.free(p)
     log("model resident (re-laid-out) in %.1f s; weight bytes per token %.1f MB" % (time.perf_counter() - t0, model.weight_bytes_per_token / 1e6))
     n_ctx = args.ctx
-    st = model.new_state(n_ctx + args.steps + args.warmup + 64)
+    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8)
     g = np.random.Generator(np.random.PCG64(args.seed + 1))
     prompt = g.integers(0, cfg.vocab, n_ctx, dtype=np.uint32)
     t0 = time.perf_counter()
@@ -236,6 +236,21 @@ def bench_decode(args):
     n_lin = cfg.n_layers - cfg.n_layers // cfg.full_every
     state_b = n_lin * (2 * cfg.lin_nv * cfg.lin_dk * cfg.lin_dv * 4 + 2 * (cfg.conv_k - 1) * cfg.ch * 4)
     all_b = wbytes + kvb + state_b
+    # the 4-token-draft speculative-verify variant: windows of [pending, 4 drafts] through pyre_forward_multi (logits of all
+    # five tokens back on the host) + pyre_spec_keep.  Random drafts are all rejected, so each window yields one token;
+    # with every draft accepted the same window would yield five.
+    spec = None
+    if args.spec_windows > 0:
+        dr = g.integers(0, cfg.vocab, (args.spec_windows, 4), dtype=np.uint32)
+        pend = nxt
+        model.forward_multi(np.concatenate([[pend], dr[0]]).astype(np.uint32), st); model.spec_keep(st, 5, 1)      # untimed
+        ctx.sync(); t0 = time.perf_counter()
+        for i in range(args.spec_windows):
+            ls = model.forward_multi(np.concatenate([[pend], dr[i]]).astype(np.uint32), st)
+            pend = int(np.argmax(ls[0])); model.spec_keep(st, 5, 1)
+        win_ms = (time.perf_counter() - t0) * 1e3 / args.spec_windows
+        spec = {"window_tokens": 5, "ms_per_window": round(win_ms, 3), "tok_s_if_all_drafts_accepted": round(5e3 / win_ms, 1), "tok_s_if_none_accepted": round(1e3 / win_ms, 1),
+                "note": "host-facing verify window incl. 5 x %d logits device->host and the host argmax; %d windows" % (cfg.vocab, args.spec_windows)}
     # second pass: per-kernel-class durations from event pairs around every launch
     ctx.prof_reset(); ctx.prof_enable(True)
     pn = min(16, args.steps)
@@ -263,6 +278,8 @@ def bench_decode(args):
                            "kernel_time_us_per_token": round(tot_ms / pn * 1e3, 1)},
         "kernels": breakdown,
     }
+    if spec:
+        out["spec_verify"] = spec
     if not args.no_cpu:
         del model, st
         out["cpu_baseline"] = cpu_baseline_decode(cfg, args.seed)
@@ -279,6 +296,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="debug: fewer layers than the 48 of the configuration")
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
     ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MiB", help="gemv workload: also run 4 plain device copies of this size (counter calibration under rocprofv3 --pmc)")
