@@ -168,6 +168,29 @@ typedef struct {
   int32_t kv_recent;  /* PYRE_QN_KV8_RECENT default 1024 */
 } pyre_model_cfg;
 
+/* ---- GGUF container (host only, no GPU needed): Gguf::open / mat / meta accessors, src/model/gguf_q.rs:250-336 --------
+ * Opens the file, or all shards of a split one given any of them (`-NNNNN-of-MMMMM.gguf`), read-only memory maps;
+ * metadata value types 0..12, `general.alignment` (default 32).  Errors come back as text in err[err_cap]. */
+typedef struct pyre_gguf pyre_gguf;
+int    pyre_gguf_open(const char* path, pyre_gguf** out, char* err, size_t err_cap);
+void   pyre_gguf_close(pyre_gguf* g);
+size_t pyre_gguf_n_shards(const pyre_gguf* g);
+size_t pyre_gguf_n_tensors(const pyre_gguf* g);
+const char* pyre_gguf_tensor_name(const pyre_gguf* g, size_t i);            /* file order */
+int    pyre_gguf_has(const pyre_gguf* g, const char* name);
+/* Gguf::mat (:326-331): the tensor as a matrix view into the map (cols = shape[0], rows = product of the rest);
+ * n_dims / dims[8] (optional) receive the stored shape.  Types other than the PYRE_* ones are reported as PYRE_E_TYPE. */
+int    pyre_gguf_tensor(const pyre_gguf* g, const char* name, pyre_tensor* out, uint32_t* n_dims, uint64_t* dims, char* err, size_t err_cap);
+/* Meta::as_u64 / as_f64 / as_str and Gguf::arr_u64 (:253-258, :323): 0 when the key exists and converts. */
+int    pyre_gguf_meta_u64(const pyre_gguf* g, const char* key, uint64_t* out);
+int    pyre_gguf_meta_f64(const pyre_gguf* g, const char* key, double* out);
+int    pyre_gguf_meta_str(const pyre_gguf* g, const char* key, char* out, size_t cap);
+long   pyre_gguf_meta_arr_u64(const pyre_gguf* g, const char* key, uint64_t* out, size_t cap);   /* element count, -1 if not an array */
+
+/* Model::load (qwen4exp_gguf.rs:462-524): `general.architecture` must be qwen4exp; configuration from the `qwen4exp.*`
+ * keys, tensors by their GGUF names (blk.N.*, token_embd, output_hc_*, output or the tied embedding).  kv_bits and
+ * kv_recent are run-time settings of the reference, not file contents.  Files with PLE layers are refused. */
+int   pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, pyre_model** out);
 /* Copies (and re-lays-out) every tensor into device memory; the caller's buffers are free afterwards. */
 int   pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* layer_tensors /*[n_layers][PYRE_LAYER_SLOTS]*/,
                         const pyre_tensor* globals /*[PYRE_GLOBAL_SLOTS]*/, pyre_model** out);

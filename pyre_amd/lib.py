@@ -44,6 +44,18 @@ def _declare(L):
         "pyre_qmatmul": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_gguf_open": (i32, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
+        "pyre_gguf_close": (None, [vp]),
+        "pyre_gguf_n_shards": (C.c_size_t, [vp]),
+        "pyre_gguf_n_tensors": (C.c_size_t, [vp]),
+        "pyre_gguf_tensor_name": (C.c_char_p, [vp, C.c_size_t]),
+        "pyre_gguf_has": (i32, [vp, C.c_char_p]),
+        "pyre_gguf_tensor": (i32, [vp, C.c_char_p, vp, vp, vp, C.c_char_p, C.c_size_t]),
+        "pyre_gguf_meta_u64": (i32, [vp, C.c_char_p, vp]),
+        "pyre_gguf_meta_f64": (i32, [vp, C.c_char_p, vp]),
+        "pyre_gguf_meta_str": (i32, [vp, C.c_char_p, C.c_char_p, C.c_size_t]),
+        "pyre_gguf_meta_arr_u64": (C.c_long, [vp, C.c_char_p, vp, C.c_size_t]),
+        "pyre_model_load_gguf": (i32, [vp, C.c_char_p, i32, i32, vp]),
         "pyre_qmatmul_mfma_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_synth_blocks": (i32, [vp, u32, sz, u64, f32, f32, vp]),
         "pyre_moe_create": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, C.POINTER(vp)]),
@@ -383,6 +395,79 @@ class TensorDesc(C.Structure):
     _fields_ = [("ggml_type", C.c_uint32), ("on_device", C.c_uint32), ("rows", C.c_uint64), ("cols", C.c_uint64), ("data", C.c_void_p)]
 
 
+class Gguf:
+    """GGUF container reader (Gguf::open of the reference, gguf_q.rs:297-336); host only, needs no GPU."""
+
+    def __init__(self, path):
+        self.L = load()
+        h = C.c_void_p(); err = C.create_string_buffer(1024)
+        rc = self.L.pyre_gguf_open(os.fsencode(path), C.byref(h), err, len(err))
+        if rc:
+            raise PyreError("gguf_open: %s" % err.value.decode(errors="replace"))
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.L.pyre_gguf_close(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def n_shards(self):
+        return self.L.pyre_gguf_n_shards(self.h)
+
+    def names(self):
+        return [self.L.pyre_gguf_tensor_name(self.h, i).decode() for i in range(self.L.pyre_gguf_n_tensors(self.h))]
+
+    def has(self, name):
+        return bool(self.L.pyre_gguf_has(self.h, name.encode()))
+
+    def tensor(self, name):
+        """(ggml type, rows, cols, stored shape, bytes as a numpy uint8 copy)"""
+        from . import synth
+        td = TensorDesc(); nd = C.c_uint32(); dims = (C.c_uint64 * 8)(); err = C.create_string_buffer(1024)
+        rc = self.L.pyre_gguf_tensor(self.h, name.encode(), C.byref(td), C.byref(nd), dims, err, len(err))
+        if rc:
+            raise PyreError("gguf_tensor: %s" % err.value.decode(errors="replace"))
+        el, bs, _ = synth.GEOM[td.ggml_type]
+        nbytes = td.rows * (td.cols // el) * bs
+        data = np.ctypeslib.as_array(C.cast(td.data, C.POINTER(C.c_uint8)), shape=(nbytes,)).copy()
+        return td.ggml_type, td.rows, td.cols, tuple(dims[i] for i in range(nd.value)), data
+
+    def u64(self, key, default=None):
+        v = C.c_uint64()
+        if self.L.pyre_gguf_meta_u64(self.h, key.encode(), C.byref(v)) == 0:
+            return v.value
+        if default is None:
+            raise KeyError(key)
+        return default
+
+    def f64(self, key):
+        v = C.c_double()
+        if self.L.pyre_gguf_meta_f64(self.h, key.encode(), C.byref(v)) != 0:
+            raise KeyError(key)
+        return v.value
+
+    def string(self, key):
+        b = C.create_string_buffer(4096)
+        if self.L.pyre_gguf_meta_str(self.h, key.encode(), b, len(b)) != 0:
+            raise KeyError(key)
+        return b.value.decode(errors="replace")
+
+    def arr_u64(self, key):
+        n = self.L.pyre_gguf_meta_arr_u64(self.h, key.encode(), None, 0)
+        if n < 0:
+            raise KeyError(key)
+        out = (C.c_uint64 * max(n, 1))()
+        self.L.pyre_gguf_meta_arr_u64(self.h, key.encode(), out, n)
+        return [out[i] for i in range(n)]
+
+
 class ModelCfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
                [("rope_base", C.c_float), ("eps", C.c_float)] + \
@@ -419,6 +504,28 @@ class Model:
         ctx.check(ctx.L.pyre_model_create(ctx.h, C.byref(self.cfg), lt, gl, C.byref(h)), "model_create")
         self.h = h
         self.vocab = self.cfg.vocab
+
+    @classmethod
+    def from_gguf(cls, ctx, path, kv_bits=4, kv_recent=1024):
+        """Model::load: configuration and tensors straight from a qwen4exp GGUF file (or its shards)."""
+        self = cls.__new__(cls)
+        self.ctx = ctx
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_model_load_gguf(ctx.h, os.fsencode(path), kv_bits, kv_recent, C.byref(h)), "model_load_gguf")
+        self.h = h
+        g = Gguf(path); a = "qwen4exp."
+        c = ModelCfg()
+        for field, key in (("n_layers", "block_count"), ("d", "embedding_length"), ("hc", "hyper_connection.count"), ("hc_lr", "hyper_connection.low_rank"),
+                           ("n_head", "attention.head_count"), ("n_kv", "attention.head_count_kv"), ("hd", "attention.key_length"), ("n_rot", "rope.dimension_count"),
+                           ("n_exp", "expert_count"), ("top_k", "expert_used_count"), ("ff_exp", "expert_feed_forward_length"), ("lin_nk", "ssm.group_count"),
+                           ("lin_nv", "ssm.time_step_rank"), ("lin_dk", "ssm.state_size"), ("lin_dv", "ssm.state_size"), ("conv_k", "ssm.conv_kernel")):
+            setattr(c, field, g.u64(a + key))
+        c.full_every = g.u64(a + "full_attention_interval", 4)
+        c.rope_base = g.f64(a + "rope.freq_base"); c.eps = g.f64(a + "attention.layer_norm_rms_epsilon")
+        c.vocab = g.tensor("token_embd.weight")[3][1]; c.kv_bits = kv_bits; c.kv_recent = kv_recent
+        g.close()
+        self.cfg = c; self.vocab = c.vocab
+        return self
 
     @property
     def weight_bytes_per_token(self):

@@ -123,3 +123,30 @@ def test_errors(ctx):
     bad = [dict(l) for l in hw.layers]; bad[0].pop(mg.ROUTER)
     with pytest.raises(lib.PyreError):
         lib.Model(ctx, c, bad, hw.globals_)                                  # missing tensor
+
+
+def test_model_loaded_from_gguf_shards_equals_the_model_built_from_the_same_tensors(ctx, tmp_path):
+    import gguf_writer as gw
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 9)
+    tens = gw.model_tensors(c, hw); half = len(tens) // 2
+    p1 = str(tmp_path / "tiny-00001-of-00002.gguf"); p2 = str(tmp_path / "tiny-00002-of-00002.gguf")
+    gw.write(p1, gw.model_meta(c), tens[:half]); gw.write(p2, [("split.no", gw.U16, 1)], tens[half:], alignment=128)
+    gg = lib.Model.from_gguf(ctx, p2, kv_bits=c.kv_bits, kv_recent=c.kv_recent)
+    assert [getattr(gg.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in ("rope_base", "eps")] == [getattr(gm.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in ("rope_base", "eps")]
+    ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88], dtype=np.uint32)
+    sa, sb = gm.new_state(64), gg.new_state(64)
+    la, lb = gm.forward(ids, sa), gg.forward(ids, sb)
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    assert relerr(lb, om.forward(ids, om.new_state())) <= 1e-4
+    # a file of another architecture, and one with a tensor missing, are refused with the reference's messages
+    bad = str(tmp_path / "other.gguf")
+    gw.write(bad, [("general.architecture", gw.STR, "llama")], [])
+    with pytest.raises(lib.PyreError, match="is not qwen4exp"):
+        lib.Model.from_gguf(ctx, bad)
+    gw.write(bad, gw.model_meta(c), [t for t in tens if t[0] != "blk.2.ssm_out.weight"])
+    with pytest.raises(lib.PyreError, match="missing tensor blk.2.ssm_out.weight"):
+        lib.Model.from_gguf(ctx, bad)
+    gw.write(bad, [m for m in gw.model_meta(c) if "expert_count" not in m[0]], tens)
+    with pytest.raises(lib.PyreError, match="gguf key qwen4exp.expert_count"):
+        lib.Model.from_gguf(ctx, bad)
