@@ -606,7 +606,7 @@ class State:
         return k, v
 
     def close(self):
-        if getattr(self, "h", None) and getattr(self.m, "h", None):
+        if getattr(self, "h", None) and getattr(self.m, "h", None) and getattr(self.m.ctx, "h", None):      # never after its context
             self.m.ctx.L.pyre_state_destroy(self.h)
         self.h = None
 
