@@ -202,6 +202,17 @@ int   pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_st
 void  pyre_state_destroy(pyre_state* s);
 int   pyre_state_reset(pyre_ctx* ctx, pyre_state* s);
 int   pyre_state_len(const pyre_state* s);
+int   pyre_state_capacity(const pyre_state* s);                 /* positions the caches have room for (Model::max_ctx of this state) */
+int   pyre_model_max_window(const pyre_model* m);               /* spec_max_window (qwen4exp_gguf.rs:2486-2493): 8; multi_ok is always true */
+/* Model::snapshot / restore (qwen4exp_gguf.rs:3277-3298; the prefix cache of engine_qn.rs:92-138 keeps these): the
+ * recurrent state and the first `len` cache positions, kept in device memory; restorable into any state of the same
+ * model with enough capacity. */
+typedef struct pyre_snap pyre_snap;
+int   pyre_state_snapshot(pyre_ctx* ctx, pyre_state* s, pyre_snap** out);
+int   pyre_state_restore(pyre_ctx* ctx, pyre_state* s, const pyre_snap* snap);
+void  pyre_snap_destroy(pyre_snap* snap);
+size_t pyre_snap_bytes(const pyre_snap* snap);
+int   pyre_snap_len(const pyre_snap* snap);
 /* Test access to the recurrent state: li-th DeltaNet layer's S [nv][dk][dv] and conv [(k-1)][ch]; ai-th attention layer's f32 K / V rows [len][nkv*hd]. */
 int   pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, float* ssm_host);
 int   pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, float* v_host);

@@ -42,6 +42,7 @@ struct pyre_state {
   std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
+  std::vector<int> graph_cur;                                    // which half of every DeltaNet double buffer the captured step works on
 };
 
 namespace {
@@ -218,6 +219,67 @@ int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
   s->len = 0; s->last_window = 0; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 int pyre_state_len(const pyre_state* s) { return s ? s->len : 0; }
+int pyre_state_capacity(const pyre_state* s) { return s ? s->cap - 8 : 0; }
+int pyre_model_max_window(const pyre_model* m) { return m ? 8 : 0; }
+
+// ---- snapshot / restore (Model::snapshot / restore, qwen4exp_gguf.rs:3277-3298), device resident ---------------------------
+// A snapshot holds the recurrent state of every DeltaNet layer and the first `len` positions of every attention
+// layer's cache (f32 and 4-bit planes; the key planes are blocked by 64 positions, so a prefix of blocks is contiguous
+// whatever the capacity).  It can be restored into any state of the same model with room for `len` positions.
+struct pyre_snap { const pyre_model* m; int len; std::vector<int> packed; void* mem; size_t bytes; };
+namespace {
+struct SnapPlan { size_t cs, ss, kf, ks_kq, kq, ksc, vf, vq, vsc, total; };
+SnapPlan snap_plan(const pyre_model* m, int len) {
+  const pyre_model_cfg& c = m->c; SnapPlan p{};
+  const size_t row = (size_t)c.n_kv * c.hd, nb = ((size_t)len + 63) / 64;
+  p.cs = al256((size_t)(c.conv_k - 1) * m->ch * 4); p.ss = al256((size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4);
+  p.kf = al256(nb * row * 64 * 4); p.kq = al256(nb * (row / 8) * 64 * 4); p.ksc = al256(nb * (row / 32) * 64 * 4);
+  p.vf = al256((size_t)len * row * 4); p.vq = al256((size_t)len * (row / 8) * 4); p.vsc = al256((size_t)len * (row / 32) * 4);
+  p.total = (size_t)m->n_lin * (p.cs + p.ss) + (size_t)m->n_attn * (p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc) + 256;
+  return p;
+}
+// dir = 0: state -> snapshot buffer, 1: snapshot buffer -> state
+int snap_copy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint8_t* buf, int len, int dir) {
+  const SnapPlan p = snap_plan(m, len); uint8_t* q = buf;
+  auto cp = [&](void* st, size_t n) -> hipError_t { hipError_t e = dir == 0 ? hipMemcpyAsync(q, st, n, hipMemcpyDeviceToDevice, ctx->stream) : hipMemcpyAsync(st, q, n, hipMemcpyDeviceToDevice, ctx->stream); return e; };
+  const pyre_model_cfg& c = m->c; const size_t row = (size_t)c.n_kv * c.hd, nb = ((size_t)len + 63) / 64;
+  for (int li = 0; li < m->n_lin; ++li) {
+    int b = s->cur[li];
+    PYRE_HIP(ctx, cp(s->conv[b][li], (size_t)(c.conv_k - 1) * m->ch * 4)); q += p.cs;
+    PYRE_HIP(ctx, cp(s->ssm[b][li], (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4)); q += p.ss;
+  }
+  for (int ai = 0; ai < m->n_attn; ++ai) {
+    KvDev& kv = s->kv[ai];
+    if (len > 0) {
+      PYRE_HIP(ctx, cp(kv.kf, nb * row * 64 * 4)); q += p.kf; PYRE_HIP(ctx, cp(kv.kq, nb * (row / 8) * 64 * 4)); q += p.kq; PYRE_HIP(ctx, cp(kv.ks, nb * (row / 32) * 64 * 4)); q += p.ksc;
+      PYRE_HIP(ctx, cp(kv.vf, (size_t)len * row * 4)); q += p.vf; PYRE_HIP(ctx, cp(kv.vq, (size_t)len * (row / 8) * 4)); q += p.vq; PYRE_HIP(ctx, cp(kv.vs, (size_t)len * (row / 32) * 4)); q += p.vsc;
+    } else q += p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc;
+  }
+  return PYRE_OK;
+}
+}  // namespace
+int pyre_state_snapshot(pyre_ctx* ctx, pyre_state* s, pyre_snap** out) {
+  if (!ctx || !s || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_snapshot: null argument");
+  *out = nullptr;
+  std::unique_ptr<pyre_snap> sn(new pyre_snap()); sn->m = s->m; sn->len = s->len; sn->packed = s->packed; sn->bytes = snap_plan(s->m, s->len).total; sn->mem = nullptr;
+  hipError_t e = hipMalloc(&sn->mem, sn->bytes);
+  if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_snapshot: hipMalloc(%zu): %s", sn->bytes, hipGetErrorString(e));
+  int rc = snap_copy(ctx, s->m, s, (uint8_t*)sn->mem, s->len, 0);
+  hipError_t e2 = hipStreamSynchronize(ctx->stream);
+  if (rc || e2 != hipSuccess) { (void)hipFree(sn->mem); return rc ? rc : pyre_fail(ctx, PYRE_E_HIP, "pyre_state_snapshot: %s", hipGetErrorString(e2)); }
+  *out = sn.release(); return PYRE_OK;
+}
+int pyre_state_restore(pyre_ctx* ctx, pyre_state* s, const pyre_snap* sn) {
+  if (!ctx || !s || !sn) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_restore: null argument");
+  if (s->m != sn->m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: the snapshot belongs to another model");
+  if (sn->len + 8 > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: %d positions do not fit the state's capacity %d", sn->len, s->cap - 8);
+  int rc = snap_copy(ctx, s->m, s, (uint8_t*)sn->mem, sn->len, 1); if (rc) return rc;
+  s->len = sn->len; s->packed = sn->packed; s->last_window = 0;
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+void pyre_snap_destroy(pyre_snap* sn) { if (!sn) return; (void)hipFree(sn->mem); delete sn; }
+size_t pyre_snap_bytes(const pyre_snap* sn) { return sn ? sn->bytes : 0; }
+int pyre_snap_len(const pyre_snap* sn) { return sn ? sn->len : 0; }
 int pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, float* ssm_host) {
   if (!ctx || !s || li < 0 || li >= (int)s->cur.size()) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_read_gdn: bad layer");
   const pyre_model_cfg& c = s->m->c; int b = s->cur[li];
@@ -246,6 +308,7 @@ struct WinOpt {
   uint32_t* toks_out = nullptr; // where the picked id is mirrored
   int* step_dev = nullptr;      // replayable form: position and output slot live in device memory (see pyre_pick_launch);
                                 // recurrent state is updated in place and no host-side bookkeeping is touched
+  bool inplace = false;         // update the recurrent state in its current buffer (no pre-window copy for spec_keep)
 };
 
 // One window of t <= 8 tokens (ids in m->ids unless from_best).
@@ -268,7 +331,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
       if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev))) return rc;
     } else {
-      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = replay ? b : b ^ 1;
+      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
       if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv))) return rc;
       if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true))) return rc;
@@ -446,7 +509,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
       return PYRE_OK;
     } }
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
-  { WinOpt o; o.greedy = true; if ((rc = run_window(ctx, m, s, 1, o))) return rc; }
+  { WinOpt o; o.greedy = true; o.inplace = true; if ((rc = run_window(ctx, m, s, 1, o))) return rc; }     // in place: the captured step below keeps pointing at the current buffers
   if (n_steps > 1) {
     static const bool no_graph = getenv("PYRE_NO_GRAPH") && atoi(getenv("PYRE_NO_GRAPH")) != 0;
     int step_host[2] = {s->len - 1, s->len};      // the pick increments [0] to the position it starts; slot = [0] - [1]
@@ -455,7 +518,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
     if (no_graph || ctx->prof_on) {
       for (int i = 1; i < n_steps; ++i) if ((rc = run_window(ctx, m, s, 1, o))) return rc;
     } else {
-      if (!s->graph_exec || s->graph_toks != m->toks) {
+      if (!s->graph_exec || s->graph_toks != m->toks || s->graph_cur != s->cur) {      // forward / forward_multi calls in between flip the double buffers
         if (s->graph_exec) { (void)hipGraphExecDestroy(s->graph_exec); s->graph_exec = nullptr; }
         hipGraph_t g = nullptr;
         PYRE_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
@@ -465,7 +528,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
         if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: stream capture failed: %s", hipGetErrorString(e));
         e = hipGraphInstantiate(&s->graph_exec, g, nullptr, nullptr, 0); (void)hipGraphDestroy(g);
         if (e != hipSuccess) { s->graph_exec = nullptr; return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: graph instantiate failed: %s", hipGetErrorString(e)); }
-        s->graph_toks = m->toks;
+        s->graph_toks = m->toks; s->graph_cur = s->cur;
       }
       for (int i = 1; i < n_steps; ++i) PYRE_HIP(ctx, hipGraphLaunch(s->graph_exec, ctx->stream));
     }

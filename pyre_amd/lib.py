@@ -56,6 +56,13 @@ def _declare(L):
         "pyre_gguf_meta_str": (i32, [vp, C.c_char_p, C.c_char_p, C.c_size_t]),
         "pyre_gguf_meta_arr_u64": (C.c_long, [vp, C.c_char_p, vp, C.c_size_t]),
         "pyre_model_load_gguf": (i32, [vp, C.c_char_p, i32, i32, vp]),
+        "pyre_state_capacity": (i32, [vp]),
+        "pyre_model_max_window": (i32, [vp]),
+        "pyre_state_snapshot": (i32, [vp, vp, vp]),
+        "pyre_state_restore": (i32, [vp, vp, vp]),
+        "pyre_snap_destroy": (None, [vp]),
+        "pyre_snap_bytes": (C.c_size_t, [vp]),
+        "pyre_snap_len": (i32, [vp]),
         "pyre_qmatmul_mfma_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_synth_blocks": (i32, [vp, u32, sz, u64, f32, f32, vp]),
         "pyre_moe_create": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, C.POINTER(vp)]),
@@ -577,6 +584,29 @@ class Model:
             pass
 
 
+class Snap:
+    def __init__(self, ctx, h):
+        self.ctx, self.h = ctx, h
+
+    def __len__(self):
+        return self.ctx.L.pyre_snap_len(self.h)
+
+    @property
+    def nbytes(self):
+        return self.ctx.L.pyre_snap_bytes(self.h)
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_snap_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class State:
     def __init__(self, model, max_ctx):
         self.m = model
@@ -604,6 +634,19 @@ class State:
         k = np.empty((n, c.n_kv * c.hd), dtype=np.float32); v = np.empty_like(k)
         self.m.ctx.check(self.m.ctx.L.pyre_state_read_kv(self.m.ctx.h, self.h, ai, _ptr(k), _ptr(v)), "state_read_kv")
         return k, v
+
+    @property
+    def capacity(self):
+        return self.m.ctx.L.pyre_state_capacity(self.h)
+
+    def snapshot(self):
+        """Model::snapshot: (handle, length, bytes); hand the handle to restore() of any state of the same model."""
+        h = C.c_void_p()
+        self.m.ctx.check(self.m.ctx.L.pyre_state_snapshot(self.m.ctx.h, self.h, C.byref(h)), "state_snapshot")
+        return Snap(self.m.ctx, h)
+
+    def restore(self, snap):
+        self.m.ctx.check(self.m.ctx.L.pyre_state_restore(self.m.ctx.h, self.h, snap.h), "state_restore")
 
     def close(self):
         if getattr(self, "h", None) and getattr(self.m, "h", None) and getattr(self.m.ctx, "h", None):      # never after its context

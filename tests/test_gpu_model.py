@@ -150,3 +150,53 @@ def test_model_loaded_from_gguf_shards_equals_the_model_built_from_the_same_tens
     gw.write(bad, [m for m in gw.model_meta(c) if "expert_count" not in m[0]], tens)
     with pytest.raises(lib.PyreError, match="gguf key qwen4exp.expert_count"):
         lib.Model.from_gguf(ctx, bad)
+
+
+def test_snapshot_restore_reproduces_the_continuation_bit_for_bit(ctx):
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 10)
+    prompt = (np.arange(150, dtype=np.uint32) * 29 + 5) % c.vocab          # 150 > recent + 64: the packed region exists
+    sa = gm.new_state(400)
+    lg = gm.forward(prompt, sa)
+    snap = sa.snapshot()
+    assert len(snap) == 150 and snap.nbytes > 0 and sa.capacity >= 400 and ctx.L.pyre_model_max_window(gm.h) == 8
+    first = int(np.argmax(lg))
+    ta = gm.decode_greedy_dev(sa, first, 40)                               # the original state moves on (and packs more positions)
+    sb = gm.new_state(200)                                                 # another capacity: the blocked key planes are prefix-compatible
+    sb.restore(snap)
+    assert len(sb) == 150
+    tb = gm.decode_greedy_dev(sb, first, 40)
+    assert np.array_equal(ta, tb)
+    sa.restore(snap)                                                       # and back onto the state it came from
+    tc = gm.decode_greedy_dev(sa, first, 40)
+    assert np.array_equal(ta, tc)
+    for li in range(3):
+        for x, y in zip(sa.gdn(li), sb.gdn(li)):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    ka, va = sa.kv(0); kb, vb = sb.kv(0)
+    assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32)) and np.array_equal(va.view(np.uint32), vb.view(np.uint32))
+    gm.decode_greedy_dev(sa, int(tc[-1]), 80)                              # 270 positions: more than a 256-position state holds
+    small = gm.new_state(100)
+    with pytest.raises(lib.PyreError, match="do not fit"):
+        small.restore(sa.snapshot())
+
+
+def test_device_greedy_loop_called_repeatedly_on_one_state_continues_the_same_stream(ctx):
+    """The captured decode step must follow the state through several calls and through forward calls in between."""
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 11)
+    prompt = np.array([5, 6, 7, 8, 9, 10, 11, 12, 13, 14], dtype=np.uint32)
+    sa, sb = gm.new_state(200), gm.new_state(200)
+    lg = gm.forward(prompt, sa); gm.forward(prompt, sb)
+    first = int(np.argmax(lg))
+    whole = gm.decode_greedy_dev(sb, first, 60)
+    parts = [gm.decode_greedy_dev(sa, first, 7)]
+    parts.append(gm.decode_greedy_dev(sa, int(parts[-1][-1]), 13))
+    lg2 = gm.forward(np.array([parts[-1][-1]], dtype=np.uint32), sa)          # a host-driven step in between flips the double buffers
+    parts.append(np.array([int(np.argmax(lg2))], dtype=np.uint32))
+    parts.append(gm.decode_greedy_dev(sa, int(parts[-1][-1]), 19))
+    parts.append(gm.decode_greedy_dev(sa, int(parts[-1][-1]), 20))
+    assert np.array_equal(np.concatenate(parts), whole)
+    os_ = om.new_state(); lo = om.forward(prompt, os_)
+    ref, _ = om.generate_greedy(os_, lo, 61)
+    assert np.array_equal(ref[1:], whole)
