@@ -1,0 +1,85 @@
+"""The benchmark's real dimensions (d 2048, 512 experts top-10, 16/32 DeltaNet heads, 16/2 attention heads of 256,
+vocabulary 151936, IQ3_S) on a few layers: size-independent properties at full width, and one comparison with the
+oracle on a two-layer slice (one Gated DeltaNet + one attention layer), the size it finishes in seconds."""
+import os
+
+import numpy as np
+import pytest
+
+import orc
+from helpers import orc_model, relerr
+from pyre_amd import lib
+from pyre_amd import modelgen as mg
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def model4(ctx):
+    cfg = mg.a3b_config(n_layers=4)
+    layers, globals_, raw = mg.build_device(ctx, cfg, seed=5)
+    m = lib.Model(ctx, cfg, layers, globals_)
+    for p in raw:
+        ctx.free(p)
+    return cfg, m
+
+
+def test_verify_window_equals_single_steps_and_rollback_at_full_width(model4):
+    cfg, gm = model4
+    g = np.random.Generator(np.random.PCG64(3))
+    prompt = g.integers(0, cfg.vocab, 37, dtype=np.uint32)
+    sa, sb = gm.new_state(128), gm.new_state(128)
+    gm.forward(prompt, sa, want_logits=False); gm.forward(prompt, sb, want_logits=False)
+    toks = g.integers(0, cfg.vocab, 5, dtype=np.uint32)
+    lv = gm.forward_multi(toks, sa)
+    singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(5)])
+    assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32))
+    gm.spec_keep(sa, 5, 2)                                                   # keep two of the five
+    sc = gm.new_state(128); gm.forward(np.concatenate([prompt, toks[:2]]), sc, want_logits=False)
+    nxt = np.array([toks[2] ^ 1], dtype=np.uint32)
+    la, lc = gm.forward(nxt, sa), gm.forward(nxt, sc)                         # rolled back == never drafted
+    assert len(sa) == len(sc) == 40 and np.array_equal(la.view(np.uint32), lc.view(np.uint32))
+
+
+def test_device_loop_persistent_kernel_and_snapshot_agree_at_full_width(model4):
+    cfg, gm = model4
+    g = np.random.Generator(np.random.PCG64(4))
+    prompt = g.integers(0, cfg.vocab, 21, dtype=np.uint32)
+    st = gm.new_state(128)
+    lg = gm.forward(prompt, st); first = int(np.argmax(lg))
+    snap = st.snapshot()
+    a = gm.decode_greedy_dev(st, first, 24)
+    st.restore(snap)
+    host = []; tok = first                                                    # the host-driven loop: forward + argmax per token
+    for _ in range(24):
+        lg = gm.forward(np.array([tok], dtype=np.uint32), st); tok = int(orc.argmax(lg)); host.append(tok)
+    assert np.array_equal(a, np.array(host, dtype=np.uint32))
+    st.restore(snap)
+    os.environ["PYRE_MEGA"] = "2"
+    try:
+        b = gm.decode_greedy_dev(st, first, 24)
+    finally:
+        os.environ.pop("PYRE_MEGA", None)
+    assert np.array_equal(a, b)
+
+
+def test_two_layer_slice_matches_the_oracle_at_full_width(ctx):
+    cfg = mg.a3b_config(n_layers=2, full_every=2)
+    hw = mg.build_host(cfg, seed=8)
+    gm = lib.Model(ctx, cfg, hw.layers, hw.globals_); om = orc_model(hw, threads=min(os.cpu_count() or 1, 16))
+    g = np.random.Generator(np.random.PCG64(9))
+    prompt = g.integers(0, cfg.vocab, 10, dtype=np.uint32)
+    gs, os_ = gm.new_state(64), om.new_state()
+    lg, lo = gm.forward(prompt, gs), om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-3 and relerr(lg, lo) <= 1e-4
+    tg, _ = gm.generate_greedy(gs, lg, 6); to, _ = om.generate_greedy(os_, lo, 6)
+    assert np.array_equal(tg, to)
+    conv, ssm = gs.gdn(0)
+    assert relerr(ssm, os_.ssm(0)) <= 1e-4 and relerr(conv, os_.conv(0)) <= 1e-5
