@@ -26,6 +26,7 @@ struct pyre_ctx {
   struct ProfAcc { long count = 0; double ms = 0, bytes = 0; };
   bool prof_on = false; std::vector<ProfPending> prof_pending; std::map<std::string, ProfAcc> prof_acc; std::vector<hipEvent_t> prof_pool;
   std::string prof_text;
+  unsigned* fuse_ctl = nullptr;                        // control words of in-launch barriers (zeroed once): [0] generation, [16] abort, [32] count
   void* mfma_buf = nullptr; size_t mfma_bytes = 0;     // split activations of the matrix-core verify GEMM (grow-only)
 };
 
@@ -47,6 +48,8 @@ int pyre_fail(pyre_ctx* ctx, int code, const char* fmt, ...);
 #define PYRE_CHECK_LAUNCH(ctx) PYRE_HIP(ctx, hipGetLastError())
 
 int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out);          // grow-only device staging buffer
+// After a stream synchronisation: fails if an in-launch barrier gave up waiting (and clears the flag).
+int pyre_fuse_check(pyre_ctx* ctx);
 
 // ---- device-side matrix view --------------------------------------------------------------------------------------
 // Weights live in "lane = row" planes: rows are grouped in tiles of 64, and for every (tile, unit) the 64 rows'

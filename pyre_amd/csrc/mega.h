@@ -60,6 +60,32 @@ __device__ __forceinline__ bool grid_sync(Bar& b, unsigned* ok_lds) {
   return *ok_lds != 0;
 }
 
+// A barrier over the nwg workgroups of ONE launch that leaves its control words ready for the next launch (no host
+// reset, so it can sit in a replayed graph): arrivals count up, the last arriver zeroes the count and bumps the
+// generation word everybody else polls.  ctl: [0] generation, [16] abort flag, [32] arrival count.  Bounded like grid_sync.
+__device__ __forceinline__ bool launch_sync(unsigned* ctl, int nwg, unsigned limit, unsigned* ok_lds) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    unsigned* gen = ctl; unsigned* abort_flag = ctl + 16; unsigned* cnt = ctl + 32;
+    const unsigned g0 = __hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // read before arriving: it cannot move until this workgroup has arrived
+    unsigned good = 1;
+    if (__hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == (unsigned)nwg) {
+      __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(gen, g0 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      unsigned spins = 0;
+      while (__hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g0) {
+        if (++spins > limit) { __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); good = 0; break; }
+        __builtin_amdgcn_s_sleep(1);
+      }
+    }
+    *ok_lds = good;
+  }
+  __syncthreads();
+  return *ok_lds != 0;
+}
+
 // ---- device-side description of the model and of one run --------------------------------------------------------------
 struct HcPlan { int nw, upw, ksplit; };
 struct GemvPlan { int nw, upw; };
@@ -708,6 +734,17 @@ template <int FMT> __device__ __forceinline__ void st_pick_embed(const uint32_t*
     decode_exact<FMT>(embd, (const uint64_t*)nullptr, (int)(id >> 6), ku, (int)(id & 63), y);
     for (int i = 0; i < 64; ++i) stc(emb + (size_t)ku * 64 + i, y[i]);
   }
+}
+
+// ---- one hyper-connection mix in one launch (single-token steps): norm + [down ; inject] slices, a barrier over the
+// launch's own workgroups instead of a kernel boundary, then slice sums + up GEMV + gated stream mean --------------------
+template <int FMT> __global__ __launch_bounds__(WGT) void k_hc_mix_fused(HcDev h, HcPlan pl, const float* x_in, int in_ss, float* x_out, Comb cb, float eps,
+                                                                       float* xn, float* part, float* mixed, float* inj, unsigned* ctl, unsigned limit) {
+  extern __shared__ __align__(16) char lds[];
+  __shared__ unsigned bar_ok;
+  st_norm_down<FMT>(h, pl, x_in, in_ss, x_out, cb, eps, xn, part, nullptr, lds);
+  if (!launch_sync(ctl, (int)gridDim.x, limit, &bar_ok)) return;
+  st_up_mix<FMT>(h, pl.ksplit, part, xn, mixed, inj, lds);
 }
 
 // ---- the kernel --------------------------------------------------------------------------------------------------------

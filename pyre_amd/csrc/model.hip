@@ -457,7 +457,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     if ((rc = run_window(ctx, m, s, t, o))) return rc;
   }
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
-  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
 }
 
 int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host) {
@@ -470,7 +470,7 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
   s->last_window = n;
   PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)n * m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
-  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
 }
 
 // The DeltaNet layers kept the window's inputs and their pre-window state (the other half of the double buffer): the
@@ -536,7 +536,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
     for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
   }
   if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr, nullptr))) return rc;
-  if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+  if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx); }
   return PYRE_OK;
 }
 
