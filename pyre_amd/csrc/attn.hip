@@ -80,8 +80,8 @@ __global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1, const int* __rest
 
 __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((int)(w << (28 - 4 * i))) >> 28); }   // sign-extended nibble i
 
-// grid (chunks of 256 positions, nkv, t), 1024 threads.  One workgroup serves the G query heads that share a KV head.
-// Wave (pw, dq) owns the 64 positions pw*64.. of the chunk and the 64 head dims dq*64.., so every cache element is read
+// grid (chunks of 64*NPW positions, nkv, t), 256*NPW threads.  One workgroup serves the G query heads that share a KV
+// head.  Wave (pw, dq) owns the 64 positions pw*64.. of the chunk and the 64 head dims dq*64.., so every cache element is read
 // once per workgroup and each wave has all of its loads in flight at once (at decode sizes the step is bound by memory
 // latency, not bandwidth).  Both products run on the fp32 matrix cores as 16x16x4 tiles with the G heads as the
 // (zero-padded) 16 columns: the query and the softmax weights are then ordinary per-lane operands instead of
@@ -95,18 +95,20 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 //           4 tiles are one float4 (or 4 nibbles of one word) per position.  The four position quarters are added in order.
 typedef float f4v __attribute__((ext_vector_type(4)));
 template <int HD, int G>
-__global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+__global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
   static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
-  __shared__ float red[4 * 256 * G];          // phase 1: [dq][position][g];  phase 3: [pw][g][dim]
-  __shared__ float sc[256][G];
-  __shared__ float wmax[4][G], wsum[4][G], cm[G];
+  constexpr int NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;
+  static_assert(4 * CH == NPW * HD, "the score and value partials share one buffer");
+  __shared__ float red[4 * CH * G];          // phase 1: [dq][position][g];  phase 3: [pw][g][dim]
+  __shared__ float sc[CH][G];
+  __shared__ float wmax[NPW][G], wsum[NPW][G], cm[G];
   const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave & 3, dq = wave >> 2;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
   const int n = start + ti + 1;
-  if (chunk * 256 >= n) return;
+  if (chunk * CH >= n) return;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
-  const int wbase = chunk * 256 + pw * 64, p = wbase + lane;
+  const int wbase = chunk * CH + pw * 64, p = wbase + lane;
   const bool valid = p < n, packed = wbase < pb, active = wbase < n;
   const float scale = 1.0f / sqrtf((float)HD);
   const int li = lane & 15, lg = lane >> 4;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
 #pragma unroll
       for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[((size_t)dq * 256 + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
+        for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
     }
   }
   __syncthreads();
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
   for (int gi = 0; gi < GH; ++gi) {
     const int g = dq + 4 * gi; sv[gi] = -INFINITY;
     if (g < G) {
-      float v = ((red[((size_t)0 * 256 + pos) * G + g] + red[((size_t)1 * 256 + pos) * G + g]) + red[((size_t)2 * 256 + pos) * G + g]) + red[((size_t)3 * 256 + pos) * G + g];
+      float v = ((red[((size_t)0 * CH + pos) * G + g] + red[((size_t)1 * CH + pos) * G + g]) + red[((size_t)2 * CH + pos) * G + g]) + red[((size_t)3 * CH + pos) * G + g];
       sv[gi] = valid ? v * scale : -INFINITY;
       float m = sv[gi];
 #pragma unroll
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
     }
   }
   __syncthreads();
-  if (tid < G) cm[tid] = fmaxf(fmaxf(wmax[0][tid], wmax[1][tid]), fmaxf(wmax[2][tid], wmax[3][tid]));
+  if (tid < G) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
   __syncthreads();
 #pragma unroll
   for (int gi = 0; gi < GH; ++gi) {
@@ -236,13 +238,15 @@ __global__ __launch_bounds__(1024) void k_attn_decode(AttnDev a, KvDev kv, const
     }
   }
   __syncthreads();
-  for (int i = tid; i < G * HD; i += 1024) {
+  for (int i = tid; i < G * HD; i += NT) {
     int g = i / HD, dd = i % HD;
-    float o = ((red[((size_t)0 * G + g) * HD + dd] + red[((size_t)1 * G + g) * HD + dd]) + red[((size_t)2 * G + g) * HD + dd]) + red[((size_t)3 * G + g) * HD + dd];
+    float o = red[((size_t)0 * G + g) * HD + dd];
+#pragma unroll
+    for (int q = 1; q < NPW; ++q) o += red[((size_t)q * G + g) * HD + dd];
     part_o[(((size_t)ti * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
   }
   if (tid < G) {
-    float l = ((wsum[0][tid] + wsum[1][tid]) + wsum[2][tid]) + wsum[3][tid];
+    float l = wsum[0][tid]; for (int q = 1; q < NPW; ++q) l += wsum[q][tid];
     float* ml = part_ml + (((size_t)ti * a.nh + (size_t)kvh * G + tid) * max_chunks + chunk) * 2;
     ml[0] = cm[tid]; ml[1] = l;
   }
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(4 * HD) void k_attn_combine(AttnDev a, const float*
                                                          int max_chunks, float* __restrict__ out) {
   __shared__ float wmax[4 * HD / 64]; __shared__ float so[4][HD]; __shared__ float sl[4];
   if (posp) start = *posp;
-  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD, n = start + ti + 1, nc = (n + 255) / 256;
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD, n = start + ti + 1, nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
   float M = -INFINITY; for (int c = tid; c < nc; c += 4 * HD) M = fmaxf(M, ml[2 * c]);
@@ -289,18 +293,18 @@ void pyre_kv_carve(const AttnDev& a, int cap, void* base, KvDev* kv) {
   kv->vq = (uint32_t*)take(c * row / 8 * 4); kv->vs = (float*)take(c * row / 32 * 4); kv->cap = cap;
 }
 size_t pyre_attn_work_bytes(const AttnDev& a, int cap) {
-  size_t mc = ((size_t)cap + 255) / 256;
+  size_t mc = ((size_t)cap + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   return 3 * 256 + 4 * (8 * (size_t)a.nh * a.hd + 8 * (size_t)a.nh * mc * a.hd + 8 * (size_t)a.nh * mc * 2);
 }
 void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
-  size_t mc = ((size_t)cap + 255) / 256;
+  size_t mc = ((size_t)cap + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
 }
 
 template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp) {
-  int n = start + t, chunks = posp ? w.max_chunks : (n + 255) / 256;      // device-side position: cover the whole cache, surplus workgroups leave at once
-  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(1024), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
+  int n = start + t, chunks = posp ? w.max_chunks : (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;      // device-side position: cover the whole cache, surplus workgroups leave at once
+  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
 }
 
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
@@ -324,7 +328,7 @@ int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const Att
   { ProfScope ps(ctx, "attn_decode", kvb);
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp); break; default: launch_decode<8>(ctx, a, kv, w, start, t, posp); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + 255) / 256 + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

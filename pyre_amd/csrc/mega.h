@@ -411,17 +411,18 @@ __device__ __forceinline__ void st_attn_prep(const AttnDev& a, const KvDev& kv, 
 // ---- stage: attention over the cache, one 256-position chunk x kv head per virtual block (k_attn_decode<256, G>) ---------
 typedef float f4m __attribute__((ext_vector_type(4)));
 template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a, const KvDev& kv, const float* qbuf, int n, float* part_o, float* part_ml, int max_chunks, char* lds) {
-  constexpr int HD = 256;
-  float* red = (float*)lds; float* scb = red + 4 * 256 * G; float* wmax = scb + 256 * G; float* wsum = wmax + 4 * G; float* cm = wsum + 4 * G;
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave & 3, dq = wave >> 2;
-  const int nchunks = (n + 255) / 256, nvb = nchunks * a.nkv;
+  constexpr int HD = 256, NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;      // the stand-alone kernel's workgroup: NT threads
+  float* red = (float*)lds; float* scb = red + 4 * CH * G; float* wmax = scb + CH * G; float* wsum = wmax + NPW * G; float* cm = wsum + NPW * G;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = (wave / NPW) & 3;
+  const bool act = tid < NT;                                // the other waves only keep the barriers company
+  const int nchunks = (n + CH - 1) / CH, nvb = nchunks * a.nkv;
   const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
   const float scale = 1.0f / sqrtf((float)HD);
   const int li = lane & 15, lg = lane >> 4, row = a.nkv * HD;
   for (int vb = blockIdx.x; vb < nvb; vb += gridDim.x) {
     const int chunk = vb % nchunks, kvh = vb / nchunks;
-    const int wbase = chunk * 256 + pw * 64, p = wbase + lane;
-    const bool valid = p < n, packed = wbase < pb, active = wbase < n;
+    const int wbase = chunk * CH + pw * 64, p = wbase + lane;
+    const bool valid = act && p < n, packed = wbase < pb, active = act && wbase < n;
     {
       f4m D[4];
 #pragma unroll
@@ -456,11 +457,11 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
 #pragma unroll
           for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
       }
-      if (li < G) {
+      if (act && li < G) {
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) red[((size_t)dq * 256 + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
+          for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
       }
     }
     __syncthreads();
@@ -470,8 +471,8 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
 #pragma unroll
     for (int gi = 0; gi < GH; ++gi) {
       const int g = dq + 4 * gi; sv[gi] = -INFINITY;
-      if (g < G) {
-        float v = ((red[((size_t)0 * 256 + pos) * G + g] + red[((size_t)1 * 256 + pos) * G + g]) + red[((size_t)2 * 256 + pos) * G + g]) + red[((size_t)3 * 256 + pos) * G + g];
+      if (act && g < G) {
+        float v = ((red[((size_t)0 * CH + pos) * G + g] + red[((size_t)1 * CH + pos) * G + g]) + red[((size_t)2 * CH + pos) * G + g]) + red[((size_t)3 * CH + pos) * G + g];
         sv[gi] = valid ? v * scale : -INFINITY;
         float mx = sv[gi];
 #pragma unroll
@@ -480,12 +481,12 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
       }
     }
     __syncthreads();
-    if (tid < G) cm[tid] = fmaxf(fmaxf(wmax[0 * G + tid], wmax[1 * G + tid]), fmaxf(wmax[2 * G + tid], wmax[3 * G + tid]));
+    if (tid < G) { float mm = wmax[tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q * G + tid]); cm[tid] = mm; }
     __syncthreads();
 #pragma unroll
     for (int gi = 0; gi < GH; ++gi) {
       const int g = dq + 4 * gi;
-      if (g < G) {
+      if (act && g < G) {
         float e = valid ? expf(sv[gi] - cm[g]) : 0.0f; scb[pos * G + g] = e;
         float l = e;
 #pragma unroll
@@ -530,7 +531,7 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
       }
-      if (li < G) {
+      if (act && li < G) {
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -540,11 +541,13 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
     __syncthreads();
     for (int i = tid; i < G * HD; i += WGT) {
       int g = i / HD, dd = i % HD;
-      float o = ((red[((size_t)0 * G + g) * HD + dd] + red[((size_t)1 * G + g) * HD + dd]) + red[((size_t)2 * G + g) * HD + dd]) + red[((size_t)3 * G + g) * HD + dd];
+      float o = red[((size_t)0 * G + g) * HD + dd];
+#pragma unroll
+      for (int q = 1; q < NPW; ++q) o += red[((size_t)q * G + g) * HD + dd];
       stc(part_o + (((size_t)kvh * G + g) * max_chunks + chunk) * HD + dd, o);
     }
     if (tid < G) {
-      float l = ((wsum[0 * G + tid] + wsum[1 * G + tid]) + wsum[2 * G + tid]) + wsum[3 * G + tid];
+      float l = wsum[tid]; for (int q = 1; q < NPW; ++q) l += wsum[q * G + tid];
       float* ml = part_ml + (((size_t)kvh * G + tid) * max_chunks + chunk) * 2;
       stc(ml, cm[tid]); stc(ml + 1, l);
     }
@@ -556,7 +559,7 @@ template <int G> __device__ __forceinline__ void st_attn_decode(const AttnDev& a
 __device__ __forceinline__ void st_attn_combine(const AttnDev& a, const float* qkv, int n, const float* part_o, const float* part_ml, int max_chunks, float* out, char* lds) {
   constexpr int HD = 256;
   float* wmax = (float*)lds; float* so = wmax + 16; float* sl = so + 4 * HD;
-  const int tid = threadIdx.x, grp = tid / HD, dd = tid % HD, nc = (n + 255) / 256;
+  const int tid = threadIdx.x, grp = tid / HD, dd = tid % HD, nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   for (int h = blockIdx.x; h < a.nh; h += gridDim.x) {
     const float* ml = part_ml + (size_t)h * max_chunks * 2;
     const float* po = part_o + (size_t)h * max_chunks * HD;
