@@ -26,7 +26,7 @@ inline float h2f(const uint8_t* b) {
   float f; memcpy(&f, &u, 4); return f;
 }
 
-struct Tables { uint32_t iq3s[512]; uint64_t iq2xs[512]; uint8_t ksigns[128]; };
+struct Tables { uint32_t iq3s[512]; uint64_t iq2xs[512]; uint8_t ksigns[128]; uint64_t iq2xxs[256]; uint64_t iq2s[1024]; uint32_t iq3xxs[256]; };
 const Tables& tables() {
   static Tables t = [] {
     Tables t{};
@@ -37,6 +37,14 @@ const Tables& tables() {
       uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(kIq2xsCode[e] >> (2 * j)) & 3] << (8 * j);
       t.iq2xs[e] = w;
     }
+    auto tri8 = [](uint16_t code) { uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(code >> (2 * j)) & 3] << (8 * j); return w; };
+    static const uint8_t lv3[8] = {4, 12, 20, 28, 36, 44, 52, 62};
+    for (int e = 0; e < 256; ++e) {
+      t.iq2xxs[e] = tri8(kIq2xxsCode[e]);
+      uint32_t v = 0; for (int j = 0; j < 4; ++j) v |= (uint32_t)lv3[(kIq3xxsCode[e] >> (3 * j)) & 7] << (8 * j);
+      t.iq3xxs[e] = v;
+    }
+    for (int e = 0; e < 1024; ++e) t.iq2s[e] = tri8(kIq2sCode[e]);
     for (int i = 0; i < 128; ++i) t.ksigns[i] = (uint8_t)(i | ((__builtin_popcount(i) & 1) << 7));
     return t;
   }();
@@ -62,11 +70,20 @@ bool geom(uint32_t ty, int* el, int* by) {
     case ORC_Q4_K: *el = 256; *by = 144; return true;
     case ORC_IQ2_XS: *el = 256; *by = 74; return true;
     case ORC_IQ3_S: *el = 256; *by = 110; return true;
+    case ORC_Q4_0: *el = 32; *by = 18; return true;
+    case ORC_Q5_0: *el = 32; *by = 22; return true;
+    case ORC_Q6_K: *el = 256; *by = 210; return true;
+    case ORC_IQ4_NL: *el = 32; *by = 18; return true;
+    case ORC_IQ4_XS: *el = 256; *by = 136; return true;
+    case ORC_IQ2_XXS: *el = 256; *by = 66; return true;
+    case ORC_IQ2_S: *el = 256; *by = 82; return true;
+    case ORC_IQ3_XXS: *el = 256; *by = 98; return true;
   }
   return false;
 }
 
-// dequant, gguf_q.rs:67-166 (arms F32 :71, F16 :72, BF16 :73, Q8_0 :79, Q4K :103-107, IQ2XS :126-129, IQ3S :141-151)
+// dequant, gguf_q.rs:67-166 (arms F32 :71, F16 :72, BF16 :73, Q4_0 :74-75, Q5_0 :76-78, Q8_0 :79, IQ4NL :82-83, IQ4XS :84-89,
+// Q4K :103-107, Q6K :114-121, IQ2XXS :122-125, IQ2XS :126-129, IQ2S :130-135, IQ3XXS :136-140, IQ3S :141-151)
 bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
   int qk, bs; if (!geom(ty, &qk, &bs)) return false;
   size_t nb = n / qk;
@@ -118,6 +135,86 @@ bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
             qs += 8; signs += 4;
           }
           qh += 2;
+        }
+      }
+      break;
+    case ORC_Q4_0:
+      for (size_t i = 0; i < nb; ++i) { const uint8_t* b = x + i * bs; float d = h2f(b); float* yy = y + i * 32;
+        for (int j = 0; j < 16; ++j) { yy[j] = (float)((int)(b[2 + j] & 0xF) - 8) * d; yy[j + 16] = (float)((int)(b[2 + j] >> 4) - 8) * d; } }
+      break;
+    case ORC_Q5_0:
+      for (size_t i = 0; i < nb; ++i) { const uint8_t* b = x + i * bs; float d = h2f(b); uint32_t qh = (uint32_t)b[2] | ((uint32_t)b[3] << 8) | ((uint32_t)b[4] << 16) | ((uint32_t)b[5] << 24);
+        const uint8_t* qs = b + 6; float* yy = y + i * 32;
+        for (int j = 0; j < 16; ++j) { uint8_t h0 = (uint8_t)(((qh >> j) << 4) & 0x10), h1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+          yy[j] = (float)((int)((qs[j] & 0xF) | h0) - 16) * d; yy[j + 16] = (float)((int)((qs[j] >> 4) | h1) - 16) * d; } }
+      break;
+    case ORC_IQ4_NL:
+      for (size_t i = 0; i < nb; ++i) { const uint8_t* b = x + i * bs; float d = h2f(b); float* lo = y + i * 32; float* hi = lo + 16;
+        for (int j = 0; j < 16; ++j) { lo[j] = d * (float)kIq4nlValues[b[2 + j] & 0xF]; hi[j] = d * (float)kIq4nlValues[b[2 + j] >> 4]; } }
+      break;
+    case ORC_IQ4_XS:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); uint32_t sh = (uint32_t)b[2] | ((uint32_t)b[3] << 8); const uint8_t* sl = b + 4; const uint8_t* qs = b + 8; float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          int ls = (int)((sl[ib / 2] >> (4 * (ib % 2))) & 0xF) | (int)(((sh >> (2 * ib)) & 3) << 4); float dl = d * (float)(ls - 32);
+          for (int j = 0; j < 16; ++j) { yy[j] = (float)kIq4nlValues[qs[j] & 0xF] * dl; yy[j + 16] = (float)kIq4nlValues[qs[j] >> 4] * dl; }
+          yy += 32; qs += 16;
+        }
+      }
+      break;
+    case ORC_Q6_K:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; const uint8_t* ql = b; const uint8_t* qh = b + 128; const int8_t* sc = (const int8_t*)(b + 192); float d = h2f(b + 208); float* yy = y + i * 256;
+        for (int n = 0; n < 2; ++n) {
+          for (int l = 0; l < 32; ++l) {
+            int is = l / 16;
+            int q1 = (int)((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32, q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+            int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32, q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+            yy[l] = d * (float)sc[is] * (float)q1; yy[l + 32] = d * (float)sc[is + 2] * (float)q2;
+            yy[l + 64] = d * (float)sc[is + 4] * (float)q3; yy[l + 96] = d * (float)sc[is + 6] * (float)q4;
+          }
+          yy += 128; ql += 64; qh += 32; sc += 8;
+        }
+      }
+      break;
+    case ORC_IQ2_XXS:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); const uint8_t* qs = b + 2; float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          const uint8_t* a0 = qs + 8 * ib; uint32_t a1 = (uint32_t)a0[4] | ((uint32_t)a0[5] << 8) | ((uint32_t)a0[6] << 16) | ((uint32_t)a0[7] << 24);
+          float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+          for (int l = 0; l < 4; ++l) {
+            uint64_t gv = T.iq2xxs[a0[l]]; float g[8]; for (int j = 0; j < 8; ++j) g[j] = (float)((gv >> (8 * j)) & 0xFF);
+            put8(yy, db, g, T.ksigns[(a1 >> (7 * l)) & 127]); yy += 8;
+          }
+        }
+      }
+      break;
+    case ORC_IQ2_S:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); const uint8_t* qs = b + 2; const uint8_t* signs = b + 34; const uint8_t* qh = b + 66; const uint8_t* sc = b + 74; float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          float db[2] = { d * (0.5f + (float)(sc[ib] & 0xF)) * 0.25f, d * (0.5f + (float)(sc[ib] >> 4)) * 0.25f };
+          for (int l = 0; l < 4; ++l) {
+            uint32_t idx = (uint32_t)qs[l] | (((uint32_t)qh[ib] << (8 - 2 * l)) & 0x300);
+            uint64_t gv = T.iq2s[idx]; float g[8]; for (int j = 0; j < 8; ++j) g[j] = (float)((gv >> (8 * j)) & 0xFF);
+            put8(yy, db[l / 2], g, signs[l]); yy += 8;
+          }
+          qs += 4; signs += 4;
+        }
+      }
+      break;
+    case ORC_IQ3_XXS:
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b); const uint8_t* qs = b + 2; const uint8_t* ss = b + 66; float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          uint32_t a = (uint32_t)ss[4 * ib] | ((uint32_t)ss[4 * ib + 1] << 8) | ((uint32_t)ss[4 * ib + 2] << 16) | ((uint32_t)ss[4 * ib + 3] << 24);
+          float db = d * (0.5f + (float)(a >> 28)) * 0.5f;
+          for (int l = 0; l < 4; ++l) {
+            uint32_t g1 = T.iq3xxs[qs[8 * ib + 2 * l]], g2 = T.iq3xxs[qs[8 * ib + 2 * l + 1]];
+            float g[8]; for (int j = 0; j < 4; ++j) { g[j] = (float)((g1 >> (8 * j)) & 0xFF); g[4 + j] = (float)((g2 >> (8 * j)) & 0xFF); }
+            put8(yy, db, g, T.ksigns[(a >> (7 * l)) & 127]); yy += 8;
+          }
         }
       }
       break;

@@ -20,7 +20,7 @@ struct pyre_ctx {
   // staging for host-pointer entry points
   void* stage = nullptr; size_t stage_bytes = 0;
   // expanded codebooks in device memory: iq3s u32[512], iq2xs u64[512]
-  uint32_t* d_iq3s = nullptr; uint64_t* d_iq2xs = nullptr;
+  uint32_t* d_iq3s = nullptr; uint64_t* d_iq2xs = nullptr; uint16_t* d_cb = nullptr;
   // optional per-kernel-class timing: an event pair around every launch, resolved at pyre_prof_report
   struct ProfPending { const char* name; double bytes; hipEvent_t a, b; };
   struct ProfAcc { long count = 0; double ms = 0, bytes = 0; };
@@ -61,7 +61,10 @@ int pyre_fuse_check(pyre_ctx* ctx);
 struct QMatDev {
   const uint8_t* p0; const uint8_t* p1; const uint8_t* p2; const uint8_t* p3; const uint8_t* pb;
   int rows, cols, U, tiles, fmt;
+  uint32_t ty; int gel, gbytes;        // GGUF type the matrix was created from and its block geometry (algorithmic byte counts)
+  uint32_t lut[4]; int bias;           // C4 value table (entry = value + bias)
 };
+inline double qmat_gguf_bytes(const QMatDev& m, double rows) { return rows * (m.cols / m.gel) * m.gbytes; }
 
 struct pyre_qmat {
   pyre_ctx* ctx; uint32_t ty; size_t rows, cols; size_t gguf_bytes;

@@ -63,7 +63,11 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
     uint32_t v = 0; for (int j = 0; j < 4; ++j) v |= (uint32_t)(2 * ((kIq3sCode[i] >> (3 * j)) & 7) + 1) << (8 * j); g3[i] = v;
     uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(kIq2xsCode[i] >> (2 * j)) & 3] << (8 * j); g2[i] = w;
   }
-  if ((e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
+  std::vector<uint16_t> cb(1536);          // compact codes as they are: [iq2xxs 256 | iq2s 1024 | iq3xxs 256], used once per matrix by the load-time re-coding
+  for (int i = 0; i < 256; ++i) { cb[i] = kIq2xxsCode[i]; cb[1280 + i] = kIq3xxsCode[i]; }
+  for (int i = 0; i < 1024; ++i) cb[256 + i] = kIq2sCode[i];
+  if ((e = hipMalloc((void**)&ctx->d_cb, 1536 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 1536 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
+      (e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
       (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->fuse_ctl, 1024)) != hipSuccess || (e = hipMemset(ctx->fuse_ctl, 0, 1024)) != hipSuccess) {
     int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: codebook upload: %s", hipGetErrorString(e)); pyre_ctx_destroy(ctx); return rc; }
@@ -88,6 +92,7 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   if (ctx->stage) (void)hipFree(ctx->stage);
   if (ctx->d_iq3s) (void)hipFree(ctx->d_iq3s);
+  if (ctx->d_cb) (void)hipFree(ctx->d_cb);
   if (ctx->mfma_buf) (void)hipFree(ctx->mfma_buf);
   if (ctx->fuse_ctl) (void)hipFree(ctx->fuse_ctl);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
@@ -134,13 +139,13 @@ const char* pyre_prof_report(pyre_ctx* ctx) {
 int pyre_synth_blocks(pyre_ctx* ctx, uint32_t ty, size_t n_blocks, uint64_t seed, float d_lo, float d_hi, void* dev_out) {
   if (!ctx || !dev_out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_synth_blocks: null argument");
   int fmt = fmt_from_ggml(ty); if (fmt < 0) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_synth_blocks: unsupported ggml type %u", ty);
-  FmtGeom g = fmt_geom(fmt); size_t nbytes = n_blocks * (size_t)g.bytes; if (!nbytes) return PYRE_OK;
+  struct { int el, bytes; } g{1, 4}; ggml_geom(ty, &g.el, &g.bytes); size_t nbytes = n_blocks * (size_t)g.bytes; if (!nbytes) return PYRE_OK;
   size_t nw = (nbytes + 7) / 8;
   hipLaunchKernelGGL(k_synth_payload, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, ctx->stream, seed, nbytes, (uint8_t*)dev_out);
   PYRE_CHECK_LAUNCH(ctx);
   int nf = fmt == FMT_Q4_K ? 2 : (fmt >= FMT_Q8_0 ? 1 : 0);
-  if (nf) {
-    hipLaunchKernelGGL(k_synth_scales, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx->stream, seed, n_blocks, g.bytes, nf, 0, 2, d_lo, d_hi, (uint8_t*)dev_out);
+  if (nf) {      // the f16 super-block scale sits at byte 0 of every block format except Q6_K (byte 208)
+    hipLaunchKernelGGL(k_synth_scales, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx->stream, seed, n_blocks, g.bytes, nf, ty == PYRE_Q6_K ? 208 : 0, 2, d_lo, d_hi, (uint8_t*)dev_out);
     PYRE_CHECK_LAUNCH(ctx);
   }
   return PYRE_OK;

@@ -2,25 +2,62 @@
 // dot products the GEMV kernels use.  Format definitions: src/model/gguf_q.rs:67-166 of the reference.
 #pragma once
 #include "common.h"
+#include "iq_codebooks.h"
 
-enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_COUNT = 7 };
+// Device formats.  The first seven keep the GGUF block's own fields; C4 and C8 are what every other supported GGUF
+// type is re-coded into at load: one f32 scale per 16 values (the exact f32 product the reference forms before its
+// last multiply) and, per value, a 4-bit code into a 16-entry table of small integers (C4) or an int8 (C8), so that
+// value = scale * integer is the reference's own last multiply.
+enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_C4 = 7, FMT_C8 = 8, FMT_COUNT = 9 };
 
-struct FmtGeom { int el, bytes; int V; int e1, e2, e3, eb; };   // GGUF block (elements, bytes); plane entry sizes
+struct FmtGeom { int V; int e1, e2, e3, eb; };   // plane entry sizes: 16-byte chunks per unit in p0; bytes per unit in p1..p3; bytes per super-block in pb
 __host__ __device__ inline FmtGeom fmt_geom(int fmt) {
   switch (fmt) {
-    case FMT_F32:    return {1, 4, 16, 0, 0, 0, 0};
-    case FMT_F16:    return {1, 2, 8, 0, 0, 0, 0};
-    case FMT_BF16:   return {1, 2, 8, 0, 0, 0, 0};
-    case FMT_Q8_0:   return {32, 34, 4, 4, 0, 0, 0};     // p1: the two f16 scales of the unit's two blocks
-    case FMT_Q4_K:   return {256, 144, 2, 0, 0, 0, 16};  // pb: d, dmin, scales[12]
-    case FMT_IQ2_XS: return {256, 74, 1, 2, 0, 0, 2};    // p1: two scale bytes; pb: d
-    default:         return {256, 110, 2, 0, 0, 1, 2};   // IQ3_S, re-coded at load: p0: 64 four-bit codes, p3: scale byte; pb: d
+    case FMT_F32:    return {16, 0, 0, 0, 0};
+    case FMT_F16:    return {8, 0, 0, 0, 0};
+    case FMT_BF16:   return {8, 0, 0, 0, 0};
+    case FMT_Q8_0:   return {4, 4, 0, 0, 0};     // p1: the two f16 scales of the unit's two blocks
+    case FMT_Q4_K:   return {2, 0, 0, 0, 16};    // pb: d, dmin, scales[12]
+    case FMT_IQ2_XS: return {1, 2, 0, 0, 2};     // p1: two scale bytes; pb: d
+    case FMT_C4:     return {2, 16, 0, 0, 0};    // p0: 64 four-bit codes; p1: four f32 scales
+    case FMT_C8:     return {4, 16, 0, 0, 0};    // p0: 64 int8 values; p1: four f32 scales
+    default:         return {2, 0, 0, 1, 2};     // IQ3_S, re-coded at load: p0: 64 four-bit codes, p3: scale byte; pb: d
   }
+}
+// GGUF block geometry (elements, bytes) of the types the library loads (QType::geom, gguf_q.rs:33-42); false for the rest
+__host__ __device__ inline bool ggml_geom(uint32_t ty, int* el, int* bytes) {
+  switch (ty) {
+    case PYRE_F32: *el = 1; *bytes = 4; return true;  case PYRE_F16: case PYRE_BF16: *el = 1; *bytes = 2; return true;
+    case PYRE_Q4_0: *el = 32; *bytes = 18; return true;  case PYRE_Q5_0: *el = 32; *bytes = 22; return true;  case PYRE_Q8_0: *el = 32; *bytes = 34; return true;
+    case PYRE_Q4_K: *el = 256; *bytes = 144; return true;  case PYRE_Q6_K: *el = 256; *bytes = 210; return true;
+    case PYRE_IQ2_XXS: *el = 256; *bytes = 66; return true;  case PYRE_IQ2_XS: *el = 256; *bytes = 74; return true;  case PYRE_IQ2_S: *el = 256; *bytes = 82; return true;
+    case PYRE_IQ3_XXS: *el = 256; *bytes = 98; return true;  case PYRE_IQ3_S: *el = 256; *bytes = 110; return true;
+    case PYRE_IQ4_NL: *el = 32; *bytes = 18; return true;  case PYRE_IQ4_XS: *el = 256; *bytes = 136; return true;
+  }
+  return false;
 }
 inline int fmt_from_ggml(uint32_t ty) {
   switch (ty) { case PYRE_F32: return FMT_F32; case PYRE_F16: return FMT_F16; case PYRE_BF16: return FMT_BF16; case PYRE_Q8_0: return FMT_Q8_0;
-    case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S; }
+    case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S;
+    case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ2_XXS: case PYRE_IQ2_S: case PYRE_IQ3_XXS: return FMT_C4;
+    case PYRE_Q5_0: case PYRE_Q6_K: return FMT_C8; }
   return -1;
+}
+// The C4 value table of a GGUF type: entry c (byte c%4 of word c/4) holds value + bias, 0..255.
+//   Q4_0: c - 8.  IQ4_NL, IQ4_XS: the sixteen non-linear levels (kIq4nlValues).  The i-quants code a value as
+//   (negative << 3) | magnitude index: magnitudes {8, 25, 43} (IQ2_XXS, IQ2_S), {4, 12, .., 52, 62} (IQ3_XXS).
+inline void c4_table(uint32_t ty, uint32_t lut[4], int* bias) {
+  int v[16] = {0}; int b = 0;
+  static const int tri[3] = {8, 25, 43}; static const int lv3[8] = {4, 12, 20, 28, 36, 44, 52, 62};
+  switch (ty) {
+    case PYRE_Q4_0: for (int c = 0; c < 16; ++c) v[c] = c - 8; b = 8; break;
+    case PYRE_IQ4_NL: case PYRE_IQ4_XS: for (int c = 0; c < 16; ++c) v[c] = kIq4nlValues[c]; b = 127; break;
+    case PYRE_IQ2_XXS: case PYRE_IQ2_S: for (int c = 0; c < 3; ++c) { v[c] = tri[c]; v[8 + c] = -tri[c]; } b = 43; break;
+    case PYRE_IQ3_XXS: for (int c = 0; c < 8; ++c) { v[c] = lv3[c]; v[8 + c] = -lv3[c]; } b = 62; break;
+    default: break;
+  }
+  for (int w = 0; w < 4; ++w) { lut[w] = 0; for (int k = 0; k < 4; ++k) lut[w] |= (uint32_t)(v[4 * w + k] + b) << (8 * k); }
+  *bias = b;
 }
 
 // ---- plane accessors ------------------------------------------------------------------------------------------------
@@ -88,6 +125,18 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
         for (int jj = 0; jj < 8; ++jj) y[32 * ib + 8 * l + jj] = flip(db * (float)(uint32_t)((g >> (8 * jj)) & 0xFF), (sg >> jj) & 1);
       }
     }
+  } else if constexpr (FMT == FMT_C4) {            // scale * table[code]: the last multiply of gguf_q.rs:75,83,88,125,135,140
+    uint4 sq = ld_small<uint4>(m.p1, m, tile, ku, lane); float sc[4] = {__uint_as_float(sq.x), __uint_as_float(sq.y), __uint_as_float(sq.z), __uint_as_float(sq.w)};
+    for (int c = 0; c < 2; ++c) {
+      uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int j = 0; j < 32; ++j) { uint32_t code = (w[j >> 3] >> (4 * (j & 7))) & 0xF; int val = (int)((m.lut[code >> 2] >> (8 * (code & 3))) & 0xFF) - m.bias; y[32 * c + j] = sc[2 * c + (j >> 4)] * (float)val; }
+    }
+  } else if constexpr (FMT == FMT_C8) {            // scale * int8: the last multiply of gguf_q.rs:78,120-121
+    uint4 sq = ld_small<uint4>(m.p1, m, tile, ku, lane); float sc[4] = {__uint_as_float(sq.x), __uint_as_float(sq.y), __uint_as_float(sq.z), __uint_as_float(sq.w)};
+    for (int c = 0; c < 4; ++c) {
+      uint4 v = ld_vec<4>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (int k = 0; k < 16; ++k) y[16 * c + k] = sc[c] * (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3)));
+    }
   } else {                                         // IQ3_S, gguf_q.rs:141-151, from the 4-bit codes (see iq3s_code)
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
     uint32_t sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
@@ -102,7 +151,7 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
 // ---- factored per-unit dot products for the GEMV ------------------------------------------------------------------
 // A unit's packed data is fetched first (unit_load) and consumed later (unit_fma), so a kernel can issue the weight
 // loads ahead of a barrier or of the previous unit's arithmetic; unit_dot does both at once.
-template <int FMT> struct UnitRaw { uint4 v[FMT == FMT_F32 ? 16 : (FMT == FMT_F16 || FMT == FMT_BF16) ? 8 : FMT == FMT_Q8_0 ? 4 : (FMT == FMT_Q4_K || FMT == FMT_IQ3_S) ? 2 : 1]; uint4 hb; uint32_t s0, s1; };
+template <int FMT> struct UnitRaw { uint4 v[FMT == FMT_F32 ? 16 : (FMT == FMT_F16 || FMT == FMT_BF16) ? 8 : (FMT == FMT_Q8_0 || FMT == FMT_C8) ? 4 : (FMT == FMT_Q4_K || FMT == FMT_IQ3_S || FMT == FMT_C4) ? 2 : 1]; uint4 hb; uint32_t s0, s1; };
 template <int FMT> __device__ __forceinline__ UnitRaw<FMT> unit_load(const QMatDev& m, int tile, int ku, int lane) {
   UnitRaw<FMT> r; r.hb = uint4{0, 0, 0, 0}; r.s0 = 0; r.s1 = 0;
   constexpr int V = sizeof(r.v) / sizeof(uint4);
@@ -110,13 +159,21 @@ template <int FMT> __device__ __forceinline__ UnitRaw<FMT> unit_load(const QMatD
   for (int c = 0; c < V; ++c) r.v[c] = ld_vec<V>(m, tile, ku, c, lane);
   if constexpr (FMT == FMT_Q8_0) r.s0 = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
   if constexpr (FMT == FMT_Q4_K) r.hb = ld_block<uint4>(m, tile, ku, lane);
+  if constexpr (FMT == FMT_C4 || FMT == FMT_C8) r.hb = ld_small<uint4>(m.p1, m, tile, ku, lane);
   if constexpr (FMT == FMT_IQ2_XS) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint16_t>(m.p1, m, tile, ku, lane); }
   if constexpr (FMT == FMT_IQ3_S) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint8_t>(m.p3, m, tile, ku, lane); }
   return r;
 }
 // xs points at the unit's 64 activations of token 0 (wave-uniform address -> scalar loads); token t is xs + t*xstride.
 // acc[t] += sum_j W[row, 64*ku + j] * x[t][64*ku + j].  The operation sequence per token does not depend on T.
-template <int FMT, int T> __device__ __forceinline__ void unit_fma(const UnitRaw<FMT>& r, int ku, const uint2* lds2, int lane,
+// Four table look-ups at once: byte k of `codes` (0..15) -> byte k of the result.  v_perm_b32 picks bytes of the
+// low / high half of the table by the codes' low three bits; bit 3 then chooses between the halves.
+__device__ __forceinline__ uint32_t c4_lookup(const QMatDev& m, uint32_t codes) {
+  uint32_t i7 = codes & 0x07070707u, b3 = codes & 0x08080808u, pick = (b3 << 5) - (b3 >> 3);     // 0xFF in every byte whose code has bit 3
+  uint32_t lo = __builtin_amdgcn_perm(m.lut[1], m.lut[0], i7), hi = __builtin_amdgcn_perm(m.lut[3], m.lut[2], i7);
+  return (lo & ~pick) | (hi & pick);
+}
+template <int FMT, int T> __device__ __forceinline__ void unit_fma(const QMatDev& m, const UnitRaw<FMT>& r, int ku, const uint2* lds2, int lane,
                                                                    const float* __restrict__ xs, int xstride, float (&acc)[T]) {
   if constexpr (FMT == FMT_F32) {
 #pragma unroll
@@ -201,6 +258,53 @@ _Pragma("unroll")
         for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
       }
     }
+  } else if constexpr (FMT == FMT_C4) {   // value = table[c] - bias: per 16-value group  scale * (sum table[c] x - bias sum x)
+    uint4 v0 = r.v[0], v1 = r.v[1];
+    uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+    float sc[4] = {__uint_as_float(r.hb.x), __uint_as_float(r.hb.y), __uint_as_float(r.hb.z), __uint_as_float(r.hb.w)};
+    float sx[T][4];            // group sums of the activations: lane j holds x[j], folded inside each quarter of the wave
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      float xv = xs[t * xstride + lane];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) xv += __shfl_xor(xv, o);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) sx[t][g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), 16 * g));
+    }
+    const float nbias = -(float)m.bias;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float part[T];
+_Pragma("unroll")
+      for (int t = 0; t < T; ++t) part[t] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        uint32_t u = w[2 * g + k], lo = c4_lookup(m, u & 0x0F0F0F0Fu), hi = c4_lookup(m, (u >> 4) & 0x0F0F0F0Fu);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          float fl = (float)((lo >> (8 * b)) & 0xFF), fh = (float)((hi >> (8 * b)) & 0xFF);
+#pragma unroll
+          for (int t = 0; t < T; ++t) { part[t] = fmaf(fl, xs[t * xstride + 16 * g + 8 * k + 2 * b], part[t]); part[t] = fmaf(fh, xs[t * xstride + 16 * g + 8 * k + 2 * b + 1], part[t]); }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(sc[g], fmaf(nbias, sx[t][g], part[t]), acc[t]);
+    }
+  } else if constexpr (FMT == FMT_C8) {
+    float sc[4] = {__uint_as_float(r.hb.x), __uint_as_float(r.hb.y), __uint_as_float(r.hb.z), __uint_as_float(r.hb.w)};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float part[T];
+_Pragma("unroll")
+      for (int t = 0; t < T; ++t) part[t] = 0.0f;
+      uint4 v = r.v[c]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 16; ++k) { float f = (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3)));
+#pragma unroll
+        for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 16 * c + k], part[t]); }
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(sc[c], part[t], acc[t]);
+    }
   } else {   // IQ3_S from 4-bit codes c = (w + 15) / 2: sum w x = 2 sum c x - 15 sum x per 32-value sub-block
     float d = h2f_bits(r.s0);
     uint32_t sc = r.s1;
@@ -238,5 +342,5 @@ _Pragma("unroll")
 template <int FMT, int T> __device__ __forceinline__ void unit_dot(const QMatDev& m, const uint2* lds2, int tile, int ku, int lane,
                                                                    const float* __restrict__ xs, int xstride, float (&acc)[T]) {
   UnitRaw<FMT> r = unit_load<FMT>(m, tile, ku, lane);
-  unit_fma<FMT, T>(r, ku, lds2, lane, xs, xstride, acc);
+  unit_fma<FMT, T>(m, r, ku, lds2, lane, xs, xstride, acc);
 }

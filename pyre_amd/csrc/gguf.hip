@@ -2,7 +2,7 @@
 // pyre_model_create is called with the tensors found).
 // Follows Gguf::open / shard_paths / Meta (src/model/gguf_q.rs:250-336) and Model::load's metadata keys and tensor
 // names (src/model/qwen4exp_gguf.rs:462-524).
-#include "common.h"
+#include "formats.h"
 #include <errno.h>
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -85,9 +85,8 @@ const char* ggml_name(uint32_t ty) {
 }
 // block geometry of the types this library computes with (QType::geom, gguf_q.rs:33-42); false for the others
 bool type_geom(uint32_t ty, size_t* el, size_t* bytes) {
-  switch (ty) { case PYRE_F32: *el = 1; *bytes = 4; return true; case PYRE_F16: case PYRE_BF16: *el = 1; *bytes = 2; return true; case PYRE_Q8_0: *el = 32; *bytes = 34; return true;
-    case PYRE_Q4_K: *el = 256; *bytes = 144; return true; case PYRE_IQ2_XS: *el = 256; *bytes = 74; return true; case PYRE_IQ3_S: *el = 256; *bytes = 110; return true; }
-  return false;
+  int e = 0, b = 0; if (!ggml_geom(ty, &e, &b)) return false;
+  *el = (size_t)e; *bytes = (size_t)b; return true;
 }
 
 }  // namespace

@@ -74,7 +74,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, T>(raw, ks * nw * upw + lu, lds2, lane, xs + lu * 64, L, acc); }
+  for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, T>(m, raw, ks * nw * upw + lu, lds2, lane, xs + lu * 64, L, acc); }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
@@ -124,7 +124,7 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  unit_fma<FMT, T>(raw, ku, lds2, lane, lo + ku * 64, lr, acc);
+  unit_fma<FMT, T>(up, raw, ku, lds2, lane, lo + ku * 64, lr, acc);
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
   __syncthreads();
@@ -160,16 +160,14 @@ DownPlan down_plan(const HcDev& h) {
 template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out,
                                                const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   const int L = p.nw * p.upw * 64; size_t lds = 4 * ((size_t)T * L + (size_t)p.nw * T * 64 + (size_t)p.nw * T);
-  FmtGeom g = fmt_geom(FMT);
-  ProfScope ps(ctx, "hc_norm_down", (double)h.di.rows * (h.di.cols / g.el) * g.bytes + 4.0 * T * h.hc * h.d * 4);
+  ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
   hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, eps,
                      w.xn, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, float* mixed, float* inj) {
   const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64);
-  FmtGeom g = fmt_geom(FMT);
-  ProfScope ps(ctx, "hc_up_mix", (double)h.up.rows * (h.up.cols / g.el) * g.bytes + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
+  ProfScope ps(ctx, "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
   hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, w.xn, h.d, mixed, inj,
                      (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
@@ -180,6 +178,7 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
 #define HC_FMT_SWITCH(fmt, BODY) \
   switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; BODY } case FMT_F16: { constexpr int F = FMT_F16; BODY } case FMT_BF16: { constexpr int F = FMT_BF16; BODY } \
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; BODY } case FMT_Q4_K: { constexpr int F = FMT_Q4_K; BODY } case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; BODY } \
+    case FMT_C4: { constexpr int F = FMT_C4; BODY } case FMT_C8: { constexpr int F = FMT_C8; BODY } \
     default: { constexpr int F = FMT_IQ3_S; BODY } }
 int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, eps))
@@ -221,8 +220,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     if (nwg <= 240 && lds <= 60000) {
       mega::Comb cb{comb_out, mega::MoeOutC{mo.partial, mo.sel_w, mo.sg, mo.d, mo.k}, comb_inj};
       mega::HcPlan pl{p.nw, p.upw, p.ksplit};
-      FmtGeom g = fmt_geom(h.di.fmt);
-      ProfScope ps(ctx, "hc_mix_fused", ((double)h.di.rows * (h.di.cols / g.el) + (double)h.up.rows * (h.up.cols / g.el)) * g.bytes + 4.0 * h.hc * h.d * 4);
+      ProfScope ps(ctx, "hc_mix_fused", qmat_gguf_bytes(h.di, h.di.rows) + qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * h.hc * h.d * 4);
       switch (h.di.fmt) {
 #define HC_FUSED_CASE(F) case F: hipLaunchKernelGGL((mega::k_hc_mix_fused<F>), dim3(nwg), dim3(mega::WGT), lds, ctx->stream, h, pl, x_in, in_ss, x_out, cb, eps, w.xn, w.o, mixed, inj, ctx->fuse_ctl, 2000000u); break;
         HC_FUSED_CASE(FMT_F32) HC_FUSED_CASE(FMT_F16) HC_FUSED_CASE(FMT_BF16) HC_FUSED_CASE(FMT_Q8_0) HC_FUSED_CASE(FMT_Q4_K) default: HC_FUSED_CASE(FMT_IQ3_S)

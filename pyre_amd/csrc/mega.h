@@ -162,7 +162,7 @@ template <int FMT> __device__ __forceinline__ void st_norm_down(const HcDev& h, 
     __syncthreads();
     if (act) {
       float acc[1] = {0.0f};
-      for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, 1>(raw, ks * nw * upw + lu, (const uint2*)nullptr, lane, xs + lu * 64, L, acc); }
+      for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, 1>(m, raw, ks * nw * upw + lu, (const uint2*)nullptr, lane, xs + lu * 64, L, acc); }
       red[wave * 64 + lane] = acc[0];
     }
     __syncthreads();
@@ -203,7 +203,7 @@ template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int
     __syncthreads();
     if (act) {
       float acc[1] = {0.0f};
-      unit_fma<FMT, 1>(raw, ku, (const uint2*)nullptr, lane, lo + ku * 64, lr, acc);
+      unit_fma<FMT, 1>(up, raw, ku, (const uint2*)nullptr, lane, lo + ku * 64, lr, acc);
       red[wave * 64 + lane] = acc[0];
     }
     __syncthreads();

@@ -55,7 +55,7 @@ struct Builder {
   int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes) {
     uint32_t ty = ts[0]->ggml_type; uint64_t cols = ts[0]->cols; uint32_t dev = ts[0]->on_device; uint64_t rows = 0; size_t total = 0;
     int fmt = fmt_from_ggml(ty); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported tensor type");
-    FmtGeom g = fmt_geom(fmt);
+    struct { int el, bytes; } g{1, 4}; ggml_geom(ty, &g.el, &g.bytes);
     for (int i = 0; i < n; ++i) {
       if (!ts[i]->data) return fail(PYRE_E_ARG, "missing tensor");
       if (ts[i]->ggml_type != ty || ts[i]->cols != cols || ts[i]->on_device != dev) return fail(PYRE_E_TYPE, "tensors of one projection group differ in type, width or location");
@@ -82,7 +82,7 @@ struct Builder {
     float* d = nullptr; PYRE_HIP(ctx, hipMalloc((void**)&d, n * 4)); m->bufs.push_back(d);
     if (t.ggml_type == PYRE_F32) { PYRE_HIP(ctx, hipMemcpy(d, t.data, n * 4, t.on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice)); }
     else {
-      pyre_qmat* q = nullptr; int fmt = fmt_from_ggml(t.ggml_type); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported vector type"); FmtGeom g = fmt_geom(fmt);
+      pyre_qmat* q = nullptr; int fmt = fmt_from_ggml(t.ggml_type); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported vector type"); struct { int el, bytes; } g{1, 4}; ggml_geom(t.ggml_type, &g.el, &g.bytes);
       size_t nb = n / g.el * g.bytes;
       int rc = t.on_device ? pyre_qmat_create_dev(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q) : pyre_qmat_create(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q); if (rc) return rc;
       rc = pyre_qmat_dequant_dev(ctx, q, d); if (!rc) rc = pyre_ctx_sync(ctx); pyre_qmat_destroy(q); if (rc) return rc;
@@ -166,7 +166,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   if ((rc = B.hc(gl[PYRE_G_OUTPUT_HC_NORM], gl[PYRE_G_OUTPUT_HC_DOWN], nullptr, gl[PYRE_G_OUTPUT_HC_UP], &m->head, &tok_bytes))) return rc;
   if ((rc = B.one(gl[PYRE_G_OUTPUT], &m->out, &tok_bytes))) return rc;
   if (m->out.rows != c.vocab || m->out.cols != c.d) return B.fail(PYRE_E_SHAPE, "output shape");
-  { FmtGeom g = fmt_geom(m->embd.fmt); tok_bytes += (size_t)c.d / g.el * g.bytes; }
+  tok_bytes += (size_t)c.d / m->embd.gel * m->embd.gbytes;
   m->token_weight_bytes = tok_bytes;
   // window workspace
   const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);

@@ -158,13 +158,14 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
 #define MOE_FMT_DISPATCH(fmt, CALL) \
   switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; CALL; } break; case FMT_F16: { constexpr int F = FMT_F16; CALL; } break; case FMT_BF16: { constexpr int F = FMT_BF16; CALL; } break; \
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
+    case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; \
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
 
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
   int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc;
-  auto mat_bytes = [](const QMatDev& q, double rows) { FmtGeom g = fmt_geom(q.fmt); return rows * (q.cols / g.el) * g.bytes; };
+  auto mat_bytes = [](const QMatDev& q, double rows) { return qmat_gguf_bytes(q, rows); };
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));

@@ -5,7 +5,7 @@
 
 // ---- repack: raw GGUF rows -> planes --------------------------------------------------------------------------------
 // One thread per (padded row, unit).  Rows beyond m.rows are written as zeros (they decode to 0 and are never stored).
-__global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_bytes, uint8_t* p0, uint8_t* p1, uint8_t* p2, uint8_t* p3, uint8_t* pb, const uint32_t* __restrict__ g3) {
+__global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_bytes, uint8_t* p0, uint8_t* p1, uint8_t* p2, uint8_t* p3, uint8_t* pb, const uint32_t* __restrict__ g3, const uint16_t* __restrict__ cb) {
   size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t total = (size_t)m.tiles * 64 * m.U;
   if (gid >= total) return;
@@ -34,6 +34,63 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
       put_vec(0, b + 2 + 16 * j);
       uint8_t* d = p1 + e * 2; d[0] = live ? b[66 + 2 * j] : 0; d[1] = live ? b[67 + 2 * j] : 0;
       if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
+    } break;
+    case FMT_C4: case FMT_C8: {
+      // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256]; code(e) and scale(e / 16) of the unit's 64 values e
+      uint32_t words[16]; float sc[4];
+      for (int i = 0; i < 16; ++i) words[i] = 0;
+      for (int i = 0; i < 4; ++i) sc[i] = 0.0f;
+      auto h2 = [](const uint8_t* q) { return __half2float(__ushort_as_half((unsigned short)(q[0] | (q[1] << 8)))); };
+      auto put4 = [&](int e, uint32_t code) { words[e >> 3] |= (code & 0xF) << (4 * (e & 7)); };
+      auto put8b = [&](int e, int q) { words[e >> 2] |= (uint32_t)(q & 0xFF) << (8 * (e & 3)); };
+      auto ks = [](uint32_t i) { return i | ((__popc(i) & 1u) << 7); };
+      if (live) switch (m.ty) {          // padding rows lie past the end of the raw buffer: never read them
+        case PYRE_Q4_0: case PYRE_IQ4_NL:                              // gguf_q.rs:74-75, 82-83: unit = two 32-value blocks
+          for (int h = 0; h < 2; ++h) { const uint8_t* b = row + (size_t)(2 * ku + h) * 18; sc[2 * h] = sc[2 * h + 1] = h2(b);
+            for (int j = 0; j < 16; ++j) { put4(32 * h + j, b[2 + j] & 0xF); put4(32 * h + 16 + j, b[2 + j] >> 4); } }
+          break;
+        case PYRE_Q5_0:                                                // gguf_q.rs:76-78
+          for (int h = 0; h < 2; ++h) { const uint8_t* b = row + (size_t)(2 * ku + h) * 22; sc[2 * h] = sc[2 * h + 1] = h2(b);
+            uint32_t qh = b[2] | (b[3] << 8) | (b[4] << 16) | ((uint32_t)b[5] << 24);
+            for (int j = 0; j < 16; ++j) { put8b(32 * h + j, (int)((b[6 + j] & 0xF) | (((qh >> j) << 4) & 0x10)) - 16); put8b(32 * h + 16 + j, (int)((b[6 + j] >> 4) | ((qh >> (j + 12)) & 0x10)) - 16); } }
+          break;
+        case PYRE_IQ4_XS: {                                            // gguf_q.rs:84-89
+          const uint8_t* b = row + (size_t)(ku >> 2) * 136; float d = h2(b); uint32_t sh = b[2] | (b[3] << 8);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; int ls = (int)((b[4 + ib / 2] >> (4 * (ib % 2))) & 0xF) | (int)(((sh >> (2 * ib)) & 3) << 4);
+            sc[2 * c] = sc[2 * c + 1] = d * (float)(ls - 32); const uint8_t* q = b + 8 + 16 * ib;
+            for (int j = 0; j < 16; ++j) { put4(32 * c + j, q[j] & 0xF); put4(32 * c + 16 + j, q[j] >> 4); } }
+        } break;
+        case PYRE_Q6_K: {                                              // gguf_q.rs:114-121
+          const uint8_t* b = row + (size_t)(ku >> 2) * 210; float d = h2(b + 208); int n = (ku & 3) >> 1;
+          for (int c = 0; c < 2; ++c) { int qd = 2 * (ku & 1) + c;      // quarter of the 128-value half
+            for (int l = 0; l < 32; ++l) { uint32_t qlb = b[64 * n + l + ((qd & 1) ? 32 : 0)], nib = qd < 2 ? (qlb & 0xF) : (qlb >> 4), hi2 = (b[128 + 32 * n + l] >> (2 * qd)) & 3;
+              put8b(32 * c + l, (int)(nib | (hi2 << 4)) - 32); }
+            for (int g = 0; g < 2; ++g) sc[2 * c + g] = d * (float)(int)(int8_t)b[192 + 8 * n + 2 * qd + g]; }
+        } break;
+        case PYRE_IQ2_XXS: {                                           // gguf_q.rs:122-125
+          const uint8_t* b = row + (size_t)(ku >> 2) * 66; float d = h2(b);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; const uint8_t* a0 = b + 2 + 8 * ib; uint32_t a1 = a0[4] | (a0[5] << 8) | (a0[6] << 16) | ((uint32_t)a0[7] << 24);
+            sc[2 * c] = sc[2 * c + 1] = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+            for (int l = 0; l < 4; ++l) { uint32_t g = cb[a0[l]], sg = ks((a1 >> (7 * l)) & 127); for (int j = 0; j < 8; ++j) put4(32 * c + 8 * l + j, ((g >> (2 * j)) & 3) | (((sg >> j) & 1) << 3)); } }
+        } break;
+        case PYRE_IQ2_S: {                                             // gguf_q.rs:130-135
+          const uint8_t* b = row + (size_t)(ku >> 2) * 82; float d = h2(b);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; uint32_t s = b[74 + ib], qh = b[66 + ib];
+            sc[2 * c] = d * (0.5f + (float)(s & 0xF)) * 0.25f; sc[2 * c + 1] = d * (0.5f + (float)(s >> 4)) * 0.25f;
+            for (int l = 0; l < 4; ++l) { uint32_t g = cb[256 + (b[2 + 4 * ib + l] | ((qh << (8 - 2 * l)) & 0x300))], sg = b[34 + 4 * ib + l];
+              for (int j = 0; j < 8; ++j) put4(32 * c + 8 * l + j, ((g >> (2 * j)) & 3) | (((sg >> j) & 1) << 3)); } }
+        } break;
+        case PYRE_IQ3_XXS: {                                           // gguf_q.rs:136-140
+          const uint8_t* b = row + (size_t)(ku >> 2) * 98; float d = h2(b);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; const uint8_t* ss = b + 66 + 4 * ib; uint32_t a = ss[0] | (ss[1] << 8) | (ss[2] << 16) | ((uint32_t)ss[3] << 24);
+            sc[2 * c] = sc[2 * c + 1] = d * (0.5f + (float)(a >> 28)) * 0.5f;
+            for (int l = 0; l < 4; ++l) { uint32_t g1 = cb[1280 + b[2 + 8 * ib + 2 * l]], g2 = cb[1280 + b[2 + 8 * ib + 2 * l + 1]], sg = ks((a >> (7 * l)) & 127);
+              for (int j = 0; j < 4; ++j) { put4(32 * c + 8 * l + j, ((g1 >> (3 * j)) & 7) | (((sg >> j) & 1) << 3)); put4(32 * c + 8 * l + 4 + j, ((g2 >> (3 * j)) & 7) | (((sg >> (4 + j)) & 1) << 3)); } } }
+        } break;
+        default: break;
+      }
+      for (int c = 0; c < g.V; ++c) { uint32_t* dst = (uint32_t*)(v + ((size_t)c * 64 + lane) * 16); for (int i = 0; i < 4; ++i) dst[i] = words[4 * c + i]; }
+      float* sd = (float*)(p1 + e * 16); for (int i = 0; i < 4; ++i) sd[i] = sc[i];
     } break;
     default: {   // IQ3_S: codebook lookups and signs are resolved here, once (gguf_q.rs:141-151), into 4-bit codes
       const uint8_t* b = row + (size_t)(ku >> 2) * 110; int j = ku & 3;
@@ -160,10 +217,9 @@ int gemv_nw(const QMatDev& m, int ksplit) {
 }
 template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
-  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s"};
+  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
-  FmtGeom g = fmt_geom(FMT);
-  ProfScope ps(ctx, name.c_str(), (double)m.rows * (m.cols / g.el) * g.bytes + 4.0 * T * ((double)m.cols + m.rows));
+  ProfScope ps(ctx, name.c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * T * ((double)m.cols + m.rows));
   hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
@@ -184,6 +240,7 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
 #define FMT_DISPATCH(fmt, CALL) \
   switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; CALL; } break; case FMT_F16: { constexpr int F = FMT_F16; CALL; } break; case FMT_BF16: { constexpr int F = FMT_BF16; CALL; } break; \
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
+    case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; \
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
 }  // namespace
 
@@ -252,10 +309,10 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
   if (!ctx || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: null argument");
   *out = nullptr;
   int fmt = fmt_from_ggml(ty); if (fmt < 0) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmat_create: unsupported ggml type %u", ty);
-  FmtGeom g = fmt_geom(fmt);
-  if (rows == 0 || cols == 0 || cols % PYRE_UNIT != 0 || cols % g.el != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu: cols must be a non-zero multiple of 64 and of the block size %d", rows, cols, g.el);
+  FmtGeom g = fmt_geom(fmt); int gel = 1, gbytes = 4; ggml_geom(ty, &gel, &gbytes);
+  if (rows == 0 || cols == 0 || cols % PYRE_UNIT != 0 || cols % gel != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu: cols must be a non-zero multiple of 64 and of the block size %d", rows, cols, gel);
   if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
-  size_t row_bytes = cols / g.el * g.bytes;
+  size_t row_bytes = cols / gel * gbytes;
   if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
   pyre_qmat* m = new pyre_qmat(); m->ctx = ctx; m->ty = ty; m->rows = rows; m->cols = cols; m->gguf_bytes = nbytes;
@@ -267,7 +324,8 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
   hipError_t e = hipMalloc(&m->base, m->dev_bytes);
   if (e != hipSuccess) { delete m; return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", s0 + s1 + s2 + s3 + sb, hipGetErrorString(e)); }
   uint8_t* b = (uint8_t*)m->base;
-  m->dv = QMatDev{b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (int)rows, (int)cols, U, tiles, fmt};
+  m->dv = QMatDev{b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (int)rows, (int)cols, U, tiles, fmt, ty, gel, gbytes, {0, 0, 0, 0}, 0};
+  if (fmt == FMT_C4) c4_table(ty, m->dv.lut, &m->dv.bias);
   const uint8_t* src = (const uint8_t*)blocks; void* tmp = nullptr;
   if (!on_device) {
     e = hipMalloc(&tmp, nbytes);
@@ -276,7 +334,7 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
     src = (const uint8_t*)tmp;
   }
   size_t total = ent * 1; unsigned nblk = (unsigned)((total + 255) / 256);
-  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (const uint32_t*)ctx->d_iq3s);
+  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (const uint32_t*)ctx->d_iq3s, (const uint16_t*)ctx->d_cb);
   e = hipGetLastError();
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (tmp) (void)hipFree(tmp);

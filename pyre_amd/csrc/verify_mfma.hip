@@ -170,8 +170,7 @@ int pyre_gemm_mfma_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t
   uint2* xb = (uint2*)buf; float* sx = (float*)((uint8_t*)buf + nb_xb); float* xscale = (float*)((uint8_t*)buf + nb_xb + nb_sx);
   { ProfScope ps(ctx, "verify_xsplit", 4.0 * t * m.cols + (double)nb_xb + nb_sx);
     hipLaunchKernelGGL(k_xsplit, dim3(1), dim3(1024), 0, ctx->stream, x, t, m.cols, xb, sx, xscale); } PYRE_CHECK_LAUNCH(ctx);
-  FmtGeom g = fmt_geom(FMT_IQ3_S);
-  { ProfScope ps(ctx, "verify_gemm_mfma", (double)m.rows * (m.cols / g.el) * g.bytes + 4.0 * t * ((double)m.cols + m.rows));
+  { ProfScope ps(ctx, "verify_gemm_mfma", qmat_gguf_bytes(m, m.rows) + 4.0 * t * ((double)m.cols + m.rows));
     // two tiles per workgroup: eight (activation operands fetched a quarter as often) measured slower on the 151936-row
     // head, 151 vs 117 us at t = 8 -- the kernel is bound by load latency per sub-block, not by operand fetches
     if (t <= 4) hipLaunchKernelGGL((k_gemm_mfma_iq3s<1, 2>), dim3((m.tiles + 1) / 2), dim3(512), 0, ctx->stream, m, xb, sx, xscale, y, t);

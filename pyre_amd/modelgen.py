@@ -111,9 +111,16 @@ HC_SLOTS_LAYER = (HCA_DOWN, HCA_INJECT, HCA_UP, HCF_DOWN, HCF_INJECT, HCF_UP)
 HC_SLOTS_GLOBAL = (G_HEAD_DOWN, G_HEAD_UP)
 
 
-def scale_range(c: Config, il, slot):
+# Random payloads of these two types decode to values about ten times larger per unit of the f16 scale than the others
+# (6-bit value x int8 sub-scale; 6-bit sub-scale x level up to 127): their scale range shrinks by that factor so that a
+# synthetic model has weights of the same size whatever type it is stored in.
+WIDE_TYPES = {synth.Q6_K: 10.0, synth.IQ4_XS: 9.0}
+
+
+def scale_range(c: Config, il, slot, ty=None):
     hc = slot in (HC_SLOTS_LAYER if il >= 0 else HC_SLOTS_GLOBAL)
-    return (c.d_lo / c.hc_d_div, c.d_hi / c.hc_d_div) if hc else (c.d_lo, c.d_hi)
+    div = (c.hc_d_div if hc else 1.0) * WIDE_TYPES.get(ty, 1.0)
+    return (c.d_lo / div, c.d_hi / div)
 
 
 def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
@@ -125,7 +132,7 @@ def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
                 return synth.bf16_normal(rows, cols, s, std)
             x = synth.normal((rows, cols), s, std)
             return (x if ty == synth.F32 else x.astype(np.float16)).view(np.uint8).reshape(-1).copy()
-        return synth.matrix(ty, rows, cols, s, *scale_range(c, il, slot))
+        return synth.matrix(ty, rows, cols, s, *scale_range(c, il, slot, ty))
     if kind == "router":
         return synth.bf16_normal(rows, cols, s, 0.02)
     name = kind.split(":")[1]
@@ -174,11 +181,11 @@ def build_device(ctx, c: Config, seed=1):
     globals_ = {}
     raw = []
     for il, slot, kind, ty, rows, cols in tensor_specs(c):
-        if kind == "q" and ty in (synth.Q8_0, synth.Q4_K, synth.IQ2_XS, synth.IQ3_S):
+        if kind == "q" and ty not in (synth.F32, synth.F16, synth.BF16):
             el, bs, _ = synth.GEOM[ty]
             nb = rows * (cols // el)
             dev = ctx.alloc(nb * bs)
-            lo, hi = scale_range(c, il, slot)
+            lo, hi = scale_range(c, il, slot, ty)
             ctx.synth_blocks(ty, nb, tensor_seed(seed, il, slot), lo, hi, dev_out=dev)
             raw.append(dev)
             entry = (ty, rows, cols, dev)

@@ -16,6 +16,11 @@ _ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 IQ3S_SHA256 = "bd1af4945a1717c65610b0284e4628b9a1ba3b306fae3a06f6e5f597356e349f"
 IQ2XS_SHA256 = "06e47aaca60b4dc1d9b5a3f34540437058a6b142b4d7a59d5ded769b4d1bf1de"
 KSIGNS_SHA256 = "a76742a603f8beca5212ecce0f1f02f11a4887fd2f7c8b15aca0ea3eb3380c31"
+IQ2XXS_SHA256 = "05826b5d3e472a3a78f196be62ac78acf81df0f909626e12ab9fa2a5d490dd54"
+IQ2S_SHA256 = "e1aa1473412b0552c2174c30ef22ab4073f6a181b85a17056e8249bd2932fd88"
+IQ3XXS_SHA256 = "46e35f5a997efdee6c99ce57854c8a0d4f0ff8ca57e5e8a60c0793ea580acf5d"
+# the IQ4_NL / IQ4_XS non-linear levels (ggml's kvalues_iq4nl, iq_tables.rs:579 of the reference)
+IQ4NL_VALUES = (-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113)
 
 
 def _codes(path, name):
@@ -40,6 +45,25 @@ def codebooks(header=None):
         par ^= (i >> b) & 1
     ks = (i | (par << 7)).astype(np.uint8)
     return g3, g2, ks
+
+
+def codebooks_more(header=None):
+    """(iq2xxs_grid u8[256,8], iq2s_grid u8[1024,8], iq3xxs_grid u8[256,4], iq4nl i8[16]) expanded from a codebook header."""
+    header = header or os.path.join(_ROOT, "oracle", "iq_codebooks.h")
+    tri = np.array([8, 25, 43], dtype=np.uint8)
+    lv3 = np.array([4, 12, 20, 28, 36, 44, 52, 62], dtype=np.uint8)
+    cxx, cs, c3 = _codes(header, "kIq2xxsCode"), _codes(header, "kIq2sCode"), _codes(header, "kIq3xxsCode")
+    gxx = np.stack([tri[(cxx >> (2 * j)) & 3] for j in range(8)], axis=1).astype(np.uint8)
+    gs = np.stack([tri[(cs >> (2 * j)) & 3] for j in range(8)], axis=1).astype(np.uint8)
+    g3 = np.stack([lv3[(c3 >> (3 * j)) & 7] for j in range(4)], axis=1).astype(np.uint8)
+    m = re.search(r"kIq4nlValues\[16\] = \{(.*?)\};", open(header).read(), re.S)
+    kv = np.array([int(v) for v in re.findall(r"-?\d+", m.group(1))], dtype=np.int8)
+    return gxx, gs, g3, kv
+
+
+def codebook_digests_more(header=None):
+    gxx, gs, g3, kv = codebooks_more(header)
+    return (hashlib.sha256(gxx.tobytes()).hexdigest(), hashlib.sha256(gs.tobytes()).hexdigest(), hashlib.sha256(g3.tobytes()).hexdigest(), tuple(int(v) for v in kv))
 
 
 def codebook_digests(header=None):
@@ -116,6 +140,83 @@ def dequant(ty, raw, n):
         grid = g3[idx].astype(np.float32).reshape(-1, 8, 4, 8)         # two 4-byte entries per group of 8 values
         s = _signs(sg)
         return ((db[:, :, None, None] * grid).astype(np.float32) * s).astype(np.float32).reshape(-1)
+    f = np.float32
+    if ty == 2:                                                        # Q4_0: (nibble - 8) * d; low nibbles first, then high
+        b = raw[:n // 32 * 18].reshape(-1, 18)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        q = np.concatenate([b[:, 2:] & 0xF, b[:, 2:] >> 4], axis=1).astype(np.int32) - 8
+        return (q.astype(f) * d).astype(f).reshape(-1)
+    if ty == 6:                                                        # Q5_0: fifth bit of element e is bit e of the u32 at byte 2
+        b = raw[:n // 32 * 22].reshape(-1, 22)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qh = b[:, 2:6].copy().view(np.uint32).reshape(-1, 1)
+        hb = ((qh >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32)
+        q = np.concatenate([b[:, 6:] & 0xF, b[:, 6:] >> 4], axis=1).astype(np.int32) + 16 * hb - 16
+        return (q.astype(f) * d).astype(f).reshape(-1)
+    gxx, gs, g3x, kv = codebooks_more()
+    kvf = kv.astype(f)
+    if ty == 20:                                                       # IQ4_NL: d * level[nibble]
+        b = raw[:n // 32 * 18].reshape(-1, 18)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        q = np.concatenate([b[:, 2:] & 0xF, b[:, 2:] >> 4], axis=1)
+        return (d * kvf[q]).astype(f).reshape(-1)
+    if ty == 23:                                                       # IQ4_XS: 6-bit sub-block scale = 4 low bits (byte 4..7) | 2 high bits (u16 at 2)
+        b = raw[:n // 256 * 136].reshape(-1, 136)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        sh = b[:, 2:4].copy().view(np.uint16).astype(np.int32).reshape(-1, 1)
+        ib = np.arange(8)
+        lo4 = (b[:, 4:8][:, ib // 2].astype(np.int32) >> (4 * (ib % 2))) & 0xF
+        ls = lo4 | (((sh >> (2 * ib)) & 3) << 4)
+        dl = (d * (ls - 32).astype(f)).astype(f)                      # [nb, 8]
+        qs = b[:, 8:].reshape(-1, 8, 16)
+        q = np.concatenate([qs & 0xF, qs >> 4], axis=2)               # [nb, 8, 32]
+        return (kvf[q] * dl[:, :, None]).astype(f).reshape(-1)
+    if ty == 14:                                                       # Q6_K: (d * scale_i8) * (6-bit value - 32), 16 values per scale
+        b = raw[:n // 256 * 210].reshape(-1, 210)
+        nb = b.shape[0]
+        ql = b[:, 0:128].reshape(nb, 2, 2, 32).astype(np.int32)        # [half][which 32 bytes][l]
+        qh = b[:, 128:192].reshape(nb, 2, 32).astype(np.int32)
+        sc = b[:, 192:208].copy().view(np.int8).reshape(nb, 2, 4, 2).astype(f)   # [half][quarter][l // 16]
+        d = f16_to_f32(b[:, 208:210].copy()).reshape(nb, 1, 1, 1)
+        q = np.empty((nb, 2, 4, 32), dtype=np.int32)
+        for qd in range(4):
+            nib = (ql[:, :, qd & 1] & 0xF) if qd < 2 else (ql[:, :, qd & 1] >> 4)
+            q[:, :, qd] = (nib | (((qh >> (2 * qd)) & 3) << 4)) - 32
+        scale = (d * sc).astype(f)                                     # [nb, 2, 4, 2]
+        scale = np.repeat(scale, 16, axis=3)                           # per element l of the quarter
+        return (scale * q.astype(f)).astype(f).reshape(-1)
+    g3, g2, ks = codebooks()
+    if ty == 16:                                                       # IQ2_XXS: 8 bytes per 32 values: 4 grid indices, then 4x7 sign bits + 4 scale bits
+        b = raw[:n // 256 * 66].reshape(-1, 66)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qs = b[:, 2:66].reshape(-1, 8, 8)
+        a1 = qs[:, :, 4:8].copy().view(np.uint32).reshape(-1, 8)
+        db = ((d * (f(0.5) + (a1 >> 28).astype(f))).astype(f) * f(0.25)).astype(f)
+        grid = gxx[qs[:, :, 0:4]].astype(f)                             # [nb, 8, 4, 8]
+        sg = _signs(ks[(a1[:, :, None] >> (7 * np.arange(4, dtype=np.uint32))) & 127])
+        return ((db[:, :, None, None] * grid).astype(f) * sg).astype(f).reshape(-1)
+    if ty == 22:                                                       # IQ2_S: 10-bit grid index = byte | 2 bits of qh; one scale nibble per 16 values
+        b = raw[:n // 256 * 82].reshape(-1, 82)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qs = b[:, 2:34].reshape(-1, 8, 4).astype(np.uint32)
+        sg = b[:, 34:66].reshape(-1, 8, 4)
+        qh = b[:, 66:74].astype(np.uint32)
+        sc = b[:, 74:82]
+        hi2 = (qh[:, :, None] >> (2 * np.arange(4, dtype=np.uint32))) & 3
+        grid = gs[qs | (hi2 << 8)].astype(f)                            # [nb, 8, 4, 8]
+        lo = ((d * (f(0.5) + (sc & 0xF).astype(f))).astype(f) * f(0.25)).astype(f)
+        hi = ((d * (f(0.5) + (sc >> 4).astype(f))).astype(f) * f(0.25)).astype(f)
+        db = np.stack([lo, lo, hi, hi], axis=2)
+        return ((db[..., None] * grid).astype(f) * _signs(sg)).astype(f).reshape(-1)
+    if ty == 18:                                                       # IQ3_XXS: 64 grid indices (4 values each), then per 32 values a u32 of 4x7 sign bits + 4 scale bits
+        b = raw[:n // 256 * 98].reshape(-1, 98)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        qs = b[:, 2:66].reshape(-1, 8, 4, 2)
+        a = b[:, 66:98].copy().view(np.uint32).reshape(-1, 8)
+        db = ((d * (f(0.5) + (a >> 28).astype(f))).astype(f) * f(0.5)).astype(f)
+        grid = g3x[qs].astype(f).reshape(-1, 8, 4, 8)
+        sg = _signs(ks[(a[:, :, None] >> (7 * np.arange(4, dtype=np.uint32))) & 127])
+        return ((db[:, :, None, None] * grid).astype(f) * sg).astype(f).reshape(-1)
     raise ValueError(ty)
 
 

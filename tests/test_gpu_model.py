@@ -33,9 +33,10 @@ def pair(ctx, c, seed, max_ctx=512):
     return hw, gm, om
 
 
-@pytest.mark.parametrize("qtype,hc_type", [(synth.IQ3_S, synth.BF16), (synth.IQ3_S, synth.IQ3_S), (synth.Q4_K, synth.F32), (synth.IQ2_XS, synth.F16), (synth.Q8_0, synth.BF16)])
+@pytest.mark.parametrize("qtype,hc_type", [(synth.IQ3_S, synth.BF16), (synth.IQ3_S, synth.IQ3_S), (synth.Q4_K, synth.F32), (synth.IQ2_XS, synth.F16), (synth.Q8_0, synth.BF16),
+                                           (synth.IQ4_XS, synth.BF16), (synth.IQ2_S, synth.Q6_K), (synth.IQ3_XXS, synth.IQ4_XS), (synth.Q6_K, synth.F32), (synth.IQ2_XXS, synth.BF16)])
 def test_forward_logits_and_state_match_oracle(ctx, qtype, hc_type):
-    c = small_cfg(qtype=qtype, hc_type=hc_type, hc_lr=256 if hc_type == synth.IQ3_S else 64)
+    c = small_cfg(qtype=qtype, hc_type=hc_type, hc_lr=256 if synth.GEOM[hc_type][0] == 256 else 64)
     hw, gm, om = pair(ctx, c, 5)
     ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88], dtype=np.uint32)
     gs, os_ = gm.new_state(64), om.new_state()

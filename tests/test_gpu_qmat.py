@@ -9,7 +9,7 @@ from helpers import relerr
 from pyre_amd import lib, synth
 
 pytestmark = pytest.mark.gpu
-FMTS = [lib.Q8_0, lib.Q4_K, lib.IQ2_XS, lib.IQ3_S]
+FMTS = [lib.Q8_0, lib.Q4_K, lib.IQ2_XS, lib.IQ3_S, lib.Q4_0, lib.Q5_0, lib.Q6_K, lib.IQ2_XXS, lib.IQ3_XXS, lib.IQ4_NL, lib.IQ2_S, lib.IQ4_XS]
 ALL = FMTS + [lib.BF16, lib.F16, lib.F32]
 TOL = 1e-5
 
@@ -66,6 +66,31 @@ def test_known_answer_blocks_on_device(ctx):
     assert np.array_equal(m.to_f32(), np.ones((1, 256), np.float32))
     z2 = np_ref.pack_iq2xs(2.0, np.zeros(32, np.uint16), np.zeros(8, np.uint8))
     assert np.array_equal(lib.QMat(ctx, lib.IQ2_XS, 1, 256, z2).to_f32(), np.full((1, 256), 2.0, np.float32))
+
+
+def test_known_answer_blocks_of_the_recoded_types(ctx):
+    def blk(n, d, off=0):
+        b = np.zeros(n, np.uint8); b[off:off + 2] = np_ref.f16_bytes(d); return b
+    # zero payload: first codebook entry, scale bits 0, no signs -> every value equals d (see the oracle's known answers)
+    for ty, n in ((lib.IQ2_XXS, 66), (lib.IQ2_S, 82), (lib.IQ3_XXS, 98)):
+        assert np.array_equal(lib.QMat(ctx, ty, 1, 256, blk(n, 3.0)).to_f32(), np.full((1, 256), 3.0, np.float32)), ty
+    assert np.array_equal(lib.QMat(ctx, lib.IQ4_XS, 1, 256, blk(136, 0.5)).to_f32(), np.full((1, 256), -127 * (0.5 * -32), np.float32))
+    b = blk(210, 0.5, off=208); b[192:208] = 1
+    assert np.array_equal(lib.QMat(ctx, lib.Q6_K, 1, 256, b).to_f32(), np.full((1, 256), -16.0, np.float32))
+    kv = np.array(np_ref.IQ4NL_VALUES, np.float32)
+    b = np.concatenate([blk(18, 2.0), blk(18, 1.0)]); b[2:18] = np.arange(16) | ((15 - np.arange(16)) << 4); b[20:36] = 0x88
+    y = lib.QMat(ctx, lib.IQ4_NL, 1, 64, b).to_f32()[0]
+    assert np.array_equal(y[:16], 2.0 * kv) and np.array_equal(y[16:32], 2.0 * kv[::-1]) and np.array_equal(y[32:], np.full(32, kv[8]))
+
+
+@pytest.mark.parametrize("ty", FMTS)
+def test_device_generator_equals_host_generator(ctx, ty):
+    el, bs, _ = synth.GEOM[ty]
+    nb = 3000
+    dev = ctx.alloc(nb * bs)
+    ctx.synth_blocks(ty, nb, 777 + ty, dev_out=dev)
+    got = ctx.download(dev, (nb * bs,), np.uint8); ctx.free(dev)
+    assert np.array_equal(got, synth.blocks(ty, nb, 777 + ty))
 
 
 @pytest.mark.parametrize("ty", ALL)

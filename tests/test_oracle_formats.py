@@ -9,6 +9,8 @@ import orc
 from pyre_amd import synth
 
 FMTS = [orc.Q8_0, orc.Q4_K, orc.IQ2_XS, orc.IQ3_S]
+# the other block types real files of this architecture use (gguf_q.rs:74-78,82-89,114-125,130-140)
+FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS]
 
 
 def bits(a):
@@ -20,6 +22,7 @@ def test_codebook_digests_match_reference_tables():
         import os
         p = os.path.join(np_ref._ROOT, hdr)
         assert np_ref.codebook_digests(p) == (np_ref.IQ3S_SHA256, np_ref.IQ2XS_SHA256, np_ref.KSIGNS_SHA256)
+        assert np_ref.codebook_digests_more(p) == (np_ref.IQ2XXS_SHA256, np_ref.IQ2S_SHA256, np_ref.IQ3XXS_SHA256, np_ref.IQ4NL_VALUES)
 
 
 def test_oracle_expansion_equals_numpy_expansion():
@@ -99,7 +102,88 @@ def test_bf16_f16_f32_passthrough():
     assert np.array_equal(orc.dequant(orc.BF16, bf.view(np.uint8), 4), (bf.astype(np.uint32) << 16).view(np.float32))
 
 
-@pytest.mark.parametrize("ty", FMTS)
+def _blk(n, d, off=0):
+    b = np.zeros(n, np.uint8); b[off:off + 2] = np_ref.f16_bytes(d); return b
+
+
+def test_q4_0_and_q5_0_known_answers():
+    b = _blk(18, 0.5); b[2:] = np.arange(16) | ((15 - np.arange(16)) << 4)       # low nibble j, high nibble 15 - j
+    y = orc.dequant(orc.Q4_0, b, 32)
+    assert np.array_equal(y[:16], (np.arange(16) - 8) * 0.5) and np.array_equal(y[16:], (7 - np.arange(16)) * 0.5)
+    b = _blk(22, 0.25); b[2:6] = np.array([(1 << 3) | (1 << 20)], np.uint32).view(np.uint8)   # fifth bit of elements 3 and 20
+    b[6:] = 0x21                                                                      # low nibble 1, high nibble 2
+    y = orc.dequant(orc.Q5_0, b, 32)
+    exp = np.concatenate([np.full(16, 1 - 16.0), np.full(16, 2 - 16.0)]); exp[3] += 16; exp[20] += 16
+    assert np.array_equal(y, (exp * 0.25).astype(np.float32))
+
+
+def test_iq4_nl_and_iq4_xs_known_answers():
+    kv = np.array(np_ref.IQ4NL_VALUES, np.float32)
+    b = _blk(18, 2.0); b[2:] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    y = orc.dequant(orc.IQ4_NL, b, 32)
+    assert np.array_equal(y[:16], 2.0 * kv) and np.array_equal(y[16:], 2.0 * kv[::-1])
+    # IQ4_XS: zero payload -> 6-bit scale 0 -> d * (0 - 32), level 0 = -127
+    assert np.array_equal(orc.dequant(orc.IQ4_XS, _blk(136, 0.5), 256), np.full(256, -127 * (0.5 * -32), np.float32))
+    b = _blk(136, 1.0)
+    b[2:4] = np.array([(2 << (2 * 5)) | (3 << (2 * 6))], np.uint16).view(np.uint8)   # high bits: sub-block 5 -> 2, sub-block 6 -> 3
+    b[4 + 2] = 0x9 << 4                                                               # low bits of sub-block 5 (high nibble of byte 2) = 9
+    b[4 + 3] = 0x4                                                                    # low bits of sub-block 6 = 4
+    b[8 + 16 * 5:8 + 16 * 6] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    y = orc.dequant(orc.IQ4_XS, b, 256).reshape(8, 32)
+    assert np.array_equal(y[5, :16], kv * float((9 | (2 << 4)) - 32)) and np.array_equal(y[5, 16:], kv[::-1] * float(41 - 32))
+    assert np.array_equal(y[6], np.full(32, -127.0 * ((4 | (3 << 4)) - 32), np.float32))
+    assert np.array_equal(y[0], np.full(32, -127.0 * -32, np.float32))
+
+
+def test_q6_k_known_answers():
+    b = _blk(210, 0.5, off=208); b[192:208] = 1
+    assert np.array_equal(orc.dequant(orc.Q6_K, b, 256), np.full(256, 0.5 * 1 * -32, np.float32))     # all six-bit values 0 -> -32
+    b = _blk(210, 1.0, off=208)
+    b[192:208] = np.array([1, 2, 3, 4, 5, 6, 7, 8, -1, -2, -3, -4, -5, -6, -7, -8], np.int8).view(np.uint8)
+    # second half (elements 128..255): element 128 + 64 + 17 is quarter 2, l = 17 -> high nibble of ql[64 + 17], bits 4..5 of qh[32 + 17],
+    # scale index 8 + 2*2 + 17 // 16 = 13 (-6)
+    b[64 + 17] = 0xB << 4; b[128 + 32 + 17] = 0x2 << 4
+    y = orc.dequant(orc.Q6_K, b, 256)
+    assert y[128 + 64 + 17] == -6.0 * ((0xB | (2 << 4)) - 32)
+    # element 33 is quarter 1, l = 1 -> low nibble of ql[32 + 1], bits 2..3 of qh[1], scale index 2
+    b[32 + 1] = 0x7; b[128 + 1] = 0x3 << 2
+    y = orc.dequant(orc.Q6_K, b, 256)
+    assert y[33] == 3.0 * ((7 | (3 << 4)) - 32)
+    assert y[0] == 1.0 * -32 and y[16] == 2.0 * -32 and y[255] == -8.0 * -32
+
+
+def test_iq2_xxs_iq2_s_iq3_xxs_known_answers():
+    gxx, gs, g3x, _ = np_ref.codebooks_more()
+    _, _, ks = np_ref.codebooks()
+    assert np.array_equal(gxx[0], [8] * 8) and np.array_equal(gs[0], [8] * 8) and np.array_equal(g3x[0], [4] * 4)
+    assert set(np.unique(gxx)) == {8, 25, 43} and set(np.unique(gs)) == {8, 25, 43} and set(np.unique(g3x)) == {4, 12, 20, 28, 36, 44, 52, 62}
+    # zero payload: entry 0, scale bits 0, no signs -> d*(0.5)*0.25*8 = d, and d*(0.5)*0.5*4 = d
+    for ty, n in ((orc.IQ2_XXS, 66), (orc.IQ2_S, 82), (orc.IQ3_XXS, 98)):
+        assert np.array_equal(orc.dequant(ty, _blk(n, 3.0), 256), np.full(256, 3.0, np.float32)), ty
+    # IQ2_XXS: sub-block 3: grid bytes (10, 0, 200, 0), sign index 9 for group 2, scale bits 6
+    b = _blk(66, 1.0); b[2 + 8 * 3 + 0] = 10; b[2 + 8 * 3 + 2] = 200
+    b[2 + 8 * 3 + 4:2 + 8 * 3 + 8] = np.array([(9 << 14) | (6 << 28)], np.uint32).view(np.uint8)
+    y = orc.dequant(orc.IQ2_XXS, b, 256).reshape(8, 4, 8)
+    db = np.float32(6.5 * 0.25)
+    sgn = np.where((ks[9] >> np.arange(8)) & 1, -1.0, 1.0).astype(np.float32)
+    assert np.array_equal(y[3, 0], db * gxx[10].astype(np.float32)) and np.array_equal(y[3, 2], db * gxx[200].astype(np.float32) * sgn)
+    assert np.array_equal(y[3, 1], np.full(8, db * 8)) and np.array_equal(y[2], np.full((4, 8), 1.0, np.float32))
+    # IQ2_S: sub-block 6: index byte 1 = 0x55 with high bits 2 (qh bits 2..3) -> entry 0x255; sign byte for group 1; scale nibbles 3 / 12
+    b = _blk(82, 1.0); b[2 + 4 * 6 + 1] = 0x55; b[66 + 6] = 2 << 2; b[34 + 4 * 6 + 1] = 0b10000001; b[74 + 6] = 3 | (12 << 4)
+    y = orc.dequant(orc.IQ2_S, b, 256).reshape(8, 4, 8)
+    lo, hi = np.float32(3.5 * 0.25), np.float32(12.5 * 0.25)
+    exp1 = lo * gs[0x255].astype(np.float32); exp1[0] *= -1; exp1[7] *= -1
+    assert np.array_equal(y[6, 1], exp1) and np.array_equal(y[6, 0], np.full(8, lo * 8)) and np.array_equal(y[6, 2], np.full(8, hi * 8))
+    # IQ3_XXS: sub-block 2: index bytes 4, 5 (group 2) = 100, 255; sign index 3 for group 2; scale bits 15
+    b = _blk(98, 1.0); b[2 + 8 * 2 + 4] = 100; b[2 + 8 * 2 + 5] = 255
+    b[66 + 4 * 2:66 + 4 * 2 + 4] = np.array([(3 << 14) | (15 << 28)], np.uint32).view(np.uint8)
+    y = orc.dequant(orc.IQ3_XXS, b, 256).reshape(8, 4, 8)
+    db = np.float32(15.5 * 0.5)
+    exp = db * np.concatenate([g3x[100], g3x[255]]).astype(np.float32); exp[0] *= -1; exp[1] *= -1
+    assert np.array_equal(y[2, 2], exp) and np.array_equal(y[2, 0], np.full(8, db * 4))
+
+
+@pytest.mark.parametrize("ty", FMTS + FMTS_MORE)
 def test_oracle_dequant_bit_equal_to_numpy_on_random_blocks(ty):
     el, bs, _ = synth.GEOM[ty]
     nb = 4096
@@ -129,7 +213,7 @@ def test_dot_small_integers_exact_and_tail():
         assert orc.dot(a, b) == float(np.dot(a.astype(np.float64), b.astype(np.float64)))
 
 
-@pytest.mark.parametrize("ty", FMTS + [orc.BF16])
+@pytest.mark.parametrize("ty", FMTS + FMTS_MORE + [orc.BF16])
 def test_matmul_index_contract_and_accuracy(ty):
     rows, cols, t = 48, 512, 3
     raw = synth.matrix(ty, rows, cols, seed=33) if ty != orc.BF16 else synth.bf16_normal(rows, cols, 3, 0.02)
