@@ -83,7 +83,10 @@ def bench_gemv(args):
     from pyre_amd import lib, synth
     ev = HipEvents()
     ctx = lib.Context(0)
-    ty, rows, cols = lib.IQ3_S, 151936, 2048
+    names = {"iq3_s": lib.IQ3_S, "iq2_xs": lib.IQ2_XS, "q4_k": lib.Q4_K, "q8_0": lib.Q8_0, "q4_0": lib.Q4_0, "q5_0": lib.Q5_0, "q6_k": lib.Q6_K, "iq2_xxs": lib.IQ2_XXS,
+             "iq2_s": lib.IQ2_S, "iq3_xxs": lib.IQ3_XXS, "iq4_nl": lib.IQ4_NL, "iq4_xs": lib.IQ4_XS}
+    ty, rows, cols = names[args.fmt], 151936, 2048
+    FN = args.fmt.upper()
     el, bs, _ = synth.GEOM[ty]
     nb = rows * cols // el
     nbuf = 5                                    # 5 x 133.7 MB = 668 MB > 512 MB
@@ -121,18 +124,18 @@ def bench_gemv(args):
     traffic = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary, when present
     try:
         for line in open(os.path.join(ROOT, "profiles", "gemv_iq3s_vocab_head_kernel_stats.txt")):
-            if t == 1 and line.startswith("traffic_bytes_per_launch:"):
+            if t == 1 and ty == lib.IQ3_S and line.startswith("traffic_bytes_per_launch:"):
                 traffic = int(line.split(":")[1])
     except OSError:
         pass
     gbs = alg_bytes / (per * 1e-3) / 1e9
     out = {
-        "metric": "IQ3_S dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=%d%s)" % (t, ", matrix cores" if args.mfma else ""), "value": round(gbs, 1), "unit": "GB/s",
+        "metric": "%s dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=%d%s)" % (FN, t, ", matrix cores" if args.mfma else ""), "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[1]: IQ3_S GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
+        "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "k_gemm_mfma_iq3s (+ k_xsplit)" if args.mfma else "k_gemv<IQ3_S,%d>" % t, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(per * 1e3, 3)},
+                     "kernel": "k_gemm_mfma_iq3s (+ k_xsplit)" if args.mfma else "k_gemv<%s,%d>" % (FN, t), "device_bytes_per_launch": mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(per * 1e3, 3)},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemv(ty, rows, cols, 9000)
@@ -298,6 +301,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
+    ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs)")
     ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MiB", help="gemv workload: also run 4 plain device copies of this size (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()

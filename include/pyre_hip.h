@@ -64,6 +64,9 @@ size_t pyre_qmat_rows(const pyre_qmat* m);
 size_t pyre_qmat_cols(const pyre_qmat* m);
 /* GGUF bytes of the matrix (rows * row_bytes): the algorithmic weight bytes of one GEMV. */
 size_t pyre_qmat_gguf_bytes(const pyre_qmat* m);
+/* Bytes the matrix occupies in device memory after the load-time re-layout (what one GEMV actually streams); the
+ * reference's counterpart is the size of the repacked Burn tensor (repack_to_burn, src/model/qn_gpu.rs:54). */
+size_t pyre_qmat_device_bytes(const pyre_qmat* m);
 /* QMat::to_f32 (gguf_q.rs:212): all rows*cols values, bit-exact with gguf_q::dequant (gguf_q.rs:67-166). */
 int    pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host);
 int    pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev);

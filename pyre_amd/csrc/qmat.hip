@@ -350,6 +350,7 @@ void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx
 size_t pyre_qmat_rows(const pyre_qmat* m) { return m ? m->rows : 0; }
 size_t pyre_qmat_cols(const pyre_qmat* m) { return m ? m->cols : 0; }
 size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; }
+size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes : 0; }
 
 int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
   if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");

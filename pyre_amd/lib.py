@@ -39,6 +39,7 @@ def _declare(L):
         "pyre_qmat_rows": (sz, [vp]),
         "pyre_qmat_cols": (sz, [vp]),
         "pyre_qmat_gguf_bytes": (sz, [vp]),
+        "pyre_qmat_device_bytes": (sz, [vp]),
         "pyre_qmat_dequant": (i32, [vp, vp, vp]),
         "pyre_qmat_dequant_dev": (i32, [vp, vp, vp]),
         "pyre_qmat_row": (i32, [vp, vp, sz, vp]),
@@ -221,6 +222,10 @@ class QMat:
     @property
     def gguf_bytes(self):
         return self.ctx.L.pyre_qmat_gguf_bytes(self.h)
+
+    @property
+    def dev_bytes(self):
+        return self.ctx.L.pyre_qmat_device_bytes(self.h)
 
     def to_f32(self):
         out = np.empty((self.rows, self.cols), dtype=np.float32)
