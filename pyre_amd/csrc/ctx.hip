@@ -63,10 +63,11 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
     uint32_t v = 0; for (int j = 0; j < 4; ++j) v |= (uint32_t)(2 * ((kIq3sCode[i] >> (3 * j)) & 7) + 1) << (8 * j); g3[i] = v;
     uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(kIq2xsCode[i] >> (2 * j)) & 3] << (8 * j); g2[i] = w;
   }
-  std::vector<uint16_t> cb(1536);          // compact codes as they are: [iq2xxs 256 | iq2s 1024 | iq3xxs 256], used once per matrix by the load-time re-coding
+  std::vector<uint16_t> cb(2048);          // compact codes as they are: [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512], used once per matrix by the load-time re-coding
   for (int i = 0; i < 256; ++i) { cb[i] = kIq2xxsCode[i]; cb[1280 + i] = kIq3xxsCode[i]; }
   for (int i = 0; i < 1024; ++i) cb[256 + i] = kIq2sCode[i];
-  if ((e = hipMalloc((void**)&ctx->d_cb, 1536 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 1536 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
+  for (int i = 0; i < 512; ++i) cb[1536 + i] = kIq2xsCode[i];
+  if ((e = hipMalloc((void**)&ctx->d_cb, 2048 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 2048 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
       (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->fuse_ctl, 1024)) != hipSuccess || (e = hipMemset(ctx->fuse_ctl, 0, 1024)) != hipSuccess) {

@@ -18,7 +18,7 @@ __host__ __device__ inline FmtGeom fmt_geom(int fmt) {
     case FMT_BF16:   return {8, 0, 0, 0, 0};
     case FMT_Q8_0:   return {4, 4, 0, 0, 0};     // p1: the two f16 scales of the unit's two blocks
     case FMT_Q4_K:   return {2, 0, 0, 0, 16};    // pb: d, dmin, scales[12]
-    case FMT_IQ2_XS: return {1, 2, 0, 0, 2};     // p1: two scale bytes; pb: d
+    case FMT_IQ2_XS: return {1, 2, 8, 0, 2};     // IQ2_XS / IQ2_XXS / IQ2_S, re-coded at load: p0: 64 two-bit magnitude codes; p1: four scale nibbles; p2: 64 sign bits; pb: d
     case FMT_C4:     return {2, 16, 0, 0, 0};    // p0: 64 four-bit codes; p1: four f32 scales
     case FMT_C8:     return {4, 16, 0, 0, 0};    // p0: 64 int8 values; p1: four f32 scales
     default:         return {2, 0, 0, 1, 2};     // IQ3_S, re-coded at load: p0: 64 four-bit codes, p3: scale byte; pb: d
@@ -39,20 +39,20 @@ __host__ __device__ inline bool ggml_geom(uint32_t ty, int* el, int* bytes) {
 inline int fmt_from_ggml(uint32_t ty) {
   switch (ty) { case PYRE_F32: return FMT_F32; case PYRE_F16: return FMT_F16; case PYRE_BF16: return FMT_BF16; case PYRE_Q8_0: return FMT_Q8_0;
     case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S;
-    case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ2_XXS: case PYRE_IQ2_S: case PYRE_IQ3_XXS: return FMT_C4;
+    case PYRE_IQ2_XXS: case PYRE_IQ2_S: return FMT_IQ2_XS;
+    case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ3_XXS: return FMT_C4;
     case PYRE_Q5_0: case PYRE_Q6_K: return FMT_C8; }
   return -1;
 }
 // The C4 value table of a GGUF type: entry c (byte c%4 of word c/4) holds value + bias, 0..255.
-//   Q4_0: c - 8.  IQ4_NL, IQ4_XS: the sixteen non-linear levels (kIq4nlValues).  The i-quants code a value as
-//   (negative << 3) | magnitude index: magnitudes {8, 25, 43} (IQ2_XXS, IQ2_S), {4, 12, .., 52, 62} (IQ3_XXS).
+//   Q4_0: c - 8.  IQ4_NL, IQ4_XS: the sixteen non-linear levels (kIq4nlValues).  IQ3_XXS codes a value as
+//   (negative << 3) | magnitude index, magnitudes {4, 12, .., 52, 62}.
 inline void c4_table(uint32_t ty, uint32_t lut[4], int* bias) {
   int v[16] = {0}; int b = 0;
-  static const int tri[3] = {8, 25, 43}; static const int lv3[8] = {4, 12, 20, 28, 36, 44, 52, 62};
+  static const int lv3[8] = {4, 12, 20, 28, 36, 44, 52, 62};
   switch (ty) {
     case PYRE_Q4_0: for (int c = 0; c < 16; ++c) v[c] = c - 8; b = 8; break;
     case PYRE_IQ4_NL: case PYRE_IQ4_XS: for (int c = 0; c < 16; ++c) v[c] = kIq4nlValues[c]; b = 127; break;
-    case PYRE_IQ2_XXS: case PYRE_IQ2_S: for (int c = 0; c < 3; ++c) { v[c] = tri[c]; v[8 + c] = -tri[c]; } b = 43; break;
     case PYRE_IQ3_XXS: for (int c = 0; c < 8; ++c) { v[c] = lv3[c]; v[8 + c] = -lv3[c]; } b = 62; break;
     default: break;
   }
@@ -86,6 +86,17 @@ __device__ __forceinline__ void scale_min_k4(int j, uint32_t a, uint32_t b, uint
 // decodes without the codebook: w = 2c - 15.
 __host__ __device__ inline uint32_t iq3s_code(uint32_t grid_byte, uint32_t neg) { int w = neg ? -(int)grid_byte : (int)grid_byte; return (uint32_t)((w + 15) >> 1); }
 
+// The 2-bit i-quants (IQ2_XS, IQ2_XXS, IQ2_S) hold sign * magnitude with magnitude in {8, 25, 43} and one scale nibble
+// per 16 values (IQ2_XXS: per 32, stored twice).  At load the codebook and sign-table lookups are resolved once; per
+// unit the device keeps, for value e = 4r + b (round r, byte b) of 16-value group g:
+//   magnitude index (0, 1, 2) at bits 8b + 2r of dword g of the unit's 16-byte chunk,
+//   sign at bit 8b + r + 4*(g & 1) of dword g / 2 of the unit's 8 sign bytes,
+// so that `round r` of a group yields four 3-bit codes (sign << 2 | index), one per byte, with two shifts and two
+// masks, and one v_perm_b32 turns them into the four biased values magnitude * sign + 43.
+__device__ __forceinline__ uint32_t iq2_mag(uint32_t idx) { return idx == 0 ? 8u : (idx == 1 ? 25u : 43u); }
+#define PYRE_IQ2_TLO 0x00564433u      // codes 0..3: 43 + {8, 25, 43}, unused
+#define PYRE_IQ2_THI 0x00001223u      // codes 4..7: 43 - {8, 25, 43}, unused
+
 // ---- bit-exact decode of one unit (64 consecutive values of one row) -----------------------------------------------
 // Same operations in the same order as gguf_q::dequant; compiled with -ffp-contract=off so nothing is fused.
 template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const uint64_t* g2, int tile, int ku, int lane, float* y) {
@@ -112,18 +123,15 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
       uint4 v = ld_vec<2>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
       for (int k = 0; k < 16; ++k) { uint32_t b = (w[k >> 2] >> (8 * (k & 3))) & 0xFF; y[16 * c + k] = d1 * (float)(b & 0xF) - M1; y[32 + 16 * c + k] = d2 * (float)(b >> 4) - M2; }
     }
-  } else if constexpr (FMT == FMT_IQ2_XS) {        // gguf_q.rs:126-129
+  } else if constexpr (FMT == FMT_IQ2_XS) {        // gguf_q.rs:122-135 from the re-coded planes: (db * magnitude) * sign
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
     uint32_t sc = ld_small<uint16_t>(m.p1, m, tile, ku, lane);
-    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
-    for (int ib = 0; ib < 2; ++ib) {
-      uint32_t s = (sc >> (8 * ib)) & 0xFF;
-      float db0 = d * (0.5f + (float)(s & 0xF)) * 0.25f, db1 = d * (0.5f + (float)(s >> 4)) * 0.25f;
-      for (int l = 0; l < 4; ++l) {
-        uint32_t q = (w[2 * ib + (l >> 1)] >> (16 * (l & 1))) & 0xFFFF;
-        uint64_t g = g2[q & 511]; uint32_t sg = ksigns(q >> 9); float db = l < 2 ? db0 : db1;
-        for (int jj = 0; jj < 8; ++jj) y[32 * ib + 8 * l + jj] = flip(db * (float)(uint32_t)((g >> (8 * jj)) & 0xFF), (sg >> jj) & 1);
-      }
+    uint2 sg = ld_small<uint2>(m.p2, m, tile, ku, lane); uint32_t S[2] = {sg.x, sg.y};
+    uint4 v = ld_vec<1>(m, tile, ku, 0, lane); uint32_t M[4] = {v.x, v.y, v.z, v.w};
+    for (int g = 0; g < 4; ++g) {
+      float db = d * (0.5f + (float)((sc >> (4 * g)) & 0xF)) * 0.25f;
+      for (int e = 0; e < 16; ++e) { int r = e >> 2, b = e & 3; uint32_t idx = (M[g] >> (8 * b + 2 * r)) & 3, neg = (S[g >> 1] >> (8 * b + r + 4 * (g & 1))) & 1;
+        y[16 * g + e] = flip(db * (float)iq2_mag(idx), neg); }
     }
   } else if constexpr (FMT == FMT_C4) {            // scale * table[code]: the last multiply of gguf_q.rs:75,83,88,125,135,140
     uint4 sq = ld_small<uint4>(m.p1, m, tile, ku, lane); float sc[4] = {__uint_as_float(sq.x), __uint_as_float(sq.y), __uint_as_float(sq.z), __uint_as_float(sq.w)};
@@ -160,7 +168,7 @@ template <int FMT> __device__ __forceinline__ UnitRaw<FMT> unit_load(const QMatD
   if constexpr (FMT == FMT_Q8_0) r.s0 = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
   if constexpr (FMT == FMT_Q4_K) r.hb = ld_block<uint4>(m, tile, ku, lane);
   if constexpr (FMT == FMT_C4 || FMT == FMT_C8) r.hb = ld_small<uint4>(m.p1, m, tile, ku, lane);
-  if constexpr (FMT == FMT_IQ2_XS) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint16_t>(m.p1, m, tile, ku, lane); }
+  if constexpr (FMT == FMT_IQ2_XS) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint16_t>(m.p1, m, tile, ku, lane); uint2 sg = ld_small<uint2>(m.p2, m, tile, ku, lane); r.hb.x = sg.x; r.hb.y = sg.y; }
   if constexpr (FMT == FMT_IQ3_S) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint8_t>(m.p3, m, tile, ku, lane); }
   return r;
 }
@@ -228,35 +236,37 @@ _Pragma("unroll")
         for (int t = 0; t < T; ++t) { acc[t] = fmaf(lo, xs[t * xstride + 16 * c + k], acc[t]); acc[t] = fmaf(hi, xs[t * xstride + 32 + 16 * c + k], acc[t]); }
       }
     }
-  } else if constexpr (FMT == FMT_IQ2_XS) {
+  } else if constexpr (FMT == FMT_IQ2_XS) {   // biased value = sign * magnitude + 43 by one byte permute per four values; per group  db * (sum biased x - 43 sum x)
     float d = h2f_bits(r.s0);
     uint32_t sc = r.s1;
-    uint4 v = r.v[0]; uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint4 v = r.v[0]; uint32_t M[4] = {v.x, v.y, v.z, v.w}; uint32_t S[2] = {r.hb.x, r.hb.y};
+    float sx[T][4];
 #pragma unroll
-    for (int ib = 0; ib < 2; ++ib) {
-      uint32_t s = (sc >> (8 * ib)) & 0xFF;
+    for (int t = 0; t < T; ++t) {
+      float xv = xs[t * xstride + lane];
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        float part[T];
+      for (int o = 8; o > 0; o >>= 1) xv += __shfl_xor(xv, o);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) sx[t][g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), 16 * g));
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float part[T];
 _Pragma("unroll")
       for (int t = 0; t < T; ++t) part[t] = 0.0f;
 #pragma unroll
-        for (int l2 = 0; l2 < 2; ++l2) {
-          int l = 2 * hf + l2;
-          uint32_t q = (w[2 * ib + (l >> 1)] >> (16 * (l & 1))) & 0xFFFF;
-          uint2 g = lds2[q & 511]; uint32_t sg = ksigns(q >> 9);
+      for (int rr = 0; rr < 4; ++rr) {
+        const int k = rr + 4 * (g & 1);
+        uint32_t idx4 = (M[g] >> (2 * rr)) & 0x03030303u, sgn = k >= 2 ? (S[g >> 1] >> (k - 2)) : (S[g >> 1] << (2 - k));
+        uint32_t bv = __builtin_amdgcn_perm(PYRE_IQ2_THI, PYRE_IQ2_TLO, (sgn & 0x04040404u) | idx4);
 #pragma unroll
-          for (int jj = 0; jj < 8; ++jj) {
-            uint32_t gw = jj < 4 ? g.x : g.y;
-            float f = __uint_as_float(__float_as_uint((float)((gw >> (8 * (jj & 3))) & 0xFF)) | ((sg << (31 - jj)) & 0x80000000u));
+        for (int b = 0; b < 4; ++b) { float f = (float)((bv >> (8 * b)) & 0xFF);
 #pragma unroll
-            for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 32 * ib + 8 * l + jj], part[t]);
-          }
-        }
-        float db = d * (0.5f + (float)((s >> (4 * hf)) & 0xF)) * 0.25f;
-#pragma unroll
-        for (int t = 0; t < T; ++t) acc[t] = fmaf(db, part[t], acc[t]);
+          for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 16 * g + 4 * rr + b], part[t]); }
       }
+      float db = d * (0.5f + (float)((sc >> (4 * g)) & 0xF)) * 0.25f;
+#pragma unroll
+      for (int t = 0; t < T; ++t) acc[t] = fmaf(db, fmaf(-43.0f, sx[t][g], part[t]), acc[t]);
     }
   } else if constexpr (FMT == FMT_C4) {   // value = table[c] - bias: per 16-value group  scale * (sum table[c] x - bias sum x)
     uint4 v0 = r.v[0], v1 = r.v[1];

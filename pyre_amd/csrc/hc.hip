@@ -28,14 +28,13 @@ __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in
 template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
     const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
-  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, nw = nthr >> 6, tid = threadIdx.x, L = nw * upw * 64;
   float* xs = sm;                         // [T][L]
   float* red = sm + (size_t)T * L;        // [nw][T][64]
   float* wsum = red + (size_t)nw * T * 64;   // [nw][T]
   const int tile = blockIdx.x, ks = blockIdx.y;
-  if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
   UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);     // in flight across both barriers
@@ -92,12 +91,11 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 // the sum of its waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc, s ascending from zero (:1380).
 template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xn, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2) {
-  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6;
   float* lo = sm;                         // [T][lr]
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
-  if constexpr (FMT == FMT_IQ2_XS) for (int i = tid; i < 512; i += nthr) lds2[i] = g2[i];
   const int n_o = lr + hc;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave / U, ku = wave - s * U;

@@ -61,14 +61,13 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 template <int FMT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2) {
-  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   __shared__ float red[2][NW][64];
   __shared__ RouteLds rl;
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
   const int nrows = shared ? m.sf : m.ff;
   if ((int)blockIdx.x * 64 >= nrows) return;
-  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const float* xs = x + (size_t)ti * m.d;
   int expert = 0;
@@ -113,11 +112,10 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
 template <int FMT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
                                                      const uint2* __restrict__ g2) {
-  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   __shared__ float red[NW][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
-  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const QMatDev& D = shared ? m.sh_down : m.down_e;
   const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.d >> 6)) + blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;

@@ -29,14 +29,35 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
       put_vec(0, b + 16 + 32 * j); put_vec(1, b + 32 + 32 * j);
       if (j == 0) { uint8_t* d = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 16; for (int i = 0; i < 16; ++i) d[i] = live ? b[i] : 0; }
     } break;
-    case FMT_IQ2_XS: {
-      const uint8_t* b = row + (size_t)(ku >> 2) * 74; int j = ku & 3;
-      put_vec(0, b + 2 + 16 * j);
-      uint8_t* d = p1 + e * 2; d[0] = live ? b[66 + 2 * j] : 0; d[1] = live ? b[67 + 2 * j] : 0;
-      if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = live ? b[0] : 0; dd[1] = live ? b[1] : 0; }
+    case FMT_IQ2_XS: {   // IQ2_XS / IQ2_XXS / IQ2_S (gguf_q.rs:122-135): grid and sign lookups resolved here, once; cb holds 2-bit magnitude indices per grid byte
+      uint32_t M[4] = {0, 0, 0, 0}, S[2] = {0, 0}; uint32_t scb = 0; int j = ku & 3;
+      auto ks = [](uint32_t i) { return i | ((__popc(i) & 1u) << 7); };
+      auto put = [&](int ev, uint32_t idx, uint32_t neg) { int gq = ev >> 4, e16 = ev & 15, r = e16 >> 2, bb = e16 & 3; M[gq] |= (idx & 3) << (8 * bb + 2 * r); S[gq >> 1] |= (neg & 1) << (8 * bb + r + 4 * (gq & 1)); };
+      const uint8_t* b = row; uint32_t dbits = 0;
+      if (live) {
+        if (m.ty == PYRE_IQ2_XS) {
+          b = row + (size_t)(ku >> 2) * 74; dbits = b[0] | (b[1] << 8); scb = b[66 + 2 * j] | (b[67 + 2 * j] << 8);
+          for (int l = 0; l < 8; ++l) { uint32_t q = b[2 + 16 * j + 2 * l] | (b[3 + 16 * j + 2 * l] << 8), gcode = cb[1536 + (q & 511)], sg = ks(q >> 9);
+            for (int jj = 0; jj < 8; ++jj) put(8 * l + jj, (gcode >> (2 * jj)) & 3, (sg >> jj) & 1); }
+        } else if (m.ty == PYRE_IQ2_XXS) {
+          b = row + (size_t)(ku >> 2) * 66; dbits = b[0] | (b[1] << 8);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * j + c; const uint8_t* a0 = b + 2 + 8 * ib; uint32_t a1 = a0[4] | (a0[5] << 8) | (a0[6] << 16) | ((uint32_t)a0[7] << 24), nib = a1 >> 28;
+            scb |= (nib | (nib << 4)) << (8 * c);
+            for (int l = 0; l < 4; ++l) { uint32_t gcode = cb[a0[l]], sg = ks((a1 >> (7 * l)) & 127); for (int jj = 0; jj < 8; ++jj) put(32 * c + 8 * l + jj, (gcode >> (2 * jj)) & 3, (sg >> jj) & 1); } }
+        } else {           // IQ2_S
+          b = row + (size_t)(ku >> 2) * 82; dbits = b[0] | (b[1] << 8);
+          for (int c = 0; c < 2; ++c) { int ib = 2 * j + c; uint32_t qh = b[66 + ib]; scb |= (uint32_t)b[74 + ib] << (8 * c);
+            for (int l = 0; l < 4; ++l) { uint32_t gcode = cb[256 + (b[2 + 4 * ib + l] | ((qh << (8 - 2 * l)) & 0x300))], sg = b[34 + 4 * ib + l];
+              for (int jj = 0; jj < 8; ++jj) put(32 * c + 8 * l + jj, (gcode >> (2 * jj)) & 3, (sg >> jj) & 1); } }
+        }
+      }
+      uint32_t* dst = (uint32_t*)(v + (size_t)lane * 16); for (int i = 0; i < 4; ++i) dst[i] = M[i];
+      uint8_t* d1 = p1 + e * 2; d1[0] = (uint8_t)(scb & 0xFF); d1[1] = (uint8_t)(scb >> 8);
+      uint32_t* d2 = (uint32_t*)(p2 + e * 8); d2[0] = S[0]; d2[1] = S[1];
+      if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = (uint8_t)(dbits & 0xFF); dd[1] = (uint8_t)(dbits >> 8); }
     } break;
     case FMT_C4: case FMT_C8: {
-      // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256]; code(e) and scale(e / 16) of the unit's 64 values e
+      // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512]; code(e) and scale(e / 16) of the unit's 64 values e
       uint32_t words[16]; float sc[4];
       for (int i = 0; i < 16; ++i) words[i] = 0;
       for (int i = 0; i < 4; ++i) sc[i] = 0.0f;
@@ -66,19 +87,6 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
             for (int l = 0; l < 32; ++l) { uint32_t qlb = b[64 * n + l + ((qd & 1) ? 32 : 0)], nib = qd < 2 ? (qlb & 0xF) : (qlb >> 4), hi2 = (b[128 + 32 * n + l] >> (2 * qd)) & 3;
               put8b(32 * c + l, (int)(nib | (hi2 << 4)) - 32); }
             for (int g = 0; g < 2; ++g) sc[2 * c + g] = d * (float)(int)(int8_t)b[192 + 8 * n + 2 * qd + g]; }
-        } break;
-        case PYRE_IQ2_XXS: {                                           // gguf_q.rs:122-125
-          const uint8_t* b = row + (size_t)(ku >> 2) * 66; float d = h2(b);
-          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; const uint8_t* a0 = b + 2 + 8 * ib; uint32_t a1 = a0[4] | (a0[5] << 8) | (a0[6] << 16) | ((uint32_t)a0[7] << 24);
-            sc[2 * c] = sc[2 * c + 1] = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
-            for (int l = 0; l < 4; ++l) { uint32_t g = cb[a0[l]], sg = ks((a1 >> (7 * l)) & 127); for (int j = 0; j < 8; ++j) put4(32 * c + 8 * l + j, ((g >> (2 * j)) & 3) | (((sg >> j) & 1) << 3)); } }
-        } break;
-        case PYRE_IQ2_S: {                                             // gguf_q.rs:130-135
-          const uint8_t* b = row + (size_t)(ku >> 2) * 82; float d = h2(b);
-          for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; uint32_t s = b[74 + ib], qh = b[66 + ib];
-            sc[2 * c] = d * (0.5f + (float)(s & 0xF)) * 0.25f; sc[2 * c + 1] = d * (0.5f + (float)(s >> 4)) * 0.25f;
-            for (int l = 0; l < 4; ++l) { uint32_t g = cb[256 + (b[2 + 4 * ib + l] | ((qh << (8 - 2 * l)) & 0x300))], sg = b[34 + 4 * ib + l];
-              for (int j = 0; j < 8; ++j) put4(32 * c + 8 * l + j, ((g >> (2 * j)) & 3) | (((sg >> j) & 1) << 3)); } }
         } break;
         case PYRE_IQ3_XXS: {                                           // gguf_q.rs:136-140
           const uint8_t* b = row + (size_t)(ku >> 2) * 98; float d = h2(b);
@@ -145,10 +153,9 @@ template <int FMT> __global__ __launch_bounds__(64) void k_rows(QMatDev m, const
 template <int FMT, int T, int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int upw,
                                                   GemvEpi ep, const uint2* __restrict__ g2) {
-  __shared__ uint2 lds2[FMT == FMT_IQ2_XS ? 512 : 1];
+  const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   __shared__ float red[NW][T][64];
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
-  if constexpr (FMT == FMT_IQ2_XS) { for (int i = threadIdx.x; i < 512; i += NW * 64) lds2[i] = g2[i]; __syncthreads(); }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // conv epilogue: wave 0 fetches its rows' taps and state first, so the loads overlap the dot products
   float cw[8], chist[8]; const bool conv_row = ep.co != nullptr && wave == 0 && tile * 64 + lane < ep.ch;
