@@ -139,6 +139,21 @@ int  pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, in
 /* Harness access: install n positions of (already normalised + rotated) keys and values [n][nkv*hd]; read them back. */
 int  pyre_attn_load_cache(pyre_ctx* ctx, pyre_attn* a, const float* k_host, const float* v_host, int n);
 int  pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_host);
+/* The QSA sparse indexer of attn_core (qwen4exp_gguf.rs:1565-1599), attached before the first position: rows given to
+ * pyre_attn_decode_kv4 then carry [.. | index queries idx_nh*idx_hd | index key idx_hd] after q/k/v.  A query that sees
+ * more than idx_budget + idx_ratio - 1 positions attends to the idx_budget / idx_ratio blocks of idx_ratio tokens with
+ * the largest sum_h relu(q_h . pooled block key) / sqrt(idx_hd) and to the incomplete tail; blocks of equal score are
+ * taken lowest index first (the reference's select_nth_unstable leaves that order open). */
+int  pyre_attn_set_indexer(pyre_ctx* ctx, pyre_attn* a, int idx_nh, int idx_hd, int idx_ratio, int idx_budget, const float* iqn /*[idx_hd]*/, const float* ikn /*[idx_hd]*/);
+/* qn_ctx::rope_inv (src/qn_ctx.rs:164-185) for a model context of ctx_tokens: YaRN frequencies and magnitude factor when
+ * ctx_tokens > ctx_train > 0. */
+int  pyre_attn_set_context(pyre_ctx* ctx, pyre_attn* a, int ctx_train, int ctx_tokens);
+/* Harness access: install the raw index keys [len][idx_hd] of the cached positions (complete blocks are pooled on the
+ * device); read the raw keys and the pooled block keys [len/idx_ratio][idx_hd]; read the positions the last decode call
+ * selected for its token ti (*count = -1: every visible position). */
+int  pyre_attn_load_index(pyre_ctx* ctx, pyre_attn* a, const float* ik_host);
+int  pyre_attn_read_index(pyre_ctx* ctx, pyre_attn* a, float* ik_host, float* ib_host);
+int  pyre_attn_read_selection(pyre_ctx* ctx, pyre_attn* a, int ti, int32_t* pos_host, int cap, int32_t* count);
 
 /* ---- model: the layer API engine_qn drives ------------------------------------------------------------------------
  * Model::{load, new_state, forward, forward_multi, spec_keep} (qwen4exp_gguf.rs:462, 1345, 2050, 2365, 2495) as
@@ -157,6 +172,7 @@ enum {
   PYRE_T_ATTN_Q, PYRE_T_ATTN_K, PYRE_T_ATTN_V, PYRE_T_ATTN_OUTPUT, PYRE_T_ATTN_Q_NORM, PYRE_T_ATTN_K_NORM,
   PYRE_T_ATTN_QKV, PYRE_T_ATTN_GATE, PYRE_T_SSM_BETA, PYRE_T_SSM_ALPHA, PYRE_T_SSM_A, PYRE_T_SSM_DT_BIAS, PYRE_T_SSM_CONV1D, PYRE_T_SSM_NORM, PYRE_T_SSM_OUT,
   PYRE_T_FFN_GATE_INP, PYRE_T_FFN_GATE_EXPS, PYRE_T_FFN_UP_EXPS, PYRE_T_FFN_DOWN_EXPS, PYRE_T_FFN_GATE_INP_SHEXP, PYRE_T_FFN_GATE_SHEXP, PYRE_T_FFN_UP_SHEXP, PYRE_T_FFN_DOWN_SHEXP,
+  PYRE_T_INDEXER_Q_PROJ, PYRE_T_INDEXER_K_PROJ, PYRE_T_INDEXER_Q_NORM, PYRE_T_INDEXER_K_NORM,   /* blk.N.indexer.* (qwen4exp_gguf.rs:501): all attention layers or none */
   PYRE_LAYER_SLOTS
 };
 enum { PYRE_G_TOKEN_EMBD = 0, PYRE_G_OUTPUT_HC_NORM, PYRE_G_OUTPUT_HC_DOWN, PYRE_G_OUTPUT_HC_UP, PYRE_G_OUTPUT, PYRE_GLOBAL_SLOTS };
@@ -170,6 +186,13 @@ typedef struct {
   int32_t vocab;
   int32_t kv_bits;    /* 4 (PYRE_QN_KV_BITS default) or 0 */
   int32_t kv_recent;  /* PYRE_QN_KV8_RECENT default 1024 */
+  /* QSA sparse indexer (qwen4exp_gguf.rs:24-25, 481-485): heads (0 = none), key length, tokens per block, token budget.
+   * Attention is dense up to idx_budget + idx_ratio - 1 visible positions and attends to idx_budget / idx_ratio
+   * selected blocks plus the incomplete tail beyond (attn_core, :1565-1599). */
+  int32_t idx_nh, idx_hd, idx_ratio, idx_budget;
+  /* trained context length and the context the model is built for (Cfg::ctx_train, Cfg::max_ctx): ctx > ctx_train > 0
+   * switches the YaRN frequency table and magnitude factor on (qn_ctx::rope_inv, src/qn_ctx.rs:164-185). */
+  int32_t ctx_train, ctx;
 } pyre_model_cfg;
 
 /* ---- GGUF container (host only, no GPU needed): Gguf::open / mat / meta accessors, src/model/gguf_q.rs:250-336 --------
@@ -193,8 +216,10 @@ long   pyre_gguf_meta_arr_u64(const pyre_gguf* g, const char* key, uint64_t* out
 
 /* Model::load (qwen4exp_gguf.rs:462-524): `general.architecture` must be qwen4exp; configuration from the `qwen4exp.*`
  * keys, tensors by their GGUF names (blk.N.*, token_embd, output_hc_*, output or the tied embedding).  kv_bits and
- * kv_recent are run-time settings of the reference, not file contents.  Files with PLE layers are refused. */
-int   pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, pyre_model** out);
+ * kv_recent are run-time settings of the reference, not file contents, and so is the context the model is built for
+ * (qn_ctx::startup_tokens, PYRE_QN_CTX).  The QSA indexer is taken when `attention.indexer.head_count` > 0 and the
+ * indexer tensors exist.  Files with PLE layers are refused. */
+int   pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, int ctx_tokens /* 0: the trained context */, pyre_model** out);
 /* Copies (and re-lays-out) every tensor into device memory; the caller's buffers are free afterwards. */
 int   pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* layer_tensors /*[n_layers][PYRE_LAYER_SLOTS]*/,
                         const pyre_tensor* globals /*[PYRE_GLOBAL_SLOTS]*/, pyre_model** out);

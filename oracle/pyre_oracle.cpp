@@ -343,39 +343,77 @@ void gdn_core(int nk, int nv, int dk, int dv, int kk, float eps, const float* a,
   }
 }
 
-// rope, qwen4exp_gguf.rs:1436-1439 with rope_cs :529-533 (mscale == 1): angle = pos as f32 * inv[i]
-void rope(float* v, int pos, int n_rot, const float* inv) {
+// rope, qwen4exp_gguf.rs:1436-1439 with rope_cs :529-533: angle = pos as f32 * inv[i]; cos and sin are multiplied by
+// the YaRN magnitude factor only when it is not 1
+void rope(float* v, int pos, int n_rot, const float* inv, float mscale = 1.0f) {
   int half = n_rot / 2;
-  for (int i = 0; i < half; ++i) { float a = (float)pos * inv[i]; float s = sinf(a), c = cosf(a); float x0 = v[i], x1 = v[i + half]; v[i] = x0 * c - x1 * s; v[i + half] = x1 * c + x0 * s; }
+  for (int i = 0; i < half; ++i) { float a = (float)pos * inv[i]; float s = sinf(a), c = cosf(a); if (mscale != 1.0f) { c = c * mscale; s = s * mscale; }
+    float x0 = v[i], x1 = v[i + half]; v[i] = x0 * c - x1 * s; v[i + half] = x1 * c + x0 * s; }
 }
 
-// attn_core, qwen4exp_gguf.rs:1558-1615, dense branch (no indexer).  Cache rows below the packed boundary are read
-// through the 4-bit round trip (kvq_roundtrip semantics, :1535), the cache itself keeps f32.
-void attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, const float* qn, const float* kn,
-               const float* qf, const float* kf_in, const float* vf, int start, int t, int kv_bits, int recent, float* kc, float* vc, float* att) {
+// attn_core, qwen4exp_gguf.rs:1558-1615.  Cache rows below the packed boundary are read through the 4-bit round trip
+// (kvq_roundtrip semantics, :1535), the cache itself keeps f32.  With an indexer (idx_nh > 0): raw index keys are
+// appended, every completed block of `ratio` tokens is pooled (mean, RMSNorm, RoPE at the block's first position,
+// :1571-1578), and a query that sees more than budget + ratio - 1 positions attends only to the budget/ratio blocks
+// with the largest  sum_h relu(q_h . block key) / sqrt(idx_hd)  plus the incomplete tail (:1589-1599).
+struct Qsa { int nh = 0, hd = 0, ratio = 1, budget = 0; const float* iqn = nullptr; const float* ikn = nullptr; const float* iq = nullptr; const float* ik = nullptr;
+             float* ikc = nullptr; float* ibc = nullptr; int32_t* sel = nullptr; int32_t* sel_n = nullptr; int sel_stride = 0; };
+void attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, float mscale, const float* qn, const float* kn,
+               const float* qf, const float* kf_in, const float* vf, int start, int t, int kv_bits, int recent, float* kc, float* vc, float* att, const Qsa& qs = Qsa()) {
   size_t row = (size_t)nkv * hd;
   std::vector<float> kf(kf_in, kf_in + (size_t)t * row);
-  for (int ti = 0; ti < t; ++ti) for (int h = 0; h < nkv; ++h) { float* kh = kf.data() + ti * row + (size_t)h * hd; rms_inplace(kh, kn, eps, hd); rope(kh, start + ti, n_rot, inv); }
+  for (int ti = 0; ti < t; ++ti) for (int h = 0; h < nkv; ++h) { float* kh = kf.data() + ti * row + (size_t)h * hd; rms_inplace(kh, kn, eps, hd); rope(kh, start + ti, n_rot, inv, mscale); }
   memcpy(kc + start * row, kf.data(), sizeof(float) * t * row); memcpy(vc + start * row, vf, sizeof(float) * t * row);
+  const int ihd = qs.hd, ir = qs.ratio, inh = qs.nh; const int dense_n = inh > 0 ? qs.budget + ir - 1 : INT32_MAX;
+  std::vector<float> iqs;
+  if (inh > 0) {
+    memcpy(qs.ikc + (size_t)start * ihd, qs.ik, sizeof(float) * (size_t)t * ihd);
+    int nt = start + t;
+    for (int b = start / ir; b < nt / ir; ++b) {          // blocks [0, start / ir) were pooled by earlier calls
+      float* pk = qs.ibc + (size_t)b * ihd; for (int i = 0; i < ihd; ++i) pk[i] = 0.0f;
+      for (int p = b * ir; p < (b + 1) * ir; ++p) for (int i = 0; i < ihd; ++i) pk[i] += qs.ikc[(size_t)p * ihd + i];
+      for (int i = 0; i < ihd; ++i) pk[i] /= (float)ir;
+      rms_inplace(pk, qs.ikn, eps, ihd); rope(pk, b * ir, n_rot, inv, mscale);
+    }
+    if (start + t > dense_n) {
+      iqs.assign(qs.iq, qs.iq + (size_t)t * inh * ihd);
+      for (int ti = 0; ti < t; ++ti) for (int h = 0; h < inh; ++h) { float* qh = iqs.data() + ((size_t)ti * inh + h) * ihd; rms_inplace(qh, qs.iqn, eps, ihd); rope(qh, start + ti, n_rot, inv, mscale); }
+    }
+  }
   float scale = 1.0f / sqrtf((float)hd); int grp = nh / nkv;
   std::vector<float> qh(hd), krt(row), vrt(row);
   for (int ti = 0; ti < t; ++ti) {
     int n = start + ti + 1; size_t pb = packed_boundary(n, kv_bits, recent);
+    std::vector<int> ps;                      // attended positions, ascending
+    bool sparse = !iqs.empty() && n > dense_n;
+    if (sparse) {
+      int nb = n / ir, kk = qs.budget / ir; float iscale = 1.0f / sqrtf((float)ihd);
+      const float* q = iqs.data() + (size_t)ti * inh * ihd;
+      std::vector<std::pair<float, int>> sc(nb);
+      for (int b = 0; b < nb; ++b) { const float* kb = qs.ibc + (size_t)b * ihd; float sm = 0.0f; for (int h = 0; h < inh; ++h) sm += fmaxf(dot(q + (size_t)h * ihd, kb, ihd), 0.0f); sc[b] = {sm * iscale, b}; }
+      std::stable_sort(sc.begin(), sc.end(), [](const std::pair<float, int>& a, const std::pair<float, int>& b) { return a.first > b.first; });   // ties: lower block first
+      std::vector<int> blocks; for (int i = 0; i < kk && i < nb; ++i) blocks.push_back(sc[i].second);
+      std::sort(blocks.begin(), blocks.end());
+      for (int b : blocks) for (int p = b * ir; p < (b + 1) * ir; ++p) ps.push_back(p);
+      for (int p = nb * ir; p < n; ++p) ps.push_back(p);
+    } else { ps.resize(n); for (int p = 0; p < n; ++p) ps[p] = p; }
+    if (qs.sel_n) { qs.sel_n[ti] = sparse ? (int32_t)ps.size() : -1; if (sparse && qs.sel) for (size_t i = 0; i < ps.size() && (int)i < qs.sel_stride; ++i) qs.sel[(size_t)ti * qs.sel_stride + i] = ps[i]; }
+    const int np = (int)ps.size();
     for (int h = 0; h < nh; ++h) {
       size_t base = (size_t)ti * nh * 2 * hd + (size_t)h * 2 * hd;
-      memcpy(qh.data(), qf + base, sizeof(float) * hd); rms_inplace(qh.data(), qn, eps, hd); rope(qh.data(), start + ti, n_rot, inv);
+      memcpy(qh.data(), qf + base, sizeof(float) * hd); rms_inplace(qh.data(), qn, eps, hd); rope(qh.data(), start + ti, n_rot, inv, mscale);
       int kvh = h / grp; float* out = att + ((size_t)ti * nh + h) * hd; for (int i = 0; i < hd; ++i) out[i] = 0.0f;
-      std::vector<float> sc(n);
-      for (int p = 0; p < n; ++p) {
-        const float* kr = kc + p * row + (size_t)kvh * hd;
+      std::vector<float> sc(np);
+      for (int j = 0; j < np; ++j) {
+        int p = ps[j]; const float* kr = kc + p * row + (size_t)kvh * hd;
         if ((size_t)p < pb) { memcpy(krt.data(), kr, sizeof(float) * hd); kvq_roundtrip(krt.data(), hd, 4); kr = krt.data(); }
-        sc[p] = dot(qh.data(), kr, hd) * scale;
+        sc[j] = dot(qh.data(), kr, hd) * scale;
       }
-      float mx = -INFINITY; for (int p = 0; p < n; ++p) mx = fmaxf(mx, sc[p]);
-      float sum = 0.0f; for (int p = 0; p < n; ++p) { sc[p] = expf(sc[p] - mx); sum += sc[p]; }
+      float mx = -INFINITY; for (int j = 0; j < np; ++j) mx = fmaxf(mx, sc[j]);
+      float sum = 0.0f; for (int j = 0; j < np; ++j) { sc[j] = expf(sc[j] - mx); sum += sc[j]; }
       float iv = 1.0f / sum;
-      for (int p = 0; p < n; ++p) {
-        float wgt = sc[p] * iv; const float* vr = vc + p * row + (size_t)kvh * hd;
+      for (int j = 0; j < np; ++j) {
+        int p = ps[j]; float wgt = sc[j] * iv; const float* vr = vc + p * row + (size_t)kvh * hd;
         if ((size_t)p < pb) { memcpy(vrt.data(), vr, sizeof(float) * hd); kvq_roundtrip(vrt.data(), hd, 4); vr = vrt.data(); }
         for (int i = 0; i < hd; ++i) out[i] += wgt * vr[i];
       }
@@ -455,7 +493,8 @@ void hc_combine(int d, int hc, float* x, const float* out, const float* inj, int
 // ---------- model ------------------------------------------------------------------------------
 struct OrcModel {
   OrcCfg c; std::vector<OrcTensor> lt; OrcTensor g[ORC_GLOBAL_SLOTS]; int threads;
-  std::vector<float> rope_inv;
+  std::vector<float> rope_inv; float mscale = 1.0f;
+  bool has_idx(int il) const { return c.idx_nh > 0 && T(il, ORC_IDX_Q).data != nullptr; }
   std::vector<std::vector<float>> vec;  // dequantized small tensors, indexed like lt (empty when unused)
   std::vector<float> head_norm;
   const OrcTensor& T(int il, int slot) const { return lt[(size_t)il * ORC_LAYER_SLOTS + slot]; }
@@ -465,7 +504,7 @@ struct OrcModel {
 struct OrcCkpt { std::vector<std::vector<float>> conv, ssm; };
 struct OrcState {
   std::vector<uint32_t> tokens;
-  std::vector<std::vector<float>> conv, ssm, k, v;
+  std::vector<std::vector<float>> conv, ssm, k, v, ik, ib;   // ik / ib: raw index keys [pos][idx_hd], pooled block keys [block][idx_hd]
   std::vector<OrcCkpt> ck;  // state after each token of the last forward_multi
 };
 
@@ -491,6 +530,22 @@ size_t orc_kv_packed_boundary(size_t n, int kv_bits, int recent) { return packed
 
 // rope_inv, qn_ctx.rs:164-170 (unscaled branch): inv[i] = base.powf(-(2 i) / n_rot)
 void orc_rope_inv(int n_rot, float base, float* inv) { for (int i = 0; i < n_rot / 2; ++i) inv[i] = powf(base, -(2.0f * (float)i) / (float)n_rot); }
+// rope_inv, qn_ctx.rs:164-185, both branches
+float orc_rope_inv_yarn(int n_rot, float base, int ctx_train, int ctx, float* inv) {
+  int half = n_rot / 2;
+  float scale = (ctx_train > 0 && ctx > ctx_train) ? (float)ctx / (float)ctx_train : 1.0f;
+  if (scale <= 1.0f) { orc_rope_inv(n_rot, base, inv); return 1.0f; }
+  float dim = (float)n_rot;
+  auto corr = [&](float rot) { return (dim * logf((float)ctx_train / (rot * 2.0f * 3.14159265358979323846f))) / (2.0f * logf(base)); };
+  float low = fmaxf(floorf(corr(32.0f)), 0.0f);
+  float high = fminf(ceilf(corr(1.0f)), (float)(half > 0 ? half - 1 : 0));
+  for (int i = 0; i < half; ++i) {
+    float extrap = powf(base, -(2.0f * (float)i) / dim), interp = extrap / scale;
+    float ramp = fabsf(high - low) < 1e-6f ? 1.0f : fminf(fmaxf(((float)i - low) / (high - low), 0.0f), 1.0f);
+    inv[i] = interp * (1.0f - ramp) + extrap * ramp;
+  }
+  return 1.0f + 0.1f * logf(scale);
+}
 // sampler::argmax, sampler.rs:142-148: first index of the maximum (strict >)
 uint32_t orc_argmax(const float* l, size_t n) { size_t best = 0; for (size_t i = 1; i < n; ++i) if (l[i] > l[best]) best = i; return (uint32_t)best; }
 int orc_top_k(const float* r, int n, int k, int32_t* idx, float* w) { return top_k(r, n, k, idx, w) ? 0 : -1; }
@@ -506,7 +561,14 @@ void orc_gdn_core(int nk, int nv, int dk, int dv, int conv_k, float eps, const f
 }
 void orc_attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, const float* qn, const float* kn, const float* q, const float* k, const float* v,
                    int start, int t, int kv_bits, int kv_recent, float* kc, float* vc, float* out) {
-  attn_core(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, start, t, kv_bits, kv_recent, kc, vc, out);
+  attn_core(nh, nkv, hd, n_rot, eps, inv, 1.0f, qn, kn, q, k, v, start, t, kv_bits, kv_recent, kc, vc, out);
+}
+void orc_attn_core_qsa(int nh, int nkv, int hd, int n_rot, float eps, const float* inv, float mscale, const float* qn, const float* kn, const float* q, const float* k, const float* v,
+                       int start, int t, int kv_bits, int kv_recent, float* kc, float* vc, int idx_nh, int idx_hd, int idx_ratio, int idx_budget, const float* iqn, const float* ikn,
+                       const float* iq, const float* ik, float* ikc, float* ibc, float* out, int32_t* sel, int32_t* sel_n, int sel_stride) {
+  Qsa qs; qs.nh = idx_nh; qs.hd = idx_hd; qs.ratio = idx_ratio < 1 ? 1 : idx_ratio; qs.budget = idx_budget; qs.iqn = iqn; qs.ikn = ikn; qs.iq = iq; qs.ik = ik; qs.ikc = ikc; qs.ibc = ibc;
+  qs.sel = sel; qs.sel_n = sel_n; qs.sel_stride = sel_stride;
+  attn_core(nh, nkv, hd, n_rot, eps, inv, mscale, qn, kn, q, k, v, start, t, kv_bits, kv_recent, kc, vc, out, qs);
 }
 int orc_moe_ffn(int d, int n_exp, int top_k_, int ff, const OrcTensor* router, const OrcTensor* gate_e, const OrcTensor* up_e, const OrcTensor* down_e,
                 const float* sh_gate_inp, const OrcTensor* sh_gate, const OrcTensor* sh_up, const OrcTensor* sh_down,
@@ -521,10 +583,10 @@ OrcModel* orc_model_create(const OrcCfg* cfg, const OrcTensor* lt, const OrcTens
   OrcModel* m = new OrcModel(); m->c = *cfg; m->threads = threads;
   m->lt.assign(lt, lt + (size_t)cfg->n_layers * ORC_LAYER_SLOTS); for (int i = 0; i < ORC_GLOBAL_SLOTS; ++i) m->g[i] = globals[i];
   m->vec.resize(m->lt.size());
-  static const int vs[] = {ORC_HCA_NORM, ORC_HCF_NORM, ORC_ATTN_QN, ORC_ATTN_KN, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_SH_GATE_INP};
+  static const int vs[] = {ORC_HCA_NORM, ORC_HCF_NORM, ORC_ATTN_QN, ORC_ATTN_KN, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_SH_GATE_INP, ORC_IDX_QN, ORC_IDX_KN};
   for (int il = 0; il < cfg->n_layers; ++il) for (int s : vs) if (!to_vec(m->T(il, s), m->vec[(size_t)il * ORC_LAYER_SLOTS + s])) { delete m; return nullptr; }
   if (!to_vec(m->g[ORC_G_HEAD_NORM], m->head_norm)) { delete m; return nullptr; }
-  m->rope_inv.resize(cfg->n_rot / 2); orc_rope_inv(cfg->n_rot, cfg->rope_base, m->rope_inv.data());
+  m->rope_inv.resize(cfg->n_rot / 2); m->mscale = orc_rope_inv_yarn(cfg->n_rot, cfg->rope_base, cfg->ctx_train, cfg->ctx, m->rope_inv.data());
   return m;
 }
 void orc_model_destroy(OrcModel* m) { delete m; }
@@ -532,7 +594,7 @@ void orc_model_destroy(OrcModel* m) { delete m; }
 OrcState* orc_state_create(const OrcModel* m) {  // new_state, qwen4exp_gguf.rs:1345-1353
   OrcState* s = new OrcState(); const OrcCfg& c = m->c; int ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv;
   for (int il = 0; il < c.n_layers; ++il) {
-    if (m->full(il)) { s->k.emplace_back(); s->v.emplace_back(); }
+    if (m->full(il)) { s->k.emplace_back(); s->v.emplace_back(); s->ik.emplace_back(); s->ib.emplace_back(); }
     else { s->conv.emplace_back((size_t)(c.conv_k - 1) * ch, 0.0f); s->ssm.emplace_back((size_t)c.lin_nv * c.lin_dk * c.lin_dv, 0.0f); }
   }
   return s;
@@ -543,6 +605,8 @@ float* orc_state_conv(OrcState* s, int li) { return s->conv[li].data(); }
 float* orc_state_ssm(OrcState* s, int li) { return s->ssm[li].data(); }
 float* orc_state_k(OrcState* s, int ai) { return s->k[ai].data(); }
 float* orc_state_v(OrcState* s, int ai) { return s->v[ai].data(); }
+float* orc_state_ik(OrcState* s, int ai) { return s->ik[ai].data(); }
+float* orc_state_ib(OrcState* s, int ai) { return s->ib[ai].data(); }
 
 // forward_inner, qwen4exp_gguf.rs:2087-2157 (host branch :2134-2142, head :2150-2153)
 int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, float* logits) {
@@ -561,7 +625,15 @@ int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, flo
       std::vector<float> q((size_t)t * nh * 2 * hd), k(t * row), v(t * row), att((size_t)t * nh * hd);
       if (!mm(&m->T(il, ORC_ATTN_Q), mixed.data(), t, q.data(), th) || !mm(&m->T(il, ORC_ATTN_K), mixed.data(), t, k.data(), th) || !mm(&m->T(il, ORC_ATTN_V), mixed.data(), t, v.data(), th)) return -3;
       st->k[ai].resize((size_t)(start + t) * row); st->v[ai].resize((size_t)(start + t) * row);
-      attn_core(nh, nkv, hd, c.n_rot, c.eps, m->rope_inv.data(), m->V(il, ORC_ATTN_QN), m->V(il, ORC_ATTN_KN), q.data(), k.data(), v.data(), start, t, c.kv_bits, c.kv_recent, st->k[ai].data(), st->v[ai].data(), att.data());
+      Qsa qs; std::vector<float> iq, ik;
+      if (m->has_idx(il)) {
+        int ihd = c.idx_hd, ir = c.idx_ratio < 1 ? 1 : c.idx_ratio; iq.resize((size_t)t * c.idx_nh * ihd); ik.resize((size_t)t * ihd);
+        if (!mm(&m->T(il, ORC_IDX_Q), mixed.data(), t, iq.data(), th) || !mm(&m->T(il, ORC_IDX_K), mixed.data(), t, ik.data(), th)) return -3;
+        st->ik[ai].resize((size_t)(start + t) * ihd); st->ib[ai].resize((size_t)((start + t) / ir) * ihd);
+        qs.nh = c.idx_nh; qs.hd = ihd; qs.ratio = ir; qs.budget = c.idx_budget; qs.iqn = m->V(il, ORC_IDX_QN); qs.ikn = m->V(il, ORC_IDX_KN); qs.iq = iq.data(); qs.ik = ik.data();
+        qs.ikc = st->ik[ai].data(); qs.ibc = st->ib[ai].data();
+      }
+      attn_core(nh, nkv, hd, c.n_rot, c.eps, m->rope_inv.data(), m->mscale, m->V(il, ORC_ATTN_QN), m->V(il, ORC_ATTN_KN), q.data(), k.data(), v.data(), start, t, c.kv_bits, c.kv_recent, st->k[ai].data(), st->v[ai].data(), att.data(), qs);
       if (!mm(&m->T(il, ORC_ATTN_O), att.data(), t, o.data(), th)) return -3;
       ++ai;
     } else {  // linear, :1617-1621
@@ -597,6 +669,9 @@ int orc_spec_keep(const OrcModel* m, OrcState* st, int t, int keep) {
   size_t n = st->tokens.size() - t + keep; st->tokens.resize(n);
   st->conv = st->ck[keep - 1].conv; st->ssm = st->ck[keep - 1].ssm;
   size_t row = (size_t)m->c.n_kv * m->c.hd; for (auto& k : st->k) k.resize(n * row); for (auto& v : st->v) v.resize(n * row);
+  size_t ihd = m->c.idx_hd, ir = m->c.idx_ratio < 1 ? 1 : m->c.idx_ratio;       // :2509-2513
+  for (auto& k : st->ik) if (!k.empty()) k.resize(n * ihd);
+  for (auto& b : st->ib) if (!b.empty()) b.resize((n / ir) * ihd);
   return 0;
 }
 // spec::generate, greedy branch (spec.rs:156-267; accept loop :229-238, keep :249), drafts from a fixed stream:

@@ -19,6 +19,10 @@
  *   orc_gdn_core           closed forms (zero state, delta-rule overwrite property, pure decay,
  *                          one-hot conv = delay) + an independent numpy statement
  *   orc_attn_core          single position, uniform keys, rope at pos 0, numpy statement
+ *   orc_attn_core_qsa      equals the dense branch up to budget + ratio - 1 positions; selection by brute force
+ *                          (numpy sort) on distinct scores; hand-built keys that force a known block set;
+ *                          block pooling closed form (identical keys -> pooled key = rope(rms(key)))
+ *   orc_rope_inv_yarn      the reference's asserted properties (qn_ctx.rs:406-419) + float64 closed form
  *   orc_moe_ffn            numpy statement built from orc_dequant'd dense weights
  *   orc_forward            numpy statement of the whole token step on a tiny model
  * Parity unpinned (only running the reference could pin): the last-ulp behaviour of
@@ -44,6 +48,7 @@ enum {
   ORC_ATTN_Q, ORC_ATTN_K, ORC_ATTN_V, ORC_ATTN_O, ORC_ATTN_QN, ORC_ATTN_KN,
   ORC_LIN_QKV, ORC_LIN_Z, ORC_LIN_BETA, ORC_LIN_ALPHA, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_LIN_OUT,
   ORC_ROUTER, ORC_GATE_E, ORC_UP_E, ORC_DOWN_E, ORC_SH_GATE_INP, ORC_SH_GATE, ORC_SH_UP, ORC_SH_DOWN,
+  ORC_IDX_Q, ORC_IDX_K, ORC_IDX_QN, ORC_IDX_KN,                     /* blk.N.indexer.{q_proj,k_proj,q_norm,k_norm}.weight (optional) */
   ORC_LAYER_SLOTS
 };
 enum { ORC_G_EMBD = 0, ORC_G_HEAD_NORM, ORC_G_HEAD_DOWN, ORC_G_HEAD_UP, ORC_G_OUT, ORC_GLOBAL_SLOTS };
@@ -56,6 +61,10 @@ typedef struct {
   int32_t vocab;
   int32_t kv_bits;    /* 0 = f32 cache everywhere, 4 = positions below the packed boundary are read through kv4 */
   int32_t kv_recent;  /* f32 window kept at the tail (reference default 1024) */
+  /* QSA sparse indexer (qwen4exp_gguf.rs:24-25): heads (0 = none), key length, block size in tokens, token budget */
+  int32_t idx_nh, idx_hd, idx_ratio, idx_budget;
+  /* trained context and the context the model is built for; ctx > ctx_train > 0 switches YaRN on (qn_ctx.rs:164-185) */
+  int32_t ctx_train, ctx;
 } OrcCfg;
 
 int    orc_type_geom(uint32_t ty, int* elems, int* bytes);
@@ -72,6 +81,8 @@ void   orc_kvq_roundtrip(float* x, size_t n, int bits);
 size_t orc_kv_packed_boundary(size_t n_visible, int kv_bits, int recent);
 
 void   orc_rope_inv(int n_rot, float base, float* inv);
+/* qn_ctx::rope_inv with the YaRN branch; returns mscale (1 when ctx <= ctx_train or ctx_train == 0). */
+float  orc_rope_inv_yarn(int n_rot, float base, int ctx_train, int ctx, float* inv);
 uint32_t orc_argmax(const float* logits, size_t n);
 int    orc_top_k(const float* r, int n, int k, int32_t* idx, float* w);
 void   orc_rms(const float* x, const float* w, float eps, float* y, size_t n);
@@ -92,6 +103,19 @@ void   orc_gdn_core(int nk, int nv, int dk, int dv, int conv_k, float eps,
 void   orc_attn_core(int nh, int nkv, int hd, int n_rot, float eps, const float* rope_inv,
                      const float* qn, const float* kn, const float* q, const float* k, const float* v,
                      int start, int t, int kv_bits, int kv_recent, float* kc, float* vc, float* out);
+
+/* attn_core with the QSA indexer (qwen4exp_gguf.rs:1565-1599) and the YaRN magnitude factor.  iq [t][idx_nh*idx_hd],
+ * ik [t][idx_hd] raw indexer projections; ikc [cap][idx_hd] raw index keys and ibc [cap/ratio][idx_hd] pooled block keys
+ * are caller-owned like kc/vc (rows [0,start) resp. [0,start/ratio) valid on entry).  sel (optional) receives, per
+ * token, the attended positions in ascending order, sel_n[ti] of them, in rows of sel_stride ints; sel_n[ti] = -1 means
+ * every visible position (dense).  Among blocks of equal score the lower block index is taken first (the reference's
+ * select_nth_unstable leaves that order unspecified). */
+void   orc_attn_core_qsa(int nh, int nkv, int hd, int n_rot, float eps, const float* rope_inv, float mscale,
+                         const float* qn, const float* kn, const float* q, const float* k, const float* v,
+                         int start, int t, int kv_bits, int kv_recent, float* kc, float* vc,
+                         int idx_nh, int idx_hd, int idx_ratio, int idx_budget, const float* iqn, const float* ikn,
+                         const float* iq, const float* ik, float* ikc, float* ibc,
+                         float* out, int32_t* sel, int32_t* sel_n, int sel_stride);
 
 /* MoE FFN (ffn + routed f32 branch).  x [t][d] -> y [t][d]. sel_idx/sel_w (optional) receive [t][k]. */
 int    orc_moe_ffn(int d, int n_exp, int top_k, int ff, const OrcTensor* router, const OrcTensor* gate_e,
@@ -117,6 +141,8 @@ float*    orc_state_conv(OrcState*, int li);
 float*    orc_state_ssm(OrcState*, int li);
 float*    orc_state_k(OrcState*, int ai);
 float*    orc_state_v(OrcState*, int ai);
+float*    orc_state_ik(OrcState*, int ai);
+float*    orc_state_ib(OrcState*, int ai);
 /* Model::forward: append ids, return logits of the last token in logits[vocab]. */
 int       orc_forward(const OrcModel*, OrcState*, const uint32_t* ids, int n, float* logits);
 /* forward_multi semantics = n sequential steps; logits [n][vocab]; keeps per-token checkpoints. */

@@ -39,6 +39,7 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
     int i = ri;
     float ang = (float)pos * rinv;
     float sn = sinf(ang), cs = cosf(ang);
+    if (a.mscale != 1.0f) { cs = cs * a.mscale; sn = sn * a.mscale; }      // YaRN magnitude factor, rope_cs (:529-533)
     float x0 = buf[i], x1 = buf[i + half];
     v = tid < half ? x0 * cs - x1 * sn : x1 * cs + x0 * sn;
   }
@@ -252,14 +253,162 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
   }
 }
 
+// The same kernel over a position list: entry i of plist[ti] (pcount[ti] entries, ascending positions) takes the place of
+// position i; pcount[ti] < 0 means every visible position (the list is not read).  Listed positions are scattered over
+// the packed and the f32 part of the cache, so the choice between them is made per lane, not per wave.
+template <int HD, int G>
+__global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
+                                                                         const int* __restrict__ plist, const int* __restrict__ pcount, int list_stride) {
+  static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
+  constexpr int NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;
+  __shared__ float red[4 * CH * G];
+  __shared__ float sc[CH][G];
+  __shared__ float wmax[NPW][G], wsum[NPW][G], cm[G];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
+  if (posp) start = *posp;
+  const int n = start + ti + 1, cnt = pcount[ti];
+  const bool listed = cnt >= 0; const int ne = listed ? cnt : n;       // entries to attend to
+  if (chunk * CH >= ne) return;
+  const int* list = plist + (size_t)ti * list_stride;
+  const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
+  const int wbase = chunk * CH + pw * 64;
+  const bool valid = wbase + lane < ne, active = wbase < ne;
+  const float scale = 1.0f / sqrtf((float)HD);
+  const int li = lane & 15, lg = lane >> 4;
+  const int row = a.nkv * HD;
+  auto pos_of = [&](int i) { int ii = min(i, ne - 1); return listed ? list[ii] : ii; };
+  {
+    f4v D[4];
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) {
+      float B[16];
+      if (li < G) {
+        const float4* q4 = (const float4*)(qbuf + ((size_t)ti * a.nh + (size_t)kvh * G + li) * HD + dq * 64 + 16 * lg);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { float4 v = q4[j]; B[4 * j] = v.x; B[4 * j + 1] = v.y; B[4 * j + 2] = v.z; B[4 * j + 3] = v.w; }
+      } else {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) B[s] = 0.0f;
+      }
+      float A[4][16];
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt) {
+        const size_t pp = (size_t)pos_of(wbase + 16 * pt + li);
+        if ((int)pp < pb) {
+          uint32_t k0 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp)], k1 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp)];
+          float ksc = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp)];
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(s < 8 ? k0 : k1, s & 7) * ksc;
+        } else {
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp)];
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < 16; ++s)
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
+    }
+    if (li < G) {
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
+    }
+  }
+  __syncthreads();
+  constexpr int GH = (G + 3) / 4;
+  const int pos = pw * 64 + lane;
+  float sv[GH];
+#pragma unroll
+  for (int gi = 0; gi < GH; ++gi) {
+    const int g = dq + 4 * gi; sv[gi] = -INFINITY;
+    if (g < G) {
+      float v = ((red[((size_t)0 * CH + pos) * G + g] + red[((size_t)1 * CH + pos) * G + g]) + red[((size_t)2 * CH + pos) * G + g]) + red[((size_t)3 * CH + pos) * G + g];
+      sv[gi] = valid ? v * scale : -INFINITY;
+      float m = sv[gi];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      if (lane == 0) wmax[pw][g] = m;
+    }
+  }
+  __syncthreads();
+  if (tid < G) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
+  __syncthreads();
+#pragma unroll
+  for (int gi = 0; gi < GH; ++gi) {
+    const int g = dq + 4 * gi;
+    if (g < G) {
+      float e = valid ? expf(sv[gi] - cm[g]) : 0.0f; sc[pos][g] = e;
+      float l = e;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+      if (lane == 0) wsum[pw][g] = l;
+    }
+  }
+  __syncthreads();
+  {
+    f4v D[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    if (active) {
+      float A[4][16];
+#pragma unroll
+      for (int s = 0; s < 16; ++s) {            // entries past the list carry weight zero; their position is clamped
+        const size_t pg = (size_t)pos_of(wbase + 4 * s + lg);
+        if ((int)pg < pb) {
+          const uint32_t vw = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
+          const float vsc = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
+          const uint32_t hw = vw >> (16 * (li & 1));
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc;
+        } else {
+          float4 v = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+          A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
+        }
+      }
+      float B[16];
+#pragma unroll
+      for (int s = 0; s < 16; ++s) B[s] = li < G ? sc[pw * 64 + 4 * s + lg][li < G ? li : 0] : 0.0f;
+#pragma unroll
+      for (int s = 0; s < 16; ++s)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
+    }
+    if (li < G) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((size_t)pw * G + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < G * HD; i += NT) {
+    int g = i / HD, dd = i % HD;
+    float o = red[((size_t)0 * G + g) * HD + dd];
+#pragma unroll
+    for (int q = 1; q < NPW; ++q) o += red[((size_t)q * G + g) * HD + dd];
+    part_o[(((size_t)ti * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
+  }
+  if (tid < G) {
+    float l = wsum[0][tid]; for (int q = 1; q < NPW; ++q) l += wsum[q][tid];
+    float* ml = part_ml + (((size_t)ti * a.nh + (size_t)kvh * G + tid) * max_chunks + chunk) * 2;
+    ml[0] = cm[tid]; ml[1] = l;
+  }
+}
+
 // grid (nh, t), 4*HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
 // Thread (grp, dim) adds the chunks grp, grp+4, ... in ascending order; the four groups are then added in order.
 template <int HD>
 __global__ __launch_bounds__(4 * HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                         int max_chunks, float* __restrict__ out) {
+                                                         int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
   __shared__ float wmax[4 * HD / 64]; __shared__ float so[4][HD]; __shared__ float sl[4];
   if (posp) start = *posp;
-  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD, n = start + ti + 1, nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD;
+  int n = start + ti + 1; if (pcount && pcount[ti] >= 0) n = pcount[ti];        // a position list: its entries are what the chunks covered
+  const int nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
   float M = -INFINITY; for (int c = tid; c < nc; c += 4 * HD) M = fmaxf(M, ml[2 * c]);
@@ -302,12 +451,18 @@ void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
   w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
 }
 
-template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp) {
+template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp, const QsaWork* qw) {
   int n = start + t, chunks = posp ? w.max_chunks : (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;      // device-side position: cover the whole cache, surplus workgroups leave at once
-  hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks);
+  if (!qw) { hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks); return; }
+  // a token attends either to all of its n <= budget + ratio - 1 visible positions or to a list: never to more than list_stride entries
+  { int lc = (qw->list_stride + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK; if (chunks > lc) chunks = lc; }
+  hipLaunchKernelGGL((k_attn_decode_sel<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, qw->plist, qw->pcount, qw->list_stride);
 }
 
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
+  return pyre_attn_launch_sel(ctx, a, kv, w, qkv, stride, start, t, packed_done, out, posp, nullptr);
+}
+int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp, const QsaWork* qw) {
   if (a.hd != 256) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: head dim %d unsupported (256 only)", a.hd);
   if (a.nkv < 1 || a.nh % a.nkv) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: %d query heads over %d kv heads", a.nh, a.nkv);
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
@@ -326,14 +481,16 @@ int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const Att
   }
   double kvb = 0; for (int ti = 0; ti < t; ++ti) { double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent); kvb += 2.0 * a.nkv * a.hd * (pb * 0.625 + (n - pb) * 4.0); }
   { ProfScope ps(ctx, "attn_decode", kvb);
-  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp); break; default: launch_decode<8>(ctx, a, kv, w, start, t, posp); } }
+  switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp, qw); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp, qw); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp, qw); break;
+    default: launch_decode<8>(ctx, a, kv, w, start, t, posp, qw); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 
 // ---- C ABI: standalone attention layer core for the block harness -----------------------------------------------------
-struct pyre_attn { pyre_ctx* ctx; AttnDev dv; KvDev kv; AttnWork w; float* params; void* kvmem; void* wmem; float* io; int len, packed, cap; };
+struct pyre_attn { pyre_ctx* ctx; AttnDev dv; KvDev kv; AttnWork w; float* params; void* kvmem; void* wmem; float* io; int len, packed, cap;
+                   QsaDev q{}; QsaBuf qb{}; QsaWork qw{}; void* qmem = nullptr; float* qparams = nullptr; float rope_base = 0; };
 
 extern "C" {
 
@@ -344,7 +501,7 @@ int pyre_attn_create(pyre_ctx* ctx, int nh, int nkv, int hd, int n_rot, float ro
   pyre_attn* a = new pyre_attn(); a->ctx = ctx; a->len = 0; a->packed = 0; a->cap = (max_ctx + 255) / 256 * 256;
   std::vector<float> hp(2 * (size_t)hd + n_rot / 2); memcpy(hp.data(), qn, 4 * hd); memcpy(hp.data() + hd, kn, 4 * hd);
   for (int i = 0; i < n_rot / 2; ++i) hp[2 * hd + i] = powf(rope_base, -(2.0f * (float)i) / (float)n_rot);    // rope_inv, src/qn_ctx.rs:168
-  a->dv = AttnDev{nullptr, nullptr, nullptr, nh, nkv, hd, n_rot, kv_bits, kv_recent, eps};
+  a->dv = AttnDev{nullptr, nullptr, nullptr, nh, nkv, hd, n_rot, kv_bits, kv_recent, eps}; a->rope_base = rope_base;
   size_t qw = (size_t)nh * 2 * hd + 2 * (size_t)nkv * hd;
   hipError_t e = hipMalloc((void**)&a->params, hp.size() * 4);
   if (e == hipSuccess) e = hipMemcpy(a->params, hp.data(), hp.size() * 4, hipMemcpyHostToDevice);
@@ -356,7 +513,7 @@ int pyre_attn_create(pyre_ctx* ctx, int nh, int nkv, int hd, int n_rot, float ro
   pyre_kv_carve(a->dv, a->cap, a->kvmem, &a->kv); pyre_attn_work_carve(a->dv, a->cap, a->wmem, &a->w);
   *out = a; return PYRE_OK;
 }
-void pyre_attn_destroy(pyre_attn* a) { if (!a) return; (void)hipStreamSynchronize(a->ctx->stream); (void)hipFree(a->params); (void)hipFree(a->kvmem); (void)hipFree(a->wmem); (void)hipFree(a->io); delete a; }
+void pyre_attn_destroy(pyre_attn* a) { if (!a) return; (void)hipStreamSynchronize(a->ctx->stream); if (a->qmem) (void)hipFree(a->qmem); if (a->qparams) (void)hipFree(a->qparams); (void)hipFree(a->params); (void)hipFree(a->kvmem); (void)hipFree(a->wmem); (void)hipFree(a->io); delete a; }
 int pyre_attn_len(const pyre_attn* a) { return a ? a->len : 0; }
 int pyre_attn_truncate(pyre_ctx* ctx, pyre_attn* a, int len) { if (!a || len < 0 || len > a->len) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_truncate: bad length"); a->len = len; return PYRE_OK; }
 
@@ -365,10 +522,12 @@ int pyre_attn_truncate(pyre_ctx* ctx, pyre_attn* a, int len) { if (!a || len < 0
 int pyre_attn_decode_kv4(pyre_ctx* ctx, pyre_attn* a, const float* qkv_host, int t, float* out_host) {
   if (!ctx || !a || !qkv_host || !out_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_decode_kv4: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_decode_kv4: t = %d outside 1..8", t);
-  size_t qw = (size_t)a->dv.nh * 2 * a->dv.hd + 2 * (size_t)a->dv.nkv * a->dv.hd, ow = (size_t)a->dv.nh * a->dv.hd;
+  size_t qb = (size_t)a->dv.nh * 2 * a->dv.hd + 2 * (size_t)a->dv.nkv * a->dv.hd, qw = qb + (a->q.nh > 0 ? (size_t)(a->q.nh + 1) * a->q.hd : 0), ow = (size_t)a->dv.nh * a->dv.hd;
   float* qd = a->io; float* od = a->io + 8 * qw;
   PYRE_HIP(ctx, hipMemcpyAsync(qd, qkv_host, (size_t)t * qw * 4, hipMemcpyHostToDevice, ctx->stream));
-  int rc = pyre_attn_launch(ctx, a->dv, a->kv, a->w, qd, (int)qw, a->len, t, &a->packed, od, nullptr); if (rc) return rc;
+  int rc = PYRE_OK;
+  if (a->q.nh > 0 && (rc = pyre_qsa_launch(ctx, a->q, a->dv, a->qb, a->qw, qd, (int)qw, (int)qb, a->len, t, nullptr))) return rc;
+  rc = pyre_attn_launch_sel(ctx, a->dv, a->kv, a->w, qd, (int)qw, a->len, t, &a->packed, od, nullptr, a->q.nh > 0 ? &a->qw : nullptr); if (rc) return rc;
   a->len += t;
   PYRE_HIP(ctx, hipMemcpyAsync(out_host, od, (size_t)t * ow * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
@@ -396,6 +555,52 @@ int pyre_attn_read_cache(pyre_ctx* ctx, pyre_attn* a, float* k_host, float* v_ho
   for (int p = 0; p < a->len; ++p) for (size_t c = 0; c < row; ++c) k_host[(size_t)p * row + c] = kt[kv_blk(c, row, p)];
   return PYRE_OK;
 }
-// kv4 pack / unpack of a flat f32 array through the device kernels' arithmetic is covered by load_cache + decode; this
-// export packs n values (multiple of 32) exactly like kv4::pack and returns words and scales.
+// Attaches a QSA indexer to the block (before any position is decoded): rows passed to pyre_attn_decode_kv4 then carry
+// [.. | index queries nh*hd | index key hd] after the q/k/v projections.
+int pyre_attn_set_indexer(pyre_ctx* ctx, pyre_attn* a, int idx_nh, int idx_hd, int idx_ratio, int idx_budget, const float* iqn_host, const float* ikn_host) {
+  if (!ctx || !a || !iqn_host || !ikn_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_set_indexer: null argument");
+  if (a->len != 0 || a->q.nh != 0) return pyre_fail(ctx, PYRE_E_STATE, "pyre_attn_set_indexer: the block already holds positions or an indexer");
+  if (idx_nh < 1 || idx_hd < 64 || idx_hd % 64 || idx_hd > 1024 || idx_hd < a->dv.n_rot || idx_ratio < 1 || idx_budget < idx_ratio || idx_budget % idx_ratio) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_attn_set_indexer: unsupported geometry");
+  QsaDev q{nullptr, nullptr, idx_nh, idx_hd, idx_ratio, idx_budget};
+  size_t bb = (pyre_qsa_buf_bytes(q, a->cap) + 255) & ~(size_t)255, wb = pyre_qsa_work_bytes(q, a->cap);
+  size_t qw = (size_t)a->dv.nh * 2 * a->dv.hd + 2 * (size_t)a->dv.nkv * a->dv.hd + (size_t)(idx_nh + 1) * idx_hd;
+  PYRE_HIP(ctx, hipMalloc(&a->qmem, bb + wb)); PYRE_HIP(ctx, hipMalloc((void**)&a->qparams, 2 * (size_t)idx_hd * 4));
+  PYRE_HIP(ctx, hipMemcpy(a->qparams, iqn_host, (size_t)idx_hd * 4, hipMemcpyHostToDevice)); PYRE_HIP(ctx, hipMemcpy(a->qparams + idx_hd, ikn_host, (size_t)idx_hd * 4, hipMemcpyHostToDevice));
+  (void)hipFree(a->io); a->io = nullptr; PYRE_HIP(ctx, hipMalloc((void**)&a->io, 8 * (qw + (size_t)a->dv.nh * a->dv.hd) * 4));
+  q.iqn = a->qparams; q.ikn = a->qparams + idx_hd; a->q = q;
+  pyre_qsa_buf_carve(q, a->cap, a->qmem, &a->qb); pyre_qsa_work_carve(q, a->cap, (uint8_t*)a->qmem + bb, &a->qw);
+  return PYRE_OK;
+}
+// Rebuilds the rotation table for a model context of ctx_tokens with a trained context of ctx_train (YaRN past it).
+int pyre_attn_set_context(pyre_ctx* ctx, pyre_attn* a, int ctx_train, int ctx_tokens) {
+  if (!ctx || !a) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_set_context: null argument");
+  if (a->len != 0) return pyre_fail(ctx, PYRE_E_STATE, "pyre_attn_set_context: the block already holds positions");
+  std::vector<float> inv(a->dv.n_rot / 2 + 1); a->dv.mscale = pyre_rope_table(a->dv.n_rot, a->rope_base, ctx_train, ctx_tokens, inv.data());
+  PYRE_HIP(ctx, hipMemcpy(a->params + 2 * a->dv.hd, inv.data(), (size_t)(a->dv.n_rot / 2) * 4, hipMemcpyHostToDevice)); return PYRE_OK;
+}
+// Harness access to the indexer: install the raw index keys of the a->len cached positions (their complete blocks are
+// pooled on the device), read keys and pooled block keys back, read the positions the last call selected for token ti
+// (*count = -1: dense).
+int pyre_attn_load_index(pyre_ctx* ctx, pyre_attn* a, const float* ik_host) {
+  if (!ctx || !a || !ik_host || a->q.nh < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_load_index: bad argument");
+  if (a->len > 0) PYRE_HIP(ctx, hipMemcpyAsync(a->qb.ik, ik_host, (size_t)a->len * a->q.hd * 4, hipMemcpyHostToDevice, ctx->stream));
+  int rc = pyre_qsa_pool_all(ctx, a->q, a->dv, a->qb, a->len); if (rc) return rc;
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
+int pyre_attn_read_index(pyre_ctx* ctx, pyre_attn* a, float* ik_host, float* ib_host) {
+  if (!ctx || !a || a->q.nh < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_read_index: bad argument");
+  const size_t hd = a->q.hd, nblk = (size_t)a->len / a->q.ratio, grp = (nblk + 63) / 64;
+  if (ik_host && a->len > 0) PYRE_HIP(ctx, hipMemcpyAsync(ik_host, a->qb.ik, (size_t)a->len * hd * 4, hipMemcpyDeviceToHost, ctx->stream));
+  std::vector<float> tmp(grp * hd * 64);
+  if (ib_host && nblk > 0) PYRE_HIP(ctx, hipMemcpyAsync(tmp.data(), a->qb.ib, tmp.size() * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  if (ib_host) for (size_t b = 0; b < nblk; ++b) for (size_t i = 0; i < hd; ++i) ib_host[b * hd + i] = tmp[qsa_ib_at(b, i, hd)];
+  return PYRE_OK;
+}
+int pyre_attn_read_selection(pyre_ctx* ctx, pyre_attn* a, int ti, int32_t* pos_host, int cap, int32_t* count) {
+  if (!ctx || !a || !count || a->q.nh < 1 || ti < 0 || ti >= 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_attn_read_selection: bad argument");
+  PYRE_HIP(ctx, hipMemcpy(count, a->qw.pcount + ti, 4, hipMemcpyDeviceToHost));
+  if (*count > 0 && pos_host) { int nrd = *count < cap ? *count : cap; PYRE_HIP(ctx, hipMemcpy(pos_host, a->qw.plist + (size_t)ti * a->qw.list_stride, (size_t)nrd * 4, hipMemcpyDeviceToHost)); }
+  return PYRE_OK;
+}
 }  // extern "C"

@@ -170,7 +170,7 @@ int pyre_gdn_prefill_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, i
                             const float* ssm_in, float* ssm_out, float* co, float* logg, float* beta, float* oraw, float* out_dev);
 
 // ---- gated attention over the KV cache (attn.hip) -----------------------------------------------------------------------
-struct AttnDev { const float* qn; const float* kn; const float* rope_inv; int nh, nkv, hd, n_rot, kv_bits, kv_recent; float eps; };
+struct AttnDev { const float* qn; const float* kn; const float* rope_inv; int nh, nkv, hd, n_rot, kv_bits, kv_recent; float eps; float mscale = 1.0f; };   // mscale: YaRN magnitude factor on cos and sin
 struct KvDev {
   // key planes are blocked by 64 positions: row r of R rows at position p sits at kv_blk(r, R, p), so the rows a wave
   // reads for its 64 positions are one contiguous range (lane = position reads stay coalesced)
@@ -197,3 +197,33 @@ void   pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w);
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
                      int* packed_done, float* out_dev, const int* posp);
 size_t pyre_packed_boundary(size_t n_visible, int kv_bits, int recent);
+// qn_ctx::rope_inv (src/qn_ctx.rs:164-185): inverse frequencies [n_rot/2]; YaRN when ctx > ctx_train > 0; returns mscale
+float pyre_rope_table(int n_rot, float base, int ctx_train, int ctx, float* inv_host);
+
+// ---- QSA sparse indexer (qsa.hip), qwen4exp_gguf.rs:1565-1599 ------------------------------------------------------------
+// Blocks of `ratio` tokens; a query that sees more than budget + ratio - 1 positions attends to the budget / ratio
+// blocks with the largest  sum_h relu(q_h . block key) / sqrt(hd)  and to the incomplete tail.
+struct QsaDev { const float* iqn; const float* ikn; int nh, hd, ratio, budget; };      // nh == 0: the layer has no indexer
+struct QsaBuf {            // per attention layer, capacity fixed with the KV cache
+  float* ik;               // [cap][hd]                 raw index keys as projected
+  float* ib;               // [cap/ratio/64][hd][64]    pooled block keys, blocked by 64 blocks (lane = block reads are coalesced)
+};
+struct QsaWork {           // per state, shared by the layers
+  float* iq;               // [8][nh][hd]   normalised, rotated index queries of the window
+  float* score;            // [8][cap/ratio]
+  int* plist;              // [8][list_stride]  attended positions, ascending
+  int* pcount;             // [8]  entries of plist in use; -1 = every visible position (dense)
+  int list_stride, max_blocks;
+};
+__host__ __device__ inline size_t qsa_ib_at(size_t b, size_t i, size_t hd) { return ((b >> 6) * hd + i) * 64 + (b & 63); }
+size_t pyre_qsa_buf_bytes(const QsaDev& q, int cap);
+void   pyre_qsa_buf_carve(const QsaDev& q, int cap, void* base, QsaBuf* b);
+size_t pyre_qsa_work_bytes(const QsaDev& q, int cap);
+void   pyre_qsa_work_carve(const QsaDev& q, int cap, void* base, QsaWork* w);
+// idx [t][..] rows hold, at column iq_off, the raw index queries [nh*hd] followed by the raw index key [hd].  Appends
+// the keys, pools the blocks the window completes, and leaves the attended positions of every token in w.plist / w.pcount.
+int pyre_qsa_launch(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaBuf& b, const QsaWork& w, const float* proj, int stride, int iq_off, int start, int t, const int* posp);
+int pyre_qsa_pool_all(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaBuf& b, int n);
+// the attention launch with an optional position list (qw == nullptr: dense)
+int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
+                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw);

@@ -196,7 +196,7 @@ long pyre_gguf_meta_arr_u64(const pyre_gguf* g, const char* key, uint64_t* out, 
 
 // Model::load (qwen4exp_gguf.rs:462-524): architecture check, configuration from the metadata, tensors by name.
 // kv_bits / kv_recent are run-time settings of the reference (qn_ctx.rs:119, PYRE_QN_KV8_RECENT), not file contents.
-int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, pyre_model** out) {
+int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, int ctx_tokens, pyre_model** out) {
   if (!ctx || !path || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_load_gguf: null argument");
   *out = nullptr; pyre_gguf* gp = nullptr; std::string e;
   int rc = gguf_open(path, &gp, &e); if (rc) return pyre_fail(ctx, rc, "pyre_model_load_gguf: %s", e.c_str());
@@ -215,6 +215,12 @@ int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_re
   c.n_exp = (int)ku("expert_count"); c.top_k = (int)ku("expert_used_count"); c.ff_exp = (int)ku("expert_feed_forward_length");
   c.lin_nk = (int)ku("ssm.group_count"); c.lin_nv = (int)ku("ssm.time_step_rank"); c.lin_dk = (int)ku("ssm.state_size"); c.lin_dv = c.lin_dk; c.conv_k = (int)ku("ssm.conv_kernel");
   c.full_every = (int)ku("full_attention_interval", 4); c.kv_bits = kv_bits; c.kv_recent = kv_recent;
+  // QSA indexer and trained context, qwen4exp_gguf.rs:481-486 (same defaults); the ratio is the largest entry of compress_ratios
+  c.idx_budget = (int)ku("attention.indexer.top_k", 2048); c.idx_nh = (int)ku("attention.indexer.head_count", 0); c.idx_hd = (int)ku("attention.indexer.key_length", 128);
+  c.idx_ratio = 4; { auto it = g->meta.find("qwen4exp.attention.compress_ratios"); if (it != g->meta.end() && it->second.kind == Meta::A && !it->second.a.empty()) { uint64_t mx = 0; for (const Meta& e2 : it->second.a) { uint64_t v = 0; if (e2.as_u64(&v) && v > mx) mx = v; } c.idx_ratio = (int)(mx > 0 ? mx : 1); } }
+  c.ctx_train = (int)ku("context_length", 262144); c.ctx = ctx_tokens > 0 ? ctx_tokens : c.ctx_train;
+  const bool has_idx = c.idx_nh > 0 && g->tensors.count("blk." + std::to_string((c.full_every > 0 ? c.full_every : 1) - 1) + ".indexer.q_proj.weight") > 0;      // :489 looks at block 3
+  if (!has_idx) c.idx_nh = 0;
   if (missing) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_load_gguf: gguf key %s", miss.c_str());
   { auto it = g->meta.find("qwen4exp.ple.layers"); if (it != g->meta.end() && it->second.kind == Meta::A && !it->second.a.empty()) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_load_gguf: per-layer-embedding (PLE) layers are not supported"); }
   auto emb = g->tensors.find("token_embd.weight");
@@ -230,7 +236,9 @@ int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_re
     const bool full = (il + 1) % (c.full_every > 0 ? c.full_every : 1) == 0;
     bool ok;
     if (full) ok = get(p + "attn_q.weight", &T[PYRE_T_ATTN_Q]) && get(p + "attn_k.weight", &T[PYRE_T_ATTN_K]) && get(p + "attn_v.weight", &T[PYRE_T_ATTN_V]) && get(p + "attn_output.weight", &T[PYRE_T_ATTN_OUTPUT]) &&
-                   get(p + "attn_q_norm.weight", &T[PYRE_T_ATTN_Q_NORM]) && get(p + "attn_k_norm.weight", &T[PYRE_T_ATTN_K_NORM]);
+                   get(p + "attn_q_norm.weight", &T[PYRE_T_ATTN_Q_NORM]) && get(p + "attn_k_norm.weight", &T[PYRE_T_ATTN_K_NORM]) &&
+                   (!has_idx || (get(p + "indexer.q_proj.weight", &T[PYRE_T_INDEXER_Q_PROJ]) && get(p + "indexer.k_proj.weight", &T[PYRE_T_INDEXER_K_PROJ]) &&
+                                 get(p + "indexer.q_norm.weight", &T[PYRE_T_INDEXER_Q_NORM]) && get(p + "indexer.k_norm.weight", &T[PYRE_T_INDEXER_K_NORM])));
     else ok = get(p + "attn_qkv.weight", &T[PYRE_T_ATTN_QKV]) && get(p + "attn_gate.weight", &T[PYRE_T_ATTN_GATE]) && get(p + "ssm_beta.weight", &T[PYRE_T_SSM_BETA]) && get(p + "ssm_alpha.weight", &T[PYRE_T_SSM_ALPHA]) &&
               get(p + "ssm_a", &T[PYRE_T_SSM_A]) && get(p + "ssm_dt.bias", &T[PYRE_T_SSM_DT_BIAS]) && get(p + "ssm_conv1d.weight", &T[PYRE_T_SSM_CONV1D]) && get(p + "ssm_norm.weight", &T[PYRE_T_SSM_NORM]) &&
               get(p + "ssm_out.weight", &T[PYRE_T_SSM_OUT]);

@@ -14,7 +14,7 @@ struct Layer {
   HcDev hca{}, hcf{};
   QMatDev proj{};            // attention: [q ; k ; v]   DeltaNet: [qkv ; z ; beta ; alpha]
   QMatDev outp{};            // attn_output / ssm_out
-  AttnDev attn{}; GdnDev gdn{}; MoeDev moe{};
+  AttnDev attn{}; GdnDev gdn{}; MoeDev moe{}; QsaDev qsa{};
   int mix_index = 0;         // index among the attention or among the DeltaNet layers
 };
 
@@ -24,6 +24,7 @@ struct pyre_model {
   pyre_ctx* ctx = nullptr; pyre_model_cfg c{};
   std::vector<Layer> layers; HcDev head{}; QMatDev embd{}, out{};
   std::vector<pyre_qmat*> owned; std::vector<void*> bufs;
+  bool has_idx = false; int iq_off = 0; float mscale = 1.0f;       // QSA indexer on every attention layer; column of the index projections in an attention row
   float* rope_inv = nullptr; int n_attn = 0, n_lin = 0, ch = 0, pw_lin = 0, pw_attn = 0;
   size_t token_weight_bytes = 0;
   // activations for a window of up to 8 tokens
@@ -40,6 +41,7 @@ struct pyre_state {
   std::vector<float*> conv[2], ssm[2]; std::vector<int> cur;     // DeltaNet double buffers
   std::vector<float*> proj_saved;                                // per DeltaNet layer [8][pw_lin]: inputs of the last window
   std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
+  std::vector<QsaBuf> qsa; QsaWork qw{};                          // indexer keys per attention layer; selection workspace
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
   std::vector<int> graph_cur;                                    // which half of every DeltaNet double buffer the captured step works on
@@ -117,9 +119,15 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   struct Guard { pyre_model* m; bool armed = true; ~Guard() { if (armed && m) { for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); } } } guard{m};
   Builder B{ctx, m};
   m->ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv; m->pw_lin = m->ch + c.lin_nv * c.lin_dv + 2 * c.lin_nv; m->pw_attn = c.n_head * 2 * c.hd + 2 * c.n_kv * c.hd;
-  std::vector<float> inv(c.n_rot / 2); for (int i = 0; i < c.n_rot / 2; ++i) inv[i] = powf(c.rope_base, -(2.0f * (float)i) / (float)c.n_rot);   // qn_ctx.rs:168
+  m->has_idx = c.idx_nh > 0 && c.full_every <= c.n_layers && lt[(size_t)(c.full_every - 1) * PYRE_LAYER_SLOTS + PYRE_T_INDEXER_Q_PROJ].data != nullptr;
+  if (m->has_idx) {
+    if (c.idx_hd < 64 || c.idx_hd % 64 || c.idx_hd > 1024 || c.idx_hd < c.n_rot || c.idx_ratio < 1 || c.idx_budget < c.idx_ratio || c.idx_budget % c.idx_ratio)
+      return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_create: indexer with %d heads of %d, block %d, budget %d is unsupported", c.idx_nh, c.idx_hd, c.idx_ratio, c.idx_budget);
+    m->iq_off = m->pw_attn; m->pw_attn += c.idx_nh * c.idx_hd + c.idx_hd;
+  }
+  std::vector<float> inv(c.n_rot / 2); const float mscale = pyre_rope_table(c.n_rot, c.rope_base, c.ctx_train, c.ctx, inv.data());   // qn_ctx.rs:164-185
   PYRE_HIP(ctx, hipMalloc((void**)&m->rope_inv, (inv.size() + 1) * 4)); m->bufs.push_back(m->rope_inv);
-  PYRE_HIP(ctx, hipMemcpy(m->rope_inv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice));
+  PYRE_HIP(ctx, hipMemcpy(m->rope_inv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice)); m->mscale = mscale;
   size_t tok_bytes = 0; int rc;
   m->layers.resize(c.n_layers);
   for (int il = 0; il < c.n_layers; ++il) {
@@ -129,14 +137,19 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
     if ((rc = B.hc(T[PYRE_T_HC_FFN_NORM], T[PYRE_T_HC_FFN_DOWN], &T[PYRE_T_HC_FFN_INJECT], T[PYRE_T_HC_FFN_UP], &L.hcf, &tok_bytes))) return rc;
     if (L.full) {
       L.mix_index = m->n_attn++;
-      const pyre_tensor* grp[3] = {&T[PYRE_T_ATTN_Q], &T[PYRE_T_ATTN_K], &T[PYRE_T_ATTN_V]};
+      const pyre_tensor* grp[5] = {&T[PYRE_T_ATTN_Q], &T[PYRE_T_ATTN_K], &T[PYRE_T_ATTN_V], &T[PYRE_T_INDEXER_Q_PROJ], &T[PYRE_T_INDEXER_K_PROJ]};
       if (grp[0]->rows != (uint64_t)c.n_head * 2 * c.hd || grp[1]->rows != (uint64_t)c.n_kv * c.hd || grp[2]->rows != (uint64_t)c.n_kv * c.hd || grp[0]->cols != (uint64_t)c.d)
         return B.fail(PYRE_E_SHAPE, "attention projection shapes");
-      if ((rc = B.cat(grp, 3, &L.proj, &tok_bytes))) return rc;
+      if (m->has_idx && (!grp[3]->data || !grp[4]->data || grp[3]->rows != (uint64_t)c.idx_nh * c.idx_hd || grp[4]->rows != (uint64_t)c.idx_hd)) return B.fail(PYRE_E_SHAPE, "indexer projection shapes (every attention layer needs them)");
+      if ((rc = B.cat(grp, m->has_idx ? 5 : 3, &L.proj, &tok_bytes))) return rc;
       if (T[PYRE_T_ATTN_OUTPUT].rows != (uint64_t)c.d || T[PYRE_T_ATTN_OUTPUT].cols != (uint64_t)c.n_head * c.hd) return B.fail(PYRE_E_SHAPE, "attn_output shape");
       if ((rc = B.one(T[PYRE_T_ATTN_OUTPUT], &L.outp, &tok_bytes))) return rc;
-      L.attn = AttnDev{nullptr, nullptr, m->rope_inv, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
+      L.attn = AttnDev{nullptr, nullptr, m->rope_inv, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps, mscale};
       if ((rc = B.vec(T[PYRE_T_ATTN_Q_NORM], c.hd, &L.attn.qn)) || (rc = B.vec(T[PYRE_T_ATTN_K_NORM], c.hd, &L.attn.kn))) return rc;
+      if (m->has_idx) {
+        L.qsa = QsaDev{nullptr, nullptr, c.idx_nh, c.idx_hd, c.idx_ratio, c.idx_budget};
+        if ((rc = B.vec(T[PYRE_T_INDEXER_Q_NORM], c.idx_hd, &L.qsa.iqn)) || (rc = B.vec(T[PYRE_T_INDEXER_K_NORM], c.idx_hd, &L.qsa.ikn))) return rc;
+      }
     } else {
       L.mix_index = m->n_lin++;
       const pyre_tensor* grp[4] = {&T[PYRE_T_ATTN_QKV], &T[PYRE_T_ATTN_GATE], &T[PYRE_T_SSM_BETA], &T[PYRE_T_SSM_ALPHA]};
@@ -199,13 +212,16 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   size_t cs = al256((size_t)(c.conv_k - 1) * m->ch * 4), ss = al256((size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4), ps = al256((size_t)8 * m->pw_lin * 4);
   AttnDev a0{nullptr, nullptr, nullptr, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
   size_t kvb = al256(pyre_kv_bytes(a0, s->cap)), awb = al256(pyre_attn_work_bytes(a0, s->cap));
-  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * kvb + awb + 4096 + 256;
+  QsaDev q0{nullptr, nullptr, m->has_idx ? c.idx_nh : 0, c.idx_hd, c.idx_ratio < 1 ? 1 : c.idx_ratio, c.idx_budget};
+  size_t qbb = al256(pyre_qsa_buf_bytes(q0, s->cap)), qwb = al256(pyre_qsa_work_bytes(q0, s->cap));
+  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * (kvb + qbb) + awb + qwb + 4096 + 256;
   hipError_t e = hipMalloc(&s->mem, total);
   if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_create: hipMalloc(%zu): %s", total, hipGetErrorString(e));
   uint8_t* p = (uint8_t*)s->mem; auto take = [&](size_t n) { void* r = p; p += n; return r; };
   for (int li = 0; li < m->n_lin; ++li) { for (int b = 0; b < 2; ++b) { s->conv[b].push_back((float*)take(cs)); s->ssm[b].push_back((float*)take(ss)); } s->proj_saved.push_back((float*)take(ps)); s->cur.push_back(0); }
   for (int ai = 0; ai < m->n_attn; ++ai) { KvDev kv; pyre_kv_carve(a0, s->cap, take(kvb), &kv); s->kv.push_back(kv); s->packed.push_back(0); }
   pyre_attn_work_carve(a0, s->cap, take(awb), &s->aw);
+  if (m->has_idx) { for (int ai = 0; ai < m->n_attn; ++ai) { QsaBuf qb; pyre_qsa_buf_carve(q0, s->cap, take(qbb), &qb); s->qsa.push_back(qb); } pyre_qsa_work_carve(q0, s->cap, take(qwb), &s->qw); }
   s->step_dev = (int*)take(256);
   int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
   *out = S.release(); return PYRE_OK;
@@ -228,14 +244,15 @@ int pyre_model_max_window(const pyre_model* m) { return m ? 8 : 0; }
 // whatever the capacity).  It can be restored into any state of the same model with room for `len` positions.
 struct pyre_snap { const pyre_model* m; int len; std::vector<int> packed; void* mem; size_t bytes; };
 namespace {
-struct SnapPlan { size_t cs, ss, kf, ks_kq, kq, ksc, vf, vq, vsc, total; };
+struct SnapPlan { size_t cs, ss, kf, ks_kq, kq, ksc, vf, vq, vsc, ik, ib, total; };
 SnapPlan snap_plan(const pyre_model* m, int len) {
   const pyre_model_cfg& c = m->c; SnapPlan p{};
   const size_t row = (size_t)c.n_kv * c.hd, nb = ((size_t)len + 63) / 64;
   p.cs = al256((size_t)(c.conv_k - 1) * m->ch * 4); p.ss = al256((size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4);
   p.kf = al256(nb * row * 64 * 4); p.kq = al256(nb * (row / 8) * 64 * 4); p.ksc = al256(nb * (row / 32) * 64 * 4);
   p.vf = al256((size_t)len * row * 4); p.vq = al256((size_t)len * (row / 8) * 4); p.vsc = al256((size_t)len * (row / 32) * 4);
-  p.total = (size_t)m->n_lin * (p.cs + p.ss) + (size_t)m->n_attn * (p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc) + 256;
+  if (m->has_idx) { p.ik = al256((size_t)len * c.idx_hd * 4); p.ib = al256(((size_t)len / c.idx_ratio + 63) / 64 * 64 * c.idx_hd * 4); }      // raw index keys; pooled block keys in whole groups of 64 blocks
+  p.total = (size_t)m->n_lin * (p.cs + p.ss) + (size_t)m->n_attn * (p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc + p.ik + p.ib) + 256;
   return p;
 }
 // dir = 0: state -> snapshot buffer, 1: snapshot buffer -> state
@@ -254,6 +271,13 @@ int snap_copy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint8_t* buf, i
       PYRE_HIP(ctx, cp(kv.kf, nb * row * 64 * 4)); q += p.kf; PYRE_HIP(ctx, cp(kv.kq, nb * (row / 8) * 64 * 4)); q += p.kq; PYRE_HIP(ctx, cp(kv.ks, nb * (row / 32) * 64 * 4)); q += p.ksc;
       PYRE_HIP(ctx, cp(kv.vf, (size_t)len * row * 4)); q += p.vf; PYRE_HIP(ctx, cp(kv.vq, (size_t)len * (row / 8) * 4)); q += p.vq; PYRE_HIP(ctx, cp(kv.vs, (size_t)len * (row / 32) * 4)); q += p.vsc;
     } else q += p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc;
+    if (m->has_idx) {
+      if (len > 0) { PYRE_HIP(ctx, cp(s->qsa[ai].ik, (size_t)len * c.idx_hd * 4)); }
+      q += p.ik;
+      size_t ibn = ((size_t)len / c.idx_ratio + 63) / 64 * 64 * c.idx_hd * 4;
+      if (ibn) { PYRE_HIP(ctx, cp(s->qsa[ai].ib, ibn)); }
+      q += p.ib;
+    }
   }
   return PYRE_OK;
 }
@@ -329,7 +353,8 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
-      if ((rc = pyre_attn_launch(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev))) return rc;
+      if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], s->qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
+      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &s->qw : nullptr))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
@@ -363,6 +388,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
 // Usable when every matrix but the router is IQ3_S, the router is bf16, and the shapes fit the kernel's stages; anything
 // else keeps the launch-per-stage path.
 bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
+  if (m->has_idx || m->mscale != 1.0f) return false;        // the persistent kernel has neither the indexer nor the YaRN factor
   if (m->mega_ok >= 0) return m->mega_ok == 1;
   m->mega_ok = 0;
   const pyre_model_cfg& c = m->c;

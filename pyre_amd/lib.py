@@ -57,7 +57,7 @@ def _declare(L):
         "pyre_gguf_meta_f64": (i32, [vp, C.c_char_p, vp]),
         "pyre_gguf_meta_str": (i32, [vp, C.c_char_p, C.c_char_p, C.c_size_t]),
         "pyre_gguf_meta_arr_u64": (C.c_long, [vp, C.c_char_p, vp, C.c_size_t]),
-        "pyre_model_load_gguf": (i32, [vp, C.c_char_p, i32, i32, vp]),
+        "pyre_model_load_gguf": (i32, [vp, C.c_char_p, i32, i32, i32, vp]),
         "pyre_state_capacity": (i32, [vp]),
         "pyre_model_max_window": (i32, [vp]),
         "pyre_state_snapshot": (i32, [vp, vp, vp]),
@@ -84,6 +84,11 @@ def _declare(L):
         "pyre_attn_decode_kv4": (i32, [vp, vp, vp, i32, vp]),
         "pyre_attn_load_cache": (i32, [vp, vp, vp, vp, i32]),
         "pyre_attn_read_cache": (i32, [vp, vp, vp, vp]),
+        "pyre_attn_set_indexer": (i32, [vp, vp, i32, i32, i32, i32, vp, vp]),
+        "pyre_attn_set_context": (i32, [vp, vp, i32, i32]),
+        "pyre_attn_load_index": (i32, [vp, vp, vp]),
+        "pyre_attn_read_index": (i32, [vp, vp, vp, vp]),
+        "pyre_attn_read_selection": (i32, [vp, vp, i32, vp, i32, vp]),
         "pyre_model_create": (i32, [vp, vp, vp, vp, C.POINTER(vp)]),
         "pyre_model_destroy": (None, [vp]),
         "pyre_model_weight_bytes_per_token": (sz, [vp]),
@@ -385,8 +390,35 @@ class Attn:
         self.ctx.check(self.ctx.L.pyre_attn_read_cache(self.ctx.h, self.h, _ptr(k), _ptr(v)), "attn_read_cache")
         return k, v
 
-    def decode(self, q, k, v):
-        qkv = np.ascontiguousarray(np.concatenate([q, k, v], axis=1), dtype=np.float32)
+    def set_indexer(self, idx_nh, idx_hd, idx_ratio, idx_budget, iqn, ikn):
+        """QSA sparse indexer (qwen4exp_gguf.rs:1565-1599); decode() then also takes the raw index projections."""
+        iqn = np.ascontiguousarray(iqn, dtype=np.float32); ikn = np.ascontiguousarray(ikn, dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_attn_set_indexer(self.ctx.h, self.h, idx_nh, idx_hd, idx_ratio, idx_budget, _ptr(iqn), _ptr(ikn)), "attn_set_indexer")
+        self.idx = (idx_nh, idx_hd, idx_ratio, idx_budget)
+
+    def set_context(self, ctx_train, ctx_tokens):
+        self.ctx.check(self.ctx.L.pyre_attn_set_context(self.ctx.h, self.h, ctx_train, ctx_tokens), "attn_set_context")
+
+    def load_index(self, ik):
+        ik = np.ascontiguousarray(ik, dtype=np.float32); assert ik.shape[0] == len(self)
+        self.ctx.check(self.ctx.L.pyre_attn_load_index(self.ctx.h, self.h, _ptr(ik)), "attn_load_index")
+
+    def read_index(self):
+        nh, hd, ratio, _ = self.idx; n = len(self)
+        ik = np.empty((n, hd), dtype=np.float32); ib = np.empty((n // ratio, hd), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_attn_read_index(self.ctx.h, self.h, _ptr(ik), _ptr(ib)), "attn_read_index")
+        return ik, ib
+
+    def selection(self, ti):
+        """Positions the last decode call attended to for its token ti (None: every visible position)."""
+        _, _, ratio, budget = self.idx
+        pos = np.empty(budget + 2 * ratio + 4, dtype=np.int32); cnt = C.c_int32()
+        self.ctx.check(self.ctx.L.pyre_attn_read_selection(self.ctx.h, self.h, ti, _ptr(pos), pos.size, C.byref(cnt)), "attn_read_selection")
+        return None if cnt.value < 0 else pos[:cnt.value].copy()
+
+    def decode(self, q, k, v, iq=None, ik=None):
+        parts = [q, k, v] + ([iq, ik] if iq is not None else [])
+        qkv = np.ascontiguousarray(np.concatenate(parts, axis=1), dtype=np.float32)
         t = qkv.shape[0]
         out = np.empty((t, self.nh * self.hd), dtype=np.float32)
         self.ctx.check(self.ctx.L.pyre_attn_decode_kv4(self.ctx.h, self.h, _ptr(qkv), t, _ptr(out)), "attn_decode_kv4")
@@ -485,10 +517,10 @@ class ModelCfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
                [("rope_base", C.c_float), ("eps", C.c_float)] + \
                [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
-                                         "full_every", "vocab", "kv_bits", "kv_recent")]
+                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")]
 
 
-LAYER_SLOTS, GLOBAL_SLOTS = 31, 5
+LAYER_SLOTS, GLOBAL_SLOTS = 35, 5
 
 
 class Model:
@@ -519,12 +551,12 @@ class Model:
         self.vocab = self.cfg.vocab
 
     @classmethod
-    def from_gguf(cls, ctx, path, kv_bits=4, kv_recent=1024):
+    def from_gguf(cls, ctx, path, kv_bits=4, kv_recent=1024, ctx_tokens=0):
         """Model::load: configuration and tensors straight from a qwen4exp GGUF file (or its shards)."""
         self = cls.__new__(cls)
         self.ctx = ctx
         h = C.c_void_p()
-        ctx.check(ctx.L.pyre_model_load_gguf(ctx.h, os.fsencode(path), kv_bits, kv_recent, C.byref(h)), "model_load_gguf")
+        ctx.check(ctx.L.pyre_model_load_gguf(ctx.h, os.fsencode(path), kv_bits, kv_recent, ctx_tokens, C.byref(h)), "model_load_gguf")
         self.h = h
         g = Gguf(path); a = "qwen4exp."
         c = ModelCfg()
@@ -536,6 +568,13 @@ class Model:
         c.full_every = g.u64(a + "full_attention_interval", 4)
         c.rope_base = g.f64(a + "rope.freq_base"); c.eps = g.f64(a + "attention.layer_norm_rms_epsilon")
         c.vocab = g.tensor("token_embd.weight")[3][1]; c.kv_bits = kv_bits; c.kv_recent = kv_recent
+        c.idx_budget = g.u64(a + "attention.indexer.top_k", 2048); c.idx_hd = g.u64(a + "attention.indexer.key_length", 128)
+        c.idx_nh = g.u64(a + "attention.indexer.head_count", 0) if g.has("blk.%d.indexer.q_proj.weight" % (c.full_every - 1)) else 0
+        try:
+            c.idx_ratio = max(max(g.arr_u64(a + "attention.compress_ratios") or [4]), 1)
+        except KeyError:
+            c.idx_ratio = 4
+        c.ctx_train = g.u64(a + "context_length", 262144); c.ctx = ctx_tokens or c.ctx_train
         g.close()
         self.cfg = c; self.vocab = c.vocab
         return self

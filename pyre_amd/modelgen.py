@@ -12,11 +12,12 @@ from . import synth
 
 (HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
  ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
- UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, LAYER_SLOTS) = range(32)
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN, LAYER_SLOTS) = range(36)
 G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
 
 CFG_FIELDS = ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot", "rope_base", "eps", "n_exp", "top_k",
-              "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k", "full_every", "vocab", "kv_bits", "kv_recent")
+              "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k", "full_every", "vocab", "kv_bits", "kv_recent",
+              "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")
 
 
 @dataclass
@@ -43,6 +44,12 @@ class Config:
     vocab: int = 512
     kv_bits: int = 4
     kv_recent: int = 1024
+    idx_nh: int = 0                   # QSA sparse indexer heads (0 = no indexer), key length, block size, token budget
+    idx_hd: int = 128
+    idx_ratio: int = 4
+    idx_budget: int = 2048
+    ctx_train: int = 0                # trained context and the context the model is built for (ctx > ctx_train > 0: YaRN)
+    ctx: int = 0
     # generation knobs (not part of the model contract)
     qtype: int = synth.IQ3_S          # type of every projection / expert / embedding / head matrix
     hc_type: int = synth.BF16         # type of the hyper-connection matrices (BF16 in real files)
@@ -87,6 +94,9 @@ def tensor_specs(c: Config):
             out += [(il, ATTN_Q, "q", c.qtype, c.n_head * 2 * c.hd, c.d), (il, ATTN_K, "q", c.qtype, c.n_kv * c.hd, c.d),
                     (il, ATTN_V, "q", c.qtype, c.n_kv * c.hd, c.d), (il, ATTN_O, "q", c.qtype, c.d, c.n_head * c.hd),
                     (il, ATTN_QN, "vec:norm1", synth.F32, 1, c.hd), (il, ATTN_KN, "vec:norm1", synth.F32, 1, c.hd)]
+            if c.idx_nh > 0:
+                out += [(il, IDX_Q, "q", c.qtype, c.idx_nh * c.idx_hd, c.d), (il, IDX_K, "q", c.qtype, c.idx_hd, c.d),
+                        (il, IDX_QN, "vec:norm1", synth.F32, 1, c.idx_hd), (il, IDX_KN, "vec:norm1", synth.F32, 1, c.idx_hd)]
         else:
             out += [(il, LIN_QKV, "q", c.qtype, c.ch, c.d), (il, LIN_Z, "q", c.qtype, c.lin_nv * c.lin_dv, c.d),
                     (il, LIN_BETA, "q", c.qtype, c.lin_nv, c.d), (il, LIN_ALPHA, "q", c.qtype, c.lin_nv, c.d),

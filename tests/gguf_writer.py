@@ -59,6 +59,7 @@ LAYER_NAMES = {
     mg.LIN_CONV: "ssm_conv1d.weight", mg.LIN_NORM: "ssm_norm.weight", mg.LIN_OUT: "ssm_out.weight",
     mg.ROUTER: "ffn_gate_inp.weight", mg.GATE_E: "ffn_gate_exps.weight", mg.UP_E: "ffn_up_exps.weight", mg.DOWN_E: "ffn_down_exps.weight",
     mg.SH_GATE_INP: "ffn_gate_inp_shexp.weight", mg.SH_GATE: "ffn_gate_shexp.weight", mg.SH_UP: "ffn_up_shexp.weight", mg.SH_DOWN: "ffn_down_shexp.weight",
+    mg.IDX_Q: "indexer.q_proj.weight", mg.IDX_K: "indexer.k_proj.weight", mg.IDX_QN: "indexer.q_norm.weight", mg.IDX_KN: "indexer.k_norm.weight",
 }
 GLOBAL_NAMES = {mg.G_EMBD: "token_embd.weight", mg.G_HEAD_NORM: "output_hc_norm.weight", mg.G_HEAD_DOWN: "output_hc_down.weight", mg.G_HEAD_UP: "output_hc_up.weight", mg.G_OUT: "output.weight"}
 
@@ -71,7 +72,9 @@ def model_meta(c):
             (a + "rope.freq_base", F32, c.rope_base), (a + "attention.layer_norm_rms_epsilon", F32, c.eps), (a + "expert_count", U32, c.n_exp),
             (a + "expert_used_count", U32, c.top_k), (a + "expert_feed_forward_length", U32, c.ff_exp), (a + "ssm.group_count", U32, c.lin_nk),
             (a + "ssm.time_step_rank", U64, c.lin_nv), (a + "ssm.state_size", I32, c.lin_dk), (a + "ssm.conv_kernel", U16, c.conv_k),
-            (a + "full_attention_interval", U8, c.full_every), (a + "context_length", U32, 262144), ("tokenizer.ggml.tokens", ARR, (STR, ["a", "b"]))]
+            (a + "full_attention_interval", U8, c.full_every), (a + "context_length", U32, c.ctx_train or 262144), ("tokenizer.ggml.tokens", ARR, (STR, ["a", "b"]))] + \
+           ([(a + "attention.indexer.head_count", U32, c.idx_nh), (a + "attention.indexer.key_length", U32, c.idx_hd), (a + "attention.indexer.top_k", U32, c.idx_budget),
+             (a + "attention.compress_ratios", ARR, (U32, [1, c.idx_ratio, 2] if c.idx_ratio > 2 else [c.idx_ratio]))] if c.idx_nh > 0 else [])
 
 
 def model_tensors(c, hw):

@@ -42,13 +42,14 @@ def dense(entry):
 def np_forward_tokens(hw, ids):
     """float64 numpy statement of the token loop (one token at a time); returns logits after each token."""
     c = hw.cfg; d, hc = c.d, c.hc
-    inv = (np.float64(np.float32(c.rope_base)) ** (-2.0 * np.arange(c.n_rot // 2) / c.n_rot))
+    inv, ms = np_ref.yarn_inv(c.n_rot, c.rope_base, c.ctx_train, c.ctx)
     L = [{s: (dense(e) if e[0] != 0 or e[1] > 1 else e[3].view(np.float32).astype(np.float64)) for s, e in lay.items()} for lay in hw.layers]
     G = {s: (dense(e) if e[1] > 1 else e[3].view(np.float32).astype(np.float64)) for s, e in hw.globals_.items()}
-    conv = {}; S = {}; K = {}; V = {}
+    conv = {}; S = {}; K = {}; V = {}; IK = {}; IB = {}
     for il in range(c.n_layers):
         if c.full(il):
             K[il] = np.zeros((0, c.n_kv * c.hd), np.float32); V[il] = np.zeros((0, c.n_kv * c.hd), np.float32)
+            IK[il] = np.zeros((0, c.idx_hd)); IB[il] = np.zeros((0, c.idx_hd))
         else:
             conv[il] = np.zeros((c.conv_k - 1, c.ch)); S[il] = np.zeros((c.lin_nv, c.lin_dk, c.lin_dv))
     out = []
@@ -60,8 +61,17 @@ def np_forward_tokens(hw, ids):
             if c.full(il):
                 n = pos + 1
                 pb = orc.packed_boundary(n, c.kv_bits, c.kv_recent)
+                positions = None
+                if c.idx_nh > 0 and mg.IDX_Q in W:
+                    IK[il] = np.concatenate([IK[il], (W[mg.IDX_K] @ m)[None]])
+                    if n % c.idx_ratio == 0:
+                        b = n // c.idx_ratio - 1
+                        IB[il] = np.concatenate([IB[il], np_ref.qsa_pool(IK[il][b * c.idx_ratio:n], W[mg.IDX_KN], c.eps, b * c.idx_ratio, c.n_rot, inv, ms)[None]])
+                    iq = (W[mg.IDX_Q] @ m).reshape(c.idx_nh, c.idx_hd)
+                    iq = np.stack([np_ref.rope(np_ref.rms(iq[h], W[mg.IDX_QN], c.eps), pos, c.n_rot, inv, ms) for h in range(c.idx_nh)])
+                    positions = np_ref.qsa_select(iq, IB[il], n, c.idx_ratio, c.idx_budget)
                 o, kr, vr = np_ref.attn_step(c.n_head, c.n_kv, c.hd, c.n_rot, c.eps, inv, W[mg.ATTN_QN], W[mg.ATTN_KN],
-                                             W[mg.ATTN_Q] @ m, W[mg.ATTN_K] @ m, W[mg.ATTN_V] @ m, pos, K[il], V[il], pb)
+                                             W[mg.ATTN_Q] @ m, W[mg.ATTN_K] @ m, W[mg.ATTN_V] @ m, pos, K[il], V[il], pb, positions=positions, mscale=ms)
                 K[il] = np.concatenate([K[il], kr[None]]); V[il] = np.concatenate([V[il], vr[None]])
                 o = W[mg.ATTN_O] @ o
             else:

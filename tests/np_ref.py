@@ -309,19 +309,51 @@ def gdn_step(nk, nv, dk, dv, conv_k, eps, a, dt, conv_w, norm_w, qkv, z, beta, a
     return out.reshape(-1), win[1:], S
 
 
-def rope(v, pos, n_rot, inv):
+def rope(v, pos, n_rot, inv, mscale=1.0):
     v = np.array(v, dtype=np.float64); half = n_rot // 2
     ang = (np.float32(pos) * np.asarray(inv, dtype=np.float32)).astype(np.float64)   # the angle itself is an f32 product (qwen4exp_gguf.rs:530)
-    c, s = np.cos(ang), np.sin(ang)
+    c, s = np.cos(ang) * mscale, np.sin(ang) * mscale
     x0, x1 = v[..., :half].copy(), v[..., half:n_rot].copy()
     v[..., :half] = x0 * c - x1 * s
     v[..., half:n_rot] = x1 * c + x0 * s
     return v
 
 
-def attn_step(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, pos, K, V, packed_below=0):
-    """One token at position pos, float64. K,V [pos, nkv*hd] caches (f32 content). Returns (out, k_row, v_row)."""
-    k = rope(rms(np.asarray(k, dtype=np.float64).reshape(nkv, hd), np.asarray(kn, dtype=np.float64), eps), pos, n_rot, inv)
+def yarn_inv(n_rot, base, ctx_train, ctx):
+    """float64 statement of the YaRN frequency table (llama.cpp / transformers defaults: beta_fast 32, beta_slow 1):
+    (inverse frequencies, magnitude factor)."""
+    i = np.arange(n_rot // 2, dtype=np.float64)
+    plain = np.float64(np.float32(base)) ** (-2.0 * i / n_rot)
+    if not (ctx_train > 0 and ctx > ctx_train):
+        return plain, 1.0
+    scale = ctx / ctx_train
+    corr = lambda rot: n_rot * np.log(ctx_train / (rot * 2 * np.pi)) / (2 * np.log(base))
+    low = max(np.floor(corr(32.0)), 0.0); high = min(np.ceil(corr(1.0)), n_rot // 2 - 1)
+    ramp = np.ones_like(i) if abs(high - low) < 1e-6 else np.clip((i - low) / (high - low), 0.0, 1.0)
+    return plain / scale * (1 - ramp) + plain * ramp, 1.0 + 0.1 * np.log(scale)
+
+
+def qsa_select(iq, ib, n, ratio, budget):
+    """Positions a query with n visible tokens attends to (ascending), or None while dense.  iq [nh][ihd] normalised and
+    rotated index queries, ib [n // ratio][ihd] pooled block keys (float64).  Blocks ordered by (score desc, index asc)."""
+    if n <= budget + ratio - 1:
+        return None
+    nb = n // ratio
+    sc = np.maximum(ib[:nb] @ iq.T, 0.0).sum(1) / np.sqrt(iq.shape[1])
+    order = sorted(range(nb), key=lambda b: (-sc[b], b))[:budget // ratio]
+    pos = [p for b in sorted(order) for p in range(b * ratio, (b + 1) * ratio)] + list(range(nb * ratio, n))
+    return np.array(pos, dtype=np.int64)
+
+
+def qsa_pool(ik_rows, ikn, eps, first_pos, n_rot, inv, mscale=1.0):
+    """Block key: mean of the block's raw index keys, RMSNorm, RoPE at the block's first position."""
+    return rope(rms(np.asarray(ik_rows, dtype=np.float64).mean(0), np.asarray(ikn, dtype=np.float64), eps), first_pos, n_rot, inv, mscale)
+
+
+def attn_step(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, pos, K, V, packed_below=0, positions=None, mscale=1.0):
+    """One token at position pos, float64. K,V [pos, nkv*hd] caches (f32 content). Returns (out, k_row, v_row).
+    positions: the attended subset (ascending), default every visible position."""
+    k = rope(rms(np.asarray(k, dtype=np.float64).reshape(nkv, hd), np.asarray(kn, dtype=np.float64), eps), pos, n_rot, inv, mscale)
     Kf = np.concatenate([np.asarray(K, dtype=np.float64).reshape(pos, nkv * hd), k.reshape(1, -1)], axis=0)
     Vf = np.concatenate([np.asarray(V, dtype=np.float64).reshape(pos, nkv * hd), np.asarray(v, dtype=np.float64).reshape(1, -1)], axis=0)
     Ke, Ve = Kf.copy(), Vf.copy()
@@ -331,11 +363,12 @@ def attn_step(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, pos, K, V, packed_b
     q = np.asarray(q, dtype=np.float64).reshape(nh, 2 * hd)
     out = np.empty((nh, hd)); grp = nh // nkv
     for h in range(nh):
-        qh = rope(rms(q[h, :hd], np.asarray(qn, dtype=np.float64), eps), pos, n_rot, inv)
+        qh = rope(rms(q[h, :hd], np.asarray(qn, dtype=np.float64), eps), pos, n_rot, inv, mscale)
         kvh = h // grp
-        sc = Ke[:, kvh * hd:(kvh + 1) * hd] @ qh / np.sqrt(hd)
+        Ks, Vs = (Ke, Ve) if positions is None else (Ke[positions], Ve[positions])
+        sc = Ks[:, kvh * hd:(kvh + 1) * hd] @ qh / np.sqrt(hd)
         w = np.exp(sc - sc.max()); w /= w.sum()
-        out[h] = (w[:, None] * Ve[:, kvh * hd:(kvh + 1) * hd]).sum(0) * sigm(q[h, hd:])
+        out[h] = (w[:, None] * Vs[:, kvh * hd:(kvh + 1) * hd]).sum(0) * sigm(q[h, hd:])
     return out.reshape(-1), Kf[-1].astype(np.float32), Vf[-1].astype(np.float32)
 
 

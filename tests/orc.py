@@ -12,7 +12,7 @@ F32, F16, Q8_0, Q4_K, IQ2_XS, IQ3_S, BF16 = 0, 1, 8, 12, 17, 21, 30
 Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS = 2, 6, 14, 16, 18, 20, 22, 23
 (HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
  ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
- UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, LAYER_SLOTS) = range(32)
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN, LAYER_SLOTS) = range(36)
 G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
 
 
@@ -24,7 +24,7 @@ class Cfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
                [("rope_base", C.c_float), ("eps", C.c_float)] + \
                [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
-                                         "full_every", "vocab", "kv_bits", "kv_recent")]
+                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")]
 
 
 def build():
@@ -51,7 +51,8 @@ def lib():
             getattr(L, n).argtypes = [C.c_float]
         L.orc_model_create.restype = C.c_void_p
         L.orc_state_create.restype = C.c_void_p
-        for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v"):
+        L.orc_rope_inv_yarn.restype = C.c_float
+        for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v", "orc_state_ik", "orc_state_ib"):
             getattr(L, n).restype = C.POINTER(C.c_float)
         _lib = L
     return _lib
@@ -159,6 +160,26 @@ def attn_core(nh, nkv, hd, n_rot, eps, inv, qn, kn, q, k, v, start, kv_bits, kv_
     return out
 
 
+def rope_inv_yarn(n_rot, base, ctx_train, ctx):
+    inv = np.empty(n_rot // 2, dtype=np.float32)
+    ms = lib().orc_rope_inv_yarn(C.c_int(n_rot), C.c_float(base), C.c_int(ctx_train), C.c_int(ctx), _p(inv))
+    return inv, float(ms)
+
+
+def attn_core_qsa(nh, nkv, hd, n_rot, eps, inv, mscale, qn, kn, q, k, v, start, kv_bits, kv_recent, kc, vc,
+                  idx_nh, idx_hd, idx_ratio, idx_budget, iqn, ikn, iq, ik, ikc, ibc):
+    """Returns (out [t][nh*hd], [positions or None per token]); the caches kc, vc, ikc, ibc are updated in place."""
+    q = f32(q); t = q.shape[0]
+    k, v, qn, kn, inv, iqn, ikn, iq, ik = (f32(a) for a in (k, v, qn, kn, inv, iqn, ikn, iq, ik))
+    out = np.empty((t, nh * hd), dtype=np.float32)
+    stride = idx_budget + 2 * idx_ratio
+    sel = np.zeros((t, stride), dtype=np.int32); sel_n = np.zeros(t, dtype=np.int32)
+    lib().orc_attn_core_qsa(nh, nkv, hd, n_rot, C.c_float(eps), _p(inv), C.c_float(mscale), _p(qn), _p(kn), _p(q), _p(k), _p(v), C.c_int(start), C.c_int(t),
+                            C.c_int(kv_bits), C.c_int(kv_recent), _p(kc), _p(vc), C.c_int(idx_nh), C.c_int(idx_hd), C.c_int(idx_ratio), C.c_int(idx_budget),
+                            _p(iqn), _p(ikn), _p(iq), _p(ik), _p(ikc), _p(ibc), _p(out), _p(sel), _p(sel_n), C.c_int(stride))
+    return out, [None if sel_n[i] < 0 else sel[i, :sel_n[i]].copy() for i in range(t)]
+
+
 def moe_ffn(d, n_exp, k, ff, router, gate_e, up_e, down_e, sh_gate_inp, sh_gate, sh_up, sh_down, x, threads=4):
     x = f32(x).reshape(-1, d); t = x.shape[0]
     y = np.empty((t, d), dtype=np.float32)
@@ -261,6 +282,13 @@ class State:
     def vcache(self, ai):
         c = self.m.cfg
         return np.ctypeslib.as_array(lib().orc_state_v(self.h, ai), shape=(len(self) * c.n_kv * c.hd,))
+
+    def ikeys(self, ai):
+        return np.ctypeslib.as_array(lib().orc_state_ik(self.h, ai), shape=(len(self) * self.m.cfg.idx_hd,))
+
+    def iblocks(self, ai):
+        c = self.m.cfg
+        return np.ctypeslib.as_array(lib().orc_state_ib(self.h, ai), shape=((len(self) // max(c.idx_ratio, 1)) * c.idx_hd,))
 
     def __del__(self):
         if getattr(self, "h", None):

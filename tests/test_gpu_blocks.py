@@ -3,6 +3,7 @@ against the CPU oracle, through the C ABI.  Tolerance 1e-5 on max|d| / max|ref| 
 import numpy as np
 import pytest
 
+import np_ref
 import orc
 from helpers import orc_tensor, relerr
 from pyre_amd import lib, synth
@@ -192,6 +193,108 @@ def test_attention_closed_forms(ctx):
     for h in (0, 9, 15):
         gate = p["q"][0].reshape(nh, 512)[h, 256:].astype(np.float64)
         assert relerr(out[0].reshape(nh, 256)[h], allv[h // 8] / (1 + np.exp(-gate))) < 1e-5
+
+
+# ---- QSA sparse indexer + YaRN ------------------------------------------------------------------------------------------------
+INH, IHD, IR, IBUD = 3, 128, 4, 64          # dense up to 67 visible positions
+
+
+def qsa_inputs(nh, nkv, seed, t):
+    g = lambda s, shape, std=1.0: synth.normal(shape, seed * 100 + s, std)
+    p = attn_inputs(nh, nkv, seed, t)
+    p.update(iq=g(11, (t, INH * IHD)), ik=g(12, (t, IHD)), iqn=1 + g(13, (IHD,), 0.1), ikn=1 + g(14, (IHD,), 0.1))
+    return p
+
+
+def pooled(ik, ikn, inv, mscale=1.0):
+    nb = ik.shape[0] // IR
+    return np.stack([np_ref.qsa_pool(ik[b * IR:(b + 1) * IR], ikn, 1e-6, b * IR, 64, inv, mscale) for b in range(nb)]).astype(np.float32) if nb else np.zeros((0, IHD), np.float32)
+
+
+@pytest.mark.parametrize("kv_bits,recent,start,t", [(0, 1024, 150, 5), (4, 64, 300, 8), (0, 1024, 64, 6), (4, 64, 1000, 3), (0, 1024, 20, 8)])
+def test_qsa_attention_selection_and_output_match_oracle(ctx, kv_bits, recent, start, t):
+    nh, nkv = 16, 2
+    row = nkv * 256
+    p = qsa_inputs(nh, nkv, 7 + start, t)
+    kc = synth.normal((start, row), 6); vc = synth.normal((start, row), 7); ikc = synth.normal((start, IHD), 8)
+    inv = orc.rope_inv(64, 1e7)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], kv_bits, recent, start + 16)
+    att.set_indexer(INH, IHD, IR, IBUD, p["iqn"], p["ikn"])
+    att.load_cache(kc, vc); att.load_index(ikc)
+    ik0, ib0 = att.read_index()
+    ibc = pooled(ikc, p["ikn"], inv)
+    assert np.array_equal(ik0, ikc) and relerr(ib0, ibc) <= 1e-6 and ib0.shape == (start // IR, IHD)
+    out = att.decode(p["q"], p["k"], p["v"], p["iq"], p["ik"])
+    K = np.zeros((start + t, row), np.float32); V = np.zeros_like(K); K[:start] = kc; V[:start] = vc
+    IK = np.zeros((start + t, IHD), np.float32); IK[:start] = ikc
+    IB = np.zeros(((start + t) // IR, IHD), np.float32); IB[:start // IR] = ib0          # the device's own pooled keys: same selection inputs on both sides
+    ref, sel = orc.attn_core_qsa(nh, nkv, 256, 64, 1e-6, inv, 1.0, p["qn"], p["kn"], p["q"], p["k"], p["v"], start, kv_bits, recent, K, V,
+                                 INH, IHD, IR, IBUD, p["iqn"], p["ikn"], p["iq"], p["ik"], IK, IB)
+    for ti in range(t):
+        got = att.selection(ti)
+        if sel[ti] is None:
+            assert got is None, ti
+        else:
+            assert got is not None and np.array_equal(got, sel[ti]), ti
+    assert relerr(out, ref) <= 2e-5
+    ik2, ib2 = att.read_index()
+    assert np.array_equal(ik2, IK) and relerr(ib2, IB) <= 1e-6
+    if start + t > IBUD + IR - 1:
+        assert sel[t - 1] is not None and len(sel[t - 1]) == IBUD + (start + t) % IR
+
+
+def test_qsa_growth_from_empty_crosses_dense_limit_and_packing_boundary(ctx):
+    nh, nkv, recent = 4, 2, 64
+    row = nkv * 256; N = 200
+    p = qsa_inputs(nh, nkv, 19, N)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, recent, 256)
+    att.set_indexer(INH, IHD, IR, IBUD, p["iqn"], p["ikn"])
+    K = np.zeros((N, row), np.float32); V = np.zeros_like(K); IK = np.zeros((N, IHD), np.float32); IB = np.zeros((N // IR, IHD), np.float32)
+    inv = orc.rope_inv(64, 1e7)
+    worst = 0.0; i = 0; sparse_seen = 0
+    for t in [1] * 75 + [8] * 10 + [3, 5, 7, 1, 1, 1, 2, 8, 8, 8, 1]:
+        sl = slice(i, i + t)
+        out = att.decode(p["q"][sl], p["k"][sl], p["v"][sl], p["iq"][sl], p["ik"][sl])
+        ref, sel = orc.attn_core_qsa(nh, nkv, 256, 64, 1e-6, inv, 1.0, p["qn"], p["kn"], p["q"][sl], p["k"][sl], p["v"][sl], i, 4, recent, K, V,
+                                     INH, IHD, IR, IBUD, p["iqn"], p["ikn"], p["iq"][sl], p["ik"][sl], IK, IB)
+        for ti in range(t):
+            got = att.selection(ti)
+            assert (got is None) == (sel[ti] is None) and (got is None or np.array_equal(got, sel[ti])), (i, ti)
+            sparse_seen += got is not None
+        worst = max(worst, relerr(out, ref)); i += t
+    assert i == N and sparse_seen == N - (IBUD + IR - 1) and worst <= 2e-5
+    _, ib = att.read_index()
+    assert relerr(ib, IB) <= 1e-6
+
+
+def test_qsa_equal_scores_take_the_lowest_blocks_and_yarn_changes_the_rotation(ctx):
+    nh, nkv = 4, 2
+    row = nkv * 256; start = 160
+    p = qsa_inputs(nh, nkv, 23, 1)
+    # index queries whose dot with every block key is negative: all scores are exactly zero -> blocks 0..15 + tail
+    u = np.zeros(IHD, np.float32); u[64:] = 1.0
+    ikc = np.tile(u, (start, 1)).astype(np.float32); p["iq"] = np.tile(-u, (1, INH)).astype(np.float32); p["iqn"] = np.ones(IHD, np.float32); p["ikn"] = np.ones(IHD, np.float32)
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 0, 1024, 256)
+    att.set_indexer(INH, IHD, IR, IBUD, p["iqn"], p["ikn"])
+    att.set_context(128, 256)                                      # YaRN x2
+    kc = synth.normal((start, row), 6); vc = synth.normal((start, row), 7)
+    att.load_cache(kc, vc); att.load_index(ikc)
+    out = att.decode(p["q"], p["k"], p["v"], p["iq"], p["ik"])
+    assert list(att.selection(0)) == list(range(IBUD)) + [start]
+    inv, ms = orc.rope_inv_yarn(64, 1e7, 128, 256)
+    assert ms > 1.0
+    K = np.zeros((start + 1, row), np.float32); V = np.zeros_like(K); K[:start] = kc; V[:start] = vc
+    IK = np.zeros((start + 1, IHD), np.float32); IK[:start] = ikc; IB = np.zeros(((start + 1) // IR, IHD), np.float32); IB[:start // IR] = pooled(ikc, p["ikn"], inv, ms)
+    ref, sel = orc.attn_core_qsa(nh, nkv, 256, 64, 1e-6, inv, ms, p["qn"], p["kn"], p["q"], p["k"], p["v"], start, 0, 1024, K, V,
+                                 INH, IHD, IR, IBUD, p["iqn"], p["ikn"], p["iq"], p["ik"], IK, IB)
+    assert list(sel[0]) == list(range(IBUD)) + [start] and relerr(out, ref) <= 2e-5
+    k2, _ = att.read_cache()
+    assert relerr(k2[start], K[start]) <= 1e-6
+    _, ib = att.read_index()
+    assert relerr(ib, IB[:start // IR]) <= 1e-6
+    # without the factor and the scaled frequencies the new key row differs
+    plain = orc.attn_core(nh, nkv, 256, 64, 1e-6, orc.rope_inv(64, 1e7), p["qn"], p["kn"], p["q"], p["k"], p["v"], start, 0, 1024, K.copy(), V.copy())
+    assert relerr(out, plain) > 1e-3
 
 
 # ---- chunked DeltaNet prefill (matrix cores) against the sequential recurrence ---------------------------------------------

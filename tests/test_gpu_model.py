@@ -134,7 +134,8 @@ def test_model_loaded_from_gguf_shards_equals_the_model_built_from_the_same_tens
     p1 = str(tmp_path / "tiny-00001-of-00002.gguf"); p2 = str(tmp_path / "tiny-00002-of-00002.gguf")
     gw.write(p1, gw.model_meta(c), tens[:half]); gw.write(p2, [("split.no", gw.U16, 1)], tens[half:], alignment=128)
     gg = lib.Model.from_gguf(ctx, p2, kv_bits=c.kv_bits, kv_recent=c.kv_recent)
-    assert [getattr(gg.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in ("rope_base", "eps")] == [getattr(gm.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in ("rope_base", "eps")]
+    skip = ("rope_base", "eps", "ctx_train", "ctx")        # floats; the file's trained context (262144 by default) is the model's context unless one is asked for
+    assert [getattr(gg.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip] == [getattr(gm.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip]
     ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88], dtype=np.uint32)
     sa, sb = gm.new_state(64), gg.new_state(64)
     la, lb = gm.forward(ids, sa), gg.forward(ids, sb)
@@ -151,6 +152,51 @@ def test_model_loaded_from_gguf_shards_equals_the_model_built_from_the_same_tens
     gw.write(bad, [m for m in gw.model_meta(c) if "expert_count" not in m[0]], tens)
     with pytest.raises(lib.PyreError, match="gguf key qwen4exp.expert_count"):
         lib.Model.from_gguf(ctx, bad)
+
+
+def idx_cfg(**kw):
+    # one attention layer with an indexer: dense up to 16 + 4 - 1 = 19 visible positions, 4 blocks + tail beyond; YaRN x2
+    return small_cfg(idx_nh=2, idx_hd=128, idx_ratio=4, idx_budget=16, ctx_train=64, ctx=128, **kw)
+
+
+def test_indexer_and_yarn_model_matches_oracle_greedy_verify_rollback_snapshot_and_device_loop(ctx, tmp_path):
+    c = idx_cfg()
+    hw, gm, om = pair(ctx, c, 12)
+    prompt = (np.arange(37, dtype=np.uint32) * 31 + 3) % c.vocab            # 37 > 19: the prompt itself already runs sparse
+    gs, os_ = gm.new_state(300), om.new_state()
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-4 and orc.argmax(lg) == orc.argmax(lo)
+    snap = gs.snapshot()
+    out_g, _ = gm.generate_greedy(gs, lg, 100)                               # host-driven loop; crosses the packing boundary at 128 + 64
+    out_o, _ = om.generate_greedy(os_, lo, 100)
+    assert np.array_equal(out_g, out_o), "first split at %d" % int(np.argmax(out_g != out_o))
+    # the device-resident loop (captured step, position on the device) from the snapshot gives the same stream
+    s2 = gm.new_state(200); s2.restore(snap)
+    assert np.array_equal(gm.decode_greedy_dev(s2, int(out_g[0]), 99), out_g[1:])
+    # verify window == single steps, rollback == never drafted (indexer keys and block keys included)
+    sa, sb = gm.new_state(64), gm.new_state(64)
+    gm.forward(prompt[:30], sa); gm.forward(prompt[:30], sb)
+    toks = np.array([9, 100, 11, 212, 13, 77], dtype=np.uint32)
+    lv = gm.forward_multi(toks, sa)
+    singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(6)])
+    assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32))
+    gm.spec_keep(sa, 6, 3)
+    sc = gm.new_state(64); gm.forward(prompt[:30], sc)
+    for i in range(3):
+        gm.forward(toks[i:i + 1], sc)
+    nxt = np.array([40, 41, 42, 43, 44], dtype=np.uint32)
+    assert np.array_equal(gm.forward(nxt, sa).view(np.uint32), gm.forward(nxt, sc).view(np.uint32))
+    # the same model through a GGUF file (indexer metadata and tensors by name; context 128 -> YaRN)
+    import gguf_writer as gw
+    p = str(tmp_path / "idx.gguf")
+    gw.write(p, gw.model_meta(c), gw.model_tensors(c, hw))
+    gg = lib.Model.from_gguf(ctx, p, kv_bits=c.kv_bits, kv_recent=c.kv_recent, ctx_tokens=128)
+    assert (gg.cfg.idx_nh, gg.cfg.idx_hd, gg.cfg.idx_ratio, gg.cfg.idx_budget, gg.cfg.ctx_train, gg.cfg.ctx) == (2, 128, 4, 16, 64, 128)
+    sg = gg.new_state(64)
+    assert np.array_equal(gg.forward(prompt, sg).view(np.uint32), lg.view(np.uint32))
+    # without the requested context the rotation table is the trained one: different logits
+    g0 = lib.Model.from_gguf(ctx, p, kv_bits=c.kv_bits, kv_recent=c.kv_recent)
+    assert relerr(g0.forward(prompt, g0.new_state(64)), lg) > 1e-4
 
 
 def test_snapshot_restore_reproduces_the_continuation_bit_for_bit(ctx):

@@ -165,6 +165,146 @@ def test_rope_rotates_pairs_i_and_i_plus_half_only_below_n_rot():
     assert relerr(got[:, NROT // 2:NROT], k0[:, NROT // 2:NROT] * np.cos(ang) + k0[:, :NROT // 2] * np.sin(ang)) < 1e-5
 
 
+# ---- QSA sparse indexer + YaRN ---------------------------------------------------------------------------------------
+INH, IHD, IR, IBUD = 3, 128, 4, 64          # dense up to 64 + 4 - 1 = 67 visible positions
+
+
+def qsa_inputs(seed, t):
+    g = lambda s, shape, std=1.0: synth.normal(shape, seed * 100 + s, std)
+    p = attn_inputs(seed, t)
+    p.update(iq=g(11, (t, INH * IHD)), ik=g(12, (t, IHD)), iqn=1 + g(13, (IHD,), 0.1), ikn=1 + g(14, (IHD,), 0.1))
+    return p
+
+
+def run_qsa(p, start, kc, vc, ikc, ibc, kv_bits=0, recent=1024, inv=None, mscale=1.0, budget=IBUD):
+    t = p["q"].shape[0]
+    K = np.zeros((start + t, NKV * HD), np.float32); V = np.zeros_like(K); K[:start] = kc; V[:start] = vc
+    IK = np.zeros((start + t, IHD), np.float32); IK[:start] = ikc
+    IB = np.zeros(((start + t) // IR, IHD), np.float32); IB[:start // IR] = ibc
+    inv = orc.rope_inv(NROT, 1e7) if inv is None else inv
+    out, sel = orc.attn_core_qsa(NH, NKV, HD, NROT, 1e-6, inv, mscale, p["qn"], p["kn"], p["q"], p["k"], p["v"], start, kv_bits, recent, K, V,
+                                 INH, IHD, IR, budget, p["iqn"], p["ikn"], p["iq"], p["ik"], IK, IB)
+    return out, sel, K, V, IK, IB
+
+
+def feed(seed, n, chunk=5, **kw):
+    """n positions through the oracle in windows of `chunk`; returns the per-token inputs and the final caches."""
+    kc = np.zeros((0, NKV * HD), np.float32); vc = kc.copy(); ikc = np.zeros((0, IHD), np.float32); ibc = ikc.copy()
+    ps, outs, sels = [], [], []
+    start = 0
+    while start < n:
+        t = min(chunk, n - start)
+        p = qsa_inputs(seed * 1000 + start, t)
+        out, sel, kc, vc, ikc, ibc = run_qsa(p, start, kc, vc, ikc, ibc, **kw)
+        ps.append(p); outs += list(out); sels += sel; start += t
+    return ps, outs, sels, kc, vc, ikc, ibc
+
+
+def test_qsa_is_dense_up_to_budget_plus_ratio_minus_one_and_equals_the_dense_branch():
+    n = IBUD + IR - 1
+    ps, outs, sels, kc, vc, ikc, ibc = feed(1, n)
+    assert all(s is None for s in sels)
+    # the dense entry point on the same inputs gives the same bits
+    kd = np.zeros((0, NKV * HD), np.float32); vd = kd.copy(); start = 0
+    for p in ps:
+        t = p["q"].shape[0]
+        o, kd, vd = run_attn(p, start, kd, vd)
+        assert np.array_equal(o, np.array(outs[start:start + t])); start += t
+    assert np.array_equal(kd, kc)
+    # one more position switches the selection on: budget/ratio blocks + tail
+    p = qsa_inputs(77, 1)
+    _, sel, *_ = run_qsa(p, n, kc, vc, ikc, ibc)
+    assert sel[0] is not None and len(sel[0]) == IBUD + (n + 1) % IR and (np.diff(sel[0]) > 0).all() and sel[0][-1] == n
+
+
+def test_qsa_block_keys_are_pooled_normalised_rotated_and_indexed_by_block():
+    n = 23
+    ps, _, _, _, _, ikc, ibc = feed(2, n, chunk=3)
+    assert ikc.shape == (n, IHD) and ibc.shape == (n // IR, IHD)
+    raw = np.concatenate([p["ik"] for p in ps]); assert np.array_equal(ikc, raw)       # raw keys stored as projected
+    inv = orc.rope_inv(NROT, 1e7); ikn = ps[0]["ikn"]
+    # all windows use differently seeded norm weights in feed(); re-run with one weight set to check the closed form
+    kc = np.zeros((0, NKV * HD), np.float32); vc = kc.copy(); ikc = np.zeros((0, IHD), np.float32); ibc = ikc.copy(); start = 0
+    rows = []
+    for w in range(6):
+        p = qsa_inputs(500 + w, 4); p["ikn"] = ikn; rows.append(p["ik"])
+        _, _, kc, vc, ikc, ibc = run_qsa(p, start, kc, vc, ikc, ibc); start += 4
+    for b in range(6):
+        exp = np_ref.qsa_pool(rows[b], ikn, 1e-6, b * IR, NROT, inv)
+        assert relerr(ibc[b], exp) < 1e-6, b
+    # identical keys in a block: the mean is the key itself
+    p = qsa_inputs(600, 4); p["ikn"] = ikn; p["ik"][:] = p["ik"][0]
+    _, _, _, _, _, ibc2 = run_qsa(p, start, kc, vc, ikc, ibc)
+    assert relerr(ibc2[6], np_ref.rope(np_ref.rms(p["ik"][0].astype(np.float64), ikn.astype(np.float64), 1e-6), 24, NROT, inv)) < 1e-6
+
+
+@pytest.mark.parametrize("kv_bits,recent", [(0, 1024), (4, 64)])
+def test_qsa_selection_and_sparse_attention_match_numpy(kv_bits, recent):
+    n0, t = 150, 6
+    ps, _, _, kc, vc, ikc, ibc = feed(3, n0, chunk=8, kv_bits=kv_bits, recent=recent)
+    p = qsa_inputs(9, t); p["iqn"] = ps[0]["iqn"]
+    out, sel, K, V, IK, IB = run_qsa(p, n0, kc, vc, ikc, ibc, kv_bits, recent)
+    inv = orc.rope_inv(NROT, 1e7)
+    Kn, Vn = kc.copy(), vc.copy()
+    for ti in range(t):
+        pos = n0 + ti; n = pos + 1
+        iq = np.stack([np_ref.rope(np_ref.rms(p["iq"][ti].reshape(INH, IHD)[h].astype(np.float64), p["iqn"].astype(np.float64), 1e-6), pos, NROT, inv) for h in range(INH)])
+        want = np_ref.qsa_select(iq, IB.astype(np.float64), n, IR, IBUD)
+        assert want is not None and np.array_equal(sel[ti], want), ti
+        assert len(want) == IBUD + n % IR
+        pb = orc.packed_boundary(n, kv_bits, recent)
+        o, kr, vr = np_ref.attn_step(NH, NKV, HD, NROT, 1e-6, inv, p["qn"], p["kn"], p["q"][ti], p["k"][ti], p["v"][ti], pos, Kn, Vn, pb, positions=want)
+        Kn = np.concatenate([Kn, kr[None]]); Vn = np.concatenate([Vn, vr[None]])
+        assert relerr(out[ti], o) < 2e-5, ti
+    if kv_bits:
+        assert orc.packed_boundary(n0 + t, kv_bits, recent) > 0
+
+
+def test_qsa_picks_the_blocks_whose_keys_point_along_the_query():
+    # block keys are pooled from raw keys; plant raw keys proportional to a direction u in chosen blocks and to -u elsewhere:
+    # with norm weights 1 and positions where RoPE leaves the planted (non-rotated) dims alone, relu(q.k) is positive only there
+    n0 = 200; nb = n0 // IR; chosen = sorted([3, 17, 18, 40, 41, 42, 5, 11, 29, 30, 31, 33, 36, 44, 47, 49])     # = budget / ratio = 16 blocks
+    u = np.zeros(IHD, np.float32); u[NROT:] = synth.normal((IHD - NROT,), 5)                                      # outside the rotated dims
+    kc = synth.normal((n0, NKV * HD), 6); vc = synth.normal((n0, NKV * HD), 7)
+    ikc = np.tile(-u, (n0, 1)).astype(np.float32)
+    for b in chosen:
+        ikc[b * IR:(b + 1) * IR] = u * (1.0 + 0.1 * b)          # distinct positive scores
+    ones = np.ones(IHD, np.float32)
+    inv = orc.rope_inv(NROT, 1e7)
+    ibc = np.stack([np_ref.qsa_pool(ikc[b * IR:(b + 1) * IR], ones, 1e-6, b * IR, NROT, inv) for b in range(nb)]).astype(np.float32)
+    p = qsa_inputs(4, 1); p["iqn"] = ones; p["ikn"] = ones; p["iq"] = np.tile(u, (1, INH)).astype(np.float32)
+    _, sel, *_ = run_qsa(p, n0, kc, vc, ikc, ibc)
+    want = [q for b in chosen for q in range(b * IR, (b + 1) * IR)] + [n0]
+    assert list(sel[0]) == want
+
+
+def test_yarn_table_reference_properties_and_closed_form():
+    inv, ms = orc.rope_inv_yarn(64, 1e7, 262144, 131072)                 # qn_ctx.rs:406-411
+    plain = orc.rope_inv(64, 1e7)
+    assert ms == 1.0 and inv[0] == 1.0 and np.array_equal(inv, plain)
+    assert np.array_equal(orc.rope_inv_yarn(64, 1e7, 0, 524288)[0], plain)
+    y, ym = orc.rope_inv_yarn(64, 1e7, 262144, 524288)                   # qn_ctx.rs:412-419
+    assert abs(ym - (1.0 + 0.1 * np.log(2.0))) < 1e-5 and ym > 1.0
+    assert y[0] < plain[0] and (abs(y[31] - plain[31]) / plain[31] < 0.05 or y[31] <= plain[31])
+    for train, ctx in ((262144, 524288), (262144, 300000), (32768, 1048576), (4096, 6000)):
+        got, gm = orc.rope_inv_yarn(64, 1e7, train, ctx)
+        exp, em = np_ref.yarn_inv(64, 1e7, train, ctx)
+        assert relerr(got, exp) < 1e-5 and abs(gm - em) < 1e-6, (train, ctx)
+        s = ctx / train
+        assert abs(got[0] * s - 1.0) < 1e-6 and abs(got[-1] / plain[-1] - 1.0) < 1e-6        # pure interpolation / pure extrapolation ends
+
+
+def test_yarn_magnitude_factor_scales_rotated_dims_only():
+    y, ym = orc.rope_inv_yarn(NROT, 1e7, 128, 256)
+    p = qsa_inputs(8, 1); p["kn"] = np.ones(HD, np.float32)
+    _, _, K, *_ = run_qsa(p, 7, np.zeros((7, NKV * HD)), np.zeros((7, NKV * HD)), np.zeros((7, IHD)), np.zeros((1, IHD)), inv=y, mscale=ym)
+    k0 = np_ref.rms(p["k"][0].reshape(NKV, HD).astype(np.float64), np.ones(HD), 1e-6)
+    got = K[7].reshape(NKV, HD).astype(np.float64)
+    assert relerr(got[:, NROT:], k0[:, NROT:]) < 1e-6
+    assert relerr(got, np_ref.rope(k0, 7, NROT, y, ym)) < 1e-5
+    assert relerr((got[:, :NROT] ** 2).sum(-1), (k0[:, :NROT] ** 2).sum(-1) * ym * ym) < 1e-5
+
+
 # ---- MoE / hyper-connections / token step --------------------------------------------------------------------------
 def small_cfg(**kw):
     c = mg.Config(n_layers=4, d=256, hc=2, hc_lr=32, n_exp=8, top_k=2, ff_exp=256, vocab=512, kv_recent=64)
@@ -223,6 +363,31 @@ def test_token_step_matches_numpy_and_prefill_equals_steps():
     lg2 = m.forward(ids, st2)                      # one prefill chunk: same arithmetic per token
     assert relerr(lg2, lg[-1]) < 1e-6
     assert relerr(st2.ssm(0), st.ssm(0)) < 1e-6 and np.array_equal(st2.kcache(0), st.kcache(0))
+
+
+def test_token_step_with_indexer_and_yarn_matches_numpy_and_rollback_restores_the_indexer_state():
+    # 4 layers (one attention layer with an indexer): dense up to 8 + 4 - 1 = 11 positions, sparse beyond; YaRN x2
+    c = small_cfg(idx_nh=2, idx_hd=128, idx_ratio=4, idx_budget=8, ctx_train=32, ctx=64)
+    hw = mg.build_host(c, seed=8)
+    m = orc_model(hw)
+    ids = ((np.arange(22, dtype=np.uint32) * 29 + 7) % c.vocab).astype(np.uint32)
+    st = m.new_state()
+    lg = np.array([m.forward(ids[i:i + 1], st) for i in range(ids.size)])
+    ref = np_forward_tokens(hw, ids)
+    for i in range(ids.size):
+        assert relerr(lg[i], ref[i]) < 1e-4, i
+    assert st.ikeys(0).size == 22 * 128 and st.iblocks(0).size == 5 * 128
+    # windows (prefill chunks) give the same per-token arithmetic
+    st2 = m.new_state(); m.forward(ids[:13], st2); lg2 = m.forward(ids[13:], st2)
+    assert relerr(lg2, lg[-1]) < 1e-6 and np.array_equal(st2.iblocks(0), st.iblocks(0)) and np.array_equal(st2.ikeys(0), st.ikeys(0))
+    # verify window + rollback: 5 tokens, keep 2 -> indexer state truncated to 15 + 2 = 17 positions, 4 blocks; continuing
+    # from there equals never having drafted
+    st3 = m.new_state(); m.forward(ids[:15], st3)
+    bad = ids[15:20].copy(); bad[2:] = (bad[2:] + 1) % c.vocab
+    m.forward_multi(bad, st3); m.spec_keep(st3, 5, 2)
+    assert len(st3) == 17 and st3.ikeys(0).size == 17 * 128 and st3.iblocks(0).size == 4 * 128
+    lg3 = np.array([m.forward(ids[i:i + 1], st3) for i in range(17, 22)])
+    assert np.array_equal(lg3, lg[17:22])
 
 
 def test_verify_rollback_and_drafted_generation_are_identical_to_plain_decode():
