@@ -199,6 +199,8 @@ def bench_decode(args):
     cfg = mg.a3b_config()
     if args.layers:
         cfg.n_layers = args.layers
+    if args.indexer:             # variant: the reference's long-context mechanism (QSA sparse indexer, its GGUF defaults: 2048-token budget, blocks of 4)
+        cfg.idx_nh, cfg.idx_hd, cfg.idx_ratio, cfg.idx_budget = args.indexer, 128, 4, 2048
     t0 = time.perf_counter()
     layers, globals_, raw = mg.build_device(ctx, cfg, seed=args.seed)
     ctx.sync()
@@ -270,7 +272,8 @@ def bench_decode(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[4]: Qwen-Next-style A3B hybrid, %d layers (3 Gated DeltaNet + 1 gated attention per group), 512 experts top-10 + shared, "
-                               "IQ3_S weights (bf16 router), 4 hyper-connection streams, 4-bit KV, greedy decode after a %d-token random prompt" % (cfg.n_layers, n_ctx),
+                               "IQ3_S weights (bf16 router), 4 hyper-connection streams, 4-bit KV, greedy decode after a %d-token random prompt%s" % (
+                                   cfg.n_layers, n_ctx, (", QSA indexer with %d heads (budget 2048, blocks of 4): variant, not the configuration of the metric" % args.indexer) if args.indexer else ""),
                    "context": n_ctx, "layers": cfg.n_layers},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel": dom_k, "algorithmic_bytes_per_launch": round(dom[2] / dom[0]), "avg_launch_us": round(dom[1] / dom[0] * 1e3, 3),
@@ -298,6 +301,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=32768, help="prompt length for the decode workload")
     ap.add_argument("--layers", type=int, default=0, help="debug: fewer layers than the 48 of the configuration")
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--indexer", type=int, default=0, metavar="HEADS", help="decode workload variant: attention layers with a QSA sparse indexer of this many heads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")

@@ -293,17 +293,40 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
         for (int s = 0; s < 16; ++s) B[s] = 0.0f;
       }
       float A[4][16];
+      // Whether a position is read from the 4-bit or the f32 part is a per-lane fact, but almost every wave is all of one
+      // kind (old selected blocks, or the tail): those take a branch the whole wave agrees on, with all loads in flight
+      // at once; only a wave that straddles the boundary decides lane by lane.
+      size_t pp[4]; bool lp = true, lf = true;
 #pragma unroll
-      for (int pt = 0; pt < 4; ++pt) {
-        const size_t pp = (size_t)pos_of(wbase + 16 * pt + li);
-        if ((int)pp < pb) {
-          uint32_t k0 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp)], k1 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp)];
-          float ksc = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp)];
+      for (int pt = 0; pt < 4; ++pt) { pp[pt] = (size_t)pos_of(wbase + 16 * pt + li); lp = lp && (int)pp[pt] < pb; lf = lf && (int)pp[pt] >= pb; }
+      if (__all(lp)) {
+        uint32_t kw[4][2]; float ksc[4];
 #pragma unroll
-          for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(s < 8 ? k0 : k1, s & 7) * ksc;
-        } else {
+        for (int pt = 0; pt < 4; ++pt) {
+          kw[pt][0] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp[pt])]; kw[pt][1] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp[pt])];
+          ksc[pt] = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp[pt])];
+        }
 #pragma unroll
-          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp)];
+        for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(kw[pt][s >> 3], s & 7) * ksc[pt];
+      } else if (__all(lf)) {
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp[pt])];
+      } else {
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt) {
+          if ((int)pp[pt] < pb) {
+            uint32_t k0 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp[pt])], k1 = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp[pt])];
+            float ksc = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp[pt])];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(s < 8 ? k0 : k1, s & 7) * ksc;
+          } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp[pt])];
+          }
         }
       }
 #pragma unroll
@@ -355,18 +378,41 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
     for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     if (active) {
       float A[4][16];
+      size_t pg[16]; bool lp = true, lf = true;             // entries past the list carry weight zero; their position is clamped
 #pragma unroll
-      for (int s = 0; s < 16; ++s) {            // entries past the list carry weight zero; their position is clamped
-        const size_t pg = (size_t)pos_of(wbase + 4 * s + lg);
-        if ((int)pg < pb) {
-          const uint32_t vw = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
-          const float vsc = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
-          const uint32_t hw = vw >> (16 * (li & 1));
+      for (int s = 0; s < 16; ++s) { pg[s] = (size_t)pos_of(wbase + 4 * s + lg); lp = lp && (int)pg[s] < pb; lf = lf && (int)pg[s] >= pb; }
+      if (__all(lp)) {
+        uint32_t vw[16]; float vsc[16];
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc;
-        } else {
-          float4 v = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+        for (int s = 0; s < 16; ++s) {
+          vw[s] = kv.vq[pg[s] * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
+          vsc[s] = kv.vs[pg[s] * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
+        }
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+          const uint32_t hw = vw[s] >> (16 * (li & 1));
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc[s];
+        }
+      } else if (__all(lf)) {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+          float4 v = *(const float4*)(kv.vf + pg[s] * row + (size_t)kvh * HD + dq * 64 + 4 * li);
           A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+          if ((int)pg[s] < pb) {
+            const uint32_t vw = kv.vq[pg[s] * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
+            const float vsc = kv.vs[pg[s] * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
+            const uint32_t hw = vw >> (16 * (li & 1));
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc;
+          } else {
+            float4 v = *(const float4*)(kv.vf + pg[s] * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+            A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
+          }
         }
       }
       float B[16];
@@ -479,7 +525,12 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
     { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn, (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
     *packed_done = pbn;
   }
-  double kvb = 0; for (int ti = 0; ti < t; ++ti) { double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent); kvb += 2.0 * a.nkv * a.hd * (pb * 0.625 + (n - pb) * 4.0); }
+  double kvb = 0;
+  for (int ti = 0; ti < t; ++ti) {
+    double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent);
+    if (qw && n > qw->list_stride) { double m = qw->list_stride, fp = n > 0 ? pb / n : 0; kvb += 2.0 * a.nkv * a.hd * m * (fp * 0.625 + (1 - fp) * 4.0); }     // a position list: its entries, packed in the cache's own proportion
+    else kvb += 2.0 * a.nkv * a.hd * (pb * 0.625 + (n - pb) * 4.0);
+  }
   { ProfScope ps(ctx, "attn_decode", kvb);
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp, qw); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp, qw); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp, qw); break;
     default: launch_decode<8>(ctx, a, kv, w, start, t, posp, qw); } }

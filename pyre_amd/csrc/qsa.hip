@@ -70,35 +70,42 @@ __global__ void k_qsa_prep(QsaDev q, AttnDev a, QsaBuf b, const float* __restric
   else b.ib[qsa_ib_at((size_t)blk, (size_t)tid, (size_t)hd)] = v;
 }
 
-// grid (ceil(max_blocks / 256), t), 256 threads: lane = block.  score[ti][b] = sum_h relu(q_h . key_b) / sqrt(hd) for the
-// n / ratio complete blocks a query with n visible positions can choose from; nothing while the query is dense.
+// grid (ceil(max_blocks / 64), t), 256 threads: lane = block, the four waves split the key length.
+// score[ti][b] = sum_h relu(q_h . key_b) / sqrt(hd) for the n / ratio complete blocks a query with n visible positions
+// can choose from; nothing while the query is dense.
 constexpr int QSA_HB = 4;
 __global__ __launch_bounds__(256) void k_qsa_score(QsaDev q, QsaBuf b, const float* __restrict__ iq, int start, const int* __restrict__ posp, float* __restrict__ score, int max_blocks) {
-  extern __shared__ float qs[];             // [round_up(nh, QSA_HB)][hd], rows past nh are zero
+  extern __shared__ float qs[];             // [round_up(nh, QSA_HB)][hd] queries (rows past nh are zero), then [4][nhp][64] partial dots
   if (posp) start = *posp;
   const int ti = blockIdx.y, n = start + ti + 1, hd = q.hd, tid = threadIdx.x;
   if (n <= q.budget + q.ratio - 1) return;
   const int nb = n / q.ratio, nhp = (q.nh + QSA_HB - 1) / QSA_HB * QSA_HB;
-  if ((int)blockIdx.x * 256 >= nb) return;
+  if ((int)blockIdx.x * 64 >= nb) return;
+  float* part = qs + (size_t)nhp * hd;
   for (int i = tid; i < nhp * hd; i += 256) qs[i] = i < q.nh * hd ? iq[(size_t)ti * q.nh * hd + i] : 0.0f;
   __syncthreads();
-  const int blk = blockIdx.x * 256 + tid, lane = tid & 63;
-  if ((blk & ~63) >= nb) return;             // the whole wave lies past the last complete block
-  const float* kb = b.ib + (size_t)(blk >> 6) * hd * 64 + lane;
-  float total = 0.0f;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), blk = blockIdx.x * 64 + lane;
+  const int seg = hd / 4, i0 = wave * seg;                      // this wave's slice of the key
+  const float* kb = b.ib + (size_t)blockIdx.x * hd * 64 + lane;
   for (int h0 = 0; h0 < nhp; h0 += QSA_HB) {
     float acc[QSA_HB];
 #pragma unroll
     for (int j = 0; j < QSA_HB; ++j) acc[j] = 0.0f;
-    for (int i = 0; i < hd; ++i) {
+#pragma unroll 8
+    for (int i = i0; i < i0 + seg; ++i) {
       const float kv = kb[(size_t)i * 64];
 #pragma unroll
       for (int j = 0; j < QSA_HB; ++j) acc[j] = fmaf(qs[(h0 + j) * hd + i], kv, acc[j]);
     }
 #pragma unroll
-    for (int j = 0; j < QSA_HB; ++j) total += fmaxf(acc[j], 0.0f);
+    for (int j = 0; j < QSA_HB; ++j) part[((size_t)wave * nhp + h0 + j) * 64 + lane] = acc[j];
   }
-  if (blk < nb) score[(size_t)ti * max_blocks + blk] = total * (1.0f / sqrtf((float)hd));
+  __syncthreads();
+  if (wave == 0 && blk < nb) {
+    float total = 0.0f;
+    for (int h = 0; h < q.nh; ++h) { float d = ((part[((size_t)0 * nhp + h) * 64 + lane] + part[((size_t)1 * nhp + h) * 64 + lane]) + part[((size_t)2 * nhp + h) * 64 + lane]) + part[((size_t)3 * nhp + h) * 64 + lane]; total += fmaxf(d, 0.0f); }
+    score[(size_t)ti * max_blocks + blk] = total * (1.0f / sqrtf((float)hd));
+  }
 }
 
 // exclusive prefix sum of one int per thread over a 1024-thread workgroup; *total receives the sum
@@ -120,7 +127,7 @@ __device__ __forceinline__ int block_excl_scan(int v, int* wtot, int* total) {
 // over the (non-negative) float bits, then every block above it plus, among the blocks equal to it, the lowest indices;
 // the chosen blocks are compacted in index order into positions, followed by the incomplete tail.
 __global__ __launch_bounds__(1024) void k_qsa_select(QsaDev q, const float* __restrict__ score, int start, const int* __restrict__ posp, int* __restrict__ plist, int* __restrict__ pcount, int list_stride, int max_blocks) {
-  __shared__ unsigned hist[256]; __shared__ unsigned s_prefix, s_need; __shared__ int wtot[16];
+  __shared__ unsigned hist[256]; __shared__ unsigned wsuf[4]; __shared__ unsigned s_prefix, s_need; __shared__ int wtot[16];
   if (posp) start = *posp;
   const int ti = blockIdx.x, tid = threadIdx.x, n = start + ti + 1;
   if (n <= q.budget + q.ratio - 1) { if (tid == 0) pcount[ti] = -1; return; }
@@ -134,10 +141,22 @@ __global__ __launch_bounds__(1024) void k_qsa_select(QsaDev q, const float* __re
     __syncthreads();
     for (int bk = tid; bk < nb; bk += 1024) { unsigned u = __float_as_uint(sc[bk]) & 0x7FFFFFFFu; if ((u & mask_hi) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u); }
     __syncthreads();
-    if (tid == 0) {
-      unsigned cum = 0; int d = 255;
-      for (; d > 0; --d) { if (cum + hist[d] >= need) break; cum += hist[d]; }
-      s_prefix = prefix | ((unsigned)d << shift); s_need = need - cum;
+    // bucket d of the current digit is the one that holds the need-th largest key when the count of keys in buckets
+    // >= d reaches need and the count in buckets > d does not: a suffix sum over the 256 buckets by threads 0..255
+    if (tid < 256) {
+      unsigned suf = hist[tid];                                // inclusive suffix sum inside the wave (this lane and the lanes above)
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) { unsigned u = __shfl_down(suf, o); if ((tid & 63) + o < 64) suf += u; }
+      if ((tid & 63) == 0) wsuf[tid >> 6] = suf;               // the wave's total
+      hist[tid] = suf;
+    }
+    __syncthreads();
+    if (tid < 256) {
+      unsigned above = 0; for (int w = (tid >> 6) + 1; w < 4; ++w) above += wsuf[w];
+      const unsigned incl = hist[tid] + above;                 // keys in buckets >= tid
+      const unsigned up = __shfl_down(incl, 1);
+      const unsigned excl = (tid & 63) == 63 ? above : up;     // keys in buckets > tid
+      if (incl >= need && excl < need) { s_prefix = prefix | ((unsigned)tid << shift); s_need = need - excl; }
     }
     __syncthreads();
     prefix = s_prefix; need = s_need;
@@ -198,8 +217,9 @@ int pyre_qsa_launch(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaB
   const int nbmax = posp ? w.max_blocks : (start + t) / q.ratio;
   if (maybe_sparse && nbmax > 0) {
     const int nhp = (q.nh + QSA_HB - 1) / QSA_HB * QSA_HB;
+    if (((size_t)nhp * q.hd + 4 * (size_t)nhp * 64) * 4 > 65536) return pyre_fail(ctx, PYRE_E_SHAPE, "indexer: %d heads of %d do not fit the score kernel's shared memory", q.nh, q.hd);
     ProfScope ps(ctx, "qsa_score", 4.0 * t * ((double)nbmax * q.hd + (double)q.nh * q.hd + nbmax));
-    hipLaunchKernelGGL(k_qsa_score, dim3((nbmax + 255) / 256, t), dim3(256), (size_t)nhp * q.hd * 4, ctx->stream, q, b, w.iq, start, posp, w.score, w.max_blocks); PYRE_CHECK_LAUNCH(ctx);
+    hipLaunchKernelGGL(k_qsa_score, dim3((nbmax + 63) / 64, t), dim3(256), ((size_t)nhp * q.hd + 4 * (size_t)nhp * 64) * 4, ctx->stream, q, b, w.iq, start, posp, w.score, w.max_blocks); PYRE_CHECK_LAUNCH(ctx);
   }
   { ProfScope ps(ctx, "qsa_select", 4.0 * t * (5.0 * nbmax + q.budget)); hipLaunchKernelGGL(k_qsa_select, dim3(t), dim3(1024), 0, ctx->stream, q, w.score, start, posp, w.plist, w.pcount, w.list_stride, w.max_blocks); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
