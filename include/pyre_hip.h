@@ -262,6 +262,26 @@ int   pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, co
  * tokens (optional, host) receives the n_steps generated ids after the call. */
 int   pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host);
 
+/* ---- request loop over one resident state: engine_qn::run (src/engine_qn.rs:92-170) --------------------------------
+ * Prefill on the absolute chunk grid (PYRE_PREFILL_CHUNK, default 256) with a prefix cache of state snapshots
+ * (PYRE_QN_PCACHE, PYRE_QN_PCACHE_MB): a prompt that strictly extends the previous request's tokens continues that
+ * state, otherwise it starts from the longest snapshot it strictly extends, otherwise from an empty state; snapshots are
+ * taken at grid boundaries and where the prompt leaves the previous prompt's common prefix, oldest dropped first beyond
+ * cache_bytes_cap (0 = no prefix cache).  Snapshots live in device memory.  The arithmetic of a token does not depend
+ * on how the prompt is split, so a resumed prompt ends in exactly the state and logits of a full prefill. */
+typedef struct pyre_session pyre_session;
+int   pyre_session_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, int prefill_chunk, size_t cache_bytes_cap, pyre_session** out);
+void  pyre_session_destroy(pyre_session* s);
+pyre_state* pyre_session_state(pyre_session* s);
+/* logits_host [vocab] after the last prompt token; *cached = prompt tokens not recomputed, *from_snapshot = 1 when they
+ * came from a snapshot rather than from the previous request's state.  A prompt of max_ctx tokens or more is refused
+ * with the reference's message. */
+int   pyre_session_prefill(pyre_ctx* ctx, pyre_session* s, const uint32_t* prompt, int n, float* logits_host, int* cached, int* from_snapshot);
+/* pyre_generate_greedy on the session's state; the tokens the state consumed are recorded for the next request. */
+int   pyre_session_generate_greedy(pyre_ctx* ctx, pyre_session* s, const float* first_logits_host, int n_out, uint32_t* out, int n_draft, const uint32_t* draft_stream, int* rounds);
+int   pyre_session_stats(const pyre_session* s, int* n_snapshots, size_t* snapshot_bytes, int* state_len);
+int   pyre_session_snapshot_len(const pyre_session* s, int i);      /* tokens of the i-th snapshot, oldest first; -1 past the end */
+
 #ifdef __cplusplus
 }
 #endif

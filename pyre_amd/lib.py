@@ -57,6 +57,13 @@ def _declare(L):
         "pyre_gguf_meta_f64": (i32, [vp, C.c_char_p, vp]),
         "pyre_gguf_meta_str": (i32, [vp, C.c_char_p, C.c_char_p, C.c_size_t]),
         "pyre_gguf_meta_arr_u64": (C.c_long, [vp, C.c_char_p, vp, C.c_size_t]),
+        "pyre_session_create": (i32, [vp, vp, i32, i32, sz, C.POINTER(vp)]),
+        "pyre_session_destroy": (None, [vp]),
+        "pyre_session_state": (vp, [vp]),
+        "pyre_session_prefill": (i32, [vp, vp, vp, i32, vp, C.POINTER(i32), C.POINTER(i32)]),
+        "pyre_session_generate_greedy": (i32, [vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32)]),
+        "pyre_session_stats": (i32, [vp, C.POINTER(i32), C.POINTER(sz), C.POINTER(i32)]),
+        "pyre_session_snapshot_len": (i32, [vp, i32]),
         "pyre_model_load_gguf": (i32, [vp, C.c_char_p, i32, i32, i32, vp]),
         "pyre_state_capacity": (i32, [vp]),
         "pyre_model_max_window": (i32, [vp]),
@@ -696,6 +703,47 @@ class State:
     def close(self):
         if getattr(self, "h", None) and getattr(self.m, "h", None) and getattr(self.m.ctx, "h", None):      # never after its context
             self.m.ctx.L.pyre_state_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Session:
+    """engine_qn::run of the reference (src/engine_qn.rs:92-170) over one resident state: chunk-grid prefill with a prefix
+    cache of device-resident snapshots, then greedy generation."""
+
+    def __init__(self, model, max_ctx, chunk=256, cache_bytes=3072 << 20):
+        self.m = model; self.ctx = model.ctx
+        h = C.c_void_p()
+        self.ctx.check(self.ctx.L.pyre_session_create(self.ctx.h, model.h, max_ctx, chunk, cache_bytes, C.byref(h)), "session_create")
+        self.h = h
+
+    def prefill(self, prompt):
+        """(logits after the prompt, prompt tokens not recomputed, whether they came from a snapshot)"""
+        ids = np.ascontiguousarray(prompt, dtype=np.uint32)
+        lg = np.empty(self.m.vocab, dtype=np.float32); cached = C.c_int32(); snap = C.c_int32()
+        self.ctx.check(self.ctx.L.pyre_session_prefill(self.ctx.h, self.h, _ptr(ids), ids.size, _ptr(lg), C.byref(cached), C.byref(snap)), "session_prefill")
+        return lg, cached.value, bool(snap.value)
+
+    def generate_greedy(self, first_logits, n_out, n_draft=0, draft_stream=None):
+        fl = np.ascontiguousarray(first_logits, dtype=np.float32); out = np.empty(n_out, dtype=np.uint32); rounds = C.c_int32()
+        ds = np.ascontiguousarray(draft_stream, dtype=np.uint32) if draft_stream is not None else None
+        self.ctx.check(self.ctx.L.pyre_session_generate_greedy(self.ctx.h, self.h, _ptr(fl), n_out, _ptr(out), n_draft, _ptr(ds) if ds is not None else None, C.byref(rounds)), "session_generate_greedy")
+        return out, rounds.value
+
+    def stats(self):
+        """(snapshots held, their bytes, tokens the state has consumed, snapshot lengths oldest first)"""
+        n = C.c_int32(); b = C.c_size_t(); ln = C.c_int32()
+        self.ctx.L.pyre_session_stats(self.h, C.byref(n), C.byref(b), C.byref(ln))
+        return n.value, b.value, ln.value, [self.ctx.L.pyre_session_snapshot_len(self.h, i) for i in range(n.value)]
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            self.ctx.L.pyre_session_destroy(self.h)
         self.h = None
 
     def __del__(self):

@@ -247,3 +247,48 @@ def test_device_greedy_loop_called_repeatedly_on_one_state_continues_the_same_st
     os_ = om.new_state(); lo = om.forward(prompt, os_)
     ref, _ = om.generate_greedy(os_, lo, 61)
     assert np.array_equal(ref[1:], whole)
+
+
+def test_session_chunk_grid_prefill_and_prefix_cache_give_the_state_of_a_full_prefill(ctx):
+    """engine_qn::run: continue the previous state, resume from the longest grid snapshot, cut at the common prefix."""
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 13)
+    rng = np.random.Generator(np.random.PCG64(5))
+    A = rng.integers(0, c.vocab, 150, dtype=np.uint32)
+    full = lambda ids: gm.forward(ids, gm.new_state(400))
+    se = lib.Session(gm, 400, chunk=32, cache_bytes=64 << 20)
+    la, cached, snap = se.prefill(A)
+    assert cached == 0 and not snap and np.array_equal(la.view(np.uint32), full(A).view(np.uint32))
+    assert se.stats()[3] == [32, 64, 96, 128] and se.stats()[2] == 150                  # grid snapshots, none at the prompt's end
+    out, _ = se.generate_greedy(la, 10)
+    so = om.new_state(); lo = om.forward(A, so)
+    assert np.array_equal(out, om.generate_greedy(so, lo, 10)[0]) and se.stats()[2] == 159     # the last token is pending
+    # 1. a prompt that strictly extends what the state consumed continues it
+    B = np.concatenate([A, out[:9], rng.integers(0, c.vocab, 20, dtype=np.uint32)]).astype(np.uint32)
+    lb, cached, snap = se.prefill(B)
+    assert cached == 159 and not snap and np.array_equal(lb.view(np.uint32), full(B).view(np.uint32))
+    # 2. a prompt that shares 100 tokens with A: longest snapshot it extends is 96; a snapshot is cut at the common prefix with
+    #    the previous prompt (B: 100 tokens) as well as on the grid
+    C2 = np.concatenate([A[:100], rng.integers(0, c.vocab, 70, dtype=np.uint32)]).astype(np.uint32)
+    lc, cached, snap = se.prefill(C2)
+    assert cached == 96 and snap and np.array_equal(lc.view(np.uint32), full(C2).view(np.uint32))
+    lens = se.stats()[3]
+    assert 100 in lens and 128 in lens and 160 in lens and lens.count(128) == 2          # A's and C2's 128-token prefixes differ
+    # 3. the same prompt again: every snapshot it strictly extends is a candidate -> the 160-token one
+    lc2, cached, snap = se.prefill(C2)
+    assert cached == 160 and snap and np.array_equal(lc2.view(np.uint32), lc.view(np.uint32))
+    # 4. an unrelated prompt starts from an empty state
+    D = rng.integers(0, c.vocab, 40, dtype=np.uint32)
+    ld, cached, snap = se.prefill(D)
+    assert cached == 0 and not snap and np.array_equal(ld.view(np.uint32), full(D).view(np.uint32))
+    # 5. the byte cap drops the oldest snapshots first; a prompt at or beyond the context size is refused
+    one = se.stats()[1] // se.stats()[0]
+    small = lib.Session(gm, 400, chunk=32, cache_bytes=3 * one)
+    small.prefill(A)
+    n, b, _, lens = small.stats()
+    assert b <= 3 * one and lens == sorted(lens) and lens[-1] == 128 and n < 4
+    with pytest.raises(lib.PyreError, match="exceeds context size"):
+        se.prefill(np.zeros(400, np.uint32))
+    off = lib.Session(gm, 400, chunk=32, cache_bytes=0)                                 # PYRE_QN_PCACHE=0
+    off.prefill(A); assert off.stats()[0] == 0
+    se.close(); small.close(); off.close()
