@@ -45,9 +45,19 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 #pragma unroll
   for (int t = 0; t < T; ++t) mine[t] = upw == 1 ? hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid) : 0.0f;
   const float mine_nv = upw == 1 ? norm[(size_t)s * d + i0 + tid] : 0.0f;
-  for (int i = tid; i < d; i += nthr) {
+  // four elements per pass with every load of the pass issued before the first square: the trip count depends on d, and
+  // a rolled loop would pay one memory round trip per element (measured: 14 of 30 us at five tokens).  Elements past d
+  // are clamped for the load and left out of the sum; each token's squares are still added in ascending element order.
+  for (int ib = tid; ib < d; ib += 4 * nthr) {
+    float vv[4][T];
 #pragma unroll
-    for (int t = 0; t < T; ++t) { float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i); ss[t] += v * v; }
+    for (int u = 0; u < 4; ++u) { const int ic = min(ib + u * nthr, d - 1);
+#pragma unroll
+      for (int t = 0; t < T; ++t) vv[u][t] = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, ic); }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) if (ib + u * nthr < d) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) ss[t] += vv[u][t] * vv[u][t]; }
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -212,7 +222,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   // (4.48 vs 4.26 ms per token) -- the dependent memory round trips of a stage cost the same inside one kernel, and
   // the barrier with its cache-bypassing hand-off costs more than the kernel boundary it replaces.
   static const bool fused_ok = getenv("PYRE_HC_FUSED") && atoi(getenv("PYRE_HC_FUSED")) != 0;
-  if (t == 1 && fused_ok && h.di.fmt == h.up.fmt && h.di.fmt != FMT_IQ2_XS && ctx->fuse_ctl) {
+  if (t == 1 && fused_ok && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
     const int nwg = std::max(h.di.tiles * p.ksplit, h.d / 64), L = p.nw * p.upw * 64;
     const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64) + 64;
     if (nwg <= 240 && lds <= 60000) {

@@ -168,7 +168,31 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
-  for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
+  if constexpr (T == 1) {
+    for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
+  } else {
+    // Several tokens: T x 64 activations per unit do not fit the scalar registers, and scalar loads in pieces cost one
+    // memory round trip per piece.  Each wave stages the activations of two units at a time in its own slice of shared
+    // memory ([token][unit][64], vector loads issued together with the units' weights) and takes them from there; a
+    // wave's shared-memory operations execute in order, so no workgroup barrier is involved.  The arithmetic per token
+    // is the single-token sequence.
+    extern __shared__ __align__(16) float xsm[];
+    float* xw = xsm + (size_t)wave * (2 * 64 * T);
+    for (int ku = k0; ku < k1; ku += 2) {
+      const bool two = ku + 1 < k1;
+      UnitRaw<FMT> r0 = unit_load<FMT>(m, tile, ku, lane), r1 = unit_load<FMT>(m, tile, two ? ku + 1 : ku, lane);
+      float xa[T], xb[T];
+#pragma unroll
+      for (int t = 0; t < T; ++t) { xa[t] = x[(size_t)t * m.cols + (size_t)ku * 64 + lane]; xb[t] = x[(size_t)t * m.cols + (size_t)(two ? ku + 1 : ku) * 64 + lane]; }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < T; ++t) { xw[(t * 2 + 0) * 64 + lane] = xa[t]; xw[(t * 2 + 1) * 64 + lane] = xb[t]; }
+      __builtin_amdgcn_wave_barrier();
+      unit_fma<FMT, T>(m, r0, ku, lds2, lane, xw, 128, acc);
+      if (two) unit_fma<FMT, T>(m, r1, ku + 1, lds2, lane, xw + 64, 128, acc);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[wave][t][lane] = acc[t];
   __syncthreads();
@@ -227,7 +251,7 @@ template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDe
   static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   ProfScope ps(ctx, name.c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * T * ((double)m.cols + m.rows));
-  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
+  hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), T > 1 ? (size_t)NW * 2 * 64 * T * 4 : 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 // Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
