@@ -143,7 +143,7 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
-struct HcWork { float* xn; float* o; };     // [8][hc*d] normalized streams, [<=32][8][tiles*64] slice sums of [down ; inject]
+struct HcWork { float* ssq; float* o; };    // [<=32][8] slice sums of squares of the streams, [<=32][8][tiles*64] slice sums of [down ; inject]
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // Streams are read from x_in (element i of stream s of token ti at x_in[ti*in_ts + s*in_ss + i]; in_ss = 0 replicates one

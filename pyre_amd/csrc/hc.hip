@@ -1,9 +1,10 @@
 // Hyper-connection mix / combine around every block: grouped RMSNorm over the hc residual streams, low-rank sigmoid
 // gate, stream mean; residual update.  Follows hc_mix / hc_combine, src/model/qwen4exp_gguf.rs:1357-1388 (f32 branch).
 //
-// One mix is two launches.  k_hc_norm_down folds the pending residual update, the grouped RMSNorm and the
-// [down ; inject] GEMV (K cut into slices, one slice per workgroup); k_hc_up_mix adds the slice sums, applies silu,
-// runs the up GEMV from shared memory and reduces the gated streams to their mean.
+// One mix is two launches.  k_hc_norm_down folds the pending residual update, the norm weights and the [down ; inject]
+// GEMV (K cut into slices, one slice per workgroup) and leaves each slice's sum of squares; k_hc_up_mix turns those
+// into the streams' RMS scales, adds the scaled slice sums, applies silu, runs the up GEMV from shared memory and
+// reduces the gated, normalized streams to their mean.
 #include "formats.h"
 #include "mega.h"
 #include <stdlib.h>
@@ -20,13 +21,39 @@ __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in
   return v;
 }
 
-// grid (row tiles of [down ; inject], K slices), nw waves.  A workgroup owns L = nw*upw*64 columns of one stream s:
-//   1. every workgroup recomputes sum(x_new^2) over the whole stream (d elements per token, tiny) -> scale
-//   2. its L columns of xn = (x_new * scale) * norm go to shared memory; the tile-0 workgroup of the slice also
-//      publishes them (xn) and the updated stream (x_out, never the buffer x_in points into)
-//   3. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
+// The slices of one output row, all loads in flight together: groups of eight behind a branch the whole launch agrees on
+// (ksplit is a kernel argument), so that unused groups cost neither loads nor instruction fetch; inside a group slices
+// past ksplit repeat the last one and are never added.  `want` is the thread's own condition (one execution mask).
+__device__ __forceinline__ void hc_load_run(float (&sv)[32], const float* __restrict__ p, int n, int stride) {      // n (<= 32) values at p, p + stride, ..
+#pragma unroll
+  for (int k = 0; k < 32; ++k) sv[k] = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) if (g * 4 < n) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sv[g * 4 + j] = p[(size_t)min(g * 4 + j, n - 1) * stride];
+  }
+}
+template <int T> __device__ __forceinline__ void hc_load_slices(float (&pv)[32], const float* __restrict__ part, bool want, int ksplit, int t, int r64, int i) {
+#pragma unroll
+  for (int ks = 0; ks < 32; ++ks) pv[ks] = 0.0f;
+  if (want) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) if (g * 8 < ksplit) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pv[g * 8 + j] = part[((size_t)min(g * 8 + j, ksplit - 1) * T + t) * r64 + i];
+    }
+  }
+}
+
+// grid (row tiles of [down ; inject], K slices), nw waves.  A workgroup owns L = nw*upw*64 columns of one stream s.
+// The RMS scale of a stream multiplies every term of a row's dot product, so it is applied after the dot (by
+// k_hc_up_mix, which also sums the slices): a workgroup never needs the sum of squares of the whole stream.
+//   1. its L columns of x_new (the pending residual update applied) times the norm weight go to shared memory; the
+//      squares of x_new are summed over the slice -> ssq[ks*T + t]; the tile-0 workgroup of the slice also publishes the
+//      updated stream (x_out, never the buffer x_in points into)
+//   2. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
 template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
-    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float eps, float* __restrict__ xn,
+    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq,
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   extern __shared__ __align__(16) float sm[];
@@ -37,27 +64,19 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   const int tile = blockIdx.x, ks = blockIdx.y;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
-  UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);     // in flight across both barriers
+  UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);     // in flight across the barrier
   float w[T], ss[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) { w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
-  float mine[T];        // upw == 1: the slice element this thread normalizes later (and its norm weight), fetched with the others
+  for (int j = tid; j < L; j += nthr) {
+    const float nv = norm[(size_t)s * d + i0 + j];
 #pragma unroll
-  for (int t = 0; t < T; ++t) mine[t] = upw == 1 ? hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid) : 0.0f;
-  const float mine_nv = upw == 1 ? norm[(size_t)s * d + i0 + tid] : 0.0f;
-  // four elements per pass with every load of the pass issued before the first square: the trip count depends on d, and
-  // a rolled loop would pay one memory round trip per element (measured: 14 of 30 us at five tokens).  Elements past d
-  // are clamped for the load and left out of the sum; each token's squares are still added in ascending element order.
-  for (int ib = tid; ib < d; ib += 4 * nthr) {
-    float vv[4][T];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) { const int ic = min(ib + u * nthr, d - 1);
-#pragma unroll
-      for (int t = 0; t < T; ++t) vv[u][t] = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, ic); }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) if (ib + u * nthr < d) {
-#pragma unroll
-      for (int t = 0; t < T; ++t) ss[t] += vv[u][t] * vv[u][t]; }
+    for (int t = 0; t < T; ++t) {
+      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
+      ss[t] += v * v;
+      xs[(size_t)t * L + j] = v * nv;
+      if (tile == 0) x_out[((size_t)t * hc + s) * d + i0 + j] = v;
+    }
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -66,20 +85,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
     if (lane == 0) wsum[wave * T + t] = ss[t];
   }
   __syncthreads();
-  float sc[T];
-#pragma unroll
-  for (int t = 0; t < T; ++t) { float tot = wsum[t]; for (int q = 1; q < nw; ++q) tot += wsum[q * T + t]; sc[t] = 1.0f / sqrtf(tot / (float)d + eps); }
-  for (int j = tid; j < L; j += nthr) {
-    const float nv = upw == 1 ? mine_nv : norm[(size_t)s * d + i0 + j];
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-      float v = upw == 1 ? mine[t] : hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
-      float o = v * sc[t] * nv;                                   // rms, :209: (x * s) * w
-      xs[(size_t)t * L + j] = o;
-      if (tile == 0) { size_t k = ((size_t)t * hc + s) * d + i0 + j; xn[k] = o; x_out[k] = v; }
-    }
-  }
-  __syncthreads();
+  if (tile == 0 && tid < T) { float tot = wsum[tid]; for (int q = 1; q < nw; ++q) tot += wsum[q * T + tid]; ssq[ks * T + tid] = tot; }
   float acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
@@ -95,57 +101,69 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
   }
 }
 
-// grid (d / 64), hc*U waves (U = lr / 64 units of the up matrix).  Prologue: o = slice sums of [down ; inject] added in
-// slice order; lo = silu(o / hc) for the first lr rows -> shared memory, inj = o[lr + s] / hc (zeros without inject)
-// (:1376-1378).  Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is
-// the sum of its waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc, s ascending from zero (:1380).
-template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, int ksplit, int r64, int lr, int hc, int has_inject,
-    const float* __restrict__ xn, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2) {
+// grid (d / 64), hc*U waves (U = lr / 64 units of the up matrix).  Prologue: the streams' RMS scales from the slice
+// sums of squares, scale_s = 1 / sqrt(sum / d + eps) (rms, :209); o = the scaled slice sums of [down ; inject];
+// lo = silu(o / hc) for the first lr rows -> shared memory, inj = o[lr + s] / hc (zeros without inject) (:1376-1378).
+// Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is the sum of its
+// waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc with xn = (x * scale_s) * norm, s ascending
+// from zero (:1380).
+template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
+    const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   extern __shared__ __align__(16) float sm[];
-  const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6;
+  const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc;
   float* lo = sm;                         // [T][lr]
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
+  float* scs = red + (size_t)(nthr >> 6) * T * 64;   // [T][8]
   const int n_o = lr + hc;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave / U, ku = wave - s * U;
   UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);        // in flight across the prologue
-  float xpre[8];                  // the epilogue's normalized-stream values of this thread's first output, fetched now
+  float xpre[8], npre[8];         // the epilogue's stream values and norm weights of this thread's first output, fetched now
 #pragma unroll
-  for (int q = 0; q < 8; ++q) xpre[q] = (tid < T * 64 && q < hc) ? xn[((size_t)(tid >> 6) * hc + q) * d + blockIdx.x * 64 + (tid & 63)] : 0.0f;
-  for (int idx = tid; idx < T * n_o; idx += nthr) {
-    int t = idx / n_o, i = idx - t * n_o;
-    float o = 0.0f;
-    if (i < lr || has_inject) {
-      float pv[32];                 // every slice is fetched before the first add: one round trip
+  for (int q = 0; q < 8; ++q) { const bool on = tid < T * 64 && q < hc;
+    xpre[q] = on ? xnew[((size_t)(tid >> 6) * hc + q) * d + blockIdx.x * 64 + (tid & 63)] : 0.0f; npre[q] = on ? norm[(size_t)q * d + blockIdx.x * 64 + (tid & 63)] : 0.0f; }
+  // the slices of this thread's first output row are fetched before the barrier the scales need
+  float pv[32]; int idx = tid; int t = idx / n_o, i = idx - t * n_o;
+  bool have = idx < T * n_o;
+  hc_load_slices<T>(pv, part, have && (i < lr || has_inject), ksplit, t, r64, i);
+  if (tid < T * hc) {
+    const int tt = tid / hc, q = tid - tt * hc;
+    float sv[32];                 // all of the stream's slices before the first add: one round trip
+    hc_load_run(sv, ssq + (size_t)(q * kps) * T + tt, kps, T);
+    float tot = sv[0];
 #pragma unroll
-      for (int ks = 0; ks < 32; ++ks) pv[ks] = ks < ksplit ? part[((size_t)ks * T + t) * r64 + i] : 0.0f;
-      o = pv[0];
-#pragma unroll
-      for (int ks = 1; ks < 32; ++ks) if (ks < ksplit) o += pv[ks];
-    }
-    float v = o / (float)hc;
+    for (int k = 1; k < 32; ++k) if (k < kps) tot += sv[k];
+    scs[tt * 8 + q] = 1.0f / sqrtf(tot / (float)d + eps);
+  }
+  __syncthreads();
+  while (have) {
+    const float o = (i < lr || has_inject) ? mega::hc_scaled_sum(pv, scs + t * 8, ksplit, kps) : 0.0f;
+    const float v = o / (float)hc;
     if (i < lr) lo[t * lr + i] = v * sigm(v);
     else if (blockIdx.x == 0) inj[t * hc + (i - lr)] = has_inject ? v : 0.0f;
+    idx += nthr; have = idx < T * n_o;
+    if (have) { t = idx / n_o; i = idx - t * n_o; hc_load_slices<T>(pv, part, i < lr || has_inject, ksplit, t, r64, i); }
   }
   __syncthreads();
   float acc[T];
 #pragma unroll
-  for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+  for (int t2 = 0; t2 < T; ++t2) acc[t2] = 0.0f;
   unit_fma<FMT, T>(up, raw, ku, lds2, lane, lo + ku * 64, lr, acc);
 #pragma unroll
-  for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
+  for (int t2 = 0; t2 < T; ++t2) red[((size_t)wave * T + t2) * 64 + lane] = acc[t2];
   __syncthreads();
-  for (int i = tid; i < T * 64; i += nthr) {
-    int t = i >> 6, l = i & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
+  for (int i2 = tid; i2 < T * 64; i2 += nthr) {
+    int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
 #pragma unroll
     for (int q = 0; q < 8; ++q) if (q < hc) {
-      float g = red[((size_t)(q * U) * T + t) * 64 + l];
-      for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t) * 64 + l];
-      const float xv = i == tid ? xpre[q] : xn[((size_t)t * hc + q) * d + col];
-      mx += xv * sigm(g);
+      float g = red[((size_t)(q * U) * T + t2) * 64 + l];
+      for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t2) * 64 + l];
+      const float xv = i2 == tid ? xpre[q] : xnew[((size_t)t2 * hc + q) * d + col];
+      const float nv = i2 == tid ? npre[q] : norm[(size_t)q * d + col];
+      mx += xv * scs[t2 * 8 + q] * nv * sigm(g);                   // rms, :209: (x * s) * w
     }
-    mixed[(size_t)t * d + col] = mx / (float)hc;
+    mixed[(size_t)t2 * d + col] = mx / (float)hc;
   }
 }
 
@@ -169,14 +187,14 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
                                                const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   const int L = p.nw * p.upw * 64; size_t lds = 4 * ((size_t)T * L + (size_t)p.nw * T * 64 + (size_t)p.nw * T);
   ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
-  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, eps,
-                     w.xn, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
+  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc,
+                     w.ssq, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
-template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, float* mixed, float* inj) {
-  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64);
+template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj) {
+  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 8);
   ProfScope ps(ctx, "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
-  hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, w.xn, h.d, mixed, inj,
+  hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, h.d, mixed, inj,
                      (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
@@ -191,8 +209,8 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
 int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, eps))
 }
-int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, float* mixed, float* inj) {
-  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, mixed, inj))
+int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj) {
+  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj))
 }
 }  // namespace
 
@@ -201,10 +219,10 @@ bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit) {
   DownPlan p = down_plan(h); *nw = p.nw; *upw = p.upw; *ksplit = p.ksplit;
   return p.ksplit >= 1 && p.ksplit <= 32 && p.ksplit * p.nw * p.upw == h.di.U;
 }
-size_t pyre_hc_work_bytes(const HcDev& h) { size_t w = (size_t)h.hc * h.d; return 256 * 3 + 4 * 8 * w + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
+size_t pyre_hc_work_bytes(const HcDev& h) { return 256 * 3 + 4 * 8 * 32 + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
 void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
-  w->xn = (float*)take(4 * 8 * (size_t)h.hc * h.d); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
+  w->ssq = (float*)take(4 * 8 * 32); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
 }
 
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
@@ -230,7 +248,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
       mega::HcPlan pl{p.nw, p.upw, p.ksplit};
       ProfScope ps(ctx, "hc_mix_fused", qmat_gguf_bytes(h.di, h.di.rows) + qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * h.hc * h.d * 4);
       switch (h.di.fmt) {
-#define HC_FUSED_CASE(F) case F: hipLaunchKernelGGL((mega::k_hc_mix_fused<F>), dim3(nwg), dim3(mega::WGT), lds, ctx->stream, h, pl, x_in, in_ss, x_out, cb, eps, w.xn, w.o, mixed, inj, ctx->fuse_ctl, 2000000u); break;
+#define HC_FUSED_CASE(F) case F: hipLaunchKernelGGL((mega::k_hc_mix_fused<F>), dim3(nwg), dim3(mega::WGT), lds, ctx->stream, h, pl, x_in, in_ss, x_out, cb, eps, w.ssq, w.o, mixed, inj, ctx->fuse_ctl, 2000000u); break;
         HC_FUSED_CASE(FMT_F32) HC_FUSED_CASE(FMT_F16) HC_FUSED_CASE(FMT_BF16) HC_FUSED_CASE(FMT_Q8_0) HC_FUSED_CASE(FMT_Q4_K) default: HC_FUSED_CASE(FMT_IQ3_S)
 #undef HC_FUSED_CASE
       }
@@ -238,7 +256,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     }
   }
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, mo, comb_inj, eps); if (rc) return rc;
-  return up_mix(ctx, h, w, p.ksplit, t, mixed, inj);
+  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj);
 }
 
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x, int t, const float* out, const float* inj) {

@@ -101,7 +101,7 @@ struct Args {
   HcDev head; HcPlan ph; QMatDev embd, out; GemvPlan gh;
   int d, hc, ch, pw_lin, pw_attn, conv_k; float eps;
   // activations (one token)
-  float *emb, *xa, *xb, *xn, *part, *mixed, *inj_a, *inj_f, *proj, *co, *core, *o, *hbuf, *vlogits;
+  float *emb, *xa, *xb, *ssq, *part, *mixed, *inj_a, *inj_f, *proj, *co, *core, *o, *hbuf, *vlogits;
   uint32_t* best; MoeWork mw; AttnWork aw;
   uint32_t* toks; uint32_t first; int start_pos, n_steps;
   unsigned* ctl; unsigned limit;
@@ -129,37 +129,31 @@ __device__ __forceinline__ float hc_x_new(const float* x_in, int in_ss, const Co
   else if (cb.out) v = v + ldc(cb.out + i) * w;
   return v;
 }
-template <int FMT> __device__ __forceinline__ void st_norm_down(const HcDev& h, const HcPlan& pl, const float* x_in, int in_ss, float* x_out, const Comb& cb, float eps,
-                                                float* xn, float* part, const uint2* g2, char* lds) {
+template <int FMT> __device__ __forceinline__ void st_norm_down(const HcDev& h, const HcPlan& pl, const float* x_in, int in_ss, float* x_out, const Comb& cb,
+                                                float* ssq, float* part, const uint2* g2, char* lds) {
   const QMatDev& m = h.di; const int d = h.d, hc = h.hc, nvb = m.tiles * pl.ksplit, VT = pl.nw * 64, upw = pl.upw, nw = pl.nw, L = nw * upw * 64;
   float* xs = (float*)lds; float* red = xs + L; float* wsum = red + nw * 64;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   for (int vb = blockIdx.x; vb < nvb; vb += gridDim.x) {
     const int tile = vb % m.tiles, ks = vb / m.tiles; const bool act = tid < VT;
     const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
-    UnitRaw<FMT> raw; float w = 0.0f, ss = 0.0f, mine = 0.0f;
+    UnitRaw<FMT> raw; float w = 0.0f, ss = 0.0f;
     if (act) {
       raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);
       w = (cb.out || cb.mo.partial) ? 2.0f * sigm(ldc(cb.inj + s)) : 0.0f;
-      mine = upw == 1 ? hc_x_new(x_in, in_ss, cb, w, d, s, i0 + tid) : 0.0f;
-      for (int i = tid; i < d; i += VT) { float v = hc_x_new(x_in, in_ss, cb, w, d, s, i); ss += v * v; }
+      for (int j = tid; j < L; j += VT) {
+        const float nv = h.norm[(size_t)s * d + i0 + j];
+        float v = hc_x_new(x_in, in_ss, cb, w, d, s, i0 + j);
+        ss += v * v;
+        xs[j] = v * nv;
+        if (tile == 0) stc(x_out + (size_t)s * d + i0 + j, v);
+      }
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
       if (lane == 0) wsum[wave] = ss;
     }
     __syncthreads();
-    if (act) {
-      float tot = wsum[0]; for (int q = 1; q < nw; ++q) tot += wsum[q];
-      const float sc = 1.0f / sqrtf(tot / (float)d + eps);
-      for (int j = tid; j < L; j += VT) {
-        const float nv = h.norm[(size_t)s * d + i0 + j];
-        float v = upw == 1 ? mine : hc_x_new(x_in, in_ss, cb, w, d, s, i0 + j);
-        float o = v * sc * nv;
-        xs[j] = o;
-        if (tile == 0) { size_t k = (size_t)s * d + i0 + j; stc(xn + k, o); stc(x_out + k, v); }
-      }
-    }
-    __syncthreads();
+    if (tile == 0 && tid == 0) { float tot = wsum[0]; for (int q = 1; q < nw; ++q) tot += wsum[q]; stc(ssq + ks, tot); }
     if (act) {
       float acc[1] = {0.0f};
       for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, 1>(m, raw, ks * nw * upw + lu, (const uint2*)nullptr, lane, xs + lu * 64, L, acc); }
@@ -175,30 +169,84 @@ template <int FMT> __device__ __forceinline__ void st_norm_down(const HcDev& h, 
   (void)g2; (void)hc;
 }
 
-// ---- stage: slice sums + silu + up GEMV + gated stream mean (k_hc_up_mix at T = 1) ---------------------------------------
-template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int ksplit, const float* part, const float* xn, float* mixed, float* inj, char* lds) {
-  const QMatDev& up = h.up; const int lr = h.lr, hc = h.hc, d = h.d, U = lr >> 6, r64 = h.di.tiles * 64, nvb = d / 64, VT = hc * U * 64, n_o = lr + hc;
-  float* lo = (float*)lds; float* red = lo + lr;
+// o = sum over the streams, in order, of  scale_s * (the stream's slice sums added in slice order):  `pv` holds the
+// slices of one output row, `sc` the streams' RMS scales, kps the slices per stream.  The usual slice counts are powers of
+// two and get straight-line code with fixed register indices; any other count takes the generic walk.
+template <int KPS> __device__ __forceinline__ float hc_scaled_sum_k(const float (&pv)[32], const float* sc, int hc) {
+  float o = 0.0f;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) if (q * KPS < 32 && q < hc) {
+    float inner = pv[(q * KPS) & 31];
+#pragma unroll
+    for (int k = 1; k < KPS; ++k) inner += pv[(q * KPS + k) & 31];
+    const float term = sc[q] * inner;
+    o = q == 0 ? term : o + term;
+  }
+  return o;
+}
+__device__ __forceinline__ float hc_scaled_sum(const float (&pv)[32], const float* sc, int ksplit, int kps) {
+  const int hc = ksplit / kps;
+  if (hc <= 8) switch (kps) {
+    case 1: return hc_scaled_sum_k<1>(pv, sc, hc); case 2: return hc_scaled_sum_k<2>(pv, sc, hc); case 4: return hc_scaled_sum_k<4>(pv, sc, hc);
+    case 8: return hc_scaled_sum_k<8>(pv, sc, hc); case 16: return hc_scaled_sum_k<16>(pv, sc, hc); case 32: return hc_scaled_sum_k<32>(pv, sc, hc);
+    default: break;
+  }
+  float o = 0.0f, inner = 0.0f; int left = kps, q = 0;
+#pragma unroll
+  for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) {
+    inner = left == kps ? pv[ks] : inner + pv[ks];
+    if (--left == 0) { const float term = sc[q] * inner; o = q == 0 ? term : o + term; ++q; left = kps; }
+  }
+  return o;
+}
+// n (<= 32) values at p, p + stride, ...: groups of four behind launch-uniform branches, all loads of a group in flight
+__device__ __forceinline__ void hc_load_run(float (&sv)[32], const float* p, int n, int stride) {
+#pragma unroll
+  for (int k = 0; k < 32; ++k) sv[k] = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) if (g * 4 < n) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sv[g * 4 + j] = ldc(p + (size_t)min(g * 4 + j, n - 1) * stride);
+  }
+}
+
+// ---- stage: stream scales + scaled slice sums + silu + up GEMV + gated stream mean (k_hc_up_mix at T = 1) ----------------
+template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int ksplit, const float* part, const float* ssq, const float* xnew, float eps, float* mixed, float* inj, char* lds) {
+  const QMatDev& up = h.up; const int lr = h.lr, hc = h.hc, d = h.d, U = lr >> 6, r64 = h.di.tiles * 64, nvb = d / 64, VT = hc * U * 64, n_o = lr + hc, kps = ksplit / hc;
+  float* lo = (float*)lds; float* red = lo + lr; float* scs = red + (size_t)hc * U * 64;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  auto load_slices = [&](float (&pv)[32], bool want, int i) {
+#pragma unroll
+    for (int ks = 0; ks < 32; ++ks) pv[ks] = 0.0f;
+    if (want) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) if (g * 8 < ksplit) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pv[g * 8 + j] = ldc(part + (size_t)min(g * 8 + j, ksplit - 1) * r64 + i);
+      }
+    }
+  };
   for (int vb = blockIdx.x; vb < nvb; vb += gridDim.x) {
     const bool act = tid < VT; const int s = wave / U, ku = wave - s * U;
-    UnitRaw<FMT> raw;
-    if (act) {
-      raw = unit_load<FMT>(up, s * (d >> 6) + vb, ku, lane);
-      for (int i = tid; i < n_o; i += VT) {
-        float o = 0.0f;
-        if (i < lr || h.has_inject) {
-          float pv[32];
+    UnitRaw<FMT> raw; float pv[32]; int i = tid; bool have = act && i < n_o;
+    if (act) raw = unit_load<FMT>(up, s * (d >> 6) + vb, ku, lane);
+    load_slices(pv, have && (i < lr || h.has_inject), i);
+    if (tid < hc) {
+      float sv[32];
+      hc_load_run(sv, ssq + tid * kps, kps, 1);
+      float tot = sv[0];
 #pragma unroll
-          for (int ks = 0; ks < 32; ++ks) pv[ks] = ks < ksplit ? ldc(part + (size_t)ks * r64 + i) : 0.0f;
-          o = pv[0];
-#pragma unroll
-          for (int ks = 1; ks < 32; ++ks) if (ks < ksplit) o += pv[ks];
-        }
-        float v = o / (float)hc;
-        if (i < lr) lo[i] = v * sigm(v);
-        else if (vb == 0) stc(inj + (i - lr), h.has_inject ? v : 0.0f);
-      }
+      for (int k = 1; k < 32; ++k) if (k < kps) tot += sv[k];
+      scs[tid] = 1.0f / sqrtf(tot / (float)d + eps);
+    }
+    __syncthreads();
+    while (have) {
+      const float o = (i < lr || h.has_inject) ? hc_scaled_sum(pv, scs, ksplit, kps) : 0.0f;
+      const float v = o / (float)hc;
+      if (i < lr) lo[i] = v * sigm(v);
+      else if (vb == 0) stc(inj + (i - lr), h.has_inject ? v : 0.0f);
+      i += VT; have = i < n_o;
+      if (have) load_slices(pv, i < lr || h.has_inject, i);
     }
     __syncthreads();
     if (act) {
@@ -212,7 +260,7 @@ template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int
       for (int q = 0; q < hc; ++q) {
         float g = red[(q * U) * 64 + lane];
         for (int k = 1; k < U; ++k) g += red[(q * U + k) * 64 + lane];
-        mx += ldc(xn + (size_t)q * d + col) * sigm(g);
+        mx += ldc(xnew + (size_t)q * d + col) * scs[q] * h.norm[(size_t)q * d + col] * sigm(g);
       }
       stc(mixed + col, mx / (float)hc);
     }
@@ -742,12 +790,12 @@ template <int FMT> __device__ __forceinline__ void st_pick_embed(const uint32_t*
 // ---- one hyper-connection mix in one launch (single-token steps): norm + [down ; inject] slices, a barrier over the
 // launch's own workgroups instead of a kernel boundary, then slice sums + up GEMV + gated stream mean --------------------
 template <int FMT> __global__ __launch_bounds__(WGT) void k_hc_mix_fused(HcDev h, HcPlan pl, const float* x_in, int in_ss, float* x_out, Comb cb, float eps,
-                                                                       float* xn, float* part, float* mixed, float* inj, unsigned* ctl, unsigned limit) {
+                                                                       float* ssq, float* part, float* mixed, float* inj, unsigned* ctl, unsigned limit) {
   extern __shared__ __align__(16) char lds[];
   __shared__ unsigned bar_ok;
-  st_norm_down<FMT>(h, pl, x_in, in_ss, x_out, cb, eps, xn, part, nullptr, lds);
+  st_norm_down<FMT>(h, pl, x_in, in_ss, x_out, cb, ssq, part, nullptr, lds);
   if (!launch_sync(ctl, (int)gridDim.x, limit, &bar_ok)) return;
-  st_up_mix<FMT>(h, pl.ksplit, part, xn, mixed, inj, lds);
+  st_up_mix<FMT>(h, pl.ksplit, part, ssq, x_out, eps, mixed, inj, lds);
 }
 
 // ---- the kernel --------------------------------------------------------------------------------------------------------
@@ -769,10 +817,10 @@ template <int FW, int FR> __global__ __launch_bounds__(WGT) void k_decode(Args a
     Comb cb{nullptr, MoeOutC{nullptr, nullptr, nullptr, 0, 0}, nullptr};
     for (int il = 0; il < a.n_layers; ++il) {
       const Layer& L = a.layers[il];
-      st_norm_down<FW>(L.hca, L.pa, xin, in_ss, xout, cb, a.eps, a.xn, a.part, nullptr, lds);
+      st_norm_down<FW>(L.hca, L.pa, xin, in_ss, xout, cb, a.ssq, a.part, nullptr, lds);
       MEGA_SYNC(1);
       xin = xout; in_ss = d; { float* q = xout; xout = xother; xother = q; }
-      st_up_mix<FW>(L.hca, L.pa.ksplit, a.part, a.xn, a.mixed, a.inj_a, lds);
+      st_up_mix<FW>(L.hca, L.pa.ksplit, a.part, a.ssq, xin, a.eps, a.mixed, a.inj_a, lds);
       MEGA_SYNC(2);
       if (L.full) {
         st_gemv<FW>(L.proj, L.gp, a.mixed, a.proj, Epi{nullptr, nullptr, nullptr, nullptr, 0, 0}, lds);
@@ -796,10 +844,10 @@ template <int FW, int FR> __global__ __launch_bounds__(WGT) void k_decode(Args a
       st_gemv<FW>(L.outp, L.go, a.core, a.o, Epi{nullptr, nullptr, nullptr, nullptr, 0, 0}, lds);
       MEGA_SYNC(8);
       Comb ca{a.o, MoeOutC{nullptr, nullptr, nullptr, 0, 0}, a.inj_a};
-      st_norm_down<FW>(L.hcf, L.pf, xin, in_ss, xout, ca, a.eps, a.xn, a.part, nullptr, lds);
+      st_norm_down<FW>(L.hcf, L.pf, xin, in_ss, xout, ca, a.ssq, a.part, nullptr, lds);
       MEGA_SYNC(1);
       xin = xout; { float* q = xout; xout = xother; xother = q; }
-      st_up_mix<FW>(L.hcf, L.pf.ksplit, a.part, a.xn, a.mixed, a.inj_f, lds);
+      st_up_mix<FW>(L.hcf, L.pf.ksplit, a.part, a.ssq, xin, a.eps, a.mixed, a.inj_f, lds);
       MEGA_SYNC(2);
       st_gemv<FR>(L.moe.router, L.gr, a.mixed, a.mw.logits, Epi{nullptr, nullptr, nullptr, nullptr, 0, 0}, lds);
       MEGA_SYNC(9);
@@ -810,9 +858,9 @@ template <int FW, int FR> __global__ __launch_bounds__(WGT) void k_decode(Args a
       MEGA_SYNC(11);
       cb = Comb{nullptr, MoeOutC{a.mw.partial, a.mw.sel_w, a.mw.sg, d, L.moe.top_k}, a.inj_f};
     }
-    st_norm_down<FW>(a.head, a.ph, xin, in_ss, xout, cb, a.eps, a.xn, a.part, nullptr, lds);
+    st_norm_down<FW>(a.head, a.ph, xin, in_ss, xout, cb, a.ssq, a.part, nullptr, lds);
     MEGA_SYNC(1);
-    st_up_mix<FW>(a.head, a.ph.ksplit, a.part, a.xn, a.hbuf, a.inj_a, lds);
+    st_up_mix<FW>(a.head, a.ph.ksplit, a.part, a.ssq, xout, a.eps, a.hbuf, a.inj_a, lds);
     MEGA_SYNC(2);
     st_gemv<FW>(a.out, a.gh, a.hbuf, a.vlogits, Epi{a.best, nullptr, nullptr, nullptr, 0, 0}, lds);
     MEGA_SYNC(12);

@@ -420,7 +420,7 @@ bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
   m->mega_wgs = wgs;
   a.n_layers = c.n_layers; a.head = m->head; a.embd = m->embd; a.out = m->out; pyre_gemv_plan(m->out, &a.gh.nw, &a.gh.upw);
   a.d = c.d; a.hc = c.hc; a.ch = m->ch; a.pw_lin = m->pw_lin; a.pw_attn = m->pw_attn; a.conv_k = c.conv_k; a.eps = c.eps;
-  a.emb = m->emb; a.xa = m->x; a.xb = m->x2; a.xn = m->hw.xn; a.part = m->hw.o; a.mixed = m->mixed; a.inj_a = m->inj_a; a.inj_f = m->inj_f; a.proj = m->proj; a.co = m->co; a.core = m->core;
+  a.emb = m->emb; a.xa = m->x; a.xb = m->x2; a.ssq = m->hw.ssq; a.part = m->hw.o; a.mixed = m->mixed; a.inj_a = m->inj_a; a.inj_f = m->inj_f; a.proj = m->proj; a.co = m->co; a.core = m->core;
   a.o = m->o; a.hbuf = m->hbuf; a.vlogits = m->logits; a.best = m->best; a.mw = m->mw; a.ctl = m->mega_ctl; a.limit = 4000000u;
   m->mega_ok = 1; return true;
 }
