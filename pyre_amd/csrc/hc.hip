@@ -36,11 +36,12 @@ __device__ __forceinline__ void hc_load_run(float (&sv)[32], const float* __rest
 template <int T> __device__ __forceinline__ void hc_load_slices(float (&pv)[32], const float* __restrict__ part, bool want, int ksplit, int t, int r64, int i) {
 #pragma unroll
   for (int ks = 0; ks < 32; ++ks) pv[ks] = 0.0f;
+  const unsigned off = (unsigned)(t * r64 + i);
   if (want) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) if (g * 8 < ksplit) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) pv[g * 8 + j] = part[((size_t)min(g * 8 + j, ksplit - 1) * T + t) * r64 + i];
+      for (int j = 0; j < 8; ++j) pv[g * 8 + j] = (part + (size_t)min(g * 8 + j, ksplit - 1) * T * r64)[off];      // launch-uniform base + the thread's 32-bit offset
     }
   }
 }
@@ -102,7 +103,8 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 }
 
 // grid (d / 64), hc*U waves (U = lr / 64 units of the up matrix).  Prologue: the streams' RMS scales from the slice
-// sums of squares, scale_s = 1 / sqrt(sum / d + eps) (rms, :209); o = the scaled slice sums of [down ; inject];
+// sums of squares, scale_s = 1 / sqrt(sum / d + eps) (rms, :209); o = the slice sums of [down ; inject], each times
+// its stream's scale, added in slice order;
 // lo = silu(o / hc) for the first lr rows -> shared memory, inj = o[lr + s] / hc (zeros without inject) (:1376-1378).
 // Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is the sum of its
 // waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc with xn = (x * scale_s) * norm, s ascending
@@ -114,15 +116,18 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc;
   float* lo = sm;                         // [T][lr]
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
-  float* scs = red + (size_t)(nthr >> 6) * T * 64;   // [T][8]
+  float* sls = red + (size_t)(nthr >> 6) * T * 64;   // [T][32]: the RMS scale of the stream each slice belongs to
   const int n_o = lr + hc;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave / U, ku = wave - s * U;
   UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);        // in flight across the prologue
   float xpre[8], npre[8];         // the epilogue's stream values and norm weights of this thread's first output, fetched now
 #pragma unroll
-  for (int q = 0; q < 8; ++q) { const bool on = tid < T * 64 && q < hc;
-    xpre[q] = on ? xnew[((size_t)(tid >> 6) * hc + q) * d + blockIdx.x * 64 + (tid & 63)] : 0.0f; npre[q] = on ? norm[(size_t)q * d + blockIdx.x * 64 + (tid & 63)] : 0.0f; }
+  for (int q = 0; q < 8; ++q) { xpre[q] = 0.0f; npre[q] = 0.0f; }
+  if (wave < T) {                  // wave t holds token t's 64 outputs
+#pragma unroll
+    for (int q = 0; q < 8; ++q) if (q < hc) { xpre[q] = (xnew + ((size_t)wave * hc + q) * d + blockIdx.x * 64)[lane]; npre[q] = (norm + (size_t)q * d + blockIdx.x * 64)[lane]; }
+  }
   // the slices of this thread's first output row are fetched before the barrier the scales need
   float pv[32]; int idx = tid; int t = idx / n_o, i = idx - t * n_o;
   bool have = idx < T * n_o;
@@ -134,11 +139,16 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
     float tot = sv[0];
 #pragma unroll
     for (int k = 1; k < 32; ++k) if (k < kps) tot += sv[k];
-    scs[tt * 8 + q] = 1.0f / sqrtf(tot / (float)d + eps);
+    const float sc = 1.0f / sqrtf(tot / (float)d + eps);
+    for (int k = 0; k < kps; ++k) sls[tt * 32 + q * kps + k] = sc;
   }
   __syncthreads();
   while (have) {
-    const float o = (i < lr || has_inject) ? mega::hc_scaled_sum(pv, scs + t * 8, ksplit, kps) : 0.0f;
+    float o = 0.0f;                 // slices in order, each times its stream's scale
+    if (i < lr || has_inject) {
+#pragma unroll
+      for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) { const float term = pv[ks] * sls[t * 32 + ks]; o = ks == 0 ? term : o + term; }
+    }
     const float v = o / (float)hc;
     if (i < lr) lo[t * lr + i] = v * sigm(v);
     else if (blockIdx.x == 0) inj[t * hc + (i - lr)] = has_inject ? v : 0.0f;
@@ -161,7 +171,7 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
       for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t2) * 64 + l];
       const float xv = i2 == tid ? xpre[q] : xnew[((size_t)t2 * hc + q) * d + col];
       const float nv = i2 == tid ? npre[q] : norm[(size_t)q * d + col];
-      mx += xv * scs[t2 * 8 + q] * nv * sigm(g);                   // rms, :209: (x * s) * w
+      mx += xv * sls[t2 * 32 + q * kps] * nv * sigm(g);            // rms, :209: (x * s) * w
     }
     mixed[(size_t)t2 * d + col] = mx / (float)hc;
   }
@@ -192,7 +202,7 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj) {
-  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 8);
+  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32);
   ProfScope ps(ctx, "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
   hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, h.d, mixed, inj,
                      (const uint2*)ctx->d_iq2xs);
@@ -242,7 +252,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   static const bool fused_ok = getenv("PYRE_HC_FUSED") && atoi(getenv("PYRE_HC_FUSED")) != 0;
   if (t == 1 && fused_ok && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
     const int nwg = std::max(h.di.tiles * p.ksplit, h.d / 64), L = p.nw * p.upw * 64;
-    const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64) + 64;
+    const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64 + 32) + 64;
     if (nwg <= 240 && lds <= 60000) {
       mega::Comb cb{comb_out, mega::MoeOutC{mo.partial, mo.sel_w, mo.sg, mo.d, mo.k}, comb_inj};
       mega::HcPlan pl{p.nw, p.upw, p.ksplit};

@@ -169,36 +169,6 @@ template <int FMT> __device__ __forceinline__ void st_norm_down(const HcDev& h, 
   (void)g2; (void)hc;
 }
 
-// o = sum over the streams, in order, of  scale_s * (the stream's slice sums added in slice order):  `pv` holds the
-// slices of one output row, `sc` the streams' RMS scales, kps the slices per stream.  The usual slice counts are powers of
-// two and get straight-line code with fixed register indices; any other count takes the generic walk.
-template <int KPS> __device__ __forceinline__ float hc_scaled_sum_k(const float (&pv)[32], const float* sc, int hc) {
-  float o = 0.0f;
-#pragma unroll
-  for (int q = 0; q < 8; ++q) if (q * KPS < 32 && q < hc) {
-    float inner = pv[(q * KPS) & 31];
-#pragma unroll
-    for (int k = 1; k < KPS; ++k) inner += pv[(q * KPS + k) & 31];
-    const float term = sc[q] * inner;
-    o = q == 0 ? term : o + term;
-  }
-  return o;
-}
-__device__ __forceinline__ float hc_scaled_sum(const float (&pv)[32], const float* sc, int ksplit, int kps) {
-  const int hc = ksplit / kps;
-  if (hc <= 8) switch (kps) {
-    case 1: return hc_scaled_sum_k<1>(pv, sc, hc); case 2: return hc_scaled_sum_k<2>(pv, sc, hc); case 4: return hc_scaled_sum_k<4>(pv, sc, hc);
-    case 8: return hc_scaled_sum_k<8>(pv, sc, hc); case 16: return hc_scaled_sum_k<16>(pv, sc, hc); case 32: return hc_scaled_sum_k<32>(pv, sc, hc);
-    default: break;
-  }
-  float o = 0.0f, inner = 0.0f; int left = kps, q = 0;
-#pragma unroll
-  for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) {
-    inner = left == kps ? pv[ks] : inner + pv[ks];
-    if (--left == 0) { const float term = sc[q] * inner; o = q == 0 ? term : o + term; ++q; left = kps; }
-  }
-  return o;
-}
 // n (<= 32) values at p, p + stride, ...: groups of four behind launch-uniform branches, all loads of a group in flight
 __device__ __forceinline__ void hc_load_run(float (&sv)[32], const float* p, int n, int stride) {
 #pragma unroll
@@ -213,7 +183,7 @@ __device__ __forceinline__ void hc_load_run(float (&sv)[32], const float* p, int
 // ---- stage: stream scales + scaled slice sums + silu + up GEMV + gated stream mean (k_hc_up_mix at T = 1) ----------------
 template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int ksplit, const float* part, const float* ssq, const float* xnew, float eps, float* mixed, float* inj, char* lds) {
   const QMatDev& up = h.up; const int lr = h.lr, hc = h.hc, d = h.d, U = lr >> 6, r64 = h.di.tiles * 64, nvb = d / 64, VT = hc * U * 64, n_o = lr + hc, kps = ksplit / hc;
-  float* lo = (float*)lds; float* red = lo + lr; float* scs = red + (size_t)hc * U * 64;
+  float* lo = (float*)lds; float* red = lo + lr; float* sls = red + (size_t)hc * U * 64;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   auto load_slices = [&](float (&pv)[32], bool want, int i) {
 #pragma unroll
@@ -237,11 +207,16 @@ template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int
       float tot = sv[0];
 #pragma unroll
       for (int k = 1; k < 32; ++k) if (k < kps) tot += sv[k];
-      scs[tid] = 1.0f / sqrtf(tot / (float)d + eps);
+      const float sc = 1.0f / sqrtf(tot / (float)d + eps);
+      for (int k = 0; k < kps; ++k) sls[tid * kps + k] = sc;
     }
     __syncthreads();
     while (have) {
-      const float o = (i < lr || h.has_inject) ? hc_scaled_sum(pv, scs, ksplit, kps) : 0.0f;
+      float o = 0.0f;
+      if (i < lr || h.has_inject) {
+#pragma unroll
+        for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) { const float term = pv[ks] * sls[ks]; o = ks == 0 ? term : o + term; }
+      }
       const float v = o / (float)hc;
       if (i < lr) lo[i] = v * sigm(v);
       else if (vb == 0) stc(inj + (i - lr), h.has_inject ? v : 0.0f);
@@ -260,7 +235,7 @@ template <int FMT> __device__ __forceinline__ void st_up_mix(const HcDev& h, int
       for (int q = 0; q < hc; ++q) {
         float g = red[(q * U) * 64 + lane];
         for (int k = 1; k < U; ++k) g += red[(q * U + k) * 64 + lane];
-        mx += ldc(xnew + (size_t)q * d + col) * scs[q] * h.norm[(size_t)q * d + col] * sigm(g);
+        mx += ldc(xnew + (size_t)q * d + col) * sls[q * kps] * h.norm[(size_t)q * d + col] * sigm(g);
       }
       stc(mixed + col, mx / (float)hc);
     }
