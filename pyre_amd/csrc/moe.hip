@@ -75,7 +75,14 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
     route_topk(logits + (size_t)ti * m.n_exp, m.n_exp, m.top_k, rl);
     expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]);
   } else if (blockIdx.x == 0) {
-    float p = 0.0f; for (int i = threadIdx.x; i < m.d; i += NW * 64) p = fmaf(m.sh_gate_inp[i], xs[i], p);
+    float p = 0.0f;
+    for (int ib = threadIdx.x; ib < m.d; ib += 4 * NW * 64) {          // four elements per pass, loads first (elements past d: weight zero)
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { const int ic = min(ib + u * NW * 64, m.d - 1); a[u] = m.sh_gate_inp[ic]; b[u] = xs[ic]; }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) if (ib + u * NW * 64 < m.d) p = fmaf(a[u], b[u], p);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
     if (lane == 0) red[0][wave][0] = p;
@@ -87,7 +94,13 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   const int tile = (shared ? 0 : expert * (m.ff >> 6)) + blockIdx.x;
   const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
   float ag[1] = {0.0f}, au[1] = {0.0f};
-  for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(G, lds2, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, lds2, tile, ku, lane, xs + ku * 64, 0, au); }
+  // two units of both matrices are fetched before the first is consumed: a rolled loop would pay a memory round trip per unit
+  for (int ku = k0; ku < kend; ku += 2) {
+    const int kb = min(ku + 1, kend - 1);
+    UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ku, lane), u0 = unit_load<FMT>(Up, tile, ku, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
+    unit_fma<FMT, 1>(G, g0, ku, lds2, lane, xs + ku * 64, 0, ag); unit_fma<FMT, 1>(Up, u0, ku, lds2, lane, xs + ku * 64, 0, au);
+    if (ku + 1 < kend) { unit_fma<FMT, 1>(G, g1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, ag); unit_fma<FMT, 1>(Up, u1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, au); }
+  }
   red[0][wave][lane] = ag[0]; red[1][wave][lane] = au[0];
   __syncthreads();
   if (threadIdx.x < 64) {
