@@ -139,7 +139,10 @@ size_t pyre_moe_work_bytes(const MoeDev& m);
 void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
 // y[t][d] = ffn(x[t][d]).  With y == nullptr (top_k <= PYRE_MOE_KMAX) the output stays unreduced in the work buffers
 // (pyre_moe_out) for a consumer that evaluates moe_out_value itself.
-int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev);
+// Router logits that arrive as K-slice sums (left by the mix that produced x, see HcRoute): logit[t][e] = the slices
+// p[(s*T + t)*r64 + e], s = 0..nsl-1, added in slice order.
+struct RouteSrc { const float* p; int nsl; int r64; };
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr);
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
@@ -150,8 +153,13 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // row over the streams), the pending residual update is applied first when comb_out (a [t][d] vector) or comb_moe (the
 // unreduced FFN output) is given (x[ti][s][:] += out[ti][:] * 2*sigmoid(comb_inj[ti][s])), and the updated streams go to x_out [t][hc][d], which
 // must not overlap x_in.  mixed [t][d] and inj [t][hc] = hc_mix(updated streams).
+// The router GEMV of the FFN block that follows a mix, riding on the mix's second launch: workgroup b of that launch
+// owns columns [64b, 64b+64) of the mixed vector, so it leaves the K-slice sum part[(b*T + t)*tiles*64 + row] of every
+// router row; the gate/up launch adds the d/64 slices (RouteSrc).  bf16 and f32 routers, at most 64 slices.
+struct HcRoute { QMatDev router; float* part; };
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed_dev, float* inj_dev);
+                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr);
+bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router);
 // waves per workgroup, units per wave and K slices of the norm + [down ; inject] kernel; false if the shape is unsupported
 bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit);
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x_dev, int t, const float* out_dev, const float* inj_dev);

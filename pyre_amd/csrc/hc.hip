@@ -109,8 +109,12 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
 // Wave (s, ku) takes unit ku of row tile s*(d/64) + blockIdx.x of `up`; the gate logit of stream s is the sum of its
 // waves in unit order; mixed[i] = (sum_s xn[s][i] * sigm(gate_s[i])) / hc with xn = (x * scale_s) * norm, s ascending
 // from zero (:1380).
-template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
-    const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2) {
+// RF >= 0: the launch also leaves its K slice of the router GEMV over the mixed vector (format RF; HcRoute): wave w
+// takes router tile w, w + nw, .. at unit blockIdx.x, the first tile's weights fetched ahead of the up GEMV.
+template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
+    const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2,
+    QMatDev router, float* __restrict__ rpart) {
+  constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc;
@@ -155,6 +159,9 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
     idx += nthr; have = idx < T * n_o;
     if (have) { t = idx / n_o; i = idx - t * n_o; hc_load_slices<T>(pv, part, i < lr || has_inject, ksplit, t, r64, i); }
   }
+  UnitRaw<RFX> rraw;              // fetched once the registers it needs are free (f32: 64 of them, after the up GEMV); in flight until the epilogue
+  constexpr bool R_EARLY = RFX != FMT_F32;
+  if (ROUTE && R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
   __syncthreads();
   float acc[T];
 #pragma unroll
@@ -162,6 +169,7 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
   unit_fma<FMT, T>(up, raw, ku, lds2, lane, lo + ku * 64, lr, acc);
 #pragma unroll
   for (int t2 = 0; t2 < T; ++t2) red[((size_t)wave * T + t2) * 64 + lane] = acc[t2];
+  if (ROUTE && !R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
   __syncthreads();
   for (int i2 = tid; i2 < T * 64; i2 += nthr) {
     int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
@@ -173,7 +181,22 @@ template <int FMT, int T> __global__ __launch_bounds__(1024) void k_hc_up_mix(QM
       const float nv = i2 == tid ? npre[q] : norm[(size_t)q * d + col];
       mx += xv * sls[t2 * 32 + q * kps] * nv * sigm(g);            // rms, :209: (x * s) * w
     }
-    mixed[(size_t)t2 * d + col] = mx / (float)hc;
+    const float mv = mx / (float)hc;
+    mixed[(size_t)t2 * d + col] = mv;
+    if (ROUTE) lo[t2 * 64 + l] = mv;          // lo is free after the barrier above
+  }
+  if (ROUTE) {
+    __syncthreads();
+    const size_t rr64 = (size_t)router.tiles * 64; const int nw = nthr >> 6;
+    for (int tile = wave; tile < router.tiles; tile += nw) {
+      if (tile != wave) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
+#pragma unroll 1
+      for (int t2 = 0; t2 < T; ++t2) {          // one token at a time (same operations per token): T tokens at once would keep 64*T activations in registers
+        float ra[1] = {0.0f};
+        unit_fma<RFX, 1>(router, rraw, blockIdx.x, lds2, lane, lo + t2 * 64, 0, ra);
+        rpart[((size_t)blockIdx.x * T + t2) * rr64 + (size_t)tile * 64 + lane] = ra[0];
+      }
+    }
   }
 }
 
@@ -201,11 +224,17 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
                      w.ssq, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
-template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj) {
+template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
   const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32);
-  ProfScope ps(ctx, "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)));
-  hipLaunchKernelGGL((k_hc_up_mix<FMT, T>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, h.d, mixed, inj,
-                     (const uint2*)ctx->d_iq2xs);
+  const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
+  ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
+               (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
+#define UP_MIX_GO(RF) hipLaunchKernelGGL((k_hc_up_mix<FMT, T, RF>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
+                     h.d, mixed, inj, (const uint2*)ctx->d_iq2xs, rq, rp)
+  if constexpr (FMT == FMT_IQ3_S || FMT == FMT_BF16 || FMT == FMT_F16 || FMT == FMT_F32) {
+    if (rt && rq.fmt == FMT_BF16) UP_MIX_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_GO(FMT_F32); else UP_MIX_GO(-1);
+  } else UP_MIX_GO(-1);
+#undef UP_MIX_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 #define HC_T_SWITCH(F, FN, ...) \
@@ -219,11 +248,15 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
 int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
   HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, eps))
 }
-int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj) {
-  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj))
+int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
+  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt))
 }
 }  // namespace
 
+bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router) {
+  const int f = h.up.fmt;
+  return (f == FMT_IQ3_S || f == FMT_BF16 || f == FMT_F16 || f == FMT_F32) && (router.fmt == FMT_BF16 || router.fmt == FMT_F32) && router.cols == h.d && h.d / 64 <= 64 && router.U == h.d / 64;
+}
 bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit) {
   if (h.d % 64 || h.lr % 64 || h.hc * h.up.U > 16 || h.up.tiles != h.hc * (h.d / 64) || h.di.U != h.hc * (h.d / 64)) return false;
   DownPlan p = down_plan(h); *nw = p.nw; *upw = p.upw; *ksplit = p.ksplit;
@@ -236,8 +269,9 @@ void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
 }
 
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed, float* inj) {
+                       float eps, float* mixed, float* inj, const HcRoute* route) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
+  if (route && !pyre_hc_route_ok(h, route->router)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: this router cannot ride on the mix");
   if (x_in == x_out) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: the updated streams must go to another buffer");
   if (h.d % 64 || h.lr % 64 || h.hc * h.up.U > 16 || h.up.tiles != h.hc * (h.d / 64) || h.di.U != h.hc * (h.d / 64))
     return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: needs d and the low rank in multiples of 64 and hc * (low rank / 64) <= 16 (d %d, low rank %d, hc %d)", h.d, h.lr, h.hc);
@@ -250,7 +284,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   // (4.48 vs 4.26 ms per token) -- the dependent memory round trips of a stage cost the same inside one kernel, and
   // the barrier with its cache-bypassing hand-off costs more than the kernel boundary it replaces.
   static const bool fused_ok = getenv("PYRE_HC_FUSED") && atoi(getenv("PYRE_HC_FUSED")) != 0;
-  if (t == 1 && fused_ok && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
+  if (t == 1 && fused_ok && !route && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
     const int nwg = std::max(h.di.tiles * p.ksplit, h.d / 64), L = p.nw * p.upw * 64;
     const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64 + 32) + 64;
     if (nwg <= 240 && lds <= 60000) {
@@ -266,7 +300,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     }
   }
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, mo, comb_inj, eps); if (rc) return rc;
-  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj);
+  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route);
 }
 
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x, int t, const float* out, const float* inj) {

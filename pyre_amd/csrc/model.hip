@@ -29,7 +29,7 @@ struct pyre_model {
   size_t token_weight_bytes = 0;
   // activations for a window of up to 8 tokens
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
-  float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr;
+  float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr, *rpart = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
   int mega_ok = -1;               // persistent-kernel decode: -1 not probed, 0 unsupported shape/types, 1 usable
   std::vector<mega::Layer> mega_layers; mega::Args mega_args{}; mega::Layer* mega_dev = nullptr; unsigned* mega_ctl = nullptr; int mega_wgs = 0;
@@ -185,8 +185,9 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
   MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
+  size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + al256(rp_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
@@ -194,6 +195,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
+  m->rpart = (float*)take(rp_b);
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   guard.armed = false; *out = M.release(); return PYRE_OK;
 }
@@ -346,6 +348,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
   const bool raw_moe = c.top_k <= PYRE_MOE_KMAX && t == 1;        // single token: the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
+  const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
     if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
@@ -363,9 +366,11 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       s->cur[li] = nb;
     }
     if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
-    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f))) return rc;
+    const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
+    HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
+    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr))) return rc;
     advance();
-    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y))) return rc;
+    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y, ride ? &rs : nullptr))) return rc;
     if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
     comb_inj = m->inj_f;
   }

@@ -11,11 +11,26 @@
 // candidates (an expert outside its wave's best k cannot be in the global best k); the candidates are then ranked
 // against each other from shared memory.  Leaves the chosen ids (ascending) in s_idx[0..k) and their logits in s_val[0..k).
 struct RouteLds { float c_val[16 * 32]; int c_idx[16 * 32]; float r_val[32]; int r_idx[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
-__device__ __forceinline__ void route_topk(const float* __restrict__ logits, int n_exp, int k, RouteLds& L) {
+// The logits are given as nsl (<= 64) K-slice sums `sstride` floats apart, added in slice order (nsl == 1: the logits
+// themselves); all slices are fetched before the first add, in groups of eight behind launch-uniform branches.
+__device__ __forceinline__ void route_topk(const float* __restrict__ logits, int nsl, int sstride, int n_exp, int k, RouteLds& L) {
   const int e = threadIdx.x, lane = e & 63, wave = e >> 6, nwa = (n_exp + 63) >> 6;
   if (wave < nwa) {
     float v = -INFINITY;
-    if (e < n_exp) { v = logits[e]; if (isnan(v)) v = -INFINITY; }      // nan_clean
+    if (e < n_exp) {
+      float sv[64];
+#pragma unroll
+      for (int q = 0; q < 64; ++q) sv[q] = 0.0f;
+#pragma unroll
+      for (int g = 0; g < 8; ++g) if (g * 8 < nsl) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sv[g * 8 + q] = (logits + (size_t)min(g * 8 + q, nsl - 1) * sstride)[e];
+      }
+      v = sv[0];
+#pragma unroll
+      for (int q = 1; q < 64; ++q) if (q < nsl) v += sv[q];
+      if (isnan(v)) v = -INFINITY;      // nan_clean
+    }
     int lr = 0;
 #pragma unroll
     for (int j = 0; j < 64; ++j) { float u = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); lr += (u > v || (u == v && j < lane)) ? 1 : 0; }
@@ -60,7 +75,7 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // entry publishes the shared-expert gate sigmoid(sh_gate_inp . x).
 template <int FMT, int NW>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
-                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2) {
+                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   __shared__ float red[2][NW][64];
   __shared__ RouteLds rl;
@@ -72,7 +87,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   const float* xs = x + (size_t)ti * m.d;
   int expert = 0;
   if (!shared) {
-    route_topk(logits + (size_t)ti * m.n_exp, m.n_exp, m.top_k, rl);
+    route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl);
     expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]);
   } else if (blockIdx.x == 0) {
     float p = 0.0f;
@@ -172,15 +187,17 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
     case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; \
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
 
-int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y) {
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y, const RouteSrc* routed) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
-  int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc;
+  if (routed && (routed->nsl < 1 || routed->nsl > 64 || routed->r64 < m.n_exp)) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: %d router slices of %d rows", routed->nsl, routed->r64);
+  if (!routed) { int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc; }
+  const float* lg = routed ? routed->p : w.logits; const int nsl = routed ? routed->nsl : 1, sstride = routed ? t * routed->r64 : 0, tstride = routed ? routed->r64 : m.n_exp;
   auto mat_bytes = [](const QMatDev& q, double rows) { return qmat_gguf_bytes(q, rows); };
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
-  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, w.logits, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2)); }
+  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride)); }
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
   MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }

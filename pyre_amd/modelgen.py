@@ -60,6 +60,7 @@ class Config:
     # reach the hundreds, every sigmoid saturates and the network becomes chaotic in f32 (f32 and f64 evaluations of
     # the same weights then differ by percents), which would make any parity statement meaningless
     hc_d_div: float = 64.0
+    router_type: int = synth.BF16         # ffn_gate_inp: bf16, f32 or f16
 
     @property
     def ch(self):
@@ -103,7 +104,7 @@ def tensor_specs(c: Config):
                     (il, LIN_A, "vec:a", synth.F32, 1, c.lin_nv), (il, LIN_DT, "vec:dt", synth.F32, 1, c.lin_nv),
                     (il, LIN_CONV, "vec:conv", synth.F32, 1, c.ch * c.conv_k), (il, LIN_NORM, "vec:norm1", synth.F32, 1, c.lin_dv),
                     (il, LIN_OUT, "q", c.qtype, c.d, c.lin_nv * c.lin_dv)]
-        out += [(il, ROUTER, "router", synth.BF16, c.n_exp, c.d), (il, GATE_E, "q", c.qtype, c.n_exp * c.ff_exp, c.d),
+        out += [(il, ROUTER, "router", c.router_type, c.n_exp, c.d), (il, GATE_E, "q", c.qtype, c.n_exp * c.ff_exp, c.d),
                 (il, UP_E, "q", c.qtype, c.n_exp * c.ff_exp, c.d), (il, DOWN_E, "q", c.qtype, c.n_exp * c.d, c.ff_exp),
                 (il, SH_GATE_INP, "vec:small", synth.F32, 1, c.d), (il, SH_GATE, "q", c.qtype, sf, c.d),
                 (il, SH_UP, "q", c.qtype, sf, c.d), (il, SH_DOWN, "q", c.qtype, c.d, sf)]
@@ -144,7 +145,10 @@ def host_tensor(c: Config, seed, il, slot, kind, ty, rows, cols):
             return (x if ty == synth.F32 else x.astype(np.float16)).view(np.uint8).reshape(-1).copy()
         return synth.matrix(ty, rows, cols, s, *scale_range(c, il, slot, ty))
     if kind == "router":
-        return synth.bf16_normal(rows, cols, s, 0.02)
+        if ty == synth.BF16:
+            return synth.bf16_normal(rows, cols, s, 0.02)
+        x = synth.normal((rows, cols), s, 0.02)
+        return (x if ty == synth.F32 else x.astype(np.float16)).view(np.uint8).reshape(-1).copy()
     name = kind.split(":")[1]
     if name == "norm1":
         v = synth.normal((cols,), s, 0.1, 1.0)

@@ -53,6 +53,32 @@ def test_forward_logits_and_state_match_oracle(ctx, qtype, hc_type):
     assert relerr(k.reshape(-1), os_.kcache(0)) <= 1e-4 and relerr(v.reshape(-1), os_.vcache(0)) <= 1e-4
 
 
+@pytest.mark.parametrize("router_type,hc_type,rides", [(synth.BF16, synth.IQ3_S, True), (synth.F32, synth.BF16, True), (synth.F32, synth.F32, True), (synth.BF16, synth.F16, True),
+                                                       (synth.F16, synth.BF16, False), (synth.BF16, synth.Q8_0, False)])
+def test_router_riding_on_the_mix_equals_the_separate_router_launch(ctx, router_type, hc_type, rides, monkeypatch):
+    """The router GEMV as K slices left by the mix's second launch (bf16 / f32 routers behind IQ3_S / bf16 / f16 / f32
+    mixes) against the separate launch: same experts, logits within 1e-5 of each other and of the oracle's 1e-4; other
+    type pairs keep the separate launch."""
+    c = small_cfg(qtype=synth.IQ3_S, hc_type=hc_type, hc_lr=256 if synth.GEOM[hc_type][0] == 256 else 64, router_type=router_type, n_exp=64, top_k=6)
+    hw, gm, om = pair(ctx, c, 31)
+    ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88, 5, 6], dtype=np.uint32)
+    out = {}
+    for on in ("1", "0"):
+        monkeypatch.setenv("PYRE_ROUTER_RIDES", on)
+        st = gm.new_state(64)
+        ctx.prof_reset(); ctx.prof_enable(True)
+        lg = [gm.forward(ids[:8], st), gm.forward(ids[8:], st)] + [gm.forward(ids[i:i + 1], st) for i in range(3)]
+        prof = ctx.prof_report(); ctx.prof_enable(False)
+        out[on] = (lg, prof)
+    assert ("hc_up_mix_router" in out["1"][1]) == rides and "hc_up_mix_router" not in out["0"][1]
+    os_ = om.new_state()
+    lo = [om.forward(ids[:8], os_), om.forward(ids[8:], os_)] + [om.forward(ids[i:i + 1], os_) for i in range(3)]
+    for a, b, o in zip(out["1"][0], out["0"][0], lo):
+        assert relerr(a, b) <= 1e-5 and relerr(a, o) <= 1e-4 and orc.argmax(a) == orc.argmax(b) == orc.argmax(o)
+        if not rides:
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_greedy_stream_identical_to_oracle_across_the_packing_boundary(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 6)

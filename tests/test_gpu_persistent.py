@@ -20,6 +20,7 @@ def ctx():
 
 def run(gm, prompt, first, n, mega):
     os.environ["PYRE_MEGA"] = "2" if mega else "0"
+    os.environ["PYRE_ROUTER_RIDES"] = "0"          # the persistent kernel mirrors the stage path with a separate router GEMV
     try:
         st = gm.new_state(len(prompt) + n + 8)
         gm.forward(prompt, st, want_logits=False)
@@ -29,7 +30,7 @@ def run(gm, prompt, first, n, mega):
         nxt = gm.forward(np.array([toks[-1]], dtype=np.uint32), st)
         return toks, conv, ssm, k, v, nxt, len(st)
     finally:
-        os.environ.pop("PYRE_MEGA", None)
+        os.environ.pop("PYRE_MEGA", None); os.environ.pop("PYRE_ROUTER_RIDES", None)
 
 
 @pytest.mark.parametrize("n_prompt,n", [(10, 24), (100, 96)])
