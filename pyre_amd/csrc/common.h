@@ -28,6 +28,7 @@ struct pyre_ctx {
   std::string prof_text;
   unsigned* fuse_ctl = nullptr;                        // control words of in-launch barriers (zeroed once): [0] generation, [16] abort, [32] count
   void* mfma_buf = nullptr; size_t mfma_bytes = 0;     // split activations of the matrix-core verify GEMM (grow-only)
+  void* i8_buf = nullptr; size_t i8_bytes = 0;         // fixed-point activation digits of the integer-dot GEMV (grow-only)
 };
 
 // Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
@@ -99,6 +100,12 @@ int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint3
 // ~1e-7 relative (not bit for bit).
 bool pyre_gemm_mfma_ok(const QMatDev& m, int t);
 int pyre_gemm_mfma_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+
+// IQ3_S GEMV with integer dot products over block-fixed-point activations (gemv_i8.hip), 1 <= t <= 8: y[t][rows] as
+// pyre_gemv_launch, within 2^-23 of each unit's largest activation of it; per-token results do not depend on t.
+// best (t = 1, optional): per-tile maxima as pyre_gemv_argmax_launch.
+bool pyre_gemv_i8_ok(const QMatDev& m, int t);
+int pyre_gemv_i8_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, uint32_t* best_dev);
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {

@@ -95,6 +95,7 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->d_iq3s) (void)hipFree(ctx->d_iq3s);
   if (ctx->d_cb) (void)hipFree(ctx->d_cb);
   if (ctx->mfma_buf) (void)hipFree(ctx->mfma_buf);
+  if (ctx->i8_buf) (void)hipFree(ctx->i8_buf);
   if (ctx->fuse_ctl) (void)hipFree(ctx->fuse_ctl);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
   for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }

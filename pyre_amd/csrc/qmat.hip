@@ -411,10 +411,17 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
+// The operator's own launch: IQ3_S goes through the integer-dot GEMV (for every t, so a token's result does not depend
+// on the window width); PYRE_QMATMUL_F32=1 keeps the f32 lane = row GEMV the model's layers use.
+static int qmatmul_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev) {
+  static const int f32_only = env_int("PYRE_QMATMUL_F32", 0);
+  if (!f32_only && pyre_gemv_i8_ok(m, t)) return pyre_gemv_i8_launch(ctx, m, x_dev, t, y_dev, nullptr);
+  return pyre_gemv_launch(ctx, m, x_dev, t, y_dev);
+}
 int pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
-  return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
+  return qmatmul_launch(ctx, m->dv, x_dev, t, y_dev);
 }
 int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) {
   if (!ctx || !m || !x_host || !y_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
@@ -423,7 +430,7 @@ int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, 
   void* st; int rc = pyre_stage(ctx, xo + yb, &st); if (rc) return rc;
   float* xd = (float*)st; float* yd = (float*)((uint8_t*)st + xo);
   PYRE_HIP(ctx, hipMemcpyAsync(xd, x_host, xb, hipMemcpyHostToDevice, ctx->stream));
-  rc = pyre_gemv_launch(ctx, m->dv, xd, t, yd); if (rc) return rc;
+  rc = qmatmul_launch(ctx, m->dv, xd, t, yd); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(y_host, yd, yb, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
