@@ -77,6 +77,14 @@ int    pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_h
  * multi-token verify pass equal one-token decode (qwen4exp_gguf.rs:2357-2360). */
 int    pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
+/* IQ3_S matrices take pyre_qmatmul through integer dot products: each 64-column unit of x is first written as block
+ * fixed point (power-of-two scale, 23-bit signed integers; |error| <= 2^-23 of the unit's largest magnitude), the
+ * products with the 4-bit codes are exact in int32 and the block scales are applied in f32.  A non-finite activation
+ * makes every output NaN.  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the model's layers use
+ * (QMat::matmul's own arithmetic, gguf_q.rs:169-197,233-241: f32 products, f32 accumulation); for every other type
+ * the two are the same code. */
+int    pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
+int    pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
 /* The batch 2..8 speculative-verify GEMM on the matrix cores (the reference's verify kernels, src/model/qn_cube.rs:17,6454,
  * and lcm_dense, qwen4exp_gguf.rs:2641-2737): IQ3_S matrices, t in 2..8.  Same contract as pyre_qmatmul; the result
  * agrees with it to about 1e-7 of max|y| but not bit for bit (f16 two-term split of the activations, f32 accumulation). */

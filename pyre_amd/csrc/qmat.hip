@@ -412,27 +412,31 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
 }
 
 // The operator's own launch: IQ3_S goes through the integer-dot GEMV (for every t, so a token's result does not depend
-// on the window width); PYRE_QMATMUL_F32=1 keeps the f32 lane = row GEMV the model's layers use.
-static int qmatmul_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev) {
+// on the window width); f32_path (or PYRE_QMATMUL_F32=1) keeps the f32 lane = row GEMV the model's layers use.
+static int qmatmul_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, bool f32_path) {
   static const int f32_only = env_int("PYRE_QMATMUL_F32", 0);
-  if (!f32_only && pyre_gemv_i8_ok(m, t)) return pyre_gemv_i8_launch(ctx, m, x_dev, t, y_dev, nullptr);
+  if (!f32_path && !f32_only && pyre_gemv_i8_ok(m, t)) return pyre_gemv_i8_launch(ctx, m, x_dev, t, y_dev, nullptr);
   return pyre_gemv_launch(ctx, m, x_dev, t, y_dev);
 }
-int pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
+static int qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev, bool f32_path) {
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
-  return qmatmul_launch(ctx, m->dv, x_dev, t, y_dev);
+  return qmatmul_launch(ctx, m->dv, x_dev, t, y_dev, f32_path);
 }
-int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) {
+static int qmatmul_host(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host, bool f32_path) {
   if (!ctx || !m || !x_host || !y_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
   size_t xb = (size_t)t * m->cols * sizeof(float), yb = (size_t)t * m->rows * sizeof(float), xo = (xb + 255) & ~(size_t)255;
   void* st; int rc = pyre_stage(ctx, xo + yb, &st); if (rc) return rc;
   float* xd = (float*)st; float* yd = (float*)((uint8_t*)st + xo);
   PYRE_HIP(ctx, hipMemcpyAsync(xd, x_host, xb, hipMemcpyHostToDevice, ctx->stream));
-  rc = qmatmul_launch(ctx, m->dv, xd, t, yd); if (rc) return rc;
+  rc = qmatmul_launch(ctx, m->dv, xd, t, yd, f32_path); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(y_host, yd, yb, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
+int pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, false); }
+int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, false); }
+int pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, true); }
+int pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, true); }
 
 }  // extern "C"

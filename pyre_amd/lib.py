@@ -45,6 +45,8 @@ def _declare(L):
         "pyre_qmat_row": (i32, [vp, vp, sz, vp]),
         "pyre_qmatmul": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_dev": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmatmul_f32": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmatmul_f32_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
         "pyre_gguf_open": (i32, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
         "pyre_gguf_close": (None, [vp]),
@@ -255,6 +257,13 @@ class QMat:
         t = x.shape[0] if t is None else t
         y = np.empty((t, self.rows), dtype=np.float32)
         self.ctx.check(self.ctx.L.pyre_qmatmul(self.ctx.h, self.h, _ptr(x), t, _ptr(y)), "qmatmul")
+        return y
+
+    def matmul_f32(self, x):
+        """matmul on the f32 multiply-add GEMV the model's layers use (IQ3_S: matmul itself takes integer dot products)."""
+        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
+        y = np.empty((x.shape[0], self.rows), dtype=np.float32)
+        self.ctx.check(self.ctx.L.pyre_qmatmul_f32(self.ctx.h, self.h, _ptr(x), x.shape[0], _ptr(y)), "qmatmul_f32")
         return y
 
     def matmul_mfma(self, x):

@@ -134,6 +134,57 @@ def test_result_for_a_token_does_not_depend_on_batch_width(ctx, ty):
     assert np.array_equal(bits(m.matmul(x[3:4])), bits(y8[3:4]))
     # and it is reproducible run to run (split-K partials are added in a fixed order)
     assert np.array_equal(bits(m.matmul(x)), bits(y8))
+    y8f = m.matmul_f32(x)
+    for t in (1, 3):
+        assert np.array_equal(bits(m.matmul_f32(x[:t])), bits(y8f[:t])), t
+
+
+# ---- IQ3_S: the operator's integer-dot path (matmul) beside the f32 multiply-add path the layers use (matmul_f32) ------
+@pytest.mark.parametrize("rows,cols", [(320, 2048), (4096, 2048), (2048, 4096), (2048, 512), (100, 256)])
+def test_iq3s_both_paths_match_truth_and_each_other(ctx, rows, cols):
+    raw = synth.matrix(lib.IQ3_S, rows, cols, 131)
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
+    W = orc.dequant(lib.IQ3_S, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    for t in (1, 2, 3, 5, 8):
+        x = synth.normal((t, cols), 141 + t)
+        truth = x.astype(np.float64) @ W.T
+        yi, yf = m.matmul(x), m.matmul_f32(x)
+        assert relerr(yi, truth) <= TOL and relerr(yf, truth) <= TOL, t
+        assert relerr(yi, yf) <= 2e-6, t
+        for i in range(t):           # per token, whatever the window width, on both paths
+            assert np.array_equal(bits(m.matmul(x[i:i + 1])), bits(yi[i:i + 1]))
+            assert np.array_equal(bits(m.matmul_f32(x[i:i + 1])), bits(yf[i:i + 1]))
+
+
+def test_iq3s_integer_path_block_fixed_point_edge_cases(ctx):
+    rows, cols = 256, 1024
+    raw = synth.matrix(lib.IQ3_S, rows, cols, 151)
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
+    W = orc.dequant(lib.IQ3_S, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    g = np.random.Generator(np.random.PCG64(152))
+    x = synth.normal((6, cols), 153)
+    x[0, 5] = 3.0e4; x[0, 700] = -2.0e4                       # outliers: only their own 64-column units lose resolution
+    x[1] *= np.exp2(g.integers(-40, 40, cols // 64).repeat(64)).astype(np.float32)      # every unit on its own power of two
+    x[2] = 0.0; x[2, 64:128] = synth.normal((64,), 154)       # all-zero units beside one live unit
+    x[3] *= 1e-30                                             # tiny but normal magnitudes
+    x[4] *= 1e30
+    x[5, ::2] = 0.0
+    with np.errstate(all="ignore"):
+        truth = x.astype(np.float64) @ W.T
+    y = m.matmul(x)
+    for i in range(6):
+        assert relerr(y[i], truth[i]) <= TOL, i
+    # exactly representable activations (small integers): the integer path is exact up to the f32 scale products
+    xi = g.integers(-1000, 1000, (1, cols)).astype(np.float32)
+    assert relerr(m.matmul(xi), xi.astype(np.float64) @ W.T) <= 2e-7
+    # a power-of-two scaling of the input scales the output exactly
+    a = synth.normal((1, cols), 155)
+    assert np.array_equal(bits(m.matmul(a * 1024.0)), bits(m.matmul(a) * 1024.0))
+    # a non-finite activation: every output is NaN (the f32 path gives inf or NaN row by row)
+    bad = synth.normal((1, cols), 156); bad[0, 3] = np.inf
+    assert np.isnan(m.matmul(bad)).all()
+    bad[0, 3] = np.nan
+    assert np.isnan(m.matmul(bad)).all()
 
 
 def test_linearity_and_zero_input(ctx):
@@ -143,6 +194,8 @@ def test_linearity_and_zero_input(ctx):
     ya, yb, yab = m.matmul(a), m.matmul(b), m.matmul(2 * a - b)
     assert relerr(yab, 2 * ya.astype(np.float64) - yb) <= 1e-5
     assert not m.matmul(np.zeros((1, cols), np.float32)).any()
+    assert not m.matmul_f32(np.zeros((1, cols), np.float32)).any()
+    assert relerr(m.matmul_f32(2 * a - b), 2 * m.matmul_f32(a).astype(np.float64) - m.matmul_f32(b)) <= 1e-5
 
 
 def test_vocab_head_shape_against_sampled_rows(ctx):
@@ -157,11 +210,14 @@ def test_vocab_head_shape_against_sampled_rows(ctx):
     raw = synth.matrix(ty, rows, cols, 4242)
     x = synth.normal((2, cols), 91)
     y = m.matmul(x)
+    yf = m.matmul_f32(x)
     sel = np.r_[0:64, 75000:75064, rows - 64:rows]
     rb = cols // el * bs
     Wsel = np.stack([orc.dequant(ty, raw[r * rb:(r + 1) * rb], cols) for r in sel]).astype(np.float64)
     truth = x.astype(np.float64) @ Wsel.T
     assert np.abs(y[:, sel] - truth).max() / np.abs(truth).max() <= TOL
+    assert np.abs(yf[:, sel] - truth).max() / np.abs(truth).max() <= TOL
+    assert relerr(y, yf) <= 2e-6
     # device generator == host generator, through the bit-exact dequant of a few rows
     for r in (0, 12345, rows - 1):
         assert np.array_equal(bits(m.row(r)), bits(orc.dequant(ty, raw[r * rb:(r + 1) * rb], cols)))
