@@ -132,7 +132,8 @@ def bench_gemv(args):
     alg_bytes = mats[0].gguf_bytes + 4 * t * cols + 4 * t * rows
     traffic = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary, when present
     try:
-        for line in open(os.path.join(ROOT, "profiles", "gemv_iq3s_vocab_head_kernel_stats.txt")):
+        prof_file = "gemv_iq3s_vocab_head_kernel_stats.txt" if os.environ.get("PYRE_QMATMUL_F32") == "1" else "gemv_i8_iq3s_vocab_head_kernel_stats.txt"
+        for line in open(os.path.join(ROOT, "profiles", prof_file)):
             if t == 1 and ty == lib.IQ3_S and line.startswith("traffic_bytes_per_launch:"):
                 traffic = int(line.split(":")[1])
     except OSError:
