@@ -77,7 +77,7 @@ struct pyre_qmat {
 //   co:   rows < ch are the channels of a causal depthwise conv1d (kernel kk, weights conv_w[ch][kk]); the lane that
 //         owns a row runs the window's tokens in order, o = w[kk-1]*cur + sum_j w[j]*state[j], co[t][row] = silu(o),
 //         and slides the row's state conv_in -> conv_out ([kk-1][ch], oldest first; in == out is fine).
-struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; };
+struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; int four_waves; };
 // launchers implemented in qmat.hip, used by the block / model code
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 // waves per workgroup and units per wave the (unsplit) GEMV uses for this matrix
@@ -85,6 +85,13 @@ void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw);
 // K range split over `ksplit` workgroups per row tile; partial[(ks*t_count + t)*tiles*64 + row] holds the slice sums and
 // the consumer adds them in slice order.
 int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit);
+// Few row tiles, long rows (an output projection): the sixteen waves of pyre_gemv_launch's plan, same units each, as
+// four workgroups of four waves per row tile (the work of a tile on four compute units instead of one).  Each
+// workgroup leaves the sum of its waves, parts[(q*t_count + t)*tiles*64 + row], q < PYRE_GEMV_PARTS; the consumer adds the
+// parts in order from the first.
+#define PYRE_GEMV_PARTS 4
+bool pyre_gemv_parts_ok(const QMatDev& m);
+int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* parts_dev);
 // t = 1 GEMV that also leaves, per row tile, (bits of the maximum, first row holding it) in best[2*tile], best[2*tile+1].
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev);
 // y as pyre_gemv_launch (raw projections), plus the conv epilogue described at GemvEpi (best ignored).
@@ -165,7 +172,7 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // router row; the gate/up launch adds the d/64 slices (RouteSrc).  bf16 and f32 routers, at most 64 slices.
 struct HcRoute { QMatDev router; float* part; };
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr);
+                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr, int comb_parts = 1);
 bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router);
 // waves per workgroup, units per wave and K slices of the norm + [down ; inject] kernel; false if the shape is unsupported
 bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit);

@@ -14,10 +14,22 @@ __device__ __forceinline__ float sigm(float x) { return 1.0f / (1.0f + expf(-x))
 
 // Stream element i of token ti with the pending residual update applied: x + out * w  (:1384-1387), w = 2*sigm(inj).
 // `out` is a plain [t][d] vector (comb_out) or the unreduced FFN output (mo.partial != nullptr).
-__device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, const MoeOut& mo, float w, int d, int ti, int s, int i) {
+// NP > 1: `out` comes as NP partial vectors, part q of token ti at comb_out + (q*T + ti)*d, added in order from the first
+// (pyre_gemv_parts_launch); all parts are fetched before the first add.
+template <int T, int NP> __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, const MoeOut& mo, float w, int d, int ti, int s, int i) {
   float v = x_in[(size_t)ti * in_ts + (size_t)s * in_ss + i];
-  if (mo.partial) v = v + moe_out_value(mo, ti, i) * w;
-  else if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
+  if constexpr (NP > 1) {
+    float sv[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) sv[q] = (comb_out + ((size_t)q * T + ti) * d)[i];
+    float o = sv[0];
+#pragma unroll
+    for (int q = 1; q < NP; ++q) o += sv[q];
+    v = v + o * w;
+  } else {
+    if (mo.partial) v = v + moe_out_value(mo, ti, i) * w;
+    else if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
+  }
   return v;
 }
 
@@ -53,7 +65,7 @@ template <int T> __device__ __forceinline__ void hc_load_slices(float (&pv)[32],
 //      squares of x_new are summed over the slice -> ssq[ks*T + t]; the tile-0 workgroup of the slice also publishes the
 //      updated stream (x_out, never the buffer x_in points into)
 //   2. each wave takes upw units of the slice; partial sums -> part[(ks*T + t)*tiles*64 + row]
-template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
+template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_norm_down(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
     const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq,
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
@@ -73,7 +85,7 @@ template <int FMT, int T> __global__ __launch_bounds__(512) void k_hc_norm_down(
     const float nv = norm[(size_t)s * d + i0 + j];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      float v = hc_x_new(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
+      float v = hc_x_new<T, NP>(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + j);
       ss[t] += v * v;
       xs[(size_t)t * L + j] = v * nv;
       if (tile == 0) x_out[((size_t)t * hc + s) * d + i0 + j] = v;
@@ -217,11 +229,13 @@ DownPlan down_plan(const HcDev& h) {
 }
 
 template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out,
-                                               const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
+                                               const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj, float eps) {
   const int L = p.nw * p.upw * 64; size_t lds = 4 * ((size_t)T * L + (size_t)p.nw * T * 64 + (size_t)p.nw * T);
   ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
-  hipLaunchKernelGGL((k_hc_norm_down<FMT, T>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc,
-                     w.ssq, w.o, p.upw, (const uint2*)ctx->d_iq2xs);
+#define NORM_DOWN_GO(NP) hipLaunchKernelGGL((k_hc_norm_down<FMT, T, NP>), dim3(h.di.tiles, p.ksplit), dim3(p.nw * 64), lds, ctx->stream, h.di, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, \
+                     w.ssq, w.o, p.upw, (const uint2*)ctx->d_iq2xs)
+  if constexpr (FMT == FMT_IQ3_S) { if (comb_parts > 1) NORM_DOWN_GO(PYRE_GEMV_PARTS); else NORM_DOWN_GO(1); } else NORM_DOWN_GO(1);
+#undef NORM_DOWN_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
@@ -245,8 +259,8 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; BODY } case FMT_Q4_K: { constexpr int F = FMT_Q4_K; BODY } case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; BODY } \
     case FMT_C4: { constexpr int F = FMT_C4; BODY } case FMT_C8: { constexpr int F = FMT_C8; BODY } \
     default: { constexpr int F = FMT_IQ3_S; BODY } }
-int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut& mo, const float* comb_inj, float eps) {
-  HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, eps))
+int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj, float eps) {
+  HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, comb_parts, mo, comb_inj, eps))
 }
 int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
   HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt))
@@ -269,8 +283,9 @@ void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
 }
 
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed, float* inj, const HcRoute* route) {
+                       float eps, float* mixed, float* inj, const HcRoute* route, int comb_parts) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
+  if (comb_parts != 1 && !(comb_parts == PYRE_GEMV_PARTS && h.di.fmt == FMT_IQ3_S && comb_out && !comb_moe)) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: %d partial vectors (1, or %d with an IQ3_S mix)", comb_parts, PYRE_GEMV_PARTS);
   if (route && !pyre_hc_route_ok(h, route->router)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: this router cannot ride on the mix");
   if (x_in == x_out) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: the updated streams must go to another buffer");
   if (h.d % 64 || h.lr % 64 || h.hc * h.up.U > 16 || h.up.tiles != h.hc * (h.d / 64) || h.di.U != h.hc * (h.d / 64))
@@ -284,7 +299,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   // (4.48 vs 4.26 ms per token) -- the dependent memory round trips of a stage cost the same inside one kernel, and
   // the barrier with its cache-bypassing hand-off costs more than the kernel boundary it replaces.
   static const bool fused_ok = getenv("PYRE_HC_FUSED") && atoi(getenv("PYRE_HC_FUSED")) != 0;
-  if (t == 1 && fused_ok && !route && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
+  if (t == 1 && fused_ok && !route && comb_parts == 1 && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
     const int nwg = std::max(h.di.tiles * p.ksplit, h.d / 64), L = p.nw * p.upw * 64;
     const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64 + 32) + 64;
     if (nwg <= 240 && lds <= 60000) {
@@ -299,7 +314,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
       PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
     }
   }
-  int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, mo, comb_inj, eps); if (rc) return rc;
+  int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj, eps); if (rc) return rc;
   return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route);
 }
 

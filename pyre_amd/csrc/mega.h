@@ -88,7 +88,7 @@ __device__ __forceinline__ bool launch_sync(unsigned* ctl, int nwg, unsigned lim
 
 // ---- device-side description of the model and of one run --------------------------------------------------------------
 struct HcPlan { int nw, upw, ksplit; };
-struct GemvPlan { int nw, upw; };
+struct GemvPlan { int nw, upw; int grp = 0; };      // grp > 1: the waves' sums are added in groups of grp, then the groups (the stage path's K slices)
 struct Layer {
   HcDev hca, hcf; HcPlan pa, pf;
   QMatDev proj, outp; GemvPlan gp, go, gr;      // gr: router
@@ -271,7 +271,10 @@ template <int FMT> __device__ __forceinline__ void st_gemv(const QMatDev& m, con
     __syncthreads();
     if (act && vt < 64) {
       float s = red[lane];
-      for (int w = 1; w < nw; ++w) s += red[w * 64 + lane];
+      if (gp.grp > 1) {
+        for (int w = 1; w < gp.grp; ++w) s += red[w * 64 + lane];
+        for (int g = gp.grp; g < nw; g += gp.grp) { float gs = red[g * 64 + lane]; for (int w = 1; w < gp.grp; ++w) gs += red[(g + w) * 64 + lane]; s += gs; }
+      } else for (int w = 1; w < nw; ++w) s += red[w * 64 + lane];
       const size_t row = (size_t)tile * 64 + lane;
       if (row < (size_t)m.rows) stc(y + row, s);
       if (ep.best != nullptr) {

@@ -186,12 +186,12 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
   MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
   size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
-  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
+  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
                  al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + al256(rp_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
-  m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
+  m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
@@ -337,6 +337,8 @@ struct WinOpt {
   bool inplace = false;         // update the recurrent state in its current buffer (no pre-window copy for spec_keep)
 };
 
+bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) && (int)L.outp.rows == d && L.hcf.di.fmt == FMT_IQ3_S; }
+
 // One window of t <= 8 tokens (ids in m->ids unless from_best).
 int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
@@ -365,10 +367,12 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true))) return rc;
       s->cur[li] = nb;
     }
-    if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
+    int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
+    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o))) return rc; }
+    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
     const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
     HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
-    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
     advance();
     if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y, ride ? &rs : nullptr))) return rc;
     if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
@@ -413,7 +417,7 @@ bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
     else if (L.gdn.nv % L.gdn.nk) return false;
     if ((size_t)L.proj.cols * 4 + 4096 > mega::LDS_BYTES || (size_t)L.outp.cols * 4 + 4096 > mega::LDS_BYTES) return false;
     M.hca = L.hca; M.hcf = L.hcf; M.proj = L.proj; M.outp = L.outp; M.moe = L.moe; M.attn = L.attn; M.gdn = L.gdn; M.full = L.full ? 1 : 0;
-    pyre_gemv_plan(L.proj, &M.gp.nw, &M.gp.upw); pyre_gemv_plan(L.outp, &M.go.nw, &M.go.upw); pyre_gemv_plan(mo.router, &M.gr.nw, &M.gr.upw);
+    pyre_gemv_plan(L.proj, &M.gp.nw, &M.gp.upw); pyre_gemv_plan(L.outp, &M.go.nw, &M.go.upw); M.go.grp = outp_in_parts(L, c.d) ? M.go.nw / PYRE_GEMV_PARTS : 0; pyre_gemv_plan(mo.router, &M.gr.nw, &M.gr.upw);
   }
   if ((size_t)c.d * 4 + 8192 + sizeof(mega::RouteLds) > mega::LDS_BYTES) return false;
   hipDeviceProp_t prop; if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return false;

@@ -257,7 +257,7 @@ template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDe
 // Waves per workgroup: enough that a row tile's whole K range is covered by one workgroup with few units per wave,
 // fewer when there are so many tiles that the chip is full anyway.
 template <int FMT, int T> int gemv_t(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
-  int nw = gemv_nw(m, ksplit);
+  int nw = ep.four_waves ? 4 : gemv_nw(m, ksplit);
   if (nw == 4) return gemv_launch_nw<FMT, T, 4>(ctx, m, x, y, ksplit, ep);
   if (nw == 8) return gemv_launch_nw<FMT, T, 8>(ctx, m, x, y, ksplit, ep);
   return gemv_launch_nw<FMT, T, 16>(ctx, m, x, y, ksplit, ep);
@@ -284,6 +284,17 @@ int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, flo
 int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* partial, int ksplit) {
   int rc = PYRE_OK;
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, partial, ksplit, GemvEpi{}));
+  return rc;
+}
+bool pyre_gemv_parts_ok(const QMatDev& m) {
+  static const int off = env_int("PYRE_GEMV_PARTS", 1) == 0;
+  return !off && m.tiles <= 64 && gemv_nw(m, 1) == 16 && m.U % 16 == 0 && m.U / 16 >= 2 && m.rows == m.tiles * 64;
+}
+int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* parts) {
+  if (!pyre_gemv_parts_ok(m)) return pyre_fail(ctx, PYRE_E_SHAPE, "gemv: the four-part form needs few row tiles and rows of a multiple of 32 units");
+  int rc = PYRE_OK;
+  GemvEpi ep{}; ep.four_waves = 1;
+  FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep));
   return rc;
 }
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best) {
