@@ -157,6 +157,8 @@ void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
 // p[(s*T + t)*r64 + e], s = 0..nsl-1, added in slice order.
 struct RouteSrc { const float* p; int nsl; int r64; };
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr);
+// K parts the gate/up dot products are summed in (1 or 2; k_moe_gu)
+int pyre_moe_gu_parts(const MoeDev& m);
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows

@@ -95,6 +95,7 @@ struct Layer {
   MoeDev moe; AttnDev attn; GdnDev gdn; KvDev kv;
   float* conv; float* ssm; float* proj_saved;    // DeltaNet: current state buffers (updated in place), raw projections [pw_lin]
   int full;
+  int gu_parts;         // K parts of the gate/up dot products (pyre_moe_gu_parts)
 };
 struct Args {
   const Layer* layers; int n_layers;
@@ -652,9 +653,9 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
     L.s_w[e] = w;
   }
 }
-template <int FMT> __device__ __forceinline__ void st_route_gu(const MoeDev& m, const float* logits, int32_t* sel_idx, float* sel_w, float* sg, const float* x, float* h, int hstride, char* lds) {
-  constexpr int NW = 16;
-  float* xs = (float*)lds; float* red = xs + m.d; RouteLds& rl = *(RouteLds*)(red + 2 * NW * 64);
+template <int FMT> __device__ __forceinline__ void st_route_gu(const MoeDev& m, const float* logits, int32_t* sel_idx, float* sel_w, float* sg, const float* x, float* h, int hstride, int parts, char* lds) {
+  constexpr int NW = 16, PMAX = 2;       // red: [gate, up][part][wave][64]
+  float* xs = (float*)lds; float* red = xs + m.d; RouteLds& rl = *(RouteLds*)(red + 2 * PMAX * NW * 64);
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int tiles = hstride / 64, k1 = m.top_k + 1, nvb = tiles * k1;
   if ((int)blockIdx.x >= nvb) return;
@@ -679,15 +680,23 @@ template <int FMT> __device__ __forceinline__ void st_route_gu(const MoeDev& m, 
     }
     const QMatDev& Gm = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
     const int tile = (shared ? 0 : expert * (m.ff >> 6)) + bx;
-    const int upw = (Gm.U + NW - 1) / NW, k0 = wave * upw, kend = min(Gm.U, k0 + upw);
-    float ag[1] = {0.0f}, au[1] = {0.0f};
-    for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(Gm, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, au); }
-    red[wave * 64 + lane] = ag[0]; red[(NW + wave) * 64 + lane] = au[0];
+    // a dot product is the sum of its K parts in order, a part the sum of its wave shares in wave order (k_moe_gu)
+    const int upw = (Gm.U + NW * parts - 1) / (NW * parts);
+    for (int p = 0; p < parts; ++p) {
+      const int k0 = min(Gm.U, (p * NW + wave) * upw), kend = min(Gm.U, k0 + upw);
+      float ag[1] = {0.0f}, au[1] = {0.0f};
+      for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(Gm, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, au); }
+      red[(p * NW + wave) * 64 + lane] = ag[0]; red[((PMAX + p) * NW + wave) * 64 + lane] = au[0];
+    }
     __syncthreads();
     if (tid < 64) {
-      float g = red[lane], u = red[NW * 64 + lane];
+      float g = 0.0f, u = 0.0f;
+      for (int p = 0; p < parts; ++p) {
+        float gp = red[(p * NW) * 64 + lane], up = red[((PMAX + p) * NW) * 64 + lane];
 #pragma unroll
-      for (int w = 1; w < NW; ++w) { g += red[w * 64 + lane]; u += red[(NW + w) * 64 + lane]; }
+        for (int w = 1; w < NW; ++w) { gp += red[(p * NW + w) * 64 + lane]; up += red[((PMAX + p) * NW + w) * 64 + lane]; }
+        if (p == 0) { g = gp; u = up; } else { g += gp; u += up; }
+      }
       float s = 1.0f / (1.0f + expf(-g));
       stc(h + (size_t)j * hstride + bx * 64 + lane, (g * s) * u);
     }
@@ -830,7 +839,7 @@ template <int FW, int FR> __global__ __launch_bounds__(WGT) void k_decode(Args a
       st_gemv<FR>(L.moe.router, L.gr, a.mixed, a.mw.logits, Epi{nullptr, nullptr, nullptr, nullptr, 0, 0}, lds);
       MEGA_SYNC(9);
       const int hs = L.moe.ff > L.moe.sf ? L.moe.ff : L.moe.sf;
-      st_route_gu<FW>(L.moe, a.mw.logits, a.mw.sel_idx, a.mw.sel_w, a.mw.sg, a.mixed, a.mw.h, hs, lds);
+      st_route_gu<FW>(L.moe, a.mw.logits, a.mw.sel_idx, a.mw.sel_w, a.mw.sg, a.mixed, a.mw.h, hs, L.gu_parts, lds);
       MEGA_SYNC(10);
       st_moe_down<FW>(L.moe, a.mw.sel_idx, a.mw.h, hs, a.mw.partial, lds);
       MEGA_SYNC(11);

@@ -416,10 +416,10 @@ bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
     if (L.full) { int G = L.attn.nh / L.attn.nkv; if (L.attn.nh % L.attn.nkv || (G != 1 && G != 2 && G != 4 && G != 8)) return false; }
     else if (L.gdn.nv % L.gdn.nk) return false;
     if ((size_t)L.proj.cols * 4 + 4096 > mega::LDS_BYTES || (size_t)L.outp.cols * 4 + 4096 > mega::LDS_BYTES) return false;
-    M.hca = L.hca; M.hcf = L.hcf; M.proj = L.proj; M.outp = L.outp; M.moe = L.moe; M.attn = L.attn; M.gdn = L.gdn; M.full = L.full ? 1 : 0;
+    M.hca = L.hca; M.hcf = L.hcf; M.proj = L.proj; M.outp = L.outp; M.moe = L.moe; M.attn = L.attn; M.gdn = L.gdn; M.full = L.full ? 1 : 0; M.gu_parts = pyre_moe_gu_parts(L.moe);
     pyre_gemv_plan(L.proj, &M.gp.nw, &M.gp.upw); pyre_gemv_plan(L.outp, &M.go.nw, &M.go.upw); M.go.grp = outp_in_parts(L, c.d) ? M.go.nw / PYRE_GEMV_PARTS : 0; pyre_gemv_plan(mo.router, &M.gr.nw, &M.gr.upw);
   }
-  if ((size_t)c.d * 4 + 8192 + sizeof(mega::RouteLds) > mega::LDS_BYTES) return false;
+  if ((size_t)c.d * 4 + 2 * 8192 + sizeof(mega::RouteLds) > mega::LDS_BYTES) return false;
   hipDeviceProp_t prop; if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return false;
   int wgs = prop.multiProcessorCount; if (wgs > 256) wgs = 256; if (wgs < 32) return false;
   int per_cu = 0;

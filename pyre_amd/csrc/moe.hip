@@ -73,11 +73,18 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // grid (row tiles, entries), 16 waves; entry = ti*(k+1) + j, j < k: the j-th chosen expert of token ti (ascending id),
 // j == k: the shared expert.  Tile 0 of entry (ti, 0) publishes the token's expert ids and weights, tile 0 of the shared
 // entry publishes the shared-expert gate sigmoid(sh_gate_inp . x).
-template <int FMT, int NW>
+// The K range is cut into P parts of NW wave shares each; a dot product is the sum of its parts in order from the
+// first, a part the sum of its wave shares in wave order -- whatever the launch shape, so a token's result does not
+// depend on it.  gridDim.z == 1: the workgroup's wave w takes share w of every part (P accumulators) and stores
+// silu(g) * u.  gridDim.z == nz > 1 (P == 1 in the template, nz parts): workgroup kz takes part kz only -- an entry's 64
+// rows on nz compute units instead of one; at one token a launch of tiles x (k+1) workgroups leaves most of the chip
+// idle -- and leaves the part's raw sums, gate at h[((entry*nz + kz)*2 + 0)*hstride + row], up at [... + 1]; the down
+// launch adds the parts and forms silu(g) * u with the same operations.
+template <int FMT, int NW, int P>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
-  __shared__ float red[2][NW][64];
+  __shared__ float red[2][P][NW][64];
   __shared__ RouteLds rl;
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
@@ -100,34 +107,60 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
-    if (lane == 0) red[0][wave][0] = p;
+    if (lane == 0) red[0][0][wave][0] = p;
     __syncthreads();
-    if (threadIdx.x == 0) { float tot = 0.0f; for (int w = 0; w < NW; ++w) tot += red[0][w][0]; rl.s_w[0] = 1.0f / (1.0f + expf(-tot)); }
+    if (threadIdx.x == 0) { float tot = 0.0f; for (int w = 0; w < NW; ++w) tot += red[0][0][w][0]; rl.s_w[0] = 1.0f / (1.0f + expf(-tot)); }
     __syncthreads();
   }
   const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
   const int tile = (shared ? 0 : expert * (m.ff >> 6)) + blockIdx.x;
-  const int upw = (G.U + NW - 1) / NW, k0 = wave * upw, kend = min(G.U, k0 + upw);
-  float ag[1] = {0.0f}, au[1] = {0.0f};
-  // two units of both matrices are fetched before the first is consumed: a rolled loop would pay a memory round trip per unit
-  for (int ku = k0; ku < kend; ku += 2) {
-    const int kb = min(ku + 1, kend - 1);
-    UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ku, lane), u0 = unit_load<FMT>(Up, tile, ku, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
-    unit_fma<FMT, 1>(G, g0, ku, lds2, lane, xs + ku * 64, 0, ag); unit_fma<FMT, 1>(Up, u0, ku, lds2, lane, xs + ku * 64, 0, au);
-    if (ku + 1 < kend) { unit_fma<FMT, 1>(G, g1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, ag); unit_fma<FMT, 1>(Up, u1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, au); }
+  const int nz = gridDim.z, kz = blockIdx.z, np = P * nz;          // np parts in all
+  const int upw = (G.U + NW * np - 1) / (NW * np);
+  float ag[P][1], au[P][1];
+#pragma unroll
+  for (int p = 0; p < P; ++p) { ag[p][0] = 0.0f; au[p][0] = 0.0f; }
+  if (P == 2 && upw == 1) {
+    // one unit per part: both parts' units of both matrices are fetched before the first is consumed
+    const int ka = min(wave, G.U - 1), kb = min(NW + wave, G.U - 1);
+    UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ka, lane), u0 = unit_load<FMT>(Up, tile, ka, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
+    if (wave < G.U) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
+    if (NW + wave < G.U) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
+  } else {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const int k0 = min(G.U, ((kz * P + p) * NW + wave) * upw), kend = min(G.U, k0 + upw);
+      // two units of both matrices are fetched before the first is consumed: a rolled loop would pay a memory round trip per unit
+      for (int ku = k0; ku < kend; ku += 2) {
+        const int kb = min(ku + 1, kend - 1);
+        UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ku, lane), u0 = unit_load<FMT>(Up, tile, ku, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
+        unit_fma<FMT, 1>(G, g0, ku, lds2, lane, xs + ku * 64, 0, ag[p]); unit_fma<FMT, 1>(Up, u0, ku, lds2, lane, xs + ku * 64, 0, au[p]);
+        if (ku + 1 < kend) { unit_fma<FMT, 1>(G, g1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, ag[p]); unit_fma<FMT, 1>(Up, u1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, au[p]); }
+      }
+    }
   }
-  red[0][wave][lane] = ag[0]; red[1][wave][lane] = au[0];
+#pragma unroll
+  for (int p = 0; p < P; ++p) { red[0][p][wave][lane] = ag[p][0]; red[1][p][wave][lane] = au[p][0]; }
   __syncthreads();
   if (threadIdx.x < 64) {
-    float g = red[0][0][lane], u = red[1][0][lane];
+    float g = 0.0f, u = 0.0f;
 #pragma unroll
-    for (int w = 1; w < NW; ++w) { g += red[0][w][lane]; u += red[1][w][lane]; }
-    float s = 1.0f / (1.0f + expf(-g));
-    h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+    for (int p = 0; p < P; ++p) {
+      float gp = red[0][p][0][lane], up = red[1][p][0][lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) { gp += red[0][p][w][lane]; up += red[1][p][w][lane]; }
+      if (p == 0) { g = gp; u = up; } else { g += gp; u += up; }
+    }
+    if (nz == 1) {
+      float s = 1.0f / (1.0f + expf(-g));
+      h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+    } else {
+      float* hp = h + ((size_t)entry * nz + kz) * 2 * hstride + blockIdx.x * 64 + lane;
+      hp[0] = g; hp[hstride] = u;
+    }
   }
   // Publishing comes last: a global store ahead of the dot products would stop the compiler from keeping the
   // activations in scalar registers (it could no longer prove them unmodified).
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && kz == 0) {
     if (shared) { if (threadIdx.x == 0) sg[ti] = rl.s_w[0]; }
     else if (j == 0) {
       route_weights(m.top_k, rl);       // thread e < k writes and then reads its own s_w entry
@@ -137,20 +170,43 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
 }
 
 // ---- expert down: partial[entry][r] = down[r] . h[entry] ---------------------------------------------------------------
-template <int FMT, int NW>
+// NZ > 1: h arrives as the gate / up sums of NZ K parts (k_moe_gu with gridDim.z = NZ); each wave forms the 64 values of
+// a unit, silu(sum of gate parts) * (sum of up parts), in its own slice of shared memory while the unit's weights are
+// on their way (a wave's shared-memory operations execute in order: no workgroup barrier).
+template <int FMT, int NW, int NZ>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
                                                      const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   __shared__ float red[NW][64];
+  __shared__ float hx[NZ > 1 ? NW : 1][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == m.top_k;
   const QMatDev& D = shared ? m.sh_down : m.down_e;
   const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.d >> 6)) + blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int upw = (D.U + NW - 1) / NW, k0 = wave * upw, kend = min(D.U, k0 + upw);
-  const float* xs = h + (size_t)entry * hstride;
   float acc[1] = {0.0f};
-  for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
+  if constexpr (NZ == 1) {
+    const float* xs = h + (size_t)entry * hstride;
+    for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
+  } else {
+    const float* hp = h + (size_t)entry * NZ * 2 * hstride + lane;
+    for (int ku = k0; ku < kend; ++ku) {
+      UnitRaw<FMT> r = unit_load<FMT>(D, tile, ku, lane);
+      float gp[NZ], up[NZ];
+#pragma unroll
+      for (int q = 0; q < NZ; ++q) { gp[q] = hp[(size_t)(2 * q) * hstride + ku * 64]; up[q] = hp[(size_t)(2 * q + 1) * hstride + ku * 64]; }
+      float g = gp[0], u = up[0];
+#pragma unroll
+      for (int q = 1; q < NZ; ++q) { g += gp[q]; u += up[q]; }
+      float s = 1.0f / (1.0f + expf(-g));
+      __builtin_amdgcn_wave_barrier();
+      hx[wave][lane] = (g * s) * u;
+      __builtin_amdgcn_wave_barrier();
+      unit_fma<FMT, 1>(D, r, ku, lds2, lane, hx[wave], 0, acc);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
   red[wave][lane] = acc[0];
   __syncthreads();
   if (threadIdx.x < 64) {
@@ -170,15 +226,16 @@ __global__ void k_moe_sum(const float* __restrict__ partial, const float* __rest
   y[(size_t)ti * d + r] = yv + o;
 }
 
+#define PYRE_MOE_GU_NZMAX 2
 size_t pyre_moe_work_bytes(const MoeDev& m) {
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
-  return 256 * 8 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs + 8 * k1 * (size_t)m.d);
+  return 256 * 8 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d);
 }
 void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
   w->logits = (float*)take(4 * 8 * (size_t)m.n_exp); w->sel_idx = (int32_t*)take(4 * 8 * (size_t)m.top_k); w->sel_w = (float*)take(4 * 8 * (size_t)m.top_k);
-  w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
+  w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
 }
 
 #define MOE_FMT_DISPATCH(fmt, CALL) \
@@ -187,6 +244,13 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
     case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; \
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
 
+// K parts of the gate/up dot products (a property of the matrices, so that every window length gives a token the
+// same bits) and whether a window of t tokens launches one workgroup per part: only a single token does, whose
+// tiles x (k+1) workgroups would leave most of the chip idle.
+int pyre_moe_gu_parts(const MoeDev& m) {
+  static const bool off = getenv("PYRE_MOE_GU_PARTS") && atoi(getenv("PYRE_MOE_GU_PARTS")) == 0;
+  return (!off && m.gate_e.U % 32 == 0 && m.sh_gate.U == m.gate_e.U) ? 2 : 1;
+}
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y, const RouteSrc* routed) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
@@ -196,11 +260,15 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   auto mat_bytes = [](const QMatDev& q, double rows) { return qmat_gguf_bytes(q, rows); };
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
+  const int P = pyre_moe_gu_parts(m), nz = (P > 1 && t == 1) ? P : 1;
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
-  MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16>), dim3(hs / 64, entries), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride)); }
+#define GU_GO(PP, NZ) MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP>), dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride))
+  if (nz > 1 || P == 1) { GU_GO(1, nz); } else { GU_GO(2, 1); } }
+#undef GU_GO
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
-  MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
+  if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
+  else { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 2>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); } }
   PYRE_CHECK_LAUNCH(ctx);
   if (y) {
     ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
