@@ -445,33 +445,50 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
   }
 }
 
-// grid (nh, t), 4*HD threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
+// grid (nh, t, HD/64), 256 threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
 // Thread (grp, dim) adds the chunks grp, grp+4, ... in ascending order; the four groups are then added in order.
+// A workgroup owns 64 dimensions of a head and goes through the chunks 256 at a time: the 64 partial outputs a thread
+// needs of such a tile do not depend on the maximum, so the first tile's are fetched at the start, together with the
+// (max, sum) pairs; thread c of the tile then leaves exp(max_c - M) and sum_c in shared memory for everybody.  Up to
+// 256 chunks (32 768 positions) the whole merge is one memory round trip.
 template <int HD>
-__global__ __launch_bounds__(4 * HD) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                         int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
-  __shared__ float wmax[4 * HD / 64]; __shared__ float so[4][HD]; __shared__ float sl[4];
+__global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                      int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
+  constexpr int B = 64;
+  __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[256], ls[256];
   if (posp) start = *posp;
-  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / HD, dd = tid % HD;
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid >> 6, dd = blockIdx.z * 64 + (tid & 63);
   int n = start + ti + 1; if (pcount && pcount[ti] >= 0) n = pcount[ti];        // a position list: its entries are what the chunks covered
   const int nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
-  float M = -INFINITY; for (int c = tid; c < nc; c += 4 * HD) M = fmaxf(M, ml[2 * c]);
+  float pv[B];
+#pragma unroll
+  for (int i = 0; i < B; ++i) pv[i] = nc > 0 ? po[(size_t)min(grp + 4 * i, nc - 1) * HD + dd] : 0.0f;
+  float m0 = -INFINITY, l0 = 0.0f; if (tid < nc) { m0 = ml[2 * tid]; l0 = ml[2 * tid + 1]; }
+  float M = m0; for (int c = tid + 256; c < nc; c += 256) M = fmaxf(M, ml[2 * c]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
   if ((tid & 63) == 0) wmax[tid >> 6] = M;
   __syncthreads();
-  M = wmax[0];
-#pragma unroll
-  for (int i = 1; i < 4 * HD / 64; ++i) M = fmaxf(M, wmax[i]);
+  M = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   float L = 0.0f, o = 0.0f;
-#pragma unroll 4
-  for (int c = grp; c < nc; c += 4) { float f = expf(ml[2 * c] - M); L = fmaf(ml[2 * c + 1], f, L); o = fmaf(po[(size_t)c * HD + dd], f, o); }
-  so[grp][dd] = o; if (dd == 0) sl[grp] = L;
+  for (int cb = 0; cb < nc; cb += 256) {
+    if (cb > 0) {
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < B; ++i) pv[i] = po[(size_t)min(cb + grp + 4 * i, nc - 1) * HD + dd];
+      m0 = -INFINITY; l0 = 0.0f; if (cb + tid < nc) { m0 = ml[2 * (cb + tid)]; l0 = ml[2 * (cb + tid) + 1]; }
+    }
+    fs[tid] = expf(m0 - M); ls[tid] = l0;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < B; ++i) if (cb + grp + 4 * i < nc) { const float f = fs[grp + 4 * i]; L = fmaf(ls[grp + 4 * i], f, L); o = fmaf(pv[i], f, o); }
+  }
+  so[grp][tid & 63] = o; if ((tid & 63) == 0) sl[grp] = L;
   __syncthreads();
   if (grp == 0) {
-    o = ((so[0][dd] + so[1][dd]) + so[2][dd]) + so[3][dd]; L = ((sl[0] + sl[1]) + sl[2]) + sl[3];
+    o = ((so[0][tid] + so[1][tid]) + so[2][tid]) + so[3][tid]; L = ((sl[0] + sl[1]) + sl[2]) + sl[3];
     float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd];
     out[((size_t)ti * a.nh + h) * HD + dd] = (o / L) * a_sigm(gate);
   }
@@ -535,7 +552,7 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp, qw); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp, qw); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp, qw); break;
     default: launch_decode<8>(ctx, a, kv, w, start, t, posp, qw); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t), dim3(1024), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t, 256 / 64), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 
