@@ -683,7 +683,7 @@ template <int FMT> __device__ __forceinline__ void st_route_gu(const MoeDev& m, 
     // a dot product is the sum of its K parts in order, a part the sum of its wave shares in wave order (k_moe_gu)
     const int upw = (Gm.U + NW * parts - 1) / (NW * parts);
     for (int p = 0; p < parts; ++p) {
-      const int k0 = min(Gm.U, (p * NW + wave) * upw), kend = min(Gm.U, k0 + upw);
+      const int k0 = min(Gm.U, (wave * parts + p) * upw), kend = min(Gm.U, k0 + upw);
       float ag[1] = {0.0f}, au[1] = {0.0f};
       for (int ku = k0; ku < kend; ++ku) { unit_dot<FMT, 1>(Gm, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, ag); unit_dot<FMT, 1>(Up, (const uint2*)nullptr, tile, ku, lane, xs + ku * 64, 0, au); }
       red[(p * NW + wave) * 64 + lane] = ag[0]; red[((PMAX + p) * NW + wave) * 64 + lane] = au[0];

@@ -121,14 +121,14 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   for (int p = 0; p < P; ++p) { ag[p][0] = 0.0f; au[p][0] = 0.0f; }
   if (P == 2 && upw == 1) {
     // one unit per part: both parts' units of both matrices are fetched before the first is consumed
-    const int ka = min(wave, G.U - 1), kb = min(NW + wave, G.U - 1);
+    const int ka = min(2 * wave, G.U - 1), kb = min(2 * wave + 1, G.U - 1);
     UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ka, lane), u0 = unit_load<FMT>(Up, tile, ka, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
-    if (wave < G.U) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
-    if (NW + wave < G.U) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
+    if (2 * wave < G.U) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
+    if (2 * wave + 1 < G.U) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
   } else {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      const int k0 = min(G.U, ((kz * P + p) * NW + wave) * upw), kend = min(G.U, k0 + upw);
+      const int k0 = min(G.U, (wave * np + kz * P + p) * upw), kend = min(G.U, k0 + upw);          // wave w's shares of the np parts are adjacent
       // two units of both matrices are fetched before the first is consumed: a rolled loop would pay a memory round trip per unit
       for (int ku = k0; ku < kend; ku += 2) {
         const int kb = min(ku + 1, kend - 1);
