@@ -279,6 +279,14 @@ def bench_decode(args):
                   "avg_launch_us": round(v[1] / v[0] * 1e3, 3), "GBps": round(v[2] / (v[1] * 1e-3) / 1e9, 1) if v[1] > 0 else None} for k, v in classes]
     dom_k, dom = classes[0]
     dom_gbs = dom[2] / (dom[1] * 1e-3) / 1e9
+    traffic = None          # HBM bytes per launch of the dominant class from the committed FETCH_SIZE / WRITE_SIZE summary, when it covers it
+    if cfg.n_layers == 48 and not args.indexer:
+        try:
+            for line in open(os.path.join(ROOT, "profiles", "decode_deltanet_slice_hbm_traffic.txt")):
+                if line.startswith("traffic_bytes_per_launch_%s:" % dom_k):
+                    traffic = int(line.split(":")[1])
+        except OSError:
+            pass
     out = {
         "metric": "decode tok/s batch-1 (A3B hybrid IQ3_S)", "value": round(tok_s, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
@@ -287,7 +295,7 @@ def bench_decode(args):
                                "IQ3_S weights (bf16 router), 4 hyper-connection streams, 4-bit KV, greedy decode after a %d-token random prompt%s" % (
                                    cfg.n_layers, n_ctx, (", QSA indexer with %d heads (budget 2048, blocks of 4): variant, not the configuration of the metric" % args.indexer) if args.indexer else ""),
                    "context": n_ctx, "layers": cfg.n_layers},
-        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": dom_k, "algorithmic_bytes_per_launch": round(dom[2] / dom[0]), "avg_launch_us": round(dom[1] / dom[0] * 1e3, 3),
                      "share_of_kernel_time": round(dom[1] / tot_ms, 3)},
         "token_roofline": {"weight_bytes_per_token": wbytes, "kv_bytes_per_token": round(kvb), "state_bytes_per_token": state_b,
