@@ -44,6 +44,24 @@ def test_moe_ffn_small(ctx, qtype, t):
     assert relerr(y, yo) <= TOL
 
 
+@pytest.mark.parametrize("qtype,d", [(synth.Q4_K, 2048), (synth.Q8_0, 2048), (synth.IQ2_XS, 2048), (synth.IQ4_NL, 2048), (synth.IQ3_S, 4096)])
+def test_moe_gate_up_in_two_k_parts(ctx, qtype, d):
+    # rows of a multiple of 32 units: the gate/up dot products are summed in two K parts -- one workgroup per part for a
+    # single token, both parts in one workgroup for a window -- and a token's bits must not depend on which (d = 4096:
+    # two units per wave and part)
+    c = mg.Config(n_layers=1, full_every=4, d=d, n_exp=16, top_k=4, ff_exp=256, qtype=qtype)
+    moe, oracle, _ = moe_pair(ctx, c, 11)
+    x = synth.normal((3, c.d), 300)
+    y, idx, w = moe.ffn(x)
+    yo, io, wo = oracle(x)
+    assert np.array_equal(idx, io) and np.abs(w - wo).max() < 1e-6
+    assert relerr(y, yo) <= TOL
+    for ti in range(3):
+        y1, i1, _ = moe.ffn(x[ti:ti + 1])
+        assert np.array_equal(i1, idx[ti:ti + 1]) and relerr(y1, yo[ti:ti + 1]) <= TOL
+        assert np.array_equal(y1.view(np.uint32), y[ti:ti + 1].view(np.uint32))
+
+
 @pytest.mark.parametrize("t", [1, 4])
 def test_moe_ffn_benchmark_geometry(ctx, t):
     # 512 routed experts + 1 shared, d 2048, expert ff 512, top-10, IQ3_S (reduced to 64 resident experts' worth of
