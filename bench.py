@@ -222,7 +222,7 @@ def bench_decode(args):
         ctx.free(p)
     log("model resident (re-laid-out) in %.1f s; weight bytes per token %.1f MB" % (time.perf_counter() - t0, model.weight_bytes_per_token / 1e6))
     n_ctx = args.ctx
-    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8)
+    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8 + args.host_steps + 1)
     g = np.random.Generator(np.random.PCG64(args.seed + 1))
     prompt = g.integers(0, cfg.vocab, n_ctx, dtype=np.uint32)
     t0 = time.perf_counter()
@@ -268,6 +268,18 @@ def bench_decode(args):
         win_ms = (time.perf_counter() - t0) * 1e3 / args.spec_windows
         spec = {"window_tokens": 5, "ms_per_window": round(win_ms, 3), "tok_s_if_all_drafts_accepted": round(5e3 / win_ms, 1), "tok_s_if_none_accepted": round(1e3 / win_ms, 1),
                 "note": "host-facing verify window incl. 5 x %d logits device->host and the host argmax; %d windows" % (cfg.vocab, args.spec_windows)}
+    # the reference's own loop shape (Model::forward -> Vec<f32> logits -> sampler::argmax on the host): every step
+    # carries 151936 logits over PCIe and a host argmax; reported beside `value`, never as it
+    host_loop = None
+    if args.host_steps > 0:
+        tok = nxt
+        lg = model.forward(np.array([tok], dtype=np.uint32), st); tok = int(np.argmax(lg))      # untimed
+        ctx.sync(); t0 = time.perf_counter()
+        for i in range(args.host_steps):
+            lg = model.forward(np.array([tok], dtype=np.uint32), st); tok = int(np.argmax(lg))
+        hms = (time.perf_counter() - t0) * 1e3 / args.host_steps
+        host_loop = {"tok_s": round(1e3 / hms, 1), "ms_per_step": round(hms, 3), "steps": args.host_steps,
+                     "note": "pyre_forward per token: ids from the host, %d f32 logits back over PCIe, argmax on the host" % cfg.vocab}
     # second pass: per-kernel-class durations from event pairs around every launch
     ctx.prof_reset(); ctx.prof_enable(True)
     pn = min(16, args.steps)
@@ -306,6 +318,8 @@ def bench_decode(args):
     }
     if spec:
         out["spec_verify"] = spec
+    if host_loop:
+        out["host_loop"] = host_loop
     if not args.no_cpu:
         del model, st
         out["cpu_baseline"] = cpu_baseline_decode(cfg, args.seed)
@@ -324,6 +338,7 @@ def main():
     ap.add_argument("--indexer", type=int, default=0, metavar="HEADS", help="decode workload variant: attention layers with a QSA sparse indexer of this many heads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
+    ap.add_argument("--host-steps", type=int, default=32, help="decode workload: steps of the host-facing loop (pyre_forward + host argmax) to time beside the device loop (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
     ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs)")
     ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
