@@ -348,7 +348,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   // leaves the updated streams in the other
   const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
   auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
-  const bool raw_moe = c.top_k <= PYRE_MOE_KMAX && t == 1;        // single token: the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum)
+  const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
   for (int il = 0; il < c.n_layers; ++il) {
