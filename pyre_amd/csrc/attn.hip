@@ -8,13 +8,48 @@ __device__ __forceinline__ float a_sigm(float x) { return 1.0f / (1.0f + expf(-x
 
 size_t pyre_packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 4 || n <= (size_t)recent + 64) return 0; return ((n - recent) / 64) * 64; }
 
+// The positions that fall below the packed boundary when the context grows from pos to pos + 1 positions.
+__device__ __forceinline__ bool kv_pack_step_range(const AttnDev& a, int pos, int* p0, int* p1) {
+  const int n = pos + 1;
+  *p1 = (a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0;
+  *p0 = (a.kv_bits == 4 && n - 1 > a.kv_recent + 64) ? ((n - 1 - a.kv_recent) / 64) * 64 : 0;
+  return *p1 > *p0;
+}
+// kv4::pack (src/model/kv4.rs:12-42), thread gid of [p0, p1): one thread per (position, 32-value block, K or V)
+template <int HD> __device__ __forceinline__ void kv_pack_thread(const AttnDev& a, const KvDev& kv, int p0, int p1, size_t gid) {
+  const int bpr = a.nkv * HD / 32;                 // blocks per cache row
+  size_t per = (size_t)(p1 - p0) * bpr;
+  if (gid >= 2 * per) return;
+  const bool is_v = gid >= per; if (is_v) gid -= per;
+  const int pos = p0 + (int)(gid / bpr), blk = (int)(gid % bpr), kvh = blk / (HD / 32), bb = blk % (HD / 32);
+  float x[32];
+  for (int i = 0; i < 32; ++i) x[i] = is_v ? kv.vf[(size_t)pos * a.nkv * HD + (size_t)blk * 32 + i] : kv.kf[kv_blk((size_t)kvh * HD + bb * 32 + i, (size_t)a.nkv * HD, pos)];
+  float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(x[i]));
+  const float s = (m > 0.0f && isfinite(m)) ? m / 7.0f : 0.0f;
+  for (int w = 0; w < 4; ++w) {
+    uint32_t u = 0;
+    for (int j = 0; j < 8; ++j) { int q = s > 0.0f ? (int)fminf(fmaxf(roundf(x[8 * w + j] / s), -7.0f), 7.0f) : 0; u |= ((uint32_t)q & 0xFu) << (4 * j); }
+    if (is_v) kv.vq[(size_t)pos * (a.nkv * HD / 8) + (size_t)blk * 4 + w] = u;
+    else kv.kq[kv_blk((size_t)kvh * (HD / 8) + bb * 4 + w, (size_t)a.nkv * (HD / 8), pos)] = u;
+  }
+  if (is_v) kv.vs[(size_t)pos * bpr + blk] = s; else kv.ks[kv_blk((size_t)kvh * (HD / 32) + bb, (size_t)a.nkv * (HD / 32), pos)] = s;
+}
+
 // grid (nkv + nh, t), hd threads.  Blocks 0..nkv-1: key head -> rms_inplace(kn) -> rope -> cache (and the raw value row);
 // blocks nkv..: query head h -> rms_inplace(qn) -> rope -> q scratch.
+// Blocks past nkv + nh (single-token steps at a device-side position): the 64-position packing step that the growth
+// of the context by this token may make due (k_kv_pack's work, old positions only: it touches nothing the other
+// blocks write), so a replayed step does not spend a launch on a check that almost always finds nothing to do.
 template <int HD>
 __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout) {
   __shared__ float buf[HD]; __shared__ float red[HD / 64];
   if (posp) start = *posp;
   const int b = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, pos = start + ti;
+  if (b >= a.nkv + a.nh) {
+    int p0, p1;
+    if (ti == 0 && kv_pack_step_range(a, start, &p0, &p1)) kv_pack_thread<HD>(a, kv, p0, p1, (size_t)(b - a.nkv - a.nh) * HD + tid);
+    return;
+  }
   const bool is_k = b < a.nkv; const int h = is_k ? b : b - a.nkv;
   const float* row = qkv + (size_t)ti * stride;
   const float* src = is_k ? row + (size_t)a.nh * 2 * HD + (size_t)h * HD : row + (size_t)h * 2 * HD;
@@ -54,29 +89,8 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
 // grows from *posp to *posp + 1 positions (nothing on most steps).
 template <int HD>
 __global__ void k_kv_pack(AttnDev a, KvDev kv, int p0, int p1, const int* __restrict__ posp) {
-  if (posp) {
-    int n = *posp + 1;
-    p1 = (a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0;
-    p0 = (a.kv_bits == 4 && n - 1 > a.kv_recent + 64) ? ((n - 1 - a.kv_recent) / 64) * 64 : 0;
-    if (p1 <= p0) return;
-  }
-  const int bpr = a.nkv * HD / 32;                 // blocks per cache row
-  size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  size_t per = (size_t)(p1 - p0) * bpr;
-  if (gid >= 2 * per) return;
-  const bool is_v = gid >= per; if (is_v) gid -= per;
-  const int pos = p0 + (int)(gid / bpr), blk = (int)(gid % bpr), kvh = blk / (HD / 32), bb = blk % (HD / 32);
-  float x[32];
-  for (int i = 0; i < 32; ++i) x[i] = is_v ? kv.vf[(size_t)pos * a.nkv * HD + (size_t)blk * 32 + i] : kv.kf[kv_blk((size_t)kvh * HD + bb * 32 + i, (size_t)a.nkv * HD, pos)];
-  float m = 0.0f; for (int i = 0; i < 32; ++i) m = fmaxf(m, fabsf(x[i]));
-  const float s = (m > 0.0f && isfinite(m)) ? m / 7.0f : 0.0f;
-  for (int w = 0; w < 4; ++w) {
-    uint32_t u = 0;
-    for (int j = 0; j < 8; ++j) { int q = s > 0.0f ? (int)fminf(fmaxf(roundf(x[8 * w + j] / s), -7.0f), 7.0f) : 0; u |= ((uint32_t)q & 0xFu) << (4 * j); }
-    if (is_v) kv.vq[(size_t)pos * (a.nkv * HD / 8) + (size_t)blk * 4 + w] = u;
-    else kv.kq[kv_blk((size_t)kvh * (HD / 8) + bb * 4 + w, (size_t)a.nkv * (HD / 8), pos)] = u;
-  }
-  if (is_v) kv.vs[(size_t)pos * bpr + blk] = s; else kv.ks[kv_blk((size_t)kvh * (HD / 32) + bb, (size_t)a.nkv * (HD / 32), pos)] = s;
+  if (posp && !kv_pack_step_range(a, *posp, &p0, &p1)) return;
+  kv_pack_thread<HD>(a, kv, p0, p1, (size_t)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((int)(w << (28 - 4 * i))) >> 28); }   // sign-extended nibble i
@@ -532,11 +546,14 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q); } PYRE_CHECK_LAUNCH(ctx);
+  // a single-token step at a device-side position: the packing check rides on the prep launch as extra blocks
+  const bool pack_rides = posp && t == 1 && a.kv_bits == 4;
+  const int pack_blocks = pack_rides ? (64 * (a.nkv * a.hd / 32) * 2 + 255) / 256 : 0;
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
   int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
   if (posp) {   // one 64-position packing step at most; the kernel decides from the device-side position
-    if (a.kv_bits == 4) { size_t thr = (size_t)64 * (a.nkv * a.hd / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, 0, 0, posp); PYRE_CHECK_LAUNCH(ctx); }
+    if (a.kv_bits == 4 && !pack_rides) { size_t thr = (size_t)64 * (a.nkv * a.hd / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, 0, 0, posp); PYRE_CHECK_LAUNCH(ctx); }
   } else if (pbn > *packed_done) {
     size_t thr = (size_t)(pbn - *packed_done) * (a.nkv * a.hd / 32) * 2;
     { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn, (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);

@@ -94,6 +94,26 @@ def test_greedy_stream_identical_to_oracle_across_the_packing_boundary(ctx):
     assert len(gs) == len(os_) == 100 + n - 1 and orc.packed_boundary(len(os_), 4, 64) == 128
 
 
+def test_device_loop_identical_to_oracle_across_the_packing_boundary(ctx):
+    # the device-resident loop (replayed step, position on the device): the 64-position packing step rides on the
+    # attention prep launch there; the stream must cross the boundary (context 129) exactly as the oracle's does
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 6)
+    prompt = (np.arange(100, dtype=np.uint32) * 37 + 11) % c.vocab
+    gs, os_ = gm.new_state(300), om.new_state()
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    n = 96
+    out_o, _ = om.generate_greedy(os_, lo, n)
+    first = int(np.argmax(lg))
+    assert first == int(out_o[0])
+    out_d = gm.decode_greedy_dev(gs, first, n - 1)
+    assert np.array_equal(out_d, out_o[1:]), "first split at %d" % int(np.argmax(out_d != out_o[1:]))
+    assert orc.packed_boundary(len(os_), 4, 64) == 128
+    # and the state it leaves continues like the oracle's
+    l2 = gm.forward(np.array([out_d[-1]], dtype=np.uint32), gs); o2 = om.forward(np.array([out_o[-1]], dtype=np.uint32), os_)
+    assert relerr(l2, o2) <= 1e-3 and orc.argmax(l2) == orc.argmax(o2)
+
+
 def test_verify_window_equals_single_steps_and_rollback(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 7)
