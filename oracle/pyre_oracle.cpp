@@ -78,6 +78,8 @@ bool geom(uint32_t ty, int* el, int* by) {
     case ORC_IQ2_XXS: *el = 256; *by = 66; return true;
     case ORC_IQ2_S: *el = 256; *by = 82; return true;
     case ORC_IQ3_XXS: *el = 256; *by = 98; return true;
+    case ORC_Q3_K: *el = 256; *by = 110; return true;
+    case ORC_Q2_0: *el = 64; *by = 18; return true;
   }
   return false;
 }
@@ -136,6 +138,27 @@ bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
           }
           qh += 2;
         }
+      }
+      break;
+    case ORC_Q2_0:          // gguf_q.rs:80-81 with lut q2 (:50): value j of byte k = ((byte >> 2j) & 3) - 1, times d
+      for (size_t i = 0; i < nb; ++i) { const uint8_t* b = x + i * bs; float d = h2f(b); float* yy = y + i * 64;
+        for (int k = 0; k < 16; ++k) for (int j = 0; j < 4; ++j) yy[4 * k + j] = (float)((int)((b[2 + k] >> (2 * j)) & 3) - 1) * d; }
+      break;
+    case ORC_Q3_K:          // gguf_q.rs:90-102
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; const uint8_t* hm = b; const uint8_t* q = b + 32; const uint8_t* sc = b + 96; const float d_all = h2f(b + 108);
+        auto a = [&](int k) { return (uint32_t)sc[4 * k] | ((uint32_t)sc[4 * k + 1] << 8) | ((uint32_t)sc[4 * k + 2] << 16) | ((uint32_t)sc[4 * k + 3] << 24); };
+        const uint32_t a0 = a(0), a1 = a(1), tmp = a(2), k1 = 0x03030303u, k2 = 0x0f0f0f0fu;
+        const uint32_t aux[4] = {(a0 & k2) | ((tmp & k1) << 4), (a1 & k2) | (((tmp >> 2) & k1) << 4), ((a0 >> 4) & k2) | (((tmp >> 4) & k1) << 4), ((a1 >> 4) & k2) | (((tmp >> 6) & k1) << 4)};
+        int8_t scales[16]; for (int k = 0; k < 16; ++k) scales[k] = (int8_t)((aux[k >> 2] >> (8 * (k & 3))) & 0xFF);
+        float* yy = y + i * 256; int is = 0; uint8_t m = 1;
+        for (int n = 0; n < 2; ++n) { int shift = 0;
+          for (int j = 0; j < 4; ++j) {
+            for (int half = 0; half < 2; ++half) { const float dl = d_all * (float)((int)scales[is] - 32); ++is;
+              for (int l = 0; l < 16; ++l) { const int o = l + 16 * half; yy[l] = dl * (float)((int)((q[o] >> shift) & 3) - ((hm[o] & m) ? 0 : 4)); }
+              yy += 16; }
+            shift += 2; m = (uint8_t)(m << 1); }
+          q += 32; }
       }
       break;
     case ORC_Q4_0:

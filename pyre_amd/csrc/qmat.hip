@@ -88,6 +88,23 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
               put8b(32 * c + l, (int)(nib | (hi2 << 4)) - 32); }
             for (int g = 0; g < 2; ++g) sc[2 * c + g] = d * (float)(int)(int8_t)b[192 + 8 * n + 2 * qd + g]; }
         } break;
+        case PYRE_Q2_0: {                                              // gguf_q.rs:80-81, lut q2 :50: one 64-value block per unit
+          const uint8_t* b = row + (size_t)ku * 18; const float d = h2(b);
+          for (int i = 0; i < 4; ++i) sc[i] = d;
+          for (int k = 0; k < 16; ++k) for (int j = 0; j < 4; ++j) put4(4 * k + j, (b[2 + k] >> (2 * j)) & 3);
+        } break;
+        case PYRE_Q3_K: {                                              // gguf_q.rs:90-102
+          const uint8_t* b = row + (size_t)(ku >> 2) * 110; const uint8_t* hm = b; const uint8_t* s12 = b + 96; const float d = h2(b + 108);
+          auto a = [&](int k) { return (uint32_t)s12[4 * k] | ((uint32_t)s12[4 * k + 1] << 8) | ((uint32_t)s12[4 * k + 2] << 16) | ((uint32_t)s12[4 * k + 3] << 24); };
+          const uint32_t a0 = a(0), a1 = a(1), tmp = a(2), k1 = 0x03030303u, k2 = 0x0f0f0f0fu;
+          const uint32_t aux[4] = {(a0 & k2) | ((tmp & k1) << 4), (a1 & k2) | (((tmp >> 2) & k1) << 4), ((a0 >> 4) & k2) | (((tmp >> 4) & k1) << 4), ((a1 >> 4) & k2) | (((tmp >> 6) & k1) << 4)};
+          const int u = ku & 3, n = u >> 1; const uint8_t* q = b + 32 + 32 * n;
+          for (int g4 = 0; g4 < 4; ++g4) {                             // 16 values: j = 2*(u&1) + g4/2, half = g4&1
+            const int j = 2 * (u & 1) + (g4 >> 1), half = g4 & 1, is = 8 * n + 2 * j + half, shift = 2 * j; const uint32_t mbit = 1u << (4 * n + j);
+            sc[g4] = d * (float)((int)(int8_t)((aux[is >> 2] >> (8 * (is & 3))) & 0xFF) - 32);
+            for (int l = 0; l < 16; ++l) { const int o = l + 16 * half; put4(16 * g4 + l, ((q[o] >> shift) & 3) | ((hm[o] & mbit) ? 4u : 0u)); }
+          }
+        } break;
         case PYRE_IQ3_XXS: {                                           // gguf_q.rs:136-140
           const uint8_t* b = row + (size_t)(ku >> 2) * 98; float d = h2(b);
           for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; const uint8_t* ss = b + 66 + 4 * ib; uint32_t a = ss[0] | (ss[1] << 8) | (ss[2] << 16) | ((uint32_t)ss[3] << 24);

@@ -153,6 +153,28 @@ def dequant(ty, raw, n):
         hb = ((qh >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32)
         q = np.concatenate([b[:, 6:] & 0xF, b[:, 6:] >> 4], axis=1).astype(np.int32) + 16 * hb - 16
         return (q.astype(f) * d).astype(f).reshape(-1)
+    if ty == 42:                                                       # Q2_0: 64 values per block, four 2-bit codes per byte (low bits first), (code - 1) * d
+        b = raw[:n // 64 * 18].reshape(-1, 18)
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)
+        q = ((b[:, 2:, None].astype(np.int32) >> (2 * np.arange(4))) & 3).reshape(-1, 64) - 1
+        return (q.astype(f) * d).astype(f).reshape(-1)
+    if ty == 11:                                                       # Q3_K: hmask[32] | qs[64] | scales[12] | d; value = d*(sc6 - 32) * (low2 - (hbit ? 0 : 4))
+        b = raw[:n // 256 * 110].reshape(-1, 110)
+        nb = b.shape[0]
+        hm = b[:, 0:32].astype(np.int32); qs = b[:, 32:96].reshape(nb, 2, 32).astype(np.int32); s12 = b[:, 96:108].astype(np.int32)
+        d = f16_to_f32(b[:, 108:110].copy()).reshape(nb, 1)
+        # sixteen 6-bit scales: low 4 bits from bytes 0..7 (low nibbles -> scales 0..7, high nibbles -> 8..15), high 2 bits from bytes 8..11
+        lo4 = np.concatenate([s12[:, 0:8] & 0xF, s12[:, 0:8] >> 4], axis=1)                                  # [nb, 16]
+        hi2 = np.stack([(s12[:, 8 + (k % 4)] >> (2 * (k // 4))) & 3 for k in range(16)], axis=1)             # scale k: byte 8 + k%4, bits 2*(k/4)
+        sc6 = (lo4 | (hi2 << 4)) - 32
+        dl = (d * sc6.astype(f)).astype(f)                                                                   # [nb, 16]: scale of values 16k .. 16k+15
+        out = np.empty((nb, 2, 4, 32), dtype=np.int32)                                                       # [half of 128][shift step j][byte o]
+        for nn in range(2):
+            for j in range(4):
+                hb = (hm >> (4 * nn + j)) & 1
+                out[:, nn, j] = ((qs[:, nn] >> (2 * j)) & 3) - 4 * (1 - hb)
+        q = out.reshape(nb, 16, 16).astype(f)                                                                # value index = nn*128 + j*32 + o; 16 per scale
+        return (dl[:, :, None] * q).astype(f).reshape(-1)
     gxx, gs, g3x, kv = codebooks_more()
     kvf = kv.astype(f)
     if ty == 20:                                                       # IQ4_NL: d * level[nibble]

@@ -10,7 +10,7 @@ from pyre_amd import synth
 
 FMTS = [orc.Q8_0, orc.Q4_K, orc.IQ2_XS, orc.IQ3_S]
 # the other block types real files of this architecture use (gguf_q.rs:74-78,82-89,114-125,130-140)
-FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS]
+FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS, orc.Q3_K, orc.Q2_0]
 
 
 def bits(a):
@@ -115,6 +115,27 @@ def test_q4_0_and_q5_0_known_answers():
     y = orc.dequant(orc.Q5_0, b, 32)
     exp = np.concatenate([np.full(16, 1 - 16.0), np.full(16, 2 - 16.0)]); exp[3] += 16; exp[20] += 16
     assert np.array_equal(y, (exp * 0.25).astype(np.float32))
+
+
+def test_q2_0_and_q3_k_known_answers():
+    # Q2_0 (gguf_q.rs:80-81, :50): byte 0b11100100 holds the codes 0, 1, 2, 3 from the low bits up -> values -1, 0, 1, 2
+    b = _blk(18, 0.5); b[2:] = 0b11100100
+    assert np.array_equal(orc.dequant(orc.Q2_0, b, 64), np.tile(np.array([-1, 0, 1, 2], np.float32) * 0.5, 16))
+    # Q3_K (gguf_q.rs:90-102): zero payload -> scale 0 - 32, low bits 0, mask clear -> -4: every value d * -32 * -4
+    assert np.array_equal(orc.dequant(orc.Q3_K, _blk(110, 0.5, 108), 256), np.full(256, 0.5 * -32 * -4, np.float32))
+    b = _blk(110, 1.0, 108)
+    b[96 + 3] = 0x5 | (0xA << 4)          # low 4 bits of scale 3 = 5, of scale 11 = 10
+    b[96 + 8 + 3] = 0b00100001            # high 2 bits: scale 3 (bits 0-1) = 1, scale 11 (bits 4-5) = 2
+    b[32 + 20] = 0b00001100               # first 128 values, byte o = 20: code 3 at shift 2 (j = 1) -> value index 32 + 20
+    b[0 + 20] = 0b00000010                # high-mask bit 1 (n = 0, j = 1) of byte 20 set: no -4
+    b[32 + 32 + 7] = 0b01000000           # second 128 values, byte o = 7: code 1 at shift 6 (j = 3) -> value index 128 + 96 + 7
+    y = orc.dequant(orc.Q3_K, b, 256)
+    exp = np.full(256, -32.0 * -4, np.float32)
+    exp[48:64] = ((5 | (1 << 4)) - 32) * -4.0           # scale 3 covers values 48..63
+    exp[176:192] = ((10 | (2 << 4)) - 32) * -4.0        # scale 11 covers values 176..191
+    exp[52] = ((5 | (1 << 4)) - 32) * 3.0               # value 32 + 20 lies in scale 3's group: code 3, mask set
+    exp[128 + 96 + 7] = -32.0 * (1 - 4)
+    assert np.array_equal(y, exp)
 
 
 def test_iq4_nl_and_iq4_xs_known_answers():
