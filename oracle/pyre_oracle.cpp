@@ -80,12 +80,13 @@ bool geom(uint32_t ty, int* el, int* by) {
     case ORC_IQ3_XXS: *el = 256; *by = 98; return true;
     case ORC_Q3_K: *el = 256; *by = 110; return true;
     case ORC_Q2_0: *el = 64; *by = 18; return true;
+    case ORC_Q5_K: *el = 256; *by = 176; return true;
   }
   return false;
 }
 
 // dequant, gguf_q.rs:67-166 (arms F32 :71, F16 :72, BF16 :73, Q4_0 :74-75, Q5_0 :76-78, Q8_0 :79, IQ4NL :82-83, IQ4XS :84-89,
-// Q4K :103-107, Q6K :114-121, IQ2XXS :122-125, IQ2XS :126-129, IQ2S :130-135, IQ3XXS :136-140, IQ3S :141-151)
+// Q2_0 :80-81, Q3K :90-102, Q4K :103-107, Q5K :108-113, Q6K :114-121, IQ2XXS :122-125, IQ2XS :126-129, IQ2S :130-135, IQ3XXS :136-140, IQ3S :141-151)
 bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
   int qk, bs; if (!geom(ty, &qk, &bs)) return false;
   size_t nb = n / qk;
@@ -105,6 +106,18 @@ bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
           float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
           for (int l = 0; l < 32; ++l) { yy[l] = d1 * (float)(q[l] & 0xF) - M1; yy[l + 32] = d2 * (float)(q[l] >> 4) - M2; }
           yy += 64; q += 32;
+        }
+      }
+      break;
+    case ORC_Q5_K:          // gguf_q.rs:108-113: as Q4_K with a fifth bit per value from qh (bit 2j for the low nibbles, 2j+1 for the high)
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; float d = h2f(b), mn = h2f(b + 2); const uint8_t* sc = b + 4; const uint8_t* qh = b + 16; const uint8_t* ql = b + 48; float* yy = y + i * 256;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 4; ++j) {
+          uint8_t s1, m1, s2, m2; scale_min_k4(2 * j, sc, &s1, &m1); scale_min_k4(2 * j + 1, sc, &s2, &m2);
+          float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
+          for (int l = 0; l < 32; ++l) { yy[l] = d1 * (float)((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0)) - M1; yy[l + 32] = d2 * (float)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - M2; }
+          yy += 64; ql += 32; u1 = (uint8_t)(u1 << 2); u2 = (uint8_t)(u2 << 2);
         }
       }
       break;

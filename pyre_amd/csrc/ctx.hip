@@ -145,7 +145,7 @@ int pyre_synth_blocks(pyre_ctx* ctx, uint32_t ty, size_t n_blocks, uint64_t seed
   size_t nw = (nbytes + 7) / 8;
   hipLaunchKernelGGL(k_synth_payload, dim3((unsigned)((nw + 255) / 256)), dim3(256), 0, ctx->stream, seed, nbytes, (uint8_t*)dev_out);
   PYRE_CHECK_LAUNCH(ctx);
-  int nf = fmt == FMT_Q4_K ? 2 : (fmt >= FMT_Q8_0 ? 1 : 0);
+  int nf = (fmt == FMT_Q4_K || ty == PYRE_Q5_K) ? 2 : (fmt >= FMT_Q8_0 ? 1 : 0);      // Q4_K, Q5_K: d and dmin
   if (nf) {      // the f16 super-block scale sits at byte 0 of every block format except Q6_K (byte 208) and Q3_K (byte 108)
     hipLaunchKernelGGL(k_synth_scales, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx->stream, seed, n_blocks, g.bytes, nf, ty == PYRE_Q6_K ? 208 : (ty == PYRE_Q3_K ? 108 : 0), 2, d_lo, d_hi, (uint8_t*)dev_out);
     PYRE_CHECK_LAUNCH(ctx);

@@ -24,13 +24,16 @@ __host__ __device__ inline FmtGeom fmt_geom(int fmt) {
     default:         return {2, 0, 0, 1, 2};     // IQ3_S, re-coded at load: p0: 64 four-bit codes, p3: scale byte; pb: d
   }
 }
+// Planes of a matrix of GGUF type ty in device format fmt: Q5_K (value = d*s*q - dmin*m, gguf_q.rs:108-113) rides on C8 with
+// a second f32 per 16 values in p2, the offset dmin*m subtracted after the scale multiply.
+__host__ __device__ inline FmtGeom qmat_geom(int fmt, uint32_t ty) { FmtGeom g = fmt_geom(fmt); if (fmt == FMT_C8 && ty == PYRE_Q5_K) g.e2 = 16; return g; }
 // GGUF block geometry (elements, bytes) of the types the library loads (QType::geom, gguf_q.rs:33-42); false for the rest
 __host__ __device__ inline bool ggml_geom(uint32_t ty, int* el, int* bytes) {
   switch (ty) {
     case PYRE_F32: *el = 1; *bytes = 4; return true;  case PYRE_F16: case PYRE_BF16: *el = 1; *bytes = 2; return true;
     case PYRE_Q4_0: *el = 32; *bytes = 18; return true;  case PYRE_Q5_0: *el = 32; *bytes = 22; return true;  case PYRE_Q8_0: *el = 32; *bytes = 34; return true;
     case PYRE_Q4_K: *el = 256; *bytes = 144; return true;  case PYRE_Q6_K: *el = 256; *bytes = 210; return true;
-    case PYRE_Q3_K: *el = 256; *bytes = 110; return true;  case PYRE_Q2_0: *el = 64; *bytes = 18; return true;
+    case PYRE_Q3_K: *el = 256; *bytes = 110; return true;  case PYRE_Q2_0: *el = 64; *bytes = 18; return true;  case PYRE_Q5_K: *el = 256; *bytes = 176; return true;
     case PYRE_IQ2_XXS: *el = 256; *bytes = 66; return true;  case PYRE_IQ2_XS: *el = 256; *bytes = 74; return true;  case PYRE_IQ2_S: *el = 256; *bytes = 82; return true;
     case PYRE_IQ3_XXS: *el = 256; *bytes = 98; return true;  case PYRE_IQ3_S: *el = 256; *bytes = 110; return true;
     case PYRE_IQ4_NL: *el = 32; *bytes = 18; return true;  case PYRE_IQ4_XS: *el = 256; *bytes = 136; return true;
@@ -42,7 +45,7 @@ inline int fmt_from_ggml(uint32_t ty) {
     case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S;
     case PYRE_IQ2_XXS: case PYRE_IQ2_S: return FMT_IQ2_XS;
     case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ3_XXS: case PYRE_Q3_K: case PYRE_Q2_0: return FMT_C4;
-    case PYRE_Q5_0: case PYRE_Q6_K: return FMT_C8; }
+    case PYRE_Q5_0: case PYRE_Q6_K: case PYRE_Q5_K: return FMT_C8; }
   return -1;
 }
 // The C4 value table of a GGUF type: entry c (byte c%4 of word c/4) holds value + bias, 0..255.
@@ -149,6 +152,10 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
       uint4 v = ld_vec<4>(m, tile, ku, c, lane); uint32_t w[4] = {v.x, v.y, v.z, v.w};
       for (int k = 0; k < 16; ++k) y[16 * c + k] = sc[c] * (float)(int)(int8_t)(w[k >> 2] >> (8 * (k & 3)));
     }
+    if (m.ty == PYRE_Q5_K) {                       // gguf_q.rs:112: d1 * q - m1, the subtraction after the rounded product
+      uint4 oq = ld_small<uint4>(m.p2, m, tile, ku, lane); float off[4] = {__uint_as_float(oq.x), __uint_as_float(oq.y), __uint_as_float(oq.z), __uint_as_float(oq.w)};
+      for (int k = 0; k < 64; ++k) y[k] = y[k] - off[k >> 4];
+    }
   } else {                                         // IQ3_S, gguf_q.rs:141-151, from the 4-bit codes (see iq3s_code)
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));
     uint32_t sc = ld_small<uint8_t>(m.p3, m, tile, ku, lane);
@@ -163,15 +170,16 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
 // ---- factored per-unit dot products for the GEMV ------------------------------------------------------------------
 // A unit's packed data is fetched first (unit_load) and consumed later (unit_fma), so a kernel can issue the weight
 // loads ahead of a barrier or of the previous unit's arithmetic; unit_dot does both at once.
-template <int FMT> struct UnitRaw { uint4 v[FMT == FMT_F32 ? 16 : (FMT == FMT_F16 || FMT == FMT_BF16) ? 8 : (FMT == FMT_Q8_0 || FMT == FMT_C8) ? 4 : (FMT == FMT_Q4_K || FMT == FMT_IQ3_S || FMT == FMT_C4) ? 2 : 1]; uint4 hb; uint32_t s0, s1; };
+template <int FMT> struct UnitRaw { uint4 v[FMT == FMT_F32 ? 16 : (FMT == FMT_F16 || FMT == FMT_BF16) ? 8 : (FMT == FMT_Q8_0 || FMT == FMT_C8) ? 4 : (FMT == FMT_Q4_K || FMT == FMT_IQ3_S || FMT == FMT_C4) ? 2 : 1]; uint4 hb; uint4 hb2; uint32_t s0, s1; };
 template <int FMT> __device__ __forceinline__ UnitRaw<FMT> unit_load(const QMatDev& m, int tile, int ku, int lane) {
-  UnitRaw<FMT> r; r.hb = uint4{0, 0, 0, 0}; r.s0 = 0; r.s1 = 0;
+  UnitRaw<FMT> r; r.hb = uint4{0, 0, 0, 0}; r.hb2 = uint4{0, 0, 0, 0}; r.s0 = 0; r.s1 = 0;
   constexpr int V = sizeof(r.v) / sizeof(uint4);
 #pragma unroll
   for (int c = 0; c < V; ++c) r.v[c] = ld_vec<V>(m, tile, ku, c, lane);
   if constexpr (FMT == FMT_Q8_0) r.s0 = ld_small<uint32_t>(m.p1, m, tile, ku, lane);
   if constexpr (FMT == FMT_Q4_K) r.hb = ld_block<uint4>(m, tile, ku, lane);
   if constexpr (FMT == FMT_C4 || FMT == FMT_C8) r.hb = ld_small<uint4>(m.p1, m, tile, ku, lane);
+  if constexpr (FMT == FMT_C8) { if (m.ty == PYRE_Q5_K) r.hb2 = ld_small<uint4>(m.p2, m, tile, ku, lane); }
   if constexpr (FMT == FMT_IQ2_XS) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint16_t>(m.p1, m, tile, ku, lane); uint2 sg = ld_small<uint2>(m.p2, m, tile, ku, lane); r.hb.x = sg.x; r.hb.y = sg.y; }
   if constexpr (FMT == FMT_IQ3_S) { r.s0 = ld_block<uint16_t>(m, tile, ku, lane); r.s1 = ld_small<uint8_t>(m.p3, m, tile, ku, lane); }
   return r;
@@ -318,6 +326,17 @@ _Pragma("unroll")
         for (int t = 0; t < T; ++t) part[t] = fmaf(f, xs[t * xstride + 16 * c + k], part[t]); }
 #pragma unroll
       for (int t = 0; t < T; ++t) acc[t] = fmaf(sc[c], part[t], acc[t]);
+    }
+    if (m.ty == PYRE_Q5_K) {             // value = scale * q - offset: the offsets leave through the groups' activation sums
+      const float off[4] = {__uint_as_float(r.hb2.x), __uint_as_float(r.hb2.y), __uint_as_float(r.hb2.z), __uint_as_float(r.hb2.w)};
+#pragma unroll
+      for (int t = 0; t < T; ++t) {
+        float xv = xs[t * xstride + lane];
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) xv += __shfl_xor(xv, o);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[t] = fmaf(-off[g], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), 16 * g)), acc[t]);
+      }
     }
   } else {   // IQ3_S from 4-bit codes c = (w + 15) / 2: sum w x = 2 sum c x - 15 sum x per 32-value sub-block
     float d = h2f_bits(r.s0);

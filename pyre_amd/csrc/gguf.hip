@@ -80,7 +80,7 @@ bool shard_paths(const std::string& path, std::vector<std::string>* out, std::st
 const char* ggml_name(uint32_t ty) {
   switch (ty) { case 0: return "F32"; case 1: return "F16"; case 2: return "Q4_0"; case 3: return "Q4_1"; case 6: return "Q5_0"; case 7: return "Q5_1"; case 8: return "Q8_0"; case 10: return "Q2_K";
     case 11: return "Q3_K"; case 12: return "Q4_K"; case 13: return "Q5_K"; case 14: return "Q6_K"; case 16: return "IQ2_XXS"; case 17: return "IQ2_XS"; case 18: return "IQ3_XXS"; case 19: return "IQ1_S";
-    case 20: return "IQ4_NL"; case 21: return "IQ3_S"; case 22: return "IQ2_S"; case 23: return "IQ4_XS"; case 30: return "BF16"; case 42: return "Q2_0"; }
+    case 20: return "IQ4_NL"; case 21: return "IQ3_S"; case 22: return "IQ2_S"; case 23: return "IQ4_XS"; case 29: return "IQ1_M"; case 30: return "BF16"; case 42: return "Q2_0"; }
   return "unknown";
 }
 // block geometry of the types this library computes with (QType::geom, gguf_q.rs:33-42); false for the others

@@ -12,7 +12,7 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
   int ku = (int)(gid % m.U); size_t r = gid / m.U; int tile = (int)(r / 64), lane = (int)(r % 64);
   bool live = r < (size_t)m.rows;
   const uint8_t* row = raw + r * row_bytes;
-  FmtGeom g = fmt_geom(m.fmt);
+  FmtGeom g = qmat_geom(m.fmt, m.ty);
   size_t e = ((size_t)tile * m.U + ku) * 64 + lane;              // entry index in per-unit planes
   uint8_t* v = p0 + ((size_t)tile * m.U + ku) * g.V * 64 * 16;     // chunk c of this lane at v + (c*64 + lane)*16
   auto put_vec = [&](int chunk, const uint8_t* src) { uint8_t* d = v + ((size_t)chunk * 64 + lane) * 16; for (int i = 0; i < 16; ++i) d[i] = live ? src[i] : 0; };
@@ -58,9 +58,9 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
     } break;
     case FMT_C4: case FMT_C8: {
       // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512]; code(e) and scale(e / 16) of the unit's 64 values e
-      uint32_t words[16]; float sc[4];
+      uint32_t words[16]; float sc[4], off[4];
       for (int i = 0; i < 16; ++i) words[i] = 0;
-      for (int i = 0; i < 4; ++i) sc[i] = 0.0f;
+      for (int i = 0; i < 4; ++i) { sc[i] = 0.0f; off[i] = 0.0f; }
       auto h2 = [](const uint8_t* q) { return __half2float(__ushort_as_half((unsigned short)(q[0] | (q[1] << 8)))); };
       auto put4 = [&](int e, uint32_t code) { words[e >> 3] |= (code & 0xF) << (4 * (e & 7)); };
       auto put8b = [&](int e, int q) { words[e >> 2] |= (uint32_t)(q & 0xFF) << (8 * (e & 3)); };
@@ -105,6 +105,14 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
             for (int l = 0; l < 16; ++l) { const int o = l + 16 * half; put4(16 * g4 + l, ((q[o] >> shift) & 3) | ((hm[o] & mbit) ? 4u : 0u)); }
           }
         } break;
+        case PYRE_Q5_K: {                                              // gguf_q.rs:108-113
+          const uint8_t* b = row + (size_t)(ku >> 2) * 176; const float d = h2(b), mn = h2(b + 2); const int j = ku & 3;
+          auto w32 = [&](int k) { return (uint32_t)b[4 + 4 * k] | ((uint32_t)b[5 + 4 * k] << 8) | ((uint32_t)b[6 + 4 * k] << 16) | ((uint32_t)b[7 + 4 * k] << 24); };
+          uint32_t s1, m1, s2, m2; scale_min_k4(2 * j, w32(0), w32(1), w32(2), s1, m1); scale_min_k4(2 * j + 1, w32(0), w32(1), w32(2), s2, m2);
+          sc[0] = sc[1] = d * (float)s1; off[0] = off[1] = mn * (float)m1; sc[2] = sc[3] = d * (float)s2; off[2] = off[3] = mn * (float)m2;
+          const uint8_t* qh = b + 16; const uint8_t* ql = b + 48 + 32 * j; const uint32_t u1 = 1u << (2 * j), u2 = 2u << (2 * j);
+          for (int l = 0; l < 32; ++l) { put8b(l, (int)((ql[l] & 0xF) + ((qh[l] & u1) ? 16 : 0))); put8b(32 + l, (int)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0))); }
+        } break;
         case PYRE_IQ3_XXS: {                                           // gguf_q.rs:136-140
           const uint8_t* b = row + (size_t)(ku >> 2) * 98; float d = h2(b);
           for (int c = 0; c < 2; ++c) { int ib = 2 * (ku & 3) + c; const uint8_t* ss = b + 66 + 4 * ib; uint32_t a = ss[0] | (ss[1] << 8) | (ss[2] << 16) | ((uint32_t)ss[3] << 24);
@@ -116,6 +124,7 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
       }
       for (int c = 0; c < g.V; ++c) { uint32_t* dst = (uint32_t*)(v + ((size_t)c * 64 + lane) * 16); for (int i = 0; i < 4; ++i) dst[i] = words[4 * c + i]; }
       float* sd = (float*)(p1 + e * 16); for (int i = 0; i < 4; ++i) sd[i] = sc[i];
+      if (g.e2 == 16) { float* od = (float*)(p2 + e * 16); for (int i = 0; i < 4; ++i) od[i] = off[i]; }
     } break;
     default: {   // IQ3_S: codebook lookups and signs are resolved here, once (gguf_q.rs:141-151), into 4-bit codes
       const uint8_t* b = row + (size_t)(ku >> 2) * 110; int j = ku & 3;
@@ -368,7 +377,7 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
   if (!ctx || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: null argument");
   *out = nullptr;
   int fmt = fmt_from_ggml(ty); if (fmt < 0) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmat_create: unsupported ggml type %u", ty);
-  FmtGeom g = fmt_geom(fmt); int gel = 1, gbytes = 4; ggml_geom(ty, &gel, &gbytes);
+  FmtGeom g = qmat_geom(fmt, ty); int gel = 1, gbytes = 4; ggml_geom(ty, &gel, &gbytes);
   if (rows == 0 || cols == 0 || cols % PYRE_UNIT != 0 || cols % gel != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu: cols must be a non-zero multiple of 64 and of the block size %d", rows, cols, gel);
   if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
   size_t row_bytes = cols / gel * gbytes;

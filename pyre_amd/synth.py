@@ -21,9 +21,9 @@ SCALE_SALT = np.uint64(0xD1B54A32D192ED03)
 GEOM = {8: (32, 34, (0,)), 12: (256, 144, (0, 2)), 17: (256, 74, (0,)), 21: (256, 110, (0,)),
         0: (1, 4, ()), 1: (1, 2, ()), 30: (1, 2, ()),
         2: (32, 18, (0,)), 6: (32, 22, (0,)), 14: (256, 210, (208,)), 16: (256, 66, (0,)), 18: (256, 98, (0,)),
-        20: (32, 18, (0,)), 22: (256, 82, (0,)), 23: (256, 136, (0,)), 11: (256, 110, (108,)), 42: (64, 18, (0,))}
+        20: (32, 18, (0,)), 22: (256, 82, (0,)), 23: (256, 136, (0,)), 11: (256, 110, (108,)), 42: (64, 18, (0,)), 13: (256, 176, (0, 2))}
 Q8_0, Q4_K, IQ2_XS, IQ3_S, F32, F16, BF16 = 8, 12, 17, 21, 0, 1, 30
-Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS, Q3_K, Q2_0 = 2, 6, 14, 16, 18, 20, 22, 23, 11, 42
+Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS, Q3_K, Q2_0, Q5_K = 2, 6, 14, 16, 18, 20, 22, 23, 11, 42, 13
 
 
 def mix64(z):

@@ -153,6 +153,26 @@ def dequant(ty, raw, n):
         hb = ((qh >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32)
         q = np.concatenate([b[:, 6:] & 0xF, b[:, 6:] >> 4], axis=1).astype(np.int32) + 16 * hb - 16
         return (q.astype(f) * d).astype(f).reshape(-1)
+    if ty == 13:                                                       # Q5_K: d | dmin | scales[12] | qh[32] | ql[128]; (d*s) * (nibble + 16*bit) - dmin*m
+        b = raw[:n // 256 * 176].reshape(-1, 176)
+        nb = b.shape[0]
+        d = f16_to_f32(b[:, 0:2].copy()).reshape(-1); mn = f16_to_f32(b[:, 2:4].copy()).reshape(-1)
+        sc = b[:, 4:16].astype(np.uint32)
+        s = np.empty((nb, 8), dtype=np.uint32); m = np.empty_like(s)
+        for j in range(8):
+            if j < 4:
+                s[:, j] = sc[:, j] & 63; m[:, j] = sc[:, j + 4] & 63
+            else:
+                s[:, j] = (sc[:, j + 4] & 0xF) | ((sc[:, j - 4] >> 6) << 4)
+                m[:, j] = (sc[:, j + 4] >> 4) | ((sc[:, j] >> 6) << 4)
+        qh = b[:, 16:48].astype(np.int32); ql = b[:, 48:].reshape(nb, 4, 32).astype(np.int32)
+        out = np.empty((nb, 8, 32), dtype=f)                               # sub-block 2j: low nibbles, 2j+1: high nibbles of the same 32 bytes
+        for sb in range(8):
+            nib = (ql[:, sb // 2] & 0xF) if sb % 2 == 0 else (ql[:, sb // 2] >> 4)
+            q = (nib + 16 * ((qh >> sb) & 1)).astype(f)
+            d1 = (d * s[:, sb].astype(f)).astype(f).reshape(nb, 1); m1 = (mn * m[:, sb].astype(f)).astype(f).reshape(nb, 1)
+            out[:, sb] = ((d1 * q).astype(f) - m1).astype(f)
+        return out.reshape(-1)
     if ty == 42:                                                       # Q2_0: 64 values per block, four 2-bit codes per byte (low bits first), (code - 1) * d
         b = raw[:n // 64 * 18].reshape(-1, 18)
         d = f16_to_f32(b[:, 0:2].copy()).reshape(-1, 1)

@@ -32,7 +32,7 @@ def moe_pair(ctx, c, seed):
     return moe, oracle, hw
 
 
-@pytest.mark.parametrize("qtype", [synth.IQ3_S, synth.IQ2_XS, synth.Q4_K, synth.Q8_0, synth.IQ2_S, synth.IQ4_NL, synth.Q6_K])
+@pytest.mark.parametrize("qtype", [synth.IQ3_S, synth.IQ2_XS, synth.Q4_K, synth.Q8_0, synth.IQ2_S, synth.IQ4_NL, synth.Q6_K, synth.Q5_K, synth.Q3_K])
 @pytest.mark.parametrize("t", [1, 4])
 def test_moe_ffn_small(ctx, qtype, t):
     c = mg.Config(n_layers=1, full_every=4, d=512, n_exp=16, top_k=4, ff_exp=256, qtype=qtype)

@@ -34,7 +34,8 @@ def pair(ctx, c, seed, max_ctx=512):
 
 
 @pytest.mark.parametrize("qtype,hc_type", [(synth.IQ3_S, synth.BF16), (synth.IQ3_S, synth.IQ3_S), (synth.Q4_K, synth.F32), (synth.IQ2_XS, synth.F16), (synth.Q8_0, synth.BF16),
-                                           (synth.IQ4_XS, synth.BF16), (synth.IQ2_S, synth.Q6_K), (synth.IQ3_XXS, synth.IQ4_XS), (synth.Q6_K, synth.F32), (synth.IQ2_XXS, synth.BF16)])
+                                           (synth.IQ4_XS, synth.BF16), (synth.IQ2_S, synth.Q6_K), (synth.IQ3_XXS, synth.IQ4_XS), (synth.Q6_K, synth.F32), (synth.IQ2_XXS, synth.BF16),
+                                           (synth.Q5_K, synth.Q3_K), (synth.Q3_K, synth.Q5_K)])
 def test_forward_logits_and_state_match_oracle(ctx, qtype, hc_type):
     c = small_cfg(qtype=qtype, hc_type=hc_type, hc_lr=256 if synth.GEOM[hc_type][0] == 256 else 64)
     hw, gm, om = pair(ctx, c, 5)

@@ -10,7 +10,7 @@ from pyre_amd import synth
 
 FMTS = [orc.Q8_0, orc.Q4_K, orc.IQ2_XS, orc.IQ3_S]
 # the other block types real files of this architecture use (gguf_q.rs:74-78,82-89,114-125,130-140)
-FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS, orc.Q3_K, orc.Q2_0]
+FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS, orc.Q3_K, orc.Q2_0, orc.Q5_K]
 
 
 def bits(a):
@@ -135,6 +135,24 @@ def test_q2_0_and_q3_k_known_answers():
     exp[176:192] = ((10 | (2 << 4)) - 32) * -4.0        # scale 11 covers values 176..191
     exp[52] = ((5 | (1 << 4)) - 32) * 3.0               # value 32 + 20 lies in scale 3's group: code 3, mask set
     exp[128 + 96 + 7] = -32.0 * (1 - 4)
+    assert np.array_equal(y, exp)
+
+
+def test_q5_k_known_answers():
+    # gguf_q.rs:108-113.  scales bytes: sub-block 0 -> (s, m) = (3, 5) through the j < 4 branch; sub-block 5 -> (s, m) = (0x2B, 0x1C)
+    # through the j >= 4 branch: low 4 bits in byte 9 (s low nibble, m high nibble), high 2 bits in bits 6-7 of bytes 1 (s) and 5 (m)
+    b = _blk(176, 0.5); b[2:4] = np_ref.f16_bytes(0.25)
+    b[4 + 0] = 3; b[4 + 4] = 5
+    b[4 + 9] = (0x2B & 0xF) | ((0x1C & 0xF) << 4); b[4 + 1] = (0x2B >> 4) << 6; b[4 + 5] = (0x1C >> 4) << 6
+    b[48 + 7] = 0x9                      # sub-block 0 (low nibbles of the first 32 bytes), value 7: nibble 9
+    b[16 + 7] = 0b00000001               # ... with its fifth bit (bit 0 of qh[7]) set -> 25
+    b[48 + 64 + 3] = 0xC0                # sub-block 5 (high nibbles of the third 32 bytes), value 3: nibble 12
+    b[16 + 3] = 1 << 5                   # ... fifth bit = bit 5 of qh[3] -> 28
+    y = orc.dequant(orc.Q5_K, b, 256).reshape(8, 32)
+    exp = np.zeros((8, 32), np.float32)
+    exp[0] = 0.5 * 3 * 0 - 0.25 * 5; exp[0, 7] = 0.5 * 3 * 25 - 0.25 * 5
+    exp[5] = -0.25 * 0x1C; exp[5, 3] = 0.5 * 0x2B * 28 - 0.25 * 0x1C
+    exp[1, 7] = 0.0                      # bytes 1 and 5 also carry the 6-bit (s, m) of sub-block 1: both 0 in their low bits
     assert np.array_equal(y, exp)
 
 
