@@ -84,7 +84,7 @@ def bench_gemv(args):
     ev = HipEvents()
     ctx = lib.Context(0)
     names = {"iq3_s": lib.IQ3_S, "iq2_xs": lib.IQ2_XS, "q4_k": lib.Q4_K, "q8_0": lib.Q8_0, "q4_0": lib.Q4_0, "q5_0": lib.Q5_0, "q6_k": lib.Q6_K, "iq2_xxs": lib.IQ2_XXS,
-             "iq2_s": lib.IQ2_S, "iq3_xxs": lib.IQ3_XXS, "iq4_nl": lib.IQ4_NL, "iq4_xs": lib.IQ4_XS}
+             "iq2_s": lib.IQ2_S, "iq3_xxs": lib.IQ3_XXS, "iq4_nl": lib.IQ4_NL, "iq4_xs": lib.IQ4_XS, "q3_k": lib.Q3_K, "q5_k": lib.Q5_K, "q2_0": lib.Q2_0}
     ty, rows, cols = names[args.fmt], 151936, 2048
     FN = args.fmt.upper()
     el, bs, _ = synth.GEOM[ty]
@@ -340,7 +340,7 @@ def main():
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
     ap.add_argument("--host-steps", type=int, default=32, help="decode workload: steps of the host-facing loop (pyre_forward + host argmax) to time beside the device loop (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
-    ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs)")
+    ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs, q3_k, q5_k, q2_0)")
     ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MiB", help="gemv workload: also run 4 plain device copies of this size (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
