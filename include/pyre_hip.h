@@ -24,7 +24,7 @@ typedef struct pyre_state pyre_state;
 
 /* ggml tensor type ids accepted by pyre_qmat_create (QType::from_id, src/model/gguf_q.rs:25-28). */
 enum { PYRE_F32 = 0, PYRE_F16 = 1, PYRE_Q4_0 = 2, PYRE_Q5_0 = 6, PYRE_Q8_0 = 8, PYRE_Q3_K = 11, PYRE_Q4_K = 12, PYRE_Q5_K = 13, PYRE_Q6_K = 14, PYRE_IQ2_XXS = 16, PYRE_IQ2_XS = 17,
-       PYRE_IQ3_XXS = 18, PYRE_IQ4_NL = 20, PYRE_IQ3_S = 21, PYRE_IQ2_S = 22, PYRE_IQ4_XS = 23, PYRE_BF16 = 30, PYRE_Q2_0 = 42 };
+       PYRE_IQ3_XXS = 18, PYRE_IQ4_NL = 20, PYRE_IQ3_S = 21, PYRE_IQ2_S = 22, PYRE_IQ4_XS = 23, PYRE_IQ1_M = 29, PYRE_BF16 = 30, PYRE_Q2_0 = 42 };
 
 enum { PYRE_OK = 0, PYRE_E_ARG = -1, PYRE_E_TYPE = -2, PYRE_E_SHAPE = -3, PYRE_E_HIP = -4, PYRE_E_STATE = -5, PYRE_E_NOMEM = -6 };
 

@@ -81,12 +81,13 @@ bool geom(uint32_t ty, int* el, int* by) {
     case ORC_Q3_K: *el = 256; *by = 110; return true;
     case ORC_Q2_0: *el = 64; *by = 18; return true;
     case ORC_Q5_K: *el = 256; *by = 176; return true;
+    case ORC_IQ1_M: *el = 256; *by = 56; return true;
   }
   return false;
 }
 
 // dequant, gguf_q.rs:67-166 (arms F32 :71, F16 :72, BF16 :73, Q4_0 :74-75, Q5_0 :76-78, Q8_0 :79, IQ4NL :82-83, IQ4XS :84-89,
-// Q2_0 :80-81, Q3K :90-102, Q4K :103-107, Q5K :108-113, Q6K :114-121, IQ2XXS :122-125, IQ2XS :126-129, IQ2S :130-135, IQ3XXS :136-140, IQ3S :141-151)
+// Q2_0 :80-81, Q3K :90-102, Q4K :103-107, Q5K :108-113, Q6K :114-121, IQ1M :152-165, IQ2XXS :122-125, IQ2XS :126-129, IQ2S :130-135, IQ3XXS :136-140, IQ3S :141-151)
 bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
   int qk, bs; if (!geom(ty, &qk, &bs)) return false;
   size_t nb = n / qk;
@@ -106,6 +107,23 @@ bool dequant(uint32_t ty, const uint8_t* x, size_t n, float* y) {
           float d1 = d * (float)s1, M1 = mn * (float)m1, d2 = d * (float)s2, M2 = mn * (float)m2;
           for (int l = 0; l < 32; ++l) { yy[l] = d1 * (float)(q[l] & 0xF) - M1; yy[l + 32] = d2 * (float)(q[l] >> 4) - M2; }
           yy += 64; q += 32;
+        }
+      }
+      break;
+    case ORC_IQ1_M:         // gguf_q.rs:152-165; grid entry e, byte j as int8 = ((kIq1sCode[e] >> 2j) & 3) - 1
+      for (size_t i = 0; i < nb; ++i) {
+        const uint8_t* b = x + i * bs; const uint8_t* qs = b; const uint8_t* qh = b + 32; const uint8_t* scb = b + 48;
+        const uint16_t sc[4] = {(uint16_t)(scb[0] | (scb[1] << 8)), (uint16_t)(scb[2] | (scb[3] << 8)), (uint16_t)(scb[4] | (scb[5] << 8)), (uint16_t)(scb[6] | (scb[7] << 8))};
+        const uint16_t su = (uint16_t)((sc[0] >> 12) | ((sc[1] >> 8) & 0x00f0) | ((sc[2] >> 4) & 0x0f00) | (sc[3] & 0xf000));
+        const uint8_t sub[2] = {(uint8_t)(su & 0xFF), (uint8_t)(su >> 8)}; const float d = h2f(sub); float* yy = y + i * 256;
+        for (int ib = 0; ib < 8; ++ib) {
+          const float dl1 = d * (float)(2 * ((sc[ib / 2] >> (6 * (ib % 2))) & 7) + 1), dl2 = d * (float)(2 * ((sc[ib / 2] >> (6 * (ib % 2) + 3)) & 7) + 1);
+          const size_t idx[4] = {(size_t)qs[0] | (((size_t)qh[0] << 8) & 0x700), (size_t)qs[1] | (((size_t)qh[0] << 4) & 0x700), (size_t)qs[2] | (((size_t)qh[1] << 8) & 0x700), (size_t)qs[3] | (((size_t)qh[1] << 4) & 0x700)};
+          const float dl[4] = {(qh[0] & 0x08) ? -0.125f : 0.125f, (qh[0] & 0x80) ? -0.125f : 0.125f, (qh[1] & 0x08) ? -0.125f : 0.125f, (qh[1] & 0x80) ? -0.125f : 0.125f};
+          for (int l = 0; l < 4; ++l) { const uint16_t gc = kIq1sCode[idx[l]]; const float s = l < 2 ? dl1 : dl2;
+            for (int j = 0; j < 8; ++j) yy[j] = s * ((float)((int)((gc >> (2 * j)) & 3) - 1) + dl[l]);
+            yy += 8; }
+          qs += 4; qh += 2;
         }
       }
       break;

@@ -42,6 +42,7 @@ __global__ void k_synth_scales(uint64_t seed, size_t n_blocks, int bs, int nfiel
     float u = (float)bits * 5.9604644775390625e-08f;    // 2^-24
     float v = lo + (hi - lo) * u;
     unsigned short h = __half_as_ushort(__float2half_rn(v));
+    if (off0 < 0) { uint8_t* q = out + b * bs + 48; for (int k = 0; k < 4; ++k) q[2 * k + 1] = (uint8_t)((q[2 * k + 1] & 0x0F) | (((h >> (4 * k)) & 0xF) << 4)); continue; }      // IQ1_M: nibble k of d in the top nibble of scale word k
     uint8_t* p = out + b * bs + (f == 0 ? off0 : off1); p[0] = (uint8_t)(h & 0xFF); p[1] = (uint8_t)(h >> 8);
   }
 }
@@ -63,11 +64,12 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
     uint32_t v = 0; for (int j = 0; j < 4; ++j) v |= (uint32_t)(2 * ((kIq3sCode[i] >> (3 * j)) & 7) + 1) << (8 * j); g3[i] = v;
     uint64_t w = 0; for (int j = 0; j < 8; ++j) w |= (uint64_t)tri[(kIq2xsCode[i] >> (2 * j)) & 3] << (8 * j); g2[i] = w;
   }
-  std::vector<uint16_t> cb(2048);          // compact codes as they are: [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512], used once per matrix by the load-time re-coding
+  std::vector<uint16_t> cb(4096);          // compact codes as they are: [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512 | iq1s 2048], used once per matrix by the load-time re-coding
+  for (int i = 0; i < 2048; ++i) cb[2048 + i] = kIq1sCode[i];
   for (int i = 0; i < 256; ++i) { cb[i] = kIq2xxsCode[i]; cb[1280 + i] = kIq3xxsCode[i]; }
   for (int i = 0; i < 1024; ++i) cb[256 + i] = kIq2sCode[i];
   for (int i = 0; i < 512; ++i) cb[1536 + i] = kIq2xsCode[i];
-  if ((e = hipMalloc((void**)&ctx->d_cb, 2048 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 2048 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
+  if ((e = hipMalloc((void**)&ctx->d_cb, 4096 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 4096 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
       (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->fuse_ctl, 1024)) != hipSuccess || (e = hipMemset(ctx->fuse_ctl, 0, 1024)) != hipSuccess) {
@@ -147,7 +149,7 @@ int pyre_synth_blocks(pyre_ctx* ctx, uint32_t ty, size_t n_blocks, uint64_t seed
   PYRE_CHECK_LAUNCH(ctx);
   int nf = (fmt == FMT_Q4_K || ty == PYRE_Q5_K) ? 2 : (fmt >= FMT_Q8_0 ? 1 : 0);      // Q4_K, Q5_K: d and dmin
   if (nf) {      // the f16 super-block scale sits at byte 0 of every block format except Q6_K (byte 208) and Q3_K (byte 108)
-    hipLaunchKernelGGL(k_synth_scales, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx->stream, seed, n_blocks, g.bytes, nf, ty == PYRE_Q6_K ? 208 : (ty == PYRE_Q3_K ? 108 : 0), 2, d_lo, d_hi, (uint8_t*)dev_out);
+    hipLaunchKernelGGL(k_synth_scales, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx->stream, seed, n_blocks, g.bytes, nf, ty == PYRE_Q6_K ? 208 : (ty == PYRE_Q3_K ? 108 : (ty == PYRE_IQ1_M ? -1 : 0)), 2, d_lo, d_hi, (uint8_t*)dev_out);
     PYRE_CHECK_LAUNCH(ctx);
   }
   return PYRE_OK;

@@ -34,6 +34,7 @@ __host__ __device__ inline bool ggml_geom(uint32_t ty, int* el, int* bytes) {
     case PYRE_Q4_0: *el = 32; *bytes = 18; return true;  case PYRE_Q5_0: *el = 32; *bytes = 22; return true;  case PYRE_Q8_0: *el = 32; *bytes = 34; return true;
     case PYRE_Q4_K: *el = 256; *bytes = 144; return true;  case PYRE_Q6_K: *el = 256; *bytes = 210; return true;
     case PYRE_Q3_K: *el = 256; *bytes = 110; return true;  case PYRE_Q2_0: *el = 64; *bytes = 18; return true;  case PYRE_Q5_K: *el = 256; *bytes = 176; return true;
+    case PYRE_IQ1_M: *el = 256; *bytes = 56; return true;
     case PYRE_IQ2_XXS: *el = 256; *bytes = 66; return true;  case PYRE_IQ2_XS: *el = 256; *bytes = 74; return true;  case PYRE_IQ2_S: *el = 256; *bytes = 82; return true;
     case PYRE_IQ3_XXS: *el = 256; *bytes = 98; return true;  case PYRE_IQ3_S: *el = 256; *bytes = 110; return true;
     case PYRE_IQ4_NL: *el = 32; *bytes = 18; return true;  case PYRE_IQ4_XS: *el = 256; *bytes = 136; return true;
@@ -44,14 +45,16 @@ inline int fmt_from_ggml(uint32_t ty) {
   switch (ty) { case PYRE_F32: return FMT_F32; case PYRE_F16: return FMT_F16; case PYRE_BF16: return FMT_BF16; case PYRE_Q8_0: return FMT_Q8_0;
     case PYRE_Q4_K: return FMT_Q4_K; case PYRE_IQ2_XS: return FMT_IQ2_XS; case PYRE_IQ3_S: return FMT_IQ3_S;
     case PYRE_IQ2_XXS: case PYRE_IQ2_S: return FMT_IQ2_XS;
-    case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ3_XXS: case PYRE_Q3_K: case PYRE_Q2_0: return FMT_C4;
+    case PYRE_Q4_0: case PYRE_IQ4_NL: case PYRE_IQ4_XS: case PYRE_IQ3_XXS: case PYRE_Q3_K: case PYRE_Q2_0: case PYRE_IQ1_M: return FMT_C4;
     case PYRE_Q5_0: case PYRE_Q6_K: case PYRE_Q5_K: return FMT_C8; }
   return -1;
 }
 // The C4 value table of a GGUF type: entry c (byte c%4 of word c/4) holds value + bias, 0..255.
 //   Q4_0: c - 8.  IQ4_NL, IQ4_XS: the sixteen non-linear levels (kIq4nlValues).  IQ3_XXS codes a value as
 //   (negative << 3) | magnitude index, magnitudes {4, 12, .., 52, 62}.  Q3_K: code = two low bits | high-mask bit << 2, value
-//   code - 4 (gguf_q.rs:99: low - (mask set ? 0 : 4)).  Q2_0: the two-bit code - 1 (gguf_q.rs:50).
+//   code - 4 (gguf_q.rs:99: low - (mask set ? 0 : 4)).  Q2_0: the two-bit code - 1 (gguf_q.rs:50).  IQ1_M (gguf_q.rs:152-165): a value is
+//   s * (g + delta), g in {-1, 0, 1}, delta = +-0.125; code = (g + 1) | (delta negative) << 2 stands for the integer 8 g +- 1 and the
+//   group's scale is s / 8 (a power-of-two scaling: the product rounds exactly as the reference's).
 inline void c4_table(uint32_t ty, uint32_t lut[4], int* bias) {
   int v[16] = {0}; int b = 0;
   static const int lv3[8] = {4, 12, 20, 28, 36, 44, 52, 62};
@@ -61,6 +64,7 @@ inline void c4_table(uint32_t ty, uint32_t lut[4], int* bias) {
     case PYRE_IQ3_XXS: for (int c = 0; c < 8; ++c) { v[c] = lv3[c]; v[8 + c] = -lv3[c]; } b = 62; break;
     case PYRE_Q3_K: for (int c = 0; c < 8; ++c) v[c] = c - 4; b = 8; break;
     case PYRE_Q2_0: for (int c = 0; c < 4; ++c) v[c] = c - 1; b = 8; break;
+    case PYRE_IQ1_M: for (int c = 0; c < 8; ++c) v[c] = 8 * ((c & 3) - 1) + ((c & 4) ? -1 : 1); b = 17; break;
     default: break;
   }
   for (int w = 0; w < 4; ++w) { lut[w] = 0; for (int k = 0; k < 4; ++k) lut[w] |= (uint32_t)(v[4 * w + k] + b) << (8 * k); }

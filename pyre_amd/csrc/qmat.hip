@@ -57,7 +57,7 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
       if (j == 0) { uint8_t* dd = pb + (((size_t)tile * (m.U >> 2) + (ku >> 2)) * 64 + lane) * 2; dd[0] = (uint8_t)(dbits & 0xFF); dd[1] = (uint8_t)(dbits >> 8); }
     } break;
     case FMT_C4: case FMT_C8: {
-      // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512]; code(e) and scale(e / 16) of the unit's 64 values e
+      // cb: compact codebooks [iq2xxs 256 | iq2s 1024 | iq3xxs 256 | iq2xs 512 | iq1s 2048]; code(e) and scale(e / 16) of the unit's 64 values e
       uint32_t words[16]; float sc[4], off[4];
       for (int i = 0; i < 16; ++i) words[i] = 0;
       for (int i = 0; i < 4; ++i) { sc[i] = 0.0f; off[i] = 0.0f; }
@@ -104,6 +104,18 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
             sc[g4] = d * (float)((int)(int8_t)((aux[is >> 2] >> (8 * (is & 3))) & 0xFF) - 32);
             for (int l = 0; l < 16; ++l) { const int o = l + 16 * half; put4(16 * g4 + l, ((q[o] >> shift) & 3) | ((hm[o] & mbit) ? 4u : 0u)); }
           }
+        } break;
+        case PYRE_IQ1_M: {                                             // gguf_q.rs:152-165
+          const uint8_t* b = row + (size_t)(ku >> 2) * 56; const uint8_t* scb = b + 48;
+          const uint32_t s16[4] = {(uint32_t)scb[0] | (scb[1] << 8), (uint32_t)scb[2] | (scb[3] << 8), (uint32_t)scb[4] | (scb[5] << 8), (uint32_t)scb[6] | (scb[7] << 8)};
+          const uint32_t su = (s16[0] >> 12) | ((s16[1] >> 8) & 0x00f0) | ((s16[2] >> 4) & 0x0f00) | (s16[3] & 0xf000);
+          const float d = __half2float(__ushort_as_half((unsigned short)su));
+          for (int c = 0; c < 2; ++c) { const int ib = 2 * (ku & 3) + c; const uint8_t* qs = b + 4 * ib; const uint8_t* qh = b + 32 + 2 * ib;
+            const float dl1 = d * (float)(2 * ((s16[ib / 2] >> (6 * (ib % 2))) & 7) + 1), dl2 = d * (float)(2 * ((s16[ib / 2] >> (6 * (ib % 2) + 3)) & 7) + 1);
+            sc[2 * c] = dl1 * 0.125f; sc[2 * c + 1] = dl2 * 0.125f;
+            const uint32_t idx[4] = {(uint32_t)qs[0] | (((uint32_t)qh[0] << 8) & 0x700), (uint32_t)qs[1] | (((uint32_t)qh[0] << 4) & 0x700), (uint32_t)qs[2] | (((uint32_t)qh[1] << 8) & 0x700), (uint32_t)qs[3] | (((uint32_t)qh[1] << 4) & 0x700)};
+            const uint32_t neg[4] = {(uint32_t)(qh[0] >> 3) & 1, (uint32_t)(qh[0] >> 7) & 1, (uint32_t)(qh[1] >> 3) & 1, (uint32_t)(qh[1] >> 7) & 1};
+            for (int l = 0; l < 4; ++l) { const uint32_t gc = cb[2048 + idx[l]]; for (int j = 0; j < 8; ++j) put4(32 * c + 8 * l + j, ((gc >> (2 * j)) & 3) | (neg[l] << 2)); } }
         } break;
         case PYRE_Q5_K: {                                              // gguf_q.rs:108-113
           const uint8_t* b = row + (size_t)(ku >> 2) * 176; const float d = h2(b), mn = h2(b + 2); const int j = ku & 3;

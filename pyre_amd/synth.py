@@ -21,9 +21,10 @@ SCALE_SALT = np.uint64(0xD1B54A32D192ED03)
 GEOM = {8: (32, 34, (0,)), 12: (256, 144, (0, 2)), 17: (256, 74, (0,)), 21: (256, 110, (0,)),
         0: (1, 4, ()), 1: (1, 2, ()), 30: (1, 2, ()),
         2: (32, 18, (0,)), 6: (32, 22, (0,)), 14: (256, 210, (208,)), 16: (256, 66, (0,)), 18: (256, 98, (0,)),
-        20: (32, 18, (0,)), 22: (256, 82, (0,)), 23: (256, 136, (0,)), 11: (256, 110, (108,)), 42: (64, 18, (0,)), 13: (256, 176, (0, 2))}
+        20: (32, 18, (0,)), 22: (256, 82, (0,)), 23: (256, 136, (0,)), 11: (256, 110, (108,)), 42: (64, 18, (0,)), 13: (256, 176, (0, 2)),
+        29: (256, 56, (-1,))}        # IQ1_M: the f16 scale is scattered over the top nibbles of the four scale words (bytes 49, 51, 53, 55)
 Q8_0, Q4_K, IQ2_XS, IQ3_S, F32, F16, BF16 = 8, 12, 17, 21, 0, 1, 30
-Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS, Q3_K, Q2_0, Q5_K = 2, 6, 14, 16, 18, 20, 22, 23, 11, 42, 13
+Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS, Q3_K, Q2_0, Q5_K, IQ1_M = 2, 6, 14, 16, 18, 20, 22, 23, 11, 42, 13, 29
 
 
 def mix64(z):
@@ -53,6 +54,11 @@ def blocks(ty, n_blocks, seed, d_lo=1e-3, d_hi=2e-2):
             bits = (w >> np.uint64(40)) if fi == 0 else ((w >> np.uint64(16)) & np.uint64(0xFFFFFF))
             u = bits.astype(np.float32) * np.float32(2.0 ** -24)
             v = (lo + (hi - lo) * u).astype(np.float32).astype(np.float16)
+            if off < 0:
+                h = v.view(np.uint16).astype(np.uint32)
+                for k in range(4):
+                    b[:, 49 + 2 * k] = (b[:, 49 + 2 * k] & 0x0F) | (((h >> (4 * k)) & 0xF) << 4).astype(np.uint8)
+                continue
             b[:, off:off + 2] = v.view(np.uint8).reshape(n_blocks, 2)
     return raw
 

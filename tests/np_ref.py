@@ -17,6 +17,7 @@ IQ3S_SHA256 = "bd1af4945a1717c65610b0284e4628b9a1ba3b306fae3a06f6e5f597356e349f"
 IQ2XS_SHA256 = "06e47aaca60b4dc1d9b5a3f34540437058a6b142b4d7a59d5ded769b4d1bf1de"
 KSIGNS_SHA256 = "a76742a603f8beca5212ecce0f1f02f11a4887fd2f7c8b15aca0ea3eb3380c31"
 IQ2XXS_SHA256 = "05826b5d3e472a3a78f196be62ac78acf81df0f909626e12ab9fa2a5d490dd54"
+IQ1S_SHA256 = "07540ffc1aeaf6ad4d97e96b0fcc765aae39671d4ae4a27bbd0e796fde167c6a"      # IQ1S_GRID (iq_tables.rs:321 of the reference), 2048 x 8 int8
 IQ2S_SHA256 = "e1aa1473412b0552c2174c30ef22ab4073f6a181b85a17056e8249bd2932fd88"
 IQ3XXS_SHA256 = "46e35f5a997efdee6c99ce57854c8a0d4f0ff8ca57e5e8a60c0793ea580acf5d"
 # the IQ4_NL / IQ4_XS non-linear levels (ggml's kvalues_iq4nl, iq_tables.rs:579 of the reference)
@@ -59,6 +60,13 @@ def codebooks_more(header=None):
     m = re.search(r"kIq4nlValues\[16\] = \{(.*?)\};", open(header).read(), re.S)
     kv = np.array([int(v) for v in re.findall(r"-?\d+", m.group(1))], dtype=np.int8)
     return gxx, gs, g3, kv
+
+
+def codebook_iq1s(header=None):
+    """iq1s_grid i8[2048, 8] expanded from a codebook header: byte j of entry e = ((code >> 2j) & 3) - 1."""
+    header = header or os.path.join(_ROOT, "oracle", "iq_codebooks.h")
+    c = _codes(header, "kIq1sCode")
+    return np.stack([((c >> (2 * j)) & 3).astype(np.int8) - 1 for j in range(8)], axis=1).astype(np.int8)
 
 
 def codebook_digests_more(header=None):
@@ -153,6 +161,24 @@ def dequant(ty, raw, n):
         hb = ((qh >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32)
         q = np.concatenate([b[:, 6:] & 0xF, b[:, 6:] >> 4], axis=1).astype(np.int32) + 16 * hb - 16
         return (q.astype(f) * d).astype(f).reshape(-1)
+    if ty == 29:                                                       # IQ1_M: qs[32] | qh[16] | four u16 scale words whose top nibbles spell the f16 d
+        b = raw[:n // 256 * 56].reshape(-1, 56)
+        nb = b.shape[0]
+        g1 = codebook_iq1s().astype(f)                                 # [2048, 8]
+        sc = b[:, 48:56].copy().view(np.uint16).reshape(nb, 4).astype(np.uint32)
+        su = ((sc[:, 0] >> 12) | ((sc[:, 1] >> 8) & 0xF0) | ((sc[:, 2] >> 4) & 0xF00) | (sc[:, 3] & 0xF000)).astype(np.uint16)
+        d = su.view(np.float16).astype(f).reshape(nb, 1)
+        qs = b[:, 0:32].reshape(nb, 8, 4).astype(np.uint32); qh = b[:, 32:48].reshape(nb, 8, 2).astype(np.uint32)
+        ib = np.arange(8)
+        w = sc[:, ib // 2]                                             # [nb, 8]: the scale word of sub-block ib
+        s3a = (w >> (6 * (ib % 2))) & 7; s3b = (w >> (6 * (ib % 2) + 3)) & 7
+        dl1 = (d * (2 * s3a + 1).astype(f)).astype(f); dl2 = (d * (2 * s3b + 1).astype(f)).astype(f)      # [nb, 8]
+        hi = np.stack([(qh[:, :, 0] << 8) & 0x700, (qh[:, :, 0] << 4) & 0x700, (qh[:, :, 1] << 8) & 0x700, (qh[:, :, 1] << 4) & 0x700], axis=2)
+        idx = qs | hi                                                  # [nb, 8, 4]
+        neg = np.stack([qh[:, :, 0] & 0x08, qh[:, :, 0] & 0x80, qh[:, :, 1] & 0x08, qh[:, :, 1] & 0x80], axis=2) != 0
+        delta = np.where(neg, f(-0.125), f(0.125)).astype(f)           # [nb, 8, 4]
+        s = np.stack([dl1, dl1, dl2, dl2], axis=2)                     # groups 0, 1 of a sub-block use the first 3-bit scale, 2, 3 the second
+        return (s[:, :, :, None] * (g1[idx] + delta[:, :, :, None]).astype(f)).astype(f).reshape(-1)
     if ty == 13:                                                       # Q5_K: d | dmin | scales[12] | qh[32] | ql[128]; (d*s) * (nibble + 16*bit) - dmin*m
         b = raw[:n // 256 * 176].reshape(-1, 176)
         nb = b.shape[0]

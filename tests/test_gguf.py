@@ -59,7 +59,7 @@ def test_refusals(tmp_path):
     with pytest.raises(lib.PyreError, match="not GGUF"):
         lib.Gguf(p)
     good = str(tmp_path / "g.gguf")
-    gw.write(good, [("k", gw.STR, "v" * 100)], [("i1", [256], 29, np.zeros(56, np.uint8)), ("q6", [256], synth.Q6_K, np.zeros(210, np.uint8)), ("odd", [48], synth.Q8_0, np.zeros(51, np.uint8)),
+    gw.write(good, [("k", gw.STR, "v" * 100)], [("q2k", [256], 10, np.zeros(84, np.uint8)), ("q6", [256], synth.Q6_K, np.zeros(210, np.uint8)), ("odd", [48], synth.Q8_0, np.zeros(51, np.uint8)),
                                                  ("t", [64, 8], synth.Q8_0, synth.matrix(synth.Q8_0, 8, 64, 1))])
     raw = open(good, "rb").read()
     for cut in (10, 30, 60, 150, len(raw) - 100):                                                   # truncated header, key, tensor info, data
@@ -77,8 +77,8 @@ def test_refusals(tmp_path):
     with pytest.raises(lib.PyreError):
         lib.Gguf(p)
     g = lib.Gguf(good)
-    with pytest.raises(lib.PyreError, match="IQ1_M.*not supported"):
-        g.tensor("i1")
+    with pytest.raises(lib.PyreError, match="Q2_K.*not supported"):
+        g.tensor("q2k")
     assert g.tensor("q6")[0] == synth.Q6_K
     with pytest.raises(lib.PyreError, match="not a multiple of block"):
         g.tensor("odd")

@@ -9,7 +9,7 @@ from helpers import relerr
 from pyre_amd import lib, synth
 
 pytestmark = pytest.mark.gpu
-FMTS = [lib.Q8_0, lib.Q4_K, lib.IQ2_XS, lib.IQ3_S, lib.Q4_0, lib.Q5_0, lib.Q6_K, lib.IQ2_XXS, lib.IQ3_XXS, lib.IQ4_NL, lib.IQ2_S, lib.IQ4_XS, lib.Q3_K, lib.Q2_0, lib.Q5_K]
+FMTS = [lib.Q8_0, lib.Q4_K, lib.IQ2_XS, lib.IQ3_S, lib.Q4_0, lib.Q5_0, lib.Q6_K, lib.IQ2_XXS, lib.IQ3_XXS, lib.IQ4_NL, lib.IQ2_S, lib.IQ4_XS, lib.Q3_K, lib.Q2_0, lib.Q5_K, lib.IQ1_M]
 ALL = FMTS + [lib.BF16, lib.F16, lib.F32]
 TOL = 1e-5
 

@@ -10,7 +10,7 @@ from pyre_amd import synth
 
 FMTS = [orc.Q8_0, orc.Q4_K, orc.IQ2_XS, orc.IQ3_S]
 # the other block types real files of this architecture use (gguf_q.rs:74-78,82-89,114-125,130-140)
-FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS, orc.Q3_K, orc.Q2_0, orc.Q5_K]
+FMTS_MORE = [orc.Q4_0, orc.Q5_0, orc.Q6_K, orc.IQ2_XXS, orc.IQ3_XXS, orc.IQ4_NL, orc.IQ2_S, orc.IQ4_XS, orc.Q3_K, orc.Q2_0, orc.Q5_K, orc.IQ1_M]
 
 
 def bits(a):
@@ -23,6 +23,8 @@ def test_codebook_digests_match_reference_tables():
         p = os.path.join(np_ref._ROOT, hdr)
         assert np_ref.codebook_digests(p) == (np_ref.IQ3S_SHA256, np_ref.IQ2XS_SHA256, np_ref.KSIGNS_SHA256)
         assert np_ref.codebook_digests_more(p) == (np_ref.IQ2XXS_SHA256, np_ref.IQ2S_SHA256, np_ref.IQ3XXS_SHA256, np_ref.IQ4NL_VALUES)
+        import hashlib
+        assert hashlib.sha256(np_ref.codebook_iq1s(p).tobytes()).hexdigest() == np_ref.IQ1S_SHA256
 
 
 def test_oracle_expansion_equals_numpy_expansion():
@@ -136,6 +138,34 @@ def test_q2_0_and_q3_k_known_answers():
     exp[52] = ((5 | (1 << 4)) - 32) * 3.0               # value 32 + 20 lies in scale 3's group: code 3, mask set
     exp[128 + 96 + 7] = -32.0 * (1 - 4)
     assert np.array_equal(y, exp)
+
+
+def test_iq1_m_known_answers():
+    # gguf_q.rs:152-165.  The IQ1S grid is ggml's; its expansion is pinned by digest like the other grids.
+    g1 = np_ref.codebook_iq1s()
+    import hashlib
+    assert hashlib.sha256(g1.tobytes()).hexdigest() == np_ref.IQ1S_SHA256
+    assert set(np.unique(g1)) == {-1, 0, 1}
+
+    def blk(d):
+        b = np.zeros(56, np.uint8); h = int(np.array([d], np.float16).view(np.uint16)[0])
+        for k in range(4):
+            b[49 + 2 * k] = ((h >> (4 * k)) & 0xF) << 4
+        return b
+    # zero payload: index 0, 3-bit scales 0 -> d * 1, delta +0.125: every value d * (grid[0] + 0.125)
+    y = orc.dequant(orc.IQ1_M, blk(2.0), 256).reshape(32, 8)
+    assert np.array_equal(y, np.tile(2.0 * (g1[0].astype(np.float32) + 0.125), (32, 1)))
+    # sub-block 5 (second half of scale word 2): first scale 3 -> x7, second scale 6 -> x13; group 1 of it: index 0x2A5 (high bits 2 from
+    # qh[0] bits 4-6), delta negative (qh[0] bit 7); group 2: index 0x733 (high bits 7 from qh[1] bits 0-2), delta positive
+    b = blk(0.5)
+    w2 = (3 << 6) | (6 << 9); b[48 + 4] |= w2 & 0xFF; b[48 + 5] |= (w2 >> 8) & 0x0F
+    b[4 * 5 + 1] = 0xA5; b[32 + 2 * 5 + 0] = (2 << 4) | 0x80
+    b[4 * 5 + 2] = 0x33; b[32 + 2 * 5 + 1] = 7
+    y = orc.dequant(orc.IQ1_M, b, 256).reshape(8, 4, 8)
+    assert np.array_equal(y[5, 1], (0.5 * 7) * (g1[0x2A5].astype(np.float32) - 0.125))
+    assert np.array_equal(y[5, 2], (0.5 * 13) * (g1[0x733].astype(np.float32) + 0.125))
+    assert np.array_equal(y[5, 0], (0.5 * 7) * (g1[0].astype(np.float32) + 0.125)) and np.array_equal(y[5, 3], (0.5 * 13) * (g1[0].astype(np.float32) + 0.125))
+    assert np.array_equal(y[4, 0], 0.5 * (g1[0].astype(np.float32) + 0.125))       # first half of the same scale word: 3-bit scales 0
 
 
 def test_q5_k_known_answers():
