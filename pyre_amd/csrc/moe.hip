@@ -80,7 +80,9 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // rows on nz compute units instead of one; at one token a launch of tiles x (k+1) workgroups leaves most of the chip
 // idle -- and leaves the part's raw sums, gate at h[((entry*nz + kz)*2 + 0)*hstride + row], up at [... + 1]; the down
 // launch adds the parts and forms silu(g) * u with the same operations.
-template <int FMT, int NW, int P>
+// PRE: the token's experts were chosen by k_moe_route (windows of several tokens: hundreds of workgroups would each redo
+// the selection otherwise); the workgroup reads its expert id and publishes nothing but the shared-expert gate.
+template <int FMT, int NW, int P, bool PRE>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
@@ -94,8 +96,8 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   const float* xs = x + (size_t)ti * m.d;
   int expert = 0;
   if (!shared) {
-    route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl);
-    expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]);
+    if constexpr (PRE) expert = __builtin_amdgcn_readfirstlane(sel_idx[ti * m.top_k + j]);
+    else { route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl); expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]); }
   } else if (blockIdx.x == 0) {
     float p = 0.0f;
     for (int ib = threadIdx.x; ib < m.d; ib += 4 * NW * 64) {          // four elements per pass, loads first (elements past d: weight zero)
@@ -162,11 +164,20 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   // activations in scalar registers (it could no longer prove them unmodified).
   if (blockIdx.x == 0 && kz == 0) {
     if (shared) { if (threadIdx.x == 0) sg[ti] = rl.s_w[0]; }
-    else if (j == 0) {
+    else if (!PRE && j == 0) {
       route_weights(m.top_k, rl);       // thread e < k writes and then reads its own s_w entry
       if (threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
     }
   }
+}
+
+// ---- routing alone (windows of several tokens): grid t, 1024 threads; ids ascending and softmax weights of token ti ------
+__global__ __launch_bounds__(1024) void k_moe_route(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int nsl, int sstride, int tstride) {
+  __shared__ RouteLds rl;
+  const int ti = blockIdx.x;
+  route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl);
+  route_weights(m.top_k, rl);
+  if ((int)threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
 }
 
 // ---- expert down: partial[entry][r] = down[r] . h[entry] ---------------------------------------------------------------
@@ -262,8 +273,12 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   const int P = pyre_moe_gu_parts(m), nz = (P > 1 && t == 1) ? P : 1;
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
-#define GU_GO(PP, NZ) MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP>), dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride))
-  if (nz > 1 || P == 1) { GU_GO(1, nz); } else { GU_GO(2, 1); } }
+#define GU_GO(PP, NZ, PRE) MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP, PRE>), dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride))
+  if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
+  else {
+    hipLaunchKernelGGL(k_moe_route, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
+    if (P == 2) { GU_GO(2, 1, true); } else { GU_GO(1, 1, true); }
+  } }
 #undef GU_GO
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
