@@ -266,6 +266,17 @@ int   pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, i
  * out [n_out] tokens; *rounds (optional) = verify rounds used. */
 int   pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
                            int n_draft, const uint32_t* draft_stream, int* rounds);
+/* Prompt-lookup drafter, spec::ngram_draft (src/spec.rs:122-139): the most recent earlier occurrence of the longest suffix
+ * (n = max_n .. min_n tokens) of history[0..len) and up to k tokens that followed it -> out [k]; returns how many (0: no
+ * match).  Host only: no context, no GPU. */
+int   pyre_ngram_draft(const uint32_t* history, size_t len, int k, int min_n, int max_n, uint32_t* out);
+/* spec::generate, greedy branch, with that drafter supplying the drafts (src/spec.rs:207: drafts = ngram_draft(history, kk,
+ * ng_min, ng_max), the reference's defaults are 3 and 8): history [n_hist] are the tokens the state has consumed (the
+ * prompt); a round without a match is a plain single-token step.  k = drafts per round at most, 1..7.  The output equals
+ * plain greedy decoding token for token.  *rounds / *drafted / *accepted (optional): verify rounds, drafts verified, drafts
+ * accepted (spec::Outcome, src/spec.rs:150-154). */
+int   pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* history, size_t n_hist, const float* first_logits_host,
+                                 int n_out, uint32_t* out, int k, int ng_min, int ng_max, int* rounds, int* drafted, int* accepted);
 /* The decode loop as the benchmark times it: n_steps greedy steps starting from token `first`, everything on the device;
  * tokens (optional, host) receives the n_steps generated ids after the call. */
 int   pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host);

@@ -606,4 +606,48 @@ int pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, cons
   return PYRE_OK;
 }
 
+int pyre_ngram_draft(const uint32_t* h, size_t len, int k, int min_n, int max_n, uint32_t* out) {
+  if (!h || !out || k <= 0 || min_n < 1 || len < (size_t)min_n + 1) return 0;
+  const size_t top = (size_t)max_n < len - 1 ? (size_t)max_n : len - 1;
+  for (size_t n = top; n >= (size_t)min_n && n <= top; --n) {          // longest suffix first
+    const uint32_t* suf = h + len - n;
+    for (size_t i = len - n; i > 0;) {                                  // start positions from the most recent down, i + n < len
+      --i;
+      if (h[i + n - 1] == suf[n - 1] && memcmp(h + i, suf, n * sizeof(uint32_t)) == 0) {
+        const size_t s0 = i + n, e = s0 + (size_t)k < len ? s0 + (size_t)k : len;
+        if (e > s0) { for (size_t q = s0; q < e; ++q) out[q - s0] = h[q]; return (int)(e - s0); }
+      }
+    }
+  }
+  return 0;
+}
+
+int pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* history, size_t n_hist, const float* first_logits, int n_out, uint32_t* out,
+                               int k, int ng_min, int ng_max, int* rounds_out, int* drafted_out, int* accepted_out) {
+  if (!ctx || !m || !s || !first_logits || !out || n_out < 1 || (n_hist && !history)) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_ngram: bad argument");
+  if (k < 1 || k > 7 || ng_min < 1 || ng_max < ng_min) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_ngram: k %d (1..7), n-gram lengths %d..%d", k, ng_min, ng_max);
+  const size_t V = m->c.vocab; int produced = 0, rounds = 0, drafted = 0, accepted = 0;
+  std::vector<uint32_t> hist(history, history + n_hist); hist.reserve(n_hist + (size_t)n_out + 8);
+  std::vector<float> ls((size_t)8 * V);
+  uint32_t pending = host_argmax(first_logits, V);
+  for (;;) {
+    hist.push_back(pending); out[produced++] = pending; if (produced >= n_out) break;
+    const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
+    uint32_t toks[8]; toks[0] = pending;
+    const int nd = kk > 0 ? pyre_ngram_draft(hist.data(), hist.size(), kk, ng_min, ng_max, toks + 1) : 0;
+    if (nd == 0) { int rc = pyre_forward(ctx, m, s, &pending, 1, ls.data()); if (rc) return rc; pending = host_argmax(ls.data(), V); continue; }
+    int rc = pyre_forward_multi(ctx, m, s, toks, nd + 1, ls.data()); if (rc) return rc;
+    int acc = 0; bool have = false; uint32_t nx = 0;
+    for (int i = 0; i < nd; ++i) { uint32_t tk = host_argmax(ls.data() + (size_t)i * V, V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = host_argmax(ls.data() + (size_t)nd * V, V);
+    if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
+    ++rounds; drafted += nd; accepted += acc;
+    bool stop = false; for (int i = 0; i < acc; ++i) { hist.push_back(toks[i + 1]); out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
+    if (stop) break;
+    pending = nx;
+  }
+  if (rounds_out) *rounds_out = rounds; if (drafted_out) *drafted_out = drafted; if (accepted_out) *accepted_out = accepted;
+  return PYRE_OK;
+}
+
 }  // extern "C"

@@ -111,6 +111,8 @@ def _declare(L):
         "pyre_forward_multi": (i32, [vp, vp, vp, vp, i32, vp]),
         "pyre_spec_keep": (i32, [vp, vp, vp, i32, i32]),
         "pyre_generate_greedy": (i32, [vp, vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32)]),
+        "pyre_ngram_draft": (i32, [vp, C.c_size_t, i32, i32, i32, vp]),
+        "pyre_generate_greedy_ngram": (i32, [vp, vp, vp, vp, C.c_size_t, vp, i32, vp, i32, i32, i32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
         "pyre_decode_greedy_dev": (i32, [vp, vp, vp, u32, i32, vp]),
     }
     for name, (res, args) in sig.items():
@@ -136,6 +138,13 @@ def load():
         _declare(L)
         _lib = L
     return _lib
+
+
+def ngram_draft(history, k, min_n, max_n):
+    """spec::ngram_draft through the library (host only, needs no GPU)."""
+    h = np.ascontiguousarray(history, dtype=np.uint32); out = np.empty(max(k, 1), dtype=np.uint32)
+    n = load().pyre_ngram_draft(h.ctypes.data_as(C.c_void_p), h.size, k, min_n, max_n, out.ctypes.data_as(C.c_void_p))
+    return out[:n].copy()
 
 
 def _ptr(a):
@@ -627,6 +636,14 @@ class Model:
         rounds = C.c_int(0)
         self.ctx.check(self.ctx.L.pyre_generate_greedy(self.ctx.h, self.h, st.h, _ptr(fl), n_out, _ptr(out), n_draft, _ptr(ds), C.byref(rounds)), "generate_greedy")
         return out, rounds.value
+
+    def generate_greedy_ngram(self, st, history, first_logits, n_out, k=4, ng_min=3, ng_max=8):
+        """spec::generate (greedy) with the prompt-lookup drafter; returns (tokens, rounds, drafted, accepted)."""
+        fl = np.ascontiguousarray(first_logits, dtype=np.float32); hs = np.ascontiguousarray(history, dtype=np.uint32)
+        out = np.empty(n_out, dtype=np.uint32); r, d, a = C.c_int(0), C.c_int(0), C.c_int(0)
+        self.ctx.check(self.ctx.L.pyre_generate_greedy_ngram(self.ctx.h, self.h, st.h, _ptr(hs), hs.size, _ptr(fl), n_out, _ptr(out), k, ng_min, ng_max,
+                                                             C.byref(r), C.byref(d), C.byref(a)), "generate_greedy_ngram")
+        return out, r.value, d.value, a.value
 
     def decode_greedy_dev(self, st, first, n_steps, fetch=True):
         out = np.empty(n_steps, dtype=np.uint32) if fetch else None

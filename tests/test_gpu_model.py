@@ -115,6 +115,26 @@ def test_device_loop_identical_to_oracle_across_the_packing_boundary(ctx):
     assert relerr(l2, o2) <= 1e-3 and orc.argmax(l2) == orc.argmax(o2)
 
 
+def test_ngram_drafted_generation_equals_plain_greedy(ctx):
+    # spec::generate with the prompt-lookup drafter (src/spec.rs:207): whatever the drafts, the stream is plain greedy's
+    c = small_cfg()
+    hw, gm, om = pair(ctx, c, 8)
+    pat = np.array([5, 9, 200, 31, 77, 12, 64, 3], dtype=np.uint32)
+    prompt = np.concatenate([pat, pat, pat, pat[:5]])                   # a repetitive prompt: the drafter finds matches from the first round
+    ga, gb, os_ = gm.new_state(200), gm.new_state(200), om.new_state()
+    la = gm.forward(prompt, ga); lb = gm.forward(prompt, gb); lo = om.forward(prompt, os_)
+    plain, _ = gm.generate_greedy(ga, la, 60)
+    drafted, rounds, nd, na = gm.generate_greedy_ngram(gb, prompt, lb, 60, k=4, ng_min=2, ng_max=8)
+    oracle, _ = om.generate_greedy(os_, lo, 60)
+    assert np.array_equal(plain, oracle)
+    assert np.array_equal(drafted, plain), "first split at %d" % int(np.argmax(drafted != plain))
+    assert rounds > 0 and nd >= rounds and 0 <= na <= nd
+    assert len(gb) == len(ga)
+    # and both states continue alike
+    t = np.array([plain[-1]], dtype=np.uint32)
+    assert np.array_equal(gm.forward(t, ga).view(np.uint32), gm.forward(t, gb).view(np.uint32))
+
+
 def test_verify_window_equals_single_steps_and_rollback(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 7)
