@@ -508,6 +508,37 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
 }
 
+// First maximum of each of t logit rows (sampler::argmax, src/sampler.rs:142-148: a scan from index 0 with strict >, so the
+// lowest index among equal maxima, NaNs never chosen unless at index 0): grid t, 1024 threads; a thread walks its indices in ascending order, the threads then meet by (value, index).
+__global__ __launch_bounds__(1024) void k_argmax_rows(const float* __restrict__ logits, int V, uint32_t* __restrict__ best) {
+  __shared__ float sv[16]; __shared__ uint32_t si[16];
+  const float* l = logits + (size_t)blockIdx.x * V; const int tid = threadIdx.x;
+  float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
+  for (int i = tid; i < V; i += 1024) { const float v = l[i]; if (!(v != v) && (bi == 0xFFFFFFFFu || v > bv)) { bv = v; bi = (uint32_t)i; } }      // a NaN is never greater
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { const float ov = __shfl_xor(bv, o); const uint32_t oi = __shfl_xor(bi, o); if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; } }
+  if ((tid & 63) == 0) { sv[tid >> 6] = bv; si[tid >> 6] = bi; }
+  __syncthreads();
+  if (tid == 0) { for (int w = 1; w < 16; ++w) if (si[w] != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || sv[w] > bv || (sv[w] == bv && si[w] < bi))) { bv = sv[w]; bi = si[w]; }
+    best[blockIdx.x] = (bi == 0xFFFFFFFFu || l[0] != l[0]) ? 0u : bi; }          // the scan starts from index 0: a NaN there is never replaced, as on the host
+}
+
+// pyre_forward_multi for a caller that only wants each token's greedy pick: the picks are formed on the device and t
+// integers come back instead of t x vocab logits.
+static int forward_multi_picks(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, uint32_t* picks_host) {
+  if (n < 1 || n > 8) return pyre_fail(ctx, PYRE_E_ARG, "forward_multi: window of %d tokens outside 1..8", n);
+  if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "forward_multi: state belongs to another model");
+  if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward_multi: context exceeds the state's capacity %d", s->cap);
+  int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
+  PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+  { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
+  s->last_window = n;
+  hipLaunchKernelGGL(k_argmax_rows, dim3(n), dim3(1024), 0, ctx->stream, m->logits, m->c.vocab, m->best);
+  PYRE_CHECK_LAUNCH(ctx);
+  PYRE_HIP(ctx, hipMemcpyAsync(picks_host, m->best, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
+}
+
 // The DeltaNet layers kept the window's inputs and their pre-window state (the other half of the double buffer): the
 // first `keep` tokens are run again from there, which reproduces the checkpoint after token `keep` bit for bit.
 int pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int keep) {
@@ -587,16 +618,15 @@ int pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, cons
     if (produced < n_out) { int rc = pyre_decode_greedy_dev(ctx, m, s, pending, n_out - 1, out + 1); if (rc) return rc; }
     if (rounds_out) *rounds_out = 0; return PYRE_OK;
   }
-  std::vector<float> ls((size_t)8 * V);
   for (;;) {
     out[produced++] = pending; if (produced >= n_out) break;
     int left = n_out - produced; int kk = n_draft < left - 1 ? n_draft : left - 1;
-    if (kk <= 0) { int rc = pyre_forward(ctx, m, s, &pending, 1, ls.data()); if (rc) return rc; pending = host_argmax(ls.data(), V); continue; }
+    if (kk <= 0) { uint32_t pk; int rc = forward_multi_picks(ctx, m, s, &pending, 1, &pk); if (rc) return rc; pending = pk; continue; }
     uint32_t toks[8]; toks[0] = pending; for (int j = 0; j < kk; ++j) toks[j + 1] = draft_stream[produced + j];
-    int rc = pyre_forward_multi(ctx, m, s, toks, kk + 1, ls.data()); if (rc) return rc;
+    uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, kk + 1, picks); if (rc) return rc;
     int acc = 0; bool have = false; uint32_t nx = 0;
-    for (int i = 0; i < kk; ++i) { uint32_t tk = host_argmax(ls.data() + (size_t)i * V, V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
-    if (!have) nx = host_argmax(ls.data() + (size_t)kk * V, V);
+    for (int i = 0; i < kk; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = picks[kk];
     if ((rc = pyre_spec_keep(ctx, m, s, kk + 1, acc + 1))) return rc; ++rounds;
     bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
     if (stop) break;
@@ -628,18 +658,17 @@ int pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s
   if (k < 1 || k > 7 || ng_min < 1 || ng_max < ng_min) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_ngram: k %d (1..7), n-gram lengths %d..%d", k, ng_min, ng_max);
   const size_t V = m->c.vocab; int produced = 0, rounds = 0, drafted = 0, accepted = 0;
   std::vector<uint32_t> hist(history, history + n_hist); hist.reserve(n_hist + (size_t)n_out + 8);
-  std::vector<float> ls((size_t)8 * V);
   uint32_t pending = host_argmax(first_logits, V);
   for (;;) {
     hist.push_back(pending); out[produced++] = pending; if (produced >= n_out) break;
     const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
     uint32_t toks[8]; toks[0] = pending;
     const int nd = kk > 0 ? pyre_ngram_draft(hist.data(), hist.size(), kk, ng_min, ng_max, toks + 1) : 0;
-    if (nd == 0) { int rc = pyre_forward(ctx, m, s, &pending, 1, ls.data()); if (rc) return rc; pending = host_argmax(ls.data(), V); continue; }
-    int rc = pyre_forward_multi(ctx, m, s, toks, nd + 1, ls.data()); if (rc) return rc;
+    if (nd == 0) { uint32_t pk; int rc = forward_multi_picks(ctx, m, s, &pending, 1, &pk); if (rc) return rc; pending = pk; continue; }
+    uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
     int acc = 0; bool have = false; uint32_t nx = 0;
-    for (int i = 0; i < nd; ++i) { uint32_t tk = host_argmax(ls.data() + (size_t)i * V, V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
-    if (!have) nx = host_argmax(ls.data() + (size_t)nd * V, V);
+    for (int i = 0; i < nd; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = picks[nd];
     if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
     ++rounds; drafted += nd; accepted += acc;
     bool stop = false; for (int i = 0; i < acc; ++i) { hist.push_back(toks[i + 1]); out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
