@@ -266,6 +266,10 @@ int   pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, i
  * out [n_out] tokens; *rounds (optional) = verify rounds used. */
 int   pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
                            int n_draft, const uint32_t* draft_stream, int* rounds);
+/* sampler::argmax (src/sampler.rs:142-148) of t rows of `vocab` logits on the device: a scan from index 0 with strict >, so
+ * the first of equal maxima; a NaN is never greater, and a NaN at index 0 is never replaced.  The drafted loops below use
+ * the same kernel on the window's logits; this entry point takes host rows (test and tooling use). */
+int   pyre_argmax_rows(pyre_ctx* ctx, const float* logits_host, int t, int vocab, uint32_t* picks_host);
 /* Prompt-lookup drafter, spec::ngram_draft (src/spec.rs:122-139): the most recent earlier occurrence of the longest suffix
  * (n = max_n .. min_n tokens) of history[0..len) and up to k tokens that followed it -> out [k]; returns how many (0: no
  * match).  Host only: no context, no GPU. */

@@ -636,6 +636,19 @@ int pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, cons
   return PYRE_OK;
 }
 
+int pyre_argmax_rows(pyre_ctx* ctx, const float* logits_host, int t, int vocab, uint32_t* picks_host) {
+  if (!ctx || !logits_host || !picks_host || t < 1 || vocab < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_argmax_rows: bad argument");
+  float* d = nullptr; uint32_t* b = nullptr; const size_t n = (size_t)t * vocab;
+  PYRE_HIP(ctx, hipMalloc((void**)&d, n * 4 + (size_t)t * 4)); b = (uint32_t*)(d + n);
+  hipError_t e = hipMemcpyAsync(d, logits_host, n * 4, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) { hipLaunchKernelGGL(k_argmax_rows, dim3(t), dim3(1024), 0, ctx->stream, d, vocab, b); e = hipGetLastError(); }
+  if (e == hipSuccess) e = hipMemcpyAsync(picks_host, b, (size_t)t * 4, hipMemcpyDeviceToHost, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  (void)hipFree(d);
+  if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "pyre_argmax_rows: %s", hipGetErrorString(e));
+  return PYRE_OK;
+}
+
 int pyre_ngram_draft(const uint32_t* h, size_t len, int k, int min_n, int max_n, uint32_t* out) {
   if (!h || !out || k <= 0 || min_n < 1 || len < (size_t)min_n + 1) return 0;
   const size_t top = (size_t)max_n < len - 1 ? (size_t)max_n : len - 1;

@@ -112,6 +112,7 @@ def _declare(L):
         "pyre_spec_keep": (i32, [vp, vp, vp, i32, i32]),
         "pyre_generate_greedy": (i32, [vp, vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32)]),
         "pyre_ngram_draft": (i32, [vp, C.c_size_t, i32, i32, i32, vp]),
+        "pyre_argmax_rows": (i32, [vp, vp, i32, i32, vp]),
         "pyre_generate_greedy_ngram": (i32, [vp, vp, vp, vp, C.c_size_t, vp, i32, vp, i32, i32, i32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
         "pyre_decode_greedy_dev": (i32, [vp, vp, vp, u32, i32, vp]),
     }

@@ -115,6 +115,31 @@ def test_device_loop_identical_to_oracle_across_the_packing_boundary(ctx):
     assert relerr(l2, o2) <= 1e-3 and orc.argmax(l2) == orc.argmax(o2)
 
 
+def test_device_argmax_rows_follows_the_host_scan(ctx):
+    # sampler::argmax (src/sampler.rs:142-148): b = 0; for i: if l[i] > l[b] { b = i }
+    def host(l):
+        b = 0
+        for i in range(len(l)):
+            if l[i] > l[b]:
+                b = i
+        return b
+    g = np.random.Generator(np.random.PCG64(4))
+    V = 5003                                                             # not a multiple of the workgroup width
+    rows = g.standard_normal((8, V)).astype(np.float32)
+    rows[0, [17, 4000, 4999]] = 9.0                                      # equal maxima: the first wins
+    rows[1, 0] = np.nan                                                  # a NaN at index 0 is never replaced
+    rows[2, [5, 1024, 3000]] = np.nan; rows[2, 2048] = 50.0              # NaNs elsewhere are never chosen
+    rows[3, :] = -np.inf                                                 # nothing is greater than the first element
+    rows[4, :] = np.nan
+    rows[5, 1023] = 7.0; rows[5, 1024] = 7.0                             # a tie across two threads' strides
+    rows[6, V - 1] = 99.0                                                # the last element
+    rows[7, 0] = 99.0
+    picks = np.empty(8, dtype=np.uint32)
+    ctx.check(ctx.L.pyre_argmax_rows(ctx.h, rows.ctypes.data_as(lib.C.c_void_p), 8, V, picks.ctypes.data_as(lib.C.c_void_p)), "argmax_rows")
+    with np.errstate(invalid="ignore"):
+        assert picks.tolist() == [host(r) for r in rows] == [17, 0, 2048, 0, 0, 1023, V - 1, 0]
+
+
 def test_ngram_drafted_generation_equals_plain_greedy(ctx):
     # spec::generate with the prompt-lookup drafter (src/spec.rs:207): whatever the drafts, the stream is plain greedy's
     c = small_cfg()
