@@ -222,7 +222,7 @@ def bench_decode(args):
         ctx.free(p)
     log("model resident (re-laid-out) in %.1f s; weight bytes per token %.1f MB" % (time.perf_counter() - t0, model.weight_bytes_per_token / 1e6))
     n_ctx = args.ctx
-    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8 + args.host_steps + 1)
+    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8 + args.host_steps + 1 + args.spec_loop_tokens + 16)
     g = np.random.Generator(np.random.PCG64(args.seed + 1))
     prompt = g.integers(0, cfg.vocab, n_ctx, dtype=np.uint32)
     t0 = time.perf_counter()
@@ -268,6 +268,29 @@ def bench_decode(args):
         win_ms = (time.perf_counter() - t0) * 1e3 / args.spec_windows
         spec = {"window_tokens": 5, "ms_per_window": round(win_ms, 3), "tok_s_if_all_drafts_accepted": round(5e3 / win_ms, 1), "tok_s_if_none_accepted": round(1e3 / win_ms, 1),
                 "note": "host-facing verify window incl. 5 x %d logits device->host and the host argmax; %d windows" % (cfg.vocab, args.spec_windows)}
+    # the variant end to end through the library's own loop (spec::generate's greedy rounds, picks formed on the device):
+    # fixed 4-token drafts that are the plain greedy run's own tokens (every draft accepted), then wrong ones (every
+    # window rolled back to one token); both from the same snapshot, both must reproduce the plain stream
+    spec_loop = None
+    if args.spec_loop_tokens > 0:
+        n_sl = args.spec_loop_tokens
+        snap = st.snapshot()
+        plain = model.decode_greedy_dev(st, nxt, n_sl)                  # tokens that follow nxt
+        stream = np.concatenate([[nxt], plain]).astype(np.uint32)       # what generate emits when its first pick is nxt
+        fl = np.zeros(cfg.vocab, dtype=np.float32); fl[nxt] = 1.0
+        res = {}
+        for name, ds in (("all_accepted", stream), ("none_accepted", (stream + 1) % cfg.vocab)):
+            st.restore(snap)
+            dsp = np.concatenate([ds, np.zeros(16, np.uint32)]).astype(np.uint32)
+            ctx.sync(); t0 = time.perf_counter()
+            out_t, rounds = model.generate_greedy(st, fl, n_sl + 1, n_draft=4, draft_stream=dsp)
+            ctx.sync(); dt = time.perf_counter() - t0
+            if not np.array_equal(out_t, stream):
+                raise SystemExit("drafted generation diverged from plain greedy decoding")
+            res[name] = {"tok_s": round(n_sl / dt, 1), "rounds": rounds}
+        st.restore(snap)
+        spec_loop = {"tokens": n_sl, "drafts_per_round": 4, **res,
+                     "note": "pyre_generate_greedy with a fixed draft stream from the same snapshot; output checked against the plain greedy stream"}
     # the reference's own loop shape (Model::forward -> Vec<f32> logits -> sampler::argmax on the host): every step
     # carries 151936 logits over PCIe and a host argmax; reported beside `value`, never as it
     host_loop = None
@@ -320,6 +343,8 @@ def bench_decode(args):
         out["spec_verify"] = spec
     if host_loop:
         out["host_loop"] = host_loop
+    if spec_loop:
+        out["spec_loop"] = spec_loop
     if not args.no_cpu:
         del model, st
         out["cpu_baseline"] = cpu_baseline_decode(cfg, args.seed)
@@ -338,6 +363,7 @@ def main():
     ap.add_argument("--indexer", type=int, default=0, metavar="HEADS", help="decode workload variant: attention layers with a QSA sparse indexer of this many heads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
+    ap.add_argument("--spec-loop-tokens", type=int, default=64, help="decode workload: tokens to generate through the drafted loop (4 fixed drafts per round, all accepted / none accepted; 0 = skip)")
     ap.add_argument("--host-steps", type=int, default=32, help="decode workload: steps of the host-facing loop (pyre_forward + host argmax) to time beside the device loop (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
     ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs, q3_k, q5_k, q2_0)")
