@@ -51,6 +51,7 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
   __shared__ float P[C][C + 1];      // e^{L_i-L_j} q_i.k_j, j <= i
   __shared__ float D[C][33];         // B, then Delta
   __shared__ float L[C], Bt[C];
+  __shared__ __align__(16) float Qs[C][DK + 4], Ks[C][DK + 4];      // the chunk's q and k rows, staged once (rows padded against bank conflicts)
   const int h = blockIdx.x, cb = blockIdx.y, kh = h % p.nk, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ch = 2 * p.nk * DK + p.nv * p.dv, w = p.nv * p.dv, r = lane & 31, kk = lane >> 5;
   const float* sin_ = ssm_in + (size_t)h * DK * p.dv + cb * 32; float* sout = ssm_out + (size_t)h * DK * p.dv + cb * 32;
@@ -60,14 +61,21 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
     const float* qc = co + (size_t)t0 * ch + (size_t)kh * DK;                 // q_i at qc + i*ch
     const float* kc = qc + (size_t)p.nk * DK;
     const float* vc = co + (size_t)t0 * ch + 2 * (size_t)p.nk * DK + (size_t)h * p.dv + cb * 32;
-    __syncthreads();                                                           // previous chunk done with L, A, P, D; S final
-    if (tid < C) Bt[tid] = beta[(size_t)(t0 + tid) * p.nv + h];
-    if (tid == 0) { float acc = 0.0f; for (int i = 0; i < C; ++i) { acc += logg[(size_t)(t0 + i) * p.nv + h]; L[i] = acc; } }
+    __syncthreads();                                                           // previous chunk done with L, A, P, D, Qs, Ks; S final
+    for (int i = tid; i < C * (DK / 4); i += 256) {                            // coalesced: a row is 512 contiguous bytes
+      const int row = i / (DK / 4), c4 = i % (DK / 4);
+      *(float4*)&Qs[row][4 * c4] = *(const float4*)(qc + (size_t)row * ch + 4 * c4); *(float4*)&Ks[row][4 * c4] = *(const float4*)(kc + (size_t)row * ch + 4 * c4);
+    }
+    // the chunk's log-decays are fetched by 64 threads at once (one thread walking them would pay a memory round trip per
+    // token), then summed in token order by one
+    if (tid < C) { Bt[tid] = beta[(size_t)(t0 + tid) * p.nv + h]; L[tid] = logg[(size_t)(t0 + tid) * p.nv + h]; }
+    __syncthreads();
+    if (tid == 0) { float acc = 0.0f; for (int i = 0; i < C; ++i) { acc += L[i]; L[i] = acc; } }
     __syncthreads();
     // ---- A and P: 64x64x128 each, tile (ti, tj) with tj <= ti; waves 0..2 take A tiles (0,0),(1,0),(1,1), then P likewise
     for (int job = wave; job < 6; job += 4) {
       const int which = job / 3, tsel = job % 3, ti = tsel == 0 ? 0 : 1, tj = tsel == 2 ? 1 : 0;
-      const float* arow = (which == 0 ? kc : qc) + (size_t)(32 * ti + r) * ch; const float* brow = kc + (size_t)(32 * tj + r) * ch;
+      const float* arow = which == 0 ? Ks[32 * ti + r] : Qs[32 * ti + r]; const float* brow = Ks[32 * tj + r];
       floatx16 acc = {0};
       for (int k0 = 0; k0 < DK; k0 += 8) {
         float4 a4 = *(const float4*)(arow + k0 + 4 * kk), b4 = *(const float4*)(brow + k0 + 4 * kk);
@@ -85,7 +93,7 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
     // ---- K S_0 (waves 0,1) and Q S_0 (waves 2,3): 64x32x128, row tile = wave & 1
     floatx16 acc1 = {0};
     {
-      const int ti = wave & 1; const float* arow = (wave < 2 ? kc : qc) + (size_t)(32 * ti + r) * ch;
+      const int ti = wave & 1; const float* arow = wave < 2 ? Ks[32 * ti + r] : Qs[32 * ti + r];
       for (int k0 = 0; k0 < DK; k0 += 8) {
         float4 a4 = *(const float4*)(arow + k0 + 4 * kk); const int kb = k0 + 4 * kk;
         acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, S[kb][r], acc1, 0, 0, 0); acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, S[kb + 1][r], acc1, 0, 0, 0);
@@ -99,11 +107,12 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
       }
     }
     __syncthreads();
-    // ---- forward substitution (I + A) Delta = B, one thread per column
-    if (tid < 32) {
-      for (int i = 1; i < C; ++i) { float s = D[i][tid]; for (int j = 0; j < i; ++j) s -= A[i][j] * D[j][tid]; D[i][tid] = s; }
+    // ---- forward substitution (I + A) Delta = B, column by column of A: once Delta_j is final every later row takes its
+    // term, all 256 threads at work; an element still receives its terms in ascending j, as a row-by-row solve would give it
+    for (int j = 0; j < C - 1; ++j) {
+      for (int idx = tid; idx < (C - 1 - j) * 32; idx += 256) { const int i = j + 1 + (idx >> 5), c = idx & 31; D[i][c] -= A[i][j] * D[j][c]; }
+      __syncthreads();
     }
-    __syncthreads();
     // ---- O = O1 + P Delta (waves 2,3): 64x32x64
     if (wave >= 2) {
       const int ti = wave & 1;
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
       floatx16 acc2; const float eLC = expf(L[C - 1]);
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc2[e] = eLC * S[32 * wave + 8 * (e >> 2) + 4 * kk + (e & 3)][r];
-      for (int k0 = 0; k0 < C; k0 += 2) { int j = k0 + kk; float a = kc[(size_t)j * ch + 32 * wave + r] * expf(L[C - 1] - L[j]); acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, D[j][r], acc2, 0, 0, 0); }
+      for (int k0 = 0; k0 < C; k0 += 2) { int j = k0 + kk; float a = Ks[j][32 * wave + r] * expf(L[C - 1] - L[j]); acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, D[j][r], acc2, 0, 0, 0); }
       __syncthreads();                                                        // every wave has read the old S
 #pragma unroll
       for (int e = 0; e < 16; ++e) S[32 * wave + 8 * (e >> 2) + 4 * kk + (e & 3)][r] = acc2[e];
