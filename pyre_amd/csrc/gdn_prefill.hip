@@ -109,10 +109,18 @@ __global__ __launch_bounds__(256) void k_gdnp_chunk(GdnDev p, const float* __res
     __syncthreads();
     // ---- forward substitution (I + A) Delta = B, column by column of A: once Delta_j is final every later row takes its
     // term, all 256 threads at work; an element still receives its terms in ascending j, as a row-by-row solve would give it
-    for (int j = 0; j < C - 1; ++j) {
-      for (int idx = tid; idx < (C - 1 - j) * 32; idx += 256) { const int i = j + 1 + (idx >> 5), c = idx & 31; D[i][c] -= A[i][j] * D[j][c]; }
-      __syncthreads();
+    // The 32 columns of Delta are independent: wave w solves columns 8w .. 8w+7 with eight lanes per column (lane t of a column
+    // takes the rows j+1+t, j+1+t+8, ..), and a wave's shared-memory operations execute in order, so the 63 steps need no
+    // workgroup barrier.
+    {
+      const int c = 8 * wave + (lane & 7), tr = lane >> 3;
+      for (int j = 0; j < C - 1; ++j) {
+        const float dj = D[j][c];
+        for (int i = j + 1 + tr; i < C; i += 8) D[i][c] -= A[i][j] * dj;
+        __builtin_amdgcn_wave_barrier();
+      }
     }
+    __syncthreads();
     // ---- O = O1 + P Delta (waves 2,3): 64x32x64
     if (wave >= 2) {
       const int ti = wave & 1;
