@@ -23,8 +23,18 @@
  *                          (numpy sort) on distinct scores; hand-built keys that force a known block set;
  *                          block pooling closed form (identical keys -> pooled key = rope(rms(key)))
  *   orc_rope_inv_yarn      the reference's asserted properties (qn_ctx.rs:406-419) + float64 closed form
- *   orc_moe_ffn            numpy statement built from orc_dequant'd dense weights
- *   orc_forward            numpy statement of the whole token step on a tiny model
+ *   orc_hc_mix             closed forms: zero up (or zero down) -> half the mean of the normalised streams;
+ *                          one-hot down / inject / up rows -> silu(x_j / hc), x_m / hc and the stream-major gate
+ *                          layout as explicit numbers; windows == single tokens
+ *   orc_hc_combine         inject 0 -> x + out exactly; -inf -> unchanged; +inf -> x + 2 out; ln 3 -> x + 1.5 out
+ *   orc_moe_ffn            closed forms: shared expert alone with a zero gate vector -> halved SwiGLU of picked
+ *                          inputs; two chosen experts, one with a zero down matrix -> w1 * down_1 (silu(g) * u) with
+ *                          w1 the two-way softmax; all-ones Q8_0 matrices -> sf silu(S) S sigmoid(x_0) + ff silu(S) S;
+ *                          + a numpy statement built from orc_dequant'd dense weights
+ *   orc_forward            all block outputs zeroed -> head(hc_mix(tiled embedding of the last token)) bit for bit;
+ *                          one live FFN / one live DeltaNet layer -> the composition of the pinned block entry
+ *                          points bit for bit (and not with the other mixer's inject factors); + a numpy statement
+ *                          of the whole token step on a tiny model
  * Parity unpinned (only running the reference could pin): the last-ulp behaviour of
  * expf/log1pf/powf/sincosf on the reference's own target libm.
  */
