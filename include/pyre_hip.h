@@ -85,6 +85,16 @@ int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, i
  * the two are the same code. */
 int    pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
+/* pyre_qmatmul_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  IQ3_S matrices only -- the one type whose GEMV
+ * needs a scratch buffer (the activations' fixed-point digits); every other type's pyre_qmatmul_dev allocates nothing
+ * already.  The digits go to a fixed device array inside the library (PYRE_QMATMUL_STATIC_MAX_TU * 256 bytes per GPU,
+ * held until the process ends) instead of the context's grow-only buffer, and the call makes no allocation, no event
+ * and no copy: two kernel launches on the context's stream.  Same kernels and launch shapes as pyre_qmatmul_dev, so
+ * the result is bit-identical to it.  t * cols / 64 above PYRE_QMATMUL_STATIC_MAX_TU is rejected with PYRE_E_SHAPE.
+ * All contexts on one GPU share that GPU's array: calls that overlap in time on one GPU (two contexts' streams) race. */
+#define PYRE_QMATMUL_STATIC_MAX_TU 4096      /* token-units: t = 8 up to 32768 columns, t = 1 up to 262144 */
+int    pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
 /* The batch 2..8 speculative-verify GEMM on the matrix cores (the reference's verify kernels, src/model/qn_cube.rs:17,6454,
  * and lcm_dense, qwen4exp_gguf.rs:2641-2737): IQ3_S matrices, t in 2..8.  Same contract as pyre_qmatmul; the result
  * agrees with it to about 1e-7 of max|y| but not bit for bit (f16 two-term split of the activations, f32 accumulation). */

@@ -29,6 +29,7 @@ struct pyre_ctx {
   unsigned* fuse_ctl = nullptr;                        // control words of in-launch barriers (zeroed once): [0] generation, [16] abort, [32] count
   void* mfma_buf = nullptr; size_t mfma_bytes = 0;     // split activations of the matrix-core verify GEMM (grow-only)
   void* i8_buf = nullptr; size_t i8_bytes = 0;         // fixed-point activation digits of the integer-dot GEMV (grow-only)
+  uint32_t* i8_static = nullptr;                       // device address of this GPU's copy of the file-scope digit array (gemv_i8.hip), resolved at creation
 };
 
 // Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
@@ -113,6 +114,10 @@ int pyre_gemm_mfma_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, i
 // best (t = 1, optional): per-tile maxima as pyre_gemv_argmax_launch.
 bool pyre_gemv_i8_ok(const QMatDev& m, int t);
 int pyre_gemv_i8_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, uint32_t* best_dev);
+// The same launches with the digits in a file-scope device array (at most PYRE_QMATMUL_STATIC_MAX_TU token-units): no
+// allocation of any kind.  pyre_i8_static_init resolves the array's address on the context's device (context creation).
+int pyre_i8_static_init(pyre_ctx* ctx);
+int pyre_gemv_i8_static_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {

@@ -74,6 +74,7 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
       (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->fuse_ctl, 1024)) != hipSuccess || (e = hipMemset(ctx->fuse_ctl, 0, 1024)) != hipSuccess) {
     int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: codebook upload: %s", hipGetErrorString(e)); pyre_ctx_destroy(ctx); return rc; }
+  if (pyre_i8_static_init(ctx) != PYRE_OK) { int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: %s", ctx->err.c_str()); pyre_ctx_destroy(ctx); return rc; }
   *out = ctx; return PYRE_OK;
 }
 

@@ -176,6 +176,42 @@ template <int T> void launch_t(pyre_ctx* ctx, const QMatDev& m, const uint32_t* 
 
 bool pyre_gemv_i8_ok(const QMatDev& m, int t) { return m.fmt == FMT_IQ3_S && t >= 1 && t <= 8; }
 
+// ---- the variant that allocates nothing -----------------------------------------------------------------------------
+// The activation digits of pyre_qmatmul_static_dev live in this file-scope array instead of the context's grow-only
+// buffer.  Every GPU the library runs on holds its own copy, at its own address, until the process ends; the name below
+// is only the host-side handle of the symbol, the device address comes from hipGetSymbolAddress (once per device, at
+// context creation) and is what the kernels and every other host-side use get.
+#define I8_STATIC_WORDS ((size_t)PYRE_QMATMUL_STATIC_MAX_TU * I8_STRIDE)
+static __device__ __align__(256) uint32_t scratch[I8_STATIC_WORDS];
+#define I8_MAX_DEVICES 64
+static uint32_t* g_static_ptr[I8_MAX_DEVICES];
+
+int pyre_i8_static_init(pyre_ctx* ctx) {      // called by pyre_ctx_create with the context's device current
+  if (ctx->device < 0 || ctx->device >= I8_MAX_DEVICES) return pyre_fail(ctx, PYRE_E_ARG, "device %d outside the static scratch table (%d devices)", ctx->device, I8_MAX_DEVICES);
+  if (!g_static_ptr[ctx->device]) {
+    void* p = nullptr;
+    PYRE_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return pyre_fail(ctx, PYRE_E_HIP, "hipGetSymbolAddress returned a null address for the static scratch");
+    g_static_ptr[ctx->device] = (uint32_t*)p;
+  }
+  ctx->i8_static = g_static_ptr[ctx->device];
+  return PYRE_OK;
+}
+
+// Same kernels, same launch shapes and therefore the same bits as pyre_gemv_i8_launch; no allocation, no event, no copy.
+int pyre_gemv_i8_static_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
+  if (!pyre_gemv_i8_ok(m, t)) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: IQ3_S and 1..8 tokens only");
+  if ((size_t)t * m.U > (size_t)PYRE_QMATMUL_STATIC_MAX_TU)
+    return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: t * cols / 64 = %zu exceeds the static scratch (at most %d: t = 8 up to %d columns)", (size_t)t * m.U, PYRE_QMATMUL_STATIC_MAX_TU, PYRE_QMATMUL_STATIC_MAX_TU / 8 * 64);
+  uint32_t* dg = ctx->i8_static;
+  if (!dg) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the static scratch of device %d was not resolved at context creation", ctx->device);
+  hipLaunchKernelGGL(k_act_digits, dim3(m.U, t), dim3(64), 0, ctx->stream, x, m.cols, dg); PYRE_CHECK_LAUNCH(ctx);
+  switch (t) { case 1: launch_t<1>(ctx, m, dg, y, nullptr); break; case 2: launch_t<2>(ctx, m, dg, y, nullptr); break; case 3: launch_t<3>(ctx, m, dg, y, nullptr); break; case 4: launch_t<4>(ctx, m, dg, y, nullptr); break;
+    case 5: launch_t<5>(ctx, m, dg, y, nullptr); break; case 6: launch_t<6>(ctx, m, dg, y, nullptr); break; case 7: launch_t<7>(ctx, m, dg, y, nullptr); break; default: launch_t<8>(ctx, m, dg, y, nullptr); break; }
+  PYRE_CHECK_LAUNCH(ctx);
+  return PYRE_OK;
+}
+
 int pyre_gemv_i8_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, uint32_t* best) {
   if (!pyre_gemv_i8_ok(m, t)) return pyre_fail(ctx, PYRE_E_ARG, "integer-dot GEMV: IQ3_S and 1..8 tokens only");
   void* buf = nullptr; int rc = i8_scratch(ctx, (size_t)t * m.U * I8_STRIDE * 4, &buf); if (rc) return rc;

@@ -485,6 +485,12 @@ static int qmatmul_host(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, 
 }
 int pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, false); }
 int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, false); }
+int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
+  if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: null argument");
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: t = %d outside 1..8", t);
+  if (m->dv.fmt != FMT_IQ3_S) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  return pyre_gemv_i8_static_launch(ctx, m->dv, x_dev, t, y_dev);
+}
 int pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, true); }
 int pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, true); }
 

@@ -47,6 +47,7 @@ def _declare(L):
         "pyre_qmatmul_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_f32": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_f32_dev": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmatmul_static_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
         "pyre_gguf_open": (i32, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
         "pyre_gguf_close": (None, [vp]),
@@ -285,6 +286,10 @@ class QMat:
 
     def matmul_mfma_dev(self, x_dev, t, y_dev):
         self.ctx.check(self.ctx.L.pyre_qmatmul_mfma_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_mfma_dev")
+
+    def matmul_static_dev(self, x_dev, t, y_dev):
+        """pyre_qmatmul_static_dev: device pointers in and out, nothing allocated by the call."""
+        self.ctx.check(self.ctx.L.pyre_qmatmul_static_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_static_dev")
 
     def matmul_dev(self, x_dev, t, y_dev):
         self.ctx.check(self.ctx.L.pyre_qmatmul_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_dev")
