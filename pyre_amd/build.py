@@ -11,28 +11,33 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-def _compile(src):
-    obj = src[:-4] + ".o"
-    cmd = ["hipcc", *FLAGS, "-c", src, "-o", obj]
+def _compile(job):
+    src, obj, extra = job
+    cmd = ["hipcc", *FLAGS, *extra, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, r.returncode, (r.stdout + r.stderr)
 
 
-def build(verbose=True, jobs=8):
+def build(verbose=True, jobs=8, extra_flags=(), out_dir=None):
+    """out_dir (with extra_flags): a diagnostics variant of the library beside the product build, e.g. -DPYRE_PHASE_TS."""
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
     objs = []
+    lib = LIB if out_dir is None else os.path.join(out_dir, "libpyre_hip.so")
+    if out_dir is not None:
+        os.makedirs(out_dir, exist_ok=True)
+    todo = [(s, (s[:-4] + ".o") if out_dir is None else os.path.join(out_dir, os.path.basename(s)[:-4] + ".o"), tuple(extra_flags)) for s in srcs]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        for src, obj, rc, out in ex.map(_compile, srcs):
+        for src, obj, rc, out in ex.map(_compile, todo):
             msg = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l and l.strip())
             if verbose and msg:
                 print(msg)
             if rc != 0:
                 raise RuntimeError("hipcc failed on %s\n%s" % (src, out))
             objs.append(obj)
-    r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], capture_output=True, text=True)
+    r = subprocess.run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed\n" + r.stdout + r.stderr)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

@@ -10,6 +10,21 @@
 #include <vector>
 #include "../../include/pyre_hip.h"
 
+// Diagnostics build (-DPYRE_PHASE_TS): workgroup 0's first thread keeps 100 MHz timestamps of a kernel's phases in
+// registers and leaves them in a per-file device array at the kernel's end (read back by pyre_debug_ts_*).
+#ifdef PYRE_PHASE_TS
+#define PYRE_TS_DECL(name) static __device__ unsigned long long name[128];
+#define PYRE_TS_VARS unsigned long long ts_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define PYRE_TS(k) ts_[k] = wall_clock64()
+#define PYRE_TS_FLUSH(name, base) do { if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) { for (int q_ = 0; q_ < 8; ++q_) name[(base) + q_] = ts_[q_]; } } while (0)
+#define PYRE_TS_EXPORT(name, fn) extern "C" int fn(unsigned long long* out) { return hipMemcpyFromSymbol(out, HIP_SYMBOL(name), sizeof(unsigned long long) * 128) == hipSuccess ? 0 : -1; }
+#else
+#define PYRE_TS_DECL(name)
+#define PYRE_TS_VARS
+#define PYRE_TS(k)
+#define PYRE_TS_FLUSH(name, base)
+#define PYRE_TS_EXPORT(name, fn)
+#endif
 #define PYRE_WAVE 64
 #define PYRE_UNIT 64            // weights per decode unit (one lane decodes one unit at a time)
 
@@ -42,6 +57,14 @@ struct ProfScope {
   }
   ~ProfScope() { if (!a) return; (void)hipEventRecord(b, ctx->stream); ctx->prof_pending.push_back({name, bytes, a, b}); }
 };
+
+#ifdef __HIPCC__
+// Workgroup barrier for exchanges that go through shared memory only: waits for the wave's own shared-memory (and
+// scalar) operations, not for its outstanding global loads, so weights requested ahead of it stay in flight across it.
+// (__syncthreads() carries a workgroup-scope fence, which on this part drains every outstanding vector memory
+// operation first: a prefetch issued before it costs its whole latency at the barrier.)
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+#endif
 
 extern thread_local std::string g_pyre_create_err;
 

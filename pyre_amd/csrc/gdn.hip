@@ -1,6 +1,7 @@
 // Gated DeltaNet recurrent step: causal depthwise conv1d + SiLU, L2-normalised q/k, gated delta rule on the fp32
 // state kept resident in HBM, gated RMSNorm.  Follows linear_core, src/model/qwen4exp_gguf.rs:1624-1673.
 #include "formats.h"
+PYRE_TS_DECL(gdn_ts) PYRE_TS_EXPORT(gdn_ts, pyre_debug_ts_gdn)
 
 __device__ __forceinline__ float g_sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float g_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
@@ -31,6 +32,7 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
                                                    const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int G = 4, R = DK / G;
+  PYRE_TS_VARS PYRE_TS(0);
   __shared__ float qs[DK], ks[DK], pm[G][DV], po[G][DV], red[8];
   const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7;
   const int ch = 2 * p.nk * DK + p.nv * DV, w = p.nv * DV;
@@ -52,24 +54,25 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
     if ((tid & 63) == 0) red[tid >> 6] = sq;
-    __syncthreads();
+    __syncthreads(); PYRE_TS(1);
     if (tid < DK) qs[tid] = v * ((1.0f / sqrtf(red[0] + red[1] + 1e-6f)) * (1.0f / sqrtf((float)DK)));
     else if (tid < 2 * DK) ks[tid - DK] = v * ((1.0f / sqrtf(red[2] + red[3] + 1e-6f)) * 1.0f);
     const float g = expf(g_softplus(alpha_raw + dtb) * a);      // alpha at [ch + nv*dv + nv + h]
     const float b = g_sigm(beta_raw);                                 // beta  at [ch + nv*dv + h]
-    __syncthreads();
+    __syncthreads(); PYRE_TS(2);
     float pmv = 0.0f;
 #pragma unroll
     for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[grp * R + r]; }
     pm[grp][j] = pmv;
-    __syncthreads();
+    PYRE_TS(3);
+    __syncthreads(); PYRE_TS(4);
     const float mem = ((pm[0][j] + pm[1][j]) + pm[2][j]) + pm[3][j];
     const float delta = (v_j - mem) * b;
     float pov = 0.0f;
 #pragma unroll
     for (int r = 0; r < R; ++r) { S[r] += ks[grp * R + r] * delta; pov += S[r] * qs[grp * R + r]; }
     po[grp][j] = pov;
-    __syncthreads();
+    __syncthreads(); PYRE_TS(5);
     if (tid < DV) {
       float o = ((po[0][j] + po[1][j]) + po[2][j]) + po[3][j];
       float ss = o * o;
@@ -84,10 +87,11 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
       float o = pm[0][j] * (sc * nw_j);                              // rms_inplace: x *= s * w  (:210)
       out[(size_t)ti * w + h * DV + j] = o * g_sigm(z_j);   // z at [ch + h*dv + j]
     }
-    __syncthreads();
+    __syncthreads(); PYRE_TS(6);
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) sout[(size_t)(grp * R + r) * DV + j] = S[r];
+  PYRE_TS(7); PYRE_TS_FLUSH(gdn_ts, 0);
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,

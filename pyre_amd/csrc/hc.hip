@@ -10,6 +10,7 @@
 #include <stdlib.h>
 #include <algorithm>
 
+PYRE_TS_DECL(hc_ts) PYRE_TS_EXPORT(hc_ts, pyre_debug_ts_hc)
 __device__ __forceinline__ float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // Stream element i of token ti with the pending residual update applied: x + out * w  (:1384-1387), w = 2*sigm(inj).
@@ -69,6 +70,7 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
     const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq,
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
+  PYRE_TS_VARS PYRE_TS(0);
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, nw = nthr >> 6, tid = threadIdx.x, L = nw * upw * 64;
   float* xs = sm;                         // [T][L]
@@ -77,11 +79,28 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
   const int tile = blockIdx.x, ks = blockIdx.y;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int c0 = ks * L, s = c0 / d, i0 = c0 - s * d;
-  UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);     // in flight across the barrier
+  // Loads return in the order they were issued: the streams (and the pending update's terms) first, since the copy into
+  // shared memory waits for them, then the first unit's weights, which stay in flight across the barrier.
   float w[T], ss[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) { w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f; ss[t] = 0.0f; }
-  for (int j = tid; j < L; j += nthr) {
+  float v0[T]; float nv0 = 0.0f;
+  if (tid < L) {
+    nv0 = norm[(size_t)s * d + i0 + tid];
+#pragma unroll
+    for (int t = 0; t < T; ++t) v0[t] = hc_x_new<T, NP>(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid);
+  }
+  UnitRaw<FMT> raw = unit_load<FMT>(m, tile, ks * nw * upw + wave * upw, lane);
+  if (tid < L) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const float v = v0[t];
+      ss[t] += v * v;
+      xs[(size_t)t * L + tid] = v * nv0;
+      if (tile == 0) x_out[((size_t)t * hc + s) * d + i0 + tid] = v;
+    }
+  }
+  for (int j = tid + nthr; j < L; j += nthr) {
     const float nv = norm[(size_t)s * d + i0 + j];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
@@ -97,7 +116,7 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
     for (int o = 32; o > 0; o >>= 1) ss[t] += __shfl_xor(ss[t], o);
     if (lane == 0) wsum[wave * T + t] = ss[t];
   }
-  __syncthreads();
+  lds_barrier(); PYRE_TS(1);
   if (tile == 0 && tid < T) { float tot = wsum[tid]; for (int q = 1; q < nw; ++q) tot += wsum[q * T + tid]; ssq[ks * T + tid] = tot; }
   float acc[T];
 #pragma unroll
@@ -105,13 +124,15 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
   for (int u = 0; u < upw; ++u) { int lu = wave * upw + u; if (u > 0) raw = unit_load<FMT>(m, tile, ks * nw * upw + lu, lane); unit_fma<FMT, T>(m, raw, ks * nw * upw + lu, lds2, lane, xs + lu * 64, L, acc); }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[((size_t)wave * T + t) * 64 + lane] = acc[t];
-  __syncthreads();
+  PYRE_TS(2);
+  lds_barrier(); PYRE_TS(3);
   const size_t r64 = (size_t)m.tiles * 64;
   for (int i = tid; i < T * 64; i += nthr) {
     int t = i >> 6, l = i & 63; float a = red[(size_t)t * 64 + l];
     for (int q = 1; q < nw; ++q) a += red[((size_t)q * T + t) * 64 + l];
     part[((size_t)ks * T + t) * r64 + (size_t)tile * 64 + l] = a;
   }
+  PYRE_TS(4); PYRE_TS_FLUSH(hc_ts, NP > 1 ? 0 : 8);
 }
 
 // grid (d / 64), hc*U waves (U = lr / 64 units of the up matrix).  Prologue: the streams' RMS scales from the slice
@@ -128,42 +149,48 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
     QMatDev router, float* __restrict__ rpart) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
+  PYRE_TS_VARS PYRE_TS(0);
   extern __shared__ __align__(16) float sm[];
-  const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc;
+  const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc, nw = nthr >> 6;
   float* lo = sm;                         // [T][lr]
   float* red = sm + (size_t)T * lr;       // [nw][T][64]
-  float* sls = red + (size_t)(nthr >> 6) * T * 64;   // [T][32]: the RMS scale of the stream each slice belongs to
+  float* sls = red + (size_t)nw * T * 64;   // [T][32]: the RMS scale of the stream each slice belongs to
+  float* term = sls + (size_t)T * 32;     // [T*hc][64]: the streams' gated, normalized values before they are added
   const int n_o = lr + hc;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave / U, ku = wave - s * U;
-  UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);        // in flight across the prologue
-  float xpre[8], npre[8];         // the epilogue's stream values and norm weights of this thread's first output, fetched now
+  // Loads return in the order they were issued, so they are issued in the order they are needed: the slice sums of
+  // squares and of [down ; inject] first (the prologue waits for nothing else), then the up weights, the epilogue's
+  // operands and the router tile, all of which stay in flight across the barriers below (which exchange through shared
+  // memory only).
+  float ssv[32];
 #pragma unroll
-  for (int q = 0; q < 8; ++q) { xpre[q] = 0.0f; npre[q] = 0.0f; }
-  if (wave < T) {                  // wave t holds token t's 64 outputs
-#pragma unroll
-    for (int q = 0; q < 8; ++q) if (q < hc) { xpre[q] = (xnew + ((size_t)wave * hc + q) * d + blockIdx.x * 64)[lane]; npre[q] = (norm + (size_t)q * d + blockIdx.x * 64)[lane]; }
-  }
-  // the slices of this thread's first output row are fetched before the barrier the scales need
+  for (int k = 0; k < 32; ++k) ssv[k] = 0.0f;
+  const int stt = tid / hc, sq = tid - stt * hc;
+  if (tid < T * hc) hc_load_run(ssv, ssq + (size_t)(sq * kps) * T + stt, kps, T);          // all of the stream's slices before the first add: one round trip
   float pv[32]; int idx = tid; int t = idx / n_o, i = idx - t * n_o;
   bool have = idx < T * n_o;
   hc_load_slices<T>(pv, part, have && (i < lr || has_inject), ksplit, t, r64, i);
+  UnitRaw<FMT> raw = unit_load<FMT>(up, s * (d >> 6) + blockIdx.x, ku, lane);
+  // the epilogue's stream value and norm weight of this wave's first (token, stream) item
+  float xpre = 0.0f, npre = 0.0f;
+  if (wave < T * hc) { const int t0 = wave / hc, q0 = wave - t0 * hc; xpre = (xnew + ((size_t)t0 * hc + q0) * d + blockIdx.x * 64)[lane]; npre = (norm + (size_t)q0 * d + blockIdx.x * 64)[lane]; }
+  UnitRaw<RFX> rraw;
+  constexpr bool R_EARLY = RFX != FMT_F32;      // an f32 tile is 64 registers: fetched once the up GEMV has freed them
+  if (ROUTE && R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
   if (tid < T * hc) {
-    const int tt = tid / hc, q = tid - tt * hc;
-    float sv[32];                 // all of the stream's slices before the first add: one round trip
-    hc_load_run(sv, ssq + (size_t)(q * kps) * T + tt, kps, T);
-    float tot = sv[0];
+    float tot = ssv[0];
 #pragma unroll
-    for (int k = 1; k < 32; ++k) if (k < kps) tot += sv[k];
+    for (int k = 1; k < 32; ++k) if (k < kps) tot += ssv[k];
     const float sc = 1.0f / sqrtf(tot / (float)d + eps);
-    for (int k = 0; k < kps; ++k) sls[tt * 32 + q * kps + k] = sc;
+    for (int k = 0; k < kps; ++k) sls[stt * 32 + sq * kps + k] = sc;
   }
-  __syncthreads();
+  lds_barrier(); PYRE_TS(1);
   while (have) {
     float o = 0.0f;                 // slices in order, each times its stream's scale
     if (i < lr || has_inject) {
 #pragma unroll
-      for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) { const float term = pv[ks] * sls[t * 32 + ks]; o = ks == 0 ? term : o + term; }
+      for (int ks = 0; ks < 32; ++ks) if (ks < ksplit) { const float tm = pv[ks] * sls[t * 32 + ks]; o = ks == 0 ? tm : o + tm; }
     }
     const float v = o / (float)hc;
     if (i < lr) lo[t * lr + i] = v * sigm(v);
@@ -171,10 +198,7 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
     idx += nthr; have = idx < T * n_o;
     if (have) { t = idx / n_o; i = idx - t * n_o; hc_load_slices<T>(pv, part, i < lr || has_inject, ksplit, t, r64, i); }
   }
-  UnitRaw<RFX> rraw;              // fetched once the registers it needs are free (f32: 64 of them, after the up GEMV); in flight until the epilogue
-  constexpr bool R_EARLY = RFX != FMT_F32;
-  if (ROUTE && R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
-  __syncthreads();
+  lds_barrier(); PYRE_TS(2);
   float acc[T];
 #pragma unroll
   for (int t2 = 0; t2 < T; ++t2) acc[t2] = 0.0f;
@@ -182,24 +206,30 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
 #pragma unroll
   for (int t2 = 0; t2 < T; ++t2) red[((size_t)wave * T + t2) * 64 + lane] = acc[t2];
   if (ROUTE && !R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
-  __syncthreads();
+  PYRE_TS(3);
+  lds_barrier(); PYRE_TS(4);
+  // one wave per (token, stream): the gate logit is the sum of the stream's waves in unit order; xn * sigm(gate) -> term
+  for (int w = wave; w < T * hc; w += nw) {
+    const int t2 = w / hc, q = w - t2 * hc, col = blockIdx.x * 64 + lane;
+    float g = red[((size_t)(q * U) * T + t2) * 64 + lane];
+    for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t2) * 64 + lane];
+    const float xv = w == wave ? xpre : xnew[((size_t)t2 * hc + q) * d + col];
+    const float nv = w == wave ? npre : norm[(size_t)q * d + col];
+    term[(size_t)w * 64 + lane] = xv * sls[t2 * 32 + q * kps] * nv * sigm(g);            // rms, :209: (x * s) * w
+  }
+  lds_barrier();
   for (int i2 = tid; i2 < T * 64; i2 += nthr) {
-    int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
+    const int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) if (q < hc) {
-      float g = red[((size_t)(q * U) * T + t2) * 64 + l];
-      for (int k = 1; k < U; ++k) g += red[((size_t)(q * U + k) * T + t2) * 64 + l];
-      const float xv = i2 == tid ? xpre[q] : xnew[((size_t)t2 * hc + q) * d + col];
-      const float nv = i2 == tid ? npre[q] : norm[(size_t)q * d + col];
-      mx += xv * sls[t2 * 32 + q * kps] * nv * sigm(g);            // rms, :209: (x * s) * w
-    }
+    for (int q = 0; q < 8; ++q) if (q < hc) mx += term[(size_t)(t2 * hc + q) * 64 + l];          // streams ascending from zero (:1380)
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
     if (ROUTE) lo[t2 * 64 + l] = mv;          // lo is free after the barrier above
   }
+  PYRE_TS(5);
   if (ROUTE) {
-    __syncthreads();
-    const size_t rr64 = (size_t)router.tiles * 64; const int nw = nthr >> 6;
+    lds_barrier(); PYRE_TS(6);
+    const size_t rr64 = (size_t)router.tiles * 64;
     for (int tile = wave; tile < router.tiles; tile += nw) {
       if (tile != wave) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
 #pragma unroll 1
@@ -210,6 +240,7 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
       }
     }
   }
+  PYRE_TS(7); PYRE_TS_FLUSH(hc_ts, ROUTE ? 16 : 24);
 }
 
 __global__ void k_hc_combine(float* __restrict__ x, const float* __restrict__ out, const float* __restrict__ inj, int d, int hc) {
@@ -239,7 +270,7 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
-  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32);
+  const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32 + (size_t)T * h.hc * 64);
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));

@@ -3,64 +3,99 @@
 // Follows ffn / routed (f32 branch) of the reference, src/model/qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793,
 // and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
 #include "formats.h"
+PYRE_TS_DECL(moe_ts) PYRE_TS_EXPORT(moe_ts, pyre_debug_ts_moe)
 
 // ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id -----------------------------
 // Runs inside every gate/up workgroup of a routed entry (all of them need the expert id before they can touch a
 // weight, and a separate launch would cost more than redoing this small selection everywhere).
-// Two-level selection: wave w < ceil(n_exp/64) ranks its own 64 logits through lane broadcasts and keeps its best k as
-// candidates (an expert outside its wave's best k cannot be in the global best k); the candidates are then ranked
-// against each other from shared memory.  Leaves the chosen ids (ascending) in s_idx[0..k) and their logits in s_val[0..k).
-struct RouteLds { float c_val[16 * 32]; int c_idx[16 * 32]; float r_val[32]; int r_idx[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
+// Thread e sums logit e's K slices (in slice order) into shared memory; wave 0 then holds the logits R per lane and
+// takes the maximum k times: a lane keeps the best of its own live logits, the wave's best of those comes out of six
+// idempotent DPP steps (no shared memory, no barrier), its owner retires it and rescans.  Leaves the chosen ids
+// (ascending) in s_idx[0..k) and their logits in s_val[0..k).
+struct RouteLds { float lv[1024]; float r_val[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
+#ifdef PYRE_PHASE_TS
+#define ROUTE_TS_PARAM , unsigned long long* rts_
+#define ROUTE_TS_ARG , ts_
+#define ROUTE_TS(k) rts_[k] = wall_clock64()
+#else
+#define ROUTE_TS_PARAM
+#define ROUTE_TS_ARG
+#define ROUTE_TS(k)
+#endif
+// A logit becomes a 32-bit key whose unsigned order is the logits' order (0 = no candidate); the largest key of the wave
+// comes out of six DPP maximum steps, the lowest index that holds it out of six DPP minimum steps.
+__device__ __forceinline__ uint32_t route_key(float v) {
+  uint32_t u = __float_as_uint(v + 0.0f);          // -0 counts as +0, as in a float comparison
+  return u ^ ((u & 0x80000000u) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float route_key_value(uint32_t u) { return __uint_as_float(u ^ ((u & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)); }
+template <int CTRL> __device__ __forceinline__ uint32_t route_dpp(uint32_t m) {          // lanes without a source see their own value
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, 0xf, 0xf, false);
+}
+__device__ __forceinline__ uint32_t route_wave_max(uint32_t m) {          // both are idempotent, so the row broadcasts need no row masks
+  m = max(m, route_dpp<0x111>(m)); m = max(m, route_dpp<0x112>(m)); m = max(m, route_dpp<0x114>(m)); m = max(m, route_dpp<0x118>(m));      // row_shr 1, 2, 4, 8: lane 15 of a row holds the row's
+  m = max(m, route_dpp<0x142>(m)); m = max(m, route_dpp<0x143>(m));          // row_bcast 15, 31: lane 63 holds the wave's
+  return (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+}
+__device__ __forceinline__ uint32_t route_wave_min(uint32_t m) {
+  m = min(m, route_dpp<0x111>(m)); m = min(m, route_dpp<0x112>(m)); m = min(m, route_dpp<0x114>(m)); m = min(m, route_dpp<0x118>(m));
+  m = min(m, route_dpp<0x142>(m)); m = min(m, route_dpp<0x143>(m));
+  return (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+}
+template <int R> __device__ __forceinline__ void route_select(int n_exp, int k, RouteLds& L, int lane) {
+  // straight-line code (selects, no divergent branches: a branch costs more here than the few operations it would skip)
+  uint32_t key[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) { const int idx = r * 64 + lane; const uint32_t kk = route_key(L.lv[min(idx, 1023)]); key[r] = idx < n_exp ? kk : 0u; }
+  uint32_t sel_k = 0u, sel_i = 0u;
+  for (int round = 0; round < k; ++round) {
+    uint32_t m = key[0];
+#pragma unroll
+    for (int r = 1; r < R; ++r) m = max(m, key[r]);
+    const uint32_t wm = route_wave_max(m);
+    uint32_t mi = 0xFFFFFFFFu;
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) mi = key[r] == wm ? (uint32_t)(r * 64 + lane) : mi;          // the lane's lowest index holding the maximum
+    const uint32_t wi = route_wave_min(mi);
+    sel_k = lane == round ? wm : sel_k; sel_i = lane == round ? wi : sel_i;
+#pragma unroll
+    for (int r = 0; r < R; ++r) key[r] = (uint32_t)(r * 64 + lane) == wi ? 0u : key[r];          // its owner retires it
+  }
+  int pos = 0;
+  for (int j = 0; j < k; ++j) { const uint32_t oj = (uint32_t)__builtin_amdgcn_readlane((int)sel_i, j); pos += oj < sel_i ? 1 : 0; }
+  if (lane < k) { L.s_idx[pos] = (int)sel_i; L.s_val[pos] = route_key_value(sel_k); }
+}
 // The logits are given as nsl (<= 64) K-slice sums `sstride` floats apart, added in slice order (nsl == 1: the logits
 // themselves); all slices are fetched before the first add, in groups of eight behind launch-uniform branches.
-__device__ __forceinline__ void route_topk(const float* __restrict__ logits, int nsl, int sstride, int n_exp, int k, RouteLds& L) {
-  const int e = threadIdx.x, lane = e & 63, wave = e >> 6, nwa = (n_exp + 63) >> 6;
-  if (wave < nwa) {
-    float v = -INFINITY;
-    if (e < n_exp) {
-      float sv[64];
+__device__ __forceinline__ void route_topk(const float* __restrict__ logits, int nsl, int sstride, int n_exp, int k, RouteLds& L ROUTE_TS_PARAM) {
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  if (e < n_exp) {
+    float sv[64];
 #pragma unroll
-      for (int q = 0; q < 64; ++q) sv[q] = 0.0f;
+    for (int q = 0; q < 64; ++q) sv[q] = 0.0f;
 #pragma unroll
-      for (int g = 0; g < 8; ++g) if (g * 8 < nsl) {
+    for (int g = 0; g < 8; ++g) if (g * 8 < nsl) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) sv[g * 8 + q] = (logits + (size_t)min(g * 8 + q, nsl - 1) * sstride)[e];
-      }
-      v = sv[0];
-#pragma unroll
-      for (int q = 1; q < 64; ++q) if (q < nsl) v += sv[q];
-      if (isnan(v)) v = -INFINITY;      // nan_clean
+      for (int q = 0; q < 8; ++q) sv[g * 8 + q] = (logits + (size_t)min(g * 8 + q, nsl - 1) * sstride)[e];
     }
-    int lr = 0;
+    float v = sv[0];
 #pragma unroll
-    for (int j = 0; j < 64; ++j) { float u = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); lr += (u > v || (u == v && j < lane)) ? 1 : 0; }
-    if (lr < k) { L.c_val[wave * k + lr] = v; L.c_idx[wave * k + lr] = e; }
+    for (int q = 1; q < 64; ++q) if (q < nsl) v += sv[q];
+    if (isnan(v)) v = -INFINITY;      // nan_clean
+    L.lv[e] = v;
   }
-  __syncthreads();
-  // candidate c is ranked by SP threads, each against a slice of the candidates; the SP counts meet through shuffles
-  const int nc = nwa * k; int SP = 8; while (SP > 1 && nc * SP > (int)blockDim.x) SP >>= 1;
-  {
-    const int c = e / SP, part = e % SP, per = (nc + SP - 1) / SP; int rank = 0;
-    float cv = 0.0f; int ci = 0;
-    if (c < nc) {
-      cv = L.c_val[c]; ci = L.c_idx[c];
-      const int j1 = min(nc, (part + 1) * per);
-#pragma unroll 4
-      for (int j = part * per; j < j1; ++j) { float u = L.c_val[j]; int ui = L.c_idx[j]; rank += (u > cv || (u == cv && ui < ci)) ? 1 : 0; }
-    }
-    for (int o = 1; o < SP; o <<= 1) rank += __shfl_xor(rank, o);
-    if (c < nc && part == 0 && rank < k) { L.r_val[rank] = cv; L.r_idx[rank] = ci; }
-  }
-  __syncthreads();
-  if (e < k) { int me = L.r_idx[e], pos = 0; for (int j = 0; j < k; ++j) pos += L.r_idx[j] < me ? 1 : 0; L.s_idx[pos] = me; L.s_val[pos] = L.r_val[e]; }
-  __syncthreads();
+  ROUTE_TS(5);
+  lds_barrier(); ROUTE_TS(6);
+  if (wave == 0) { if (n_exp <= 512) route_select<8>(n_exp, k, L, lane); else route_select<16>(n_exp, k, L, lane); }
+  ROUTE_TS(7);
+  lds_barrier();
 }
 // softmax over the chosen logits in ascending expert id (soft_top); called by the whole workgroup after route_topk
 __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
   const int e = threadIdx.x;
   float mx = -INFINITY, ex = 1.0f;
   if (e < k) { for (int i = 0; i < k; ++i) mx = fmaxf(mx, L.s_val[i]); ex = isfinite(mx) ? expf(L.s_val[e] - mx) : 1.0f; L.r_val[e] = ex; }
-  __syncthreads();
+  lds_barrier();
   if (e < k) {
     float w;
     if (!isfinite(mx)) w = 1.0f / (float)k;
@@ -86,6 +121,7 @@ template <int FMT, int NW, int P, bool PRE>
 __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
+  PYRE_TS_VARS PYRE_TS(0);
   __shared__ float red[2][P][NW][64];
   __shared__ RouteLds rl;
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
@@ -97,7 +133,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   int expert = 0;
   if (!shared) {
     if constexpr (PRE) expert = __builtin_amdgcn_readfirstlane(sel_idx[ti * m.top_k + j]);
-    else { route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl); expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]); }
+    else { route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl ROUTE_TS_ARG); expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]); }
   } else if (blockIdx.x == 0) {
     float p = 0.0f;
     for (int ib = threadIdx.x; ib < m.d; ib += 4 * NW * 64) {          // four elements per pass, loads first (elements past d: weight zero)
@@ -110,10 +146,11 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
     if (lane == 0) red[0][0][wave][0] = p;
-    __syncthreads();
+    lds_barrier();
     if (threadIdx.x == 0) { float tot = 0.0f; for (int w = 0; w < NW; ++w) tot += red[0][0][w][0]; rl.s_w[0] = 1.0f / (1.0f + expf(-tot)); }
-    __syncthreads();
+    lds_barrier();
   }
+  PYRE_TS(1);
   const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
   const int tile = (shared ? 0 : expert * (m.ff >> 6)) + blockIdx.x;
   const int nz = gridDim.z, kz = blockIdx.z, np = P * nz;          // np parts in all
@@ -142,7 +179,8 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
   }
 #pragma unroll
   for (int p = 0; p < P; ++p) { red[0][p][wave][lane] = ag[p][0]; red[1][p][wave][lane] = au[p][0]; }
-  __syncthreads();
+  PYRE_TS(2);
+  lds_barrier(); PYRE_TS(3);
   if (threadIdx.x < 64) {
     float g = 0.0f, u = 0.0f;
 #pragma unroll
@@ -169,13 +207,17 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
       if (threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
     }
   }
+  PYRE_TS(4); PYRE_TS_FLUSH(moe_ts, 0);
 }
 
 // ---- routing alone (windows of several tokens): grid t, 1024 threads; ids ascending and softmax weights of token ti ------
 __global__ __launch_bounds__(1024) void k_moe_route(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int nsl, int sstride, int tstride) {
   __shared__ RouteLds rl;
   const int ti = blockIdx.x;
-  route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl);
+#ifdef PYRE_PHASE_TS
+  unsigned long long ts_[8];
+#endif
+  route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl ROUTE_TS_ARG);
   route_weights(m.top_k, rl);
   if ((int)threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
 }
@@ -188,6 +230,7 @@ template <int FMT, int NW, int NZ>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
                                                      const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
+  PYRE_TS_VARS PYRE_TS(0);
   __shared__ float red[NW][64];
   __shared__ float hx[NZ > 1 ? NW : 1][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
@@ -219,13 +262,15 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
     }
   }
   red[wave][lane] = acc[0];
-  __syncthreads();
+  PYRE_TS(1);
+  lds_barrier(); PYRE_TS(2);
   if (threadIdx.x < 64) {
     float s = red[0][lane];
 #pragma unroll
     for (int w = 1; w < NW; ++w) s += red[w][lane];
     partial[(size_t)entry * m.d + blockIdx.x * 64 + lane] = s;
   }
+  PYRE_TS(3); PYRE_TS_FLUSH(moe_ts, 8);
 }
 
 // y[ti][r] = shared[ti][r] * sg[ti] + (sum over the token's experts, ascending id, from zero, of w * partial)

@@ -2,6 +2,7 @@
 // Drop-in for QMat / QMat::matmul of the reference (src/model/gguf_q.rs:201-247).
 #include "formats.h"
 #include <stdlib.h>
+PYRE_TS_DECL(qmat_ts) PYRE_TS_EXPORT(qmat_ts, pyre_debug_ts_qmat)
 
 // ---- repack: raw GGUF rows -> planes --------------------------------------------------------------------------------
 // One thread per (padded row, unit).  Rows beyond m.rows are written as zeros (they decode to 0 and are never stored).
@@ -192,6 +193,7 @@ template <int FMT, int T, int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __restrict__ x, float* __restrict__ y, int upw,
                                                   GemvEpi ep, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
+  PYRE_TS_VARS PYRE_TS(0);
   __shared__ float red[NW][T][64];
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -207,6 +209,10 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = 0.0f;
   if constexpr (T == 1) {
+    // One token: a unit's 64 activations reach all lanes as scalar loads, and every multiply-add takes its activation
+    // straight from a scalar register.  (Copying the K range into shared memory first, all loads in flight at once, was
+    // measured slower: 4.2 against 2.3 us for a 2048-column projection -- 64 shared-memory reads per unit and vector
+    // operands cost more than the units' scalar round trips save.)
     for (int ku = k0; ku < k1; ++ku) unit_dot<FMT, T>(m, lds2, tile, ku, lane, x + (size_t)ku * 64, m.cols, acc);
   } else {
     // Several tokens: T x 64 activations per unit do not fit the scalar registers, and scalar loads in pieces cost one
@@ -233,7 +239,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) red[wave][t][lane] = acc[t];
-  __syncthreads();
+  PYRE_TS(1);
+  lds_barrier(); PYRE_TS(2);
   const size_t r64 = (size_t)m.tiles * 64;
   for (int i = threadIdx.x; i < T * 64; i += NW * 64) {
     int t = i >> 6, l = i & 63; float s = red[0][t][l];
@@ -270,6 +277,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemv(QMatDev m, const float* __rest
 #pragma unroll
     for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
   }
+  PYRE_TS(3); PYRE_TS_FLUSH(qmat_ts, (NW == 16 ? 0 : (gridDim.y > 1 ? 8 : 16)));
 }
 
 namespace {
