@@ -91,6 +91,15 @@ struct QMatDev {
 };
 inline double qmat_gguf_bytes(const QMatDev& m, double rows) { return rows * (m.cols / m.gel) * m.gbytes; }
 
+#ifdef __HIPCC__
+// Kernel arguments are scalar loads from the argument block, which the compiler otherwise issues where each value is
+// first needed: behind branches that is one memory round trip after another before the first vector load can go out.
+// Naming the values here makes every such load leave at the kernel's first instruction, under one wait.
+template <typename A> __device__ __forceinline__ void arg_now(A a) { asm volatile("" ::"s"(a)); }
+template <typename... A> __device__ __forceinline__ void args_now(A... a) { (arg_now(a), ...); }
+__device__ __forceinline__ void qmat_args_now(const QMatDev& m) { args_now(m.p0, m.p1, m.p2, m.p3, m.pb, m.rows, m.cols, m.U, m.tiles); }
+#endif
+
 struct pyre_qmat {
   pyre_ctx* ctx; uint32_t ty; size_t rows, cols; size_t gguf_bytes;
   void* base; size_t dev_bytes; QMatDev dv;

@@ -33,6 +33,7 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int G = 4, R = DK / G;
   PYRE_TS_VARS PYRE_TS(0);
+  args_now(p.a, p.dt, p.norm_w, p.nk, p.nv, p.eps, proj, stride, t, co_all, ssm_in, ssm_out, out);
   __shared__ float qs[DK], ks[DK], pm[G][DV], po[G][DV], red[8];
   const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7;
   const int ch = 2 * p.nk * DK + p.nv * DV, w = p.nv * DV;

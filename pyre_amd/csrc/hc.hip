@@ -71,6 +71,7 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
     float* __restrict__ part, int upw, const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
+  qmat_args_now(m); args_now(x_in, in_ss, in_ts, x_out, comb_out, mo.partial, mo.sel_w, mo.sg, mo.d, mo.k, comb_inj, norm, d, hc, ssq, part, upw);
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, nw = nthr >> 6, tid = threadIdx.x, L = nw * upw * 64;
   float* xs = sm;                         // [T][L]
@@ -150,6 +151,8 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
+  qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj);
+
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, U = lr >> 6, kps = ksplit / hc, nw = nthr >> 6;
   float* lo = sm;                         // [T][lr]

@@ -122,6 +122,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __res
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
+  args_now(m.n_exp, m.top_k, logits, nsl, sstride, tstride);          // what the selection needs; the rest would crowd the scalar registers the activations go through
   __shared__ float red[2][P][NW][64];
   __shared__ RouteLds rl;
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
@@ -231,6 +232,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
                                                      const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
+  qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, partial);
   __shared__ float red[NW][64];
   __shared__ float hx[NZ > 1 ? NW : 1][64];
   const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
