@@ -8,6 +8,11 @@ Workloads (synthetic weights and inputs, resident in HBM before the timed region
           One step = one generated token; the whole loop runs on the device without host round trips.
   gemv    one IQ3_S dequant-GEMV of the vocabulary-head shape (151936 x 2048, t = 1) per step, rotating over enough
           distinct weight buffers (> 512 MB) that nothing is served from the 256 MB Infinity Cache.
+  gemv0   configs[0]: the single 4096 x 4096 IQ3_S GEMV, rotating over 128 matrices, plus cache-resident rate and call latency.
+  sweep   configs[1]: IQ2_XS / IQ3_S / Q4_K / Q8_0 x five shapes x t in 1, 2, 4, 8 (one table under "sweep").
+  moe     configs[2]: the MoE FFN step (512 experts top-10 + shared) at t = 1 and 4.
+  gdn     configs[3]: the Gated DeltaNet decode step and the 4096-token chunked prefill (kernel durations).
+  attn    the attention layer core of configs[4] at --ctx cached positions (kernel durations).
 Timed regions are bracketed by HIP events recorded on the library's own stream; per-kernel-class durations come from
 the library's event-pair profiler in a second, separately timed pass.
 """
@@ -152,6 +157,252 @@ def bench_gemv(args):
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_gemv(ty, rows, cols, 9000)
     return out
+
+
+# ------------------------------------------------------------------------------------------ the other configurations
+def _dev_matrix(ctx, lib, synth, ty, rows, cols, seed):
+    el, bs, _ = synth.GEOM[ty]
+    nb = rows * (cols // el)
+    dev = ctx.alloc(nb * bs)
+    ctx.synth_blocks(ty, nb, seed, dev_out=dev)
+    m = lib.QMat(ctx, ty, rows, cols, dev_blocks=dev, nbytes=nb * bs)
+    ctx.free(dev)
+    return m
+
+
+def _timed(ev, ctx, n, fn):
+    e0, e1 = ev.event(), ev.event()
+    ctx.sync(); ev.record(e0, ctx.stream)
+    for i in range(n):
+        fn(i)
+    ev.record(e1, ctx.stream)
+    return ev.elapsed_ms(e0, e1) / n
+
+
+def _prof(ctx, n, fn):
+    """{kernel class: (launches per step, avg launch us, algorithmic bytes per launch)} from the library's event pairs."""
+    ctx.prof_reset(); ctx.prof_enable(True)
+    for i in range(n):
+        fn(i)
+    ctx.sync()
+    rep = ctx.prof_report(); ctx.prof_enable(False)
+    return {k: (v[0] / n, v[1] / v[0] * 1e3, v[2] / v[0]) for k, v in rep.items()}
+
+
+def _line(metric, value, unit, args, per_ms, dtype, workload, roofline, extra):
+    out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per_ms, 5),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": {"workload": workload}, "roofline": roofline}
+    out.update(extra)
+    return out
+
+
+def bench_gemv0(args):
+    """configs[0]: one IQ3_S GEMV, 4096 x 4096, t = 1.  The matrix (7.2 MB) fits the 256 MB Infinity Cache many times over, so
+    the timed loop rotates over 128 distinct matrices (923 MB); the cache-resident rate and the latency of one synchronised call
+    are reported beside it."""
+    from pyre_amd import lib, synth
+    ev = HipEvents(); ctx = lib.Context(0)
+    rows = cols = 4096; ty = lib.IQ3_S; nbuf = 128
+    mats = [_dev_matrix(ctx, lib, synth, ty, rows, cols, 100 + i) for i in range(nbuf)]
+    x = ctx.upload(synth.normal((1, cols), 3)); y = ctx.alloc(rows * 4)
+    alg = mats[0].gguf_bytes + 4 * cols + 4 * rows
+    res = {}
+    for name, call in (("operator_i8", lambda m: m.matmul_dev(x, 1, y)), ("f32", lambda m: m.matmul_f32_dev(x, 1, y))):
+        for i in range(args.warmup):
+            call(mats[i % nbuf])
+        per = _timed(ev, ctx, args.steps, lambda i: call(mats[i % nbuf]))
+        hot = _timed(ev, ctx, args.steps, lambda i: call(mats[0]))
+        pr = _prof(ctx, min(args.steps, 128), lambda i: call(mats[i % nbuf]))
+        lat = []
+        for i in range(20):
+            ctx.sync(); t0 = time.perf_counter(); call(mats[(7 * i) % nbuf]); ctx.sync(); lat.append((time.perf_counter() - t0) * 1e6)
+        dom = max(pr.items(), key=lambda kv: kv[1][1] * kv[1][0])
+        res[name] = {"us_per_call_rotating": round(per * 1e3, 3), "GBps_rotating": round(alg / (per * 1e-3) / 1e9, 1), "us_per_call_cache_resident": round(hot * 1e3, 3),
+                     "GBps_cache_resident": round(alg / (hot * 1e-3) / 1e9, 1), "single_synchronised_call_us_median": round(float(np.median(lat)), 2),
+                     "kernels": {k: {"launches_per_call": round(v[0], 2), "avg_launch_us": round(v[1], 3)} for k, v in pr.items()},
+                     "dominant_kernel": dom[0], "dominant_kernel_us": round(dom[1][1], 3), "dominant_kernel_GBps": round(alg / (dom[1][1] * 1e-6) / 1e9, 1)}
+    op = res["operator_i8"]
+    roof = {"bound": "hbm", "achieved": op["dominant_kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(op["dominant_kernel_GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": op["dominant_kernel"], "algorithmic_bytes_per_launch": alg, "device_bytes_per_launch": mats[0].dev_bytes, "avg_launch_us": op["dominant_kernel_us"]}
+    extra = {"paths": res}
+    if not args.no_cpu:
+        import orc
+        threads = min(os.cpu_count() or 1, 16)
+        raw = synth.matrix(ty, rows, cols, 100); xh = synth.normal((1, cols), 3)
+        orc.matmul(ty, raw, rows, cols, xh, threads=threads); n = 0; t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 10.0 and n < 400:
+            orc.matmul(ty, raw, rows, cols, xh, threads=threads); n += 1
+        dt = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": round(n * alg / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+                                 "sample": "%d calls of the oracle matmul (row dequant + f32 dot, rows over %d threads) on the whole 4096 x 4096 IQ3_S matrix, t=1" % (n, threads)}
+    return _line("IQ3_S dequant-GEMV achieved HBM GB/s (4096x4096, t=1)", op["GBps_rotating"], "GB/s", args, op["us_per_call_rotating"] / 1e3, "f32",
+                 "configs[0]: IQ3_S GEMV 4096x4096, batch 1, rotating over %d weight buffers (%.0f MB); operator path (integer dot) and f32 path" % (nbuf, nbuf * mats[0].gguf_bytes / 1e6), roof, extra)
+
+
+def bench_sweep(args):
+    """configs[1]: IQ2_XS, IQ3_S, Q4_K, Q8_0 x five shapes x t in 1, 2, 4, 8; every case rotates over enough matrices to exceed
+    600 MB (at most 512 of them: the smallest shapes stay partly cache resident, their working set is stated)."""
+    from pyre_amd import lib, synth
+    ev = HipEvents(); ctx = lib.Context(0)
+    fmts = [("IQ2_XS", lib.IQ2_XS), ("IQ3_S", lib.IQ3_S), ("Q4_K", lib.Q4_K), ("Q8_0", lib.Q8_0)]
+    shapes = [(4096, 2048), (2048, 4096), (512, 2048), (2048, 512), (151936, 2048)]
+    table = []
+    steps = max(16, min(args.steps, 200))
+    for fname, ty in fmts:
+        for rows, cols in shapes:
+            el, bs, _ = synth.GEOM[ty]
+            gbytes = rows * (cols // el) * bs
+            nbuf = int(min(512, max(2, -(-600e6 // gbytes))))
+            mats = [_dev_matrix(ctx, lib, synth, ty, rows, cols, 7000 + 31 * i + ty) for i in range(nbuf)]
+            x = ctx.upload(synth.normal((8, cols), 5)); y = ctx.alloc(8 * rows * 4)
+            for t in (1, 2, 4, 8):
+                for i in range(4):
+                    mats[i % nbuf].matmul_dev(x, t, y)
+                per = _timed(ev, ctx, steps, lambda i: mats[i % nbuf].matmul_dev(x, t, y))
+                alg = gbytes + 4 * t * (cols + rows)
+                table.append({"fmt": fname, "rows": rows, "cols": cols, "t": t, "us_per_call": round(per * 1e3, 3), "GBps": round(alg / (per * 1e-3) / 1e9, 1),
+                              "frac_of_peak": round(alg / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "working_set_MB": round(nbuf * gbytes / 1e6)})
+            for m in mats:
+                m.close()
+            ctx.free(x); ctx.free(y)
+        log("sweep: %s done" % fname)
+    head = next(r for r in table if r["fmt"] == "IQ3_S" and r["rows"] == 151936 and r["t"] == 1)
+    gm = float(np.exp(np.mean([np.log(r["GBps"]) for r in table])))
+    roof = {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac_of_peak"], "traffic": None,
+            "kernel": "operator call (every launch of pyre_qmatmul_dev), IQ3_S 151936x2048 t=1", "avg_launch_us": head["us_per_call"]}
+    extra = {"sweep": table, "geometric_mean_GBps": round(gm, 1)}
+    if not args.no_cpu:
+        extra["cpu_baseline"] = cpu_baseline_gemv(lib.IQ3_S, 151936, 2048, 9000)
+    return _line("quant-format GEMV sweep, achieved HBM GB/s per operator call (value: IQ3_S vocab head, t=1)", head["GBps"], "GB/s", args, head["us_per_call"] / 1e3, "f32",
+                 "configs[1]: IQ2_XS / IQ3_S / Q4_K / Q8_0 x {4096<-2048, 2048<-4096, 512<-2048, 2048<-512, 151936<-2048} x t in {1,2,4,8}, rotating weight buffers", roof, extra)
+
+
+def bench_moe(args):
+    """configs[2]: the MoE FFN step, 512 routed experts top-10 + 1 shared, d 2048, expert ff 512, IQ3_S, bf16 router, t in 1, 4.
+    Two layers' worth of experts (1.4 GB) alternate and the token activations rotate, so the chosen experts are cold."""
+    from pyre_amd import lib, synth
+    from pyre_amd import modelgen as mg
+    ev = HipEvents(); ctx = lib.Context(0)
+    c = mg.a3b_config(n_layers=2, full_every=8)
+    layers, globals_, raw = mg.build_device(ctx, c, seed=17)
+    moes = []
+    for L in layers:
+        qm = {s: (lib.QMat(ctx, L[s][0], L[s][1], L[s][2], dev_blocks=L[s][3], nbytes=L[s][1] * (L[s][2] // synth.GEOM[L[s][0]][0]) * synth.GEOM[L[s][0]][1]) if not isinstance(L[s][3], np.ndarray)
+                  else lib.QMat(ctx, L[s][0], L[s][1], L[s][2], L[s][3])) for s in (mg.ROUTER, mg.GATE_E, mg.UP_E, mg.DOWN_E, mg.SH_GATE, mg.SH_UP, mg.SH_DOWN)}
+        moes.append((lib.Moe(ctx, c.top_k, qm[mg.ROUTER], qm[mg.GATE_E], qm[mg.UP_E], qm[mg.DOWN_E], L[mg.SH_GATE_INP][3].view(np.float32), qm[mg.SH_GATE], qm[mg.SH_UP], qm[mg.SH_DOWN]), qm))
+    host_raw = None
+    if not args.no_cpu:          # the oracle's copy of layer 0, before the raw blocks are freed
+        host_raw = {s: ((layers[0][s][0], layers[0][s][1], layers[0][s][2], ctx.download(layers[0][s][3], (layers[0][s][1] * (layers[0][s][2] // synth.GEOM[layers[0][s][0]][0]) * synth.GEOM[layers[0][s][0]][1],), np.uint8))
+                        if not isinstance(layers[0][s][3], np.ndarray) else layers[0][s]) for s in (mg.ROUTER, mg.GATE_E, mg.UP_E, mg.DOWN_E, mg.SH_GATE, mg.SH_UP, mg.SH_DOWN, mg.SH_GATE_INP)}
+    for p in raw:
+        ctx.free(p)
+    nx = 64
+    xs = synth.normal((nx * 4, c.d), 23)
+    xd = ctx.upload(xs); yd = ctx.alloc(4 * c.d * 4)
+    el, bs, _ = synth.GEOM[synth.IQ3_S]
+    per_expert = (2 * c.ff_exp * (c.d // el) + c.d * (c.ff_exp // el)) * bs
+    res = {}
+    for t in (1, 4):
+        call = lambda i: moes[i % 2][0].ffn_dev(xd + ((i % nx) * 4) * c.d * 4, t, yd)
+        for i in range(args.warmup):
+            call(i)
+        per = _timed(ev, ctx, args.steps, call)
+        pr = _prof(ctx, min(args.steps, 64), call)
+        alg = c.n_exp * c.d * 2 + (min(t * c.top_k, c.n_exp) + 1) * per_expert + 4 * t * 2 * c.d          # bf16 router + distinct experts (upper bound: all distinct) + shared
+        ksum = sum(v[0] * v[1] for v in pr.values())
+        res["t%d" % t] = {"us_per_step": round(per * 1e3, 3), "algorithmic_bytes": alg, "GBps": round(alg / (per * 1e-3) / 1e9, 1), "frac_of_peak": round(alg / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                          "kernel_us_per_step": round(ksum, 3), "kernels": {k: {"launches_per_step": round(v[0], 2), "avg_launch_us": round(v[1], 3), "GBps": round(v[2] / (v[1] * 1e-6) / 1e9, 1) if v[2] else None} for k, v in pr.items()}}
+    r1 = res["t1"]; dom = max(r1["kernels"].items(), key=lambda kv: kv[1]["avg_launch_us"] * kv[1]["launches_per_step"])
+    roof = {"bound": "hbm", "achieved": dom[1]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round((dom[1]["GBps"] or 0) / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom[0], "avg_launch_us": dom[1]["avg_launch_us"]}
+    extra = {"steps_by_width": res}
+    if host_raw is not None:
+        import orc
+        threads = min(os.cpu_count() or 1, 16)
+        T = {s: orc.tensor(*host_raw[s]) for s in (mg.ROUTER, mg.GATE_E, mg.UP_E, mg.DOWN_E, mg.SH_GATE, mg.SH_UP, mg.SH_DOWN)}
+        sgi = host_raw[mg.SH_GATE_INP][3].view(np.float32)
+        f = lambda i: orc.moe_ffn(c.d, c.n_exp, c.top_k, c.ff_exp, T[mg.ROUTER], T[mg.GATE_E], T[mg.UP_E], T[mg.DOWN_E], sgi, T[mg.SH_GATE], T[mg.SH_UP], T[mg.SH_DOWN], xs[4 * (i % nx):4 * (i % nx) + 1], threads=threads)
+        f(0); n = 0; t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 10.0 and n < 2000:
+            f(n); n += 1
+        dt = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": round(n / dt, 2), "unit": "MoE steps/s (t=1)", "cores": threads, "kind": "port",
+                                 "sample": "%d single-token steps of the oracle's moe_ffn on layer 0's tensors (512 experts resident, top-10 + shared)" % n}
+    return _line("MoE FFN step (512 experts top-10 + shared, IQ3_S): steps/s at t=1", round(1e3 / r1["us_per_step"] * 1e3, 1), "steps/s", args, r1["us_per_step"] / 1e3, "f32",
+                 "configs[2]: MoE FFN step, d 2048, ff 512, 512 experts top-10 + 1 shared, IQ3_S, bf16 router, batch 1 and 4; two layers' experts alternate, 64 activations rotate", roof, extra)
+
+
+def bench_gdn(args):
+    """configs[3]: the Gated DeltaNet layer core, 16 QK / 32 V heads of 128: the decode step at batch 1 and the chunked prefill of
+    4096 tokens (chunks of 64).  The block entry points take host buffers, so the figures are the kernels' own durations (event
+    pairs on the library's stream around each launch): inputs are in HBM when a timed region starts."""
+    from pyre_amd import lib
+    ctx = lib.Context(0)
+    nk, nv, T = 16, 32, 4096
+    ch = 2 * nk * 128 + nv * 128
+    g = np.random.Generator(np.random.PCG64(41))
+    a = (-np.exp(g.uniform(0.0, np.log(16.0), nv))).astype(np.float32); dt = np.zeros(nv, np.float32)
+    conv_w = (0.5 * g.standard_normal(ch * 4)).astype(np.float32); norm_w = (1 + 0.1 * g.standard_normal(128)).astype(np.float32)
+    gd = lib.Gdn(ctx, nk, nv, 128, 128, 4, 1e-6, a, dt, conv_w, norm_w)
+    S0 = (0.01 * g.standard_normal((nv, 128, 128))).astype(np.float32)
+    gd.set_state(None, S0)
+    qkv = g.standard_normal((T, ch), dtype=np.float32); z = g.standard_normal((T, nv * 128), dtype=np.float32)
+    beta = g.standard_normal((T, nv), dtype=np.float32); alpha = g.standard_normal((T, nv), dtype=np.float32)
+    n = max(8, min(args.steps, 128))
+    for i in range(args.warmup):
+        gd.step(qkv[i:i + 1], z[i:i + 1], beta[i:i + 1], alpha[i:i + 1])
+    pr = _prof(ctx, n, lambda i: gd.step(qkv[i:i + 1], z[i:i + 1], beta[i:i + 1], alpha[i:i + 1]))
+    step_us = sum(v[0] * v[1] for v in pr.values())
+    state_b = 2 * nv * 128 * 128 * 4 + 2 * 3 * ch * 4 + 4 * (ch + nv * 128 + 2 * nv) + 4 * nv * 128
+    gd.set_state(None, S0)
+    gd.prefill_chunked(qkv, z, beta, alpha)                  # untimed
+    gd.set_state(None, S0)
+    pp = _prof(ctx, 1, lambda i: gd.prefill_chunked(qkv, z, beta, alpha))
+    pre_us = sum(v[0] * v[1] for v in pp.values())
+    # fp32 matrix work of the chunked form per (head, chunk of 64): A = K K^T (64x64x128), B-ish products and the state update: ~ 2*(64*64*128*3 + 64*128*128*3) flop
+    flop = nv * (T // 64) * 2.0 * (3 * 64 * 64 * 128 + 3 * 64 * 128 * 128)
+    res = {"decode_step": {"kernel_us": round(step_us, 3), "algorithmic_bytes": state_b, "GBps": round(state_b / (step_us * 1e-6) / 1e9, 1), "frac_of_hbm_peak": round(state_b / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                           "kernels": {k: {"launches_per_step": round(v[0], 2), "avg_launch_us": round(v[1], 3)} for k, v in pr.items()}},
+           "prefill_4096": {"kernel_ms": round(pre_us / 1e3, 3), "us_per_token": round(pre_us / T, 4), "matrix_TFLOPs": round(flop / (pre_us * 1e-6) / 1e12, 2), "frac_of_fp32_mfma_peak": round(flop / (pre_us * 1e-6) / 1e12 / 157.3, 4),
+                            "kernels": {k: {"launches": round(v[0], 2), "avg_launch_us": round(v[1], 3)} for k, v in pp.items()}}}
+    roof = {"bound": "hbm", "achieved": res["decode_step"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["decode_step"]["frac_of_hbm_peak"], "traffic": None, "kernel": "gdn_delta", "avg_launch_us": round(step_us, 3)}
+    extra = {"gdn": res}
+    if not args.no_cpu:
+        import orc
+        so, co = S0.copy().reshape(-1), np.zeros(3 * ch, np.float32)
+        m = 0; t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 10.0 and m < T:
+            orc.gdn_core(nk, nv, 128, 128, 4, 1e-6, a, dt, conv_w, norm_w, qkv[m:m + 64], z[m:m + 64], beta[m:m + 64], alpha[m:m + 64], co, so); m += 64
+        dtc = time.perf_counter() - t0
+        extra["cpu_baseline"] = {"value": round(m / dtc, 1), "unit": "tokens/s (sequential recurrence)", "cores": 1, "kind": "port", "sample": "%d tokens of the oracle's linear_core restatement, one thread" % m}
+    return _line("Gated DeltaNet decode step (16/32 heads of 128): steps/s by kernel time", round(1e6 / step_us, 1), "steps/s", args, step_us / 1e3, "f32",
+                 "configs[3]: Gated DeltaNet layer core, post-projection inputs, conv 4, state N(0,0.01), A_log~U(0,ln16); decode step at batch 1 and chunked prefill of 4096 tokens (chunk 64)", roof, extra)
+
+
+def bench_attn(args):
+    """The gated attention layer core over the 4-bit cache at the metric's context (16 / 2 heads of 256, 32768 positions, newest
+    1024 in f32), t = 1: kernel durations from the library's event pairs (the block entry point takes host buffers)."""
+    from pyre_amd import lib
+    ctx = lib.Context(0)
+    nh, nkv, n0 = 16, 2, args.ctx
+    row = nkv * 256
+    g = np.random.Generator(np.random.PCG64(43))
+    att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, np.ones(256, np.float32), np.ones(256, np.float32), 4, 1024, n0 + 512)
+    att.load_cache(g.standard_normal((n0, row), dtype=np.float32), g.standard_normal((n0, row), dtype=np.float32))
+    q = g.standard_normal((256, nh * 512), dtype=np.float32); k = g.standard_normal((256, row), dtype=np.float32); v = g.standard_normal((256, row), dtype=np.float32)
+    n = max(8, min(args.steps, 128))
+    for i in range(args.warmup):
+        att.decode(q[i:i + 1], k[i:i + 1], v[i:i + 1])
+    pr = _prof(ctx, n, lambda i: att.decode(q[8 + i:9 + i], k[8 + i:9 + i], v[8 + i:9 + i]))
+    us = sum(v_[0] * v_[1] for v_ in pr.values())
+    nn = n0 + args.warmup + n // 2
+    pb = ((nn - 1024) // 64) * 64 if nn > 1024 + 64 else 0
+    alg = 2 * row * (pb * 0.625 + (nn - pb) * 4.0)
+    dom = max(pr.items(), key=lambda kv: kv[1][0] * kv[1][1])
+    roof = {"bound": "hbm", "achieved": round(alg / (dom[1][1] * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg / (dom[1][1] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": dom[0], "algorithmic_bytes_per_launch": round(alg), "avg_launch_us": round(dom[1][1], 3)}
+    extra = {"kernels": {k_: {"launches_per_step": round(v_[0], 2), "avg_launch_us": round(v_[1], 3)} for k_, v_ in pr.items()}, "kernel_us_per_step": round(us, 3)}
+    return _line("gated attention decode step over the 4-bit KV cache: steps/s by kernel time", round(1e6 / us, 1), "steps/s", args, us / 1e3, "f32",
+                 "attention layer core of configs[4]: 16 Q / 2 KV heads of 256, %d cached positions (4-bit below the newest 1024), batch 1" % n0, roof, extra)
 
 
 # -------------------------------------------------------------------------------------------------------------- decode
@@ -356,7 +607,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="decode", choices=["decode", "gemv"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "gemv", "gemv0", "sweep", "moe", "gdn", "attn"])
     ap.add_argument("--ctx", type=int, default=32768, help="prompt length for the decode workload")
     ap.add_argument("--layers", type=int, default=0, help="debug: fewer layers than the 48 of the configuration")
     ap.add_argument("--seed", type=int, default=1)
@@ -373,7 +624,7 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the reference path is single-GPU, single-process); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    out = {"gemv": bench_gemv, "decode": bench_decode}[args.workload](args)
+    out = {"gemv": bench_gemv, "decode": bench_decode, "gemv0": bench_gemv0, "sweep": bench_sweep, "moe": bench_moe, "gdn": bench_gdn, "attn": bench_attn}[args.workload](args)
     print(json.dumps(out))
 
 

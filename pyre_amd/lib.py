@@ -294,6 +294,9 @@ class QMat:
     def matmul_dev(self, x_dev, t, y_dev):
         self.ctx.check(self.ctx.L.pyre_qmatmul_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_dev")
 
+    def matmul_f32_dev(self, x_dev, t, y_dev):
+        self.ctx.check(self.ctx.L.pyre_qmatmul_f32_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_f32_dev")
+
     def close(self):
         if getattr(self, "h", None) and getattr(self.ctx, "h", None):
             self.ctx.L.pyre_qmat_destroy(self.h)
