@@ -77,27 +77,30 @@ int    pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_h
  * multi-token verify pass equal one-token decode (qwen4exp_gguf.rs:2357-2360). */
 int    pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
-/* IQ3_S matrices take pyre_qmatmul through integer dot products: each 64-column unit of x is first written as block
- * fixed point (power-of-two scale, 23-bit signed integers; |error| <= 2^-23 of the unit's largest magnitude), the
- * products with the 4-bit codes are exact in int32 and the block scales are applied in f32.  A non-finite activation
- * makes every output NaN.  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the model's layers use
- * (QMat::matmul's own arithmetic, gguf_q.rs:169-197,233-241: f32 products, f32 accumulation); for every other type
- * the two are the same code. */
+/* IQ3_S matrices take pyre_qmatmul through the f16 matrix cores, for every t with one kernel (the reference's verify
+ * kernels, src/model/qn_cube.rs:17,6454, and lcm_dense, qwen4exp_gguf.rs:2641-2737, are this product with t > 1): each
+ * 256-column stretch of a token is scaled by its own power of two and every value is written as two f16 halves (22
+ * significant bits; values more than 2^14 / 6e-5 below the largest magnitude of their stretch lose resolution), the 4-bit
+ * codes times their sub-block scales are exact in f16, products are exact and summed in f32.  A non-finite activation
+ * makes every output of its token NaN.  An IQ3_S matrix created through pyre_qmat_create* is held in two layouts (one per
+ * kernel; pyre_qmat_device_bytes counts both).  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the
+ * model's expert matrices use (QMat::matmul's own arithmetic, gguf_q.rs:169-197,233-241: f32 products, f32 accumulation);
+ * for every other type the two are the same code. */
 int    pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
 /* pyre_qmatmul_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  IQ3_S matrices only -- the one type whose GEMV
- * needs a scratch buffer (the activations' fixed-point digits); every other type's pyre_qmatmul_dev allocates nothing
- * already.  The digits go to a fixed device array inside the library (PYRE_QMATMUL_STATIC_MAX_TU * 256 bytes per GPU,
- * held until the process ends) instead of the context's grow-only buffer, and the call makes no allocation, no event
- * and no copy: two kernel launches on the context's stream.  Same kernels and launch shapes as pyre_qmatmul_dev, so
- * the result is bit-identical to it.  t * cols / 64 above PYRE_QMATMUL_STATIC_MAX_TU is rejected with PYRE_E_SHAPE.
+ * needs a scratch buffer (the activations as f16 operand rows); every other type's pyre_qmatmul_dev allocates nothing
+ * already.  The operand goes to a fixed device array inside the library (PYRE_QMATMUL_STATIC_MAX_COLS * 32 bytes plus
+ * the scale factors, about 1 MiB per GPU, held until the process ends) instead of the context's grow-only buffer, and the
+ * call makes no allocation, no event and no copy: two kernel launches on the context's stream.  Same kernels and launch
+ * shapes as pyre_qmatmul_dev, so the result is bit-identical to it.  Matrices with more than
+ * PYRE_QMATMUL_STATIC_MAX_COLS columns are rejected with PYRE_E_SHAPE.
  * All contexts on one GPU share that GPU's array: calls that overlap in time on one GPU (two contexts' streams) race. */
-#define PYRE_QMATMUL_STATIC_MAX_TU 4096      /* token-units: t = 8 up to 32768 columns, t = 1 up to 262144 */
+#define PYRE_QMATMUL_STATIC_MAX_COLS 32768
 int    pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
-/* The batch 2..8 speculative-verify GEMM on the matrix cores (the reference's verify kernels, src/model/qn_cube.rs:17,6454,
- * and lcm_dense, qwen4exp_gguf.rs:2641-2737): IQ3_S matrices, t in 2..8.  Same contract as pyre_qmatmul; the result
- * agrees with it to about 1e-7 of max|y| but not bit for bit (f16 two-term split of the activations, f32 accumulation). */
+/* pyre_qmatmul restricted to IQ3_S (PYRE_E_TYPE otherwise): kept for callers written against a separate verify-window
+ * entry point; t in 1..8, bit-identical to pyre_qmatmul. */
 int    pyre_qmatmul_mfma(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_mfma_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
 

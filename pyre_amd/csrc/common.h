@@ -41,10 +41,8 @@ struct pyre_ctx {
   struct ProfAcc { long count = 0; double ms = 0, bytes = 0; };
   bool prof_on = false; std::vector<ProfPending> prof_pending; std::map<std::string, ProfAcc> prof_acc; std::vector<hipEvent_t> prof_pool;
   std::string prof_text;
-  unsigned* fuse_ctl = nullptr;                        // control words of in-launch barriers (zeroed once): [0] generation, [16] abort, [32] count
-  void* mfma_buf = nullptr; size_t mfma_bytes = 0;     // split activations of the matrix-core verify GEMM (grow-only)
-  void* i8_buf = nullptr; size_t i8_bytes = 0;         // fixed-point activation digits of the integer-dot GEMV (grow-only)
-  uint32_t* i8_static = nullptr;                       // device address of this GPU's copy of the file-scope digit array (gemv_i8.hip), resolved at creation
+  void* aop_buf = nullptr; size_t aop_bytes = 0;       // split activations of the operator's matrix-core GEMM (grow-only)
+  void* aop_static = nullptr;                          // device address of this GPU's copy of the file-scope operand array (gemm_m.hip), resolved at creation
 };
 
 // Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
@@ -73,8 +71,6 @@ int pyre_fail(pyre_ctx* ctx, int code, const char* fmt, ...);
 #define PYRE_CHECK_LAUNCH(ctx) PYRE_HIP(ctx, hipGetLastError())
 
 int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out);          // grow-only device staging buffer
-// After a stream synchronisation: fails if an in-launch barrier gave up waiting (and clears the flag).
-int pyre_fuse_check(pyre_ctx* ctx);
 
 // ---- device-side matrix view --------------------------------------------------------------------------------------
 // Weights live in "lane = row" planes: rows are grouped in tiles of 64, and for every (tile, unit) the 64 rows'
@@ -83,11 +79,18 @@ int pyre_fuse_check(pyre_ctx* ctx);
 //   vector plane  p0: [tile][unit][chunk < V][lane] x 16 B
 //   small planes  p1..p3: [tile][unit][lane] x e bytes
 //   block plane   pb: [tile][unit/4][lane] x e bytes    (per 256-value super-block)
+// FMT_IQ3_S_M (IQ3_S for the matrix cores): rows in groups of 16, columns in steps of 32 (one sub-block).  In
+// v_mfma_f32_16x16x32_f16 lane l supplies, for the operand that carries the weights, row l % 16 of the group and the eight
+// consecutive columns 8 * (l / 16) .. + 7 of the step, so a lane's share of a step is eight 4-bit codes = one dword:
+//   mq: [row group][128-column chunk][lane] x 16 B: dword s = step s of the chunk; the code of column element e of the lane's
+//       eight sits at nibble e/2 + 4*(e&1), so that or-ing nibbles p and p + 4 into one register yields elements 2p, 2p + 1
+//   mh: [row group][super-block][row] x 8 B: f16 d, 16 zero bits, the eight 4-bit sub-block scales (nibble i = sub-block i)
 struct QMatDev {
   const uint8_t* p0; const uint8_t* p1; const uint8_t* p2; const uint8_t* p3; const uint8_t* pb;
   int rows, cols, U, tiles, fmt;
   uint32_t ty; int gel, gbytes;        // GGUF type the matrix was created from and its block geometry (algorithmic byte counts)
   uint32_t lut[4]; int bias;           // C4 value table (entry = value + bias)
+  const uint8_t* mq; const uint8_t* mh; int SB;      // FMT_IQ3_S_M planes; SB = super-blocks (256 columns) per row
 };
 inline double qmat_gguf_bytes(const QMatDev& m, double rows) { return rows * (m.cols / m.gel) * m.gbytes; }
 
@@ -100,10 +103,16 @@ template <typename... A> __device__ __forceinline__ void args_now(A... a) { (arg
 __device__ __forceinline__ void qmat_args_now(const QMatDev& m) { args_now(m.p0, m.p1, m.p2, m.p3, m.pb, m.rows, m.cols, m.U, m.tiles); }
 #endif
 
+// dv: the lane = row planes (every type).  dvm: the matrix-core layout, IQ3_S only (fmt == FMT_IQ3_S_M when present).
+// Which of the two an IQ3_S matrix holds is decided at creation: the stand-alone operator keeps both (its entry points
+// cover both kernels), the model keeps one per matrix.
+enum { PYRE_LAYOUT_ROWS = 0, PYRE_LAYOUT_M = 1, PYRE_LAYOUT_BOTH = 2 };
 struct pyre_qmat {
   pyre_ctx* ctx; uint32_t ty; size_t rows, cols; size_t gguf_bytes;
   void* base; size_t dev_bytes; QMatDev dv;
+  void* base_m = nullptr; size_t dev_bytes_m = 0; QMatDev dvm{};
 };
+int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, int layout, pyre_qmat** out);
 
 // Optional work folded into the end of a GEMV launch (qmat.hip):
 //   best: t = 1, per row tile (bits of the maximum, first row holding it) -> best[2*tile], best[2*tile+1]
@@ -112,23 +121,26 @@ struct pyre_qmat {
 //         and slides the row's state conv_in -> conv_out ([kk-1][ch], oldest first; in == out is fine).
 struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; int four_waves; };
 // launchers implemented in qmat.hip, used by the block / model code
-int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+// Matrices in the matrix-core layout (FMT_IQ3_S_M) take their activations as the f16 operand `a` when the caller has one (a
+// producer kernel wrote it); otherwise x_dev is split into the context's operand buffer by one more launch.
+struct PyreAop;
+int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, const PyreAop* a = nullptr);
 // waves per workgroup and units per wave the (unsplit) GEMV uses for this matrix
 void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw);
 // K range split over `ksplit` workgroups per row tile; partial[(ks*t_count + t)*tiles*64 + row] holds the slice sums and
 // the consumer adds them in slice order.
-int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit);
+int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* partial_dev, int ksplit, const PyreAop* a = nullptr);
 // Few row tiles, long rows (an output projection): the sixteen waves of pyre_gemv_launch's plan, same units each, as
 // four workgroups of four waves per row tile (the work of a tile on four compute units instead of one).  Each
 // workgroup leaves the sum of its waves, parts[(q*t_count + t)*tiles*64 + row], q < PYRE_GEMV_PARTS; the consumer adds the
 // parts in order from the first.
 #define PYRE_GEMV_PARTS 4
 bool pyre_gemv_parts_ok(const QMatDev& m);
-int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* parts_dev);
+int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* parts_dev, const PyreAop* a = nullptr);
 // t = 1 GEMV that also leaves, per row tile, (bits of the maximum, first row holding it) in best[2*tile], best[2*tile+1].
-int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev);
+int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev, const PyreAop* a = nullptr);
 // y as pyre_gemv_launch (raw projections), plus the conv epilogue described at GemvEpi (best ignored).
-int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, const GemvEpi& conv);
+int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, const GemvEpi& conv, const PyreAop* a = nullptr);
 int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev, int n, float* out_dev, int out_stride);
 // Greedy pick from per-tile maxima (first maximum overall) -> id_out[0] (and mirror[0] if given); when m is given the
 // chosen row is dequantized into out_dev in the same launch (the next token's embedding).
@@ -136,20 +148,36 @@ int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev
 // id goes to mirror[step_dev[0] - step_dev[1]] instead of mirror[0].
 int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev, int* step_dev);
 
-// Verify GEMM on the matrix cores (verify_mfma.hip): IQ3_S, 2 <= t <= 8; y[t][rows] as pyre_gemv_launch, equal to it to
-// ~1e-7 relative (not bit for bit).
-bool pyre_gemm_mfma_ok(const QMatDev& m, int t);
-int pyre_gemm_mfma_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
-
-// IQ3_S GEMV with integer dot products over block-fixed-point activations (gemv_i8.hip), 1 <= t <= 8: y[t][rows] as
-// pyre_gemv_launch, within 2^-23 of each unit's largest activation of it; per-token results do not depend on t.
-// best (t = 1, optional): per-tile maxima as pyre_gemv_argmax_launch.
-bool pyre_gemv_i8_ok(const QMatDev& m, int t);
-int pyre_gemv_i8_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, uint32_t* best_dev);
-// The same launches with the digits in a file-scope device array (at most PYRE_QMATMUL_STATIC_MAX_TU token-units): no
-// allocation of any kind.  pyre_i8_static_init resolves the array's address on the context's device (context creation).
-int pyre_i8_static_init(pyre_ctx* ctx);
-int pyre_gemv_i8_static_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+// ---- IQ3_S GEMM on the matrix cores (gemm_m.hip), 1 <= t <= 8, matrices in FMT_IQ3_S_M ------------------------------------
+// The activations reach the kernel as its f16 operand: every value as two halves, x = h1 + h2 * 2^-11 with h1 = f16(x) and
+// h2 = f16((x - h1) * 2^11) (22 significant bits), token ti's halves as operand rows 2 ti and 2 ti + 1 of R = 2, 4, 8 or 16
+// rows (the power of two that holds the window, pyre_aop_rows), laid out [8-column group][row] x 16 B.  ainv (optional):
+// [super-block][8] factors the super-block's sums are multiplied by per token (the inverse of the power of two the splitter
+// scaled that stretch of the token by); null = 1.  Rows 2t .. R - 1 may hold anything finite or not: a row of the operand
+// only ever reaches its own token's sums, so a token's result is bit-identical for every window width.
+struct PyreAop { const uint4* op; const float* ainv; };
+int pyre_aop_rows(int t);
+size_t pyre_aop_bytes(int cols, int t);                            // operand bytes for a K range of `cols` and a window of t
+// splits x [t][cols] (any magnitudes: each 256-column stretch of a token is scaled by its own power of two) into op / ainv
+int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv);
+// y as pyre_gemv_launch / pyre_gemv_split_launch (ksplit > 1: slice sums) with the epilogues of GemvEpi
+int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep);
+// K parts / waves per workgroup the kernel uses for this matrix (ksplit parts)
+void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* hb_per_wave);
+// the operator's own scratch for the split operand (grow-only, per context), and the fixed per-GPU array of the entry point
+// that allocates nothing (resolved at context creation)
+int pyre_gemm_m_scratch(pyre_ctx* ctx, int cols, uint4** op, float** ainv);
+int pyre_static_init(pyre_ctx* ctx);
+int pyre_gemm_m_static(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
+#ifdef __HIPCC__
+// One activation into the operand a producer kernel leaves for the GEMM that follows it, unscaled (|v| < 65504: the
+// producers' outputs are normalised vectors): element k of token ti of a window with R operand rows.
+__device__ __forceinline__ void aop_store(uint16_t* __restrict__ op, int R, int k, int ti, float v) {
+  const _Float16 h1 = (_Float16)v, h2 = (_Float16)((v - (float)h1) * 2048.0f);
+  const size_t base = ((size_t)(k >> 3) * R + 2 * ti) * 8 + (k & 7);
+  op[base] = __builtin_bit_cast(unsigned short, h1); op[base + 8] = __builtin_bit_cast(unsigned short, h2);
+}
+#endif
 
 // ---- MoE FFN block (moe.hip) ----------------------------------------------------------------------------------------
 struct MoeDev {

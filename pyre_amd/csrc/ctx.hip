@@ -71,22 +71,13 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
   for (int i = 0; i < 512; ++i) cb[1536 + i] = kIq2xsCode[i];
   if ((e = hipMalloc((void**)&ctx->d_cb, 4096 * 2)) != hipSuccess || (e = hipMemcpy(ctx->d_cb, cb.data(), 4096 * 2, hipMemcpyHostToDevice)) != hipSuccess ||
       (e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
-      (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess ||
-      (e = hipMalloc((void**)&ctx->fuse_ctl, 1024)) != hipSuccess || (e = hipMemset(ctx->fuse_ctl, 0, 1024)) != hipSuccess) {
+      (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess) {
     int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: codebook upload: %s", hipGetErrorString(e)); pyre_ctx_destroy(ctx); return rc; }
-  if (pyre_i8_static_init(ctx) != PYRE_OK) { int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: %s", ctx->err.c_str()); pyre_ctx_destroy(ctx); return rc; }
+  if (pyre_static_init(ctx) != PYRE_OK) { int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: %s", ctx->err.c_str()); pyre_ctx_destroy(ctx); return rc; }
   *out = ctx; return PYRE_OK;
 }
 
 }  // extern "C"
-
-int pyre_fuse_check(pyre_ctx* ctx) {
-  unsigned flag = 0;
-  PYRE_HIP(ctx, hipMemcpy(&flag, ctx->fuse_ctl + 16, 4, hipMemcpyDeviceToHost));
-  if (!flag) return PYRE_OK;
-  PYRE_HIP(ctx, hipMemset(ctx->fuse_ctl, 0, 1024));
-  return pyre_fail(ctx, PYRE_E_HIP, "an in-launch barrier gave up waiting for its workgroups (results of this call are invalid)");
-}
 
 extern "C" {
 
@@ -97,9 +88,7 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->stage) (void)hipFree(ctx->stage);
   if (ctx->d_iq3s) (void)hipFree(ctx->d_iq3s);
   if (ctx->d_cb) (void)hipFree(ctx->d_cb);
-  if (ctx->mfma_buf) (void)hipFree(ctx->mfma_buf);
-  if (ctx->i8_buf) (void)hipFree(ctx->i8_buf);
-  if (ctx->fuse_ctl) (void)hipFree(ctx->fuse_ctl);
+  if (ctx->aop_buf) (void)hipFree(ctx->aop_buf);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
   for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto e : ctx->prof_pool) (void)hipEventDestroy(e);

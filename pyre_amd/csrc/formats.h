@@ -8,7 +8,9 @@
 // type is re-coded into at load: one f32 scale per 16 values (the exact f32 product the reference forms before its
 // last multiply) and, per value, a 4-bit code into a 16-entry table of small integers (C4) or an int8 (C8), so that
 // value = scale * integer is the reference's own last multiply.
-enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_C4 = 7, FMT_C8 = 8, FMT_COUNT = 9 };
+// FMT_IQ3_S_M is the second home of an IQ3_S matrix: the same 4-bit codes laid out for the matrix cores (see QMatDev), used by
+// the matrices that only ever meet a GEMV (projections, the vocabulary head, the stand-alone operator).
+enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_C4 = 7, FMT_C8 = 8, FMT_IQ3_S_M = 9, FMT_COUNT = 10 };
 
 struct FmtGeom { int V; int e1, e2, e3, eb; };   // plane entry sizes: 16-byte chunks per unit in p0; bytes per unit in p1..p3; bytes per super-block in pb
 __host__ __device__ inline FmtGeom fmt_geom(int fmt) {
@@ -159,6 +161,19 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
     if (m.ty == PYRE_Q5_K) {                       // gguf_q.rs:112: d1 * q - m1, the subtraction after the rounded product
       uint4 oq = ld_small<uint4>(m.p2, m, tile, ku, lane); float off[4] = {__uint_as_float(oq.x), __uint_as_float(oq.y), __uint_as_float(oq.z), __uint_as_float(oq.w)};
       for (int k = 0; k < 64; ++k) y[k] = y[k] - off[k >> 4];
+    }
+  } else if constexpr (FMT == FMT_IQ3_S_M) {       // the same codes in the matrix-core layout (QMatDev::mq / mh)
+    const size_t row = (size_t)tile * 64 + lane, rgi = row >> 4; const int j = (int)(row & 15);
+    const int sb = ku >> 2, k128 = ku >> 1;
+    const uint2 hdr = ((const uint2*)m.mh)[(rgi * m.SB + sb) * 16 + j];
+    const float d = h2f_bits(hdr.x);
+    for (int c = 0; c < 2; ++c) {                  // sub-block 2*(ku&3) + c of the super-block = step 2*(ku&1) + c of its 128-column half
+      const int sbi = 2 * (ku & 3) + c, st = 2 * (ku & 1) + c;
+      const float db = d * (float)(1 + 2 * ((hdr.y >> (4 * sbi)) & 0xF));
+      for (int kg = 0; kg < 4; ++kg) {
+        const uint32_t w = ((const uint32_t*)m.mq)[((rgi * (size_t)(m.cols >> 7) + k128) * 64 + kg * 16 + j) * 4 + st];
+        for (int e = 0; e < 8; ++e) { const int sv = 2 * (int)((w >> (4 * ((e >> 1) + 4 * (e & 1)))) & 0xF) - 15; y[32 * c + 8 * kg + e] = flip(db * (float)(sv < 0 ? -sv : sv), sv < 0 ? 1u : 0u); }
+      }
     }
   } else {                                         // IQ3_S, gguf_q.rs:141-151, from the 4-bit codes (see iq3s_code)
     float d = h2f_bits(ld_block<uint16_t>(m, tile, ku, lane));

@@ -1,0 +1,273 @@
+// IQ3_S dequant-GEMM on the f16 matrix cores, 1..8 tokens (QMat::matmul, src/model/gguf_q.rs:217-242; the verify window of
+// lcm_dense / the MTP drafter, qwen4exp_gguf.rs:2641-2737, is the same product with t > 1).
+//
+// The lane = row GEMV spends about 2.7 vector instructions per weight and token (nibble -> byte -> float -> fma); on the
+// 151 936 x 2048 head that is as long as streaming its bytes, and every further token of a window costs the same again.
+// Here a weight costs about 1.6 instructions whatever the number of tokens:
+//   * the 4-bit code c of a weight w = (2c - 15) * (2n + 1) * d becomes the f16 number 16 + c by or-ing it into a
+//     mantissa (0x4C00 | c << 6), two per register;
+//   * one packed f16 fma per register pair folds the sub-block scale in: (16 + c) * 2s - 47s = (2c - 15) * s, s = 2n + 1,
+//     every intermediate an integer below 2048 and therefore exact in f16;
+//   * v_mfma_f32_16x16x32_f16 multiplies 16 weight rows x 32 columns with 16 activation rows.  An activation row is one
+//     half of a token: x = h1 + h2 * 2^-11 with h1 = f16(x), h2 = f16((x - h1) * 2^11), 22 significant bits, so eight
+//     tokens fill the sixteen rows and one token costs what eight do;
+//   * d (per super-block and row) and the power of two the activations were scaled by meet the f32 sums once per
+//     128 columns.
+// Products are exact in f32 and are summed in f32, so the result differs from the exact dot product by the 2^-22
+// representation of x and the usual f32 summation error.  A token's operand rows are read by nobody else's sums: its
+// result is bit-identical for every window width.
+//
+// grid (row tiles of 64, K slices), NW waves.  Wave w of slice ks walks 128-column chunks [(ks*NW + w) * cpw, + cpw).
+#include "formats.h"
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+int pyre_aop_rows(int t) { return t <= 1 ? 2 : (t == 2 ? 4 : (t <= 4 ? 8 : 16)); }
+size_t pyre_aop_bytes(int cols, int t) { return (size_t)(cols / 8) * pyre_aop_rows(t) * 16; }
+
+// ---- the activation operand from f32 rows: grid = super-blocks (256 columns), 256 threads, thread = column ---------------------
+// Each 256-column stretch of a token is scaled by its own power of two so that its largest magnitude lands in [2^13, 2^14):
+// the f16 halves then keep 22 bits of every value that matters to the sum, whatever the magnitudes of x.
+__global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, int T, int R, int cols, uint16_t* __restrict__ op, float* __restrict__ ainv) {
+  __shared__ float mx[4][8];
+  const int sb = blockIdx.x, i = threadIdx.x, k = sb * 256 + i, wave = i >> 6, lane = i & 63;
+  float v[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) v[t] = t < T ? x[(size_t)t * cols + k] : 0.0f;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    float a = fabsf(v[t]); a = a == a ? a : INFINITY;         // a NaN anywhere makes the stretch non-finite
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o));
+    if (lane == 0) mx[wave][t] = a;
+  }
+  __syncthreads();
+  uint16_t* o = op + (size_t)(k >> 3) * R * 8 + (k & 7);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const float m = fmaxf(fmaxf(mx[0][t], mx[1][t]), fmaxf(mx[2][t], mx[3][t]));
+    int e = 0;                                                // m * 2^e in [2^13, 2^14); zero and non-finite stretches stay as they are
+    if (m > 0.0f && m < INFINITY) { e = 140 - (int)((__float_as_uint(m) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+    const float up = __uint_as_float((uint32_t)(127 + e) << 23), dn = __uint_as_float((uint32_t)(127 - e) << 23);
+    const float xs = v[t] * up;
+    const _Float16 h1 = (_Float16)xs, h2 = (_Float16)((xs - (float)h1) * 2048.0f);
+    if (2 * t < R) { o[(2 * t) * 8] = __builtin_bit_cast(unsigned short, h1); o[(2 * t + 1) * 8] = __builtin_bit_cast(unsigned short, h2); }
+    if (i == 0) ainv[sb * 8 + t] = t < T ? dn : 0.0f;
+  }
+}
+
+int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv) {
+  ProfScope ps(ctx, "act_split_f16", 4.0 * t * cols + (double)pyre_aop_bytes(cols, t));
+  hipLaunchKernelGGL(k_act_split, dim3(cols / 256), dim3(256), 0, ctx->stream, x_dev, t, pyre_aop_rows(t), cols, (uint16_t*)op, ainv);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+
+// ---- the product -----------------------------------------------------------------------------------------------------------------
+struct ChunkRaw { uint4 w[4]; uint2 h[4]; uint4 a[4]; float ai0, ai1; };
+
+__device__ __forceinline__ ChunkRaw chunk_load(const QMatDev& m, const uint4* __restrict__ aop, const float* __restrict__ ainv, int R, int tile, int c, int lane, int K128) {
+  ChunkRaw r;
+  const bool live = (lane & 15) < R;         // operand rows the window does not have are zero
+#pragma unroll
+  for (int s = 0; s < 4; ++s) r.a[s] = live ? aop[(((size_t)c * 4 + s) * 4 + (lane >> 4)) * R + (lane & 15)] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const size_t rg = (size_t)tile * 4 + g;
+    r.w[g] = ((const uint4*)m.mq)[(rg * K128 + c) * 64 + lane];
+    r.h[g] = ((const uint2*)m.mh)[(rg * m.SB + (c >> 1)) * 16 + (lane & 15)];
+  }
+  r.ai0 = 1.0f; r.ai1 = 1.0f;
+  if (ainv) { const float2 p = ((const float2*)ainv)[(c >> 1) * 4 + (lane >> 4)]; r.ai0 = p.x; r.ai1 = p.y; }
+  return r;
+}
+
+// tot[g] += (this chunk's 128 columns of row group g) x (the sixteen activation rows), scaled
+__device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const uint2* __restrict__ sctab, v4f (&tot)[4]) {
+  const int sh = 16 * (c & 1);               // the chunk's four sub-block scales: nibbles 4 (c & 1) .. + 3 of the header's scale word
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t wd[4] = {r.w[g].x, r.w[g].y, r.w[g].z, r.w[g].w};
+    const uint32_t a4[4][4] = {{r.a[0].x, r.a[0].y, r.a[0].z, r.a[0].w}, {r.a[1].x, r.a[1].y, r.a[1].z, r.a[1].w}, {r.a[2].x, r.a[2].y, r.a[2].z, r.a[2].w}, {r.a[3].x, r.a[3].y, r.a[3].z, r.a[3].w}};
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint32_t n = (r.h[g].y >> (sh + 4 * s)) & 0xFu;
+      const uint2 sc = sctab[n];
+      const v2h vs2 = __builtin_bit_cast(v2h, sc.x), vs47 = __builtin_bit_cast(v2h, sc.y);
+      const uint32_t u = wd[s], K = 0x03C003C0u, E = 0x4C004C00u;
+      const uint32_t p[4] = {((u << 6) & K) | E, ((u << 2) & K) | E, ((u >> 2) & K) | E, ((u >> 6) & K) | E};
+      uint32_t q[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) q[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(v2h, p[i]), vs2, vs47));
+      struct U4 { uint32_t x[4]; };
+      const v8h B = __builtin_bit_cast(v8h, (U4{{q[0], q[1], q[2], q[3]}}));
+      const v8h A = __builtin_bit_cast(v8h, (U4{{a4[s][0], a4[s][1], a4[s][2], a4[s][3]}}));
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, acc, 0, 0, 0);
+    }
+    const float d = h2f_bits(r.h[g].x & 0xFFFFu);
+    const float d0 = d * r.ai0, d1 = d * r.ai1;
+    tot[g][0] = fmaf(acc[0], d0, tot[g][0]); tot[g][1] = fmaf(acc[1], d0, tot[g][1]);
+    tot[g][2] = fmaf(acc[2], d1, tot[g][2]); tot[g][3] = fmaf(acc[3], d1, tot[g][3]);
+  }
+}
+
+//   ksplit == 1: y[t*rows + row] = sum.
+//   ksplit  > 1: y is a partial buffer, y[(ks*T + t)*tiles*64 + row] = slice sum (the consumer adds the slices in order).
+//   ep.best (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
+//   ep.co: conv1d + SiLU of the leading ep.ch rows (linear_core, qwen4exp_gguf.rs:1643-1647), as in the lane = row GEMV.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
+  __shared__ float red[NW][4][2][64];
+  __shared__ uint2 sctab[16];                 // scale nibble n -> packed f16 pairs (2s, 2s) and (-47s, -47s), s = 2n + 1
+  if (threadIdx.x < 16) {
+    const uint32_t a = __builtin_bit_cast(unsigned short, (_Float16)(float)(4 * (int)threadIdx.x + 2)), b = __builtin_bit_cast(unsigned short, (_Float16)(-47.0f * (float)(2 * (int)threadIdx.x + 1)));
+    sctab[threadIdx.x] = uint2{a | (a << 16), b | (b << 16)};
+  }
+  const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int K128 = m.cols >> 7;
+  float cw[8], chist[8]; const bool conv_row = ep.co != nullptr && wave == 0 && tile * 64 + lane < ep.ch;
+  if (conv_row) {
+    const size_t row = (size_t)tile * 64 + lane;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { cw[k] = k < ep.kk ? ep.conv_w[row * ep.kk + k] : 0.0f; chist[k] = k < ep.kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
+  }
+  const int c0 = (ks * NW + wave) * cpw, c1 = min(K128, c0 + cpw);
+  v4f tot[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane, no look-ahead
+    ChunkRaw cur;
+    if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
+    lds_barrier();                            // the scale table; the chunk's loads stay in flight
+    for (int c = c0; c < c1; ++c) {
+      if (c > c0) cur = chunk_load(m, aop, ainv, R, tile, c, lane, K128);
+      chunk_mac(cur, c, sctab, tot);
+    }
+  } else {
+    ChunkRaw cur;
+    if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
+    lds_barrier();
+    for (int c = c0; c < c1; ++c) {
+      const int cn = c + 1 < c1 ? c + 1 : c;
+      ChunkRaw nxt = chunk_load(m, aop, ainv, R, tile, cn, lane, K128);
+      chunk_mac(cur, c, sctab, tot);
+      cur = nxt;
+    }
+  }
+  // lane (q, j) holds, for row group g, token 2q (rows 0, 1 of its four) and token 2q + 1 (rows 2, 3): halves h1, h2 * 2^11
+#pragma unroll
+  for (int g = 0; g < 4; ++g) { red[wave][g][0][lane] = tot[g][0] + tot[g][1] * (1.0f / 2048.0f); red[wave][g][1][lane] = tot[g][2] + tot[g][3] * (1.0f / 2048.0f); }
+  lds_barrier();
+  auto rsum = [&](int t, int rl) { const int l = (t >> 1) * 16 + (rl & 15), g = rl >> 4, h = t & 1; float s = red[0][g][h][l];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) s += red[w][g][h][l];
+    return s; };
+  const size_t r64 = (size_t)m.tiles * 64;
+  for (int i = threadIdx.x; i < T * 64; i += NW * 64) {
+    const int t = i >> 6, l = i & 63; const float s = rsum(t, l);
+    const size_t row = (size_t)tile * 64 + l;
+    if (ksplit == 1) { if (row < (size_t)m.rows) y[(size_t)t * m.rows + row] = s; }
+    else y[((size_t)ks * T + t) * r64 + row] = s;
+    if (T == 1 && ep.best != nullptr) {       // threads 0..63 = wave 0: first maximum of the tile (sampler::argmax order)
+      float bv = row < (size_t)m.rows ? s : -INFINITY; uint32_t bi = (uint32_t)row;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; } }
+      if (l == 0) { ep.best[2 * tile] = __float_as_uint(bv); ep.best[2 * tile + 1] = bi; }
+    }
+  }
+  if (conv_row) {
+    const size_t row = (size_t)tile * 64 + lane;
+    for (int t = 0; t < T; ++t) {
+      const float cur = rsum(t, lane);
+      float o = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) if (k == ep.kk - 1) o = cw[k] * cur;
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) o += cw[k] * chist[k];
+      ep.co[(size_t)t * ep.ch + row] = o * (1.0f / (1.0f + expf(-o)));
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k + 1 < ep.kk - 1) chist[k] = chist[k + 1];
+#pragma unroll
+      for (int k = 0; k < 7; ++k) if (k == ep.kk - 2) chist[k] = cur;
+    }
+#pragma unroll
+    for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
+  }
+}
+
+namespace {
+int env_i(const char* n, int dflt) { const char* v = getenv(n); return v && *v ? atoi(v) : dflt; }
+int gemm_m_nw(const QMatDev& m, int ksplit) {
+  static const int force = env_i("PYRE_GEMM_M_NW", 0);
+  const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit;
+  int nw = m.tiles >= 1024 ? 4 : (m.tiles >= 256 ? 8 : 16);
+  while (nw > 1 && nw / 2 >= per_wg) nw /= 2;          // no idle waves
+  if (nw < 4) nw = 4;
+  if (force == 4 || force == 8 || force == 16) nw = force;
+  return nw;
+}
+template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep) {
+  hipLaunchKernelGGL((k_gemm_m<NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep);
+}
+}  // namespace
+
+void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* cpw) {
+  *nw = gemm_m_nw(m, ksplit);
+  const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit; *cpw = (per_wg + *nw - 1) / *nw; if (*cpw < 1) *cpw = 1;
+}
+
+int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, const GemvEpi& ep) {
+  if (m.fmt != FMT_IQ3_S_M || !m.mq || !m.mh) return pyre_fail(ctx, PYRE_E_TYPE, "gemm_m: the matrix is not held in the matrix-core layout");
+  if (t < 1 || t > 8 || ksplit < 1 || !a.op || !y) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: t = %d, %d K slices", t, ksplit);
+  if (m.cols % 256 != 0 || m.SB != m.cols / 256) return pyre_fail(ctx, PYRE_E_SHAPE, "gemm_m: %d columns", m.cols);
+  int nw, cpw; pyre_gemm_m_plan(m, ksplit, &nw, &cpw);
+  if (ep.four_waves) { nw = 4; const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit; cpw = (per_wg + 3) / 4; }
+  static const std::string names[9] = {"", "gemm_m_iq3s_t1", "gemm_m_iq3s_t2", "gemm_m_iq3s_t3", "gemm_m_iq3s_t4", "gemm_m_iq3s_t5", "gemm_m_iq3s_t6", "gemm_m_iq3s_t7", "gemm_m_iq3s_t8"};
+  ProfScope ps(ctx, names[t].c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * t * ((double)m.cols + m.rows));
+  if (nw == 4) gemm_m_go<4>(ctx, m, a, t, y, ksplit, cpw, ep);
+  else if (nw == 8) gemm_m_go<8>(ctx, m, a, t, y, ksplit, cpw, ep);
+  else gemm_m_go<16>(ctx, m, a, t, y, ksplit, cpw, ep);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+
+// ---- operand scratch: the context's grow-only buffer, and the fixed per-GPU array -------------------------------------------------
+int pyre_gemm_m_scratch(pyre_ctx* ctx, int cols, uint4** op, float** ainv) {
+  const size_t ob = (pyre_aop_bytes(cols, 8) + 255) & ~(size_t)255, need = ob + (size_t)(cols / 256) * 8 * 4;
+  if (ctx->aop_bytes < need) {
+    PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->aop_buf) (void)hipFree(ctx->aop_buf);
+    ctx->aop_buf = nullptr; ctx->aop_bytes = 0;
+    PYRE_HIP(ctx, hipMalloc(&ctx->aop_buf, need)); ctx->aop_bytes = need;
+  }
+  *op = (uint4*)ctx->aop_buf; *ainv = (float*)((uint8_t*)ctx->aop_buf + ob);
+  return PYRE_OK;
+}
+
+// The entry point that allocates nothing keeps its operand here: PYRE_QMATMUL_STATIC_MAX_COLS columns of operand rows
+// (32 bytes a column) and their scale factors.  One copy per GPU, held until the process ends; calls on one GPU share it.
+#define STATIC_MAX_COLS 32768
+#define STATIC_OP_BYTES ((size_t)STATIC_MAX_COLS * 32)
+static __device__ __align__(256) uint8_t scratch[STATIC_OP_BYTES + (STATIC_MAX_COLS / 256) * 8 * 4];
+static void* g_scratch_ptr[64];
+
+int pyre_static_init(pyre_ctx* ctx) {
+  if (ctx->device < 0 || ctx->device >= 64) return pyre_fail(ctx, PYRE_E_ARG, "device %d outside 0..63", ctx->device);
+  if (!g_scratch_ptr[ctx->device]) {
+    void* p = nullptr;
+    PYRE_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[ctx->device] = p;
+  }
+  ctx->aop_static = g_scratch_ptr[ctx->device];
+  return PYRE_OK;
+}
+
+int pyre_gemm_m_static(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev) {
+  if (m.cols > STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %d columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m.cols, STATIC_MAX_COLS);
+  if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
+  uint4* op = (uint4*)ctx->aop_static; float* ainv = (float*)((uint8_t*)ctx->aop_static + STATIC_OP_BYTES);
+  int rc = pyre_act_split_launch(ctx, x_dev, t, m.cols, op, ainv); if (rc) return rc;
+  return pyre_gemm_m_launch(ctx, m, PyreAop{op, ainv}, t, y_dev, 1, GemvEpi{});
+}

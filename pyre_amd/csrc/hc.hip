@@ -6,7 +6,6 @@
 // into the streams' RMS scales, adds the scaled slice sums, applies silu, runs the up GEMV from shared memory and
 // reduces the gated, normalized streams to their mean.
 #include "formats.h"
-#include "mega.h"
 #include <stdlib.h>
 #include <algorithm>
 
@@ -328,26 +327,6 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
   MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
   if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);
-  // PYRE_HC_FUSED=1 (single-token steps): both halves in one launch, separated by a barrier over the launch's own
-  // workgroups (same arithmetic, see mega.h).  Off by default: measured 2 us per mix slower than the two launches
-  // (4.48 vs 4.26 ms per token) -- the dependent memory round trips of a stage cost the same inside one kernel, and
-  // the barrier with its cache-bypassing hand-off costs more than the kernel boundary it replaces.
-  static const bool fused_ok = getenv("PYRE_HC_FUSED") && atoi(getenv("PYRE_HC_FUSED")) != 0;
-  if (t == 1 && fused_ok && !route && comb_parts == 1 && h.di.fmt == h.up.fmt && (h.di.fmt <= FMT_Q4_K || h.di.fmt == FMT_IQ3_S) && ctx->fuse_ctl) {
-    const int nwg = std::max(h.di.tiles * p.ksplit, h.d / 64), L = p.nw * p.upw * 64;
-    const size_t lds = 4 * std::max((size_t)L + (size_t)p.nw * 64 + p.nw, (size_t)h.lr + (size_t)h.hc * h.up.U * 64 + 32) + 64;
-    if (nwg <= 240 && lds <= 60000) {
-      mega::Comb cb{comb_out, mega::MoeOutC{mo.partial, mo.sel_w, mo.sg, mo.d, mo.k}, comb_inj};
-      mega::HcPlan pl{p.nw, p.upw, p.ksplit};
-      ProfScope ps(ctx, "hc_mix_fused", qmat_gguf_bytes(h.di, h.di.rows) + qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * h.hc * h.d * 4);
-      switch (h.di.fmt) {
-#define HC_FUSED_CASE(F) case F: hipLaunchKernelGGL((mega::k_hc_mix_fused<F>), dim3(nwg), dim3(mega::WGT), lds, ctx->stream, h, pl, x_in, in_ss, x_out, cb, eps, w.ssq, w.o, mixed, inj, ctx->fuse_ctl, 2000000u); break;
-        HC_FUSED_CASE(FMT_F32) HC_FUSED_CASE(FMT_F16) HC_FUSED_CASE(FMT_BF16) HC_FUSED_CASE(FMT_Q8_0) HC_FUSED_CASE(FMT_Q4_K) default: HC_FUSED_CASE(FMT_IQ3_S)
-#undef HC_FUSED_CASE
-      }
-      PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
-    }
-  }
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj, eps); if (rc) return rc;
   return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route);
 }

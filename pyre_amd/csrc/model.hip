@@ -3,7 +3,6 @@
 // greedy loop.  Follows Model::forward_inner / forward_multi / spec_keep (src/model/qwen4exp_gguf.rs:2087-2157,
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
-#include "mega.h"
 #include <memory>
 #include <stdlib.h>
 
@@ -31,8 +30,6 @@ struct pyre_model {
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
   float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr, *rpart = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
-  int mega_ok = -1;               // persistent-kernel decode: -1 not probed, 0 unsupported shape/types, 1 usable
-  std::vector<mega::Layer> mega_layers; mega::Args mega_args{}; mega::Layer* mega_dev = nullptr; unsigned* mega_ctl = nullptr; int mega_wgs = 0;
 };
 
 struct pyre_state {
@@ -54,7 +51,9 @@ struct Builder {
   int fail(int code, const char* what) { return pyre_fail(ctx, code, "pyre_model_create: %s", what); }
 
   // one matrix out of `n` row-concatenated tensors of one type and width
-  int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes) {
+  // layout: PYRE_LAYOUT_M for the matrices that only ever meet a GEMV or a row look-up (projections, head, embedding),
+  // PYRE_LAYOUT_ROWS for those the hyper-connection and MoE kernels walk themselves
+  int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS) {
     uint32_t ty = ts[0]->ggml_type; uint64_t cols = ts[0]->cols; uint32_t dev = ts[0]->on_device; uint64_t rows = 0; size_t total = 0;
     int fmt = fmt_from_ggml(ty); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported tensor type");
     struct { int el, bytes; } g{1, 4}; ggml_geom(ty, &g.el, &g.bytes);
@@ -64,18 +63,19 @@ struct Builder {
       rows += ts[i]->rows; total += ts[i]->rows * (cols / g.el * g.bytes);
     }
     pyre_qmat* q = nullptr; int rc;
-    if (n == 1) rc = dev ? pyre_qmat_create_dev(ctx, ty, rows, cols, ts[0]->data, total, &q) : pyre_qmat_create(ctx, ty, rows, cols, ts[0]->data, total, &q);
+    if (cols % 256) layout = PYRE_LAYOUT_ROWS;
+    if (n == 1) rc = pyre_qmat_create_layout(ctx, ty, rows, cols, ts[0]->data, dev != 0, total, layout, &q);
     else {
       void* tmp = nullptr; PYRE_HIP(ctx, hipMalloc(&tmp, total)); size_t off = 0;
       for (int i = 0; i < n; ++i) { size_t nb = ts[i]->rows * (cols / g.el * g.bytes);
         hipError_t e = hipMemcpy((uint8_t*)tmp + off, ts[i]->data, nb, dev ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
         if (e != hipSuccess) { (void)hipFree(tmp); return pyre_fail(ctx, PYRE_E_HIP, "pyre_model_create: copy: %s", hipGetErrorString(e)); } off += nb; }
-      rc = pyre_qmat_create_dev(ctx, ty, rows, cols, tmp, total, &q); (void)hipFree(tmp);
+      rc = pyre_qmat_create_layout(ctx, ty, rows, cols, tmp, true, total, layout, &q); (void)hipFree(tmp);
     }
     if (rc) return rc;
     m->owned.push_back(q); *out = q->dv; if (gguf_bytes) *gguf_bytes += total; return PYRE_OK;
   }
-  int one(const pyre_tensor& t, QMatDev* out, size_t* gguf_bytes) { const pyre_tensor* p = &t; return cat(&p, 1, out, gguf_bytes); }
+  int one(const pyre_tensor& t, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS) { const pyre_tensor* p = &t; return cat(&p, 1, out, gguf_bytes, layout); }
 
   // Gguf::vec: a small tensor fully dequantized to f32 on the device
   int vec(const pyre_tensor& t, size_t expect, const float** out) {
@@ -86,7 +86,7 @@ struct Builder {
     else {
       pyre_qmat* q = nullptr; int fmt = fmt_from_ggml(t.ggml_type); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported vector type"); struct { int el, bytes; } g{1, 4}; ggml_geom(t.ggml_type, &g.el, &g.bytes);
       size_t nb = n / g.el * g.bytes;
-      int rc = t.on_device ? pyre_qmat_create_dev(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q) : pyre_qmat_create(ctx, t.ggml_type, t.rows, t.cols, t.data, nb, &q); if (rc) return rc;
+      int rc = pyre_qmat_create_layout(ctx, t.ggml_type, t.rows, t.cols, t.data, t.on_device != 0, nb, PYRE_LAYOUT_ROWS, &q); if (rc) return rc;
       rc = pyre_qmat_dequant_dev(ctx, q, d); if (!rc) rc = pyre_ctx_sync(ctx); pyre_qmat_destroy(q); if (rc) return rc;
     }
     *out = d; return PYRE_OK;
@@ -129,6 +129,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   PYRE_HIP(ctx, hipMalloc((void**)&m->rope_inv, (inv.size() + 1) * 4)); m->bufs.push_back(m->rope_inv);
   PYRE_HIP(ctx, hipMemcpy(m->rope_inv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice)); m->mscale = mscale;
   size_t tok_bytes = 0; int rc;
+  const int mlay = [] { const char* e = getenv("PYRE_MODEL_ROWS"); return e && *e && atoi(e) != 0; }() ? PYRE_LAYOUT_ROWS : PYRE_LAYOUT_M;      // 1: every matrix in the lane = row layout
   m->layers.resize(c.n_layers);
   for (int il = 0; il < c.n_layers; ++il) {
     const pyre_tensor* T = lt + (size_t)il * PYRE_LAYER_SLOTS; Layer& L = m->layers[il];
@@ -141,9 +142,9 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
       if (grp[0]->rows != (uint64_t)c.n_head * 2 * c.hd || grp[1]->rows != (uint64_t)c.n_kv * c.hd || grp[2]->rows != (uint64_t)c.n_kv * c.hd || grp[0]->cols != (uint64_t)c.d)
         return B.fail(PYRE_E_SHAPE, "attention projection shapes");
       if (m->has_idx && (!grp[3]->data || !grp[4]->data || grp[3]->rows != (uint64_t)c.idx_nh * c.idx_hd || grp[4]->rows != (uint64_t)c.idx_hd)) return B.fail(PYRE_E_SHAPE, "indexer projection shapes (every attention layer needs them)");
-      if ((rc = B.cat(grp, m->has_idx ? 5 : 3, &L.proj, &tok_bytes))) return rc;
+      if ((rc = B.cat(grp, m->has_idx ? 5 : 3, &L.proj, &tok_bytes, mlay))) return rc;
       if (T[PYRE_T_ATTN_OUTPUT].rows != (uint64_t)c.d || T[PYRE_T_ATTN_OUTPUT].cols != (uint64_t)c.n_head * c.hd) return B.fail(PYRE_E_SHAPE, "attn_output shape");
-      if ((rc = B.one(T[PYRE_T_ATTN_OUTPUT], &L.outp, &tok_bytes))) return rc;
+      if ((rc = B.one(T[PYRE_T_ATTN_OUTPUT], &L.outp, &tok_bytes, mlay))) return rc;
       L.attn = AttnDev{nullptr, nullptr, m->rope_inv, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps, mscale};
       if ((rc = B.vec(T[PYRE_T_ATTN_Q_NORM], c.hd, &L.attn.qn)) || (rc = B.vec(T[PYRE_T_ATTN_K_NORM], c.hd, &L.attn.kn))) return rc;
       if (m->has_idx) {
@@ -155,9 +156,9 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
       const pyre_tensor* grp[4] = {&T[PYRE_T_ATTN_QKV], &T[PYRE_T_ATTN_GATE], &T[PYRE_T_SSM_BETA], &T[PYRE_T_SSM_ALPHA]};
       if (grp[0]->rows != (uint64_t)m->ch || grp[1]->rows != (uint64_t)c.lin_nv * c.lin_dv || grp[2]->rows != (uint64_t)c.lin_nv || grp[3]->rows != (uint64_t)c.lin_nv || grp[0]->cols != (uint64_t)c.d)
         return B.fail(PYRE_E_SHAPE, "DeltaNet projection shapes");
-      if ((rc = B.cat(grp, 4, &L.proj, &tok_bytes))) return rc;
+      if ((rc = B.cat(grp, 4, &L.proj, &tok_bytes, mlay))) return rc;
       if (T[PYRE_T_SSM_OUT].rows != (uint64_t)c.d || T[PYRE_T_SSM_OUT].cols != (uint64_t)c.lin_nv * c.lin_dv) return B.fail(PYRE_E_SHAPE, "ssm_out shape");
-      if ((rc = B.one(T[PYRE_T_SSM_OUT], &L.outp, &tok_bytes))) return rc;
+      if ((rc = B.one(T[PYRE_T_SSM_OUT], &L.outp, &tok_bytes, mlay))) return rc;
       L.gdn = GdnDev{nullptr, nullptr, nullptr, nullptr, c.lin_nk, c.lin_nv, c.lin_dk, c.lin_dv, c.conv_k, c.eps};
       if ((rc = B.vec(T[PYRE_T_SSM_A], c.lin_nv, &L.gdn.a)) || (rc = B.vec(T[PYRE_T_SSM_DT_BIAS], c.lin_nv, &L.gdn.dt)) ||
           (rc = B.vec(T[PYRE_T_SSM_CONV1D], (size_t)m->ch * c.conv_k, &L.gdn.conv_w)) || (rc = B.vec(T[PYRE_T_SSM_NORM], c.lin_dv, &L.gdn.norm_w))) return rc;
@@ -174,10 +175,10 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
     if ((rc = B.vec(T[PYRE_T_FFN_GATE_INP_SHEXP], c.d, &mo.sh_gate_inp))) return rc;
     tok_bytes += router_b + sh + (ge + ue + de) / c.n_exp * c.top_k;
   }
-  if ((rc = B.one(gl[PYRE_G_TOKEN_EMBD], &m->embd, nullptr))) return rc;
+  if ((rc = B.one(gl[PYRE_G_TOKEN_EMBD], &m->embd, nullptr, mlay))) return rc;
   if (m->embd.rows != c.vocab || m->embd.cols != c.d) return B.fail(PYRE_E_SHAPE, "token_embd shape");
   if ((rc = B.hc(gl[PYRE_G_OUTPUT_HC_NORM], gl[PYRE_G_OUTPUT_HC_DOWN], nullptr, gl[PYRE_G_OUTPUT_HC_UP], &m->head, &tok_bytes))) return rc;
-  if ((rc = B.one(gl[PYRE_G_OUTPUT], &m->out, &tok_bytes))) return rc;
+  if ((rc = B.one(gl[PYRE_G_OUTPUT], &m->out, &tok_bytes, mlay))) return rc;
   if (m->out.rows != c.vocab || m->out.cols != c.d) return B.fail(PYRE_E_SHAPE, "output shape");
   tok_bytes += (size_t)c.d / m->embd.gel * m->embd.gbytes;
   m->token_weight_bytes = tok_bytes;
@@ -196,6 +197,8 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
   m->rpart = (float*)take(rp_b);
+  { uint4* op; float* ainv; int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));      // the operand buffer of the widest GEMV input, so that no step allocates
+    if ((rc = pyre_gemm_m_scratch(ctx, (kmax + 255) / 256 * 256, &op, &ainv))) return rc; }
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   guard.armed = false; *out = M.release(); return PYRE_OK;
 }
@@ -203,7 +206,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
 void pyre_model_destroy(pyre_model* m) {
   if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
   for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); if (m->toks) (void)hipFree(m->toks);
-  if (m->mega_dev) (void)hipFree(m->mega_dev); if (m->mega_ctl) (void)hipFree(m->mega_ctl); delete m;
+  delete m;
 }
 size_t pyre_model_weight_bytes_per_token(const pyre_model* m) { return m ? m->token_weight_bytes : 0; }
 
@@ -393,83 +396,6 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
 }
 
-// ---- persistent-kernel decode (mega.h) ------------------------------------------------------------------------------------
-// Usable when every matrix but the router is IQ3_S, the router is bf16, and the shapes fit the kernel's stages; anything
-// else keeps the launch-per-stage path.
-bool mega_probe(pyre_ctx* ctx, pyre_model* m) {
-  if (m->has_idx || m->mscale != 1.0f) return false;        // the persistent kernel has neither the indexer nor the YaRN factor
-  if (m->mega_ok >= 0) return m->mega_ok == 1;
-  m->mega_ok = 0;
-  const pyre_model_cfg& c = m->c;
-  auto w_ok = [](const QMatDev& q) { return q.fmt == FMT_IQ3_S; };
-  auto hc_ok = [&](const HcDev& h, mega::HcPlan* p) { return w_ok(h.di) && w_ok(h.up) && pyre_hc_plan(h, &p->nw, &p->upw, &p->ksplit); };
-  if (c.top_k > PYRE_MOE_KMAX || c.hd != 256 || c.lin_dk != 128 || c.lin_dv != 128 || c.conv_k < 2 || c.conv_k > 8 || c.n_exp > 1024) return false;
-  if (!w_ok(m->embd) || !w_ok(m->out)) return false;
-  mega::Args& a = m->mega_args; a = mega::Args{};
-  if (!hc_ok(m->head, &a.ph)) return false;
-  m->mega_layers.assign(c.n_layers, mega::Layer{});
-  for (int il = 0; il < c.n_layers; ++il) {
-    const Layer& L = m->layers[il]; mega::Layer& M = m->mega_layers[il];
-    if (!hc_ok(L.hca, &M.pa) || !hc_ok(L.hcf, &M.pf) || !w_ok(L.proj) || !w_ok(L.outp)) return false;
-    const MoeDev& mo = L.moe;
-    if (mo.router.fmt != FMT_BF16 || !w_ok(mo.gate_e) || !w_ok(mo.up_e) || !w_ok(mo.down_e) || !w_ok(mo.sh_gate) || !w_ok(mo.sh_up) || !w_ok(mo.sh_down)) return false;
-    if (L.full) { int G = L.attn.nh / L.attn.nkv; if (L.attn.nh % L.attn.nkv || (G != 1 && G != 2 && G != 4 && G != 8)) return false; }
-    else if (L.gdn.nv % L.gdn.nk) return false;
-    if ((size_t)L.proj.cols * 4 + 4096 > mega::LDS_BYTES || (size_t)L.outp.cols * 4 + 4096 > mega::LDS_BYTES) return false;
-    M.hca = L.hca; M.hcf = L.hcf; M.proj = L.proj; M.outp = L.outp; M.moe = L.moe; M.attn = L.attn; M.gdn = L.gdn; M.full = L.full ? 1 : 0; M.gu_parts = pyre_moe_gu_parts(L.moe);
-    pyre_gemv_plan(L.proj, &M.gp.nw, &M.gp.upw); pyre_gemv_plan(L.outp, &M.go.nw, &M.go.upw); M.go.grp = outp_in_parts(L, c.d) ? M.go.nw / PYRE_GEMV_PARTS : 0; pyre_gemv_plan(mo.router, &M.gr.nw, &M.gr.upw);
-  }
-  if ((size_t)c.d * 4 + 2 * 8192 + sizeof(mega::RouteLds) > mega::LDS_BYTES) return false;
-  hipDeviceProp_t prop; if (hipGetDeviceProperties(&prop, ctx->device) != hipSuccess) return false;
-  int wgs = prop.multiProcessorCount; if (wgs > 256) wgs = 256; if (wgs < 32) return false;
-  int per_cu = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)mega::k_decode<FMT_IQ3_S, FMT_BF16>, mega::WGT, mega::LDS_BYTES) != hipSuccess || per_cu < 1) return false;
-  if (hipMalloc((void**)&m->mega_dev, sizeof(mega::Layer) * c.n_layers) != hipSuccess) return false;
-  if (hipMalloc((void**)&m->mega_ctl, 4096) != hipSuccess) return false;
-  m->mega_wgs = wgs;
-  a.n_layers = c.n_layers; a.head = m->head; a.embd = m->embd; a.out = m->out; pyre_gemv_plan(m->out, &a.gh.nw, &a.gh.upw);
-  a.d = c.d; a.hc = c.hc; a.ch = m->ch; a.pw_lin = m->pw_lin; a.pw_attn = m->pw_attn; a.conv_k = c.conv_k; a.eps = c.eps;
-  a.emb = m->emb; a.xa = m->x; a.xb = m->x2; a.ssq = m->hw.ssq; a.part = m->hw.o; a.mixed = m->mixed; a.inj_a = m->inj_a; a.inj_f = m->inj_f; a.proj = m->proj; a.co = m->co; a.core = m->core;
-  a.o = m->o; a.hbuf = m->hbuf; a.vlogits = m->logits; a.best = m->best; a.mw = m->mw; a.ctl = m->mega_ctl; a.limit = 4000000u;
-  m->mega_ok = 1; return true;
-}
-
-int mega_decode(pyre_ctx* ctx, pyre_model* m, pyre_state* s, uint32_t first, int n_steps) {
-  // per-state pointers: recurrent state in place in the current buffers, KV caches, raw-projection rows
-  int li = 0, ai = 0;
-  for (int il = 0; il < m->c.n_layers; ++il) {
-    mega::Layer& M = m->mega_layers[il];
-    if (M.full) { M.kv = s->kv[ai]; ++ai; }
-    else { M.conv = s->conv[s->cur[li]][li]; M.ssm = s->ssm[s->cur[li]][li]; M.proj_saved = s->proj_saved[li]; ++li; }
-  }
-  PYRE_HIP(ctx, hipMemcpyAsync(m->mega_dev, m->mega_layers.data(), sizeof(mega::Layer) * m->mega_layers.size(), hipMemcpyHostToDevice, ctx->stream));
-  const int chunk = 256;                       // tokens per launch
-  for (int done = 0; done < n_steps; done += chunk) {
-    int n = n_steps - done < chunk ? n_steps - done : chunk;
-    mega::Args a = m->mega_args; a.layers = m->mega_dev; a.aw = s->aw; a.toks = m->toks + done; a.n_steps = n; a.start_pos = s->len + done;
-    a.first = first;
-    if (done > 0) {   // continue from the previous launch's last pick
-      PYRE_HIP(ctx, hipMemcpyAsync(&a.first, m->toks + done - 1, 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    }
-    PYRE_HIP(ctx, hipMemsetAsync(m->mega_ctl, 0, 4096, ctx->stream));
-    { const char* e = getenv("PYRE_MEGA_TIMES"); a.stage_ticks = e && atoi(e) ? (unsigned long long*)(m->mega_ctl + 512) : nullptr; }
-    void* args[] = {&a};
-    { ProfScope ps(ctx, "decode_persistent", 0.0);
-      PYRE_HIP(ctx, hipLaunchCooperativeKernel((const void*)mega::k_decode<FMT_IQ3_S, FMT_BF16>, dim3(m->mega_wgs), dim3(mega::WGT), args, mega::LDS_BYTES, ctx->stream)); }
-    unsigned flags[32];
-    PYRE_HIP(ctx, hipMemcpyAsync(flags, m->mega_ctl, sizeof(flags), hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    if (a.stage_ticks) {
-      unsigned long long tk[16]; PYRE_HIP(ctx, hipMemcpy(tk, a.stage_ticks, sizeof(tk), hipMemcpyDeviceToHost));
-      static const char* nm[13] = {"pick_embed", "hc_norm_down", "hc_up_mix", "proj_gemv", "attn_prep", "attn_decode", "attn_combine", "gdn_delta", "out_gemv", "router_gemv", "route_gate_up", "moe_down", "head_gemv"};
-      fprintf(stderr, "[pyre] persistent decode, %d tokens, us per token by stage class (incl. the barrier after it):\n", n);
-      double tot = 0; for (int i = 0; i < 13; ++i) { double us = tk[i] * 0.01 / n; tot += us; fprintf(stderr, "[pyre]   %-14s %9.1f\n", nm[i], us); }
-      fprintf(stderr, "[pyre]   %-14s %9.1f\n", "total", tot);
-    }
-    if (flags[16]) return pyre_fail(ctx, PYRE_E_HIP, "pyre_decode_greedy_dev: the persistent kernel gave up waiting at barrier round %u", flags[0]);
-  }
-  return PYRE_OK;
-}
-
 int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
   for (int i = 0; i < n; ++i) if (ids[i] >= (uint32_t)m->c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "forward: token id %u outside the vocabulary (%d)", ids[i], m->c.vocab);
   return PYRE_OK;
@@ -492,7 +418,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     if ((rc = run_window(ctx, m, s, t, o))) return rc;
   }
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
-  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
 int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host) {
@@ -505,7 +431,7 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
   s->last_window = n;
   PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)n * m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
-  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
 // First maximum of each of t logit rows (sampler::argmax, src/sampler.rs:142-148: a scan from index 0 with strict >, so the
@@ -536,7 +462,7 @@ static int forward_multi_picks(pyre_ctx* ctx, const pyre_model* m, pyre_state* s
   hipLaunchKernelGGL(k_argmax_rows, dim3(n), dim3(1024), 0, ctx->stream, m->logits, m->c.vocab, m->best);
   PYRE_CHECK_LAUNCH(ctx);
   PYRE_HIP(ctx, hipMemcpyAsync(picks_host, m->best, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
-  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx);
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
 // The DeltaNet layers kept the window's inputs and their pre-window state (the other half of the double buffer): the
@@ -565,19 +491,10 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
   int rc = check_ids(ctx, m, &first, 1); if (rc) return rc;
   if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }
   s->last_window = 0;
-  { const char* e = getenv("PYRE_MEGA"); const int want = e && *e ? atoi(e) : 0;      // 1: use it when the model qualifies, 2: fail if it does not
-    if (want == 2 && !mega_probe(ctx, m)) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_decode_greedy_dev: the persistent decode kernel does not support this model (types or shapes)");
-    if (want && !ctx->prof_on && mega_probe(ctx, m)) {
-      if ((rc = mega_decode(ctx, m, s, first, n_steps))) return rc;
-      s->len += n_steps;
-      for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
-      if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
-      return PYRE_OK;
-    } }
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, &first, 4, hipMemcpyHostToDevice, ctx->stream));
   { WinOpt o; o.greedy = true; o.inplace = true; if ((rc = run_window(ctx, m, s, 1, o))) return rc; }     // in place: the captured step below keeps pointing at the current buffers
   if (n_steps > 1) {
-    static const bool no_graph = getenv("PYRE_NO_GRAPH") && atoi(getenv("PYRE_NO_GRAPH")) != 0;
+    const bool no_graph = getenv("PYRE_NO_GRAPH") && atoi(getenv("PYRE_NO_GRAPH")) != 0;          // read per call (tests switch it)
     int step_host[2] = {s->len - 1, s->len};      // the pick increments [0] to the position it starts; slot = [0] - [1]
     PYRE_HIP(ctx, hipMemcpyAsync(s->step_dev, step_host, 8, hipMemcpyHostToDevice, ctx->stream));
     WinOpt o; o.greedy = true; o.from_best = true; o.toks_out = m->toks; o.step_dev = s->step_dev;
@@ -602,7 +519,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
     for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
   }
   if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr, nullptr))) return rc;
-  if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return pyre_fuse_check(ctx); }
+  if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK; }
   return PYRE_OK;
 }
 

@@ -157,6 +157,28 @@ __global__ void k_repack(QMatDev m, const uint8_t* __restrict__ raw, size_t row_
   }
 }
 
+// IQ3_S into the matrix-core layout (QMatDev::mq / mh): one thread per (row of the padded row groups, super-block).
+__global__ __launch_bounds__(256) void k_repack_m(int rows, int rows_pad, int SB, const uint8_t* __restrict__ raw, size_t row_bytes, uint32_t* __restrict__ mq, uint2* __restrict__ mh, const uint32_t* __restrict__ g3) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; if (idx >= (size_t)rows_pad * SB) return;
+  const int row = (int)(idx / SB), sb = (int)(idx % SB); const bool live = row < rows;      // padding rows lie past the end of the raw buffer: never read them
+  const size_t rg = (size_t)(row >> 4); const int j = row & 15; const size_t K128 = (size_t)SB * 2;
+  const uint8_t* b = raw + (size_t)row * row_bytes + (size_t)sb * 110;
+  for (int ib = 0; ib < 8; ++ib) {               // sub-block ib: 32 values = step ib & 3 of 128-column chunk 2 sb + ib / 4
+    const uint32_t h = live ? b[66 + ib] : 0;
+    for (int l = 0; l < 4; ++l) {                // eight consecutive values = the share of lane group l
+      uint32_t wd = 0;
+      if (live) {
+        const uint32_t gA = g3[b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256)], gB = g3[b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256)], sg = b[74 + 4 * ib + l];
+        for (int e = 0; e < 8; ++e) { const uint32_t gb = ((e < 4 ? gA : gB) >> (8 * (e & 3))) & 0xFF; wd |= iq3s_code(gb, (sg >> e) & 1) << (4 * ((e >> 1) + 4 * (e & 1))); }
+      }
+      mq[((rg * K128 + 2 * sb + (ib >> 2)) * 64 + l * 16 + j) * 4 + (ib & 3)] = wd;
+    }
+  }
+  uint2 hd{0u, 0u};
+  if (live) { hd.x = (uint32_t)b[0] | ((uint32_t)b[1] << 8); hd.y = (uint32_t)b[106] | ((uint32_t)b[107] << 8) | ((uint32_t)b[108] << 16) | ((uint32_t)b[109] << 24); }
+  mh[(rg * SB + sb) * 16 + j] = hd;
+}
+
 // ---- bit-exact dequant export -----------------------------------------------------------------------------------------
 // grid (U, tiles), 64 threads: lane l decodes unit ku of row tile*64+l, the tile is transposed through LDS so that
 // each row's 64 values leave as one contiguous 256-byte store.
@@ -319,39 +341,60 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
     case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
     case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; \
     default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
+// the kernels that only decode (export, rows by index, the greedy pick) also read the matrix-core layout
+#define FMT_DISPATCH_X(fmt, CALL) \
+  switch (fmt) { case FMT_F32: { constexpr int F = FMT_F32; CALL; } break; case FMT_F16: { constexpr int F = FMT_F16; CALL; } break; case FMT_BF16: { constexpr int F = FMT_BF16; CALL; } break; \
+    case FMT_Q8_0: { constexpr int F = FMT_Q8_0; CALL; } break; case FMT_Q4_K: { constexpr int F = FMT_Q4_K; CALL; } break; case FMT_IQ2_XS: { constexpr int F = FMT_IQ2_XS; CALL; } break; \
+    case FMT_C4: { constexpr int F = FMT_C4; CALL; } break; case FMT_C8: { constexpr int F = FMT_C8; CALL; } break; case FMT_IQ3_S_M: { constexpr int F = FMT_IQ3_S_M; CALL; } break; \
+    default: { constexpr int F = FMT_IQ3_S; CALL; } break; }
+
+// A matrix in the matrix-core layout whose caller has no f16 operand at hand: the activations are split into the
+// context's operand buffer first (sized by pyre_gemm_m_scratch; grows only outside stream capture).
+int gemm_m_from_f32(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, const GemvEpi& ep, const PyreAop* a) {
+  if (a && a->op) return pyre_gemm_m_launch(ctx, m, *a, t, y, ksplit, ep);
+  uint4* op; float* ainv; int rc = pyre_gemm_m_scratch(ctx, m.cols, &op, &ainv); if (rc) return rc;
+  if ((rc = pyre_act_split_launch(ctx, x, t, m.cols, op, ainv))) return rc;
+  return pyre_gemm_m_launch(ctx, m, PyreAop{op, ainv}, t, y, ksplit, ep);
+}
 }  // namespace
 
 void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw) { *nw = gemv_nw(m, 1); *upw = (m.U + *nw - 1) / *nw; if (*upw < 1) *upw = 1; }
-int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y) {
+int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, const PyreAop* a) {
+  if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, y, 1, GemvEpi{}, a);
   int rc = PYRE_OK;
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, GemvEpi{}));
   return rc;
 }
-int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* partial, int ksplit) {
+int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* partial, int ksplit, const PyreAop* a) {
+  if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, partial, ksplit, GemvEpi{}, a);
   int rc = PYRE_OK;
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, partial, ksplit, GemvEpi{}));
   return rc;
 }
 bool pyre_gemv_parts_ok(const QMatDev& m) {
   static const int off = env_int("PYRE_GEMV_PARTS", 1) == 0;
+  if (m.fmt == FMT_IQ3_S_M) return !off && m.tiles <= 64 && m.cols % (128 * PYRE_GEMV_PARTS * 4) == 0 && m.rows == m.tiles * 64;
   return !off && m.tiles <= 64 && gemv_nw(m, 1) == 16 && m.U % 16 == 0 && m.U / 16 >= 2 && m.rows == m.tiles * 64;
 }
-int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* parts) {
+int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* parts, const PyreAop* a) {
   if (!pyre_gemv_parts_ok(m)) return pyre_fail(ctx, PYRE_E_SHAPE, "gemv: the four-part form needs few row tiles and rows of a multiple of 32 units");
   int rc = PYRE_OK;
   GemvEpi ep{}; ep.four_waves = 1;
+  if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep, a);
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep));
   return rc;
 }
-int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best) {
+int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best, const PyreAop* a) {
   int rc = PYRE_OK;
   GemvEpi ep{}; ep.best = best;
+  if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, 1, y, 1, ep, a);
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, 1, y, 1, ep));
   return rc;
 }
-int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, const GemvEpi& conv) {
+int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, const GemvEpi& conv, const PyreAop* a) {
   if (!conv.co || !conv.conv_w || !conv.conv_in || !conv.conv_out || conv.kk < 2 || conv.kk > 8 || conv.ch < 1 || conv.ch > m.rows) return pyre_fail(ctx, PYRE_E_ARG, "gemv: bad conv epilogue (kernel %d, %d channels of %d rows)", conv.kk, conv.ch, m.rows);
   GemvEpi ep = conv; ep.best = nullptr; int rc = PYRE_OK;
+  if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, y, 1, ep, a);
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, ep));
   return rc;
 }
@@ -381,7 +424,7 @@ int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t*
   ProfScope ps(ctx, "pick_embed", 8.0 * n_tiles);
   if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step); }
   else { dim3 grid((m->U + 63) / 64);
-    FMT_DISPATCH(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step)); }
+    FMT_DISPATCH_X(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step)); }
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
@@ -389,11 +432,11 @@ int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* idx, int n,
   if (n <= 0) return PYRE_OK;
   dim3 grid((m.U + 63) / 64, n);
   ProfScope ps(ctx, "embed_rows", 0.0);
-  FMT_DISPATCH(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
+  FMT_DISPATCH_X(m.fmt, hipLaunchKernelGGL((k_rows<F>), grid, dim3(64), 0, ctx->stream, m, (const uint64_t*)ctx->d_iq2xs, idx, out, out_stride));
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
-static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, pyre_qmat** out) {
+int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, int layout, pyre_qmat** out) {
   if (!ctx || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: null argument");
   *out = nullptr;
   int fmt = fmt_from_ggml(ty); if (fmt < 0) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmat_create: unsupported ggml type %u", ty);
@@ -402,48 +445,73 @@ static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t co
   if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
   size_t row_bytes = cols / gel * gbytes;
   if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
+  if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // only IQ3_S has a matrix-core layout
+  const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
   pyre_qmat* m = new pyre_qmat(); m->ctx = ctx; m->ty = ty; m->rows = rows; m->cols = cols; m->gguf_bytes = nbytes;
+  auto drop = [&]() { if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); delete m; };
   int U = (int)(cols / PYRE_UNIT), tiles = (int)((rows + 63) / 64);
   size_t ent = (size_t)tiles * U * 64;
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
-  size_t s0 = al(ent * g.V * 16), s1 = al(ent * g.e1), s2 = al(ent * g.e2), s3 = al(ent * g.e3), sb = al(ent / 4 * g.eb + 256);
-  m->dev_bytes = s0 + s1 + s2 + s3 + sb;
-  hipError_t e = hipMalloc(&m->base, m->dev_bytes);
-  if (e != hipSuccess) { delete m; return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", s0 + s1 + s2 + s3 + sb, hipGetErrorString(e)); }
-  uint8_t* b = (uint8_t*)m->base;
-  m->dv = QMatDev{b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (int)rows, (int)cols, U, tiles, fmt, ty, gel, gbytes, {0, 0, 0, 0}, 0};
-  if (fmt == FMT_C4) c4_table(ty, m->dv.lut, &m->dv.bias);
-  const uint8_t* src = (const uint8_t*)blocks; void* tmp = nullptr;
+  const uint8_t* src = (const uint8_t*)blocks; void* tmp = nullptr; hipError_t e = hipSuccess;
   if (!on_device) {
     e = hipMalloc(&tmp, nbytes);
     if (e == hipSuccess) e = hipMemcpyAsync(tmp, blocks, nbytes, hipMemcpyHostToDevice, ctx->stream);
-    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); (void)hipFree(m->base); delete m; return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: upload failed: %s", hipGetErrorString(e)); }
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: upload failed: %s", hipGetErrorString(e)); }
     src = (const uint8_t*)tmp;
   }
-  size_t total = ent * 1; unsigned nblk = (unsigned)((total + 255) / 256);
-  hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (const uint32_t*)ctx->d_iq3s, (const uint16_t*)ctx->d_cb);
-  e = hipGetLastError();
+  const QMatDev shape{nullptr, nullptr, nullptr, nullptr, nullptr, (int)rows, (int)cols, U, tiles, fmt, ty, gel, gbytes, {0, 0, 0, 0}, 0, nullptr, nullptr, 0};
+  if (want_rows) {
+    size_t s0 = al(ent * g.V * 16), s1 = al(ent * g.e1), s2 = al(ent * g.e2), s3 = al(ent * g.e3), sb = al(ent / 4 * g.eb + 256);
+    m->dev_bytes = s0 + s1 + s2 + s3 + sb;
+    e = hipMalloc(&m->base, m->dev_bytes);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", s0 + s1 + s2 + s3 + sb, hipGetErrorString(e)); }
+    uint8_t* b = (uint8_t*)m->base;
+    m->dv = shape; m->dv.p0 = b; m->dv.p1 = b + s0; m->dv.p2 = b + s0 + s1; m->dv.p3 = b + s0 + s1 + s2; m->dv.pb = b + s0 + s1 + s2 + s3;
+    if (fmt == FMT_C4) c4_table(ty, m->dv.lut, &m->dv.bias);
+    size_t total = ent * 1; unsigned nblk = (unsigned)((total + 255) / 256);
+    hipLaunchKernelGGL(k_repack, dim3(nblk), dim3(256), 0, ctx->stream, m->dv, src, row_bytes, b, b + s0, b + s0 + s1, b + s0 + s1 + s2, b + s0 + s1 + s2 + s3, (const uint32_t*)ctx->d_iq3s, (const uint16_t*)ctx->d_cb);
+    e = hipGetLastError();
+  }
+  if (want_m && e == hipSuccess) {
+    if (cols % 256) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: IQ3_S rows are whole super-blocks of 256 columns, got %zu", cols); }
+    const int SB = (int)(cols / 256); const size_t rows_pad = (size_t)tiles * 64;
+    const size_t sq = al(rows_pad * cols / 2), sh = al(rows_pad * SB * 8);
+    m->dev_bytes_m = sq + sh;
+    e = hipMalloc(&m->base_m, m->dev_bytes_m);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", sq + sh, hipGetErrorString(e)); }
+    uint8_t* b = (uint8_t*)m->base_m;
+    m->dvm = shape; m->dvm.fmt = FMT_IQ3_S_M; m->dvm.mq = b; m->dvm.mh = b + sq; m->dvm.SB = SB;
+    const size_t total = rows_pad * SB;
+    hipLaunchKernelGGL(k_repack_m, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, src, row_bytes, (uint32_t*)b, (uint2*)(b + sq), (const uint32_t*)ctx->d_iq3s);
+    e = hipGetLastError();
+    if (!want_rows) m->dv = m->dvm;         // the only layout the matrix has is the one every user sees
+  }
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (tmp) (void)hipFree(tmp);
-  if (e != hipSuccess) { (void)hipFree(m->base); delete m; return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: repack failed: %s", hipGetErrorString(e)); }
+  if (e != hipSuccess) { drop(); return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: repack failed: %s", hipGetErrorString(e)); }
   *out = m; return PYRE_OK;
+}
+// the stand-alone operator keeps an IQ3_S matrix in both layouts: pyre_qmatmul runs on the matrix cores, pyre_qmatmul_f32
+// on the lane = row GEMV that the model's expert matrices use
+static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, pyre_qmat** out) {
+  return pyre_qmat_create_layout(ctx, ty, rows, cols, blocks, on_device, nbytes, PYRE_LAYOUT_BOTH, out);
 }
 
 extern "C" {
 
 int pyre_qmat_create(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* host_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, host_blocks, false, nbytes, out); }
 int pyre_qmat_create_dev(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* dev_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, dev_blocks, true, nbytes, out); }
-void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); (void)hipFree(m->base); delete m; }
+void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); delete m; }
 size_t pyre_qmat_rows(const pyre_qmat* m) { return m ? m->rows : 0; }
 size_t pyre_qmat_cols(const pyre_qmat* m) { return m ? m->cols : 0; }
 size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; }
-size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes : 0; }
+size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes + m->dev_bytes_m : 0; }
 
 int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
   if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");
   dim3 grid(m->dv.U, m->dv.tiles);
-  FMT_DISPATCH(m->dv.fmt, hipLaunchKernelGGL((k_dequant<F>), grid, dim3(64), 0, ctx->stream, m->dv, (const uint64_t*)ctx->d_iq2xs, out_dev));
+  FMT_DISPATCH_X(m->dv.fmt, hipLaunchKernelGGL((k_dequant<F>), grid, dim3(64), 0, ctx->stream, m->dv, (const uint64_t*)ctx->d_iq2xs, out_dev));
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 int pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host) {
@@ -463,22 +531,23 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
   void* st; int rc = pyre_stage(ctx, m->cols * sizeof(float) + 256, &st); if (rc) return rc;
   uint32_t r = (uint32_t)row; uint32_t* idx = (uint32_t*)((uint8_t*)st + m->cols * sizeof(float));
   PYRE_HIP(ctx, hipMemcpyAsync(idx, &r, 4, hipMemcpyHostToDevice, ctx->stream));
-  rc = pyre_row_launch(ctx, m->dv, idx, 1, (float*)st, (int)m->cols); if (rc) return rc;
+  rc = pyre_row_launch(ctx, m->dvm.mq ? m->dvm : m->dv, idx, 1, (float*)st, (int)m->cols); if (rc) return rc;      // a matrix held in both layouts: rows come from the matrix-core one, pyre_qmat_dequant from the other
   PYRE_HIP(ctx, hipMemcpyAsync(out_host, st, m->cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 
-// The operator's own launch: IQ3_S goes through the integer-dot GEMV (for every t, so a token's result does not depend
-// on the window width); f32_path (or PYRE_QMATMUL_F32=1) keeps the f32 lane = row GEMV the model's layers use.
-static int qmatmul_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, bool f32_path) {
+// The operator's own launch: an IQ3_S matrix goes through the matrix-core GEMM (for every t, so a token's result does not
+// depend on the window width); f32_path (or PYRE_QMATMUL_F32=1) takes the f32 lane = row GEMV the model's expert matrices use.
+static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev, bool f32_path) {
   static const int f32_only = env_int("PYRE_QMATMUL_F32", 0);
-  if (!f32_path && !f32_only && pyre_gemv_i8_ok(m, t)) return pyre_gemv_i8_launch(ctx, m, x_dev, t, y_dev, nullptr);
-  return pyre_gemv_launch(ctx, m, x_dev, t, y_dev);
+  const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
+  if (has_m && (!has_rows || (!f32_path && !f32_only))) return pyre_gemv_launch(ctx, m->dvm, x_dev, t, y_dev);
+  return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
 }
 static int qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev, bool f32_path) {
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: t = %d outside 1..8", t);
-  return qmatmul_launch(ctx, m->dv, x_dev, t, y_dev, f32_path);
+  return qmatmul_launch(ctx, m, x_dev, t, y_dev, f32_path);
 }
 static int qmatmul_host(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host, bool f32_path) {
   if (!ctx || !m || !x_host || !y_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul: null argument");
@@ -487,7 +556,7 @@ static int qmatmul_host(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, 
   void* st; int rc = pyre_stage(ctx, xo + yb, &st); if (rc) return rc;
   float* xd = (float*)st; float* yd = (float*)((uint8_t*)st + xo);
   PYRE_HIP(ctx, hipMemcpyAsync(xd, x_host, xb, hipMemcpyHostToDevice, ctx->stream));
-  rc = qmatmul_launch(ctx, m->dv, xd, t, yd, f32_path); if (rc) return rc;
+  rc = qmatmul_launch(ctx, m, xd, t, yd, f32_path); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(y_host, yd, yb, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
@@ -496,8 +565,18 @@ int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, 
 int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: t = %d outside 1..8", t);
-  if (m->dv.fmt != FMT_IQ3_S) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
-  return pyre_gemv_i8_static_launch(ctx, m->dv, x_dev, t, y_dev);
+  if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  return pyre_gemm_m_static(ctx, m->dvm, x_dev, t, y_dev);
+}
+// kept for callers written against the separate verify-window entry: since pyre_qmatmul itself runs on the matrix cores
+// for every window width, these are the same call restricted to IQ3_S
+int pyre_qmatmul_mfma_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
+  if (m && !(m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq)) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_mfma: IQ3_S matrices only");
+  return qmatmul_dev(ctx, m, x_dev, t, y_dev, false);
+}
+int pyre_qmatmul_mfma(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) {
+  if (m && !(m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq)) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_mfma: IQ3_S matrices only");
+  return qmatmul_host(ctx, m, x_host, t, y_host, false);
 }
 int pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, true); }
 int pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, true); }

@@ -48,7 +48,7 @@ def test_verify_window_equals_single_steps_and_rollback_at_full_width(model4):
     assert len(sa) == len(sc) == 40 and np.array_equal(la.view(np.uint32), lc.view(np.uint32))
 
 
-def test_device_loop_persistent_kernel_and_snapshot_agree_at_full_width(model4):
+def test_device_loop_host_loop_and_snapshot_agree_at_full_width(model4):
     cfg, gm = model4
     g = np.random.Generator(np.random.PCG64(4))
     prompt = g.integers(0, cfg.vocab, 21, dtype=np.uint32)
@@ -62,11 +62,11 @@ def test_device_loop_persistent_kernel_and_snapshot_agree_at_full_width(model4):
         lg = gm.forward(np.array([tok], dtype=np.uint32), st); tok = int(orc.argmax(lg)); host.append(tok)
     assert np.array_equal(a, np.array(host, dtype=np.uint32))
     st.restore(snap)
-    os.environ["PYRE_MEGA"] = "2"
+    os.environ["PYRE_NO_GRAPH"] = "1"                                         # the same step as ordinary launches instead of a replayed graph
     try:
         b = gm.decode_greedy_dev(st, first, 24)
     finally:
-        os.environ.pop("PYRE_MEGA", None)
+        os.environ.pop("PYRE_NO_GRAPH", None)
     assert np.array_equal(a, b)
 
 

@@ -31,10 +31,10 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_consecutive_cal
     big = lib.QMat(ctx, lib.IQ3_S, 4096, 4096, synth.matrix(lib.IQ3_S, 4096, 4096, 501))
     small = lib.QMat(ctx, lib.IQ3_S, 320, 512, synth.matrix(lib.IQ3_S, 320, 512, 502))
     xa = synth.normal((8, 4096), 503); xb = synth.normal((1, 512), 504)
-    a, b = both(ctx, big, 4096, 4096, xa)                  # first call: 8 tokens x 64 units of digits
+    a, b = both(ctx, big, 4096, 4096, xa)                  # first call: 4096 columns of sixteen operand rows
     assert np.isfinite(a).all() and np.abs(a).max() > 0
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
-    a, b = both(ctx, small, 320, 512, xb)                  # second call, smaller: the array still holds the first call's digits beyond its own
+    a, b = both(ctx, small, 320, 512, xb)                  # second call, smaller: the array still holds the first call's operand beyond its own
     assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
     a, b = both(ctx, big, 4096, 4096, xa[:3])              # and back to a larger one, another width
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
@@ -48,19 +48,20 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_consecutive_cal
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit_and_other_types(ctx):
-    rows, cols = 64, 65536                                 # 8 tokens x 1024 units = 8192 token-units > 4096
-    wide = lib.QMat(ctx, lib.IQ3_S, rows, cols, synth.matrix(lib.IQ3_S, rows, cols, 505))
-    xd = ctx.upload(synth.normal((8, cols), 506)); yd = ctx.alloc(8 * rows * 4)
-    with pytest.raises(lib.PyreError, match="static scratch"):
-        wide.matmul_static_dev(xd, 8, yd)
-    wide.matmul_static_dev(xd, 4, yd)                      # 4 x 1024 = 4096 token-units: exactly the limit
-    ya = ctx.alloc(4 * rows * 4); wide.matmul_dev(xd, 4, ya)
-    assert np.array_equal(ctx.download(yd, (4, rows)).view(np.uint32), ctx.download(ya, (4, rows)).view(np.uint32))
+    rows = 64
+    wide = lib.QMat(ctx, lib.IQ3_S, rows, 65536, synth.matrix(lib.IQ3_S, rows, 65536, 505))      # twice the 32 768 columns the array holds
+    edge = lib.QMat(ctx, lib.IQ3_S, rows, 32768, synth.matrix(lib.IQ3_S, rows, 32768, 508))      # exactly the limit
+    xd = ctx.upload(synth.normal((8, 65536), 506)); yd = ctx.alloc(8 * rows * 4); ya = ctx.alloc(8 * rows * 4)
+    for t in (1, 8):
+        with pytest.raises(lib.PyreError, match="static scratch"):
+            wide.matmul_static_dev(xd, t, yd)
+    edge.matmul_static_dev(xd, 8, yd); edge.matmul_dev(xd, 8, ya)
+    assert np.array_equal(ctx.download(yd, (8, rows)).view(np.uint32), ctx.download(ya, (8, rows)).view(np.uint32))
     with pytest.raises(lib.PyreError):
-        wide.matmul_static_dev(xd, 9, yd)
+        edge.matmul_static_dev(xd, 9, yd)
     q8 = lib.QMat(ctx, lib.Q8_0, 64, 256, synth.matrix(lib.Q8_0, 64, 256, 507))
     with pytest.raises(lib.PyreError, match="IQ3_S"):
         q8.matmul_static_dev(xd, 1, yd)
     for p in (xd, yd, ya):
         ctx.free(p)
-    wide.close(); q8.close()
+    wide.close(); edge.close(); q8.close()
