@@ -106,7 +106,7 @@ def bench_gemv(args):
     t = args.t
     if t > 1:
         x = ctx.upload(synth.normal((t, cols), 3)); y = ctx.alloc(t * rows * 4)
-    run = (lambda m: m.matmul_mfma_dev(x, t, y)) if args.mfma else (lambda m: m.matmul_dev(x, t, y))
+    run = lambda m: m.matmul_dev(x, t, y)
     for i in range(args.warmup):
         run(mats[i % nbuf])
     ctx.sync()
@@ -137,7 +137,7 @@ def bench_gemv(args):
     alg_bytes = mats[0].gguf_bytes + 4 * t * cols + 4 * t * rows
     traffic = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary, when present
     try:
-        prof_file = "gemv_iq3s_vocab_head_kernel_stats.txt" if os.environ.get("PYRE_QMATMUL_F32") == "1" else "gemv_i8_iq3s_vocab_head_kernel_stats.txt"
+        prof_file = "gemv_iq3s_vocab_head_kernel_stats.txt" if os.environ.get("PYRE_QMATMUL_F32") == "1" else "gemm_m_iq3s_vocab_head_kernel_stats.txt"
         for line in open(os.path.join(ROOT, "profiles", prof_file)):
             if t == 1 and ty == lib.IQ3_S and line.startswith("traffic_bytes_per_launch:"):
                 traffic = int(line.split(":")[1])
@@ -146,12 +146,12 @@ def bench_gemv(args):
     gbs = alg_bytes / (per * 1e-3) / 1e9                 # whole step (every launch of the operator call)
     kgbs = alg_bytes / (dom_us * 1e-6) / 1e9             # the dominant kernel alone
     out = {
-        "metric": "%s dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=%d%s)" % (FN, t, ", matrix cores" if args.mfma else ""), "value": round(gbs, 1), "unit": "GB/s",
+        "metric": "%s dequant-GEMV achieved HBM GB/s (vocab head 151936x2048, t=%d%s)" % (FN, t, ""), "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": kernels[0]["kernel"] if kernels else None, "device_bytes_per_launch": mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
+                     "kernel": kernels[0]["kernel"] if kernels else None, "device_bytes_per_launch": mats[0].layout_bytes(ty == lib.IQ3_S and os.environ.get("PYRE_QMATMUL_F32") != "1") or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
         "kernels": kernels,
     }
     if not args.no_cpu:
@@ -207,7 +207,7 @@ def bench_gemv0(args):
     x = ctx.upload(synth.normal((1, cols), 3)); y = ctx.alloc(rows * 4)
     alg = mats[0].gguf_bytes + 4 * cols + 4 * rows
     res = {}
-    for name, call in (("operator_i8", lambda m: m.matmul_dev(x, 1, y)), ("f32", lambda m: m.matmul_f32_dev(x, 1, y))):
+    for name, call in (("operator", lambda m: m.matmul_dev(x, 1, y)), ("f32", lambda m: m.matmul_f32_dev(x, 1, y))):
         for i in range(args.warmup):
             call(mats[i % nbuf])
         per = _timed(ev, ctx, args.steps, lambda i: call(mats[i % nbuf]))
@@ -221,9 +221,9 @@ def bench_gemv0(args):
                      "GBps_cache_resident": round(alg / (hot * 1e-3) / 1e9, 1), "single_synchronised_call_us_median": round(float(np.median(lat)), 2),
                      "kernels": {k: {"launches_per_call": round(v[0], 2), "avg_launch_us": round(v[1], 3)} for k, v in pr.items()},
                      "dominant_kernel": dom[0], "dominant_kernel_us": round(dom[1][1], 3), "dominant_kernel_GBps": round(alg / (dom[1][1] * 1e-6) / 1e9, 1)}
-    op = res["operator_i8"]
+    op = res["operator"]
     roof = {"bound": "hbm", "achieved": op["dominant_kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(op["dominant_kernel_GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": op["dominant_kernel"], "algorithmic_bytes_per_launch": alg, "device_bytes_per_launch": mats[0].dev_bytes, "avg_launch_us": op["dominant_kernel_us"]}
+            "kernel": op["dominant_kernel"], "algorithmic_bytes_per_launch": alg, "device_bytes_per_launch": mats[0].layout_bytes(True), "avg_launch_us": op["dominant_kernel_us"]}
     extra = {"paths": res}
     if not args.no_cpu:
         import orc
@@ -618,7 +618,6 @@ def main():
     ap.add_argument("--host-steps", type=int, default=32, help="decode workload: steps of the host-facing loop (pyre_forward + host argmax) to time beside the device loop (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
     ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs, q3_k, q5_k, q2_0)")
-    ap.add_argument("--mfma", action="store_true", help="gemv workload, t >= 2: the matrix-core verify GEMM instead of the T-accumulator GEMV")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MiB", help="gemv workload: also run 4 plain device copies of this size (counter calibration under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:

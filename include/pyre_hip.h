@@ -67,6 +67,9 @@ size_t pyre_qmat_gguf_bytes(const pyre_qmat* m);
 /* Bytes the matrix occupies in device memory after the load-time re-layout (what one GEMV actually streams); the
  * reference's counterpart is the size of the repacked Burn tensor (repack_to_burn, src/model/qn_gpu.rs:54). */
 size_t pyre_qmat_device_bytes(const pyre_qmat* m);
+/* The same per layout: 0 = the lane-per-row planes (every type; what pyre_qmatmul_f32 streams), 1 = the matrix-core layout
+ * (IQ3_S only, 0 otherwise; what pyre_qmatmul streams for IQ3_S).  No counterpart in the reference. */
+size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int matrix_core_layout);
 /* QMat::to_f32 (gguf_q.rs:212): all rows*cols values, bit-exact with gguf_q::dequant (gguf_q.rs:67-166). */
 int    pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host);
 int    pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev);

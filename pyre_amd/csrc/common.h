@@ -84,7 +84,8 @@ int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out);          // grow-only 
 // consecutive columns 8 * (l / 16) .. + 7 of the step, so a lane's share of a step is eight 4-bit codes = one dword:
 //   mq: [row group][128-column chunk][lane] x 16 B: dword s = step s of the chunk; the code of column element e of the lane's
 //       eight sits at nibble e/2 + 4*(e&1), so that or-ing nibbles p and p + 4 into one register yields elements 2p, 2p + 1
-//   mh: [row group][super-block][row] x 8 B: f16 d, 16 zero bits, the eight 4-bit sub-block scales (nibble i = sub-block i)
+//   mh: [row group][super-block][row] x 8 B: f16 d, 16 zero bits, the eight 4-bit sub-block scales (sub-block i at nibble
+//       i/2 + 4*(i&1), the same order)
 struct QMatDev {
   const uint8_t* p0; const uint8_t* p1; const uint8_t* p2; const uint8_t* p3; const uint8_t* pb;
   int rows, cols, U, tiles, fmt;

@@ -169,7 +169,7 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
     const float d = h2f_bits(hdr.x);
     for (int c = 0; c < 2; ++c) {                  // sub-block 2*(ku&3) + c of the super-block = step 2*(ku&1) + c of its 128-column half
       const int sbi = 2 * (ku & 3) + c, st = 2 * (ku & 1) + c;
-      const float db = d * (float)(1 + 2 * ((hdr.y >> (4 * sbi)) & 0xF));
+      const float db = d * (float)(1 + 2 * ((hdr.y >> (4 * ((sbi >> 1) + 4 * (sbi & 1)))) & 0xF));
       for (int kg = 0; kg < 4; ++kg) {
         const uint32_t w = ((const uint32_t*)m.mq)[((rgi * (size_t)(m.cols >> 7) + k128) * 64 + kg * 16 + j) * 4 + st];
         for (int e = 0; e < 8; ++e) { const int sv = 2 * (int)((w >> (4 * ((e >> 1) + 4 * (e & 1)))) & 0xF) - 15; y[32 * c + 8 * kg + e] = flip(db * (float)(sv < 0 ? -sv : sv), sv < 0 ? 1u : 0u); }

@@ -23,6 +23,7 @@
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+PYRE_TS_DECL(gemm_ts) PYRE_TS_EXPORT(gemm_ts, pyre_debug_ts_gemm)
 
 int pyre_aop_rows(int t) { return t <= 1 ? 2 : (t == 2 ? 4 : (t <= 4 ? 8 : 16)); }
 size_t pyre_aop_bytes(int cols, int t) { return (size_t)(cols / 8) * pyre_aop_rows(t) * 16; }
@@ -32,6 +33,7 @@ size_t pyre_aop_bytes(int cols, int t) { return (size_t)(cols / 8) * pyre_aop_ro
 // the f16 halves then keep 22 bits of every value that matters to the sum, whatever the magnitudes of x.
 __global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, int T, int R, int cols, uint16_t* __restrict__ op, float* __restrict__ ainv) {
   __shared__ float mx[4][8];
+  PYRE_TS_VARS PYRE_TS(0);
   const int sb = blockIdx.x, i = threadIdx.x, k = sb * 256 + i, wave = i >> 6, lane = i & 63;
   float v[8];
 #pragma unroll
@@ -56,6 +58,7 @@ __global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, 
     if (2 * t < R) { o[(2 * t) * 8] = __builtin_bit_cast(unsigned short, h1); o[(2 * t + 1) * 8] = __builtin_bit_cast(unsigned short, h2); }
     if (i == 0) ainv[sb * 8 + t] = t < T ? dn : 0.0f;
   }
+  PYRE_TS(1); PYRE_TS_FLUSH(gemm_ts, 24);
 }
 
 int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv) {
@@ -83,22 +86,35 @@ __device__ __forceinline__ ChunkRaw chunk_load(const QMatDev& m, const uint4* __
   return r;
 }
 
+// The two constants of the nibble -> f16 step.  They are kept in registers the compiler cannot see through, so that
+// (x & K) | E stays one instruction (a second literal would split it).
+struct NibK { uint32_t K, E; };
+__device__ __forceinline__ NibK nib_consts() { NibK k; asm volatile("s_mov_b32 %0, 0x03C003C0" : "=s"(k.K)); asm volatile("v_mov_b32 %0, 0x4C004C00" : "=v"(k.E)); return k; }
+// eight 4-bit fields of u -> four registers of two f16 numbers 16 + field: fields 0 and 4, 1 and 5, 2 and 6, 3 and 7
+__device__ __forceinline__ void nib_f16(uint32_t u, const NibK& k, uint32_t (&p)[4]) {
+  p[0] = ((u << 6) & k.K) | k.E; p[1] = ((u << 2) & k.K) | k.E; p[2] = ((u >> 2) & k.K) | k.E; p[3] = ((u >> 6) & k.K) | k.E;
+}
+
 // tot[g] += (this chunk's 128 columns of row group g) x (the sixteen activation rows), scaled
-__device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const uint2* __restrict__ sctab, v4f (&tot)[4]) {
-  const int sh = 16 * (c & 1);               // the chunk's four sub-block scales: nibbles 4 (c & 1) .. + 3 of the header's scale word
+__device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const NibK& nk, v4f (&tot)[4]) {
+  const int sh = 8 * (c & 1);                // the chunk's four sub-block scales: header fields (0, 4, 1, 5) of the scale word shifted by this
+  const v2h four = {(_Float16)4.0f, (_Float16)4.0f}, m62 = {(_Float16)-62.0f, (_Float16)-62.0f}, m235 = {(_Float16)-23.5f, (_Float16)-23.5f};
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
     const uint32_t wd[4] = {r.w[g].x, r.w[g].y, r.w[g].z, r.w[g].w};
     const uint32_t a4[4][4] = {{r.a[0].x, r.a[0].y, r.a[0].z, r.a[0].w}, {r.a[1].x, r.a[1].y, r.a[1].z, r.a[1].w}, {r.a[2].x, r.a[2].y, r.a[2].z, r.a[2].w}, {r.a[3].x, r.a[3].y, r.a[3].z, r.a[3].w}};
+    // the sub-block scales as f16 pairs: 16 + n -> 2s = 4 (16 + n) - 62 and -47s = -23.5 * 2s, s = 2n + 1, all exact
+    const uint32_t hs = r.h[g].y >> sh;
+    const uint32_t np0 = ((hs << 6) & nk.K) | nk.E, np1 = ((hs << 2) & nk.K) | nk.E;
+    v2h s2[2], s47[2];
+    s2[0] = __builtin_elementwise_fma(__builtin_bit_cast(v2h, np0), four, m62); s2[1] = __builtin_elementwise_fma(__builtin_bit_cast(v2h, np1), four, m62);
+    s47[0] = s2[0] * m235; s47[1] = s2[1] * m235;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const uint32_t n = (r.h[g].y >> (sh + 4 * s)) & 0xFu;
-      const uint2 sc = sctab[n];
-      const v2h vs2 = __builtin_bit_cast(v2h, sc.x), vs47 = __builtin_bit_cast(v2h, sc.y);
-      const uint32_t u = wd[s], K = 0x03C003C0u, E = 0x4C004C00u;
-      const uint32_t p[4] = {((u << 6) & K) | E, ((u << 2) & K) | E, ((u >> 2) & K) | E, ((u >> 6) & K) | E};
-      uint32_t q[4];
+      const v2h vs2 = {s2[s >> 1][s & 1], s2[s >> 1][s & 1]}, vs47 = {s47[s >> 1][s & 1], s47[s >> 1][s & 1]};
+      uint32_t p[4], q[4];
+      nib_f16(wd[s], nk, p);
 #pragma unroll
       for (int i = 0; i < 4; ++i) q[i] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(v2h, p[i]), vs2, vs47));
       struct U4 { uint32_t x[4]; };
@@ -120,47 +136,44 @@ __device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const uint2*
 template <int NW>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
-  __shared__ uint2 sctab[16];                 // scale nibble n -> packed f16 pairs (2s, 2s) and (-47s, -47s), s = 2n + 1
-  if (threadIdx.x < 16) {
-    const uint32_t a = __builtin_bit_cast(unsigned short, (_Float16)(float)(4 * (int)threadIdx.x + 2)), b = __builtin_bit_cast(unsigned short, (_Float16)(-47.0f * (float)(2 * (int)threadIdx.x + 1)));
-    sctab[threadIdx.x] = uint2{a | (a << 16), b | (b << 16)};
-  }
+  PYRE_TS_VARS PYRE_TS(0);
+  qmat_args_now(m); args_now(aop, ainv, y, T, R, cpw, ep.best, ep.conv_w, ep.conv_in, ep.conv_out, ep.co, ep.ch, ep.kk);
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int K128 = m.cols >> 7;
+  const int c0 = (ks * NW + wave) * cpw, c1 = min(K128, c0 + cpw);
+  v4f tot[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  const NibK nk = nib_consts();
+  ChunkRaw cur;
+  if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
+  // conv epilogue: wave 0 fetches its rows' taps and state now, behind the weights, so the loads overlap the products
   float cw[8], chist[8]; const bool conv_row = ep.co != nullptr && wave == 0 && tile * 64 + lane < ep.ch;
   if (conv_row) {
     const size_t row = (size_t)tile * 64 + lane;
 #pragma unroll
     for (int k = 0; k < 8; ++k) { cw[k] = k < ep.kk ? ep.conv_w[row * ep.kk + k] : 0.0f; chist[k] = k < ep.kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
   }
-  const int c0 = (ks * NW + wave) * cpw, c1 = min(K128, c0 + cpw);
-  v4f tot[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  PYRE_TS(1);
   if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane, no look-ahead
-    ChunkRaw cur;
-    if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
-    lds_barrier();                            // the scale table; the chunk's loads stay in flight
     for (int c = c0; c < c1; ++c) {
       if (c > c0) cur = chunk_load(m, aop, ainv, R, tile, c, lane, K128);
-      chunk_mac(cur, c, sctab, tot);
+      chunk_mac(cur, c, nk, tot);
     }
   } else {
-    ChunkRaw cur;
-    if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
-    lds_barrier();
     for (int c = c0; c < c1; ++c) {
       const int cn = c + 1 < c1 ? c + 1 : c;
       ChunkRaw nxt = chunk_load(m, aop, ainv, R, tile, cn, lane, K128);
-      chunk_mac(cur, c, sctab, tot);
+      chunk_mac(cur, c, nk, tot);
       cur = nxt;
     }
   }
+  PYRE_TS(2);
   // lane (q, j) holds, for row group g, token 2q (rows 0, 1 of its four) and token 2q + 1 (rows 2, 3): halves h1, h2 * 2^11
 #pragma unroll
   for (int g = 0; g < 4; ++g) { red[wave][g][0][lane] = tot[g][0] + tot[g][1] * (1.0f / 2048.0f); red[wave][g][1][lane] = tot[g][2] + tot[g][3] * (1.0f / 2048.0f); }
-  lds_barrier();
+  lds_barrier(); PYRE_TS(3);
   auto rsum = [&](int t, int rl) { const int l = (t >> 1) * 16 + (rl & 15), g = rl >> 4, h = t & 1; float s = red[0][g][h][l];
 #pragma unroll
     for (int w = 1; w < NW; ++w) s += red[w][g][h][l];
@@ -196,6 +209,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
 #pragma unroll
     for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
   }
+  PYRE_TS(4); PYRE_TS_FLUSH(gemm_ts, (NW == 16 ? 0 : (gridDim.y > 1 ? 8 : 16)));
 }
 
 namespace {

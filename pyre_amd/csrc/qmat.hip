@@ -175,7 +175,10 @@ __global__ __launch_bounds__(256) void k_repack_m(int rows, int rows_pad, int SB
     }
   }
   uint2 hd{0u, 0u};
-  if (live) { hd.x = (uint32_t)b[0] | ((uint32_t)b[1] << 8); hd.y = (uint32_t)b[106] | ((uint32_t)b[107] << 8) | ((uint32_t)b[108] << 16) | ((uint32_t)b[109] << 24); }
+  if (live) {       // sub-block i's scale at field i/2 + 4*(i&1) of the scale word, the order the codes of a step are in
+    hd.x = (uint32_t)b[0] | ((uint32_t)b[1] << 8);
+    for (int i = 0; i < 8; ++i) hd.y |= (uint32_t)((b[106 + (i >> 1)] >> (4 * (i & 1))) & 0xF) << (4 * ((i >> 1) + 4 * (i & 1)));
+  }
   mh[(rg * SB + sb) * 16 + j] = hd;
 }
 
@@ -507,6 +510,7 @@ size_t pyre_qmat_rows(const pyre_qmat* m) { return m ? m->rows : 0; }
 size_t pyre_qmat_cols(const pyre_qmat* m) { return m ? m->cols : 0; }
 size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; }
 size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes + m->dev_bytes_m : 0; }
+size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int matrix_core_layout) { return !m ? 0 : (matrix_core_layout ? m->dev_bytes_m : m->dev_bytes); }
 
 int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
   if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");

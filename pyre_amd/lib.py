@@ -49,6 +49,7 @@ def _declare(L):
         "pyre_qmatmul_f32_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_static_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
+        "pyre_qmat_layout_bytes": (sz, [vp, i32]),
         "pyre_gguf_open": (i32, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
         "pyre_gguf_close": (None, [vp]),
         "pyre_gguf_n_shards": (C.c_size_t, [vp]),
@@ -251,6 +252,10 @@ class QMat:
     @property
     def dev_bytes(self):
         return self.ctx.L.pyre_qmat_device_bytes(self.h)
+
+    def layout_bytes(self, matrix_core):
+        """Device bytes of one layout: False = the lane-per-row planes, True = the matrix-core layout (IQ3_S only)."""
+        return self.ctx.L.pyre_qmat_layout_bytes(self.h, 1 if matrix_core else 0)
 
     def to_f32(self):
         out = np.empty((self.rows, self.cols), dtype=np.float32)
