@@ -240,7 +240,10 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // router row; the gate/up launch adds the d/64 slices (RouteSrc).  bf16 and f32 routers, at most 64 slices.
 struct HcRoute { QMatDev router; float* part; };
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr, int comb_parts = 1);
+                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr, int comb_parts = 1, uint16_t* aop = nullptr);
+// aop (here and in pyre_gdn_launch / pyre_attn_launch_sel): when given, the kernel that writes the f32 result also leaves it
+// as the f16 operand of a matrix-core GEMM (PyreAop::op, pyre_aop_rows(t) rows, unscaled), so the GEMM that follows needs no
+// separate split launch.
 bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router);
 // waves per workgroup, units per wave and K slices of the norm + [down ; inject] kernel; false if the shape is unsupported
 bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit);
@@ -252,7 +255,7 @@ struct GdnDev { const float* a; const float* dt; const float* conv_w; const floa
 // conv_in/conv_out [(k-1)][ch], ssm_in/ssm_out [nv][dk][dv] (in != out).  co_scratch [8][ch].  out [t][nv*dv].
 // conv_done: co_scratch already holds silu(conv) of the window and the conv state has been advanced (GemvEpi).
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false);
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr);
 
 // Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
 // scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].
@@ -316,4 +319,4 @@ int pyre_qsa_launch(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaB
 int pyre_qsa_pool_all(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaBuf& b, int n);
 // the attention launch with an optional position list (qw == nullptr: dense)
 int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
-                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw);
+                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw, uint16_t* aop = nullptr);

@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj
 // 128x128 state in registers across the whole token window, so the state is read once and written once per launch.
 template <int DK, int DV>
 __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
-                                                   const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out) {
+                                                   const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out, uint16_t* __restrict__ aop, int aop_rows) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int G = 4, R = DK / G;
   PYRE_TS_VARS PYRE_TS(0);
@@ -86,7 +86,9 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     if (tid < DV) {
       float sc = 1.0f / sqrtf((red[4] + red[5]) / (float)DV + p.eps);
       float o = pm[0][j] * (sc * nw_j);                              // rms_inplace: x *= s * w  (:210)
-      out[(size_t)ti * w + h * DV + j] = o * g_sigm(z_j);   // z at [ch + h*dv + j]
+      const float ov = o * g_sigm(z_j);                             // z at [ch + h*dv + j]
+      out[(size_t)ti * w + h * DV + j] = ov;
+      if (aop) aop_store(aop, aop_rows, h * DV + j, ti, ov);        // the f16 operand of the output projection (matrix-core layout)
     }
     __syncthreads(); PYRE_TS(6);
   }
@@ -96,13 +98,14 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done) {
+                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done, uint16_t* aop) {
+  if (aop && t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: an f16 operand holds at most 8 tokens, not %d", t);
   if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
   if (g.conv_k < 2 || g.conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: conv kernel %d outside 2..8", g.conv_k);
   if (t < 1) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d", t);
   int ch = 2 * g.nk * g.dk + g.nv * g.dv;
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

@@ -146,7 +146,7 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
 // takes router tile w, w + nw, .. at unit blockIdx.x, the first tile's weights fetched ahead of the up GEMV.
 template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2,
-    QMatDev router, float* __restrict__ rpart) {
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
@@ -226,6 +226,7 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
     for (int q = 0; q < 8; ++q) if (q < hc) mx += term[(size_t)(t2 * hc + q) * 64 + l];          // streams ascending from zero (:1380)
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
+    if (aop) aop_store(aop, aop_rows, col, t2, mv);          // the f16 operand of the GEMM that follows (matrix-core layout)
     if (ROUTE) lo[t2 * 64 + l] = mv;          // lo is free after the barrier above
   }
   PYRE_TS(5);
@@ -271,13 +272,13 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
 #undef NORM_DOWN_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
-template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
+template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
   const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32 + (size_t)T * h.hc * 64);
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
 #define UP_MIX_GO(RF) hipLaunchKernelGGL((k_hc_up_mix<FMT, T, RF>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, (const uint2*)ctx->d_iq2xs, rq, rp)
+                     h.d, mixed, inj, (const uint2*)ctx->d_iq2xs, rq, rp, aop, pyre_aop_rows(T))
   if constexpr (FMT == FMT_IQ3_S || FMT == FMT_BF16 || FMT == FMT_F16 || FMT == FMT_F32) {
     if (rt && rq.fmt == FMT_BF16) UP_MIX_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_GO(FMT_F32); else UP_MIX_GO(-1);
   } else UP_MIX_GO(-1);
@@ -295,8 +296,8 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
 int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj, float eps) {
   HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, comb_parts, mo, comb_inj, eps))
 }
-int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
-  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt))
+int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
+  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt, aop))
 }
 }  // namespace
 
@@ -316,7 +317,7 @@ void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
 }
 
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed, float* inj, const HcRoute* route, int comb_parts) {
+                       float eps, float* mixed, float* inj, const HcRoute* route, int comb_parts, uint16_t* aop) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
   if (comb_parts != 1 && !(comb_parts == PYRE_GEMV_PARTS && h.di.fmt == FMT_IQ3_S && comb_out && !comb_moe)) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: %d partial vectors (1, or %d with an IQ3_S mix)", comb_parts, PYRE_GEMV_PARTS);
   if (route && !pyre_hc_route_ok(h, route->router)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: this router cannot ride on the mix");
@@ -328,7 +329,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
   if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj, eps); if (rc) return rc;
-  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route);
+  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route, aop);
 }
 
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x, int t, const float* out, const float* inj) {

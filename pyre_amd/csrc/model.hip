@@ -30,6 +30,7 @@ struct pyre_model {
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
   float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr, *rpart = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
+  uint16_t* aop = nullptr;      // the f16 operand a producer kernel leaves for the matrix-core GEMV that follows it (one at a time: the launches are stream-ordered)
 };
 
 struct pyre_state {
@@ -187,8 +188,10 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
   MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
   size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
+  int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));
+  const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + al256(rp_b) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + al256(rp_b) + al256(aop_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
@@ -196,8 +199,9 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
-  m->rpart = (float*)take(rp_b);
-  { uint4* op; float* ainv; int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));      // the operand buffer of the widest GEMV input, so that no step allocates
+  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
+  PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
+  { uint4* op; float* ainv;      // and the context's operand buffer for a GEMV whose producer leaves f32 only, so that no step allocates
     if ((rc = pyre_gemm_m_scratch(ctx, (kmax + 255) / 256 * 256, &op, &ainv))) return rc; }
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   guard.armed = false; *out = M.release(); return PYRE_OK;
@@ -354,25 +358,29 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
+  const bool fuse_aop = [] { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }();      // 1: separate split launches instead of the producers' own operand stores
+  const PyreAop aop{(const uint4*)m->aop, nullptr};
+  auto opnd = [&](const QMatDev& q) -> const PyreAop* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? &aop : nullptr; };
+  auto opw = [&](const QMatDev& q) -> uint16_t* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? m->aop : nullptr; };
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, 1, opw(L.proj)))) return rc;
     advance();
     if (L.full) {
       int ai = L.mix_index;
-      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj))) return rc;
+      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.proj)))) return rc;
       if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], s->qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
-      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &s->qw : nullptr))) return rc;
+      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &s->qw : nullptr, opw(L.outp)))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
-      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv))) return rc;
-      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true))) return rc;
+      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.proj)))) return rc;
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, opw(L.outp)))) return rc;
       s->cur[li] = nb;
     }
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
-    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o))) return rc; }
-    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o))) return rc;
+    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc; }
+    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc;
     const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
     HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
@@ -384,16 +392,16 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   if (!replay) s->len = start + t;
   if (o.head_tokens == 0) return PYRE_OK;       // prompt window whose logits nobody reads
   if (o.head_tokens >= t) {
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a))) return rc;
-    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
-    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits);
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->out)))) return rc;
+    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->out));
+    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->out));
   }
   // last token only: fold the pending ffn output into its streams, then the head
   const size_t last = (size_t)(t - 1) * hc * d;
   MoeOut mol{}; if (comb_moe) mol = pyre_moe_out(m->layers.back().moe, m->mw, t - 1);
-  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a))) return rc;
-  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best);
-  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits);
+  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->out)))) return rc;
+  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->out));
+  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits, opnd(m->out));
 }
 
 int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
