@@ -82,10 +82,11 @@ int pyre_stage(pyre_ctx* ctx, size_t nbytes, void** out);          // grow-only 
 // FMT_IQ3_S_M (IQ3_S for the matrix cores): rows in groups of 16, columns in steps of 32 (one sub-block).  In
 // v_mfma_f32_16x16x32_f16 lane l supplies, for the operand that carries the weights, row l % 16 of the group and the eight
 // consecutive columns 8 * (l / 16) .. + 7 of the step, so a lane's share of a step is eight 4-bit codes = one dword:
-//   mq: [row group][128-column chunk][lane] x 16 B: dword s = step s of the chunk; the code of column element e of the lane's
+//   mq: [row tile of 64][128-column chunk][row group of the tile][lane] x 16 B (a tile's chunk is 4 KB contiguous, a tile's
+//       whole K range one contiguous run): dword s = step s of the chunk; the code of column element e of the lane's
 //       eight sits at nibble e/2 + 4*(e&1), so that or-ing nibbles p and p + 4 into one register yields elements 2p, 2p + 1
-//   mh: [row group][super-block][row] x 8 B: f16 d, 16 zero bits, the eight 4-bit sub-block scales (sub-block i at nibble
-//       i/2 + 4*(i&1), the same order)
+//   mh: [row tile][super-block][row group][row] x 8 B: f16 d, 16 zero bits, the eight 4-bit sub-block scales (sub-block i
+//       at nibble i/2 + 4*(i&1), the same order)
 struct QMatDev {
   const uint8_t* p0; const uint8_t* p1; const uint8_t* p2; const uint8_t* p3; const uint8_t* pb;
   int rows, cols, U, tiles, fmt;
@@ -104,6 +105,9 @@ template <typename... A> __device__ __forceinline__ void args_now(A... a) { (arg
 __device__ __forceinline__ void qmat_args_now(const QMatDev& m) { args_now(m.p0, m.p1, m.p2, m.p3, m.pb, m.rows, m.cols, m.U, m.tiles); }
 #endif
 
+// index of row group rg's 64 lane slots (16 B each) for chunk c in mq, and of its 16 header slots (8 B each) for super-block sb in mh
+inline __host__ __device__ size_t mq_slot(size_t rg, int c, int K128) { return (((rg >> 2) * K128 + c) * 4 + (rg & 3)) * 64; }
+inline __host__ __device__ size_t mh_slot(size_t rg, int sb, int SB) { return (((rg >> 2) * SB + sb) * 4 + (rg & 3)) * 16; }
 // dv: the lane = row planes (every type).  dvm: the matrix-core layout, IQ3_S only (fmt == FMT_IQ3_S_M when present).
 // Which of the two an IQ3_S matrix holds is decided at creation: the stand-alone operator keeps both (its entry points
 // cover both kernels), the model keeps one per matrix.
@@ -139,6 +143,8 @@ int pyre_gemv_split_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, 
 bool pyre_gemv_parts_ok(const QMatDev& m);
 int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* parts_dev, const PyreAop* a = nullptr);
 // t = 1 GEMV that also leaves, per row tile, (bits of the maximum, first row holding it) in best[2*tile], best[2*tile+1].
+// (value bits, first row) pairs the argmax form leaves in best_dev for this matrix: one per row tile
+int pyre_gemv_best_count(const QMatDev& m);
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, float* y_dev, uint32_t* best_dev, const PyreAop* a = nullptr);
 // y as pyre_gemv_launch (raw projections), plus the conv epilogue described at GemvEpi (best ignored).
 int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, const GemvEpi& conv, const PyreAop* a = nullptr);
@@ -162,6 +168,7 @@ size_t pyre_aop_bytes(int cols, int t);                            // operand by
 // splits x [t][cols] (any magnitudes: each 256-column stretch of a token is scaled by its own power of two) into op / ainv
 int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv);
 // y as pyre_gemv_launch / pyre_gemv_split_launch (ksplit > 1: slice sums) with the epilogues of GemvEpi
+int pyre_gemm_m_best_count(const QMatDev& m);
 int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep);
 // K parts / waves per workgroup the kernel uses for this matrix (ksplit parts)
 void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* hb_per_wave);

@@ -165,13 +165,13 @@ template <int FMT> __device__ inline void decode_exact(const QMatDev& m, const u
   } else if constexpr (FMT == FMT_IQ3_S_M) {       // the same codes in the matrix-core layout (QMatDev::mq / mh)
     const size_t row = (size_t)tile * 64 + lane, rgi = row >> 4; const int j = (int)(row & 15);
     const int sb = ku >> 2, k128 = ku >> 1;
-    const uint2 hdr = ((const uint2*)m.mh)[(rgi * m.SB + sb) * 16 + j];
+    const uint2 hdr = ((const uint2*)m.mh)[mh_slot(rgi, sb, m.SB) + j];
     const float d = h2f_bits(hdr.x);
     for (int c = 0; c < 2; ++c) {                  // sub-block 2*(ku&3) + c of the super-block = step 2*(ku&1) + c of its 128-column half
       const int sbi = 2 * (ku & 3) + c, st = 2 * (ku & 1) + c;
       const float db = d * (float)(1 + 2 * ((hdr.y >> (4 * ((sbi >> 1) + 4 * (sbi & 1)))) & 0xF));
       for (int kg = 0; kg < 4; ++kg) {
-        const uint32_t w = ((const uint32_t*)m.mq)[((rgi * (size_t)(m.cols >> 7) + k128) * 64 + kg * 16 + j) * 4 + st];
+        const uint32_t w = ((const uint32_t*)m.mq)[(mq_slot(rgi, k128, m.cols >> 7) + kg * 16 + j) * 4 + st];
         for (int e = 0; e < 8; ++e) { const int sv = 2 * (int)((w >> (4 * ((e >> 1) + 4 * (e & 1)))) & 0xF) - 15; y[32 * c + 8 * kg + e] = flip(db * (float)(sv < 0 ? -sv : sv), sv < 0 ? 1u : 0u); }
       }
     }

@@ -68,22 +68,34 @@ int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, ui
 }
 
 // ---- the product -----------------------------------------------------------------------------------------------------------------
-struct ChunkRaw { uint4 w[4]; uint2 h[4]; uint4 a[4]; float ai0, ai1; };
+// What a wave fetches for one chunk: from the matrix (memory) its row groups' codes and super-block headers, from the
+// operand (second-level cache) the sixteen activation rows and their scale factors.
+template <int G> struct WBuf { uint4 w[G]; uint2 h[G]; };
+struct ABuf { uint4 a[4]; float ai0, ai1; };
 
-__device__ __forceinline__ ChunkRaw chunk_load(const QMatDev& m, const uint4* __restrict__ aop, const float* __restrict__ ainv, int R, int tile, int c, int lane, int K128) {
-  ChunkRaw r;
-  const bool live = (lane & 15) < R;         // operand rows the window does not have are zero
+template <int G> __device__ __forceinline__ void load_w(const QMatDev& m, int rg0, int c, int lane, int K128, WBuf<G>& b) {
 #pragma unroll
-  for (int s = 0; s < 4; ++s) r.a[s] = live ? aop[(((size_t)c * 4 + s) * 4 + (lane >> 4)) * R + (lane & 15)] : make_uint4(0, 0, 0, 0);
+  for (int g = 0; g < G; ++g) b.w[g] = ((const uint4*)m.mq)[mq_slot((size_t)rg0 + g, c, K128) + lane];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const size_t rg = (size_t)tile * 4 + g;
-    r.w[g] = ((const uint4*)m.mq)[(rg * K128 + c) * 64 + lane];
-    r.h[g] = ((const uint2*)m.mh)[(rg * m.SB + (c >> 1)) * 16 + (lane & 15)];
+  for (int g = 0; g < G; ++g) b.h[g] = ((const uint2*)m.mh)[mh_slot((size_t)rg0 + g, c >> 1, m.SB) + (lane & 15)];
+}
+// Every load is unconditional, so that the compiler's count of outstanding loads is exact and a wait for one chunk never
+// drains the chunks requested after it: operand rows the window does not have are read through a buffer descriptor at an
+// offset past its end, which returns zeros without touching memory.
+struct AopRsrc { __amdgpu_buffer_rsrc_t r; int lane_off; };       // lane_off: byte offset of the lane's row inside an (8-column group) x R block, or -1
+__device__ __forceinline__ AopRsrc aop_rsrc(const uint4* aop, int cols, int R, int lane) {
+  AopRsrc a; a.r = __builtin_amdgcn_make_buffer_rsrc((void*)aop, 0, (cols >> 3) * R * 16, 0x00020000);
+  a.lane_off = (lane & 15) < R ? ((lane >> 4) * R + (lane & 15)) * 16 : -1; return a;
+}
+template <bool SC> __device__ __forceinline__ void load_a(const AopRsrc& ar, const float* __restrict__ ainv, int R, int c, int lane, ABuf& b) {
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int off = ar.lane_off < 0 ? -1 : ar.lane_off + (c * 4 + s) * 4 * R * 16;
+    const auto v = __builtin_amdgcn_raw_buffer_load_b128(ar.r, off, 0, 0);
+    b.a[s] = make_uint4(v[0], v[1], v[2], v[3]);
   }
-  r.ai0 = 1.0f; r.ai1 = 1.0f;
-  if (ainv) { const float2 p = ((const float2*)ainv)[(c >> 1) * 4 + (lane >> 4)]; r.ai0 = p.x; r.ai1 = p.y; }
-  return r;
+  b.ai0 = 1.0f; b.ai1 = 1.0f;
+  if constexpr (SC) { const float2 p = ((const float2*)ainv)[(c >> 1) * 4 + (lane >> 4)]; b.ai0 = p.x; b.ai1 = p.y; }
 }
 
 // The two constants of the nibble -> f16 step.  They are kept in registers the compiler cannot see through, so that
@@ -96,16 +108,20 @@ __device__ __forceinline__ void nib_f16(uint32_t u, const NibK& k, uint32_t (&p)
 }
 
 // tot[g] += (this chunk's 128 columns of row group g) x (the sixteen activation rows), scaled
-__device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const NibK& nk, v4f (&tot)[4]) {
+template <int G> __device__ __forceinline__ void chunk_mac(const WBuf<G>& wb, const ABuf& ab, int c, const NibK& nk, v4f (&tot)[G]) {
+#ifdef PYRE_DIAG_NOMAC
+  for (int g = 0; g < G; ++g) { tot[g][0] += __uint_as_float((wb.w[g].x ^ wb.w[g].y ^ wb.w[g].z ^ wb.w[g].w ^ wb.h[g].x ^ wb.h[g].y) & 0x3FFFFFFF); tot[g][1] += __uint_as_float((ab.a[g].x ^ ab.a[g].y ^ ab.a[g].z ^ ab.a[g].w) & 0x3FFFFFFF) + ab.ai0 + ab.ai1; }
+  return;
+#endif
   const int sh = 8 * (c & 1);                // the chunk's four sub-block scales: header fields (0, 4, 1, 5) of the scale word shifted by this
   const v2h four = {(_Float16)4.0f, (_Float16)4.0f}, m62 = {(_Float16)-62.0f, (_Float16)-62.0f}, m235 = {(_Float16)-23.5f, (_Float16)-23.5f};
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < G; ++g) {
     v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    const uint32_t wd[4] = {r.w[g].x, r.w[g].y, r.w[g].z, r.w[g].w};
-    const uint32_t a4[4][4] = {{r.a[0].x, r.a[0].y, r.a[0].z, r.a[0].w}, {r.a[1].x, r.a[1].y, r.a[1].z, r.a[1].w}, {r.a[2].x, r.a[2].y, r.a[2].z, r.a[2].w}, {r.a[3].x, r.a[3].y, r.a[3].z, r.a[3].w}};
+    const uint32_t wd[4] = {wb.w[g].x, wb.w[g].y, wb.w[g].z, wb.w[g].w};
+    const uint32_t a4[4][4] = {{ab.a[0].x, ab.a[0].y, ab.a[0].z, ab.a[0].w}, {ab.a[1].x, ab.a[1].y, ab.a[1].z, ab.a[1].w}, {ab.a[2].x, ab.a[2].y, ab.a[2].z, ab.a[2].w}, {ab.a[3].x, ab.a[3].y, ab.a[3].z, ab.a[3].w}};
     // the sub-block scales as f16 pairs: 16 + n -> 2s = 4 (16 + n) - 62 and -47s = -23.5 * 2s, s = 2n + 1, all exact
-    const uint32_t hs = r.h[g].y >> sh;
+    const uint32_t hs = wb.h[g].y >> sh;
     const uint32_t np0 = ((hs << 6) & nk.K) | nk.E, np1 = ((hs << 2) & nk.K) | nk.E;
     v2h s2[2], s47[2];
     s2[0] = __builtin_elementwise_fma(__builtin_bit_cast(v2h, np0), four, m62); s2[1] = __builtin_elementwise_fma(__builtin_bit_cast(v2h, np1), four, m62);
@@ -122,8 +138,8 @@ __device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const NibK& 
       const v8h A = __builtin_bit_cast(v8h, (U4{{a4[s][0], a4[s][1], a4[s][2], a4[s][3]}}));
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, acc, 0, 0, 0);
     }
-    const float d = h2f_bits(r.h[g].x & 0xFFFFu);
-    const float d0 = d * r.ai0, d1 = d * r.ai1;
+    const float d = h2f_bits(wb.h[g].x & 0xFFFFu);
+    const float d0 = d * ab.ai0, d1 = d * ab.ai1;
     tot[g][0] = fmaf(acc[0], d0, tot[g][0]); tot[g][1] = fmaf(acc[1], d0, tot[g][1]);
     tot[g][2] = fmaf(acc[2], d1, tot[g][2]); tot[g][3] = fmaf(acc[3], d1, tot[g][3]);
   }
@@ -133,7 +149,7 @@ __device__ __forceinline__ void chunk_mac(const ChunkRaw& r, int c, const NibK& 
 //   ksplit  > 1: y is a partial buffer, y[(ks*T + t)*tiles*64 + row] = slice sum (the consumer adds the slices in order).
 //   ep.best (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 //   ep.co: conv1d + SiLU of the leading ep.ch rows (linear_core, qwen4exp_gguf.rs:1643-1647), as in the lane = row GEMV.
-template <int NW>
+template <int NW, bool SC, bool CONV>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
@@ -146,27 +162,33 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
 #pragma unroll
   for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   const NibK nk = nib_consts();
-  ChunkRaw cur;
-  if (c0 < c1) cur = chunk_load(m, aop, ainv, R, tile, c0, lane, K128);
+  const AopRsrc ar = aop_rsrc(aop, m.cols, R, lane);
+  WBuf<4> w0; ABuf a0;
+  if (c0 < c1) { load_a<SC>(ar, ainv, R, c0, lane, a0); load_w<4>(m, tile * 4, c0, lane, K128, w0); }
   // conv epilogue: wave 0 fetches its rows' taps and state now, behind the weights, so the loads overlap the products
-  float cw[8], chist[8]; const bool conv_row = ep.co != nullptr && wave == 0 && tile * 64 + lane < ep.ch;
-  if (conv_row) {
+  float cw[CONV ? 8 : 1], chist[CONV ? 8 : 1]; const bool conv_row = CONV && wave == 0 && tile * 64 + lane < ep.ch;
+  if constexpr (CONV) if (conv_row) {
     const size_t row = (size_t)tile * 64 + lane;
 #pragma unroll
     for (int k = 0; k < 8; ++k) { cw[k] = k < ep.kk ? ep.conv_w[row * ep.kk + k] : 0.0f; chist[k] = k < ep.kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
   }
   PYRE_TS(1);
-  if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane, no look-ahead
+  if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane: one buffer, no look-ahead
     for (int c = c0; c < c1; ++c) {
-      if (c > c0) cur = chunk_load(m, aop, ainv, R, tile, c, lane, K128);
-      chunk_mac(cur, c, nk, tot);
+      if (c > c0) { load_a<SC>(ar, ainv, R, c, lane, a0); load_w<4>(m, tile * 4, c, lane, K128, w0); }
+      chunk_mac<4>(w0, a0, c, nk, tot);
     }
-  } else {
-    for (int c = c0; c < c1; ++c) {
-      const int cn = c + 1 < c1 ? c + 1 : c;
-      ChunkRaw nxt = chunk_load(m, aop, ainv, R, tile, cn, lane, K128);
-      chunk_mac(cur, c, nk, tot);
-      cur = nxt;
+  } else {                                    // two buffers taking turns (a copy from one to the other would wait for the loads just issued)
+    WBuf<4> w1; ABuf a1;
+    for (int c = c0; c < c1; c += 2) {
+      if (c + 1 < c1) { load_a<SC>(ar, ainv, R, c + 1, lane, a1); load_w<4>(m, tile * 4, c + 1, lane, K128, w1); }
+      __builtin_amdgcn_sched_barrier(0);      // (keeps the compiler from sinking the loads down to their first use)
+      chunk_mac<4>(w0, a0, c, nk, tot);
+      __builtin_amdgcn_sched_barrier(0);
+      if (c + 2 < c1) { load_a<SC>(ar, ainv, R, c + 2, lane, a0); load_w<4>(m, tile * 4, c + 2, lane, K128, w0); }
+      __builtin_amdgcn_sched_barrier(0);
+      if (c + 1 < c1) chunk_mac<4>(w1, a1, c + 1, nk, tot);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   PYRE_TS(2);
@@ -191,7 +213,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
       if (l == 0) { ep.best[2 * tile] = __float_as_uint(bv); ep.best[2 * tile + 1] = bi; }
     }
   }
-  if (conv_row) {
+  if constexpr (CONV) if (conv_row) {
     const size_t row = (size_t)tile * 64 + lane;
     for (int t = 0; t < T; ++t) {
       const float cur = rsum(t, lane);
@@ -224,7 +246,10 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
   return nw;
 }
 template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep) {
-  hipLaunchKernelGGL((k_gemm_m<NW>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep);
+#define GEMM_M_GO(SC, CONV) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
+  if (ep.co) { if (a.ainv) GEMM_M_GO(true, true); else GEMM_M_GO(false, true); }
+  else { if (a.ainv) GEMM_M_GO(true, false); else GEMM_M_GO(false, false); }
+#undef GEMM_M_GO
 }
 }  // namespace
 
@@ -232,6 +257,8 @@ void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* cpw) {
   *nw = gemm_m_nw(m, ksplit);
   const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit; *cpw = (per_wg + *nw - 1) / *nw; if (*cpw < 1) *cpw = 1;
 }
+
+int pyre_gemm_m_best_count(const QMatDev& m) { return m.tiles; }
 
 int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, const GemvEpi& ep) {
   if (m.fmt != FMT_IQ3_S_M || !m.mq || !m.mh) return pyre_fail(ctx, PYRE_E_TYPE, "gemm_m: the matrix is not held in the matrix-core layout");

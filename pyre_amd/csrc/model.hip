@@ -191,14 +191,14 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));
   const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 64 + 2)) + al256(rp_b) + al256(aop_b) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
   m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
-  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 64 + 2));
+  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
   m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
   PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
   { uint4* op; float* ainv;      // and the context's operand buffer for a GEMV whose producer leaves f32 only, so that no step allocates
@@ -350,7 +350,7 @@ bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) &&
 int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, o.toks_out, &m->embd, m->emb, o.step_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
   // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
   // leaves the updated streams in the other
   const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
@@ -526,7 +526,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
     s->len += n_steps - 1;
     for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
   }
-  if ((rc = pyre_pick_launch(ctx, m->best, m->out.tiles, m->ids, m->toks + n_steps - 1, nullptr, nullptr, nullptr))) return rc;
+  if ((rc = pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, m->toks + n_steps - 1, nullptr, nullptr, nullptr))) return rc;
   if (tokens_host) { PYRE_HIP(ctx, hipMemcpyAsync(tokens_host, m->toks, (size_t)n_steps * 4, hipMemcpyDeviceToHost, ctx->stream)); PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK; }
   return PYRE_OK;
 }

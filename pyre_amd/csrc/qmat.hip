@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void k_repack_m(int rows, int rows_pad, int SB
         const uint32_t gA = g3[b[2 + 8 * ib + 2 * l] | ((h << (8 - 2 * l)) & 256)], gB = g3[b[2 + 8 * ib + 2 * l + 1] | ((h << (7 - 2 * l)) & 256)], sg = b[74 + 4 * ib + l];
         for (int e = 0; e < 8; ++e) { const uint32_t gb = ((e < 4 ? gA : gB) >> (8 * (e & 3))) & 0xFF; wd |= iq3s_code(gb, (sg >> e) & 1) << (4 * ((e >> 1) + 4 * (e & 1))); }
       }
-      mq[((rg * K128 + 2 * sb + (ib >> 2)) * 64 + l * 16 + j) * 4 + (ib & 3)] = wd;
+      mq[(mq_slot(rg, 2 * sb + (ib >> 2), (int)K128) + l * 16 + j) * 4 + (ib & 3)] = wd;
     }
   }
   uint2 hd{0u, 0u};
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256) void k_repack_m(int rows, int rows_pad, int SB
     hd.x = (uint32_t)b[0] | ((uint32_t)b[1] << 8);
     for (int i = 0; i < 8; ++i) hd.y |= (uint32_t)((b[106 + (i >> 1)] >> (4 * (i & 1))) & 0xF) << (4 * ((i >> 1) + 4 * (i & 1)));
   }
-  mh[(rg * SB + sb) * 16 + j] = hd;
+  mh[mh_slot(rg, sb, SB) + j] = hd;
 }
 
 // ---- bit-exact dequant export -----------------------------------------------------------------------------------------
@@ -387,6 +387,7 @@ int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int 
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep));
   return rc;
 }
+int pyre_gemv_best_count(const QMatDev& m) { return m.fmt == FMT_IQ3_S_M ? pyre_gemm_m_best_count(m) : m.tiles; }
 int pyre_gemv_argmax_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, uint32_t* best, const PyreAop* a) {
   int rc = PYRE_OK;
   GemvEpi ep{}; ep.best = best;
