@@ -135,12 +135,12 @@ def bench_gemv(args):
     kernels = [{"kernel": k, "launches_per_step": round(v[0] / pn, 2), "avg_launch_us": round(v[1] / v[0] * 1e3, 3)} for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])]
     dom_us = kernels[0]["avg_launch_us"] if kernels else per * 1e3
     alg_bytes = mats[0].gguf_bytes + 4 * t * cols + 4 * t * rows
-    traffic = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary, when present
+    traffic = None; traffic_source = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary (not this run), when present
     try:
         prof_file = "gemv_iq3s_vocab_head_kernel_stats.txt" if os.environ.get("PYRE_QMATMUL_F32") == "1" else "gemm_m_iq3s_vocab_head_kernel_stats.txt"
         for line in open(os.path.join(ROOT, "profiles", prof_file)):
             if t == 1 and ty == lib.IQ3_S and line.startswith("traffic_bytes_per_launch:"):
-                traffic = int(line.split(":")[1])
+                traffic = int(line.split(":")[1]); traffic_source = "profiles/%s: rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, not this run" % prof_file
     except OSError:
         pass
     gbs = alg_bytes / (per * 1e-3) / 1e9                 # whole step (every launch of the operator call)
@@ -150,7 +150,7 @@ def bench_gemv(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
-        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": kernels[0]["kernel"] if kernels else None, "device_bytes_per_launch": mats[0].layout_bytes(ty == lib.IQ3_S and os.environ.get("PYRE_QMATMUL_F32") != "1") or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
         "kernels": kernels,
     }
@@ -565,12 +565,15 @@ def bench_decode(args):
                   "avg_launch_us": round(v[1] / v[0] * 1e3, 3), "GBps": round(v[2] / (v[1] * 1e-3) / 1e9, 1) if v[1] > 0 else None} for k, v in classes]
     dom_k, dom = classes[0]
     dom_gbs = dom[2] / (dom[1] * 1e-3) / 1e9
-    traffic = None          # HBM bytes per launch of the dominant class from the committed FETCH_SIZE / WRITE_SIZE summary, when it covers it
+    # HBM bytes per launch of the dominant class: not measured by this run but read from the committed FETCH_SIZE /
+    # WRITE_SIZE summary (a three-layer slice of the same step), when that covers the class; traffic_source says so
+    traffic = None; traffic_source = None
     if cfg.n_layers == 48 and not args.indexer:
         try:
             for line in open(os.path.join(ROOT, "profiles", "decode_deltanet_slice_hbm_traffic.txt")):
                 if line.startswith("traffic_bytes_per_launch_%s:" % dom_k):
                     traffic = int(line.split(":")[1])
+                    traffic_source = "profiles/decode_deltanet_slice_hbm_traffic.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE on a three-layer slice of this step, not this run; attention-layer launches of the class are not covered"
         except OSError:
             pass
     out = {
@@ -578,10 +581,11 @@ def bench_decode(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[4]: Qwen-Next-style A3B hybrid, %d layers (3 Gated DeltaNet + 1 gated attention per group), 512 experts top-10 + shared, "
-                               "IQ3_S weights (bf16 router), 4 hyper-connection streams, 4-bit KV, greedy decode after a %d-token random prompt%s" % (
-                                   cfg.n_layers, n_ctx, (", QSA indexer with %d heads (budget 2048, blocks of 4): variant, not the configuration of the metric" % args.indexer) if args.indexer else ""),
-                   "context": n_ctx, "layers": cfg.n_layers},
-        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                               "IQ3_S weights (bf16 router), 4 hyper-connection streams (their synthetic matrices' block scales divided by hc_d_div = %g so that the streams stay bounded over 48 layers), "
+                               "4-bit KV, greedy decode after a %d-token random prompt%s" % (
+                                   cfg.n_layers, cfg.hc_d_div, n_ctx, (", QSA indexer with %d heads (budget 2048, blocks of 4): variant, not the configuration of the metric" % args.indexer) if args.indexer else ""),
+                   "context": n_ctx, "layers": cfg.n_layers, "hc_d_div": cfg.hc_d_div},
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": dom_k, "algorithmic_bytes_per_launch": round(dom[2] / dom[0]), "avg_launch_us": round(dom[1] / dom[0] * 1e3, 3),
                      "share_of_kernel_time": round(dom[1] / tot_ms, 3)},
         "token_roofline": {"weight_bytes_per_token": wbytes, "kv_bytes_per_token": round(kvb), "state_bytes_per_token": state_b,
