@@ -54,6 +54,35 @@ def test_forward_logits_and_state_match_oracle(ctx, qtype, hc_type):
     assert relerr(k.reshape(-1), os_.kcache(0)) <= 1e-4 and relerr(v.reshape(-1), os_.vcache(0)) <= 1e-4
 
 
+def test_matrix_core_layout_equals_the_lane_per_row_layout_and_the_separate_operand_split(ctx, monkeypatch):
+    # the same IQ3_S model three ways: projections, head and embedding on the matrix cores with the operand left by the
+    # producer kernels (default); the same with every GEMV splitting its own input; every matrix in the lane = row layout.
+    # All three against the oracle, single steps and a verify window, and the same greedy stream.
+    c = small_cfg(qtype=synth.IQ3_S, hc_type=synth.IQ3_S, hc_lr=256)
+    hw = mg.build_host(c, seed=41); om = orc_model(hw)
+    prompt = np.random.Generator(np.random.PCG64(42)).integers(0, c.vocab, 21, dtype=np.uint32)
+    os_ = om.new_state(); lo = om.forward(prompt, os_)
+    want = []; tok = int(orc.argmax(lo))
+    for _ in range(12):
+        want.append(tok); tok = int(orc.argmax(om.forward(np.array([tok], dtype=np.uint32), os_)))
+    outs = {}
+    for name, env in (("default", {}), ("split", {"PYRE_AOP_SPLIT": "1"}), ("rows", {"PYRE_MODEL_ROWS": "1"})):
+        for k in ("PYRE_AOP_SPLIT", "PYRE_MODEL_ROWS"):
+            monkeypatch.delenv(k, raising=False)
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        gm = lib.Model(ctx, c, hw.layers, hw.globals_); st = gm.new_state(128)
+        lg = gm.forward(prompt, st)
+        assert relerr(lg, lo) <= 1e-3, name
+        got = gm.decode_greedy_dev(st, int(orc.argmax(lg)), 12)
+        assert [int(orc.argmax(lg))] + [int(x) for x in got[:11]] == want, name
+        win = gm.forward_multi(np.array(want[:5], dtype=np.uint32), st)          # a verify window on top
+        outs[name] = (lg, win)
+        st.close(); gm.close()
+    for name in ("split", "rows"):
+        assert relerr(outs[name][0], outs["default"][0]) <= 1e-4 and relerr(outs[name][1], outs["default"][1]) <= 1e-4, name
+
+
 @pytest.mark.parametrize("router_type,hc_type,rides", [(synth.BF16, synth.IQ3_S, True), (synth.F32, synth.BF16, True), (synth.F32, synth.F32, True), (synth.BF16, synth.F16, True),
                                                        (synth.F16, synth.BF16, False), (synth.BF16, synth.Q8_0, False)])
 def test_router_riding_on_the_mix_equals_the_separate_router_launch(ctx, router_type, hc_type, rides, monkeypatch):
