@@ -197,9 +197,10 @@ enum {
   PYRE_T_ATTN_QKV, PYRE_T_ATTN_GATE, PYRE_T_SSM_BETA, PYRE_T_SSM_ALPHA, PYRE_T_SSM_A, PYRE_T_SSM_DT_BIAS, PYRE_T_SSM_CONV1D, PYRE_T_SSM_NORM, PYRE_T_SSM_OUT,
   PYRE_T_FFN_GATE_INP, PYRE_T_FFN_GATE_EXPS, PYRE_T_FFN_UP_EXPS, PYRE_T_FFN_DOWN_EXPS, PYRE_T_FFN_GATE_INP_SHEXP, PYRE_T_FFN_GATE_SHEXP, PYRE_T_FFN_UP_SHEXP, PYRE_T_FFN_DOWN_SHEXP,
   PYRE_T_INDEXER_Q_PROJ, PYRE_T_INDEXER_K_PROJ, PYRE_T_INDEXER_Q_NORM, PYRE_T_INDEXER_K_NORM,   /* blk.N.indexer.* (qwen4exp_gguf.rs:501): all attention layers or none */
+  PYRE_T_PLE_KEY, PYRE_T_PLE_VALUE, PYRE_T_PLE_NORM_KEY, PYRE_T_PLE_NORM_QUERY, PYRE_T_PLE_NORM_CONV, PYRE_T_PLE_CONV1D,   /* blk.N.ple_{key,value,norm_key,norm_query,norm_conv,conv1d}.weight (:505): the layers of ple.layers; a layer has all six or none */
   PYRE_LAYER_SLOTS
 };
-enum { PYRE_G_TOKEN_EMBD = 0, PYRE_G_OUTPUT_HC_NORM, PYRE_G_OUTPUT_HC_DOWN, PYRE_G_OUTPUT_HC_UP, PYRE_G_OUTPUT, PYRE_GLOBAL_SLOTS };
+enum { PYRE_G_TOKEN_EMBD = 0, PYRE_G_OUTPUT_HC_NORM, PYRE_G_OUTPUT_HC_DOWN, PYRE_G_OUTPUT_HC_UP, PYRE_G_OUTPUT, PYRE_G_PLE_TOKEN_EMBD /* per_layer_token_embd.weight (:512) */, PYRE_GLOBAL_SLOTS };
 
 /* Cfg (qwen4exp_gguf.rs:18-26), the fields the decode loop uses. */
 typedef struct {
@@ -217,6 +218,13 @@ typedef struct {
   /* trained context length and the context the model is built for (Cfg::ctx_train, Cfg::max_ctx): ctx > ctx_train > 0
    * switches the YaRN frequency table and magnitude factor on (qn_ctx::rope_inv, src/qn_ctx.rs:164-185). */
   int32_t ctx_train, ctx;
+  /* Per-layer n-gram embeddings, PLE (qwen4exp_gguf.rs:22-23, 477-480, ple_rows :1390-1407, ple :1409-1434): n-gram length
+   * (0 or 1 = none; at most 8), table heads per n-gram length ((ple_ngram - 1) * ple_per_gram <= 16 heads), conv kernel
+   * length (dilation = ple_ngram), width of a table row, the token id that cuts an n-gram's context; per n-gram position a
+   * 64-bit multiplier, per head an offset into the table and a modulus.  A layer has PLE when its PYRE_T_PLE_* slots are set. */
+  int32_t ple_ngram, ple_per_gram, ple_conv_k, ple_dim;
+  uint32_t ple_eos; int32_t ple_reserved;
+  uint64_t ple_mult[8], ple_off[16], ple_vocab[16];
 } pyre_model_cfg;
 
 /* ---- GGUF container (host only, no GPU needed): Gguf::open / mat / meta accessors, src/model/gguf_q.rs:250-336 --------
@@ -242,7 +250,7 @@ long   pyre_gguf_meta_arr_u64(const pyre_gguf* g, const char* key, uint64_t* out
  * keys, tensors by their GGUF names (blk.N.*, token_embd, output_hc_*, output or the tied embedding).  kv_bits and
  * kv_recent are run-time settings of the reference, not file contents, and so is the context the model is built for
  * (qn_ctx::startup_tokens, PYRE_QN_CTX).  The QSA indexer is taken when `attention.indexer.head_count` > 0 and the
- * indexer tensors exist.  Files with PLE layers are refused. */
+ * indexer tensors exist; PLE layers (`ple.layers` and the ple.* keys, :468-480) when the file lists them. */
 int   pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_recent, int ctx_tokens /* 0: the trained context */, pyre_model** out);
 /* Copies (and re-lays-out) every tensor into device memory; the caller's buffers are free afterwards. */
 int   pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* layer_tensors /*[n_layers][PYRE_LAYER_SLOTS]*/,
@@ -266,7 +274,9 @@ int   pyre_state_restore(pyre_ctx* ctx, pyre_state* s, const pyre_snap* snap);
 void  pyre_snap_destroy(pyre_snap* snap);
 size_t pyre_snap_bytes(const pyre_snap* snap);
 int   pyre_snap_len(const pyre_snap* snap);
-/* Test access to the recurrent state: li-th DeltaNet layer's S [nv][dk][dv] and conv [(k-1)][ch]; ai-th attention layer's f32 K / V rows [len][nkv*hd]. */
+/* Test access to the recurrent state: li-th DeltaNet layer's S [nv][dk][dv] and conv [(k-1)][ch]; ai-th attention layer's f32 K / V rows [len][nkv*hd];
+ * pi-th PLE layer's history [(ple_conv_k-1)*ple_ngram][hc*d], oldest first (State::ple_hist, :196; rows before position 0 are zero). */
+int   pyre_state_read_ple(pyre_ctx* ctx, pyre_state* s, int pi, float* hist_host);
 int   pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, float* ssm_host);
 int   pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, float* v_host);
 /* forward: append n tokens (any n >= 1; processed in windows of up to 8), logits of the last one -> logits_host[vocab]. */

@@ -542,6 +542,62 @@ void hc_combine(int d, int hc, float* x, const float* out, const float* inj, int
   for (int ti = 0; ti < t; ++ti) for (int s = 0; s < hc; ++s) { float w = 2.0f * sigm(inj[ti * hc + s]); float* r = x + ((size_t)ti * hc + s) * d; for (int i = 0; i < d; ++i) r[i] += out[(size_t)ti * d + i] * w; }
 }
 
+
+// ---------- per-layer n-gram embeddings (PLE) ------------------------------------------------------
+// ple_rows, qwen4exp_gguf.rs:1390-1407
+bool ple_rows(const OrcCfg& c, const OrcTensor& tab, const uint32_t* tokens, int start, int t, float* emb) {
+  const int ng = c.ple_ngram, nh = (ng - 1) * c.ple_per_gram, hd = c.ple_dim;
+  int qk, bs; if (!geom(tab.ty, &qk, &bs) || hd % qk || (int)tab.cols != hd) return false; const size_t rb = (size_t)hd / qk * bs;
+  for (int ti = 0; ti < t; ++ti) {
+    const int p = start + ti;
+    uint64_t ctx[8]; for (int s = 0; s < ng; ++s) ctx[s] = tokens[p];
+    bool cut = false;
+    for (int s = 1; s < ng; ++s) {
+      const bool none = cut || p < s; const uint32_t tk = none ? 0 : tokens[p - s];
+      cut = cut || none || tk == c.ple_eos; ctx[s] = cut ? (uint64_t)c.ple_eos : (uint64_t)tk;
+    }
+    for (int n = 2; n <= ng; ++n) {
+      uint64_t mixed = ctx[0] * c.ple_mult[0];                       // wrapping
+      for (int j = 1; j < n; ++j) mixed ^= ctx[j] * c.ple_mult[j];
+      for (int gi = 0; gi < c.ple_per_gram; ++gi) {
+        const int h = (n - 2) * c.ple_per_gram + gi; const uint64_t row = mixed % c.ple_vocab[h] + c.ple_off[h];
+        if (row >= tab.rows) return false;
+        if (!dequant(tab.ty, (const uint8_t*)tab.data + row * rb, hd, emb + ((size_t)ti * nh + h) * hd)) return false;
+      }
+    }
+  }
+  return true;
+}
+// ple, qwen4exp_gguf.rs:1409-1434
+bool ple_apply(const OrcCfg& c, const OrcTensor* key, const OrcTensor* value, const float* nk, const float* nq, const float* nc, const float* conv,
+               std::vector<float>& hist, const float* emb, float* x, int t, int th) {
+  const int d = c.d, hc = c.hc, w = hc * d, dil = c.ple_ngram, K = c.ple_conv_k, hl = (K - 1) * dil;
+  if ((int)key->rows != w || (int)value->rows != d || key->cols != value->cols || (int)hist.size() != hl * w) return false;
+  std::vector<float> kt((size_t)t * w), vt((size_t)t * d);
+  if (!mm(key, emb, t, kt.data(), th) || !mm(value, emb, t, vt.data(), th)) return false;
+  std::vector<float> gated(w), nrm(w), kk(d), q(d);
+  for (int ti = 0; ti < t; ++ti) {
+    float* xt = x + (size_t)ti * w;
+    for (int s = 0; s < hc; ++s) {
+      memcpy(kk.data(), &kt[(size_t)ti * w + (size_t)s * d], sizeof(float) * d); rms_inplace(kk.data(), nk + (size_t)s * d, c.eps, d);
+      rms(xt + (size_t)s * d, nq + (size_t)s * d, c.eps, q.data(), d);
+      const float sc = dot(kk.data(), q.data(), d) / sqrtf((float)d);
+      const float g = sc != sc ? sc : sigm(copysignf(1.0f, sc) * sqrtf(fmaxf(fabsf(sc), 1e-6f)));      // f32::signum: +-1 by the sign bit (also of zero), NaN for NaN
+      for (int i = 0; i < d; ++i) gated[(size_t)s * d + i] = vt[(size_t)ti * d + i] * g;
+    }
+    nrm = gated;
+    for (int s = 0; s < hc; ++s) rms_inplace(nrm.data() + (size_t)s * d, nc + (size_t)s * d, c.eps, d);
+    // depthwise causal conv, dilation = n-gram length: taps K-1 (now), then (K-1-k)*dil rows back; hist oldest first
+    for (int ch = 0; ch < w; ++ch) {
+      float o = conv[(size_t)ch * K + K - 1] * nrm[ch];
+      for (int k = 0; k < K - 1; ++k) { const int back = (K - 1 - k) * dil; o += conv[(size_t)ch * K + k] * hist[(size_t)(hl - back) * w + ch]; }
+      xt[ch] += gated[ch] + silu(o);
+    }
+    hist.erase(hist.begin(), hist.begin() + w); hist.insert(hist.end(), nrm.begin(), nrm.end());
+  }
+  return true;
+}
+
 }  // namespace
 
 // ---------- model ------------------------------------------------------------------------------
@@ -554,11 +610,13 @@ struct OrcModel {
   const OrcTensor& T(int il, int slot) const { return lt[(size_t)il * ORC_LAYER_SLOTS + slot]; }
   const float* V(int il, int slot) const { return vec[(size_t)il * ORC_LAYER_SLOTS + slot].data(); }
   bool full(int il) const { return (il + 1) % c.full_every == 0; }
+  bool has_ple(int il) const { return c.ple_ngram > 1 && T(il, ORC_PLE_KEY).data != nullptr; }
 };
-struct OrcCkpt { std::vector<std::vector<float>> conv, ssm; };
+struct OrcCkpt { std::vector<std::vector<float>> conv, ssm, ple_hist; };
 struct OrcState {
   std::vector<uint32_t> tokens;
   std::vector<std::vector<float>> conv, ssm, k, v, ik, ib;   // ik / ib: raw index keys [pos][idx_hd], pooled block keys [block][idx_hd]
+  std::vector<std::vector<float>> ple_hist;                  // per PLE layer: the last (conv_k-1)*ngram normalised rows [hc*d], oldest first (:196)
   std::vector<OrcCkpt> ck;  // state after each token of the last forward_multi
 };
 
@@ -637,7 +695,9 @@ OrcModel* orc_model_create(const OrcCfg* cfg, const OrcTensor* lt, const OrcTens
   OrcModel* m = new OrcModel(); m->c = *cfg; m->threads = threads;
   m->lt.assign(lt, lt + (size_t)cfg->n_layers * ORC_LAYER_SLOTS); for (int i = 0; i < ORC_GLOBAL_SLOTS; ++i) m->g[i] = globals[i];
   m->vec.resize(m->lt.size());
-  static const int vs[] = {ORC_HCA_NORM, ORC_HCF_NORM, ORC_ATTN_QN, ORC_ATTN_KN, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_SH_GATE_INP, ORC_IDX_QN, ORC_IDX_KN};
+  if (cfg->ple_ngram > 8 || (cfg->ple_ngram > 1 && ((cfg->ple_ngram - 1) * cfg->ple_per_gram > 16 || cfg->ple_conv_k < 1))) { delete m; return nullptr; }
+  static const int vs[] = {ORC_HCA_NORM, ORC_HCF_NORM, ORC_ATTN_QN, ORC_ATTN_KN, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_SH_GATE_INP, ORC_IDX_QN, ORC_IDX_KN,
+                           ORC_PLE_NK, ORC_PLE_NQ, ORC_PLE_NC, ORC_PLE_CONV};
   for (int il = 0; il < cfg->n_layers; ++il) for (int s : vs) if (!to_vec(m->T(il, s), m->vec[(size_t)il * ORC_LAYER_SLOTS + s])) { delete m; return nullptr; }
   if (!to_vec(m->g[ORC_G_HEAD_NORM], m->head_norm)) { delete m; return nullptr; }
   m->rope_inv.resize(cfg->n_rot / 2); m->mscale = orc_rope_inv_yarn(cfg->n_rot, cfg->rope_base, cfg->ctx_train, cfg->ctx, m->rope_inv.data());
@@ -650,6 +710,7 @@ OrcState* orc_state_create(const OrcModel* m) {  // new_state, qwen4exp_gguf.rs:
   for (int il = 0; il < c.n_layers; ++il) {
     if (m->full(il)) { s->k.emplace_back(); s->v.emplace_back(); s->ik.emplace_back(); s->ib.emplace_back(); }
     else { s->conv.emplace_back((size_t)(c.conv_k - 1) * ch, 0.0f); s->ssm.emplace_back((size_t)c.lin_nv * c.lin_dk * c.lin_dv, 0.0f); }
+    if (m->has_ple(il)) s->ple_hist.emplace_back((size_t)(c.ple_conv_k - 1) * c.ple_ngram * c.hc * c.d, 0.0f);      // :1350
   }
   return s;
 }
@@ -661,6 +722,14 @@ float* orc_state_k(OrcState* s, int ai) { return s->k[ai].data(); }
 float* orc_state_v(OrcState* s, int ai) { return s->v[ai].data(); }
 float* orc_state_ik(OrcState* s, int ai) { return s->ik[ai].data(); }
 float* orc_state_ib(OrcState* s, int ai) { return s->ib[ai].data(); }
+float* orc_state_ple_hist(OrcState* s, int pi) { return s->ple_hist[pi].data(); }
+int orc_ple_rows(const OrcCfg* c, const OrcTensor* tab, const uint32_t* tokens, int start, int t, float* emb) { return ple_rows(*c, *tab, tokens, start, t, emb) ? 0 : -1; }
+int orc_ple(const OrcCfg* c, const OrcTensor* key, const OrcTensor* value, const float* nk, const float* nq, const float* nc, const float* conv,
+            float* hist, const float* emb, float* x, int t, int threads) {
+  const size_t n = (size_t)(c->ple_conv_k - 1) * c->ple_ngram * c->hc * c->d; std::vector<float> h(hist, hist + n);
+  if (!ple_apply(*c, key, value, nk, nq, nc, conv, h, emb, x, t, threads)) return -1;
+  memcpy(hist, h.data(), n * sizeof(float)); return 0;
+}
 
 // forward_inner, qwen4exp_gguf.rs:2087-2157 (host branch :2134-2142, head :2150-2153)
 int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, float* logits) {
@@ -670,9 +739,18 @@ int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, flo
   std::vector<float> x((size_t)t * hc * d), e(d);
   const OrcTensor& embd = m->g[ORC_G_EMBD]; int qk, bs; if (!geom(embd.ty, &qk, &bs)) return -1; size_t erb = (size_t)d / qk * bs;
   for (int ti = 0; ti < t; ++ti) { dequant(embd.ty, (const uint8_t*)embd.data + ids[ti] * erb, d, e.data()); for (int s = 0; s < hc; ++s) memcpy(&x[((size_t)ti * hc + s) * d], e.data(), sizeof(float) * d); }
-  int li = 0, ai = 0;
-  std::vector<float> mixed((size_t)t * d), inj((size_t)t * hc), o((size_t)t * d);
+  int li = 0, ai = 0, pi = 0;
+  std::vector<float> mixed((size_t)t * d), inj((size_t)t * hc), o((size_t)t * d), emb;
+  if (c.ple_ngram > 1 && m->g[ORC_G_PLE_TAB].data) {      // :2093
+    emb.resize((size_t)t * (c.ple_ngram - 1) * c.ple_per_gram * c.ple_dim);
+    if (!ple_rows(c, m->g[ORC_G_PLE_TAB], st->tokens.data(), start, t, emb.data())) return -9;
+  }
   for (int il = 0; il < c.n_layers; ++il) {
+    if (m->has_ple(il)) {                                   // :2112
+      if (emb.empty() || !ple_apply(c, &m->T(il, ORC_PLE_KEY), &m->T(il, ORC_PLE_VALUE), m->V(il, ORC_PLE_NK), m->V(il, ORC_PLE_NQ), m->V(il, ORC_PLE_NC), m->V(il, ORC_PLE_CONV),
+                                    st->ple_hist[pi], emb.data(), x.data(), t, th)) return -9;
+      ++pi;
+    }
     if (hc_mix(d, hc, c.eps, m->V(il, ORC_HCA_NORM), &m->T(il, ORC_HCA_DOWN), &m->T(il, ORC_HCA_INJECT), &m->T(il, ORC_HCA_UP), x.data(), t, mixed.data(), inj.data(), th) == false) return -2;
     if (m->full(il)) {  // attn, :1441-1446
       int nh = c.n_head, nkv = c.n_kv, hd = c.hd; size_t row = (size_t)nkv * hd;
@@ -714,14 +792,14 @@ int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, flo
 // decode (:2357-2360), recurrent-state checkpoints after each token for spec_keep.
 int orc_forward_multi(const OrcModel* m, OrcState* st, const uint32_t* ids, int n, float* logits) {
   st->ck.clear();
-  for (int i = 0; i < n; ++i) { int rc = orc_forward(m, st, ids + i, 1, logits + (size_t)i * m->c.vocab); if (rc) return rc; st->ck.push_back({st->conv, st->ssm}); }
+  for (int i = 0; i < n; ++i) { int rc = orc_forward(m, st, ids + i, 1, logits + (size_t)i * m->c.vocab); if (rc) return rc; st->ck.push_back({st->conv, st->ssm, st->ple_hist}); }
   return 0;
 }
 // spec_keep, qwen4exp_gguf.rs:2495-2515
 int orc_spec_keep(const OrcModel* m, OrcState* st, int t, int keep) {
   if (keep >= t || t < 2) return 0; if (keep < 1) keep = 1; if ((int)st->ck.size() < t) return -1;
   size_t n = st->tokens.size() - t + keep; st->tokens.resize(n);
-  st->conv = st->ck[keep - 1].conv; st->ssm = st->ck[keep - 1].ssm;
+  st->conv = st->ck[keep - 1].conv; st->ssm = st->ck[keep - 1].ssm; st->ple_hist = st->ck[keep - 1].ple_hist;      // ple_ck, :2417
   size_t row = (size_t)m->c.n_kv * m->c.hd; for (auto& k : st->k) k.resize(n * row); for (auto& v : st->v) v.resize(n * row);
   size_t ihd = m->c.idx_hd, ir = m->c.idx_ratio < 1 ? 1 : m->c.idx_ratio;       // :2509-2513
   for (auto& k : st->ik) if (!k.empty()) k.resize(n * ihd);

@@ -59,9 +59,10 @@ enum {
   ORC_LIN_QKV, ORC_LIN_Z, ORC_LIN_BETA, ORC_LIN_ALPHA, ORC_LIN_A, ORC_LIN_DT, ORC_LIN_CONV, ORC_LIN_NORM, ORC_LIN_OUT,
   ORC_ROUTER, ORC_GATE_E, ORC_UP_E, ORC_DOWN_E, ORC_SH_GATE_INP, ORC_SH_GATE, ORC_SH_UP, ORC_SH_DOWN,
   ORC_IDX_Q, ORC_IDX_K, ORC_IDX_QN, ORC_IDX_KN,                     /* blk.N.indexer.{q_proj,k_proj,q_norm,k_norm}.weight (optional) */
+  ORC_PLE_KEY, ORC_PLE_VALUE, ORC_PLE_NK, ORC_PLE_NQ, ORC_PLE_NC, ORC_PLE_CONV,   /* blk.N.ple_{key,value,norm_key,norm_query,norm_conv,conv1d}.weight (layers listed in ple.layers, :505) */
   ORC_LAYER_SLOTS
 };
-enum { ORC_G_EMBD = 0, ORC_G_HEAD_NORM, ORC_G_HEAD_DOWN, ORC_G_HEAD_UP, ORC_G_OUT, ORC_GLOBAL_SLOTS };
+enum { ORC_G_EMBD = 0, ORC_G_HEAD_NORM, ORC_G_HEAD_DOWN, ORC_G_HEAD_UP, ORC_G_OUT, ORC_G_PLE_TAB /* per_layer_token_embd.weight (:512) */, ORC_GLOBAL_SLOTS };
 
 typedef struct {
   int32_t n_layers, d, hc, hc_lr, n_head, n_kv, hd, n_rot;
@@ -75,6 +76,12 @@ typedef struct {
   int32_t idx_nh, idx_hd, idx_ratio, idx_budget;
   /* trained context and the context the model is built for; ctx > ctx_train > 0 switches YaRN on (qn_ctx.rs:164-185) */
   int32_t ctx_train, ctx;
+  /* per-layer n-gram embeddings (qwen4exp_gguf.rs:22-23, 477-480): n-gram length (0 = none), table heads per n-gram length,
+   * conv kernel length, width of a table row, the token that cuts an n-gram's context; per position of the n-gram a 64-bit
+   * multiplier, per head an offset into the table and a modulus */
+  int32_t ple_ngram, ple_per_gram, ple_conv_k, ple_dim;
+  uint32_t ple_eos; int32_t ple_reserved;
+  uint64_t ple_mult[8], ple_off[16], ple_vocab[16];
 } OrcCfg;
 
 int    orc_type_geom(uint32_t ty, int* elems, int* bytes);
@@ -152,6 +159,12 @@ float*    orc_state_ssm(OrcState*, int li);
 float*    orc_state_k(OrcState*, int ai);
 float*    orc_state_v(OrcState*, int ai);
 float*    orc_state_ik(OrcState*, int ai);
+float*    orc_state_ple_hist(OrcState*, int pi);      /* pi-th PLE layer: [(conv_k-1)*ngram][hc*d], oldest first */
+/* ple_rows (qwen4exp_gguf.rs:1390-1407): table rows of positions start .. start+t-1 of `tokens` -> emb [t][heads*dim] */
+int       orc_ple_rows(const OrcCfg* c, const OrcTensor* tab, const uint32_t* tokens, int start, int t, float* emb);
+/* ple (qwen4exp_gguf.rs:1409-1434): x [t][hc*d] += gated + silu(conv); hist [(conv_k-1)*ngram][hc*d] advanced by t rows */
+int       orc_ple(const OrcCfg* c, const OrcTensor* key, const OrcTensor* value, const float* nk, const float* nq, const float* nc, const float* conv,
+                  float* hist, const float* emb, float* x, int t, int threads);
 float*    orc_state_ib(OrcState*, int ai);
 /* Model::forward: append ids, return logits of the last token in logits[vocab]. */
 int       orc_forward(const OrcModel*, OrcState*, const uint32_t* ids, int n, float* logits);

@@ -153,7 +153,8 @@ int pyre_row_launch(pyre_ctx* ctx, const QMatDev& m, const uint32_t* row_idx_dev
 // chosen row is dequantized into out_dev in the same launch (the next token's embedding).
 // step_dev (optional, device int[2]): step_dev[0] is incremented first (the position of the token being started) and the
 // id goes to mirror[step_dev[0] - step_dev[1]] instead of mirror[0].
-int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev, int* step_dev);
+// hist (optional, with step_dev): the token history by position; the pick is also stored at the position it starts
+int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out_dev, int* step_dev, uint32_t* hist = nullptr);
 
 // ---- IQ3_S GEMM on the matrix cores (gemm_m.hip), 1 <= t <= 8, matrices in FMT_IQ3_S_M ------------------------------------
 // The activations reach the kernel as its f16 operand: every value as two halves, x = h1 + h2 * 2^-11 with h1 = f16(x) and
@@ -232,6 +233,22 @@ struct RouteSrc { const float* p; int nsl; int r64; };
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr);
 // K parts the gate/up dot products are summed in (1 or 2; k_moe_gu)
 int pyre_moe_gu_parts(const MoeDev& m);
+
+// ---- per-layer n-gram embeddings, PLE (ple.hip; ple_rows / ple, qwen4exp_gguf.rs:1390-1434) ----------------------------------
+struct PleCfg { int ngram, per_gram, conv_k, dim; uint32_t eos; unsigned long long mult[8], off[16], vocab[16]; };
+// kv = [key ; value] rows (hc*d + d) x (heads * dim); ring: the normalised rows of the last positions, row of position p at
+// ring[(p & mask) * hc*d] (a ring indexed by position: a rollback needs no copy, the rows are rewritten when their positions
+// come again); mask + 1 >= (conv_k - 1) * ngram + 8.
+struct PleDev { QMatDev kv; const float* nk; const float* nq; const float* nc; const float* conv; float* ring; int mask; };
+struct PleWork { uint32_t* idx; float* emb; float* kv; float* gated; };     // [8*16] table rows, [8][heads*dim], [8][hc*d + d], [8][hc*d]
+size_t pyre_ple_work_bytes(const PleCfg& c, int d, int hc);
+void   pyre_ple_work_carve(const PleCfg& c, int d, int hc, void* base, PleWork* w);
+// table rows of the window's positions (start or *posp .. + t - 1 of the token history) -> w.emb; once per window
+int pyre_ple_rows_launch(pyre_ctx* ctx, const PleCfg& c, const QMatDev& tab, const PleWork& w, const uint32_t* tokens_dev, int start, const int* posp, int t);
+// One PLE layer: the streams are read from x_in as in pyre_hc_mix_launch (pending residual update applied first), and
+// x_out [t][hc][d] = updated streams + gated + silu(conv); the layer's ring advances by t positions.
+int pyre_ple_launch(pyre_ctx* ctx, const PleCfg& c, const PleDev& p, const PleWork& w, int d, int hc, float eps, const float* x_in, int in_ss, int in_ts, float* x_out,
+                    const float* comb_out, const MoeOut* comb_moe, const float* comb_inj, int start, const int* posp, int t);
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows

@@ -3,6 +3,7 @@
 // Follows Gguf::open / shard_paths / Meta (src/model/gguf_q.rs:250-336) and Model::load's metadata keys and tensor
 // names (src/model/qwen4exp_gguf.rs:462-524).
 #include "formats.h"
+#include <algorithm>
 #include <errno.h>
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -222,7 +223,19 @@ int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_re
   const bool has_idx = c.idx_nh > 0 && g->tensors.count("blk." + std::to_string((c.full_every > 0 ? c.full_every : 1) - 1) + ".indexer.q_proj.weight") > 0;      // :489 looks at block 3
   if (!has_idx) c.idx_nh = 0;
   if (missing) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_load_gguf: gguf key %s", miss.c_str());
-  { auto it = g->meta.find("qwen4exp.ple.layers"); if (it != g->meta.end() && it->second.kind == Meta::A && !it->second.a.empty()) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_load_gguf: per-layer-embedding (PLE) layers are not supported"); }
+  // PLE, qwen4exp_gguf.rs:468-480: the listed layers carry blk.N.ple_*; the hash parameters are arrays of u64
+  std::vector<int> ple_layers;
+  { auto it = g->meta.find("qwen4exp.ple.layers"); if (it != g->meta.end() && it->second.kind == Meta::A) for (const Meta& e2 : it->second.a) { uint64_t v = 0; if (e2.as_u64(&v)) ple_layers.push_back((int)v); } }
+  if (!ple_layers.empty()) {
+    c.ple_ngram = (int)ku("ple.ngram_size", 0); c.ple_per_gram = (int)ku("ple.heads_per_ngram", 0); c.ple_conv_k = (int)ku("ple.conv_kernel", 0);
+    c.ple_eos = (uint32_t)ku("ple.eos_token_id", 0); c.ple_dim = (int)ku("embedding_length_per_layer_input", 0);
+    auto arr = [&](const char* key, uint64_t* dst, size_t cap) -> long { auto it = g->meta.find(std::string("qwen4exp.") + key); if (it == g->meta.end() || it->second.kind != Meta::A) return -1;
+      size_t n = 0; for (const Meta& e2 : it->second.a) { uint64_t v = 0; if (!e2.as_u64(&v)) return -1; if (n < cap) dst[n] = v; ++n; } return (long)n; };
+    const long nm = arr("ple.layer_multipliers", c.ple_mult, 8), no = arr("ple.head_offsets", c.ple_off, 16), nv = arr("ple.head_vocab_sizes", c.ple_vocab, 16);
+    const long nh = (long)(c.ple_ngram - 1) * c.ple_per_gram;
+    if (c.ple_ngram < 2 || c.ple_ngram > 8 || nh < 1 || nh > 16 || nm < c.ple_ngram || nm > 8 || no < nh || nv < nh || no > 16 || nv > 16)
+      return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_load_gguf: PLE with n-grams of %d, %d heads per length, %ld multipliers, %ld offsets, %ld sizes is unsupported", c.ple_ngram, c.ple_per_gram, nm, no, nv);
+  }
   auto emb = g->tensors.find("token_embd.weight");
   if (emb == g->tensors.end() || emb->second.shape.size() < 2) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_load_gguf: token_embd");
   c.vocab = (int)emb->second.shape[1];
@@ -245,8 +258,12 @@ int pyre_model_load_gguf(pyre_ctx* ctx, const char* path, int kv_bits, int kv_re
     ok = ok && get(p + "ffn_gate_inp.weight", &T[PYRE_T_FFN_GATE_INP]) && get(p + "ffn_gate_exps.weight", &T[PYRE_T_FFN_GATE_EXPS]) && get(p + "ffn_up_exps.weight", &T[PYRE_T_FFN_UP_EXPS]) &&
          get(p + "ffn_down_exps.weight", &T[PYRE_T_FFN_DOWN_EXPS]) && get(p + "ffn_gate_inp_shexp.weight", &T[PYRE_T_FFN_GATE_INP_SHEXP]) && get(p + "ffn_gate_shexp.weight", &T[PYRE_T_FFN_GATE_SHEXP]) &&
          get(p + "ffn_up_shexp.weight", &T[PYRE_T_FFN_UP_SHEXP]) && get(p + "ffn_down_shexp.weight", &T[PYRE_T_FFN_DOWN_SHEXP]);
+    if (ok && std::find(ple_layers.begin(), ple_layers.end(), il) != ple_layers.end())
+      ok = get(p + "ple_key.weight", &T[PYRE_T_PLE_KEY]) && get(p + "ple_value.weight", &T[PYRE_T_PLE_VALUE]) && get(p + "ple_norm_key.weight", &T[PYRE_T_PLE_NORM_KEY]) &&
+           get(p + "ple_norm_query.weight", &T[PYRE_T_PLE_NORM_QUERY]) && get(p + "ple_norm_conv.weight", &T[PYRE_T_PLE_NORM_CONV]) && get(p + "ple_conv1d.weight", &T[PYRE_T_PLE_CONV1D]);
     if (!ok) return pyre_fail(ctx, rc, "pyre_model_load_gguf: %s", e.c_str());
   }
+  if (!ple_layers.empty() && !get("per_layer_token_embd.weight", &gl[PYRE_G_PLE_TOKEN_EMBD])) return pyre_fail(ctx, rc, "pyre_model_load_gguf: %s", e.c_str());
   bool ok = get("token_embd.weight", &gl[PYRE_G_TOKEN_EMBD]) && get("output_hc_norm.weight", &gl[PYRE_G_OUTPUT_HC_NORM]) && get("output_hc_down.weight", &gl[PYRE_G_OUTPUT_HC_DOWN]) &&
             get("output_hc_up.weight", &gl[PYRE_G_OUTPUT_HC_UP]) && get(g->tensors.count("output.weight") ? "output.weight" : "token_embd.weight", &gl[PYRE_G_OUTPUT]);
   if (!ok) return pyre_fail(ctx, rc, "pyre_model_load_gguf: %s", e.c_str());

@@ -14,6 +14,7 @@ struct Layer {
   QMatDev proj{};            // attention: [q ; k ; v]   DeltaNet: [qkv ; z ; beta ; alpha]
   QMatDev outp{};            // attn_output / ssm_out
   AttnDev attn{}; GdnDev gdn{}; MoeDev moe{}; QsaDev qsa{};
+  bool ple = false; PleDev pld{}; int ple_index = 0;      // per-layer n-gram embeddings in front of the layer (ring pointer lives in the state)
   int mix_index = 0;         // index among the attention or among the DeltaNet layers
 };
 
@@ -30,6 +31,7 @@ struct pyre_model {
   void* work = nullptr; HcWork hw{}; MoeWork mw{};
   float *x = nullptr, *x2 = nullptr, *mixed = nullptr, *inj_a = nullptr, *inj_f = nullptr, *proj = nullptr, *core = nullptr, *o = nullptr, *y = nullptr, *hbuf = nullptr, *logits = nullptr, *co = nullptr, *emb = nullptr, *rpart = nullptr;
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
+  PleCfg plc{}; QMatDev ple_tab{}; PleWork pw{}; int n_ple = 0, ple_ring = 0;      // PLE: hash parameters, the token table, window workspace, ring rows per layer
   uint16_t* aop = nullptr;      // the f16 operand a producer kernel leaves for the matrix-core GEMV that follows it (one at a time: the launches are stream-ordered)
 };
 
@@ -41,6 +43,7 @@ struct pyre_state {
   std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
   std::vector<QsaBuf> qsa; QsaWork qw{};                          // indexer keys per attention layer; selection workspace
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
+  uint32_t* tokens_dev = nullptr; std::vector<float*> ple_ring;     // PLE models: the token history by position; per PLE layer the ring of normalised rows
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
   std::vector<int> graph_cur;                                    // which half of every DeltaNet double buffer the captured step works on
 };
@@ -137,6 +140,15 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
     L.full = (il + 1) % c.full_every == 0;
     if ((rc = B.hc(T[PYRE_T_HC_ATTN_NORM], T[PYRE_T_HC_ATTN_DOWN], &T[PYRE_T_HC_ATTN_INJECT], T[PYRE_T_HC_ATTN_UP], &L.hca, &tok_bytes))) return rc;
     if ((rc = B.hc(T[PYRE_T_HC_FFN_NORM], T[PYRE_T_HC_FFN_DOWN], &T[PYRE_T_HC_FFN_INJECT], T[PYRE_T_HC_FFN_UP], &L.hcf, &tok_bytes))) return rc;
+    if (c.ple_ngram > 1 && T[PYRE_T_PLE_KEY].data) {
+      const pyre_tensor* kvg[2] = {&T[PYRE_T_PLE_KEY], &T[PYRE_T_PLE_VALUE]}; const size_t wd = (size_t)c.hc * c.d; const int ein = (c.ple_ngram - 1) * c.ple_per_gram * c.ple_dim;
+      if (!gl[PYRE_G_PLE_TOKEN_EMBD].data || !T[PYRE_T_PLE_VALUE].data) return B.fail(PYRE_E_ARG, "a PLE layer needs per_layer_token_embd and all six ple_* tensors");
+      if (kvg[0]->rows != wd || kvg[1]->rows != (uint64_t)c.d || kvg[0]->cols != (uint64_t)ein || kvg[1]->cols != (uint64_t)ein) return B.fail(PYRE_E_SHAPE, "ple_key / ple_value shapes");
+      L.ple = true; L.ple_index = m->n_ple++; size_t pb = 0;
+      if ((rc = B.cat(kvg, 2, &L.pld.kv, &pb)) || (rc = B.vec(T[PYRE_T_PLE_NORM_KEY], wd, &L.pld.nk)) || (rc = B.vec(T[PYRE_T_PLE_NORM_QUERY], wd, &L.pld.nq)) ||
+          (rc = B.vec(T[PYRE_T_PLE_NORM_CONV], wd, &L.pld.nc)) || (rc = B.vec(T[PYRE_T_PLE_CONV1D], wd * c.ple_conv_k, &L.pld.conv))) return rc;
+      tok_bytes += pb;
+    }
     if (L.full) {
       L.mix_index = m->n_attn++;
       const pyre_tensor* grp[5] = {&T[PYRE_T_ATTN_Q], &T[PYRE_T_ATTN_K], &T[PYRE_T_ATTN_V], &T[PYRE_T_INDEXER_Q_PROJ], &T[PYRE_T_INDEXER_K_PROJ]};
@@ -176,6 +188,18 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
     if ((rc = B.vec(T[PYRE_T_FFN_GATE_INP_SHEXP], c.d, &mo.sh_gate_inp))) return rc;
     tok_bytes += router_b + sh + (ge + ue + de) / c.n_exp * c.top_k;
   }
+  if (m->n_ple > 0) {
+    if (c.ple_ngram > 8 || c.ple_per_gram < 1 || (c.ple_ngram - 1) * c.ple_per_gram > 16 || c.ple_conv_k < 1 || c.ple_conv_k > 64 || c.ple_dim < 64 || c.ple_dim % 64)
+      return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_model_create: PLE with n-grams of %d, %d heads per length, conv kernel %d, rows of %d is unsupported", c.ple_ngram, c.ple_per_gram, c.ple_conv_k, c.ple_dim);
+    if ((rc = B.one(gl[PYRE_G_PLE_TOKEN_EMBD], &m->ple_tab, nullptr))) return rc;
+    m->plc.ngram = c.ple_ngram; m->plc.per_gram = c.ple_per_gram; m->plc.conv_k = c.ple_conv_k; m->plc.dim = c.ple_dim; m->plc.eos = c.ple_eos;
+    for (int i = 0; i < 8; ++i) m->plc.mult[i] = c.ple_mult[i];
+    for (int i = 0; i < 16; ++i) { m->plc.off[i] = c.ple_off[i]; m->plc.vocab[i] = c.ple_vocab[i]; }
+    for (int h = 0; h < (c.ple_ngram - 1) * c.ple_per_gram; ++h) if (c.ple_vocab[h] == 0 || c.ple_off[h] + c.ple_vocab[h] > (uint64_t)m->ple_tab.rows) return B.fail(PYRE_E_SHAPE, "a PLE head's rows lie outside per_layer_token_embd");
+    if (m->ple_tab.cols != c.ple_dim) return B.fail(PYRE_E_SHAPE, "per_layer_token_embd row width");
+    int ring = 16; while (ring < (c.ple_conv_k - 1) * c.ple_ngram + 8) ring *= 2; m->ple_ring = ring;
+    tok_bytes += (size_t)(c.ple_ngram - 1) * c.ple_per_gram * (c.ple_dim / m->ple_tab.gel * m->ple_tab.gbytes);
+  }
   if ((rc = B.one(gl[PYRE_G_TOKEN_EMBD], &m->embd, nullptr, mlay))) return rc;
   if (m->embd.rows != c.vocab || m->embd.cols != c.d) return B.fail(PYRE_E_SHAPE, "token_embd shape");
   if ((rc = B.hc(gl[PYRE_G_OUTPUT_HC_NORM], gl[PYRE_G_OUTPUT_HC_DOWN], nullptr, gl[PYRE_G_OUTPUT_HC_UP], &m->head, &tok_bytes))) return rc;
@@ -190,8 +214,9 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
   int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));
   const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
+  const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(ple_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
@@ -200,6 +225,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
   m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
+  if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
   PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
   { uint4* op; float* ainv;      // and the context's operand buffer for a GEMV whose producer leaves f32 only, so that no step allocates
     if ((rc = pyre_gemm_m_scratch(ctx, (kmax + 255) / 256 * 256, &op, &ainv))) return rc; }
@@ -223,7 +249,8 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   size_t kvb = al256(pyre_kv_bytes(a0, s->cap)), awb = al256(pyre_attn_work_bytes(a0, s->cap));
   QsaDev q0{nullptr, nullptr, m->has_idx ? c.idx_nh : 0, c.idx_hd, c.idx_ratio < 1 ? 1 : c.idx_ratio, c.idx_budget};
   size_t qbb = al256(pyre_qsa_buf_bytes(q0, s->cap)), qwb = al256(pyre_qsa_work_bytes(q0, s->cap));
-  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * (kvb + qbb) + awb + qwb + 4096 + 256;
+  const size_t tkb = m->n_ple > 0 ? al256((size_t)s->cap * 4) : 0, prb = m->n_ple > 0 ? al256((size_t)m->ple_ring * c.hc * c.d * 4) : 0;
+  size_t total = (size_t)m->n_lin * (2 * cs + 2 * ss + ps) + (size_t)m->n_attn * (kvb + qbb) + awb + qwb + tkb + (size_t)m->n_ple * prb + 4096 + 256;
   hipError_t e = hipMalloc(&s->mem, total);
   if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_create: hipMalloc(%zu): %s", total, hipGetErrorString(e));
   uint8_t* p = (uint8_t*)s->mem; auto take = [&](size_t n) { void* r = p; p += n; return r; };
@@ -231,6 +258,7 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   for (int ai = 0; ai < m->n_attn; ++ai) { KvDev kv; pyre_kv_carve(a0, s->cap, take(kvb), &kv); s->kv.push_back(kv); s->packed.push_back(0); }
   pyre_attn_work_carve(a0, s->cap, take(awb), &s->aw);
   if (m->has_idx) { for (int ai = 0; ai < m->n_attn; ++ai) { QsaBuf qb; pyre_qsa_buf_carve(q0, s->cap, take(qbb), &qb); s->qsa.push_back(qb); } pyre_qsa_work_carve(q0, s->cap, take(qwb), &s->qw); }
+  if (m->n_ple > 0) { s->tokens_dev = (uint32_t*)take(tkb); for (int pi = 0; pi < m->n_ple; ++pi) s->ple_ring.push_back((float*)take(prb)); }
   s->step_dev = (int*)take(256);
   int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
   *out = S.release(); return PYRE_OK;
@@ -253,7 +281,7 @@ int pyre_model_max_window(const pyre_model* m) { return m ? 8 : 0; }
 // whatever the capacity).  It can be restored into any state of the same model with room for `len` positions.
 struct pyre_snap { const pyre_model* m; int len; std::vector<int> packed; void* mem; size_t bytes; };
 namespace {
-struct SnapPlan { size_t cs, ss, kf, ks_kq, kq, ksc, vf, vq, vsc, ik, ib, total; };
+struct SnapPlan { size_t cs, ss, kf, ks_kq, kq, ksc, vf, vq, vsc, ik, ib, tk, pl, total; };
 SnapPlan snap_plan(const pyre_model* m, int len) {
   const pyre_model_cfg& c = m->c; SnapPlan p{};
   const size_t row = (size_t)c.n_kv * c.hd, nb = ((size_t)len + 63) / 64;
@@ -261,7 +289,8 @@ SnapPlan snap_plan(const pyre_model* m, int len) {
   p.kf = al256(nb * row * 64 * 4); p.kq = al256(nb * (row / 8) * 64 * 4); p.ksc = al256(nb * (row / 32) * 64 * 4);
   p.vf = al256((size_t)len * row * 4); p.vq = al256((size_t)len * (row / 8) * 4); p.vsc = al256((size_t)len * (row / 32) * 4);
   if (m->has_idx) { p.ik = al256((size_t)len * c.idx_hd * 4); p.ib = al256(((size_t)len / c.idx_ratio + 63) / 64 * 64 * c.idx_hd * 4); }      // raw index keys; pooled block keys in whole groups of 64 blocks
-  p.total = (size_t)m->n_lin * (p.cs + p.ss) + (size_t)m->n_attn * (p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc + p.ik + p.ib) + 256;
+  if (m->n_ple > 0) { p.tk = al256((size_t)len * 4 + 4); p.pl = al256((size_t)(c.ple_conv_k - 1) * c.ple_ngram * c.hc * c.d * 4 + 4); }      // token history; per PLE layer the conv history
+  p.total = (size_t)m->n_lin * (p.cs + p.ss) + (size_t)m->n_attn * (p.kf + p.kq + p.ksc + p.vf + p.vq + p.vsc + p.ik + p.ib) + p.tk + (size_t)m->n_ple * p.pl + 256;
   return p;
 }
 // dir = 0: state -> snapshot buffer, 1: snapshot buffer -> state
@@ -286,6 +315,16 @@ int snap_copy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint8_t* buf, i
       size_t ibn = ((size_t)len / c.idx_ratio + 63) / 64 * 64 * c.idx_hd * 4;
       if (ibn) { PYRE_HIP(ctx, cp(s->qsa[ai].ib, ibn)); }
       q += p.ib;
+    }
+  }
+  if (m->n_ple > 0) {
+    if (len > 0) { PYRE_HIP(ctx, cp(s->tokens_dev, (size_t)len * 4)); }
+    q += p.tk;
+    const size_t wb = (size_t)c.hc * c.d * 4; const int hl = (c.ple_conv_k - 1) * c.ple_ngram;
+    for (int pi = 0; pi < m->n_ple; ++pi) {      // the rows of the last hl positions, oldest first (positions before 0 have no row)
+      uint8_t* q0 = q;
+      for (int j = 0; j < hl; ++j) { const int pos = len - hl + j; if (pos >= 0) { q = q0 + (size_t)j * wb; PYRE_HIP(ctx, cp(s->ple_ring[pi] + (size_t)(pos & (m->ple_ring - 1)) * c.hc * c.d, wb)); } }
+      q = q0 + p.pl;
     }
   }
   return PYRE_OK;
@@ -320,6 +359,16 @@ int pyre_state_read_gdn(pyre_ctx* ctx, pyre_state* s, int li, float* conv_host, 
   if (ssm_host) PYRE_HIP(ctx, hipMemcpyAsync(ssm_host, s->ssm[b][li], (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
+int pyre_state_read_ple(pyre_ctx* ctx, pyre_state* s, int pi, float* hist_host) {
+  if (!ctx || !s || !hist_host || pi < 0 || pi >= (int)s->ple_ring.size()) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_read_ple: bad argument");
+  const pyre_model_cfg& c = s->m->c; const size_t w = (size_t)c.hc * c.d; const int hl = (c.ple_conv_k - 1) * c.ple_ngram;
+  for (int j = 0; j < hl; ++j) {
+    const int pos = s->len - hl + j;
+    if (pos < 0) memset(hist_host + (size_t)j * w, 0, w * 4);
+    else PYRE_HIP(ctx, hipMemcpyAsync(hist_host + (size_t)j * w, s->ple_ring[pi] + (size_t)(pos & (s->m->ple_ring - 1)) * w, w * 4, hipMemcpyDeviceToHost, ctx->stream));
+  }
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+}
 int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, float* v_host) {
   if (!ctx || !s || ai < 0 || ai >= (int)s->kv.size() || !k_host || !v_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_read_kv: bad argument");
   const pyre_model_cfg& c = s->m->c; size_t row = (size_t)c.n_kv * c.hd; std::vector<float> kt(row * s->cap);
@@ -350,7 +399,7 @@ bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) &&
 int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev, s->tokens_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
   // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
   // leaves the updated streams in the other
   const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
@@ -358,12 +407,21 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
+  if (m->n_ple > 0) {      // the window's tokens join the history, then every position's n-gram rows are fetched once for all PLE layers
+    if (!o.from_best) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, m->ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));
+    if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
+  }
   const bool fuse_aop = [] { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }();      // 1: separate split launches instead of the producers' own operand stores
   const PyreAop aop{(const uint4*)m->aop, nullptr};
   auto opnd = [&](const QMatDev& q) -> const PyreAop* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? &aop : nullptr; };
   auto opw = [&](const QMatDev& q) -> uint16_t* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? m->aop : nullptr; };
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
+    if (L.ple) {      // resolves the pending residual update itself and leaves plain streams
+      PleDev pd = L.pld; pd.ring = s->ple_ring[L.ple_index]; pd.mask = m->ple_ring - 1;
+      if ((rc = pyre_ple_launch(ctx, m->plc, pd, m->pw, d, hc, c.eps, xin, in_ss, in_ts, xout, comb_out, comb_moe, comb_inj, start, o.step_dev, t))) return rc;
+      advance(); comb_out = nullptr; comb_moe = nullptr; comb_inj = nullptr;
+    }
     if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, 1, opw(L.proj)))) return rc;
     advance();
     if (L.full) {

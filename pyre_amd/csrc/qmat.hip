@@ -406,7 +406,7 @@ int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t
 // 64 threads per block: every block redoes the (tiny) scan of the per-tile maxima, block 0 publishes the id, and when a
 // matrix is given thread u of block b then dequantizes unit 64*b+u of the chosen row.
 template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* __restrict__ best, int n_tiles, uint32_t* id_out, uint32_t* mirror, QMatDev m, int have_m,
-                                                               const uint64_t* g2, float* __restrict__ out, int* step) {
+                                                               const uint64_t* g2, float* __restrict__ out, int* step, uint32_t* hist) {
   const int tid = threadIdx.x;
   float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
   const uint2* b2 = (const uint2*)best;
@@ -415,7 +415,7 @@ template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* 
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; } }
   if (bi == 0xFFFFFFFFu) bi = 0;
-  if (blockIdx.x == 0 && tid == 0) { int slot = 0; if (step) { int p = step[0] + 1; step[0] = p; slot = p - step[1]; } id_out[0] = bi; if (mirror) mirror[slot] = bi; }
+  if (blockIdx.x == 0 && tid == 0) { int slot = 0; if (step) { int p = step[0] + 1; step[0] = p; slot = p - step[1]; if (hist) hist[p] = bi; } id_out[0] = bi; if (mirror) mirror[slot] = bi; }
   if (!have_m) return;
   int ku = blockIdx.x * 64 + tid; if (ku >= m.U || bi >= (uint32_t)m.rows) return;
   float y[64];
@@ -424,11 +424,11 @@ template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* 
   for (int i = 0; i < 64; ++i) o[i] = y[i];
 }
 
-int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out, int* step) {
+int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out, int* step, uint32_t* hist) {
   ProfScope ps(ctx, "pick_embed", 8.0 * n_tiles);
-  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step); }
+  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step, hist); }
   else { dim3 grid((m->U + 63) / 64);
-    FMT_DISPATCH_X(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step)); }
+    FMT_DISPATCH_X(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step, hist)); }
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 

@@ -109,6 +109,7 @@ def _declare(L):
         "pyre_state_len": (i32, [vp]),
         "pyre_state_read_gdn": (i32, [vp, vp, i32, vp, vp]),
         "pyre_state_read_kv": (i32, [vp, vp, i32, vp, vp]),
+        "pyre_state_read_ple": (i32, [vp, vp, i32, vp]),
         "pyre_forward": (i32, [vp, vp, vp, vp, i32, vp]),
         "pyre_forward_multi": (i32, [vp, vp, vp, vp, i32, vp]),
         "pyre_spec_keep": (i32, [vp, vp, vp, i32, i32]),
@@ -556,10 +557,27 @@ class ModelCfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
                [("rope_base", C.c_float), ("eps", C.c_float)] + \
                [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
-                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")]
+                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")] + \
+               [(n, C.c_int32) for n in ("ple_ngram", "ple_per_gram", "ple_conv_k", "ple_dim")] + [("ple_eos", C.c_uint32), ("ple_reserved", C.c_int32),
+                ("ple_mult", C.c_uint64 * 8), ("ple_off", C.c_uint64 * 16), ("ple_vocab", C.c_uint64 * 16)]
 
 
-LAYER_SLOTS, GLOBAL_SLOTS = 35, 5
+LAYER_SLOTS, GLOBAL_SLOTS = 41, 6
+
+
+def fill_cfg(dst, src):
+    """Copies the configuration fields of `src` (any object with the field names; PLE fields optional) into the ctypes struct."""
+    for name, ty in dst._fields_:
+        if name == "ple_reserved":
+            continue
+        v = getattr(src, name, 0)
+        if name in ("ple_mult", "ple_off", "ple_vocab"):
+            arr = getattr(dst, name)
+            for i, x in enumerate(list(v or ())[:len(arr)]):
+                arr[i] = int(x)
+        else:
+            setattr(dst, name, v)
+    return dst
 
 
 class Model:
@@ -569,9 +587,7 @@ class Model:
         """cfg: object with the ModelCfg field names; layer_tensors: per layer dict slot -> (ty, rows, cols, data) where
         data is a numpy uint8 array (host) or an int device pointer; globals_: dict slot -> the same."""
         self.ctx = ctx
-        self.cfg = ModelCfg()
-        for name, _ in ModelCfg._fields_:
-            setattr(self.cfg, name, getattr(cfg, name))
+        self.cfg = fill_cfg(ModelCfg(), cfg)
         keep = []
 
         def desc(e):
@@ -614,6 +630,13 @@ class Model:
         except KeyError:
             c.idx_ratio = 4
         c.ctx_train = g.u64(a + "context_length", 262144); c.ctx = ctx_tokens or c.ctx_train
+        try:
+            has_ple = bool(g.arr_u64(a + "ple.layers"))
+        except KeyError:
+            has_ple = False
+        if has_ple:
+            c.ple_ngram = g.u64(a + "ple.ngram_size", 0); c.ple_per_gram = g.u64(a + "ple.heads_per_ngram", 0); c.ple_conv_k = g.u64(a + "ple.conv_kernel", 0)
+            c.ple_eos = g.u64(a + "ple.eos_token_id", 0); c.ple_dim = g.u64(a + "embedding_length_per_layer_input", 0)
         g.close()
         self.cfg = c; self.vocab = c.vocab
         return self
@@ -719,6 +742,12 @@ class State:
         ssm = np.empty((c.lin_nv * c.lin_dk * c.lin_dv,), dtype=np.float32)
         self.m.ctx.check(self.m.ctx.L.pyre_state_read_gdn(self.m.ctx.h, self.h, li, _ptr(conv), _ptr(ssm)), "state_read_gdn")
         return conv, ssm
+
+    def ple_hist(self, pi):
+        c = self.m.cfg
+        h = np.empty(((c.ple_conv_k - 1) * c.ple_ngram, c.hc * c.d), dtype=np.float32)
+        self.m.ctx.check(self.m.ctx.L.pyre_state_read_ple(self.m.ctx.h, self.h, pi, _ptr(h)), "state_read_ple")
+        return h
 
     def kv(self, ai):
         c = self.m.cfg

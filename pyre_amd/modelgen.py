@@ -12,12 +12,14 @@ from . import synth
 
 (HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
  ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
- UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN, LAYER_SLOTS) = range(36)
-G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN,
+ PLE_KEY, PLE_VALUE, PLE_NK, PLE_NQ, PLE_NC, PLE_CONV, LAYER_SLOTS) = range(42)
+G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, G_PLE_TAB, GLOBAL_SLOTS = range(7)
 
 CFG_FIELDS = ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot", "rope_base", "eps", "n_exp", "top_k",
               "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k", "full_every", "vocab", "kv_bits", "kv_recent",
-              "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")
+              "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx",
+              "ple_ngram", "ple_per_gram", "ple_conv_k", "ple_dim", "ple_eos", "ple_mult", "ple_off", "ple_vocab")
 
 
 @dataclass
@@ -50,6 +52,19 @@ class Config:
     idx_budget: int = 2048
     ctx_train: int = 0                # trained context and the context the model is built for (ctx > ctx_train > 0: YaRN)
     ctx: int = 0
+    # per-layer n-gram embeddings (PLE): n-gram length (0 = none), table heads per length, conv kernel, table row width,
+    # the token that cuts a context, hash multipliers per n-gram position, per head table offset and modulus; ple_layers
+    # lists the layers that carry the ple_* tensors (see with_ple)
+    ple_ngram: int = 0
+    ple_per_gram: int = 0
+    ple_conv_k: int = 0
+    ple_dim: int = 0
+    ple_eos: int = 0
+    ple_mult: tuple = ()
+    ple_off: tuple = ()
+    ple_vocab: tuple = ()
+    ple_layers: tuple = ()
+    ple_type: int = synth.Q8_0        # type of per_layer_token_embd and of ple_key / ple_value
     # generation knobs (not part of the model contract)
     qtype: int = synth.IQ3_S          # type of every projection / expert / embedding / head matrix
     hc_type: int = synth.BF16         # type of the hyper-connection matrices (BF16 in real files)
@@ -81,6 +96,17 @@ def a3b_config(**kw):
     return c
 
 
+def with_ple(c: Config, layers=(0, 2), ngram=3, per_gram=2, conv_k=3, dim=64, eos=7, sizes=(97, 131, 61, 251)):
+    """Switches PLE on for `layers`: (ngram - 1) * per_gram heads with the given table sizes (cycled), stacked in one table."""
+    nh = (ngram - 1) * per_gram
+    vocab = [sizes[i % len(sizes)] + 2 * i for i in range(nh)]
+    off = [sum(vocab[:i]) for i in range(nh)]
+    mult = [(0x9E3779B97F4A7C15 * (2 * i + 1) + 0x1234567 * i) & 0xFFFFFFFFFFFFFFFF | 1 for i in range(ngram)]
+    c.ple_ngram, c.ple_per_gram, c.ple_conv_k, c.ple_dim, c.ple_eos = ngram, per_gram, conv_k, dim, eos
+    c.ple_mult, c.ple_off, c.ple_vocab, c.ple_layers = tuple(mult), tuple(off), tuple(vocab), tuple(layers)
+    return c
+
+
 def tensor_specs(c: Config):
     """[(layer or -1, slot, kind, ty, rows, cols)] for every tensor of the model; kind in {'q','vec:<name>'}."""
     sf = c.ff_sh or c.ff_exp
@@ -91,6 +117,10 @@ def tensor_specs(c: Config):
             out += [(il, base, "vec:norm1", synth.F32, 1, w), (il, base + 1, "q", c.hc_type, c.hc_lr, w),
                     (il, base + 2, "q", c.hc_type, c.hc, w),
                     (il, base + 3, "q", c.hc_type, w, c.hc_lr)]
+        if il in c.ple_layers:
+            ein = (c.ple_ngram - 1) * c.ple_per_gram * c.ple_dim
+            out += [(il, PLE_KEY, "q", c.ple_type, w, ein), (il, PLE_VALUE, "q", c.ple_type, c.d, ein), (il, PLE_NK, "vec:norm1", synth.F32, 1, w),
+                    (il, PLE_NQ, "vec:norm1", synth.F32, 1, w), (il, PLE_NC, "vec:norm1", synth.F32, 1, w), (il, PLE_CONV, "vec:conv", synth.F32, 1, w * c.ple_conv_k)]
         if c.full(il):
             out += [(il, ATTN_Q, "q", c.qtype, c.n_head * 2 * c.hd, c.d), (il, ATTN_K, "q", c.qtype, c.n_kv * c.hd, c.d),
                     (il, ATTN_V, "q", c.qtype, c.n_kv * c.hd, c.d), (il, ATTN_O, "q", c.qtype, c.d, c.n_head * c.hd),
@@ -111,6 +141,9 @@ def tensor_specs(c: Config):
     out += [(-1, G_EMBD, "q", c.qtype, c.vocab, c.d), (-1, G_HEAD_NORM, "vec:norm1", synth.F32, 1, w),
             (-1, G_HEAD_DOWN, "q", c.hc_type, c.hc_lr, w), (-1, G_HEAD_UP, "q", c.hc_type, w, c.hc_lr),
             (-1, G_OUT, "q", c.qtype, c.vocab, c.d)]
+    if c.ple_layers:
+        nh = (c.ple_ngram - 1) * c.ple_per_gram
+        out += [(-1, G_PLE_TAB, "q", c.ple_type, max(c.ple_off[h] + c.ple_vocab[h] for h in range(nh)), c.ple_dim)]
     return out
 
 

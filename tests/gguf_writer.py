@@ -60,8 +60,10 @@ LAYER_NAMES = {
     mg.ROUTER: "ffn_gate_inp.weight", mg.GATE_E: "ffn_gate_exps.weight", mg.UP_E: "ffn_up_exps.weight", mg.DOWN_E: "ffn_down_exps.weight",
     mg.SH_GATE_INP: "ffn_gate_inp_shexp.weight", mg.SH_GATE: "ffn_gate_shexp.weight", mg.SH_UP: "ffn_up_shexp.weight", mg.SH_DOWN: "ffn_down_shexp.weight",
     mg.IDX_Q: "indexer.q_proj.weight", mg.IDX_K: "indexer.k_proj.weight", mg.IDX_QN: "indexer.q_norm.weight", mg.IDX_KN: "indexer.k_norm.weight",
+    mg.PLE_KEY: "ple_key.weight", mg.PLE_VALUE: "ple_value.weight", mg.PLE_NK: "ple_norm_key.weight", mg.PLE_NQ: "ple_norm_query.weight", mg.PLE_NC: "ple_norm_conv.weight",
+    mg.PLE_CONV: "ple_conv1d.weight",
 }
-GLOBAL_NAMES = {mg.G_EMBD: "token_embd.weight", mg.G_HEAD_NORM: "output_hc_norm.weight", mg.G_HEAD_DOWN: "output_hc_down.weight", mg.G_HEAD_UP: "output_hc_up.weight", mg.G_OUT: "output.weight"}
+GLOBAL_NAMES = {mg.G_EMBD: "token_embd.weight", mg.G_HEAD_NORM: "output_hc_norm.weight", mg.G_HEAD_DOWN: "output_hc_down.weight", mg.G_HEAD_UP: "output_hc_up.weight", mg.G_OUT: "output.weight", mg.G_PLE_TAB: "per_layer_token_embd.weight"}
 
 
 def model_meta(c):
@@ -74,7 +76,10 @@ def model_meta(c):
             (a + "ssm.time_step_rank", U64, c.lin_nv), (a + "ssm.state_size", I32, c.lin_dk), (a + "ssm.conv_kernel", U16, c.conv_k),
             (a + "full_attention_interval", U8, c.full_every), (a + "context_length", U32, c.ctx_train or 262144), ("tokenizer.ggml.tokens", ARR, (STR, ["a", "b"]))] + \
            ([(a + "attention.indexer.head_count", U32, c.idx_nh), (a + "attention.indexer.key_length", U32, c.idx_hd), (a + "attention.indexer.top_k", U32, c.idx_budget),
-             (a + "attention.compress_ratios", ARR, (U32, [1, c.idx_ratio, 2] if c.idx_ratio > 2 else [c.idx_ratio]))] if c.idx_nh > 0 else [])
+             (a + "attention.compress_ratios", ARR, (U32, [1, c.idx_ratio, 2] if c.idx_ratio > 2 else [c.idx_ratio]))] if c.idx_nh > 0 else []) + \
+           ([(a + "ple.layers", ARR, (U32, list(c.ple_layers))), (a + "ple.ngram_size", U32, c.ple_ngram), (a + "ple.heads_per_ngram", U32, c.ple_per_gram), (a + "ple.conv_kernel", U32, c.ple_conv_k),
+             (a + "ple.eos_token_id", U32, c.ple_eos), (a + "embedding_length_per_layer_input", U32, c.ple_dim), (a + "ple.layer_multipliers", ARR, (U64, list(c.ple_mult))),
+             (a + "ple.head_offsets", ARR, (U64, list(c.ple_off))), (a + "ple.head_vocab_sizes", ARR, (U64, list(c.ple_vocab)))] if c.ple_layers else [])
 
 
 def model_tensors(c, hw):

@@ -17,10 +17,8 @@ def orc_tensor(entry):
 
 
 def orc_cfg(c):
-    cfg = orc.Cfg()
-    for f in mg.CFG_FIELDS:
-        setattr(cfg, f, getattr(c, f))
-    return cfg
+    from pyre_amd.lib import fill_cfg
+    return fill_cfg(orc.Cfg(), c)
 
 
 def orc_model(hw, threads=4):
@@ -30,7 +28,7 @@ def orc_model(hw, threads=4):
         for slot in range(mg.LAYER_SLOTS):
             e = hw.layers[il].get(slot)
             lt.append(orc_tensor(e) if e is not None else orc.Tensor(0, 0, 0, None))
-    g = [orc_tensor(hw.globals_[s]) for s in range(mg.GLOBAL_SLOTS)]
+    g = [orc_tensor(hw.globals_[s]) if s in hw.globals_ else orc.Tensor(0, 0, 0, None) for s in range(mg.GLOBAL_SLOTS)]
     return orc.Model(orc_cfg(c), lt, g, threads=threads, keep=(hw,))
 
 

@@ -12,8 +12,9 @@ F32, F16, Q8_0, Q4_K, IQ2_XS, IQ3_S, BF16 = 0, 1, 8, 12, 17, 21, 30
 Q4_0, Q5_0, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_NL, IQ2_S, IQ4_XS, Q3_K, Q2_0, Q5_K, IQ1_M = 2, 6, 14, 16, 18, 20, 22, 23, 11, 42, 13, 29
 (HCA_NORM, HCA_DOWN, HCA_INJECT, HCA_UP, HCF_NORM, HCF_DOWN, HCF_INJECT, HCF_UP, ATTN_Q, ATTN_K, ATTN_V, ATTN_O,
  ATTN_QN, ATTN_KN, LIN_QKV, LIN_Z, LIN_BETA, LIN_ALPHA, LIN_A, LIN_DT, LIN_CONV, LIN_NORM, LIN_OUT, ROUTER, GATE_E,
- UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN, LAYER_SLOTS) = range(36)
-G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, GLOBAL_SLOTS = range(6)
+ UP_E, DOWN_E, SH_GATE_INP, SH_GATE, SH_UP, SH_DOWN, IDX_Q, IDX_K, IDX_QN, IDX_KN,
+ PLE_KEY, PLE_VALUE, PLE_NK, PLE_NQ, PLE_NC, PLE_CONV, LAYER_SLOTS) = range(42)
+G_EMBD, G_HEAD_NORM, G_HEAD_DOWN, G_HEAD_UP, G_OUT, G_PLE_TAB, GLOBAL_SLOTS = range(7)
 
 
 class Tensor(C.Structure):
@@ -24,7 +25,9 @@ class Cfg(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "hc", "hc_lr", "n_head", "n_kv", "hd", "n_rot")] + \
                [("rope_base", C.c_float), ("eps", C.c_float)] + \
                [(n, C.c_int32) for n in ("n_exp", "top_k", "ff_exp", "lin_nk", "lin_nv", "lin_dk", "lin_dv", "conv_k",
-                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")]
+                                         "full_every", "vocab", "kv_bits", "kv_recent", "idx_nh", "idx_hd", "idx_ratio", "idx_budget", "ctx_train", "ctx")] + \
+               [(n, C.c_int32) for n in ("ple_ngram", "ple_per_gram", "ple_conv_k", "ple_dim")] + [("ple_eos", C.c_uint32), ("ple_reserved", C.c_int32),
+                ("ple_mult", C.c_uint64 * 8), ("ple_off", C.c_uint64 * 16), ("ple_vocab", C.c_uint64 * 16)]
 
 
 def build():
@@ -52,7 +55,7 @@ def lib():
         L.orc_model_create.restype = C.c_void_p
         L.orc_state_create.restype = C.c_void_p
         L.orc_rope_inv_yarn.restype = C.c_float
-        for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v", "orc_state_ik", "orc_state_ib"):
+        for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v", "orc_state_ik", "orc_state_ib", "orc_state_ple_hist"):
             getattr(L, n).restype = C.POINTER(C.c_float)
         _lib = L
     return _lib
@@ -208,6 +211,25 @@ def hc_combine(d, hc, x, out, inj):
     return x
 
 
+def ple_rows(cfg, tab, tokens, start, t):
+    """cfg: orc.Cfg with the ple_* fields; tab: orc.Tensor; tokens: the history (uint32).  Returns emb [t][heads*dim]."""
+    tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+    emb = np.empty((t, (cfg.ple_ngram - 1) * cfg.ple_per_gram * cfg.ple_dim), dtype=np.float32)
+    rc = lib().orc_ple_rows(C.byref(cfg), C.byref(tab), _p(tokens), C.c_int(start), C.c_int(t), _p(emb))
+    assert rc == 0, rc
+    return emb
+
+
+def ple(cfg, key, value, nk, nq, nc, conv, hist, emb, x, threads=2):
+    """One PLE layer on t tokens: returns the updated x [t][hc*d]; hist [(conv_k-1)*ngram][hc*d] is advanced in place."""
+    x = f32(x).copy().reshape(-1, cfg.hc * cfg.d); t = x.shape[0]
+    nk, nq, nc, conv, emb = f32(nk), f32(nq), f32(nc), f32(conv), f32(emb)
+    assert hist.dtype == np.float32 and hist.flags.c_contiguous
+    rc = lib().orc_ple(C.byref(cfg), C.byref(key), C.byref(value), _p(nk), _p(nq), _p(nc), _p(conv), _p(hist), _p(emb), _p(x), C.c_int(t), C.c_int(threads))
+    assert rc == 0, rc
+    return x
+
+
 class Model:
     """Oracle model over a weight set (see tests/modelgen.py for the container)."""
 
@@ -274,6 +296,10 @@ class State:
         c = self.m.cfg
         ch = 2 * c.lin_nk * c.lin_dk + c.lin_nv * c.lin_dv
         return np.ctypeslib.as_array(lib().orc_state_conv(self.h, li), shape=((c.conv_k - 1) * ch,))
+
+    def ple_hist(self, pi):
+        c = self.m.cfg
+        return np.ctypeslib.as_array(lib().orc_state_ple_hist(self.h, pi), shape=((c.ple_conv_k - 1) * c.ple_ngram, c.hc * c.d))
 
     def kcache(self, ai):
         c = self.m.cfg

@@ -75,7 +75,7 @@ def test_twelve_layer_full_width_greedy_stream_matches_oracle(ctx):
         for slot in range(mg.LAYER_SLOTS):
             e = hl[il].get(slot)
             lt.append(orc.tensor(*e) if e is not None else orc.Tensor(0, 0, 0, None))
-    om = orc.Model(orc_cfg(cfg), lt, [orc.tensor(*hg[s]) for s in range(mg.GLOBAL_SLOTS)], threads=THREADS, keep=(hl, hg))
+    om = orc.Model(orc_cfg(cfg), lt, [orc.tensor(*hg[s]) if s in hg else orc.Tensor(0, 0, 0, None) for s in range(mg.GLOBAL_SLOTS)], threads=THREADS, keep=(hl, hg))
     prompt = rnd(22).integers(0, cfg.vocab, 24, dtype=np.uint32)
     gs, os_ = gm.new_state(128), om.new_state()
     lg, lo = gm.forward(prompt, gs), om.forward(prompt, os_)

@@ -232,6 +232,70 @@ def test_drafted_generation_identical_to_plain_and_to_oracle(ctx):
         assert np.array_equal(oo, plain) and orounds == rounds
 
 
+# ---- per-layer n-gram embeddings (PLE) -----------------------------------------------------------------------------------
+def ple_pair(ctx, seed, **kw):
+    c = mg.with_ple(small_cfg(**kw), layers=(0, 2, 3), ngram=3, per_gram=2, conv_k=3, dim=64, eos=7)
+    return (c,) + pair(ctx, c, seed)
+
+
+def test_ple_model_matches_oracle_steps_window_rollback_device_loop_and_snapshot(ctx, tmp_path):
+    c, hw, gm, om = ple_pair(ctx, 61)
+    g = np.random.Generator(np.random.PCG64(62))
+    prompt = g.integers(0, c.vocab, 27, dtype=np.uint32); prompt[[4, 5, 13]] = c.ple_eos          # eos tokens cut the n-gram contexts
+    gs, os_ = gm.new_state(160), om.new_state()
+    lg, lo = gm.forward(prompt, gs), om.forward(prompt, os_)                                  # windows of 8, 8, 8, 3 against the oracle's one call
+    assert relerr(lg, lo) <= 1e-3
+    for pi in range(3):
+        assert relerr(gs.ple_hist(pi), os_.ple_hist(pi)) <= 1e-4, pi
+    # single steps: the same greedy stream
+    toks = []
+    for _ in range(10):
+        tg, to = int(orc.argmax(lg)), int(orc.argmax(lo)); assert tg == to
+        toks.append(to); t1 = np.array([to], dtype=np.uint32); lg, lo = gm.forward(t1, gs), om.forward(t1, os_)
+        assert relerr(lg, lo) <= 1e-3
+    # a verify window equals single steps bit for bit, and a rollback equals never having drafted
+    snap = gs.snapshot()
+    win = np.array([int(orc.argmax(lg)), 3, c.ple_eos, 200, 41], dtype=np.uint32)
+    lv = gm.forward_multi(win, gs)
+    sb = gm.new_state(160); sb.restore(snap)
+    singles = np.array([gm.forward(win[i:i + 1], sb) for i in range(5)])
+    assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32))
+    so = om.new_state(); om.forward(np.concatenate([prompt, np.array(toks, np.uint32)]), so)
+    assert relerr(lv, om.forward_multi(win, so)) <= 1e-3
+    gm.spec_keep(gs, 5, 2); om.spec_keep(so, 5, 2)
+    sc = gm.new_state(160); sc.restore(snap); gm.forward(win[0:1], sc); gm.forward(win[1:2], sc)
+    nxt = np.array([77], dtype=np.uint32)
+    la = gm.forward(nxt, gs)
+    assert np.array_equal(la.view(np.uint32), gm.forward(nxt, sc).view(np.uint32)) and relerr(la, om.forward(nxt, so)) <= 1e-3
+    for pi in range(3):
+        assert np.array_equal(gs.ple_hist(pi).view(np.uint32), sc.ple_hist(pi).view(np.uint32)) and relerr(gs.ple_hist(pi), so.ple_hist(pi)) <= 1e-4
+    # the device-resident loop (token history and position on the device, replayed) against the oracle's loop
+    first = int(orc.argmax(la)); dev = gm.decode_greedy_dev(gs, first, 30)
+    want = []; tok = first
+    for _ in range(30):
+        tok = int(orc.argmax(om.forward(np.array([tok], dtype=np.uint32), so))); want.append(tok)
+    assert np.array_equal(dev, np.array(want, dtype=np.uint32))
+    # and once more from a restored snapshot, eagerly replayed
+    sd = gm.new_state(160); sd.restore(snap)
+    gm.forward(win[0:1], sd); gm.forward(win[1:2], sd); gm.forward(nxt, sd)
+    assert np.array_equal(gm.decode_greedy_dev(sd, first, 30), dev)
+    # the same model through a GGUF file with the ple.* keys
+    import gguf_writer as gw
+    p = str(tmp_path / "ple.gguf")
+    gw.write(p, gw.model_meta(c), gw.model_tensors(c, hw))
+    gg = lib.Model.from_gguf(ctx, p, kv_bits=c.kv_bits, kv_recent=c.kv_recent)
+    sg = gg.new_state(64)
+    assert np.array_equal(gg.forward(prompt, sg).view(np.uint32), gm.forward(prompt, gm.new_state(64)).view(np.uint32))
+
+
+def test_ple_table_rows_outside_the_table_are_refused(ctx):
+    c = mg.with_ple(small_cfg(), layers=(1,))
+    hw = mg.build_host(c, seed=63)
+    c.ple_vocab = tuple(v + 1000 for v in c.ple_vocab)
+    with pytest.raises(lib.PyreError, match="per_layer_token_embd"):
+        lib.Model(ctx, c, hw.layers, hw.globals_)
+
+
 def test_errors(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 9)
@@ -256,7 +320,8 @@ def test_model_loaded_from_gguf_shards_equals_the_model_built_from_the_same_tens
     gw.write(p1, gw.model_meta(c), tens[:half]); gw.write(p2, [("split.no", gw.U16, 1)], tens[half:], alignment=128)
     gg = lib.Model.from_gguf(ctx, p2, kv_bits=c.kv_bits, kv_recent=c.kv_recent)
     skip = ("rope_base", "eps", "ctx_train", "ctx")        # floats; the file's trained context (262144 by default) is the model's context unless one is asked for
-    assert [getattr(gg.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip] == [getattr(gm.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip]
+    val = lambda cfg, f: list(getattr(cfg, f)) if f in ("ple_mult", "ple_off", "ple_vocab") else getattr(cfg, f)
+    assert [val(gg.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip] == [val(gm.cfg, f) for f, _ in lib.ModelCfg._fields_ if f not in skip]
     ids = np.array([3, 77, 500, 12, 9, 311, 4, 4, 250, 17, 88], dtype=np.uint32)
     sa, sb = gm.new_state(64), gg.new_state(64)
     la, lb = gm.forward(ids, sa), gg.forward(ids, sb)
