@@ -35,6 +35,10 @@
  *                          one live FFN / one live DeltaNet layer -> the composition of the pinned block entry
  *                          points bit for bit (and not with the other mixer's inject factors); + a numpy statement
  *                          of the whole token step on a tiny model
+ *   orc_ple_rows / orc_ple closed forms: multipliers that single out one context token (operand order, cut at the
+ *                          sequence start and at eos, 64-bit wrap, xor); zero value -> the conv over a hand-set history
+ *                          tap by tap; zero key -> the gate floor; one-hot key / stream -> the gate in closed form;
+ *                          constant gated stream -> the norm weight; window == single tokens
  * Parity unpinned (only running the reference could pin): the last-ulp behaviour of
  * expf/log1pf/powf/sincosf on the reference's own target libm.
  */
