@@ -150,6 +150,8 @@ def bench_gemv(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
+        "path": ("f32 multiply-add GEMV, lane = row (k_gemv)" if ty != lib.IQ3_S or os.environ.get("PYRE_QMATMUL_F32") == "1" else
+                 "f16 matrix cores (k_gemm_m, preceded by the operand split k_act_split): the kernel the model's projections and head run"),
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": kernels[0]["kernel"] if kernels else None, "device_bytes_per_launch": mats[0].layout_bytes(ty == lib.IQ3_S and os.environ.get("PYRE_QMATMUL_F32") != "1") or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
         "kernels": kernels,
