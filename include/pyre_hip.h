@@ -307,6 +307,50 @@ int   pyre_ngram_draft(const uint32_t* history, size_t len, int k, int min_n, in
  * accepted (spec::Outcome, src/spec.rs:150-154). */
 int   pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* history, size_t n_hist, const float* first_logits_host,
                                  int n_out, uint32_t* out, int k, int ng_min, int ng_max, int* rounds, int* drafted, int* accepted);
+/* ---- the multi-token-prediction (MTP) drafter: src/model/mtp.rs, Model::mtp_draft (src/model/qwen4exp_gguf.rs:2180-2277) ----
+ * One extra block that pairs the main model's final residual streams R_i with the token at position i + 1 (cell i, rope
+ * position i, the unscaled table) and predicts token i + 2: pre-norms and two d x d matrices form its streams, then
+ * hyper-connection mix -> gated attention over its own last `window` cells -> mix -> MoE FFN -> mixer -> the draft
+ * vocabulary rows of the output matrix.  Its own residual feeds the next draft step.  Only draft quality depends on it:
+ * every emitted token comes from the verify window.  Tensors come in any supported type (the reference builds int8
+ * copies of a BF16 checkpoint, mtp.rs:11-13); norm vectors already carry their "1 + w" (mtp.rs:44-45); the fused
+ * mlp.experts.gate_up_proj is given as its gate and up halves. */
+enum {
+  PYRE_MTP_PRE_E = 0, PYRE_MTP_PRE_H,                       /* pre_fc_norm_embedding [d], pre_fc_norm_hidden [hc*d] */
+  PYRE_MTP_FC_E, PYRE_MTP_FC_H,                             /* fc_embedding, fc_hidden [d x d] */
+  PYRE_MTP_HCA_NORM, PYRE_MTP_HCA_DOWN, PYRE_MTP_HCA_INJECT, PYRE_MTP_HCA_UP,      /* attn_hyper_connection.* */
+  PYRE_MTP_HCF_NORM, PYRE_MTP_HCF_DOWN, PYRE_MTP_HCF_INJECT, PYRE_MTP_HCF_UP,      /* mlp_hyper_connection.* */
+  PYRE_MTP_MIX_NORM, PYRE_MTP_MIX_DOWN, PYRE_MTP_MIX_UP,                           /* hyper_connection_mixer.* (no inject) */
+  PYRE_MTP_Q, PYRE_MTP_K, PYRE_MTP_V, PYRE_MTP_O, PYRE_MTP_QN, PYRE_MTP_KN,        /* self_attn.* */
+  PYRE_MTP_ROUTER, PYRE_MTP_GATE_E, PYRE_MTP_UP_E, PYRE_MTP_DOWN_E,                /* mlp.gate, mlp.experts.* */
+  PYRE_MTP_SH_GATE_INP, PYRE_MTP_SH_GATE, PYRE_MTP_SH_UP, PYRE_MTP_SH_DOWN,        /* mlp.shared_expert_gate, mlp.shared_expert.* */
+  PYRE_MTP_HEAD,                                            /* rows draft_ids[0..n_draft_vocab) of the main model's output matrix */
+  PYRE_MTP_SLOTS
+};
+/* geometry beyond the main model's (Geo, mtp.rs:95): routed experts, experts per token, expert width, attention window
+ * in cells (PYRE_MTP_WINDOW, 128 in the reference), rows of the draft head */
+typedef struct { int32_t n_exp, top_k, ff, window, n_draft_vocab; } pyre_mtp_cfg;
+typedef struct pyre_mtp pyre_mtp;
+int   pyre_mtp_create(pyre_ctx* ctx, const pyre_model* main, const pyre_mtp_cfg* cfg, const pyre_tensor* tensors /*[PYRE_MTP_SLOTS]*/,
+                      const uint32_t* draft_ids /*[n_draft_vocab], host*/, pyre_mtp** out);
+void  pyre_mtp_destroy(pyre_mtp* m);
+/* From now on every forward call leaves the final residual streams of its last `window` tokens in a ring on the device
+ * (mtp_keep_r, qwen4exp_gguf.rs:2279-2285: window + 16 positions are kept) and the state owns the drafter's K/V cells.
+ * Snapshots do not carry either: after pyre_state_restore the drafter starts over (no drafts until a forward call has
+ * left the residual of the last position again). */
+int   pyre_state_attach_mtp(pyre_ctx* ctx, pyre_state* s, const pyre_mtp* m);
+/* mtp_draft, host-loop form with the draft policy off: catches the drafter's cells up over the positions whose token is
+ * committed, then runs up to k (1..7) draft steps from (R_{len-1}, pending) on the device and reads ids and
+ * probabilities back once.  A later draft is kept only while the drafter's probability of its choice is >= min_p
+ * (spec::draft_gate, src/spec.rs:326-327).  *n_out = drafts in ids_host / probs_host [k] (0 when the residual of the
+ * last position is not there). */
+int   pyre_mtp_draft(pyre_ctx* ctx, const pyre_mtp* m, pyre_state* s, uint32_t pending, int k, float min_p, uint32_t* ids_host, float* probs_host, int* n_out);
+/* test access: cells [*c0, *c0 + *n) of the drafter's cache, k_host / v_host [*n][n_kv*hd] (either may be NULL; pass room for `window` cells) */
+int   pyre_mtp_read_kv(pyre_ctx* ctx, pyre_state* s, int* c0, int* n, float* k_host, float* v_host);
+/* spec::generate's greedy branch with this drafter proposing (src/spec.rs:156-267): each round verifies [pending, drafts]
+ * in one window and keeps the agreeing prefix.  The output equals plain greedy decoding token for token. */
+int   pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
+                               int k, float min_p, int* rounds, int* drafted, int* accepted);
 /* The decode loop as the benchmark times it: n_steps greedy steps starting from token `first`, everything on the device;
  * tokens (optional, host) receives the n_steps generated ids after the call. */
 int   pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host);

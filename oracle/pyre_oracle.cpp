@@ -2,6 +2,7 @@
 // Every function cites the reference lines it follows (paths relative to the reference tree).
 // Build: g++ -O2 -std=c++17 -mavx2 -mfma -ffp-contract=off -fPIC -shared -pthread (see oracle/Makefile).
 #include "pyre_oracle.h"
+#include <deque>
 #include "iq_codebooks.h"
 #include <algorithm>
 #include <atomic>
@@ -618,6 +619,9 @@ struct OrcState {
   std::vector<std::vector<float>> conv, ssm, k, v, ik, ib;   // ik / ib: raw index keys [pos][idx_hd], pooled block keys [block][idx_hd]
   std::vector<std::vector<float>> ple_hist;                  // per PLE layer: the last (conv_k-1)*ngram normalised rows [hc*d], oldest first (:196)
   std::vector<OrcCkpt> ck;  // state after each token of the last forward_multi
+  // MTP drafter (mtp_r / mtp_kv, qwen4exp_gguf.rs:206): the last final residuals by position; the drafter's own K/V cells
+  int mtp_window = 0; std::deque<std::pair<int, std::vector<float>>> mtp_r;
+  int mtp_c0 = 0, mtp_n = 0; std::vector<float> mtp_k, mtp_v;
 };
 
 static bool to_vec(const OrcTensor& t, std::vector<float>& out) {
@@ -782,6 +786,15 @@ int orc_forward(const OrcModel* m, OrcState* st, const uint32_t* ids, int t, flo
                  &m->T(il, ORC_SH_GATE), &m->T(il, ORC_SH_UP), &m->T(il, ORC_SH_DOWN), mixed.data(), t, o.data(), nullptr, nullptr, th)) return -6;
     hc_combine(d, hc, x.data(), o.data(), inj.data(), t);
   }
+  if (st->mtp_window > 0) {      // mtp_keep_r for the last `window` tokens of the call, :2148-2150, :2279-2285
+    for (int ti = std::max(0, t - st->mtp_window); ti < t; ++ti) {
+      const int pos = start + ti;
+      while (!st->mtp_r.empty() && st->mtp_r.back().first >= pos) st->mtp_r.pop_back();
+      if (!st->mtp_r.empty() && st->mtp_r.back().first + 1 != pos) st->mtp_r.clear();
+      st->mtp_r.emplace_back(pos, std::vector<float>(x.begin() + (size_t)ti * hc * d, x.begin() + (size_t)(ti + 1) * hc * d));
+      while ((int)st->mtp_r.size() > st->mtp_window + 16) st->mtp_r.pop_front();
+    }
+  }
   std::vector<float> h(d), dummy(hc);
   if (!hc_mix(d, hc, c.eps, m->head_norm.data(), &m->g[ORC_G_HEAD_DOWN], nullptr, &m->g[ORC_G_HEAD_UP], x.data() + (size_t)(t - 1) * hc * d, 1, h.data(), dummy.data(), th)) return -7;
   if (!mm(&m->g[ORC_G_OUT], h.data(), 1, logits, th)) return -8;  // head_logits, :2361-2364
@@ -827,4 +840,138 @@ int orc_generate_greedy(const OrcModel* m, OrcState* st, const float* first_logi
   return rounds;
 }
 
+}  // extern "C"
+
+// ---------- MTP drafter, src/model/mtp.rs ------------------------------------------------------------------------------
+struct OrcMtp {
+  OrcMtpCfg c; OrcTensor t[ORC_MTP_SLOTS]; std::vector<uint32_t> ids; const OrcModel* main;
+  std::vector<float> pre_e, pre_h, hca_norm, hcf_norm, mix_norm, qn, kn, sgate, rope_inv;
+};
+namespace {
+const float* mtp_r_get(const OrcState* st, int pos) {      // mtp_r_get, :2286
+  if (st->mtp_r.empty()) return nullptr; const int f = st->mtp_r.front().first; if (pos < f || pos - f >= (int)st->mtp_r.size()) return nullptr;
+  const auto& e = st->mtp_r[pos - f]; return e.first == pos ? e.second.data() : nullptr;
+}
+// input, mtp.rs:151-160: t rows of main-model residuals r [t][hc*d] and token embeddings emb [t][d] -> [t][hc][d]
+bool mtp_input(const OrcMtp* m, const float* r, const float* emb, int t, std::vector<float>& out) {
+  const OrcCfg& c = m->main->c; const int d = c.d, hc = c.hc, w = hc * d, th = m->main->threads;
+  std::vector<float> en((size_t)t * d), e2((size_t)t * d), hn((size_t)t * w);
+  for (int ti = 0; ti < t; ++ti) rms(emb + (size_t)ti * d, m->pre_e.data(), c.eps, en.data() + (size_t)ti * d, d);
+  if (!mm(&m->t[ORC_MTP_FC_E], en.data(), t, e2.data(), th)) return false;
+  for (int ti = 0; ti < t; ++ti) rms(r + (size_t)ti * w, m->pre_h.data(), c.eps, hn.data() + (size_t)ti * w, w);
+  out.assign((size_t)t * w, 0.0f);
+  if (!mm(&m->t[ORC_MTP_FC_H], hn.data(), t * hc, out.data(), th)) return false;
+  for (int ti = 0; ti < t; ++ti) for (int s = 0; s < hc; ++s) for (int i = 0; i < d; ++i) out[((size_t)ti * hc + s) * d + i] += e2[(size_t)ti * d + i];
+  return true;
+}
+// kv_append, mtp.rs:163-176: K/V of t cells starting at pos0 appended (window kept); returns R after input, mixed, inject
+bool mtp_kv_append(const OrcMtp* m, OrcState* st, const float* r, const float* emb, int t, int pos0, std::vector<float>& rr, std::vector<float>& mixed, std::vector<float>& inj) {
+  const OrcCfg& c = m->main->c; const int d = c.d, hc = c.hc, row = c.n_kv * c.hd, th = m->main->threads;
+  if (st->mtp_c0 + st->mtp_n != pos0) { st->mtp_c0 = pos0; st->mtp_n = 0; st->mtp_k.clear(); st->mtp_v.clear(); }
+  if (!mtp_input(m, r, emb, t, rr)) return false;
+  mixed.assign((size_t)t * d, 0.0f); inj.assign((size_t)t * hc, 0.0f);
+  if (!hc_mix(d, hc, c.eps, m->hca_norm.data(), &m->t[ORC_MTP_HCA_DOWN], &m->t[ORC_MTP_HCA_INJECT], &m->t[ORC_MTP_HCA_UP], rr.data(), t, mixed.data(), inj.data(), th)) return false;
+  std::vector<float> kf((size_t)t * row), vf((size_t)t * row), y(c.hd);
+  if (!mm(&m->t[ORC_MTP_K], mixed.data(), t, kf.data(), th) || !mm(&m->t[ORC_MTP_V], mixed.data(), t, vf.data(), th)) return false;
+  for (int ti = 0; ti < t; ++ti) for (int h = 0; h < c.n_kv; ++h) { float* kh = kf.data() + (size_t)ti * row + (size_t)h * c.hd; rms(kh, m->kn.data(), c.eps, y.data(), c.hd); memcpy(kh, y.data(), sizeof(float) * c.hd); rope(kh, pos0 + ti, c.n_rot, m->rope_inv.data()); }
+  st->mtp_k.insert(st->mtp_k.end(), kf.begin(), kf.end()); st->mtp_v.insert(st->mtp_v.end(), vf.begin(), vf.end()); st->mtp_n += t;
+  if (st->mtp_n > m->c.window) { const int drop = st->mtp_n - m->c.window; st->mtp_k.erase(st->mtp_k.begin(), st->mtp_k.begin() + (size_t)drop * row); st->mtp_v.erase(st->mtp_v.begin(), st->mtp_v.begin() + (size_t)drop * row); st->mtp_c0 += drop; st->mtp_n -= drop; }
+  return true;
+}
+// step, mtp.rs:190-236: one draft step at cell pos; s = the final mixer's output for the head, rr = the drafter's residual.
+// The routed experts go through the main model's MoE statement (chosen experts summed in ascending id; the reference's
+// select_nth_unstable leaves their order open).
+bool mtp_step(const OrcMtp* m, OrcState* st, const float* r, const float* emb, int pos, std::vector<float>& s_out, std::vector<float>& rr) {
+  const OrcCfg& c = m->main->c; const int d = c.d, hc = c.hc, nh = c.n_head, hd = c.hd, row = c.n_kv * hd, grp = nh / c.n_kv, th = m->main->threads;
+  std::vector<float> mx, inj;
+  if (!mtp_kv_append(m, st, r, emb, 1, pos, rr, mx, inj)) return false;
+  std::vector<float> qf((size_t)nh * 2 * hd), att((size_t)nh * hd, 0.0f), qh(hd), sc;
+  if (!mm(&m->t[ORC_MTP_Q], mx.data(), 1, qf.data(), th)) return false;
+  const int n = st->mtp_n; const float scale = 1.0f / sqrtf((float)hd);
+  for (int h = 0; h < nh; ++h) {
+    const size_t base = (size_t)h * 2 * hd; rms(qf.data() + base, m->qn.data(), c.eps, qh.data(), hd); rope(qh.data(), pos, c.n_rot, m->rope_inv.data());
+    const int kvh = h / grp; sc.assign(n, 0.0f); float mxs = -INFINITY;
+    for (int p = 0; p < n; ++p) { const float* k = st->mtp_k.data() + (size_t)p * row + (size_t)kvh * hd; float a = 0.0f; for (int i = 0; i < hd; ++i) a += qh[i] * k[i]; sc[p] = a * scale; mxs = fmaxf(mxs, sc[p]); }
+    float sum = 0.0f; for (int p = 0; p < n; ++p) { sc[p] = expf(sc[p] - mxs); sum += sc[p]; }
+    float* o = att.data() + (size_t)h * hd;
+    for (int p = 0; p < n; ++p) { const float wgt = sc[p] / sum; const float* v = st->mtp_v.data() + (size_t)p * row + (size_t)kvh * hd; for (int i = 0; i < hd; ++i) o[i] += wgt * v[i]; }
+    for (int i = 0; i < hd; ++i) o[i] *= sigm(qf[base + hd + i]);
+  }
+  std::vector<float> bo(d), m2(d), inj2(hc), y(d), dummy(hc);
+  if (!mm(&m->t[ORC_MTP_O], att.data(), 1, bo.data(), th)) return false;
+  hc_combine(d, hc, rr.data(), bo.data(), inj.data(), 1);
+  if (!hc_mix(d, hc, c.eps, m->hcf_norm.data(), &m->t[ORC_MTP_HCF_DOWN], &m->t[ORC_MTP_HCF_INJECT], &m->t[ORC_MTP_HCF_UP], rr.data(), 1, m2.data(), inj2.data(), th)) return false;
+  if (!moe_ffn(d, m->c.n_exp, m->c.top_k, m->c.ff, &m->t[ORC_MTP_ROUTER], &m->t[ORC_MTP_GATE_E], &m->t[ORC_MTP_UP_E], &m->t[ORC_MTP_DOWN_E], m->sgate.data(),
+               &m->t[ORC_MTP_SH_GATE], &m->t[ORC_MTP_SH_UP], &m->t[ORC_MTP_SH_DOWN], m2.data(), 1, y.data(), nullptr, nullptr, th)) return false;
+  hc_combine(d, hc, rr.data(), y.data(), inj2.data(), 1);
+  s_out.assign(d, 0.0f);
+  return hc_mix(d, hc, c.eps, m->mix_norm.data(), &m->t[ORC_MTP_MIX_DOWN], nullptr, &m->t[ORC_MTP_MIX_UP], rr.data(), 1, s_out.data(), dummy.data(), th);
+}
+bool embd_row(const OrcModel* m, uint32_t id, float* e) { const OrcTensor& embd = m->g[ORC_G_EMBD]; int qk, bs; if (!geom(embd.ty, &qk, &bs)) return false; return dequant(embd.ty, (const uint8_t*)embd.data + (size_t)id * ((size_t)m->c.d / qk * bs), m->c.d, e); }
+}  // namespace
+
+extern "C" {
+OrcMtp* orc_mtp_create(const OrcModel* main, const OrcMtpCfg* cfg, const OrcTensor* tensors, const uint32_t* draft_ids) {
+  OrcMtp* m = new OrcMtp(); m->c = *cfg; m->main = main; for (int i = 0; i < ORC_MTP_SLOTS; ++i) m->t[i] = tensors[i];
+  m->ids.assign(draft_ids, draft_ids + cfg->n_draft_vocab);
+  bool ok = to_vec(m->t[ORC_MTP_PRE_E], m->pre_e) && to_vec(m->t[ORC_MTP_PRE_H], m->pre_h) && to_vec(m->t[ORC_MTP_HCA_NORM], m->hca_norm) && to_vec(m->t[ORC_MTP_HCF_NORM], m->hcf_norm) &&
+            to_vec(m->t[ORC_MTP_MIX_NORM], m->mix_norm) && to_vec(m->t[ORC_MTP_QN], m->qn) && to_vec(m->t[ORC_MTP_KN], m->kn) && to_vec(m->t[ORC_MTP_SH_GATE_INP], m->sgate);
+  if (!ok || (int)m->t[ORC_MTP_HEAD].rows != cfg->n_draft_vocab) { delete m; return nullptr; }
+  m->rope_inv.resize(main->c.n_rot / 2); orc_rope_inv(main->c.n_rot, main->c.rope_base, m->rope_inv.data());      // mtp.rs:111: the unscaled table
+  return m;
+}
+void orc_mtp_destroy(OrcMtp* m) { delete m; }
+void orc_state_attach_mtp(OrcState* st, const OrcMtp* m) { st->mtp_window = m->c.window; }
+const float* orc_mtp_r(const OrcState* st, int pos) { return mtp_r_get(st, pos); }
+int orc_mtp_kv(const OrcState* st, int* c0, const float** k, const float** v) { *c0 = st->mtp_c0; *k = st->mtp_k.data(); *v = st->mtp_v.data(); return st->mtp_n; }
+
+int orc_mtp_draft(const OrcMtp* m, const OrcModel* main, OrcState* st, uint32_t pending, int k, float min_p, uint32_t* ids, float* probs) {
+  const OrcCfg& c = main->c; const int n = (int)st->tokens.size(), d = c.d, w = c.hc * d, row = c.n_kv * c.hd;
+  if (n == 0 || k <= 0) return 0;
+  // kv.truncate(n - 1)
+  if (n - 1 < st->mtp_c0 + st->mtp_n) { const int keep = std::max(0, n - 1 - st->mtp_c0); st->mtp_n = keep; st->mtp_k.resize((size_t)keep * row); st->mtp_v.resize((size_t)keep * row); }
+  // catch-up over the cells whose residual is known and whose token is committed, :2194-2217
+  const int first = st->mtp_r.empty() ? n : st->mtp_r.front().first;
+  const int end = st->mtp_c0 + st->mtp_n;
+  const int lo = (st->mtp_n > 0 && end >= first) ? end : std::max(first, std::max(0, (n - 1) - m->c.window));
+  if (lo < n - 1) {
+    const int nc = n - 1 - lo; std::vector<float> rs((size_t)nc * w), es((size_t)nc * d); bool ok = true;
+    for (int j = 0; j < nc; ++j) { const float* r = mtp_r_get(st, lo + j); if (!r) { ok = false; break; } memcpy(&rs[(size_t)j * w], r, sizeof(float) * w); if (!embd_row(main, st->tokens[lo + j + 1], &es[(size_t)j * d])) return -1; }
+    if (ok) { std::vector<float> rr, mx, inj; for (int c0 = 0; c0 < nc; c0 += 64) { const int nn = std::min(64, nc - c0); if (!mtp_kv_append(m, st, &rs[(size_t)c0 * w], &es[(size_t)c0 * d], nn, lo + c0, rr, mx, inj)) return -1; } }
+    else { st->mtp_c0 = 0; st->mtp_n = 0; st->mtp_k.clear(); st->mtp_v.clear(); }
+  }
+  const float* r0 = mtp_r_get(st, n - 1); if (!r0) return 0;
+  std::vector<float> r(r0, r0 + w), e(d), s, r2, lg(m->c.n_draft_vocab); uint32_t tok = pending; int out = 0;
+  for (int j = 0; j < k; ++j) {
+    if (!embd_row(main, tok, e.data())) return -1;
+    if (!mtp_step(m, st, r.data(), e.data(), n - 1 + j, s, r2)) return -1;
+    if (!mm(&m->t[ORC_MTP_HEAD], s.data(), 1, lg.data(), main->threads)) return -1;
+    size_t bi = 0; float bv = -INFINITY; for (size_t i = 0; i < lg.size(); ++i) if (lg[i] > bv) { bv = lg[i]; bi = i; }      // best, mtp.rs:424-427
+    float z = 0.0f; for (float v : lg) z += expf(v - bv); const float p = 1.0f / z;
+    if (j > 0 && p < min_p) break;                                                        // draft_gate with the policy off
+    ids[out] = m->ids[bi]; probs[out] = p; ++out; r = r2; tok = ids[out - 1];
+  }
+  // kv.truncate(n)
+  if (n < st->mtp_c0 + st->mtp_n) { const int keep = std::max(0, n - st->mtp_c0); st->mtp_n = keep; st->mtp_k.resize((size_t)keep * row); st->mtp_v.resize((size_t)keep * row); }
+  return out;
+}
+
+int orc_generate_greedy_mtp(const OrcModel* m, const OrcMtp* mtp, OrcState* st, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* drafted, int* accepted) {
+  const size_t V = m->c.vocab; int produced = 0, nd = 0, na = 0; uint32_t pending = orc_argmax(first_logits, V); std::vector<float> ls;
+  for (;;) {
+    out[produced++] = pending; if (produced >= n_out) break;
+    const int left = n_out - produced; const int kk = std::min(k, left - 1);
+    uint32_t dr[8]; float dp[8]; int got = kk > 0 ? orc_mtp_draft(mtp, m, st, pending, std::min(kk, 7), min_p, dr, dp) : 0; if (got < 0) return -1;
+    std::vector<uint32_t> toks{pending}; for (int j = 0; j < got; ++j) toks.push_back(dr[j]);
+    ls.resize(toks.size() * V); if (orc_forward_multi(m, st, toks.data(), (int)toks.size(), ls.data())) return -1;
+    int acc = 0; bool have = false; uint32_t nx = 0;
+    for (int i = 0; i < got; ++i) { const uint32_t tk = orc_argmax(&ls[(size_t)i * V], V); if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = orc_argmax(&ls[(size_t)got * V], V);
+    orc_spec_keep(m, st, (int)toks.size(), acc + 1); nd += got; na += acc;
+    bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
+    if (stop) break;
+    pending = nx;
+  }
+  if (drafted) *drafted = nd; if (accepted) *accepted = na; return 0;
+}
 }  // extern "C"

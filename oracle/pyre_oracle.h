@@ -39,6 +39,13 @@
  *                          sequence start and at eos, 64-bit wrap, xor); zero value -> the conv over a hand-set history
  *                          tap by tap; zero key -> the gate floor; one-hot key / stream -> the gate in closed form;
  *                          constant gated stream -> the norm weight; window == single tokens
+ *   orc_mtp_draft          closed forms: a zero head -> the first draft id with probability exactly 1 / n and the min_p gate
+ *                          sparing only the first draft; a zero fc_hidden -> a cell depends only on the token one position
+ *                          ahead and its key is that token's key turned by the plain rope table at the cell's index (under
+ *                          a YaRN-scaled main model); a zero fc_embedding -> a cell depends only on its position's residual;
+ *                          catch-up start / window / both truncations as numbers worked out by hand; the draft step as the
+ *                          composition of the pinned block entry points (matmul, hc_mix, hc_combine, attn_core, moe_ffn);
+ *                          generation with the drafter proposing == plain greedy
  * Parity unpinned (only running the reference could pin): the last-ulp behaviour of
  * expf/log1pf/powf/sincosf on the reference's own target libm.
  */
@@ -149,8 +156,40 @@ int    orc_hc_mix(int d, int hc, float eps, const float* norm, const OrcTensor* 
                   const OrcTensor* up, const float* x, int t, float* mixed, float* inj, int threads);
 void   orc_hc_combine(int d, int hc, float* x, const float* out, const float* inj, int t);
 
+/* ---- the multi-token-prediction (MTP) drafter, src/model/mtp.rs ------------------------------------------------------
+ * One extra block that pairs the main model's final residual streams R_i with the token at i + 1 (cell i, rope position
+ * i) and predicts token i + 2; its own residual feeds the next draft step.  Only draft quality depends on it: every
+ * emitted token comes from the verify pass.  Tensors are given in the types the caller chose (the reference builds
+ * int8 copies of a BF16 checkpoint, mtp.rs:11-13); norm weights already carry their "1 + w" (mtp.rs:44-45). */
+enum {
+  ORC_MTP_PRE_E = 0, ORC_MTP_PRE_H,                       /* pre_fc_norm_embedding [d], pre_fc_norm_hidden [hc*d] */
+  ORC_MTP_FC_E, ORC_MTP_FC_H,                             /* fc_embedding [d x d], fc_hidden [d x d] (applied per stream) */
+  ORC_MTP_HCA_NORM, ORC_MTP_HCA_DOWN, ORC_MTP_HCA_INJECT, ORC_MTP_HCA_UP,      /* attn_hyper_connection.* */
+  ORC_MTP_HCF_NORM, ORC_MTP_HCF_DOWN, ORC_MTP_HCF_INJECT, ORC_MTP_HCF_UP,      /* mlp_hyper_connection.* */
+  ORC_MTP_MIX_NORM, ORC_MTP_MIX_DOWN, ORC_MTP_MIX_UP,                          /* hyper_connection_mixer.* (no inject) */
+  ORC_MTP_Q, ORC_MTP_K, ORC_MTP_V, ORC_MTP_O, ORC_MTP_QN, ORC_MTP_KN,          /* self_attn.* */
+  ORC_MTP_ROUTER, ORC_MTP_GATE_E, ORC_MTP_UP_E, ORC_MTP_DOWN_E,                /* mlp.gate, mlp.experts.{gate,up}_proj halves, down_proj */
+  ORC_MTP_SH_GATE_INP, ORC_MTP_SH_GATE, ORC_MTP_SH_UP, ORC_MTP_SH_DOWN,        /* mlp.shared_expert_gate, mlp.shared_expert.* */
+  ORC_MTP_HEAD,                                            /* the draft-vocabulary rows of the main model's output matrix */
+  ORC_MTP_SLOTS
+};
+typedef struct { int32_t n_exp, top_k, ff, window, n_draft_vocab; } OrcMtpCfg;      /* geometry beyond the main model's (Geo, mtp.rs:100) */
+typedef struct OrcMtp OrcMtp;
 typedef struct OrcModel OrcModel;
 typedef struct OrcState OrcState;
+OrcMtp*   orc_mtp_create(const OrcModel* main, const OrcMtpCfg* cfg, const OrcTensor* tensors /*[ORC_MTP_SLOTS]*/, const uint32_t* draft_ids /*[n_draft_vocab]*/);
+void      orc_mtp_destroy(OrcMtp*);
+/* the state keeps the last window + 16 final residuals from now on (mtp_keep_r, qwen4exp_gguf.rs:2279-2285) */
+void      orc_state_attach_mtp(OrcState*, const OrcMtp*);
+/* mtp_draft (qwen4exp_gguf.rs:2180-2277, host path, draft policy off): catch the drafter's K/V up over the cells whose token is
+ * committed, then up to k draft steps from (R_{n-1}, pending); a later draft is kept only while the drafter's probability of
+ * its choice is >= min_p (spec::draft_gate, spec.rs:326-327).  Returns the number of drafts; ids / probabilities out. */
+int       orc_mtp_draft(const OrcMtp*, const OrcModel* main, OrcState*, uint32_t pending, int k, float min_p, uint32_t* ids, float* probs);
+/* test access: the kept final residual streams [hc*d] of position pos (NULL when not kept); cells [c0, c0 + n) of the drafter's K / V [n][nkv*hd] */
+const float* orc_mtp_r(const OrcState*, int pos);
+int       orc_mtp_kv(const OrcState*, int* c0, const float** k, const float** v);
+/* spec::generate's greedy branch with the drafter proposing (spec.rs:156-267): n_out tokens; rounds / drafted / accepted counts out */
+int       orc_generate_greedy_mtp(const OrcModel*, const OrcMtp*, OrcState*, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* drafted, int* accepted);
 OrcModel* orc_model_create(const OrcCfg* cfg, const OrcTensor* layer_tensors /*[n_layers][ORC_LAYER_SLOTS]*/,
                            const OrcTensor* globals /*[ORC_GLOBAL_SLOTS]*/, int threads);
 void      orc_model_destroy(OrcModel*);

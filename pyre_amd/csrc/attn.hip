@@ -575,6 +575,14 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   return PYRE_OK;
 }
 
+// K / V of positions start..start+t-1 into an f32 cache, nothing attended (the drafter's catch-up over committed cells)
+int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t) {
+  if (a.hd != 256 || a.kv_bits != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "attention append: head dim %d, %d-bit cache (256, f32 only)", a.hd, a.kv_bits);
+  if (t < 1 || t > 8 || start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention append: positions %d..%d outside the cache (%d)", start, start + t, kv.cap);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, (const int*)nullptr, w.q); } PYRE_CHECK_LAUNCH(ctx);
+  return PYRE_OK;
+}
+
 // ---- C ABI: standalone attention layer core for the block harness -----------------------------------------------------
 struct pyre_attn { pyre_ctx* ctx; AttnDev dv; KvDev kv; AttnWork w; float* params; void* kvmem; void* wmem; float* io; int len, packed, cap;
                    QsaDev q{}; QsaBuf qb{}; QsaWork qw{}; void* qmem = nullptr; float* qparams = nullptr; float rope_base = 0; };

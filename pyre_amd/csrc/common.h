@@ -344,3 +344,4 @@ int pyre_qsa_pool_all(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const Qs
 // the attention launch with an optional position list (qw == nullptr: dense)
 int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
                          int* packed_done, float* out_dev, const int* posp, const QsaWork* qw, uint16_t* aop = nullptr);
+int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t);      // K / V only

@@ -46,6 +46,16 @@ struct pyre_state {
   uint32_t* tokens_dev = nullptr; std::vector<float*> ple_ring;     // PLE models: the token history by position; per PLE layer the ring of normalised rows
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
   std::vector<int> graph_cur;                                    // which half of every DeltaNet double buffer the captured step works on
+  // MTP drafter (attached by pyre_state_attach_mtp): the ring of final residual streams by position, of which positions
+  // [r_first, r_next) are valid; the drafter's own K/V cache by cell, of which cells [m_c0, m_c0 + m_n) are valid
+  const pyre_mtp* mtp = nullptr; void* mtp_mem = nullptr; float* r_ring = nullptr; int r_mask = 0, r_first = 0, r_next = 0;
+  KvDev mkv{}; int* mlist = nullptr; int* mcount = nullptr; int m_c0 = 0, m_n = 0;
+  // mtp_keep_r (qwen4exp_gguf.rs:2279-2285) for positions start .. start+t-1, whose rows a kernel on the stream writes
+  void r_push(int start, int t, int window) {
+    if (r_next > start) r_next = start;                          // newer rows are dropped (a rolled-back window)
+    if (r_next <= r_first || r_next != start) r_first = start;   // a gap empties the ring
+    r_next = start + t; if (r_next - r_first > window + 16) r_first = r_next - (window + 16);
+  }
 };
 
 namespace {
@@ -263,13 +273,13 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
   *out = S.release(); return PYRE_OK;
 }
-void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec); (void)hipFree(s->mem); delete s; }
+void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec); (void)hipFree(s->mem); if (s->mtp_mem) (void)hipFree(s->mtp_mem); delete s; }
 int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
   if (!ctx || !s) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_reset: null argument");
   const pyre_model_cfg& c = s->m->c; size_t cs = (size_t)(c.conv_k - 1) * s->m->ch * 4, ss = (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4;
   for (size_t li = 0; li < s->cur.size(); ++li) { s->cur[li] = 0; PYRE_HIP(ctx, hipMemsetAsync(s->conv[0][li], 0, cs, ctx->stream)); PYRE_HIP(ctx, hipMemsetAsync(s->ssm[0][li], 0, ss, ctx->stream)); }
   for (auto& pk : s->packed) pk = 0;
-  s->len = 0; s->last_window = 0; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+  s->len = 0; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 int pyre_state_len(const pyre_state* s) { return s ? s->len : 0; }
 int pyre_state_capacity(const pyre_state* s) { return s ? s->cap - 8 : 0; }
@@ -346,7 +356,7 @@ int pyre_state_restore(pyre_ctx* ctx, pyre_state* s, const pyre_snap* sn) {
   if (s->m != sn->m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: the snapshot belongs to another model");
   if (sn->len + 8 > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: %d positions do not fit the state's capacity %d", sn->len, s->cap - 8);
   int rc = snap_copy(ctx, s->m, s, (uint8_t*)sn->mem, sn->len, 1); if (rc) return rc;
-  s->len = sn->len; s->packed = sn->packed; s->last_window = 0;
+  s->len = sn->len; s->packed = sn->packed; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0;      // the drafter starts over
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 void pyre_snap_destroy(pyre_snap* sn) { if (!sn) return; (void)hipFree(sn->mem); delete sn; }
@@ -391,7 +401,16 @@ struct WinOpt {
   int* step_dev = nullptr;      // replayable form: position and output slot live in device memory (see pyre_pick_launch);
                                 // recurrent state is updated in place and no host-side bookkeeping is touched
   bool inplace = false;         // update the recurrent state in its current buffer (no pre-window copy for spec_keep)
+  int keep_from = 0;            // with a drafter attached: the final residual streams of tokens keep_from .. t-1 go to the state's ring
 };
+
+// rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
+__global__ __launch_bounds__(256) void k_ring_store(const float* __restrict__ x, float* __restrict__ ring, int mask, int start, const int* __restrict__ posp, int from, int w) {
+  if (posp) start = *posp;
+  const int i = blockIdx.x * 256 + threadIdx.x, ti = from + blockIdx.y; if (i >= w) return;
+  ring[(size_t)((start + ti) & mask) * w + i] = x[(size_t)ti * w + i];
+}
+int mtp_window_of(const pyre_mtp* m);
 
 bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) && (int)L.outp.rows == d && L.hcf.di.fmt == FMT_IQ3_S; }
 
@@ -407,8 +426,9 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
-  if (m->n_ple > 0) {      // the window's tokens join the history, then every position's n-gram rows are fetched once for all PLE layers
-    if (!o.from_best) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, m->ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  // the window's tokens join the history (PLE models and states with a drafter keep one)
+  if (s->tokens_dev && !o.from_best) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, m->ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  if (m->n_ple > 0) {      // every position's n-gram rows are fetched once for all PLE layers
     if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
   }
   const bool fuse_aop = [] { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }();      // 1: separate split launches instead of the producers' own operand stores
@@ -448,9 +468,18 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     comb_inj = m->inj_f;
   }
   if (!replay) s->len = start + t;
-  if (o.head_tokens == 0) return PYRE_OK;       // prompt window whose logits nobody reads
-  if (o.head_tokens >= t) {
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->out)))) return rc;
+  const bool want_r = s->mtp && o.keep_from < t;      // the head mix resolves the pending update of every token: its x_out rows are the final residual streams
+  if (o.head_tokens == 0 && !want_r) return PYRE_OK;       // prompt window whose logits nobody reads
+  if (o.head_tokens >= t || want_r) {
+    const bool all = o.head_tokens >= t;
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, 1, all ? opw(m->out) : nullptr))) return rc;
+    if (want_r) {
+      const int w = hc * d;
+      hipLaunchKernelGGL(k_ring_store, dim3((w + 255) / 256, t - o.keep_from), dim3(256), 0, ctx->stream, xout, s->r_ring, s->r_mask, start, o.step_dev, o.keep_from, w); PYRE_CHECK_LAUNCH(ctx);
+      if (!replay) s->r_push(start + o.keep_from, t - o.keep_from, mtp_window_of(s->mtp));
+    }
+    if (o.head_tokens == 0) return PYRE_OK;
+    if (!all) return pyre_gemv_launch(ctx, m->out, m->hbuf + (size_t)(t - 1) * d, 1, m->logits);      // the last token's logits only
     if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->out));
     return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->out));
   }
@@ -481,6 +510,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     int t = n - i < 8 ? n - i : 8; bool last = i + t >= n;
     PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
     WinOpt o; o.head_tokens = last && logits_host ? 1 : 0;
+    if (s->mtp) { const int k0 = n - mtp_window_of(s->mtp) - i; o.keep_from = k0 < 0 ? 0 : k0; }      // the last `window` tokens of a call (qwen4exp_gguf.rs:2148-2150)
     if ((rc = run_window(ctx, m, s, t, o))) return rc;
   }
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
@@ -494,7 +524,7 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
-  { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
+  { WinOpt o; o.head_tokens = n; if (s->mtp && n > mtp_window_of(s->mtp)) o.keep_from = n - mtp_window_of(s->mtp); if ((rc = run_window(ctx, m, s, n, o))) return rc; }
   s->last_window = n;
   PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)n * m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
@@ -523,7 +553,7 @@ static int forward_multi_picks(pyre_ctx* ctx, const pyre_model* m, pyre_state* s
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward_multi: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
-  { WinOpt o; o.head_tokens = n; if ((rc = run_window(ctx, m, s, n, o))) return rc; }
+  { WinOpt o; o.head_tokens = n; if (s->mtp && n > mtp_window_of(s->mtp)) o.keep_from = n - mtp_window_of(s->mtp); if ((rc = run_window(ctx, m, s, n, o))) return rc; }
   s->last_window = n;
   hipLaunchKernelGGL(k_argmax_rows, dim3(n), dim3(1024), 0, ctx->stream, m->logits, m->c.vocab, m->best);
   PYRE_CHECK_LAUNCH(ctx);
@@ -581,6 +611,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
       }
       for (int i = 1; i < n_steps; ++i) PYRE_HIP(ctx, hipGraphLaunch(s->graph_exec, ctx->stream));
     }
+    if (s->mtp) s->r_push(s->len, n_steps - 1, mtp_window_of(s->mtp));      // the replayed steps stored their rows themselves
     s->len += n_steps - 1;
     for (size_t ai = 0; ai < s->packed.size(); ++ai) { int pb = (int)pyre_packed_boundary((size_t)s->len, m->c.kv_bits, m->c.kv_recent); if (pb > s->packed[ai]) s->packed[ai] = pb; }
   }
@@ -668,6 +699,273 @@ int pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s
     if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
     ++rounds; drafted += nd; accepted += acc;
     bool stop = false; for (int i = 0; i < acc; ++i) { hist.push_back(toks[i + 1]); out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
+    if (stop) break;
+    pending = nx;
+  }
+  if (rounds_out) *rounds_out = rounds; if (drafted_out) *drafted_out = drafted; if (accepted_out) *accepted_out = accepted;
+  return PYRE_OK;
+}
+
+}  // extern "C"
+
+// ---- the MTP drafter (src/model/mtp.rs; Model::mtp_draft, src/model/qwen4exp_gguf.rs:2180-2277) --------------------------------
+// Launch sequence of one draft step at cell p (R = the main model's final residual streams of position p for the first
+// step, the drafter's own residual afterwards; token = the token at position p + 1):
+//   row look-up of the token's embedding -> k_mtp_in (the two pre-norms) -> fc_embedding GEMV, fc_hidden GEMV over the
+//   hc streams -> attention mix (adds the embedding part to every stream on the way: a pending update with weight
+//   2 * sigmoid(0) = 1) -> [q ; k ; v] GEMV -> attention over the cells of the window (a position list) -> output GEMV
+//   -> FFN mix -> MoE FFN -> mixer -> head GEMV over the draft vocabulary -> k_mtp_best (id, probability, next token).
+// The catch-up over committed cells stops after the K / V append.
+struct pyre_mtp {
+  pyre_ctx* ctx = nullptr; const pyre_model* main = nullptr; pyre_mtp_cfg c{};
+  pyre_model shell;                 // owner of the drafter's matrices and vectors (Builder's bookkeeping)
+  QMatDev fc_e{}, fc_h{}, qkv{}, outp{}, head{}; HcDev hca{}, hcf{}, mix{}; MoeDev moe{}; AttnDev attn{};
+  const float *pre_e = nullptr, *pre_h = nullptr; uint32_t* ids_dev = nullptr;
+  void* work = nullptr; HcWork hw{}; MoeWork mw{};
+  float *emb, *en, *e2, *hn, *xh, *ra, *rb, *rc, *mixed, *inj_a, *inj_f, *inj_m, *zeros, *proj, *core, *bo, *y, *sh, *logits, *out_p;
+  uint32_t *out_ids, *tok; int pw = 0;
+};
+
+namespace {
+int mtp_window_of(const pyre_mtp* m) { return m->c.window; }
+
+// grid t, 256 threads: en = rms(emb row, pre_e) [t][d]; hn = rms(R row over all hc*d values, pre_h) [t][hc*d].
+// R row of cell ti: ring row (pos0 + ti) & mask, or row ti of a plain buffer when mask < 0.
+__global__ __launch_bounds__(256) void k_mtp_in(const float* __restrict__ emb, const float* __restrict__ r, int mask, int pos0, const float* __restrict__ pre_e, const float* __restrict__ pre_h,
+                                                int d, int w, float eps, float* __restrict__ en, float* __restrict__ hn) {
+  __shared__ float red[4];
+  const int ti = blockIdx.x, tid = threadIdx.x;
+  const float* e = emb + (size_t)ti * d; const float* rr = r + (size_t)(mask < 0 ? ti : ((pos0 + ti) & mask)) * w;
+  float se = 0.0f, sr = 0.0f;
+  for (int i = tid; i < d; i += 256) se += e[i] * e[i];
+  for (int i = tid; i < w; i += 256) sr += rr[i] * rr[i];
+  auto bsum = [&](float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads(); if ((tid & 63) == 0) red[tid >> 6] = v; __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]); };
+  se = bsum(se); sr = bsum(sr);
+  const float ke = 1.0f / sqrtf(se / (float)d + eps), kr = 1.0f / sqrtf(sr / (float)w + eps);
+  for (int i = tid; i < d; i += 256) en[(size_t)ti * d + i] = e[i] * ke * pre_e[i];
+  for (int i = tid; i < w; i += 256) hn[(size_t)ti * w + i] = rr[i] * kr * pre_h[i];
+}
+
+// best (mtp.rs:424-427) of the draft head's logits: the first maximum, its probability 1 / sum exp(v - max); one block
+__global__ __launch_bounds__(1024) void k_mtp_best(const float* __restrict__ l, int n, const uint32_t* __restrict__ ids, uint32_t* __restrict__ out_id, float* __restrict__ out_p, uint32_t* __restrict__ tok) {
+  __shared__ float sv[16]; __shared__ uint32_t si[16]; __shared__ float bvs; __shared__ uint32_t bis;
+  const int tid = threadIdx.x;
+  float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
+  for (int i = tid; i < n; i += 1024) { const float v = l[i]; if (v > bv) { bv = v; bi = (uint32_t)i; } }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { const float ov = __shfl_xor(bv, o); const uint32_t oi = __shfl_xor(bi, o); if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; } }
+  if ((tid & 63) == 0) { sv[tid >> 6] = bv; si[tid >> 6] = bi; }
+  __syncthreads();
+  if (tid == 0) { for (int q = 1; q < 16; ++q) if (si[q] != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || sv[q] > bv || (sv[q] == bv && si[q] < bi))) { bv = sv[q]; bi = si[q]; }
+    bvs = bv; bis = bi == 0xFFFFFFFFu ? 0u : bi; }
+  __syncthreads();
+  bv = bvs; float z = 0.0f;
+  for (int i = tid; i < n; i += 1024) z += expf(l[i] - bv);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) z += __shfl_xor(z, o);
+  __syncthreads();
+  if ((tid & 63) == 0) sv[tid >> 6] = z;
+  __syncthreads();
+  if (tid == 0) { float t = 0.0f; for (int q = 0; q < 16; ++q) t += sv[q]; const uint32_t id = ids[bis]; *out_id = id; *out_p = 1.0f / t; *tok = id; }
+}
+
+struct MtpCounts { int c[8]; };
+// the position list of a draft call: list[i] = lo + i; count[j] = cells step j attends to
+__global__ void k_mtp_list(int* __restrict__ list, int lo, int n, int* __restrict__ count, MtpCounts cn) {
+  const int i = blockIdx.x * 256 + threadIdx.x; if (i < n) list[i] = lo + i; if (i < 8) count[i] = cn.c[i];
+}
+
+// cells pos0 .. pos0+t-1 (t * hc <= 8): input, attention mix, [q ; k ; v]; leaves the streams in m->ra, the mix's inject logits in m->inj_a
+int mtp_cells(pyre_ctx* ctx, const pyre_mtp* m, const float* r, int mask, int pos0, int t) {
+  const pyre_model_cfg& c = m->main->c; const int d = c.d, hc = c.hc, w = hc * d; int rc;
+  hipLaunchKernelGGL(k_mtp_in, dim3(t), dim3(256), 0, ctx->stream, m->emb, r, mask, pos0, m->pre_e, m->pre_h, d, w, c.eps, m->en, m->hn); PYRE_CHECK_LAUNCH(ctx);
+  if ((rc = pyre_gemv_launch(ctx, m->fc_e, m->en, t, m->e2))) return rc;
+  if ((rc = pyre_gemv_launch(ctx, m->fc_h, m->hn, t * hc, m->xh))) return rc;
+  if ((rc = pyre_hc_mix_launch(ctx, m->hca, m->hw, m->xh, d, w, m->ra, t, m->e2, nullptr, m->zeros, c.eps, m->mixed, m->inj_a, nullptr, 1, nullptr))) return rc;
+  return pyre_gemv_launch(ctx, m->qkv, m->mixed, t, m->proj);
+}
+}  // namespace
+
+extern "C" {
+
+int pyre_mtp_create(pyre_ctx* ctx, const pyre_model* main, const pyre_mtp_cfg* cfg, const pyre_tensor* T, const uint32_t* draft_ids, pyre_mtp** out) {
+  if (!ctx || !main || !cfg || !T || !draft_ids || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_create: null argument");
+  *out = nullptr; const pyre_model_cfg& c = main->c; const int d = c.d, hc = c.hc, w = hc * d;
+  if (cfg->n_exp < 1 || cfg->n_exp > 1024 || cfg->top_k < 1 || cfg->top_k > 32 || cfg->top_k > cfg->n_exp || cfg->ff < 64 || cfg->ff % 64 || cfg->window < 1 || cfg->n_draft_vocab < 1 || 8 / hc < 1)
+    return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_mtp_create: %d experts top %d of width %d, window %d, %d draft rows", cfg->n_exp, cfg->top_k, cfg->ff, cfg->window, cfg->n_draft_vocab);
+  for (int i = 0; i < cfg->n_draft_vocab; ++i) if (draft_ids[i] >= (uint32_t)c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_create: draft id %u outside the vocabulary (%d)", draft_ids[i], c.vocab);
+  PYRE_HIP(ctx, hipSetDevice(ctx->device));
+  std::unique_ptr<pyre_mtp> M(new pyre_mtp()); pyre_mtp* m = M.get(); m->ctx = ctx; m->main = main; m->c = *cfg; m->shell.ctx = ctx; m->shell.c = c;
+  struct Guard { pyre_mtp* m; bool armed = true; ~Guard() { if (armed) { for (auto q : m->shell.owned) pyre_qmat_destroy(q); for (auto b : m->shell.bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); } } } guard{m};
+  Builder B{ctx, &m->shell}; int rc;
+  const int mlay = [] { const char* e = getenv("PYRE_MODEL_ROWS"); return e && *e && atoi(e) != 0; }() ? PYRE_LAYOUT_ROWS : PYRE_LAYOUT_M;
+  if ((rc = B.vec(T[PYRE_MTP_PRE_E], d, &m->pre_e)) || (rc = B.vec(T[PYRE_MTP_PRE_H], w, &m->pre_h))) return rc;
+  if ((rc = B.one(T[PYRE_MTP_FC_E], &m->fc_e, nullptr, mlay)) || (rc = B.one(T[PYRE_MTP_FC_H], &m->fc_h, nullptr, mlay))) return rc;
+  if (m->fc_e.rows != d || m->fc_e.cols != d || m->fc_h.rows != d || m->fc_h.cols != d) return B.fail(PYRE_E_SHAPE, "fc_embedding / fc_hidden must be d x d");
+  auto hcb = [&](int norm, int down, int inject, int up, HcDev* h) { m->shell.c.hc_lr = (int)T[down].rows; return B.hc(T[norm], T[down], inject >= 0 ? &T[inject] : nullptr, T[up], h, nullptr); };
+  if ((rc = hcb(PYRE_MTP_HCA_NORM, PYRE_MTP_HCA_DOWN, PYRE_MTP_HCA_INJECT, PYRE_MTP_HCA_UP, &m->hca)) || (rc = hcb(PYRE_MTP_HCF_NORM, PYRE_MTP_HCF_DOWN, PYRE_MTP_HCF_INJECT, PYRE_MTP_HCF_UP, &m->hcf)) ||
+      (rc = hcb(PYRE_MTP_MIX_NORM, PYRE_MTP_MIX_DOWN, -1, PYRE_MTP_MIX_UP, &m->mix))) return rc;
+  { const pyre_tensor* grp[3] = {&T[PYRE_MTP_Q], &T[PYRE_MTP_K], &T[PYRE_MTP_V]};
+    if (grp[0]->rows != (uint64_t)c.n_head * 2 * c.hd || grp[1]->rows != (uint64_t)c.n_kv * c.hd || grp[2]->rows != (uint64_t)c.n_kv * c.hd || grp[0]->cols != (uint64_t)d) return B.fail(PYRE_E_SHAPE, "drafter attention projection shapes");
+    if ((rc = B.cat(grp, 3, &m->qkv, nullptr, mlay))) return rc; m->pw = c.n_head * 2 * c.hd + 2 * c.n_kv * c.hd; }
+  if (T[PYRE_MTP_O].rows != (uint64_t)d || T[PYRE_MTP_O].cols != (uint64_t)c.n_head * c.hd) return B.fail(PYRE_E_SHAPE, "drafter o_proj shape");
+  if ((rc = B.one(T[PYRE_MTP_O], &m->outp, nullptr, mlay))) return rc;
+  std::vector<float> inv(c.n_rot / 2 + 1); (void)pyre_rope_table(c.n_rot, c.rope_base, 0, 0, inv.data());      // mtp.rs:111: the unscaled table
+  float* rinv = nullptr; PYRE_HIP(ctx, hipMalloc((void**)&rinv, inv.size() * 4)); m->shell.bufs.push_back(rinv);
+  PYRE_HIP(ctx, hipMemcpy(rinv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice));
+  m->attn = AttnDev{nullptr, nullptr, rinv, c.n_head, c.n_kv, c.hd, c.n_rot, 0, 0, c.eps, 1.0f};
+  if ((rc = B.vec(T[PYRE_MTP_QN], c.hd, &m->attn.qn)) || (rc = B.vec(T[PYRE_MTP_KN], c.hd, &m->attn.kn))) return rc;
+  MoeDev& mo = m->moe;
+  if ((rc = B.one(T[PYRE_MTP_ROUTER], &mo.router, nullptr)) || (rc = B.one(T[PYRE_MTP_GATE_E], &mo.gate_e, nullptr)) || (rc = B.one(T[PYRE_MTP_UP_E], &mo.up_e, nullptr)) || (rc = B.one(T[PYRE_MTP_DOWN_E], &mo.down_e, nullptr)) ||
+      (rc = B.one(T[PYRE_MTP_SH_GATE], &mo.sh_gate, nullptr)) || (rc = B.one(T[PYRE_MTP_SH_UP], &mo.sh_up, nullptr)) || (rc = B.one(T[PYRE_MTP_SH_DOWN], &mo.sh_down, nullptr))) return rc;
+  mo.d = d; mo.n_exp = cfg->n_exp; mo.top_k = cfg->top_k; mo.ff = cfg->ff; mo.sf = mo.sh_gate.rows;
+  if (mo.router.rows != cfg->n_exp || mo.router.cols != d || mo.gate_e.rows != cfg->n_exp * cfg->ff || mo.up_e.rows != cfg->n_exp * cfg->ff || mo.gate_e.cols != d || mo.up_e.cols != d ||
+      (size_t)mo.down_e.rows != (size_t)cfg->n_exp * d || mo.down_e.cols != cfg->ff || mo.sh_up.rows != mo.sf || mo.sh_down.rows != d || mo.sh_down.cols != mo.sf || mo.sf % 64)
+    return B.fail(PYRE_E_SHAPE, "drafter expert tensor shapes");
+  if (mo.gate_e.fmt != mo.up_e.fmt || mo.sh_gate.fmt != mo.gate_e.fmt || mo.sh_up.fmt != mo.gate_e.fmt || mo.sh_down.fmt != mo.down_e.fmt) return B.fail(PYRE_E_TYPE, "gate/up (and shared) expert types must agree");
+  if ((rc = B.vec(T[PYRE_MTP_SH_GATE_INP], d, &mo.sh_gate_inp))) return rc;
+  if ((rc = B.one(T[PYRE_MTP_HEAD], &m->head, nullptr, mlay))) return rc;
+  if (m->head.rows != cfg->n_draft_vocab || m->head.cols != d) return B.fail(PYRE_E_SHAPE, "the draft head must hold n_draft_vocab rows of d");
+  PYRE_HIP(ctx, hipMalloc((void**)&m->ids_dev, (size_t)cfg->n_draft_vocab * 4)); m->shell.bufs.push_back(m->ids_dev);
+  PYRE_HIP(ctx, hipMemcpy(m->ids_dev, draft_ids, (size_t)cfg->n_draft_vocab * 4, hipMemcpyHostToDevice));
+  // workspace for up to 8 rows
+  HcDev hmax = m->hca; hmax.lr = std::max(m->hca.lr, std::max(m->hcf.lr, m->mix.lr));
+  const size_t moe_b = pyre_moe_work_bytes(mo), f8d = 4 * 8 * (size_t)d, nhd = (size_t)c.n_head * c.hd;
+  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 13 * al256(f8d) + 5 * al256(4 * 64) + al256(4 * 8 * (size_t)m->pw) + al256(4 * 8 * nhd) + al256(4 * (size_t)cfg->n_draft_vocab) + 3 * 256 + 4096;
+  PYRE_HIP(ctx, hipMalloc(&m->work, total)); PYRE_HIP(ctx, hipMemset(m->work, 0, total));
+  uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
+  pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(mo, take(moe_b), &m->mw);
+  m->emb = (float*)take(f8d); m->en = (float*)take(f8d); m->e2 = (float*)take(f8d); m->hn = (float*)take(f8d); m->xh = (float*)take(f8d); m->ra = (float*)take(f8d); m->rb = (float*)take(f8d); m->rc = (float*)take(f8d);
+  m->mixed = (float*)take(f8d); m->bo = (float*)take(f8d); m->y = (float*)take(f8d); m->sh = (float*)take(f8d); (void)take(f8d);
+  m->inj_a = (float*)take(4 * 64); m->inj_f = (float*)take(4 * 64); m->inj_m = (float*)take(4 * 64); m->zeros = (float*)take(4 * 64); (void)take(4 * 64);
+  m->proj = (float*)take(4 * 8 * (size_t)m->pw); m->core = (float*)take(4 * 8 * nhd); m->logits = (float*)take(4 * (size_t)cfg->n_draft_vocab);
+  m->out_p = (float*)take(4 * 8); m->out_ids = (uint32_t*)take(4 * 8); m->tok = (uint32_t*)take(4 * 8);
+  { uint4* op; float* ainv; const int kmax = std::max(d, (int)nhd); if ((rc = pyre_gemm_m_scratch(ctx, (kmax + 255) / 256 * 256, &op, &ainv))) return rc; }      // no draft step allocates
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  guard.armed = false; *out = M.release(); return PYRE_OK;
+}
+
+void pyre_mtp_destroy(pyre_mtp* m) {
+  if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
+  for (auto q : m->shell.owned) pyre_qmat_destroy(q); for (auto b : m->shell.bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work);
+  delete m;
+}
+
+int pyre_state_attach_mtp(pyre_ctx* ctx, pyre_state* s, const pyre_mtp* m) {
+  if (!ctx || !s || !m) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_attach_mtp: null argument");
+  if (s->m != m->main) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_attach_mtp: the drafter was built for another model");
+  if (s->mtp) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_attach_mtp: the state already has a drafter");
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  const pyre_model_cfg& c = s->m->c; const size_t w = (size_t)c.hc * c.d;
+  int rows = 32; while (rows < m->c.window + 24) rows *= 2;      // a window of 8 lands before the oldest of window + 16 kept rows is dropped
+  const size_t rb = al256((size_t)rows * w * 4), kvb = al256(pyre_kv_bytes(m->attn, s->cap)), lb = al256(4 * ((size_t)m->c.window + 16)), tkb = s->tokens_dev ? 0 : al256((size_t)s->cap * 4);
+  hipError_t e = hipMalloc(&s->mtp_mem, rb + kvb + lb + 256 + tkb);
+  if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_attach_mtp: hipMalloc(%zu): %s", rb + kvb + lb + 256 + tkb, hipGetErrorString(e));
+  uint8_t* p = (uint8_t*)s->mtp_mem; auto take = [&](size_t n) { void* r = p; p += n; return r; };
+  s->r_ring = (float*)take(rb); s->r_mask = rows - 1; pyre_kv_carve(m->attn, s->cap, take(kvb), &s->mkv); s->mlist = (int*)take(lb); s->mcount = (int*)take(256);
+  if (tkb) { s->tokens_dev = (uint32_t*)take(tkb); PYRE_HIP(ctx, hipMemset(s->tokens_dev, 0, tkb)); }
+  s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0; s->mtp = m;
+  if (s->graph_exec) { (void)hipGraphExecDestroy(s->graph_exec); s->graph_exec = nullptr; }      // a captured step does not store its residual yet
+  return PYRE_OK;
+}
+
+int pyre_mtp_draft(pyre_ctx* ctx, const pyre_mtp* m, pyre_state* s, uint32_t pending, int k, float min_p, uint32_t* ids_host, float* probs_host, int* n_out) {
+  if (!ctx || !m || !s || !ids_host || !probs_host || !n_out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_draft: null argument");
+  *n_out = 0;
+  if (s->mtp != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_mtp_draft: this drafter is not attached to the state");
+  if (k > 7) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_draft: k = %d above 7", k);
+  const pyre_model* main = m->main; const pyre_model_cfg& c = main->c; const int n = s->len, d = c.d, hc = c.hc, window = m->c.window; int rc;
+  if (n == 0 || k <= 0) return PYRE_OK;
+  if (pending >= (uint32_t)c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_draft: token id %u outside the vocabulary (%d)", pending, c.vocab);
+  if (n - 1 + k > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_mtp_draft: cells up to %d exceed the state's capacity %d", n - 1 + k, s->cap);
+  auto have_r = [&](int pos) { return pos >= s->r_first && pos < s->r_next; };
+  auto grow = [&](int pos0, int t) { if (s->m_c0 + s->m_n != pos0) { s->m_c0 = pos0; s->m_n = 0; } s->m_n += t; if (s->m_n > window) { s->m_c0 += s->m_n - window; s->m_n = window; } };      // kv_append's bookkeeping, mtp.rs:163-176
+  if (n - 1 < s->m_c0 + s->m_n) s->m_n = std::max(0, n - 1 - s->m_c0);                                     // kv.truncate(n - 1)
+  // catch-up over the cells whose residual is known and whose token is committed (:2194-2217)
+  const int first = s->r_next > s->r_first ? s->r_first : n, end = s->m_c0 + s->m_n;
+  const int lo = (s->m_n > 0 && end >= first) ? end : std::max(first, std::max(0, (n - 1) - window));
+  if (lo < n - 1) {
+    bool ok = true; for (int i = lo; i < n - 1; ++i) ok = ok && have_r(i);
+    if (ok) {
+      const int per = 8 / hc;
+      for (int p0 = lo; p0 < n - 1; p0 += per) {
+        const int t = std::min(per, n - 1 - p0);
+        if ((rc = pyre_row_launch(ctx, main->embd, s->tokens_dev + p0 + 1, t, m->emb, d))) return rc;
+        if ((rc = mtp_cells(ctx, m, s->r_ring, s->r_mask, p0, t))) return rc;
+        if ((rc = pyre_attn_append_launch(ctx, m->attn, s->mkv, s->aw, m->proj, m->pw, p0, t))) return rc;
+        grow(p0, t);
+      }
+    } else { s->m_c0 = 0; s->m_n = 0; }
+  }
+  if (!have_r(n - 1)) return PYRE_OK;
+  // the k draft steps: cell n-1+j attends to the window's cells, which the host knows in advance
+  int c0 = s->m_c0, cn = s->m_n, lo0 = 0; MtpCounts cnt{}; int c0j[8];
+  for (int j = 0; j < k; ++j) { const int pos = n - 1 + j; if (c0 + cn != pos) { c0 = pos; cn = 0; } ++cn; if (cn > window) { c0 += cn - window; cn = window; } c0j[j] = c0; cnt.c[j] = cn; if (j == 0) lo0 = c0; }
+  const int nlist = n - 1 + k - lo0;
+  hipLaunchKernelGGL(k_mtp_list, dim3((std::max(nlist, 8) + 255) / 256), dim3(256), 0, ctx->stream, s->mlist, lo0, nlist, s->mcount, cnt); PYRE_CHECK_LAUNCH(ctx);
+  PYRE_HIP(ctx, hipMemcpyAsync(m->tok, &pending, 4, hipMemcpyHostToDevice, ctx->stream));
+  const float* r = s->r_ring; int mask = s->r_mask, rpos = n - 1;
+  for (int j = 0; j < k; ++j) {
+    const int pos = n - 1 + j;
+    if ((rc = pyre_row_launch(ctx, main->embd, m->tok, 1, m->emb, d))) return rc;
+    if ((rc = mtp_cells(ctx, m, r, mask, rpos, 1))) return rc;
+    QsaWork qw{}; qw.plist = s->mlist + (c0j[j] - lo0); qw.pcount = s->mcount + j; qw.list_stride = window;
+    int packed = 0;
+    if ((rc = pyre_attn_launch_sel(ctx, m->attn, s->mkv, s->aw, m->proj, m->pw, pos, 1, &packed, m->core, nullptr, &qw, nullptr))) return rc;
+    if ((rc = pyre_gemv_launch(ctx, m->outp, m->core, 1, m->bo))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->hcf, m->hw, m->ra, d, hc * d, m->rb, 1, m->bo, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, nullptr, 1, nullptr))) return rc;
+    if ((rc = pyre_moe_launch(ctx, m->moe, m->mw, m->mixed, 1, m->y, nullptr))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->mix, m->hw, m->rb, d, hc * d, m->rc, 1, m->y, nullptr, m->inj_f, c.eps, m->sh, m->inj_m, nullptr, 1, nullptr))) return rc;
+    if ((rc = pyre_gemv_launch(ctx, m->head, m->sh, 1, m->logits))) return rc;
+    hipLaunchKernelGGL(k_mtp_best, dim3(1), dim3(1024), 0, ctx->stream, m->logits, m->c.n_draft_vocab, m->ids_dev, m->out_ids + j, m->out_p + j, m->tok); PYRE_CHECK_LAUNCH(ctx);
+    grow(pos, 1);
+    r = m->rc; mask = -1; rpos = 0;      // the drafter's own residual feeds the next step
+  }
+  uint32_t ids[8]; float ps[8];
+  PYRE_HIP(ctx, hipMemcpyAsync(ids, m->out_ids, (size_t)k * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipMemcpyAsync(ps, m->out_p, (size_t)k * 4, hipMemcpyDeviceToHost, ctx->stream));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  int got = 0; for (int j = 0; j < k; ++j) { if (j > 0 && ps[j] < min_p) break; ids_host[got] = ids[j]; probs_host[got] = ps[j]; ++got; }      // draft_gate, policy off (spec.rs:326-327)
+  if (n < s->m_c0 + s->m_n) s->m_n = std::max(0, n - s->m_c0);                                            // kv.truncate(n): the drafted cells go
+  *n_out = got; return PYRE_OK;
+}
+
+int pyre_mtp_read_kv(pyre_ctx* ctx, pyre_state* s, int* c0, int* n, float* k_host, float* v_host) {
+  if (!ctx || !s || !s->mtp || !c0 || !n) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_read_kv: bad argument");
+  const AttnDev& a = s->mtp->attn; const size_t row = (size_t)a.nkv * a.hd; *c0 = s->m_c0; *n = s->m_n;
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  if (s->m_n == 0) return PYRE_OK;
+  if (v_host) PYRE_HIP(ctx, hipMemcpy(v_host, s->mkv.vf + (size_t)s->m_c0 * row, (size_t)s->m_n * row * 4, hipMemcpyDeviceToHost));
+  if (k_host) {      // keys are blocked by 64 positions: fetch the blocks that hold the cells and pick the rows out on the host
+    const size_t b0 = (size_t)s->m_c0 / 64, b1 = ((size_t)s->m_c0 + s->m_n + 63) / 64; std::vector<float> tmp((b1 - b0) * row * 64);
+    PYRE_HIP(ctx, hipMemcpy(tmp.data(), s->mkv.kf + b0 * row * 64, tmp.size() * 4, hipMemcpyDeviceToHost));
+    for (int i = 0; i < s->m_n; ++i) { const size_t p = (size_t)s->m_c0 + i; for (size_t r = 0; r < row; ++r) k_host[(size_t)i * row + r] = tmp[kv_blk(r, row, p) - b0 * row * 64]; }
+  }
+  return PYRE_OK;
+}
+
+int pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* rounds_out, int* drafted_out, int* accepted_out) {
+  if (!ctx || !m || !mtp || !s || !first_logits || !out || n_out < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp: bad argument");
+  if (k < 1 || k > 7) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp: k %d outside 1..7", k);
+  if (s->mtp != mtp) return pyre_fail(ctx, PYRE_E_STATE, "pyre_generate_greedy_mtp: this drafter is not attached to the state");
+  const size_t V = m->c.vocab; int produced = 0, rounds = 0, drafted = 0, accepted = 0;
+  uint32_t pending = host_argmax(first_logits, V);
+  for (;;) {
+    out[produced++] = pending; if (produced >= n_out) break;
+    const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
+    uint32_t toks[8]; float ps[8]; toks[0] = pending; int nd = 0;
+    if (kk > 0) { int rc = pyre_mtp_draft(ctx, mtp, s, pending, kk, min_p, toks + 1, ps, &nd); if (rc) return rc; }
+    uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
+    int acc = 0; bool have = false; uint32_t nx = 0;
+    for (int i = 0; i < nd; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
+    if (!have) nx = picks[nd];
+    if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
+    if (nd > 0) ++rounds; drafted += nd; accepted += acc;
+    bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
     if (stop) break;
     pending = nx;
   }

@@ -118,6 +118,12 @@ def _declare(L):
         "pyre_argmax_rows": (i32, [vp, vp, i32, i32, vp]),
         "pyre_generate_greedy_ngram": (i32, [vp, vp, vp, vp, C.c_size_t, vp, i32, vp, i32, i32, i32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
         "pyre_decode_greedy_dev": (i32, [vp, vp, vp, u32, i32, vp]),
+        "pyre_mtp_create": (i32, [vp, vp, vp, vp, vp, C.POINTER(vp)]),
+        "pyre_mtp_destroy": (None, [vp]),
+        "pyre_state_attach_mtp": (i32, [vp, vp, vp]),
+        "pyre_mtp_draft": (i32, [vp, vp, vp, u32, i32, f32, vp, vp, C.POINTER(i32)]),
+        "pyre_mtp_read_kv": (i32, [vp, vp, C.POINTER(i32), C.POINTER(i32), vp, vp]),
+        "pyre_generate_greedy_mtp": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, f32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -690,6 +696,72 @@ class Model:
     def close(self):
         if getattr(self, "h", None) and getattr(self.ctx, "h", None):
             self.ctx.L.pyre_model_destroy(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+MTP_SLOTS = 30
+
+
+class MtpCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_exp", "top_k", "ff", "window", "n_draft_vocab")]
+
+
+class Mtp:
+    """The MTP drafter (src/model/mtp.rs) beside a Model: tensors is a dict slot -> (ty, rows, cols, data) over the
+    PYRE_MTP_* slots, draft_ids the vocabulary ids of the draft head's rows."""
+
+    def __init__(self, model, n_exp, top_k, ff, window, tensors, draft_ids):
+        self.m = model; ctx = model.ctx
+        ids = np.ascontiguousarray(draft_ids, dtype=np.uint32)
+        self.cfg = MtpCfg(n_exp, top_k, ff, window, ids.size)
+        keep = []
+
+        def desc(e):
+            if e is None:
+                return TensorDesc(0, 0, 0, 0, None)
+            ty, rows, cols, data = e
+            if isinstance(data, np.ndarray):
+                data = np.ascontiguousarray(data); keep.append(data)
+                return TensorDesc(ty, 0, rows, cols, data.ctypes.data)
+            return TensorDesc(ty, 1, rows, cols, int(data))
+        ts = (TensorDesc * MTP_SLOTS)(*[desc(tensors.get(s)) for s in range(MTP_SLOTS)])
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_mtp_create(ctx.h, model.h, C.byref(self.cfg), ts, _ptr(ids), C.byref(h)), "mtp_create")
+        self.h = h
+
+    def attach(self, st):
+        self.m.ctx.check(self.m.ctx.L.pyre_state_attach_mtp(self.m.ctx.h, st.h, self.h), "state_attach_mtp")
+
+    def draft(self, st, pending, k, min_p=0.0):
+        """Model::mtp_draft: (ids, probabilities) of up to k drafts after `pending`."""
+        ids = np.zeros(8, dtype=np.uint32); ps = np.zeros(8, dtype=np.float32); n = C.c_int(0)
+        self.m.ctx.check(self.m.ctx.L.pyre_mtp_draft(self.m.ctx.h, self.h, st.h, int(pending), k, min_p, _ptr(ids), _ptr(ps), C.byref(n)), "mtp_draft")
+        return ids[:n.value].copy(), ps[:n.value].copy()
+
+    def kv(self, st):
+        """(first cell, K [n][n_kv*hd], V) of the drafter's cache."""
+        c = self.m.cfg; row = c.n_kv * c.hd
+        k = np.zeros((self.cfg.window + 8, row), dtype=np.float32); v = np.zeros_like(k); c0, n = C.c_int(0), C.c_int(0)
+        self.m.ctx.check(self.m.ctx.L.pyre_mtp_read_kv(self.m.ctx.h, st.h, C.byref(c0), C.byref(n), _ptr(k), _ptr(v)), "mtp_read_kv")
+        return c0.value, k[:n.value].copy(), v[:n.value].copy()
+
+    def generate_greedy(self, st, first_logits, n_out, k=3, min_p=0.0):
+        """spec::generate (greedy) with this drafter; returns (tokens, rounds, drafted, accepted)."""
+        fl = np.ascontiguousarray(first_logits, dtype=np.float32)
+        out = np.empty(n_out, dtype=np.uint32); r, d, a = C.c_int(0), C.c_int(0), C.c_int(0)
+        self.m.ctx.check(self.m.ctx.L.pyre_generate_greedy_mtp(self.m.ctx.h, self.m.h, self.h, st.h, _ptr(fl), n_out, _ptr(out), k, min_p,
+                                                               C.byref(r), C.byref(d), C.byref(a)), "generate_greedy_mtp")
+        return out, r.value, d.value, a.value
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.m, "h", None) and getattr(self.m.ctx, "h", None):
+            self.m.ctx.L.pyre_mtp_destroy(self.h)
         self.h = None
 
     def __del__(self):

@@ -240,3 +240,46 @@ def build_device(ctx, c: Config, seed=1):
             entry = (ty, rows, cols, host_tensor(c, seed, il, slot, kind, ty, rows, cols))
         (layers[il] if il >= 0 else globals_)[slot] = entry
     return layers, globals_, raw
+
+
+# ---- the MTP drafter's tensors (slots of include/pyre_hip.h's PYRE_MTP_* enum; names of src/model/mtp.rs:99-117) -----------
+(MTP_PRE_E, MTP_PRE_H, MTP_FC_E, MTP_FC_H, MTP_HCA_NORM, MTP_HCA_DOWN, MTP_HCA_INJECT, MTP_HCA_UP, MTP_HCF_NORM, MTP_HCF_DOWN,
+ MTP_HCF_INJECT, MTP_HCF_UP, MTP_MIX_NORM, MTP_MIX_DOWN, MTP_MIX_UP, MTP_Q, MTP_K, MTP_V, MTP_O, MTP_QN, MTP_KN, MTP_ROUTER,
+ MTP_GATE_E, MTP_UP_E, MTP_DOWN_E, MTP_SH_GATE_INP, MTP_SH_GATE, MTP_SH_UP, MTP_SH_DOWN, MTP_HEAD, MTP_SLOTS) = range(31)
+
+
+def mtp_specs(c: Config, n_exp, ff, lr=None):
+    """[(slot, kind, ty, rows, cols)] of the drafter's tensors except the head (rows of the main output matrix)."""
+    w = c.hc * c.d; lr = lr or c.hc_lr; sf = c.ff_sh or ff
+    out = [(MTP_PRE_E, "vec:norm1", synth.F32, 1, c.d), (MTP_PRE_H, "vec:norm1", synth.F32, 1, w),
+           (MTP_FC_E, "q", c.qtype, c.d, c.d), (MTP_FC_H, "q", c.qtype, c.d, c.d)]
+    for base, inj in ((MTP_HCA_NORM, True), (MTP_HCF_NORM, True)):
+        out += [(base, "vec:norm1", synth.F32, 1, w), (base + 1, "hc", c.hc_type, lr, w), (base + 2, "hc", c.hc_type, c.hc, w), (base + 3, "hc", c.hc_type, w, lr)]
+    out += [(MTP_MIX_NORM, "vec:norm1", synth.F32, 1, w), (MTP_MIX_DOWN, "hc", c.hc_type, lr, w), (MTP_MIX_UP, "hc", c.hc_type, w, lr)]
+    out += [(MTP_Q, "q", c.qtype, c.n_head * 2 * c.hd, c.d), (MTP_K, "q", c.qtype, c.n_kv * c.hd, c.d), (MTP_V, "q", c.qtype, c.n_kv * c.hd, c.d),
+            (MTP_O, "q", c.qtype, c.d, c.n_head * c.hd), (MTP_QN, "vec:norm1", synth.F32, 1, c.hd), (MTP_KN, "vec:norm1", synth.F32, 1, c.hd),
+            (MTP_ROUTER, "router", c.router_type, n_exp, c.d), (MTP_GATE_E, "q", c.qtype, n_exp * ff, c.d), (MTP_UP_E, "q", c.qtype, n_exp * ff, c.d),
+            (MTP_DOWN_E, "q", c.qtype, n_exp * c.d, ff), (MTP_SH_GATE_INP, "vec:small", synth.F32, 1, c.d), (MTP_SH_GATE, "q", c.qtype, sf, c.d),
+            (MTP_SH_UP, "q", c.qtype, sf, c.d), (MTP_SH_DOWN, "q", c.qtype, c.d, sf)]
+    return out
+
+
+def build_mtp_host(c: Config, hw: HostWeights, n_exp, ff, draft_ids, seed=7, lr=None):
+    """dict slot -> (ty, rows, cols, bytes): synthetic drafter tensors, and as head the rows `draft_ids` of the main
+    model's output matrix in its own type (the reference re-quantizes those rows to int8, mtp.rs:107)."""
+    out = {}
+    for slot, kind, ty, rows, cols in mtp_specs(c, n_exp, ff, lr):
+        il, sl = (0, HCA_DOWN) if kind == "hc" else (0, ATTN_Q)          # scale range of a hyper-connection matrix or of a projection
+        k2 = "q" if kind == "hc" else kind
+        s = tensor_seed(seed, 99, slot)
+        if k2 == "q" and ty not in (synth.F32, synth.F16, synth.BF16):
+            b = synth.matrix(ty, rows, cols, s, *scale_range(c, il, sl, ty))
+        else:
+            b = host_tensor(c, seed, 99, slot, k2, ty, rows, cols)
+        out[slot] = (ty, rows, cols, b)
+    ty, rows, cols, b = hw.globals_[G_OUT]
+    el, bs, _ = synth.GEOM[ty] if ty in synth.GEOM else (1, {synth.F32: 4, synth.F16: 2, synth.BF16: 2}[ty], None)
+    rb = cols // el * bs
+    ids = np.asarray(draft_ids, dtype=np.int64)
+    out[MTP_HEAD] = (ty, ids.size, cols, np.ascontiguousarray(b.reshape(rows, rb)[ids]).reshape(-1))
+    return out

@@ -88,3 +88,9 @@ def np_forward_tokens(hw, ids):
         h, _ = np_ref.hc_mix(d, hc, c.eps, G[mg.G_HEAD_NORM], G[mg.G_HEAD_DOWN], None, G[mg.G_HEAD_UP], x)
         out.append(G[mg.G_OUT] @ h)
     return np.array(out)
+
+
+def orc_mtp(om, mt, n_exp, top_k, ff, window, draft_ids):
+    """The oracle's drafter over a modelgen.build_mtp_host tensor dict."""
+    ts = [orc_tensor(mt[s]) if s in mt else orc.Tensor(0, 0, 0, None) for s in range(mg.MTP_SLOTS)]
+    return orc.Mtp(om, n_exp, top_k, ff, window, ts, draft_ids, keep=(mt,))

@@ -57,6 +57,8 @@ def lib():
         L.orc_rope_inv_yarn.restype = C.c_float
         for n in ("orc_state_conv", "orc_state_ssm", "orc_state_k", "orc_state_v", "orc_state_ik", "orc_state_ib", "orc_state_ple_hist"):
             getattr(L, n).restype = C.POINTER(C.c_float)
+        L.orc_mtp_create.restype = C.c_void_p
+        L.orc_mtp_r.restype = C.POINTER(C.c_float)
         _lib = L
     return _lib
 
@@ -276,6 +278,58 @@ class Model:
     def __del__(self):
         if getattr(self, "h", None):
             lib().orc_model_destroy(self.h)
+            self.h = None
+
+
+MTP_SLOTS = 30
+
+
+class MtpCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_exp", "top_k", "ff", "window", "n_draft_vocab")]
+
+
+class Mtp:
+    """The oracle's MTP drafter beside a Model; tensors: list of MTP_SLOTS orc.Tensor, draft_ids: uint32 ids of the head's rows."""
+
+    def __init__(self, model, n_exp, top_k, ff, window, tensors, draft_ids, keep=()):
+        self.m = model; self._keep = keep
+        self.ids = np.ascontiguousarray(draft_ids, dtype=np.uint32)
+        self.cfg = MtpCfg(n_exp, top_k, ff, window, self.ids.size)
+        self._t = (Tensor * MTP_SLOTS)(*tensors)
+        self.h = C.c_void_p(lib().orc_mtp_create(model.h, C.byref(self.cfg), self._t, _p(self.ids)))
+        assert self.h
+
+    def attach(self, st):
+        lib().orc_state_attach_mtp(st.h, self.h)
+
+    def draft(self, st, pending, k, min_p=0.0):
+        ids = np.zeros(8, dtype=np.uint32); ps = np.zeros(8, dtype=np.float32)
+        n = lib().orc_mtp_draft(self.h, self.m.h, st.h, C.c_uint32(int(pending)), C.c_int(k), C.c_float(min_p), _p(ids), _p(ps))
+        assert n >= 0
+        return ids[:n].copy(), ps[:n].copy()
+
+    def kv(self, st):
+        c = self.m.cfg; row = c.n_kv * c.hd
+        c0 = C.c_int(0); k = C.POINTER(C.c_float)(); v = C.POINTER(C.c_float)()
+        n = lib().orc_mtp_kv(st.h, C.byref(c0), C.byref(k), C.byref(v))
+        if n == 0:
+            return c0.value, np.zeros((0, row), np.float32), np.zeros((0, row), np.float32)
+        return c0.value, np.ctypeslib.as_array(k, shape=(n, row)).copy(), np.ctypeslib.as_array(v, shape=(n, row)).copy()
+
+    def residual(self, st, pos):
+        c = self.m.cfg
+        p = lib().orc_mtp_r(st.h, C.c_int(pos))
+        return np.ctypeslib.as_array(p, shape=(c.hc * c.d,)).copy() if p else None
+
+    def generate_greedy(self, st, first_logits, n_out, k=3, min_p=0.0):
+        out = np.empty(n_out, dtype=np.uint32); fl = f32(first_logits); d, a = C.c_int(0), C.c_int(0)
+        rc = lib().orc_generate_greedy_mtp(self.m.h, self.h, st.h, _p(fl), C.c_int(n_out), _p(out), C.c_int(k), C.c_float(min_p), C.byref(d), C.byref(a))
+        assert rc == 0
+        return out, d.value, a.value
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_mtp_destroy(self.h)
             self.h = None
 
 
