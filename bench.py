@@ -475,7 +475,7 @@ def bench_decode(args):
         ctx.free(p)
     log("model resident (re-laid-out) in %.1f s; weight bytes per token %.1f MB" % (time.perf_counter() - t0, model.weight_bytes_per_token / 1e6))
     n_ctx = args.ctx
-    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8 + args.host_steps + 1 + args.spec_loop_tokens + 16)
+    st = model.new_state(n_ctx + args.steps + args.warmup + 64 + args.spec_windows + 8 + args.host_steps + 1 + args.spec_loop_tokens + 16 + 256)
     g = np.random.Generator(np.random.PCG64(args.seed + 1))
     prompt = g.integers(0, cfg.vocab, n_ctx, dtype=np.uint32)
     t0 = time.perf_counter()
@@ -578,6 +578,35 @@ def bench_decode(args):
                     traffic_source = "profiles/decode_deltanet_slice_hbm_traffic.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE on a three-layer slice of this step, not this run; attention-layer launches of the class are not covered"
         except OSError:
             pass
+    # the MTP drafter beside the model (synthetic weights of the main layers' geometry, draft head of the reference's
+    # default draft vocabulary size): cost of a draft call and of a drafted round.  Random weights draft tokens the model
+    # does not pick, so the acceptance seen here says nothing; tok/s at a given acceptance follows from the two costs.
+    mtp = None
+    if args.mtp_draft > 0:
+        kd = args.mtp_draft
+        mt, mraw = mg.build_mtp_device(ctx, cfg, cfg.n_exp, cfg.ff_exp, args.mtp_vocab, seed=args.seed + 5)
+        dr_ = lib.Mtp(model, cfg.n_exp, cfg.top_k, cfg.ff_exp, 128, mt, np.arange(args.mtp_vocab, dtype=np.uint32) * (cfg.vocab // args.mtp_vocab))
+        for p in mraw:
+            ctx.free(p)
+        snap = st.snapshot()
+        dr_.attach(st)
+        tail = model.decode_greedy_dev(st, nxt, 136)                    # fills the residual ring over a full window
+        pend = int(tail[-1])
+        dr_.draft(st, pend, kd)                                         # untimed: the catch-up over the window's cells
+        ctx.sync(); t0 = time.perf_counter()
+        for i in range(8):
+            dr_.draft(st, pend, kd)
+        d_ms = (time.perf_counter() - t0) * 1e3 / 8
+        fl = np.zeros(cfg.vocab, dtype=np.float32); fl[pend] = 1.0
+        n_g = 33
+        ctx.sync(); t0 = time.perf_counter()
+        out_t, rounds, drafted, accepted = dr_.generate_greedy(st, fl, n_g, k=kd)
+        ctx.sync(); g_dt = time.perf_counter() - t0
+        mtp = {"drafts_per_call": kd, "draft_vocab": args.mtp_vocab, "window": 128, "ms_per_draft_call": round(d_ms, 3), "ms_per_draft_step": round(d_ms / kd, 3),
+               "generate": {"tokens": n_g - 1, "rounds": rounds, "drafted": drafted, "accepted": accepted, "tok_s": round((n_g - 1) / g_dt, 1), "ms_per_round": round(g_dt * 1e3 / max(rounds, 1), 3)},
+               "note": "synthetic drafter: 512 experts top-10 of width 512 like a main layer; a call = catch-up of the newly committed cells + k draft steps + one readback"}
+        dr_.close()
+        st.restore(snap)
     out = {
         "metric": "decode tok/s batch-1 (A3B hybrid IQ3_S)", "value": round(tok_s, 2), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
@@ -602,6 +631,8 @@ def bench_decode(args):
         out["host_loop"] = host_loop
     if spec_loop:
         out["spec_loop"] = spec_loop
+    if mtp:
+        out["mtp_drafter"] = mtp
     if not args.no_cpu:
         del model, st
         out["cpu_baseline"] = cpu_baseline_decode(cfg, args.seed)
@@ -621,6 +652,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--spec-windows", type=int, default=8, help="decode workload: verify windows of 5 tokens to time after the greedy run (0 = skip)")
     ap.add_argument("--spec-loop-tokens", type=int, default=64, help="decode workload: tokens to generate through the drafted loop (4 fixed drafts per round, all accepted / none accepted; 0 = skip)")
+    ap.add_argument("--mtp-draft", type=int, default=3, metavar="K", help="decode workload: also time the MTP drafter (K drafts per call, 1..7; 0 = skip)")
+    ap.add_argument("--mtp-vocab", type=int, default=40525, help="decode workload: rows of the drafter's head (the reference's default draft vocabulary has 40525 ids)")
     ap.add_argument("--host-steps", type=int, default=32, help="decode workload: steps of the host-facing loop (pyre_forward + host argmax) to time beside the device loop (0 = skip)")
     ap.add_argument("--t", type=int, default=1, help="gemv workload: tokens per launch (1..8)")
     ap.add_argument("--fmt", default="iq3_s", help="gemv workload: GGUF block type of the matrix (iq3_s, iq2_xs, q4_k, q8_0, q4_0, q5_0, q6_k, iq2_xxs, iq2_s, iq3_xxs, iq4_nl, iq4_xs, q3_k, q5_k, q2_0)")

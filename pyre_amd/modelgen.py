@@ -283,3 +283,25 @@ def build_mtp_host(c: Config, hw: HostWeights, n_exp, ff, draft_ids, seed=7, lr=
     ids = np.asarray(draft_ids, dtype=np.int64)
     out[MTP_HEAD] = (ty, ids.size, cols, np.ascontiguousarray(b.reshape(rows, rb)[ids]).reshape(-1))
     return out
+
+
+def build_mtp_device(ctx, c: Config, n_exp, ff, n_draft, seed=7, lr=None):
+    """The drafter's tensors with every quantized matrix generated on the device (benchmark sizes).  The head is a
+    synthetic [n_draft][d] matrix of the main output matrix's type, not rows of that matrix: same shape and cost.
+    Returns (tensors, raw_device_buffers)."""
+    out, raw = {}, []
+    specs = mtp_specs(c, n_exp, ff, lr) + [(MTP_HEAD, "q", c.qtype, n_draft, c.d)]
+    for slot, kind, ty, rows, cols in specs:
+        il, sl = (0, HCA_DOWN) if kind == "hc" else (0, ATTN_Q)
+        k2 = "q" if kind == "hc" else kind
+        if k2 == "q" and ty not in (synth.F32, synth.F16, synth.BF16):
+            el, bs, _ = synth.GEOM[ty]
+            nb = rows * (cols // el)
+            dev = ctx.alloc(nb * bs)
+            lo, hi = scale_range(c, il, sl, ty)
+            ctx.synth_blocks(ty, nb, tensor_seed(seed, 99, slot), lo, hi, dev_out=dev)
+            raw.append(dev)
+            out[slot] = (ty, rows, cols, dev)
+        else:
+            out[slot] = (ty, rows, cols, host_tensor(c, seed, 99, slot, k2, ty, rows, cols))
+    return out, raw
