@@ -83,3 +83,28 @@ def test_two_layer_slice_matches_the_oracle_at_full_width(ctx):
     assert np.array_equal(tg, to)
     conv, ssm = gs.gdn(0)
     assert relerr(ssm, os_.ssm(0)) <= 1e-4 and relerr(conv, os_.conv(0)) <= 1e-5
+
+
+def test_drafter_matches_the_oracle_at_full_width(ctx):
+    # the drafter block at the benchmark's width (4 streams of 2048, 512 experts top-10 of width 512, 16 / 2 heads of
+    # 256) over a two-layer model; a 4096-row draft head
+    import helpers
+    cfg = mg.a3b_config(n_layers=2, full_every=2)
+    hw = mg.build_host(cfg, seed=8)
+    ids = (np.arange(4096, dtype=np.uint32) * 37) % cfg.vocab
+    mt = mg.build_mtp_host(cfg, hw, 512, 512, ids, seed=18)
+    gm = lib.Model(ctx, cfg, hw.layers, hw.globals_); om = orc_model(hw, threads=min(os.cpu_count() or 1, 16))
+    gd = lib.Mtp(gm, 512, 10, 512, 128, mt, ids); od = helpers.orc_mtp(om, mt, 512, 10, 512, 128, ids)
+    g = np.random.Generator(np.random.PCG64(19))
+    prompt = g.integers(0, cfg.vocab, 11, dtype=np.uint32)
+    gs, os_ = gm.new_state(64), om.new_state(); gd.attach(gs); od.attach(os_)
+    lg, lo = gm.forward(prompt, gs), om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-3
+    pending = int(orc.argmax(lo))
+    gi, gp = gd.draft(gs, pending, 3); oi, op = od.draft(os_, pending, 3)
+    assert list(gi) == list(oi) and np.allclose(gp, op, rtol=2e-3, atol=0)
+    gc0, gk, gv = gd.kv(gs); oc0, ok, ov = od.kv(os_)
+    assert (gc0, len(gk)) == (oc0, len(ok)) == (0, 11) and relerr(gk, ok) <= 1e-5 and relerr(gv, ov) <= 1e-5
+    out, rounds, drafted, accepted = gd.generate_greedy(gs, lg, 9, k=3)
+    oo, od_n, oa_n = od.generate_greedy(os_, lo, 9, k=3)
+    assert np.array_equal(out, oo) and (drafted, accepted) == (od_n, oa_n)
