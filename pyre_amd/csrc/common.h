@@ -251,7 +251,8 @@ int pyre_ple_launch(pyre_ctx* ctx, const PleCfg& c, const PleDev& p, const PleWo
                     const float* comb_out, const MoeOut* comb_moe, const float* comb_inj, int start, const int* posp, int t);
 
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
-struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject; };   // di = [down ; inject] rows
+struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject;      // di = [down ; inject] rows
+               QMatDev di_m{}, up_m{}; };      // the same two matrices in the matrix-core layout (fmt == FMT_IQ3_S_M) when they are IQ3_S of whole super-blocks
 struct HcWork { float* ssq; float* o; };    // [<=32][8] slice sums of squares of the streams, [<=32][8][tiles*64] slice sums of [down ; inject]
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);

@@ -5,7 +5,7 @@
 // GEMV (K cut into slices, one slice per workgroup) and leaves each slice's sum of squares; k_hc_up_mix turns those
 // into the streams' RMS scales, adds the scaled slice sums, applies silu, runs the up GEMV from shared memory and
 // reduces the gated, normalized streams to their mean.
-#include "formats.h"
+#include "gemm_m.h"
 #include <stdlib.h>
 #include <algorithm>
 
@@ -246,6 +246,235 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
   PYRE_TS(7); PYRE_TS_FLUSH(hc_ts, ROUTE ? 16 : 24);
 }
 
+// ---- the same two launches with both GEMVs on the f16 matrix cores -------------------------------------------------------
+// For [down ; inject] and up held in the IQ3_S matrix-core layout (QMatDev::mq / mh).  The lane = row kernels above pay
+// one multiply-add per weight and token on top of the decode; here a weight costs the same whatever the window width,
+// and a token's sums do not depend on the width either (its two operand rows are its own), so a window still equals
+// single steps bit for bit.  The operand rows are formed inside the kernels, in shared memory: x = h1 + h2 * 2^-11 after
+// a power-of-two scaling per token and slice (k_act_split's rule).
+__device__ __forceinline__ void hc_scale_of(float m, float* up, float* dn) {      // m * 2^e in [2^13, 2^14); zero and non-finite maxima leave e = 0
+  int e = 0;
+  if (m > 0.0f && m < INFINITY) { e = 140 - (int)((__float_as_uint(m) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+  *up = __uint_as_float((uint32_t)(127 + e) << 23); *dn = __uint_as_float((uint32_t)(127 - e) << 23);
+}
+__device__ __forceinline__ void hc_split_store(uint16_t* ah, int k, int t, float xs) {      // operand rows 2t, 2t+1 of column k: [8-column group][16 rows][8]
+  const _Float16 h1 = (_Float16)xs, h2 = (_Float16)((xs - (float)h1) * 2048.0f);
+  uint16_t* o = ah + ((size_t)(k >> 3) * 16 + 2 * t) * 8 + (k & 7);
+  o[0] = __builtin_bit_cast(unsigned short, h1); o[8] = __builtin_bit_cast(unsigned short, h2);
+}
+__device__ __forceinline__ void hc_lds_a(const uint16_t* ah, int c, int lane, ABuf& b) {      // chunk c (128 columns) of the operand in shared memory
+#pragma unroll
+  for (int s = 0; s < 4; ++s) b.a[s] = ((const uint4*)ah)[((c * 4 + s) * 4 + (lane >> 4)) * 16 + (lane & 15)];
+}
+
+// grid (row tiles of [down ; inject], slices of 256*CS columns), 4*CS waves, a thread prepares one column of the slice.
+// Wave (p, g) takes row group g of the tile over chunk pair p of the slice; with CS = 2 the two pairs' sums meet in
+// shared memory (pair 0 + pair 1).  Outputs as k_hc_norm_down: ssq[ks*T + t], part[(ks*T + t)*tiles*64 + row], x_out.
+template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_hc_norm_down_m(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
+    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part) {
+  constexpr int NW = 4 * CS;
+  __shared__ __align__(16) uint16_t ah[CS * 32 * 16 * 8];
+  __shared__ float wsum[NW][8], wmax[NW][8], hsum[4][2][64];
+  qmat_args_now(m); args_now(x_in, in_ss, in_ts, x_out, comb_out, mo.partial, mo.sel_w, mo.sg, mo.d, mo.k, comb_inj, norm, d, hc, ssq, part);
+  const int tile = blockIdx.x, ks = blockIdx.y, tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = wave & 3, p = wave >> 2;
+  const int c0 = ks * 256 * CS, s = c0 / d, i0 = c0 - s * d, K128 = m.cols >> 7;
+  float w[T], v[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f;
+  const float nv = norm[(size_t)s * d + i0 + tid];
+#pragma unroll
+  for (int t = 0; t < T; ++t) v[t] = hc_x_new<T, NP>(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid);
+  const int ch0 = ks * 2 * CS + 2 * p;
+  WBuf<1> w0, w1; load_w<1>(m, tile * 4 + g, ch0, lane, K128, w0); load_w<1>(m, tile * 4 + g, ch0 + 1, lane, K128, w1);
+  const NibK nk = nib_consts();
+  float xs[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    float ss = v[t] * v[t]; xs[t] = v[t] * nv;
+    if (tile == 0) x_out[((size_t)t * hc + s) * d + i0 + tid] = v[t];
+    float a = fabsf(xs[t]); a = a == a ? a : INFINITY;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { ss += __shfl_xor(ss, o); a = fmaxf(a, __shfl_xor(a, o)); }
+    if (lane == 0) { wsum[wave][t] = ss; wmax[wave][t] = a; }
+  }
+#pragma unroll
+  for (int r = 2 * T; r < 16; ++r) ah[((size_t)(tid >> 3) * 16 + r) * 8 + (tid & 7)] = 0;      // rows no token of the window owns
+  lds_barrier();
+  auto slice_max = [&](int t) { float mx = wmax[0][t];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) mx = fmaxf(mx, wmax[k][t]);
+    return mx; };
+  if (tile == 0 && tid < T) { float tot = wsum[0][tid];
+#pragma unroll
+    for (int k = 1; k < NW; ++k) tot += wsum[k][tid];
+    ssq[ks * T + tid] = tot; }
+#pragma unroll
+  for (int t = 0; t < T; ++t) { float up, dn; hc_scale_of(slice_max(t), &up, &dn); hc_split_store(ah, tid, t, xs[t] * up); }
+  lds_barrier();
+  const int q = lane >> 4;
+  float upf, dn0 = 0.0f, dn1 = 0.0f;
+  if (2 * q < T) hc_scale_of(slice_max(2 * q), &upf, &dn0);
+  if (2 * q + 1 < T) hc_scale_of(slice_max(2 * q + 1), &upf, &dn1);
+  v4f tot[1] = {v4f{0.0f, 0.0f, 0.0f, 0.0f}};
+  { ABuf a0, a1; hc_lds_a(ah, 2 * p, lane, a0); hc_lds_a(ah, 2 * p + 1, lane, a1); a0.ai0 = dn0; a0.ai1 = dn1; a1.ai0 = dn0; a1.ai1 = dn1;
+    chunk_mac<1>(w0, a0, ch0, nk, tot); chunk_mac<1>(w1, a1, ch0 + 1, nk, tot); }
+  float r0 = tot[0][0] + tot[0][1] * (1.0f / 2048.0f), r1 = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
+  if constexpr (CS == 2) {
+    if (p == 1) { hsum[g][0][lane] = r0; hsum[g][1][lane] = r1; }
+    lds_barrier();
+    if (p == 1) return;
+    r0 += hsum[g][0][lane]; r1 += hsum[g][1][lane];
+  }
+  const size_t r64 = (size_t)m.tiles * 64, row = (size_t)tile * 64 + g * 16 + (lane & 15);
+  if (2 * q < T) part[((size_t)ks * T + 2 * q) * r64 + row] = r0;
+  if (2 * q + 1 < T) part[((size_t)ks * T + 2 * q + 1) * r64 + row] = r1;
+}
+
+__device__ __forceinline__ void hc_load_run16(float (&sv)[16], const float* __restrict__ p, int n, int stride) {      // n (<= 16) values at p, p + stride, ..
+#pragma unroll
+  for (int k = 0; k < 16; ++k) sv[k] = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) if (g * 4 < n) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sv[g * 4 + j] = p[(size_t)min(g * 4 + j, n - 1) * stride];
+  }
+}
+// up to sixteen slice sums of one output row, all loads in flight together (as hc_load_slices)
+template <int T> __device__ __forceinline__ void hc_load_slices16(float (&pv)[16], const float* __restrict__ part, bool want, int ksplit, int t, int r64, int i) {
+#pragma unroll
+  for (int ks = 0; ks < 16; ++ks) pv[ks] = 0.0f;
+  const unsigned off = (unsigned)(t * r64 + i);
+  if (want) {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) if (g * 8 < ksplit) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pv[g * 8 + j] = (part + (size_t)min(g * 8 + j, ksplit - 1) * T * r64)[off];
+    }
+  }
+}
+__device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const float* sls_t, int ksplit) {      // slices in order, each times its stream's scale
+  float o = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < 16; ++ks) if (ks < ksplit) { const float tm = pv[ks] * sls_t[ks]; o = ks == 0 ? tm : o + tm; }
+  return o;
+}
+
+// grid (d / 64), hc*4 waves: wave (s, g) takes row group g of row tile s*(d/64) + blockIdx.x of `up` over all lr columns
+// (at most sixteen slices).  Prologue, epilogue and the riding router GEMV as k_hc_up_mix, except that every load the
+// prologue and the epilogue need is issued at the start (two rows of lo and one inject row a thread, two (token, stream)
+// items a wave), and lo goes through shared memory twice: f32, then as operand rows scaled per token by the power of two
+// of its largest magnitude.
+template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
+    const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows) {
+  constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
+  const uint2* lds2 = nullptr;
+  qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj);
+  extern __shared__ __align__(16) float sm[];
+  const int nthr = blockDim.x, tid = threadIdx.x, kps = ksplit / hc, nw = nthr >> 6;
+  float* lo = sm;                                 // [T][lr]
+  float* red = lo + (size_t)T * lr;               // [hc][T][64]: the gate logits
+  float* sls = red + (size_t)hc * T * 64;         // [T][16]
+  float* term = sls + (size_t)T * 16;             // [T*hc][64]
+  uint32_t* lmax = (uint32_t*)(term + (size_t)T * hc * 64);      // [8]: bits of the largest |lo| of each token
+  uint16_t* ah = (uint16_t*)(lmax + 8);           // [lr/8][16][8]
+  const int K128 = lr >> 7, n_lo = T * lr;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int s = wave >> 2, g = wave & 3, q = lane >> 4;
+  float ssv[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) ssv[k] = 0.0f;
+  const int stt = tid / hc, sq = tid - stt * hc;
+  const bool own_stream = tid < T * hc;                      // thread (token stt, stream sq): the stream's scale, and the stream's inject row
+  if (own_stream) hc_load_run16(ssv, ssq + (size_t)(sq * kps) * T + stt, kps, T);
+  float pva[16], pvb[16], pvi[16];
+  const int ia = tid, ib = tid + nthr;
+  const int ta = ia / lr, ra = ia - ta * lr, tb = ib / lr, rb = ib - tb * lr;
+  hc_load_slices16<T>(pva, part, ia < n_lo, ksplit, ta, r64, ra);
+  hc_load_slices16<T>(pvb, part, ib < n_lo, ksplit, tb, r64, rb);
+  hc_load_slices16<T>(pvi, part, own_stream && has_inject, ksplit, stt, r64, lr + sq);
+  const int rg = (s * (d >> 6) + blockIdx.x) * 4 + g;
+  WBuf<1> w0, w1; load_w<1>(up, rg, 0, lane, K128, w0); load_w<1>(up, rg, 1, lane, K128, w1);
+  const NibK nk = nib_consts();
+  // the epilogue's stream value and norm weight of this wave's (token, stream) items: wave, wave + nw
+  float xpre[2] = {0.0f, 0.0f}, npre[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 2; ++j) { const int w = wave + j * nw; if (w < T * hc) { const int t0 = w / hc, q0 = w - t0 * hc; xpre[j] = (xnew + ((size_t)t0 * hc + q0) * d + blockIdx.x * 64)[lane]; npre[j] = (norm + (size_t)q0 * d + blockIdx.x * 64)[lane]; } }
+  UnitRaw<RFX> rraw;
+  constexpr bool R_EARLY = RFX != FMT_F32;      // an f32 tile is 64 registers: fetched once the up GEMV has freed them; others once the slice sums are used up
+  if (tid < 8) lmax[tid] = 0u;
+  for (int j = tid; j < (16 - 2 * T) * lr; j += nthr) { const int r = 2 * T + j / lr, k = j - (r - 2 * T) * lr; ah[((size_t)(k >> 3) * 16 + r) * 8 + (k & 7)] = 0; }
+  if (own_stream) {
+    float tot = ssv[0];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) if (k < kps) tot += ssv[k];
+    const float sc = 1.0f / sqrtf(tot / (float)d + eps);
+    for (int k = 0; k < kps; ++k) sls[stt * 16 + sq * kps + k] = sc;
+  }
+  lds_barrier();
+  auto put_lo = [&](int t, int i, const float (&pv)[16]) {
+    const float v = hc_slice_sum16(pv, sls + t * 16, ksplit) / (float)hc, lv = v * sigm(v);
+    lo[t * lr + i] = lv; float a = fabsf(lv); a = a == a ? a : INFINITY; atomicMax(&lmax[t], __float_as_uint(a)); };
+  if (ia < n_lo) put_lo(ta, ra, pva);
+  if (ib < n_lo) put_lo(tb, rb, pvb);
+  for (int idx = tid + 2 * nthr; idx < n_lo; idx += nthr) { const int t = idx / lr, i = idx - t * lr; hc_load_slices16<T>(pva, part, true, ksplit, t, r64, i); put_lo(t, i, pva); }
+  if (own_stream && blockIdx.x == 0) inj[stt * hc + sq] = has_inject ? hc_slice_sum16(pvi, sls + stt * 16, ksplit) / (float)hc : 0.0f;
+  if (ROUTE && R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
+  lds_barrier();
+  for (int j = tid; j < n_lo; j += nthr) {
+    const int t2 = j / lr, k = j - t2 * lr; float upf, dn; hc_scale_of(__uint_as_float(lmax[t2]), &upf, &dn);
+    hc_split_store(ah, k, t2, lo[j] * upf);
+  }
+  lds_barrier();
+  v4f tot[1] = {v4f{0.0f, 0.0f, 0.0f, 0.0f}};
+  { float upf, dn0 = 0.0f, dn1 = 0.0f;
+    if (2 * q < T) hc_scale_of(__uint_as_float(lmax[2 * q]), &upf, &dn0);
+    if (2 * q + 1 < T) hc_scale_of(__uint_as_float(lmax[2 * q + 1]), &upf, &dn1);
+    for (int c = 0; c < K128; c += 2) {
+      if (c > 0) { load_w<1>(up, rg, c, lane, K128, w0); load_w<1>(up, rg, c + 1, lane, K128, w1); }
+      ABuf a0, a1; hc_lds_a(ah, c, lane, a0); hc_lds_a(ah, c + 1, lane, a1);
+      a0.ai0 = dn0; a0.ai1 = dn1; a1.ai0 = dn0; a1.ai1 = dn1;
+      chunk_mac<1>(w0, a0, c, nk, tot); chunk_mac<1>(w1, a1, c + 1, nk, tot);
+    } }
+  if (2 * q < T) red[((size_t)s * T + 2 * q) * 64 + g * 16 + (lane & 15)] = tot[0][0] + tot[0][1] * (1.0f / 2048.0f);
+  if (2 * q + 1 < T) red[((size_t)s * T + 2 * q + 1) * 64 + g * 16 + (lane & 15)] = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
+  if (ROUTE && !R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {          // one wave per (token, stream): xn * sigm(gate) -> term
+    const int w = wave + j * nw;
+    if (w < T * hc) {
+      const int t2 = w / hc, qs = w - t2 * hc;
+      const float gl = red[((size_t)qs * T + t2) * 64 + lane];
+      term[(size_t)w * 64 + lane] = xpre[j] * sls[t2 * 16 + qs * kps] * npre[j] * sigm(gl);            // rms: (x * s) * w
+    }
+  }
+  lds_barrier();
+  for (int i2 = tid; i2 < T * 64; i2 += nthr) {
+    const int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
+#pragma unroll
+    for (int qs = 0; qs < 8; ++qs) if (qs < hc) mx += term[(size_t)(t2 * hc + qs) * 64 + l];
+    const float mv = mx / (float)hc;
+    mixed[(size_t)t2 * d + col] = mv;
+    if (aop) aop_store(aop, aop_rows, col, t2, mv);
+    if (ROUTE) lo[t2 * 64 + l] = mv;
+  }
+  if (ROUTE) {
+    lds_barrier();
+    const size_t rr64 = (size_t)router.tiles * 64;
+    for (int tile = wave; tile < router.tiles; tile += nw) {
+      if (tile != wave) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
+#pragma unroll 1
+      for (int t2 = 0; t2 < T; ++t2) {
+        float ra[1] = {0.0f};
+        unit_fma<RFX, 1>(router, rraw, blockIdx.x, lds2, lane, lo + t2 * 64, 0, ra);
+        rpart[((size_t)blockIdx.x * T + t2) * rr64 + (size_t)tile * 64 + lane] = ra[0];
+      }
+    }
+  }
+}
+
 __global__ void k_hc_combine(float* __restrict__ x, const float* __restrict__ out, const float* __restrict__ inj, int d, int hc) {
   int i = blockIdx.x * blockDim.x + threadIdx.x, s = blockIdx.y, ti = blockIdx.z; if (i >= d) return;
   float w = 2.0f * sigm(inj[ti * hc + s]);
@@ -284,6 +513,40 @@ template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const
   } else UP_MIX_GO(-1);
 #undef UP_MIX_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+int hc_m_cs(const HcDev& h) { return h.d % 512 == 0 ? 2 : 1; }      // columns a thread of k_hc_norm_down_m prepares
+int hc_m_slices(const HcDev& h) { return h.hc * h.d / (256 * hc_m_cs(h)); }
+bool hc_on_matrix_cores(const HcDev& h) {
+  static const bool off = [] { const char* e = getenv("PYRE_HC_ROWS"); return e && *e && atoi(e) != 0; }();      // 1: the lane = row kernels for every window width
+  return !off && h.di_m.fmt == FMT_IQ3_S_M && h.up_m.fmt == FMT_IQ3_S_M && h.d % 256 == 0 && hc_m_slices(h) <= 16 && h.lr % 256 == 0 && h.hc * 4 <= 16 && h.di_m.tiles == h.di.tiles;
+}
+template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
+  ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
+#define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o)
+  if (hc_m_cs(h) == 2) { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 2); else NORM_DOWN_M_GO(1, 2); }
+  else { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 1); else NORM_DOWN_M_GO(1, 1); }
+#undef NORM_DOWN_M_GO
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
+  const int nw = h.hc * 4; const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + (size_t)T * h.hc * 64 + 8) + (size_t)h.lr * 32;
+  const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
+  ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
+               (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
+#define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
+                     h.d, mixed, inj, rq, rp, aop, pyre_aop_rows(T))
+  if (rt && rq.fmt == FMT_BF16) UP_MIX_M_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_GO(FMT_F32); else UP_MIX_M_GO(-1);
+#undef UP_MIX_M_GO
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+}
+#define HC_M_T_SWITCH(FN, ...) \
+  switch (t) { case 1: return FN<1>(__VA_ARGS__); case 2: return FN<2>(__VA_ARGS__); case 3: return FN<3>(__VA_ARGS__); case 4: return FN<4>(__VA_ARGS__); \
+    case 5: return FN<5>(__VA_ARGS__); case 6: return FN<6>(__VA_ARGS__); case 7: return FN<7>(__VA_ARGS__); default: return FN<8>(__VA_ARGS__); }
+int norm_down_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
+  HC_M_T_SWITCH(norm_down_m_launch, ctx, h, w, x_in, in_ss, in_ts, x_out, comb_out, comb_parts, mo, comb_inj)
+}
+int up_mix_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
+  HC_M_T_SWITCH(up_mix_m_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt, aop)
 }
 #define HC_T_SWITCH(F, FN, ...) \
   switch (t) { case 1: return FN<F, 1>(__VA_ARGS__); case 2: return FN<F, 2>(__VA_ARGS__); case 3: return FN<F, 3>(__VA_ARGS__); case 4: return FN<F, 4>(__VA_ARGS__); \
@@ -326,8 +589,13 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: needs d and the low rank in multiples of 64 and hc * (low rank / 64) <= 16 (d %d, low rank %d, hc %d)", h.d, h.lr, h.hc);
   DownPlan p = down_plan(h);
   if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
+  const bool on_m = hc_on_matrix_cores(h);
   MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
   if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);
+  if (on_m) {
+    int rc = norm_down_m(ctx, h, w, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj); if (rc) return rc;
+    return up_mix_m(ctx, h, w, hc_m_slices(h), t, x_out, eps, mixed, inj, route, aop);
+  }
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj, eps); if (rc) return rc;
   return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route, aop);
 }

@@ -67,7 +67,7 @@ struct Builder {
   // one matrix out of `n` row-concatenated tensors of one type and width
   // layout: PYRE_LAYOUT_M for the matrices that only ever meet a GEMV or a row look-up (projections, head, embedding),
   // PYRE_LAYOUT_ROWS for those the hyper-connection and MoE kernels walk themselves
-  int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS) {
+  int cat(const pyre_tensor* const* ts, int n, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS, QMatDev* out_m = nullptr) {
     uint32_t ty = ts[0]->ggml_type; uint64_t cols = ts[0]->cols; uint32_t dev = ts[0]->on_device; uint64_t rows = 0; size_t total = 0;
     int fmt = fmt_from_ggml(ty); if (fmt < 0) return fail(PYRE_E_TYPE, "unsupported tensor type");
     struct { int el, bytes; } g{1, 4}; ggml_geom(ty, &g.el, &g.bytes);
@@ -87,9 +87,9 @@ struct Builder {
       rc = pyre_qmat_create_layout(ctx, ty, rows, cols, tmp, true, total, layout, &q); (void)hipFree(tmp);
     }
     if (rc) return rc;
-    m->owned.push_back(q); *out = q->dv; if (gguf_bytes) *gguf_bytes += total; return PYRE_OK;
+    m->owned.push_back(q); *out = q->dv; if (out_m) *out_m = q->dvm; if (gguf_bytes) *gguf_bytes += total; return PYRE_OK;
   }
-  int one(const pyre_tensor& t, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS) { const pyre_tensor* p = &t; return cat(&p, 1, out, gguf_bytes, layout); }
+  int one(const pyre_tensor& t, QMatDev* out, size_t* gguf_bytes, int layout = PYRE_LAYOUT_ROWS, QMatDev* out_m = nullptr) { const pyre_tensor* p = &t; return cat(&p, 1, out, gguf_bytes, layout, out_m); }
 
   // Gguf::vec: a small tensor fully dequantized to f32 on the device
   int vec(const pyre_tensor& t, size_t expect, const float** out) {
@@ -109,8 +109,9 @@ struct Builder {
     const pyre_model_cfg& c = m->c; size_t w = (size_t)c.hc * c.d;
     if (down.rows != (uint64_t)c.hc_lr || down.cols != w || up.rows != w || up.cols != (uint64_t)c.hc_lr) return fail(PYRE_E_SHAPE, "hyper-connection matrix shapes");
     if (inject && (inject->rows != (uint64_t)c.hc || inject->cols != w)) return fail(PYRE_E_SHAPE, "hyper-connection inject shape");
-    const pyre_tensor* grp[2] = {&down, inject}; int rc = cat(grp, inject ? 2 : 1, &h->di, bytes); if (rc) return rc;
-    rc = one(up, &h->up, bytes); if (rc) return rc;
+    // both layouts: the mixes run on the matrix cores when both matrices are IQ3_S of whole super-blocks, and the lane = row kernels stay available (PYRE_HC_ROWS)
+    const pyre_tensor* grp[2] = {&down, inject}; int rc = cat(grp, inject ? 2 : 1, &h->di, bytes, PYRE_LAYOUT_BOTH, &h->di_m); if (rc) return rc;
+    rc = one(up, &h->up, bytes, PYRE_LAYOUT_BOTH, &h->up_m); if (rc) return rc;
     rc = vec(norm, w, &h->norm); if (rc) return rc;
     h->d = c.d; h->hc = c.hc; h->lr = c.hc_lr; h->has_inject = inject != nullptr; return PYRE_OK;
   }
