@@ -25,76 +25,76 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj
   for (int k = 0; k < kk - 1; ++k) conv_out[(size_t)k * ch + c] = hist[k];
 }
 
-// grid nv, 512 threads.  Thread (grp = tid/128, j = tid%128) keeps rows 32*grp..32*grp+31 of column j of the head's
-// 128x128 state in registers across the whole token window, so the state is read once and written once per launch.
+// grid nv, 512 threads (8 waves), at most 8 tokens.  Thread (grp = tid/128, j = tid%128) keeps rows 32*grp..32*grp+31 of
+// column j of the head's 128x128 state in registers across the whole window, so the state is read once and written once
+// per launch.  Whatever does not depend on the state is done per token by one wave each, before the recurrence (wave ti
+// fetches token ti's q, k, v, z and gate inputs -- eight requests a lane, all tokens in flight together -- and leaves
+// the L2-normalised q and k, v, z, the decay and beta in shared memory) and after it (wave ti: RMSNorm and gate of token
+// ti's output).  A token of the recurrence itself costs one barrier:
+//   S *= g; mem = S^T k -> barrier -> delta = (v - mem) beta; S += k (x) delta; o = S^T q      (linear_core, :1655-1668)
 template <int DK, int DV>
 __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
                                                    const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out, uint16_t* __restrict__ aop, int aop_rows) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
-  constexpr int G = 4, R = DK / G;
+  constexpr int G = 4, R = DK / G, MT = 8;
   PYRE_TS_VARS PYRE_TS(0);
   args_now(p.a, p.dt, p.norm_w, p.nk, p.nv, p.eps, proj, stride, t, co_all, ssm_in, ssm_out, out);
-  __shared__ float qs[DK], ks[DK], pm[G][DV], po[G][DV], red[8];
-  const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7;
+  __shared__ float qs[MT][DK], ks[MT][DK], vs[MT][DV], zs[MT][DV], pm[2][G][DV], po[MT][G][DV], gs[MT], bs[MT];
+  const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ch = 2 * p.nk * DK + p.nv * DV, w = p.nv * DV;
   const float* sin_ = ssm_in + (size_t)h * DK * DV; float* sout = ssm_out + (size_t)h * DK * DV;
+  float q0 = 0.0f, q1 = 0.0f, k0 = 0.0f, k1 = 0.0f, v0 = 0.0f, v1 = 0.0f, z0 = 0.0f, z1 = 0.0f, alpha_raw = 0.0f, beta_raw = 0.0f;
+  if (wave < t) {
+    const float* co = co_all + (size_t)wave * ch; const float* pr = proj + (size_t)wave * stride;
+    q0 = co[kh * DK + lane]; q1 = co[kh * DK + lane + 64]; k0 = co[p.nk * DK + kh * DK + lane]; k1 = co[p.nk * DK + kh * DK + lane + 64];
+    v0 = co[2 * p.nk * DK + h * DV + lane]; v1 = co[2 * p.nk * DK + h * DV + lane + 64];
+    z0 = pr[ch + h * DV + lane]; z1 = pr[ch + h * DV + lane + 64];                      // z at [ch + h*dv + j]
+    alpha_raw = pr[ch + w + p.nv + h]; beta_raw = pr[ch + w + h];                        // alpha at [ch + nv*dv + nv + h], beta at [ch + nv*dv + h]
+  }
+  const float a = p.a[h], dtb = p.dt[h], nw0 = p.norm_w[lane], nw1 = p.norm_w[lane + 64];
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) S[r] = sin_[(size_t)(grp * R + r) * DV + j];
-  const float a = p.a[h], dtb = p.dt[h];
-  for (int ti = 0; ti < t; ++ti) {
-    const float* co = co_all + (size_t)ti * ch;
-    const float* pr = proj + (size_t)ti * stride;
-    // L2 norms of q (threads 0..127) and k (threads 128..255) of key head kh (:1649-1651)
-    float v = 0.0f;
-    if (tid < DK) v = co[kh * DK + tid]; else if (tid < 2 * DK) v = co[p.nk * DK + kh * DK + (tid - DK)];
-    // everything else this token needs from memory is fetched now, ahead of the barriers
-    const float alpha_raw = pr[ch + w + p.nv + h], beta_raw = pr[ch + w + h], v_j = co[2 * p.nk * DK + h * DV + j];
-    const float z_j = tid < DV ? pr[ch + h * DV + j] : 0.0f, nw_j = tid < DV ? p.norm_w[j] : 0.0f;
-    float sq = v * v;
+  auto wsum = [](float x) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
-    if ((tid & 63) == 0) red[tid >> 6] = sq;
-    __syncthreads(); PYRE_TS(1);
-    if (tid < DK) qs[tid] = v * ((1.0f / sqrtf(red[0] + red[1] + 1e-6f)) * (1.0f / sqrtf((float)DK)));
-    else if (tid < 2 * DK) ks[tid - DK] = v * ((1.0f / sqrtf(red[2] + red[3] + 1e-6f)) * 1.0f);
-    const float g = expf(g_softplus(alpha_raw + dtb) * a);      // alpha at [ch + nv*dv + nv + h]
-    const float b = g_sigm(beta_raw);                                 // beta  at [ch + nv*dv + h]
-    __syncthreads(); PYRE_TS(2);
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x; };
+  if (wave < t) {          // L2 norms of q and k (:1649-1651): the sum of each half of the vector, then the two halves
+    const float sq = wsum(q0 * q0) + wsum(q1 * q1), sk = wsum(k0 * k0) + wsum(k1 * k1);
+    const float fq = (1.0f / sqrtf(sq + 1e-6f)) * (1.0f / sqrtf((float)DK)), fk = (1.0f / sqrtf(sk + 1e-6f)) * 1.0f;
+    qs[wave][lane] = q0 * fq; qs[wave][lane + 64] = q1 * fq; ks[wave][lane] = k0 * fk; ks[wave][lane + 64] = k1 * fk;
+    vs[wave][lane] = v0; vs[wave][lane + 64] = v1; zs[wave][lane] = z0; zs[wave][lane + 64] = z1;
+    if (lane == 0) { gs[wave] = expf(g_softplus(alpha_raw + dtb) * a); bs[wave] = g_sigm(beta_raw); }
+  }
+  lds_barrier(); PYRE_TS(1);
+  for (int ti = 0; ti < t; ++ti) {
+    const float g = gs[ti], b = bs[ti];
     float pmv = 0.0f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[grp * R + r]; }
-    pm[grp][j] = pmv;
-    PYRE_TS(3);
-    __syncthreads(); PYRE_TS(4);
-    const float mem = ((pm[0][j] + pm[1][j]) + pm[2][j]) + pm[3][j];
-    const float delta = (v_j - mem) * b;
+    for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[ti][grp * R + r]; }
+    pm[ti & 1][grp][j] = pmv;
+    lds_barrier();
+    const float mem = ((pm[ti & 1][0][j] + pm[ti & 1][1][j]) + pm[ti & 1][2][j]) + pm[ti & 1][3][j];
+    const float delta = (vs[ti][j] - mem) * b;
     float pov = 0.0f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) { S[r] += ks[grp * R + r] * delta; pov += S[r] * qs[grp * R + r]; }
-    po[grp][j] = pov;
-    __syncthreads(); PYRE_TS(5);
-    if (tid < DV) {
-      float o = ((po[0][j] + po[1][j]) + po[2][j]) + po[3][j];
-      float ss = o * o;
-#pragma unroll
-      for (int d = 32; d > 0; d >>= 1) ss += __shfl_xor(ss, d);
-      if ((tid & 63) == 0) red[4 + (tid >> 6)] = ss;
-      pm[0][j] = o;                       // pm is free again: keep o across the barrier below
-    }
-    __syncthreads();
-    if (tid < DV) {
-      float sc = 1.0f / sqrtf((red[4] + red[5]) / (float)DV + p.eps);
-      float o = pm[0][j] * (sc * nw_j);                              // rms_inplace: x *= s * w  (:210)
-      const float ov = o * g_sigm(z_j);                             // z at [ch + h*dv + j]
-      out[(size_t)ti * w + h * DV + j] = ov;
-      if (aop) aop_store(aop, aop_rows, h * DV + j, ti, ov);        // the f16 operand of the output projection (matrix-core layout)
-    }
-    __syncthreads(); PYRE_TS(6);
+    for (int r = 0; r < R; ++r) { S[r] += ks[ti][grp * R + r] * delta; pov += S[r] * qs[ti][grp * R + r]; }
+    po[ti][grp][j] = pov;
   }
+  PYRE_TS(2);
 #pragma unroll
   for (int r = 0; r < R; ++r) sout[(size_t)(grp * R + r) * DV + j] = S[r];
-  PYRE_TS(7); PYRE_TS_FLUSH(gdn_ts, 0);
+  lds_barrier(); PYRE_TS(3);
+  if (wave < t) {
+    const float o0 = ((po[wave][0][lane] + po[wave][1][lane]) + po[wave][2][lane]) + po[wave][3][lane];
+    const float o1 = ((po[wave][0][lane + 64] + po[wave][1][lane + 64]) + po[wave][2][lane + 64]) + po[wave][3][lane + 64];
+    const float sc = 1.0f / sqrtf((wsum(o0 * o0) + wsum(o1 * o1)) / (float)DV + p.eps);
+    const float r0 = (o0 * (sc * nw0)) * g_sigm(zs[wave][lane]), r1 = (o1 * (sc * nw1)) * g_sigm(zs[wave][lane + 64]);      // rms_inplace: x *= s * w  (:210)
+    out[(size_t)wave * w + h * DV + lane] = r0; out[(size_t)wave * w + h * DV + lane + 64] = r1;
+    if (aop) { aop_store(aop, aop_rows, h * DV + lane, wave, r0); aop_store(aop, aop_rows, h * DV + lane + 64, wave, r1); }      // the f16 operand of the output projection (matrix-core layout)
+  }
+  PYRE_TS(4); PYRE_TS(5); PYRE_TS(6); PYRE_TS(7); PYRE_TS_FLUSH(gdn_ts, 0);
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
@@ -102,7 +102,7 @@ int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int strid
   if (aop && t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: an f16 operand holds at most 8 tokens, not %d", t);
   if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
   if (g.conv_k < 2 || g.conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: conv kernel %d outside 2..8", g.conv_k);
-  if (t < 1) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d", t);
+  if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d outside 1..8", t);
   int ch = 2 * g.nk * g.dk + g.nv * g.dv;
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0); } PYRE_CHECK_LAUNCH(ctx);
