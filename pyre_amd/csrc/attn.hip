@@ -108,26 +108,34 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 //  phase 2: chunk-local max / exp / sum per head (thread = position x head group)
 //  phase 3: D[dim][head] += V[position][dim] e[position][head]; row i of tile dt stands for dim 4*i + dt, so a lane's
 //           4 tiles are one float4 (or 4 nibbles of one word) per position.  The four position quarters are added in order.
+// A window's tokens share the pass over the cache: the 16 columns hold the G heads of up to 16 / G tokens (token k of the
+// pass in columns k*G .. k*G+G-1), each with its own view (token k sees one position more than token k-1) -- a column's
+// sums do not depend on its neighbours, so a token's result is what a pass of its own gives.  The 4-bit boundary is a
+// property of a token's view; when it moves inside a window (one window in 64 / t) the launch gives every token a pass
+// of its own (tp = 1).
 typedef float f4v __attribute__((ext_vector_type(4)));
-template <int HD, int G>
-__global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+// NC: columns the buffers hold -- G for launches of one token a pass (tp = 1), 16 otherwise.
+template <int HD, int G, int NC>
+__global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int t, int tp) {
   static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
   constexpr int NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;
   static_assert(4 * CH == NPW * HD, "the score and value partials share one buffer");
-  __shared__ float red[4 * CH * G];          // phase 1: [dq][position][g];  phase 3: [pw][g][dim]
-  __shared__ float sc[CH][G];
-  __shared__ float wmax[NPW][G], wsum[NPW][G], cm[G];
-  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  __shared__ float red[4 * CH * NC];          // phase 1: [dq][position][column];  phase 3: [pw][column][dim]
+  __shared__ float sc[CH][NC];
+  __shared__ float wmax[NPW][NC], wsum[NPW][NC], cm[NC];
+  const int chunk = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
-  const int n = start + ti + 1;
+  const int tk0 = blockIdx.z * tp, nk = min(tp, t - tk0), ncol = nk * G;          // tokens tk0 .. tk0+nk-1 in columns 0 .. ncol-1
+  const int n = start + tk0 + nk;                                                  // the widest view of the pass
   if (chunk * CH >= n) return;
-  const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
-  const int wbase = chunk * CH + pw * 64, p = wbase + lane;
-  const bool valid = p < n, packed = wbase < pb, active = wbase < n;
   const float scale = 1.0f / sqrtf((float)HD);
   const int li = lane & 15, lg = lane >> 4;
   const int row = a.nkv * HD;
+  const int pb = (int)((a.kv_bits == 4 && n > a.kv_recent + 64) ? ((n - a.kv_recent) / 64) * 64 : 0);
+  const int wbase = chunk * CH + pw * 64, p = wbase + lane;
+  const bool packed = wbase < pb, active = wbase < n;
+  const int ctok = li / G, chead = li - ctok * G;                                              // the lane's column: token of the pass, head of the group
   // ---- phase 1
   {
     f4v D[4];
@@ -135,8 +143,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
     for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     if (active) {
       float B[16];
-      if (li < G) {
-        const float4* q4 = (const float4*)(qbuf + ((size_t)ti * a.nh + (size_t)kvh * G + li) * HD + dq * 64 + 16 * lg);
+      if (li < ncol) {
+        const float4* q4 = (const float4*)(qbuf + ((size_t)(tk0 + ctok) * a.nh + (size_t)kvh * G + chead) * HD + dq * 64 + 16 * lg);
 #pragma unroll
         for (int j = 0; j < 4; ++j) { float4 v = q4[j]; B[4 * j] = v.x; B[4 * j + 1] = v.y; B[4 * j + 2] = v.z; B[4 * j + 3] = v.w; }
       } else {
@@ -169,42 +177,44 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
     }
-    if (li < G) {
+    if (li < ncol) {
 #pragma unroll
       for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * G + li] = D[pt][r];
+        for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * NC + li] = D[pt][r];
     }
   }
   __syncthreads();
-  // ---- phase 2: this thread's position is pw*64 + lane, its heads are dq, dq + 4, ...
-  constexpr int GH = (G + 3) / 4;
+  // ---- phase 2: this thread's position is pw*64 + lane, its columns are dq, dq + 4, dq + 8, dq + 12
   const int pos = pw * 64 + lane;
+  constexpr int GH = (NC + 3) / 4;
   float sv[GH];
 #pragma unroll
   for (int gi = 0; gi < GH; ++gi) {
-    const int g = dq + 4 * gi; sv[gi] = -INFINITY;
-    if (g < G) {
-      float v = ((red[((size_t)0 * CH + pos) * G + g] + red[((size_t)1 * CH + pos) * G + g]) + red[((size_t)2 * CH + pos) * G + g]) + red[((size_t)3 * CH + pos) * G + g];
+    const int c = dq + 4 * gi; sv[gi] = -INFINITY;
+    if (c < ncol) {
+      const bool valid = p < start + tk0 + c / G + 1;          // the column's token sees positions below its own + 1
+      float v = ((red[((size_t)0 * CH + pos) * NC + c] + red[((size_t)1 * CH + pos) * NC + c]) + red[((size_t)2 * CH + pos) * NC + c]) + red[((size_t)3 * CH + pos) * NC + c];
       sv[gi] = valid ? v * scale : -INFINITY;
       float m = sv[gi];
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-      if (lane == 0) wmax[pw][g] = m;
+      if (lane == 0) wmax[pw][c] = m;
     }
   }
   __syncthreads();
-  if (tid < G) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
+  if (tid < ncol) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
   __syncthreads();
 #pragma unroll
   for (int gi = 0; gi < GH; ++gi) {
-    const int g = dq + 4 * gi;
-    if (g < G) {
-      float e = valid ? expf(sv[gi] - cm[g]) : 0.0f; sc[pos][g] = e;
+    const int c = dq + 4 * gi;
+    if (c < ncol) {
+      const bool valid = p < start + tk0 + c / G + 1;
+      float e = valid ? expf(sv[gi] - cm[c]) : 0.0f; sc[pos][c] = e;
       float l = e;
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
-      if (lane == 0) wsum[pw][g] = l;
+      if (lane == 0) wsum[pw][c] = l;
     }
   }
   __syncthreads();   // weights of every position visible; the score partials in `red` are dead
@@ -239,30 +249,30 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
       }
       float B[16];
 #pragma unroll
-      for (int s = 0; s < 16; ++s) B[s] = li < G ? sc[pw * 64 + 4 * s + lg][li < G ? li : 0] : 0.0f;
+      for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
 #pragma unroll
       for (int s = 0; s < 16; ++s)
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
     }
-    if (li < G) {
+    if (li < ncol) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[((size_t)pw * G + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
+        for (int r = 0; r < 4; ++r) red[((size_t)pw * NC + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
     }
   }
   __syncthreads();
-  for (int i = tid; i < G * HD; i += NT) {
-    int g = i / HD, dd = i % HD;
-    float o = red[((size_t)0 * G + g) * HD + dd];
+  for (int i = tid; i < ncol * HD; i += NT) {
+    const int c = i / HD, dd = i % HD, tk = tk0 + c / G, g = c % G;
+    float o = red[((size_t)0 * NC + c) * HD + dd];
 #pragma unroll
-    for (int q = 1; q < NPW; ++q) o += red[((size_t)q * G + g) * HD + dd];
-    part_o[(((size_t)ti * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
+    for (int q = 1; q < NPW; ++q) o += red[((size_t)q * NC + c) * HD + dd];
+    part_o[(((size_t)tk * a.nh + (size_t)kvh * G + g) * max_chunks + chunk) * HD + dd] = o;
   }
-  if (tid < G) {
+  if (tid < ncol) {
     float l = wsum[0][tid]; for (int q = 1; q < NPW; ++q) l += wsum[q][tid];
-    float* ml = part_ml + (((size_t)ti * a.nh + (size_t)kvh * G + tid) * max_chunks + chunk) * 2;
+    float* ml = part_ml + (((size_t)(tk0 + tid / G) * a.nh + (size_t)kvh * G + tid % G) * max_chunks + chunk) * 2;
     ml[0] = cm[tid]; ml[1] = l;
   }
 }
@@ -532,7 +542,12 @@ void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
 
 template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp, const QsaWork* qw) {
   int n = start + t, chunks = posp ? w.max_chunks : (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;      // device-side position: cover the whole cache, surplus workgroups leave at once
-  if (!qw) { hipLaunchKernelGGL((k_attn_decode<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks); return; }
+  if (!qw) {          // tokens that share a pass over the cache: as many as the 16 columns hold, one when the 4-bit boundary moves inside the window
+    int tp = 16 / G > 8 ? 8 : 16 / G;
+    if (posp || pyre_packed_boundary((size_t)start + 1, a.kv_bits, a.kv_recent) != pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent)) tp = 1;
+    if (tp == 1 || t == 1) hipLaunchKernelGGL((k_attn_decode<256, G, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, t, 1);
+    else hipLaunchKernelGGL((k_attn_decode<256, G, 16>), dim3(chunks, a.nkv, (t + tp - 1) / tp), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, t, tp);
+    return; }
   // a token attends either to all of its n <= budget + ratio - 1 visible positions or to a list: never to more than list_stride entries
   { int lc = (qw->list_stride + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK; if (chunks > lc) chunks = lc; }
   hipLaunchKernelGGL((k_attn_decode_sel<256, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, qw->plist, qw->pcount, qw->list_stride);

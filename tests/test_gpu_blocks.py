@@ -177,8 +177,9 @@ def test_attention_matches_oracle(ctx, nh, nkv, kv_bits, recent, start):
     assert len(att) == start + t and relerr(k2, K) <= 1e-6 and np.array_equal(v2, V)
 
 
-def test_attention_token_by_token_growth_crosses_the_packing_boundary(ctx):
-    nh, nkv, recent = 4, 2, 64
+@pytest.mark.parametrize("nh", [4, 16])          # 2 and 8 heads per KV head: eight and two tokens of a window share a pass over the cache
+def test_attention_token_by_token_growth_crosses_the_packing_boundary(ctx, nh):
+    nkv, recent = 2, 64
     row = nkv * 256
     p = attn_inputs(nh, nkv, 9, 200)
     att = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, recent, 256)
@@ -191,6 +192,14 @@ def test_attention_token_by_token_growth_crosses_the_packing_boundary(ctx):
         ref = orc.attn_core(nh, nkv, 256, 64, 1e-6, inv, p["qn"], p["kn"], p["q"][i:i + t], p["k"][i:i + t], p["v"][i:i + t], i, 4, recent, K, V)
         worst = max(worst, relerr(out, ref)); i += t
     assert i == 200 and orc.packed_boundary(200, 4, recent) == 128 and worst <= 2e-5
+    # the windows' rows are bit for bit what single steps give (the window 186..193 spans the move of the 4-bit boundary at 192)
+    att2 = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, recent, 256)
+    att2.load_cache(*[x[:186] for x in att.read_cache()])
+    att3 = lib.Attn(ctx, nh, nkv, 256, 64, 1e7, 1e-6, p["qn"], p["kn"], 4, recent, 256)
+    att3.load_cache(*[x[:186] for x in att.read_cache()])
+    win = att2.decode(p["q"][186:194], p["k"][186:194], p["v"][186:194])
+    one = np.concatenate([att3.decode(p["q"][j:j + 1], p["k"][j:j + 1], p["v"][j:j + 1]) for j in range(186, 194)])
+    assert np.array_equal(win.view(np.uint32), one.view(np.uint32))
 
 
 def test_attention_closed_forms(ctx):
