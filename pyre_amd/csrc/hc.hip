@@ -362,8 +362,8 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
 
 // grid (d / 64), hc*4 waves: wave (s, g) takes row group g of row tile s*(d/64) + blockIdx.x of `up` over all lr columns
 // (at most sixteen slices).  Prologue, epilogue and the riding router GEMV as k_hc_up_mix, except that every load the
-// prologue and the epilogue need is issued at the start (two rows of lo and one inject row a thread, two (token, stream)
-// items a wave), and lo goes through shared memory twice: f32, then as operand rows scaled per token by the power of two
+// prologue and the epilogue need is issued at the start (two rows of lo and one inject row a thread, the streams of one
+// column a thread), and lo goes through shared memory twice: f32, then as operand rows scaled per token by the power of two
 // of its largest magnitude.
 template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
@@ -376,8 +376,7 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   float* lo = sm;                                 // [T][lr]
   float* red = lo + (size_t)T * lr;               // [hc][T][64]: the gate logits
   float* sls = red + (size_t)hc * T * 64;         // [T][16]
-  float* term = sls + (size_t)T * 16;             // [T*hc][64]
-  uint32_t* lmax = (uint32_t*)(term + (size_t)T * hc * 64);      // [8]: bits of the largest |lo| of each token
+  uint32_t* lmax = (uint32_t*)(sls + (size_t)T * 16);      // [8]: bits of the largest |lo| of each token
   uint16_t* ah = (uint16_t*)(lmax + 8);           // [lr/8][16][8]
   const int K128 = lr >> 7, n_lo = T * lr;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -397,10 +396,12 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   const int rg = (s * (d >> 6) + blockIdx.x) * 4 + g;
   WBuf<1> w0, w1; load_w<1>(up, rg, 0, lane, K128, w0); load_w<1>(up, rg, 1, lane, K128, w1);
   const NibK nk = nib_consts();
-  // the epilogue's stream value and norm weight of this wave's (token, stream) items: wave, wave + nw
-  float xpre[2] = {0.0f, 0.0f}, npre[2] = {0.0f, 0.0f};
+  // the epilogue's operands: thread (token tid / 64, column tid % 64) adds the streams of its column itself
+  float xpre[4] = {0.0f, 0.0f, 0.0f, 0.0f}, npre[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (tid < T * 64) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j) { const int w = wave + j * nw; if (w < T * hc) { const int t0 = w / hc, q0 = w - t0 * hc; xpre[j] = (xnew + ((size_t)t0 * hc + q0) * d + blockIdx.x * 64)[lane]; npre[j] = (norm + (size_t)q0 * d + blockIdx.x * 64)[lane]; } }
+    for (int qs = 0; qs < 4; ++qs) if (qs < hc) { xpre[qs] = xnew[((size_t)(tid >> 6) * hc + qs) * d + blockIdx.x * 64 + lane]; npre[qs] = norm[(size_t)qs * d + blockIdx.x * 64 + lane]; }
+  }
   UnitRaw<RFX> rraw;
   constexpr bool R_EARLY = RFX != FMT_F32;      // an f32 tile is 64 registers: fetched once the up GEMV has freed them; others once the slice sums are used up
   if (tid < 8) lmax[tid] = 0u;
@@ -441,20 +442,10 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   if (2 * q + 1 < T) red[((size_t)s * T + 2 * q + 1) * 64 + g * 16 + (lane & 15)] = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
   if (ROUTE && !R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
   lds_barrier();
+  if (tid < T * 64) {          // the gated, normalised streams of the column, streams ascending from zero (:1380)
+    const int t2 = tid >> 6, l = lane, col = blockIdx.x * 64 + l; float mx = 0.0f;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {          // one wave per (token, stream): xn * sigm(gate) -> term
-    const int w = wave + j * nw;
-    if (w < T * hc) {
-      const int t2 = w / hc, qs = w - t2 * hc;
-      const float gl = red[((size_t)qs * T + t2) * 64 + lane];
-      term[(size_t)w * 64 + lane] = xpre[j] * sls[t2 * 16 + qs * kps] * npre[j] * sigm(gl);            // rms: (x * s) * w
-    }
-  }
-  lds_barrier();
-  for (int i2 = tid; i2 < T * 64; i2 += nthr) {
-    const int t2 = i2 >> 6, l = i2 & 63, col = blockIdx.x * 64 + l; float mx = 0.0f;
-#pragma unroll
-    for (int qs = 0; qs < 8; ++qs) if (qs < hc) mx += term[(size_t)(t2 * hc + qs) * 64 + l];
+    for (int qs = 0; qs < 4; ++qs) if (qs < hc) mx += xpre[qs] * sls[t2 * 16 + qs * kps] * npre[qs] * sigm(red[((size_t)qs * T + t2) * 64 + l]);            // rms: (x * s) * w
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
     if (aop) aop_store(aop, aop_rows, col, t2, mv);
@@ -529,7 +520,7 @@ template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcW
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
-  const int nw = h.hc * 4; const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + (size_t)T * h.hc * 64 + 8) + (size_t)h.lr * 32;
+  const int nw = h.hc * 4; const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + 8) + (size_t)h.lr * 32;
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
