@@ -198,3 +198,24 @@ def test_restore_starts_the_drafter_over_and_errors_are_reported(ctx):
         gd.attach(so)
     for o in (so, other, snap, gd, gs, gm):
         o.close()
+
+
+def test_drafter_beside_a_model_with_per_layer_ngram_embeddings(ctx):
+    # both keep a token history by position on the device: the state's one serves the n-gram hashes and the drafter's catch-up
+    c = mg.with_ple(small_cfg(qtype=synth.IQ3_S, hc_type=synth.IQ3_S, hc_lr=256), layers=(0, 2))
+    gm, gd, om, od = pair(ctx, c, 97, window=8)
+    gs, os_ = gm.new_state(128), om.new_state(); gd.attach(gs); od.attach(os_)
+    prompt = np.random.Generator(np.random.PCG64(98)).integers(0, c.vocab, 19, dtype=np.uint32)
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-3
+    pending = int(orc.argmax(lo))
+    d = same_drafts(gd, gs, od, os_, pending, 3)
+    toks = np.array([pending] + [int(x) for x in d], dtype=np.uint32)
+    gm.forward_multi(toks, gs); om.forward_multi(toks, os_); gm.spec_keep(gs, 4, 1); om.spec_keep(os_, 4, 1)
+    same_drafts(gd, gs, od, os_, 5, 2)
+    s0 = gm.new_state(128); fl = gm.forward(prompt, s0); plain, _ = gm.generate_greedy(s0, fl, 16)
+    s1 = gm.new_state(128); gd.attach(s1); fl1 = gm.forward(prompt, s1)
+    out, rounds, drafted, accepted = gd.generate_greedy(s1, fl1, 16, k=3)
+    assert np.array_equal(out, plain)
+    for o in (gd, gs, s0, s1, gm):
+        o.close()
