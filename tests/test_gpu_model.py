@@ -212,6 +212,40 @@ def test_verify_window_equals_single_steps_and_rollback(ctx):
         gm.spec_keep(sa, 5, 2)                                        # not armed any more
 
 
+@pytest.mark.parametrize("d,hc,rows", [(256, 2, False), (512, 4, False), (1024, 2, False), (512, 4, True)])
+def test_matrix_core_hyper_connection_mixes_windows_equal_steps_and_the_oracle(ctx, monkeypatch, d, hc, rows):
+    # IQ3_S hyper-connection matrices with a low rank of 256: the mixes run on the matrix cores (slices of 256 or 512
+    # columns, 2 or 4 streams); every window width gives a token the bits of a single step, and the oracle's logits.
+    # rows: the same through the lane = row kernels (PYRE_HC_ROWS) -- the two agree within the logits' bound.
+    monkeypatch.delenv("PYRE_HC_ROWS", raising=False)
+    c = small_cfg(d=d, hc=hc, hc_lr=256, qtype=synth.IQ3_S, hc_type=synth.IQ3_S, n_layers=4)
+    hw, gm, om = pair(ctx, c, 23)
+    g = np.random.Generator(np.random.PCG64(24))
+    prompt = g.integers(0, c.vocab, 13, dtype=np.uint32)
+    sa, sb, so = gm.new_state(64), gm.new_state(64), om.new_state()
+    la = gm.forward(prompt, sa); gm.forward(prompt, sb); lo = om.forward(prompt, so)
+    assert relerr(la, lo) <= 1e-3
+    for t in (8, 5, 3, 2):
+        toks = g.integers(0, c.vocab, t, dtype=np.uint32)
+        lv = gm.forward_multi(toks, sa)
+        singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(t)])
+        assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32)), t
+        assert relerr(lv, om.forward_multi(toks, so)) <= 1e-3, t
+    if rows:          # one of the geometries again through the other kernels (the switch is read once per process: a fresh one)
+        import subprocess, sys, os
+        code = ("import numpy as np, sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+                "from pyre_amd import lib, synth, modelgen as mg\n"
+                "c = mg.Config(n_layers=4, d=%d, hc=%d, hc_lr=256, n_exp=8, top_k=2, ff_exp=256, vocab=512, kv_recent=64, qtype=synth.IQ3_S, hc_type=synth.IQ3_S)\n"
+                "ctx = lib.Context(0); hw = mg.build_host(c, seed=23); gm = lib.Model(ctx, c, hw.layers, hw.globals_); st = gm.new_state(64)\n"
+                "lg = gm.forward(np.frombuffer(bytes.fromhex(%r), dtype=np.uint32), st); sys.stdout.write(lg.tobytes().hex())\n") % (
+                    os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)), d, hc, prompt.tobytes().hex())
+        env = dict(os.environ, PYRE_HC_ROWS="1")
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        lr = np.frombuffer(bytes.fromhex(out.stdout.strip()), dtype=np.float32)
+        assert relerr(lr, lo) <= 1e-3 and relerr(lr, la) <= 1e-3 and int(np.argmax(lr)) == int(np.argmax(la))
+
+
 def test_drafted_generation_identical_to_plain_and_to_oracle(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 8)
