@@ -8,11 +8,12 @@ PYRE_TS_DECL(moe_ts) PYRE_TS_EXPORT(moe_ts, pyre_debug_ts_moe)
 // ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id -----------------------------
 // Runs inside every gate/up workgroup of a routed entry (all of them need the expert id before they can touch a
 // weight, and a separate launch would cost more than redoing this small selection everywhere).
-// Thread e sums logit e's K slices (in slice order) into shared memory; wave 0 then holds the logits R per lane and
-// takes the maximum k times: a lane keeps the best of its own live logits, the wave's best of those comes out of six
-// idempotent DPP steps (no shared memory, no barrier), its owner retires it and rescans.  Leaves the chosen ids
-// (ascending) in s_idx[0..k) and their logits in s_val[0..k).
-struct RouteLds { float lv[1024]; float r_val[32]; float s_val[32]; int s_idx[32]; float s_w[32]; };
+// Thread e sums logit e's K slices (in slice order) into shared memory.  The selection is a tournament: every wave
+// of 64 logits takes its own k largest (k rounds of: the wave's largest key out of six DPP maximum steps, its lowest lane
+// -- the lowest index -- from a ballot, that lane retires its key), the waves' candidates meet in shared memory, each
+// candidate counts the candidates that beat it (larger key, or equal key and lower index) and the k that are beaten by
+// fewer than k others are the choice.  Leaves the chosen ids (ascending) in s_idx[0..k) and their logits in s_val[0..k).
+struct RouteLds { float lv[1024]; float r_val[32]; float s_val[32]; int s_idx[32]; float s_w[32]; uint64_t cand[512]; uint64_t win[32]; };
 #ifdef PYRE_PHASE_TS
 #define ROUTE_TS_PARAM , unsigned long long* rts_
 #define ROUTE_TS_ARG , ts_
@@ -22,48 +23,58 @@ struct RouteLds { float lv[1024]; float r_val[32]; float s_val[32]; int s_idx[32
 #define ROUTE_TS_ARG
 #define ROUTE_TS(k)
 #endif
-// A logit becomes a 32-bit key whose unsigned order is the logits' order (0 = no candidate); the largest key of the wave
-// comes out of six DPP maximum steps, the lowest index that holds it out of six DPP minimum steps.
+// A logit becomes a 32-bit key whose unsigned order is the logits' order (0 = no candidate).
 __device__ __forceinline__ uint32_t route_key(float v) {
   uint32_t u = __float_as_uint(v + 0.0f);          // -0 counts as +0, as in a float comparison
   return u ^ ((u & 0x80000000u) ? 0xFFFFFFFFu : 0x80000000u);
 }
 __device__ __forceinline__ float route_key_value(uint32_t u) { return __uint_as_float(u ^ ((u & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu)); }
-template <int CTRL> __device__ __forceinline__ uint32_t route_dpp(uint32_t m) {          // lanes without a source see their own value
-  return (uint32_t)__builtin_amdgcn_update_dpp((int)m, (int)m, CTRL, 0xf, 0xf, false);
+template <int CTRL> __device__ __forceinline__ uint32_t route_dpp(uint32_t m) {          // lanes without a source see 0, the maximum's identity: the move folds into the v_max
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, CTRL, 0xf, 0xf, true);
 }
-__device__ __forceinline__ uint32_t route_wave_max(uint32_t m) {          // both are idempotent, so the row broadcasts need no row masks
+__device__ __forceinline__ uint32_t route_wave_max(uint32_t m) {          // idempotent, so the row broadcasts need no row masks
   m = max(m, route_dpp<0x111>(m)); m = max(m, route_dpp<0x112>(m)); m = max(m, route_dpp<0x114>(m)); m = max(m, route_dpp<0x118>(m));      // row_shr 1, 2, 4, 8: lane 15 of a row holds the row's
   m = max(m, route_dpp<0x142>(m)); m = max(m, route_dpp<0x143>(m));          // row_bcast 15, 31: lane 63 holds the wave's
   return (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
 }
-__device__ __forceinline__ uint32_t route_wave_min(uint32_t m) {
-  m = min(m, route_dpp<0x111>(m)); m = min(m, route_dpp<0x112>(m)); m = min(m, route_dpp<0x114>(m)); m = min(m, route_dpp<0x118>(m));
-  m = min(m, route_dpp<0x142>(m)); m = min(m, route_dpp<0x143>(m));
-  return (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
-}
-template <int R> __device__ __forceinline__ void route_select(int n_exp, int k, RouteLds& L, int lane) {
-  // straight-line code (selects, no divergent branches: a branch costs more here than the few operations it would skip)
-  uint32_t key[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) { const int idx = r * 64 + lane; const uint32_t kk = route_key(L.lv[min(idx, 1023)]); key[r] = idx < n_exp ? kk : 0u; }
-  uint32_t sel_k = 0u, sel_i = 0u;
-  for (int round = 0; round < k; ++round) {
-    uint32_t m = key[0];
-#pragma unroll
-    for (int r = 1; r < R; ++r) m = max(m, key[r]);
-    const uint32_t wm = route_wave_max(m);
-    uint32_t mi = 0xFFFFFFFFu;
-#pragma unroll
-    for (int r = R - 1; r >= 0; --r) mi = key[r] == wm ? (uint32_t)(r * 64 + lane) : mi;          // the lane's lowest index holding the maximum
-    const uint32_t wi = route_wave_min(mi);
-    sel_k = lane == round ? wm : sel_k; sel_i = lane == round ? wi : sel_i;
-#pragma unroll
-    for (int r = 0; r < R; ++r) key[r] = (uint32_t)(r * 64 + lane) == wi ? 0u : key[r];          // its owner retires it
+// called by the whole workgroup (at least n_exp threads, a multiple of 64), after lv[] is complete
+__device__ __forceinline__ void route_select(int n_exp, int k, RouteLds& L) {
+  const int e = threadIdx.x, lane = e & 63, wave = e >> 6, nwv = (n_exp + 63) >> 6;
+  if (wave < nwv) {
+    uint32_t key = e < n_exp ? route_key(L.lv[e]) : 0u;
+    uint32_t ck = 0u, cl = 0u;          // lane r keeps the wave's r-th candidate
+    for (int round = 0; round < k; ++round) {
+      const uint32_t wm = route_wave_max(key);
+      const int ol = __ffsll((unsigned long long)__ballot(key == wm)) - 1;          // the lowest lane that holds it = the lowest index
+      ck = lane == round ? wm : ck; cl = lane == round ? (uint32_t)ol : cl;
+      key = lane == ol ? 0u : key;
+    }
+    if (lane < k) L.cand[wave * k + lane] = ((uint64_t)ck << 32) | (uint32_t)(0xFFFFFFFFu - ((uint32_t)(wave * 64) + cl));
   }
-  int pos = 0;
-  for (int j = 0; j < k; ++j) { const uint32_t oj = (uint32_t)__builtin_amdgcn_readlane((int)sel_i, j); pos += oj < sel_i ? 1 : 0; }
-  if (lane < k) { L.s_idx[pos] = (int)sel_i; L.s_val[pos] = route_key_value(sel_k); }
+  lds_barrier();
+  // eight neighbouring lanes share a candidate and split the others among them; larger 64-bit word = larger key, or the
+  // same key at a lower index: a strict order, so the k winners hold the ranks 0 .. k-1
+  const int nc = nwv * k, sub = e & 7;
+  for (int i = e >> 3; i < nc; i += (int)(blockDim.x >> 3)) {
+    const uint64_t ci = L.cand[i];
+    int beaten = 0;
+    for (int j = sub; j < nc; j += 32) {
+      const uint64_t c0 = L.cand[min(j, 511)], c1 = L.cand[min(j + 8, 511)], c2 = L.cand[min(j + 16, 511)], c3 = L.cand[min(j + 24, 511)];
+      beaten += (c0 > ci ? 1 : 0) + ((j + 8 < nc && c1 > ci) ? 1 : 0) + ((j + 16 < nc && c2 > ci) ? 1 : 0) + ((j + 24 < nc && c3 > ci) ? 1 : 0);
+    }
+    beaten += __builtin_amdgcn_mov_dpp(beaten, 0xB1, 0xf, 0xf, true);          // quad_perm [1,0,3,2]
+    beaten += __builtin_amdgcn_mov_dpp(beaten, 0x4E, 0xf, 0xf, true);          // quad_perm [2,3,0,1]
+    beaten += __builtin_amdgcn_mov_dpp(beaten, 0x141, 0xf, 0xf, true);         // row_half_mirror: the other quad of the eight
+    if (sub == 0 && (uint32_t)(ci >> 32) != 0u && beaten < k) L.win[beaten] = ci;
+  }
+  lds_barrier();
+  if (wave == 0) {
+    const uint64_t w = L.win[min(lane, 31)];
+    const uint32_t idx = 0xFFFFFFFFu - (uint32_t)w;
+    int pos = 0;
+    for (int j = 0; j < k; ++j) { const uint32_t oj = (uint32_t)__builtin_amdgcn_readlane((int)idx, j); pos += oj < idx ? 1 : 0; }
+    if (lane < k) { L.s_idx[pos] = (int)idx; L.s_val[pos] = route_key_value((uint32_t)(w >> 32)); }
+  }
 }
 // The logits are given as nsl (<= 64) K-slice sums `sstride` floats apart, added in slice order (nsl == 1: the logits
 // themselves); all slices are fetched before the first add, in groups of eight behind launch-uniform branches.
@@ -86,7 +97,7 @@ __device__ __forceinline__ void route_topk(const float* __restrict__ logits, int
   }
   ROUTE_TS(5);
   lds_barrier(); ROUTE_TS(6);
-  if (wave == 0) { if (n_exp <= 512) route_select<8>(n_exp, k, L, lane); else route_select<16>(n_exp, k, L, lane); }
+  route_select(n_exp, k, L);
   ROUTE_TS(7);
   lds_barrier();
 }
