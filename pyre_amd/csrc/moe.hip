@@ -126,10 +126,13 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // rows on nz compute units instead of one; at one token a launch of tiles x (k+1) workgroups leaves most of the chip
 // idle -- and leaves the part's raw sums, gate at h[((entry*nz + kz)*2 + 0)*hstride + row], up at [... + 1]; the down
 // launch adds the parts and forms silu(g) * u with the same operations.
+// The window form (PRE, both parts in the workgroup) is held to 64 registers for the formats whose decode fits them
+// (next to) without spilling, so that two workgroups share a compute unit: five tokens' 440 workgroups are then resident
+// at once instead of taking a second turn on the 256 compute units.
 // PRE: the token's experts were chosen by k_moe_route (windows of several tokens: hundreds of workgroups would each redo
 // the selection otherwise); the workgroup reads its expert id and publishes nothing but the shared-expert gate.
 template <int FMT, int NW, int P, bool PRE>
-__global__ __launch_bounds__(NW * 64) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
+__global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 8 : 1) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
