@@ -116,7 +116,7 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 typedef float f4v __attribute__((ext_vector_type(4)));
 // NC: columns the buffers hold -- G for launches of one token a pass (tp = 1), 16 otherwise.
 template <int HD, int G, int NC>
-__global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int t, int tp) {
+__global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int t, int tp) {
   static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
   constexpr int NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;
   static_assert(4 * CH == NPW * HD, "the score and value partials share one buffer");
@@ -136,6 +136,16 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
   const int wbase = chunk * CH + pw * 64, p = wbase + lane;
   const bool packed = wbase < pb, active = wbase < n;
   const int ctok = li / G, chead = li - ctok * G;                                              // the lane's column: token of the pass, head of the group
+  // The packed values do not depend on the scores: their loads go out with the keys', one memory round trip for both.
+  uint32_t vw[16]; float vsc[16];
+  if (active && packed) {
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const size_t pg = (size_t)wbase + 4 * s + lg;
+      vw[s] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
+      vsc[s] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
+    }
+  }
   // ---- phase 1
   {
     f4v D[4];
@@ -151,8 +161,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
 #pragma unroll
         for (int s = 0; s < 16; ++s) B[s] = 0.0f;
       }
-      float A[4][16];
-      if (packed) {
+      if (packed) {             // the keys stay packed until the step that uses them: four values live, not sixty-four
         uint32_t kw[4][2]; float ksc[4];
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) {
@@ -161,21 +170,22 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
           ksc[pt] = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp)];
         }
 #pragma unroll
-        for (int pt = 0; pt < 4; ++pt)
+        for (int s = 0; s < 16; ++s)
 #pragma unroll
-          for (int s = 0; s < 16; ++s) A[pt][s] = nib_val(kw[pt][s >> 3], s & 7) * ksc[pt];
+          for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(nib_val(kw[pt][s >> 3], s & 7) * ksc[pt], B[s], D[pt], 0, 0, 0);
       } else {
+        float A[4][16];
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) {
           const size_t pp = (size_t)min(wbase + 16 * pt + li, n - 1);
 #pragma unroll
           for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp)];
         }
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+#pragma unroll
+          for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
       }
-#pragma unroll
-      for (int s = 0; s < 16; ++s)
-#pragma unroll
-        for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
     }
     if (li < ncol) {
 #pragma unroll
@@ -224,36 +234,31 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode(AttnDev a, 
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     if (active) {
-      float A[4][16];
+      float B[16];
       if (packed) {             // packed positions lie below the boundary, hence inside the view
-        uint32_t vw[16]; float vsc[16];
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-          const size_t pg = (size_t)wbase + 4 * s + lg;
-          vw[s] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
-          vsc[s] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
-        }
+        for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
           const uint32_t hw = vw[s] >> (16 * (li & 1));      // the lane's four nibbles
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) A[dt][s] = nib_val(hw, dt) * vsc[s];
+          for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(nib_val(hw, dt) * vsc[s], B[s], D[dt], 0, 0, 0);
         }
       } else {                  // positions past the view carry weight zero; their address is clamped
+        float A[4][16];
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
           const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);
           float4 v = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
           A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
         }
+#pragma unroll
+        for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
       }
-      float B[16];
-#pragma unroll
-      for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
-#pragma unroll
-      for (int s = 0; s < 16; ++s)
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
     }
     if (li < ncol) {
 #pragma unroll
