@@ -403,32 +403,48 @@ int pyre_gemv_conv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t
   return rc;
 }
 
-// 64 threads per block: every block redoes the (tiny) scan of the per-tile maxima, block 0 publishes the id, and when a
-// matrix is given thread u of block b then dequantizes unit 64*b+u of the chosen row.
-template <int FMT> __global__ __launch_bounds__(64) void k_pick(const uint32_t* __restrict__ best, int n_tiles, uint32_t* id_out, uint32_t* mirror, QMatDev m, int have_m,
-                                                               const uint64_t* g2, float* __restrict__ out, int* step, uint32_t* hist) {
+// 256 threads per block: every block redoes the (tiny) scan of the per-tile maxima -- a thread's candidates are all fetched
+// before the first is looked at, so the scan is one memory round trip up to 4096 tiles -- block 0 publishes the id, and when
+// a matrix is given thread u < 64 of block b then dequantizes unit 64*b+u of the chosen row.
+__device__ __forceinline__ void pick_better(float& bv, uint32_t& bi, float v, uint32_t r) {          // larger value, then lower row; 0xFFFFFFFF = no candidate yet
+  if (r != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || v > bv || (v == bv && r < bi))) { bv = v; bi = r; }
+}
+template <int FMT> __global__ __launch_bounds__(256) void k_pick(const uint32_t* __restrict__ best, int n_tiles, uint32_t* id_out, uint32_t* mirror, QMatDev m, int have_m,
+                                                                const uint64_t* g2, float* __restrict__ out, int* step, uint32_t* hist) {
+  __shared__ float wv[4]; __shared__ uint32_t wi[4];
   const int tid = threadIdx.x;
   float bv = -INFINITY; uint32_t bi = 0xFFFFFFFFu;
   const uint2* b2 = (const uint2*)best;
-#pragma unroll 8
-  for (int i = tid; i < n_tiles; i += 64) { uint2 e = b2[i]; float v = __uint_as_float(e.x); uint32_t r = e.y; if (bi == 0xFFFFFFFFu || v > bv || (v == bv && r < bi)) { bv = v; bi = r; } }
+  for (int i0 = tid; i0 < n_tiles; i0 += 256 * 16) {
+    uint2 e[16];
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; } }
+    for (int q = 0; q < 16; ++q) e[q] = b2[min(i0 + 256 * q, n_tiles - 1)];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) if (i0 + 256 * q < n_tiles) pick_better(bv, bi, __uint_as_float(e[q].x), e[q].y);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { float ov = __shfl_xor(bv, o); uint32_t oi = __shfl_xor(bi, o); pick_better(bv, bi, ov, oi); }
+  if ((tid & 63) == 0) { wv[tid >> 6] = bv; wi[tid >> 6] = bi; }
+  __syncthreads();
+  bv = wv[0]; bi = wi[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) pick_better(bv, bi, wv[w], wi[w]);
   if (bi == 0xFFFFFFFFu) bi = 0;
   if (blockIdx.x == 0 && tid == 0) { int slot = 0; if (step) { int p = step[0] + 1; step[0] = p; slot = p - step[1]; if (hist) hist[p] = bi; } id_out[0] = bi; if (mirror) mirror[slot] = bi; }
-  if (!have_m) return;
+  if (!have_m || tid >= 64) return;
   int ku = blockIdx.x * 64 + tid; if (ku >= m.U || bi >= (uint32_t)m.rows) return;
   float y[64];
   decode_exact<FMT>(m, g2, (int)(bi >> 6), ku, (int)(bi & 63), y);
-  float* o = out + (size_t)ku * 64;
-  for (int i = 0; i < 64; ++i) o[i] = y[i];
+  float4* o = (float4*)(out + (size_t)ku * 64);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o[i] = float4{y[4 * i], y[4 * i + 1], y[4 * i + 2], y[4 * i + 3]};
 }
 
 int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best, int n_tiles, uint32_t* id_out, uint32_t* mirror, const QMatDev* m, float* out, int* step, uint32_t* hist) {
   ProfScope ps(ctx, "pick_embed", 8.0 * n_tiles);
-  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step, hist); }
+  if (!m) { QMatDev z{}; hipLaunchKernelGGL((k_pick<FMT_F32>), dim3(1), dim3(256), 0, ctx->stream, best, n_tiles, id_out, mirror, z, 0, (const uint64_t*)ctx->d_iq2xs, out, step, hist); }
   else { dim3 grid((m->U + 63) / 64);
-    FMT_DISPATCH_X(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(64), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step, hist)); }
+    FMT_DISPATCH_X(m->fmt, hipLaunchKernelGGL((k_pick<F>), grid, dim3(256), 0, ctx->stream, best, n_tiles, id_out, mirror, *m, 1, (const uint64_t*)ctx->d_iq2xs, out, step, hist)); }
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
