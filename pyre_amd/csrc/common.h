@@ -201,11 +201,19 @@ struct MoeWork {            // scratch for up to 8 tokens, owned by whoever laun
   float* sg;                // [8] sigmoid(sh_gate_inp . x)
   float* h;                 // [8*(top_k+1)][max(ff, sf)]
   float* partial;           // [8*(top_k+1)][d]
+  float* parts;             // [PYRE_MOE_GROUPS][t][d]: a window's output as group sums (pyre_moe_launch with in_groups)
 };
-// The FFN output of a window, left unreduced for the consumer to fold:
-//   y[ti][r] = partial[ti*(k+1)+k][r] * sg[ti] + (sum_j sel_w[ti*k+j] * partial[ti*(k+1)+j][r], j ascending, from zero)
+// The FFN output of a window, left unreduced for the consumer to fold.  The k expert terms (ascending id) and the shared
+// expert's form PYRE_MOE_GROUPS groups of g = (k + 4) / 4 consecutive experts, the shared expert in the last:
+//   P_q = sum over the group's experts, in order, from zero, of sel_w * partial      (+ partial[shared] * sg for the last)
+//   y[ti][r] = ((P_0 + P_1) + P_2) + P_3
+// -- the association a window's down projection uses when it leaves the four group sums instead (k_moe_down_groups), so
+// that a token's value does not depend on which of the two forms produced it.
 struct MoeOut { const float* partial; const float* sel_w; const float* sg; int d, k; };
 #define PYRE_MOE_KMAX 16      // moe_out_value keeps up to this many expert terms in registers
+#define PYRE_MOE_GROUPS 4     // == PYRE_GEMV_PARTS: the mix reads the group sums as it reads an output projection's K parts
+#define PYRE_MOE_GMAX 5       // entries of a group: (PYRE_MOE_KMAX + 4) / 4, the last group holds at most that many with the shared expert
+static_assert(PYRE_MOE_GROUPS == PYRE_GEMV_PARTS, "the mix adds the group sums as it adds an output projection's K parts");
 #ifdef __HIPCC__
 // All loads are issued before the first add, so the value costs one memory round trip, not k + 1.
 __device__ __forceinline__ float moe_out_value(const MoeOut& mo, int ti, int r) {
@@ -214,10 +222,17 @@ __device__ __forceinline__ float moe_out_value(const MoeOut& mo, int ti, int r) 
 #pragma unroll
   for (int j = 0; j < PYRE_MOE_KMAX; ++j) { pv[j] = j < mo.k ? p[(size_t)j * mo.d] : 0.0f; wv[j] = j < mo.k ? w[j] : 0.0f; }
   float sh = p[(size_t)mo.k * mo.d], g = mo.sg[ti];
-  float o = 0.0f;
+  const int gsz = (mo.k + 4) / 4;
+  float P[PYRE_MOE_GROUPS];
 #pragma unroll
-  for (int j = 0; j < PYRE_MOE_KMAX; ++j) if (j < mo.k) o += wv[j] * pv[j];
-  return sh * g + o;
+  for (int q = 0; q < PYRE_MOE_GROUPS; ++q) {
+    float o = 0.0f;
+#pragma unroll
+    for (int e = 0; e < PYRE_MOE_GMAX; ++e) { const int j = q * gsz + e; if (e < gsz && j < mo.k) o = fmaf(wv[j < PYRE_MOE_KMAX ? j : 0], pv[j < PYRE_MOE_KMAX ? j : 0], o); }
+    P[q] = o;
+  }
+  P[PYRE_MOE_GROUPS - 1] = fmaf(sh, g, P[PYRE_MOE_GROUPS - 1]);
+  return ((P[0] + P[1]) + P[2]) + P[3];
 }
 #endif
 inline MoeOut pyre_moe_out(const MoeDev& m, const MoeWork& w, int first_token) {
@@ -230,7 +245,10 @@ void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
 // Router logits that arrive as K-slice sums (left by the mix that produced x, see HcRoute): logit[t][e] = the slices
 // p[(s*T + t)*r64 + e], s = 0..nsl-1, added in slice order.
 struct RouteSrc { const float* p; int nsl; int r64; };
-int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr);
+// in_groups (t > 1, y == nullptr, pyre_moe_groups_ok): the down projection leaves the PYRE_MOE_GROUPS group sums of every
+// token in w.parts, group q of token ti at parts + (q*t + ti)*d, instead of the unreduced terms.
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr, bool in_groups = false);
+inline bool pyre_moe_groups_ok(const MoeDev& m) { return m.top_k <= PYRE_MOE_KMAX; }
 // K parts the gate/up dot products are summed in (1 or 2; k_moe_gu)
 int pyre_moe_gu_parts(const MoeDev& m);
 

@@ -426,6 +426,8 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
   const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
+  int comb_np = 1;          // vectors the pending update comes in: 1, or PYRE_GEMV_PARTS == PYRE_MOE_GROUPS to be added in order
+  const bool moe_groups = [] { const char* e = getenv("PYRE_MOE_GROUPS"); return !(e && *e && atoi(e) == 0); }();      // 0: windows leave the unreduced terms as a single token does
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
   // the window's tokens join the history (PLE models and states with a drafter keep one)
   if (s->tokens_dev && !o.from_best) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, m->ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));
@@ -443,8 +445,8 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_ple_launch(ctx, m->plc, pd, m->pw, d, hc, c.eps, xin, in_ss, in_ts, xout, comb_out, comb_moe, comb_inj, start, o.step_dev, t))) return rc;
       advance(); comb_out = nullptr; comb_moe = nullptr; comb_inj = nullptr;
     }
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, 1, opw(L.proj)))) return rc;
-    advance();
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.proj)))) return rc;
+    advance(); comb_np = 1;
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.proj)))) return rc;
@@ -464,8 +466,16 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
     advance();
-    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y, ride ? &rs : nullptr))) return rc;
-    if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
+    // A window's FFN output goes to the next mix as four group sums a token when that mix can add partial vectors (an
+    // IQ3_S mix over all of the window's tokens, no PLE layer in between); otherwise, and for a single token, unreduced.
+    bool groups = raw_moe && t > 1 && moe_groups && pyre_moe_groups_ok(L.moe);
+    if (groups) {
+      if (il + 1 < c.n_layers) { const Layer& Ln = m->layers[il + 1]; groups = !Ln.ple && Ln.hca.di.fmt == FMT_IQ3_S; }
+      else groups = (o.head_tokens >= t || (s->mtp && o.keep_from < t)) && m->head.di.fmt == FMT_IQ3_S;
+    }
+    if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y, ride ? &rs : nullptr, groups))) return rc;
+    if (groups) { comb_out = m->mw.parts; comb_moe = nullptr; comb_np = PYRE_MOE_GROUPS; }
+    else if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
     comb_inj = m->inj_f;
   }
   if (!replay) s->len = start + t;
@@ -473,7 +483,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   if (o.head_tokens == 0 && !want_r) return PYRE_OK;       // prompt window whose logits nobody reads
   if (o.head_tokens >= t || want_r) {
     const bool all = o.head_tokens >= t;
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, 1, all ? opw(m->out) : nullptr))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, comb_np, all ? opw(m->out) : nullptr))) return rc;
     if (want_r) {
       const int w = hc * d;
       hipLaunchKernelGGL(k_ring_store, dim3((w + 255) / 256, t - o.keep_from), dim3(256), 0, ctx->stream, xout, s->r_ring, s->r_mask, start, o.step_dev, o.keep_from, w); PYRE_CHECK_LAUNCH(ctx);

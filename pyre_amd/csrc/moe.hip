@@ -289,25 +289,97 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
   PYRE_TS(3); PYRE_TS_FLUSH(moe_ts, 8);
 }
 
-// y[ti][r] = shared[ti][r] * sg[ti] + (sum over the token's experts, ascending id, from zero, of w * partial)
+// y[ti][r]: the four group sums of moe_out_value, added in order (few experts only: top_k <= PYRE_MOE_KMAX; more experts
+// take the plain sum shared * sg + (the experts' terms in ascending id, from zero))
 __global__ void k_moe_sum(const float* __restrict__ partial, const float* __restrict__ sel_w, const float* __restrict__ sg, int d, int k, float* __restrict__ y) {
   int r = blockIdx.x * blockDim.x + threadIdx.x, ti = blockIdx.y; if (r >= d) return;
+  if (k <= PYRE_MOE_KMAX) { const MoeOut mo{partial, sel_w, sg, d, k}; y[(size_t)ti * d + r] = moe_out_value(mo, ti, r); return; }
   const float* p = partial + (size_t)ti * (k + 1) * d;
   float o = 0.0f; for (int j = 0; j < k; ++j) o += sel_w[ti * k + j] * p[(size_t)j * d + r];
   float yv = p[(size_t)k * d + r] * sg[ti];
   y[(size_t)ti * d + r] = yv + o;
 }
 
+// ---- expert down of a window, summed by groups: parts[(q*t + ti)*d + r] = P_q of moe_out_value -------------------------------
+// grid (d/64, t, PYRE_MOE_GROUPS), NW waves.  The workgroup computes the down rows of its group's (at most PYRE_MOE_GMAX)
+// entries as k_moe_down does -- wave w the K share w of every entry, the shares added in wave order -- and folds them with
+// the routing weights in the group's order: the consumer then reads four vectors a token instead of k + 1, and the value is
+// bit for bit what moe_out_value forms from k_moe_down's unreduced terms.  A wave's weights of all entries and its slices
+// of their activations (through its own shared memory: no workgroup barrier) are fetched before the first is used.
+// GE: entries a group can hold in this instance (3 covers top_k <= 11, PYRE_MOE_GMAX the rest) -- the register budget follows it.
+template <int FMT, int NW, int GE>
+__global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1) void k_moe_down_groups(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ sel_w, const float* __restrict__ sg,
+                                                            const float* __restrict__ h, int hstride, float* __restrict__ parts, const uint2* __restrict__ g2) {
+  static_assert(GE <= PYRE_MOE_GMAX, "a group holds at most PYRE_MOE_GMAX entries");
+  const uint2* lds2 = nullptr;
+  qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, parts);
+  __shared__ float red[GE][NW][64];
+  __shared__ float hx[NW][GE][64];
+  const int ti = blockIdx.y, q = blockIdx.z, k = m.top_k, gsz = (k + 4) / 4;
+  const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;          // the group's routed entries j0 .. j0+nr-1
+  const bool with_shared = q == PYRE_MOE_GROUPS - 1;
+  const int ne = nr + (with_shared ? 1 : 0);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  // the routed and the shared matrices may differ in width: each has its own K shares (as in k_moe_down)
+  const int Ur = m.down_e.U, Us = m.sh_down.U, upr = (Ur + NW - 1) / NW, ups = (Us + NW - 1) / NW;
+  const int niter = max(nr > 0 ? upr : 0, with_shared ? ups : 0);
+  int tile[GE]; const float* xs[GE];
+#pragma unroll
+  for (int e = 0; e < GE; ++e) {
+    const bool shared = with_shared && e == nr; const int j = shared ? k : min(j0 + e, k - 1);
+    tile[e] = (shared ? 0 : __builtin_amdgcn_readfirstlane(sel_idx[ti * k + j]) * (m.d >> 6)) + blockIdx.x;
+    xs[e] = h + (size_t)(ti * (k + 1) + j) * hstride;
+  }
+  float acc[GE][1];
+#pragma unroll
+  for (int e = 0; e < GE; ++e) acc[e][0] = 0.0f;
+  for (int it = 0; it < niter; ++it) {
+    UnitRaw<FMT> r[GE]; float hv[GE]; bool on[GE]; int ku[GE];
+#pragma unroll
+    for (int e = 0; e < GE; ++e) {
+      const bool shared = with_shared && e == nr; const int up = shared ? ups : upr, U = shared ? Us : Ur;
+      ku[e] = wave * up + it; on[e] = e < ne && it < up && ku[e] < U;
+      if (on[e]) { const QMatDev& D = shared ? m.sh_down : m.down_e; r[e] = unit_load<FMT>(D, tile[e], ku[e], lane); hv[e] = xs[e][ku[e] * 64 + lane]; }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int e = 0; e < GE; ++e) if (on[e]) hx[wave][e][lane] = hv[e];
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int e = 0; e < GE; ++e) if (on[e]) { const QMatDev& D = (with_shared && e == nr) ? m.sh_down : m.down_e; unit_fma<FMT, 1>(D, r[e], ku[e], lds2, lane, hx[wave][e], 0, acc[e]); }
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int e = 0; e < GE; ++e) if (e < ne) red[e][wave][lane] = acc[e][0];
+  lds_barrier();
+  if (threadIdx.x < 64) {
+    float wv[GE];
+#pragma unroll
+    for (int e = 0; e < GE; ++e) wv[e] = e < nr ? sel_w[ti * k + j0 + e] : 0.0f;
+    const float g = with_shared ? sg[ti] : 0.0f;
+    float o = 0.0f;
+#pragma unroll
+    for (int e = 0; e < GE; ++e) if (e < ne) {
+      float pv = red[e][0][lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) pv += red[e][w][lane];
+      if (e < nr) o = fmaf(wv[e], pv, o); else o = fmaf(pv, g, o);          // the shared expert comes last
+    }
+    parts[((size_t)q * gridDim.y + ti) * m.d + blockIdx.x * 64 + lane] = o;
+  }
+}
+
 #define PYRE_MOE_GU_NZMAX 2
 size_t pyre_moe_work_bytes(const MoeDev& m) {
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
-  return 256 * 8 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d);
+  return 256 * 9 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d + 8 * PYRE_MOE_GROUPS * (size_t)m.d);
 }
 void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
   w->logits = (float*)take(4 * 8 * (size_t)m.n_exp); w->sel_idx = (int32_t*)take(4 * 8 * (size_t)m.top_k); w->sel_w = (float*)take(4 * 8 * (size_t)m.top_k);
   w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
+  w->parts = (float*)take(4 * 8 * PYRE_MOE_GROUPS * (size_t)m.d);
 }
 
 #define MOE_FMT_DISPATCH(fmt, CALL) \
@@ -323,7 +395,8 @@ int pyre_moe_gu_parts(const MoeDev& m) {
   static const bool off = getenv("PYRE_MOE_GU_PARTS") && atoi(getenv("PYRE_MOE_GU_PARTS")) == 0;
   return (!off && m.gate_e.U % 32 == 0 && m.sh_gate.U == m.gate_e.U) ? 2 : 1;
 }
-int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y, const RouteSrc* routed) {
+int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x, int t, float* y, const RouteSrc* routed, bool in_groups) {
+  if (in_groups && (y || t < 2 || !pyre_moe_groups_ok(m))) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: group sums are for unreduced windows of 2..8 tokens with top_k <= %d", PYRE_MOE_KMAX);
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
   if (routed && (routed->nsl < 1 || routed->nsl > 64 || routed->r64 < m.n_exp)) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: %d router slices of %d rows", routed->nsl, routed->r64);
@@ -343,7 +416,13 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
 #undef GU_GO
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
-  if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
+  if (in_groups) {
+    const int gsz = (m.top_k + 4) / 4, last = m.top_k - min(m.top_k, (PYRE_MOE_GROUPS - 1) * gsz) + 1;          // entries of a full group, of the last (with the shared expert)
+#define DOWN_G_GO(GE) MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down_groups<F, 8, GE>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2))
+    if (gsz <= 3 && last <= 3) { DOWN_G_GO(3); } else { DOWN_G_GO(PYRE_MOE_GMAX); }
+#undef DOWN_G_GO
+  }
+  else if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
   else { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 2>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); } }
   PYRE_CHECK_LAUNCH(ctx);
   if (y) {

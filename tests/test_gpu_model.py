@@ -212,6 +212,27 @@ def test_verify_window_equals_single_steps_and_rollback(ctx):
         gm.spec_keep(sa, 5, 2)                                        # not armed any more
 
 
+@pytest.mark.parametrize("n_exp,top_k,ff_sh,qtype", [(32, 13, 512, synth.IQ3_S), (16, 3, 0, synth.IQ3_S), (16, 2, 0, synth.IQ3_S), (16, 10, 0, synth.Q4_K), (16, 11, 512, synth.Q8_0)])
+def test_window_ffn_output_as_group_sums_equals_single_steps_and_the_oracle(ctx, n_exp, top_k, ff_sh, qtype):
+    # With IQ3_S hyper-connection matrices a window's FFN output reaches the next mix as four group sums a token (groups of
+    # (k + 4) / 4 experts, the shared expert in the last; here groups of 4, 1, 1, 3 and 3 experts, an empty third group, a
+    # shared expert wider than the routed ones); a single token leaves the unreduced terms and the mix forms the same sums.
+    c = small_cfg(n_exp=n_exp, top_k=top_k, ff_sh=ff_sh, hc_lr=256, qtype=qtype, hc_type=synth.IQ3_S)
+    hw, gm, om = pair(ctx, c, 31)
+    g = np.random.Generator(np.random.PCG64(32))
+    prompt = g.integers(0, c.vocab, 11, dtype=np.uint32)
+    sa, sb, so = gm.new_state(64), gm.new_state(64), om.new_state()
+    la = gm.forward(prompt, sa); lo = om.forward(prompt, so)
+    for tok in prompt: lb = gm.forward(np.array([tok], dtype=np.uint32), sb)
+    assert relerr(la, lo) <= 1e-3 and np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    for t in (8, 5, 2):
+        toks = g.integers(0, c.vocab, t, dtype=np.uint32)
+        lv = gm.forward_multi(toks, sa)
+        singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(t)])
+        assert np.array_equal(lv.view(np.uint32), singles.view(np.uint32)), t
+        assert relerr(lv, om.forward_multi(toks, so)) <= 1e-3, t
+
+
 @pytest.mark.parametrize("d,hc,rows", [(256, 2, False), (512, 4, False), (1024, 2, False), (512, 4, True)])
 def test_matrix_core_hyper_connection_mixes_windows_equal_steps_and_the_oracle(ctx, monkeypatch, d, hc, rows):
     # IQ3_S hyper-connection matrices with a low rank of 256: the mixes run on the matrix cores (slices of 256 or 512
