@@ -20,6 +20,8 @@ struct Layer {
 
 }  // namespace
 
+struct PromptPipe; void prompt_pipe_free(PromptPipe* P);
+
 struct pyre_model {
   pyre_ctx* ctx = nullptr; pyre_model_cfg c{};
   std::vector<Layer> layers; HcDev head{}; QMatDev embd{}, out{};
@@ -33,6 +35,7 @@ struct pyre_model {
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
   PleCfg plc{}; QMatDev ple_tab{}; PleWork pw{}; int n_ple = 0, ple_ring = 0;      // PLE: hash parameters, the token table, window workspace, ring rows per layer
   uint16_t* aop = nullptr;      // the f16 operand a producer kernel leaves for the matrix-core GEMV that follows it (one at a time: the launches are stream-ordered)
+  PromptPipe* pipe = nullptr;      // further window workspaces and streams for a long prompt (prompt_pipe), made at the first one
 };
 
 struct pyre_state {
@@ -42,6 +45,7 @@ struct pyre_state {
   std::vector<float*> proj_saved;                                // per DeltaNet layer [8][pw_lin]: inputs of the last window
   std::vector<KvDev> kv; std::vector<int> packed; AttnWork aw{};
   std::vector<QsaBuf> qsa; QsaWork qw{};                          // indexer keys per attention layer; selection workspace
+  void* pipe_mem = nullptr; std::vector<AttnWork> aw_more; std::vector<QsaWork> qw_more;      // one more attention / selection workspace per further prompt stream
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
   uint32_t* tokens_dev = nullptr; std::vector<float*> ple_ring;     // PLE models: the token history by position; per PLE layer the ring of normalised rows
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
@@ -122,6 +126,32 @@ size_t al256(size_t n) { return (n + 255) & ~(size_t)255; }
 }  // namespace
 
 extern "C" {
+
+// The activations of one window of up to 8 tokens: everything a window's launches write apart from the state.
+static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
+  const pyre_model_cfg& c = m->c;
+  const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
+  HcDev hmax = m->head; hmax.lr = c.hc_lr;
+  MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
+  size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
+  int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));
+  const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
+  const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
+  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(ple_b) + 4096;
+  PYRE_HIP(ctx, hipMalloc(&m->work, total));
+  uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
+  pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
+  m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
+  m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
+  m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
+  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
+  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
+  if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
+  PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
+  if (kmax_out) *kmax_out = kmax;
+  return PYRE_OK;
+}
 
 int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tensor* lt, const pyre_tensor* gl, pyre_model** out) {
   if (!ctx || !cfg || !lt || !gl || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_model_create: null argument");
@@ -218,26 +248,8 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
   if (m->out.rows != c.vocab || m->out.cols != c.d) return B.fail(PYRE_E_SHAPE, "output shape");
   tok_bytes += (size_t)c.d / m->embd.gel * m->embd.gbytes;
   m->token_weight_bytes = tok_bytes;
-  // window workspace
-  const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
-  HcDev hmax = m->head; hmax.lr = c.hc_lr;
-  MoeDev& m0 = m->layers[0].moe; size_t moe_b = 0; for (auto& L : m->layers) { size_t b = pyre_moe_work_bytes(L.moe); if (b > moe_b) moe_b = b; }
-  size_t rp_b = 4; for (auto& L : m->layers) if (pyre_hc_route_ok(L.hcf, L.moe.router)) rp_b = std::max(rp_b, (size_t)4 * 8 * (c.d / 64) * L.moe.router.tiles * 64);      // router K-slice sums
-  int kmax = c.d; for (auto& L : m->layers) kmax = std::max(kmax, std::max(L.proj.cols, L.outp.cols));
-  const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
-  const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
-  size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(ple_b) + 4096;
-  PYRE_HIP(ctx, hipMalloc(&m->work, total));
-  uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
-  pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
-  m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
-  m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
-  m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
-  m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
-  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
-  if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
-  PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
+  int kmax = 0;
+  if ((rc = model_alloc_work(ctx, m, &kmax))) return rc;
   { uint4* op; float* ainv;      // and the context's operand buffer for a GEMV whose producer leaves f32 only, so that no step allocates
     if ((rc = pyre_gemm_m_scratch(ctx, (kmax + 255) / 256 * 256, &op, &ainv))) return rc; }
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -246,6 +258,7 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
 
 void pyre_model_destroy(pyre_model* m) {
   if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
+  prompt_pipe_free(m->pipe);
   for (auto q : m->owned) pyre_qmat_destroy(q); for (auto b : m->bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work); if (m->toks) (void)hipFree(m->toks);
   delete m;
 }
@@ -274,7 +287,7 @@ int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_stat
   int rc = pyre_state_reset(ctx, s); if (rc) { (void)hipFree(s->mem); return rc; }
   *out = S.release(); return PYRE_OK;
 }
-void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec); (void)hipFree(s->mem); if (s->mtp_mem) (void)hipFree(s->mtp_mem); delete s; }
+void pyre_state_destroy(pyre_state* s) { if (!s) return; (void)hipStreamSynchronize(s->ctx->stream); if (s->graph_exec) (void)hipGraphExecDestroy(s->graph_exec); (void)hipFree(s->mem); if (s->mtp_mem) (void)hipFree(s->mtp_mem); if (s->pipe_mem) (void)hipFree(s->pipe_mem); delete s; }
 int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
   if (!ctx || !s) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_reset: null argument");
   const pyre_model_cfg& c = s->m->c; size_t cs = (size_t)(c.conv_k - 1) * s->m->ch * 4, ss = (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4;
@@ -394,6 +407,75 @@ int pyre_state_read_kv(pyre_ctx* ctx, pyre_state* s, int ai, float* k_host, floa
 
 namespace {
 
+}  // namespace
+
+// A long prompt runs its windows on several streams at once: window w+1 may work on layer l as soon as window w has left
+// that layer's state (an event per layer), each stream with a window workspace of its own -- a shallow copy of the model
+// whose activations are separate -- and an attention workspace of its own in the state.  The launches of a window of 8
+// tokens leave most of the chip idle most of the time; two or three windows in flight fill it.  Arithmetic and order per
+// window are unchanged, so the state and the logits are bit for bit those of one stream.
+struct PromptPipe {
+  std::vector<pyre_ctx*> ctx;                  // contexts of the further streams
+  std::vector<pyre_model*> mdl;                // the model's shallow copies, one per further stream
+  std::vector<std::vector<hipEvent_t>> ev;     // [set][layer]; set 0 is the model's own stream
+  std::vector<hipEvent_t> done;                // [set] end of the set's last window
+  hipEvent_t start = nullptr;
+  uint32_t* ids = nullptr; size_t ids_cap = 0; // the call's token ids on the device
+};
+static int prompt_streams() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_STREAMS"); int v = e && *e ? atoi(e) : 3; return v < 1 ? 1 : (v > 4 ? 4 : v); }(); return k; }
+void prompt_pipe_free(PromptPipe* P) {
+  if (!P) return;
+  for (auto* mc : P->mdl) if (mc) { (void)hipStreamSynchronize(mc->ctx->stream); if (mc->work) (void)hipFree(mc->work); delete mc; }
+  for (auto* cx : P->ctx) if (cx) pyre_ctx_destroy(cx);
+  for (auto& v : P->ev) for (auto e : v) if (e) (void)hipEventDestroy(e);
+  for (auto e : P->done) if (e) (void)hipEventDestroy(e);
+  if (P->start) (void)hipEventDestroy(P->start);
+  if (P->ids) (void)hipFree(P->ids);
+  delete P;
+}
+static int prompt_pipe_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe** out) {
+  pyre_model* mm = const_cast<pyre_model*>(m);          // the workspaces are the model's, like its own activations
+  if (mm->pipe) { *out = mm->pipe; return PYRE_OK; }
+  const int k = prompt_streams();
+  std::unique_ptr<PromptPipe, void (*)(PromptPipe*)> P(new PromptPipe(), prompt_pipe_free);
+  for (int i = 1; i < k; ++i) {
+    pyre_ctx* cx = nullptr; int rc = pyre_ctx_create(ctx->device, &cx); if (rc) return pyre_fail(ctx, rc, "prompt streams: %s", pyre_last_error(nullptr));
+    P->ctx.push_back(cx);
+    pyre_model* mc = new pyre_model(*m); mc->ctx = cx; mc->owned.clear(); mc->bufs.clear(); mc->work = nullptr; mc->toks = nullptr; mc->toks_cap = 0; mc->pipe = nullptr;
+    P->mdl.push_back(mc);
+    int kmax = 0; rc = model_alloc_work(cx, mc, &kmax);
+    if (!rc) { uint4* op; float* ainv; rc = pyre_gemm_m_scratch(cx, (kmax + 255) / 256 * 256, &op, &ainv); }
+    if (rc) return pyre_fail(ctx, rc, "prompt streams: %s", cx->err.c_str());
+    PYRE_HIP(ctx, hipStreamSynchronize(cx->stream));
+  }
+  P->ev.resize(k); P->done.resize(k, nullptr);
+  for (int i = 0; i < k; ++i) {
+    P->ev[i].resize(m->c.n_layers, nullptr);
+    for (auto& e : P->ev[i]) PYRE_HIP(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    PYRE_HIP(ctx, hipEventCreateWithFlags(&P->done[i], hipEventDisableTiming));
+  }
+  PYRE_HIP(ctx, hipEventCreateWithFlags(&P->start, hipEventDisableTiming));
+  mm->pipe = P.release(); *out = mm->pipe; return PYRE_OK;
+}
+// the state's further attention / selection workspaces (one per further stream)
+static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int k) {
+  if ((int)s->aw_more.size() >= k - 1) return PYRE_OK;
+  const pyre_model_cfg& c = m->c;
+  AttnDev a0{nullptr, nullptr, nullptr, c.n_head, c.n_kv, c.hd, c.n_rot, c.kv_bits, c.kv_recent, c.eps};
+  QsaDev q0{nullptr, nullptr, m->has_idx ? c.idx_nh : 0, c.idx_hd, c.idx_ratio < 1 ? 1 : c.idx_ratio, c.idx_budget};
+  const size_t awb = al256(pyre_attn_work_bytes(a0, s->cap)), qwb = al256(pyre_qsa_work_bytes(q0, s->cap));
+  if (s->pipe_mem) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); (void)hipFree(s->pipe_mem); s->pipe_mem = nullptr; s->aw_more.clear(); s->qw_more.clear(); }
+  PYRE_HIP(ctx, hipMalloc(&s->pipe_mem, (size_t)(k - 1) * (awb + qwb) + 256));
+  uint8_t* p = (uint8_t*)s->pipe_mem;
+  for (int i = 1; i < k; ++i) {
+    AttnWork aw{}; pyre_attn_work_carve(a0, s->cap, p, &aw); p += awb; s->aw_more.push_back(aw);
+    QsaWork qw{}; if (m->has_idx) pyre_qsa_work_carve(q0, s->cap, p, &qw); p += qwb; s->qw_more.push_back(qw);
+  }
+  return PYRE_OK;
+}
+
+namespace {
+
 struct WinOpt {
   int head_tokens = 1;          // 0 = no logits, 1 = last token only, t = every token (rows 0..t-1 of m->logits)
   bool greedy = false;          // t == 1: the head GEMV also leaves per-tile maxima in m->best
@@ -403,6 +485,9 @@ struct WinOpt {
                                 // recurrent state is updated in place and no host-side bookkeeping is touched
   bool inplace = false;         // update the recurrent state in its current buffer (no pre-window copy for spec_keep)
   int keep_from = 0;            // with a drafter attached: the final residual streams of tokens keep_from .. t-1 go to the state's ring
+  // a prompt window that shares the GPU with its neighbours (prompt_pipe): its ids, the attention / selection workspace
+  // it uses instead of the state's, and per layer the event it waits for (the previous window has left the layer) and records
+  const uint32_t* ids_dev = nullptr; const AttnWork* aw = nullptr; const QsaWork* qw = nullptr; const hipEvent_t* wait_ev = nullptr; const hipEvent_t* rec_ev = nullptr;
 };
 
 // rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
@@ -419,7 +504,8 @@ bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) &&
 int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev, s->tokens_dev) : pyre_row_launch(ctx, m->embd, m->ids, t, m->emb, d); if (rc) return rc;
+  const uint32_t* ids = o.ids_dev ? o.ids_dev : m->ids; const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
+  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev, s->tokens_dev) : pyre_row_launch(ctx, m->embd, ids, t, m->emb, d); if (rc) return rc;
   // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
   // leaves the updated streams in the other
   const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
@@ -430,7 +516,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   const bool moe_groups = [] { const char* e = getenv("PYRE_MOE_GROUPS"); return !(e && *e && atoi(e) == 0); }();      // 0: windows leave the unreduced terms as a single token does
   const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
   // the window's tokens join the history (PLE models and states with a drafter keep one)
-  if (s->tokens_dev && !o.from_best) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, m->ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));
+  if (s->tokens_dev && !o.from_best && !o.ids_dev) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));      // (a prompt on several streams has stored the whole call's ids already)
   if (m->n_ple > 0) {      // every position's n-gram rows are fetched once for all PLE layers
     if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
   }
@@ -440,6 +526,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   auto opw = [&](const QMatDev& q) -> uint16_t* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? m->aop : nullptr; };
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
+    if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
     if (L.ple) {      // resolves the pending residual update itself and leaves plain streams
       PleDev pd = L.pld; pd.ring = s->ple_ring[L.ple_index]; pd.mask = m->ple_ring - 1;
       if ((rc = pyre_ple_launch(ctx, m->plc, pd, m->pw, d, hc, c.eps, xin, in_ss, in_ts, xout, comb_out, comb_moe, comb_inj, start, o.step_dev, t))) return rc;
@@ -447,11 +534,13 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     }
     if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.proj)))) return rc;
     advance(); comb_np = 1;
+    // the layer's state (cache, recurrent state, saved projection) is the previous window's until that window has left it
+    if (o.wait_ev) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.proj)))) return rc;
-      if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], s->qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
-      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], s->aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &s->qw : nullptr, opw(L.outp)))) return rc;
+      if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
+      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr, opw(L.outp)))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
@@ -459,6 +548,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, opw(L.outp)))) return rc;
       s->cur[li] = nb;
     }
+    if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
     if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc; }
     else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc;
@@ -517,13 +607,37 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: %d + %d tokens exceed the state's capacity %d", s->len, n, s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   s->last_window = 0;
-  for (int i = 0; i < n; i += 8) {
+  const int nwin = (n + 7) / 8, K = prompt_streams();
+  PromptPipe* P = nullptr;
+  if (K > 1 && nwin >= 2 * K && !ctx->prof_on) {      // a long prompt: K windows in flight (the per-class timing wants one stream)
+    if ((rc = prompt_pipe_get(ctx, m, &P)) || (rc = prompt_pipe_state(ctx, m, s, K))) return rc;
+    if (P->ids_cap < (size_t)n) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); if (P->ids) (void)hipFree(P->ids); P->ids = nullptr; P->ids_cap = 0;
+      PYRE_HIP(ctx, hipMalloc((void**)&P->ids, (size_t)n * 4)); P->ids_cap = (size_t)n; }
+    PYRE_HIP(ctx, hipMemcpyAsync(P->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
+    if (s->tokens_dev) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + s->len, P->ids, (size_t)n * 4, hipMemcpyDeviceToDevice, ctx->stream));      // the history every window's n-gram rows read
+    PYRE_HIP(ctx, hipEventRecord(P->start, ctx->stream));      // the other streams begin after everything already queued here
+    for (auto* cx : P->ctx) PYRE_HIP(ctx, hipStreamWaitEvent(cx->stream, P->start, 0));
+  }
+  int prev = -1;
+  for (int i = 0, w = 0; i < n; i += 8, ++w) {
     int t = n - i < 8 ? n - i : 8; bool last = i + t >= n;
-    PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
     WinOpt o; o.head_tokens = last && logits_host ? 1 : 0;
     if (s->mtp) { const int k0 = n - mtp_window_of(s->mtp) - i; o.keep_from = k0 < 0 ? 0 : k0; }      // the last `window` tokens of a call (qwen4exp_gguf.rs:2148-2150)
-    if ((rc = run_window(ctx, m, s, t, o))) return rc;
+    if (!P) {
+      PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
+      if ((rc = run_window(ctx, m, s, t, o))) return rc;
+      continue;
+    }
+    const int set = (nwin - 1 - w) % K;          // the last window runs on the model's own stream and workspace: its logits are the call's
+    pyre_ctx* cx = set ? P->ctx[set - 1] : ctx; const pyre_model* mx = set ? P->mdl[set - 1] : m;
+    o.ids_dev = P->ids + i; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
+    o.wait_ev = prev >= 0 ? P->ev[prev].data() : nullptr; o.rec_ev = P->ev[set].data();
+    rc = run_window(cx, mx, s, t, o);
+    if (!rc && hipEventRecord(P->done[set], cx->stream) != hipSuccess) rc = pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
+    if (rc) { if (cx != ctx) pyre_fail(ctx, rc, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return rc; }
+    prev = set;
   }
+  if (P) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, P->done[k], 0));      // everything the other streams did precedes what follows here
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }

@@ -212,6 +212,37 @@ def test_verify_window_equals_single_steps_and_rollback(ctx):
         gm.spec_keep(sa, 5, 2)                                        # not armed any more
 
 
+@pytest.mark.parametrize("kind", ["plain", "iq3s_mixes", "ple", "indexer"])
+def test_long_prompt_on_several_streams_equals_short_calls_on_one(ctx, kind):
+    # A call of 2 * 3 windows or more runs its windows on three streams, a window entering a layer when the previous one has
+    # left that layer's state; shorter calls run on the model's own stream.  Same logits, recurrent state, caches and
+    # continuation, bit for bit (250 tokens: the 4-bit boundary moves several times, ragged last window).
+    if kind == "plain": c = small_cfg()
+    elif kind == "iq3s_mixes": c = small_cfg(hc_lr=256, qtype=synth.IQ3_S, hc_type=synth.IQ3_S, n_exp=16, top_k=10)
+    elif kind == "ple": c = mg.with_ple(small_cfg(), layers=(0, 2, 3), ngram=3, per_gram=2, conv_k=3, dim=64, eos=7)
+    else: c = idx_cfg(); c.ctx = 512
+    hw = mg.build_host(c, seed=41)
+    gm = lib.Model(ctx, c, hw.layers, hw.globals_)
+    g = np.random.Generator(np.random.PCG64(42))
+    prompt = g.integers(0, c.vocab, 250, dtype=np.uint32)
+    sa, sb = gm.new_state(320), gm.new_state(320)
+    la = gm.forward(prompt, sa)                                     # 32 windows: three in flight
+    for i in range(0, 250, 40): lb = gm.forward(prompt[i:i + 40], sb)      # 5 windows a call: one stream
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    n_lin = sum(1 for il in range(c.n_layers) if not c.full(il))
+    for li in range(n_lin):
+        ca, xa = sa.gdn(li); cb, xb = sb.gdn(li)
+        assert np.array_equal(ca.view(np.uint32), cb.view(np.uint32)) and np.array_equal(xa.view(np.uint32), xb.view(np.uint32)), li
+    for ai in range(c.n_layers - n_lin):
+        ka, va = sa.kv(ai); kb, vb = sb.kv(ai)
+        assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32)) and np.array_equal(va.view(np.uint32), vb.view(np.uint32)), ai
+    more = g.integers(0, c.vocab, 60, dtype=np.uint32)              # and again on top of the state a long call left
+    la = gm.forward(more, sa)
+    for i in range(0, 60, 30): lb = gm.forward(more[i:i + 30], sb)
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)) and len(sa) == len(sb) == 310
+    assert np.array_equal(gm.decode_greedy_dev(sa, int(np.argmax(la)), 12), gm.decode_greedy_dev(sb, int(np.argmax(lb)), 12))
+
+
 @pytest.mark.parametrize("n_exp,top_k,ff_sh,qtype", [(32, 13, 512, synth.IQ3_S), (16, 3, 0, synth.IQ3_S), (16, 2, 0, synth.IQ3_S), (16, 10, 0, synth.Q4_K), (16, 11, 512, synth.Q8_0)])
 def test_window_ffn_output_as_group_sums_equals_single_steps_and_the_oracle(ctx, n_exp, top_k, ff_sh, qtype):
     # With IQ3_S hyper-connection matrices a window's FFN output reaches the next mix as four group sums a token (groups of

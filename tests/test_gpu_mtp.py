@@ -120,6 +120,20 @@ def test_window_shorter_than_the_prompt_and_than_a_verify_window(ctx):
         o.close()
 
 
+def test_drafter_after_a_long_prompt_on_several_streams(ctx):
+    # 123 tokens = 16 windows, three in flight on three streams; the last 16 residual rows come from the last three windows
+    # (the last one ragged), i.e. from all three streams; the drafts are the oracle's
+    c = small_cfg(qtype=synth.IQ3_S, hc_type=synth.IQ3_S, hc_lr=256)
+    gm, gd, om, od = pair(ctx, c, 65, window=16)
+    gs, os_ = gm.new_state(192), om.new_state(); gd.attach(gs); od.attach(os_)
+    prompt = np.random.Generator(np.random.PCG64(66)).integers(0, c.vocab, 123, dtype=np.uint32)
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-3 and int(np.argmax(lg)) == int(np.argmax(lo))
+    same_drafts(gd, gs, od, os_, int(np.argmax(lo)), 3)
+    for o in (gd, gs, gm):
+        o.close()
+
+
 def test_zero_head_closed_form_and_the_probability_gate(ctx):
     c = small_cfg(qtype=synth.IQ3_S, hc_type=synth.BF16)
     gm, gd, om, od = pair(ctx, c, 71, window=16, zero=(mg.MTP_HEAD,))
