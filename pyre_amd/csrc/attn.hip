@@ -476,15 +476,16 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
 
 // grid (nh, t, HD/64), 256 threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
 // Thread (grp, dim) adds the chunks grp, grp+4, ... in ascending order; the four groups are then added in order.
-// A workgroup owns 64 dimensions of a head and goes through the chunks 256 at a time: the 64 partial outputs a thread
+// A workgroup owns 64 dimensions of a head and goes through the chunks 320 at a time: the 80 partial outputs a thread
 // needs of such a tile do not depend on the maximum, so the first tile's are fetched at the start, together with the
-// (max, sum) pairs; thread c of the tile then leaves exp(max_c - M) and sum_c in shared memory for everybody.  Up to
-// 256 chunks (32 768 positions) the whole merge is one memory round trip.
+// (max, sum) pairs; thread c of the tile (and again thread c - 256 for the last 64) then leaves exp(max_c - M) and sum_c
+// in shared memory for everybody.  Up to 320 chunks (40 960 positions) the whole merge is one memory round trip -- the
+// step after a 32 768-token prompt has 257 chunks.
 template <int HD>
 __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                       int max_chunks, float* __restrict__ out, const int* __restrict__ pcount, uint16_t* __restrict__ aop, int aop_rows) {
-  constexpr int B = 64;
-  __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[256], ls[256];
+  constexpr int CB = 320, B = CB / 4;
+  __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[CB], ls[CB];
   if (posp) start = *posp;
   const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid >> 6, dd = blockIdx.z * 64 + (tid & 63);
   int n = start + ti + 1; if (pcount && pcount[ti] >= 0) n = pcount[ti];        // a position list: its entries are what the chunks covered
@@ -494,7 +495,9 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   float pv[B];
 #pragma unroll
   for (int i = 0; i < B; ++i) pv[i] = nc > 0 ? po[(size_t)min(grp + 4 * i, nc - 1) * HD + dd] : 0.0f;
-  float m0 = -INFINITY, l0 = 0.0f; if (tid < nc) { m0 = ml[2 * tid]; l0 = ml[2 * tid + 1]; }
+  float m0 = -INFINITY, l0 = 0.0f, m1 = -INFINITY, l1 = 0.0f;          // the tile's chunks tid and (threads below 64) 256 + tid
+  if (tid < nc) { m0 = ml[2 * tid]; l0 = ml[2 * tid + 1]; }
+  if (tid < CB - 256 && 256 + tid < nc) { m1 = ml[2 * (256 + tid)]; l1 = ml[2 * (256 + tid) + 1]; }
   float M = m0; for (int c = tid + 256; c < nc; c += 256) M = fmaxf(M, ml[2 * c]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
@@ -502,14 +505,16 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   __syncthreads();
   M = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   float L = 0.0f, o = 0.0f;
-  for (int cb = 0; cb < nc; cb += 256) {
+  for (int cb = 0; cb < nc; cb += CB) {
     if (cb > 0) {
       __syncthreads();
 #pragma unroll
       for (int i = 0; i < B; ++i) pv[i] = po[(size_t)min(cb + grp + 4 * i, nc - 1) * HD + dd];
       m0 = -INFINITY; l0 = 0.0f; if (cb + tid < nc) { m0 = ml[2 * (cb + tid)]; l0 = ml[2 * (cb + tid) + 1]; }
+      m1 = -INFINITY; l1 = 0.0f; if (tid < CB - 256 && cb + 256 + tid < nc) { m1 = ml[2 * (cb + 256 + tid)]; l1 = ml[2 * (cb + 256 + tid) + 1]; }
     }
     fs[tid] = expf(m0 - M); ls[tid] = l0;
+    if (tid < CB - 256) { fs[256 + tid] = expf(m1 - M); ls[256 + tid] = l1; }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < B; ++i) if (cb + grp + 4 * i < nc) { const float f = fs[grp + 4 * i]; L = fmaf(ls[grp + 4 * i], f, L); o = fmaf(pv[i], f, o); }
