@@ -194,6 +194,16 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
         for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * NC + li] = D[pt][r];
     }
   }
+  // f32 values: requested now, while the scores are being normalised (the keys' registers are free again; __syncthreads
+  // waits for outstanding loads, so the round trip is paid at the first barrier of phase 2 instead of after the last)
+  float4 vf4[16];
+  if (active && !packed) {
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);          // positions past the view carry weight zero; their address is clamped
+      vf4[s] = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+    }
+  }
   __syncthreads();
   // ---- phase 2: this thread's position is pw*64 + lane, its columns are dq, dq + 4, dq + 8, dq + 12
   const int pos = pw * 64 + lane;
@@ -244,20 +254,15 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(nib_val(hw, dt) * vsc[s], B[s], D[dt], 0, 0, 0);
         }
-      } else {                  // positions past the view carry weight zero; their address is clamped
-        float A[4][16];
-#pragma unroll
-        for (int s = 0; s < 16; ++s) {
-          const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);
-          float4 v = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
-          A[0][s] = v.x; A[1][s] = v.y; A[2][s] = v.z; A[3][s] = v.w;
-        }
+      } else {
 #pragma unroll
         for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
 #pragma unroll
-        for (int s = 0; s < 16; ++s)
+        for (int s = 0; s < 16; ++s) {
+          const float A[4] = {vf4[s].x, vf4[s].y, vf4[s].z, vf4[s].w};
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt][s], B[s], D[dt], 0, 0, 0);
+          for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt], B[s], D[dt], 0, 0, 0);
+        }
       }
     }
     if (li < ncol) {
