@@ -421,7 +421,10 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   if (ib < n_lo) put_lo(tb, rb, pvb);
   for (int idx = tid + 2 * nthr; idx < n_lo; idx += nthr) { const int t = idx / lr, i = idx - t * lr; hc_load_slices16<T>(pva, part, true, ksplit, t, r64, i); put_lo(t, i, pva); }
   if (own_stream && blockIdx.x == 0) inj[stt * hc + sq] = has_inject ? hc_slice_sum16(pvi, sls + stt * 16, ksplit) / (float)hc : 0.0f;
-  if (ROUTE && R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
+  // the router's tiles go round the waves; with waves to spare (16 waves, 8 tiles) wave w and wave w + tiles share tile w and split the tokens
+  const int rnt = ROUTE ? max(1, (int)router.tiles) : 1, rsets = max(1, nw / rnt), rtile = wave % rnt, rset = wave / rnt;
+  const bool rwave = ROUTE && rset < rsets;
+  if (rwave && R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
   lds_barrier();
   for (int j = tid; j < n_lo; j += nthr) {
     const int t2 = j / lr, k = j - t2 * lr; float upf, dn; hc_scale_of(__uint_as_float(lmax[t2]), &upf, &dn);
@@ -440,7 +443,7 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
     } }
   if (2 * q < T) red[((size_t)s * T + 2 * q) * 64 + g * 16 + (lane & 15)] = tot[0][0] + tot[0][1] * (1.0f / 2048.0f);
   if (2 * q + 1 < T) red[((size_t)s * T + 2 * q + 1) * 64 + g * 16 + (lane & 15)] = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
-  if (ROUTE && !R_EARLY && wave < router.tiles) rraw = unit_load<RFX>(router, wave, blockIdx.x, lane);
+  if (rwave && !R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
   lds_barrier();
   if (tid < T * 64) {          // the gated, normalised streams of the column, streams ascending from zero (:1380)
     const int t2 = tid >> 6, l = lane, col = blockIdx.x * 64 + l; float mx = 0.0f;
@@ -454,10 +457,10 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   if (ROUTE) {
     lds_barrier();
     const size_t rr64 = (size_t)router.tiles * 64;
-    for (int tile = wave; tile < router.tiles; tile += nw) {
-      if (tile != wave) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
+    for (int tile = rtile; rwave && tile < rnt; tile += nw) {          // (more tiles than waves: one set, the tiles in turns)
+      if (tile != rtile) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
 #pragma unroll 1
-      for (int t2 = 0; t2 < T; ++t2) {
+      for (int t2 = rset; t2 < T; t2 += rsets) {
         float ra[1] = {0.0f};
         unit_fma<RFX, 1>(router, rraw, blockIdx.x, lds2, lane, lo + t2 * 64, 0, ra);
         rpart[((size_t)blockIdx.x * T + t2) * rr64 + (size_t)tile * 64 + lane] = ra[0];
