@@ -423,7 +423,7 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   if (own_stream && blockIdx.x == 0) inj[stt * hc + sq] = has_inject ? hc_slice_sum16(pvi, sls + stt * 16, ksplit) / (float)hc : 0.0f;
   // the router's tiles go round the waves; with waves to spare (16 waves, 8 tiles) wave w and wave w + tiles share tile w and split the tokens
   const int rnt = ROUTE ? max(1, (int)router.tiles) : 1, rsets = max(1, nw / rnt), rtile = wave % rnt, rset = wave / rnt;
-  const bool rwave = ROUTE && rset < rsets;
+  const bool rwave = ROUTE && rset < rsets && rset < T;          // (a set without a token fetches nothing)
   if (rwave && R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
   lds_barrier();
   for (int j = tid; j < n_lo; j += nthr) {
