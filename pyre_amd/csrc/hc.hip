@@ -422,8 +422,8 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   for (int idx = tid + 2 * nthr; idx < n_lo; idx += nthr) { const int t = idx / lr, i = idx - t * lr; hc_load_slices16<T>(pva, part, true, ksplit, t, r64, i); put_lo(t, i, pva); }
   if (own_stream && blockIdx.x == 0) inj[stt * hc + sq] = has_inject ? hc_slice_sum16(pvi, sls + stt * 16, ksplit) / (float)hc : 0.0f;
   // the router's tiles go round the waves; with waves to spare (16 waves, 8 tiles) wave w and wave w + tiles share tile w and split the tokens
-  const int rnt = ROUTE ? max(1, (int)router.tiles) : 1, rsets = max(1, nw / rnt), rtile = wave % rnt, rset = wave / rnt;
-  const bool rwave = ROUTE && rset < rsets && rset < T;          // (a set without a token fetches nothing)
+  const int rnt = ROUTE ? max(1, (int)router.tiles) : 1, rsets = T == 1 ? 1 : max(1, nw / rnt), rtile = T == 1 ? wave : wave % rnt, rset = T == 1 ? 0 : wave / rnt;
+  const bool rwave = ROUTE && (T == 1 ? wave < rnt : (rset < rsets && rset < T));          // (a set without a token fetches nothing; a single token: one set, no division)
   if (rwave && R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
   lds_barrier();
   for (int j = tid; j < n_lo; j += nthr) {
