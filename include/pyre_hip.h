@@ -68,8 +68,9 @@ size_t pyre_qmat_gguf_bytes(const pyre_qmat* m);
  * reference's counterpart is the size of the repacked Burn tensor (repack_to_burn, src/model/qn_gpu.rs:54). */
 size_t pyre_qmat_device_bytes(const pyre_qmat* m);
 /* The same per layout: 0 = the lane-per-row planes (every type; what pyre_qmatmul_f32 streams), 1 = the matrix-core layout
- * (IQ3_S only, 0 otherwise; what pyre_qmatmul streams for IQ3_S).  No counterpart in the reference. */
-size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int matrix_core_layout);
+ * (IQ3_S only, 0 otherwise; what pyre_qmatmul streams for IQ3_S windows of 2..8 tokens), 2 = IQ3_S at the file's bits per
+ * weight (112 bytes per 256 weights; what pyre_qmatmul streams for one token).  No counterpart in the reference. */
+size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int layout);
 /* QMat::to_f32 (gguf_q.rs:212): all rows*cols values, bit-exact with gguf_q::dequant (gguf_q.rs:67-166). */
 int    pyre_qmat_dequant(pyre_ctx* ctx, const pyre_qmat* m, float* out_host);
 int    pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev);
@@ -77,16 +78,24 @@ int    pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev);
 int    pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host);
 /* QMat::matmul (gguf_q.rs:216-217): y[ti*rows + r] = sum_c W[r,c] * x[ti*cols + c], t in 1..8.
  * The result for a token does not depend on t (same operations in the same order), which is what lets a
- * multi-token verify pass equal one-token decode (qwen4exp_gguf.rs:2357-2360). */
+ * multi-token verify pass equal one-token decode (qwen4exp_gguf.rs:2357-2360) -- with one exception: a single token of
+ * an IQ3_S matrix takes a kernel of its own (below), so t = 1 and t >= 2 agree to rounding (both within 1e-5 of the exact
+ * product), not bit for bit; PYRE_QMATMUL_NATIVE=0 in the environment sends t = 1 through the window's kernel as well. */
 int    pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
 int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
-/* IQ3_S matrices take pyre_qmatmul through the f16 matrix cores, for every t with one kernel (the reference's verify
+/* One token of an IQ3_S matrix (t = 1; the reference's GPU decode of this type, src/model/qn_cube.rs:3354-3382): the
+ * matrix is streamed at the file's bits per weight -- per four weights the 9-bit codebook index and four sign bits, the
+ * codebook with the signs folded in (8192 x four signed bytes) in shared memory -- and the activations are block fixed
+ * point, three signed bytes per value with one power of two per 64 columns (|x - su q| <= 2^-22 of the 64 columns'
+ * largest magnitude), so that four weights meet their columns in v_dot4_i32_i8; the integer sums are exact, the scales
+ * d * (1 + 2 s) and the accumulation are f32.
+ * Windows of 2..8 tokens of an IQ3_S matrix go through the f16 matrix cores with one kernel (the reference's verify
  * kernels, src/model/qn_cube.rs:17,6454, and lcm_dense, qwen4exp_gguf.rs:2641-2737, are this product with t > 1): each
  * 256-column stretch of a token is scaled by its own power of two and every value is written as two f16 halves (22
  * significant bits; values more than 2^14 / 6e-5 below the largest magnitude of their stretch lose resolution), the 4-bit
  * codes times their sub-block scales are exact in f16, products are exact and summed in f32.  A non-finite activation
- * makes every output of its token NaN.  An IQ3_S matrix created through pyre_qmat_create* is held in two layouts (one per
- * kernel; pyre_qmat_device_bytes counts both).  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the
+ * makes every output of its token NaN.  An IQ3_S matrix created through pyre_qmat_create* is held in three layouts (one per
+ * kernel; pyre_qmat_device_bytes counts them all, pyre_qmat_layout_bytes each).  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the
  * model's expert matrices use (QMat::matmul's own arithmetic, gguf_q.rs:169-197,233-241: f32 products, f32 accumulation);
  * for every other type the two are the same code. */
 int    pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
@@ -102,11 +111,6 @@ int    pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
  * All contexts on one GPU share that GPU's array: calls that overlap in time on one GPU (two contexts' streams) race. */
 #define PYRE_QMATMUL_STATIC_MAX_COLS 32768
 int    pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
-/* pyre_qmatmul restricted to IQ3_S (PYRE_E_TYPE otherwise): kept for callers written against a separate verify-window
- * entry point; t in 1..8, bit-identical to pyre_qmatmul. */
-int    pyre_qmatmul_mfma(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
-int    pyre_qmatmul_mfma_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev);
-
 /* ---- synthetic tensors (no counterpart in the reference's API; its micro-benchmarks build the same kind of data
  * inline, src/model/qdot.rs:823-859, src/model/qn_cube.rs:7216-7249) ---------------------------------------------
  * Fills n_blocks raw GGUF blocks on the device: counter-based random payload bytes, every f16 scale field drawn

@@ -73,7 +73,7 @@ int pyre_ctx_create(int device, pyre_ctx** out) {
       (e = hipMalloc((void**)&ctx->d_iq3s, 512 * 4)) != hipSuccess || (e = hipMalloc((void**)&ctx->d_iq2xs, 512 * 8)) != hipSuccess ||
       (e = hipMemcpy(ctx->d_iq3s, g3.data(), 512 * 4, hipMemcpyHostToDevice)) != hipSuccess || (e = hipMemcpy(ctx->d_iq2xs, g2.data(), 512 * 8, hipMemcpyHostToDevice)) != hipSuccess) {
     int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: codebook upload: %s", hipGetErrorString(e)); pyre_ctx_destroy(ctx); return rc; }
-  if (pyre_static_init(ctx) != PYRE_OK) { int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: %s", ctx->err.c_str()); pyre_ctx_destroy(ctx); return rc; }
+  if (pyre_gemv_n_table(ctx) != PYRE_OK || pyre_static_init(ctx) != PYRE_OK) { int rc = pyre_fail(nullptr, PYRE_E_HIP, "pyre_ctx_create: %s", ctx->err.c_str()); pyre_ctx_destroy(ctx); return rc; }
   *out = ctx; return PYRE_OK;
 }
 
@@ -90,6 +90,8 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->d_cb) (void)hipFree(ctx->d_cb);
   if (ctx->aop_buf) (void)hipFree(ctx->aop_buf);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
+  if (ctx->d_iq3s_sgn) (void)hipFree(ctx->d_iq3s_sgn);
+  if (ctx->dgn_buf) (void)hipFree(ctx->dgn_buf);
   for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto e : ctx->prof_pool) (void)hipEventDestroy(e);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);

@@ -275,6 +275,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   constexpr int NW = 4 * CS;
   __shared__ __align__(16) uint16_t ah[CS * 32 * 16 * 8];
   __shared__ float wsum[NW][8], wmax[NW][8], hsum[4][2][64];
+  PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m); args_now(x_in, in_ss, in_ts, x_out, comb_out, mo.partial, mo.sel_w, mo.sg, mo.d, mo.k, comb_inj, norm, d, hc, ssq, part);
   const int tile = blockIdx.x, ks = blockIdx.y, tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = wave & 3, p = wave >> 2;
@@ -300,7 +301,8 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   }
 #pragma unroll
   for (int r = 2 * T; r < 16; ++r) ah[((size_t)(tid >> 3) * 16 + r) * 8 + (tid & 7)] = 0;      // rows no token of the window owns
-  lds_barrier();
+  PYRE_TS(1);
+  lds_barrier(); PYRE_TS(2);
   auto slice_max = [&](int t) { float mx = wmax[0][t];
 #pragma unroll
     for (int k = 1; k < NW; ++k) mx = fmaxf(mx, wmax[k][t]);
@@ -311,7 +313,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
     ssq[ks * T + tid] = tot; }
 #pragma unroll
   for (int t = 0; t < T; ++t) { float up, dn; hc_scale_of(slice_max(t), &up, &dn); hc_split_store(ah, tid, t, xs[t] * up); }
-  lds_barrier();
+  lds_barrier(); PYRE_TS(3);
   const int q = lane >> 4;
   float upf, dn0 = 0.0f, dn1 = 0.0f;
   if (2 * q < T) hc_scale_of(slice_max(2 * q), &upf, &dn0);
@@ -319,6 +321,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   v4f tot[1] = {v4f{0.0f, 0.0f, 0.0f, 0.0f}};
   { ABuf a0, a1; hc_lds_a(ah, 2 * p, lane, a0); hc_lds_a(ah, 2 * p + 1, lane, a1); a0.ai0 = dn0; a0.ai1 = dn1; a1.ai0 = dn0; a1.ai1 = dn1;
     chunk_mac<1>(w0, a0, ch0, nk, tot); chunk_mac<1>(w1, a1, ch0 + 1, nk, tot); }
+  PYRE_TS(4);
   float r0 = tot[0][0] + tot[0][1] * (1.0f / 2048.0f), r1 = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
   if constexpr (CS == 2) {
     if (p == 1) { hsum[g][0][lane] = r0; hsum[g][1][lane] = r1; }
@@ -329,6 +332,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   const size_t r64 = (size_t)m.tiles * 64, row = (size_t)tile * 64 + g * 16 + (lane & 15);
   if (2 * q < T) part[((size_t)ks * T + 2 * q) * r64 + row] = r0;
   if (2 * q + 1 < T) part[((size_t)ks * T + 2 * q + 1) * r64 + row] = r1;
+  PYRE_TS(5); PYRE_TS(6); PYRE_TS(7); PYRE_TS_FLUSH(hc_ts, NP > 1 ? 48 : 56);
 }
 
 __device__ __forceinline__ void hc_load_run16(float (&sv)[16], const float* __restrict__ p, int n, int stride) {      // n (<= 16) values at p, p + stride, ..
@@ -360,27 +364,33 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
   return o;
 }
 
-// grid (d / 64), hc*4 waves: wave (s, g) takes row group g of row tile s*(d/64) + blockIdx.x of `up` over all lr columns
-// (at most sixteen slices).  Prologue, epilogue and the riding router GEMV as k_hc_up_mix, except that every load the
-// prologue and the epilogue need is issued at the start (two rows of lo and one inject row a thread, the streams of one
-// column a thread), and lo goes through shared memory twice: f32, then as operand rows scaled per token by the power of two
-// of its largest magnitude.
+// grid (d / CW), hc * (CW / 16) waves, CW = 1 << lcw = 16, 32 or 64 columns of the mixed vector per workgroup: wave (s, g)
+// takes row group g of the workgroup's CW rows of stream s of `up` over all lr columns (at most sixteen slices).  A single
+// token without a riding router runs on d / 16 workgroups of hc waves: the launch is bound by the vector instructions a
+// compute unit issues, not by bytes, so 128 compute units with one wave per SIMD finish the same arithmetic four times
+// sooner than 32 with four.  Prologue, epilogue and the riding router GEMV (CW = 64 only: a workgroup owns one 64-column
+// unit of the router) as k_hc_up_mix, except that every load the prologue and the epilogue need is issued at the start
+// (two rows of lo and one inject row a thread, the streams of one column a thread), and lo goes through shared memory
+// twice: f32, then as operand rows scaled per token by the power of two of its largest magnitude.  Operand rows no token
+// of the window owns are left as they are: a row only ever reaches its own sums.  A value's arithmetic does not depend on CW.
 template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
-    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows) {
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;
-  qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj);
+  PYRE_TS_VARS PYRE_TS(0);
+  qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj, lcw);
   extern __shared__ __align__(16) float sm[];
-  const int nthr = blockDim.x, tid = threadIdx.x, kps = ksplit / hc, nw = nthr >> 6;
+  const int nthr = blockDim.x, tid = threadIdx.x, kps = ksplit / hc, nw = nthr >> 6, CW = 1 << lcw, lg = lcw - 4;
   float* lo = sm;                                 // [T][lr]
-  float* red = lo + (size_t)T * lr;               // [hc][T][64]: the gate logits
+  float* red = lo + (size_t)T * lr;               // [hc][T][CW]: the gate logits
   float* sls = red + (size_t)hc * T * 64;         // [T][16]
   uint32_t* lmax = (uint32_t*)(sls + (size_t)T * 16);      // [8]: bits of the largest |lo| of each token
   uint16_t* ah = (uint16_t*)(lmax + 8);           // [lr/8][16][8]
   const int K128 = lr >> 7, n_lo = T * lr;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int s = wave >> 2, g = wave & 3, q = lane >> 4;
+  const int s = wave >> lg, g = wave & ((1 << lg) - 1), q = lane >> 4;
+  const int col0 = blockIdx.x << lcw;
   float ssv[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) ssv[k] = 0.0f;
@@ -393,19 +403,19 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   hc_load_slices16<T>(pva, part, ia < n_lo, ksplit, ta, r64, ra);
   hc_load_slices16<T>(pvb, part, ib < n_lo, ksplit, tb, r64, rb);
   hc_load_slices16<T>(pvi, part, own_stream && has_inject, ksplit, stt, r64, lr + sq);
-  const int rg = (s * (d >> 6) + blockIdx.x) * 4 + g;
+  const int rg = ((s * d + col0) >> 4) + g;
   WBuf<1> w0, w1; load_w<1>(up, rg, 0, lane, K128, w0); load_w<1>(up, rg, 1, lane, K128, w1);
   const NibK nk = nib_consts();
-  // the epilogue's operands: thread (token tid / 64, column tid % 64) adds the streams of its column itself
+  // the epilogue's operands: thread (token tid / CW, column tid % CW) adds the streams of its column itself
   float xpre[4] = {0.0f, 0.0f, 0.0f, 0.0f}, npre[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (tid < T * 64) {
+  const int et = tid >> lcw, el = tid & (CW - 1);
+  if (tid < (T << lcw)) {
 #pragma unroll
-    for (int qs = 0; qs < 4; ++qs) if (qs < hc) { xpre[qs] = xnew[((size_t)(tid >> 6) * hc + qs) * d + blockIdx.x * 64 + lane]; npre[qs] = norm[(size_t)qs * d + blockIdx.x * 64 + lane]; }
+    for (int qs = 0; qs < 4; ++qs) if (qs < hc) { xpre[qs] = xnew[((size_t)et * hc + qs) * d + col0 + el]; npre[qs] = norm[(size_t)qs * d + col0 + el]; }
   }
   UnitRaw<RFX> rraw;
   constexpr bool R_EARLY = RFX != FMT_F32;      // an f32 tile is 64 registers: fetched once the up GEMV has freed them; others once the slice sums are used up
   if (tid < 8) lmax[tid] = 0u;
-  for (int j = tid; j < (16 - 2 * T) * lr; j += nthr) { const int r = 2 * T + j / lr, k = j - (r - 2 * T) * lr; ah[((size_t)(k >> 3) * 16 + r) * 8 + (k & 7)] = 0; }
   if (own_stream) {
     float tot = ssv[0];
 #pragma unroll
@@ -413,7 +423,8 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
     const float sc = 1.0f / sqrtf(tot / (float)d + eps);
     for (int k = 0; k < kps; ++k) sls[stt * 16 + sq * kps + k] = sc;
   }
-  lds_barrier();
+  PYRE_TS(1);
+  lds_barrier(); PYRE_TS(2);
   auto put_lo = [&](int t, int i, const float (&pv)[16]) {
     const float v = hc_slice_sum16(pv, sls + t * 16, ksplit) / (float)hc, lv = v * sigm(v);
     lo[t * lr + i] = lv; float a = fabsf(lv); a = a == a ? a : INFINITY; atomicMax(&lmax[t], __float_as_uint(a)); };
@@ -425,12 +436,12 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   const int rnt = ROUTE ? max(1, (int)router.tiles) : 1, rsets = T == 1 ? 1 : max(1, nw / rnt), rtile = T == 1 ? wave : wave % rnt, rset = T == 1 ? 0 : wave / rnt;
   const bool rwave = ROUTE && (T == 1 ? wave < rnt : (rset < rsets && rset < T));          // (a set without a token fetches nothing; a single token: one set, no division)
   if (rwave && R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
-  lds_barrier();
+  lds_barrier(); PYRE_TS(3);
   for (int j = tid; j < n_lo; j += nthr) {
     const int t2 = j / lr, k = j - t2 * lr; float upf, dn; hc_scale_of(__uint_as_float(lmax[t2]), &upf, &dn);
     hc_split_store(ah, k, t2, lo[j] * upf);
   }
-  lds_barrier();
+  lds_barrier(); PYRE_TS(4);
   v4f tot[1] = {v4f{0.0f, 0.0f, 0.0f, 0.0f}};
   { float upf, dn0 = 0.0f, dn1 = 0.0f;
     if (2 * q < T) hc_scale_of(__uint_as_float(lmax[2 * q]), &upf, &dn0);
@@ -441,14 +452,15 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
       a0.ai0 = dn0; a0.ai1 = dn1; a1.ai0 = dn0; a1.ai1 = dn1;
       chunk_mac<1>(w0, a0, c, nk, tot); chunk_mac<1>(w1, a1, c + 1, nk, tot);
     } }
-  if (2 * q < T) red[((size_t)s * T + 2 * q) * 64 + g * 16 + (lane & 15)] = tot[0][0] + tot[0][1] * (1.0f / 2048.0f);
-  if (2 * q + 1 < T) red[((size_t)s * T + 2 * q + 1) * 64 + g * 16 + (lane & 15)] = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
+  if (2 * q < T) red[(((size_t)s * T + 2 * q) << lcw) + g * 16 + (lane & 15)] = tot[0][0] + tot[0][1] * (1.0f / 2048.0f);
+  if (2 * q + 1 < T) red[(((size_t)s * T + 2 * q + 1) << lcw) + g * 16 + (lane & 15)] = tot[0][2] + tot[0][3] * (1.0f / 2048.0f);
   if (rwave && !R_EARLY) rraw = unit_load<RFX>(router, rtile, blockIdx.x, lane);
-  lds_barrier();
-  if (tid < T * 64) {          // the gated, normalised streams of the column, streams ascending from zero (:1380)
-    const int t2 = tid >> 6, l = lane, col = blockIdx.x * 64 + l; float mx = 0.0f;
+  PYRE_TS(5);
+  lds_barrier(); PYRE_TS(6);
+  if (tid < (T << lcw)) {          // the gated, normalised streams of the column, streams ascending from zero (:1380)
+    const int t2 = et, l = el, col = col0 + l; float mx = 0.0f;
 #pragma unroll
-    for (int qs = 0; qs < 4; ++qs) if (qs < hc) mx += xpre[qs] * sls[t2 * 16 + qs * kps] * npre[qs] * sigm(red[((size_t)qs * T + t2) * 64 + l]);            // rms: (x * s) * w
+    for (int qs = 0; qs < 4; ++qs) if (qs < hc) mx += xpre[qs] * sls[t2 * 16 + qs * kps] * npre[qs] * sigm(red[(((size_t)qs * T + t2) << lcw) + l]);            // rms: (x * s) * w
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
     if (aop) aop_store(aop, aop_rows, col, t2, mv);
@@ -467,6 +479,7 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
       }
     }
   }
+  PYRE_TS(7); PYRE_TS_FLUSH(hc_ts, ROUTE ? 32 : 40);
 }
 
 __global__ void k_hc_combine(float* __restrict__ x, const float* __restrict__ out, const float* __restrict__ inj, int d, int hc) {
@@ -522,13 +535,22 @@ template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcW
 #undef NORM_DOWN_M_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
+// columns of the mixed vector a workgroup of the matrix-core up / mix launch owns (log2): a single token without a riding
+// router spreads over d / 16 workgroups, everything else keeps 64 (the router rides in units of 64 columns; a window's
+// prologue grows with its width and would be redone by four times as many workgroups)
+int hc_m_lcw(const HcDev& h, int t, bool route) {
+  static const int force = [] { const char* e = getenv("PYRE_HC_CW"); return e && *e ? atoi(e) : 0; }();      // 16 / 32 / 64: one width for every launch without a router
+  if (route) return 6;
+  if (force == 16) return 4; if (force == 32) return 5; if (force == 64) return 6;
+  return t == 1 ? 4 : 6;
+}
 template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
-  const int nw = h.hc * 4; const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + 8) + (size_t)h.lr * 32;
+  const int lcw = hc_m_lcw(h, T, rt != nullptr), nw = h.hc << (lcw - 4); const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + 8) + (size_t)h.lr * 32;
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
-#define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, rq, rp, aop, pyre_aop_rows(T))
+#define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
+                     h.d, mixed, inj, rq, rp, aop, pyre_aop_rows(T), lcw)
   if (rt && rq.fmt == FMT_BF16) UP_MIX_M_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_GO(FMT_F32); else UP_MIX_M_GO(-1);
 #undef UP_MIX_M_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;

@@ -469,7 +469,7 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
   const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
   pyre_qmat* m = new pyre_qmat(); m->ctx = ctx; m->ty = ty; m->rows = rows; m->cols = cols; m->gguf_bytes = nbytes;
-  auto drop = [&]() { if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); delete m; };
+  auto drop = [&]() { if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); if (m->base_n) (void)hipFree(m->base_n); delete m; };
   int U = (int)(cols / PYRE_UNIT), tiles = (int)((rows + 63) / 64);
   size_t ent = (size_t)tiles * U * 64;
   auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
@@ -507,6 +507,12 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
     e = hipGetLastError();
     if (!want_rows) m->dv = m->dvm;         // the only layout the matrix has is the one every user sees
   }
+  if (layout == PYRE_LAYOUT_BOTH && fmt == FMT_IQ3_S && cols % 256 == 0 && e == hipSuccess) {      // the stand-alone operator's single-token kernel streams the file's 3.44 bit/weight
+    m->dev_bytes_n = pyre_gemv_n_bytes(rows, cols);
+    e = hipMalloc(&m->base_n, m->dev_bytes_n);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_n, hipGetErrorString(e)); }
+    if (pyre_gemv_n_repack(ctx, rows, cols, src, row_bytes, m->base_n) != PYRE_OK) e = hipErrorLaunchFailure;
+  }
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (tmp) (void)hipFree(tmp);
   if (e != hipSuccess) { drop(); return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmat_create: repack failed: %s", hipGetErrorString(e)); }
@@ -522,12 +528,12 @@ extern "C" {
 
 int pyre_qmat_create(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* host_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, host_blocks, false, nbytes, out); }
 int pyre_qmat_create_dev(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* dev_blocks, size_t nbytes, pyre_qmat** out) { return qmat_create_common(ctx, ty, rows, cols, dev_blocks, true, nbytes, out); }
-void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); delete m; }
+void pyre_qmat_destroy(pyre_qmat* m) { if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream); if (m->base) (void)hipFree(m->base); if (m->base_m) (void)hipFree(m->base_m); if (m->base_n) (void)hipFree(m->base_n); delete m; }
 size_t pyre_qmat_rows(const pyre_qmat* m) { return m ? m->rows : 0; }
 size_t pyre_qmat_cols(const pyre_qmat* m) { return m ? m->cols : 0; }
 size_t pyre_qmat_gguf_bytes(const pyre_qmat* m) { return m ? m->gguf_bytes : 0; }
-size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes + m->dev_bytes_m : 0; }
-size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int matrix_core_layout) { return !m ? 0 : (matrix_core_layout ? m->dev_bytes_m : m->dev_bytes); }
+size_t pyre_qmat_device_bytes(const pyre_qmat* m) { return m ? m->dev_bytes + m->dev_bytes_m + m->dev_bytes_n : 0; }
+size_t pyre_qmat_layout_bytes(const pyre_qmat* m, int which) { return !m ? 0 : (which == 2 ? m->dev_bytes_n : (which ? m->dev_bytes_m : m->dev_bytes)); }
 
 int pyre_qmat_dequant_dev(pyre_ctx* ctx, const pyre_qmat* m, float* out_dev) {
   if (!ctx || !m || !out_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_dequant: null argument");
@@ -560,7 +566,9 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
 // The operator's own launch: an IQ3_S matrix goes through the matrix-core GEMM (for every t, so a token's result does not
 // depend on the window width); f32_path (or PYRE_QMATMUL_F32=1) takes the f32 lane = row GEMV the model's expert matrices use.
 static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev, bool f32_path) {
-  static const int f32_only = env_int("PYRE_QMATMUL_F32", 0);
+  static const int f32_only = env_int("PYRE_QMATMUL_F32", 0), native = env_int("PYRE_QMATMUL_NATIVE", 1);
+  // one token of an IQ3_S matrix: the kernel that streams the file's 3.44 bit/weight (PYRE_QMATMUL_NATIVE=0: the matrix cores as for a window)
+  if (t == 1 && m->base_n && native && !f32_path && !f32_only) return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
   if (has_m && (!has_rows || (!f32_path && !f32_only))) return pyre_gemv_launch(ctx, m->dvm, x_dev, t, y_dev);
   return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
@@ -587,17 +595,12 @@ int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: t = %d outside 1..8", t);
   if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  if (t == 1 && m->base_n && env_int("PYRE_QMATMUL_NATIVE", 1)) {      // one token: the native-format kernel, as in pyre_qmatmul_dev, its activation digits in the static array
+    if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
+    if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
+    return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, ctx->aop_static);
+  }
   return pyre_gemm_m_static(ctx, m->dvm, x_dev, t, y_dev);
-}
-// kept for callers written against the separate verify-window entry: since pyre_qmatmul itself runs on the matrix cores
-// for every window width, these are the same call restricted to IQ3_S
-int pyre_qmatmul_mfma_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
-  if (m && !(m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq)) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_mfma: IQ3_S matrices only");
-  return qmatmul_dev(ctx, m, x_dev, t, y_dev, false);
-}
-int pyre_qmatmul_mfma(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) {
-  if (m && !(m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq)) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_mfma: IQ3_S matrices only");
-  return qmatmul_host(ctx, m, x_host, t, y_host, false);
 }
 int pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) { return qmatmul_dev(ctx, m, x_dev, t, y_dev, true); }
 int pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host) { return qmatmul_host(ctx, m, x_host, t, y_host, true); }

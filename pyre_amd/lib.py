@@ -48,7 +48,6 @@ def _declare(L):
         "pyre_qmatmul_f32": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_f32_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmatmul_static_dev": (i32, [vp, vp, vp, i32, vp]),
-        "pyre_qmatmul_mfma": (i32, [vp, vp, vp, i32, vp]),
         "pyre_qmat_layout_bytes": (sz, [vp, i32]),
         "pyre_gguf_open": (i32, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
         "pyre_gguf_close": (None, [vp]),
@@ -76,7 +75,6 @@ def _declare(L):
         "pyre_snap_destroy": (None, [vp]),
         "pyre_snap_bytes": (C.c_size_t, [vp]),
         "pyre_snap_len": (i32, [vp]),
-        "pyre_qmatmul_mfma_dev": (i32, [vp, vp, vp, i32, vp]),
         "pyre_synth_blocks": (i32, [vp, u32, sz, u64, f32, f32, vp]),
         "pyre_moe_create": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, C.POINTER(vp)]),
         "pyre_moe_destroy": (None, [vp]),
@@ -260,9 +258,10 @@ class QMat:
     def dev_bytes(self):
         return self.ctx.L.pyre_qmat_device_bytes(self.h)
 
-    def layout_bytes(self, matrix_core):
-        """Device bytes of one layout: False = the lane-per-row planes, True = the matrix-core layout (IQ3_S only)."""
-        return self.ctx.L.pyre_qmat_layout_bytes(self.h, 1 if matrix_core else 0)
+    def layout_bytes(self, layout):
+        """Device bytes of one layout: 0 / False = the lane-per-row planes, 1 / True = the matrix-core layout (IQ3_S only),
+        2 = IQ3_S at the file's bits per weight (what a single-token matmul streams)."""
+        return self.ctx.L.pyre_qmat_layout_bytes(self.h, int(layout))
 
     def to_f32(self):
         out = np.empty((self.rows, self.cols), dtype=np.float32)
@@ -283,21 +282,11 @@ class QMat:
         return y
 
     def matmul_f32(self, x):
-        """matmul on the f32 multiply-add GEMV the model's layers use (IQ3_S: matmul itself takes integer dot products)."""
+        """matmul on the f32 multiply-add GEMV the model's expert matrices use (IQ3_S: matmul itself takes the native-format integer-dot kernel for one token and the matrix cores for a window)."""
         x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
         y = np.empty((x.shape[0], self.rows), dtype=np.float32)
         self.ctx.check(self.ctx.L.pyre_qmatmul_f32(self.ctx.h, self.h, _ptr(x), x.shape[0], _ptr(y)), "qmatmul_f32")
         return y
-
-    def matmul_mfma(self, x):
-        """The matrix-core verify GEMM (IQ3_S, 2..8 tokens): same contract as matmul, ~1e-7 of max|y| from it."""
-        x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, self.cols)
-        y = np.empty((x.shape[0], self.rows), dtype=np.float32)
-        self.ctx.check(self.ctx.L.pyre_qmatmul_mfma(self.ctx.h, self.h, _ptr(x), x.shape[0], _ptr(y)), "qmatmul_mfma")
-        return y
-
-    def matmul_mfma_dev(self, x_dev, t, y_dev):
-        self.ctx.check(self.ctx.L.pyre_qmatmul_mfma_dev(self.ctx.h, self.h, _ptr(x_dev), t, _ptr(y_dev)), "qmatmul_mfma_dev")
 
     def matmul_static_dev(self, x_dev, t, y_dev):
         """pyre_qmatmul_static_dev: device pointers in and out, nothing allocated by the call."""

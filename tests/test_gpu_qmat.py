@@ -130,8 +130,14 @@ def test_result_for_a_token_does_not_depend_on_batch_width(ctx, ty):
     y8 = m.matmul(x)
     for t in (1, 2, 4):
         yt = m.matmul(x[:t])
-        assert np.array_equal(bits(yt), bits(y8[:t])), t
-    assert np.array_equal(bits(m.matmul(x[3:4])), bits(y8[3:4]))
+        if ty == lib.IQ3_S and t == 1:          # one token of an IQ3_S matrix has a kernel of its own: equal to rounding, and to itself
+            assert relerr(yt, y8[:1]) <= 2e-6 and np.array_equal(bits(yt), bits(m.matmul(x[:1])))
+        else:
+            assert np.array_equal(bits(yt), bits(y8[:t])), t
+    if ty == lib.IQ3_S:
+        assert relerr(m.matmul(x[3:4]), y8[3:4]) <= 2e-6 and np.array_equal(bits(m.matmul(x[2:4])[1:]), bits(y8[3:4]))
+    else:
+        assert np.array_equal(bits(m.matmul(x[3:4])), bits(y8[3:4]))
     # and it is reproducible run to run (split-K partials are added in a fixed order)
     assert np.array_equal(bits(m.matmul(x)), bits(y8))
     y8f = m.matmul_f32(x)
@@ -151,8 +157,11 @@ def test_iq3s_both_paths_match_truth_and_each_other(ctx, rows, cols):
         yi, yf = m.matmul(x), m.matmul_f32(x)
         assert relerr(yi, truth) <= TOL and relerr(yf, truth) <= TOL, t
         assert relerr(yi, yf) <= 2e-6, t
-        for i in range(t):           # per token, whatever the window width, on both paths
-            assert np.array_equal(bits(m.matmul(x[i:i + 1])), bits(yi[i:i + 1]))
+        for i in range(t):           # per token, whatever the window width (a single token of `matmul` runs the native-format kernel: equal to rounding)
+            if t >= 2:
+                pair = x[[i, (i + 1) % t]]
+                assert np.array_equal(bits(m.matmul(pair)[:1]), bits(yi[i:i + 1]))
+            assert relerr(m.matmul(x[i:i + 1]), yi[i:i + 1]) <= 2e-6
             assert np.array_equal(bits(m.matmul_f32(x[i:i + 1])), bits(yf[i:i + 1]))
 
 
@@ -237,7 +246,7 @@ def test_argument_errors_are_reported(ctx):
         m.row(64)
 
 
-# ---- the verify window on the matrix cores (IQ3_S): the same kernel as t = 1 ---------------------------------------------
+# ---- the verify window on the matrix cores (IQ3_S, t >= 2) and the native-format kernel (t = 1) ------------------------------
 @pytest.mark.parametrize("t", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("rows,cols", [(320, 2048), (4096, 2048), (2048, 4096), (2048, 512), (100, 256)])
 def test_verify_gemm_on_matrix_cores_matches_truth(ctx, rows, cols, t):
@@ -248,19 +257,41 @@ def test_verify_gemm_on_matrix_cores_matches_truth(ctx, rows, cols, t):
     x[0] *= 3000.0                                   # a token far outside the half range: the exact power-of-two rescaling
     x[-1] *= 1e-6
     truth = x.astype(np.float64) @ W.T
-    y = m.matmul_mfma(x)
+    y = m.matmul(x)
     for i in range(t):                               # per token: the tokens differ by nine orders of magnitude
         assert relerr(y[i], truth[i]) <= TOL, i
-    assert np.array_equal(bits(y), bits(m.matmul(x)))          # one kernel behind both entry points
     yf = m.matmul_f32(x)
     for i in range(t):
         assert relerr(y[i], yf[i]) <= 2e-6, i
 
 
-def test_verify_gemm_on_matrix_cores_rejects_other_types_and_widths(ctx):
-    m = lib.QMat(ctx, lib.Q8_0, 64, 256, synth.matrix(lib.Q8_0, 64, 256, 3))
-    with pytest.raises(lib.PyreError):
-        m.matmul_mfma(synth.normal((2, 256), 1))
-    m3 = lib.QMat(ctx, lib.IQ3_S, 64, 256, synth.matrix(lib.IQ3_S, 64, 256, 3))
-    with pytest.raises(lib.PyreError):
-        m3.matmul_mfma(synth.normal((9, 256), 1))
+# ---- one token of an IQ3_S matrix: the file's bits per weight, codebook with signs in shared memory, integer dots --------------
+@pytest.mark.parametrize("rows,cols", [(64, 256), (100, 256), (65, 512), (320, 2048), (4096, 2048), (2048, 4096), (1000, 768), (130, 8192)])
+def test_iq3s_native_format_single_token(ctx, rows, cols):
+    raw = synth.matrix(lib.IQ3_S, rows, cols, 300 + rows % 97)
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
+    assert m.layout_bytes(2) == (rows + 63) // 64 * 64 * (cols // 256) * 112
+    W = orc.dequant(lib.IQ3_S, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    g = np.random.Generator(np.random.PCG64(rows + cols))
+    for case in range(6):
+        x = synth.normal((1, cols), 400 + case)
+        if case == 1: x *= np.exp2(g.integers(-40, 40, cols // 64).repeat(64)).astype(np.float32)      # every 64 columns on their own power of two
+        if case == 2: x[0, 5] = 3.0e4; x[0, cols - 3] = -2.0e7                                          # outliers
+        if case == 3: x *= 1e-30
+        if case == 4: x *= 1e30
+        if case == 5: x[0, ::2] = 0.0; x[0, :64] = 0.0                                                  # an all-zero unit
+        with np.errstate(all="ignore"):
+            truth = x.astype(np.float64) @ W.T
+        y = m.matmul(x)
+        assert relerr(y, truth) <= TOL, case
+        assert np.array_equal(bits(y), bits(m.matmul(x)))          # run to run
+        assert relerr(y, m.matmul(np.concatenate([x, x]))[:1]) <= 2e-6          # the window's kernel agrees to rounding
+    xi = g.integers(-1000, 1000, (1, cols)).astype(np.float32)          # integers: exact digits, exact sums, only the f32 scaling rounds
+    assert relerr(m.matmul(xi), xi.astype(np.float64) @ W.T) <= 2e-7
+    a = synth.normal((1, cols), 155)
+    assert np.array_equal(bits(m.matmul(a * 1024.0)), bits(m.matmul(a) * 1024.0))          # a power of two scales the result exactly
+    bad = synth.normal((1, cols), 156); bad[0, 3] = np.inf
+    assert np.isnan(m.matmul(bad)).all()
+    bad[0, 3] = np.nan
+    assert np.isnan(m.matmul(bad)).all()
+    assert not m.matmul(np.zeros((1, cols), np.float32)).any()
