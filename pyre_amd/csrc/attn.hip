@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
 // step after a 32 768-token prompt has 257 chunks.
 template <int HD>
 __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                      int max_chunks, float* __restrict__ out, const int* __restrict__ pcount, uint16_t* __restrict__ aop, int aop_rows) {
+                                                      int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
   constexpr int CB = 320, B = CB / 4;
   __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[CB], ls[CB];
   if (posp) start = *posp;
@@ -531,7 +531,6 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
     float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd];
     const float ov = (o / L) * a_sigm(gate);
     out[((size_t)ti * a.nh + h) * HD + dd] = ov;
-    if (aop) aop_store(aop, aop_rows, h * HD + dd, ti, ov);          // the f16 operand of the output projection (matrix-core layout)
   }
 }
 
@@ -571,7 +570,7 @@ template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, cons
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
   return pyre_attn_launch_sel(ctx, a, kv, w, qkv, stride, start, t, packed_done, out, posp, nullptr);
 }
-int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp, const QsaWork* qw, uint16_t* aop) {
+int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp, const QsaWork* qw) {
   if (a.hd != 256) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: head dim %d unsupported (256 only)", a.hd);
   if (a.nkv < 1 || a.nh % a.nkv) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: %d query heads over %d kv heads", a.nh, a.nkv);
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
@@ -601,7 +600,7 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp, qw); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp, qw); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp, qw); break;
     default: launch_decode<8>(ctx, a, kv, w, start, t, posp, qw); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t, 256 / 64), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr, aop, aop ? pyre_aop_rows(t) : 0); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t, 256 / 64), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

@@ -188,8 +188,9 @@ int pyre_gemm_m_scratch(pyre_ctx* ctx, int cols, uint4** op, float** ainv);
 int pyre_static_init(pyre_ctx* ctx);
 int pyre_gemm_m_static(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev);
 #ifdef __HIPCC__
-// One activation into the operand a producer kernel leaves for the GEMM that follows it, unscaled (|v| < 65504: the
-// producers' outputs are normalised vectors): element k of token ti of a window with R operand rows.
+// One activation into the operand a producer kernel leaves for the GEMM that follows it: element k of token ti of a window
+// with R operand rows.  v is the value already multiplied by the power of two its producer scales the token by (AopOut:
+// the factor brings a bound of the token's largest magnitude into [2^13, 2^14), the GEMM multiplies the sums by its inverse).
 __device__ __forceinline__ void aop_store(uint16_t* __restrict__ op, int R, int k, int ti, float v) {
   const _Float16 h1 = (_Float16)v, h2 = (_Float16)((v - (float)h1) * 2048.0f);
   const size_t base = ((size_t)(k >> 3) * R + 2 * ti) * 8 + (k & 7);
@@ -280,7 +281,7 @@ int pyre_ple_launch(pyre_ctx* ctx, const PleCfg& c, const PleDev& p, const PleWo
 // ---- hyper-connections (hc.hip) ---------------------------------------------------------------------------------------
 struct HcDev { QMatDev di; QMatDev up; const float* norm; int d, hc, lr; bool has_inject;      // di = [down ; inject] rows
                QMatDev di_m{}, up_m{}; };      // the same two matrices in the matrix-core layout (fmt == FMT_IQ3_S_M) when they are IQ3_S of whole super-blocks
-struct HcWork { float* ssq; float* o; };    // [<=32][8] slice sums of squares of the streams, [<=32][8][tiles*64] slice sums of [down ; inject]
+struct HcWork { float* ssq; float* o; float* smx; };    // [<=32][8] slice sums of squares of the streams, [<=32][8][tiles*64] slice sums of [down ; inject], [<=32][8] largest |x * norm weight| of each slice
 size_t pyre_hc_work_bytes(const HcDev& h);
 void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // Streams are read from x_in (element i of stream s of token ti at x_in[ti*in_ts + s*in_ss + i]; in_ss = 0 replicates one
@@ -291,11 +292,18 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // owns columns [64b, 64b+64) of the mixed vector, so it leaves the K-slice sum part[(b*T + t)*tiles*64 + row] of every
 // router row; the gate/up launch adds the d/64 slices (RouteSrc).  bf16 and f32 routers, at most 64 slices.
 struct HcRoute { QMatDev router; float* part; };
+// Where a producer kernel leaves its result as the f16 operand of the matrix-core GEMM that follows (so that GEMM needs no
+// split launch of its own): op = PyreAop::op (pyre_aop_rows(t) rows), ainv = PyreAop::ainv, [nsb super-blocks][8 tokens].
+// Every token is scaled by one power of two that brings a bound of its largest magnitude into [2^13, 2^14) -- a bound every
+// workgroup of the producer can form without talking to the others -- and ainv holds the inverse for every super-block:
+//   hyper-connection mix: |mixed_i| <= max over the streams of (RMS scale * largest |x * norm weight| of the stream), from
+//     the slice maxima the mix's first launch leaves (matrix-core mixes only: pyre_hc_aop_ok)
+//   Gated DeltaNet: |o_i * scale| <= sqrt(dv) after the RMS normalisation, times the largest norm weight: a constant of the
+//     layer (pyre_gdn_launch takes the factor, the model keeps the matching ainv)
+struct AopOut { uint16_t* op; float* ainv; int nsb; };
+bool pyre_hc_aop_ok(const HcDev& h);
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr, int comb_parts = 1, uint16_t* aop = nullptr);
-// aop (here and in pyre_gdn_launch / pyre_attn_launch_sel): when given, the kernel that writes the f32 result also leaves it
-// as the f16 operand of a matrix-core GEMM (PyreAop::op, pyre_aop_rows(t) rows, unscaled), so the GEMM that follows needs no
-// separate split launch.
+                       float eps, float* mixed_dev, float* inj_dev, const HcRoute* route = nullptr, int comb_parts = 1, const AopOut* aop = nullptr);
 bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router);
 // waves per workgroup, units per wave and K slices of the norm + [down ; inject] kernel; false if the shape is unsupported
 bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit);
@@ -307,7 +315,7 @@ struct GdnDev { const float* a; const float* dt; const float* conv_w; const floa
 // conv_in/conv_out [(k-1)][ch], ssm_in/ssm_out [nv][dk][dv] (in != out).  co_scratch [8][ch].  out [t][nv*dv].
 // conv_done: co_scratch already holds silu(conv) of the window and the conv state has been advanced (GemvEpi).
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr);
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f);
 
 // Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
 // scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].
@@ -371,5 +379,5 @@ int pyre_qsa_launch(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaB
 int pyre_qsa_pool_all(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaBuf& b, int n);
 // the attention launch with an optional position list (qw == nullptr: dense)
 int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
-                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw, uint16_t* aop = nullptr);
+                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw);
 int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t);      // K / V only

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj
 //   S *= g; mem = S^T k -> barrier -> delta = (v - mem) beta; S += k (x) delta; o = S^T q      (linear_core, :1655-1668)
 template <int DK, int DV>
 __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
-                                                   const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out, uint16_t* __restrict__ aop, int aop_rows) {
+                                                   const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out, uint16_t* __restrict__ aop, int aop_rows, float aop_up) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int G = 4, R = DK / G, MT = 8;
   PYRE_TS_VARS PYRE_TS(0);
@@ -92,20 +92,20 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
     const float sc = 1.0f / sqrtf((wsum(o0 * o0) + wsum(o1 * o1)) / (float)DV + p.eps);
     const float r0 = (o0 * (sc * nw0)) * g_sigm(zs[wave][lane]), r1 = (o1 * (sc * nw1)) * g_sigm(zs[wave][lane + 64]);      // rms_inplace: x *= s * w  (:210)
     out[(size_t)wave * w + h * DV + lane] = r0; out[(size_t)wave * w + h * DV + lane + 64] = r1;
-    if (aop) { aop_store(aop, aop_rows, h * DV + lane, wave, r0); aop_store(aop, aop_rows, h * DV + lane + 64, wave, r1); }      // the f16 operand of the output projection (matrix-core layout)
+    if (aop) { aop_store(aop, aop_rows, h * DV + lane, wave, r0 * aop_up); aop_store(aop, aop_rows, h * DV + lane + 64, wave, r1 * aop_up); }      // the f16 operand of the output projection (matrix-core layout), scaled by the layer's power of two
   }
   PYRE_TS(4); PYRE_TS(5); PYRE_TS(6); PYRE_TS(7); PYRE_TS_FLUSH(gdn_ts, 0);
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done, uint16_t* aop) {
+                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done, uint16_t* aop, float aop_up) {
   if (aop && t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: an f16 operand holds at most 8 tokens, not %d", t);
   if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
   if (g.conv_k < 2 || g.conv_k > 8) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: conv kernel %d outside 2..8", g.conv_k);
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d outside 1..8", t);
   int ch = 2 * g.nk * g.dk + g.nv * g.dv;
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

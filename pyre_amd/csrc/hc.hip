@@ -146,7 +146,7 @@ template <int FMT, int T, int NP> __global__ __launch_bounds__(512) void k_hc_no
 // takes router tile w, w + nw, .. at unit blockIdx.x, the first tile's weights fetched ahead of the up GEMV.
 template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj, const uint2* __restrict__ g2,
-    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows) {
+    QMatDev router, float* __restrict__ rpart) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
@@ -226,7 +226,6 @@ template <int FMT, int T, int RF> __global__ __launch_bounds__(1024) void k_hc_u
     for (int q = 0; q < 8; ++q) if (q < hc) mx += term[(size_t)(t2 * hc + q) * 64 + l];          // streams ascending from zero (:1380)
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
-    if (aop) aop_store(aop, aop_rows, col, t2, mv);          // the f16 operand of the GEMM that follows (matrix-core layout)
     if (ROUTE) lo[t2 * 64 + l] = mv;          // lo is free after the barrier above
   }
   PYRE_TS(5);
@@ -271,7 +270,7 @@ __device__ __forceinline__ void hc_lds_a(const uint16_t* ah, int c, int lane, AB
 // Wave (p, g) takes row group g of the tile over chunk pair p of the slice; with CS = 2 the two pairs' sums meet in
 // shared memory (pair 0 + pair 1).  Outputs as k_hc_norm_down: ssq[ks*T + t], part[(ks*T + t)*tiles*64 + row], x_out.
 template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_hc_norm_down_m(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
-    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part) {
+    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part, float* __restrict__ smx) {
   constexpr int NW = 4 * CS;
   __shared__ __align__(16) uint16_t ah[CS * 32 * 16 * 8];
   __shared__ float wsum[NW][8], wmax[NW][8], hsum[4][2][64];
@@ -310,7 +309,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   if (tile == 0 && tid < T) { float tot = wsum[0][tid];
 #pragma unroll
     for (int k = 1; k < NW; ++k) tot += wsum[k][tid];
-    ssq[ks * T + tid] = tot; }
+    ssq[ks * T + tid] = tot; smx[ks * T + tid] = slice_max(tid); }          // (the largest |x * norm weight| of the slice: the second launch bounds the mixed vector with it)
 #pragma unroll
   for (int t = 0; t < T; ++t) { float up, dn; hc_scale_of(slice_max(t), &up, &dn); hc_split_store(ah, tid, t, xs[t] * up); }
   lds_barrier(); PYRE_TS(3);
@@ -375,7 +374,7 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
 // of the window owns are left as they are: a row only ever reaches its own sums.  A value's arithmetic does not depend on CW.
 template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
-    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw) {
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;
   PYRE_TS_VARS PYRE_TS(0);
@@ -386,7 +385,8 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   float* red = lo + (size_t)T * lr;               // [hc][T][CW]: the gate logits
   float* sls = red + (size_t)hc * T * 64;         // [T][16]
   uint32_t* lmax = (uint32_t*)(sls + (size_t)T * 16);      // [8]: bits of the largest |lo| of each token
-  uint16_t* ah = (uint16_t*)(lmax + 8);           // [lr/8][16][8]
+  float* bnd = (float*)(lmax + 8);                // [T][4]: RMS scale * largest |x * norm weight| of each stream
+  uint16_t* ah = (uint16_t*)(bnd + 32);           // [lr/8][16][8]
   const int K128 = lr >> 7, n_lo = T * lr;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int s = wave >> lg, g = wave & ((1 << lg) - 1), q = lane >> 4;
@@ -396,7 +396,10 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   for (int k = 0; k < 16; ++k) ssv[k] = 0.0f;
   const int stt = tid / hc, sq = tid - stt * hc;
   const bool own_stream = tid < T * hc;                      // thread (token stt, stream sq): the stream's scale, and the stream's inject row
-  if (own_stream) hc_load_run16(ssv, ssq + (size_t)(sq * kps) * T + stt, kps, T);
+  float smv[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) smv[k] = 0.0f;
+  if (own_stream) { hc_load_run16(ssv, ssq + (size_t)(sq * kps) * T + stt, kps, T); if (aop) hc_load_run16(smv, smx + (size_t)(sq * kps) * T + stt, kps, T); }
   float pva[16], pvb[16], pvi[16];
   const int ia = tid, ib = tid + nthr;
   const int ta = ia / lr, ra = ia - ta * lr, tb = ib / lr, rb = ib - tb * lr;
@@ -422,6 +425,10 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
     for (int k = 1; k < 16; ++k) if (k < kps) tot += ssv[k];
     const float sc = 1.0f / sqrtf(tot / (float)d + eps);
     for (int k = 0; k < kps; ++k) sls[stt * 16 + sq * kps + k] = sc;
+    float mxs = smv[0];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) if (k < kps) mxs = fmaxf(mxs, smv[k]);
+    bnd[stt * 4 + (sq & 3)] = sc * mxs;          // |x_i * scale * norm_i| <= this for every column i of the stream
   }
   PYRE_TS(1);
   lds_barrier(); PYRE_TS(2);
@@ -463,7 +470,15 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
     for (int qs = 0; qs < 4; ++qs) if (qs < hc) mx += xpre[qs] * sls[t2 * 16 + qs * kps] * npre[qs] * sigm(red[(((size_t)qs * T + t2) << lcw) + l]);            // rms: (x * s) * w
     const float mv = mx / (float)hc;
     mixed[(size_t)t2 * d + col] = mv;
-    if (aop) aop_store(aop, aop_rows, col, t2, mv);
+    if (aop) {          // the f16 operand of the GEMM that follows: the token scaled by the power of two of a bound of its largest magnitude
+      float b = bnd[t2 * 4];
+#pragma unroll
+      for (int qs = 1; qs < 4; ++qs) if (qs < hc) b = fmaxf(b, bnd[t2 * 4 + qs]);
+      b = b == b ? b : INFINITY;
+      float upf, dn; hc_scale_of(b, &upf, &dn);
+      aop_store(aop, aop_rows, col, t2, mv * upf);
+      if (blockIdx.x == 0 && l == 0) for (int sb = 0; sb < aop_nsb; ++sb) aop_inv[sb * 8 + t2] = dn;
+    }
     if (ROUTE) lo[t2 * 64 + l] = mv;
   }
   if (ROUTE) {
@@ -508,13 +523,13 @@ template <int FMT, int T> int norm_down_launch(pyre_ctx* ctx, const HcDev& h, co
 #undef NORM_DOWN_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
-template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
+template <int FMT, int T> int up_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
   const int nw = h.hc * h.up.U; size_t lds = 4 * ((size_t)T * h.lr + (size_t)nw * T * 64 + (size_t)T * 32 + (size_t)T * h.hc * 64);
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
 #define UP_MIX_GO(RF) hipLaunchKernelGGL((k_hc_up_mix<FMT, T, RF>), dim3(h.d / 64), dim3(nw * 64), lds, ctx->stream, h.up, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, (const uint2*)ctx->d_iq2xs, rq, rp, aop, pyre_aop_rows(T))
+                     h.d, mixed, inj, (const uint2*)ctx->d_iq2xs, rq, rp)
   if constexpr (FMT == FMT_IQ3_S || FMT == FMT_BF16 || FMT == FMT_F16 || FMT == FMT_F32) {
     if (rt && rq.fmt == FMT_BF16) UP_MIX_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_GO(FMT_F32); else UP_MIX_GO(-1);
   } else UP_MIX_GO(-1);
@@ -529,7 +544,7 @@ bool hc_on_matrix_cores(const HcDev& h) {
 }
 template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
   ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
-#define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o)
+#define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
   if (hc_m_cs(h) == 2) { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 2); else NORM_DOWN_M_GO(1, 2); }
   else { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 1); else NORM_DOWN_M_GO(1, 1); }
 #undef NORM_DOWN_M_GO
@@ -544,13 +559,13 @@ int hc_m_lcw(const HcDev& h, int t, bool route) {
   if (force == 16) return 4; if (force == 32) return 5; if (force == 64) return 6;
   return t == 1 ? 4 : 6;
 }
-template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
-  const int lcw = hc_m_lcw(h, T, rt != nullptr), nw = h.hc << (lcw - 4); const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + 8) + (size_t)h.lr * 32;
+template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, const AopOut* aop) {
+  const int lcw = hc_m_lcw(h, T, rt != nullptr), nw = h.hc << (lcw - 4); const size_t lds = 4 * ((size_t)T * h.lr + (size_t)h.hc * T * 64 + (size_t)T * 16 + 8 + 32) + (size_t)h.lr * 32;
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
 #define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, rq, rp, aop, pyre_aop_rows(T), lcw)
+                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0)
   if (rt && rq.fmt == FMT_BF16) UP_MIX_M_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_GO(FMT_F32); else UP_MIX_M_GO(-1);
 #undef UP_MIX_M_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
@@ -561,7 +576,7 @@ template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork
 int norm_down_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
   HC_M_T_SWITCH(norm_down_m_launch, ctx, h, w, x_in, in_ss, in_ts, x_out, comb_out, comb_parts, mo, comb_inj)
 }
-int up_mix_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
+int up_mix_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, const AopOut* aop) {
   HC_M_T_SWITCH(up_mix_m_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt, aop)
 }
 #define HC_T_SWITCH(F, FN, ...) \
@@ -575,11 +590,12 @@ int up_mix_m(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, 
 int norm_down(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const DownPlan& p, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj, float eps) {
   HC_FMT_SWITCH(h.di.fmt, HC_T_SWITCH(F, norm_down_launch, ctx, h, w, p, x_in, in_ss, in_ts, x_out, comb_out, comb_parts, mo, comb_inj, eps))
 }
-int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt, uint16_t* aop) {
-  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt, aop))
+int up_mix(pyre_ctx* ctx, const HcDev& h, const HcWork& w, int ksplit, int t, const float* xnew, float eps, float* mixed, float* inj, const HcRoute* rt) {
+  HC_FMT_SWITCH(h.up.fmt, HC_T_SWITCH(F, up_mix_launch, ctx, h, w, ksplit, xnew, eps, mixed, inj, rt))
 }
 }  // namespace
 
+bool pyre_hc_aop_ok(const HcDev& h) { return hc_on_matrix_cores(h) && h.hc <= 4; }
 bool pyre_hc_route_ok(const HcDev& h, const QMatDev& router) {
   const int f = h.up.fmt;
   return (f == FMT_IQ3_S || f == FMT_BF16 || f == FMT_F16 || f == FMT_F32) && (router.fmt == FMT_BF16 || router.fmt == FMT_F32) && router.cols == h.d && h.d / 64 <= 64 && router.U == h.d / 64;
@@ -589,14 +605,14 @@ bool pyre_hc_plan(const HcDev& h, int* nw, int* upw, int* ksplit) {
   DownPlan p = down_plan(h); *nw = p.nw; *upw = p.upw; *ksplit = p.ksplit;
   return p.ksplit >= 1 && p.ksplit <= 32 && p.ksplit * p.nw * p.upw == h.di.U;
 }
-size_t pyre_hc_work_bytes(const HcDev& h) { return 256 * 3 + 4 * 8 * 32 + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
+size_t pyre_hc_work_bytes(const HcDev& h) { return 256 * 4 + 2 * 4 * 8 * 32 + 4 * 8 * 32 * ((size_t)h.lr + h.hc + 64); }
 void pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
-  w->ssq = (float*)take(4 * 8 * 32); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
+  w->ssq = (float*)take(4 * 8 * 32); w->smx = (float*)take(4 * 8 * 32); w->o = (float*)take(4 * 8 * 32 * ((size_t)h.lr + h.hc + 64));
 }
 
 int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, int t, const float* comb_out, const MoeOut* comb_moe, const float* comb_inj,
-                       float eps, float* mixed, float* inj, const HcRoute* route, int comb_parts, uint16_t* aop) {
+                       float eps, float* mixed, float* inj, const HcRoute* route, int comb_parts, const AopOut* aop) {
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: t = %d outside 1..8", t);
   if (comb_parts != 1 && !(comb_parts == PYRE_GEMV_PARTS && h.di.fmt == FMT_IQ3_S && comb_out && !comb_moe)) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: %d partial vectors (1, or %d with an IQ3_S mix)", comb_parts, PYRE_GEMV_PARTS);
   if (route && !pyre_hc_route_ok(h, route->router)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: this router cannot ride on the mix");
@@ -606,6 +622,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   DownPlan p = down_plan(h);
   if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
   const bool on_m = hc_on_matrix_cores(h);
+  if (aop && !(on_m && aop->op && aop->ainv && aop->nsb >= 1 && h.hc <= 4)) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: only the matrix-core mix leaves an operand (pyre_hc_aop_ok)");
   MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
   if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);
   if (on_m) {
@@ -613,7 +630,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
     return up_mix_m(ctx, h, w, hc_m_slices(h), t, x_out, eps, mixed, inj, route, aop);
   }
   int rc = norm_down(ctx, h, w, p, x_in, in_ss, in_ts, x_out, t, comb_out, comb_parts, mo, comb_inj, eps); if (rc) return rc;
-  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route, aop);
+  return up_mix(ctx, h, w, p.ksplit, t, x_out, eps, mixed, inj, route);
 }
 
 int pyre_hc_combine_launch(pyre_ctx* ctx, int d, int hc, float* x, int t, const float* out, const float* inj) {

@@ -16,6 +16,7 @@ struct Layer {
   AttnDev attn{}; GdnDev gdn{}; MoeDev moe{}; QsaDev qsa{};
   bool ple = false; PleDev pld{}; int ple_index = 0;      // per-layer n-gram embeddings in front of the layer (ring pointer lives in the state)
   int mix_index = 0;         // index among the attention or among the DeltaNet layers
+  float gdn_up = 1.0f; const float* gdn_ainv = nullptr;      // DeltaNet: the power of two its output is scaled by as the f16 operand of ssm_out, and the [super-block][8] array of its inverse
 };
 
 }  // namespace
@@ -35,6 +36,7 @@ struct pyre_model {
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
   PleCfg plc{}; QMatDev ple_tab{}; PleWork pw{}; int n_ple = 0, ple_ring = 0;      // PLE: hash parameters, the token table, window workspace, ring rows per layer
   uint16_t* aop = nullptr;      // the f16 operand a producer kernel leaves for the matrix-core GEMV that follows it (one at a time: the launches are stream-ordered)
+  float* aop_inv = nullptr;     // [super-blocks][8]: the inverse of the power of two the hyper-connection mix scaled each token of that operand by
   PromptPipe* pipe = nullptr;      // further window workspaces and streams for a long prompt (prompt_pipe), made at the first one
 };
 
@@ -138,7 +140,7 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
   const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(ple_b) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(4 * 8 * (size_t)((kmax + 255) / 256)) + al256(ple_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
@@ -146,7 +148,7 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
-  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b);
+  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b); m->aop_inv = (float*)take(4 * 8 * (size_t)((kmax + 255) / 256));
   if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
   PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
   if (kmax_out) *kmax_out = kmax;
@@ -216,6 +218,16 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
       L.gdn = GdnDev{nullptr, nullptr, nullptr, nullptr, c.lin_nk, c.lin_nv, c.lin_dk, c.lin_dv, c.conv_k, c.eps};
       if ((rc = B.vec(T[PYRE_T_SSM_A], c.lin_nv, &L.gdn.a)) || (rc = B.vec(T[PYRE_T_SSM_DT_BIAS], c.lin_nv, &L.gdn.dt)) ||
           (rc = B.vec(T[PYRE_T_SSM_CONV1D], (size_t)m->ch * c.conv_k, &L.gdn.conv_w)) || (rc = B.vec(T[PYRE_T_SSM_NORM], c.lin_dv, &L.gdn.norm_w))) return rc;
+      {      // the layer's output as an f16 operand: |o_i * rms scale * w_i * sigmoid(z_i)| <= sqrt(dv) * max |w|, brought into [2^13, 2^14) by a power of two
+        std::vector<float> nw(c.lin_dv); PYRE_HIP(ctx, hipMemcpy(nw.data(), L.gdn.norm_w, (size_t)c.lin_dv * 4, hipMemcpyDeviceToHost));
+        float mx = 0.0f; bool fin = true; for (float v : nw) { if (!(fabsf(v) <= 3.0e38f)) fin = false; mx = fmaxf(mx, fabsf(v)); }
+        const float bound = sqrtf((float)c.lin_dv) * mx; int e = 0;
+        if (fin && bound > 0.0f) { uint32_t bits; memcpy(&bits, &bound, 4); e = 140 - (int)((bits >> 23) & 0xFF); e = e > 100 ? 100 : (e < -100 ? -100 : e); }
+        L.gdn_up = ldexpf(1.0f, e);
+        const int nsb = (c.lin_nv * c.lin_dv + 255) / 256; std::vector<float> inv((size_t)nsb * 8, ldexpf(1.0f, -e));
+        float* dv = nullptr; PYRE_HIP(ctx, hipMalloc((void**)&dv, inv.size() * 4)); m->bufs.push_back(dv);
+        PYRE_HIP(ctx, hipMemcpy(dv, inv.data(), inv.size() * 4, hipMemcpyHostToDevice)); L.gdn_ainv = dv;
+      }
     }
     MoeDev& mo = L.moe; size_t router_b = 0, ge = 0, ue = 0, de = 0, sh = 0;
     if ((rc = B.one(T[PYRE_T_FFN_GATE_INP], &mo.router, &router_b)) || (rc = B.one(T[PYRE_T_FFN_GATE_EXPS], &mo.gate_e, &ge)) || (rc = B.one(T[PYRE_T_FFN_UP_EXPS], &mo.up_e, &ue)) ||
@@ -521,9 +533,15 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
   }
   const bool fuse_aop = [] { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }();      // 1: separate split launches instead of the producers' own operand stores
-  const PyreAop aop{(const uint4*)m->aop, nullptr};
-  auto opnd = [&](const QMatDev& q) -> const PyreAop* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? &aop : nullptr; };
-  auto opw = [&](const QMatDev& q) -> uint16_t* { return fuse_aop && q.fmt == FMT_IQ3_S_M ? m->aop : nullptr; };
+  // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
+  // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
+  // own split launch (its magnitude has no bound a single workgroup of the merge could form)
+  const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
+  const AopOut aout{m->aop, m->aop_inv, d / 256};
+  auto hc_fused = [&](const HcDev& h, const QMatDev& q) { return fuse_aop && q.fmt == FMT_IQ3_S_M && q.cols == d && d % 256 == 0 && pyre_hc_aop_ok(h); };
+  auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
+  auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
+  auto gdn_fused = [&](const Layer& L) { return fuse_aop && L.outp.fmt == FMT_IQ3_S_M && L.gdn_ainv != nullptr; };
   for (int il = 0; il < c.n_layers; ++il) {
     const Layer& L = m->layers[il];
     if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
@@ -532,26 +550,27 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       if ((rc = pyre_ple_launch(ctx, m->plc, pd, m->pw, d, hc, c.eps, xin, in_ss, in_ts, xout, comb_out, comb_moe, comb_inj, start, o.step_dev, t))) return rc;
       advance(); comb_out = nullptr; comb_moe = nullptr; comb_inj = nullptr;
     }
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.proj)))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.hca, L.proj)))) return rc;
     advance(); comb_np = 1;
     // the layer's state (cache, recurrent state, saved projection) is the previous window's until that window has left it
     if (o.wait_ev) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));
     if (L.full) {
       int ai = L.mix_index;
-      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.proj)))) return rc;
+      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.hca, L.proj)))) return rc;
       if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
-      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr, opw(L.outp)))) return rc;
+      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
-      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.proj)))) return rc;
-      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, opw(L.outp)))) return rc;
+      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.hca, L.proj)))) return rc;
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, gdn_fused(L) ? m->aop : nullptr, L.gdn_up))) return rc;
       s->cur[li] = nb;
     }
     if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
-    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc; }
-    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, opnd(L.outp)))) return rc;
+    const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}; const PyreAop* oa = (!L.full && gdn_fused(L)) ? &aop_gdn : nullptr;
+    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc; }
+    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc;
     const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
     HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
@@ -573,7 +592,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   if (o.head_tokens == 0 && !want_r) return PYRE_OK;       // prompt window whose logits nobody reads
   if (o.head_tokens >= t || want_r) {
     const bool all = o.head_tokens >= t;
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, comb_np, all ? opw(m->out) : nullptr))) return rc;
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, comb_np, all ? opw(m->head, m->out) : nullptr))) return rc;
     if (want_r) {
       const int w = hc * d;
       hipLaunchKernelGGL(k_ring_store, dim3((w + 255) / 256, t - o.keep_from), dim3(256), 0, ctx->stream, xout, s->r_ring, s->r_mask, start, o.step_dev, o.keep_from, w); PYRE_CHECK_LAUNCH(ctx);
@@ -581,15 +600,15 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     }
     if (o.head_tokens == 0) return PYRE_OK;
     if (!all) return pyre_gemv_launch(ctx, m->out, m->hbuf + (size_t)(t - 1) * d, 1, m->logits);      // the last token's logits only
-    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->out));
-    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->out));
+    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
+    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->head, m->out));
   }
   // last token only: fold the pending ffn output into its streams, then the head
   const size_t last = (size_t)(t - 1) * hc * d;
   MoeOut mol{}; if (comb_moe) mol = pyre_moe_out(m->layers.back().moe, m->mw, t - 1);
-  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->out)))) return rc;
-  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->out));
-  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits, opnd(m->out));
+  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->head, m->out)))) return rc;
+  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
+  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits, opnd(m->head, m->out));
 }
 
 int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
@@ -1040,7 +1059,7 @@ int pyre_mtp_draft(pyre_ctx* ctx, const pyre_mtp* m, pyre_state* s, uint32_t pen
     if ((rc = mtp_cells(ctx, m, r, mask, rpos, 1))) return rc;
     QsaWork qw{}; qw.plist = s->mlist + (c0j[j] - lo0); qw.pcount = s->mcount + j; qw.list_stride = window;
     int packed = 0;
-    if ((rc = pyre_attn_launch_sel(ctx, m->attn, s->mkv, s->aw, m->proj, m->pw, pos, 1, &packed, m->core, nullptr, &qw, nullptr))) return rc;
+    if ((rc = pyre_attn_launch_sel(ctx, m->attn, s->mkv, s->aw, m->proj, m->pw, pos, 1, &packed, m->core, nullptr, &qw))) return rc;
     if ((rc = pyre_gemv_launch(ctx, m->outp, m->core, 1, m->bo))) return rc;
     if ((rc = pyre_hc_mix_launch(ctx, m->hcf, m->hw, m->ra, d, hc * d, m->rb, 1, m->bo, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, nullptr, 1, nullptr))) return rc;
     if ((rc = pyre_moe_launch(ctx, m->moe, m->mw, m->mixed, 1, m->y, nullptr))) return rc;

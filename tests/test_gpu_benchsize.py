@@ -100,6 +100,47 @@ def test_twelve_layer_full_width_greedy_stream_matches_oracle(ctx):
     gs.close(); gm.close()
 
 
+def test_all_48_layers_full_width_greedy_stream_matches_oracle(ctx, capsys):
+    # the benchmark's own depth and width: 48 layers (36 Gated DeltaNet + 12 attention, 512 experts each), an 8-token prompt
+    # and 16 greedy tokens against the oracle's token loop on the same weights (generated on the device, downloaded once)
+    def say(msg):
+        with capsys.disabled():
+            print(msg, flush=True)
+    cfg = mg.a3b_config(n_layers=48)
+    layers, globals_, raw = mg.build_device(ctx, cfg, seed=23)
+    gm = lib.Model(ctx, cfg, layers, globals_)
+    say("\n48-layer model on the device; downloading the weights for the oracle")
+    hl, hg = host_weights_from_device(ctx, cfg, layers, globals_)
+    for p in raw:
+        ctx.free(p)
+    lt = []
+    for il in range(cfg.n_layers):
+        for slot in range(mg.LAYER_SLOTS):
+            e = hl[il].get(slot)
+            lt.append(orc.tensor(*e) if e is not None else orc.Tensor(0, 0, 0, None))
+    om = orc.Model(orc_cfg(cfg), lt, [orc.tensor(*hg[s]) if s in hg else orc.Tensor(0, 0, 0, None) for s in range(mg.GLOBAL_SLOTS)], threads=THREADS, keep=(hl, hg))
+    prompt = rnd(24).integers(0, cfg.vocab, 8, dtype=np.uint32)
+    gs, os_ = gm.new_state(64), om.new_state()
+    lg, lo = gm.forward(prompt, gs), om.forward(prompt, os_)
+    say("prompt done: logits rel err %.3e" % relerr(lg, lo))
+    worst = relerr(lg, lo); rows = []
+    for i in range(16):
+        tg, to = int(orc.argmax(lg)), int(orc.argmax(lo))
+        top2 = np.partition(lo, -2)[-2:]; margin = float(top2[1] - top2[0]); dl = float(np.abs(lg - lo).max())
+        rows.append((i, to, margin, dl))
+        assert tg == to, "token %d: device %d, oracle %d, oracle top-2 margin %.3e, max |dlogit| %.3e" % (i, tg, to, margin, dl)
+        tok = np.array([to], dtype=np.uint32)
+        lg, lo = gm.forward(tok, gs), om.forward(tok, os_)
+        worst = max(worst, relerr(lg, lo))
+        if i % 4 == 3:
+            say("  %d tokens identical, worst logits rel err so far %.3e" % (i + 1, worst))
+    say("48-layer full-width greedy stream: token, id, oracle top-2 margin, max |dlogit|")
+    for r in rows:
+        say("  %2d %6d  %.3e  %.3e" % r)
+    assert worst <= 1e-3
+    gs.close(); gm.close()
+
+
 def test_device_loop_equals_host_loop_beyond_32k_context(ctx):
     # one layer group (3 Gated DeltaNet + 1 attention layer) at full width with a 32 800-token prompt: the replayed
     # device-resident step (positions read from device memory, packing check folded into the prep launch) against the

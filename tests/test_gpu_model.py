@@ -298,6 +298,45 @@ def test_matrix_core_hyper_connection_mixes_windows_equal_steps_and_the_oracle(c
         assert relerr(lr, lo) <= 1e-3 and relerr(lr, la) <= 1e-3 and int(np.argmax(lr)) == int(np.argmax(la))
 
 
+@pytest.mark.parametrize("scale,mixes", [(1.0e5, False), (1.0e4, False), (1.0e5, True), (1.0e-6, True), (1.0e-9, True)])
+def test_large_and_tiny_activations_through_the_producer_operands(ctx, scale, mixes):
+    # The kernels that produce a matrix-core GEMV's input (attention-side mix -> projections, Gated DeltaNet -> ssm_out,
+    # head mix -> vocabulary head) leave it as that GEMV's f16 operand, every token scaled by a power of two.  With the
+    # DeltaNet norm weights and the head's norm weights (and, `mixes`, the attention-side hyper-connection norm weights)
+    # multiplied by 1e5 .. 1e-9 those inputs leave the range an unscaled f16 half could hold (65504 overflows, below 6e-5
+    # loses bits): the logits must be finite and the oracle's, and a window must still equal single steps bit for bit.
+    # (Large hyper-connection norm weights also saturate the mixes' sigmoid gates, which makes the network itself
+    # ill-conditioned -- the oracle's f32 evaluation and any other f32 evaluation part by percents, with the operand split
+    # exactly as with the producers' operands -- so that case checks finiteness and the bit equality only.)
+    c = small_cfg(d=512, hc=4, hc_lr=256, qtype=synth.IQ3_S, hc_type=synth.IQ3_S, n_layers=4)
+    hw = mg.build_host(c, seed=29)
+    def mul(e):
+        ty, rows, cols, b = e; assert ty == synth.F32
+        return (ty, rows, cols, (b.view(np.float32) * np.float32(scale)).view(np.uint8).copy())
+    for L in hw.layers:
+        if mixes: L[mg.HCA_NORM] = mul(L[mg.HCA_NORM])
+        if mg.LIN_NORM in L: L[mg.LIN_NORM] = mul(L[mg.LIN_NORM])
+    hw.globals_[mg.G_HEAD_NORM] = mul(hw.globals_[mg.G_HEAD_NORM])
+    gm = lib.Model(ctx, c, hw.layers, hw.globals_); om = orc_model(hw)
+    well_conditioned = not (mixes and scale > 1.0)
+    g = np.random.Generator(np.random.PCG64(30))
+    prompt = g.integers(0, c.vocab, 11, dtype=np.uint32)
+    sa, sb, so = gm.new_state(64), gm.new_state(64), om.new_state()
+    la = gm.forward(prompt, sa); gm.forward(prompt, sb); lo = om.forward(prompt, so)
+    assert np.isfinite(la).all() and np.isfinite(lo).all() and np.abs(la).max() > 0
+    if well_conditioned:
+        assert relerr(la, lo) <= 1e-3, relerr(la, lo)
+    for t in (5, 2):
+        toks = g.integers(0, c.vocab, t, dtype=np.uint32)
+        lv = gm.forward_multi(toks, sa)
+        singles = np.array([gm.forward(toks[i:i + 1], sb) for i in range(t)])
+        assert np.isfinite(lv).all() and np.array_equal(lv.view(np.uint32), singles.view(np.uint32)), t
+        lw = om.forward_multi(toks, so)
+        if well_conditioned:
+            assert relerr(lv, lw) <= 1e-3, t
+    sa.close(); sb.close(); gm.close()
+
+
 def test_drafted_generation_identical_to_plain_and_to_oracle(ctx):
     c = small_cfg()
     hw, gm, om = pair(ctx, c, 8)

@@ -117,7 +117,7 @@ def test_gemv_sweep_shapes(ctx, ty, rows, cols):
     raw = synth.matrix(ty, rows, cols, 41 + ty)
     m = lib.QMat(ctx, ty, rows, cols, raw)
     W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
-    for t in (1, 4, 8):
+    for t in (1, 2, 4, 8):
         x = synth.normal((t, cols), 51 + t)
         assert relerr(m.matmul(x), x.astype(np.float64) @ W.T) <= TOL, t
 

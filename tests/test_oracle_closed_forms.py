@@ -269,3 +269,34 @@ def test_forward_with_one_live_deltanet_layer_is_mix_projections_core_out_combin
         x1 = orc.hc_combine(c.d, c.hc, x, o, inj).reshape(1, -1)
         assert np.abs(o).max() > 0 and np.array_equal(lg, head_of(c, hw, x1)), tok
     assert np.array_equal(st.ssm(0), ssm) and np.array_equal(st.conv(0), conv)
+
+
+def test_forward_with_one_live_attention_layer_is_mix_projections_core_out_combine():
+    # only layer 3's gated attention writes to the streams (every FFN and every DeltaNet output projection is zeroed): over
+    # three tokens the logits are head(combine(tile(e), attn_output(attn_core(q, k, v over the layer's own cache)), inject))
+    # with the attention-side mix, the [q ; k ; v] projections of the mixed vector, the cache carried across the tokens and
+    # the token's own position -- from the block entry points pinned in test_oracle_blocks.py.
+    c, hw = tiny_model(34, zero_slots=(mg.LIN_OUT, mg.DOWN_E, mg.SH_DOWN))
+    m = orc_model(hw); st = m.new_state()
+    L = hw.layers[3]; assert mg.ATTN_O in L
+    row = c.n_kv * c.hd
+    K = np.zeros((16, row), np.float32); V = np.zeros((16, row), np.float32)
+    inv = orc.rope_inv(c.n_rot, c.rope_base)
+    mm = lambda s, x: orc.matmul(L[s][0], L[s][3], L[s][1], L[s][2], x)
+    for pos, tok in enumerate((5, 250, 77)):
+        lg = m.forward(np.array([tok], dtype=np.uint32), st)
+        x = np.tile(embedding(c, hw, tok), c.hc)[None]
+        mixed, inj = orc.hc_mix(c.d, c.hc, c.eps, hw.f32(3, mg.HCA_NORM), orc_tensor(L[mg.HCA_DOWN]), orc_tensor(L[mg.HCA_INJECT]), orc_tensor(L[mg.HCA_UP]), x)
+        q, k, v = mm(mg.ATTN_Q, mixed), mm(mg.ATTN_K, mixed), mm(mg.ATTN_V, mixed)
+        oa = orc.attn_core(c.n_head, c.n_kv, c.hd, c.n_rot, c.eps, inv, hw.f32(3, mg.ATTN_QN), hw.f32(3, mg.ATTN_KN), q, k, v, pos, c.kv_bits, c.kv_recent, K, V)
+        o = mm(mg.ATTN_O, oa)
+        x1 = orc.hc_combine(c.d, c.hc, x, o, inj).reshape(1, -1)
+        assert np.abs(o).max() > 0 and np.array_equal(lg, head_of(c, hw, x1)), pos
+        # the FFN-side mixer's inject factors, or a cache that forgot the earlier tokens, give something else
+        _, inj_f = orc.hc_mix(c.d, c.hc, c.eps, hw.f32(3, mg.HCF_NORM), orc_tensor(L[mg.HCF_DOWN]), orc_tensor(L[mg.HCF_INJECT]), orc_tensor(L[mg.HCF_UP]), x)
+        assert not np.array_equal(lg, head_of(c, hw, orc.hc_combine(c.d, c.hc, x, o, inj_f).reshape(1, -1)))
+        if pos > 0:
+            K0 = np.zeros_like(K); V0 = np.zeros_like(V)
+            o0 = mm(mg.ATTN_O, orc.attn_core(c.n_head, c.n_kv, c.hd, c.n_rot, c.eps, inv, hw.f32(3, mg.ATTN_QN), hw.f32(3, mg.ATTN_KN), q, k, v, 0, c.kv_bits, c.kv_recent, K0, V0))
+            assert not np.array_equal(o0, o)
+    assert np.array_equal(st.kcache(0).reshape(-1, row)[:3], K[:3]) and np.array_equal(st.vcache(0).reshape(-1, row)[:3], V[:3])
