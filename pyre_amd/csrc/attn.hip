@@ -5,6 +5,7 @@
 #include "formats.h"
 
 __device__ __forceinline__ float a_sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
+PYRE_TS_DECL(attn_ts) PYRE_TS_EXPORT(attn_ts, pyre_debug_ts_attn)
 
 size_t pyre_packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 4 || n <= (size_t)recent + 64) return 0; return ((n - recent) / 64) * 64; }
 
@@ -58,9 +59,7 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
   const int half = a.n_rot / 2, ri = tid < half ? tid : tid - half;
   const float nwt = is_k ? a.kn[tid] : a.qn[tid], rinv = tid < a.n_rot ? a.rope_inv[ri] : 0.0f;
   const float vrow = is_k ? row[(size_t)a.nh * 2 * HD + (size_t)a.nkv * HD + (size_t)h * HD + tid] : 0.0f;
-  float ss = v * v;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  float ss = wave_sum(v * v);
   if ((tid & 63) == 0) red[tid >> 6] = ss;
   __syncthreads();
   float tot = 0.0f;
@@ -123,6 +122,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   __shared__ float red[4 * CH * NC];          // phase 1: [dq][position][column];  phase 3: [pw][column][dim]
   __shared__ float sc[CH][NC];
   __shared__ float wmax[NPW][NC], wsum[NPW][NC], cm[NC];
+  PYRE_TS_VARS PYRE_TS(0);
   const int chunk = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
@@ -146,6 +146,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
       vsc[s] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
     }
   }
+  PYRE_TS(1);
   // ---- phase 1
   {
     f4v D[4];
@@ -204,7 +205,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
       vf4[s] = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
     }
   }
-  __syncthreads();
+  PYRE_TS(2);
+  __syncthreads(); PYRE_TS(3);
   // ---- phase 2: this thread's position is pw*64 + lane, its columns are dq, dq + 4, dq + 8, dq + 12
   const int pos = pw * 64 + lane;
   constexpr int GH = (NC + 3) / 4;
@@ -216,9 +218,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
       const bool valid = p < start + tk0 + c / G + 1;          // the column's token sees positions below its own + 1
       float v = ((red[((size_t)0 * CH + pos) * NC + c] + red[((size_t)1 * CH + pos) * NC + c]) + red[((size_t)2 * CH + pos) * NC + c]) + red[((size_t)3 * CH + pos) * NC + c];
       sv[gi] = valid ? v * scale : -INFINITY;
-      float m = sv[gi];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      const float m = wave_max(sv[gi]);
       if (lane == 0) wmax[pw][c] = m;
     }
   }
@@ -231,13 +231,11 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
     if (c < ncol) {
       const bool valid = p < start + tk0 + c / G + 1;
       float e = valid ? expf(sv[gi] - cm[c]) : 0.0f; sc[pos][c] = e;
-      float l = e;
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+      const float l = wave_sum(e);
       if (lane == 0) wsum[pw][c] = l;
     }
   }
-  __syncthreads();   // weights of every position visible; the score partials in `red` are dead
+  __syncthreads(); PYRE_TS(4);   // weights of every position visible; the score partials in `red` are dead
   // ---- phase 3
   {
     f4v D[4];
@@ -272,7 +270,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
         for (int r = 0; r < 4; ++r) red[((size_t)pw * NC + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
     }
   }
-  __syncthreads();
+  PYRE_TS(5);
+  __syncthreads(); PYRE_TS(6);
   for (int i = tid; i < ncol * HD; i += NT) {
     const int c = i / HD, dd = i % HD, tk = tk0 + c / G, g = c % G;
     float o = red[((size_t)0 * NC + c) * HD + dd];
@@ -285,6 +284,10 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
     float* ml = part_ml + (((size_t)(tk0 + tid / G) * a.nh + (size_t)kvh * G + tid % G) * max_chunks + chunk) * 2;
     ml[0] = cm[tid]; ml[1] = l;
   }
+#ifdef PYRE_PHASE_TS
+  PYRE_TS(7);
+  if (tid == 0 && blockIdx.y == 0 && blockIdx.z == 0 && (chunk == 0 || chunk == (n - 1) / CH)) { for (int q_ = 0; q_ < 8; ++q_) attn_ts[(chunk == 0 ? 0 : 8) + q_] = ts_[q_]; }
+#endif
 }
 
 // The same kernel over a position list: entry i of plist[ti] (pcount[ti] entries, ascending positions) takes the place of
@@ -385,9 +388,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
     if (g < G) {
       float v = ((red[((size_t)0 * CH + pos) * G + g] + red[((size_t)1 * CH + pos) * G + g]) + red[((size_t)2 * CH + pos) * G + g]) + red[((size_t)3 * CH + pos) * G + g];
       sv[gi] = valid ? v * scale : -INFINITY;
-      float m = sv[gi];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      const float m = wave_max(sv[gi]);
       if (lane == 0) wmax[pw][g] = m;
     }
   }
@@ -399,9 +400,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
     const int g = dq + 4 * gi;
     if (g < G) {
       float e = valid ? expf(sv[gi] - cm[g]) : 0.0f; sc[pos][g] = e;
-      float l = e;
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+      const float l = wave_sum(e);
       if (lane == 0) wsum[pw][g] = l;
     }
   }
@@ -490,6 +489,7 @@ template <int HD>
 __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                       int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
   constexpr int CB = 320, B = CB / 4;
+  PYRE_TS_VARS PYRE_TS(0);
   __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[CB], ls[CB];
   if (posp) start = *posp;
   const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid >> 6, dd = blockIdx.z * 64 + (tid & 63);
@@ -504,8 +504,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   if (tid < nc) { m0 = ml[2 * tid]; l0 = ml[2 * tid + 1]; }
   if (tid < CB - 256 && 256 + tid < nc) { m1 = ml[2 * (256 + tid)]; l1 = ml[2 * (256 + tid) + 1]; }
   float M = m0; for (int c = tid + 256; c < nc; c += 256) M = fmaxf(M, ml[2 * c]);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  M = wave_max(M);
   if ((tid & 63) == 0) wmax[tid >> 6] = M;
   __syncthreads();
   M = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
@@ -532,6 +531,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
     const float ov = (o / L) * a_sigm(gate);
     out[((size_t)ti * a.nh + h) * HD + dd] = ov;
   }
+  PYRE_TS(1); PYRE_TS(2); PYRE_TS(3); PYRE_TS(4); PYRE_TS(5); PYRE_TS(6); PYRE_TS(7); PYRE_TS_FLUSH(attn_ts, 16);
 }
 
 size_t pyre_kv_bytes(const AttnDev& a, int cap) {

@@ -66,6 +66,25 @@ struct ProfScope {
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 #endif
 
+#ifdef __HIPCC__
+// Wave-wide sum / maximum on the data-parallel-primitive path: four steps inside each row of sixteen lanes (quad swaps, half
+// mirror, mirror: every lane then holds its row's value), two row broadcasts, one lane read -- seven short instructions
+// where six __shfl_xor steps are six trips through the shared-memory crossbar.  Every lane gets the result.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float wave_dpp(float old, float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v += wave_dpp<0xB1, 0xf>(0.0f, v); v += wave_dpp<0x4E, 0xf>(0.0f, v); v += wave_dpp<0x141, 0xf>(0.0f, v); v += wave_dpp<0x140, 0xf>(0.0f, v);
+  v += wave_dpp<0x142, 0xa>(0.0f, v); v += wave_dpp<0x143, 0xc>(0.0f, v);          // lane 15 of rows 0, 2 into rows 1, 3; lane 31 into rows 2, 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, wave_dpp<0xB1, 0xf>(v, v)); v = fmaxf(v, wave_dpp<0x4E, 0xf>(v, v)); v = fmaxf(v, wave_dpp<0x141, 0xf>(v, v)); v = fmaxf(v, wave_dpp<0x140, 0xf>(v, v));
+  v = fmaxf(v, wave_dpp<0x142, 0xa>(v, v)); v = fmaxf(v, wave_dpp<0x143, 0xc>(v, v));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+#endif
+
 extern thread_local std::string g_pyre_create_err;
 
 int pyre_fail(pyre_ctx* ctx, int code, const char* fmt, ...);

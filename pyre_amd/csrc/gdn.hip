@@ -56,10 +56,7 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) S[r] = sin_[(size_t)(grp * R + r) * DV + j];
-  auto wsum = [](float x) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
-    return x; };
+  auto wsum = [](float x) { return wave_sum(x); };
   if (wave < t) {          // L2 norms of q and k (:1649-1651): the sum of each half of the vector, then the two halves
     const float sq = wsum(q0 * q0) + wsum(q1 * q1), sk = wsum(k0 * k0) + wsum(k1 * k1);
     const float fq = (1.0f / sqrtf(sq + 1e-6f)) * (1.0f / sqrtf((float)DK)), fk = (1.0f / sqrtf(sk + 1e-6f)) * 1.0f;

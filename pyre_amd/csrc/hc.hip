@@ -294,8 +294,7 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
     float ss = v[t] * v[t]; xs[t] = v[t] * nv;
     if (tile == 0) x_out[((size_t)t * hc + s) * d + i0 + tid] = v[t];
     float a = fabsf(xs[t]); a = a == a ? a : INFINITY;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { ss += __shfl_xor(ss, o); a = fmaxf(a, __shfl_xor(a, o)); }
+    ss = wave_sum(ss); a = wave_max(a);
     if (lane == 0) { wsum[wave][t] = ss; wmax[wave][t] = a; }
   }
 #pragma unroll
@@ -432,8 +431,11 @@ template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(Q
   }
   PYRE_TS(1);
   lds_barrier(); PYRE_TS(2);
+  const bool hc_p2 = (hc & (hc - 1)) == 0; const float rhc = 1.0f / (float)hc;          // a power-of-two stream count: the division is a multiplication, bit for bit
   auto put_lo = [&](int t, int i, const float (&pv)[16]) {
-    const float v = hc_slice_sum16(pv, sls + t * 16, ksplit) / (float)hc, lv = v * sigm(v);
+    const float sv = hc_slice_sum16(pv, sls + t * 16, ksplit); float v;
+    if (hc_p2) v = sv * rhc; else v = sv / (float)hc;
+    const float lv = v * sigm(v);
     lo[t * lr + i] = lv; float a = fabsf(lv); a = a == a ? a : INFINITY; atomicMax(&lmax[t], __float_as_uint(a)); };
   if (ia < n_lo) put_lo(ta, ra, pva);
   if (ib < n_lo) put_lo(tb, rb, pvb);
