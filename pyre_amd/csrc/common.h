@@ -245,19 +245,23 @@ struct MoeOut { const float* partial; const float* sel_w; const float* sg; int d
 static_assert(PYRE_MOE_GROUPS == PYRE_GEMV_PARTS, "the mix adds the group sums as it adds an output projection's K parts");
 #ifdef __HIPCC__
 // All loads are issued before the first add, so the value costs one memory round trip, not k + 1.
-__device__ __forceinline__ float moe_out_value(const MoeOut& mo, int ti, int r) {
-  const float* p = mo.partial + (size_t)ti * (mo.k + 1) * mo.d + r; const float* w = mo.sel_w + ti * mo.k;
-  float pv[PYRE_MOE_KMAX], wv[PYRE_MOE_KMAX];
+// FK > 0: the number of routed experts as a compile-time constant (the caller guarantees mo.k == FK): the loads and the
+// grouping carry no predicates; the arithmetic is the same.
+template <int FK = 0> __device__ __forceinline__ float moe_out_value(const MoeOut& mo, int ti, int r) {
+  const int k = FK ? FK : mo.k;
+  const float* p = mo.partial + (size_t)ti * (k + 1) * mo.d + r; const float* w = mo.sel_w + ti * k;
+  constexpr int KM = FK ? FK : PYRE_MOE_KMAX;
+  float pv[KM], wv[KM];
 #pragma unroll
-  for (int j = 0; j < PYRE_MOE_KMAX; ++j) { pv[j] = j < mo.k ? p[(size_t)j * mo.d] : 0.0f; wv[j] = j < mo.k ? w[j] : 0.0f; }
-  float sh = p[(size_t)mo.k * mo.d], g = mo.sg[ti];
-  const int gsz = (mo.k + 4) / 4;
+  for (int j = 0; j < KM; ++j) { pv[j] = j < k ? p[(size_t)j * mo.d] : 0.0f; wv[j] = j < k ? w[j] : 0.0f; }
+  float sh = p[(size_t)k * mo.d], g = mo.sg[ti];
+  const int gsz = (k + 4) / 4;
   float P[PYRE_MOE_GROUPS];
 #pragma unroll
   for (int q = 0; q < PYRE_MOE_GROUPS; ++q) {
     float o = 0.0f;
 #pragma unroll
-    for (int e = 0; e < PYRE_MOE_GMAX; ++e) { const int j = q * gsz + e; if (e < gsz && j < mo.k) o = fmaf(wv[j < PYRE_MOE_KMAX ? j : 0], pv[j < PYRE_MOE_KMAX ? j : 0], o); }
+    for (int e = 0; e < PYRE_MOE_GMAX; ++e) { const int j = q * gsz + e; if (e < gsz && j < k) o = fmaf(wv[j < KM ? j : 0], pv[j < KM ? j : 0], o); }
     P[q] = o;
   }
   P[PYRE_MOE_GROUPS - 1] = fmaf(sh, g, P[PYRE_MOE_GROUPS - 1]);

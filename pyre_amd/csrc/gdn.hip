@@ -32,13 +32,15 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj
 // the L2-normalised q and k, v, z, the decay and beta in shared memory) and after it (wave ti: RMSNorm and gate of token
 // ti's output).  A token of the recurrence itself costs one barrier:
 //   S *= g; mem = S^T k -> barrier -> delta = (v - mem) beta; S += k (x) delta; o = S^T q      (linear_core, :1655-1668)
-template <int DK, int DV>
+// FT, FNK, FNV > 0: the window width and the head counts as compile-time constants (the launcher checks them) -- same arithmetic.
+template <int DK, int DV, int FT = 0, int FNK = 0, int FNV = 0>
 __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
                                                    const float* __restrict__ ssm_in, float* __restrict__ ssm_out, float* __restrict__ out, uint16_t* __restrict__ aop, int aop_rows, float aop_up) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int G = 4, R = DK / G, MT = 8;
   PYRE_TS_VARS PYRE_TS(0);
   args_now(p.a, p.dt, p.norm_w, p.nk, p.nv, p.eps, proj, stride, t, co_all, ssm_in, ssm_out, out);
+  if constexpr (FT > 0) { t = FT; p.nk = FNK; p.nv = FNV; }
   __shared__ float qs[MT][DK], ks[MT][DK], vs[MT][DV], zs[MT][DV], pm[2][G][DV], po[MT][G][DV], gs[MT], bs[MT];
   const int h = blockIdx.x, kh = h % p.nk, tid = threadIdx.x, j = tid & (DV - 1), grp = tid >> 7, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -102,7 +104,8 @@ int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int strid
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: t = %d outside 1..8", t);
   int ch = 2 * g.nk * g.dk + g.nv * g.dv;
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); if (t == 1 && g.nk == 16 && g.nv == 32) hipLaunchKernelGGL((k_gdn_delta<128, 128, 1, 16, 32>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up);          // a single token of the A3B geometry: constants folded in
+    else hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

@@ -16,7 +16,7 @@ __device__ __forceinline__ float sigm(float x) { return 1.0f / (1.0f + expf(-x))
 // `out` is a plain [t][d] vector (comb_out) or the unreduced FFN output (mo.partial != nullptr).
 // NP > 1: `out` comes as NP partial vectors, part q of token ti at comb_out + (q*T + ti)*d, added in order from the first
 // (pyre_gemv_parts_launch); all parts are fetched before the first add.
-template <int T, int NP> __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, const MoeOut& mo, float w, int d, int ti, int s, int i) {
+template <int T, int NP, int FK = 0> __device__ __forceinline__ float hc_x_new(const float* __restrict__ x_in, int in_ss, int in_ts, const float* __restrict__ comb_out, const MoeOut& mo, float w, int d, int ti, int s, int i) {
   float v = x_in[(size_t)ti * in_ts + (size_t)s * in_ss + i];
   if constexpr (NP > 1) {
     float sv[NP];
@@ -27,7 +27,7 @@ template <int T, int NP> __device__ __forceinline__ float hc_x_new(const float* 
     for (int q = 1; q < NP; ++q) o += sv[q];
     v = v + o * w;
   } else {
-    if (mo.partial) v = v + moe_out_value(mo, ti, i) * w;
+    if (mo.partial) v = v + moe_out_value<FK>(mo, ti, i) * w;
     else if (comb_out) v = v + comb_out[(size_t)ti * d + i] * w;
   }
   return v;
@@ -269,7 +269,9 @@ __device__ __forceinline__ void hc_lds_a(const uint16_t* ah, int c, int lane, AB
 // grid (row tiles of [down ; inject], slices of 256*CS columns), 4*CS waves, a thread prepares one column of the slice.
 // Wave (p, g) takes row group g of the tile over chunk pair p of the slice; with CS = 2 the two pairs' sums meet in
 // shared memory (pair 0 + pair 1).  Outputs as k_hc_norm_down: ssq[ks*T + t], part[(ks*T + t)*tiles*64 + row], x_out.
-template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_hc_norm_down_m(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
+// FD, FK > 0: the model width d and the routed experts per token as compile-time constants (the launcher checks them): the
+// stream index of a slice is a shift, the gather of the unreduced FFN output carries no predicates -- same arithmetic.
+template <int T, int NP, int CS, int FD = 0, int FK = 0> __global__ __launch_bounds__(256 * CS) void k_hc_norm_down_m(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
     const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part, float* __restrict__ smx) {
   constexpr int NW = 4 * CS;
   __shared__ __align__(16) uint16_t ah[CS * 32 * 16 * 8];
@@ -278,13 +280,14 @@ template <int T, int NP, int CS> __global__ __launch_bounds__(256 * CS) void k_h
   qmat_args_now(m); args_now(x_in, in_ss, in_ts, x_out, comb_out, mo.partial, mo.sel_w, mo.sg, mo.d, mo.k, comb_inj, norm, d, hc, ssq, part);
   const int tile = blockIdx.x, ks = blockIdx.y, tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = wave & 3, p = wave >> 2;
+  if constexpr (FD > 0) d = FD;
   const int c0 = ks * 256 * CS, s = c0 / d, i0 = c0 - s * d, K128 = m.cols >> 7;
   float w[T], v[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) w[t] = (comb_out || mo.partial) ? 2.0f * sigm(comb_inj[t * hc + s]) : 0.0f;
   const float nv = norm[(size_t)s * d + i0 + tid];
 #pragma unroll
-  for (int t = 0; t < T; ++t) v[t] = hc_x_new<T, NP>(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid);
+  for (int t = 0; t < T; ++t) v[t] = hc_x_new<T, NP, FK>(x_in, in_ss, in_ts, comb_out, mo, w[t], d, t, s, i0 + tid);
   const int ch0 = ks * 2 * CS + 2 * p;
   WBuf<1> w0, w1; load_w<1>(m, tile * 4 + g, ch0, lane, K128, w0); load_w<1>(m, tile * 4 + g, ch0 + 1, lane, K128, w1);
   const NibK nk = nib_consts();
@@ -371,13 +374,16 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
 // (two rows of lo and one inject row a thread, the streams of one column a thread), and lo goes through shared memory
 // twice: f32, then as operand rows scaled per token by the power of two of its largest magnitude.  Operand rows no token
 // of the window owns are left as they are: a row only ever reaches its own sums.  A value's arithmetic does not depend on CW.
-template <int T, int RF> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
+// FHC, FLR, FKS > 0: the stream count, the low rank and the slice count as compile-time constants (the launcher checks
+// them): divisions become shifts, the slice loops lose their predicates -- same arithmetic.
+template <int T, int RF, int FHC = 0, int FLR = 0, int FKS = 0> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
     QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   const uint2* lds2 = nullptr;
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj, lcw);
+  if constexpr (FHC > 0) { hc = FHC; lr = FLR; ksplit = FKS; }
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, kps = ksplit / hc, nw = nthr >> 6, CW = 1 << lcw, lg = lcw - 4;
   float* lo = sm;                                 // [T][lr]
@@ -547,9 +553,16 @@ bool hc_on_matrix_cores(const HcDev& h) {
 template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
   ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
 #define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
-  if (hc_m_cs(h) == 2) { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 2); else NORM_DOWN_M_GO(1, 2); }
+#define NORM_DOWN_M_FIX(NP) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, 2, 2048, 10>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(512), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
+  bool done = false;
+  if constexpr (T == 1) {          // a single token at the width of the A3B configuration: the instance with its constants folded in
+    if (h.d == 2048 && (!mo.partial || mo.k == 10)) { if (comb_parts > 1) NORM_DOWN_M_FIX(PYRE_GEMV_PARTS); else NORM_DOWN_M_FIX(1); done = true; }
+  }
+  if (done) {}
+  else if (hc_m_cs(h) == 2) { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 2); else NORM_DOWN_M_GO(1, 2); }
   else { if (comb_parts > 1) NORM_DOWN_M_GO(PYRE_GEMV_PARTS, 1); else NORM_DOWN_M_GO(1, 1); }
 #undef NORM_DOWN_M_GO
+#undef NORM_DOWN_M_FIX
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 // columns of the mixed vector a workgroup of the matrix-core up / mix launch owns (log2): a single token without a riding
@@ -566,9 +579,18 @@ template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
-#define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0)
-  if (rt && rq.fmt == FMT_BF16) UP_MIX_M_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_GO(FMT_F32); else UP_MIX_M_GO(-1);
+#define UP_MIX_M_ARGS dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
+                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0
+#define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), UP_MIX_M_ARGS)
+#define UP_MIX_M_FIX(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF, 4, 256, 16>), UP_MIX_M_ARGS)
+  bool done = false;
+  if constexpr (T == 1) {          // a single token with four streams, a low rank of 256 and sixteen slices (the A3B configuration): constants folded in
+    if (h.hc == 4 && h.lr == 256 && ksplit == 16) { if (rt && rq.fmt == FMT_BF16) UP_MIX_M_FIX(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_FIX(FMT_F32); else UP_MIX_M_FIX(-1); done = true; }
+  }
+  if (done) {}
+  else if (rt && rq.fmt == FMT_BF16) UP_MIX_M_GO(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_GO(FMT_F32); else UP_MIX_M_GO(-1);
+#undef UP_MIX_M_FIX
+#undef UP_MIX_M_ARGS
 #undef UP_MIX_M_GO
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }

@@ -131,32 +131,36 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // at once instead of taking a second turn on the 256 compute units.
 // PRE: the token's experts were chosen by k_moe_route (windows of several tokens: hundreds of workgroups would each redo
 // the selection otherwise); the workgroup reads its expert id and publishes nothing but the shared-expert gate.
-template <int FMT, int NW, int P, bool PRE>
+// FIX: the A3B configuration's constants (512 experts, top 10, d = 2048 in 32 router slices, ff = 512) folded in at compile
+// time (the launcher checks them) -- same arithmetic.
+template <int FMT, int NW, int P, bool PRE, bool FIX = false>
 __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 8 : 1) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
                                                    const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
   args_now(m.n_exp, m.top_k, logits, nsl, sstride, tstride);          // what the selection needs; the rest would crowd the scalar registers the activations go through
+  const int n_exp = FIX ? 512 : m.n_exp, top_k = FIX ? 10 : m.top_k, d = FIX ? 2048 : m.d, ff = FIX ? 512 : m.ff;
+  if constexpr (FIX) nsl = 32;
   __shared__ float red[2][P][NW][64];
   __shared__ RouteLds rl;
-  const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
-  const bool shared = j == m.top_k;
-  const int nrows = shared ? m.sf : m.ff;
+  const int entry = blockIdx.y, k1 = top_k + 1, ti = entry / k1, j = entry % k1;
+  const bool shared = j == top_k;
+  const int nrows = shared ? m.sf : ff;
   if ((int)blockIdx.x * 64 >= nrows) return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const float* xs = x + (size_t)ti * m.d;
+  const float* xs = x + (size_t)ti * d;
   int expert = 0;
   if (!shared) {
-    if constexpr (PRE) expert = __builtin_amdgcn_readfirstlane(sel_idx[ti * m.top_k + j]);
-    else { route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl ROUTE_TS_ARG); expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]); }
+    if constexpr (PRE) expert = __builtin_amdgcn_readfirstlane(sel_idx[ti * top_k + j]);
+    else { route_topk(logits + (size_t)ti * tstride, nsl, sstride, n_exp, top_k, rl ROUTE_TS_ARG); expert = __builtin_amdgcn_readfirstlane(rl.s_idx[j]); }
   } else if (blockIdx.x == 0) {
     float p = 0.0f;
-    for (int ib = threadIdx.x; ib < m.d; ib += 4 * NW * 64) {          // four elements per pass, loads first (elements past d: weight zero)
+    for (int ib = threadIdx.x; ib < d; ib += 4 * NW * 64) {          // four elements per pass, loads first (elements past d: weight zero)
       float a[4], b[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) { const int ic = min(ib + u * NW * 64, m.d - 1); a[u] = m.sh_gate_inp[ic]; b[u] = xs[ic]; }
+      for (int u = 0; u < 4; ++u) { const int ic = min(ib + u * NW * 64, d - 1); a[u] = m.sh_gate_inp[ic]; b[u] = xs[ic]; }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) if (ib + u * NW * 64 < m.d) p = fmaf(a[u], b[u], p);
+      for (int u = 0; u < 4; ++u) if (ib + u * NW * 64 < d) p = fmaf(a[u], b[u], p);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) p += __shfl_xor(p, o);
@@ -167,22 +171,23 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
   }
   PYRE_TS(1);
   const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
-  const int tile = (shared ? 0 : expert * (m.ff >> 6)) + blockIdx.x;
-  const int nz = gridDim.z, kz = blockIdx.z, np = P * nz;          // np parts in all
-  const int upw = (G.U + NW * np - 1) / (NW * np);
+  const int tile = (shared ? 0 : expert * (ff >> 6)) + blockIdx.x;
+  const int nz = FIX ? 2 : (int)gridDim.z, kz = blockIdx.z, np = P * nz;          // np parts in all
+  const int GU = FIX ? 32 : G.U;          // 64-column units of a row (both matrices, routed or shared: d / 64)
+  const int upw = (GU + NW * np - 1) / (NW * np);
   float ag[P][1], au[P][1];
 #pragma unroll
   for (int p = 0; p < P; ++p) { ag[p][0] = 0.0f; au[p][0] = 0.0f; }
   if (P == 2 && upw == 1) {
     // one unit per part: both parts' units of both matrices are fetched before the first is consumed
-    const int ka = min(2 * wave, G.U - 1), kb = min(2 * wave + 1, G.U - 1);
+    const int ka = min(2 * wave, GU - 1), kb = min(2 * wave + 1, GU - 1);
     UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ka, lane), u0 = unit_load<FMT>(Up, tile, ka, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
-    if (2 * wave < G.U) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
-    if (2 * wave + 1 < G.U) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
+    if (2 * wave < GU) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
+    if (2 * wave + 1 < GU) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
   } else {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      const int k0 = min(G.U, (wave * np + kz * P + p) * upw), kend = min(G.U, k0 + upw);          // wave w's shares of the np parts are adjacent
+      const int k0 = min(GU, (wave * np + kz * P + p) * upw), kend = min(GU, k0 + upw);          // wave w's shares of the np parts are adjacent
       // two units of both matrices are fetched before the first is consumed: a rolled loop would pay a memory round trip per unit
       for (int ku = k0; ku < kend; ku += 2) {
         const int kb = min(ku + 1, kend - 1);
@@ -218,8 +223,8 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
   if (blockIdx.x == 0 && kz == 0) {
     if (shared) { if (threadIdx.x == 0) sg[ti] = rl.s_w[0]; }
     else if (!PRE && j == 0) {
-      route_weights(m.top_k, rl);       // thread e < k writes and then reads its own s_w entry
-      if (threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
+      route_weights(top_k, rl);       // thread e < k writes and then reads its own s_w entry
+      if ((int)threadIdx.x < top_k) { sel_idx[ti * top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
     }
   }
   PYRE_TS(4); PYRE_TS_FLUSH(moe_ts, 0);
@@ -241,20 +246,22 @@ __global__ __launch_bounds__(1024) void k_moe_route(MoeDev m, const float* __res
 // NZ > 1: h arrives as the gate / up sums of NZ K parts (k_moe_gu with gridDim.z = NZ); each wave forms the 64 values of
 // a unit, silu(sum of gate parts) * (sum of up parts), in its own slice of shared memory while the unit's weights are
 // on their way (a wave's shared-memory operations execute in order: no workgroup barrier).
-template <int FMT, int NW, int NZ>
+template <int FMT, int NW, int NZ, bool FIX = false>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
                                                      const uint2* __restrict__ g2) {
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, partial);
+  const int top_k = FIX ? 10 : m.top_k, d = FIX ? 2048 : m.d;          // FIX: the A3B configuration (top 10, d = 2048, routed and shared experts 512 wide), checked by the launcher
   __shared__ float red[NW][64];
   __shared__ float hx[NZ > 1 ? NW : 1][64];
-  const int entry = blockIdx.y, k1 = m.top_k + 1, ti = entry / k1, j = entry % k1;
-  const bool shared = j == m.top_k;
+  const int entry = blockIdx.y, k1 = top_k + 1, ti = entry / k1, j = entry % k1;
+  const bool shared = j == top_k;
   const QMatDev& D = shared ? m.sh_down : m.down_e;
-  const int tile = (shared ? 0 : sel_idx[ti * m.top_k + j] * (m.d >> 6)) + blockIdx.x;
+  const int tile = (shared ? 0 : sel_idx[ti * top_k + j] * (d >> 6)) + blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int upw = (D.U + NW - 1) / NW, k0 = wave * upw, kend = min(D.U, k0 + upw);
+  const int DU = FIX ? 8 : D.U;
+  const int upw = (DU + NW - 1) / NW, k0 = wave * upw, kend = min(DU, k0 + upw);
   float acc[1] = {0.0f};
   if constexpr (NZ == 1) {
     const float* xs = h + (size_t)entry * hstride;
@@ -284,7 +291,7 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
     float s = red[0][lane];
 #pragma unroll
     for (int w = 1; w < NW; ++w) s += red[w][lane];
-    partial[(size_t)entry * m.d + blockIdx.x * 64 + lane] = s;
+    partial[(size_t)entry * d + blockIdx.x * 64 + lane] = s;
   }
   PYRE_TS(3); PYRE_TS_FLUSH(moe_ts, 8);
 }
@@ -406,9 +413,11 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   const int P = pyre_moe_gu_parts(m), nz = (P > 1 && t == 1) ? P : 1;
+  const bool a3b = t == 1 && m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512;          // the instances with these constants folded in
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
 #define GU_GO(PP, NZ, PRE) MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP, PRE>), dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride))
-  if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
+  if (t == 1 && a3b && nsl == 32 && nz == 2) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true>), dim3(hs / 64, entries, 2), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride);
+  else if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
   else {
     hipLaunchKernelGGL(k_moe_route, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
     if (P == 2) { GU_GO(2, 1, true); } else { GU_GO(1, 1, true); }
@@ -422,6 +431,7 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
     if (gsz <= 3 && last <= 3) { DOWN_G_GO(3); } else { DOWN_G_GO(PYRE_MOE_GMAX); }
 #undef DOWN_G_GO
   }
+  else if (a3b && nz == 2) hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, true>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2);
   else if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
   else { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 2>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); } }
   PYRE_CHECK_LAUNCH(ctx);
