@@ -6,6 +6,11 @@
 
 __device__ __forceinline__ float a_sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
 PYRE_TS_DECL(attn_ts) PYRE_TS_EXPORT(attn_ts, pyre_debug_ts_attn)
+#ifdef PYRE_PHASE_TS
+// diagnostics build: start, end and hardware id of every workgroup of the last k_attn_decode launch
+__device__ unsigned long long attn_wg[4096 * 10];
+extern "C" int pyre_debug_attn_wg(unsigned long long* out) { return hipMemcpyFromSymbol(out, HIP_SYMBOL(attn_wg), sizeof(unsigned long long) * 4096 * 10) == hipSuccess ? 0 : -1; }
+#endif
 
 size_t pyre_packed_boundary(size_t n, int kv_bits, int recent) { if (kv_bits != 4 || n <= (size_t)recent + 64) return 0; return ((n - recent) / 64) * 64; }
 
@@ -41,9 +46,13 @@ template <int HD> __device__ __forceinline__ void kv_pack_thread(const AttnDev& 
 // Blocks past nkv + nh (single-token steps at a device-side position): the 64-position packing step that the growth
 // of the context by this token may make due (k_kv_pack's work, old positions only: it touches nothing the other
 // blocks write), so a replayed step does not spend a launch on a check that almost always finds nothing to do.
+// A query head also leaves as two f16 halves, q * 2^e = h1 + h2 (e: the head's largest magnitude lands in
+// [2^13, 2^14); elements below 2^-3 after scaling keep fewer than 22 bits, 2^-27 of the largest), with 2^-e in qsc: the operand of the packed-key product.  Within
+// each group of eight dims the halves are stored in the order 0 4 1 5 2 6 3 7, the order in which a 32-bit word of
+// eight 4-bit keys unpacks into f16 pairs.
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout) {
-  __shared__ float buf[HD]; __shared__ float red[HD / 64];
+__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout, uint16_t* __restrict__ qh, float* __restrict__ qsc) {
+  __shared__ float buf[HD]; __shared__ float red[HD / 64]; __shared__ float redm[HD / 64];
   if (posp) start = *posp;
   const int b = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, pos = start + ti;
   if (b >= a.nkv + a.nh) {
@@ -80,7 +89,23 @@ __global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const flo
   if (is_k) {
     kv.kf[kv_blk((size_t)h * HD + tid, (size_t)a.nkv * HD, pos)] = v;
     kv.vf[(size_t)pos * a.nkv * HD + (size_t)h * HD + tid] = vrow;
-  } else qout[((size_t)ti * a.nh + h) * HD + tid] = v;
+  } else {
+    qout[((size_t)ti * a.nh + h) * HD + tid] = v;
+    float am = fabsf(v); am = am == am ? am : INFINITY;
+    am = wave_max(am);
+    if ((tid & 63) == 0) redm[tid >> 6] = am;
+    __syncthreads();
+    float m = redm[0];
+#pragma unroll
+    for (int i = 1; i < HD / 64; ++i) m = fmaxf(m, redm[i]);
+    int e = 0;
+    if (m > 0.0f && m < INFINITY) { e = 140 - (int)((__float_as_uint(m) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+    const float xs = v * __uint_as_float((uint32_t)(127 + e) << 23);
+    const _Float16 h1 = (_Float16)xs, h2 = (_Float16)(xs - (float)h1);
+    uint16_t* o = qh + ((size_t)ti * a.nh + h) * 2 * HD + (tid & ~7) + ((tid & 3) * 2 + ((tid >> 2) & 1));
+    o[0] = __builtin_bit_cast(unsigned short, h1); o[HD] = __builtin_bit_cast(unsigned short, h2);
+    if (tid == 0) qsc[(size_t)ti * a.nh + h] = __uint_as_float((uint32_t)(127 - e) << 23);
+  }
 }
 
 // kv4::pack for positions [p0, p1): one thread per (position, 32-value block, K or V).
@@ -113,17 +138,37 @@ __device__ __forceinline__ float nib_val(uint32_t w, int i) { return (float)(((i
 // property of a token's view; when it moves inside a window (one window in 64 / t) the launch gives every token a pass
 // of its own (tp = 1).
 typedef float f4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h8v __attribute__((ext_vector_type(8)));
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+// lane 2 * q + O of the caller's row of sixteen lanes, for every lane of the row (q = 0..3 unrolled by the caller)
+template <int O> __device__ __forceinline__ int row_bcast(int v, int q) {
+  switch (q) { case 0: return __builtin_amdgcn_update_dpp(0, v, 0x150 + O, 0xf, 0xf, true); case 1: return __builtin_amdgcn_update_dpp(0, v, 0x150 + O + 2, 0xf, 0xf, true);
+    case 2: return __builtin_amdgcn_update_dpp(0, v, 0x150 + O + 4, 0xf, 0xf, true); default: return __builtin_amdgcn_update_dpp(0, v, 0x150 + O + 6, 0xf, 0xf, true); }
+}
+// eight 4-bit two's-complement fields of w -> eight f16 numbers in the order 0 4 1 5 2 6 3 7: field ^ 8 is the value + 8,
+// or-ed into the mantissa of 1024 it is the f16 number 1032 + value, and one packed subtraction leaves the value
+__device__ __forceinline__ h8v nib8_f16(uint32_t w) {
+  const uint32_t x = w ^ 0x88888888u;
+  const h2v off = {(_Float16)1032.0f, (_Float16)1032.0f};
+  struct U4 { uint32_t v[4]; } u;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) u.v[q] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2v, ((x >> (4 * q)) & 0x000F000Fu) | 0x64006400u) - off);
+  return __builtin_bit_cast(h8v, u);
+}
 // NC: columns the buffers hold -- G for launches of one token a pass (tp = 1), 16 otherwise.
 template <int HD, int G, int NC>
-__global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int t, int tp) {
+__global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev a, KvDev kv, const float* __restrict__ qbuf, const uint16_t* __restrict__ qh, const float* __restrict__ qsc, int start, const int* __restrict__ posp, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int t, int tp) {
   static_assert(HD == 256, "the wave layout assumes 4 x 64 head dims");
   constexpr int NPW = PYRE_ATTN_NPW, CH = PYRE_ATTN_CHUNK, NT = 256 * NPW;
   static_assert(4 * CH == NPW * HD, "the score and value partials share one buffer");
   __shared__ float red[4 * CH * NC];          // phase 1: [dq][position][column];  phase 3: [pw][column][dim]
-  __shared__ float sc[CH][NC];
+  __shared__ __align__(16) float sc[NC][CH + 4];          // [column][position]: eight consecutive positions of a column are two 16-byte reads
   __shared__ float wmax[NPW][NC], wsum[NPW][NC], cm[NC];
   PYRE_TS_VARS PYRE_TS(0);
-  const int chunk = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  // chunks in descending order: the workgroups past the view (a captured launch covers the whole cache) and the partly
+  // filled last chunk go first and free their slots at once; when the grid exceeds what the chip holds, the workgroups
+  // that wait are full ones either way, and they now wait for the short ones
+  const int chunk = (int)gridDim.x - 1 - (int)blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
   const int tk0 = blockIdx.z * tp, nk = min(tp, t - tk0), ncol = nk * G;          // tokens tk0 .. tk0+nk-1 in columns 0 .. ncol-1
@@ -137,44 +182,184 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   const bool packed = wbase < pb, active = wbase < n;
   const int ctok = li / G, chead = li - ctok * G;                                              // the lane's column: token of the pass, head of the group
   // The packed values do not depend on the scores: their loads go out with the keys', one memory round trip for both.
-  uint32_t vw[16]; float vsc[16];
-  if (active && packed) {
+  // Lane (li, lg) of the value product stands for two dims of a scale block (word li & 3, nibbles 2 * (li >> 2) + m) at
+  // the eight positions 8 * lg .. of a 32-position group: vw[g][b][p] is the word of position 32 * g + 8 * lg + p in block
+  // dq * 2 + b.  vsl[g]: the scale of position 32 * g + 8 * lg + (li & 7) in block dq * 2 + (li >> 3); the lanes of a row of
+  // sixteen hold the 8 x 2 scales the row needs and pass them round with row broadcasts.
+  // All of it through buffer descriptors: one 32-bit offset per array and lane, the rest of an address is a constant
+  // of the instruction or a scalar.
+  const int pos = pw * 64 + lane;
+  constexpr int GH = (NC + 3) / 4;
+  // chunk-local max / exp / sum per head; called by every wave after the barrier that follows its scores
+  auto softmax_phase = [&]() {
+    float sv[GH];
 #pragma unroll
-    for (int s = 0; s < 16; ++s) {
-      const size_t pg = (size_t)wbase + 4 * s + lg;
-      vw[s] = kv.vq[pg * (row / 8) + (size_t)kvh * (HD / 8) + dq * 8 + (li >> 1)];
-      vsc[s] = kv.vs[pg * (row / 32) + (size_t)kvh * (HD / 32) + dq * 2 + (li >> 3)];
-    }
-  }
-  PYRE_TS(1);
-  // ---- phase 1
-  {
-    f4v D[4];
-#pragma unroll
-    for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-    if (active) {
-      float B[16];
-      if (li < ncol) {
-        const float4* q4 = (const float4*)(qbuf + ((size_t)(tk0 + ctok) * a.nh + (size_t)kvh * G + chead) * HD + dq * 64 + 16 * lg);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) { float4 v = q4[j]; B[4 * j] = v.x; B[4 * j + 1] = v.y; B[4 * j + 2] = v.z; B[4 * j + 3] = v.w; }
-      } else {
-#pragma unroll
-        for (int s = 0; s < 16; ++s) B[s] = 0.0f;
+    for (int gi = 0; gi < GH; ++gi) {
+      const int c = dq + 4 * gi; sv[gi] = -INFINITY;
+      if (c < ncol) {
+        const bool valid = p < start + tk0 + c / G + 1;          // the column's token sees positions below its own + 1
+        float v = ((red[((size_t)0 * CH + pos) * NC + c] + red[((size_t)1 * CH + pos) * NC + c]) + red[((size_t)2 * CH + pos) * NC + c]) + red[((size_t)3 * CH + pos) * NC + c];
+        sv[gi] = valid ? v * scale : -INFINITY;
+        const float m = wave_max(sv[gi]);
+        if (lane == 0) wmax[pw][c] = m;
       }
-      if (packed) {             // the keys stay packed until the step that uses them: four values live, not sixty-four
-        uint32_t kw[4][2]; float ksc[4];
+    }
+    __syncthreads();
+    if (tid < ncol) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
+    __syncthreads();
 #pragma unroll
-        for (int pt = 0; pt < 4; ++pt) {
-          const size_t pp = (size_t)wbase + 16 * pt + li;
-          kw[pt][0] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg, (size_t)a.nkv * (HD / 8), pp)]; kw[pt][1] = kv.kq[kv_blk((size_t)kvh * (HD / 8) + dq * 8 + 2 * lg + 1, (size_t)a.nkv * (HD / 8), pp)];
-          ksc[pt] = kv.ks[kv_blk((size_t)kvh * (HD / 32) + dq * 2 + (lg >> 1), (size_t)a.nkv * (HD / 32), pp)];
+    for (int gi = 0; gi < GH; ++gi) {
+      const int c = dq + 4 * gi;
+      if (c < ncol) {
+        const bool valid = p < start + tk0 + c / G + 1;
+        float e = valid ? expf(sv[gi] - cm[c]) : 0.0f; sc[c][pos] = e;
+        const float l = wave_sum(e);
+        if (lane == 0) wsum[pw][c] = l;
+      }
+    }
+    __syncthreads();          // weights of every position visible; the score partials in `red` are dead
+  };
+  // A wave is on one of two paths for the whole kernel -- packed positions or f32 ones (the branch is scalar: wbase is a
+  // wave's) -- each with its own registers; both pass the same five barriers.
+  if (active && packed) {             // packed positions lie below the boundary, hence inside the view
+    // Lane (li, lg) of the value product stands for two dims of a scale block (word li & 3, nibbles 2 * (li >> 2) + m) at
+    // the eight positions 8 * lg .. of a 32-position group: vw[g][b][p] is the word of position 32 * g + 8 * lg + p in
+    // block dq * 2 + b.  vsl[g]: the scale of position 32 * g + 8 * lg + (li & 7) in block dq * 2 + (li >> 3); the lanes of a
+    // row of sixteen hold the 8 x 2 scales the row needs and pass them round with row broadcasts.  The values do not
+    // depend on the scores: their loads go out with the keys', one memory round trip for both.  All of it through
+    // buffer descriptors: one 32-bit offset per array and lane, the rest of an address is a constant or a scalar.
+    uint32_t vw[2][2][8]; float vsl[2]; uint32_t kw[4][2]; float ksc[4][2];
+    {
+      const __amdgpu_buffer_rsrc_t rvq = __builtin_amdgcn_make_buffer_rsrc((void*)kv.vq, 0, 0xFFFFFFFF, 0x00020000), rvs = __builtin_amdgcn_make_buffer_rsrc((void*)kv.vs, 0, 0xFFFFFFFF, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rkq = __builtin_amdgcn_make_buffer_rsrc((void*)kv.kq, 0, 0xFFFFFFFF, 0x00020000), rks = __builtin_amdgcn_make_buffer_rsrc((void*)kv.ks, 0, 0xFFFFFFFF, 0x00020000);
+      const int vrow = (row / 8) * 4, srow = (row / 32) * 4;          // bytes of a position's packed values and of its scales
+      const int vq_off = (wbase + 8 * lg) * vrow + (kvh * (HD / 8) + dq * 8 + (li & 3)) * 4, vs_off = (wbase + 8 * lg + (li & 7)) * srow + (kvh * (HD / 32) + dq * 2 + (li >> 3)) * 4;
+      const int kq_off = (((wbase >> 6) * (a.nkv * (HD / 8)) + kvh * (HD / 8) + dq * 8 + lg) * 64 + li) * 4, ks_off = (((wbase >> 6) * (a.nkv * (HD / 32)) + kvh * (HD / 32) + dq * 2) * 64 + li) * 4;
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {          // key word (block dq*2 + b, dims 8*lg ..) and block scale of position wbase + 16*pt + li
+          kw[pt][b] = __builtin_amdgcn_raw_buffer_load_b32(rkq, kq_off, (b * 4 * 64 + 16 * pt) * 4, 0);
+          ksc[pt][b] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rks, ks_off, (b * 64 + 16 * pt) * 4, 0));
         }
 #pragma unroll
-        for (int s = 0; s < 16; ++s)
+      for (int g = 0; g < 2; ++g) {
 #pragma unroll
-          for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(nib_val(kw[pt][s >> 3], s & 7) * ksc[pt], B[s], D[pt], 0, 0, 0);
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int q = 0; q < 8; ++q) vw[g][b][q] = __builtin_amdgcn_raw_buffer_load_b32(rvq, vq_off, (32 * g + q) * vrow + b * 16, 0);
+        vsl[g] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rvs, vs_off, 32 * g * srow, 0));
+      }
+    }
+    PYRE_TS(1);
+    {
+      f4v D[4];
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+      // 4-bit keys on the f16 matrix cores: one v_mfma_f32_16x16x32_f16 per query half covers 16 positions x a 32-dim
+      // scale block.  A = the query halves (row = column of the pass), B = the keys (column = position, a lane's word
+      // is its eight dims), so a lane's sums belong to its own position and meet that position's block scale in f32.
+      // Products (4 bits x 11 bits) and the 32-term sums are exact in f32.
+      h8v qa[2][2];
+      if (li < ncol) {
+        const uint4* qp = (const uint4*)(qh + ((size_t)(tk0 + ctok) * a.nh + (size_t)kvh * G + chead) * 2 * HD);
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf) qa[b][hf] = __builtin_bit_cast(h8v, qp[(hf * HD + (dq * 2 + b) * 32 + lg * 8) >> 3]);
       } else {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf) qa[b][hf] = __builtin_bit_cast(h8v, make_uint4(0, 0, 0, 0));
+      }
+      float qinv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) { const int c = 4 * lg + r; qinv[r] = c < ncol ? qsc[(size_t)(tk0 + c / G) * a.nh + (size_t)kvh * G + c % G] : 0.0f; }
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const h8v Bk = nib8_f16(kw[pt][b]);
+          const f4v z = {0.0f, 0.0f, 0.0f, 0.0f};
+          const f4v d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[b][1], Bk, __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[b][0], Bk, z, 0, 0, 0), 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) D[pt][r] = fmaf(ksc[pt][b], d[r], D[pt][r]);
+        }
+      // register r of tile pt: column 4*lg + r, position 16*pt + li
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) if (4 * lg + r < ncol) red[((size_t)dq * CH + pw * 64 + 16 * pt + li) * NC + 4 * lg + r] = D[pt][r] * qinv[r];
+    }
+    PYRE_TS(2);
+    __syncthreads(); PYRE_TS(3);
+    softmax_phase(); PYRE_TS(4);
+    {
+      // 4-bit values on the f16 matrix cores, 32 positions x 16 dims a step.  A = the weights times the position's block
+      // scale times a power of two of the wave (the largest scale lands in [2^13, 2^14)), as two f16 numbers h1 + h2
+      // (rounded towards zero; row = column of the pass); B = the values, a lane's eight positions of one dim.
+      float vm = wave_max(fmaxf(vsl[0], vsl[1]));
+      int E = 0;
+      if (vm > 0.0f && vm < INFINITY) { E = 140 - (int)((__float_as_uint(vm) >> 23) & 0xFF); E = E > 100 ? 100 : E; }
+      const float up = __uint_as_float((uint32_t)(127 + E) << 23), dn = __uint_as_float((uint32_t)(127 - E) << 23);
+      f4v Dv[2][2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int m = 0; m < 2; ++m) Dv[b][m] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+      const h2v off = {(_Float16)1032.0f, (_Float16)1032.0f};
+      const int bsh = 8 * (li >> 2);
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        float ev[8];
+        { const float4* e4 = (const float4*)&sc[li < NC ? li : 0][pw * 64 + 32 * g + 8 * lg];
+          const float4 e0 = e4[0], e1 = e4[1]; const bool on = li < ncol;
+          ev[0] = on ? e0.x : 0.0f; ev[1] = on ? e0.y : 0.0f; ev[2] = on ? e0.z : 0.0f; ev[3] = on ? e0.w : 0.0f; ev[4] = on ? e1.x : 0.0f; ev[5] = on ? e1.y : 0.0f; ev[6] = on ? e1.z : 0.0f; ev[7] = on ? e1.w : 0.0f; }
+        const int vs_bits = __float_as_int(vsl[g] * up);
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          struct U4 { uint32_t v[4]; } ah, al, b0, b1;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float s0 = __int_as_float(b == 0 ? row_bcast<2 * 0>(vs_bits, q) : row_bcast<8>(vs_bits, q)), s1 = __int_as_float(b == 0 ? row_bcast<1>(vs_bits, q) : row_bcast<9>(vs_bits, q));
+            const float x0 = ev[2 * q] * s0, x1 = ev[2 * q + 1] * s1;
+            const auto h = __builtin_amdgcn_cvt_pkrtz(x0, x1);
+            const auto l = __builtin_amdgcn_cvt_pkrtz(x0 - (float)h[0], x1 - (float)h[1]);
+            ah.v[q] = __builtin_bit_cast(uint32_t, h); al.v[q] = __builtin_bit_cast(uint32_t, l);
+            const uint32_t y = (((vw[g][b][2 * q] >> bsh) & 0xFFu) | (((vw[g][b][2 * q + 1] >> bsh) & 0xFFu) << 16)) ^ 0x00880088u;
+            b0.v[q] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2v, (y & 0x000F000Fu) | 0x64006400u) - off);
+            b1.v[q] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2v, ((y >> 4) & 0x000F000Fu) | 0x64006400u) - off);
+          }
+          const h8v A1 = __builtin_bit_cast(h8v, ah), A2 = __builtin_bit_cast(h8v, al), B0 = __builtin_bit_cast(h8v, b0), B1 = __builtin_bit_cast(h8v, b1);
+          Dv[b][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, B0, __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, B0, Dv[b][0], 0, 0, 0), 0, 0, 0);
+          Dv[b][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, B1, __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, B1, Dv[b][1], 0, 0, 0), 0, 0, 0);
+        }
+      }
+      // register r of (b, m): column 4*lg + r, dim dq*64 + b*32 + 8*(li & 3) + 2*(li >> 2) + m
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) if (4 * lg + r < ncol) red[((size_t)pw * NC + 4 * lg + r) * HD + dq * 64 + b * 32 + 8 * (li & 3) + 2 * (li >> 2) + m] = Dv[b][m][r] * dn;
+    }
+  } else {
+    PYRE_TS(1);
+    {
+      f4v D[4];
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt) D[pt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+      if (active) {
+        float B[16];
+        if (li < ncol) {
+          const float4* q4 = (const float4*)(qbuf + ((size_t)(tk0 + ctok) * a.nh + (size_t)kvh * G + chead) * HD + dq * 64 + 16 * lg);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) { float4 v = q4[j]; B[4 * j] = v.x; B[4 * j + 1] = v.y; B[4 * j + 2] = v.z; B[4 * j + 3] = v.w; }
+        } else {
+#pragma unroll
+          for (int s = 0; s < 16; ++s) B[s] = 0.0f;
+        }
         float A[4][16];
 #pragma unroll
         for (int pt = 0; pt < 4; ++pt) {
@@ -186,75 +371,40 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
         for (int s = 0; s < 16; ++s)
 #pragma unroll
           for (int pt = 0; pt < 4; ++pt) D[pt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[pt][s], B[s], D[pt], 0, 0, 0);
+        if (li < ncol) {
+#pragma unroll
+          for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * NC + li] = D[pt][r];
+        }
+      } else if (li < ncol) {          // a wave past the view: its positions carry no weight, their scores are read all the same
+#pragma unroll
+        for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * NC + li] = 0.0f;
       }
     }
-    if (li < ncol) {
-#pragma unroll
-      for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) red[((size_t)dq * CH + pw * 64 + 16 * pt + 4 * lg + r) * NC + li] = D[pt][r];
-    }
-  }
-  // f32 values: requested now, while the scores are being normalised (the keys' registers are free again; __syncthreads
-  // waits for outstanding loads, so the round trip is paid at the first barrier of phase 2 instead of after the last)
-  float4 vf4[16];
-  if (active && !packed) {
-#pragma unroll
-    for (int s = 0; s < 16; ++s) {
-      const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);          // positions past the view carry weight zero; their address is clamped
-      vf4[s] = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
-    }
-  }
-  PYRE_TS(2);
-  __syncthreads(); PYRE_TS(3);
-  // ---- phase 2: this thread's position is pw*64 + lane, its columns are dq, dq + 4, dq + 8, dq + 12
-  const int pos = pw * 64 + lane;
-  constexpr int GH = (NC + 3) / 4;
-  float sv[GH];
-#pragma unroll
-  for (int gi = 0; gi < GH; ++gi) {
-    const int c = dq + 4 * gi; sv[gi] = -INFINITY;
-    if (c < ncol) {
-      const bool valid = p < start + tk0 + c / G + 1;          // the column's token sees positions below its own + 1
-      float v = ((red[((size_t)0 * CH + pos) * NC + c] + red[((size_t)1 * CH + pos) * NC + c]) + red[((size_t)2 * CH + pos) * NC + c]) + red[((size_t)3 * CH + pos) * NC + c];
-      sv[gi] = valid ? v * scale : -INFINITY;
-      const float m = wave_max(sv[gi]);
-      if (lane == 0) wmax[pw][c] = m;
-    }
-  }
-  __syncthreads();
-  if (tid < ncol) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
-  __syncthreads();
-#pragma unroll
-  for (int gi = 0; gi < GH; ++gi) {
-    const int c = dq + 4 * gi;
-    if (c < ncol) {
-      const bool valid = p < start + tk0 + c / G + 1;
-      float e = valid ? expf(sv[gi] - cm[c]) : 0.0f; sc[pos][c] = e;
-      const float l = wave_sum(e);
-      if (lane == 0) wsum[pw][c] = l;
-    }
-  }
-  __syncthreads(); PYRE_TS(4);   // weights of every position visible; the score partials in `red` are dead
-  // ---- phase 3
-  {
-    f4v D[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    // f32 values: requested now, while the scores are being normalised (the keys' registers are free again; __syncthreads
+    // waits for outstanding loads, so the round trip is paid at the first barrier of the softmax phase instead of after the last)
+    float4 vf4[16];
     if (active) {
-      float B[16];
-      if (packed) {             // packed positions lie below the boundary, hence inside the view
 #pragma unroll
-        for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
+      for (int s = 0; s < 16; ++s) {
+        const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);          // positions past the view carry weight zero; their address is clamped
+        vf4[s] = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+      }
+    }
+    PYRE_TS(2);
+    __syncthreads(); PYRE_TS(3);
+    softmax_phase(); PYRE_TS(4);
+    {
+      f4v D[4];
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-          const uint32_t hw = vw[s] >> (16 * (li & 1));      // the lane's four nibbles
+      for (int dt = 0; dt < 4; ++dt) D[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+      if (active) {
+        float B[16];
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(nib_val(hw, dt) * vsc[s], B[s], D[dt], 0, 0, 0);
-        }
-      } else {
-#pragma unroll
-        for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[pw * 64 + 4 * s + lg][li < NC ? li : 0] : 0.0f;
+        for (int s = 0; s < 16; ++s) B[s] = li < ncol ? sc[li < NC ? li : 0][pw * 64 + 4 * s + lg] : 0.0f;
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
           const float A[4] = {vf4[s].x, vf4[s].y, vf4[s].z, vf4[s].w};
@@ -262,12 +412,12 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
           for (int dt = 0; dt < 4; ++dt) D[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[dt], B[s], D[dt], 0, 0, 0);
         }
       }
-    }
-    if (li < ncol) {
+      if (li < ncol) {
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[((size_t)pw * NC + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
+          for (int r = 0; r < 4; ++r) red[((size_t)pw * NC + li) * HD + dq * 64 + 4 * (4 * lg + r) + dt] = D[dt][r];
+      }
     }
   }
   PYRE_TS(5);
@@ -287,6 +437,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
 #ifdef PYRE_PHASE_TS
   PYRE_TS(7);
   if (tid == 0 && blockIdx.y == 0 && blockIdx.z == 0 && (chunk == 0 || chunk == (n - 1) / CH)) { for (int q_ = 0; q_ < 8; ++q_) attn_ts[(chunk == 0 ? 0 : 8) + q_] = ts_[q_]; }
+  if (tid == 0 && blockIdx.z == 0) { const unsigned w_ = blockIdx.y * gridDim.x + blockIdx.x; if (w_ < 4096) { for (int q_ = 0; q_ < 8; ++q_) attn_wg[10 * w_ + q_] = ts_[q_];
+    attn_wg[10 * w_ + 8] = ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32) | (unsigned)__builtin_amdgcn_s_getreg(4 | (31 << 11)); attn_wg[10 * w_ + 9] = ((unsigned long long)kvh << 32) | (unsigned)chunk; } }
 #endif
 }
 
@@ -301,7 +453,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
   __shared__ float red[4 * CH * G];
   __shared__ float sc[CH][G];
   __shared__ float wmax[NPW][G], wsum[NPW][G], cm[G];
-  const int chunk = blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
+  const int chunk = (int)gridDim.x - 1 - (int)blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;          // descending, as in k_attn_decode
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
   const int n = start + ti + 1, cnt = pcount[ti];
@@ -497,6 +649,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   const int nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
   const float* po = part_o + ((size_t)ti * a.nh + h) * max_chunks * HD;
+  const float gate = grp == 0 ? qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd] : 0.0f;          // fetched with the partials, not after them
   float pv[B];
 #pragma unroll
   for (int i = 0; i < B; ++i) pv[i] = nc > 0 ? po[(size_t)min(grp + 4 * i, nc - 1) * HD + dd] : 0.0f;
@@ -527,7 +680,6 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   __syncthreads();
   if (grp == 0) {
     o = ((so[0][tid] + so[1][tid]) + so[2][tid]) + so[3][tid]; L = ((sl[0] + sl[1]) + sl[2]) + sl[3];
-    float gate = qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd];
     const float ov = (o / L) * a_sigm(gate);
     out[((size_t)ti * a.nh + h) * HD + dd] = ov;
   }
@@ -546,12 +698,12 @@ void pyre_kv_carve(const AttnDev& a, int cap, void* base, KvDev* kv) {
 }
 size_t pyre_attn_work_bytes(const AttnDev& a, int cap) {
   size_t mc = ((size_t)cap + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
-  return 3 * 256 + 4 * (8 * (size_t)a.nh * a.hd + 8 * (size_t)a.nh * mc * a.hd + 8 * (size_t)a.nh * mc * 2);
+  return 5 * 256 + 4 * (2 * 8 * (size_t)a.nh * a.hd + 8 * (size_t)a.nh + 8 * (size_t)a.nh * mc * a.hd + 8 * (size_t)a.nh * mc * 2);
 }
 void pyre_attn_work_carve(const AttnDev& a, int cap, void* base, AttnWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
   size_t mc = ((size_t)cap + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
-  w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
+  w->q = (float*)take(4 * 8 * (size_t)a.nh * a.hd); w->qh = (uint16_t*)take(2 * 2 * 8 * (size_t)a.nh * a.hd); w->qsc = (float*)take(4 * 8 * (size_t)a.nh); w->part_o = (float*)take(4 * 8 * (size_t)a.nh * mc * a.hd); w->part_ml = (float*)take(4 * 8 * (size_t)a.nh * mc * 2); w->max_chunks = (int)mc;
 }
 
 template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, int start, int t, const int* posp, const QsaWork* qw) {
@@ -559,8 +711,8 @@ template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, cons
   if (!qw) {          // tokens that share a pass over the cache: as many as the 16 columns hold, one when the 4-bit boundary moves inside the window
     int tp = 16 / G > 8 ? 8 : 16 / G;
     if (posp || pyre_packed_boundary((size_t)start + 1, a.kv_bits, a.kv_recent) != pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent)) tp = 1;
-    if (tp == 1 || t == 1) hipLaunchKernelGGL((k_attn_decode<256, G, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, t, 1);
-    else hipLaunchKernelGGL((k_attn_decode<256, G, 16>), dim3(chunks, a.nkv, (t + tp - 1) / tp), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, start, posp, w.part_o, w.part_ml, w.max_chunks, t, tp);
+    if (tp == 1 || t == 1) hipLaunchKernelGGL((k_attn_decode<256, G, G>), dim3(chunks, a.nkv, t), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, w.qh, w.qsc, start, posp, w.part_o, w.part_ml, w.max_chunks, t, 1);
+    else hipLaunchKernelGGL((k_attn_decode<256, G, 16>), dim3(chunks, a.nkv, (t + tp - 1) / tp), dim3(256 * PYRE_ATTN_NPW), 0, ctx->stream, a, kv, w.q, w.qh, w.qsc, start, posp, w.part_o, w.part_ml, w.max_chunks, t, tp);
     return; }
   // a token attends either to all of its n <= budget + ratio - 1 visible positions or to a list: never to more than list_stride entries
   { int lc = (qw->list_stride + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK; if (chunks > lc) chunks = lc; }
@@ -576,11 +728,12 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
+  if (a.kv_bits == 4 && (size_t)kv.cap * (size_t)(a.nkv * a.hd / 8) * 4 >= ((size_t)1 << 31)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: a 4-bit cache of %d positions exceeds the 2 GiB a kernel addresses with 32-bit offsets", kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
   // a single-token step at a device-side position: the packing check rides on the prep launch as extra blocks
   const bool pack_rides = posp && t == 1 && a.kv_bits == 4;
   const int pack_blocks = pack_rides ? (64 * (a.nkv * a.hd / 32) * 2 + 255) / 256 : 0;
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q, w.qh, w.qsc); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
   int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
   if (posp) {   // one 64-position packing step at most; the kernel decides from the device-side position
@@ -608,7 +761,7 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
 int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t) {
   if (a.hd != 256 || a.kv_bits != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "attention append: head dim %d, %d-bit cache (256, f32 only)", a.hd, a.kv_bits);
   if (t < 1 || t > 8 || start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention append: positions %d..%d outside the cache (%d)", start, start + t, kv.cap);
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, (const int*)nullptr, w.q); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, (const int*)nullptr, w.q, w.qh, w.qsc); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

@@ -69,11 +69,14 @@ int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, ui
 //   ksplit  > 1: y is a partial buffer, y[(ks*T + t)*tiles*64 + row] = slice sum (the consumer adds the slices in order).
 //   ep.best (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 //   ep.co: conv1d + SiLU of the leading ep.ch rows (linear_core, qwen4exp_gguf.rs:1643-1647), as in the lane = row GEMV.
-template <int NW, bool SC, bool CONV>
+//   ONE: the single-token instance -- T = 1, two operand rows and (CONV) four taps are compile-time constants.
+template <int NW, bool SC, bool CONV, bool ONE = false>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m); args_now(aop, ainv, y, T, R, cpw, ep.best, ep.conv_w, ep.conv_in, ep.conv_out, ep.co, ep.ch, ep.kk);
+  if constexpr (ONE) { T = 1; R = 2; }
+  const int kk = ONE ? 4 : ep.kk;
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int K128 = m.cols >> 7;
@@ -90,7 +93,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
   if constexpr (CONV) if (conv_row) {
     const size_t row = (size_t)tile * 64 + lane;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { cw[k] = k < ep.kk ? ep.conv_w[row * ep.kk + k] : 0.0f; chist[k] = k < ep.kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
+    for (int k = 0; k < 8; ++k) { cw[k] = k < kk ? ep.conv_w[row * kk + k] : 0.0f; chist[k] = k < kk - 1 ? ep.conv_in[(size_t)k * ep.ch + row] : 0.0f; }
   }
   PYRE_TS(1);
   if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane: one buffer, no look-ahead
@@ -139,17 +142,17 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
       const float cur = rsum(t, lane);
       float o = 0.0f;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) if (k == ep.kk - 1) o = cw[k] * cur;
+      for (int k = 0; k < 8; ++k) if (k == kk - 1) o = cw[k] * cur;
 #pragma unroll
-      for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) o += cw[k] * chist[k];
+      for (int k = 0; k < 7; ++k) if (k < kk - 1) o += cw[k] * chist[k];
       ep.co[(size_t)t * ep.ch + row] = o * (1.0f / (1.0f + expf(-o)));
 #pragma unroll
-      for (int k = 0; k < 7; ++k) if (k + 1 < ep.kk - 1) chist[k] = chist[k + 1];
+      for (int k = 0; k < 7; ++k) if (k + 1 < kk - 1) chist[k] = chist[k + 1];
 #pragma unroll
-      for (int k = 0; k < 7; ++k) if (k == ep.kk - 2) chist[k] = cur;
+      for (int k = 0; k < 7; ++k) if (k == kk - 2) chist[k] = cur;
     }
 #pragma unroll
-    for (int k = 0; k < 7; ++k) if (k < ep.kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
+    for (int k = 0; k < 7; ++k) if (k < kk - 1) ep.conv_out[(size_t)k * ep.ch + row] = chist[k];
   }
   PYRE_TS(4); PYRE_TS_FLUSH(gemm_ts, (NW == 16 ? 0 : (gridDim.y > 1 ? 8 : 16)));
 }
@@ -166,9 +169,10 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
   return nw;
 }
 template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep) {
-#define GEMM_M_GO(SC, CONV) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
-  if (ep.co) { if (a.ainv) GEMM_M_GO(true, true); else GEMM_M_GO(false, true); }
-  else { if (a.ainv) GEMM_M_GO(true, false); else GEMM_M_GO(false, false); }
+#define GEMM_M_GO(SC, CONV, ONE) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, ONE>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
+  if (t == 1 && a.ainv && (!ep.co || ep.kk == 4)) { if (ep.co) GEMM_M_GO(true, true, true); else GEMM_M_GO(true, false, true); }          // a single token with scaled operand rows: the instance with its constants folded in
+  else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true, false); else GEMM_M_GO(false, true, false); }
+  else { if (a.ainv) GEMM_M_GO(true, false, false); else GEMM_M_GO(false, false, false); }
 #undef GEMM_M_GO
 }
 }  // namespace

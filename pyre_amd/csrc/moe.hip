@@ -58,9 +58,11 @@ __device__ __forceinline__ void route_select(int n_exp, int k, RouteLds& L) {
   for (int i = e >> 3; i < nc; i += (int)(blockDim.x >> 3)) {
     const uint64_t ci = L.cand[i];
     int beaten = 0;
-    for (int j = sub; j < nc; j += 32) {
+#pragma unroll
+    for (int jb = 0; jb < 512; jb += 32) if (jb < nc) {          // (uniform branches: with nc known at compile time every read is issued before the first comparison)
+      const int j = jb + sub;
       const uint64_t c0 = L.cand[min(j, 511)], c1 = L.cand[min(j + 8, 511)], c2 = L.cand[min(j + 16, 511)], c3 = L.cand[min(j + 24, 511)];
-      beaten += (c0 > ci ? 1 : 0) + ((j + 8 < nc && c1 > ci) ? 1 : 0) + ((j + 16 < nc && c2 > ci) ? 1 : 0) + ((j + 24 < nc && c3 > ci) ? 1 : 0);
+      beaten += ((j < nc && c0 > ci) ? 1 : 0) + ((j + 8 < nc && c1 > ci) ? 1 : 0) + ((j + 16 < nc && c2 > ci) ? 1 : 0) + ((j + 24 < nc && c3 > ci) ? 1 : 0);
     }
     beaten += __builtin_amdgcn_mov_dpp(beaten, 0xB1, 0xf, 0xf, true);          // quad_perm [1,0,3,2]
     beaten += __builtin_amdgcn_mov_dpp(beaten, 0x4E, 0xf, 0xf, true);          // quad_perm [2,3,0,1]
