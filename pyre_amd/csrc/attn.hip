@@ -165,10 +165,12 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   __shared__ __align__(16) float sc[NC][CH + 4];          // [column][position]: eight consecutive positions of a column are two 16-byte reads
   __shared__ float wmax[NPW][NC], wsum[NPW][NC], cm[NC];
   PYRE_TS_VARS PYRE_TS(0);
-  // chunks in descending order: the workgroups past the view (a captured launch covers the whole cache) and the partly
-  // filled last chunk go first and free their slots at once; when the grid exceeds what the chip holds, the workgroups
-  // that wait are full ones either way, and they now wait for the short ones
-  const int chunk = (int)gridDim.x - 1 - (int)blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+  // Workgroups in dispatch order (x fastest): chunks descending, the KV heads of a chunk next to each other.  The
+  // workgroups past the view (a captured launch covers the whole cache) leave first; the chunks of the f32 window, which
+  // move eight times the bytes of a packed chunk, follow as neighbours in the order and so land on different compute
+  // units, where each later shares its unit with a packed chunk instead of another f32 one.
+  const int lin = (int)blockIdx.x + (int)gridDim.x * (int)blockIdx.y;
+  const int chunk = (int)gridDim.x - 1 - lin / (int)gridDim.y, kvh = lin % (int)gridDim.y, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
   const int tk0 = blockIdx.z * tp, nk = min(tp, t - tk0), ncol = nk * G;          // tokens tk0 .. tk0+nk-1 in columns 0 .. ncol-1
@@ -230,11 +232,12 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
     // buffer descriptors: one 32-bit offset per array and lane, the rest of an address is a constant or a scalar.
     uint32_t vw[2][2][8]; float vsl[2]; uint32_t kw[4][2]; float ksc[4][2];
     {
-      const __amdgpu_buffer_rsrc_t rvq = __builtin_amdgcn_make_buffer_rsrc((void*)kv.vq, 0, 0xFFFFFFFF, 0x00020000), rvs = __builtin_amdgcn_make_buffer_rsrc((void*)kv.vs, 0, 0xFFFFFFFF, 0x00020000);
-      const __amdgpu_buffer_rsrc_t rkq = __builtin_amdgcn_make_buffer_rsrc((void*)kv.kq, 0, 0xFFFFFFFF, 0x00020000), rks = __builtin_amdgcn_make_buffer_rsrc((void*)kv.ks, 0, 0xFFFFFFFF, 0x00020000);
+      // the descriptors start at the wave's 64 positions: every offset below is small
       const int vrow = (row / 8) * 4, srow = (row / 32) * 4;          // bytes of a position's packed values and of its scales
-      const int vq_off = (wbase + 8 * lg) * vrow + (kvh * (HD / 8) + dq * 8 + (li & 3)) * 4, vs_off = (wbase + 8 * lg + (li & 7)) * srow + (kvh * (HD / 32) + dq * 2 + (li >> 3)) * 4;
-      const int kq_off = (((wbase >> 6) * (a.nkv * (HD / 8)) + kvh * (HD / 8) + dq * 8 + lg) * 64 + li) * 4, ks_off = (((wbase >> 6) * (a.nkv * (HD / 32)) + kvh * (HD / 32) + dq * 2) * 64 + li) * 4;
+      const __amdgpu_buffer_rsrc_t rvq = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kv.vq + (size_t)wbase * vrow), 0, 0xFFFFFFFF, 0x00020000), rvs = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kv.vs + (size_t)wbase * srow), 0, 0xFFFFFFFF, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rkq = __builtin_amdgcn_make_buffer_rsrc((void*)(kv.kq + (size_t)(wbase >> 6) * (a.nkv * (HD / 8)) * 64), 0, 0xFFFFFFFF, 0x00020000), rks = __builtin_amdgcn_make_buffer_rsrc((void*)(kv.ks + (size_t)(wbase >> 6) * (a.nkv * (HD / 32)) * 64), 0, 0xFFFFFFFF, 0x00020000);
+      const int vq_off = 8 * lg * vrow + (kvh * (HD / 8) + dq * 8 + (li & 3)) * 4, vs_off = (8 * lg + (li & 7)) * srow + (kvh * (HD / 32) + dq * 2 + (li >> 3)) * 4;
+      const int kq_off = ((kvh * (HD / 8) + dq * 8 + lg) * 64 + li) * 4, ks_off = ((kvh * (HD / 32) + dq * 2) * 64 + li) * 4;
 #pragma unroll
       for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
@@ -360,13 +363,15 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
 #pragma unroll
           for (int s = 0; s < 16; ++s) B[s] = 0.0f;
         }
+        // one descriptor at the wave's 64-position block, one offset per lane; positions past the view (the last chunk)
+        // read what the cache holds there, and their scores are discarded
         float A[4][16];
+        const __amdgpu_buffer_rsrc_t rkf = __builtin_amdgcn_make_buffer_rsrc((void*)(kv.kf + (size_t)(wbase >> 6) * row * 64), 0, 0xFFFFFFFF, 0x00020000);
+        const int kf_off = ((kvh * HD + dq * 64 + 16 * lg) * 64 + li) * 4;
 #pragma unroll
-        for (int pt = 0; pt < 4; ++pt) {
-          const size_t pp = (size_t)min(wbase + 16 * pt + li, n - 1);
+        for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-          for (int s = 0; s < 16; ++s) A[pt][s] = kv.kf[kv_blk((size_t)kvh * HD + dq * 64 + 16 * lg + s, (size_t)a.nkv * HD, pp)];
-        }
+          for (int s = 0; s < 16; ++s) A[pt][s] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rkf, kf_off, (s * 64 + 16 * pt) * 4, 0));
 #pragma unroll
         for (int s = 0; s < 16; ++s)
 #pragma unroll
@@ -388,10 +393,12 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
     // waits for outstanding loads, so the round trip is paid at the first barrier of the softmax phase instead of after the last)
     float4 vf4[16];
     if (active) {
+      const __amdgpu_buffer_rsrc_t rvf = __builtin_amdgcn_make_buffer_rsrc((void*)(kv.vf + (size_t)wbase * row), 0, 0xFFFFFFFF, 0x00020000);
+      const int vf_off = (kvh * HD + dq * 64 + 4 * li) * 4, last = n - 1 - wbase;
 #pragma unroll
-      for (int s = 0; s < 16; ++s) {
-        const size_t pg = (size_t)min(wbase + 4 * s + lg, n - 1);          // positions past the view carry weight zero; their address is clamped
-        vf4[s] = *(const float4*)(kv.vf + pg * row + (size_t)kvh * HD + dq * 64 + 4 * li);
+      for (int s = 0; s < 16; ++s) {          // positions past the view carry weight zero; their address is clamped
+        const auto v = __builtin_amdgcn_raw_buffer_load_b128(rvf, vf_off + min(4 * s + lg, last) * (row * 4), 0, 0);
+        vf4[s] = make_float4(__int_as_float(v[0]), __int_as_float(v[1]), __int_as_float(v[2]), __int_as_float(v[3]));
       }
     }
     PYRE_TS(2);
@@ -436,7 +443,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   }
 #ifdef PYRE_PHASE_TS
   PYRE_TS(7);
-  if (tid == 0 && blockIdx.y == 0 && blockIdx.z == 0 && (chunk == 0 || chunk == (n - 1) / CH)) { for (int q_ = 0; q_ < 8; ++q_) attn_ts[(chunk == 0 ? 0 : 8) + q_] = ts_[q_]; }
+  if (tid == 0 && kvh == 0 && blockIdx.z == 0 && (chunk == 0 || chunk == (n - 1) / CH)) { for (int q_ = 0; q_ < 8; ++q_) attn_ts[(chunk == 0 ? 0 : 8) + q_] = ts_[q_]; }
   if (tid == 0 && blockIdx.z == 0) { const unsigned w_ = blockIdx.y * gridDim.x + blockIdx.x; if (w_ < 4096) { for (int q_ = 0; q_ < 8; ++q_) attn_wg[10 * w_ + q_] = ts_[q_];
     attn_wg[10 * w_ + 8] = ((unsigned long long)__builtin_amdgcn_s_getreg(20 | (31 << 11)) << 32) | (unsigned)__builtin_amdgcn_s_getreg(4 | (31 << 11)); attn_wg[10 * w_ + 9] = ((unsigned long long)kvh << 32) | (unsigned)chunk; } }
 #endif
@@ -453,7 +460,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
   __shared__ float red[4 * CH * G];
   __shared__ float sc[CH][G];
   __shared__ float wmax[NPW][G], wsum[NPW][G], cm[G];
-  const int chunk = (int)gridDim.x - 1 - (int)blockIdx.x, kvh = blockIdx.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;          // descending, as in k_attn_decode
+  const int lin = (int)blockIdx.x + (int)gridDim.x * (int)blockIdx.y;          // dispatch order as in k_attn_decode
+  const int chunk = (int)gridDim.x - 1 - lin / (int)gridDim.y, kvh = lin % (int)gridDim.y, ti = blockIdx.z, tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), pw = wave % NPW, dq = wave / NPW;
   if (posp) start = *posp;
   const int n = start + ti + 1, cnt = pcount[ti];
@@ -728,7 +736,6 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "attention: t = %d outside 1..8", t);
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
-  if (a.kv_bits == 4 && (size_t)kv.cap * (size_t)(a.nkv * a.hd / 8) * 4 >= ((size_t)1 << 31)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: a 4-bit cache of %d positions exceeds the 2 GiB a kernel addresses with 32-bit offsets", kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
   // a single-token step at a device-side position: the packing check rides on the prep launch as extra blocks
   const bool pack_rides = posp && t == 1 && a.kv_bits == 4;

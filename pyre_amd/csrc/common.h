@@ -198,7 +198,9 @@ size_t pyre_aop_bytes(int cols, int t);                            // operand by
 int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv);
 // y as pyre_gemv_launch / pyre_gemv_split_launch (ksplit > 1: slice sums) with the epilogues of GemvEpi
 int pyre_gemm_m_best_count(const QMatDev& m);
-int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep);
+int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep, const float* xf = nullptr);
+// xf: the single token's f32 activations instead of `a` (the kernel forms the operand rows itself); where that pays
+bool pyre_gemm_m_x_ok(const QMatDev& m, int t, const GemvEpi& ep);
 // K parts / waves per workgroup the kernel uses for this matrix (ksplit parts)
 void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* hb_per_wave);
 // the operator's own scratch for the split operand (grow-only, per context), and the fixed per-GPU array of the entry point

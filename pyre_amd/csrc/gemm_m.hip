@@ -70,7 +70,41 @@ int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, ui
 //   ep.best (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 //   ep.co: conv1d + SiLU of the leading ep.ch rows (linear_core, qwen4exp_gguf.rs:1643-1647), as in the lane = row GEMV.
 //   ONE: the single-token instance -- T = 1, two operand rows and (CONV) four taps are compile-time constants.
-template <int NW, bool SC, bool CONV, bool ONE = false>
+//   XF (with ONE): `aop` is the token's f32 activations; every wave forms the operand rows of its chunks itself, with the
+//   arithmetic of k_act_split (the 256-column stretch's power of two from a wave maximum over the stretch), so the sums
+//   are bit for bit those of the split launch followed by this one -- a launch less where the producer of x cannot
+//   scale (it does not know the stretch's maximum) and the matrix has few row tiles to repeat the conversion in.
+__device__ __forceinline__ void load_a_x(const float* __restrict__ x, int c, int lane, ABuf& b) {
+  const int row = lane & 15, kg = lane >> 4;
+  const float4 sv = ((const float4*)(x + (size_t)(c >> 1) * 256))[lane];
+  float4 xv[4][2];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) { const float4* p = (const float4*)(x + (size_t)c * 128 + s * 32 + kg * 8); xv[s][0] = p[0]; xv[s][1] = p[1]; }
+  auto nn = [](float v) { float a = fabsf(v); return a == a ? a : INFINITY; };          // a NaN anywhere makes the stretch non-finite
+  const float m = wave_max(fmaxf(fmaxf(nn(sv.x), nn(sv.y)), fmaxf(nn(sv.z), nn(sv.w))));
+  int e = 0;
+  if (m > 0.0f && m < INFINITY) { e = 140 - (int)((__float_as_uint(m) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+  const float up = __uint_as_float((uint32_t)(127 + e) << 23), dn = __uint_as_float((uint32_t)(127 - e) << 23);
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const float v[8] = {xv[s][0].x, xv[s][0].y, xv[s][0].z, xv[s][0].w, xv[s][1].x, xv[s][1].y, xv[s][1].z, xv[s][1].w};
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t hh[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const float xs = v[2 * q + u] * up;
+        const _Float16 h1 = (_Float16)xs, h2 = (_Float16)((xs - (float)h1) * 2048.0f);
+        hh[u] = row == 0 ? __builtin_bit_cast(unsigned short, h1) : (row == 1 ? __builtin_bit_cast(unsigned short, h2) : 0u);
+      }
+      w[q] = hh[0] | (hh[1] << 16);
+    }
+    b.a[s] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  b.ai0 = kg == 0 ? dn : 0.0f; b.ai1 = 0.0f;
+}
+template <int NW, bool SC, bool CONV, bool ONE = false, bool XF = false>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
@@ -85,9 +119,12 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
 #pragma unroll
   for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
   const NibK nk = nib_consts();
+  static_assert(!XF || (ONE && !CONV), "f32 activations: the single-token instance without the conv epilogue");
   const AopRsrc ar = aop_rsrc(aop, m.cols, R, lane);
+  const float* xf = (const float*)aop;
+  auto get_a = [&](int c, ABuf& b) { if constexpr (XF) load_a_x(xf, c, lane, b); else load_a<SC>(ar, ainv, R, c, lane, b); };
   WBuf<4> w0; ABuf a0;
-  if (c0 < c1) { load_a<SC>(ar, ainv, R, c0, lane, a0); load_w<4>(m, tile * 4, c0, lane, K128, w0); }
+  if (c0 < c1) { get_a(c0, a0); load_w<4>(m, tile * 4, c0, lane, K128, w0); }
   // conv epilogue: wave 0 fetches its rows' taps and state now, behind the weights, so the loads overlap the products
   float cw[CONV ? 8 : 1], chist[CONV ? 8 : 1]; const bool conv_row = CONV && wave == 0 && tile * 64 + lane < ep.ch;
   if constexpr (CONV) if (conv_row) {
@@ -98,17 +135,17 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
   PYRE_TS(1);
   if constexpr (NW == 16) {                   // sixteen waves: one or two chunks a wave and 128 registers a lane: one buffer, no look-ahead
     for (int c = c0; c < c1; ++c) {
-      if (c > c0) { load_a<SC>(ar, ainv, R, c, lane, a0); load_w<4>(m, tile * 4, c, lane, K128, w0); }
+      if (c > c0) { get_a(c, a0); load_w<4>(m, tile * 4, c, lane, K128, w0); }
       chunk_mac<4>(w0, a0, c, nk, tot);
     }
   } else {                                    // two buffers taking turns (a copy from one to the other would wait for the loads just issued)
     WBuf<4> w1; ABuf a1;
     for (int c = c0; c < c1; c += 2) {
-      if (c + 1 < c1) { load_a<SC>(ar, ainv, R, c + 1, lane, a1); load_w<4>(m, tile * 4, c + 1, lane, K128, w1); }
+      if (c + 1 < c1) { get_a(c + 1, a1); load_w<4>(m, tile * 4, c + 1, lane, K128, w1); }
       __builtin_amdgcn_sched_barrier(0);      // (keeps the compiler from sinking the loads down to their first use)
       chunk_mac<4>(w0, a0, c, nk, tot);
       __builtin_amdgcn_sched_barrier(0);
-      if (c + 2 < c1) { load_a<SC>(ar, ainv, R, c + 2, lane, a0); load_w<4>(m, tile * 4, c + 2, lane, K128, w0); }
+      if (c + 2 < c1) { get_a(c + 2, a0); load_w<4>(m, tile * 4, c + 2, lane, K128, w0); }
       __builtin_amdgcn_sched_barrier(0);
       if (c + 1 < c1) chunk_mac<4>(w1, a1, c + 1, nk, tot);
       __builtin_amdgcn_sched_barrier(0);
@@ -168,7 +205,8 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
   if (force == 4 || force == 8 || force == 16) nw = force;
   return nw;
 }
-template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep) {
+template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep, const float* xf = nullptr) {
+  if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, true, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep); return; }
 #define GEMM_M_GO(SC, CONV, ONE) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, ONE>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
   if (t == 1 && a.ainv && (!ep.co || ep.kk == 4)) { if (ep.co) GEMM_M_GO(true, true, true); else GEMM_M_GO(true, false, true); }          // a single token with scaled operand rows: the instance with its constants folded in
   else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true, false); else GEMM_M_GO(false, true, false); }
@@ -184,17 +222,22 @@ void pyre_gemm_m_plan(const QMatDev& m, int ksplit, int* nw, int* cpw) {
 
 int pyre_gemm_m_best_count(const QMatDev& m) { return m.tiles; }
 
-int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, const GemvEpi& ep) {
+bool pyre_gemm_m_x_ok(const QMatDev& m, int t, const GemvEpi& ep) {
+  static const bool off = env_i("PYRE_GEMM_M_X", 1) == 0;
+  return !off && t == 1 && !ep.co && m.tiles <= 128;
+}
+int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, const GemvEpi& ep, const float* xf) {
   if (m.fmt != FMT_IQ3_S_M || !m.mq || !m.mh) return pyre_fail(ctx, PYRE_E_TYPE, "gemm_m: the matrix is not held in the matrix-core layout");
-  if (t < 1 || t > 8 || ksplit < 1 || !a.op || !y) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: t = %d, %d K slices", t, ksplit);
+  if (xf && !pyre_gemm_m_x_ok(m, t, ep)) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: f32 activations are for a single token, no conv epilogue and at most 128 row tiles");
+  if (t < 1 || t > 8 || ksplit < 1 || (!a.op && !xf) || !y) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: t = %d, %d K slices", t, ksplit);
   if (m.cols % 256 != 0 || m.SB != m.cols / 256) return pyre_fail(ctx, PYRE_E_SHAPE, "gemm_m: %d columns", m.cols);
   int nw, cpw; pyre_gemm_m_plan(m, ksplit, &nw, &cpw);
   if (ep.four_waves) { nw = 4; const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit; cpw = (per_wg + 3) / 4; }
   static const std::string names[9] = {"", "gemm_m_iq3s_t1", "gemm_m_iq3s_t2", "gemm_m_iq3s_t3", "gemm_m_iq3s_t4", "gemm_m_iq3s_t5", "gemm_m_iq3s_t6", "gemm_m_iq3s_t7", "gemm_m_iq3s_t8"};
   ProfScope ps(ctx, names[t].c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * t * ((double)m.cols + m.rows));
-  if (nw == 4) gemm_m_go<4>(ctx, m, a, t, y, ksplit, cpw, ep);
-  else if (nw == 8) gemm_m_go<8>(ctx, m, a, t, y, ksplit, cpw, ep);
-  else gemm_m_go<16>(ctx, m, a, t, y, ksplit, cpw, ep);
+  if (nw == 4) gemm_m_go<4>(ctx, m, a, t, y, ksplit, cpw, ep, xf);
+  else if (nw == 8) gemm_m_go<8>(ctx, m, a, t, y, ksplit, cpw, ep, xf);
+  else gemm_m_go<16>(ctx, m, a, t, y, ksplit, cpw, ep, xf);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 

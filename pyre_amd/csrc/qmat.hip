@@ -355,6 +355,7 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
 // context's operand buffer first (sized by pyre_gemm_m_scratch; grows only outside stream capture).
 int gemm_m_from_f32(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, const GemvEpi& ep, const PyreAop* a) {
   if (a && a->op) return pyre_gemm_m_launch(ctx, m, *a, t, y, ksplit, ep);
+  if (pyre_gemm_m_x_ok(m, t, ep)) return pyre_gemm_m_launch(ctx, m, PyreAop{nullptr, nullptr}, 1, y, ksplit, ep, x);          // few row tiles: the product converts x itself, a launch less
   uint4* op; float* ainv; int rc = pyre_gemm_m_scratch(ctx, m.cols, &op, &ainv); if (rc) return rc;
   if ((rc = pyre_act_split_launch(ctx, x, t, m.cols, op, ainv))) return rc;
   return pyre_gemm_m_launch(ctx, m, PyreAop{op, ainv}, t, y, ksplit, ep);
