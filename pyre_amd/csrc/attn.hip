@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   static_assert(4 * CH == NPW * HD, "the score and value partials share one buffer");
   __shared__ float red[4 * CH * NC];          // phase 1: [dq][position][column];  phase 3: [pw][column][dim]
   __shared__ __align__(16) float sc[NC][CH + 4];          // [column][position]: eight consecutive positions of a column are two 16-byte reads
-  __shared__ float wmax[NPW][NC], wsum[NPW][NC], cm[NC];
+  __shared__ float wmax[NPW][NC], wsum[NPW][NC];
   PYRE_TS_VARS PYRE_TS(0);
   // Workgroups in dispatch order (x fastest): chunks descending, the KV heads of a chunk next to each other.  The
   // workgroups past the view (a captured launch covers the whole cache) leave first; the chunks of the f32 window, which
@@ -207,14 +207,15 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
       }
     }
     __syncthreads();
-    if (tid < ncol) { float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]); cm[tid] = mm; }
-    __syncthreads();
 #pragma unroll
     for (int gi = 0; gi < GH; ++gi) {
       const int c = dq + 4 * gi;
       if (c < ncol) {
         const bool valid = p < start + tk0 + c / G + 1;
-        float e = valid ? expf(sv[gi] - cm[c]) : 0.0f; sc[c][pos] = e;
+        float mm = wmax[0][c];          // the chunk's maximum of the column: every thread takes it from the waves' maxima itself
+#pragma unroll
+        for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][c]);
+        float e = valid ? expf(sv[gi] - mm) : 0.0f; sc[c][pos] = e;
         const float l = wave_sum(e);
         if (lane == 0) wsum[pw][c] = l;
       }
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
     __syncthreads();          // weights of every position visible; the score partials in `red` are dead
   };
   // A wave is on one of two paths for the whole kernel -- packed positions or f32 ones (the branch is scalar: wbase is a
-  // wave's) -- each with its own registers; both pass the same five barriers.
+  // wave's) -- each with its own registers; both pass the same four barriers.
   if (active && packed) {             // packed positions lie below the boundary, hence inside the view
     // Lane (li, lg) of the value product stands for two dims of a scale block (word li & 3, nibbles 2 * (li >> 2) + m) at
     // the eight positions 8 * lg .. of a 32-position group: vw[g][b][p] is the word of position 32 * g + 8 * lg + p in
@@ -439,7 +440,8 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW, 4) void k_attn_decode(AttnDev 
   if (tid < ncol) {
     float l = wsum[0][tid]; for (int q = 1; q < NPW; ++q) l += wsum[q][tid];
     float* ml = part_ml + (((size_t)(tk0 + tid / G) * a.nh + (size_t)kvh * G + tid % G) * max_chunks + chunk) * 2;
-    ml[0] = cm[tid]; ml[1] = l;
+    float mm = wmax[0][tid]; for (int q = 1; q < NPW; ++q) mm = fmaxf(mm, wmax[q][tid]);
+    ml[0] = mm; ml[1] = l;
   }
 #ifdef PYRE_PHASE_TS
   PYRE_TS(7);
@@ -638,21 +640,22 @@ __global__ __launch_bounds__(256 * PYRE_ATTN_NPW) void k_attn_decode_sel(AttnDev
   }
 }
 
-// grid (nh, t, HD/64), 256 threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
-// Thread (grp, dim) adds the chunks grp, grp+4, ... in ascending order; the four groups are then added in order.
-// A workgroup owns 64 dimensions of a head and goes through the chunks 320 at a time: the 80 partial outputs a thread
-// needs of such a tile do not depend on the maximum, so the first tile's are fetched at the start, together with the
-// (max, sum) pairs; thread c of the tile (and again thread c - 256 for the last 64) then leaves exp(max_c - M) and sum_c
-// in shared memory for everybody.  Up to 320 chunks (40 960 positions) the whole merge is one memory round trip -- the
-// step after a 32 768-token prompt has 257 chunks.
+// grid (nh, t, HD/16), 256 threads: merge the chunk partials (log-sum-exp), normalise, multiply by sigmoid(gate).
+// Thread (grp, dim) adds the chunks grp, grp+16, ... in ascending order; the sixteen groups are then added in order.
+// A workgroup owns 16 dimensions of a head -- the partial outputs are most of what a long context makes this kernel read,
+// and a compute unit fetches them no faster than about 20 GB/s, so they are spread over nh * 16 workgroups -- and goes
+// through the chunks 320 at a time: the 20 partial outputs a thread needs of such a tile do not depend on the maximum,
+// so the first tile's are fetched at the start, together with the (max, sum) pairs and the gate; thread c of the tile
+// (and again thread c - 256 for the last 64) then leaves exp(max_c - M) and sum_c in shared memory for everybody.  Up to
+// 320 chunks (40 960 positions) the whole merge is one memory round trip -- the step after a 32 768-token prompt has 257.
 template <int HD>
 __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                       int max_chunks, float* __restrict__ out, const int* __restrict__ pcount) {
-  constexpr int CB = 320, B = CB / 4;
+  constexpr int CB = 320, DW = PYRE_ATTN_CDIMS, NG = 256 / DW, B = CB / NG;
   PYRE_TS_VARS PYRE_TS(0);
-  __shared__ float wmax[4]; __shared__ float so[4][64]; __shared__ float sl[4]; __shared__ float fs[CB], ls[CB];
+  __shared__ float wmax[4]; __shared__ float so[NG][DW]; __shared__ float sl[NG]; __shared__ float fs[CB], ls[CB];
   if (posp) start = *posp;
-  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid >> 6, dd = blockIdx.z * 64 + (tid & 63);
+  const int h = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, grp = tid / DW, dl = tid % DW, dd = blockIdx.z * DW + dl;
   int n = start + ti + 1; if (pcount && pcount[ti] >= 0) n = pcount[ti];        // a position list: its entries are what the chunks covered
   const int nc = (n + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK;
   const float* ml = part_ml + ((size_t)ti * a.nh + h) * max_chunks * 2;
@@ -660,7 +663,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
   const float gate = grp == 0 ? qkv[(size_t)ti * stride + (size_t)h * 2 * HD + HD + dd] : 0.0f;          // fetched with the partials, not after them
   float pv[B];
 #pragma unroll
-  for (int i = 0; i < B; ++i) pv[i] = nc > 0 ? po[(size_t)min(grp + 4 * i, nc - 1) * HD + dd] : 0.0f;
+  for (int i = 0; i < B; ++i) pv[i] = nc > 0 ? po[(size_t)min(grp + NG * i, nc - 1) * HD + dd] : 0.0f;
   float m0 = -INFINITY, l0 = 0.0f, m1 = -INFINITY, l1 = 0.0f;          // the tile's chunks tid and (threads below 64) 256 + tid
   if (tid < nc) { m0 = ml[2 * tid]; l0 = ml[2 * tid + 1]; }
   if (tid < CB - 256 && 256 + tid < nc) { m1 = ml[2 * (256 + tid)]; l1 = ml[2 * (256 + tid) + 1]; }
@@ -674,7 +677,7 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
     if (cb > 0) {
       __syncthreads();
 #pragma unroll
-      for (int i = 0; i < B; ++i) pv[i] = po[(size_t)min(cb + grp + 4 * i, nc - 1) * HD + dd];
+      for (int i = 0; i < B; ++i) pv[i] = po[(size_t)min(cb + grp + NG * i, nc - 1) * HD + dd];
       m0 = -INFINITY; l0 = 0.0f; if (cb + tid < nc) { m0 = ml[2 * (cb + tid)]; l0 = ml[2 * (cb + tid) + 1]; }
       m1 = -INFINITY; l1 = 0.0f; if (tid < CB - 256 && cb + 256 + tid < nc) { m1 = ml[2 * (cb + 256 + tid)]; l1 = ml[2 * (cb + 256 + tid) + 1]; }
     }
@@ -682,12 +685,14 @@ __global__ __launch_bounds__(256) void k_attn_combine(AttnDev a, const float* __
     if (tid < CB - 256) { fs[256 + tid] = expf(m1 - M); ls[256 + tid] = l1; }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < B; ++i) if (cb + grp + 4 * i < nc) { const float f = fs[grp + 4 * i]; L = fmaf(ls[grp + 4 * i], f, L); o = fmaf(pv[i], f, o); }
+    for (int i = 0; i < B; ++i) if (cb + grp + NG * i < nc) { const float f = fs[grp + NG * i]; L = fmaf(ls[grp + NG * i], f, L); o = fmaf(pv[i], f, o); }
   }
-  so[grp][tid & 63] = o; if ((tid & 63) == 0) sl[grp] = L;
+  so[grp][dl] = o; if (dl == 0) sl[grp] = L;
   __syncthreads();
   if (grp == 0) {
-    o = ((so[0][tid] + so[1][tid]) + so[2][tid]) + so[3][tid]; L = ((sl[0] + sl[1]) + sl[2]) + sl[3];
+    o = so[0][dl]; L = sl[0];
+#pragma unroll
+    for (int g = 1; g < NG; ++g) { o += so[g][dl]; L += sl[g]; }
     const float ov = (o / L) * a_sigm(gate);
     out[((size_t)ti * a.nh + h) * HD + dd] = ov;
   }
@@ -760,7 +765,7 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   switch (G) { case 1: launch_decode<1>(ctx, a, kv, w, start, t, posp, qw); break; case 2: launch_decode<2>(ctx, a, kv, w, start, t, posp, qw); break; case 4: launch_decode<4>(ctx, a, kv, w, start, t, posp, qw); break;
     default: launch_decode<8>(ctx, a, kv, w, start, t, posp, qw); } }
   PYRE_CHECK_LAUNCH(ctx);
-  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t, 256 / 64), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_combine", 4.0 * t * a.nh * a.hd * ((start + t + PYRE_ATTN_CHUNK - 1) / PYRE_ATTN_CHUNK + 2)); hipLaunchKernelGGL((k_attn_combine<256>), dim3(a.nh, t, 256 / PYRE_ATTN_CDIMS), dim3(256), 0, ctx->stream, a, qkv, stride, start, posp, w.part_o, w.part_ml, w.max_chunks, out, qw ? qw->pcount : (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

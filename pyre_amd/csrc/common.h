@@ -362,6 +362,7 @@ struct KvDev {
 };
 __host__ __device__ inline size_t kv_blk(size_t r, size_t R, size_t p) { return ((p >> 6) * R + r) * 64 + (p & 63); }
 #define PYRE_ATTN_NPW 2                       // 64-position groups per attention workgroup
+#define PYRE_ATTN_CDIMS 16                    // head dims a workgroup of the chunk merge owns
 #define PYRE_ATTN_CHUNK (64 * PYRE_ATTN_NPW)   // positions per chunk (one workgroup per chunk and KV head)
 struct AttnWork { float* q; uint16_t* qh; float* qsc; float* part_o; float* part_ml; int max_chunks; };   // q [8][nh][hd], its f16 halves [8][nh][2][hd] and their scale [8][nh]; partials per (token, head, chunk)
 size_t pyre_kv_bytes(const AttnDev& a, int cap);
