@@ -135,14 +135,31 @@ def bench_gemv(args):
     kernels = [{"kernel": k, "launches_per_step": round(v[0] / pn, 2), "avg_launch_us": round(v[1] / v[0] * 1e3, 3)} for k, v in sorted(prof.items(), key=lambda kv: -kv[1][1])]
     dom_us = kernels[0]["avg_launch_us"] if kernels else per * 1e3
     alg_bytes = mats[0].gguf_bytes + 4 * t * cols + 4 * t * rows
-    traffic = None; traffic_source = None          # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary (not this run), when present
-    try:
-        prof_file = "gemv_iq3s_vocab_head_kernel_stats.txt" if os.environ.get("PYRE_QMATMUL_F32") == "1" else "gemm_m_iq3s_vocab_head_kernel_stats.txt"
-        for line in open(os.path.join(ROOT, "profiles", prof_file)):
-            if t == 1 and ty == lib.IQ3_S and line.startswith("traffic_bytes_per_launch:"):
-                traffic = int(line.split(":")[1]); traffic_source = "profiles/%s: rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, not this run" % prof_file
-    except OSError:
-        pass
+    dom_name = kernels[0]["kernel"] if kernels else None
+    # which kernel the operator took: one token of an IQ3_S matrix streams the native layout (the file's bits per weight)
+    # through integer dot products, a window the matrix-core layout; PYRE_QMATMUL_F32=1 / other block types the lane = row GEMV
+    if ty != lib.IQ3_S or os.environ.get("PYRE_QMATMUL_F32") == "1":
+        layout, path = 0, "f32 multiply-add GEMV, lane = row (k_gemv)"
+    elif t == 1 and os.environ.get("PYRE_QMATMUL_NATIVE", "1") != "0":
+        layout, path = 2, "native-format GEMV (k_gemv_n: 13-bit codebook-index + sign fields, signed codebook in shared memory, v_dot4_i32_i8), preceded by the activation digits launch k_act_digits_n"
+    else:
+        layout, path = 1, "f16 matrix cores (k_gemm_m, preceded by the operand split k_act_split): the kernel the model's projections and head run on a window"
+    # HBM bytes per launch and the kernel-trace duration come from the committed counter summary of this very kernel
+    # (not from this run); a summary that names another kernel is not quoted
+    traffic = None; traffic_source = None; trace_us = None
+    prof_file = {0: "gemv_lane_row_iq3s_vocab_head_kernel_stats.txt", 1: "gemm_m_iq3s_vocab_head_kernel_stats.txt", 2: "gemv_n_iq3s_vocab_head_kernel_stats.txt"}[layout]
+    if ty == lib.IQ3_S:
+        try:
+            fields = {}
+            for line in open(os.path.join(ROOT, "profiles", prof_file)):
+                if ":" in line and not line.startswith(" "):
+                    k_, v_ = line.split(":", 1); fields[k_.strip()] = v_.strip()
+            if fields.get("profiled_kernel_class") == dom_name and fields.get("tokens_per_launch") == str(t):
+                traffic = int(fields["traffic_bytes_per_launch"]) if "traffic_bytes_per_launch" in fields else None
+                trace_us = float(fields["kernel_trace_avg_us"]) if "kernel_trace_avg_us" in fields else None
+                traffic_source = "profiles/%s: rocprofv3 FETCH_SIZE + WRITE_SIZE and --kernel-trace runs of this command, not this run" % prof_file
+        except (OSError, ValueError):
+            pass
     gbs = alg_bytes / (per * 1e-3) / 1e9                 # whole step (every launch of the operator call)
     kgbs = alg_bytes / (dom_us * 1e-6) / 1e9             # the dominant kernel alone
     out = {
@@ -150,10 +167,12 @@ def bench_gemv(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
-        "path": ("f32 multiply-add GEMV, lane = row (k_gemv)" if ty != lib.IQ3_S or os.environ.get("PYRE_QMATMUL_F32") == "1" else
-                 "f16 matrix cores (k_gemm_m, preceded by the operand split k_act_split): the kernel the model's projections and head run"),
-        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": kernels[0]["kernel"] if kernels else None, "device_bytes_per_launch": mats[0].layout_bytes(ty == lib.IQ3_S and os.environ.get("PYRE_QMATMUL_F32") != "1") or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
+        "path": path,
+        "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4),
+                     "frac_is": "algorithmic bytes / this run's event-pair duration of the dominant kernel (an event pair reads about 0.3 us longer than the kernel trace on this kernel)",
+                     "frac_kernel_trace": round(alg_bytes / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if trace_us else None, "kernel_trace_avg_us": trace_us,
+                     "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": dom_name, "device_bytes_per_launch": mats[0].layout_bytes(layout) or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
         "kernels": kernels,
     }
     if not args.no_cpu:
@@ -487,6 +506,7 @@ def bench_decode(args):
         done += piece.size
         if done % 8192 == 0 or last:
             log("prefill %d / %d tokens (%.1f s)" % (done, n_ctx, time.perf_counter() - t0))
+    ctx.sync(); prefill_s = time.perf_counter() - t0
     first = int(np.argmax(lg))
     toks = model.decode_greedy_dev(st, first, args.warmup) if args.warmup else np.array([first], dtype=np.uint32)
     nxt = int(toks[-1])
@@ -567,17 +587,31 @@ def bench_decode(args):
                   "avg_launch_us": round(v[1] / v[0] * 1e3, 3), "GBps": round(v[2] / (v[1] * 1e-3) / 1e9, 1) if v[1] > 0 else None} for k, v in classes]
     dom_k, dom = classes[0]
     dom_gbs = dom[2] / (dom[1] * 1e-3) / 1e9
-    # HBM bytes per launch of the dominant class: not measured by this run but read from the committed FETCH_SIZE /
-    # WRITE_SIZE summary (a three-layer slice of the same step), when that covers the class; traffic_source says so
-    traffic = None; traffic_source = None
-    if cfg.n_layers == 48 and not args.indexer:
+    # HBM bytes per launch of the dominant class and its kernel-trace duration: not measured by this run but read from
+    # the committed counter summaries (FETCH_SIZE / WRITE_SIZE on a three-layer slice of this step; --kernel-trace of this
+    # command).  A summary whose kernel classes are not the classes this run reports is stale and is not quoted.
+    traffic = None; traffic_source = None; trace_us = None
+    def prof_fields(name):
+        f = {}
         try:
-            for line in open(os.path.join(ROOT, "profiles", "decode_deltanet_slice_hbm_traffic.txt")):
-                if line.startswith("traffic_bytes_per_launch_%s:" % dom_k):
-                    traffic = int(line.split(":")[1])
-                    traffic_source = "profiles/decode_deltanet_slice_hbm_traffic.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE on a three-layer slice of this step, not this run; attention-layer launches of the class are not covered"
+            for line in open(os.path.join(ROOT, "profiles", name)):
+                if ":" in line and not line.startswith(" "):
+                    k_, v_ = line.split(":", 1); f[k_.strip()] = v_.strip()
         except OSError:
             pass
+        return f
+    mine = set(prof.keys())
+    if cfg.n_layers == 48 and not args.indexer:
+        f = prof_fields("decode_deltanet_slice_hbm_traffic.txt")
+        theirs = set(x.strip() for x in f.get("profiled_kernel_classes", "").split(",") if x.strip())
+        if theirs and theirs <= mine and ("traffic_bytes_per_launch_%s" % dom_k) in f:
+            traffic = int(f["traffic_bytes_per_launch_%s" % dom_k])
+            traffic_source = ("profiles/decode_deltanet_slice_hbm_traffic.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE on a three-layer DeltaNet slice of this step launched kernel by kernel, not this run; "
+                              "the attention layers' launches of the class and the traffic under graph replay are not measured")
+        f = prof_fields("decode_a3b_ctx%d_kernel_stats.txt" % n_ctx)
+        theirs = set(x.strip() for x in f.get("profiled_kernel_classes", "").split(",") if x.strip())
+        if theirs and theirs <= mine and ("kernel_trace_avg_us_%s" % dom_k) in f:
+            trace_us = float(f["kernel_trace_avg_us_%s" % dom_k])
     # the MTP drafter beside the model (synthetic weights of the main layers' geometry, draft head of the reference's
     # default draft vocabulary size): cost of a draft call and of a drafted round.  Random weights draft tokens the model
     # does not pick, so the acceptance seen here says nothing; tok/s at a given acceptance follows from the two costs.
@@ -588,23 +622,51 @@ def bench_decode(args):
         dr_ = lib.Mtp(model, cfg.n_exp, cfg.top_k, cfg.ff_exp, 128, mt, np.arange(args.mtp_vocab, dtype=np.uint32) * (cfg.vocab // args.mtp_vocab))
         for p in mraw:
             ctx.free(p)
+        n_g = 33
         snap = st.snapshot()
+        plain_all = model.decode_greedy_dev(st, nxt, 136 + n_g + 16)    # the plain greedy stream the drafted loops must reproduce
+        st.restore(snap)
         dr_.attach(st)
-        tail = model.decode_greedy_dev(st, nxt, 136)                    # fills the residual ring over a full window
-        pend = int(tail[-1])
-        dr_.draft(st, pend, kd)                                         # untimed: the catch-up over the window's cells
+        def warm():
+            tail = model.decode_greedy_dev(st, nxt, 136)                # fills the residual ring over a full window
+            p_ = int(tail[-1])
+            dr_.draft(st, p_, kd)                                       # untimed: the catch-up over the window's cells
+            return p_
+        pend = warm()
         ctx.sync(); t0 = time.perf_counter()
         for i in range(8):
             dr_.draft(st, pend, kd)
         d_ms = (time.perf_counter() - t0) * 1e3 / 8
         fl = np.zeros(cfg.vocab, dtype=np.float32); fl[pend] = 1.0
-        n_g = 33
+        # (1) every draft accepted: the drafter runs, then its ids are replaced by the plain stream's (the accepted path end to end)
+        forced = np.concatenate([plain_all[135:], np.zeros(16, np.uint32)]).astype(np.uint32)
+        ctx.sync(); t0 = time.perf_counter()
+        out_a, rounds_a, drafted_a, accepted_a = dr_.generate_greedy_forced(st, fl, n_g, forced, k=kd)
+        ctx.sync(); a_dt = time.perf_counter() - t0
+        if not np.array_equal(out_a, plain_all[135:135 + n_g]):
+            raise SystemExit("drafted generation (forced drafts) diverged from plain greedy decoding")
+        # (2) the synthetic drafter's own drafts (random weights: the model picks none of them): the rejected path
+        st.restore(snap); pend = warm()
         ctx.sync(); t0 = time.perf_counter()
         out_t, rounds, drafted, accepted = dr_.generate_greedy(st, fl, n_g, k=kd)
         ctx.sync(); g_dt = time.perf_counter() - t0
+        if not np.array_equal(out_t, plain_all[135:135 + n_g]):
+            raise SystemExit("drafted generation diverged from plain greedy decoding")
+        r_acc, r_rej = a_dt * 1e3 / max(rounds_a, 1), g_dt * 1e3 / max(rounds, 1)
+        def implied(a):          # per-draft acceptance a, kd drafts a round: 1 + a + .. + a^kd tokens per round; a round costs between the two measured ones
+            toks = (1.0 - a ** (kd + 1)) / (1.0 - a) if a < 1.0 else kd + 1.0
+            full = a ** kd                                              # rounds whose drafts are all kept take the accepted-path cost
+            return round(toks / ((full * r_acc + (1.0 - full) * r_rej) * 1e-3), 1)
         mtp = {"drafts_per_call": kd, "draft_vocab": args.mtp_vocab, "window": 128, "ms_per_draft_call": round(d_ms, 3), "ms_per_draft_step": round(d_ms / kd, 3),
-               "generate": {"tokens": n_g - 1, "rounds": rounds, "drafted": drafted, "accepted": accepted, "tok_s": round((n_g - 1) / g_dt, 1), "ms_per_round": round(g_dt * 1e3 / max(rounds, 1), 3)},
-               "note": "synthetic drafter: 512 experts top-10 of width 512 like a main layer; a call = catch-up of the newly committed cells + k draft steps + one readback"}
+               "drafted_round_ms": {"all_drafts_accepted": round(r_acc, 3), "no_draft_accepted": round(r_rej, 3),
+                                    "rounds": [rounds_a, rounds], "drafted": [drafted_a, drafted], "accepted": [accepted_a, accepted]},
+               "accepted_path_tok_s": round((n_g - 1) / a_dt, 1),
+               "implied_tok_s_at_acceptance": {"0.68": implied(0.68), "0.8": implied(0.8), "0.87": implied(0.87)},
+               "plain_decode_tok_s": round(tok_s, 1),
+               "note": "synthetic drafter (512 experts top-10 of width 512 like a main layer, random weights): its own drafts are never the model's pick, so the rate a trained drafter "
+                       "would give is not measured; measured are the cost of a draft call (catch-up of the newly committed cells + k draft steps + one readback) and of a drafted round "
+                       "with every draft accepted (the drafter's ids replaced by the plain stream's after it ran) and with none; implied = expected tokens per round at the "
+                       "reference's per-draft acceptance range / the round cost"}
         dr_.close()
         st.restore(snap)
     out = {
@@ -616,15 +678,21 @@ def bench_decode(args):
                                "4-bit KV, greedy decode after a %d-token random prompt%s" % (
                                    cfg.n_layers, cfg.hc_d_div, n_ctx, (", QSA indexer with %d heads (budget 2048, blocks of 4): variant, not the configuration of the metric" % args.indexer) if args.indexer else ""),
                    "context": n_ctx, "layers": cfg.n_layers, "hc_d_div": cfg.hc_d_div},
-        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(dom_gbs / HBM_PEAK_GBS, 4),
+                     "frac_is": "algorithmic bytes / this run's event-pair duration of the class (launches of a few microseconds read 3 to 4 us longer between two events than in the kernel trace)",
+                     "frac_kernel_trace": round(dom[2] / dom[0] / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if trace_us else None, "kernel_trace_avg_us": trace_us,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": dom_k, "algorithmic_bytes_per_launch": round(dom[2] / dom[0]), "avg_launch_us": round(dom[1] / dom[0] * 1e3, 3),
                      "share_of_kernel_time": round(dom[1] / tot_ms, 3)},
         "token_roofline": {"weight_bytes_per_token": wbytes, "kv_bytes_per_token": round(kvb), "state_bytes_per_token": state_b,
                            "weights_only": {"GBps": round(wbytes / (per * 1e-3) / 1e9, 1), "frac": round(wbytes / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
                            "all_bytes": {"GBps": round(all_b / (per * 1e-3) / 1e9, 1), "frac": round(all_b / (per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
-                           "kernel_time_us_per_token": round(tot_ms / pn * 1e3, 1)},
+                           "kernel_time_us_per_token": round(tot_ms / pn * 1e3, 1),
+                           "hyper_connection_share_of_kernel_time": round(sum(v[1] for k, v in prof.items() if k.startswith("hc_")) / tot_ms, 3)},
         "kernels": breakdown,
     }
+    out["prompt"] = {"tokens": n_ctx, "seconds": round(prefill_s, 2), "tok_s": round(n_ctx / prefill_s, 1),
+                     "note": "pyre_forward over the prompt in calls of 2048 tokens (windows of 8 tokens, three windows in flight), logits of the last token only; untimed part of the step metric"}
     if spec:
         out["spec_verify"] = spec
     if host_loop:

@@ -355,6 +355,12 @@ int   pyre_mtp_read_kv(pyre_ctx* ctx, pyre_state* s, int* c0, int* n, float* k_h
  * in one window and keeps the agreeing prefix.  The output equals plain greedy decoding token for token. */
 int   pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
                                int k, float min_p, int* rounds, int* drafted, int* accepted);
+/* The same loop for measurements of the accepted path: the drafter runs every round (its cost is paid), then its ids are
+ * replaced by forced_stream[produced ..] (at least n_out + 8 ids).  With the plain greedy output there (entry i = the
+ * i-th token of that output, entry 0 the first pick) every draft is accepted, whatever the drafter's weights would draft.
+ * No counterpart in the reference; the reference reports acceptance of trained drafters (docs/HANDOFF.md:28). */
+int   pyre_generate_greedy_mtp_forced(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits_host, int n_out, uint32_t* out,
+                                      int k, const uint32_t* forced_stream, int* rounds, int* drafted, int* accepted);
 /* The decode loop as the benchmark times it: n_steps greedy steps starting from token `first`, everything on the device;
  * tokens (optional, host) receives the n_steps generated ids after the call. */
 int   pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint32_t first, int n_steps, uint32_t* tokens_host);

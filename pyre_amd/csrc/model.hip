@@ -1092,7 +1092,9 @@ int pyre_mtp_read_kv(pyre_ctx* ctx, pyre_state* s, int* c0, int* n, float* k_hos
   return PYRE_OK;
 }
 
-int pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* rounds_out, int* drafted_out, int* accepted_out) {
+// forced: the drafter runs (its cost is paid) and its ids are then replaced by forced[produced ..] -- with the plain greedy
+// stream there, every draft is accepted: the accepted path timed end to end, whatever the drafter's weights would draft
+static int generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* rounds_out, int* drafted_out, int* accepted_out, const uint32_t* forced) {
   if (!ctx || !m || !mtp || !s || !first_logits || !out || n_out < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp: bad argument");
   if (k < 1 || k > 7) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp: k %d outside 1..7", k);
   if (s->mtp != mtp) return pyre_fail(ctx, PYRE_E_STATE, "pyre_generate_greedy_mtp: this drafter is not attached to the state");
@@ -1103,6 +1105,7 @@ int pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp*
     const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
     uint32_t toks[8]; float ps[8]; toks[0] = pending; int nd = 0;
     if (kk > 0) { int rc = pyre_mtp_draft(ctx, mtp, s, pending, kk, min_p, toks + 1, ps, &nd); if (rc) return rc; }
+    if (forced && kk > 0) { nd = kk; for (int j = 0; j < kk; ++j) toks[j + 1] = forced[produced + j]; }
     uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
     int acc = 0; bool have = false; uint32_t nx = 0;
     for (int i = 0; i < nd; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
@@ -1115,6 +1118,13 @@ int pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp*
   }
   if (rounds_out) *rounds_out = rounds; if (drafted_out) *drafted_out = drafted; if (accepted_out) *accepted_out = accepted;
   return PYRE_OK;
+}
+int pyre_generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int k, float min_p, int* rounds_out, int* drafted_out, int* accepted_out) {
+  return generate_greedy_mtp(ctx, m, mtp, s, first_logits, n_out, out, k, min_p, rounds_out, drafted_out, accepted_out, nullptr);
+}
+int pyre_generate_greedy_mtp_forced(pyre_ctx* ctx, const pyre_model* m, const pyre_mtp* mtp, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int k, const uint32_t* forced_stream, int* rounds_out, int* drafted_out, int* accepted_out) {
+  if (!forced_stream) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp_forced: null draft stream");
+  return generate_greedy_mtp(ctx, m, mtp, s, first_logits, n_out, out, k, 0.0f, rounds_out, drafted_out, accepted_out, forced_stream);
 }
 
 }  // extern "C"

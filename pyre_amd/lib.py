@@ -122,6 +122,7 @@ def _declare(L):
         "pyre_mtp_draft": (i32, [vp, vp, vp, u32, i32, f32, vp, vp, C.POINTER(i32)]),
         "pyre_mtp_read_kv": (i32, [vp, vp, C.POINTER(i32), C.POINTER(i32), vp, vp]),
         "pyre_generate_greedy_mtp": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, f32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
+        "pyre_generate_greedy_mtp_forced": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -746,6 +747,15 @@ class Mtp:
         out = np.empty(n_out, dtype=np.uint32); r, d, a = C.c_int(0), C.c_int(0), C.c_int(0)
         self.m.ctx.check(self.m.ctx.L.pyre_generate_greedy_mtp(self.m.ctx.h, self.m.h, self.h, st.h, _ptr(fl), n_out, _ptr(out), k, min_p,
                                                                C.byref(r), C.byref(d), C.byref(a)), "generate_greedy_mtp")
+        return out, r.value, d.value, a.value
+
+    def generate_greedy_forced(self, st, first_logits, n_out, forced_stream, k=3):
+        """The same loop with the drafter's ids replaced (after it ran) by forced_stream: the accepted path end to end."""
+        fl = np.ascontiguousarray(first_logits, dtype=np.float32); fs = np.ascontiguousarray(forced_stream, dtype=np.uint32)
+        assert fs.size >= n_out + 8
+        out = np.empty(n_out, dtype=np.uint32); r, d, a = C.c_int(0), C.c_int(0), C.c_int(0)
+        self.m.ctx.check(self.m.ctx.L.pyre_generate_greedy_mtp_forced(self.m.ctx.h, self.m.h, self.h, st.h, _ptr(fl), n_out, _ptr(out), k, _ptr(fs),
+                                                                      C.byref(r), C.byref(d), C.byref(a)), "generate_greedy_mtp_forced")
         return out, r.value, d.value, a.value
 
     def close(self):
