@@ -169,7 +169,7 @@ def bench_gemv(args):
         "config": {"workload": "configs[1]: %s GEMV 2048->151936, batch %d, rotating over %d weight buffers (%.0f MB)" % (FN, t, nbuf, nbuf * mats[0].gguf_bytes / 1e6)},
         "path": path,
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(kgbs / HBM_PEAK_GBS, 4),
-                     "frac_is": "algorithmic bytes / this run's event-pair duration of the dominant kernel (an event pair reads about 0.3 us longer than the kernel trace on this kernel)",
+                     "frac_is": "algorithmic bytes / this run's event-pair duration of the dominant kernel; frac_kernel_trace: the same bytes / the kernel-trace duration in the committed profile",
                      "frac_kernel_trace": round(alg_bytes / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if trace_us else None, "kernel_trace_avg_us": trace_us,
                      "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": dom_name, "device_bytes_per_launch": mats[0].layout_bytes(layout) or mats[0].dev_bytes, "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": dom_us},
@@ -244,7 +244,7 @@ def bench_gemv0(args):
                      "dominant_kernel": dom[0], "dominant_kernel_us": round(dom[1][1], 3), "dominant_kernel_GBps": round(alg / (dom[1][1] * 1e-6) / 1e9, 1)}
     op = res["operator"]
     roof = {"bound": "hbm", "achieved": op["dominant_kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(op["dominant_kernel_GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": op["dominant_kernel"], "algorithmic_bytes_per_launch": alg, "device_bytes_per_launch": mats[0].layout_bytes(True), "avg_launch_us": op["dominant_kernel_us"]}
+            "kernel": op["dominant_kernel"], "algorithmic_bytes_per_launch": alg, "device_bytes_per_launch": mats[0].layout_bytes(0), "avg_launch_us": op["dominant_kernel_us"]}
     extra = {"paths": res}
     if not args.no_cpu:
         import orc
@@ -257,7 +257,7 @@ def bench_gemv0(args):
         extra["cpu_baseline"] = {"value": round(n * alg / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
                                  "sample": "%d calls of the oracle matmul (row dequant + f32 dot, rows over %d threads) on the whole 4096 x 4096 IQ3_S matrix, t=1" % (n, threads)}
     return _line("IQ3_S dequant-GEMV achieved HBM GB/s (4096x4096, t=1)", op["GBps_rotating"], "GB/s", args, op["us_per_call_rotating"] / 1e3, "f32",
-                 "configs[0]: IQ3_S GEMV 4096x4096, batch 1, rotating over %d weight buffers (%.0f MB); operator path (integer dot) and f32 path" % (nbuf, nbuf * mats[0].gguf_bytes / 1e6), roof, extra)
+                 "configs[0]: IQ3_S GEMV 4096x4096, batch 1, rotating over %d weight buffers (%.0f MB); the operator (a single token of a matrix of at most 128 row tiles takes the one-launch lane = row f32 GEMV, the kernel of pyre_qmatmul_f32) and pyre_qmatmul_f32" % (nbuf, nbuf * mats[0].gguf_bytes / 1e6), roof, extra)
 
 
 def bench_sweep(args):

@@ -566,8 +566,15 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
 
 // The operator's own launch: an IQ3_S matrix goes through the matrix-core GEMM (for every t, so a token's result does not
 // depend on the window width); f32_path (or PYRE_QMATMUL_F32=1) takes the f32 lane = row GEMV the model's expert matrices use.
+static bool qmat_small_one_token(const pyre_qmat* m, int t) {
+  const int on = env_int("PYRE_QMATMUL_SMALL", 1);          // read at every call: tests switch it to reach the native-format kernel with small shapes
+  return on && t == 1 && m->dvm.fmt == FMT_IQ3_S_M && m->base != nullptr && m->dv.fmt == FMT_IQ3_S && m->dv.tiles <= 128;
+}
 static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev, bool f32_path) {
   static const int f32_only = env_int("PYRE_QMATMUL_F32", 0), native = env_int("PYRE_QMATMUL_NATIVE", 1);
+  // one token of a small IQ3_S matrix (at most 128 row tiles): the lane = row f32 GEMV -- one launch where the other two
+  // paths need a second one for the activations, and a call of this size is its launches, not its bytes
+  if (qmat_small_one_token(m, t) && !f32_path && !f32_only) return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   // one token of an IQ3_S matrix: the kernel that streams the file's 3.44 bit/weight (PYRE_QMATMUL_NATIVE=0: the matrix cores as for a window)
   if (t == 1 && m->base_n && native && !f32_path && !f32_only) return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
@@ -596,6 +603,8 @@ int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: t = %d outside 1..8", t);
   if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
+  if (qmat_small_one_token(m, t) && !env_int("PYRE_QMATMUL_F32", 0)) return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);      // as pyre_qmatmul_dev (a launch that happens to need no scratch; the limit above holds for every call alike)
   if (t == 1 && m->base_n && env_int("PYRE_QMATMUL_NATIVE", 1)) {      // one token: the native-format kernel, as in pyre_qmatmul_dev, its activation digits in the static array
     if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
     if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");

@@ -267,7 +267,8 @@ def test_verify_gemm_on_matrix_cores_matches_truth(ctx, rows, cols, t):
 
 # ---- one token of an IQ3_S matrix: the file's bits per weight, codebook with signs in shared memory, integer dots --------------
 @pytest.mark.parametrize("rows,cols", [(64, 256), (100, 256), (65, 512), (320, 2048), (4096, 2048), (2048, 4096), (1000, 768), (130, 8192)])
-def test_iq3s_native_format_single_token(ctx, rows, cols):
+def test_iq3s_native_format_single_token(ctx, rows, cols, monkeypatch):
+    monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the native-format kernel (the operator sends them to the one-launch f32 GEMV otherwise)
     raw = synth.matrix(lib.IQ3_S, rows, cols, 300 + rows % 97)
     m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
     assert m.layout_bytes(2) == (rows + 63) // 64 * 64 * (cols // 256) * 112
@@ -295,3 +296,21 @@ def test_iq3s_native_format_single_token(ctx, rows, cols):
     bad[0, 3] = np.nan
     assert np.isnan(m.matmul(bad)).all()
     assert not m.matmul(np.zeros((1, cols), np.float32)).any()
+
+
+@pytest.mark.gpu
+def test_small_iq3s_single_token_takes_one_launch(ctx):
+    """A single token of an IQ3_S matrix of at most 128 row tiles goes through the lane = row f32 GEMV (one launch): the
+    result is bit for bit pyre_qmatmul_f32's; a window and a large matrix are unaffected."""
+    rows, cols = 4096, 4096
+    raw = synth.matrix(lib.IQ3_S, rows, cols, 77)
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, raw)
+    x = synth.normal((1, cols), 78)
+    y = m.matmul(x)
+    assert np.array_equal(bits(y), bits(m.matmul_f32(x)))
+    W = orc.dequant(lib.IQ3_S, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    assert relerr(y, x.astype(np.float64) @ W.T) <= TOL
+    ctx.prof_reset(); ctx.prof_enable(True)
+    m.matmul(x); ctx.sync()
+    rep = ctx.prof_report(); ctx.prof_enable(False)
+    assert sum(v[0] for v in rep.values()) == 1, rep          # one kernel launch for the call
