@@ -19,6 +19,7 @@
 //
 // grid (row tiles of 64, K slices), NW waves.  Wave w of slice ks walks 128-column chunks [(ks*NW + w) * cpw, + cpw).
 #include "gemm_m.h"
+#include <mutex>
 
 PYRE_TS_DECL(gemm_ts) PYRE_TS_EXPORT(gemm_ts, pyre_debug_ts_gemm)
 
@@ -260,9 +261,11 @@ int pyre_gemm_m_scratch(pyre_ctx* ctx, int cols, uint4** op, float** ainv) {
 #define STATIC_OP_BYTES ((size_t)STATIC_MAX_COLS * 32)
 static __device__ __align__(256) uint8_t scratch[STATIC_OP_BYTES + (STATIC_MAX_COLS / 256) * 8 * 4];
 static void* g_scratch_ptr[64];
+static std::mutex g_scratch_mu;          // contexts may be created from several threads
 
 int pyre_static_init(pyre_ctx* ctx) {
   if (ctx->device < 0 || ctx->device >= 64) return pyre_fail(ctx, PYRE_E_ARG, "device %d outside 0..63", ctx->device);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
   if (!g_scratch_ptr[ctx->device]) {
     void* p = nullptr;
     PYRE_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));

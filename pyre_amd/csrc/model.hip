@@ -49,6 +49,7 @@ struct pyre_state {
   std::vector<QsaBuf> qsa; QsaWork qw{};                          // indexer keys per attention layer; selection workspace
   void* pipe_mem = nullptr; std::vector<AttnWork> aw_more; std::vector<QsaWork> qw_more;      // one more attention / selection workspace per further prompt stream
   int last_window = 0;                                           // tokens of the last forward_multi (0 = spec_keep unarmed)
+  bool broken = false;                                           // a call failed after it had begun to advance this state: every call but reset / restore refuses it
   uint32_t* tokens_dev = nullptr; std::vector<float*> ple_ring;     // PLE models: the token history by position; per PLE layer the ring of normalised rows
   int* step_dev = nullptr; hipGraphExec_t graph_exec = nullptr; const uint32_t* graph_toks = nullptr;   // replayed decode step
   std::vector<int> graph_cur;                                    // which half of every DeltaNet double buffer the captured step works on
@@ -305,7 +306,7 @@ int pyre_state_reset(pyre_ctx* ctx, pyre_state* s) {
   const pyre_model_cfg& c = s->m->c; size_t cs = (size_t)(c.conv_k - 1) * s->m->ch * 4, ss = (size_t)c.lin_nv * c.lin_dk * c.lin_dv * 4;
   for (size_t li = 0; li < s->cur.size(); ++li) { s->cur[li] = 0; PYRE_HIP(ctx, hipMemsetAsync(s->conv[0][li], 0, cs, ctx->stream)); PYRE_HIP(ctx, hipMemsetAsync(s->ssm[0][li], 0, ss, ctx->stream)); }
   for (auto& pk : s->packed) pk = 0;
-  s->len = 0; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
+  s->len = 0; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0; s->broken = false; PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 int pyre_state_len(const pyre_state* s) { return s ? s->len : 0; }
 int pyre_state_capacity(const pyre_state* s) { return s ? s->cap - 8 : 0; }
@@ -369,6 +370,7 @@ int snap_copy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, uint8_t* buf, i
 int pyre_state_snapshot(pyre_ctx* ctx, pyre_state* s, pyre_snap** out) {
   if (!ctx || !s || !out) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_snapshot: null argument");
   *out = nullptr;
+  if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "pyre_state_snapshot");
   std::unique_ptr<pyre_snap> sn(new pyre_snap()); sn->m = s->m; sn->len = s->len; sn->packed = s->packed; sn->bytes = snap_plan(s->m, s->len).total; sn->mem = nullptr;
   hipError_t e = hipMalloc(&sn->mem, sn->bytes);
   if (e != hipSuccess) return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_state_snapshot: hipMalloc(%zu): %s", sn->bytes, hipGetErrorString(e));
@@ -382,7 +384,7 @@ int pyre_state_restore(pyre_ctx* ctx, pyre_state* s, const pyre_snap* sn) {
   if (s->m != sn->m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: the snapshot belongs to another model");
   if (sn->len + 8 > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_state_restore: %d positions do not fit the state's capacity %d", sn->len, s->cap - 8);
   int rc = snap_copy(ctx, s->m, s, (uint8_t*)sn->mem, sn->len, 1); if (rc) return rc;
-  s->len = sn->len; s->packed = sn->packed; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0;      // the drafter starts over
+  s->len = sn->len; s->packed = sn->packed; s->last_window = 0; s->r_first = s->r_next = 0; s->m_c0 = s->m_n = 0; s->broken = false;      // the drafter starts over
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
 void pyre_snap_destroy(pyre_snap* sn) { if (!sn) return; (void)hipFree(sn->mem); delete sn; }
@@ -623,6 +625,7 @@ extern "C" {
 int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, float* logits_host) {
   if (!ctx || !m || !s || !ids || n < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward: bad argument");
   if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: state belongs to another model");
+  if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "pyre_forward");
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: %d + %d tokens exceed the state's capacity %d", s->len, n, s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   s->last_window = 0;
@@ -644,7 +647,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     if (s->mtp) { const int k0 = n - mtp_window_of(s->mtp) - i; o.keep_from = k0 < 0 ? 0 : k0; }      // the last `window` tokens of a call (qwen4exp_gguf.rs:2148-2150)
     if (!P) {
       PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids + i, (size_t)t * 4, hipMemcpyHostToDevice, ctx->stream));
-      if ((rc = run_window(ctx, m, s, t, o))) return rc;
+      if ((rc = run_window(ctx, m, s, t, o))) { s->broken = true; return rc; }
       continue;
     }
     const int set = (nwin - 1 - w) % K;          // the last window runs on the model's own stream and workspace: its logits are the call's
@@ -653,7 +656,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     o.wait_ev = prev >= 0 ? P->ev[prev].data() : nullptr; o.rec_ev = P->ev[set].data();
     rc = run_window(cx, mx, s, t, o);
     if (!rc && hipEventRecord(P->done[set], cx->stream) != hipSuccess) rc = pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
-    if (rc) { if (cx != ctx) pyre_fail(ctx, rc, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return rc; }
+    if (rc) { s->broken = true; if (cx != ctx) pyre_fail(ctx, rc, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return rc; }      // windows already issued have advanced the bookkeeping and part of the state
     prev = set;
   }
   if (P) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, P->done[k], 0));      // everything the other streams did precedes what follows here
@@ -665,6 +668,7 @@ int pyre_forward_multi(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const 
   if (!ctx || !m || !s || !ids || !logits_host) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward_multi: null argument");
   if (n < 1 || n > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_forward_multi: window of %d tokens outside 1..8", n);
   if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: state belongs to another model");
+  if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "pyre_forward_multi");
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward_multi: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
@@ -694,6 +698,7 @@ __global__ __launch_bounds__(1024) void k_argmax_rows(const float* __restrict__ 
 static int forward_multi_picks(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* ids, int n, uint32_t* picks_host) {
   if (n < 1 || n > 8) return pyre_fail(ctx, PYRE_E_ARG, "forward_multi: window of %d tokens outside 1..8", n);
   if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "forward_multi: state belongs to another model");
+  if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "forward_multi");
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward_multi: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   PYRE_HIP(ctx, hipMemcpyAsync(m->ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, ctx->stream));
@@ -727,6 +732,7 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
   pyre_model* m = const_cast<pyre_model*>(mc);
   if (!ctx || !m || !s || n_steps < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_decode_greedy_dev: bad argument");
   if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_decode_greedy_dev: state belongs to another model");
+  if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "pyre_decode_greedy_dev");
   if (s->len + n_steps > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_decode_greedy_dev: context exceeds the state's capacity %d", s->cap);
   int rc = check_ids(ctx, m, &first, 1); if (rc) return rc;
   if (m->toks_cap < n_steps) { if (m->toks) { PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); PYRE_HIP(ctx, hipFree(m->toks)); m->toks = nullptr; } PYRE_HIP(ctx, hipMalloc((void**)&m->toks, (size_t)n_steps * 4)); m->toks_cap = n_steps; }

@@ -65,3 +65,48 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit_and_other_types(ct
     for p in (xd, yd, ya):
         ctx.free(p)
     wide.close(); edge.close(); q8.close()
+
+
+def test_static_entry_point_under_stream_capture(ctx):
+    """The claim 'no allocation, no event, no synchronisation' checked by the runtime itself: a stream capture fails on any
+    of them.  The call is captured for one token of a large matrix (the native-format kernel, activation digits in the
+    array) and for a window (operand rows in the array), the graphs are replayed with other calls on the array in between,
+    and every replay gives the bits of pyre_qmatmul_dev."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]; hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    stream = C.c_void_p(ctx.stream)
+    rows, cols = 8320, 2048          # 130 row tiles: a single token takes the native-format kernel
+    m = lib.QMat(ctx, lib.IQ3_S, rows, cols, synth.matrix(lib.IQ3_S, rows, cols, 601))
+    other = lib.QMat(ctx, lib.IQ3_S, 320, 4096, synth.matrix(lib.IQ3_S, 320, 4096, 602))
+    x = synth.normal((8, cols), 603); xo = ctx.upload(synth.normal((8, 4096), 604)); yo = ctx.alloc(8 * 320 * 4)
+    xd = ctx.upload(x)
+    for t in (1, 5):
+        yref = ctx.alloc(t * rows * 4); ycap = ctx.alloc(t * rows * 4)
+        m.matmul_dev(xd, t, yref); ctx.sync()
+        want = ctx.download(yref, (t, rows)).view(np.uint32)
+        assert hip.hipStreamBeginCapture(stream, 0) == 0          # hipStreamCaptureModeGlobal: unsafe calls from any thread fail
+        try:
+            m.matmul_static_dev(xd, t, ycap)
+        finally:
+            graph = C.c_void_p(); rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0 and graph.value
+        ex = C.c_void_p()
+        assert hip.hipGraphInstantiate(C.byref(ex), graph, None, None, 0) == 0
+        for rep in range(3):
+            other.matmul_static_dev(xo, 8 if rep else 1, yo)          # eager work on the same array between the replays
+            z = ctx.upload(np.zeros((t, rows), np.float32)); ctx.sync()
+            assert hip.hipGraphLaunch(ex, stream) == 0
+            ctx.sync()
+            got = ctx.download(ycap, (t, rows)).view(np.uint32)
+            assert np.array_equal(got, want), (t, rep)
+            ctx.free(z)
+        assert hip.hipGraphExecDestroy(ex) == 0 and hip.hipGraphDestroy(graph) == 0
+        ctx.free(yref); ctx.free(ycap)
+    for p_ in (xd, xo, yo):
+        ctx.free(p_)
+    m.close(); other.close()
