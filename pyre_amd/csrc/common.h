@@ -152,7 +152,7 @@ int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, 
 //   co:   rows < ch are the channels of a causal depthwise conv1d (kernel kk, weights conv_w[ch][kk]); the lane that
 //         owns a row runs the window's tokens in order, o = w[kk-1]*cur + sum_j w[j]*state[j], co[t][row] = silu(o),
 //         and slides the row's state conv_in -> conv_out ([kk-1][ch], oldest first; in == out is fine).
-struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; int four_waves; };
+struct GemvEpi { uint32_t* best; const float* conv_w; const float* conv_in; float* conv_out; float* co; int ch, kk; int four_waves; int sq_heads = 0; float sq_eps = 0.0f; };          // sq_*: PyreAop::sq travels to the kernel here
 // launchers implemented in qmat.hip, used by the block / model code
 // Matrices in the matrix-core layout (FMT_IQ3_S_M) take their activations as the f16 operand `a` when the caller has one (a
 // producer kernel wrote it); otherwise x_dev is split into the context's operand buffer by one more launch.
@@ -191,7 +191,12 @@ int pyre_pick_launch(pyre_ctx* ctx, const uint32_t* best_dev, int n_tiles, uint3
 // [super-block][8] factors the super-block's sums are multiplied by per token (the inverse of the power of two the splitter
 // scaled that stretch of the token by); null = 1.  Rows 2t .. R - 1 may hold anything finite or not: a row of the operand
 // only ever reaches its own token's sums, so a token's result is bit-identical for every window width.
-struct PyreAop { const uint4* op; const float* ainv; };
+struct PyreAop { const uint4* op; const float* ainv; const float* sq = nullptr; int sq_heads = 0; float sq_eps = 0.0f; };
+// sq (with op; ainv unused): the operand of a Gated DeltaNet output projection as its four workgroups per head leave it
+// (GdnQ): one 128-column chunk = one head, one 32-column sub-block = one workgroup's columns, each scaled by its own power
+// of two; sq[(t*heads + h)*4 + q] = that factor's inverse, sq[8*heads*4 + (t*heads + h)*4 + q] = the quarter's sum of
+// squares of the un-normalised output.  The product brings a chunk's sub-blocks to a common power of two and applies
+// 1 / sqrt(mean square + eps), the head's RMS norm, with the chunk's scale.
 int pyre_aop_rows(int t);
 size_t pyre_aop_bytes(int cols, int t);                            // operand bytes for a K range of `cols` and a window of t
 // splits x [t][cols] (any magnitudes: each 256-column stretch of a token is scaled by its own power of two) into op / ainv
@@ -339,8 +344,13 @@ struct GdnDev { const float* a; const float* dt; const float* conv_w; const floa
 // proj [t][ch + nv*dv + 2*nv] = [qkv | z | beta | alpha] per token (row stride = proj_stride floats).
 // conv_in/conv_out [(k-1)][ch], ssm_in/ssm_out [nv][dk][dv] (in != out).  co_scratch [8][ch].  out [t][nv*dv].
 // conv_done: co_scratch already holds silu(conv) of the window and the conv state has been advanced (GemvEpi).
+// gq: the launch runs on nv x 4 workgroups (a workgroup owns 32 columns of a head's state) and leaves, instead of out_dev,
+// the un-normalised gated output as f16 operand rows with the per-quarter factors and sums of squares of PyreAop::sq.
+// The state it leaves differs in rounding from the nv-workgroup form's (the column sums meet in another order): a layer
+// uses one form for every call.
+struct GdnQ { uint16_t* op; float* sq; };
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f);
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f, const GdnQ* gq = nullptr);
 
 // Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
 // scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].

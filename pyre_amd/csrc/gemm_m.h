@@ -38,6 +38,36 @@ template <bool SC> __device__ __forceinline__ void load_a(const AopRsrc& ar, con
   if constexpr (SC) { const float2 p = ((const float2*)ainv)[(c >> 1) * 4 + (lane >> 4)]; b.ai0 = p.x; b.ai1 = p.y; }
 }
 
+// The operand of PyreAop::sq: chunk c is head c, sub-block s the columns of the head's workgroup s.  A lane rescales its
+// row's four sub-blocks from their own powers of two to the largest factor's inverse (exact: a multiplication of an f16
+// number by a power of two not above one; what falls below the subnormals is 2^-24 of the chunk's largest value) and takes,
+// for the two tokens whose sums it holds, that factor times 1 / sqrt(mean square + eps) as the chunk's scale.
+__device__ __forceinline__ void load_a_sq(const AopRsrc& ar, const float* __restrict__ sq, int heads, float eps, int R, int c, int lane, ABuf& b) {
+  typedef _Float16 h2v_ __attribute__((ext_vector_type(2)));
+  const int trow = (lane & 15) >> 1, q = lane >> 4;
+  const float4 dr = *(const float4*)(sq + ((size_t)trow * heads + c) * 4);
+  const float4 d0 = *(const float4*)(sq + ((size_t)(2 * q) * heads + c) * 4), d1 = *(const float4*)(sq + ((size_t)(2 * q + 1) * heads + c) * 4);
+  const float* ssq = sq + (size_t)8 * heads * 4;
+  const float4 s0 = *(const float4*)(ssq + ((size_t)(2 * q) * heads + c) * 4), s1 = *(const float4*)(ssq + ((size_t)(2 * q + 1) * heads + c) * 4);
+  const float mr = fmaxf(fmaxf(dr.x, dr.y), fmaxf(dr.z, dr.w));
+  // the quotients of two powers of two, by their exponents (no division on this path)
+  const uint32_t mb = __float_as_uint(mr) - 0x3F800000u;
+  const float fr[4] = {__uint_as_float(__float_as_uint(dr.x) - mb), __uint_as_float(__float_as_uint(dr.y) - mb), __uint_as_float(__float_as_uint(dr.z) - mb), __uint_as_float(__float_as_uint(dr.w) - mb)};
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int off = ar.lane_off < 0 ? -1 : ar.lane_off + (c * 4 + s) * 4 * R * 16;
+    const auto v = __builtin_amdgcn_raw_buffer_load_b128(ar.r, off, 0, 0);
+    const h2v_ f = {(_Float16)fr[s], (_Float16)fr[s]};
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2v_, (uint32_t)v[k]) * f);
+    b.a[s] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  const float m0 = fmaxf(fmaxf(d0.x, d0.y), fmaxf(d0.z, d0.w)), m1 = fmaxf(fmaxf(d1.x, d1.y), fmaxf(d1.z, d1.w));
+  b.ai0 = m0 * __builtin_amdgcn_rsqf((((s0.x + s0.y) + s0.z) + s0.w) * (1.0f / 128.0f) + eps);          // (the hardware reciprocal square root: one unit in the last place)
+  b.ai1 = m1 * __builtin_amdgcn_rsqf((((s1.x + s1.y) + s1.z) + s1.w) * (1.0f / 128.0f) + eps);
+}
+
 // The two constants of the nibble -> f16 step.  They are kept in registers the compiler cannot see through, so that
 // (x & K) | E stays one instruction (a second literal would split it).
 struct NibK { uint32_t K, E; };

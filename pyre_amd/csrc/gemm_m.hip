@@ -105,7 +105,8 @@ __device__ __forceinline__ void load_a_x(const float* __restrict__ x, int c, int
   }
   b.ai0 = kg == 0 ? dn : 0.0f; b.ai1 = 0.0f;
 }
-template <int NW, bool SC, bool CONV, bool ONE = false, bool XF = false>
+//   SQ: the operand of a Gated DeltaNet output projection with per-sub-block scales and the head norm (load_a_sq).
+template <int NW, bool SC, bool CONV, bool ONE = false, bool XF = false, bool SQ = false>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __re
   static_assert(!XF || (ONE && !CONV), "f32 activations: the single-token instance without the conv epilogue");
   const AopRsrc ar = aop_rsrc(aop, m.cols, R, lane);
   const float* xf = (const float*)aop;
-  auto get_a = [&](int c, ABuf& b) { if constexpr (XF) load_a_x(xf, c, lane, b); else load_a<SC>(ar, ainv, R, c, lane, b); };
+  auto get_a = [&](int c, ABuf& b) { if constexpr (XF) load_a_x(xf, c, lane, b); else if constexpr (SQ) load_a_sq(ar, ainv, ep.sq_heads, ep.sq_eps, R, c, lane, b); else load_a<SC>(ar, ainv, R, c, lane, b); };
   WBuf<4> w0; ABuf a0;
   if (c0 < c1) { get_a(c0, a0); load_w<4>(m, tile * 4, c0, lane, K128, w0); }
   // conv epilogue: wave 0 fetches its rows' taps and state now, behind the weights, so the loads overlap the products
@@ -208,6 +209,12 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
 }
 template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep, const float* xf = nullptr) {
   if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, true, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep); return; }
+  if (a.sq) {          // (the launcher has checked: no conv epilogue, chunks = heads)
+    GemvEpi e2 = ep; e2.sq_heads = a.sq_heads; e2.sq_eps = a.sq_eps;
+    if (t == 1) hipLaunchKernelGGL((k_gemm_m<NW, true, false, true, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, 1, 2, cpw, e2);
+    else hipLaunchKernelGGL((k_gemm_m<NW, true, false, false, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, t, pyre_aop_rows(t), cpw, e2);
+    return;
+  }
 #define GEMM_M_GO(SC, CONV, ONE) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, ONE>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
   if (t == 1 && a.ainv && (!ep.co || ep.kk == 4)) { if (ep.co) GEMM_M_GO(true, true, true); else GEMM_M_GO(true, false, true); }          // a single token with scaled operand rows: the instance with its constants folded in
   else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true, false); else GEMM_M_GO(false, true, false); }
@@ -231,6 +238,7 @@ int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t,
   if (m.fmt != FMT_IQ3_S_M || !m.mq || !m.mh) return pyre_fail(ctx, PYRE_E_TYPE, "gemm_m: the matrix is not held in the matrix-core layout");
   if (xf && !pyre_gemm_m_x_ok(m, t, ep)) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: f32 activations are for a single token, no conv epilogue and at most 128 row tiles");
   if (t < 1 || t > 8 || ksplit < 1 || (!a.op && !xf) || !y) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: t = %d, %d K slices", t, ksplit);
+  if (a.sq && (ep.co || xf || a.sq_heads * 128 != m.cols)) return pyre_fail(ctx, PYRE_E_ARG, "gemm_m: per-quarter scales need %d heads of 128 columns and no conv epilogue", a.sq_heads);
   if (m.cols % 256 != 0 || m.SB != m.cols / 256) return pyre_fail(ctx, PYRE_E_SHAPE, "gemm_m: %d columns", m.cols);
   int nw, cpw; pyre_gemm_m_plan(m, ksplit, &nw, &cpw);
   if (ep.four_waves) { nw = 4; const int per_wg = ((m.cols >> 7) + ksplit - 1) / ksplit; cpw = (per_wg + 3) / 4; }

@@ -36,6 +36,7 @@ struct pyre_model {
   uint32_t* ids = nullptr; uint32_t* toks = nullptr; int toks_cap = 0; uint32_t* best = nullptr;
   PleCfg plc{}; QMatDev ple_tab{}; PleWork pw{}; int n_ple = 0, ple_ring = 0;      // PLE: hash parameters, the token table, window workspace, ring rows per layer
   uint16_t* aop = nullptr;      // the f16 operand a producer kernel leaves for the matrix-core GEMV that follows it (one at a time: the launches are stream-ordered)
+  float* gdn_sq = nullptr;      // [2][8][nv][4]: per token, head and quarter the inverse power of two of the Gated DeltaNet operand and the quarter's sum of squares (PyreAop::sq)
   float* aop_inv = nullptr;     // [super-blocks][8]: the inverse of the power of two the hyper-connection mix scaled each token of that operand by
   PromptPipe* pipe = nullptr;      // further window workspaces and streams for a long prompt (prompt_pipe), made at the first one
 };
@@ -141,7 +142,7 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   const size_t aop_b = pyre_aop_bytes((kmax + 255) / 256 * 256, 8);
   const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
-                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(4 * 8 * (size_t)((kmax + 255) / 256)) + al256(ple_b) + 4096;
+                 al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(4 * 8 * (size_t)((kmax + 255) / 256)) + al256(4 * 2 * 8 * 4 * (size_t)c.lin_nv) + al256(ple_b) + 4096;
   PYRE_HIP(ctx, hipMalloc(&m->work, total));
   uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
@@ -149,7 +150,7 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
   m->inj_a = (float*)take(4 * 8 * c.hc); m->inj_f = (float*)take(4 * 8 * c.hc); m->proj = (float*)take(4 * 8 * pmax); m->core = (float*)take(4 * 8 * cmax);
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
-  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b); m->aop_inv = (float*)take(4 * 8 * (size_t)((kmax + 255) / 256));
+  m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b); m->aop_inv = (float*)take(4 * 8 * (size_t)((kmax + 255) / 256)); m->gdn_sq = (float*)take(4 * 2 * 8 * 4 * (size_t)c.lin_nv);
   if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
   PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
   if (kmax_out) *kmax_out = kmax;
@@ -515,6 +516,14 @@ int mtp_window_of(const pyre_mtp* m);
 bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) && (int)L.outp.rows == d && L.hcf.di.fmt == FMT_IQ3_S; }
 
 // One window of t <= 8 tokens (ids in m->ids unless from_best).
+static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
+// A Gated DeltaNet layer whose output projection is on the matrix cores runs its recurrence on nv x 4 workgroups and leaves
+// the head norm to that projection (GdnQ / PyreAop::sq) -- in every call that touches the layer's state, the re-run of
+// pyre_spec_keep included: the two forms of the kernel round the state differently.  PYRE_GDN_Q=0: nv workgroups.
+static bool gdn_q_on(const pyre_model* m, const Layer& L) {
+  const char* e = getenv("PYRE_GDN_Q");
+  return !(e && *e && atoi(e) == 0) && fuse_aop_on() && !L.full && L.outp.fmt == FMT_IQ3_S_M && L.gdn.dv == 128 && L.gdn.dk == 128 && L.outp.cols == L.gdn.nv * 128 && m->gdn_sq != nullptr;
+}
 int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
   const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
   if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
@@ -534,7 +543,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
   if (m->n_ple > 0) {      // every position's n-gram rows are fetched once for all PLE layers
     if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
   }
-  const bool fuse_aop = [] { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }();      // 1: separate split launches instead of the producers' own operand stores
+  const bool fuse_aop = fuse_aop_on();      // PYRE_AOP_SPLIT=1: separate split launches instead of the producers' own operand stores
   // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
   // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
   // own split launch (its magnitude has no bound a single workgroup of the merge could form)
@@ -565,12 +574,14 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
       if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.hca, L.proj)))) return rc;
-      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, gdn_fused(L) ? m->aop : nullptr, L.gdn_up))) return rc;
+      const GdnQ gq{m->aop, m->gdn_sq};
+      if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, gdn_fused(L) ? m->aop : nullptr, L.gdn_up, gdn_q_on(m, L) ? &gq : nullptr))) return rc;
       s->cur[li] = nb;
     }
     if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
-    const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}; const PyreAop* oa = (!L.full && gdn_fused(L)) ? &aop_gdn : nullptr;
+    const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
+    const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
     if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc; }
     else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc;
     const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
@@ -719,7 +730,8 @@ int pyre_spec_keep(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, int
   if (s->last_window != t) return pyre_fail(ctx, PYRE_E_STATE, "pyre_spec_keep: the last forward_multi window had %d tokens, not %d", s->last_window, t);
   for (const Layer& L : m->layers) if (!L.full) {
     int li = L.mix_index, after = s->cur[li], before = after ^ 1;
-    int rc = pyre_gdn_launch(ctx, L.gdn, s->proj_saved[li], m->pw_lin, keep, s->conv[before][li], s->conv[after][li], s->ssm[before][li], s->ssm[after][li], m->co, m->core); if (rc) return rc;
+    const GdnQ gq{m->aop, m->gdn_sq};          // (its operand and scales are not used: the call is for the state)
+    int rc = pyre_gdn_launch(ctx, L.gdn, s->proj_saved[li], m->pw_lin, keep, s->conv[before][li], s->conv[after][li], s->ssm[before][li], s->ssm[after][li], m->co, m->core, false, nullptr, 1.0f, gdn_q_on(m, L) ? &gq : nullptr); if (rc) return rc;
   }
   s->len -= t - keep; s->last_window = 0;
   return PYRE_OK;
