@@ -179,7 +179,11 @@ int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int strid
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
   if (gq) {
     ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv));
-    if (t == 1 && g.nk == 16 && g.nv == 32) hipLaunchKernelGGL((k_gdn_delta_q<128, 128, 1, 16, 32>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq);
+#define GDN_Q_FIX(FT) hipLaunchKernelGGL((k_gdn_delta_q<128, 128, FT, 16, 32>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq)
+    if (g.nk == 16 && g.nv == 32) {          // the A3B geometry: the window width and the head counts folded in
+      switch (t) { case 1: GDN_Q_FIX(1); break; case 2: GDN_Q_FIX(2); break; case 3: GDN_Q_FIX(3); break; case 4: GDN_Q_FIX(4); break; case 5: GDN_Q_FIX(5); break; case 6: GDN_Q_FIX(6); break; case 7: GDN_Q_FIX(7); break; default: GDN_Q_FIX(8); break; }
+    }
+#undef GDN_Q_FIX
     else hipLaunchKernelGGL((k_gdn_delta_q<128, 128>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq);
     PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
   }

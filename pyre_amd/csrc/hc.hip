@@ -555,7 +555,7 @@ template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcW
 #define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
 #define NORM_DOWN_M_FIX(NP) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, 2, 2048, 10>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(512), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
   bool done = false;
-  if constexpr (T == 1) {          // a single token at the width of the A3B configuration: the instance with its constants folded in
+  {          // the width of the A3B configuration: the instances with its constants folded in
     if (h.d == 2048 && (!mo.partial || mo.k == 10)) { if (comb_parts > 1) NORM_DOWN_M_FIX(PYRE_GEMV_PARTS); else NORM_DOWN_M_FIX(1); done = true; }
   }
   if (done) {}
@@ -584,7 +584,7 @@ template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork
 #define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), UP_MIX_M_ARGS)
 #define UP_MIX_M_FIX(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF, 4, 256, 16>), UP_MIX_M_ARGS)
   bool done = false;
-  if constexpr (T == 1) {          // a single token with four streams, a low rank of 256 and sixteen slices (the A3B configuration): constants folded in
+  {          // four streams, a low rank of 256 and sixteen slices (the A3B configuration): constants folded in
     if (h.hc == 4 && h.lr == 256 && ksplit == 16) { if (rt && rq.fmt == FMT_BF16) UP_MIX_M_FIX(FMT_BF16); else if (rt && rq.fmt == FMT_F32) UP_MIX_M_FIX(FMT_F32); else UP_MIX_M_FIX(-1); done = true; }
   }
   if (done) {}

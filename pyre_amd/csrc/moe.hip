@@ -174,7 +174,7 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
   PYRE_TS(1);
   const QMatDev& G = shared ? m.sh_gate : m.gate_e; const QMatDev& Up = shared ? m.sh_up : m.up_e;
   const int tile = (shared ? 0 : expert * (ff >> 6)) + blockIdx.x;
-  const int nz = FIX ? 2 : (int)gridDim.z, kz = blockIdx.z, np = P * nz;          // np parts in all
+  const int nz = (FIX && !PRE) ? 2 : (FIX ? 1 : (int)gridDim.z), kz = blockIdx.z, np = P * nz;          // np parts in all (FIX: two workgroups a single token's entry, one a window's)
   const int GU = FIX ? 32 : G.U;          // 64-column units of a row (both matrices, routed or shared: d / 64)
   const int upw = (GU + NW * np - 1) / (NW * np);
   float ag[P][1], au[P][1];
@@ -233,15 +233,18 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
 }
 
 // ---- routing alone (windows of several tokens): grid t, 1024 threads; ids ascending and softmax weights of token ti ------
+template <bool FIX = false>
 __global__ __launch_bounds__(1024) void k_moe_route(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, int nsl, int sstride, int tstride) {
   __shared__ RouteLds rl;
   const int ti = blockIdx.x;
+  const int n_exp = FIX ? 512 : m.n_exp, top_k = FIX ? 10 : m.top_k;          // FIX: the A3B configuration (and 32 router slices), checked by the launcher
+  if constexpr (FIX) nsl = 32;
 #ifdef PYRE_PHASE_TS
   unsigned long long ts_[8];
 #endif
-  route_topk(logits + (size_t)ti * tstride, nsl, sstride, m.n_exp, m.top_k, rl ROUTE_TS_ARG);
-  route_weights(m.top_k, rl);
-  if ((int)threadIdx.x < m.top_k) { sel_idx[ti * m.top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * m.top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
+  route_topk(logits + (size_t)ti * tstride, nsl, sstride, n_exp, top_k, rl ROUTE_TS_ARG);
+  route_weights(top_k, rl);
+  if ((int)threadIdx.x < top_k) { sel_idx[ti * top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; sel_w[ti * top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
 }
 
 // ---- expert down: partial[entry][r] = down[r] . h[entry] ---------------------------------------------------------------
@@ -316,7 +319,7 @@ __global__ void k_moe_sum(const float* __restrict__ partial, const float* __rest
 // bit for bit what moe_out_value forms from k_moe_down's unreduced terms.  A wave's weights of all entries and its slices
 // of their activations (through its own shared memory: no workgroup barrier) are fetched before the first is used.
 // GE: entries a group can hold in this instance (3 covers top_k <= 11, PYRE_MOE_GMAX the rest) -- the register budget follows it.
-template <int FMT, int NW, int GE>
+template <int FMT, int NW, int GE, bool FIX = false>
 __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1) void k_moe_down_groups(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ sel_w, const float* __restrict__ sg,
                                                             const float* __restrict__ h, int hstride, float* __restrict__ parts, const uint2* __restrict__ g2) {
   static_assert(GE <= PYRE_MOE_GMAX, "a group holds at most PYRE_MOE_GMAX entries");
@@ -324,19 +327,19 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, parts);
   __shared__ float red[GE][NW][64];
   __shared__ float hx[NW][GE][64];
-  const int ti = blockIdx.y, q = blockIdx.z, k = m.top_k, gsz = (k + 4) / 4;
+  const int ti = blockIdx.y, q = blockIdx.z, k = FIX ? 10 : m.top_k, gsz = (k + 4) / 4, d = FIX ? 2048 : m.d;          // FIX: the A3B configuration (top 10, d = 2048, experts 512 wide), checked by the launcher
   const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;          // the group's routed entries j0 .. j0+nr-1
   const bool with_shared = q == PYRE_MOE_GROUPS - 1;
   const int ne = nr + (with_shared ? 1 : 0);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // the routed and the shared matrices may differ in width: each has its own K shares (as in k_moe_down)
-  const int Ur = m.down_e.U, Us = m.sh_down.U, upr = (Ur + NW - 1) / NW, ups = (Us + NW - 1) / NW;
+  const int Ur = FIX ? 8 : m.down_e.U, Us = FIX ? 8 : m.sh_down.U, upr = (Ur + NW - 1) / NW, ups = (Us + NW - 1) / NW;
   const int niter = max(nr > 0 ? upr : 0, with_shared ? ups : 0);
   int tile[GE]; const float* xs[GE];
 #pragma unroll
   for (int e = 0; e < GE; ++e) {
     const bool shared = with_shared && e == nr; const int j = shared ? k : min(j0 + e, k - 1);
-    tile[e] = (shared ? 0 : __builtin_amdgcn_readfirstlane(sel_idx[ti * k + j]) * (m.d >> 6)) + blockIdx.x;
+    tile[e] = (shared ? 0 : __builtin_amdgcn_readfirstlane(sel_idx[ti * k + j]) * (d >> 6)) + blockIdx.x;
     xs[e] = h + (size_t)(ti * (k + 1) + j) * hstride;
   }
   float acc[GE][1];
@@ -374,7 +377,7 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
       for (int w = 1; w < NW; ++w) pv += red[e][w][lane];
       if (e < nr) o = fmaf(wv[e], pv, o); else o = fmaf(pv, g, o);          // the shared expert comes last
     }
-    parts[((size_t)q * gridDim.y + ti) * m.d + blockIdx.x * 64 + lane] = o;
+    parts[((size_t)q * gridDim.y + ti) * d + blockIdx.x * 64 + lane] = o;
   }
 }
 
@@ -421,8 +424,11 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   if (t == 1 && a3b && nsl == 32 && nz == 2) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true>), dim3(hs / 64, entries, 2), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride);
   else if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
   else {
-    hipLaunchKernelGGL(k_moe_route, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
-    if (P == 2) { GU_GO(2, 1, true); } else { GU_GO(1, 1, true); }
+    const bool a3bw = m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512 && nsl == 32;          // a window of the A3B configuration: constants folded in
+    if (a3bw) hipLaunchKernelGGL(k_moe_route<true>, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
+    else hipLaunchKernelGGL(k_moe_route<false>, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
+    if (a3bw && P == 2) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 2, true, true>), dim3(hs / 64, entries, 1), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride);
+    else if (P == 2) { GU_GO(2, 1, true); } else { GU_GO(1, 1, true); }
   } }
 #undef GU_GO
   PYRE_CHECK_LAUNCH(ctx);
@@ -430,7 +436,9 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   if (in_groups) {
     const int gsz = (m.top_k + 4) / 4, last = m.top_k - min(m.top_k, (PYRE_MOE_GROUPS - 1) * gsz) + 1;          // entries of a full group, of the last (with the shared expert)
 #define DOWN_G_GO(GE) MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down_groups<F, 8, GE>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2))
-    if (gsz <= 3 && last <= 3) { DOWN_G_GO(3); } else { DOWN_G_GO(PYRE_MOE_GMAX); }
+    if (m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512)          // the A3B configuration: constants folded in
+      hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, 3, true>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2);
+    else if (gsz <= 3 && last <= 3) { DOWN_G_GO(3); } else { DOWN_G_GO(PYRE_MOE_GMAX); }
 #undef DOWN_G_GO
   }
   else if (a3b && nz == 2) hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, true>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2);
