@@ -70,7 +70,8 @@ int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, ui
 //   ksplit  > 1: y is a partial buffer, y[(ks*T + t)*tiles*64 + row] = slice sum (the consumer adds the slices in order).
 //   ep.best (T == 1, ksplit == 1): best[2*tile] = bits of the tile's maximum, best[2*tile+1] = its first row.
 //   ep.co: conv1d + SiLU of the leading ep.ch rows (linear_core, qwen4exp_gguf.rs:1643-1647), as in the lane = row GEMV.
-//   ONE: the single-token instance -- T = 1, two operand rows and (CONV) four taps are compile-time constants.
+//   FT > 0: the window width as a compile-time constant -- T = FT, its operand rows and (CONV) four taps folded in; FT = 1 is
+//   the single-token instance ("ONE" below).
 //   XF (with ONE): `aop` is the token's f32 activations; every wave forms the operand rows of its chunks itself, with the
 //   arithmetic of k_act_split (the 256-column stretch's power of two from a wave maximum over the stretch), so the sums
 //   are bit for bit those of the split launch followed by this one -- a launch less where the producer of x cannot
@@ -106,13 +107,14 @@ __device__ __forceinline__ void load_a_x(const float* __restrict__ x, int c, int
   b.ai0 = kg == 0 ? dn : 0.0f; b.ai1 = 0.0f;
 }
 //   SQ: the operand of a Gated DeltaNet output projection with per-sub-block scales and the head norm (load_a_sq).
-template <int NW, bool SC, bool CONV, bool ONE = false, bool XF = false, bool SQ = false>
+template <int NW, bool SC, bool CONV, int FT = 0, bool XF = false, bool SQ = false>
 __global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m); args_now(aop, ainv, y, T, R, cpw, ep.best, ep.conv_w, ep.conv_in, ep.conv_out, ep.co, ep.ch, ep.kk);
-  if constexpr (ONE) { T = 1; R = 2; }
-  const int kk = ONE ? 4 : ep.kk;
+  constexpr bool ONE = FT == 1;
+  if constexpr (FT > 0) { T = FT; R = FT <= 1 ? 2 : (FT == 2 ? 4 : (FT <= 4 ? 8 : 16)); }
+  const int kk = FT > 0 ? 4 : ep.kk;
   const int tile = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int K128 = m.cols >> 7;
@@ -208,17 +210,22 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
   return nw;
 }
 template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep, const float* xf = nullptr) {
-  if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, true, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep); return; }
+  if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, 1, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep); return; }
+#define GEMM_M_T(CALL) switch (t) { case 1: { constexpr int FT = 1; CALL; } break; case 2: { constexpr int FT = 2; CALL; } break; case 3: { constexpr int FT = 3; CALL; } break; case 4: { constexpr int FT = 4; CALL; } break; \
+    case 5: { constexpr int FT = 5; CALL; } break; case 6: { constexpr int FT = 6; CALL; } break; case 7: { constexpr int FT = 7; CALL; } break; default: { constexpr int FT = 8; CALL; } break; }
   if (a.sq) {          // (the launcher has checked: no conv epilogue, chunks = heads)
     GemvEpi e2 = ep; e2.sq_heads = a.sq_heads; e2.sq_eps = a.sq_eps;
-    if (t == 1) hipLaunchKernelGGL((k_gemm_m<NW, true, false, true, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, 1, 2, cpw, e2);
-    else hipLaunchKernelGGL((k_gemm_m<NW, true, false, false, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, t, pyre_aop_rows(t), cpw, e2);
+    GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, t, pyre_aop_rows(t), cpw, e2));
     return;
   }
-#define GEMM_M_GO(SC, CONV, ONE) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, ONE>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
-  if (t == 1 && a.ainv && (!ep.co || ep.kk == 4)) { if (ep.co) GEMM_M_GO(true, true, true); else GEMM_M_GO(true, false, true); }          // a single token with scaled operand rows: the instance with its constants folded in
-  else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true, false); else GEMM_M_GO(false, true, false); }
-  else { if (a.ainv) GEMM_M_GO(true, false, false); else GEMM_M_GO(false, false, false); }
+#define GEMM_M_GO(SC, CONV) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, 0>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
+  if (a.ainv && (!ep.co || ep.kk == 4)) {          // scaled operand rows (every launch of the model and of the operator): the instance with the window width folded in
+    if (ep.co) { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, true, FT>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)); }
+    else { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)); }
+  }
+  else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true); else GEMM_M_GO(false, true); }
+  else { if (a.ainv) GEMM_M_GO(true, false); else GEMM_M_GO(false, false); }
+#undef GEMM_M_T
 #undef GEMM_M_GO
 }
 }  // namespace
