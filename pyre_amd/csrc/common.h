@@ -43,6 +43,7 @@ struct pyre_ctx {
   std::string prof_text;
   void* aop_buf = nullptr; size_t aop_bytes = 0;       // split activations of the operator's matrix-core GEMM (grow-only)
   void* aop_static = nullptr;                          // device address of this GPU's copy of the file-scope operand array (gemm_m.hip), resolved at creation
+  uint32_t* d_iq2xs_sgn = nullptr;                     // IQ2_XS likewise: two tables of 8192 x four signed bytes (weights 0..3 / 4..7 of an entry)
   uint32_t* d_iq3s_sgn = nullptr;                      // IQ3_S codebook with the signs folded in: 8192 x four signed bytes (gemv_n.hip), made at first use
   void* dgn_buf = nullptr; size_t dgn_bytes = 0;       // activation digits of the native-format IQ3_S GEMV (grow-only)
 };
@@ -141,11 +142,11 @@ struct pyre_qmat {
 };
 int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, int layout, pyre_qmat** out);
 // IQ3_S at the file's bits per weight with the codebook in shared memory, one token (gemv_n.hip)
-size_t pyre_gemv_n_bytes(size_t rows, size_t cols);
-int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev);
+size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt = 6);          // fmt: FMT_IQ3_S (6) or FMT_IQ2_XS (5)
+int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev, int fmt = 6);
 int pyre_gemv_n_table(pyre_ctx* ctx);                             // the codebook table, made at context creation
 size_t pyre_gemv_n_digit_bytes(size_t cols);
-int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, const float* x_dev, float* y_dev, void* digits = nullptr);
+int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, const float* x_dev, float* y_dev, void* digits = nullptr, int fmt = 6);
 
 // Optional work folded into the end of a GEMV launch (qmat.hip):
 //   best: t = 1, per row tile (bits of the maximum, first row holding it) -> best[2*tile], best[2*tile+1]

@@ -91,6 +91,7 @@ void pyre_ctx_destroy(pyre_ctx* ctx) {
   if (ctx->aop_buf) (void)hipFree(ctx->aop_buf);
   if (ctx->d_iq2xs) (void)hipFree(ctx->d_iq2xs);
   if (ctx->d_iq3s_sgn) (void)hipFree(ctx->d_iq3s_sgn);
+  if (ctx->d_iq2xs_sgn) (void)hipFree(ctx->d_iq2xs_sgn);
   if (ctx->dgn_buf) (void)hipFree(ctx->dgn_buf);
   for (auto& p : ctx->prof_pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
   for (auto e : ctx->prof_pool) (void)hipEventDestroy(e);

@@ -18,6 +18,13 @@
 //           scaled by d * (1 + 2 s) * su in f32.
 // The only rounding beyond the f32 path's is the representation of x: |x - su q| <= 2^-22 of the 64 columns' largest
 // magnitude.  t >= 2 stays on the matrix cores, where a window costs what a token does.
+//
+// IQ2_XS (F = 1 below; gguf_q.rs:126-129) goes the same way.  The file keeps per eight weights a 16-bit word (9-bit codebook
+// index, 7-bit index into the sign table, whose eighth sign is the parity of the seven); here the parity is resolved at load
+// and a field is 17 bits: index | signs of weights 0..3 << 9 | signs of weights 4..7 << 13.  32 fields + 8 scale bytes + d =
+// 78 bytes, kept as five 16-byte pieces: 80 bytes per 256 weights (2.5 bit/weight against the file's 2.3125).  The signed
+// codebook is two tables of 8192 entries (weights 0..3 and 4..7 of an entry: index | four signs << 9), 64 KB of shared
+// memory; a 16-weight half of a sub-block has its own 4-bit scale, (2 n + 1) / 8, so the digit sums are joined per half.
 #include "formats.h"
 #include "iq_codebooks.h"
 
@@ -46,6 +53,28 @@ __global__ __launch_bounds__(256) void k_repack_n(int rows, int rows_pad, int SB
   }
   const size_t tile = (size_t)(row >> 6); const int lane = row & 63;
   for (int p = 0; p < 7; ++p) nq[((tile * SB + sb) * 7 + p) * 64 + lane] = make_uint4(w[4 * p], w[4 * p + 1], w[4 * p + 2], w[4 * p + 3]);
+}
+
+// IQ2_XS: raw GGUF rows -> five pieces per (row, super-block); one thread per (padded row, super-block)
+__global__ __launch_bounds__(256) void k_repack_n2(int rows, int rows_pad, int SB, const uint8_t* __restrict__ raw, size_t row_bytes, uint4* __restrict__ nq) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; if (idx >= (size_t)rows_pad * SB) return;
+  const int row = (int)(idx / SB), sb = (int)(idx % SB); const bool live = row < rows;
+  uint32_t w[20];
+  for (int i = 0; i < 20; ++i) w[i] = 0;
+  if (live) {
+    const uint8_t* b = raw + (size_t)row * row_bytes + (size_t)sb * 74;
+    auto put = [&](int bit, uint32_t val, int nbits) { w[bit >> 5] |= val << (bit & 31); if ((bit & 31) + nbits > 32) w[(bit >> 5) + 1] |= val >> (32 - (bit & 31)); };
+    for (int e = 0; e < 32; ++e) {
+      const uint32_t q = (uint32_t)b[2 + 2 * e] | ((uint32_t)b[3 + 2 * e] << 8);
+      const uint32_t s7 = q >> 9, s8 = s7 | ((uint32_t)(__popc(s7) & 1) << 7);          // ksigns(i) = i | parity(i) << 7
+      put(17 * e, (q & 511u) | (s8 << 9), 17);
+    }
+    w[17] = (uint32_t)b[66] | ((uint32_t)b[67] << 8) | ((uint32_t)b[68] << 16) | ((uint32_t)b[69] << 24);
+    w[18] = (uint32_t)b[70] | ((uint32_t)b[71] << 8) | ((uint32_t)b[72] << 16) | ((uint32_t)b[73] << 24);
+    w[19] = (uint32_t)b[0] | ((uint32_t)b[1] << 8);
+  }
+  const size_t tile = (size_t)(row >> 6); const int lane = row & 63;
+  for (int p = 0; p < 5; ++p) nq[((tile * SB + sb) * 5 + p) * 64 + lane] = make_uint4(w[4 * p], w[4 * p + 1], w[4 * p + 2], w[4 * p + 3]);
 }
 
 // ---- activation digits: grid = 64-column units, one wave per unit -------------------------------------------------------------
@@ -118,22 +147,61 @@ __device__ __forceinline__ float n_superblock(const uint4 (&r)[7], const uint8_t
   return acc;
 }
 
+// ---- IQ2_XS: entry E (eight weights) of the 20 words: the two table offsets (weights 0..3: first table; 4..7: second, 32 KB on)
+template <int E> __device__ __forceinline__ void n2_offs(const uint32_t (&w)[20], uint32_t& o0, uint32_t& o1) {
+  constexpr int bit = 17 * E - 2;                   // the window starts two bits below the field: index at bits 2..10, signs at 11..14 and 15..18
+  uint32_t f;
+  if constexpr (bit < 0) f = w[0] << 2;
+  else { constexpr int wi = bit >> 5, sh = bit & 31; if constexpr (sh + 19 <= 32) f = w[wi] >> sh; else f = __builtin_amdgcn_alignbit(w[wi + 1], w[wi], sh); }
+  o0 = f & 0x7FFCu;
+  o1 = ((f & 0x07FCu) | ((f >> 4) & 0x7800u)) + 32768u;
+}
+template <int IB, int L> __device__ __forceinline__ void n2_group(const uint32_t (&w)[20], const uint8_t* lt, const uint32_t* __restrict__ p, int (&ia)[3], int (&ib)[3]) {
+  if constexpr (L < 4) {
+    uint32_t o0, o1; n2_offs<IB * 4 + L>(w, o0, o1);
+    const int e0 = (int)*(const uint32_t*)(lt + o0), e1 = (int)*(const uint32_t*)(lt + o1);
+    int (&acc)[3] = L < 2 ? ia : ib;                 // entries 0, 1: the sub-block's first sixteen weights; 2, 3: its second
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { acc[k] = __builtin_amdgcn_sdot4(e0, (int)p[(2 * L) * 3 + k], acc[k], false); acc[k] = __builtin_amdgcn_sdot4(e1, (int)p[(2 * L + 1) * 3 + k], acc[k], false); }
+    n2_group<IB, L + 1>(w, lt, p, ia, ib);
+  }
+}
+template <int IB> __device__ __forceinline__ float n2_subblock(const uint32_t (&w)[20], const uint8_t* lt, const uint32_t* __restrict__ dgs, float dsu, float acc) {
+  int ia[3] = {0, 0, 0}, ib[3] = {0, 0, 0};
+  n2_group<IB, 0>(w, lt, dgs + (IB & 1) * 24, ia, ib);
+  const int ta = (int)(((uint32_t)ia[0] << 16) + ((uint32_t)ia[1] << 8) + (uint32_t)ia[2]), tb = (int)(((uint32_t)ib[0] << 16) + ((uint32_t)ib[1] << 8) + (uint32_t)ib[2]);      // |t| < 2^31: |i1| <= 16 * 43 * 33
+  const uint32_t sc = (w[17 + (IB >> 2)] >> (8 * (IB & 3))) & 0xFFu;
+  const float sa = (float)(1 + 2 * (int)(sc & 0xFu)) * 0.125f, sbf = (float)(1 + 2 * (int)(sc >> 4)) * 0.125f;          // (0.5 + n) * 0.25
+  return fmaf(dsu * sbf, (float)tb, fmaf(dsu * sa, (float)ta, acc));
+}
+__device__ __forceinline__ float n_superblock(const uint4 (&r)[5], const uint8_t* lt, const uint32_t* __restrict__ dg, float acc) {
+  const uint32_t w[20] = {r[0].x, r[0].y, r[0].z, r[0].w, r[1].x, r[1].y, r[1].z, r[1].w, r[2].x, r[2].y, r[2].z, r[2].w, r[3].x, r[3].y, r[3].z, r[3].w, r[4].x, r[4].y, r[4].z, r[4].w};
+  const float d = h2f_bits(w[19] & 0xFFFFu);
+  { const float dsu = d * __uint_as_float(dg[0 * DGN_STRIDE + 48]); acc = n2_subblock<0>(w, lt, dg + 0 * DGN_STRIDE, dsu, acc); acc = n2_subblock<1>(w, lt, dg + 0 * DGN_STRIDE, dsu, acc); }
+  { const float dsu = d * __uint_as_float(dg[1 * DGN_STRIDE + 48]); acc = n2_subblock<2>(w, lt, dg + 1 * DGN_STRIDE, dsu, acc); acc = n2_subblock<3>(w, lt, dg + 1 * DGN_STRIDE, dsu, acc); }
+  { const float dsu = d * __uint_as_float(dg[2 * DGN_STRIDE + 48]); acc = n2_subblock<4>(w, lt, dg + 2 * DGN_STRIDE, dsu, acc); acc = n2_subblock<5>(w, lt, dg + 2 * DGN_STRIDE, dsu, acc); }
+  { const float dsu = d * __uint_as_float(dg[3 * DGN_STRIDE + 48]); acc = n2_subblock<6>(w, lt, dg + 3 * DGN_STRIDE, dsu, acc); acc = n2_subblock<7>(w, lt, dg + 3 * DGN_STRIDE, dsu, acc); }
+  return acc;
+}
+
 // grid = min(tiles, what the chip holds at once), NW waves; the workgroup fills its table, then takes row tiles
 // blockIdx.x, + gridDim.x, ..; wave w walks super-blocks [w * spw, + spw) of the tile, lane l owns row tile * 64 + l; the
 // waves' sums meet in shared memory in wave order.  The next super-block's seven pieces are requested before the current
 // one's arithmetic starts.
-template <int NW> __global__ __launch_bounds__(NW * 64) void k_gemv_n(const uint4* __restrict__ nq, int rows, int tiles, int SB, const uint4* __restrict__ tab, const uint32_t* __restrict__ dg, float* __restrict__ y, int spw) {
-  __shared__ __align__(16) uint8_t lt[8192 * 4];
+// P: 16-byte pieces a super-block has (7: IQ3_S, one 32 KB table; 5: IQ2_XS, two)
+template <int NW, int P = 7> __global__ __launch_bounds__(NW * 64) void k_gemv_n(const uint4* __restrict__ nq, int rows, int tiles, int SB, const uint4* __restrict__ tab, const uint32_t* __restrict__ dg, float* __restrict__ y, int spw) {
+  constexpr int TW = P == 7 ? 2048 : 4096;          // 16-byte words of the table(s)
+  __shared__ __align__(16) uint8_t lt[TW * 16];
   __shared__ float red[NW][64];
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  for (int i = tid; i < 2048; i += NW * 64) ((uint4*)lt)[i] = tab[i];
+  for (int i = tid; i < TW; i += NW * 64) ((uint4*)lt)[i] = tab[i];
   __syncthreads();
   const int s0 = min(SB, wave * spw), s1 = min(SB, s0 + spw);
-  uint4 bufa[7], bufb[7];
-  const size_t tstride = (size_t)SB * 7 * 64;
+  uint4 bufa[P], bufb[P];
+  const size_t tstride = (size_t)SB * P * 64;
   if (s0 < s1 && (int)blockIdx.x < tiles) {
 #pragma unroll
-    for (int p = 0; p < 7; ++p) bufa[p] = nq[(size_t)blockIdx.x * tstride + ((size_t)s0 * 7 + p) * 64 + lane];
+    for (int p = 0; p < P; ++p) bufa[p] = nq[(size_t)blockIdx.x * tstride + ((size_t)s0 * P + p) * 64 + lane];
   }
   for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     float acc = 0.0f;
@@ -143,17 +211,17 @@ template <int NW> __global__ __launch_bounds__(NW * 64) void k_gemv_n(const uint
       const uint4* nbase = nq + (size_t)tn * tstride + lane;
       for (int sb = s0; sb < s1; sb += 2) {          // two buffers taking turns (a copy from one to the other would cost 28 moves a super-block)
         const bool last1 = sb + 1 >= s1, last2 = sb + 2 >= s1;
-        const uint4* b1 = last1 ? nbase + (size_t)s0 * 7 * 64 : base + (size_t)(sb + 1) * 7 * 64;
+        const uint4* b1 = last1 ? nbase + (size_t)s0 * P * 64 : base + (size_t)(sb + 1) * P * 64;
 #pragma unroll
-        for (int p = 0; p < 7; ++p) bufb[p] = b1[(size_t)p * 64];
+        for (int p = 0; p < P; ++p) bufb[p] = b1[(size_t)p * 64];
         acc = n_superblock(bufa, lt, dg + (size_t)sb * 4 * DGN_STRIDE, acc);
         if (last1) {
 #pragma unroll
-          for (int p = 0; p < 7; ++p) bufa[p] = bufb[p];          // (an odd count of super-blocks a wave: the prefetched one is the next tile's first)
+          for (int p = 0; p < P; ++p) bufa[p] = bufb[p];          // (an odd count of super-blocks a wave: the prefetched one is the next tile's first)
         } else {
-          const uint4* b2 = last2 ? nbase + (size_t)s0 * 7 * 64 : base + (size_t)(sb + 2) * 7 * 64;
+          const uint4* b2 = last2 ? nbase + (size_t)s0 * P * 64 : base + (size_t)(sb + 2) * P * 64;
 #pragma unroll
-          for (int p = 0; p < 7; ++p) bufa[p] = b2[(size_t)p * 64];
+          for (int p = 0; p < P; ++p) bufa[p] = b2[(size_t)p * 64];
           acc = n_superblock(bufb, lt, dg + (size_t)(sb + 1) * 4 * DGN_STRIDE, acc);
         }
       }
@@ -175,10 +243,11 @@ namespace {
 int env_i(const char* n, int dflt) { const char* s = getenv(n); return s && *s ? atoi(s) : dflt; }
 }
 
-size_t pyre_gemv_n_bytes(size_t rows, size_t cols) { return ((rows + 63) / 64) * 64 * (cols / 256) * 112; }
+size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt) { return ((rows + 63) / 64) * 64 * (cols / 256) * (fmt == FMT_IQ2_XS ? 80 : 112); }
 
-int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev) {
+int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev, int fmt) {
   const int SB = (int)(cols / 256); const size_t rows_pad = (rows + 63) / 64 * 64, total = rows_pad * SB;
+  if (fmt == FMT_IQ2_XS) { hipLaunchKernelGGL(k_repack_n2, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, raw_dev, row_bytes, (uint4*)nq_dev); PYRE_CHECK_LAUNCH(ctx); return PYRE_OK; }
   hipLaunchKernelGGL(k_repack_n, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, raw_dev, row_bytes, (uint4*)nq_dev);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
@@ -186,6 +255,18 @@ int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* r
 // the table: entry (index | signs << 9) = the four codebook values of `index`, value j negated where sign bit j is set
 int pyre_gemv_n_table(pyre_ctx* ctx) {
   if (ctx->d_iq3s_sgn) return PYRE_OK;
+  {      // IQ2_XS: table h (h = 0: weights 0..3 of an entry, 1: weights 4..7), entry (index | four signs << 9)
+    std::vector<uint32_t> t2(16384);
+    static const int tri[3] = {8, 25, 43};
+    for (int h = 0; h < 2; ++h) for (int i = 0; i < 8192; ++i) {
+      uint32_t v = 0;
+      for (int j = 0; j < 4; ++j) { const int g = tri[(kIq2xsCode[i & 511] >> (2 * (4 * h + j))) & 3]; const int sgn = ((i >> (9 + j)) & 1) ? -g : g; v |= (uint32_t)(uint8_t)(int8_t)sgn << (8 * j); }
+      t2[(size_t)h * 8192 + i] = v;
+    }
+    PYRE_HIP(ctx, hipMalloc((void**)&ctx->d_iq2xs_sgn, 16384 * 4));
+    PYRE_HIP(ctx, hipMemcpyAsync(ctx->d_iq2xs_sgn, t2.data(), 16384 * 4, hipMemcpyHostToDevice, ctx->stream));
+    PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  }
   std::vector<uint32_t> t(8192);
   for (int i = 0; i < 8192; ++i) {
     uint32_t v = 0;
@@ -201,9 +282,9 @@ int pyre_gemv_n_table(pyre_ctx* ctx) {
 size_t pyre_gemv_n_digit_bytes(size_t cols) { return cols / 64 * DGN_STRIDE * 4; }
 
 // digits: where the activation digits go (pyre_gemv_n_digit_bytes(cols) bytes); null = the context's grow-only buffer
-int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, const float* x_dev, float* y_dev, void* digits) {
+int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, const float* x_dev, float* y_dev, void* digits, int fmt) {
   if (cols % 256) return pyre_fail(ctx, PYRE_E_SHAPE, "gemv_n: %zu columns are not whole super-blocks", cols);
-  if (!ctx->d_iq3s_sgn) return pyre_fail(ctx, PYRE_E_HIP, "gemv_n: the codebook table was not made at context creation");
+  if (!ctx->d_iq3s_sgn || !ctx->d_iq2xs_sgn) return pyre_fail(ctx, PYRE_E_HIP, "gemv_n: the codebook tables were not made at context creation");
   const int U = (int)(cols / 64), SB = (int)(cols / 256), tiles = (int)((rows + 63) / 64);
   const size_t need = pyre_gemv_n_digit_bytes(cols);
   if (!digits && ctx->dgn_bytes < need) {
@@ -223,6 +304,18 @@ int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, 
   int grid = fwg > 0 ? fwg : 256 * per_cu;
   static const int fgrid = env_i("PYRE_GEMV_N_GRID", 0); if (fgrid > 0) grid = fgrid;
   if (grid > tiles) grid = tiles;
+  if (fmt == FMT_IQ2_XS) {          // two 32 KB tables a workgroup: eight waves, two workgroups a compute unit
+    ProfScope ps(ctx, "gemv_n_iq2_xs_t1", (double)rows * (cols / 256) * 74 + 4.0 * ((double)cols + rows));
+    const uint4* q = (const uint4*)nq; const uint4* tb = (const uint4*)ctx->d_iq2xs_sgn;
+    if (grid > 512 && fgrid <= 0) grid = 512 < tiles ? 512 : tiles;
+    switch (nw) {
+      case 1: hipLaunchKernelGGL((k_gemv_n<1, 5>), dim3(grid), dim3(64), 0, ctx->stream, q, (int)rows, tiles, SB, tb, dg, y_dev, spw); break;
+      case 2: hipLaunchKernelGGL((k_gemv_n<2, 5>), dim3(grid), dim3(128), 0, ctx->stream, q, (int)rows, tiles, SB, tb, dg, y_dev, spw); break;
+      case 8: hipLaunchKernelGGL((k_gemv_n<8, 5>), dim3(grid), dim3(512), 0, ctx->stream, q, (int)rows, tiles, SB, tb, dg, y_dev, spw); break;
+      default: hipLaunchKernelGGL((k_gemv_n<4, 5>), dim3(grid), dim3(256), 0, ctx->stream, q, (int)rows, tiles, SB, tb, dg, y_dev, spw); break;
+    }
+    PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+  }
   { ProfScope ps(ctx, "gemv_n_iq3_s_t1", (double)rows * (cols / 256) * 110 + 4.0 * ((double)cols + rows));
     const uint4* q = (const uint4*)nq; const uint4* tb = (const uint4*)ctx->d_iq3s_sgn;
     switch (nw) {

@@ -298,6 +298,42 @@ def test_iq3s_native_format_single_token(ctx, rows, cols, monkeypatch):
     assert not m.matmul(np.zeros((1, cols), np.float32)).any()
 
 
+# ---- one token of an IQ2_XS matrix: 80 bytes per 256 weights, two signed codebook tables in shared memory, integer dots ----------
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(64, 256), (100, 256), (65, 512), (320, 2048), (4096, 2048), (1000, 768), (130, 8192), (8256, 1024)])
+def test_iq2xs_native_format_single_token(ctx, rows, cols, monkeypatch):
+    monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the native-format kernel
+    raw = synth.matrix(lib.IQ2_XS, rows, cols, 500 + rows % 97)
+    m = lib.QMat(ctx, lib.IQ2_XS, rows, cols, raw)
+    assert m.layout_bytes(2) == (rows + 63) // 64 * 64 * (cols // 256) * 80
+    W = orc.dequant(lib.IQ2_XS, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    g = np.random.Generator(np.random.PCG64(rows + cols + 1))
+    for case in range(6):
+        x = synth.normal((1, cols), 600 + case)
+        if case == 1: x *= np.exp2(g.integers(-40, 40, cols // 64).repeat(64)).astype(np.float32)
+        if case == 2: x[0, 5] = 3.0e4; x[0, cols - 3] = -2.0e7
+        if case == 3: x *= 1e-30
+        if case == 4: x *= 1e30
+        if case == 5: x[0, ::2] = 0.0; x[0, :64] = 0.0
+        with np.errstate(all="ignore"):
+            truth = x.astype(np.float64) @ W.T
+        y = m.matmul(x)
+        assert relerr(y, truth) <= TOL, case
+        assert np.array_equal(bits(y), bits(m.matmul(x)))          # run to run
+        assert relerr(y, m.matmul_f32(x)) <= 2e-6                  # the f32 GEMV agrees to rounding
+        assert relerr(y, m.matmul(np.concatenate([x, x]))[:1]) <= 2e-6
+    xi = g.integers(-1000, 1000, (1, cols)).astype(np.float32)          # integers: exact digits, exact sums, only the f32 scaling rounds
+    assert relerr(m.matmul(xi), xi.astype(np.float64) @ W.T) <= 4e-7          # (sixteen f32 additions a super-block: two scales a sub-block)
+    a = synth.normal((1, cols), 155)
+    assert np.array_equal(bits(m.matmul(a * 1024.0)), bits(m.matmul(a) * 1024.0))
+    bad = synth.normal((1, cols), 156); bad[0, 3] = np.inf
+    assert np.isnan(m.matmul(bad)).all()
+    assert not m.matmul(np.zeros((1, cols), np.float32)).any()
+    monkeypatch.setenv("PYRE_QMATMUL_SMALL", "1")
+    if (rows + 63) // 64 <= 128:                                        # a small matrix: the one-launch f32 GEMV
+        assert np.array_equal(bits(m.matmul(a)), bits(m.matmul_f32(a)))
+
+
 @pytest.mark.gpu
 def test_small_iq3s_single_token_takes_one_launch(ctx):
     """A single token of an IQ3_S matrix of at most 128 row tiles goes through the lane = row f32 GEMV (one launch): the
