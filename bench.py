@@ -140,6 +140,8 @@ def bench_gemv(args):
     # through integer dot products, a window the matrix-core layout; PYRE_QMATMUL_F32=1 / other block types the lane = row GEMV
     if ty == lib.IQ2_XS and t == 1 and os.environ.get("PYRE_QMATMUL_NATIVE", "1") != "0" and os.environ.get("PYRE_QMATMUL_F32") != "1":
         layout, path = 2, "native-format GEMV (k_gemv_n over 80 bytes per 256 weights: 17-bit codebook-index + sign fields, two signed codebook tables in shared memory, v_dot4_i32_i8), preceded by the activation digits launch k_act_digits_n"
+    elif ty == lib.Q4_K and t == 1 and os.environ.get("PYRE_QMATMUL_NATIVE", "1") != "0" and os.environ.get("PYRE_QMATMUL_F32") != "1":
+        layout, path = 2, "native-format GEMV (k_gemv_n over the file's 144-byte blocks: nibbles into v_dot4_i32_i8, minima through the digit sums), preceded by the activation digits launch k_act_digits_n"
     elif ty != lib.IQ3_S or os.environ.get("PYRE_QMATMUL_F32") == "1":
         layout, path = 0, "f32 multiply-add GEMV, lane = row (k_gemv)"
     elif t == 1 and os.environ.get("PYRE_QMATMUL_NATIVE", "1") != "0":

@@ -142,7 +142,7 @@ struct pyre_qmat {
 };
 int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, int layout, pyre_qmat** out);
 // IQ3_S at the file's bits per weight with the codebook in shared memory, one token (gemv_n.hip)
-size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt = 6);          // fmt: FMT_IQ3_S (6) or FMT_IQ2_XS (5)
+size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt = 6);          // fmt: FMT_IQ3_S (6), FMT_IQ2_XS (5) or FMT_Q4_K (4)
 int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev, int fmt = 6);
 int pyre_gemv_n_table(pyre_ctx* ctx);                             // the codebook table, made at context creation
 size_t pyre_gemv_n_digit_bytes(size_t cols);

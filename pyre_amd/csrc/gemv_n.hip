@@ -25,10 +25,15 @@
 // 78 bytes, kept as five 16-byte pieces: 80 bytes per 256 weights (2.5 bit/weight against the file's 2.3125).  The signed
 // codebook is two tables of 8192 entries (weights 0..3 and 4..7 of an entry: index | four signs << 9), 64 KB of shared
 // memory; a 16-weight half of a sub-block has its own 4-bit scale, (2 n + 1) / 8, so the digit sums are joined per half.
+//
+// Q4_K (P = 9; gguf_q.rs:96-120) needs no table: a block's 144 bytes are kept as they are, nine lane = row pieces (the header
+// with d, dmin and the twelve scale bytes, then the 128 bytes of nibbles).  A dword of nibbles is four weights of one
+// sub-block (low nibbles) and four of the next (high nibbles): two masks give the two byte vectors for v_dot4_i32_i8, and
+// the dmin * min term leaves through the sub-block's sum of activation digits, which the digits launch provides.
 #include "formats.h"
 #include "iq_codebooks.h"
 
-#define DGN_STRIDE 64      // dwords per 64-column unit: 48 digit words [(sub-block*8 + group)*3 + digit], then su, pad
+#define DGN_STRIDE 64      // dwords per 64-column unit: 48 digit words [(sub-block*8 + group)*3 + digit], then su, the two sub-blocks' integer sums, pad
 
 // ---- the matrix: raw GGUF rows -> nq; one thread per (padded row, super-block) ---------------------------------------------
 __global__ __launch_bounds__(256) void k_repack_n(int rows, int rows_pad, int SB, const uint8_t* __restrict__ raw, size_t row_bytes, uint4* __restrict__ nq) {
@@ -77,6 +82,20 @@ __global__ __launch_bounds__(256) void k_repack_n2(int rows, int rows_pad, int S
   for (int p = 0; p < 5; ++p) nq[((tile * SB + sb) * 5 + p) * 64 + lane] = make_uint4(w[4 * p], w[4 * p + 1], w[4 * p + 2], w[4 * p + 3]);
 }
 
+// Q4_K: the block's nine 16-byte pieces as they are, transposed to lane = row planes; one thread per (padded row, super-block, piece)
+__global__ __launch_bounds__(256) void k_repack_n4(int rows, int rows_pad, int SB, const uint8_t* __restrict__ raw, size_t row_bytes, uint4* __restrict__ nq) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; if (idx >= (size_t)rows_pad * SB * 9) return;
+  const int p = (int)(idx % 9); const size_t rs = idx / 9; const int row = (int)(rs / SB), sb = (int)(rs % SB);
+  uint32_t w[4] = {0, 0, 0, 0};
+  if (row < rows) {
+    const uint8_t* b = raw + (size_t)row * row_bytes + (size_t)sb * 144 + p * 16;          // (rows of 144-byte blocks are 16-byte aligned only if the buffer is: bytes)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = (uint32_t)b[4 * k] | ((uint32_t)b[4 * k + 1] << 8) | ((uint32_t)b[4 * k + 2] << 16) | ((uint32_t)b[4 * k + 3] << 24);
+  }
+  const size_t tile = (size_t)(row >> 6); const int lane = row & 63;
+  nq[((tile * SB + sb) * 9 + p) * 64 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // ---- activation digits: grid = 64-column units, one wave per unit -------------------------------------------------------------
 __global__ __launch_bounds__(64) void k_act_digits_n(const float* __restrict__ x, uint32_t* __restrict__ dg) {
   __shared__ __align__(16) uint8_t sm[3][64];
@@ -96,8 +115,13 @@ __global__ __launch_bounds__(64) void k_act_digits_n(const float* __restrict__ x
   sm[0][lane] = (uint8_t)a1; sm[1][lane] = (uint8_t)a2; sm[2][lane] = (uint8_t)a3;      // byte b of group g = column 4 g + b
   __builtin_amdgcn_wave_barrier();      // one wave: its shared-memory operations execute in order
   uint32_t* o = dg + (size_t)ku * DGN_STRIDE;
+  int qs = q;                                            // the sum of each half's integers (|sum| <= 2^26), for the formats with an offset per sub-block
+#pragma unroll
+  for (int o2 = 16; o2 > 0; o2 >>= 1) qs += __shfl_xor(qs, o2);
   if (lane < 48) o[lane] = ((const uint32_t*)sm[lane % 3])[lane / 3];
   else if (lane == 48) o[48] = __float_as_uint(su);
+  if (lane == 0) o[49] = (uint32_t)qs;
+  if (lane == 32) o[50] = (uint32_t)qs;
 }
 
 // byte offset into the table of group G's entry: the 13-bit field at bit 13 G of the 28 words, times four
@@ -184,18 +208,46 @@ __device__ __forceinline__ float n_superblock(const uint4 (&r)[5], const uint8_t
   return acc;
 }
 
+// ---- Q4_K: unit C (64 weights: sub-blocks 2C and 2C + 1) of the block's 36 words
+template <int C> __device__ __forceinline__ float n4_unit(const uint32_t (&w)[36], const uint32_t* __restrict__ dgu, float d, float dmin, float acc) {
+  int ia[3] = {0, 0, 0}, ib[3] = {0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t u = w[4 + 8 * C + j]; const int lo = (int)(u & 0x0F0F0F0Fu), hi = (int)((u >> 4) & 0x0F0F0F0Fu);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { ia[k] = __builtin_amdgcn_sdot4(lo, (int)dgu[j * 3 + k], ia[k], false); ib[k] = __builtin_amdgcn_sdot4(hi, (int)dgu[(8 + j) * 3 + k], ib[k], false); }
+  }
+  const int ta = (int)(((uint32_t)ia[0] << 16) + ((uint32_t)ia[1] << 8) + (uint32_t)ia[2]), tb = (int)(((uint32_t)ib[0] << 16) + ((uint32_t)ib[1] << 8) + (uint32_t)ib[2]);      // |t| < 2^31: |i1| <= 32 * 15 * 33
+  uint32_t s1, m1, s2, m2; scale_min_k4(2 * C, w[1], w[2], w[3], s1, m1); scale_min_k4(2 * C + 1, w[1], w[2], w[3], s2, m2);
+  const float su = __uint_as_float(dgu[48]), dsu = d * su, msu = dmin * su;
+  acc = fmaf(dsu * (float)s1, (float)ta, acc); acc = fmaf(-(msu * (float)m1), (float)(int)dgu[49], acc);
+  acc = fmaf(dsu * (float)s2, (float)tb, acc); acc = fmaf(-(msu * (float)m2), (float)(int)dgu[50], acc);
+  return acc;
+}
+__device__ __forceinline__ float n_superblock(const uint4 (&r)[9], const uint8_t* lt, const uint32_t* __restrict__ dg, float acc) {
+  uint32_t w[36];
+#pragma unroll
+  for (int p = 0; p < 9; ++p) { w[4 * p] = r[p].x; w[4 * p + 1] = r[p].y; w[4 * p + 2] = r[p].z; w[4 * p + 3] = r[p].w; }
+  const float d = h2f_bits(w[0] & 0xFFFFu), dmin = h2f_bits(w[0] >> 16);
+  acc = n4_unit<0>(w, dg + 0 * DGN_STRIDE, d, dmin, acc); acc = n4_unit<1>(w, dg + 1 * DGN_STRIDE, d, dmin, acc);
+  acc = n4_unit<2>(w, dg + 2 * DGN_STRIDE, d, dmin, acc); acc = n4_unit<3>(w, dg + 3 * DGN_STRIDE, d, dmin, acc);
+  return acc;
+}
+
 // grid = min(tiles, what the chip holds at once), NW waves; the workgroup fills its table, then takes row tiles
 // blockIdx.x, + gridDim.x, ..; wave w walks super-blocks [w * spw, + spw) of the tile, lane l owns row tile * 64 + l; the
 // waves' sums meet in shared memory in wave order.  The next super-block's seven pieces are requested before the current
 // one's arithmetic starts.
-// P: 16-byte pieces a super-block has (7: IQ3_S, one 32 KB table; 5: IQ2_XS, two)
+// P: 16-byte pieces a super-block has (7: IQ3_S, one 32 KB table; 5: IQ2_XS, two; 9: Q4_K, none)
 template <int NW, int P = 7> __global__ __launch_bounds__(NW * 64) void k_gemv_n(const uint4* __restrict__ nq, int rows, int tiles, int SB, const uint4* __restrict__ tab, const uint32_t* __restrict__ dg, float* __restrict__ y, int spw) {
-  constexpr int TW = P == 7 ? 2048 : 4096;          // 16-byte words of the table(s)
-  __shared__ __align__(16) uint8_t lt[TW * 16];
+  constexpr int TW = P == 7 ? 2048 : (P == 5 ? 4096 : 0);          // 16-byte words of the table(s)
+  __shared__ __align__(16) uint8_t lt[TW ? TW * 16 : 16];
   __shared__ float red[NW][64];
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  for (int i = tid; i < TW; i += NW * 64) ((uint4*)lt)[i] = tab[i];
-  __syncthreads();
+  if constexpr (TW > 0) {
+    for (int i = tid; i < TW; i += NW * 64) ((uint4*)lt)[i] = tab[i];
+    __syncthreads();
+  }
   const int s0 = min(SB, wave * spw), s1 = min(SB, s0 + spw);
   uint4 bufa[P], bufb[P];
   const size_t tstride = (size_t)SB * P * 64;
@@ -243,10 +295,11 @@ namespace {
 int env_i(const char* n, int dflt) { const char* s = getenv(n); return s && *s ? atoi(s) : dflt; }
 }
 
-size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt) { return ((rows + 63) / 64) * 64 * (cols / 256) * (fmt == FMT_IQ2_XS ? 80 : 112); }
+size_t pyre_gemv_n_bytes(size_t rows, size_t cols, int fmt) { return ((rows + 63) / 64) * 64 * (cols / 256) * (fmt == FMT_IQ2_XS ? 80 : (fmt == FMT_Q4_K ? 144 : 112)); }
 
 int pyre_gemv_n_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* nq_dev, int fmt) {
   const int SB = (int)(cols / 256); const size_t rows_pad = (rows + 63) / 64 * 64, total = rows_pad * SB;
+  if (fmt == FMT_Q4_K) { hipLaunchKernelGGL(k_repack_n4, dim3((unsigned)((total * 9 + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, raw_dev, row_bytes, (uint4*)nq_dev); PYRE_CHECK_LAUNCH(ctx); return PYRE_OK; }
   if (fmt == FMT_IQ2_XS) { hipLaunchKernelGGL(k_repack_n2, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, raw_dev, row_bytes, (uint4*)nq_dev); PYRE_CHECK_LAUNCH(ctx); return PYRE_OK; }
   hipLaunchKernelGGL(k_repack_n, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, (int)rows, (int)rows_pad, SB, raw_dev, row_bytes, (uint4*)nq_dev);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
@@ -304,6 +357,17 @@ int pyre_gemv_n_launch(pyre_ctx* ctx, const void* nq, size_t rows, size_t cols, 
   int grid = fwg > 0 ? fwg : 256 * per_cu;
   static const int fgrid = env_i("PYRE_GEMV_N_GRID", 0); if (fgrid > 0) grid = fgrid;
   if (grid > tiles) grid = tiles;
+  if (fmt == FMT_Q4_K) {
+    ProfScope ps(ctx, "gemv_n_q4_k_t1", (double)rows * (cols / 256) * 144 + 4.0 * ((double)cols + rows));
+    const uint4* q = (const uint4*)nq;
+    switch (nw) {
+      case 1: hipLaunchKernelGGL((k_gemv_n<1, 9>), dim3(grid), dim3(64), 0, ctx->stream, q, (int)rows, tiles, SB, nullptr, dg, y_dev, spw); break;
+      case 2: hipLaunchKernelGGL((k_gemv_n<2, 9>), dim3(grid), dim3(128), 0, ctx->stream, q, (int)rows, tiles, SB, nullptr, dg, y_dev, spw); break;
+      case 8: hipLaunchKernelGGL((k_gemv_n<8, 9>), dim3(grid), dim3(512), 0, ctx->stream, q, (int)rows, tiles, SB, nullptr, dg, y_dev, spw); break;
+      default: hipLaunchKernelGGL((k_gemv_n<4, 9>), dim3(grid), dim3(256), 0, ctx->stream, q, (int)rows, tiles, SB, nullptr, dg, y_dev, spw); break;
+    }
+    PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
+  }
   if (fmt == FMT_IQ2_XS) {          // two 32 KB tables a workgroup: eight waves, two workgroups a compute unit
     ProfScope ps(ctx, "gemv_n_iq2_xs_t1", (double)rows * (cols / 256) * 74 + 4.0 * ((double)cols + rows));
     const uint4* q = (const uint4*)nq; const uint4* tb = (const uint4*)ctx->d_iq2xs_sgn;

@@ -466,7 +466,7 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
   if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
   size_t row_bytes = cols / gel * gbytes;
   if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
-  const bool want_n = layout == PYRE_LAYOUT_BOTH && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS) && cols % 256 == 0;      // the single token's native-format layout
+  const bool want_n = layout == PYRE_LAYOUT_BOTH && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS || (fmt == FMT_Q4_K && ty == PYRE_Q4_K)) && cols % 256 == 0;      // the single token's native-format layout
   if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // only IQ3_S has a matrix-core layout
   const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
@@ -577,9 +577,9 @@ static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev,
   // paths need a second one for the activations, and a call of this size is its launches, not its bytes
   if (qmat_small_one_token(m, t) && !f32_path && !f32_only) return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   // one token of an IQ3_S matrix: the kernel that streams the file's 3.44 bit/weight (PYRE_QMATMUL_NATIVE=0: the matrix cores as for a window)
-  // (IQ2_XS has the same kernel over its own 2.5 bit/weight layout; a small matrix of it stays with the one-launch f32 GEMV likewise)
-  const bool iq2 = m->dv.fmt == FMT_IQ2_XS;
-  if (t == 1 && m->base_n && native && !f32_path && !f32_only && !(iq2 && m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, nullptr, iq2 ? FMT_IQ2_XS : FMT_IQ3_S);
+  // (IQ2_XS and Q4_K have the same kernel over their own layouts, 2.5 and 4.5 bit/weight; a small matrix of them stays with the one-launch f32 GEMV likewise)
+  const bool rows_only = m->dv.fmt == FMT_IQ2_XS || m->dv.fmt == FMT_Q4_K;          // (the formats without a matrix-core layout)
+  if (t == 1 && m->base_n && native && !f32_path && !f32_only && !(rows_only && m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, nullptr, rows_only ? m->dv.fmt : FMT_IQ3_S);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
   if (has_m && (!has_rows || (!f32_path && !f32_only))) return pyre_gemv_launch(ctx, m->dvm, x_dev, t, y_dev);
   return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
@@ -605,15 +605,15 @@ int pyre_qmatmul(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, 
 int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, int t, float* y_dev) {
   if (!ctx || !m || !x_dev || !y_dev) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: null argument");
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmatmul_static_dev: t = %d outside 1..8", t);
-  if (m->dv.fmt == FMT_IQ2_XS && m->base_n) {      // IQ2_XS: only the single token of a large matrix uses scratch (the native-format kernel's activation digits)
+  if ((m->dv.fmt == FMT_IQ2_XS || m->dv.fmt == FMT_Q4_K) && m->base_n) {      // IQ2_XS, Q4_K: only the single token of a large matrix uses scratch (the native-format kernel's activation digits)
     if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
     if (t == 1 && env_int("PYRE_QMATMUL_NATIVE", 1) && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {
       if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
-      return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, ctx->aop_static, FMT_IQ2_XS);
+      return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, ctx->aop_static, m->dv.fmt);
     }
     return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   }
-  if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S and IQ2_XS matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S, IQ2_XS and Q4_K matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
   if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
   if (qmat_small_one_token(m, t) && !env_int("PYRE_QMATMUL_F32", 0)) return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);      // as pyre_qmatmul_dev (a launch that happens to need no scratch; the limit above holds for every call alike)
   if (t == 1 && m->base_n && env_int("PYRE_QMATMUL_NATIVE", 1)) {      // one token: the native-format kernel, as in pyre_qmatmul_dev, its activation digits in the static array

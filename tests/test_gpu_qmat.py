@@ -298,15 +298,17 @@ def test_iq3s_native_format_single_token(ctx, rows, cols, monkeypatch):
     assert not m.matmul(np.zeros((1, cols), np.float32)).any()
 
 
-# ---- one token of an IQ2_XS matrix: 80 bytes per 256 weights, two signed codebook tables in shared memory, integer dots ----------
+# ---- one token of an IQ2_XS matrix: 80 bytes per 256 weights, two signed codebook tables in shared memory, integer dots;
+# ---- of a Q4_K matrix: the file's 144 bytes, nibbles straight into the integer dots, the minima through the digit sums ----------
 @pytest.mark.gpu
+@pytest.mark.parametrize("ty,piece_bytes", [(lib.IQ2_XS, 80), (lib.Q4_K, 144)])
 @pytest.mark.parametrize("rows,cols", [(64, 256), (100, 256), (65, 512), (320, 2048), (4096, 2048), (1000, 768), (130, 8192), (8256, 1024)])
-def test_iq2xs_native_format_single_token(ctx, rows, cols, monkeypatch):
+def test_iq2xs_q4k_native_format_single_token(ctx, rows, cols, ty, piece_bytes, monkeypatch):
     monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the native-format kernel
-    raw = synth.matrix(lib.IQ2_XS, rows, cols, 500 + rows % 97)
-    m = lib.QMat(ctx, lib.IQ2_XS, rows, cols, raw)
-    assert m.layout_bytes(2) == (rows + 63) // 64 * 64 * (cols // 256) * 80
-    W = orc.dequant(lib.IQ2_XS, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    raw = synth.matrix(ty, rows, cols, 500 + rows % 97)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
+    assert m.layout_bytes(2) == (rows + 63) // 64 * 64 * (cols // 256) * piece_bytes
+    W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
     g = np.random.Generator(np.random.PCG64(rows + cols + 1))
     for case in range(6):
         x = synth.normal((1, cols), 600 + case)

@@ -47,9 +47,10 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_consecutive_cal
     big.close(); small.close()
 
 
-def test_static_scratch_entry_point_iq2xs_single_token(ctx):
-    big = lib.QMat(ctx, lib.IQ2_XS, 8256, 2048, synth.matrix(lib.IQ2_XS, 8256, 2048, 511))          # 129 row tiles: the native-format kernel, digits in the array
-    small = lib.QMat(ctx, lib.IQ2_XS, 320, 512, synth.matrix(lib.IQ2_XS, 320, 512, 512))          # one launch, no scratch
+@pytest.mark.parametrize("ty", [lib.IQ2_XS, lib.Q4_K])
+def test_static_scratch_entry_point_iq2xs_q4k_single_token(ctx, ty):
+    big = lib.QMat(ctx, ty, 8256, 2048, synth.matrix(ty, 8256, 2048, 511))          # 129 row tiles: the native-format kernel, digits in the array
+    small = lib.QMat(ctx, ty, 320, 512, synth.matrix(ty, 320, 512, 512))          # one launch, no scratch
     for m, rows, cols, t in ((big, 8256, 2048, 1), (small, 320, 512, 1), (big, 8256, 2048, 4), (big, 8256, 2048, 1)):
         a, b = both(ctx, m, rows, cols, synth.normal((t, cols), 513 + t))
         assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
