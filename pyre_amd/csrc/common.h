@@ -239,6 +239,7 @@ struct MoeWork {            // scratch for up to 8 tokens, owned by whoever laun
   float* h;                 // [8*(top_k+1)][max(ff, sf)]
   float* partial;           // [8*(top_k+1)][d]
   float* parts;             // [PYRE_MOE_GROUPS][t][d]: a window's output as group sums (pyre_moe_launch with in_groups)
+  uint32_t* dgx;            // [8][d/64][64]: the activations' digits for the integer-dot gate/up products (IQ3_S experts)
 };
 // The FFN output of a window, left unreduced for the consumer to fold.  The k expert terms (ascending id) and the shared
 // expert's form PYRE_MOE_GROUPS groups of g = (k + 4) / 4 consecutive experts, the shared expert in the last:
@@ -285,7 +286,7 @@ void   pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w);
 // (pyre_moe_out) for a consumer that evaluates moe_out_value itself.
 // Router logits that arrive as K-slice sums (left by the mix that produced x, see HcRoute): logit[t][e] = the slices
 // p[(s*T + t)*r64 + e], s = 0..nsl-1, added in slice order.
-struct RouteSrc { const float* p; int nsl; int r64; };
+struct RouteSrc { const float* p; int nsl; int r64; const uint32_t* dgx = nullptr; };          // dgx: the activations' digits (digits.h), left by the same mix, or null
 // in_groups (t > 1, y == nullptr, pyre_moe_groups_ok): the down projection leaves the PYRE_MOE_GROUPS group sums of every
 // token in w.parts, group q of token ti at parts + (q*t + ti)*d, instead of the unreduced terms.
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr, bool in_groups = false);
@@ -322,7 +323,7 @@ void   pyre_hc_work_carve(const HcDev& h, void* base, HcWork* w);
 // The router GEMV of the FFN block that follows a mix, riding on the mix's second launch: workgroup b of that launch
 // owns columns [64b, 64b+64) of the mixed vector, so it leaves the K-slice sum part[(b*T + t)*tiles*64 + row] of every
 // router row; the gate/up launch adds the d/64 slices (RouteSrc).  bf16 and f32 routers, at most 64 slices.
-struct HcRoute { QMatDev router; float* part; };
+struct HcRoute { QMatDev router; float* part; uint32_t* dgx = nullptr; };          // dgx: where the mix leaves the digits of its output for the expert products (digits.h), or null
 // Where a producer kernel leaves its result as the f16 operand of the matrix-core GEMM that follows (so that GEMM needs no
 // split launch of its own): op = PyreAop::op (pyre_aop_rows(t) rows), ainv = PyreAop::ainv, [nsb super-blocks][8 tokens].
 // Every token is scaled by one power of two that brings a bound of its largest magnitude into [2^13, 2^14) -- a bound every

@@ -6,6 +6,7 @@
 // into the streams' RMS scales, adds the scaled slice sums, applies silu, runs the up GEMV from shared memory and
 // reduces the gated, normalized streams to their mean.
 #include "gemm_m.h"
+#include "digits.h"
 #include <stdlib.h>
 #include <algorithm>
 
@@ -378,8 +379,9 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
 // them): divisions become shifts, the slice loops lose their predicates -- same arithmetic.
 template <int T, int RF, int FHC = 0, int FLR = 0, int FKS = 0> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
-    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb) {
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb, uint32_t* __restrict__ dgx) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
+  __shared__ uint8_t dsm[ROUTE ? T : 1][3][64];          // the digit waves' staging
   const uint2* lds2 = nullptr;
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj, lcw);
@@ -491,6 +493,8 @@ template <int T, int RF, int FHC = 0, int FLR = 0, int FKS = 0> __global__ __lau
   }
   if (ROUTE) {
     lds_barrier();
+    // the digits of the workgroup's 64 columns for the expert products that follow: token t2 by wave nw - 1 - t2 (the waves the router's tiles leave idle)
+    if (dgx && lcw == 6) for (int t2 = nw - 1 - wave; t2 < T; t2 += nw) digits_eo_wave(lo[t2 * 64 + lane], lane, dsm[ROUTE ? t2 : 0], dgx + ((size_t)t2 * (d >> 6) + blockIdx.x) * DGX_STRIDE);
     const size_t rr64 = (size_t)router.tiles * 64;
     for (int tile = rtile; rwave && tile < rnt; tile += nw) {          // (more tiles than waves: one set, the tiles in turns)
       if (tile != rtile) rraw = unit_load<RFX>(router, tile, blockIdx.x, lane);
@@ -580,7 +584,7 @@ template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
 #define UP_MIX_M_ARGS dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0
+                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0, rt ? rt->dgx : nullptr
 #define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), UP_MIX_M_ARGS)
 #define UP_MIX_M_FIX(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF, 4, 256, 16>), UP_MIX_M_ARGS)
   bool done = false;

@@ -585,7 +585,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc; }
     else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc;
     const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
-    HcRoute hr{L.moe.router, m->rpart}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64};
+    HcRoute hr{L.moe.router, m->rpart, m->mw.dgx}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64, pyre_hc_aop_ok(L.hcf) ? m->mw.dgx : nullptr};          // (the matrix-core mix leaves the digits of its output; after another mix the expert launch makes them)
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
     advance();
     // A window's FFN output goes to the next mix as four group sums a token when that mix can add partial vectors (an

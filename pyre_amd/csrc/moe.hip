@@ -3,6 +3,7 @@
 // Follows ffn / routed (f32 branch) of the reference, src/model/qwen4exp_gguf.rs:1675-1684, 1721-1732, 1754-1793,
 // and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
 #include "formats.h"
+#include "digits.h"
 PYRE_TS_DECL(moe_ts) PYRE_TS_EXPORT(moe_ts, pyre_debug_ts_moe)
 
 // ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id -----------------------------
@@ -135,9 +136,12 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // the selection otherwise); the workgroup reads its expert id and publishes nothing but the shared-expert gate.
 // FIX: the A3B configuration's constants (512 experts, top 10, d = 2048 in 32 router slices, ff = 512) folded in at compile
 // time (the launcher checks them) -- same arithmetic.
-template <int FMT, int NW, int P, bool PRE, bool FIX = false>
+// ID (IQ3_S): the dot products in the integer form of digits.h -- 1.4 vector instructions a weight where byte -> float and
+// multiply-add take 3; dgx holds the digits of the window's activations, token ti at dgx + ti * (d / 64) * DGX_STRIDE.
+template <int FMT, int NW, int P, bool PRE, bool FIX = false, bool ID = false>
 __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 8 : 1) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
-                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride) {
+                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride, const uint32_t* __restrict__ dgx) {
+  static_assert(!ID || FMT == FMT_IQ3_S, "the integer form is IQ3_S's");
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
   args_now(m.n_exp, m.top_k, logits, nsl, sstride, tstride);          // what the selection needs; the rest would crowd the scalar registers the activations go through
@@ -177,6 +181,12 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
   const int nz = (FIX && !PRE) ? 2 : (FIX ? 1 : (int)gridDim.z), kz = blockIdx.z, np = P * nz;          // np parts in all (FIX: two workgroups a single token's entry, one a window's)
   const int GU = FIX ? 32 : G.U;          // 64-column units of a row (both matrices, routed or shared: d / 64)
   const int upw = (GU + NW * np - 1) / (NW * np);
+  const uint32_t* dgs = ID ? dgx + (size_t)ti * GU * DGX_STRIDE : nullptr;
+  // one unit of a matrix into an accumulator, in the f32 or the integer form
+  auto mac = [&](const QMatDev& Q, const UnitRaw<FMT>& r, int ku, float (&a)[1]) {
+    if constexpr (ID) unit_idot_iq3s(r, dgs + (size_t)ku * DGX_STRIDE, a[0]);
+    else unit_fma<FMT, 1>(Q, r, ku, lds2, lane, xs + ku * 64, 0, a);
+  };
   float ag[P][1], au[P][1];
 #pragma unroll
   for (int p = 0; p < P; ++p) { ag[p][0] = 0.0f; au[p][0] = 0.0f; }
@@ -184,8 +194,8 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
     // one unit per part: both parts' units of both matrices are fetched before the first is consumed
     const int ka = min(2 * wave, GU - 1), kb = min(2 * wave + 1, GU - 1);
     UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ka, lane), u0 = unit_load<FMT>(Up, tile, ka, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
-    if (2 * wave < GU) { unit_fma<FMT, 1>(G, g0, ka, lds2, lane, xs + ka * 64, 0, ag[0]); unit_fma<FMT, 1>(Up, u0, ka, lds2, lane, xs + ka * 64, 0, au[0]); }
-    if (2 * wave + 1 < GU) { unit_fma<FMT, 1>(G, g1, kb, lds2, lane, xs + kb * 64, 0, ag[P - 1]); unit_fma<FMT, 1>(Up, u1, kb, lds2, lane, xs + kb * 64, 0, au[P - 1]); }
+    if (2 * wave < GU) { mac(G, g0, ka, ag[0]); mac(Up, u0, ka, au[0]); }
+    if (2 * wave + 1 < GU) { mac(G, g1, kb, ag[P - 1]); mac(Up, u1, kb, au[P - 1]); }
   } else {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
@@ -194,8 +204,8 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
       for (int ku = k0; ku < kend; ku += 2) {
         const int kb = min(ku + 1, kend - 1);
         UnitRaw<FMT> g0 = unit_load<FMT>(G, tile, ku, lane), u0 = unit_load<FMT>(Up, tile, ku, lane), g1 = unit_load<FMT>(G, tile, kb, lane), u1 = unit_load<FMT>(Up, tile, kb, lane);
-        unit_fma<FMT, 1>(G, g0, ku, lds2, lane, xs + ku * 64, 0, ag[p]); unit_fma<FMT, 1>(Up, u0, ku, lds2, lane, xs + ku * 64, 0, au[p]);
-        if (ku + 1 < kend) { unit_fma<FMT, 1>(G, g1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, ag[p]); unit_fma<FMT, 1>(Up, u1, ku + 1, lds2, lane, xs + (ku + 1) * 64, 0, au[p]); }
+        mac(G, g0, ku, ag[p]); mac(Up, u0, ku, au[p]);
+        if (ku + 1 < kend) { mac(G, g1, ku + 1, ag[p]); mac(Up, u1, ku + 1, au[p]); }
       }
     }
   }
@@ -381,10 +391,17 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   }
 }
 
+// the digits of t tokens' activations as a launch of its own (callers whose producer kernel does not leave them): grid (d / 64, t), one wave
+__global__ __launch_bounds__(64) void k_act_digits_eo(const float* __restrict__ x, int d, uint32_t* __restrict__ dgx) {
+  __shared__ uint8_t sm[3][64];
+  const int ku = blockIdx.x, ti = blockIdx.y, lane = threadIdx.x;
+  digits_eo_wave(x[(size_t)ti * d + ku * 64 + lane], lane, sm, dgx + ((size_t)ti * (d >> 6) + ku) * DGX_STRIDE);
+}
+
 #define PYRE_MOE_GU_NZMAX 2
 size_t pyre_moe_work_bytes(const MoeDev& m) {
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
-  return 256 * 9 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d + 8 * PYRE_MOE_GROUPS * (size_t)m.d);
+  return 256 * 10 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d + 8 * PYRE_MOE_GROUPS * (size_t)m.d + 8 * (size_t)(m.d / 64) * DGX_STRIDE);
 }
 void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
@@ -392,6 +409,7 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   w->logits = (float*)take(4 * 8 * (size_t)m.n_exp); w->sel_idx = (int32_t*)take(4 * 8 * (size_t)m.top_k); w->sel_w = (float*)take(4 * 8 * (size_t)m.top_k);
   w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
   w->parts = (float*)take(4 * 8 * PYRE_MOE_GROUPS * (size_t)m.d);
+  w->dgx = (uint32_t*)take(4 * 8 * (size_t)(m.d / 64) * DGX_STRIDE);
 }
 
 #define MOE_FMT_DISPATCH(fmt, CALL) \
@@ -418,19 +436,29 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   const int hs = m.ff > m.sf ? m.ff : m.sf, entries = t * (m.top_k + 1);
   const uint2* g2 = (const uint2*)ctx->d_iq2xs;
   const int P = pyre_moe_gu_parts(m), nz = (P > 1 && t == 1) ? P : 1;
+  // IQ3_S experts: gate/up in the integer form, on the digits the mix left beside the activations or on a launch of their own
+  static const bool idot_on = !(getenv("PYRE_MOE_IDOT") && atoi(getenv("PYRE_MOE_IDOT")) == 0);
+  const bool idot = idot_on && m.gate_e.fmt == FMT_IQ3_S && m.sh_gate.fmt == FMT_IQ3_S;
+  const uint32_t* dgx = nullptr;
+  if (idot) {
+    if (routed && routed->dgx) dgx = routed->dgx;
+    else { ProfScope ps(ctx, "moe_digits", 4.0 * t * m.d * 2); hipLaunchKernelGGL(k_act_digits_eo, dim3(m.d / 64, t), dim3(64), 0, ctx->stream, x, m.d, w.dgx); PYRE_CHECK_LAUNCH(ctx); dgx = w.dgx; }
+  }
   const bool a3b = t == 1 && m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512;          // the instances with these constants folded in
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
-#define GU_GO(PP, NZ, PRE) MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP, PRE>), dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride))
-  if (t == 1 && a3b && nsl == 32 && nz == 2) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true>), dim3(hs / 64, entries, 2), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride);
+#define GU_ARGS(NZ) dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride, dgx
+#define GU_GO(PP, NZ, PRE) do { if (idot) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, PP, PRE, false, true>), GU_ARGS(NZ)); else MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP, PRE>), GU_ARGS(NZ))); } while (0)
+  if (t == 1 && a3b && nsl == 32 && nz == 2) { if (idot) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true, true>), GU_ARGS(2)); else hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true>), GU_ARGS(2)); }
   else if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
   else {
     const bool a3bw = m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512 && nsl == 32;          // a window of the A3B configuration: constants folded in
     if (a3bw) hipLaunchKernelGGL(k_moe_route<true>, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
     else hipLaunchKernelGGL(k_moe_route<false>, dim3(t), dim3(1024), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, nsl, sstride, tstride);
-    if (a3bw && P == 2) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 2, true, true>), dim3(hs / 64, entries, 1), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride);
+    if (a3bw && P == 2) { if (idot) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 2, true, true, true>), GU_ARGS(1)); else hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 2, true, true>), GU_ARGS(1)); }
     else if (P == 2) { GU_GO(2, 1, true); } else { GU_GO(1, 1, true); }
   } }
 #undef GU_GO
+#undef GU_ARGS
   PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
   if (in_groups) {
