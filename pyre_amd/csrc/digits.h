@@ -1,6 +1,6 @@
 // Activations as block fixed point for the integer-dot form of a GEMV over 4-bit codes: per 64 columns one power of two
-// and, per value, three signed-byte digits in base 256 (|q| <= 2^21), so that sum(code * x) is three v_dot4_i32_i8 sums
-// joined in integers.  The digit bytes are arranged for the lane = row layout of the 4-bit codes (QMatDev::p0 of an IQ3_S
+// and, per value, three signed-byte digits in base 256 (|q| <= 2^22: with codes of at most 15 a 32-value sub-block's
+// sum stays below 2^31), so that sum(code * x) is three v_dot4_i32_i8 sums joined in integers.  The digit bytes are arranged for the lane = row layout of the 4-bit codes (QMatDev::p0 of an IQ3_S
 // matrix: nibble i of word k is value 8k + i): word 2k of a digit plane holds columns 8k, 8k+2, 8k+4, 8k+6 -- what the
 // mask 0x0F0F0F0F leaves of code word k -- and word 2k+1 columns 8k+1, .., 8k+7 -- what it leaves after a shift by four.
 //   unit u of a token: dg[u * 64 + w * 3 + j], w = 0..15 the word, j = 0..2 the digit (most significant first);
@@ -20,12 +20,12 @@ __device__ __forceinline__ void digits_eo_wave(float v, int lane, uint8_t (*sm)[
   if (!fin) su = __uint_as_float(0x7FC00000u);            // a non-finite activation makes the unit's contribution NaN
   else if (mx > 0.0f) {
     int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 126; if (e < -100) e = -100;      // mx < 2^e (subnormal maxima take the clamp)
-    su = __uint_as_float((uint32_t)(e - 21 + 127) << 23); q = (int)rintf(v * __uint_as_float((uint32_t)(21 - e + 127) << 23));      // |q| <= 2^21
+    su = __uint_as_float((uint32_t)(e - 22 + 127) << 23); q = (int)rintf(v * __uint_as_float((uint32_t)(22 - e + 127) << 23));      // |q| <= 2^22
   }
   const int a3 = (int)(int8_t)(q & 0xFF), q1 = (q - a3) >> 8, a2 = (int)(int8_t)(q1 & 0xFF), a1 = (q1 - a2) >> 8;
   const int pos = (((lane >> 3) * 2 + (lane & 1)) << 2) + ((lane & 7) >> 1);
   sm[0][pos] = (uint8_t)a1; sm[1][pos] = (uint8_t)a2; sm[2][pos] = (uint8_t)a3;
-  int qs = q;
+  int qs = q;                                            // (|sum of 32| <= 2^27)
 #pragma unroll
   for (int s = 16; s > 0; s >>= 1) qs += __shfl_xor(qs, s);
   __builtin_amdgcn_wave_barrier();      // one wave: its shared-memory operations execute in order
@@ -52,7 +52,7 @@ __device__ __forceinline__ void unit_idot_iq3s(const UnitRaw<FMT_IQ3_S>& r, cons
       i1 = __builtin_amdgcn_sdot4(lo, (int)p[0], i1, false); i2 = __builtin_amdgcn_sdot4(lo, (int)p[1], i2, false); i3 = __builtin_amdgcn_sdot4(lo, (int)p[2], i3, false);
       i1 = __builtin_amdgcn_sdot4(hi, (int)p[3], i1, false); i2 = __builtin_amdgcn_sdot4(hi, (int)p[4], i2, false); i3 = __builtin_amdgcn_sdot4(hi, (int)p[5], i3, false);
     }
-    const int t = (int)(((uint32_t)i1 << 16) + ((uint32_t)i2 << 8) + (uint32_t)i3);          // |t| <= 32 * 15 * 2^21 < 2^31
+    const int t = (int)(((uint32_t)i1 << 16) + ((uint32_t)i2 << 8) + (uint32_t)i3);          // |t| <= 32 * 15 * 2^22 < 2^31
     const float db = d * (float)(1 + 2 * ((sc >> (4 * sb)) & 0xF));
     acc = fmaf(db, fmaf(-15.0f, (float)(int)dgu[49 + sb], 2.0f * (float)t), acc);
   }
