@@ -7,14 +7,13 @@
 //   dg[u * 64 + 48] the unit's power of two (f32 bits), [49] / [50] the integer sums of the values of columns 0..31 / 32..63.
 #pragma once
 #include "formats.h"
+#include "common.h"
 
 #define DGX_STRIDE 64
 
 // one wave, lane = column: v is the lane's activation; sm is [3][64] bytes of the wave's own shared memory
 __device__ __forceinline__ void digits_eo_wave(float v, int lane, uint8_t (*sm)[64], uint32_t* __restrict__ o) {
-  float mx = fabsf(v);
-#pragma unroll
-  for (int s = 32; s > 0; s >>= 1) mx = fmaxf(mx, __shfl_xor(mx, s));
+  const float mx = wave_max(fabsf(v));
   const bool fin = __all(isfinite(v));
   float su = 0.0f; int q = 0;
   if (!fin) su = __uint_as_float(0x7FC00000u);            // a non-finite activation makes the unit's contribution NaN
@@ -25,14 +24,17 @@ __device__ __forceinline__ void digits_eo_wave(float v, int lane, uint8_t (*sm)[
   const int a3 = (int)(int8_t)(q & 0xFF), q1 = (q - a3) >> 8, a2 = (int)(int8_t)(q1 & 0xFF), a1 = (q1 - a2) >> 8;
   const int pos = (((lane >> 3) * 2 + (lane & 1)) << 2) + ((lane & 7) >> 1);
   sm[0][pos] = (uint8_t)a1; sm[1][pos] = (uint8_t)a2; sm[2][pos] = (uint8_t)a3;
-  int qs = q;                                            // (|sum of 32| <= 2^27)
-#pragma unroll
-  for (int s = 16; s > 0; s >>= 1) qs += __shfl_xor(qs, s);
+  // the integer sums of the two halves (|sum of 32| <= 2^27): four steps inside each row of sixteen lanes, then lane 15 of rows 0 and 2
+  // into rows 1 and 3 -- lanes 16..31 hold the first half's sum, lanes 48..63 the second's
+  int qs = q;
+  qs += __builtin_amdgcn_update_dpp(0, qs, 0xB1, 0xf, 0xf, false); qs += __builtin_amdgcn_update_dpp(0, qs, 0x4E, 0xf, 0xf, false);
+  qs += __builtin_amdgcn_update_dpp(0, qs, 0x141, 0xf, 0xf, false); qs += __builtin_amdgcn_update_dpp(0, qs, 0x140, 0xf, 0xf, false);
+  qs += __builtin_amdgcn_update_dpp(0, qs, 0x142, 0xa, 0xf, false);
   __builtin_amdgcn_wave_barrier();      // one wave: its shared-memory operations execute in order
   if (lane < 48) o[lane] = ((const uint32_t*)sm[lane % 3])[lane / 3];
   else if (lane == 48) o[48] = __float_as_uint(su);
-  if (lane == 0) o[49] = (uint32_t)qs;
-  if (lane == 32) o[50] = (uint32_t)qs;
+  if (lane == 16) o[49] = (uint32_t)qs;
+  if (lane == 48) o[50] = (uint32_t)qs;
 }
 
 // acc += sum_j W[row, unit's 64 columns] * x[j] for the lane's row of an IQ3_S unit in the lane = row layout, the

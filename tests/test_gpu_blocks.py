@@ -62,6 +62,47 @@ def test_moe_gate_up_in_two_k_parts(ctx, qtype, d):
         assert np.array_equal(y1.view(np.uint32), y[ti:ti + 1].view(np.uint32))
 
 
+def test_moe_iq3s_gate_up_in_the_integer_form_over_the_activation_range(ctx):
+    # IQ3_S experts multiply gate/up in integers: per 64 columns the activations become a power of two and three signed-byte
+    # digits.  Activations whose 64-column stretches sit on powers of two of their own, outliers, tiny and huge values must
+    # still give the oracle's result; a window equals its single steps bit for bit; PYRE_MOE_IDOT=0 (the f32 multiply-add
+    # form, read once per process: a fresh one) agrees to rounding and chooses the same experts.
+    c = mg.Config(n_layers=1, full_every=4, d=2048, n_exp=16, top_k=4, ff_exp=256, qtype=synth.IQ3_S)
+    moe, oracle, _ = moe_pair(ctx, c, 13)
+    g = np.random.Generator(np.random.PCG64(77))
+    xs = []
+    for case in range(5):
+        x = synth.normal((3, c.d), 700 + case)
+        if case == 1: x *= np.exp2(g.integers(-20, 20, c.d // 64).repeat(64)).astype(np.float32)
+        if case == 2: x[0, 5] = 3.0e3; x[1, c.d - 3] = -2.0e4
+        if case == 3: x *= 1e-20
+        if case == 4: x[:, ::2] = 0.0; x[:, :64] = 0.0
+        xs.append(x)
+        y, idx, w = moe.ffn(x)
+        yo, io, wo = oracle(x)
+        assert np.array_equal(idx, io), case
+        assert relerr(y, yo) <= TOL, case
+        for ti in range(3):
+            y1, _, _ = moe.ffn(x[ti:ti + 1])
+            assert np.array_equal(y1.view(np.uint32), y[ti:ti + 1].view(np.uint32)), (case, ti)
+    import subprocess, sys, os
+    code = ("import numpy as np, sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+            "from pyre_amd import lib, synth, modelgen as mg\n"
+            "import test_gpu_blocks as tb\n"
+            "ctx = lib.Context(0); c = mg.Config(n_layers=1, full_every=4, d=2048, n_exp=16, top_k=4, ff_exp=256, qtype=synth.IQ3_S)\n"
+            "moe, _, _ = tb.moe_pair(ctx, c, 13)\n"
+            "x = np.frombuffer(bytes.fromhex(sys.stdin.read()), dtype=np.float32).reshape(3, 2048)\n"
+            "y, idx, w = moe.ffn(x); sys.stdout.write(y.tobytes().hex() + ' ' + idx.astype(np.int32).tobytes().hex())\n") % (
+                os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, PYRE_MOE_IDOT="0"), input=xs[1].tobytes().hex(), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    yh, ih = out.stdout.strip().split(" ")
+    yf = np.frombuffer(bytes.fromhex(yh), dtype=np.float32).reshape(3, c.d)
+    y, idx, _ = moe.ffn(xs[1])
+    assert np.array_equal(np.frombuffer(bytes.fromhex(ih), dtype=np.int32).reshape(idx.shape), idx.astype(np.int32))
+    assert relerr(y, yf) <= 2e-6 and not np.array_equal(y.view(np.uint32), yf.view(np.uint32))          # (two forms: equal to rounding, not bit for bit)
+
+
 @pytest.mark.parametrize("t", [1, 4])
 def test_moe_ffn_benchmark_geometry(ctx, t):
     # 512 routed experts + 1 shared, d 2048, expert ff 512, top-10, IQ3_S (reduced to 64 resident experts' worth of
