@@ -46,6 +46,7 @@ struct pyre_ctx {
   uint32_t* d_iq2xs_sgn = nullptr;                     // IQ2_XS likewise: two tables of 8192 x four signed bytes (weights 0..3 / 4..7 of an entry)
   uint32_t* d_iq3s_sgn = nullptr;                      // IQ3_S codebook with the signs folded in: 8192 x four signed bytes (gemv_n.hip), made at first use
   void* dgn_buf = nullptr; size_t dgn_bytes = 0;       // activation digits of the native-format IQ3_S GEMV (grow-only)
+  int spec_adapt = -1;                                 // adaptive draft length of the drafted greedy loops: 1 on, 0 off, -1 PYRE_SPEC_ADAPT in the environment (unset: off)
 };
 
 // Wraps one kernel launch when profiling is on (bytes = algorithmic bytes the launch moves).
@@ -240,6 +241,7 @@ struct MoeWork {            // scratch for up to 8 tokens, owned by whoever laun
   float* partial;           // [8*(top_k+1)][d]
   float* parts;             // [PYRE_MOE_GROUPS][t][d]: a window's output as group sums (pyre_moe_launch with in_groups)
   uint32_t* dgx;            // [8][d/64][64]: the activations' digits for the integer-dot gate/up products (IQ3_S experts)
+  uint32_t* dgh;            // [8*(top_k+1)][max(ff, sf)/64][64]: the digits of h for the integer-dot down products, left by the gate/up launch of a window
 };
 // The FFN output of a window, left unreduced for the consumer to fold.  The k expert terms (ascending id) and the shared
 // expert's form PYRE_MOE_GROUPS groups of g = (k + 4) / 4 consecutive experts, the shared expert in the last:

@@ -82,7 +82,7 @@ __device__ __forceinline__ void route_select(int n_exp, int k, RouteLds& L) {
 // The logits are given as nsl (<= 64) K-slice sums `sstride` floats apart, added in slice order (nsl == 1: the logits
 // themselves); all slices are fetched before the first add, in groups of eight behind launch-uniform branches.
 __device__ __forceinline__ void route_topk(const float* __restrict__ logits, int nsl, int sstride, int n_exp, int k, RouteLds& L ROUTE_TS_PARAM) {
-  const int e = threadIdx.x, lane = e & 63, wave = e >> 6;
+  const int e = threadIdx.x;
   if (e < n_exp) {
     float sv[64];
 #pragma unroll
@@ -140,7 +140,8 @@ __device__ __forceinline__ void route_weights(int k, RouteLds& L) {
 // multiply-add take 3; dgx holds the digits of the window's activations, token ti at dgx + ti * (d / 64) * DGX_STRIDE.
 template <int FMT, int NW, int P, bool PRE, bool FIX = false, bool ID = false>
 __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 8 : 1) void k_moe_gu(MoeDev m, const float* __restrict__ logits, int32_t* __restrict__ sel_idx, float* __restrict__ sel_w, float* __restrict__ sg,
-                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride, const uint32_t* __restrict__ dgx) {
+                                                   const float* __restrict__ x, float* __restrict__ h, int hstride, const uint2* __restrict__ g2, int nsl, int sstride, int tstride, const uint32_t* __restrict__ dgx,
+                                                   uint32_t* __restrict__ dgh) {
   static_assert(!ID || FMT == FMT_IQ3_S, "the integer form is IQ3_S's");
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
@@ -149,6 +150,7 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
   if constexpr (FIX) nsl = 32;
   __shared__ float red[2][P][NW][64];
   __shared__ RouteLds rl;
+  __shared__ uint8_t hsm[ID ? 3 : 1][64];
   const int entry = blockIdx.y, k1 = top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == top_k;
   const int nrows = shared ? m.sf : ff;
@@ -224,7 +226,10 @@ __global__ __launch_bounds__(NW * 64, (PRE && P == 2 && FMT >= 5 && FMT <= 7) ? 
     }
     if (nz == 1) {
       float s = 1.0f / (1.0f + expf(-g));
-      h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+      const float hv = (g * s) * u;      // silu(g) * u, silu(x) = x * sigm(x)
+      h[(size_t)entry * hstride + blockIdx.x * 64 + lane] = hv;
+      // the tile's 64 rows are one unit of the down product's columns: their digits for its integer form
+      if constexpr (ID) { if (dgh) digits_eo_wave(hv, lane, hsm, dgh + ((size_t)entry * (hstride >> 6) + blockIdx.x) * DGX_STRIDE); }
     } else {
       float* hp = h + ((size_t)entry * nz + kz) * 2 * hstride + blockIdx.x * 64 + lane;
       hp[0] = g; hp[hstride] = u;
@@ -261,15 +266,20 @@ __global__ __launch_bounds__(1024) void k_moe_route(MoeDev m, const float* __res
 // NZ > 1: h arrives as the gate / up sums of NZ K parts (k_moe_gu with gridDim.z = NZ); each wave forms the 64 values of
 // a unit, silu(sum of gate parts) * (sum of up parts), in its own slice of shared memory while the unit's weights are
 // on their way (a wave's shared-memory operations execute in order: no workgroup barrier).
-template <int FMT, int NW, int NZ, bool FIX = false>
+// ID (IQ3_S): the integer form of digits.h on the digits of h -- left by k_moe_gu beside h (NZ == 1), or formed here by
+// the wave that forms the unit's values (NZ > 1); the same digits either way, so a token's bits do not depend on the form.
+template <int FMT, int NW, int NZ, bool FIX = false, bool ID = false>
 __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ h, int hstride, float* __restrict__ partial,
-                                                     const uint2* __restrict__ g2) {
+                                                     const uint2* __restrict__ g2, const uint32_t* __restrict__ dgh) {
+  static_assert(!ID || FMT == FMT_IQ3_S, "the integer form is IQ3_S's");
   const uint2* lds2 = nullptr;          // no format needs a codebook in shared memory any more
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, partial);
   const int top_k = FIX ? 10 : m.top_k, d = FIX ? 2048 : m.d;          // FIX: the A3B configuration (top 10, d = 2048, routed and shared experts 512 wide), checked by the launcher
   __shared__ float red[NW][64];
-  __shared__ float hx[NZ > 1 ? NW : 1][64];
+  __shared__ float hx[(NZ > 1 && !ID) ? NW : 1][64];
+  __shared__ __align__(16) uint32_t hdg[(NZ > 1 && ID) ? NW : 1][DGX_STRIDE];
+  __shared__ uint8_t hsm[(NZ > 1 && ID) ? NW : 1][3][64];
   const int entry = blockIdx.y, k1 = top_k + 1, ti = entry / k1, j = entry % k1;
   const bool shared = j == top_k;
   const QMatDev& D = shared ? m.sh_down : m.down_e;
@@ -280,6 +290,10 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
   float acc[1] = {0.0f};
   if constexpr (NZ == 1) {
     const float* xs = h + (size_t)entry * hstride;
+    if constexpr (ID) {
+      const uint32_t* dge = dgh + (size_t)entry * (hstride >> 6) * DGX_STRIDE;
+      for (int ku = k0; ku < kend; ++ku) { UnitRaw<FMT> r = unit_load<FMT>(D, tile, ku, lane); unit_idot_iq3s(r, dge + (size_t)ku * DGX_STRIDE, acc[0]); }
+    } else
     for (int ku = k0; ku < kend; ++ku) unit_dot<FMT, 1>(D, lds2, tile, ku, lane, xs + ku * 64, 0, acc);
   } else {
     const float* hp = h + (size_t)entry * NZ * 2 * hstride + lane;
@@ -293,9 +307,15 @@ __global__ __launch_bounds__(NW * 64) void k_moe_down(MoeDev m, const int32_t* _
       for (int q = 1; q < NZ; ++q) { g += gp[q]; u += up[q]; }
       float s = 1.0f / (1.0f + expf(-g));
       __builtin_amdgcn_wave_barrier();
-      hx[wave][lane] = (g * s) * u;
-      __builtin_amdgcn_wave_barrier();
-      unit_fma<FMT, 1>(D, r, ku, lds2, lane, hx[wave], 0, acc);
+      if constexpr (ID) {
+        digits_eo_wave((g * s) * u, lane, hsm[wave], hdg[wave]);
+        __builtin_amdgcn_wave_barrier();
+        unit_idot_iq3s(r, hdg[wave], acc[0]);
+      } else {
+        hx[wave][lane] = (g * s) * u;
+        __builtin_amdgcn_wave_barrier();
+        unit_fma<FMT, 1>(D, r, ku, lds2, lane, hx[wave], 0, acc);
+      }
       __builtin_amdgcn_wave_barrier();
     }
   }
@@ -329,14 +349,16 @@ __global__ void k_moe_sum(const float* __restrict__ partial, const float* __rest
 // bit for bit what moe_out_value forms from k_moe_down's unreduced terms.  A wave's weights of all entries and its slices
 // of their activations (through its own shared memory: no workgroup barrier) are fetched before the first is used.
 // GE: entries a group can hold in this instance (3 covers top_k <= 11, PYRE_MOE_GMAX the rest) -- the register budget follows it.
-template <int FMT, int NW, int GE, bool FIX = false>
+// ID (IQ3_S): the integer form on the digits k_moe_gu left beside h, as k_moe_down<.., ID>.
+template <int FMT, int NW, int GE, bool FIX = false, bool ID = false>
 __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1) void k_moe_down_groups(MoeDev m, const int32_t* __restrict__ sel_idx, const float* __restrict__ sel_w, const float* __restrict__ sg,
-                                                            const float* __restrict__ h, int hstride, float* __restrict__ parts, const uint2* __restrict__ g2) {
+                                                            const float* __restrict__ h, int hstride, float* __restrict__ parts, const uint2* __restrict__ g2, const uint32_t* __restrict__ dgh) {
   static_assert(GE <= PYRE_MOE_GMAX, "a group holds at most PYRE_MOE_GMAX entries");
+  static_assert(!ID || FMT == FMT_IQ3_S, "the integer form is IQ3_S's");
   const uint2* lds2 = nullptr;
   qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, parts);
   __shared__ float red[GE][NW][64];
-  __shared__ float hx[NW][GE][64];
+  __shared__ float hx[ID ? 1 : NW][GE][64];
   const int ti = blockIdx.y, q = blockIdx.z, k = FIX ? 10 : m.top_k, gsz = (k + 4) / 4, d = FIX ? 2048 : m.d;          // FIX: the A3B configuration (top 10, d = 2048, experts 512 wide), checked by the launcher
   const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;          // the group's routed entries j0 .. j0+nr-1
   const bool with_shared = q == PYRE_MOE_GROUPS - 1;
@@ -345,12 +367,13 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   // the routed and the shared matrices may differ in width: each has its own K shares (as in k_moe_down)
   const int Ur = FIX ? 8 : m.down_e.U, Us = FIX ? 8 : m.sh_down.U, upr = (Ur + NW - 1) / NW, ups = (Us + NW - 1) / NW;
   const int niter = max(nr > 0 ? upr : 0, with_shared ? ups : 0);
-  int tile[GE]; const float* xs[GE];
+  int tile[GE]; const float* xs[GE]; const uint32_t* dge[GE];
 #pragma unroll
   for (int e = 0; e < GE; ++e) {
     const bool shared = with_shared && e == nr; const int j = shared ? k : min(j0 + e, k - 1);
     tile[e] = (shared ? 0 : __builtin_amdgcn_readfirstlane(sel_idx[ti * k + j]) * (d >> 6)) + blockIdx.x;
     xs[e] = h + (size_t)(ti * (k + 1) + j) * hstride;
+    dge[e] = ID ? dgh + (size_t)(ti * (k + 1) + j) * (hstride >> 6) * DGX_STRIDE : nullptr;
   }
   float acc[GE][1];
 #pragma unroll
@@ -361,15 +384,20 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
     for (int e = 0; e < GE; ++e) {
       const bool shared = with_shared && e == nr; const int up = shared ? ups : upr, U = shared ? Us : Ur;
       ku[e] = wave * up + it; on[e] = e < ne && it < up && ku[e] < U;
-      if (on[e]) { const QMatDev& D = shared ? m.sh_down : m.down_e; r[e] = unit_load<FMT>(D, tile[e], ku[e], lane); hv[e] = xs[e][ku[e] * 64 + lane]; }
+      if (on[e]) { const QMatDev& D = shared ? m.sh_down : m.down_e; r[e] = unit_load<FMT>(D, tile[e], ku[e], lane); if constexpr (!ID) hv[e] = xs[e][ku[e] * 64 + lane]; }
     }
-    __builtin_amdgcn_wave_barrier();
+    if constexpr (ID) {
 #pragma unroll
-    for (int e = 0; e < GE; ++e) if (on[e]) hx[wave][e][lane] = hv[e];
-    __builtin_amdgcn_wave_barrier();
+      for (int e = 0; e < GE; ++e) if (on[e]) unit_idot_iq3s(r[e], dge[e] + (size_t)ku[e] * DGX_STRIDE, acc[e][0]);
+    } else {
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int e = 0; e < GE; ++e) if (on[e]) { const QMatDev& D = (with_shared && e == nr) ? m.sh_down : m.down_e; unit_fma<FMT, 1>(D, r[e], ku[e], lds2, lane, hx[wave][e], 0, acc[e]); }
-    __builtin_amdgcn_wave_barrier();
+      for (int e = 0; e < GE; ++e) if (on[e]) hx[wave][e][lane] = hv[e];
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int e = 0; e < GE; ++e) if (on[e]) { const QMatDev& D = (with_shared && e == nr) ? m.sh_down : m.down_e; unit_fma<FMT, 1>(D, r[e], ku[e], lds2, lane, hx[wave][e], 0, acc[e]); }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
 #pragma unroll
   for (int e = 0; e < GE; ++e) if (e < ne) red[e][wave][lane] = acc[e][0];
@@ -401,7 +429,7 @@ __global__ __launch_bounds__(64) void k_act_digits_eo(const float* __restrict__ 
 #define PYRE_MOE_GU_NZMAX 2
 size_t pyre_moe_work_bytes(const MoeDev& m) {
   size_t hs = (size_t)(m.ff > m.sf ? m.ff : m.sf), k1 = m.top_k + 1;
-  return 256 * 10 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d + 8 * PYRE_MOE_GROUPS * (size_t)m.d + 8 * (size_t)(m.d / 64) * DGX_STRIDE);
+  return 256 * 11 + sizeof(float) * (8 * (size_t)m.n_exp + 8 * (size_t)m.top_k * 2 + 8 + 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX + 8 * k1 * (size_t)m.d + 8 * PYRE_MOE_GROUPS * (size_t)m.d + 8 * (size_t)(m.d / 64) * DGX_STRIDE + 8 * k1 * (hs / 64) * DGX_STRIDE);
 }
 void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
@@ -410,6 +438,7 @@ void pyre_moe_work_carve(const MoeDev& m, void* base, MoeWork* w) {
   w->sg = (float*)take(4 * 8); w->h = (float*)take(4 * 8 * k1 * hs * 2 * PYRE_MOE_GU_NZMAX); w->partial = (float*)take(4 * 8 * k1 * (size_t)m.d);
   w->parts = (float*)take(4 * 8 * PYRE_MOE_GROUPS * (size_t)m.d);
   w->dgx = (uint32_t*)take(4 * 8 * (size_t)(m.d / 64) * DGX_STRIDE);
+  w->dgh = (uint32_t*)take(4 * 8 * k1 * (hs / 64) * DGX_STRIDE);
 }
 
 #define MOE_FMT_DISPATCH(fmt, CALL) \
@@ -444,9 +473,13 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
     if (routed && routed->dgx) dgx = routed->dgx;
     else { ProfScope ps(ctx, "moe_digits", 4.0 * t * m.d * 2); hipLaunchKernelGGL(k_act_digits_eo, dim3(m.d / 64, t), dim3(64), 0, ctx->stream, x, m.d, w.dgx); PYRE_CHECK_LAUNCH(ctx); dgx = w.dgx; }
   }
+  // ... and the down products on the digits of h, which a window's gate/up launch leaves and a single token's down launch forms
+  static const bool idot_gu_only = getenv("PYRE_MOE_IDOT") && atoi(getenv("PYRE_MOE_IDOT")) == 1;
+  const bool idot_dn = idot && !idot_gu_only && m.down_e.fmt == FMT_IQ3_S && m.sh_down.fmt == FMT_IQ3_S;
+  uint32_t* dgh = idot_dn ? w.dgh : nullptr;
   const bool a3b = t == 1 && m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512;          // the instances with these constants folded in
   { ProfScope ps(ctx, "moe_route_gate_up", t * (2.0 * m.top_k * mat_bytes(m.gate_e, m.ff) + 2.0 * mat_bytes(m.sh_gate, m.sf)) + 4.0 * t * (m.n_exp + 2.0 * m.d));
-#define GU_ARGS(NZ) dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride, dgx
+#define GU_ARGS(NZ) dim3(hs / 64, entries, NZ), dim3(16 * 64), 0, ctx->stream, m, lg, w.sel_idx, w.sel_w, w.sg, x, w.h, hs, g2, nsl, sstride, tstride, dgx, dgh
 #define GU_GO(PP, NZ, PRE) do { if (idot) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, PP, PRE, false, true>), GU_ARGS(NZ)); else MOE_FMT_DISPATCH(m.gate_e.fmt, hipLaunchKernelGGL((k_moe_gu<F, 16, PP, PRE>), GU_ARGS(NZ))); } while (0)
   if (t == 1 && a3b && nsl == 32 && nz == 2) { if (idot) hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true, true>), GU_ARGS(2)); else hipLaunchKernelGGL((k_moe_gu<FMT_IQ3_S, 16, 1, false, true>), GU_ARGS(2)); }
   else if (t == 1) { GU_GO(1, nz, false); }          // the selection inside the launch; one workgroup per K part
@@ -463,15 +496,21 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   { ProfScope ps(ctx, "moe_down", t * (m.top_k * mat_bytes(m.down_e, m.d) + mat_bytes(m.sh_down, m.d)));
   if (in_groups) {
     const int gsz = (m.top_k + 4) / 4, last = m.top_k - min(m.top_k, (PYRE_MOE_GROUPS - 1) * gsz) + 1;          // entries of a full group, of the last (with the shared expert)
-#define DOWN_G_GO(GE) MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down_groups<F, 8, GE>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2))
-    if (m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512)          // the A3B configuration: constants folded in
-      hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, 3, true>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2);
+#define DOWN_G_GO(GE) MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down_groups<F, 8, GE>), dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2, dgh))
+#define DOWN_G_ARGS dim3(m.d / 64, t, PYRE_MOE_GROUPS), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.sel_w, w.sg, w.h, hs, w.parts, g2, dgh
+    if (m.gate_e.fmt == FMT_IQ3_S && m.down_e.fmt == FMT_IQ3_S && m.n_exp == 512 && m.top_k == 10 && m.d == 2048 && m.ff == 512 && m.sf == 512) {          // the A3B configuration: constants folded in
+      if (idot_dn) hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, 3, true, true>), DOWN_G_ARGS); else hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, 3, true>), DOWN_G_ARGS);
+    } else if (idot_dn) { if (gsz <= 3 && last <= 3) hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, 3, false, true>), DOWN_G_ARGS); else hipLaunchKernelGGL((k_moe_down_groups<FMT_IQ3_S, 8, PYRE_MOE_GMAX, false, true>), DOWN_G_ARGS); }
     else if (gsz <= 3 && last <= 3) { DOWN_G_GO(3); } else { DOWN_G_GO(PYRE_MOE_GMAX); }
+#undef DOWN_G_ARGS
 #undef DOWN_G_GO
   }
-  else if (a3b && nz == 2) hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, true>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2);
-  else if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); }
-  else { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 2>), dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2)); } }
+#define DOWN_ARGS dim3(m.d / 64, entries), dim3(8 * 64), 0, ctx->stream, m, w.sel_idx, w.h, hs, w.partial, g2, dgh
+  else if (a3b && nz == 2) { if (idot_dn) hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, true, true>), DOWN_ARGS); else hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, true>), DOWN_ARGS); }
+  else if (idot_dn) { if (nz == 1) hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 1, false, true>), DOWN_ARGS); else hipLaunchKernelGGL((k_moe_down<FMT_IQ3_S, 8, 2, false, true>), DOWN_ARGS); }
+  else if (nz == 1) { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 1>), DOWN_ARGS)); }
+  else { MOE_FMT_DISPATCH(m.down_e.fmt, hipLaunchKernelGGL((k_moe_down<F, 8, 2>), DOWN_ARGS)); } }
+#undef DOWN_ARGS
   PYRE_CHECK_LAUNCH(ctx);
   if (y) {
     ProfScope ps(ctx, "moe_sum", 4.0 * t * m.d * (m.top_k + 2));
