@@ -311,6 +311,18 @@ int   pyre_ngram_draft(const uint32_t* history, size_t len, int k, int min_n, in
  * accepted (spec::Outcome, src/spec.rs:150-154). */
 int   pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32_t* history, size_t n_hist, const float* first_logits_host,
                                  int n_out, uint32_t* out, int k, int ng_min, int ng_max, int* rounds, int* drafted, int* accepted);
+/* Adaptive draft length, spec::adapt_plan (src/spec.rs:144-152): the draft count k in 0..min(n, 8) with the best expected
+ * tokens per second relative to plain decoding, from the plain step time ts, the measured verify time tv[t] of a t-token
+ * window (tv[10]; an entry of 0 = unmeasured: ts * (1 + 0.75 (t - 1))), the running acceptance p and the drafter's time per
+ * round td.  0 = no window is expected to beat plain steps.  Host only: no context, no GPU. */
+int   pyre_adapt_plan(int n, double ts, const double* tv, double p, double td);
+/* Whether pyre_generate_greedy_ngram and pyre_generate_greedy_mtp apply that plan as spec::generate does (src/spec.rs:162-167,
+ * 186-193, 213-217): timings and acceptance tracked online, the decision taken before drafting (so a drafter that does not
+ * pay is not run either, apart from a probe window now and then) and again on what the drafter produced.  on = 1 / 0, or
+ * -1: PYRE_SPEC_ADAPT in the environment.  The reference's default is on (spec::adapt_on, src/spec.rs:34); here an unset
+ * variable means off, so that the drafted / accepted counts of a run do not depend on the clock -- a binding passes
+ * spec::adapt_on().  The generated tokens are the same either way. */
+void  pyre_spec_set_adapt(pyre_ctx* ctx, int on);
 /* ---- the multi-token-prediction (MTP) drafter: src/model/mtp.rs, Model::mtp_draft (src/model/qwen4exp_gguf.rs:2180-2277) ----
  * One extra block that pairs the main model's final residual streams R_i with the token at position i + 1 (cell i, rope
  * position i, the unscaled table) and predicts token i + 2: pre-norms and two d x d matrices form its streams, then
@@ -338,6 +350,24 @@ typedef struct pyre_mtp pyre_mtp;
 int   pyre_mtp_create(pyre_ctx* ctx, const pyre_model* main, const pyre_mtp_cfg* cfg, const pyre_tensor* tensors /*[PYRE_MTP_SLOTS]*/,
                       const uint32_t* draft_ids /*[n_draft_vocab], host*/, pyre_mtp** out);
 void  pyre_mtp_destroy(pyre_mtp* m);
+/* The drafter's checkpoint file: the safetensors reader of src/model/mtp.rs:24-50 (St::open / raw).  An 8-byte header
+ * length, a JSON header, BF16 tensors only (anything else: PYRE_E_TYPE); names have their "mtp." and "layers.0." prefixes
+ * trimmed.  Host only.  pyre_st_tensor: *data points into the mapping (valid until pyre_st_close), dims[8] / *n_dims
+ * (optional) receive the shape. */
+typedef struct pyre_st pyre_st;
+int    pyre_st_open(const char* path, pyre_st** out, char* err, size_t err_cap);
+void   pyre_st_close(pyre_st* s);
+size_t pyre_st_n_tensors(const pyre_st* s);
+const char* pyre_st_tensor_name(const pyre_st* s, size_t i);            /* file (header) order */
+int    pyre_st_tensor(const pyre_st* s, const char* name, const void** data, uint32_t* n_dims, uint64_t* dims, char* err, size_t err_cap);
+/* Mtp::load (src/model/mtp.rs:99-118): the drafter from that file.  Tensor names as the reference reads them; norm vectors
+ * become 1 + w; mlp.experts.gate_up_proj [experts][2 ff][d] is split into gate (rows 0 .. ff of an expert) and up; experts
+ * and width come from mlp.experts.down_proj [experts][d][ff]; matrices stay BF16 (the reference re-quantizes them to int8).
+ * top_k: experts per token, capped by the main model's (PYRE_MTP_TOPK; 0 = the main model's); window: 0 = 128
+ * (PYRE_MTP_WINDOW); head: the draft head [n_draft_vocab][d] in any supported type, or NULL = rows draft_ids of the main
+ * model's output matrix dequantized to f32. */
+int   pyre_mtp_load_safetensors(pyre_ctx* ctx, const pyre_model* main, const char* path, int top_k, int window,
+                                const uint32_t* draft_ids, int n_draft_vocab, const pyre_tensor* head, pyre_mtp** out);
 /* From now on every forward call leaves the final residual streams of its last `window` tokens in a ring on the device
  * (mtp_keep_r, qwen4exp_gguf.rs:2279-2285: window + 16 positions are kept) and the state owns the drafter's K/V cells.
  * Snapshots do not carry either: after pyre_state_restore the drafter starts over (no drafts until a forward call has

@@ -3,6 +3,7 @@
 // greedy loop.  Follows Model::forward_inner / forward_multi / spec_keep (src/model/qwen4exp_gguf.rs:2087-2157,
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
+#include <chrono>
 #include <memory>
 #include <stdlib.h>
 
@@ -782,7 +783,48 @@ int pyre_decode_greedy_dev(pyre_ctx* ctx, const pyre_model* mc, pyre_state* s, u
   return PYRE_OK;
 }
 
+// Adaptive draft length of spec::generate (src/spec.rs:162-167, 186-193, 213-217, 221, 229, 258): the plain step time ts and the
+// verify time tv[t] of a t-token window as running means, the running acceptance p_acc, the drafter's time per round td_avg.
+// Before drafting the plan picks the draft count (0 = a plain step; now and then a probe window of at most two drafts so the
+// estimates can recover); after drafting the most profitable prefix of what the drafter produced is kept.  Nothing
+// happens before the first plain step has been timed.  It only chooses which drafts are verified: the output is unchanged.
+struct SpecAdapt {
+  bool on = false; double ts = 0, tv[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, p_acc = 0.7, td_avg = 0; int skipped = 0; bool probe = false;
+  std::chrono::steady_clock::time_point t0;
+  explicit SpecAdapt(const pyre_ctx* ctx) { const char* e = getenv("PYRE_SPEC_ADAPT"); on = ctx->spec_adapt >= 0 ? ctx->spec_adapt != 0 : (e && *e && strcmp(e, "0") != 0); }
+  void tick() { t0 = std::chrono::steady_clock::now(); }
+  double tock() const { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count(); }
+  int plan(int kk) {
+    probe = false;
+    if (!on || kk <= 0 || ts <= 0.0) return kk;
+    const int bk = pyre_adapt_plan(kk, ts, tv, p_acc, td_avg);
+    bool none = true; for (int t = 2; t < 10; ++t) if (tv[t] != 0.0) none = false;
+    const int every = none ? 2 : 24;            // sooner while no window has been timed yet
+    if (bk > 0) { skipped = 0; return bk; }
+    if (skipped >= every) { skipped = 0; probe = true; return kk < 2 ? kk : 2; }
+    ++skipped; return 0;
+  }
+  int trim(int nd) const { return (on && !probe && nd > 0 && ts > 0.0) ? pyre_adapt_plan(nd, ts, tv, p_acc, 0.0) : nd; }
+  void drafted(double dt) { td_avg = td_avg == 0.0 ? dt : 0.8 * td_avg + 0.2 * dt; }
+  void plain(double dt) { ts = ts == 0.0 ? dt : 0.8 * ts + 0.2 * dt; }
+  void verified(int t, double dt) { tv[t] = tv[t] == 0.0 ? dt : 0.7 * tv[t] + 0.3 * dt; }
+  void accepted(int acc, int nd) { p_acc = 0.7 * p_acc + 0.3 * ((double)acc / (double)nd); }
+};
+
 static uint32_t host_argmax(const float* l, size_t n) { size_t b = 0; for (size_t i = 1; i < n; ++i) if (l[i] > l[b]) b = i; return (uint32_t)b; }
+
+int pyre_adapt_plan(int n, double ts, const double* tv, double p, double td) {            // spec::adapt_plan, src/spec.rs:147-152
+  if (!tv) return 0;
+  double best = 1.0, e = 1.0, pp = 1.0; int bk = 0;
+  for (int kq = 1; kq <= (n < 8 ? n : 8); ++kq) {
+    pp *= p; e += pp;
+    const double est = tv[kq + 1] > 0.0 ? tv[kq + 1] : ts * (1.0 + 0.75 * ((double)(kq + 1) - 1.0));
+    const double g = e * ts / (est + td);
+    if (g > best) { best = g; bk = kq; }
+  }
+  return bk;
+}
+void pyre_spec_set_adapt(pyre_ctx* ctx, int on) { if (ctx) ctx->spec_adapt = on < 0 ? -1 : (on != 0); }
 
 int pyre_generate_greedy(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const float* first_logits, int n_out, uint32_t* out, int n_draft, const uint32_t* draft_stream, int* rounds_out) {
   if (!ctx || !m || !s || !first_logits || !out || n_out < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy: bad argument");
@@ -847,18 +889,20 @@ int pyre_generate_greedy_ngram(pyre_ctx* ctx, const pyre_model* m, pyre_state* s
   if (k < 1 || k > 7 || ng_min < 1 || ng_max < ng_min) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_ngram: k %d (1..7), n-gram lengths %d..%d", k, ng_min, ng_max);
   const size_t V = m->c.vocab; int produced = 0, rounds = 0, drafted = 0, accepted = 0;
   std::vector<uint32_t> hist(history, history + n_hist); hist.reserve(n_hist + (size_t)n_out + 8);
+  SpecAdapt ad(ctx);
   uint32_t pending = host_argmax(first_logits, V);
   for (;;) {
     hist.push_back(pending); out[produced++] = pending; if (produced >= n_out) break;
-    const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
+    const int left = n_out - produced; const int kk = ad.plan(k < left - 1 ? k : left - 1);
     uint32_t toks[8]; toks[0] = pending;
-    const int nd = kk > 0 ? pyre_ngram_draft(hist.data(), hist.size(), kk, ng_min, ng_max, toks + 1) : 0;
-    if (nd == 0) { uint32_t pk; int rc = forward_multi_picks(ctx, m, s, &pending, 1, &pk); if (rc) return rc; pending = pk; continue; }
-    uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
+    const int nd = ad.trim(kk > 0 ? pyre_ngram_draft(hist.data(), hist.size(), kk, ng_min, ng_max, toks + 1) : 0);
+    if (nd == 0) { uint32_t pk; ad.tick(); int rc = forward_multi_picks(ctx, m, s, &pending, 1, &pk); if (rc) return rc; ad.plain(ad.tock()); pending = pk; continue; }
+    uint32_t picks[8]; ad.tick(); int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc; ad.verified(nd + 1, ad.tock());
     int acc = 0; bool have = false; uint32_t nx = 0;
     for (int i = 0; i < nd; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
     if (!have) nx = picks[nd];
     if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
+    ad.accepted(acc, nd);
     ++rounds; drafted += nd; accepted += acc;
     bool stop = false; for (int i = 0; i < acc; ++i) { hist.push_back(toks[i + 1]); out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
     if (stop) break;
@@ -1011,6 +1055,65 @@ int pyre_mtp_create(pyre_ctx* ctx, const pyre_model* main, const pyre_mtp_cfg* c
   guard.armed = false; *out = M.release(); return PYRE_OK;
 }
 
+// Mtp::load (src/model/mtp.rs:99-118) from the one-file BF16 checkpoint: tensor names as the reference reads them, norm
+// vectors as 1 + w, the fused mlp.experts.gate_up_proj [experts][2 ff][d] split into its gate (rows 0 .. ff of an expert)
+// and up (rows ff .. 2 ff) halves, experts and width from mlp.experts.down_proj [experts][d][ff]; the matrices stay BF16
+// (the reference re-quantizes them to int8 at load, mtp.rs:11-13).  head == NULL: the draft head is the rows draft_ids
+// of the main model's output matrix, dequantized exactly (f32).
+int pyre_mtp_load_safetensors(pyre_ctx* ctx, const pyre_model* main, const char* path, int top_k, int window, const uint32_t* draft_ids, int n_draft_vocab, const pyre_tensor* head, pyre_mtp** out) {
+  if (!ctx || !main || !path || !draft_ids || !out || n_draft_vocab < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_load_safetensors: bad argument");
+  *out = nullptr; const pyre_model_cfg& c = main->c;
+  char err[512] = {0}; pyre_st* st = nullptr;
+  int rc = pyre_st_open(path, &st, err, sizeof err); if (rc) return pyre_fail(ctx, rc, "pyre_mtp_load_safetensors: %s", err);
+  struct Closer { pyre_st* s; ~Closer() { pyre_st_close(s); } } closer{st};
+  std::vector<std::vector<float>> f32s; std::vector<std::vector<uint16_t>> halves; f32s.reserve(16); halves.reserve(4);
+  pyre_tensor T[PYRE_MTP_SLOTS]; memset(T, 0, sizeof T);
+  auto raw = [&](const std::string& n, const uint16_t** d, std::vector<uint64_t>* sh) { const void* p; uint32_t nd; uint64_t dims[8]; int r = pyre_st_tensor(st, n.c_str(), &p, &nd, dims, err, sizeof err);
+    if (r) return pyre_fail(ctx, r, "pyre_mtp_load_safetensors: %s", err); *d = (const uint16_t*)p; sh->assign(dims, dims + nd); return (int)PYRE_OK; };
+  auto mat = [&](int slot, const std::string& n) { const uint16_t* d; std::vector<uint64_t> sh; int r = raw(n, &d, &sh); if (r) return r;
+    if (sh.size() != 2) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_mtp_load_safetensors: %s is not a matrix", n.c_str());
+    T[slot] = pyre_tensor{PYRE_BF16, 0, sh[0], sh[1], d}; return (int)PYRE_OK; };
+  auto vec = [&](int slot, const std::string& n, float add) { const uint16_t* d; std::vector<uint64_t> sh; int r = raw(n, &d, &sh); if (r) return r;
+    uint64_t cnt = 1; for (uint64_t v : sh) cnt *= v;
+    f32s.emplace_back((size_t)cnt); std::vector<float>& y = f32s.back();
+    for (size_t i = 0; i < (size_t)cnt; ++i) { const uint32_t u = (uint32_t)d[i] << 16; float f; memcpy(&f, &u, 4); y[i] = f + add; }            // St::row, St::norm
+    T[slot] = pyre_tensor{PYRE_F32, 0, 1, cnt, y.data()}; return (int)PYRE_OK; };
+  if ((rc = vec(PYRE_MTP_PRE_E, "pre_fc_norm_embedding.weight", 1.0f)) || (rc = vec(PYRE_MTP_PRE_H, "pre_fc_norm_hidden.weight", 1.0f)) ||
+      (rc = mat(PYRE_MTP_FC_E, "fc_embedding.weight")) || (rc = mat(PYRE_MTP_FC_H, "fc_hidden.weight"))) return rc;
+  const struct { const char* p; int norm, down, inject, up; } hcs[3] = {{"attn_hyper_connection", PYRE_MTP_HCA_NORM, PYRE_MTP_HCA_DOWN, PYRE_MTP_HCA_INJECT, PYRE_MTP_HCA_UP},
+    {"mlp_hyper_connection", PYRE_MTP_HCF_NORM, PYRE_MTP_HCF_DOWN, PYRE_MTP_HCF_INJECT, PYRE_MTP_HCF_UP}, {"hyper_connection_mixer", PYRE_MTP_MIX_NORM, PYRE_MTP_MIX_DOWN, -1, PYRE_MTP_MIX_UP}};
+  for (const auto& h : hcs) { const std::string b = h.p;
+    if ((rc = vec(h.norm, b + ".hc_norm.weight", 1.0f)) || (rc = mat(h.down, b + ".input_mix_weight_down.weight")) || (rc = mat(h.up, b + ".input_mix_weight_up.weight"))) return rc;
+    if (h.inject >= 0 && (rc = mat(h.inject, b + ".block_inject_weight.weight"))) return rc; }
+  if ((rc = mat(PYRE_MTP_Q, "self_attn.q_proj.weight")) || (rc = mat(PYRE_MTP_K, "self_attn.k_proj.weight")) || (rc = mat(PYRE_MTP_V, "self_attn.v_proj.weight")) || (rc = mat(PYRE_MTP_O, "self_attn.o_proj.weight")) ||
+      (rc = vec(PYRE_MTP_QN, "self_attn.q_norm.weight", 1.0f)) || (rc = vec(PYRE_MTP_KN, "self_attn.k_norm.weight", 1.0f)) ||
+      (rc = mat(PYRE_MTP_ROUTER, "mlp.gate.weight")) || (rc = mat(PYRE_MTP_SH_GATE, "mlp.shared_expert.gate_proj.weight")) || (rc = mat(PYRE_MTP_SH_UP, "mlp.shared_expert.up_proj.weight")) ||
+      (rc = mat(PYRE_MTP_SH_DOWN, "mlp.shared_expert.down_proj.weight")) || (rc = vec(PYRE_MTP_SH_GATE_INP, "mlp.shared_expert_gate.weight", 0.0f))) return rc;
+  const uint16_t *gu, *dn; std::vector<uint64_t> sg, sd;
+  if ((rc = raw("mlp.experts.gate_up_proj", &gu, &sg)) || (rc = raw("mlp.experts.down_proj", &dn, &sd))) return rc;
+  if (sd.size() != 3 || sg.size() != 3 || sg[0] != sd[0] || sg[1] != 2 * sd[2] || sg[2] != sd[1] || sd[1] != (uint64_t)c.d)
+    return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_mtp_load_safetensors: mlp.experts.gate_up_proj / down_proj are not [experts][2 ff][d] / [experts][d][ff]");
+  const size_t ne = (size_t)sd[0], ff = (size_t)sd[2], d = (size_t)c.d;            // mtp.rs:104
+  halves.emplace_back(ne * ff * d); halves.emplace_back(ne * ff * d);
+  for (size_t e = 0; e < ne; ++e) { memcpy(halves[0].data() + e * ff * d, gu + e * 2 * ff * d, ff * d * 2); memcpy(halves[1].data() + e * ff * d, gu + (e * 2 + 1) * ff * d, ff * d * 2); }
+  T[PYRE_MTP_GATE_E] = pyre_tensor{PYRE_BF16, 0, ne * ff, d, halves[0].data()}; T[PYRE_MTP_UP_E] = pyre_tensor{PYRE_BF16, 0, ne * ff, d, halves[1].data()};
+  T[PYRE_MTP_DOWN_E] = pyre_tensor{PYRE_BF16, 0, ne * d, ff, dn};
+  float* head_dev = nullptr; uint32_t* ids_dev = nullptr;
+  struct Free { float** a; uint32_t** b; ~Free() { if (*a) (void)hipFree(*a); if (*b) (void)hipFree(*b); } } fr{&head_dev, &ids_dev};
+  if (head) T[PYRE_MTP_HEAD] = *head;
+  else {            // Q8Mat::from_fn(ids.len(), d, head_row(ids[r])), mtp.rs:106, without the int8 step
+    for (int i = 0; i < n_draft_vocab; ++i) if (draft_ids[i] >= (uint32_t)c.vocab) return pyre_fail(ctx, PYRE_E_ARG, "pyre_mtp_load_safetensors: draft id %u outside the vocabulary (%d)", draft_ids[i], c.vocab);
+    PYRE_HIP(ctx, hipSetDevice(ctx->device));
+    PYRE_HIP(ctx, hipMalloc((void**)&head_dev, (size_t)n_draft_vocab * d * 4)); PYRE_HIP(ctx, hipMalloc((void**)&ids_dev, (size_t)n_draft_vocab * 4));
+    PYRE_HIP(ctx, hipMemcpy(ids_dev, draft_ids, (size_t)n_draft_vocab * 4, hipMemcpyHostToDevice));
+    for (int r0 = 0; r0 < n_draft_vocab; r0 += 32768) { const int nr = std::min(32768, n_draft_vocab - r0); if ((rc = pyre_row_launch(ctx, main->out, ids_dev + r0, nr, head_dev + (size_t)r0 * d, (int)d))) return rc; }
+    PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    T[PYRE_MTP_HEAD] = pyre_tensor{PYRE_F32, 1, (uint64_t)n_draft_vocab, (uint64_t)d, head_dev};
+  }
+  pyre_mtp_cfg cfg{(int32_t)ne, top_k > 0 ? std::min(top_k, c.top_k) : c.top_k, (int32_t)ff, window > 0 ? window : 128, n_draft_vocab};            // PYRE_MTP_TOPK capped by the model's, PYRE_MTP_WINDOW 128: mtp.rs:108,117
+  return pyre_mtp_create(ctx, main, &cfg, T, draft_ids, out);
+}
+
 void pyre_mtp_destroy(pyre_mtp* m) {
   if (!m) return; (void)hipSetDevice(m->ctx->device); (void)hipStreamSynchronize(m->ctx->stream);
   for (auto q : m->shell.owned) pyre_qmat_destroy(q); for (auto b : m->shell.bufs) (void)hipFree(b); if (m->work) (void)hipFree(m->work);
@@ -1117,18 +1220,22 @@ static int generate_greedy_mtp(pyre_ctx* ctx, const pyre_model* m, const pyre_mt
   if (k < 1 || k > 7) return pyre_fail(ctx, PYRE_E_ARG, "pyre_generate_greedy_mtp: k %d outside 1..7", k);
   if (s->mtp != mtp) return pyre_fail(ctx, PYRE_E_STATE, "pyre_generate_greedy_mtp: this drafter is not attached to the state");
   const size_t V = m->c.vocab; int produced = 0, rounds = 0, drafted = 0, accepted = 0;
+  SpecAdapt ad(ctx); if (forced) ad.on = false;
   uint32_t pending = host_argmax(first_logits, V);
   for (;;) {
     out[produced++] = pending; if (produced >= n_out) break;
-    const int left = n_out - produced; const int kk = k < left - 1 ? k : left - 1;
+    const int left = n_out - produced; const int kk = ad.plan(k < left - 1 ? k : left - 1);
     uint32_t toks[8]; float ps[8]; toks[0] = pending; int nd = 0;
-    if (kk > 0) { int rc = pyre_mtp_draft(ctx, mtp, s, pending, kk, min_p, toks + 1, ps, &nd); if (rc) return rc; }
+    if (kk > 0) { ad.tick(); int rc = pyre_mtp_draft(ctx, mtp, s, pending, kk, min_p, toks + 1, ps, &nd); if (rc) return rc; ad.drafted(ad.tock()); }
     if (forced && kk > 0) { nd = kk; for (int j = 0; j < kk; ++j) toks[j + 1] = forced[produced + j]; }
-    uint32_t picks[8]; int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
+    nd = ad.trim(nd);
+    uint32_t picks[8]; ad.tick(); int rc = forward_multi_picks(ctx, m, s, toks, nd + 1, picks); if (rc) return rc;
+    if (nd == 0) ad.plain(ad.tock()); else ad.verified(nd + 1, ad.tock());
     int acc = 0; bool have = false; uint32_t nx = 0;
     for (int i = 0; i < nd; ++i) { uint32_t tk = picks[i]; if (tk == toks[i + 1]) { ++acc; continue; } nx = tk; have = true; break; }
     if (!have) nx = picks[nd];
     if ((rc = pyre_spec_keep(ctx, m, s, nd + 1, acc + 1))) return rc;
+    if (nd > 0) ad.accepted(acc, nd);
     if (nd > 0) ++rounds; drafted += nd; accepted += acc;
     bool stop = false; for (int i = 0; i < acc; ++i) { out[produced++] = toks[i + 1]; if (produced >= n_out) { stop = true; break; } }
     if (stop) break;

@@ -123,6 +123,14 @@ def _declare(L):
         "pyre_mtp_read_kv": (i32, [vp, vp, C.POINTER(i32), C.POINTER(i32), vp, vp]),
         "pyre_generate_greedy_mtp": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, f32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
         "pyre_generate_greedy_mtp_forced": (i32, [vp, vp, vp, vp, vp, i32, vp, i32, vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32)]),
+        "pyre_adapt_plan": (i32, [i32, C.c_double, vp, C.c_double, C.c_double]),
+        "pyre_spec_set_adapt": (None, [vp, i32]),
+        "pyre_st_open": (i32, [C.c_char_p, C.POINTER(vp), C.c_char_p, C.c_size_t]),
+        "pyre_st_close": (None, [vp]),
+        "pyre_st_n_tensors": (C.c_size_t, [vp]),
+        "pyre_st_tensor_name": (C.c_char_p, [vp, C.c_size_t]),
+        "pyre_st_tensor": (i32, [vp, C.c_char_p, C.POINTER(vp), C.POINTER(u32), vp, C.c_char_p, C.c_size_t]),
+        "pyre_mtp_load_safetensors": (i32, [vp, vp, C.c_char_p, i32, i32, vp, i32, vp, C.POINTER(vp)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -156,6 +164,39 @@ def ngram_draft(history, k, min_n, max_n):
     return out[:n].copy()
 
 
+def adapt_plan(n, ts, tv, p, td):
+    """spec::adapt_plan through the library (host only, needs no GPU); tv: ten verify times, 0 = unmeasured."""
+    t = np.ascontiguousarray(tv, dtype=np.float64); assert t.size == 10
+    return int(load().pyre_adapt_plan(n, ts, t.ctypes.data_as(C.c_void_p), p, td))
+
+
+class Safetensors:
+    """The drafter checkpoint's container (St of src/model/mtp.rs) through the library (host only, needs no GPU)."""
+
+    def __init__(self, path):
+        self.L = load(); h = C.c_void_p(); err = C.create_string_buffer(512)
+        rc = self.L.pyre_st_open(os.fsencode(path), C.byref(h), err, 512)
+        if rc != 0:
+            raise PyreError("pyre_st_open (%d): %s" % (rc, err.value.decode()))
+        self.h = h; self.rc = rc
+
+    def names(self):
+        return [self.L.pyre_st_tensor_name(self.h, i).decode() for i in range(self.L.pyre_st_n_tensors(self.h))]
+
+    def tensor(self, name):
+        """(shape, raw bf16 bits as a uint16 array)"""
+        d = C.c_void_p(); nd = C.c_uint32(); dims = (C.c_uint64 * 8)(); err = C.create_string_buffer(512)
+        rc = self.L.pyre_st_tensor(self.h, name.encode(), C.byref(d), C.byref(nd), dims, err, 512)
+        if rc != 0:
+            raise PyreError("pyre_st_tensor (%d): %s" % (rc, err.value.decode()))
+        shape = [int(dims[i]) for i in range(nd.value)]; n = int(np.prod(shape)) if shape else 1
+        return shape, np.ctypeslib.as_array(C.cast(d, C.POINTER(C.c_uint16)), shape=(n,)).copy()
+
+    def close(self):
+        if self.h:
+            self.L.pyre_st_close(self.h); self.h = None
+
+
 def _ptr(a):
     if a is None:
         return None
@@ -183,6 +224,10 @@ class Context:
 
     def sync(self):
         self.check(self.L.pyre_ctx_sync(self.h), "sync")
+
+    def set_spec_adapt(self, on):
+        """Adaptive draft length of the drafted greedy loops (spec::adapt_on): 1 / 0, or -1 = PYRE_SPEC_ADAPT."""
+        self.L.pyre_spec_set_adapt(self.h, int(on))
 
     @property
     def stream(self):
@@ -724,6 +769,19 @@ class Mtp:
         h = C.c_void_p()
         ctx.check(ctx.L.pyre_mtp_create(ctx.h, model.h, C.byref(self.cfg), ts, _ptr(ids), C.byref(h)), "mtp_create")
         self.h = h
+
+    @classmethod
+    def from_safetensors(cls, model, path, draft_ids, top_k=0, window=0, head=None):
+        """Mtp::load: the drafter from its one-file BF16 checkpoint; head = (ty, rows, cols, data) or None (rows of the
+        main model's output matrix, f32)."""
+        self = cls.__new__(cls); self.m = model; ctx = model.ctx
+        ids = np.ascontiguousarray(draft_ids, dtype=np.uint32); hd = None; keep = None
+        if head is not None:
+            ty, rows, cols, data = head; keep = np.ascontiguousarray(data); hd = C.byref(TensorDesc(ty, 0, rows, cols, keep.ctypes.data))
+        h = C.c_void_p()
+        ctx.check(ctx.L.pyre_mtp_load_safetensors(ctx.h, model.h, os.fsencode(path), top_k, window, _ptr(ids), ids.size, hd, C.byref(h)), "mtp_load_safetensors")
+        self.h = h; self.cfg = MtpCfg(0, top_k, 0, window or 128, ids.size)
+        return self
 
     def attach(self, st):
         self.m.ctx.check(self.m.ctx.L.pyre_state_attach_mtp(self.m.ctx.h, st.h, self.h), "state_attach_mtp")

@@ -94,3 +94,19 @@ def orc_mtp(om, mt, n_exp, top_k, ff, window, draft_ids):
     """The oracle's drafter over a modelgen.build_mtp_host tensor dict."""
     ts = [orc_tensor(mt[s]) if s in mt else orc.Tensor(0, 0, 0, None) for s in range(mg.MTP_SLOTS)]
     return orc.Mtp(om, n_exp, top_k, ff, window, ts, draft_ids, keep=(mt,))
+
+
+def write_safetensors(path, tensors, meta=None, dtype="BF16"):
+    """A safetensors file of 16-bit tensors given as uint16 arrays (name -> array), in dict order."""
+    import json
+    hdr = {}; off = 0; blobs = []
+    if meta is not None:
+        hdr["__metadata__"] = meta
+    for name, arr in tensors.items():
+        b = np.ascontiguousarray(arr, dtype=np.uint16).tobytes()
+        hdr[name] = {"dtype": dtype, "shape": list(arr.shape), "data_offsets": [off, off + len(b)]}; off += len(b); blobs.append(b)
+    h = json.dumps(hdr).encode(); h += b" " * (-len(h) % 8)
+    with open(path, "wb") as f:
+        f.write(len(h).to_bytes(8, "little")); f.write(h)
+        for b in blobs:
+            f.write(b)

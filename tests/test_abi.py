@@ -4,6 +4,7 @@ import os
 
 import pytest
 
+import helpers
 from pyre_amd import lib
 
 
@@ -50,6 +51,81 @@ def test_ngram_drafter_reference_vectors_and_brute_force():
     for _ in range(300):
         h = g.integers(0, 4, int(g.integers(1, 40))).tolist(); k = int(g.integers(0, 6)); lo = int(g.integers(1, 4)); hi = lo + int(g.integers(0, 5))
         assert lib.ngram_draft(h, k, lo, hi).tolist() == brute(h, k, lo, hi), (h, k, lo, hi)
+
+
+def test_adapt_plan_reference_vectors_and_brute_force():
+    # the reference's own test (src/spec.rs:362-370)
+    tv = [0.0] * 10
+    assert lib.adapt_plan(2, 0.1, tv, 0.7, 0.0) == 0            # a 2-token verify at 1.75 plain steps with 70 % acceptance does not pay
+    tv2 = list(tv); tv2[2] = 0.12; tv2[3] = 0.14
+    assert lib.adapt_plan(2, 0.1, tv2, 0.75, 0.0) >= 1
+    assert lib.adapt_plan(2, 0.1, tv2, 0.75, 0.1) == 0          # a draft cost as large as a plain step kills it again
+    # values worked out from the definition: gain(k) = (1 + p + .. + p^k) ts / (tv[k + 1] + td), best k with gain > 1, first on ties
+    assert lib.adapt_plan(2, 0.1, tv2, 0.75, 0.0) == 2          # 1.75 / 1.2 = 1.458 < (1.75 + 0.5625) / 1.4 = 1.652
+    assert lib.adapt_plan(1, 0.1, tv2, 0.75, 0.0) == 1
+    assert lib.adapt_plan(3, 1.0, tv, 1.0, 0.0) == 3            # unmeasured windows: (k + 1) / (1 + 0.75 k) = 1.143, 1.2, 1.231
+    assert lib.adapt_plan(9, 1.0, tv, 1.0, 0.0) == 8            # never more than eight drafts
+    assert lib.adapt_plan(3, 1.0, tv, 0.0, 0.0) == 0 and lib.adapt_plan(0, 1.0, tv, 1.0, 0.0) == 0
+    import numpy as np
+    g = np.random.Generator(np.random.PCG64(11))
+
+    def brute(n, ts, tv, p, td):
+        best, bk = 1.0, 0
+        for k in range(1, min(n, 8) + 1):
+            e = sum(p ** i for i in range(k + 1))
+            est = tv[k + 1] if tv[k + 1] > 0 else ts * (1 + 0.75 * k)
+            gain = e * ts / (est + td)
+            if gain > best * (1 + 1e-12):
+                best, bk = gain, k
+        return bk
+    for _ in range(500):
+        n = int(g.integers(0, 10)); ts = float(g.uniform(0.001, 0.1)); p = float(g.uniform(0, 1)); td = float(g.uniform(0, 0.02))
+        tv = [0.0] * 10
+        for t in range(2, 10):
+            if g.random() < 0.6:
+                tv[t] = ts * float(g.uniform(0.8, 3.0))
+        got = lib.adapt_plan(n, ts, tv, p, td)
+        assert 0 <= got <= min(n, 8)
+        # the brute force sums the series afresh (the library accumulates it): accept either side of a numerical tie
+        want = brute(n, ts, tv, p, td)
+        if got != want:
+            def gain(k):
+                e = sum(p ** i for i in range(k + 1)); est = tv[k + 1] if tv[k + 1] > 0 else ts * (1 + 0.75 * k); return e * ts / (est + td) if k else 1.0
+            assert abs(gain(got) - gain(want)) <= 1e-9 * gain(want), (n, ts, tv, p, td, got, want)
+
+
+def test_safetensors_reader_names_shapes_bytes_and_errors(tmp_path):
+    import numpy as np
+    g = np.random.Generator(np.random.PCG64(5))
+    ts = {"mtp.layers.0.self_attn.q_proj.weight": g.integers(0, 65536, (6, 4), dtype=np.uint16),
+          "mtp.fc_embedding.weight": g.integers(0, 65536, (4, 4), dtype=np.uint16),
+          "mtp.layers.0.mlp.experts.down_proj": g.integers(0, 65536, (3, 4, 2), dtype=np.uint16),
+          "plain \"quoted\" \u00e9 name": g.integers(0, 65536, (5,), dtype=np.uint16)}
+    p = str(tmp_path / "mtp.safetensors")
+    helpers.write_safetensors(p, ts, meta={"format": "pt", "nested": {"a": [1, 2, {"b": None}], "c": True}})
+    st = lib.Safetensors(p)
+    assert st.names() == ["self_attn.q_proj.weight", "fc_embedding.weight", "mlp.experts.down_proj", 'plain "quoted" \u00e9 name']      # prefixes trimmed (mtp.rs:37)
+    for k, a in ts.items():
+        nm = k.replace("mtp.", "", 1).replace("layers.0.", "", 1)
+        shape, bits = st.tensor(nm)
+        assert shape == list(a.shape) and np.array_equal(bits, a.reshape(-1))
+    with pytest.raises(lib.PyreError, match="mtp tensor nope"):
+        st.tensor("nope")
+    st.close()
+    # anything but BF16 is refused (mtp.rs:34); offsets that do not match the shape, a header longer than the file
+    helpers.write_safetensors(p, {"a": np.zeros((2, 2), dtype=np.uint16)}, dtype="F16")
+    with pytest.raises(lib.PyreError, match="dtype F16"):
+        lib.Safetensors(p)
+    import json
+    h = json.dumps({"a": {"dtype": "BF16", "shape": [2, 3], "data_offsets": [0, 8]}}).encode()
+    open(p, "wb").write(len(h).to_bytes(8, "little") + h + b"\0" * 12)
+    with pytest.raises(lib.PyreError, match="data_offsets"):
+        lib.Safetensors(p)
+    open(p, "wb").write((1 << 40).to_bytes(8, "little") + b"{}")
+    with pytest.raises(lib.PyreError, match="header length"):
+        lib.Safetensors(p)
+    with pytest.raises(lib.PyreError, match="open"):
+        lib.Safetensors(str(tmp_path / "missing.safetensors"))
 
 
 def test_create_without_gpu_fails_loudly_not_silently():

@@ -233,3 +233,94 @@ def test_drafter_beside_a_model_with_per_layer_ngram_embeddings(ctx):
     assert np.array_equal(out, plain)
     for o in (gd, gs, s0, s1, gm):
         o.close()
+
+
+def test_drafter_loaded_from_its_safetensors_checkpoint_equals_the_drafter_given_the_same_tensors(ctx, tmp_path):
+    """Mtp::load (mtp.rs:99-118): names with their prefixes, norms as 1 + w, the fused gate_up_proj split per expert."""
+    import copy
+    c = small_cfg(qtype=synth.IQ3_S, hc_type=synth.BF16)
+    hw = mg.build_host(c, seed=101)
+    cd = copy.copy(c); cd.qtype = synth.BF16; cd.router_type = synth.BF16
+    mt = mg.build_mtp_host(cd, hw, N_EXP, FF, DRAFT_IDS, seed=111)
+
+    def bf16_bits(x):      # round to nearest even, as numpy has no bf16
+        u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+    def f32_of(bits):
+        return (bits.astype(np.uint32) << 16).view(np.float32)
+    names = {mg.MTP_PRE_E: "mtp.pre_fc_norm_embedding.weight", mg.MTP_PRE_H: "mtp.pre_fc_norm_hidden.weight", mg.MTP_FC_E: "mtp.fc_embedding.weight", mg.MTP_FC_H: "mtp.fc_hidden.weight",
+             mg.MTP_Q: "mtp.layers.0.self_attn.q_proj.weight", mg.MTP_K: "mtp.layers.0.self_attn.k_proj.weight", mg.MTP_V: "mtp.layers.0.self_attn.v_proj.weight",
+             mg.MTP_O: "mtp.layers.0.self_attn.o_proj.weight", mg.MTP_QN: "mtp.layers.0.self_attn.q_norm.weight", mg.MTP_KN: "mtp.layers.0.self_attn.k_norm.weight",
+             mg.MTP_ROUTER: "mtp.layers.0.mlp.gate.weight", mg.MTP_SH_GATE_INP: "mtp.layers.0.mlp.shared_expert_gate.weight", mg.MTP_SH_GATE: "mtp.layers.0.mlp.shared_expert.gate_proj.weight",
+             mg.MTP_SH_UP: "mtp.layers.0.mlp.shared_expert.up_proj.weight", mg.MTP_SH_DOWN: "mtp.layers.0.mlp.shared_expert.down_proj.weight"}
+    for base, pre, inj in ((mg.MTP_HCA_NORM, "attn_hyper_connection", True), (mg.MTP_HCF_NORM, "mlp_hyper_connection", True), (mg.MTP_MIX_NORM, "hyper_connection_mixer", False)):
+        names[base] = "mtp.layers.0.%s.hc_norm.weight" % pre; names[base + 1] = "mtp.layers.0.%s.input_mix_weight_down.weight" % pre
+        if inj:
+            names[base + 2] = "mtp.layers.0.%s.block_inject_weight.weight" % pre
+        names[base + (3 if inj else 2)] = "mtp.layers.0.%s.input_mix_weight_up.weight" % pre
+    norms = (mg.MTP_PRE_E, mg.MTP_PRE_H, mg.MTP_HCA_NORM, mg.MTP_HCF_NORM, mg.MTP_MIX_NORM, mg.MTP_QN, mg.MTP_KN)
+    file = {}
+    for slot, name in names.items():
+        ty, rows, cols, b = mt[slot]
+        if ty == synth.F32:      # a vector: the file holds bf16(w - 1) for a norm, bf16(w) otherwise; the drafter built from tensors gets what the loader must form
+            w = np.ascontiguousarray(b).view(np.float32)
+            bits = bf16_bits(w - np.float32(1.0) if slot in norms else w)
+            file[name] = bits
+            mt[slot] = (synth.F32, rows, cols, (f32_of(bits) + np.float32(1.0 if slot in norms else 0.0)).astype(np.float32).view(np.uint8))
+        else:
+            assert ty == synth.BF16
+            file[name] = np.ascontiguousarray(b).view(np.uint16).reshape(rows, cols)
+    g3 = lambda s, r, q: np.ascontiguousarray(mt[s][3]).view(np.uint16).reshape(N_EXP, r, q)
+    file["mtp.layers.0.mlp.experts.gate_up_proj"] = np.concatenate([g3(mg.MTP_GATE_E, FF, c.d), g3(mg.MTP_UP_E, FF, c.d)], axis=1)
+    file["mtp.layers.0.mlp.experts.down_proj"] = g3(mg.MTP_DOWN_E, c.d, FF)
+    path = str(tmp_path / "mtp.safetensors")
+    helpers.write_safetensors(path, file, meta={"format": "pt"})
+    gm = lib.Model(ctx, c, hw.layers, hw.globals_)
+    ga = lib.Mtp(gm, N_EXP, TOP_K, FF, 16, mt, DRAFT_IDS)
+    gb = lib.Mtp.from_safetensors(gm, path, DRAFT_IDS, top_k=TOP_K, window=16, head=mt[mg.MTP_HEAD])
+    gc = lib.Mtp.from_safetensors(gm, path, DRAFT_IDS, top_k=TOP_K, window=16)            # head: rows of the main output matrix as f32
+    prompt = np.random.Generator(np.random.PCG64(102)).integers(0, c.vocab, 21, dtype=np.uint32)
+    res = []
+    for gd in (ga, gb, gc):
+        gs = gm.new_state(96); gd.attach(gs); lg = gm.forward(prompt, gs)
+        ids, ps = gd.draft(gs, int(np.argmax(lg)), 4); c0, k, v = gd.kv(gs)
+        res.append((ids, ps, c0, k, v)); gs.close()
+    assert len(res[0][0]) == 4
+    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1].view(np.uint32), res[1][1].view(np.uint32))
+    assert res[0][2] == res[1][2] and np.array_equal(res[0][3].view(np.uint32), res[1][3].view(np.uint32)) and np.array_equal(res[0][4].view(np.uint32), res[1][4].view(np.uint32))
+    assert np.array_equal(res[0][0], res[2][0]) and np.allclose(res[0][1], res[2][1], rtol=1e-4, atol=0)
+    # the experts per token are capped by the main model's (PYRE_MTP_TOPK, mtp.rs:108); a missing tensor is named
+    gd = lib.Mtp.from_safetensors(gm, path, DRAFT_IDS, top_k=99, window=16); gd.close()
+    del file["mtp.layers.0.self_attn.k_norm.weight"]
+    helpers.write_safetensors(path, file)
+    with pytest.raises(lib.PyreError, match="mtp tensor self_attn.k_norm.weight"):
+        lib.Mtp.from_safetensors(gm, path, DRAFT_IDS)
+    for o in (ga, gb, gc, gm):
+        o.close()
+
+
+def test_adaptive_draft_length_changes_which_drafts_are_verified_not_the_tokens(ctx):
+    """spec::generate's adaptive plan (spec.rs:162-217): with it on, the drafted loops still produce the plain greedy stream;
+    a drafter whose drafts are never accepted is verified less often once a plain step has been timed."""
+    c = small_cfg(qtype=synth.IQ3_S, hc_type=synth.IQ3_S, hc_lr=256)
+    gm, gd, om, od = pair(ctx, c, 121, window=8)
+    prompt = np.random.Generator(np.random.PCG64(122)).integers(0, c.vocab, 13, dtype=np.uint32)
+    s0 = gm.new_state(160); fl = gm.forward(prompt, s0); plain, _ = gm.generate_greedy(s0, fl, 60)
+    ctx.set_spec_adapt(1)
+    try:
+        s1 = gm.new_state(160); gd.attach(s1); fl1 = gm.forward(prompt, s1)
+        out, rounds, drafted, accepted = gd.generate_greedy(s1, fl1, 60, k=3)
+        assert np.array_equal(out, plain) and 0 <= accepted <= drafted
+        # the prompt-lookup drafter misses often, so plain steps get timed and the plan engages
+        s2 = gm.new_state(160); fl2 = gm.forward(prompt, s2)
+        out2, r2, d2, a2 = gm.generate_greedy_ngram(s2, prompt, fl2, 60, k=4, ng_min=1, ng_max=4)
+        assert np.array_equal(out2, plain) and 0 <= a2 <= d2
+        ctx.set_spec_adapt(0)
+        s3 = gm.new_state(160); fl3 = gm.forward(prompt, s3)
+        out3, r3, d3, a3 = gm.generate_greedy_ngram(s3, prompt, fl3, 60, k=4, ng_min=1, ng_max=4)
+        assert np.array_equal(out3, plain) and 0 <= a3 <= d3
+    finally:
+        ctx.set_spec_adapt(-1)
+    for o in (gd, s0, s1, s2, s3, gm):
+        o.close()
