@@ -86,6 +86,8 @@ def test_moe_iq3s_gate_up_in_the_integer_form_over_the_activation_range(ctx):
             y1, _, _ = moe.ffn(x[ti:ti + 1])
             assert np.array_equal(y1.view(np.uint32), y[ti:ti + 1].view(np.uint32)), (case, ti)
     import subprocess, sys, os
+    if os.environ.get("PYRE_MOE_IDOT", "") == "0":
+        return                                                              # this process already runs the f32 form: nothing to compare
     code = ("import numpy as np, sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
             "from pyre_amd import lib, synth, modelgen as mg\n"
             "import test_gpu_blocks as tb\n"
