@@ -359,6 +359,7 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   qmat_args_now(m.down_e); qmat_args_now(m.sh_down); args_now(m.d, m.top_k, sel_idx, h, hstride, parts);
   __shared__ float red[GE][NW][64];
   __shared__ float hx[ID ? 1 : NW][GE][64];
+  __shared__ __align__(16) uint32_t hdg[ID ? NW : 1][GE][DGX_STRIDE];
   const int ti = blockIdx.y, q = blockIdx.z, k = FIX ? 10 : m.top_k, gsz = (k + 4) / 4, d = FIX ? 2048 : m.d;          // FIX: the A3B configuration (top 10, d = 2048, experts 512 wide), checked by the launcher
   const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;          // the group's routed entries j0 .. j0+nr-1
   const bool with_shared = q == PYRE_MOE_GROUPS - 1;
@@ -378,6 +379,11 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   float acc[GE][1];
 #pragma unroll
   for (int e = 0; e < GE; ++e) acc[e][0] = 0.0f;
+  // the routing weights and the shared expert's gate are requested now, not behind the products
+  float wv[GE];
+#pragma unroll
+  for (int e = 0; e < GE; ++e) wv[e] = e < nr ? sel_w[ti * k + j0 + e] : 0.0f;
+  const float g = with_shared ? sg[ti] : 0.0f;
   for (int it = 0; it < niter; ++it) {
     UnitRaw<FMT> r[GE]; float hv[GE]; bool on[GE]; int ku[GE];
 #pragma unroll
@@ -387,8 +393,18 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
       if (on[e]) { const QMatDev& D = shared ? m.sh_down : m.down_e; r[e] = unit_load<FMT>(D, tile[e], ku[e], lane); if constexpr (!ID) hv[e] = xs[e][ku[e] * 64 + lane]; }
     }
     if constexpr (ID) {
+      // the units' digits through the wave's own shared memory: one coalesced load an entry, all in flight with the weights
+      // (as scalar loads they would come one entry after the other: three entries' digits do not fit the scalar registers)
+      uint32_t dv[GE];
 #pragma unroll
-      for (int e = 0; e < GE; ++e) if (on[e]) unit_idot_iq3s(r[e], dge[e] + (size_t)ku[e] * DGX_STRIDE, acc[e][0]);
+      for (int e = 0; e < GE; ++e) dv[e] = on[e] ? (dge[e] + (size_t)ku[e] * DGX_STRIDE)[lane] : 0u;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int e = 0; e < GE; ++e) if (on[e]) hdg[wave][e][lane] = dv[e];
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int e = 0; e < GE; ++e) if (on[e]) unit_idot_iq3s(r[e], hdg[wave][e], acc[e][0]);
+      __builtin_amdgcn_wave_barrier();
     } else {
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -403,10 +419,6 @@ __global__ __launch_bounds__(NW * 64, (GE <= 3 && FMT >= 5 && FMT <= 7) ? 6 : 1)
   for (int e = 0; e < GE; ++e) if (e < ne) red[e][wave][lane] = acc[e][0];
   lds_barrier();
   if (threadIdx.x < 64) {
-    float wv[GE];
-#pragma unroll
-    for (int e = 0; e < GE; ++e) wv[e] = e < nr ? sel_w[ti * k + j0 + e] : 0.0f;
-    const float g = with_shared ? sg[ti] : 0.0f;
     float o = 0.0f;
 #pragma unroll
     for (int e = 0; e < GE; ++e) if (e < ne) {
