@@ -128,6 +128,32 @@ def test_safetensors_reader_names_shapes_bytes_and_errors(tmp_path):
         lib.Safetensors(str(tmp_path / "missing.safetensors"))
 
 
+def test_safetensors_reader_against_files_the_safetensors_library_writes(tmp_path):
+    """The container as the reference's checkpoint comes (scripts/mtp_fetch.py writes it with the safetensors library): BF16
+    tensors saved by safetensors.torch.save_file, with metadata, read back name by name, shape by shape, bit by bit."""
+    import numpy as np
+    torch = pytest.importorskip("torch")
+    st_torch = pytest.importorskip("safetensors.torch")
+    g = torch.Generator().manual_seed(7)
+    ts = {"mtp.fc_embedding.weight": torch.randn(6, 8, generator=g).to(torch.bfloat16),
+          "mtp.layers.0.mlp.experts.gate_up_proj": torch.randn(3, 4, 8, generator=g).to(torch.bfloat16),
+          "mtp.layers.0.self_attn.q_norm.weight": torch.randn(5, generator=g).to(torch.bfloat16),
+          "mtp.pre_fc_norm_hidden.weight": torch.zeros(0, dtype=torch.bfloat16)}
+    p = str(tmp_path / "lib.safetensors")
+    st_torch.save_file(ts, p, metadata={"format": "pt", "note": "written by the safetensors library"})
+    st = lib.Safetensors(p)
+    assert sorted(st.names()) == sorted(["fc_embedding.weight", "mlp.experts.gate_up_proj", "self_attn.q_norm.weight", "pre_fc_norm_hidden.weight"])
+    for k, t in ts.items():
+        nm = k.replace("mtp.", "", 1).replace("layers.0.", "", 1)
+        shape, bits = st.tensor(nm)
+        want = t.contiguous().view(torch.int16).numpy().view(np.uint16).reshape(-1)
+        assert shape == list(t.shape) and np.array_equal(bits[:want.size], want)
+    st.close()
+    st_torch.save_file({"a": torch.zeros(2, 2, dtype=torch.float16)}, p)
+    with pytest.raises(lib.PyreError, match="dtype F16"):
+        lib.Safetensors(p)
+
+
 def test_create_without_gpu_fails_loudly_not_silently():
     import torch
     if torch.cuda.is_available():
