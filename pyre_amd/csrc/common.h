@@ -134,7 +134,7 @@ inline __host__ __device__ size_t mh_slot(size_t rg, int sb, int SB) { return ((
 // dv: the lane = row planes (every type).  dvm: the matrix-core layout, IQ3_S only (fmt == FMT_IQ3_S_M when present).
 // Which of the two an IQ3_S matrix holds is decided at creation: the stand-alone operator keeps both (its entry points
 // cover both kernels), the model keeps one per matrix.
-enum { PYRE_LAYOUT_ROWS = 0, PYRE_LAYOUT_M = 1, PYRE_LAYOUT_BOTH = 2 };
+enum { PYRE_LAYOUT_ROWS = 0, PYRE_LAYOUT_M = 1, PYRE_LAYOUT_BOTH = 2, PYRE_LAYOUT_ALL = 3 };      // ALL (the stand-alone operator): rows, the matrix-core layout (IQ3_S, Q4_K) and the single token's native-format layout
 struct pyre_qmat {
   pyre_ctx* ctx; uint32_t ty; size_t rows, cols; size_t gguf_bytes;
   void* base; size_t dev_bytes; QMatDev dv;
@@ -205,6 +205,11 @@ size_t pyre_aop_bytes(int cols, int t);                            // operand by
 int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv);
 // y as pyre_gemv_launch / pyre_gemv_split_launch (ksplit > 1: slice sums) with the epilogues of GemvEpi
 int pyre_gemm_m_best_count(const QMatDev& m);
+// Q4_K on the matrix cores (gemm_q4.hip): the operator's windows
+size_t pyre_gemm_q4_bytes(size_t rows, size_t cols, size_t* codes);
+int pyre_gemm_q4_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* base);
+size_t pyre_gemm_q4_scratch_bytes(int cols);
+int pyre_gemm_q4_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, void* scratch = nullptr);
 int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep, const float* xf = nullptr);
 // xf: the single token's f32 activations instead of `a` (the kernel forms the operand rows itself); where that pays
 bool pyre_gemm_m_x_ok(const QMatDev& m, int t, const GemvEpi& ep);

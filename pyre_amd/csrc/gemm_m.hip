@@ -274,7 +274,7 @@ int pyre_gemm_m_scratch(pyre_ctx* ctx, int cols, uint4** op, float** ainv) {
 // (32 bytes a column) and their scale factors.  One copy per GPU, held until the process ends; calls on one GPU share it.
 #define STATIC_MAX_COLS 32768
 #define STATIC_OP_BYTES ((size_t)STATIC_MAX_COLS * 32)
-static __device__ __align__(256) uint8_t scratch[STATIC_OP_BYTES + (STATIC_MAX_COLS / 256) * 8 * 4];
+static __device__ __align__(256) uint8_t scratch[STATIC_OP_BYTES + (STATIC_MAX_COLS / 256) * 8 * 4 + 256 + (STATIC_MAX_COLS / 32) * 8 * 4];      // (operand rows, scale factors; a Q4_K window's sub-block sums)
 static void* g_scratch_ptr[64];
 static std::mutex g_scratch_mu;          // contexts may be created from several threads
 

@@ -319,7 +319,7 @@ int gemv_nw(const QMatDev& m, int ksplit) {
 }
 template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
-  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8"};
+  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8", "iq3_s", "q4_k"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   ProfScope ps(ctx, name.c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * T * ((double)m.cols + m.rows));
   hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), T > 1 ? (size_t)NW * 2 * 64 * T * 4 : 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
@@ -466,8 +466,10 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
   if (rows > (size_t)1 << 30 || cols > (size_t)1 << 24) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmat_create: %zu x %zu too large", rows, cols);
   size_t row_bytes = cols / gel * gbytes;
   if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
-  const bool want_n = layout == PYRE_LAYOUT_BOTH && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS || (fmt == FMT_Q4_K && ty == PYRE_Q4_K)) && cols % 256 == 0;      // the single token's native-format layout
-  if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // only IQ3_S has a matrix-core layout
+  const bool want_n = layout == PYRE_LAYOUT_ALL && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS || (fmt == FMT_Q4_K && ty == PYRE_Q4_K)) && cols % 256 == 0;      // the single token's native-format layout
+  const bool want_q4m = layout == PYRE_LAYOUT_ALL && fmt == FMT_Q4_K && ty == PYRE_Q4_K && cols % 256 == 0;      // Q4_K for the matrix cores: the operator's windows
+  if (layout == PYRE_LAYOUT_ALL) layout = PYRE_LAYOUT_BOTH;
+  if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // in a model only IQ3_S has a matrix-core layout
   const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
   PYRE_HIP(ctx, hipSetDevice(ctx->device));
   pyre_qmat* m = new pyre_qmat(); m->ctx = ctx; m->ty = ty; m->rows = rows; m->cols = cols; m->gguf_bytes = nbytes;
@@ -509,6 +511,13 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
     e = hipGetLastError();
     if (!want_rows) m->dv = m->dvm;         // the only layout the matrix has is the one every user sees
   }
+  if (want_q4m && e == hipSuccess) {
+    size_t sq; m->dev_bytes_m = pyre_gemm_q4_bytes(rows, cols, &sq);
+    e = hipMalloc(&m->base_m, m->dev_bytes_m);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_m, hipGetErrorString(e)); }
+    m->dvm = shape; m->dvm.fmt = FMT_Q4_K_M; m->dvm.mq = (const uint8_t*)m->base_m; m->dvm.mh = (const uint8_t*)m->base_m + sq; m->dvm.SB = (int)(cols / 256);
+    if (pyre_gemm_q4_repack(ctx, rows, cols, src, row_bytes, m->base_m) != PYRE_OK) e = hipErrorLaunchFailure;
+  }
   if (want_n && e == hipSuccess) {      // the stand-alone operator's single-token kernel streams (close to) the file's bits per weight
     m->dev_bytes_n = pyre_gemv_n_bytes(rows, cols, fmt);
     e = hipMalloc(&m->base_n, m->dev_bytes_n);
@@ -523,7 +532,7 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
 // the stand-alone operator keeps an IQ3_S matrix in both layouts: pyre_qmatmul runs on the matrix cores, pyre_qmatmul_f32
 // on the lane = row GEMV that the model's expert matrices use
 static int qmat_create_common(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols, const void* blocks, bool on_device, size_t nbytes, pyre_qmat** out) {
-  return pyre_qmat_create_layout(ctx, ty, rows, cols, blocks, on_device, nbytes, PYRE_LAYOUT_BOTH, out);
+  return pyre_qmat_create_layout(ctx, ty, rows, cols, blocks, on_device, nbytes, PYRE_LAYOUT_ALL, out);
 }
 
 extern "C" {
@@ -560,7 +569,7 @@ int pyre_qmat_row(pyre_ctx* ctx, const pyre_qmat* m, size_t row, float* out_host
   void* st; int rc = pyre_stage(ctx, m->cols * sizeof(float) + 256, &st); if (rc) return rc;
   uint32_t r = (uint32_t)row; uint32_t* idx = (uint32_t*)((uint8_t*)st + m->cols * sizeof(float));
   PYRE_HIP(ctx, hipMemcpyAsync(idx, &r, 4, hipMemcpyHostToDevice, ctx->stream));
-  rc = pyre_row_launch(ctx, m->dvm.mq ? m->dvm : m->dv, idx, 1, (float*)st, (int)m->cols); if (rc) return rc;      // a matrix held in both layouts: rows come from the matrix-core one, pyre_qmat_dequant from the other
+  rc = pyre_row_launch(ctx, (m->dvm.mq && m->dvm.fmt == FMT_IQ3_S_M) ? m->dvm : m->dv, idx, 1, (float*)st, (int)m->cols); if (rc) return rc;      // a matrix held in both layouts: rows come from the matrix-core one, pyre_qmat_dequant from the other
   PYRE_HIP(ctx, hipMemcpyAsync(out_host, st, m->cols * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;
 }
@@ -580,6 +589,9 @@ static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev,
   // (IQ2_XS and Q4_K have the same kernel over their own layouts, 2.5 and 4.5 bit/weight; a small matrix of them stays with the one-launch f32 GEMV likewise)
   const bool rows_only = m->dv.fmt == FMT_IQ2_XS || m->dv.fmt == FMT_Q4_K;          // (the formats without a matrix-core layout)
   if (t == 1 && m->base_n && native && !f32_path && !f32_only && !(rows_only && m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, nullptr, rows_only ? m->dv.fmt : FMT_IQ3_S);
+  // a window of a large Q4_K matrix: the matrix cores, where eight tokens cost what two do (PYRE_QMATMUL_Q4M=0: the lane = row GEMV);
+  // small matrices stay with the one-launch GEMV, as above
+  if (t >= 2 && env_int("PYRE_QMATMUL_Q4M", 1) && m->dvm.fmt == FMT_Q4_K_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q4_launch(ctx, m->dvm, x_dev, t, y_dev);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
   if (has_m && (!has_rows || (!f32_path && !f32_only))) return pyre_gemv_launch(ctx, m->dvm, x_dev, t, y_dev);
   return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
@@ -610,6 +622,10 @@ int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
     if (t == 1 && env_int("PYRE_QMATMUL_NATIVE", 1) && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {
       if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
       return pyre_gemv_n_launch(ctx, m->base_n, m->rows, m->cols, x_dev, y_dev, ctx->aop_static, m->dv.fmt);
+    }
+    if (t >= 2 && env_int("PYRE_QMATMUL_Q4M", 1) && m->dvm.fmt == FMT_Q4_K_M && m->dvm.mq && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {      // a Q4_K window on the matrix cores, as in pyre_qmatmul_dev
+      if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
+      return pyre_gemm_q4_launch(ctx, m->dvm, x_dev, t, y_dev, ctx->aop_static);
     }
     return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   }

@@ -352,3 +352,38 @@ def test_small_iq3s_single_token_takes_one_launch(ctx):
     m.matmul(x); ctx.sync()
     rep = ctx.prof_report(); ctx.prof_enable(False)
     assert sum(v[0] for v in rep.values()) == 1, rep          # one kernel launch for the call
+
+
+# ---- a window of a Q4_K matrix on the matrix cores: codes -> f16 by or-ing, scales folded before the product, minima through
+# ---- the sub-block sums of the activations -----------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(64, 256), (100, 512), (320, 2048), (8256, 1024), (1000, 768), (130, 8192)])
+def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, monkeypatch):
+    monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the matrix-core kernel
+    raw = synth.matrix(lib.Q4_K, rows, cols, 900 + rows % 97)
+    m = lib.QMat(ctx, lib.Q4_K, rows, cols, raw)
+    assert m.layout_bytes(1) >= (rows + 63) // 64 * 64 * (cols // 256) * 144          # 4.5 bit/weight: 128 bytes of codes + a 16-byte header
+    W = orc.dequant(lib.Q4_K, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    g = np.random.Generator(np.random.PCG64(rows + cols + 3))
+    for case in range(6):
+        x = synth.normal((8, cols), 910 + case)
+        if case == 1: x *= np.exp2(g.integers(-30, 30, cols // 256).repeat(256)).astype(np.float32)
+        if case == 2: x[0, 5] = 3.0e4; x[3, cols - 3] = -2.0e7
+        if case == 3: x *= 1e-25
+        if case == 4: x[5] *= 1e20
+        if case == 5: x[:, ::2] = 0.0; x[:, :64] = 0.0
+        with np.errstate(all="ignore"):
+            truth = x.astype(np.float64) @ W.T
+        y = m.matmul(x)
+        for ti in range(8):                                     # per token: each has its own largest magnitude
+            assert relerr(y[ti], truth[ti]) <= TOL, (case, ti)
+        assert np.array_equal(bits(y), bits(m.matmul(x)))          # run to run
+        for t in (2, 3, 5):                                     # a token's bits do not depend on the window's width
+            assert np.array_equal(bits(m.matmul(x[:t])), bits(y[:t])), (case, t)
+        assert relerr(y[:2], m.matmul_f32(x[:2])) <= 4e-6       # the f32 GEMV agrees to rounding
+    assert not m.matmul(np.zeros((4, cols), np.float32)).any()
+    bad = synth.normal((3, cols), 920); bad[1, 7] = np.nan
+    yb = m.matmul(bad)
+    assert np.isnan(yb[1]).all() and np.isfinite(yb[0]).all() and np.isfinite(yb[2]).all()          # a token's NaN stays its own
+    monkeypatch.setenv("PYRE_QMATMUL_Q4M", "0")
+    assert relerr(m.matmul(x), truth) <= TOL                     # (the lane = row window path stays available)
