@@ -319,7 +319,7 @@ int gemv_nw(const QMatDev& m, int ksplit) {
 }
 template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
-  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8", "iq3_s", "q4_k"};
+  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8", "iq3_s", "q4_k", "iq2_xs"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   ProfScope ps(ctx, name.c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * T * ((double)m.cols + m.rows));
   hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), T > 1 ? (size_t)NW * 2 * 64 * T * 4 : 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
@@ -468,6 +468,7 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
   if (!blocks || nbytes != rows * row_bytes) return pyre_fail(ctx, PYRE_E_ARG, "pyre_qmat_create: expected %zu bytes of blocks, got %zu", rows * row_bytes, nbytes);
   const bool want_n = layout == PYRE_LAYOUT_ALL && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS || (fmt == FMT_Q4_K && ty == PYRE_Q4_K)) && cols % 256 == 0;      // the single token's native-format layout
   const bool want_q4m = layout == PYRE_LAYOUT_ALL && fmt == FMT_Q4_K && ty == PYRE_Q4_K && cols % 256 == 0;      // Q4_K for the matrix cores: the operator's windows
+  const bool want_q2m = layout == PYRE_LAYOUT_ALL && fmt == FMT_IQ2_XS && ty == PYRE_IQ2_XS && cols % 256 == 0;      // IQ2_XS likewise
   if (layout == PYRE_LAYOUT_ALL) layout = PYRE_LAYOUT_BOTH;
   if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // in a model only IQ3_S has a matrix-core layout
   const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
@@ -517,6 +518,13 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
     if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_m, hipGetErrorString(e)); }
     m->dvm = shape; m->dvm.fmt = FMT_Q4_K_M; m->dvm.mq = (const uint8_t*)m->base_m; m->dvm.mh = (const uint8_t*)m->base_m + sq; m->dvm.SB = (int)(cols / 256);
     if (pyre_gemm_q4_repack(ctx, rows, cols, src, row_bytes, m->base_m) != PYRE_OK) e = hipErrorLaunchFailure;
+  }
+  if (want_q2m && e == hipSuccess) {
+    size_t sq; m->dev_bytes_m = pyre_gemm_q2_bytes(rows, cols, &sq);
+    e = hipMalloc(&m->base_m, m->dev_bytes_m);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_m, hipGetErrorString(e)); }
+    m->dvm = shape; m->dvm.fmt = FMT_IQ2_XS_M; m->dvm.mq = (const uint8_t*)m->base_m; m->dvm.mh = (const uint8_t*)m->base_m + sq; m->dvm.SB = (int)(cols / 256);
+    if (pyre_gemm_q2_repack(ctx, rows, cols, src, row_bytes, m->base_m) != PYRE_OK) e = hipErrorLaunchFailure;
   }
   if (want_n && e == hipSuccess) {      // the stand-alone operator's single-token kernel streams (close to) the file's bits per weight
     m->dev_bytes_n = pyre_gemv_n_bytes(rows, cols, fmt);
@@ -592,6 +600,8 @@ static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev,
   // a window of a large Q4_K matrix: the matrix cores, where eight tokens cost what two do (PYRE_QMATMUL_Q4M=0: the lane = row GEMV);
   // small matrices stay with the one-launch GEMV, as above
   if (t >= 2 && env_int("PYRE_QMATMUL_Q4M", 1) && m->dvm.fmt == FMT_Q4_K_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q4_launch(ctx, m->dvm, x_dev, t, y_dev);
+  // a window of a large IQ2_XS matrix likewise (PYRE_QMATMUL_Q2M=0: the lane = row GEMV)
+  if (t >= 2 && env_int("PYRE_QMATMUL_Q2M", 1) && m->dvm.fmt == FMT_IQ2_XS_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q2_launch(ctx, m->dvm, x_dev, t, y_dev);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
   if (has_m && (!has_rows || (!f32_path && !f32_only))) return pyre_gemv_launch(ctx, m->dvm, x_dev, t, y_dev);
   return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
@@ -626,6 +636,10 @@ int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
     if (t >= 2 && env_int("PYRE_QMATMUL_Q4M", 1) && m->dvm.fmt == FMT_Q4_K_M && m->dvm.mq && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {      // a Q4_K window on the matrix cores, as in pyre_qmatmul_dev
       if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
       return pyre_gemm_q4_launch(ctx, m->dvm, x_dev, t, y_dev, ctx->aop_static);
+    }
+    if (t >= 2 && env_int("PYRE_QMATMUL_Q2M", 1) && m->dvm.fmt == FMT_IQ2_XS_M && m->dvm.mq && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {      // an IQ2_XS window likewise
+      if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
+      return pyre_gemm_q2_launch(ctx, m->dvm, x_dev, t, y_dev, ctx->aop_static);
     }
     return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   }

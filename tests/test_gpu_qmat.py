@@ -355,15 +355,16 @@ def test_small_iq3s_single_token_takes_one_launch(ctx):
 
 
 # ---- a window of a Q4_K matrix on the matrix cores: codes -> f16 by or-ing, scales folded before the product, minima through
-# ---- the sub-block sums of the activations -----------------------------------------------------------------------------------
+# ---- the sub-block sums of the activations; of an IQ2_XS matrix: codes -> f16 by byte permutes through a table in registers ----
 @pytest.mark.gpu
+@pytest.mark.parametrize("ty,switch", [(lib.Q4_K, "PYRE_QMATMUL_Q4M"), (lib.IQ2_XS, "PYRE_QMATMUL_Q2M")], ids=["q4_k", "iq2_xs"])
 @pytest.mark.parametrize("rows,cols", [(64, 256), (100, 512), (320, 2048), (8256, 1024), (1000, 768), (130, 8192)])
-def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, monkeypatch):
+def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, ty, switch, monkeypatch):
     monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the matrix-core kernel
-    raw = synth.matrix(lib.Q4_K, rows, cols, 900 + rows % 97)
-    m = lib.QMat(ctx, lib.Q4_K, rows, cols, raw)
+    raw = synth.matrix(ty, rows, cols, 900 + rows % 97)
+    m = lib.QMat(ctx, ty, rows, cols, raw)
     assert m.layout_bytes(1) >= (rows + 63) // 64 * 64 * (cols // 256) * 144          # 4.5 bit/weight: 128 bytes of codes + a 16-byte header
-    W = orc.dequant(lib.Q4_K, raw, rows * cols).reshape(rows, cols).astype(np.float64)
+    W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
     g = np.random.Generator(np.random.PCG64(rows + cols + 3))
     for case in range(6):
         x = synth.normal((8, cols), 910 + case)
@@ -385,5 +386,9 @@ def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, monkeypatch):
     bad = synth.normal((3, cols), 920); bad[1, 7] = np.nan
     yb = m.matmul(bad)
     assert np.isnan(yb[1]).all() and np.isfinite(yb[0]).all() and np.isfinite(yb[2]).all()          # a token's NaN stays its own
-    monkeypatch.setenv("PYRE_QMATMUL_Q4M", "0")
+    ctx.prof_reset(); ctx.prof_enable(True)
+    m.matmul(x[:4]); ctx.sync()
+    assert any(k.startswith("gemm_q4k_t4" if ty == lib.Q4_K else "gemm_iq2xs_t4") for k in ctx.prof_report()), ctx.prof_report()          # the kernel under test is the one that ran
+    ctx.prof_enable(False)
+    monkeypatch.setenv(switch, "0")
     assert relerr(m.matmul(x), truth) <= TOL                     # (the lane = row window path stays available)
