@@ -95,7 +95,7 @@ int    pyre_qmatmul_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev, i
  * significant bits; values more than 2^14 / 6e-5 below the largest magnitude of their stretch lose resolution), the 4-bit
  * codes times their sub-block scales are exact in f16, products are exact and summed in f32.  A non-finite activation
  * makes every output of its token NaN.  An IQ3_S matrix created through pyre_qmat_create* is held in three layouts (one per
- * kernel; an IQ2_XS or Q4_K matrix in three as well: rows, the single token's native format and, for a window of a matrix of more than 128 row tiles, a matrix-core layout of its own, 4.5 bit/weight; pyre_qmat_device_bytes counts them all, pyre_qmat_layout_bytes each).  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the
+ * kernel; an IQ2_XS or Q4_K matrix in three as well: rows, the single token's native format and, for a window of a matrix of more than 128 row tiles, a matrix-core layout of its own, 4.5 bit/weight; a Q8_0 matrix in two: rows and such a matrix-core layout, 8.5 bit/weight; pyre_qmat_device_bytes counts them all, pyre_qmat_layout_bytes each).  pyre_qmatmul_f32 is the same contract on the f32 multiply-add GEMV the
  * model's expert matrices use (QMat::matmul's own arithmetic, gguf_q.rs:169-197,233-241: f32 products, f32 accumulation);
  * for every other type the two are the same code. */
 int    pyre_qmatmul_f32(pyre_ctx* ctx, const pyre_qmat* m, const float* x_host, int t, float* y_host);
@@ -104,7 +104,7 @@ int    pyre_qmatmul_f32_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  IQ3_S matrices (whose kernels take the
  * activations from a scratch buffer, as f16 operand rows or as fixed-point digits) and IQ2_XS and Q4_K matrices (whose
  * single-token kernel takes the digits likewise, and whose windows' matrix-core kernels take operand rows -- Q4_K also the activations'
- * sub-block sums); every other type's pyre_qmatmul_dev allocates nothing already.  The operand goes to a fixed device array inside the library (PYRE_QMATMUL_STATIC_MAX_COLS * 32 bytes plus
+ * sub-block sums) and Q8_0 matrices (a window's matrix-core kernel likewise); every other type's pyre_qmatmul_dev allocates nothing already.  The operand goes to a fixed device array inside the library (PYRE_QMATMUL_STATIC_MAX_COLS * 32 bytes plus
  * the scale factors and the sums, 1 MiB + 36 KiB per GPU, held until the process ends) instead of the context's grow-only buffer, and the
  * call makes no allocation, no event and no copy: two kernel launches on the context's stream.  Same kernels and launch
  * shapes as pyre_qmatmul_dev, so the result is bit-identical to it.  Matrices with more than

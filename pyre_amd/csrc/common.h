@@ -214,6 +214,10 @@ int pyre_gemm_q4_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int
 size_t pyre_gemm_q2_bytes(size_t rows, size_t cols, size_t* codes);
 int pyre_gemm_q2_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* base);
 int pyre_gemm_q2_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, void* scratch = nullptr);
+// Q8_0 on the matrix cores (gemm_q8.hip): likewise
+size_t pyre_gemm_q8_bytes(size_t rows, size_t cols, size_t* codes);
+int pyre_gemm_q8_repack(pyre_ctx* ctx, size_t rows, size_t cols, const uint8_t* raw_dev, size_t row_bytes, void* base);
+int pyre_gemm_q8_launch(pyre_ctx* ctx, const QMatDev& m, const float* x_dev, int t, float* y_dev, void* scratch = nullptr);
 int pyre_gemm_m_launch(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y_dev, int ksplit, const GemvEpi& ep, const float* xf = nullptr);
 // xf: the single token's f32 activations instead of `a` (the kernel forms the operand rows itself); where that pays
 bool pyre_gemm_m_x_ok(const QMatDev& m, int t, const GemvEpi& ep);

@@ -10,7 +10,7 @@
 // value = scale * integer is the reference's own last multiply.
 // FMT_IQ3_S_M is the second home of an IQ3_S matrix: the same 4-bit codes laid out for the matrix cores (see QMatDev), used by
 // the matrices that only ever meet a GEMV (projections, the vocabulary head, the stand-alone operator).
-enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_C4 = 7, FMT_C8 = 8, FMT_IQ3_S_M = 9, FMT_Q4_K_M = 10, FMT_IQ2_XS_M = 11, FMT_COUNT = 12 };      // FMT_Q4_K_M, FMT_IQ2_XS_M: Q4_K / IQ2_XS codes and headers laid out for the matrix cores (gemm_q4.hip, gemm_q2.hip; the operator's windows only)
+enum { FMT_F32 = 0, FMT_F16 = 1, FMT_BF16 = 2, FMT_Q8_0 = 3, FMT_Q4_K = 4, FMT_IQ2_XS = 5, FMT_IQ3_S = 6, FMT_C4 = 7, FMT_C8 = 8, FMT_IQ3_S_M = 9, FMT_Q4_K_M = 10, FMT_IQ2_XS_M = 11, FMT_Q8_0_M = 12, FMT_COUNT = 13 };      // FMT_Q4_K_M, FMT_IQ2_XS_M, FMT_Q8_0_M: Q4_K / IQ2_XS / Q8_0 codes and headers laid out for the matrix cores (gemm_q4.hip, gemm_q2.hip, gemm_q8.hip; the operator's windows only)
 
 struct FmtGeom { int V; int e1, e2, e3, eb; };   // plane entry sizes: 16-byte chunks per unit in p0; bytes per unit in p1..p3; bytes per super-block in pb
 __host__ __device__ inline FmtGeom fmt_geom(int fmt) {

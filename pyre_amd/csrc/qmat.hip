@@ -319,7 +319,7 @@ int gemv_nw(const QMatDev& m, int ksplit) {
 }
 template <int FMT, int T, int NW> int gemv_launch_nw(pyre_ctx* ctx, const QMatDev& m, const float* x, float* y, int ksplit, const GemvEpi& ep) {
   int per_wg = (m.U + ksplit - 1) / ksplit, upw = (per_wg + NW - 1) / NW; if (upw < 1) upw = 1;
-  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8", "iq3_s", "q4_k", "iq2_xs"};
+  static const char* fn[FMT_COUNT] = {"f32", "f16", "bf16", "q8_0", "q4_k", "iq2_xs", "iq3_s", "c4", "c8", "iq3_s", "q4_k", "iq2_xs", "q8_0"};
   static const std::string name = std::string("gemv_") + fn[FMT] + "_t" + std::to_string(T);
   ProfScope ps(ctx, name.c_str(), qmat_gguf_bytes(m, m.rows) + 4.0 * T * ((double)m.cols + m.rows));
   hipLaunchKernelGGL((k_gemv<FMT, T, NW>), dim3(m.tiles, ksplit), dim3(NW * 64), T > 1 ? (size_t)NW * 2 * 64 * T * 4 : 0, ctx->stream, m, x, y, upw, ep, (const uint2*)ctx->d_iq2xs);
@@ -469,6 +469,7 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
   const bool want_n = layout == PYRE_LAYOUT_ALL && (fmt == FMT_IQ3_S || fmt == FMT_IQ2_XS || (fmt == FMT_Q4_K && ty == PYRE_Q4_K)) && cols % 256 == 0;      // the single token's native-format layout
   const bool want_q4m = layout == PYRE_LAYOUT_ALL && fmt == FMT_Q4_K && ty == PYRE_Q4_K && cols % 256 == 0;      // Q4_K for the matrix cores: the operator's windows
   const bool want_q2m = layout == PYRE_LAYOUT_ALL && fmt == FMT_IQ2_XS && ty == PYRE_IQ2_XS && cols % 256 == 0;      // IQ2_XS likewise
+  const bool want_q8m = layout == PYRE_LAYOUT_ALL && fmt == FMT_Q8_0 && ty == PYRE_Q8_0 && cols % 256 == 0;      // Q8_0 likewise
   if (layout == PYRE_LAYOUT_ALL) layout = PYRE_LAYOUT_BOTH;
   if (fmt != FMT_IQ3_S) layout = PYRE_LAYOUT_ROWS;       // in a model only IQ3_S has a matrix-core layout
   const bool want_rows = layout != PYRE_LAYOUT_M, want_m = layout != PYRE_LAYOUT_ROWS;
@@ -525,6 +526,13 @@ int pyre_qmat_create_layout(pyre_ctx* ctx, uint32_t ty, size_t rows, size_t cols
     if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_m, hipGetErrorString(e)); }
     m->dvm = shape; m->dvm.fmt = FMT_IQ2_XS_M; m->dvm.mq = (const uint8_t*)m->base_m; m->dvm.mh = (const uint8_t*)m->base_m + sq; m->dvm.SB = (int)(cols / 256);
     if (pyre_gemm_q2_repack(ctx, rows, cols, src, row_bytes, m->base_m) != PYRE_OK) e = hipErrorLaunchFailure;
+  }
+  if (want_q8m && e == hipSuccess) {
+    size_t sq; m->dev_bytes_m = pyre_gemm_q8_bytes(rows, cols, &sq);
+    e = hipMalloc(&m->base_m, m->dev_bytes_m);
+    if (e != hipSuccess) { if (tmp) (void)hipFree(tmp); drop(); return pyre_fail(ctx, PYRE_E_NOMEM, "pyre_qmat_create: hipMalloc(%zu) failed: %s", m->dev_bytes_m, hipGetErrorString(e)); }
+    m->dvm = shape; m->dvm.fmt = FMT_Q8_0_M; m->dvm.mq = (const uint8_t*)m->base_m; m->dvm.mh = (const uint8_t*)m->base_m + sq; m->dvm.SB = (int)(cols / 256);
+    if (pyre_gemm_q8_repack(ctx, rows, cols, src, row_bytes, m->base_m) != PYRE_OK) e = hipErrorLaunchFailure;
   }
   if (want_n && e == hipSuccess) {      // the stand-alone operator's single-token kernel streams (close to) the file's bits per weight
     m->dev_bytes_n = pyre_gemv_n_bytes(rows, cols, fmt);
@@ -600,6 +608,8 @@ static int qmatmul_launch(pyre_ctx* ctx, const pyre_qmat* m, const float* x_dev,
   // a window of a large Q4_K matrix: the matrix cores, where eight tokens cost what two do (PYRE_QMATMUL_Q4M=0: the lane = row GEMV);
   // small matrices stay with the one-launch GEMV, as above
   if (t >= 2 && env_int("PYRE_QMATMUL_Q4M", 1) && m->dvm.fmt == FMT_Q4_K_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q4_launch(ctx, m->dvm, x_dev, t, y_dev);
+  // a window of a large Q8_0 matrix likewise (PYRE_QMATMUL_Q8M=0: the lane = row GEMV)
+  if (t >= 2 && env_int("PYRE_QMATMUL_Q8M", 1) && m->dvm.fmt == FMT_Q8_0_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q8_launch(ctx, m->dvm, x_dev, t, y_dev);
   // a window of a large IQ2_XS matrix likewise (PYRE_QMATMUL_Q2M=0: the lane = row GEMV)
   if (t >= 2 && env_int("PYRE_QMATMUL_Q2M", 1) && m->dvm.fmt == FMT_IQ2_XS_M && m->dvm.mq && !f32_path && !f32_only && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) return pyre_gemm_q2_launch(ctx, m->dvm, x_dev, t, y_dev);
   const bool has_m = m->dvm.fmt == FMT_IQ3_S_M && m->dvm.mq, has_rows = m->base != nullptr;
@@ -643,7 +653,15 @@ int pyre_qmatmul_static_dev(pyre_ctx* ctx, const pyre_qmat* m, const float* x_de
     }
     return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
   }
-  if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S, IQ2_XS and Q4_K matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
+  if (m->dvm.fmt == FMT_Q8_0_M && m->dvm.mq) {      // Q8_0: only a window of a large matrix uses scratch (the matrix-core kernel's operand rows)
+    if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
+    if (t >= 2 && env_int("PYRE_QMATMUL_Q8M", 1) && !env_int("PYRE_QMATMUL_F32", 0) && !(m->dv.tiles <= 128 && env_int("PYRE_QMATMUL_SMALL", 1))) {
+      if (!ctx->aop_static) return pyre_fail(ctx, PYRE_E_HIP, "pyre_qmatmul_static_dev: the device array was not resolved at context creation");
+      return pyre_gemm_q8_launch(ctx, m->dvm, x_dev, t, y_dev, ctx->aop_static);
+    }
+    return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);
+  }
+  if (m->dvm.fmt != FMT_IQ3_S_M || !m->dvm.mq) return pyre_fail(ctx, PYRE_E_TYPE, "pyre_qmatmul_static_dev: IQ3_S, IQ2_XS, Q4_K and Q8_0 matrices only (the other types' GEMV uses no scratch: pyre_qmatmul_dev allocates nothing for them)");
   if (m->cols > PYRE_QMATMUL_STATIC_MAX_COLS) return pyre_fail(ctx, PYRE_E_SHAPE, "pyre_qmatmul_static_dev: %zu columns exceed the static scratch of %d columns; use pyre_qmatmul_dev", m->cols, PYRE_QMATMUL_STATIC_MAX_COLS);
   if (qmat_small_one_token(m, t) && !env_int("PYRE_QMATMUL_F32", 0)) return pyre_gemv_launch(ctx, m->dv, x_dev, t, y_dev);      // as pyre_qmatmul_dev (a launch that happens to need no scratch; the limit above holds for every call alike)
   if (t == 1 && m->base_n && env_int("PYRE_QMATMUL_NATIVE", 1)) {      // one token: the native-format kernel, as in pyre_qmatmul_dev, its activation digits in the static array

@@ -355,15 +355,16 @@ def test_small_iq3s_single_token_takes_one_launch(ctx):
 
 
 # ---- a window of a Q4_K matrix on the matrix cores: codes -> f16 by or-ing, scales folded before the product, minima through
-# ---- the sub-block sums of the activations; of an IQ2_XS matrix: codes -> f16 by byte permutes through a table in registers ----
+# ---- the sub-block sums of the activations; of an IQ2_XS matrix: codes -> f16 by byte permutes through a table in registers;
+# ---- of a Q8_0 matrix: bytes -> f16 by one byte permute and an addition, the block's d after the product ----------------------
 @pytest.mark.gpu
-@pytest.mark.parametrize("ty,switch", [(lib.Q4_K, "PYRE_QMATMUL_Q4M"), (lib.IQ2_XS, "PYRE_QMATMUL_Q2M")], ids=["q4_k", "iq2_xs"])
+@pytest.mark.parametrize("ty,switch", [(lib.Q4_K, "PYRE_QMATMUL_Q4M"), (lib.IQ2_XS, "PYRE_QMATMUL_Q2M"), (lib.Q8_0, "PYRE_QMATMUL_Q8M")], ids=["q4_k", "iq2_xs", "q8_0"])
 @pytest.mark.parametrize("rows,cols", [(64, 256), (100, 512), (320, 2048), (8256, 1024), (1000, 768), (130, 8192)])
 def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, ty, switch, monkeypatch):
     monkeypatch.setenv("PYRE_QMATMUL_SMALL", "0")          # small shapes too through the matrix-core kernel
     raw = synth.matrix(ty, rows, cols, 900 + rows % 97)
     m = lib.QMat(ctx, ty, rows, cols, raw)
-    assert m.layout_bytes(1) >= (rows + 63) // 64 * 64 * (cols // 256) * 144          # 4.5 bit/weight: 128 bytes of codes + a 16-byte header
+    assert m.layout_bytes(1) >= (rows + 63) // 64 * 64 * (cols // 256) * (272 if ty == lib.Q8_0 else 144)          # 4.5 bit/weight: 128 bytes of codes + a 16-byte header (Q8_0: 8.5: 256 + 16)
     W = orc.dequant(ty, raw, rows * cols).reshape(rows, cols).astype(np.float64)
     g = np.random.Generator(np.random.PCG64(rows + cols + 3))
     for case in range(6):
@@ -388,7 +389,7 @@ def test_q4k_window_on_the_matrix_cores(ctx, rows, cols, ty, switch, monkeypatch
     assert np.isnan(yb[1]).all() and np.isfinite(yb[0]).all() and np.isfinite(yb[2]).all()          # a token's NaN stays its own
     ctx.prof_reset(); ctx.prof_enable(True)
     m.matmul(x[:4]); ctx.sync()
-    assert any(k.startswith("gemm_q4k_t4" if ty == lib.Q4_K else "gemm_iq2xs_t4") for k in ctx.prof_report()), ctx.prof_report()          # the kernel under test is the one that ran
+    assert any(k.startswith({lib.Q4_K: "gemm_q4k_t4", lib.IQ2_XS: "gemm_iq2xs_t4", lib.Q8_0: "gemm_q8_0_t4"}[ty]) for k in ctx.prof_report()), ctx.prof_report()          # the kernel under test is the one that ran
     ctx.prof_enable(False)
     monkeypatch.setenv(switch, "0")
     assert relerr(m.matmul(x), truth) <= TOL                     # (the lane = row window path stays available)

@@ -47,8 +47,8 @@ def test_static_scratch_entry_point_equals_the_allocating_one_on_consecutive_cal
     big.close(); small.close()
 
 
-@pytest.mark.parametrize("ty", [lib.IQ2_XS, lib.Q4_K])
-def test_static_scratch_entry_point_iq2xs_q4k_single_token(ctx, ty):
+@pytest.mark.parametrize("ty", [lib.IQ2_XS, lib.Q4_K, lib.Q8_0])
+def test_static_scratch_entry_point_iq2xs_q4k_single_token(ctx, ty):          # (Q8_0: its window alone uses scratch)
     big = lib.QMat(ctx, ty, 8256, 2048, synth.matrix(ty, 8256, 2048, 511))          # 129 row tiles: the native-format kernel, digits in the array
     small = lib.QMat(ctx, ty, 320, 512, synth.matrix(ty, 320, 512, 512))          # one launch, no scratch
     for m, rows, cols, t in ((big, 8256, 2048, 1), (small, 320, 512, 1), (big, 8256, 2048, 4), (big, 8256, 2048, 1)):
@@ -69,7 +69,7 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit_and_other_types(ct
     assert np.array_equal(ctx.download(yd, (8, rows)).view(np.uint32), ctx.download(ya, (8, rows)).view(np.uint32))
     with pytest.raises(lib.PyreError):
         edge.matmul_static_dev(xd, 9, yd)
-    q8 = lib.QMat(ctx, lib.Q8_0, 64, 256, synth.matrix(lib.Q8_0, 64, 256, 507))
+    q8 = lib.QMat(ctx, lib.Q6_K, 64, 256, synth.matrix(lib.Q6_K, 64, 256, 507))
     with pytest.raises(lib.PyreError, match="IQ3_S"):
         q8.matmul_static_dev(xd, 1, yd)
     for p in (xd, yd, ya):
