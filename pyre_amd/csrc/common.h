@@ -244,6 +244,7 @@ struct MoeDev {
   QMatDev router, gate_e, up_e, down_e, sh_gate, sh_up, sh_down;
   const float* sh_gate_inp;
   int d, n_exp, top_k, ff, sf;
+  QMatDev gate_m{}, up_m{}, down_m{}, sh_gate_m{}, sh_up_m{}, sh_down_m{};      // the expert matrices once more in the matrix-core layout (FMT_IQ3_S_M), when the model keeps it: a long prompt's blocks (pyre_moe_block_launch)
 };
 struct MoeWork {            // scratch for up to 8 tokens, owned by whoever launches the block
   float* logits;            // [8][n_exp]
@@ -306,6 +307,22 @@ struct RouteSrc { const float* p; int nsl; int r64; const uint32_t* dgx = nullpt
 // token in w.parts, group q of token ti at parts + (q*t + ti)*d, instead of the unreduced terms.
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr, bool in_groups = false);
 inline bool pyre_moe_groups_ok(const MoeDev& m) { return m.top_k <= PYRE_MOE_KMAX; }
+// The FFN of a block of prompt windows (T = 8 * windows tokens) with the tokens grouped by expert, on the matrix cores (moe.hip):
+// what the windows' mixes leave -- x [T][d], the router's K-slice sums (window w's at rpart + w * nsl * 8 * r64, slice s of
+// token ti at (s * 8 + ti) * r64) -- and where window w's group sums go: parts + w * 4 * 8 * d, laid out as MoeWork::parts of
+// a window of eight.  The rest is the block's own scratch (pyre_moe_block_carve): the routing, the (token, choice) pairs by
+// expert, x and h as f16 operand rows a token (xh [T + 1][2][d], hh [T * (k + 1) + 1][2][ff], the last row of each zero) with
+// their scale factors, the gate and up products and the unreduced down terms.
+struct MoeBlk {
+  const float* x; const float* rpart; float* parts;
+  int32_t* sel_idx; float* sel_w; float* sg; int32_t* eoff; int32_t* elist; float* g; float* u; float* partial;
+  uint16_t* xh; float* xinv; uint16_t* hh; float* hinv;
+};
+bool   pyre_moe_block_ok(const MoeDev& m);
+size_t pyre_moe_block_bytes(const MoeDev& m, int T);
+void   pyre_moe_block_carve(const MoeDev& m, int T, void* base, MoeBlk* b);
+int    pyre_moe_block_zero_rows(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T);
+int    pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64);
 // K parts the gate/up dot products are summed in (1 or 2; k_moe_gu)
 int pyre_moe_gu_parts(const MoeDev& m);
 

@@ -3,7 +3,10 @@
 // greedy loop.  Follows Model::forward_inner / forward_multi / spec_keep (src/model/qwen4exp_gguf.rs:2087-2157,
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
+#include "digits.h"
+#include <atomic>
 #include <chrono>
+#include <thread>
 #include <memory>
 #include <stdlib.h>
 
@@ -22,7 +25,7 @@ struct Layer {
 
 }  // namespace
 
-struct PromptPipe; void prompt_pipe_free(PromptPipe* P);
+struct PromptPipe; void prompt_pipe_free(PromptPipe* P); size_t prompt_pipe_blocks(const PromptPipe* P);
 
 struct pyre_model {
   pyre_ctx* ctx = nullptr; pyre_model_cfg c{};
@@ -68,6 +71,9 @@ struct pyre_state {
 };
 
 namespace {
+
+// PYRE_PROMPT_BLOCK=0: no second layout of the expert matrices, every prompt in windows (prompt_block_ok)
+static bool prompt_block_env() { static const bool on = [] { const char* e = getenv("PYRE_PROMPT_BLOCK"); return !(e && *e && atoi(e) == 0); }(); return on; }
 
 struct Builder {
   pyre_ctx* ctx; pyre_model* m;
@@ -233,9 +239,12 @@ int pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_tenso
       }
     }
     MoeDev& mo = L.moe; size_t router_b = 0, ge = 0, ue = 0, de = 0, sh = 0;
-    if ((rc = B.one(T[PYRE_T_FFN_GATE_INP], &mo.router, &router_b)) || (rc = B.one(T[PYRE_T_FFN_GATE_EXPS], &mo.gate_e, &ge)) || (rc = B.one(T[PYRE_T_FFN_UP_EXPS], &mo.up_e, &ue)) ||
-        (rc = B.one(T[PYRE_T_FFN_DOWN_EXPS], &mo.down_e, &de)) || (rc = B.one(T[PYRE_T_FFN_GATE_SHEXP], &mo.sh_gate, &sh)) || (rc = B.one(T[PYRE_T_FFN_UP_SHEXP], &mo.sh_up, &sh)) ||
-        (rc = B.one(T[PYRE_T_FFN_DOWN_SHEXP], &mo.sh_down, &sh))) return rc;
+    // the expert matrices in the lane = row layout the decode and window kernels walk and, unless PYRE_PROMPT_BLOCK=0, once more in
+    // the matrix-core layout a long prompt's blocks use (4.25 bit/weight on top of the first layout's bytes)
+    const int elay = prompt_block_env() ? PYRE_LAYOUT_BOTH : PYRE_LAYOUT_ROWS;
+    if ((rc = B.one(T[PYRE_T_FFN_GATE_INP], &mo.router, &router_b)) || (rc = B.one(T[PYRE_T_FFN_GATE_EXPS], &mo.gate_e, &ge, elay, &mo.gate_m)) || (rc = B.one(T[PYRE_T_FFN_UP_EXPS], &mo.up_e, &ue, elay, &mo.up_m)) ||
+        (rc = B.one(T[PYRE_T_FFN_DOWN_EXPS], &mo.down_e, &de, elay, &mo.down_m)) || (rc = B.one(T[PYRE_T_FFN_GATE_SHEXP], &mo.sh_gate, &sh, elay, &mo.sh_gate_m)) || (rc = B.one(T[PYRE_T_FFN_UP_SHEXP], &mo.sh_up, &sh, elay, &mo.sh_up_m)) ||
+        (rc = B.one(T[PYRE_T_FFN_DOWN_SHEXP], &mo.sh_down, &sh, elay, &mo.sh_down_m))) return rc;
     mo.d = c.d; mo.n_exp = c.n_exp; mo.top_k = c.top_k; mo.ff = c.ff_exp; mo.sf = mo.sh_gate.rows;
     if (mo.router.rows != c.n_exp || mo.router.cols != c.d || mo.gate_e.rows != c.n_exp * c.ff_exp || mo.up_e.rows != c.n_exp * c.ff_exp || mo.gate_e.cols != c.d || mo.up_e.cols != c.d ||
         (size_t)mo.down_e.rows != (size_t)c.n_exp * c.d || mo.down_e.cols != c.ff_exp || mo.sh_up.rows != mo.sf || mo.sh_down.rows != c.d || mo.sh_down.cols != mo.sf || c.ff_exp % 64 || mo.sf % 64)
@@ -278,6 +287,7 @@ void pyre_model_destroy(pyre_model* m) {
   delete m;
 }
 size_t pyre_model_weight_bytes_per_token(const pyre_model* m) { return m ? m->token_weight_bytes : 0; }
+size_t pyre_model_prompt_blocks(const pyre_model* m) { return m && m->pipe ? prompt_pipe_blocks(m->pipe) : 0; }
 
 int pyre_state_create(pyre_ctx* ctx, const pyre_model* m, int max_ctx, pyre_state** out) {
   if (!ctx || !m || !out || max_ctx < 1) return pyre_fail(ctx, PYRE_E_ARG, "pyre_state_create: bad argument");
@@ -437,7 +447,12 @@ struct PromptPipe {
   std::vector<hipEvent_t> done;                // [set] end of the set's last window
   hipEvent_t start = nullptr;
   uint32_t* ids = nullptr; size_t ids_cap = 0; // the call's token ids on the device
+  // blocks of windows taken layer by layer with the FFN of all their tokens grouped by expert (prompt_block_get)
+  std::vector<pyre_model*> wmdl;               // a window workspace per window of a block
+  void* blk_mem = nullptr; MoeBlk blk{}; int blk_nsl = 0, blk_r64 = 0;
+  hipEvent_t moe_done = nullptr; std::vector<hipEvent_t> front_done; size_t blocks_done = 0;
 };
+size_t prompt_pipe_blocks(const PromptPipe* P) { return P->blocks_done; }
 static int prompt_streams() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_STREAMS"); int v = e && *e ? atoi(e) : 3; return v < 1 ? 1 : (v > 4 ? 4 : v); }(); return k; }
 void prompt_pipe_free(PromptPipe* P) {
   if (!P) return;
@@ -447,6 +462,10 @@ void prompt_pipe_free(PromptPipe* P) {
   for (auto e : P->done) if (e) (void)hipEventDestroy(e);
   if (P->start) (void)hipEventDestroy(P->start);
   if (P->ids) (void)hipFree(P->ids);
+  for (auto* mc : P->wmdl) if (mc) { if (mc->work) (void)hipFree(mc->work); delete mc; }
+  if (P->blk_mem) (void)hipFree(P->blk_mem);
+  if (P->moe_done) (void)hipEventDestroy(P->moe_done);
+  for (auto e : P->front_done) if (e) (void)hipEventDestroy(e);
   delete P;
 }
 static int prompt_pipe_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe** out) {
@@ -490,7 +509,63 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
   return PYRE_OK;
 }
 
+// ---- a long prompt in blocks of windows, layer by layer ---------------------------------------------------------------------
+// Windows of eight tokens share nothing in the FFN (eight tokens pick 74 of 512 experts), which makes the expert products
+// the largest part of a prompt window.  A block of PROMPT_BLOCK_WINDOWS windows is therefore taken layer by layer: every
+// window's part of the layer up to the FFN mix (on the prompt's streams, the layer's state passing from window to window as
+// before), then the FFN of all of the block's tokens in one set of launches with the tokens grouped by expert, on the
+// matrix cores (pyre_moe_block_launch), whose group sums the windows' next mixes read.  Everything but the FFN is the
+// windows' kernels and arithmetic; the FFN's products are those of the matrix-core GEMM (f16 halves of the activations
+// instead of fixed-point digits): equal to rounding, not bit for bit.  For models whose every layer qualifies
+// (prompt_block_ok); the call's last tokens (the window whose logits are read, the rows a drafter keeps) take the windows'
+// path.  PYRE_PROMPT_BLOCK=0 switches it off.
+#define PROMPT_BLOCK_WINDOWS 32
+#define PROMPT_BLOCK_MIN 8
+static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
+static bool prompt_block_ok(const pyre_model* m) {
+  if (!prompt_block_env()) return false;
+  { const char* r = getenv("PYRE_ROUTER_RIDES"); if (r && *r && atoi(r) == 0) return false; }
+  { const char* r = getenv("PYRE_MOE_GROUPS"); if (r && *r && atoi(r) == 0) return false; }
+  const pyre_model_cfg& c = m->c;
+  if (m->n_ple > 0 || c.top_k > PYRE_MOE_KMAX || c.d % 256 || !fuse_aop_on()) return false;
+  for (int il = 0; il < c.n_layers; ++il) { const Layer& L = m->layers[il];
+    if (!pyre_moe_block_ok(L.moe) || !pyre_hc_route_ok(L.hcf, L.moe.router) || !pyre_hc_aop_ok(L.hcf) || L.hca.di.fmt != FMT_IQ3_S || L.moe.router.tiles != m->layers[0].moe.router.tiles ||
+        L.moe.ff != m->layers[0].moe.ff || L.moe.sf != m->layers[0].moe.sf || L.moe.top_k != m->layers[0].moe.top_k || L.moe.n_exp != m->layers[0].moe.n_exp) return false; }
+  return true;
+}
+static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
+  if (!P->wmdl.empty()) return PYRE_OK;
+  const pyre_model_cfg& c = m->c; const int NB = PROMPT_BLOCK_WINDOWS, d = c.d, K = (int)P->ctx.size() + 1;
+  const MoeDev& m0 = m->layers[0].moe;
+  const int nsl = d / 64, r64 = m0.router.tiles * 64;
+  const size_t xb = al256((size_t)NB * 8 * d * 4), rb = al256((size_t)NB * nsl * 8 * r64 * 4), db = al256((size_t)NB * 8 * (d / 64) * DGX_STRIDE * 4), pb = al256((size_t)NB * PYRE_MOE_GROUPS * 8 * d * 4),
+               mb = al256(pyre_moe_block_bytes(m0, NB * 8));
+  PYRE_HIP(ctx, hipMalloc(&P->blk_mem, xb + rb + db + pb + mb + 256));
+  uint8_t* p = (uint8_t*)P->blk_mem;
+  float* x_all = (float*)p; p += xb; float* r_all = (float*)p; p += rb; uint32_t* d_all = (uint32_t*)p; p += db; float* p_all = (float*)p; p += pb;
+  pyre_moe_block_carve(m0, NB * 8, p, &P->blk);
+  P->blk.x = x_all; P->blk.rpart = r_all; P->blk.parts = p_all; P->blk_nsl = nsl; P->blk_r64 = r64;
+  { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk, NB * 8); if (rc) return rc; }
+  for (int j = 0; j < NB; ++j) {
+    pyre_model* mc = new pyre_model(*m); mc->owned.clear(); mc->bufs.clear(); mc->work = nullptr; mc->toks = nullptr; mc->toks_cap = 0; mc->pipe = nullptr;
+    P->wmdl.push_back(mc);
+    int rc = model_alloc_work(ctx, mc, nullptr); if (rc) return rc;
+    mc->mixed = x_all + (size_t)j * 8 * d; mc->rpart = r_all + (size_t)j * nsl * 8 * r64; mc->mw.dgx = d_all + (size_t)j * 8 * (d / 64) * DGX_STRIDE; mc->mw.parts = p_all + (size_t)j * PYRE_MOE_GROUPS * 8 * d;
+  }
+  PYRE_HIP(ctx, hipEventCreateWithFlags(&P->moe_done, hipEventDisableTiming));
+  P->front_done.resize(K, nullptr);
+  for (auto& e : P->front_done) PYRE_HIP(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return PYRE_OK;
+}
+
 namespace {
+
+// The windows of a block are enqueued by one host thread per stream.  A window's wait for the previous window's event of a
+// layer must be issued after that event's record (a wait on an event not yet recorded passes at once): issued[j] counts the
+// layers whose record window j's thread has issued; quit ends every host-side wait when a thread has failed.
+struct BlkSync { std::atomic<int> issued[PROMPT_BLOCK_WINDOWS]; std::atomic<int> go{-1}, done{0}; std::atomic<bool> quit{false}; };
+static inline void cpu_relax() { __builtin_ia32_pause(); }
 
 struct WinOpt {
   int head_tokens = 1;          // 0 = no logits, 1 = last token only, t = every token (rows 0..t-1 of m->logits)
@@ -504,6 +579,9 @@ struct WinOpt {
   // a prompt window that shares the GPU with its neighbours (prompt_pipe): its ids, the attention / selection workspace
   // it uses instead of the state's, and per layer the event it waits for (the previous window has left the layer) and records
   const uint32_t* ids_dev = nullptr; const AttnWork* aw = nullptr; const QsaWork* qw = nullptr; const hipEvent_t* wait_ev = nullptr; const hipEvent_t* rec_ev = nullptr;
+  int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
+  bool no_len = false;          // ... and the state's length is then advanced by the caller
+  BlkSync* bs = nullptr; int bj = 0;      // a block's windows enqueued from several host threads: this window's index in the block (BlkSync)
 };
 
 // rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
@@ -517,7 +595,6 @@ int mtp_window_of(const pyre_mtp* m);
 bool outp_in_parts(const Layer& L, int d) { return pyre_gemv_parts_ok(L.outp) && (int)L.outp.rows == d && L.hcf.di.fmt == FMT_IQ3_S; }
 
 // One window of t <= 8 tokens (ids in m->ids unless from_best).
-static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
 // A Gated DeltaNet layer whose output projection is on the matrix cores runs its recurrence on nv x 4 workgroups and leaves
 // the head norm to that projection (GdnQ / PyreAop::sq) -- in every call that touches the layer's state, the re-run of
 // pyre_spec_keep included: the two forms of the kernel round the state differently.  PYRE_GDN_Q=0: nv workgroups.
@@ -525,36 +602,63 @@ static bool gdn_q_on(const pyre_model* m, const Layer& L) {
   const char* e = getenv("PYRE_GDN_Q");
   return !(e && *e && atoi(e) == 0) && fuse_aop_on() && !L.full && L.outp.fmt == FMT_IQ3_S_M && L.gdn.dv == 128 && L.gdn.dk == 128 && L.outp.cols == L.gdn.nv * 128 && m->gdn_sq != nullptr;
 }
-int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
-  const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; const int start = s->len; const bool replay = o.step_dev != nullptr;
-  if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
-  const uint32_t* ids = o.ids_dev ? o.ids_dev : m->ids; const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
-  int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev, s->tokens_dev) : pyre_row_launch(ctx, m->embd, ids, t, m->emb, d); if (rc) return rc;
-  // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
-  // leaves the updated streams in the other
-  const float* xin = m->emb; int in_ss = 0, in_ts = d; float* xout = m->x; float* xother = m->x2;
-  auto advance = [&]() { xin = xout; in_ss = d; in_ts = hc * d; float* q = xout; xout = xother; xother = q; };
-  const bool raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
+// One window of t <= 8 tokens as an object, so that a block of prompt windows can be taken layer by layer: begin() (embedding
+// rows, history, n-gram rows), per layer front(il) (everything up to the FFN mix, whose output is the FFN's input) and
+// moe(il) (the FFN; the block path runs pyre_moe_block_launch for all of its windows instead and calls moe_from_block),
+// finish() (bookkeeping, head).  run_window is the four in order.
+struct WinRun {
+  pyre_ctx* ctx; const pyre_model* m; pyre_state* s; int t; WinOpt o;
+  int start = 0; bool replay = false;
+  const float* xin = nullptr; int in_ss = 0, in_ts = 0; float* xout = nullptr; float* xother = nullptr;
   MoeOut mo{}; const MoeOut* comb_moe = nullptr; const float* comb_out = nullptr; const float* comb_inj = nullptr;
   int comb_np = 1;          // vectors the pending update comes in: 1, or PYRE_GEMV_PARTS == PYRE_MOE_GROUPS to be added in order
-  const bool moe_groups = [] { const char* e = getenv("PYRE_MOE_GROUPS"); return !(e && *e && atoi(e) == 0); }();      // 0: windows leave the unreduced terms as a single token does
-  const bool route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
-  // the window's tokens join the history (PLE models and states with a drafter keep one)
-  if (s->tokens_dev && !o.from_best && !o.ids_dev) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));      // (a prompt on several streams has stored the whole call's ids already)
-  if (m->n_ple > 0) {      // every position's n-gram rows are fetched once for all PLE layers
-    if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
+  bool raw_moe = false, moe_groups = true, route_rides = true, fuse_aop = true, ride = false;
+  WinRun(pyre_ctx* c, const pyre_model* mm, pyre_state* ss, int tt, const WinOpt& oo) : ctx(c), m(mm), s(ss), t(tt), o(oo) {}
+  void advance() { xin = xout; in_ss = m->c.d; in_ts = m->c.hc * m->c.d; float* q = xout; xout = xother; xother = q; }
+  bool hc_fused(const HcDev& h, const QMatDev& q) const { const int d = m->c.d; return fuse_aop && q.fmt == FMT_IQ3_S_M && q.cols == d && d % 256 == 0 && pyre_hc_aop_ok(h); }
+  bool gdn_fused(const Layer& L) const { return fuse_aop && L.outp.fmt == FMT_IQ3_S_M && L.gdn_ainv != nullptr; }
+  int begin() {
+    const pyre_model_cfg& c = m->c; const int d = c.d;
+    start = o.start >= 0 ? o.start : s->len; replay = o.step_dev != nullptr;
+    if (start + t > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "forward: context %d exceeds the state's capacity %d", start + t, s->cap);
+    const uint32_t* ids = o.ids_dev ? o.ids_dev : m->ids;
+    int rc = o.from_best ? pyre_pick_launch(ctx, m->best, pyre_gemv_best_count(m->out), m->ids, o.toks_out, &m->embd, m->emb, o.step_dev, s->tokens_dev) : pyre_row_launch(ctx, m->embd, ids, t, m->emb, d); if (rc) return rc;
+    // the residual streams alternate between two buffers: every mix reads one (first the embedding row, replicated) and
+    // leaves the updated streams in the other
+    xin = m->emb; in_ss = 0; in_ts = d; xout = m->x; xother = m->x2;
+    raw_moe = c.top_k <= PYRE_MOE_KMAX;        // the next mix folds the unreduced FFN output itself (same arithmetic as k_moe_sum, one launch fewer per layer)
+    moe_groups = [] { const char* e = getenv("PYRE_MOE_GROUPS"); return !(e && *e && atoi(e) == 0); }();      // 0: windows leave the unreduced terms as a single token does
+    route_rides = [] { const char* e = getenv("PYRE_ROUTER_RIDES"); return !(e && *e && atoi(e) == 0); }();      // 0: separate router launch (what the persistent kernel mirrors)
+    // the window's tokens join the history (PLE models and states with a drafter keep one)
+    if (s->tokens_dev && !o.from_best && !o.ids_dev) PYRE_HIP(ctx, hipMemcpyAsync(s->tokens_dev + start, ids, (size_t)t * 4, hipMemcpyDeviceToDevice, ctx->stream));      // (a prompt on several streams has stored the whole call's ids already)
+    if (m->n_ple > 0) {      // every position's n-gram rows are fetched once for all PLE layers
+      if ((rc = pyre_ple_rows_launch(ctx, m->plc, m->ple_tab, m->pw, s->tokens_dev, start, o.step_dev, t))) return rc;
+    }
+    fuse_aop = fuse_aop_on();      // PYRE_AOP_SPLIT=1: separate split launches instead of the producers' own operand stores
+    return PYRE_OK;
   }
-  const bool fuse_aop = fuse_aop_on();      // PYRE_AOP_SPLIT=1: separate split launches instead of the producers' own operand stores
-  // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
-  // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
-  // own split launch (its magnitude has no bound a single workgroup of the merge could form)
-  const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
-  const AopOut aout{m->aop, m->aop_inv, d / 256};
-  auto hc_fused = [&](const HcDev& h, const QMatDev& q) { return fuse_aop && q.fmt == FMT_IQ3_S_M && q.cols == d && d % 256 == 0 && pyre_hc_aop_ok(h); };
-  auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
-  auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
-  auto gdn_fused = [&](const Layer& L) { return fuse_aop && L.outp.fmt == FMT_IQ3_S_M && L.gdn_ainv != nullptr; };
-  for (int il = 0; il < c.n_layers; ++il) {
+  // whether layer il's FFN output of a window of several tokens goes to the next mix as four group sums a token: when that mix
+  // can add partial vectors (an IQ3_S mix over all of the window's tokens, no PLE layer in between); otherwise, and for a
+  // single token, unreduced
+  bool groups_at(int il) const {
+    const pyre_model_cfg& c = m->c; const Layer& L = m->layers[il];
+    bool groups = raw_moe && t > 1 && moe_groups && pyre_moe_groups_ok(L.moe);
+    if (groups) {
+      if (il + 1 < c.n_layers) { const Layer& Ln = m->layers[il + 1]; groups = !Ln.ple && Ln.hca.di.fmt == FMT_IQ3_S; }
+      else groups = (o.head_tokens >= t || (s->mtp && o.keep_from < t)) && m->head.di.fmt == FMT_IQ3_S;
+    }
+    return groups;
+  }
+  int front(int il) {
+    const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; int rc;
+    const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
+    // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
+    // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
+    // own split launch (its magnitude has no bound a single workgroup of the merge could form)
+    const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
+    const AopOut aout{m->aop, m->aop_inv, d / 256};
+    auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
+    auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
     const Layer& L = m->layers[il];
     if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
     if (L.ple) {      // resolves the pending residual update itself and leaves plain streams
@@ -565,6 +669,7 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
     if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.hca, L.proj)))) return rc;
     advance(); comb_np = 1;
     // the layer's state (cache, recurrent state, saved projection) is the previous window's until that window has left it
+    if (o.bs && o.bj > 0) { while (o.bs->issued[o.bj - 1].load(std::memory_order_acquire) <= il) { if (o.bs->quit.load(std::memory_order_relaxed)) return pyre_fail(ctx, PYRE_E_HIP, "a neighbouring window failed"); cpu_relax(); } }
     if (o.wait_ev) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));
     if (L.full) {
       int ai = L.mix_index;
@@ -580,49 +685,65 @@ int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const W
       s->cur[li] = nb;
     }
     if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
+    if (o.bs) o.bs->issued[o.bj].store(il + 1, std::memory_order_release);
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
     if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc; }
     else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc;
-    const bool ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
-    HcRoute hr{L.moe.router, m->rpart, m->mw.dgx}; RouteSrc rs{m->rpart, d / 64, L.moe.router.tiles * 64, pyre_hc_aop_ok(L.hcf) ? m->mw.dgx : nullptr};          // (the matrix-core mix leaves the digits of its output; after another mix the expert launch makes them)
+    ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
+    HcRoute hr{L.moe.router, m->rpart, m->mw.dgx};          // (the matrix-core mix leaves the digits of its output; after another mix the expert launch makes them)
     if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
     advance();
-    // A window's FFN output goes to the next mix as four group sums a token when that mix can add partial vectors (an
-    // IQ3_S mix over all of the window's tokens, no PLE layer in between); otherwise, and for a single token, unreduced.
-    bool groups = raw_moe && t > 1 && moe_groups && pyre_moe_groups_ok(L.moe);
-    if (groups) {
-      if (il + 1 < c.n_layers) { const Layer& Ln = m->layers[il + 1]; groups = !Ln.ple && Ln.hca.di.fmt == FMT_IQ3_S; }
-      else groups = (o.head_tokens >= t || (s->mtp && o.keep_from < t)) && m->head.di.fmt == FMT_IQ3_S;
-    }
+    return PYRE_OK;
+  }
+  int moe(int il) {
+    const pyre_model_cfg& c = m->c; const Layer& L = m->layers[il]; int rc;
+    RouteSrc rs{m->rpart, c.d / 64, L.moe.router.tiles * 64, pyre_hc_aop_ok(L.hcf) ? m->mw.dgx : nullptr};
+    const bool groups = groups_at(il);
     if ((rc = pyre_moe_launch(ctx, L.moe, m->mw, m->mixed, t, raw_moe ? nullptr : m->y, ride ? &rs : nullptr, groups))) return rc;
     if (groups) { comb_out = m->mw.parts; comb_moe = nullptr; comb_np = PYRE_MOE_GROUPS; }
     else if (raw_moe) { mo = pyre_moe_out(L.moe, m->mw, 0); comb_moe = &mo; comb_out = nullptr; } else comb_out = m->y;
     comb_inj = m->inj_f;
+    return PYRE_OK;
   }
-  if (!replay) s->len = start + t;
-  const bool want_r = s->mtp && o.keep_from < t;      // the head mix resolves the pending update of every token: its x_out rows are the final residual streams
-  if (o.head_tokens == 0 && !want_r) return PYRE_OK;       // prompt window whose logits nobody reads
-  if (o.head_tokens >= t || want_r) {
-    const bool all = o.head_tokens >= t;
-    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, comb_np, all ? opw(m->head, m->out) : nullptr))) return rc;
-    if (want_r) {
-      const int w = hc * d;
-      hipLaunchKernelGGL(k_ring_store, dim3((w + 255) / 256, t - o.keep_from), dim3(256), 0, ctx->stream, xout, s->r_ring, s->r_mask, start, o.step_dev, o.keep_from, w); PYRE_CHECK_LAUNCH(ctx);
-      if (!replay) s->r_push(start + o.keep_from, t - o.keep_from, mtp_window_of(s->mtp));
+  // the block's FFN launch has left this window's group sums in m->mw.parts
+  void moe_from_block() { comb_out = m->mw.parts; comb_moe = nullptr; comb_np = PYRE_MOE_GROUPS; comb_inj = m->inj_f; }
+  int finish() {
+    const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; int rc;
+    const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
+    const AopOut aout{m->aop, m->aop_inv, d / 256};
+    auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
+    auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
+    if (!replay && !o.no_len) s->len = start + t;
+    const bool want_r = s->mtp && o.keep_from < t;      // the head mix resolves the pending update of every token: its x_out rows are the final residual streams
+    if (o.head_tokens == 0 && !want_r) return PYRE_OK;       // prompt window whose logits nobody reads
+    if (o.head_tokens >= t || want_r) {
+      const bool all = o.head_tokens >= t;
+      if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->hbuf, m->inj_a, nullptr, comb_np, all ? opw(m->head, m->out) : nullptr))) return rc;
+      if (want_r) {
+        const int w = hc * d;
+        hipLaunchKernelGGL(k_ring_store, dim3((w + 255) / 256, t - o.keep_from), dim3(256), 0, ctx->stream, xout, s->r_ring, s->r_mask, start, o.step_dev, o.keep_from, w); PYRE_CHECK_LAUNCH(ctx);
+        if (!replay) s->r_push(start + o.keep_from, t - o.keep_from, mtp_window_of(s->mtp));
+      }
+      if (o.head_tokens == 0) return PYRE_OK;
+      if (!all) return pyre_gemv_launch(ctx, m->out, m->hbuf + (size_t)(t - 1) * d, 1, m->logits);      // the last token's logits only
+      if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
+      return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->head, m->out));
     }
-    if (o.head_tokens == 0) return PYRE_OK;
-    if (!all) return pyre_gemv_launch(ctx, m->out, m->hbuf + (size_t)(t - 1) * d, 1, m->logits);      // the last token's logits only
-    if (o.greedy && t == 1) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
-    return pyre_gemv_launch(ctx, m->out, m->hbuf, t, m->logits, opnd(m->head, m->out));
+    // last token only: fold the pending ffn output into its streams, then the head
+    const size_t last = (size_t)(t - 1) * hc * d;
+    MoeOut mol{}; if (comb_moe) mol = pyre_moe_out(m->layers.back().moe, m->mw, t - 1);
+    if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->head, m->out)))) return rc;
+    if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
+    return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits, opnd(m->head, m->out));
   }
-  // last token only: fold the pending ffn output into its streams, then the head
-  const size_t last = (size_t)(t - 1) * hc * d;
-  MoeOut mol{}; if (comb_moe) mol = pyre_moe_out(m->layers.back().moe, m->mw, t - 1);
-  if ((rc = pyre_hc_mix_launch(ctx, m->head, m->hw, xin + last, in_ss, in_ts, xout + last, 1, comb_out ? comb_out + (size_t)(t - 1) * d : nullptr, comb_moe ? &mol : nullptr, comb_inj + (size_t)(t - 1) * hc, c.eps, m->hbuf, m->inj_a, nullptr, 1, opw(m->head, m->out)))) return rc;
-  if (o.greedy) return pyre_gemv_argmax_launch(ctx, m->out, m->hbuf, m->logits, m->best, opnd(m->head, m->out));
-  return pyre_gemv_launch(ctx, m->out, m->hbuf, 1, m->logits, opnd(m->head, m->out));
+};
+int run_window(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, int t, const WinOpt& o) {
+  WinRun w(ctx, m, s, t, o);
+  int rc = w.begin(); if (rc) return rc;
+  for (int il = 0; il < m->c.n_layers; ++il) { if ((rc = w.front(il)) || (rc = w.moe(il))) return rc; }
+  return w.finish();
 }
 
 int check_ids(pyre_ctx* ctx, const pyre_model* m, const uint32_t* ids, int n) {
@@ -639,6 +760,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
   if (s->m != m) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: state belongs to another model");
   if (s->broken) return pyre_fail(ctx, PYRE_E_STATE, "%s: an earlier call failed half way through this state; pyre_state_reset or pyre_state_restore first", "pyre_forward");
   if (s->len + n > s->cap) return pyre_fail(ctx, PYRE_E_STATE, "pyre_forward: %d + %d tokens exceed the state's capacity %d", s->len, n, s->cap);
+  const auto t_enter = std::chrono::steady_clock::now();
   int rc = check_ids(ctx, m, ids, n); if (rc) return rc;
   s->last_window = 0;
   const int nwin = (n + 7) / 8, K = prompt_streams();
@@ -652,8 +774,80 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     PYRE_HIP(ctx, hipEventRecord(P->start, ctx->stream));      // the other streams begin after everything already queued here
     for (auto* cx : P->ctx) PYRE_HIP(ctx, hipStreamWaitEvent(cx->stream, P->start, 0));
   }
-  int prev = -1;
-  for (int i = 0, w = 0; i < n; i += 8, ++w) {
+  int prev = -1, i_first = 0;
+  const bool windows_only = [] { const char* e = getenv("PYRE_PROMPT_WINDOWS"); return e && *e && atoi(e) != 0; }();      // (read per call: 1 = this call in windows, whatever layouts the model keeps)
+  if (P && !windows_only && prompt_block_ok(m)) {      // whole blocks of windows in front of the call's last tokens: layer by layer, the FFN grouped by expert
+    // (a call's last block may be shorter, down to PROMPT_BLOCK_MIN windows: fewer tokens than that share too few experts to pay)
+    const int NBMAX = PROMPT_BLOCK_WINDOWS, tail = 8 + (s->mtp ? mtp_window_of(s->mtp) : 0);
+    int wins = n > tail ? (n - tail) / 8 : 0;
+    if (wins >= PROMPT_BLOCK_MIN && (rc = prompt_block_get(ctx, m, P))) return rc;
+    const int nl = m->c.n_layers;
+    const bool threads = K > 1 && [] { const char* e = getenv("PYRE_PROMPT_THREADS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_THREADS=0: one host thread enqueues every stream
+    for (int bi = 0; wins >= PROMPT_BLOCK_MIN; ++bi) {
+      const int NB = wins < NBMAX ? wins : NBMAX; wins -= NB;
+      std::vector<WinRun> runs; runs.reserve(NB);
+      auto cx_of = [&](int j) { const int set = j % K; return set ? P->ctx[set - 1] : ctx; };
+      auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
+      const int pos0 = s->len;
+      BlkSync bsync; for (auto& a : bsync.issued) a.store(0);
+      for (int j = 0; j < NB; ++j) {
+        const int set = j % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos0 + 8 * j; o.no_len = true;
+        if (threads) { o.bs = &bsync; o.bj = j; }
+        o.ids_dev = P->ids + i_first + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
+        const int pset = j > 0 ? (j - 1) % K : prev;            // (prev: the set of the block before this one's last window)
+        o.wait_ev = pset >= 0 ? P->ev[pset].data() : nullptr; o.rec_ev = P->ev[set].data();
+        runs.emplace_back(cx_of(j), P->wmdl[j], s, 8, o);
+        if ((rc = runs.back().begin())) return bail(rc, cx_of(j));
+      }
+      // the layer's fronts: stream k's windows from host thread k (the launches of a front cost the host what they cost the GPU)
+      std::vector<int> trc(K, PYRE_OK);
+      auto fronts_of = [&](int k, int il) -> int {
+        for (int j = k; j < NB; j += K) {
+          pyre_ctx* cx = cx_of(j);
+          if (il > 0 && j < K && j % K != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
+          int r = runs[j].front(il); if (r) return r;
+        }
+        return PYRE_OK;
+      };
+      std::vector<std::thread> workers;
+      if (threads) for (int k = 1; k < K; ++k) workers.emplace_back([&, k] {
+        (void)hipSetDevice(ctx->device);
+        for (int il = 0; il < nl; ++il) {
+          while (bsync.go.load(std::memory_order_acquire) < il) { if (bsync.quit.load(std::memory_order_relaxed)) return; cpu_relax(); }
+          const int r = fronts_of(k, il);
+          if (r) { trc[k] = r; bsync.quit.store(true); bsync.done.fetch_add(1, std::memory_order_release); return; }
+          bsync.done.fetch_add(1, std::memory_order_release);
+        }
+      });
+      auto join = [&] { bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); };
+      for (int il = 0; il < nl; ++il) {
+        if (threads) {
+          bsync.go.store(il, std::memory_order_release);
+          rc = fronts_of(0, il);
+          if (rc) { join(); return bail(rc, ctx); }
+          while (bsync.done.load(std::memory_order_acquire) < (il + 1) * (K - 1)) cpu_relax();
+          for (int k = 1; k < K; ++k) if (trc[k]) { join(); return bail(trc[k], cx_of(k)); }
+        } else {
+          for (int j = 0; j < NB; ++j) {
+            pyre_ctx* cx = cx_of(j);
+            if (il > 0 && j < K && j % K != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
+            if ((rc = runs[j].front(il))) return bail(rc, cx);
+          }
+        }
+        if (il == nl - 1) break;            // the last layer's FFN output has no reader in these windows
+        for (int k = 1; k < K; ++k) { if (hipEventRecord(P->front_done[k], P->ctx[k - 1]->stream) != hipSuccess || hipStreamWaitEvent(ctx->stream, P->front_done[k], 0) != hipSuccess) { join(); return bail(pyre_fail(ctx, PYRE_E_HIP, "event failed"), ctx); } }
+        if ((rc = pyre_moe_block_launch(ctx, m->layers[il].moe, P->blk, NB * 8, NBMAX * 8, P->blk_nsl, P->blk_r64))) { join(); return bail(rc, ctx); }
+        if (hipEventRecord(P->moe_done, ctx->stream) != hipSuccess) { join(); return bail(pyre_fail(ctx, PYRE_E_HIP, "hipEventRecord failed"), ctx); }
+        for (int j = 0; j < NB; ++j) runs[j].moe_from_block();
+      }
+      for (auto& w : workers) w.join();
+      workers.clear();
+      s->len = pos0 + NB * 8; i_first += NB * 8; prev = (NB - 1) % K; ++P->blocks_done;
+    }
+    if (i_first > 0) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipEventRecord(P->done[k], P->ctx[k - 1]->stream));
+  }
+  const int nwin_tail = (n - i_first + 7) / 8;
+  for (int i = i_first, w = 0; i < n; i += 8, ++w) {
     int t = n - i < 8 ? n - i : 8; bool last = i + t >= n;
     WinOpt o; o.head_tokens = last && logits_host ? 1 : 0;
     if (s->mtp) { const int k0 = n - mtp_window_of(s->mtp) - i; o.keep_from = k0 < 0 ? 0 : k0; }      // the last `window` tokens of a call (qwen4exp_gguf.rs:2148-2150)
@@ -662,7 +856,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
       if ((rc = run_window(ctx, m, s, t, o))) { s->broken = true; return rc; }
       continue;
     }
-    const int set = (nwin - 1 - w) % K;          // the last window runs on the model's own stream and workspace: its logits are the call's
+    const int set = (nwin_tail - 1 - w) % K;          // the last window runs on the model's own stream and workspace: its logits are the call's
     pyre_ctx* cx = set ? P->ctx[set - 1] : ctx; const pyre_model* mx = set ? P->mdl[set - 1] : m;
     o.ids_dev = P->ids + i; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
     o.wait_ev = prev >= 0 ? P->ev[prev].data() : nullptr; o.rec_ev = P->ev[set].data();
@@ -671,6 +865,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     if (rc) { s->broken = true; if (cx != ctx) pyre_fail(ctx, rc, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return rc; }      // windows already issued have advanced the bookkeeping and part of the state
     prev = set;
   }
+  if (getenv("PYRE_DEBUG_ENQ")) { static auto t_prev = std::chrono::steady_clock::now(); auto t1 = std::chrono::steady_clock::now(); fprintf(stderr, "enq %d tokens (%d in blocks): %.3f ms since entry\n", n, i_first, std::chrono::duration<double>(t1 - t_enter).count() * 1e3); (void)t_prev; }
   if (P) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, P->done[k], 0));      // everything the other streams did precedes what follows here
   if (logits_host) PYRE_HIP(ctx, hipMemcpyAsync(logits_host, m->logits, (size_t)m->c.vocab * 4, hipMemcpyDeviceToHost, ctx->stream));
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream)); return PYRE_OK;

@@ -4,6 +4,7 @@
 // and top_k / soft_top / nan_clean, :3121-3139.  All experts are resident in HBM, so there is no host split.
 #include "formats.h"
 #include "digits.h"
+#include "gemm_m.h"
 PYRE_TS_DECL(moe_ts) PYRE_TS_EXPORT(moe_ts, pyre_debug_ts_moe)
 
 // ---- router: top-k (ties -> lower index), softmax over the chosen k in ascending expert id -----------------------------
@@ -471,6 +472,7 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
   if (t < 1 || t > 8) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: t = %d outside 1..8", t);
   if (!y && m.top_k > PYRE_MOE_KMAX) return pyre_fail(ctx, PYRE_E_SHAPE, "moe_ffn: an unreduced output needs top_k <= %d", PYRE_MOE_KMAX);
   if (routed && (routed->nsl < 1 || routed->nsl > 64 || routed->r64 < m.n_exp)) return pyre_fail(ctx, PYRE_E_ARG, "moe_ffn: %d router slices of %d rows", routed->nsl, routed->r64);
+  if (t > 1 && getenv("PYRE_DEBUG_SKIP_MOE")) return PYRE_OK;
   if (!routed) { int rc = pyre_gemv_launch(ctx, m.router, x, t, w.logits); if (rc) return rc; }
   const float* lg = routed ? routed->p : w.logits; const int nsl = routed ? routed->nsl : 1, sstride = routed ? t * routed->r64 : 0, tstride = routed ? routed->r64 : m.n_exp;
   auto mat_bytes = [](const QMatDev& q, double rows) { return qmat_gguf_bytes(q, rows); };
@@ -529,6 +531,217 @@ int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const floa
     hipLaunchKernelGGL(k_moe_sum, dim3((m.d + 255) / 256, t), dim3(256), 0, ctx->stream, w.partial, w.sel_w, w.sg, m.d, m.top_k, y);
     PYRE_CHECK_LAUNCH(ctx);
   }
+  return PYRE_OK;
+}
+
+// ---- the FFN of a block of prompt windows, the tokens grouped by expert ------------------------------------------------------
+// A long prompt is run layer by layer over blocks of up to 32 windows of eight tokens (model.hip); between a layer's FFN mixes
+// and the next layer the FFN of all of the block's tokens runs here: an expert's weights are fetched once for all of its
+// tokens (a window by itself picks eight tokens x 10 of 512 experts and shares nothing).  A token's arithmetic is that of
+// the window kernels above, in the same order (k_moe_route, k_moe_gu<.., 2, true, .., ID>, k_moe_down_groups<.., ID>): its
+// bits do not depend on which path ran.  IQ3_S experts in the integer form only, gate / up rows of 32 units, expert widths
+// of at most 8 units.
+template <bool FIX>
+__global__ __launch_bounds__(1024) void k_moe_route_blk(MoeDev m, MoeBlk b, int nsl, int r64) {
+  __shared__ RouteLds rl;
+  const int ti = blockIdx.x, w = ti >> 3, tw = ti & 7;
+  const int n_exp = FIX ? 512 : m.n_exp, top_k = FIX ? 10 : m.top_k;
+  if constexpr (FIX) nsl = 32;
+#ifdef PYRE_PHASE_TS
+  unsigned long long ts_[8];
+#endif
+  route_topk(b.rpart + ((size_t)w * nsl * 8 + tw) * r64, nsl, 8 * r64, n_exp, top_k, rl ROUTE_TS_ARG);
+  route_weights(top_k, rl);
+  if ((int)threadIdx.x < top_k) { b.sel_idx[ti * top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; b.sel_w[ti * top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
+}
+// the (token, choice) pairs of the block by expert: eoff[e] .. eoff[e + 1] of elist hold expert e's entries token * (k + 1) + j
+// (in no particular order: a token's sums do not depend on its neighbours).  One workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void k_moe_lists(MoeDev m, MoeBlk b, int T) {
+  __shared__ int cnt[1024], cur[1024];
+  const int tid = threadIdx.x, k = m.top_k, np = T * k;
+  cnt[tid] = 0;
+  __syncthreads();
+  for (int p = tid; p < np; p += 1024) atomicAdd(&cnt[b.sel_idx[p]], 1);
+  __syncthreads();
+  const int own = cnt[tid]; int v = own;
+  for (int o = 1; o < 1024; o <<= 1) { cur[tid] = v; __syncthreads(); const int a = tid >= o ? cur[tid - o] : 0; __syncthreads(); v += a; }
+  cur[tid] = v - own;            // exclusive prefix
+  if (tid <= m.n_exp) b.eoff[tid] = tid < m.n_exp ? v - own : np;
+  __syncthreads();
+  for (int p = tid; p < np; p += 1024) { const int pos = atomicAdd(&cur[b.sel_idx[p]], 1); b.elist[pos] = (p / k) * (k + 1) + p % k; }
+}
+// What a workgroup of the two kernels below works on: blockIdx.y < n_exp: the routed expert's entries; above: eight tokens'
+// entries of the shared expert.
+struct BlkEntries { int n; const int32_t* list; int first; int step; };
+__device__ __forceinline__ BlkEntries blk_entries(const MoeDev& m, const MoeBlk& b, int T, int ye) {
+  BlkEntries e;
+  if (ye < m.n_exp) { const int e0 = b.eoff[ye]; e.n = b.eoff[ye + 1] - e0; e.list = b.elist + e0; e.first = 0; e.step = 0; }
+  else { const int t0 = (ye - m.n_exp) * 8; e.n = min(8, T - t0); e.list = nullptr; e.first = t0 * (m.top_k + 1) + m.top_k; e.step = m.top_k + 1; }
+  return e;
+}
+__device__ __forceinline__ int blk_entry(const BlkEntries& e, int i) { return e.list ? e.list[i] : e.first + i * e.step; }
+
+// f32 rows -> the matrix cores' operand, a row at a time: row r of x [n][cols] as its two f16 halves xh[r][0 / 1][cols], each
+// 256-column stretch on its own power of two (the arithmetic of k_act_split, gemm_m.hip), the inverse factors in
+// inv[r][cols / 256].  x2 given: the row is silu(x) * x2 (an expert's h out of its gate and up products).  gate_inp given:
+// sg[r] = sigmoid(gate_inp . x[r]) as well (the shared expert's gate).  grid (n), 256 threads, a stretch a round.  Row n of
+// xh is kept zero by the owner: the operand rows a pass has no token for point there.
+__global__ __launch_bounds__(256) void k_blk_split(const float* __restrict__ x, const float* __restrict__ x2, int cols, uint16_t* __restrict__ xh, float* __restrict__ inv, const float* __restrict__ gate_inp, float* __restrict__ sg) {
+  __shared__ float mx[2][4]; __shared__ float dp[4];
+  const int r = blockIdx.x, i = threadIdx.x, wave = i >> 6, lane = i & 63;
+  float dot = 0.0f;
+  for (int sb = 0; sb < (cols >> 8); ++sb) {
+    const int k = sb * 256 + i;
+    float v = x[(size_t)r * cols + k];
+    if (x2) { const float sgm = 1.0f / (1.0f + expf(-v)); v = (v * sgm) * x2[(size_t)r * cols + k]; }
+    if (gate_inp) dot = fmaf(gate_inp[k], v, dot);
+    float a = fabsf(v); a = a == a ? a : INFINITY;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) a = fmaxf(a, __shfl_xor(a, o));
+    if (lane == 0) mx[sb & 1][wave] = a;
+    __syncthreads();            // (the two halves of mx take turns: one barrier a round)
+    const float mv = fmaxf(fmaxf(mx[sb & 1][0], mx[sb & 1][1]), fmaxf(mx[sb & 1][2], mx[sb & 1][3]));
+    int e = 0;
+    if (mv > 0.0f && mv < INFINITY) { e = 140 - (int)((__float_as_uint(mv) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+    const float up = __uint_as_float((uint32_t)(127 + e) << 23), dn = __uint_as_float((uint32_t)(127 - e) << 23);
+    const float xs = v * up;
+    const _Float16 h1 = (_Float16)xs, h2 = (_Float16)((xs - (float)h1) * 2048.0f);
+    xh[((size_t)r * 2) * cols + k] = __builtin_bit_cast(unsigned short, h1); xh[((size_t)r * 2 + 1) * cols + k] = __builtin_bit_cast(unsigned short, h2);
+    if (i == 0) inv[(size_t)r * (cols >> 8) + sb] = dn;
+  }
+  if (gate_inp) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
+    if (lane == 0) dp[wave] = dot;
+    __syncthreads();
+    if (i == 0) sg[r] = 1.0f / (1.0f + expf(-(((dp[0] + dp[1]) + dp[2]) + dp[3])));
+  }
+}
+// the sixteen operand rows of a pass for chunk c: lane (kg, r) takes the eight columns 32 s + 8 kg .. of half r & 1 of the row
+// its slot r >> 1 names; the scale factors of the two slots whose sums the lane holds
+__device__ __forceinline__ void load_a_rows(const uint16_t* __restrict__ p, const float* __restrict__ i0, const float* __restrict__ i1, int c, ABuf& b) {
+#pragma unroll
+  for (int s = 0; s < 4; ++s) b.a[s] = *(const uint4*)(p + c * 128 + s * 32);
+  b.ai0 = i0[c >> 1]; b.ai1 = i1[c >> 1];
+}
+
+// The expert products of a block on the matrix cores.  DOWN = false: gate and up (blockIdx.z), grid (ff / 64, n_exp +
+// ceil(T / 8), 2), operand rows of x by token, out g / u [entry][ff]; DOWN = true: grid (d / 64, same, 1), operand rows of h
+// by entry, out the unreduced terms partial[entry][d].  4 waves: the workgroup owns 64 rows of its expert's matrix
+// (FMT_IQ3_S_M); its entries go through in passes of eight (sixteen operand rows); wave w walks the 128-column chunks
+// [w * cpw, + cpw) with two register buffers taking turns, the waves' sums meet in shared memory in wave order.  A weight is
+// decoded once a pass, whatever the pass holds.
+template <bool DOWN>
+__global__ __launch_bounds__(256, 3) void k_moe_mm_blk(MoeDev m, MoeBlk b, int T, int zrow) {            // zrow: the operand's zero row
+  constexpr int NW = 4;
+  __shared__ float red[NW][4][2][64];
+  __shared__ float zero_inv[64];
+  const int ye = blockIdx.y; const bool shared = ye >= m.n_exp;
+  const BlkEntries E = blk_entries(m, b, T, ye);
+  if (E.n <= 0) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, k1 = m.top_k + 1;
+  const QMatDev& W = DOWN ? (shared ? m.sh_down_m : m.down_m) : (blockIdx.z ? (shared ? m.sh_up_m : m.up_m) : (shared ? m.sh_gate_m : m.gate_m));
+  const int rows = DOWN ? m.d : m.ff, kc = DOWN ? m.ff : m.d;
+  const uint16_t* opnd = DOWN ? b.hh : b.xh; const float* inv = DOWN ? b.hinv : b.xinv;
+  float* out = DOWN ? b.partial : (blockIdx.z ? b.u : b.g);
+  const int tile = (shared ? 0 : ye * (rows >> 6)) + blockIdx.x;
+  const int K128 = kc >> 7, nsb = kc >> 8, cpw = (K128 + NW - 1) / NW, c0 = min(K128, wave * cpw), c1 = min(K128, c0 + cpw);
+  if (threadIdx.x < 64) zero_inv[threadIdx.x] = 0.0f;
+  lds_barrier();
+  const NibK nk = nib_consts();
+  const int kg = lane >> 4, r = lane & 15, slot = r >> 1, half = r & 1, q = lane >> 4;
+  for (int i0 = 0; i0 < E.n; i0 += 8) {
+    const int np = min(8, E.n - i0);
+    auto row_of = [&](int sl) { const int en = blk_entry(E, i0 + sl); return DOWN ? en : en / k1; };
+    const size_t myrow = slot < np ? (size_t)row_of(slot) : (size_t)zrow;
+    const uint16_t* ap = opnd + (myrow * 2 + half) * kc + kg * 8;
+    const float* ip0 = 2 * q < np ? inv + (size_t)row_of(2 * q) * nsb : zero_inv;            // (a slot without a token: factor 0, its sums are never read)
+    const float* ip1 = 2 * q + 1 < np ? inv + (size_t)row_of(2 * q + 1) * nsb : zero_inv;
+    v4f tot[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    WBuf<4> w0, w1; ABuf a0, a1;
+    if (c0 < c1) { load_a_rows(ap, ip0, ip1, c0, a0); load_w<4>(W, tile * 4, c0, lane, K128, w0); }
+    for (int c = c0; c < c1; c += 2) {
+      if (c + 1 < c1) { load_a_rows(ap, ip0, ip1, c + 1, a1); load_w<4>(W, tile * 4, c + 1, lane, K128, w1); }
+      __builtin_amdgcn_sched_barrier(0);
+      chunk_mac<4>(w0, a0, c, nk, tot);
+      __builtin_amdgcn_sched_barrier(0);
+      if (c + 2 < c1) { load_a_rows(ap, ip0, ip1, c + 2, a0); load_w<4>(W, tile * 4, c + 2, lane, K128, w0); }
+      __builtin_amdgcn_sched_barrier(0);
+      if (c + 1 < c1) chunk_mac<4>(w1, a1, c + 1, nk, tot);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) { red[wave][g][0][lane] = tot[g][0] + tot[g][1] * (1.0f / 2048.0f); red[wave][g][1][lane] = tot[g][2] + tot[g][3] * (1.0f / 2048.0f); }
+    lds_barrier();
+    for (int i = threadIdx.x; i < np * 64; i += NW * 64) {
+      const int t = i >> 6, rl = i & 63, l = (t >> 1) * 16 + (rl & 15), g = rl >> 4, h = t & 1;
+      float sv = red[0][g][h][l];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) sv += red[w][g][h][l];
+      out[(size_t)blk_entry(E, i0 + t) * rows + blockIdx.x * 64 + rl] = sv;
+    }
+    lds_barrier();
+  }
+}
+// the four group sums of every token (moe_out_value's groups, folded as k_moe_down_groups folds them) into the token's
+// window: grid (d / 256, T), thread = row
+__global__ __launch_bounds__(256) void k_moe_groups_blk(MoeDev m, MoeBlk b, int T) {
+  const int r = blockIdx.x * 256 + threadIdx.x, ti = blockIdx.y, k = m.top_k, d = m.d, gsz = (k + 4) / 4;
+  if (r >= d) return;
+  const float* pt = b.partial + (size_t)ti * (k + 1) * d + r;
+  float* out = b.parts + (size_t)(ti >> 3) * PYRE_MOE_GROUPS * 8 * d + (size_t)(ti & 7) * d + r;
+#pragma unroll
+  for (int q = 0; q < PYRE_MOE_GROUPS; ++q) {
+    const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;
+    float o = 0.0f;
+    for (int e = 0; e < nr; ++e) o = fmaf(b.sel_w[ti * k + j0 + e], pt[(size_t)(j0 + e) * d], o);
+    if (q == PYRE_MOE_GROUPS - 1) o = fmaf(pt[(size_t)k * d], b.sg[ti], o);            // the shared expert comes last
+    out[(size_t)q * 8 * d] = o;
+  }
+}
+
+static bool is_m(const QMatDev& q) { return q.fmt == FMT_IQ3_S_M && q.mq && q.mh; }
+bool pyre_moe_block_ok(const MoeDev& m) {
+  return is_m(m.gate_m) && is_m(m.up_m) && is_m(m.down_m) && is_m(m.sh_gate_m) && is_m(m.sh_up_m) && is_m(m.sh_down_m) && m.d % 256 == 0 && m.ff % 256 == 0 && m.sf == m.ff &&
+         m.n_exp <= 1023 && pyre_moe_groups_ok(m);
+}
+size_t pyre_moe_block_bytes(const MoeDev& m, int T) {
+  const size_t hs = (size_t)m.ff, k1 = m.top_k + 1, n = (size_t)T, ne = n * k1;
+  return 256 * 12 + 4 * (2 * n * m.top_k + n + 1024 + n * m.top_k + 2 * ne * hs + ne * (size_t)m.d + ne * (hs / 256) + n * (m.d / 256)) + 2 * (2 * (n + 1) * m.d + 2 * (ne + 1) * hs);
+}
+void pyre_moe_block_carve(const MoeDev& m, int T, void* base, MoeBlk* b) {
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += (n + 255) & ~(size_t)255; return r; };
+  const size_t hs = (size_t)m.ff, k1 = m.top_k + 1, n = (size_t)T, ne = n * k1;
+  b->sel_idx = (int32_t*)take(4 * n * m.top_k); b->sel_w = (float*)take(4 * n * m.top_k); b->sg = (float*)take(4 * n); b->eoff = (int32_t*)take(4 * 1024); b->elist = (int32_t*)take(4 * n * m.top_k);
+  b->g = (float*)take(4 * ne * hs); b->u = (float*)take(4 * ne * hs); b->partial = (float*)take(4 * ne * (size_t)m.d);
+  b->xh = (uint16_t*)take(2 * 2 * (n + 1) * m.d); b->xinv = (float*)take(4 * n * (m.d / 256));
+  b->hh = (uint16_t*)take(2 * 2 * (ne + 1) * hs); b->hinv = (float*)take(4 * ne * (hs / 256));
+}
+// the rows no token owns: row T of xh, row T * (top_k + 1) of hh (once, when the block's scratch is made: for the largest T)
+int pyre_moe_block_zero_rows(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T) {
+  const size_t hs = (size_t)m.ff, ne = (size_t)T * (m.top_k + 1);
+  PYRE_HIP(ctx, hipMemsetAsync(b.xh + (size_t)2 * T * m.d, 0, 2 * 2 * (size_t)m.d, ctx->stream));
+  PYRE_HIP(ctx, hipMemsetAsync(b.hh + 2 * ne * hs, 0, 2 * 2 * hs, ctx->stream));
+  return PYRE_OK;
+}
+// T = 8 * windows tokens (T_max: the T the scratch was carved and its zero rows were set for); the router's K-slice sums (nsl
+// slices of r64 rows a token) come from the mixes
+int pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64) {
+  if (!pyre_moe_block_ok(m) || T < 8 || T % 8 || T > T_max || nsl < 1 || nsl > 64 || r64 < m.n_exp) return pyre_fail(ctx, PYRE_E_ARG, "moe block: unsupported shape (T = %d, %d router slices)", T, nsl);
+  const int hs = m.ff, ny = m.n_exp + (T + 7) / 8, ne = T * (m.top_k + 1), ne_max = T_max * (m.top_k + 1);
+  const bool fix = m.n_exp == 512 && m.top_k == 10 && nsl == 32;
+  { ProfScope ps(ctx, "moe_block_route", 4.0 * T * nsl * m.n_exp);
+    if (fix) hipLaunchKernelGGL(k_moe_route_blk<true>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64); else hipLaunchKernelGGL(k_moe_route_blk<false>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64);
+    hipLaunchKernelGGL(k_moe_lists, dim3(1), dim3(1024), 0, ctx->stream, m, b, T);
+    hipLaunchKernelGGL(k_blk_split, dim3(T), dim3(256), 0, ctx->stream, b.x, (const float*)nullptr, m.d, b.xh, b.xinv, m.sh_gate_inp, b.sg); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "moe_block_gate_up", 2.0 * m.n_exp * qmat_gguf_bytes(m.gate_e, m.ff) + 2.0 * qmat_gguf_bytes(m.sh_gate, m.sf));
+    hipLaunchKernelGGL(k_moe_mm_blk<false>, dim3(hs / 64, ny, 2), dim3(256), 0, ctx->stream, m, b, T, T_max);
+    hipLaunchKernelGGL(k_blk_split, dim3(ne), dim3(256), 0, ctx->stream, (const float*)b.g, (const float*)b.u, hs, b.hh, b.hinv, (const float*)nullptr, (float*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "moe_block_down", (double)m.n_exp * qmat_gguf_bytes(m.down_e, m.d) + qmat_gguf_bytes(m.sh_down, m.d));
+    hipLaunchKernelGGL(k_moe_mm_blk<true>, dim3(m.d / 64, ny, 1), dim3(256), 0, ctx->stream, m, b, T, ne_max);
+    hipLaunchKernelGGL(k_moe_groups_blk, dim3((m.d + 255) / 256, T), dim3(256), 0, ctx->stream, m, b, T); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

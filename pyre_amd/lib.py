@@ -101,6 +101,7 @@ def _declare(L):
         "pyre_model_create": (i32, [vp, vp, vp, vp, C.POINTER(vp)]),
         "pyre_model_destroy": (None, [vp]),
         "pyre_model_weight_bytes_per_token": (sz, [vp]),
+        "pyre_model_prompt_blocks": (sz, [vp]),
         "pyre_state_create": (i32, [vp, vp, i32, C.POINTER(vp)]),
         "pyre_state_destroy": (None, [vp]),
         "pyre_state_reset": (i32, [vp, vp]),
@@ -685,6 +686,10 @@ class Model:
     @property
     def weight_bytes_per_token(self):
         return self.ctx.L.pyre_model_weight_bytes_per_token(self.h)
+
+    def prompt_blocks(self):
+        """Blocks of 256 prompt tokens taken layer by layer with the FFN grouped by expert since the model was created."""
+        return self.ctx.L.pyre_model_prompt_blocks(self.h)
 
     def new_state(self, max_ctx):
         return State(self, max_ctx)

@@ -202,7 +202,7 @@ def test_vocab_head_every_sweep_format_and_width(ctx, ty):
         assert np.isfinite(y).all()
         if y8 is None:
             y8 = y
-        elif ty in (lib.IQ3_S, lib.IQ2_XS, lib.Q4_K) and t == 1:        # (one token of an IQ3_S, IQ2_XS or Q4_K matrix takes the native-format kernel: equal to rounding)
+        elif ty in (lib.IQ3_S, lib.IQ2_XS, lib.Q4_K, lib.Q8_0) and t == 1:        # (one token of an IQ3_S, IQ2_XS or Q4_K matrix takes the native-format kernel, of a Q8_0 matrix the lane = row one, windows the matrix cores: equal to rounding)
             assert relerr(y, y8[:1]) <= 2e-6
         else:                                   # a token's row does not depend on the window it was computed in
             assert np.array_equal(y.view(np.uint32), y8[:t].view(np.uint32)), t

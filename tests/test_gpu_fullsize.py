@@ -108,3 +108,48 @@ def test_drafter_matches_the_oracle_at_full_width(ctx):
     out, rounds, drafted, accepted = gd.generate_greedy(gs, lg, 9, k=3)
     oo, od_n, oa_n = od.generate_greedy(os_, lo, 9, k=3)
     assert np.array_equal(out, oo) and (drafted, accepted) == (od_n, oa_n)
+
+
+def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows_path(ctx, model4, monkeypatch):
+    """A long prompt takes blocks of 32 windows layer by layer, the FFN of a block's 256 tokens grouped by expert on the
+    matrix cores: logits agree with the windows' path (PYRE_PROMPT_BLOCK=0 at run time) to rounding, the tokens that follow
+    and the state's length are the same, for a call that is whole blocks plus a ragged tail, and for a state that continues
+    with a second long call."""
+    cfg, gm = model4
+    g = np.random.Generator(np.random.PCG64(21))
+    prompt = g.integers(0, cfg.vocab, 2 * 256 + 45, dtype=np.uint32)
+    more = g.integers(0, cfg.vocab, 256 + 100 + 9, dtype=np.uint32)          # a full block and a shorter one
+    out = {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("PYRE_PROMPT_WINDOWS", "1" if mode == "0" else "0")
+        st = gm.new_state(1024)
+        n0 = gm.prompt_blocks()
+        lg = gm.forward(prompt, st)
+        assert gm.prompt_blocks() - n0 == (2 if mode == "1" else 0)          # the path under test is the one that ran
+        toks = gm.decode_greedy_dev(st, int(np.argmax(lg)), 6)
+        lg2 = gm.forward(more, st)                                           # (starts at a position that is no multiple of eight)
+        toks2 = gm.decode_greedy_dev(st, int(np.argmax(lg2)), 4)
+        out[mode] = (lg.copy(), toks.copy(), lg2.copy(), toks2.copy(), len(st))
+        st.close()
+    a, b = out["0"], out["1"]
+    assert a[4] == b[4] == prompt.size + 6 + more.size + 4
+    assert relerr(b[0], a[0]) <= 1e-4 and np.array_equal(a[1], b[1])
+    assert relerr(b[2], a[2]) <= 1e-4 and np.array_equal(a[3], b[3])
+
+
+def test_prompt_in_blocks_matches_the_oracle_at_full_width(ctx):
+    """One block of 256 tokens plus a tail through the two-layer slice against the oracle's token-by-token prompt."""
+    cfg = mg.a3b_config(n_layers=2, full_every=2)
+    hw = mg.build_host(cfg, seed=8)
+    gm = lib.Model(ctx, cfg, hw.layers, hw.globals_); om = orc_model(hw, threads=min(os.cpu_count() or 1, 16))
+    g = np.random.Generator(np.random.PCG64(23))
+    prompt = g.integers(0, cfg.vocab, 256 + 19, dtype=np.uint32)
+    gs, os_ = gm.new_state(512), om.new_state()
+    lg = gm.forward(prompt, gs)
+    assert gm.prompt_blocks() == 1
+    lo = om.forward(prompt, os_)
+    assert relerr(lg, lo) <= 1e-3
+    tg, _ = gm.generate_greedy(gs, lg, 4); to, _ = om.generate_greedy(os_, lo, 4)
+    assert np.array_equal(tg, to)
+    conv, ssm = gs.gdn(0)
+    assert relerr(ssm, os_.ssm(0)) <= 1e-3 and relerr(conv, os_.conv(0)) <= 1e-4

@@ -213,7 +213,8 @@ def test_verify_window_equals_single_steps_and_rollback(ctx):
 
 
 @pytest.mark.parametrize("kind", ["plain", "iq3s_mixes", "ple", "indexer"])
-def test_long_prompt_on_several_streams_equals_short_calls_on_one(ctx, kind):
+def test_long_prompt_on_several_streams_equals_short_calls_on_one(ctx, kind, monkeypatch):
+    monkeypatch.setenv("PYRE_PROMPT_WINDOWS", "1")          # (the windows' path: a model whose experts qualify would take the long call in blocks, equal to rounding only)
     # A call of 2 * 3 windows or more runs its windows on three streams, a window entering a layer when the previous one has
     # left that layer's state; shorter calls run on the model's own stream.  Same logits, recurrent state, caches and
     # continuation, bit for bit (250 tokens: the 4-bit boundary moves several times, ragged last window).
