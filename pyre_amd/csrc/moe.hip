@@ -625,29 +625,26 @@ __device__ __forceinline__ void load_a_rows(const uint16_t* __restrict__ p, cons
   b.ai0 = i0[c >> 1]; b.ai1 = i1[c >> 1];
 }
 
-// The expert products of a block on the matrix cores.  DOWN = false: gate and up (blockIdx.z), grid (ff / 64, n_exp +
-// ceil(T / 8), 2), operand rows of x by token, out g / u [entry][ff]; DOWN = true: grid (d / 64, same, 1), operand rows of h
-// by entry, out the unreduced terms partial[entry][d].  4 waves: the workgroup owns 64 rows of its expert's matrix
-// (FMT_IQ3_S_M); its entries go through in passes of eight (sixteen operand rows); wave w walks the 128-column chunks
-// [w * cpw, + cpw) with two register buffers taking turns, the waves' sums meet in shared memory in wave order.  A weight is
-// decoded once a pass, whatever the pass holds.
+// The expert products of a block on the matrix cores.  DOWN = false: gate and up (blockIdx.z), grid (ff / 256, n_exp +
+// ceil(T / 8), 2), operand rows of x by token, out g / u [entry][ff]; DOWN = true: grid (d / 256, same, 1), operand rows of h
+// by entry, out the unreduced terms partial[entry][d].  4 waves, each with 64 rows of its expert's matrix (FMT_IQ3_S_M) of
+// its own: the wave walks all of the row tile's 128-column chunks with two register buffers taking turns and writes its sums
+// itself -- no shared memory, no barrier.  The workgroup's entries go through in passes of eight (sixteen operand rows); a
+// weight is decoded once a pass, whatever the pass holds.
 template <bool DOWN>
 __global__ __launch_bounds__(256, 3) void k_moe_mm_blk(MoeDev m, MoeBlk b, int T, int zrow) {            // zrow: the operand's zero row
-  constexpr int NW = 4;
-  __shared__ float red[NW][4][2][64];
-  __shared__ float zero_inv[64];
   const int ye = blockIdx.y; const bool shared = ye >= m.n_exp;
   const BlkEntries E = blk_entries(m, b, T, ye);
   if (E.n <= 0) return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, k1 = m.top_k + 1;
   const QMatDev& W = DOWN ? (shared ? m.sh_down_m : m.down_m) : (blockIdx.z ? (shared ? m.sh_up_m : m.up_m) : (shared ? m.sh_gate_m : m.gate_m));
   const int rows = DOWN ? m.d : m.ff, kc = DOWN ? m.ff : m.d;
+  const int rt = blockIdx.x * 4 + wave;            // the wave's row tile inside the expert
+  if (rt * 64 >= rows) return;
   const uint16_t* opnd = DOWN ? b.hh : b.xh; const float* inv = DOWN ? b.hinv : b.xinv;
   float* out = DOWN ? b.partial : (blockIdx.z ? b.u : b.g);
-  const int tile = (shared ? 0 : ye * (rows >> 6)) + blockIdx.x;
-  const int K128 = kc >> 7, nsb = kc >> 8, cpw = (K128 + NW - 1) / NW, c0 = min(K128, wave * cpw), c1 = min(K128, c0 + cpw);
-  if (threadIdx.x < 64) zero_inv[threadIdx.x] = 0.0f;
-  lds_barrier();
+  const int tile = (shared ? 0 : ye * (rows >> 6)) + rt;
+  const int K128 = kc >> 7, nsb = kc >> 8;
   const NibK nk = nib_consts();
   const int kg = lane >> 4, r = lane & 15, slot = r >> 1, half = r & 1, q = lane >> 4;
   for (int i0 = 0; i0 < E.n; i0 += 8) {
@@ -655,34 +652,32 @@ __global__ __launch_bounds__(256, 3) void k_moe_mm_blk(MoeDev m, MoeBlk b, int T
     auto row_of = [&](int sl) { const int en = blk_entry(E, i0 + sl); return DOWN ? en : en / k1; };
     const size_t myrow = slot < np ? (size_t)row_of(slot) : (size_t)zrow;
     const uint16_t* ap = opnd + (myrow * 2 + half) * kc + kg * 8;
-    const float* ip0 = 2 * q < np ? inv + (size_t)row_of(2 * q) * nsb : zero_inv;            // (a slot without a token: factor 0, its sums are never read)
-    const float* ip1 = 2 * q + 1 < np ? inv + (size_t)row_of(2 * q + 1) * nsb : zero_inv;
+    const bool on0 = 2 * q < np, on1 = 2 * q + 1 < np;
+    const float* ip0 = inv + (size_t)(on0 ? row_of(2 * q) : 0) * nsb;            // (a slot without a token reads some row's factors: its sums are never written)
+    const float* ip1 = inv + (size_t)(on1 ? row_of(2 * q + 1) : 0) * nsb;
     v4f tot[4];
 #pragma unroll
     for (int g = 0; g < 4; ++g) tot[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     WBuf<4> w0, w1; ABuf a0, a1;
-    if (c0 < c1) { load_a_rows(ap, ip0, ip1, c0, a0); load_w<4>(W, tile * 4, c0, lane, K128, w0); }
-    for (int c = c0; c < c1; c += 2) {
-      if (c + 1 < c1) { load_a_rows(ap, ip0, ip1, c + 1, a1); load_w<4>(W, tile * 4, c + 1, lane, K128, w1); }
+    load_a_rows(ap, ip0, ip1, 0, a0); load_w<4>(W, tile * 4, 0, lane, K128, w0);
+    for (int c = 0; c < K128; c += 2) {
+      if (c + 1 < K128) { load_a_rows(ap, ip0, ip1, c + 1, a1); load_w<4>(W, tile * 4, c + 1, lane, K128, w1); }
       __builtin_amdgcn_sched_barrier(0);
       chunk_mac<4>(w0, a0, c, nk, tot);
       __builtin_amdgcn_sched_barrier(0);
-      if (c + 2 < c1) { load_a_rows(ap, ip0, ip1, c + 2, a0); load_w<4>(W, tile * 4, c + 2, lane, K128, w0); }
+      if (c + 2 < K128) { load_a_rows(ap, ip0, ip1, c + 2, a0); load_w<4>(W, tile * 4, c + 2, lane, K128, w0); }
       __builtin_amdgcn_sched_barrier(0);
-      if (c + 1 < c1) chunk_mac<4>(w1, a1, c + 1, nk, tot);
+      if (c + 1 < K128) chunk_mac<4>(w1, a1, c + 1, nk, tot);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // lane (q, j) holds, for row group g, token slot 2q (halves h1, h2 * 2^11 in rows 0, 1 of its four) and slot 2q + 1
+    float* o0 = on0 ? out + (size_t)blk_entry(E, i0 + 2 * q) * rows + rt * 64 + r : nullptr;
+    float* o1 = on1 ? out + (size_t)blk_entry(E, i0 + 2 * q + 1) * rows + rt * 64 + r : nullptr;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) { red[wave][g][0][lane] = tot[g][0] + tot[g][1] * (1.0f / 2048.0f); red[wave][g][1][lane] = tot[g][2] + tot[g][3] * (1.0f / 2048.0f); }
-    lds_barrier();
-    for (int i = threadIdx.x; i < np * 64; i += NW * 64) {
-      const int t = i >> 6, rl = i & 63, l = (t >> 1) * 16 + (rl & 15), g = rl >> 4, h = t & 1;
-      float sv = red[0][g][h][l];
-#pragma unroll
-      for (int w = 1; w < NW; ++w) sv += red[w][g][h][l];
-      out[(size_t)blk_entry(E, i0 + t) * rows + blockIdx.x * 64 + rl] = sv;
+    for (int g = 0; g < 4; ++g) {
+      if (o0) o0[g * 16] = tot[g][0] + tot[g][1] * (1.0f / 2048.0f);
+      if (o1) o1[g * 16] = tot[g][2] + tot[g][3] * (1.0f / 2048.0f);
     }
-    lds_barrier();
   }
 }
 // the four group sums of every token (moe_out_value's groups, folded as k_moe_down_groups folds them) into the token's
@@ -737,10 +732,10 @@ int pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T
     hipLaunchKernelGGL(k_moe_lists, dim3(1), dim3(1024), 0, ctx->stream, m, b, T);
     hipLaunchKernelGGL(k_blk_split, dim3(T), dim3(256), 0, ctx->stream, b.x, (const float*)nullptr, m.d, b.xh, b.xinv, m.sh_gate_inp, b.sg); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_block_gate_up", 2.0 * m.n_exp * qmat_gguf_bytes(m.gate_e, m.ff) + 2.0 * qmat_gguf_bytes(m.sh_gate, m.sf));
-    hipLaunchKernelGGL(k_moe_mm_blk<false>, dim3(hs / 64, ny, 2), dim3(256), 0, ctx->stream, m, b, T, T_max);
+    hipLaunchKernelGGL(k_moe_mm_blk<false>, dim3((hs + 255) / 256, ny, 2), dim3(256), 0, ctx->stream, m, b, T, T_max);
     hipLaunchKernelGGL(k_blk_split, dim3(ne), dim3(256), 0, ctx->stream, (const float*)b.g, (const float*)b.u, hs, b.hh, b.hinv, (const float*)nullptr, (float*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_block_down", (double)m.n_exp * qmat_gguf_bytes(m.down_e, m.d) + qmat_gguf_bytes(m.sh_down, m.d));
-    hipLaunchKernelGGL(k_moe_mm_blk<true>, dim3(m.d / 64, ny, 1), dim3(256), 0, ctx->stream, m, b, T, ne_max);
+    hipLaunchKernelGGL(k_moe_mm_blk<true>, dim3((m.d + 255) / 256, ny, 1), dim3(256), 0, ctx->stream, m, b, T, ne_max);
     hipLaunchKernelGGL(k_moe_groups_blk, dim3((m.d + 255) / 256, T), dim3(256), 0, ctx->stream, m, b, T); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
