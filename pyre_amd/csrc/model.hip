@@ -809,8 +809,8 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
         }
         return PYRE_OK;
       };
-      std::vector<std::thread> workers;
-      if (threads) for (int k = 1; k < K; ++k) workers.emplace_back([&, k] {
+      std::vector<std::thread> workers; bool thr = threads;
+      if (thr) try { for (int k = 1; k < K; ++k) workers.emplace_back([&, k] {
         (void)hipSetDevice(ctx->device);
         for (int il = 0; il < nl; ++il) {
           while (bsync.go.load(std::memory_order_acquire) < il) { if (bsync.quit.load(std::memory_order_relaxed)) return; cpu_relax(); }
@@ -818,10 +818,12 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           if (r) { trc[k] = r; bsync.quit.store(true); bsync.done.fetch_add(1, std::memory_order_release); return; }
           bsync.done.fetch_add(1, std::memory_order_release);
         }
-      });
+      }); } catch (...) {            // no thread to be had: this block from the calling thread alone (the windows' host-side waits are then met in order)
+        bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); bsync.quit.store(false); thr = false;
+      }
       auto join = [&] { bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); };
       for (int il = 0; il < nl; ++il) {
-        if (threads) {
+        if (thr) {
           bsync.go.store(il, std::memory_order_release);
           rc = fronts_of(0, il);
           if (rc) { join(); return bail(rc, ctx); }
