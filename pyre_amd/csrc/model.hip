@@ -521,6 +521,7 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
 // path.  PYRE_PROMPT_BLOCK=0 switches it off.
 #define PROMPT_BLOCK_WINDOWS 32
 #define PROMPT_BLOCK_MIN 8
+#define PROMPT_BLOCK_GROUP 2
 static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
 static bool prompt_block_ok(const pyre_model* m) {
   if (!prompt_block_env()) return false;
@@ -561,9 +562,9 @@ static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
 
 namespace {
 
-// The windows of a block are enqueued by one host thread per stream.  A window's wait for the previous window's event of a
-// layer must be issued after that event's record (a wait on an event not yet recorded passes at once): issued[j] counts the
-// layers whose record window j's thread has issued; quit ends every host-side wait when a thread has failed.
+// The windows of a block are enqueued by one host thread per stream, in groups.  A group's wait for the previous group's event
+// of a layer must be issued after that event's record (a wait on an event not yet recorded passes at once): issued[g] counts
+// the layers whose record group g's thread has issued; quit ends every host-side wait when a thread has failed.
 struct BlkSync { std::atomic<int> issued[PROMPT_BLOCK_WINDOWS]; std::atomic<int> go{-1}, done{0}; std::atomic<bool> quit{false}; };
 static inline void cpu_relax() { __builtin_ia32_pause(); }
 
@@ -581,7 +582,6 @@ struct WinOpt {
   const uint32_t* ids_dev = nullptr; const AttnWork* aw = nullptr; const QsaWork* qw = nullptr; const hipEvent_t* wait_ev = nullptr; const hipEvent_t* rec_ev = nullptr;
   int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
   bool no_len = false;          // ... and the state's length is then advanced by the caller
-  BlkSync* bs = nullptr; int bj = 0;      // a block's windows enqueued from several host threads: this window's index in the block (BlkSync)
 };
 
 // rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
@@ -649,28 +649,32 @@ struct WinRun {
     }
     return groups;
   }
-  int front(int il) {
+  // A layer up to its FFN in three parts: the mix in front of the layer's state (pre), what reads and writes that state --
+  // projection with its convolution and the recurrence, or projection and attention -- (mid), the output projection and the FFN
+  // mix (post).  Only mid follows the previous window's mid; front() is the three in a row with the events around mid.
+  int front_pre(int il) {
     const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; int rc;
-    const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
-    // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
-    // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
-    // own split launch (its magnitude has no bound a single workgroup of the merge could form)
-    const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
     const AopOut aout{m->aop, m->aop_inv, d / 256};
-    auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
     auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
     const Layer& L = m->layers[il];
-    if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
     if (L.ple) {      // resolves the pending residual update itself and leaves plain streams
       PleDev pd = L.pld; pd.ring = s->ple_ring[L.ple_index]; pd.mask = m->ple_ring - 1;
       if ((rc = pyre_ple_launch(ctx, m->plc, pd, m->pw, d, hc, c.eps, xin, in_ss, in_ts, xout, comb_out, comb_moe, comb_inj, start, o.step_dev, t))) return rc;
       advance(); comb_out = nullptr; comb_moe = nullptr; comb_inj = nullptr;
     }
+    // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
+    // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
+    // own split launch (its magnitude has no bound a single workgroup of the merge could form)
     if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.hca, L.proj)))) return rc;
     advance(); comb_np = 1;
-    // the layer's state (cache, recurrent state, saved projection) is the previous window's until that window has left it
-    if (o.bs && o.bj > 0) { while (o.bs->issued[o.bj - 1].load(std::memory_order_acquire) <= il) { if (o.bs->quit.load(std::memory_order_relaxed)) return pyre_fail(ctx, PYRE_E_HIP, "a neighbouring window failed"); cpu_relax(); } }
-    if (o.wait_ev) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));
+    return PYRE_OK;
+  }
+  int front_mid(int il) {
+    const pyre_model_cfg& c = m->c; int rc;
+    const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
+    const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
+    auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
+    const Layer& L = m->layers[il];
     if (L.full) {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.hca, L.proj)))) return rc;
@@ -684,8 +688,11 @@ struct WinRun {
       if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, gdn_fused(L) ? m->aop : nullptr, L.gdn_up, gdn_q_on(m, L) ? &gq : nullptr))) return rc;
       s->cur[li] = nb;
     }
-    if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
-    if (o.bs) o.bs->issued[o.bj].store(il + 1, std::memory_order_release);
+    return PYRE_OK;
+  }
+  int front_post(int il) {
+    const pyre_model_cfg& c = m->c; const int d = c.d; int rc;
+    const Layer& L = m->layers[il];
     int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
@@ -697,6 +704,17 @@ struct WinRun {
     advance();
     return PYRE_OK;
   }
+  int front(int il) {
+    int rc; const Layer& L = m->layers[il];
+    if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
+    if ((rc = front_pre(il))) return rc;
+    // the layer's state (cache, recurrent state, saved projection) is the previous window's until that window has left it
+    if (o.wait_ev) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));
+    if ((rc = front_mid(il))) return rc;
+    if (o.rec_ev) PYRE_HIP(ctx, hipEventRecord(o.rec_ev[il], ctx->stream));
+    return front_post(il);
+  }
+
   int moe(int il) {
     const pyre_model_cfg& c = m->c; const Layer& L = m->layers[il]; int rc;
     RouteSrc rs{m->rpart, c.d / 64, L.moe.router.tiles * 64, pyre_hc_aop_ok(L.hcf) ? m->mw.dgx : nullptr};
@@ -782,30 +800,43 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     int wins = n > tail ? (n - tail) / 8 : 0;
     if (wins >= PROMPT_BLOCK_MIN && (rc = prompt_block_get(ctx, m, P))) return rc;
     const int nl = m->c.n_layers;
-    const bool threads = K > 1 && [] { const char* e = getenv("PYRE_PROMPT_THREADS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_THREADS=0: one host thread enqueues every stream
+    const bool threads = K > 1 && [] { const char* e = getenv("PYRE_PROMPT_THREADS"); return e && *e && atoi(e) != 0; }();      // PYRE_PROMPT_THREADS=1: one host thread per stream enqueues (no faster where measured: the streams, not the host, bound a block)
     for (int bi = 0; wins >= PROMPT_BLOCK_MIN; ++bi) {
       const int NB = wins < NBMAX ? wins : NBMAX; wins -= NB;
+      // Windows go to the streams in groups of PROMPT_BLOCK_GROUP consecutive ones, a group's launches in the order pre x G,
+      // mid x G, post x G: the mids of a group follow one another in their stream without an event, one event hands the layer's
+      // state to the next group's stream, and while that stream waits for it it has its own pres behind it, not in front.
+      // (8192 tokens: groups of one 2.17 s, two 1.98, four 2.05, eight 2.29, sixteen 2.58.)
+      const int G = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : PROMPT_BLOCK_GROUP; return v < 1 ? 1 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }(), NG = (NB + G - 1) / G;      // PYRE_PROMPT_GROUP: windows a group
       std::vector<WinRun> runs; runs.reserve(NB);
-      auto cx_of = [&](int j) { const int set = j % K; return set ? P->ctx[set - 1] : ctx; };
+      auto set_of = [&](int j) { return (j / G) % K; };
+      auto cx_of = [&](int j) { const int set = set_of(j); return set ? P->ctx[set - 1] : ctx; };
       auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
       const int pos0 = s->len;
       BlkSync bsync; for (auto& a : bsync.issued) a.store(0);
       for (int j = 0; j < NB; ++j) {
-        const int set = j % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos0 + 8 * j; o.no_len = true;
-        if (threads) { o.bs = &bsync; o.bj = j; }
+        const int set = set_of(j); WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos0 + 8 * j; o.no_len = true;
         o.ids_dev = P->ids + i_first + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
-        const int pset = j > 0 ? (j - 1) % K : prev;            // (prev: the set of the block before this one's last window)
-        o.wait_ev = pset >= 0 ? P->ev[pset].data() : nullptr; o.rec_ev = P->ev[set].data();
         runs.emplace_back(cx_of(j), P->wmdl[j], s, 8, o);
         if ((rc = runs.back().begin())) return bail(rc, cx_of(j));
       }
-      // the layer's fronts: stream k's windows from host thread k (the launches of a front cost the host what they cost the GPU)
+      const int prev_in = prev;            // the set whose events carry the state into this block (-1: the call's first windows)
+      // stream k's groups of layer il, from host thread k.  A group's wait for the previous group's event is issued only after
+      // that event's record has been (BlkSync::issued, here a count per group).
       std::vector<int> trc(K, PYRE_OK);
-      auto fronts_of = [&](int k, int il) -> int {
-        for (int j = k; j < NB; j += K) {
-          pyre_ctx* cx = cx_of(j);
-          if (il > 0 && j < K && j % K != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
-          int r = runs[j].front(il); if (r) return r;
+      auto groups_of = [&](int k, int il) -> int {
+        pyre_ctx* cx = k ? P->ctx[k - 1] : ctx;
+        if (il > 0 && k != 0 && k < NG && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
+        for (int g = k; g < NG; g += K) {
+          const int j0 = g * G, j1 = j0 + G < NB ? j0 + G : NB; int r;
+          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_pre(il))) return r;
+          if (g > 0) { while (bsync.issued[g - 1].load(std::memory_order_acquire) <= il) { if (bsync.quit.load(std::memory_order_relaxed)) return pyre_fail(cx, PYRE_E_HIP, "a neighbouring group failed"); cpu_relax(); } }
+          const int pset = g > 0 ? (g - 1) % K : prev_in;
+          if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
+          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_mid(il))) return r;
+          if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
+          bsync.issued[g].store(il + 1, std::memory_order_release);
+          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_post(il))) return r;
         }
         return PYRE_OK;
       };
@@ -814,26 +845,33 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
         (void)hipSetDevice(ctx->device);
         for (int il = 0; il < nl; ++il) {
           while (bsync.go.load(std::memory_order_acquire) < il) { if (bsync.quit.load(std::memory_order_relaxed)) return; cpu_relax(); }
-          const int r = fronts_of(k, il);
+          const int r = groups_of(k, il);
           if (r) { trc[k] = r; bsync.quit.store(true); bsync.done.fetch_add(1, std::memory_order_release); return; }
           bsync.done.fetch_add(1, std::memory_order_release);
         }
-      }); } catch (...) {            // no thread to be had: this block from the calling thread alone (the windows' host-side waits are then met in order)
+      }); } catch (...) {            // no thread to be had: this block from the calling thread alone
         bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); bsync.quit.store(false); thr = false;
       }
       auto join = [&] { bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); };
       for (int il = 0; il < nl; ++il) {
         if (thr) {
           bsync.go.store(il, std::memory_order_release);
-          rc = fronts_of(0, il);
+          rc = groups_of(0, il);
           if (rc) { join(); return bail(rc, ctx); }
           while (bsync.done.load(std::memory_order_acquire) < (il + 1) * (K - 1)) cpu_relax();
-          for (int k = 1; k < K; ++k) if (trc[k]) { join(); return bail(trc[k], cx_of(k)); }
+          for (int k = 1; k < K; ++k) if (trc[k]) { join(); return bail(trc[k], P->ctx[k - 1]); }
         } else {
-          for (int j = 0; j < NB; ++j) {
-            pyre_ctx* cx = cx_of(j);
-            if (il > 0 && j < K && j % K != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
-            if ((rc = runs[j].front(il))) return bail(rc, cx);
+          // one thread: group by group in order, so that every record is issued before the wait that names it
+          for (int g = 0; g < NG; ++g) {
+            const int k = g % K; pyre_ctx* cx = k ? P->ctx[k - 1] : ctx;
+            if (il > 0 && g < K && k != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
+            const int j0 = g * G, j1 = j0 + G < NB ? j0 + G : NB;
+            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_pre(il))) return bail(rc, cx);
+            const int pset = g > 0 ? (g - 1) % K : prev_in;
+            if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
+            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_mid(il))) return bail(rc, cx);
+            if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed"), cx);
+            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_post(il))) return bail(rc, cx);
           }
         }
         if (il == nl - 1) break;            // the last layer's FFN output has no reader in these windows
@@ -844,7 +882,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
       }
       for (auto& w : workers) w.join();
       workers.clear();
-      s->len = pos0 + NB * 8; i_first += NB * 8; prev = (NB - 1) % K; ++P->blocks_done;
+      s->len = pos0 + NB * 8; i_first += NB * 8; prev = (NG - 1) % K; ++P->blocks_done;
     }
     if (i_first > 0) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipEventRecord(P->done[k], P->ctx[k - 1]->stream));
   }

@@ -120,9 +120,10 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
     prompt = g.integers(0, cfg.vocab, 2 * 256 + 45, dtype=np.uint32)
     more = g.integers(0, cfg.vocab, 256 + 100 + 9, dtype=np.uint32)          # a full block and a shorter one
     out = {}
-    for mode in ("0", "1", "1 one thread"):
+    for mode in ("0", "1", "1 threads", "1 groups of 5"):
         monkeypatch.setenv("PYRE_PROMPT_WINDOWS", "1" if mode == "0" else "0")
-        monkeypatch.setenv("PYRE_PROMPT_THREADS", "0" if mode == "1 one thread" else "1")
+        monkeypatch.setenv("PYRE_PROMPT_THREADS", "1" if mode == "1 threads" else "0")          # one host thread per stream enqueues
+        monkeypatch.setenv("PYRE_PROMPT_GROUP", "5" if mode == "1 groups of 5" else "2")        # consecutive windows a stream takes together
         st = gm.new_state(1024)
         n0 = gm.prompt_blocks()
         lg = gm.forward(prompt, st)
@@ -132,9 +133,10 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
         toks2 = gm.decode_greedy_dev(st, int(np.argmax(lg2)), 4)
         out[mode] = (lg.copy(), toks.copy(), lg2.copy(), toks2.copy(), len(st))
         st.close()
-    a, b, c = out["0"], out["1"], out["1 one thread"]
-    for i in range(4):          # who enqueues does not change a bit
-        assert np.array_equal(np.asarray(b[i]).view(np.uint32), np.asarray(c[i]).view(np.uint32)), i
+    a, b = out["0"], out["1"]
+    for other in ("1 threads", "1 groups of 5"):          # who enqueues, and in which groups, does not change a bit
+        for i in range(4):
+            assert np.array_equal(np.asarray(b[i]).view(np.uint32), np.asarray(out[other][i]).view(np.uint32)), (other, i)
     assert a[4] == b[4] == prompt.size + 6 + more.size + 4
     assert relerr(b[0], a[0]) <= 1e-4 and np.array_equal(a[1], b[1])
     assert relerr(b[2], a[2]) <= 1e-4 and np.array_equal(a[3], b[3])
