@@ -4,9 +4,7 @@
 // 2365-2480, 2495-2515) and spec::generate's greedy branch (src/spec.rs:156-267).
 #include "formats.h"
 #include "digits.h"
-#include <atomic>
 #include <chrono>
-#include <thread>
 #include <memory>
 #include <stdlib.h>
 
@@ -449,8 +447,9 @@ struct PromptPipe {
   uint32_t* ids = nullptr; size_t ids_cap = 0; // the call's token ids on the device
   // blocks of windows taken layer by layer with the FFN of all their tokens grouped by expert (prompt_block_get)
   std::vector<pyre_model*> wmdl;               // a window workspace per window of a block
-  void* blk_mem = nullptr; MoeBlk blk{}; int blk_nsl = 0, blk_r64 = 0;
-  hipEvent_t moe_done = nullptr; std::vector<hipEvent_t> front_done; size_t blocks_done = 0;
+  void* blk_mem = nullptr; MoeBlk blk[2]{}; int blk_nsl = 0, blk_r64 = 0;          // two blocks in flight: one's FFN beside the other's windows
+  hipEvent_t moe_done[2] = {nullptr, nullptr}; std::vector<hipEvent_t> front_done[2]; size_t blocks_done = 0;
+  pyre_ctx* moe_ctx = nullptr;                 // the stream of the blocks' FFN launches
 };
 size_t prompt_pipe_blocks(const PromptPipe* P) { return P->blocks_done; }
 static int prompt_streams() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_STREAMS"); int v = e && *e ? atoi(e) : 3; return v < 1 ? 1 : (v > 4 ? 4 : v); }(); return k; }
@@ -464,8 +463,9 @@ void prompt_pipe_free(PromptPipe* P) {
   if (P->ids) (void)hipFree(P->ids);
   for (auto* mc : P->wmdl) if (mc) { if (mc->work) (void)hipFree(mc->work); delete mc; }
   if (P->blk_mem) (void)hipFree(P->blk_mem);
-  if (P->moe_done) (void)hipEventDestroy(P->moe_done);
-  for (auto e : P->front_done) if (e) (void)hipEventDestroy(e);
+  for (auto e : P->moe_done) if (e) (void)hipEventDestroy(e);
+  for (auto& v : P->front_done) for (auto e : v) if (e) (void)hipEventDestroy(e);
+  if (P->moe_ctx) pyre_ctx_destroy(P->moe_ctx);
   delete P;
 }
 static int prompt_pipe_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe** out) {
@@ -521,7 +521,6 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
 // path.  PYRE_PROMPT_BLOCK=0 switches it off.
 #define PROMPT_BLOCK_WINDOWS 32
 #define PROMPT_BLOCK_MIN 8
-#define PROMPT_BLOCK_GROUP 2
 static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
 static bool prompt_block_ok(const pyre_model* m) {
   if (!prompt_block_env()) return false;
@@ -541,32 +540,33 @@ static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
   const int nsl = d / 64, r64 = m0.router.tiles * 64;
   const size_t xb = al256((size_t)NB * 8 * d * 4), rb = al256((size_t)NB * nsl * 8 * r64 * 4), db = al256((size_t)NB * 8 * (d / 64) * DGX_STRIDE * 4), pb = al256((size_t)NB * PYRE_MOE_GROUPS * 8 * d * 4),
                mb = al256(pyre_moe_block_bytes(m0, NB * 8));
-  PYRE_HIP(ctx, hipMalloc(&P->blk_mem, xb + rb + db + pb + mb + 256));
+  PYRE_HIP(ctx, hipMalloc(&P->blk_mem, 2 * (xb + rb + db + pb) + mb + 256));
   uint8_t* p = (uint8_t*)P->blk_mem;
-  float* x_all = (float*)p; p += xb; float* r_all = (float*)p; p += rb; uint32_t* d_all = (uint32_t*)p; p += db; float* p_all = (float*)p; p += pb;
-  pyre_moe_block_carve(m0, NB * 8, p, &P->blk);
-  P->blk.x = x_all; P->blk.rpart = r_all; P->blk.parts = p_all; P->blk_nsl = nsl; P->blk_r64 = r64;
-  { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk, NB * 8); if (rc) return rc; }
-  for (int j = 0; j < NB; ++j) {
+  // what the windows write and read, once per block in flight; the FFN's own scratch once (its launches share a stream)
+  float* x_all[2]; float* r_all[2]; uint32_t* d_all[2]; float* p_all[2];
+  for (int w = 0; w < 2; ++w) { x_all[w] = (float*)p; p += xb; r_all[w] = (float*)p; p += rb; d_all[w] = (uint32_t*)p; p += db; p_all[w] = (float*)p; p += pb; }
+  pyre_moe_block_carve(m0, NB * 8, p, &P->blk[0]);
+  P->blk[1] = P->blk[0];
+  for (int w = 0; w < 2; ++w) { P->blk[w].x = x_all[w]; P->blk[w].rpart = r_all[w]; P->blk[w].parts = p_all[w]; }
+  P->blk_nsl = nsl; P->blk_r64 = r64;
+  { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk[0], NB * 8); if (rc) return rc; }
+  for (int w = 0; w < 2; ++w) for (int j = 0; j < NB; ++j) {
     pyre_model* mc = new pyre_model(*m); mc->owned.clear(); mc->bufs.clear(); mc->work = nullptr; mc->toks = nullptr; mc->toks_cap = 0; mc->pipe = nullptr;
     P->wmdl.push_back(mc);
     int rc = model_alloc_work(ctx, mc, nullptr); if (rc) return rc;
-    mc->mixed = x_all + (size_t)j * 8 * d; mc->rpart = r_all + (size_t)j * nsl * 8 * r64; mc->mw.dgx = d_all + (size_t)j * 8 * (d / 64) * DGX_STRIDE; mc->mw.parts = p_all + (size_t)j * PYRE_MOE_GROUPS * 8 * d;
+    mc->mixed = x_all[w] + (size_t)j * 8 * d; mc->rpart = r_all[w] + (size_t)j * nsl * 8 * r64; mc->mw.dgx = d_all[w] + (size_t)j * 8 * (d / 64) * DGX_STRIDE; mc->mw.parts = p_all[w] + (size_t)j * PYRE_MOE_GROUPS * 8 * d;
   }
-  PYRE_HIP(ctx, hipEventCreateWithFlags(&P->moe_done, hipEventDisableTiming));
-  P->front_done.resize(K, nullptr);
-  for (auto& e : P->front_done) PYRE_HIP(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  { int rc = pyre_ctx_create(ctx->device, &P->moe_ctx); if (rc) return pyre_fail(ctx, rc, "prompt blocks: %s", pyre_last_error(nullptr)); }
+  for (int w = 0; w < 2; ++w) {
+    PYRE_HIP(ctx, hipEventCreateWithFlags(&P->moe_done[w], hipEventDisableTiming));
+    P->front_done[w].resize(K, nullptr);
+    for (auto& e : P->front_done[w]) PYRE_HIP(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  }
   PYRE_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return PYRE_OK;
 }
 
 namespace {
-
-// The windows of a block are enqueued by one host thread per stream, in groups.  A group's wait for the previous group's event
-// of a layer must be issued after that event's record (a wait on an event not yet recorded passes at once): issued[g] counts
-// the layers whose record group g's thread has issued; quit ends every host-side wait when a thread has failed.
-struct BlkSync { std::atomic<int> issued[PROMPT_BLOCK_WINDOWS]; std::atomic<int> go{-1}, done{0}; std::atomic<bool> quit{false}; };
-static inline void cpu_relax() { __builtin_ia32_pause(); }
 
 struct WinOpt {
   int head_tokens = 1;          // 0 = no logits, 1 = last token only, t = every token (rows 0..t-1 of m->logits)
@@ -800,89 +800,60 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     int wins = n > tail ? (n - tail) / 8 : 0;
     if (wins >= PROMPT_BLOCK_MIN && (rc = prompt_block_get(ctx, m, P))) return rc;
     const int nl = m->c.n_layers;
-    const bool threads = K > 1 && [] { const char* e = getenv("PYRE_PROMPT_THREADS"); return e && *e && atoi(e) != 0; }();      // PYRE_PROMPT_THREADS=1: one host thread per stream enqueues (no faster where measured: the streams, not the host, bound a block)
-    for (int bi = 0; wins >= PROMPT_BLOCK_MIN; ++bi) {
-      const int NB = wins < NBMAX ? wins : NBMAX; wins -= NB;
-      // Windows go to the streams in groups of PROMPT_BLOCK_GROUP consecutive ones, a group's launches in the order pre x G,
-      // mid x G, post x G: the mids of a group follow one another in their stream without an event, one event hands the layer's
-      // state to the next group's stream, and while that stream waits for it it has its own pres behind it, not in front.
-      // (8192 tokens: groups of one 2.17 s, two 1.98, four 2.05, eight 2.29, sixteen 2.58.)
-      const int G = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : PROMPT_BLOCK_GROUP; return v < 1 ? 1 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }(), NG = (NB + G - 1) / G;      // PYRE_PROMPT_GROUP: windows a group
-      std::vector<WinRun> runs; runs.reserve(NB);
-      auto set_of = [&](int j) { return (j / G) % K; };
-      auto cx_of = [&](int j) { const int set = set_of(j); return set ? P->ctx[set - 1] : ctx; };
-      auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
-      const int pos0 = s->len;
-      BlkSync bsync; for (auto& a : bsync.issued) a.store(0);
-      for (int j = 0; j < NB; ++j) {
-        const int set = set_of(j); WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos0 + 8 * j; o.no_len = true;
-        o.ids_dev = P->ids + i_first + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
-        runs.emplace_back(cx_of(j), P->wmdl[j], s, 8, o);
-        if ((rc = runs.back().begin())) return bail(rc, cx_of(j));
+    const int G_env = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : 0; return v < 0 ? 0 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }();      // PYRE_PROMPT_GROUP: windows a group (default: a group a stream)
+    const bool pairs = [] { const char* e = getenv("PYRE_PROMPT_PAIRS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_PAIRS=0: one block at a time
+    auto cxk = [&](int k) { return k ? P->ctx[k - 1] : ctx; };
+    auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(P->moe_ctx->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
+    // Blocks are taken two at a time, layer by layer: the windows of block A, A's FFN on the FFN stream, the windows of block B
+    // beside it, B's FFN beside A's windows of the next layer.  Within a block the windows go to the streams in groups of G
+    // consecutive ones, a group's launches in the order pre x G, mid x G, post x G: the mids of a group follow one another in
+    // their stream without an event, one event hands the layer's state to the next group's stream, and a stream that waits for
+    // it has its own pres behind it, not in front.  (8192 tokens, one block at a time: groups of one 2.17 s, two 1.98, four
+    // 2.05, eight 2.29, sixteen 2.58.)
+    struct Blk { int which, NB, G, NG, prev_in; std::vector<WinRun> runs; };
+    while (wins >= PROMPT_BLOCK_MIN) {
+      Blk B[2]; int nb = 0; int pos = s->len, i0 = i_first, pin = prev;
+      for (int w = 0; w < (pairs ? 2 : 1) && wins >= PROMPT_BLOCK_MIN; ++w) {
+        Blk& b = B[nb++]; b.which = w; b.NB = wins < NBMAX ? wins : NBMAX; wins -= b.NB; b.G = G_env ? G_env : (b.NB + K - 1) / K; b.NG = (b.NB + b.G - 1) / b.G; const int G = b.G; b.prev_in = pin; b.runs.reserve(b.NB);
+        for (int j = 0; j < b.NB; ++j) {
+          const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
+          o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
+          b.runs.emplace_back(cxk(set), P->wmdl[w * NBMAX + j], s, 8, o);
+          if ((rc = b.runs.back().begin())) return bail(rc, cxk(set));
+        }
+        pos += b.NB * 8; i0 += b.NB * 8; pin = (b.NG - 1) % K;
       }
-      const int prev_in = prev;            // the set whose events carry the state into this block (-1: the call's first windows)
-      // stream k's groups of layer il, from host thread k.  A group's wait for the previous group's event is issued only after
-      // that event's record has been (BlkSync::issued, here a count per group).
-      std::vector<int> trc(K, PYRE_OK);
-      auto groups_of = [&](int k, int il) -> int {
-        pyre_ctx* cx = k ? P->ctx[k - 1] : ctx;
-        if (il > 0 && k != 0 && k < NG && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
-        for (int g = k; g < NG; g += K) {
-          const int j0 = g * G, j1 = j0 + G < NB ? j0 + G : NB; int r;
-          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_pre(il))) return r;
-          if (g > 0) { while (bsync.issued[g - 1].load(std::memory_order_acquire) <= il) { if (bsync.quit.load(std::memory_order_relaxed)) return pyre_fail(cx, PYRE_E_HIP, "a neighbouring group failed"); cpu_relax(); } }
-          const int pset = g > 0 ? (g - 1) % K : prev_in;
+      // a block's windows of layer il: group by group in order, so that every record is issued before the wait that names it
+      auto fronts = [&](Blk& b, int il) -> int {
+        const int G = b.G;
+        for (int g = 0; g < b.NG; ++g) {
+          const int k = g % K; pyre_ctx* cx = cxk(k); int r;
+          if (il > 0 && g < K && hipStreamWaitEvent(cx->stream, P->moe_done[b.which], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
+          const int j0 = g * G, j1 = j0 + G < b.NB ? j0 + G : b.NB;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre(il))) return r;
+          const int pset = g > 0 ? (g - 1) % K : b.prev_in;
           if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
-          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_mid(il))) return r;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
-          bsync.issued[g].store(il + 1, std::memory_order_release);
-          for (int j = j0; j < j1; ++j) if ((r = runs[j].front_post(il))) return r;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post(il))) return r;
         }
         return PYRE_OK;
       };
-      std::vector<std::thread> workers; bool thr = threads;
-      if (thr) try { for (int k = 1; k < K; ++k) workers.emplace_back([&, k] {
-        (void)hipSetDevice(ctx->device);
-        for (int il = 0; il < nl; ++il) {
-          while (bsync.go.load(std::memory_order_acquire) < il) { if (bsync.quit.load(std::memory_order_relaxed)) return; cpu_relax(); }
-          const int r = groups_of(k, il);
-          if (r) { trc[k] = r; bsync.quit.store(true); bsync.done.fetch_add(1, std::memory_order_release); return; }
-          bsync.done.fetch_add(1, std::memory_order_release);
-        }
-      }); } catch (...) {            // no thread to be had: this block from the calling thread alone
-        bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); bsync.quit.store(false); thr = false;
+      auto ffn = [&](Blk& b, int il) -> int {
+        pyre_ctx* mx = P->moe_ctx;
+        for (int k = 0; k < K && k < b.NG; ++k) { if (hipEventRecord(P->front_done[b.which][k], cxk(k)->stream) != hipSuccess || hipStreamWaitEvent(mx->stream, P->front_done[b.which][k], 0) != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "event failed"); }
+        int r = pyre_moe_block_launch(mx, m->layers[il].moe, P->blk[b.which], b.NB * 8, NBMAX * 8, P->blk_nsl, P->blk_r64);
+        if (r) return pyre_fail(ctx, r, "%s", mx->err.c_str());
+        if (hipEventRecord(P->moe_done[b.which], mx->stream) != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "hipEventRecord failed");
+        for (int j = 0; j < b.NB; ++j) b.runs[j].moe_from_block();
+        return PYRE_OK;
+      };
+      for (int il = 0; il < nl; ++il) for (int w = 0; w < nb; ++w) {
+        if ((rc = fronts(B[w], il))) return bail(rc, ctx);
+        if (il < nl - 1 && (rc = ffn(B[w], il))) return bail(rc, ctx);            // the last layer's FFN output has no reader in these windows
       }
-      auto join = [&] { bsync.quit.store(true); for (auto& w : workers) w.join(); workers.clear(); };
-      for (int il = 0; il < nl; ++il) {
-        if (thr) {
-          bsync.go.store(il, std::memory_order_release);
-          rc = groups_of(0, il);
-          if (rc) { join(); return bail(rc, ctx); }
-          while (bsync.done.load(std::memory_order_acquire) < (il + 1) * (K - 1)) cpu_relax();
-          for (int k = 1; k < K; ++k) if (trc[k]) { join(); return bail(trc[k], P->ctx[k - 1]); }
-        } else {
-          // one thread: group by group in order, so that every record is issued before the wait that names it
-          for (int g = 0; g < NG; ++g) {
-            const int k = g % K; pyre_ctx* cx = k ? P->ctx[k - 1] : ctx;
-            if (il > 0 && g < K && k != 0 && hipStreamWaitEvent(cx->stream, P->moe_done, 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
-            const int j0 = g * G, j1 = j0 + G < NB ? j0 + G : NB;
-            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_pre(il))) return bail(rc, cx);
-            const int pset = g > 0 ? (g - 1) % K : prev_in;
-            if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed"), cx);
-            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_mid(il))) return bail(rc, cx);
-            if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return bail(pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed"), cx);
-            for (int j = j0; j < j1; ++j) if ((rc = runs[j].front_post(il))) return bail(rc, cx);
-          }
-        }
-        if (il == nl - 1) break;            // the last layer's FFN output has no reader in these windows
-        for (int k = 1; k < K; ++k) { if (hipEventRecord(P->front_done[k], P->ctx[k - 1]->stream) != hipSuccess || hipStreamWaitEvent(ctx->stream, P->front_done[k], 0) != hipSuccess) { join(); return bail(pyre_fail(ctx, PYRE_E_HIP, "event failed"), ctx); } }
-        if ((rc = pyre_moe_block_launch(ctx, m->layers[il].moe, P->blk, NB * 8, NBMAX * 8, P->blk_nsl, P->blk_r64))) { join(); return bail(rc, ctx); }
-        if (hipEventRecord(P->moe_done, ctx->stream) != hipSuccess) { join(); return bail(pyre_fail(ctx, PYRE_E_HIP, "hipEventRecord failed"), ctx); }
-        for (int j = 0; j < NB; ++j) runs[j].moe_from_block();
-      }
-      for (auto& w : workers) w.join();
-      workers.clear();
-      s->len = pos0 + NB * 8; i_first += NB * 8; prev = (NG - 1) % K; ++P->blocks_done;
+      for (int w = 0; w < nb; ++w) { s->len += B[w].NB * 8; i_first += B[w].NB * 8; ++P->blocks_done; }
+      prev = pin;
     }
     if (i_first > 0) for (int k = 1; k < K; ++k) PYRE_HIP(ctx, hipEventRecord(P->done[k], P->ctx[k - 1]->stream));
   }
