@@ -511,7 +511,7 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
 
 // ---- a long prompt in blocks of windows, layer by layer ---------------------------------------------------------------------
 // Windows of eight tokens share nothing in the FFN (eight tokens pick 74 of 512 experts), which makes the expert products
-// the largest part of a prompt window.  A block of PROMPT_BLOCK_WINDOWS windows is therefore taken layer by layer: every
+// the largest part of a prompt window.  A block of up to PROMPT_BLOCK_WINDOWS windows is therefore taken layer by layer: every
 // window's part of the layer up to the FFN mix (on the prompt's streams, the layer's state passing from window to window as
 // before), then the FFN of all of the block's tokens in one set of launches with the tokens grouped by expert, on the
 // matrix cores (pyre_moe_block_launch), whose group sums the windows' next mixes read.  Everything but the FFN is the
@@ -519,7 +519,8 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
 // instead of fixed-point digits): equal to rounding, not bit for bit.  For models whose every layer qualifies
 // (prompt_block_ok); the call's last tokens (the window whose logits are read, the rows a drafter keeps) take the windows'
 // path.  PYRE_PROMPT_BLOCK=0 switches it off.
-#define PROMPT_BLOCK_WINDOWS 32
+static int prompt_block_windows() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_BLOCK_WINDOWS"); int v = e && *e ? atoi(e) : 64; return v < 8 ? 8 : (v > 128 ? 128 : v); }(); return k; }      // the most windows a block has (read once)
+#define PROMPT_BLOCK_WINDOWS prompt_block_windows()
 #define PROMPT_BLOCK_MIN 8
 static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
 static bool prompt_block_ok(const pyre_model* m) {
@@ -811,10 +812,17 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     // it has its own pres behind it, not in front.  (8192 tokens, one block at a time: groups of one 2.17 s, two 1.98, four
     // 2.05, eight 2.29, sixteen 2.58.)
     struct Blk { int which, NB, G, NG, prev_in; std::vector<WinRun> runs; };
-    while (wins >= PROMPT_BLOCK_MIN) {
+    // the call's windows in an even number of blocks of (nearly) equal size, so that every block has a partner
+    int nblk = 0, bsz = 0, brem = 0;
+    if (wins >= PROMPT_BLOCK_MIN) {
+      nblk = pairs ? 2 * ((wins + 2 * NBMAX - 1) / (2 * NBMAX)) : (wins + NBMAX - 1) / NBMAX;
+      while (nblk > 1 && wins / nblk < PROMPT_BLOCK_MIN) --nblk;
+      bsz = wins / nblk; brem = wins % nblk;
+    }
+    for (int bi = 0; bi < nblk; ) {
       Blk B[2]; int nb = 0; int pos = s->len, i0 = i_first, pin = prev;
-      for (int w = 0; w < (pairs ? 2 : 1) && wins >= PROMPT_BLOCK_MIN; ++w) {
-        Blk& b = B[nb++]; b.which = w; b.NB = wins < NBMAX ? wins : NBMAX; wins -= b.NB; b.G = G_env ? G_env : (b.NB + K - 1) / K; b.NG = (b.NB + b.G - 1) / b.G; const int G = b.G; b.prev_in = pin; b.runs.reserve(b.NB);
+      for (int w = 0; w < (pairs ? 2 : 1) && bi < nblk; ++w, ++bi) {
+        Blk& b = B[nb++]; b.which = w; b.NB = bsz + (bi < brem ? 1 : 0); wins -= b.NB; b.G = G_env ? G_env : (b.NB + K - 1) / K; b.NG = (b.NB + b.G - 1) / b.G; const int G = b.G; b.prev_in = pin; b.runs.reserve(b.NB);
         for (int j = 0; j < b.NB; ++j) {
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }

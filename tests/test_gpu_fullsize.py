@@ -151,7 +151,7 @@ def test_prompt_in_blocks_matches_the_oracle_at_full_width(ctx):
     prompt = g.integers(0, cfg.vocab, 256 + 19, dtype=np.uint32)
     gs, os_ = gm.new_state(512), om.new_state()
     lg = gm.forward(prompt, gs)
-    assert gm.prompt_blocks() == 1
+    assert gm.prompt_blocks() == 2          # 33 whole windows in front of the last tokens: a pair of blocks
     lo = om.forward(prompt, os_)
     assert relerr(lg, lo) <= 1e-3
     tg, _ = gm.generate_greedy(gs, lg, 4); to, _ = om.generate_greedy(os_, lo, 4)
