@@ -140,7 +140,23 @@ def test_all_48_layers_full_width_greedy_stream_matches_oracle(ctx, capsys):
     for r in rows:
         say("  %2d %6d  %.3e  %.3e" % r)
     assert worst <= 1e-3
-    gs.close(); gm.close()
+    gs.close()
+    # the same depth through a long prompt: 1100 tokens in blocks (the FFN grouped by expert on the matrix cores) against
+    # the same prompt in windows of eight: logits within 1e-3, the sixteen greedy tokens that follow identical
+    longp = rnd(25).integers(0, cfg.vocab, 1100, dtype=np.uint32); res = {}
+    for mode in ("1", "0"):
+        os.environ["PYRE_PROMPT_WINDOWS"] = mode
+        try:
+            st = gm.new_state(1100 + 32); b0 = gm.prompt_blocks()
+            lgl = gm.forward(longp, st)
+            res[mode] = (lgl.copy(), gm.decode_greedy_dev(st, int(np.argmax(lgl)), 16).copy(), gm.prompt_blocks() - b0)
+            st.close()
+        finally:
+            os.environ.pop("PYRE_PROMPT_WINDOWS", None)
+    assert res["1"][2] == 0 and res["0"][2] == 4
+    say("1100-token prompt at 48 layers, blocks against windows: logits rel err %.3e" % relerr(res["0"][0], res["1"][0]))
+    assert relerr(res["0"][0], res["1"][0]) <= 1e-3 and np.array_equal(res["0"][1], res["1"][1])
+    gm.close()
 
 
 def test_device_loop_equals_host_loop_beyond_32k_context(ctx):
