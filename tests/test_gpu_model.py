@@ -244,6 +244,36 @@ def test_long_prompt_on_several_streams_equals_short_calls_on_one(ctx, kind, mon
     assert np.array_equal(gm.decode_greedy_dev(sa, int(np.argmax(la)), 12), gm.decode_greedy_dev(sb, int(np.argmax(lb)), 12))
 
 
+@pytest.mark.parametrize("kind", ["iq3s_mixes", "indexer"])
+def test_long_prompt_in_blocks_matches_the_oracle(ctx, kind):
+    # A long call of a model whose experts qualify (IQ3_S, equal widths in multiples of 256) takes the whole windows in front of
+    # its last tokens in blocks, layer by layer, the FFN of a block grouped by expert on the matrix cores: logits, recurrent
+    # state and the tokens that follow against the oracle's token-by-token prompt; with a sparse indexer in the attention
+    # layers as well; a second long call continues the state (ragged tails, a position that is no multiple of eight).
+    kw = dict(hc_lr=256, qtype=synth.IQ3_S, hc_type=synth.IQ3_S, n_exp=16, top_k=10)
+    if kind == "iq3s_mixes": c = small_cfg(**kw)
+    else: c = idx_cfg(**kw); c.ctx = 512
+    hw, gm, om = pair(ctx, c, 43)
+    g = np.random.Generator(np.random.PCG64(44))
+    prompt = g.integers(0, c.vocab, 250, dtype=np.uint32)
+    gs, os_ = gm.new_state(480), om.new_state()
+    lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert gm.prompt_blocks() == 2                                     # 30 whole windows: a pair of blocks
+    assert relerr(lg, lo) <= 1e-3 and int(np.argmax(lg)) == int(np.argmax(lo))
+    n_lin = sum(1 for il in range(c.n_layers) if not c.full(il))
+    for li in range(n_lin):
+        conv, ssm = gs.gdn(li)
+        assert relerr(ssm, os_.ssm(li)) <= 1e-3 and relerr(conv, os_.conv(li)) <= 1e-4, li
+    tg, _ = gm.generate_greedy(gs, lg, 6); to, _ = om.generate_greedy(os_, lo, 6)
+    assert np.array_equal(tg, to)
+    more = g.integers(0, c.vocab, 131, dtype=np.uint32)
+    lg = gm.forward(more, gs); lo = om.forward(more, os_)
+    assert gm.prompt_blocks() == 3 and len(gs) == 250 + 5 + 131     # 15 whole windows: one block (the sixth generated token has not been fed)
+    assert relerr(lg, lo) <= 1e-3 and int(np.argmax(lg)) == int(np.argmax(lo))
+    tg, _ = gm.generate_greedy(gs, lg, 6); to, _ = om.generate_greedy(os_, lo, 6)
+    assert np.array_equal(tg, to)
+
+
 @pytest.mark.parametrize("n_exp,top_k,ff_sh,qtype", [(32, 13, 512, synth.IQ3_S), (16, 3, 0, synth.IQ3_S), (16, 2, 0, synth.IQ3_S), (16, 10, 0, synth.Q4_K), (16, 11, 512, synth.Q8_0)])
 def test_window_ffn_output_as_group_sums_equals_single_steps_and_the_oracle(ctx, n_exp, top_k, ff_sh, qtype):
     # With IQ3_S hyper-connection matrices a window's FFN output reaches the next mix as four group sums a token (groups of

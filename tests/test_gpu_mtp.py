@@ -128,6 +128,7 @@ def test_drafter_after_a_long_prompt_on_several_streams(ctx):
     gs, os_ = gm.new_state(192), om.new_state(); gd.attach(gs); od.attach(os_)
     prompt = np.random.Generator(np.random.PCG64(66)).integers(0, c.vocab, 123, dtype=np.uint32)
     lg = gm.forward(prompt, gs); lo = om.forward(prompt, os_)
+    assert gm.prompt_blocks() == 1          # (the twelve whole windows in front of the drafter's rows and the last window: one block, the FFN grouped by expert)
     assert relerr(lg, lo) <= 1e-3 and int(np.argmax(lg)) == int(np.argmax(lo))
     same_drafts(gd, gs, od, os_, int(np.argmax(lo)), 3)
     for o in (gd, gs, gm):
