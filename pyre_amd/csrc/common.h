@@ -308,13 +308,13 @@ struct RouteSrc { const float* p; int nsl; int r64; const uint32_t* dgx = nullpt
 int pyre_moe_launch(pyre_ctx* ctx, const MoeDev& m, const MoeWork& w, const float* x_dev, int t, float* y_dev, const RouteSrc* routed = nullptr, bool in_groups = false);
 inline bool pyre_moe_groups_ok(const MoeDev& m) { return m.top_k <= PYRE_MOE_KMAX; }
 // The FFN of a block of prompt windows (T = 8 * windows tokens) with the tokens grouped by expert, on the matrix cores (moe.hip):
-// what the windows' mixes leave -- x [T][d], the router's K-slice sums (window w's at rpart + w * nsl * 8 * r64, slice s of
-// token ti at (s * 8 + ti) * r64) -- and where window w's group sums go: parts + w * 4 * 8 * d, laid out as MoeWork::parts of
-// a window of eight.  The rest is the block's own scratch (pyre_moe_block_carve): the routing, the (token, choice) pairs by
+// what the windows' mixes leave in their workspaces -- window w's x [8][d] at x + w * ws, its router K-slice sums at rpart + w * ws
+// (slice s of token ti at (s * 8 + ti) * r64) -- and where window w's group sums go: parts + w * ws, laid out as
+// MoeWork::parts of a window of eight.  The rest is the block's own scratch (pyre_moe_block_carve): the routing, the (token, choice) pairs by
 // expert, x and h as f16 operand rows a token (xh [T + 1][2][d], hh [T * (k + 1) + 1][2][ff], the last row of each zero) with
 // their scale factors, the gate and up products and the unreduced down terms.
 struct MoeBlk {
-  const float* x; const float* rpart; float* parts;
+  const float* x; const float* rpart; float* parts; size_t ws;      // window w's x, router sums and group sums at these + w * ws floats (the windows' workspaces: one stride)
   int32_t* sel_idx; float* sel_w; float* sg; int32_t* eoff; int32_t* elist; float* g; float* u; float* partial;
   uint16_t* xh; float* xinv; uint16_t* hh; float* hinv;
 };

@@ -137,7 +137,8 @@ size_t al256(size_t n) { return (n + 255) & ~(size_t)255; }
 extern "C" {
 
 // The activations of one window of up to 8 tokens: everything a window's launches write apart from the state.
-static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
+// the window workspace of a model (activations of up to eight tokens): its size, and its pieces carved out of `base`
+static size_t model_work_layout(pyre_model* m, void* base, int* kmax_out, size_t* aop_bytes) {
   const pyre_model_cfg& c = m->c;
   const size_t w = (size_t)c.hc * c.d, pmax = (size_t)(m->pw_lin > m->pw_attn ? m->pw_lin : m->pw_attn), cmax = (size_t)((c.lin_nv * c.lin_dv) > (c.n_head * c.hd) ? c.lin_nv * c.lin_dv : c.n_head * c.hd);
   HcDev hmax = m->head; hmax.lr = c.hc_lr;
@@ -148,8 +149,10 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   const size_t ple_b = m->n_ple > 0 ? pyre_ple_work_bytes(m->plc, c.d, c.hc) : 0;
   size_t total = al256(pyre_hc_work_bytes(hmax)) + al256(moe_b) + 2 * al256(4 * 8 * w) + 6 * al256(4 * 8 * (size_t)c.d) + al256(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d) + 2 * al256(4 * 8 * c.hc) + al256(4 * 8 * pmax) + al256(4 * 8 * cmax) +
                  al256(4 * 8 * (size_t)c.vocab) + al256(4 * 8 * (size_t)m->ch) + al256(4 * 16) + al256(8 * ((size_t)c.vocab / 32 + 4)) + al256(rp_b) + al256(aop_b) + al256(4 * 8 * (size_t)((kmax + 255) / 256)) + al256(4 * 2 * 8 * 4 * (size_t)c.lin_nv) + al256(ple_b) + 4096;
-  PYRE_HIP(ctx, hipMalloc(&m->work, total));
-  uint8_t* p = (uint8_t*)m->work; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
+  if (kmax_out) *kmax_out = kmax;
+  if (aop_bytes) *aop_bytes = aop_b;
+  if (!base) return total;
+  uint8_t* p = (uint8_t*)base; auto take = [&](size_t n) { void* r = p; p += al256(n); return r; };
   pyre_hc_work_carve(hmax, take(pyre_hc_work_bytes(hmax)), &m->hw); pyre_moe_work_carve(m0, take(moe_b), &m->mw);
   m->x = (float*)take(4 * 8 * w); m->x2 = (float*)take(4 * 8 * w); m->mixed = (float*)take(4 * 8 * (size_t)c.d); m->o = (float*)take(4 * 8 * PYRE_GEMV_PARTS * (size_t)c.d); m->y = (float*)take(4 * 8 * (size_t)c.d); m->hbuf = (float*)take(4 * 8 * (size_t)c.d);
   m->emb = (float*)take(4 * 8 * (size_t)c.d); (void)take(4 * 8 * (size_t)c.d);
@@ -157,8 +160,13 @@ static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
   m->logits = (float*)take(4 * 8 * (size_t)c.vocab); m->co = (float*)take(4 * 8 * (size_t)m->ch); m->ids = (uint32_t*)take(4 * 16); m->best = (uint32_t*)take(8 * ((size_t)c.vocab / 32 + 4));
   m->rpart = (float*)take(rp_b); m->aop = (uint16_t*)take(aop_b); m->aop_inv = (float*)take(4 * 8 * (size_t)((kmax + 255) / 256)); m->gdn_sq = (float*)take(4 * 2 * 8 * 4 * (size_t)c.lin_nv);
   if (m->n_ple > 0) pyre_ple_work_carve(m->plc, c.d, c.hc, take(ple_b), &m->pw);
+  return total;
+}
+static int model_alloc_work(pyre_ctx* ctx, pyre_model* m, int* kmax_out) {
+  size_t aop_b = 0; const size_t total = model_work_layout(m, nullptr, kmax_out, &aop_b);
+  PYRE_HIP(ctx, hipMalloc(&m->work, total));
+  (void)model_work_layout(m, m->work, nullptr, nullptr);
   PYRE_HIP(ctx, hipMemsetAsync(m->aop, 0, aop_b, ctx->stream));
-  if (kmax_out) *kmax_out = kmax;
   return PYRE_OK;
 }
 
@@ -450,6 +458,7 @@ struct PromptPipe {
   void* blk_mem = nullptr; MoeBlk blk[2]{}; int blk_nsl = 0, blk_r64 = 0;          // two blocks in flight: one's FFN beside the other's windows
   hipEvent_t moe_done[2] = {nullptr, nullptr}; std::vector<hipEvent_t> front_done[2]; size_t blocks_done = 0;
   pyre_ctx* moe_ctx = nullptr;                 // the stream of the blocks' FFN launches
+  size_t win_stride = 0;                       // bytes between the workspaces of consecutive windows of a block
 };
 size_t prompt_pipe_blocks(const PromptPipe* P) { return P->blocks_done; }
 static int prompt_streams() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_STREAMS"); int v = e && *e ? atoi(e) : 3; return v < 1 ? 1 : (v > 4 ? 4 : v); }(); return k; }
@@ -539,24 +548,22 @@ static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
   const pyre_model_cfg& c = m->c; const int NB = PROMPT_BLOCK_WINDOWS, d = c.d, K = (int)P->ctx.size() + 1;
   const MoeDev& m0 = m->layers[0].moe;
   const int nsl = d / 64, r64 = m0.router.tiles * 64;
-  const size_t xb = al256((size_t)NB * 8 * d * 4), rb = al256((size_t)NB * nsl * 8 * r64 * 4), db = al256((size_t)NB * 8 * (d / 64) * DGX_STRIDE * 4), pb = al256((size_t)NB * PYRE_MOE_GROUPS * 8 * d * 4),
-               mb = al256(pyre_moe_block_bytes(m0, NB * 8));
-  PYRE_HIP(ctx, hipMalloc(&P->blk_mem, 2 * (xb + rb + db + pb) + mb + 256));
+  // the windows' workspaces of both blocks in flight in one piece, a workspace every ws bytes: what a launch does for one
+  // window it can do for the next ones at the same addresses + ws; the FFN's own scratch once (its launches share a stream)
+  size_t aop_b = 0; const size_t ws = model_work_layout(const_cast<pyre_model*>(m), nullptr, nullptr, &aop_b), mb = al256(pyre_moe_block_bytes(m0, NB * 8));
+  PYRE_HIP(ctx, hipMalloc(&P->blk_mem, 2 * (size_t)NB * ws + mb + 256));
+  PYRE_HIP(ctx, hipMemsetAsync(P->blk_mem, 0, 2 * (size_t)NB * ws, ctx->stream));
   uint8_t* p = (uint8_t*)P->blk_mem;
-  // what the windows write and read, once per block in flight; the FFN's own scratch once (its launches share a stream)
-  float* x_all[2]; float* r_all[2]; uint32_t* d_all[2]; float* p_all[2];
-  for (int w = 0; w < 2; ++w) { x_all[w] = (float*)p; p += xb; r_all[w] = (float*)p; p += rb; d_all[w] = (uint32_t*)p; p += db; p_all[w] = (float*)p; p += pb; }
-  pyre_moe_block_carve(m0, NB * 8, p, &P->blk[0]);
-  P->blk[1] = P->blk[0];
-  for (int w = 0; w < 2; ++w) { P->blk[w].x = x_all[w]; P->blk[w].rpart = r_all[w]; P->blk[w].parts = p_all[w]; }
-  P->blk_nsl = nsl; P->blk_r64 = r64;
-  { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk[0], NB * 8); if (rc) return rc; }
   for (int w = 0; w < 2; ++w) for (int j = 0; j < NB; ++j) {
     pyre_model* mc = new pyre_model(*m); mc->owned.clear(); mc->bufs.clear(); mc->work = nullptr; mc->toks = nullptr; mc->toks_cap = 0; mc->pipe = nullptr;
     P->wmdl.push_back(mc);
-    int rc = model_alloc_work(ctx, mc, nullptr); if (rc) return rc;
-    mc->mixed = x_all[w] + (size_t)j * 8 * d; mc->rpart = r_all[w] + (size_t)j * nsl * 8 * r64; mc->mw.dgx = d_all[w] + (size_t)j * 8 * (d / 64) * DGX_STRIDE; mc->mw.parts = p_all[w] + (size_t)j * PYRE_MOE_GROUPS * 8 * d;
+    (void)model_work_layout(mc, p + ((size_t)w * NB + j) * ws, nullptr, nullptr);
   }
+  pyre_moe_block_carve(m0, NB * 8, p + 2 * (size_t)NB * ws, &P->blk[0]);
+  P->blk[1] = P->blk[0];
+  for (int w = 0; w < 2; ++w) { const pyre_model* f = P->wmdl[(size_t)w * NB]; P->blk[w].x = f->mixed; P->blk[w].rpart = f->rpart; P->blk[w].parts = f->mw.parts; P->blk[w].ws = ws / 4; }
+  P->blk_nsl = nsl; P->blk_r64 = r64; P->win_stride = ws;
+  { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk[0], NB * 8); if (rc) return rc; }
   { int rc = pyre_ctx_create(ctx->device, &P->moe_ctx); if (rc) return pyre_fail(ctx, rc, "prompt blocks: %s", pyre_last_error(nullptr)); }
   for (int w = 0; w < 2; ++w) {
     PYRE_HIP(ctx, hipEventCreateWithFlags(&P->moe_done[w], hipEventDisableTiming));

@@ -550,7 +550,7 @@ __global__ __launch_bounds__(1024) void k_moe_route_blk(MoeDev m, MoeBlk b, int 
 #ifdef PYRE_PHASE_TS
   unsigned long long ts_[8];
 #endif
-  route_topk(b.rpart + ((size_t)w * nsl * 8 + tw) * r64, nsl, 8 * r64, n_exp, top_k, rl ROUTE_TS_ARG);
+  route_topk(b.rpart + (size_t)w * b.ws + (size_t)tw * r64, nsl, 8 * r64, n_exp, top_k, rl ROUTE_TS_ARG);
   route_weights(top_k, rl);
   if ((int)threadIdx.x < top_k) { b.sel_idx[ti * top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; b.sel_w[ti * top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
 }
@@ -586,13 +586,13 @@ __device__ __forceinline__ int blk_entry(const BlkEntries& e, int i) { return e.
 // inv[r][cols / 256].  x2 given: the row is silu(x) * x2 (an expert's h out of its gate and up products).  gate_inp given:
 // sg[r] = sigmoid(gate_inp . x[r]) as well (the shared expert's gate).  grid (n), 256 threads, a stretch a round.  Row n of
 // xh is kept zero by the owner: the operand rows a pass has no token for point there.
-__global__ __launch_bounds__(256) void k_blk_split(const float* __restrict__ x, const float* __restrict__ x2, int cols, uint16_t* __restrict__ xh, float* __restrict__ inv, const float* __restrict__ gate_inp, float* __restrict__ sg) {
+__global__ __launch_bounds__(256) void k_blk_split(const float* __restrict__ x, const float* __restrict__ x2, int cols, uint16_t* __restrict__ xh, float* __restrict__ inv, const float* __restrict__ gate_inp, float* __restrict__ sg, size_t ws) {      // ws > 0: row r of x at x + (r / 8) * ws + (r % 8) * cols (a window's eight rows in its workspace)
   __shared__ float mx[2][4]; __shared__ float dp[4];
   const int r = blockIdx.x, i = threadIdx.x, wave = i >> 6, lane = i & 63;
   float dot = 0.0f;
   for (int sb = 0; sb < (cols >> 8); ++sb) {
     const int k = sb * 256 + i;
-    float v = x[(size_t)r * cols + k];
+    float v = (ws ? x + (size_t)(r >> 3) * ws + (size_t)(r & 7) * cols : x + (size_t)r * cols)[k];
     if (x2) { const float sgm = 1.0f / (1.0f + expf(-v)); v = (v * sgm) * x2[(size_t)r * cols + k]; }
     if (gate_inp) dot = fmaf(gate_inp[k], v, dot);
     float a = fabsf(v); a = a == a ? a : INFINITY;
@@ -686,7 +686,7 @@ __global__ __launch_bounds__(256) void k_moe_groups_blk(MoeDev m, MoeBlk b, int 
   const int r = blockIdx.x * 256 + threadIdx.x, ti = blockIdx.y, k = m.top_k, d = m.d, gsz = (k + 4) / 4;
   if (r >= d) return;
   const float* pt = b.partial + (size_t)ti * (k + 1) * d + r;
-  float* out = b.parts + (size_t)(ti >> 3) * PYRE_MOE_GROUPS * 8 * d + (size_t)(ti & 7) * d + r;
+  float* out = b.parts + (size_t)(ti >> 3) * b.ws + (size_t)(ti & 7) * d + r;
 #pragma unroll
   for (int q = 0; q < PYRE_MOE_GROUPS; ++q) {
     const int j0 = min(k, q * gsz), nr = min(k, j0 + gsz) - j0;
@@ -730,10 +730,10 @@ int pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T
   { ProfScope ps(ctx, "moe_block_route", 4.0 * T * nsl * m.n_exp);
     if (fix) hipLaunchKernelGGL(k_moe_route_blk<true>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64); else hipLaunchKernelGGL(k_moe_route_blk<false>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64);
     hipLaunchKernelGGL(k_moe_lists, dim3(1), dim3(1024), 0, ctx->stream, m, b, T);
-    hipLaunchKernelGGL(k_blk_split, dim3(T), dim3(256), 0, ctx->stream, b.x, (const float*)nullptr, m.d, b.xh, b.xinv, m.sh_gate_inp, b.sg); } PYRE_CHECK_LAUNCH(ctx);
+    hipLaunchKernelGGL(k_blk_split, dim3(T), dim3(256), 0, ctx->stream, b.x, (const float*)nullptr, m.d, b.xh, b.xinv, m.sh_gate_inp, b.sg, b.ws); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_block_gate_up", 2.0 * m.n_exp * qmat_gguf_bytes(m.gate_e, m.ff) + 2.0 * qmat_gguf_bytes(m.sh_gate, m.sf));
     hipLaunchKernelGGL(k_moe_mm_blk<false>, dim3((hs + 255) / 256, ny, 2), dim3(256), 0, ctx->stream, m, b, T, T_max);
-    hipLaunchKernelGGL(k_blk_split, dim3(ne), dim3(256), 0, ctx->stream, (const float*)b.g, (const float*)b.u, hs, b.hh, b.hinv, (const float*)nullptr, (float*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
+    hipLaunchKernelGGL(k_blk_split, dim3(ne), dim3(256), 0, ctx->stream, (const float*)b.g, (const float*)b.u, hs, b.hh, b.hinv, (const float*)nullptr, (float*)nullptr, (size_t)0); } PYRE_CHECK_LAUNCH(ctx);
   { ProfScope ps(ctx, "moe_block_down", (double)m.n_exp * qmat_gguf_bytes(m.down_e, m.d) + qmat_gguf_bytes(m.sh_down, m.d));
     hipLaunchKernelGGL(k_moe_mm_blk<true>, dim3((m.d + 255) / 256, ny, 1), dim3(256), 0, ctx->stream, m, b, T, ne_max);
     hipLaunchKernelGGL(k_moe_groups_blk, dim3((m.d + 255) / 256, T), dim3(256), 0, ctx->stream, m, b, T); } PYRE_CHECK_LAUNCH(ctx);
