@@ -273,12 +273,18 @@ __device__ __forceinline__ void hc_lds_a(const uint16_t* ah, int c, int lane, AB
 // FD, FK > 0: the model width d and the routed experts per token as compile-time constants (the launcher checks them): the
 // stream index of a slice is a shift, the gather of the unreduced FFN output carries no predicates -- same arithmetic.
 template <int T, int NP, int CS, int FD = 0, int FK = 0> __global__ __launch_bounds__(256 * CS) void k_hc_norm_down_m(QMatDev m, const float* __restrict__ x_in, int in_ss, int in_ts, float* __restrict__ x_out,
-    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part, float* __restrict__ smx) {
+    const float* __restrict__ comb_out, MoeOut mo, const float* __restrict__ comb_inj, const float* __restrict__ norm, int d, int hc, float* __restrict__ ssq, float* __restrict__ part, float* __restrict__ smx, size_t wz) {
   constexpr int NW = 4 * CS;
   __shared__ __align__(16) uint16_t ah[CS * 32 * 16 * 8];
   __shared__ float wsum[NW][8], wmax[NW][8], hsum[4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m); args_now(x_in, in_ss, in_ts, x_out, comb_out, mo.partial, mo.sel_w, mo.sg, mo.d, mo.k, comb_inj, norm, d, hc, ssq, part);
+  if (wz) {          // a launch for several windows: blockIdx.z's window has everything that is its own wz bytes further on per window
+    const size_t zo = (size_t)blockIdx.z * wz;
+    x_in = (const float*)((const char*)x_in + zo); x_out = (float*)((char*)x_out + zo); ssq = (float*)((char*)ssq + zo); part = (float*)((char*)part + zo); smx = (float*)((char*)smx + zo);
+    if (comb_out) comb_out = (const float*)((const char*)comb_out + zo);
+    if (comb_inj) comb_inj = (const float*)((const char*)comb_inj + zo);
+  }
   const int tile = blockIdx.x, ks = blockIdx.y, tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = wave & 3, p = wave >> 2;
   if constexpr (FD > 0) d = FD;
@@ -379,12 +385,21 @@ __device__ __forceinline__ float hc_slice_sum16(const float (&pv)[16], const flo
 // them): divisions become shifts, the slice loops lose their predicates -- same arithmetic.
 template <int T, int RF, int FHC = 0, int FLR = 0, int FKS = 0> __global__ __launch_bounds__(1024) void k_hc_up_mix_m(QMatDev up, const float* __restrict__ part, const float* __restrict__ ssq, int ksplit, int r64, int lr, int hc, int has_inject,
     const float* __restrict__ xnew, const float* __restrict__ norm, float eps, int d, float* __restrict__ mixed, float* __restrict__ inj,
-    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb, uint32_t* __restrict__ dgx) {
+    QMatDev router, float* __restrict__ rpart, uint16_t* __restrict__ aop, int aop_rows, int lcw, const float* __restrict__ smx, float* __restrict__ aop_inv, int aop_nsb, uint32_t* __restrict__ dgx, size_t wz) {
   constexpr bool ROUTE = RF >= 0; constexpr int RFX = ROUTE ? RF : FMT_F32;
   __shared__ uint8_t dsm[ROUTE ? T : 1][3][64];          // the digit waves' staging
   const uint2* lds2 = nullptr;
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(up); args_now(part, ssq, ksplit, r64, lr, hc, has_inject, xnew, norm, eps, d, mixed, inj, lcw);
+  if (wz) {          // a launch for several windows, as k_hc_norm_down_m
+    const size_t zo = (size_t)blockIdx.z * wz;
+    part = (const float*)((const char*)part + zo); ssq = (const float*)((const char*)ssq + zo); xnew = (const float*)((const char*)xnew + zo); smx = (const float*)((const char*)smx + zo);
+    mixed = (float*)((char*)mixed + zo); inj = (float*)((char*)inj + zo);
+    if (rpart) rpart = (float*)((char*)rpart + zo);
+    if (aop) aop = (uint16_t*)((char*)aop + zo);
+    if (aop_inv) aop_inv = (float*)((char*)aop_inv + zo);
+    if (dgx) dgx = (uint32_t*)((char*)dgx + zo);
+  }
   if constexpr (FHC > 0) { hc = FHC; lr = FLR; ksplit = FKS; }
   extern __shared__ __align__(16) float sm[];
   const int nthr = blockDim.x, tid = threadIdx.x, kps = ksplit / hc, nw = nthr >> 6, CW = 1 << lcw, lg = lcw - 4;
@@ -556,8 +571,8 @@ bool hc_on_matrix_cores(const HcDev& h) {
 }
 template <int T> int norm_down_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const float* x_in, int in_ss, int in_ts, float* x_out, const float* comb_out, int comb_parts, const MoeOut& mo, const float* comb_inj) {
   ProfScope ps(ctx, "hc_norm_down", qmat_gguf_bytes(h.di, h.di.rows) + 4.0 * T * h.hc * h.d * 4);
-#define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
-#define NORM_DOWN_M_FIX(NP) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, 2, 2048, 10>), dim3(h.di_m.tiles, hc_m_slices(h)), dim3(512), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx)
+#define NORM_DOWN_M_GO(NP, CS) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, CS>), dim3(h.di_m.tiles, hc_m_slices(h), ctx->batch_n), dim3(256 * CS), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx, ctx->batch_stride)
+#define NORM_DOWN_M_FIX(NP) hipLaunchKernelGGL((k_hc_norm_down_m<T, NP, 2, 2048, 10>), dim3(h.di_m.tiles, hc_m_slices(h), ctx->batch_n), dim3(512), 0, ctx->stream, h.di_m, x_in, in_ss, in_ts, x_out, comb_out, mo, comb_inj, h.norm, h.d, h.hc, w.ssq, w.o, w.smx, ctx->batch_stride)
   bool done = false;
   {          // the width of the A3B configuration: the instances with its constants folded in
     if (h.d == 2048 && (!mo.partial || mo.k == 10)) { if (comb_parts > 1) NORM_DOWN_M_FIX(PYRE_GEMV_PARTS); else NORM_DOWN_M_FIX(1); done = true; }
@@ -583,8 +598,8 @@ template <int T> int up_mix_m_launch(pyre_ctx* ctx, const HcDev& h, const HcWork
   const QMatDev rq = rt ? rt->router : QMatDev{}; float* rp = rt ? rt->part : nullptr;
   ProfScope ps(ctx, rt ? "hc_up_mix_router" : "hc_up_mix", qmat_gguf_bytes(h.up, h.up.rows) + 4.0 * T * (h.hc * h.d + h.d + (double)ksplit * (h.lr + h.hc)) +
                (rt ? qmat_gguf_bytes(rq, rq.rows) + 4.0 * T * (h.d / 64) * rq.tiles * 64 : 0.0));
-#define UP_MIX_M_ARGS dim3(h.d >> lcw), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
-                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0, rt ? rt->dgx : nullptr
+#define UP_MIX_M_ARGS dim3(h.d >> lcw, 1, ctx->batch_n), dim3(nw * 64), lds, ctx->stream, h.up_m, w.o, w.ssq, ksplit, h.di.tiles * 64, h.lr, h.hc, h.has_inject ? 1 : 0, xnew, h.norm, eps, \
+                     h.d, mixed, inj, rq, rp, aop ? aop->op : nullptr, pyre_aop_rows(T), lcw, w.smx, aop ? aop->ainv : nullptr, aop ? aop->nsb : 0, rt ? rt->dgx : nullptr, ctx->batch_stride
 #define UP_MIX_M_GO(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF>), UP_MIX_M_ARGS)
 #define UP_MIX_M_FIX(RF) hipLaunchKernelGGL((k_hc_up_mix_m<T, RF, 4, 256, 16>), UP_MIX_M_ARGS)
   bool done = false;
@@ -650,6 +665,7 @@ int pyre_hc_mix_launch(pyre_ctx* ctx, const HcDev& h, const HcWork& w, const flo
   DownPlan p = down_plan(h);
   if (p.ksplit < 1 || p.ksplit > 32 || p.ksplit * p.nw * p.upw != h.di.U) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: d = %d cannot be cut into at most 32 slices of whole waves", h.d);
   const bool on_m = hc_on_matrix_cores(h);
+  if (ctx->batch_n > 1 && !on_m) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: only the matrix-core mix serves several windows a launch");
   if (aop && !(on_m && aop->op && aop->ainv && aop->nsb >= 1 && h.hc <= 4)) return pyre_fail(ctx, PYRE_E_ARG, "hc_mix: only the matrix-core mix leaves an operand (pyre_hc_aop_ok)");
   MoeOut mo = comb_moe ? *comb_moe : MoeOut{nullptr, nullptr, nullptr, 0, 0};
   if (mo.partial && (mo.k > PYRE_MOE_KMAX || mo.d != h.d)) return pyre_fail(ctx, PYRE_E_SHAPE, "hc_mix: unreduced FFN output with top_k %d / width %d", mo.k, mo.d);

@@ -590,6 +590,7 @@ struct WinOpt {
   const uint32_t* ids_dev = nullptr; const AttnWork* aw = nullptr; const QsaWork* qw = nullptr; const hipEvent_t* wait_ev = nullptr; const hipEvent_t* rec_ev = nullptr;
   int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
   bool no_len = false;          // ... and the state's length is then advanced by the caller
+  size_t win_stride = 0;        // bytes between this window's workspace and the next window's of its block (0: it stands alone)
 };
 
 // rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
@@ -660,7 +661,9 @@ struct WinRun {
   // A layer up to its FFN in three parts: the mix in front of the layer's state (pre), what reads and writes that state --
   // projection with its convolution and the recurrence, or projection and attention -- (mid), the output projection and the FFN
   // mix (post).  Only mid follows the previous window's mid; front() is the three in a row with the events around mid.
-  int front_pre(int il) {
+  // nz: windows this launch serves (this one and the nz - 1 after it, their workspaces o.win_stride bytes apart); 0: none -- a
+  // launch of an earlier window of the group has served this one, only the bookkeeping is left
+  int front_pre(int il, int nz = 1) {
     const pyre_model_cfg& c = m->c; const int d = c.d, hc = c.hc; int rc;
     const AopOut aout{m->aop, m->aop_inv, d / 256};
     auto opw = [&](const HcDev& h, const QMatDev& q) -> const AopOut* { return hc_fused(h, q) ? &aout : nullptr; };
@@ -673,7 +676,12 @@ struct WinRun {
     // the mix that produces a matrix-core GEMV's input also leaves it as that GEMV's f16 operand, every token scaled by a power of
     // two (AopOut); the Gated DeltaNet step likewise with a constant of the layer; the attention output goes through the GEMV's
     // own split launch (its magnitude has no bound a single workgroup of the merge could form)
-    if ((rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.hca, L.proj)))) return rc;
+    if (nz > 0) {
+      ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
+      rc = pyre_hc_mix_launch(ctx, L.hca, m->hw, xin, in_ss, in_ts, xout, t, comb_out, comb_moe, comb_inj, c.eps, m->mixed, m->inj_a, nullptr, comb_np, opw(L.hca, L.proj));
+      ctx->batch_n = 1; ctx->batch_stride = 0;
+      if (rc) return rc;
+    }
     advance(); comb_np = 1;
     return PYRE_OK;
   }
@@ -698,20 +706,31 @@ struct WinRun {
     }
     return PYRE_OK;
   }
-  int front_post(int il) {
-    const pyre_model_cfg& c = m->c; const int d = c.d; int rc;
+  int front_post_proj(int il) {          // the output projection
+    const pyre_model_cfg& c = m->c; const int d = c.d;
     const Layer& L = m->layers[il];
-    int o_parts = 1;          // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
-    if (outp_in_parts(L, d)) { o_parts = PYRE_GEMV_PARTS; if ((rc = pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc; }
-    else if ((rc = pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa))) return rc;
+    // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
+    if (outp_in_parts(L, d)) return pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa);
+    return pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa);
+  }
+  int front_post_mix(int il, int nz = 1) {          // the FFN mix (nz as in front_pre)
+    const pyre_model_cfg& c = m->c; const int d = c.d; int rc;
+    const Layer& L = m->layers[il];
+    const int o_parts = outp_in_parts(L, d) ? PYRE_GEMV_PARTS : 1;
     ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
     HcRoute hr{L.moe.router, m->rpart, m->mw.dgx};          // (the matrix-core mix leaves the digits of its output; after another mix the expert launch makes them)
-    if ((rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts))) return rc;
+    if (nz > 0) {
+      ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
+      rc = pyre_hc_mix_launch(ctx, L.hcf, m->hw, xin, in_ss, in_ts, xout, t, m->o, nullptr, m->inj_a, c.eps, m->mixed, m->inj_f, ride ? &hr : nullptr, o_parts);
+      ctx->batch_n = 1; ctx->batch_stride = 0;
+      if (rc) return rc;
+    }
     advance();
     return PYRE_OK;
   }
+  int front_post(int il) { int rc = front_post_proj(il); return rc ? rc : front_post_mix(il); }
   int front(int il) {
     int rc; const Layer& L = m->layers[il];
     if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
@@ -809,6 +828,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     if (wins >= PROMPT_BLOCK_MIN && (rc = prompt_block_get(ctx, m, P))) return rc;
     const int nl = m->c.n_layers;
     const int G_env = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : 0; return v < 0 ? 0 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }();      // PYRE_PROMPT_GROUP: windows a group (default: a group a stream)
+    const bool batch = [&] { const char* e = getenv("PYRE_PROMPT_BATCH"); if (e && *e && atoi(e) == 0) return false; for (const Layer& L : m->layers) if (!pyre_hc_aop_ok(L.hca) || !pyre_hc_aop_ok(L.hcf)) return false; return true; }();      // a group's mixes in one launch each (the matrix-core mixes; PYRE_PROMPT_BATCH=0: a launch a window)
     const bool pairs = [] { const char* e = getenv("PYRE_PROMPT_PAIRS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_PAIRS=0: one block at a time
     auto cxk = [&](int k) { return k ? P->ctx[k - 1] : ctx; };
     auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(P->moe_ctx->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
@@ -833,6 +853,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
         for (int j = 0; j < b.NB; ++j) {
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
+          o.win_stride = P->win_stride;
           b.runs.emplace_back(cxk(set), P->wmdl[w * NBMAX + j], s, 8, o);
           if ((rc = b.runs.back().begin())) return bail(rc, cxk(set));
         }
@@ -845,12 +866,13 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           const int k = g % K; pyre_ctx* cx = cxk(k); int r;
           if (il > 0 && g < K && hipStreamWaitEvent(cx->stream, P->moe_done[b.which], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
           const int j0 = g * G, j1 = j0 + G < b.NB ? j0 + G : b.NB;
-          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre(il))) return r;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;            // the group's mixes: one launch each
           const int pset = g > 0 ? (g - 1) % K : b.prev_in;
           if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
-          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post(il))) return r;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il))) return r;
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_mix(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;
         }
         return PYRE_OK;
       };
