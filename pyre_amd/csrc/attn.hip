@@ -735,7 +735,7 @@ template <int G> static void launch_decode(pyre_ctx* ctx, const AttnDev& a, cons
 int pyre_attn_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp) {
   return pyre_attn_launch_sel(ctx, a, kv, w, qkv, stride, start, t, packed_done, out, posp, nullptr);
 }
-int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp, const QsaWork* qw) {
+int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t, int* packed_done, float* out, const int* posp, const QsaWork* qw, int part) {
   if (a.hd != 256) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: head dim %d unsupported (256 only)", a.hd);
   if (a.nkv < 1 || a.nh % a.nkv) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: %d query heads over %d kv heads", a.nh, a.nkv);
   int G = a.nh / a.nkv; if (G != 1 && G != 2 && G != 4 && G != 8) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: group size %d unsupported (1, 2, 4, 8)", G);
@@ -743,8 +743,13 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   if (start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention: position %d exceeds the cache capacity %d", start + t, kv.cap);
   if (a.n_rot > a.hd || (a.n_rot & 1)) return pyre_fail(ctx, PYRE_E_SHAPE, "attention: n_rot %d", a.n_rot);
   // a single-token step at a device-side position: the packing check rides on the prep launch as extra blocks
+  // part 1: the cache write (rotated q into w.q / qh / qsc, K and V into the cache, packing); part 2: the attention pass over
+  // the cache and the merge, which read only what part 1 of this and of earlier windows has written (w.q* must then be this
+  // window's own until part 2 has run); 0: both
+  if (part < 0 || part > 2 || (part && posp)) return pyre_fail(ctx, PYRE_E_ARG, "attention: part %d", part);
   const bool pack_rides = posp && t == 1 && a.kv_bits == 4;
   const int pack_blocks = pack_rides ? (64 * (a.nkv * a.hd / 32) * 2 + 255) / 256 : 0;
+  if (part != 2) {
   { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q, w.qh, w.qsc); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
   int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
@@ -755,6 +760,8 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
     { ProfScope ps(ctx, "kv_pack", (double)(pbn - *packed_done) * a.nkv * a.hd * 2 * 4.625); hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, *packed_done, pbn, (const int*)nullptr); } PYRE_CHECK_LAUNCH(ctx);
     *packed_done = pbn;
   }
+  }
+  if (part == 1) return PYRE_OK;
   double kvb = 0;
   for (int ti = 0; ti < t; ++ti) {
     double n = start + ti + 1, pb = (double)pyre_packed_boundary((size_t)n, a.kv_bits, a.kv_recent);

@@ -450,5 +450,5 @@ int pyre_qsa_launch(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaB
 int pyre_qsa_pool_all(pyre_ctx* ctx, const QsaDev& q, const AttnDev& a, const QsaBuf& b, int n);
 // the attention launch with an optional position list (qw == nullptr: dense)
 int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int qkv_stride, int start, int t,
-                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw);
+                         int* packed_done, float* out_dev, const int* posp, const QsaWork* qw, int part = 0);      // part: 1 = the cache write alone, 2 = the pass over the cache and the merge alone (w.q / qh / qsc kept in between), 0 = both
 int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t);      // K / V only

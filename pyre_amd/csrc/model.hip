@@ -459,6 +459,7 @@ struct PromptPipe {
   hipEvent_t moe_done[2] = {nullptr, nullptr}; std::vector<hipEvent_t> front_done[2]; size_t blocks_done = 0;
   pyre_ctx* moe_ctx = nullptr;                 // the stream of the blocks' FFN launches
   size_t win_stride = 0;                       // bytes between the workspaces of consecutive windows of a block
+  void* qmem = nullptr; size_t q_stride = 0, q_off[2] = {0, 0};      // per window of a block: the rotated queries (f32, f16 halves, scales) of an attention layer, kept from the cache write to the pass over the cache
 };
 size_t prompt_pipe_blocks(const PromptPipe* P) { return P->blocks_done; }
 static int prompt_streams() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_STREAMS"); int v = e && *e ? atoi(e) : 3; return v < 1 ? 1 : (v > 4 ? 4 : v); }(); return k; }
@@ -475,6 +476,7 @@ void prompt_pipe_free(PromptPipe* P) {
   for (auto e : P->moe_done) if (e) (void)hipEventDestroy(e);
   for (auto& v : P->front_done) for (auto e : v) if (e) (void)hipEventDestroy(e);
   if (P->moe_ctx) pyre_ctx_destroy(P->moe_ctx);
+  if (P->qmem) (void)hipFree(P->qmem);
   delete P;
 }
 static int prompt_pipe_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe** out) {
@@ -564,6 +566,11 @@ static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
   for (int w = 0; w < 2; ++w) { const pyre_model* f = P->wmdl[(size_t)w * NB]; P->blk[w].x = f->mixed; P->blk[w].rpart = f->rpart; P->blk[w].parts = f->mw.parts; P->blk[w].ws = ws / 4; }
   P->blk_nsl = nsl; P->blk_r64 = r64; P->win_stride = ws;
   { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk[0], NB * 8); if (rc) return rc; }
+  if (!m->has_idx && !(getenv("PYRE_PROMPT_ATTN_SPLIT") && atoi(getenv("PYRE_PROMPT_ATTN_SPLIT")) == 0)) {      // (with a sparse indexer the selection and the pass stay together in the chain; PYRE_PROMPT_ATTN_SPLIT=0: likewise)
+    const size_t nq = (size_t)8 * c.n_head * c.hd;
+    P->q_off[0] = al256(4 * nq); P->q_off[1] = P->q_off[0] + al256(2 * 2 * nq); P->q_stride = P->q_off[1] + al256(4 * 8 * (size_t)c.n_head);
+    PYRE_HIP(ctx, hipMalloc(&P->qmem, 2 * (size_t)NB * P->q_stride));
+  }
   { int rc = pyre_ctx_create(ctx->device, &P->moe_ctx); if (rc) return pyre_fail(ctx, rc, "prompt blocks: %s", pyre_last_error(nullptr)); }
   for (int w = 0; w < 2; ++w) {
     PYRE_HIP(ctx, hipEventCreateWithFlags(&P->moe_done[w], hipEventDisableTiming));
@@ -591,6 +598,7 @@ struct WinOpt {
   int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
   bool no_len = false;          // ... and the state's length is then advanced by the caller
   size_t win_stride = 0;        // bytes between this window's workspace and the next window's of its block (0: it stands alone)
+  bool attn_split = false; AttnWork aw_own{};      // a block's window: the attention pass over the cache leaves the chain through the layer's state (front_post_proj runs it); aw_own: the stream's attention workspace with q buffers of this window's own
 };
 
 // rows `from` .. t-1 of the window's final residual streams x [t][w] into the ring at their positions; grid (ceil(w/256), t - from)
@@ -687,7 +695,7 @@ struct WinRun {
   }
   int front_mid(int il) {
     const pyre_model_cfg& c = m->c; int rc;
-    const AttnWork& aw = o.aw ? *o.aw : s->aw; const QsaWork& qw = o.qw ? *o.qw : s->qw;
+    const AttnWork& aw = o.attn_split ? o.aw_own : (o.aw ? *o.aw : s->aw); const QsaWork& qw = o.qw ? *o.qw : s->qw;
     const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
     auto opnd = [&](const HcDev& h, const QMatDev& q) -> const PyreAop* { return hc_fused(h, q) ? &aop_hc : nullptr; };
     const Layer& L = m->layers[il];
@@ -695,7 +703,7 @@ struct WinRun {
       int ai = L.mix_index;
       if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.hca, L.proj)))) return rc;
       if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
-      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr))) return rc;
+      if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr, o.attn_split ? 1 : 0))) return rc;
     } else {
       int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
@@ -706,9 +714,10 @@ struct WinRun {
     }
     return PYRE_OK;
   }
-  int front_post_proj(int il) {          // the output projection
+  int front_post_proj(int il) {          // the output projection (in front of it, for a block's window, the attention pass its mid left out)
     const pyre_model_cfg& c = m->c; const int d = c.d;
     const Layer& L = m->layers[il];
+    if (L.full && o.attn_split) { int rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[L.mix_index], o.aw_own, m->proj, m->pw_attn, start, t, &s->packed[L.mix_index], m->core, nullptr, nullptr, 2); if (rc) return rc; }
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
     // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
@@ -854,6 +863,11 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
           o.win_stride = P->win_stride;
+          if (P->qmem) {          // q buffers of the window's own; the partial sums stay the stream's
+            o.attn_split = true; o.aw_own = set ? s->aw_more[set - 1] : s->aw;
+            uint8_t* qb = (uint8_t*)P->qmem + (size_t)(w * NBMAX + j) * P->q_stride;
+            o.aw_own.q = (float*)qb; o.aw_own.qh = (uint16_t*)(qb + P->q_off[0]); o.aw_own.qsc = (float*)(qb + P->q_off[1]);
+          }
           b.runs.emplace_back(cxk(set), P->wmdl[w * NBMAX + j], s, 8, o);
           if ((rc = b.runs.back().begin())) return bail(rc, cxk(set));
         }
