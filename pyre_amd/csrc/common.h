@@ -384,6 +384,8 @@ struct GdnDev { const float* a; const float* dt; const float* conv_w; const floa
 // The state it leaves differs in rounding from the nv-workgroup form's (the column sums meet in another order): a layer
 // uses one form for every call.
 struct GdnQ { uint16_t* op; float* sq; };
+// the convolution of n consecutive windows of t tokens in one launch (gdn.hip: k_gdn_conv_blk)
+int pyre_gdn_conv_block_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, int n, size_t ws, const float* prev, int prev_stride, float* conv_out, float* co);
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
                     const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f, const GdnQ* gq = nullptr);
 

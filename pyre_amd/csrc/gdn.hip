@@ -25,6 +25,31 @@ __global__ __launch_bounds__(256) void k_gdn_conv(const float* __restrict__ proj
   for (int k = 0; k < kk - 1; ++k) conv_out[(size_t)k * ch + c] = hist[k];
 }
 
+// The same for n consecutive windows of t tokens in one launch (a long prompt's blocks): grid (ceil(ch/256), n).  Window z's
+// projection rows lie at proj + z * ws, its output at co + z * ws (the windows' workspaces, ws floats apart); its history is
+// the last kk - 1 rows of window z - 1's projection -- for window 0 the kk - 1 rows at prev (row stride prev_stride: the
+// layer's convolution state, or the projection rows of the window in front of the group).  The last window leaves the state
+// in conv_out if that is given.  A channel's arithmetic is k_gdn_conv's, so are its bits.  Needs t >= kk - 1.
+__global__ __launch_bounds__(256) void k_gdn_conv_blk(const float* __restrict__ proj, int stride, int t, int ch, int kk, const float* __restrict__ conv_w, size_t ws,
+                                                      const float* __restrict__ prev, int prev_stride, float* __restrict__ conv_out, float* __restrict__ co) {
+  const int c = blockIdx.x * 256 + threadIdx.x, z = blockIdx.y; if (c >= ch) return;
+  const float* pz = proj + (size_t)z * ws;
+  float w[8], hist[8];
+  for (int k = 0; k < kk; ++k) w[k] = conv_w[(size_t)c * kk + k];
+  if (z == 0) { for (int k = 0; k < kk - 1; ++k) hist[k] = prev[(size_t)k * prev_stride + c]; }
+  else { const float* pp = pz - ws + (size_t)(t - (kk - 1)) * stride; for (int k = 0; k < kk - 1; ++k) hist[k] = pp[(size_t)k * stride + c]; }
+  float* cz = co + (size_t)z * ws;
+  for (int ti = 0; ti < t; ++ti) {
+    float cur = pz[(size_t)ti * stride + c];
+    float o = w[kk - 1] * cur;
+    for (int k = 0; k < kk - 1; ++k) o += w[k] * hist[k];
+    cz[(size_t)ti * ch + c] = o * g_sigm(o);
+    for (int k = 0; k + 1 < kk - 1; ++k) hist[k] = hist[k + 1];
+    hist[kk - 2] = cur;
+  }
+  if (conv_out && z == (int)gridDim.y - 1) for (int k = 0; k < kk - 1; ++k) conv_out[(size_t)k * ch + c] = hist[k];
+}
+
 // grid nv, 512 threads (8 waves), at most 8 tokens.  Thread (grp = tid/128, j = tid%128) keeps rows 32*grp..32*grp+31 of
 // column j of the head's 128x128 state in registers across the whole window, so the state is read once and written once
 // per launch.  Whatever does not depend on the state is done per token by one wave each, before the recurrence (wave ti
@@ -190,6 +215,14 @@ int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int strid
   { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); if (t == 1 && g.nk == 16 && g.nv == 32) hipLaunchKernelGGL((k_gdn_delta<128, 128, 1, 16, 32>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up);          // a single token of the A3B geometry: constants folded in
     else hipLaunchKernelGGL((k_gdn_delta<128, 128>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
+}
+
+int pyre_gdn_conv_block_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, int n, size_t ws, const float* prev, int prev_stride, float* conv_out, float* co) {
+  if (g.conv_k < 2 || g.conv_k > 8 || t < g.conv_k - 1 || t > 8 || n < 1) return pyre_fail(ctx, PYRE_E_ARG, "gdn block conv: kernel %d, %d windows of %d tokens", g.conv_k, n, t);
+  const int ch = 2 * g.nk * g.dk + g.nv * g.dv;
+  ProfScope ps(ctx, "gdn_conv", 4.0 * ch * n * (g.conv_k + 2.0 * t));
+  hipLaunchKernelGGL(k_gdn_conv_blk, dim3((ch + 255) / 256, n), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, ws, prev, prev_stride, conv_out, co);
+  PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 
 // ---- C ABI: standalone layer core for the block harness ---------------------------------------------------------------

@@ -598,6 +598,7 @@ struct WinOpt {
   int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
   bool no_len = false;          // ... and the state's length is then advanced by the caller
   size_t win_stride = 0;        // bytes between this window's workspace and the next window's of its block (0: it stands alone)
+  bool proj_early = false;      // a block's window: the layer's projection is launched with the mix in front of it (front_pre_proj), a Gated DeltaNet layer's convolution once for the group (front_mid_conv): neither needs the layer's state
   bool attn_split = false; AttnWork aw_own{};      // a block's window: the attention pass over the cache leaves the chain through the layer's state (front_post_proj runs it); aw_own: the stream's attention workspace with q buffers of this window's own
 };
 
@@ -693,6 +694,20 @@ struct WinRun {
     advance(); comb_np = 1;
     return PYRE_OK;
   }
+  int front_pre_proj(int il) {          // (proj_early) the layer's projection, without the convolution
+    const Layer& L = m->layers[il];
+    const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
+    return pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, hc_fused(L.hca, L.proj) ? &aop_hc : nullptr);
+  }
+  // (proj_early) the convolution of this window and the n - 1 after it, a Gated DeltaNet layer: the history in front of this
+  // window is the layer's state (first: the block's first window) or the last rows of the window before it; the last window
+  // of the block leaves the state where the windows' recurrences will have turned the layer's buffers to
+  int front_mid_conv(int il, int n, bool first, bool last) {
+    const pyre_model_cfg& c = m->c; const Layer& L = m->layers[il]; if (L.full) return PYRE_OK;
+    const int li = L.mix_index, b = s->cur[li], K1 = c.conv_k - 1;
+    const float* prev = first ? s->conv[b][li] : m->proj - o.win_stride / 4 + (size_t)(t - K1) * m->pw_lin;
+    return pyre_gdn_conv_block_launch(ctx, L.gdn, m->proj, m->pw_lin, t, n, o.win_stride / 4, prev, first ? m->ch : m->pw_lin, last ? s->conv[b ^ (n & 1)][li] : nullptr, m->co);
+  }
   int front_mid(int il) {
     const pyre_model_cfg& c = m->c; int rc;
     const AttnWork& aw = o.attn_split ? o.aw_own : (o.aw ? *o.aw : s->aw); const QsaWork& qw = o.qw ? *o.qw : s->qw;
@@ -701,13 +716,13 @@ struct WinRun {
     const Layer& L = m->layers[il];
     if (L.full) {
       int ai = L.mix_index;
-      if ((rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.hca, L.proj)))) return rc;
+      if (!o.proj_early && (rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, opnd(L.hca, L.proj)))) return rc;
       if (m->has_idx && (rc = pyre_qsa_launch(ctx, L.qsa, L.attn, s->qsa[ai], qw, m->proj, m->pw_attn, m->iq_off, start, t, o.step_dev))) return rc;
       if ((rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], aw, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, o.step_dev, m->has_idx ? &qw : nullptr, o.attn_split ? 1 : 0))) return rc;
     } else {
-      int li = L.mix_index; float* pj = s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
+      int li = L.mix_index; float* pj = o.proj_early ? m->proj : s->proj_saved[li]; int b = s->cur[li], nb = (replay || o.inplace) ? b : b ^ 1;
       GemvEpi cv{nullptr, L.gdn.conv_w, s->conv[b][li], s->conv[nb][li], m->co, m->ch, c.conv_k};      // conv1d + SiLU ride on the projection
-      if ((rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.hca, L.proj)))) return rc;
+      if (!o.proj_early && (rc = pyre_gemv_conv_launch(ctx, L.proj, m->mixed, t, pj, cv, opnd(L.hca, L.proj)))) return rc;
       const GdnQ gq{m->aop, m->gdn_sq};
       if ((rc = pyre_gdn_launch(ctx, L.gdn, pj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, gdn_fused(L) ? m->aop : nullptr, L.gdn_up, gdn_q_on(m, L) ? &gq : nullptr))) return rc;
       s->cur[li] = nb;
@@ -838,6 +853,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     const int nl = m->c.n_layers;
     const int G_env = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : 0; return v < 0 ? 0 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }();      // PYRE_PROMPT_GROUP: windows a group (default: a group a stream)
     const bool batch = [&] { const char* e = getenv("PYRE_PROMPT_BATCH"); if (e && *e && atoi(e) == 0) return false; for (const Layer& L : m->layers) if (!pyre_hc_aop_ok(L.hca) || !pyre_hc_aop_ok(L.hcf)) return false; return true; }();      // a group's mixes in one launch each (the matrix-core mixes; PYRE_PROMPT_BATCH=0: a launch a window)
+    const bool early = batch && m->c.conv_k >= 2 && m->c.conv_k <= 9 && !(getenv("PYRE_PROMPT_PROJ_EARLY") && atoi(getenv("PYRE_PROMPT_PROJ_EARLY")) == 0);      // the projections in front of the chain through the layer's state, the convolution once a group (PYRE_PROMPT_PROJ_EARLY=0: both in the chain, a window at a time)
     const bool pairs = [] { const char* e = getenv("PYRE_PROMPT_PAIRS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_PAIRS=0: one block at a time
     auto cxk = [&](int k) { return k ? P->ctx[k - 1] : ctx; };
     auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(P->moe_ctx->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
@@ -862,7 +878,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
         for (int j = 0; j < b.NB; ++j) {
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
-          o.win_stride = P->win_stride;
+          o.win_stride = P->win_stride; o.proj_early = early;
           if (P->qmem) {          // q buffers of the window's own; the partial sums stay the stream's
             o.attn_split = true; o.aw_own = set ? s->aw_more[set - 1] : s->aw;
             uint8_t* qb = (uint8_t*)P->qmem + (size_t)(w * NBMAX + j) * P->q_stride;
@@ -881,8 +897,10 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           if (il > 0 && g < K && hipStreamWaitEvent(cx->stream, P->moe_done[b.which], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
           const int j0 = g * G, j1 = j0 + G < b.NB ? j0 + G : b.NB;
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;            // the group's mixes: one launch each
+          if (early) for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre_proj(il))) return r;
           const int pset = g > 0 ? (g - 1) % K : b.prev_in;
           if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
+          if (early && (r = b.runs[j0].front_mid_conv(il, j1 - j0, j0 == 0, j1 == b.NB))) return r;
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il))) return r;
