@@ -108,10 +108,14 @@ __device__ __forceinline__ void load_a_x(const float* __restrict__ x, int c, int
 }
 //   SQ: the operand of a Gated DeltaNet output projection with per-sub-block scales and the head norm (load_a_sq).
 template <int NW, bool SC, bool CONV, int FT = 0, bool XF = false, bool SQ = false>
-__global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep) {
+__global__ __launch_bounds__(NW * 64) void k_gemm_m(QMatDev m, const uint4* __restrict__ aop, const float* __restrict__ ainv, float* __restrict__ y, int T, int R, int cpw, GemvEpi ep, size_t wz) {
   __shared__ float red[NW][4][2][64];
   PYRE_TS_VARS PYRE_TS(0);
   qmat_args_now(m); args_now(aop, ainv, y, T, R, cpw, ep.best, ep.conv_w, ep.conv_in, ep.conv_out, ep.co, ep.ch, ep.kk);
+  if (wz) {          // a launch for several windows (a long prompt's blocks): blockIdx.z's operand, scale factors and output lie wz bytes further on per window
+    const size_t zo = (size_t)blockIdx.z * wz;
+    aop = (const uint4*)((const char*)aop + zo); y = (float*)((char*)y + zo); if (ainv) ainv = (const float*)((const char*)ainv + zo);
+  }
   constexpr bool ONE = FT == 1;
   if constexpr (FT > 0) { T = FT; R = FT <= 1 ? 2 : (FT == 2 ? 4 : (FT <= 4 ? 8 : 16)); }
   const int kk = FT > 0 ? 4 : ep.kk;
@@ -210,18 +214,18 @@ int gemm_m_nw(const QMatDev& m, int ksplit) {
   return nw;
 }
 template <int NW> void gemm_m_go(pyre_ctx* ctx, const QMatDev& m, const PyreAop& a, int t, float* y, int ksplit, int cpw, const GemvEpi& ep, const float* xf = nullptr) {
-  if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, 1, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep); return; }
+  if (xf) { hipLaunchKernelGGL((k_gemm_m<NW, true, false, 1, true>), dim3(m.tiles, ksplit, ctx->batch_n), dim3(NW * 64), 0, ctx->stream, m, (const uint4*)xf, (const float*)nullptr, y, 1, 2, cpw, ep, ctx->batch_stride); return; }
 #define GEMM_M_T(CALL) switch (t) { case 1: { constexpr int FT = 1; CALL; } break; case 2: { constexpr int FT = 2; CALL; } break; case 3: { constexpr int FT = 3; CALL; } break; case 4: { constexpr int FT = 4; CALL; } break; \
     case 5: { constexpr int FT = 5; CALL; } break; case 6: { constexpr int FT = 6; CALL; } break; case 7: { constexpr int FT = 7; CALL; } break; default: { constexpr int FT = 8; CALL; } break; }
   if (a.sq) {          // (the launcher has checked: no conv epilogue, chunks = heads)
     GemvEpi e2 = ep; e2.sq_heads = a.sq_heads; e2.sq_eps = a.sq_eps;
-    GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT, false, true>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, t, pyre_aop_rows(t), cpw, e2));
+    GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT, false, true>), dim3(m.tiles, ksplit, ctx->batch_n), dim3(NW * 64), 0, ctx->stream, m, a.op, a.sq, y, t, pyre_aop_rows(t), cpw, e2, ctx->batch_stride));
     return;
   }
-#define GEMM_M_GO(SC, CONV) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, 0>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)
+#define GEMM_M_GO(SC, CONV) hipLaunchKernelGGL((k_gemm_m<NW, SC, CONV, 0>), dim3(m.tiles, ksplit, ctx->batch_n), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep, ctx->batch_stride)
   if (a.ainv && (!ep.co || ep.kk == 4)) {          // scaled operand rows (every launch of the model and of the operator): the instance with the window width folded in
-    if (ep.co) { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, true, FT>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)); }
-    else { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT>), dim3(m.tiles, ksplit), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep)); }
+    if (ep.co) { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, true, FT>), dim3(m.tiles, ksplit, ctx->batch_n), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep, ctx->batch_stride)); }
+    else { GEMM_M_T(hipLaunchKernelGGL((k_gemm_m<NW, true, false, FT>), dim3(m.tiles, ksplit, ctx->batch_n), dim3(NW * 64), 0, ctx->stream, m, a.op, a.ainv, y, t, pyre_aop_rows(t), cpw, ep, ctx->batch_stride)); }
   }
   else if (ep.co) { if (a.ainv) GEMM_M_GO(true, true); else GEMM_M_GO(false, true); }
   else { if (a.ainv) GEMM_M_GO(true, false); else GEMM_M_GO(false, false); }

@@ -694,10 +694,17 @@ struct WinRun {
     advance(); comb_np = 1;
     return PYRE_OK;
   }
-  int front_pre_proj(int il) {          // (proj_early) the layer's projection, without the convolution
-    const Layer& L = m->layers[il];
+  // whether one launch of layer il's projection / output projection can serve several windows: the operand comes from the
+  // window's own workspace (the mix's, the recurrence's per-quarter form), not through the context's split buffer
+  bool proj_batchable(int il) const { const Layer& L = m->layers[il]; return hc_fused(L.hca, L.proj); }
+  bool outp_batchable(int il) const { const Layer& L = m->layers[il]; return !L.full && gdn_q_on(m, L) && L.outp.fmt == FMT_IQ3_S_M; }
+  int front_pre_proj(int il, int nz = 1) {          // (proj_early) the layer's projection, without the convolution (nz as in front_pre)
+    const Layer& L = m->layers[il]; if (nz <= 0) return PYRE_OK;
     const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
-    return pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, hc_fused(L.hca, L.proj) ? &aop_hc : nullptr);
+    ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
+    const int rc = pyre_gemv_launch(ctx, L.proj, m->mixed, t, m->proj, hc_fused(L.hca, L.proj) ? &aop_hc : nullptr);
+    ctx->batch_n = 1; ctx->batch_stride = 0;
+    return rc;
   }
   // (proj_early) the convolution of this window and the n - 1 after it, a Gated DeltaNet layer: the history in front of this
   // window is the layer's state (first: the block's first window) or the last rows of the window before it; the last window
@@ -729,15 +736,18 @@ struct WinRun {
     }
     return PYRE_OK;
   }
-  int front_post_proj(int il) {          // the output projection (in front of it, for a block's window, the attention pass its mid left out)
+  int front_post_proj(int il, int nz = 1) {          // the output projection (nz as in front_pre; in front of it, for a block's window, the attention pass its mid left out)
     const pyre_model_cfg& c = m->c; const int d = c.d;
     const Layer& L = m->layers[il];
     if (L.full && o.attn_split) { int rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[L.mix_index], o.aw_own, m->proj, m->pw_attn, start, t, &s->packed[L.mix_index], m->core, nullptr, nullptr, 2); if (rc) return rc; }
+    if (nz <= 0) return PYRE_OK;
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
+    ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
     // few row tiles, long rows: four workgroups per row tile leave partial sums, the mix below adds them
-    if (outp_in_parts(L, d)) return pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa);
-    return pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa);
+    const int rc = outp_in_parts(L, d) ? pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, oa) : pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, oa);
+    ctx->batch_n = 1; ctx->batch_stride = 0;
+    return rc;
   }
   int front_post_mix(int il, int nz = 1) {          // the FFN mix (nz as in front_pre)
     const pyre_model_cfg& c = m->c; const int d = c.d; int rc;
@@ -897,13 +907,13 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           if (il > 0 && g < K && hipStreamWaitEvent(cx->stream, P->moe_done[b.which], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
           const int j0 = g * G, j1 = j0 + G < b.NB ? j0 + G : b.NB;
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;            // the group's mixes: one launch each
-          if (early) for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre_proj(il))) return r;
+          if (early) { const bool pb = b.runs[j0].proj_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre_proj(il, pb ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
           const int pset = g > 0 ? (g - 1) % K : b.prev_in;
           if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
           if (early && (r = b.runs[j0].front_mid_conv(il, j1 - j0, j0 == 0, j1 == b.NB))) return r;
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
-          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il))) return r;
+          { const bool ob = batch && b.runs[j0].outp_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il, ob ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_mix(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;
         }
         return PYRE_OK;

@@ -355,6 +355,7 @@ template <int FMT> int gemv_f(pyre_ctx* ctx, const QMatDev& m, const float* x, i
 // context's operand buffer first (sized by pyre_gemm_m_scratch; grows only outside stream capture).
 int gemm_m_from_f32(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, int ksplit, const GemvEpi& ep, const PyreAop* a) {
   if (a && a->op) return pyre_gemm_m_launch(ctx, m, *a, t, y, ksplit, ep);
+  if (ctx->batch_n > 1) return pyre_fail(ctx, PYRE_E_ARG, "gemv: a launch for several windows needs the windows' own operands");
   if (pyre_gemm_m_x_ok(m, t, ep)) return pyre_gemm_m_launch(ctx, m, PyreAop{nullptr, nullptr}, 1, y, ksplit, ep, x);          // few row tiles: the product converts x itself, a launch less
   uint4* op; float* ainv; int rc = pyre_gemm_m_scratch(ctx, m.cols, &op, &ainv); if (rc) return rc;
   if ((rc = pyre_act_split_launch(ctx, x, t, m.cols, op, ainv))) return rc;
@@ -365,6 +366,7 @@ int gemm_m_from_f32(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, floa
 void pyre_gemv_plan(const QMatDev& m, int* nw, int* upw) { *nw = gemv_nw(m, 1); *upw = (m.U + *nw - 1) / *nw; if (*upw < 1) *upw = 1; }
 int pyre_gemv_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int t, float* y, const PyreAop* a) {
   if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, y, 1, GemvEpi{}, a);
+  if (ctx->batch_n > 1) return pyre_fail(ctx, PYRE_E_ARG, "gemv: only the matrix-core GEMM serves several windows a launch");
   int rc = PYRE_OK;
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, y, 1, GemvEpi{}));
   return rc;
@@ -385,6 +387,7 @@ int pyre_gemv_parts_launch(pyre_ctx* ctx, const QMatDev& m, const float* x, int 
   int rc = PYRE_OK;
   GemvEpi ep{}; ep.four_waves = 1;
   if (m.fmt == FMT_IQ3_S_M) return gemm_m_from_f32(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep, a);
+  if (ctx->batch_n > 1) return pyre_fail(ctx, PYRE_E_ARG, "gemv: only the matrix-core GEMM serves several windows a launch");
   FMT_DISPATCH(m.fmt, rc = gemv_f<F>(ctx, m, x, t, parts, PYRE_GEMV_PARTS, ep));
   return rc;
 }
