@@ -387,7 +387,7 @@ struct GdnQ { uint16_t* op; float* sq; };
 // the convolution of n consecutive windows of t tokens in one launch (gdn.hip: k_gdn_conv_blk)
 int pyre_gdn_conv_block_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, int n, size_t ws, const float* prev, int prev_stride, float* conv_out, float* co);
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int proj_stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f, const GdnQ* gq = nullptr);
+                    const float* ssm_in, float* ssm_out, float* co_scratch, float* out_dev, bool conv_done = false, uint16_t* aop = nullptr, float aop_up = 1.0f, const GdnQ* gq = nullptr, int nwin = 1, size_t ws = 0);      // nwin > 1: that many consecutive windows, their projections, convolution outputs and operands ws floats apart, in one launch (the per-quarter form, conv_done)
 
 // Chunked (64-token) form of the same recurrence on the fp32 matrix cores; T must be a positive multiple of 64.
 // scratch: co [T][ch], logg [T][nv], beta [T][nv], oraw [T][nv*dv].

@@ -127,9 +127,12 @@ __global__ __launch_bounds__(512) void k_gdn_delta(GdnDev p, const float* __rest
 // all 128 columns, so it is left to the consumer (the output projection, PyreAop::sq): wave ti leaves token ti's
 // un-normalised gated output u = (o * norm_w) * sigmoid(z) of its 32 columns as f16 operand rows scaled by the quarter's own
 // power of two (its largest magnitude into [2^13, 2^14)), that factor's inverse, and the quarter's sum of o^2.
+// nwin > 1 (a long prompt's blocks): nwin consecutive windows of t tokens in one launch -- window wi's projection, convolution
+// output, operand rows and sums lie ws floats further on per window (the windows' workspaces); the state stays in registers
+// from window to window, is fetched once and stored once.  A token's arithmetic is the same whatever nwin.
 template <int DK, int DV, int FT = 0, int FNK = 0, int FNV = 0>
 __global__ __launch_bounds__(512) void k_gdn_delta_q(GdnDev p, const float* __restrict__ proj, int stride, int t, const float* __restrict__ co_all,
-                                                     const float* __restrict__ ssm_in, float* __restrict__ ssm_out, uint16_t* __restrict__ aop, int aop_rows, float* __restrict__ sq) {
+                                                     const float* __restrict__ ssm_in, float* __restrict__ ssm_out, uint16_t* __restrict__ aop, int aop_rows, float* __restrict__ sq, int nwin, size_t ws) {
   static_assert(DK == 128 && DV == 128, "tiling assumes 128x128 heads");
   constexpr int QC = 32, G = 16, R = DK / G, MT = 8;
   args_now(p.a, p.dt, p.norm_w, p.nk, p.nv, p.eps, proj, stride, t, co_all, ssm_in, ssm_out, aop, sq);
@@ -140,61 +143,72 @@ __global__ __launch_bounds__(512) void k_gdn_delta_q(GdnDev p, const float* __re
   const int ch = 2 * p.nk * DK + p.nv * DV, w = p.nv * DV, jc = qd * QC + j;
   const float* sin_ = ssm_in + (size_t)h * DK * DV; float* sout = ssm_out + (size_t)h * DK * DV;
   float q0 = 0.0f, q1 = 0.0f, k0 = 0.0f, k1 = 0.0f, v0 = 0.0f, z0 = 0.0f, alpha_raw = 0.0f, beta_raw = 0.0f;
-  if (wave < t) {
-    const float* co = co_all + (size_t)wave * ch; const float* pr = proj + (size_t)wave * stride;
-    q0 = co[kh * DK + lane]; q1 = co[kh * DK + lane + 64]; k0 = co[p.nk * DK + kh * DK + lane]; k1 = co[p.nk * DK + kh * DK + lane + 64];
-    v0 = co[2 * p.nk * DK + h * DV + qd * QC + (lane & 31)]; z0 = pr[ch + h * DV + qd * QC + (lane & 31)];
-    alpha_raw = pr[ch + w + p.nv + h]; beta_raw = pr[ch + w + h];
-  }
+  auto fetch = [&](int wi) {          // wave ti: token ti's inputs of window wi
+    if (wave < t) {
+      const float* co = co_all + (size_t)wi * ws + (size_t)wave * ch; const float* pr = proj + (size_t)wi * ws + (size_t)wave * stride;
+      q0 = co[kh * DK + lane]; q1 = co[kh * DK + lane + 64]; k0 = co[p.nk * DK + kh * DK + lane]; k1 = co[p.nk * DK + kh * DK + lane + 64];
+      v0 = co[2 * p.nk * DK + h * DV + qd * QC + (lane & 31)]; z0 = pr[ch + h * DV + qd * QC + (lane & 31)];
+      alpha_raw = pr[ch + w + p.nv + h]; beta_raw = pr[ch + w + h];
+    }
+  };
+  fetch(0);
   const float a = p.a[h], dtb = p.dt[h], nw = p.norm_w[qd * QC + (lane & 31)];
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) S[r] = sin_[(size_t)(rg * R + r) * DV + jc];
-  if (wave < t) {          // L2 norms of q and k (:1649-1651): the sum of each half of the vector, then the two halves -- as in k_gdn_delta
-    const float sq_ = wave_sum(q0 * q0) + wave_sum(q1 * q1), sk = wave_sum(k0 * k0) + wave_sum(k1 * k1);
-    const float fq = (1.0f / sqrtf(sq_ + 1e-6f)) * (1.0f / sqrtf((float)DK)), fk = (1.0f / sqrtf(sk + 1e-6f)) * 1.0f;
-    qs[wave][lane] = q0 * fq; qs[wave][lane + 64] = q1 * fq; ks[wave][lane] = k0 * fk; ks[wave][lane + 64] = k1 * fk;
-    if (lane < QC) { vs[wave][lane] = v0; zs[wave][lane] = z0; }
-    if (lane == 0) { gs[wave] = expf(g_softplus(alpha_raw + dtb) * a); bs[wave] = g_sigm(beta_raw); }
-  }
-  lds_barrier();
-  for (int ti = 0; ti < t; ++ti) {
-    const float g = gs[ti], b = bs[ti];
-    float pmv = 0.0f;
-#pragma unroll
-    for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[ti][rg * R + r]; }
-    pm[ti & 1][rg][j] = pmv;
+  for (int wi = 0; wi < nwin; ++wi) {
+    if (wave < t) {          // L2 norms of q and k (:1649-1651): the sum of each half of the vector, then the two halves -- as in k_gdn_delta
+      const float sq_ = wave_sum(q0 * q0) + wave_sum(q1 * q1), sk = wave_sum(k0 * k0) + wave_sum(k1 * k1);
+      const float fq = (1.0f / sqrtf(sq_ + 1e-6f)) * (1.0f / sqrtf((float)DK)), fk = (1.0f / sqrtf(sk + 1e-6f)) * 1.0f;
+      qs[wave][lane] = q0 * fq; qs[wave][lane + 64] = q1 * fq; ks[wave][lane] = k0 * fk; ks[wave][lane + 64] = k1 * fk;
+      if (lane < QC) { vs[wave][lane] = v0; zs[wave][lane] = z0; }
+      if (lane == 0) { gs[wave] = expf(g_softplus(alpha_raw + dtb) * a); bs[wave] = g_sigm(beta_raw); }
+    }
+    if (wi + 1 < nwin) fetch(wi + 1);          // the next window's inputs travel behind this window's recurrence
     lds_barrier();
-    float mem = pm[ti & 1][0][j];
+    for (int ti = 0; ti < t; ++ti) {
+      const float g = gs[ti], b = bs[ti];
+      float pmv = 0.0f;
 #pragma unroll
-    for (int k = 1; k < G; ++k) mem += pm[ti & 1][k][j];
-    const float delta = (vs[ti][j] - mem) * b;
-    float pov = 0.0f;
+      for (int r = 0; r < R; ++r) { S[r] *= g; pmv += S[r] * ks[ti][rg * R + r]; }
+      pm[ti & 1][rg][j] = pmv;
+      lds_barrier();
+      float mem = pm[ti & 1][0][j];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { S[r] += ks[ti][rg * R + r] * delta; pov += S[r] * qs[ti][rg * R + r]; }
-    po[ti][rg][j] = pov;
-  }
+      for (int k = 1; k < G; ++k) mem += pm[ti & 1][k][j];
+      const float delta = (vs[ti][j] - mem) * b;
+      float pov = 0.0f;
 #pragma unroll
-  for (int r = 0; r < R; ++r) sout[(size_t)(rg * R + r) * DV + jc] = S[r];
-  lds_barrier();
-  if (wave < t) {
-    const int jl = lane & 31; const bool on = lane < QC;
-    float o = po[wave][0][jl];
+      for (int r = 0; r < R; ++r) { S[r] += ks[ti][rg * R + r] * delta; pov += S[r] * qs[ti][rg * R + r]; }
+      po[ti][rg][j] = pov;
+    }
+    if (wi + 1 == nwin) {
 #pragma unroll
-    for (int k = 1; k < G; ++k) o += po[wave][k][jl];
-    const float ss = wave_sum(on ? o * o : 0.0f);
-    const float u = (o * nw) * g_sigm(zs[wave][jl]);
-    float am = on ? fabsf(u) : 0.0f; am = am == am ? am : INFINITY;
-    am = wave_max(am);
-    int e = 0;
-    if (am > 0.0f && am < INFINITY) { e = 140 - (int)((__float_as_uint(am) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
-    if (on) aop_store(aop, aop_rows, h * DV + qd * QC + jl, wave, u * __uint_as_float((uint32_t)(127 + e) << 23));
-    if (lane == 0) { sq[((size_t)wave * p.nv + h) * 4 + qd] = __uint_as_float((uint32_t)(127 - e) << 23); sq[(size_t)8 * p.nv * 4 + ((size_t)wave * p.nv + h) * 4 + qd] = ss; }
+      for (int r = 0; r < R; ++r) sout[(size_t)(rg * R + r) * DV + jc] = S[r];
+    }
+    lds_barrier();
+    if (wave < t) {
+      const int jl = lane & 31; const bool on = lane < QC;
+      float o = po[wave][0][jl];
+#pragma unroll
+      for (int k = 1; k < G; ++k) o += po[wave][k][jl];
+      const float ss = wave_sum(on ? o * o : 0.0f);
+      const float u = (o * nw) * g_sigm(zs[wave][jl]);
+      float am = on ? fabsf(u) : 0.0f; am = am == am ? am : INFINITY;
+      am = wave_max(am);
+      int e = 0;
+      if (am > 0.0f && am < INFINITY) { e = 140 - (int)((__float_as_uint(am) >> 23) & 0xFF); e = e > 100 ? 100 : e; }
+      uint16_t* aw = aop + (size_t)wi * ws * 2; float* sw = sq + (size_t)wi * ws;
+      if (on) aop_store(aw, aop_rows, h * DV + qd * QC + jl, wave, u * __uint_as_float((uint32_t)(127 + e) << 23));
+      if (lane == 0) { sw[((size_t)wave * p.nv + h) * 4 + qd] = __uint_as_float((uint32_t)(127 - e) << 23); sw[(size_t)8 * p.nv * 4 + ((size_t)wave * p.nv + h) * 4 + qd] = ss; }
+    }
+    if (wi + 1 < nwin) lds_barrier();          // the next window's inputs overwrite what this window's outputs were read from
   }
 }
 
 int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int stride, int t, const float* conv_in, float* conv_out,
-                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done, uint16_t* aop, float aop_up, const GdnQ* gq) {
+                    const float* ssm_in, float* ssm_out, float* co, float* out, bool conv_done, uint16_t* aop, float aop_up, const GdnQ* gq, int nwin, size_t ws) {
+  if (nwin < 1 || (nwin > 1 && !(gq && conv_done))) return pyre_fail(ctx, PYRE_E_ARG, "gdn: several windows a launch need the per-quarter form behind a finished convolution");
   if (aop && t > 8) return pyre_fail(ctx, PYRE_E_ARG, "gdn: an f16 operand holds at most 8 tokens, not %d", t);
   if (gq && (!gq->op || !gq->sq)) return pyre_fail(ctx, PYRE_E_ARG, "gdn: the per-quarter form needs its operand and scale arrays");
   if (g.dk != 128 || g.dv != 128) return pyre_fail(ctx, PYRE_E_SHAPE, "gdn: head dims %dx%d unsupported (128x128 only)", g.dk, g.dv);
@@ -204,12 +218,12 @@ int pyre_gdn_launch(pyre_ctx* ctx, const GdnDev& g, const float* proj, int strid
   if (!conv_done) { ProfScope ps(ctx, "gdn_conv", 4.0 * ch * (2.0 * (g.conv_k - 1) + g.conv_k + 2.0 * t)); hipLaunchKernelGGL(k_gdn_conv, dim3((ch + 255) / 256), dim3(256), 0, ctx->stream, proj, stride, t, ch, g.conv_k, g.conv_w, conv_in, conv_out, co); } PYRE_CHECK_LAUNCH(ctx);
   if (gq) {
     ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv));
-#define GDN_Q_FIX(FT) hipLaunchKernelGGL((k_gdn_delta_q<128, 128, FT, 16, 32>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq)
+#define GDN_Q_FIX(FT) hipLaunchKernelGGL((k_gdn_delta_q<128, 128, FT, 16, 32>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq, nwin, ws)
     if (g.nk == 16 && g.nv == 32) {          // the A3B geometry: the window width and the head counts folded in
       switch (t) { case 1: GDN_Q_FIX(1); break; case 2: GDN_Q_FIX(2); break; case 3: GDN_Q_FIX(3); break; case 4: GDN_Q_FIX(4); break; case 5: GDN_Q_FIX(5); break; case 6: GDN_Q_FIX(6); break; case 7: GDN_Q_FIX(7); break; default: GDN_Q_FIX(8); break; }
     }
 #undef GDN_Q_FIX
-    else hipLaunchKernelGGL((k_gdn_delta_q<128, 128>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq);
+    else hipLaunchKernelGGL((k_gdn_delta_q<128, 128>), dim3(g.nv, 4), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, gq->op, pyre_aop_rows(t), gq->sq, nwin, ws);
     PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
   }
   { ProfScope ps(ctx, "gdn_delta", 8.0 * g.nv * g.dk * g.dv + 4.0 * t * (ch + 2.0 * g.nv * g.dv)); if (t == 1 && g.nk == 16 && g.nv == 32) hipLaunchKernelGGL((k_gdn_delta<128, 128, 1, 16, 32>), dim3(g.nv), dim3(512), 0, ctx->stream, g, proj, stride, t, co, ssm_in, ssm_out, out, aop, aop ? pyre_aop_rows(t) : 0, aop_up);          // a single token of the A3B geometry: constants folded in

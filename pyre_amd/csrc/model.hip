@@ -709,11 +709,21 @@ struct WinRun {
   // (proj_early) the convolution of this window and the n - 1 after it, a Gated DeltaNet layer: the history in front of this
   // window is the layer's state (first: the block's first window) or the last rows of the window before it; the last window
   // of the block leaves the state where the windows' recurrences will have turned the layer's buffers to
-  int front_mid_conv(int il, int n, bool first, bool last) {
+  int front_mid_conv(int il, int n, bool first, bool last, int flips) {          // flips: turns of the layer's state buffers between here and the end of these windows' recurrences
     const pyre_model_cfg& c = m->c; const Layer& L = m->layers[il]; if (L.full) return PYRE_OK;
     const int li = L.mix_index, b = s->cur[li], K1 = c.conv_k - 1;
     const float* prev = first ? s->conv[b][li] : m->proj - o.win_stride / 4 + (size_t)(t - K1) * m->pw_lin;
-    return pyre_gdn_conv_block_launch(ctx, L.gdn, m->proj, m->pw_lin, t, n, o.win_stride / 4, prev, first ? m->ch : m->pw_lin, last ? s->conv[b ^ (n & 1)][li] : nullptr, m->co);
+    return pyre_gdn_conv_block_launch(ctx, L.gdn, m->proj, m->pw_lin, t, n, o.win_stride / 4, prev, first ? m->ch : m->pw_lin, last ? s->conv[b ^ (flips & 1)][li] : nullptr, m->co);
+  }
+  // (proj_early) the recurrence of this window and the n - 1 after it in one launch: the state stays in registers from window to window
+  bool gdn_group_ok(int il) const { const Layer& L = m->layers[il]; return !L.full && gdn_q_on(m, L); }
+  int front_mid_gdn(int il, int n) {
+    const Layer& L = m->layers[il]; const int li = L.mix_index, b = s->cur[li], nb = b ^ 1;
+    const GdnQ gq{m->aop, m->gdn_sq};
+    int rc = pyre_gdn_launch(ctx, L.gdn, m->proj, m->pw_lin, t, s->conv[b][li], s->conv[nb][li], s->ssm[b][li], s->ssm[nb][li], m->co, m->core, true, nullptr, L.gdn_up, &gq, n, o.win_stride / 4);
+    if (rc) return rc;
+    s->cur[li] = nb;
+    return PYRE_OK;
   }
   int front_mid(int il) {
     const pyre_model_cfg& c = m->c; int rc;
@@ -910,8 +920,10 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           if (early) { const bool pb = b.runs[j0].proj_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_pre_proj(il, pb ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
           const int pset = g > 0 ? (g - 1) % K : b.prev_in;
           if (pset >= 0 && pset != k && hipStreamWaitEvent(cx->stream, P->ev[pset][il], 0) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipStreamWaitEvent failed");
-          if (early && (r = b.runs[j0].front_mid_conv(il, j1 - j0, j0 == 0, j1 == b.NB))) return r;
-          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
+          const bool gg = early && b.runs[j0].gdn_group_ok(il);          // the group's recurrences in one launch
+          if (early && (r = b.runs[j0].front_mid_conv(il, j1 - j0, j0 == 0, j1 == b.NB, gg ? 1 : j1 - j0))) return r;
+          if (gg) { if ((r = b.runs[j0].front_mid_gdn(il, j1 - j0))) return r; }
+          else for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
           { const bool ob = batch && b.runs[j0].outp_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il, ob ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_mix(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;
