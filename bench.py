@@ -696,7 +696,7 @@ def bench_decode(args):
         "kernels": breakdown,
     }
     out["prompt"] = {"tokens": n_ctx, "seconds": round(prefill_s, 2), "tok_s": round(n_ctx / prefill_s, 1),
-                     "note": "pyre_forward over the prompt in calls of 2048 tokens (windows of 8 tokens, three in flight, taken in blocks of up to 512 tokens layer by layer, two blocks at a time, each block's FFN grouped by expert on the matrix cores beside the other block's windows), logits of the last token only; untimed part of the step metric"}
+                     "note": "pyre_forward over the prompt in calls of 2048 tokens (windows of 8 tokens, three in flight, taken in blocks of up to 1024 tokens layer by layer, two blocks at a time, each block's FFN grouped by expert on the matrix cores beside the other block's windows), logits of the last token only; untimed part of the step metric"}
     if spec:
         out["spec_verify"] = spec
     if host_loop:

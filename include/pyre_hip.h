@@ -263,7 +263,7 @@ int   pyre_model_create(pyre_ctx* ctx, const pyre_model_cfg* cfg, const pyre_ten
 void  pyre_model_destroy(pyre_model* m);
 /* GGUF bytes of the weights one decode step reads (dense matrices, router, top_k + 1 experts, head, one embedding row). */
 size_t pyre_model_weight_bytes_per_token(const pyre_model* m);
-/* Blocks of up to 512 prompt tokens this model's pyre_forward calls have taken layer by layer with the FFN grouped by expert on the
+/* Blocks of up to 1024 prompt tokens this model's pyre_forward calls have taken layer by layer with the FFN grouped by expert on the
  * matrix cores since it was created (the prompt path at t >= 16: QMat::matmul's switch to a GEMM, src/model/gguf_q.rs:219-232, and
  * the chunk loop of src/engine_qn.rs:117-138).  A call takes that path for the whole blocks in front of its last tokens when every
  * layer's experts are IQ3_S with equal widths that are multiples of 256; PYRE_PROMPT_BLOCK=0 at model creation keeps the experts in one

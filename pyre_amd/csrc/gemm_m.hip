@@ -29,8 +29,9 @@ size_t pyre_aop_bytes(int cols, int t) { return (size_t)(cols / 8) * pyre_aop_ro
 // ---- the activation operand from f32 rows: grid = super-blocks (256 columns), 256 threads, thread = column ---------------------
 // Each 256-column stretch of a token is scaled by its own power of two so that its largest magnitude lands in [2^13, 2^14):
 // the f16 halves then keep 22 bits of every value that matters to the sum, whatever the magnitudes of x.
-__global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, int T, int R, int cols, uint16_t* __restrict__ op, float* __restrict__ ainv) {
+__global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, int T, int R, int cols, uint16_t* __restrict__ op, float* __restrict__ ainv, size_t wz) {
   __shared__ float mx[4][8];
+  if (wz) { const size_t zo = (size_t)blockIdx.y * wz; x = (const float*)((const char*)x + zo); op = (uint16_t*)((char*)op + zo); ainv = (float*)((char*)ainv + zo); }      // a launch for several windows, their buffers wz bytes apart
   PYRE_TS_VARS PYRE_TS(0);
   const int sb = blockIdx.x, i = threadIdx.x, k = sb * 256 + i, wave = i >> 6, lane = i & 63;
   float v[8];
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(256) void k_act_split(const float* __restrict__ x, 
 
 int pyre_act_split_launch(pyre_ctx* ctx, const float* x_dev, int t, int cols, uint4* op, float* ainv) {
   ProfScope ps(ctx, "act_split_f16", 4.0 * t * cols + (double)pyre_aop_bytes(cols, t));
-  hipLaunchKernelGGL(k_act_split, dim3(cols / 256), dim3(256), 0, ctx->stream, x_dev, t, pyre_aop_rows(t), cols, (uint16_t*)op, ainv);
+  hipLaunchKernelGGL(k_act_split, dim3(cols / 256, ctx->batch_n), dim3(256), 0, ctx->stream, x_dev, t, pyre_aop_rows(t), cols, (uint16_t*)op, ainv, ctx->batch_stride);
   PYRE_CHECK_LAUNCH(ctx); return PYRE_OK;
 }
 

@@ -530,7 +530,7 @@ static int prompt_pipe_state(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, 
 // instead of fixed-point digits): equal to rounding, not bit for bit.  For models whose every layer qualifies
 // (prompt_block_ok); the call's last tokens (the window whose logits are read, the rows a drafter keeps) take the windows'
 // path.  PYRE_PROMPT_BLOCK=0 switches it off.
-static int prompt_block_windows() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_BLOCK_WINDOWS"); int v = e && *e ? atoi(e) : 64; return v < 8 ? 8 : (v > 128 ? 128 : v); }(); return k; }      // the most windows a block has (read once)
+static int prompt_block_windows() { static const int k = [] { const char* e = getenv("PYRE_PROMPT_BLOCK_WINDOWS"); int v = e && *e ? atoi(e) : 128; return v < 8 ? 8 : (v > 128 ? 128 : v); }(); return k; }      // the most windows a block has (read once)
 #define PROMPT_BLOCK_WINDOWS prompt_block_windows()
 #define PROMPT_BLOCK_MIN 8
 static bool fuse_aop_on() { const char* e = getenv("PYRE_AOP_SPLIT"); return !(e && *e && atoi(e) != 0); }
@@ -697,7 +697,7 @@ struct WinRun {
   // whether one launch of layer il's projection / output projection can serve several windows: the operand comes from the
   // window's own workspace (the mix's, the recurrence's per-quarter form), not through the context's split buffer
   bool proj_batchable(int il) const { const Layer& L = m->layers[il]; return hc_fused(L.hca, L.proj); }
-  bool outp_batchable(int il) const { const Layer& L = m->layers[il]; return !L.full && gdn_q_on(m, L) && L.outp.fmt == FMT_IQ3_S_M; }
+  bool outp_batchable(int il) const { const Layer& L = m->layers[il]; return L.outp.fmt == FMT_IQ3_S_M && (L.full ? (o.attn_split && L.outp.cols % 256 == 0) : gdn_q_on(m, L)); }
   int front_pre_proj(int il, int nz = 1) {          // (proj_early) the layer's projection, without the convolution (nz as in front_pre)
     const Layer& L = m->layers[il]; if (nz <= 0) return PYRE_OK;
     const PyreAop aop_hc{(const uint4*)m->aop, m->aop_inv};
@@ -746,11 +746,23 @@ struct WinRun {
     }
     return PYRE_OK;
   }
-  int front_post_proj(int il, int nz = 1) {          // the output projection (nz as in front_pre; in front of it, for a block's window, the attention pass its mid left out)
+  int front_post_attn(int il) {          // for a block's window: the attention pass its mid left out
+    const Layer& L = m->layers[il];
+    if (!(L.full && o.attn_split)) return PYRE_OK;
+    return pyre_attn_launch_sel(ctx, L.attn, s->kv[L.mix_index], o.aw_own, m->proj, m->pw_attn, start, t, &s->packed[L.mix_index], m->core, nullptr, nullptr, 2);
+  }
+  int front_post_proj(int il, int nz = 1) {          // the output projection (nz as in front_pre)
     const pyre_model_cfg& c = m->c; const int d = c.d;
     const Layer& L = m->layers[il];
-    if (L.full && o.attn_split) { int rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[L.mix_index], o.aw_own, m->proj, m->pw_attn, start, t, &s->packed[L.mix_index], m->core, nullptr, nullptr, 2); if (rc) return rc; }
     if (nz <= 0) return PYRE_OK;
+    if (L.full && nz > 1) {          // an attention layer's output projection for several windows: the split into each window's own operand buffer (free since its projection), then the product
+      const PyreAop own{(const uint4*)m->aop, m->aop_inv};
+      ctx->batch_n = nz; ctx->batch_stride = o.win_stride;
+      int rc = pyre_act_split_launch(ctx, m->core, t, L.outp.cols, (uint4*)m->aop, m->aop_inv);
+      if (!rc) rc = outp_in_parts(L, d) ? pyre_gemv_parts_launch(ctx, L.outp, m->core, t, m->o, &own) : pyre_gemv_launch(ctx, L.outp, m->core, t, m->o, &own);
+      ctx->batch_n = 1; ctx->batch_stride = 0;
+      return rc;
+    }
     const PyreAop aop_gdn{(const uint4*)m->aop, L.gdn_ainv}, aop_gdq{(const uint4*)m->aop, nullptr, m->gdn_sq, L.gdn.nv, L.gdn.eps};
     const PyreAop* oa = (!L.full && gdn_q_on(m, L)) ? &aop_gdq : ((!L.full && gdn_fused(L)) ? &aop_gdn : nullptr);
     ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
@@ -774,7 +786,7 @@ struct WinRun {
     advance();
     return PYRE_OK;
   }
-  int front_post(int il) { int rc = front_post_proj(il); return rc ? rc : front_post_mix(il); }
+  int front_post(int il) { int rc = front_post_attn(il); if (!rc) rc = front_post_proj(il); return rc ? rc : front_post_mix(il); }
   int front(int il) {
     int rc; const Layer& L = m->layers[il];
     if (o.wait_ev && L.ple) PYRE_HIP(ctx, hipStreamWaitEvent(ctx->stream, o.wait_ev[il], 0));      // the layer's ring of rows is state
@@ -925,7 +937,8 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           if (gg) { if ((r = b.runs[j0].front_mid_gdn(il, j1 - j0))) return r; }
           else for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
-          { const bool ob = batch && b.runs[j0].outp_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il, ob ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
+          for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_attn(il))) return r;
+          { const bool ob = batch && j1 - j0 > 1 && b.runs[j0].outp_batchable(il); for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_proj(il, ob ? (j == j0 ? j1 - j0 : 0) : 1))) return r; }
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_mix(il, batch ? (j == j0 ? j1 - j0 : 0) : 1))) return r;
         }
         return PYRE_OK;

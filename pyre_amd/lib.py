@@ -688,7 +688,7 @@ class Model:
         return self.ctx.L.pyre_model_weight_bytes_per_token(self.h)
 
     def prompt_blocks(self):
-        """Blocks of up to 512 prompt tokens taken layer by layer with the FFN grouped by expert since the model was created."""
+        """Blocks of up to 1024 prompt tokens taken layer by layer with the FFN grouped by expert since the model was created."""
         return self.ctx.L.pyre_model_prompt_blocks(self.h)
 
     def new_state(self, max_ctx):
