@@ -566,7 +566,7 @@ static int prompt_block_get(pyre_ctx* ctx, const pyre_model* m, PromptPipe* P) {
   for (int w = 0; w < 2; ++w) { const pyre_model* f = P->wmdl[(size_t)w * NB]; P->blk[w].x = f->mixed; P->blk[w].rpart = f->rpart; P->blk[w].parts = f->mw.parts; P->blk[w].ws = ws / 4; }
   P->blk_nsl = nsl; P->blk_r64 = r64; P->win_stride = ws;
   { int rc = pyre_moe_block_zero_rows(ctx, m0, P->blk[0], NB * 8); if (rc) return rc; }
-  if (!m->has_idx && !(getenv("PYRE_PROMPT_ATTN_SPLIT") && atoi(getenv("PYRE_PROMPT_ATTN_SPLIT")) == 0)) {      // (with a sparse indexer the selection and the pass stay together in the chain; PYRE_PROMPT_ATTN_SPLIT=0: likewise)
+  if (!m->has_idx) {      // (with a sparse indexer the selection and the pass stay together in the chain)
     const size_t nq = (size_t)8 * c.n_head * c.hd;
     P->q_off[0] = al256(4 * nq); P->q_off[1] = P->q_off[0] + al256(2 * 2 * nq); P->q_stride = P->q_off[1] + al256(4 * 8 * (size_t)c.n_head);
     PYRE_HIP(ctx, hipMalloc(&P->qmem, 2 * (size_t)NB * P->q_stride));
@@ -886,6 +886,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     const int G_env = [] { const char* e = getenv("PYRE_PROMPT_GROUP"); int v = e && *e ? atoi(e) : 0; return v < 0 ? 0 : (v > PROMPT_BLOCK_WINDOWS ? PROMPT_BLOCK_WINDOWS : v); }();      // PYRE_PROMPT_GROUP: windows a group (default: a group a stream)
     const bool batch = [&] { const char* e = getenv("PYRE_PROMPT_BATCH"); if (e && *e && atoi(e) == 0) return false; for (const Layer& L : m->layers) if (!pyre_hc_aop_ok(L.hca) || !pyre_hc_aop_ok(L.hcf)) return false; return true; }();      // a group's mixes in one launch each (the matrix-core mixes; PYRE_PROMPT_BATCH=0: a launch a window)
     const bool early = batch && m->c.conv_k >= 2 && m->c.conv_k <= 9 && !(getenv("PYRE_PROMPT_PROJ_EARLY") && atoi(getenv("PYRE_PROMPT_PROJ_EARLY")) == 0);      // the projections in front of the chain through the layer's state, the convolution once a group (PYRE_PROMPT_PROJ_EARLY=0: both in the chain, a window at a time)
+    const bool asplit = P->qmem && !(getenv("PYRE_PROMPT_ATTN_SPLIT") && atoi(getenv("PYRE_PROMPT_ATTN_SPLIT")) == 0);      // an attention layer's pass over the cache outside the chain (PYRE_PROMPT_ATTN_SPLIT=0: in it)
     const bool pairs = [] { const char* e = getenv("PYRE_PROMPT_PAIRS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_PAIRS=0: one block at a time
     auto cxk = [&](int k) { return k ? P->ctx[k - 1] : ctx; };
     auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(P->moe_ctx->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
@@ -911,7 +912,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
           o.win_stride = P->win_stride; o.proj_early = early;
-          if (P->qmem) {          // q buffers of the window's own; the partial sums stay the stream's
+          if (asplit) {          // q buffers of the window's own; the partial sums stay the stream's
             o.attn_split = true; o.aw_own = set ? s->aw_more[set - 1] : s->aw;
             uint8_t* qb = (uint8_t*)P->qmem + (size_t)(w * NBMAX + j) * P->q_stride;
             o.aw_own.q = (float*)qb; o.aw_own.qh = (uint16_t*)(qb + P->q_off[0]); o.aw_own.qsc = (float*)(qb + P->q_off[1]);

@@ -120,10 +120,14 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
     prompt = g.integers(0, cfg.vocab, 2 * 256 + 45, dtype=np.uint32)
     more = g.integers(0, cfg.vocab, 256 + 100 + 9, dtype=np.uint32)          # a full block and a shorter one
     out = {}
-    for mode in ("0", "1", "1 one block at a time", "1 groups of 5"):
+    modes = ("0", "1", "1 one block at a time", "1 groups of 5", "1 a launch a window", "1 projection in the chain", "1 attention in the chain")
+    for mode in modes:
         monkeypatch.setenv("PYRE_PROMPT_WINDOWS", "1" if mode == "0" else "0")
         monkeypatch.setenv("PYRE_PROMPT_PAIRS", "0" if mode == "1 one block at a time" else "1")     # two blocks in flight, one's FFN beside the other's windows
         monkeypatch.setenv("PYRE_PROMPT_GROUP", "5" if mode == "1 groups of 5" else "0")              # consecutive windows a stream takes together
+        monkeypatch.setenv("PYRE_PROMPT_BATCH", "0" if mode == "1 a launch a window" else "1")        # a group's mixes, projections, convolution and recurrences in one launch each
+        monkeypatch.setenv("PYRE_PROMPT_PROJ_EARLY", "0" if mode == "1 projection in the chain" else "1")     # projection (and convolution) outside the chain through the layer's state
+        monkeypatch.setenv("PYRE_PROMPT_ATTN_SPLIT", "0" if mode == "1 attention in the chain" else "1")      # the pass over the cache outside it
         st = gm.new_state(1024)
         n0 = gm.prompt_blocks()
         lg = gm.forward(prompt, st)
@@ -134,7 +138,7 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
         out[mode] = (lg.copy(), toks.copy(), lg2.copy(), toks2.copy(), len(st))
         st.close()
     a, b = out["0"], out["1"]
-    for other in ("1 one block at a time", "1 groups of 5"):          # the order of the launches does not change a bit
+    for other in modes[2:]:          # the order and the grouping of the launches do not change a bit
         for i in range(4):
             assert np.array_equal(np.asarray(b[i]).view(np.uint32), np.asarray(out[other][i]).view(np.uint32)), (other, i)
     assert a[4] == b[4] == prompt.size + 6 + more.size + 4
