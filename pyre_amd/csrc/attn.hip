@@ -51,9 +51,13 @@ template <int HD> __device__ __forceinline__ void kv_pack_thread(const AttnDev& 
 // each group of eight dims the halves are stored in the order 0 4 1 5 2 6 3 7, the order in which a 32-bit word of
 // eight 4-bit keys unpacks into f16 pairs.
 template <int HD>
-__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout, uint16_t* __restrict__ qh, float* __restrict__ qsc) {
+__global__ __launch_bounds__(HD) void k_attn_prep(AttnDev a, KvDev kv, const float* __restrict__ qkv, int stride, int start, const int* __restrict__ posp, float* __restrict__ qout, uint16_t* __restrict__ qh, float* __restrict__ qsc, size_t wz_qkv, size_t wz_q) {
   __shared__ float buf[HD]; __shared__ float red[HD / 64]; __shared__ float redm[HD / 64];
   if (posp) start = *posp;
+  if (gridDim.z > 1) {          // consecutive windows in one launch (a long prompt's blocks): window z's projection wz_qkv bytes, its query buffers wz_q bytes further on per window, its positions behind the window before
+    const size_t z = blockIdx.z; start += (int)z * (int)gridDim.y;
+    qkv = (const float*)((const char*)qkv + z * wz_qkv); qout = (float*)((char*)qout + z * wz_q); qh = (uint16_t*)((char*)qh + z * wz_q); qsc = (float*)((char*)qsc + z * wz_q);
+  }
   const int b = blockIdx.x, ti = blockIdx.y, tid = threadIdx.x, pos = start + ti;
   if (b >= a.nkv + a.nh) {
     int p0, p1;
@@ -747,12 +751,14 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
   // the cache and the merge, which read only what part 1 of this and of earlier windows has written (w.q* must then be this
   // window's own until part 2 has run); 0: both
   if (part < 0 || part > 2 || (part && posp)) return pyre_fail(ctx, PYRE_E_ARG, "attention: part %d", part);
+  const int nwin = ctx->batch_n;          // part 1 for that many consecutive windows of t tokens in one launch (ctx->batch_stride / batch_stride2: the windows' projections / query buffers apart)
+  if (nwin > 1 && (part != 1 || qw || start + nwin * t > kv.cap)) return pyre_fail(ctx, PYRE_E_ARG, "attention: %d windows a launch (the cache write alone, dense, inside the cache)", nwin);
   const bool pack_rides = posp && t == 1 && a.kv_bits == 4;
   const int pack_blocks = pack_rides ? (64 * (a.nkv * a.hd / 32) * 2 + 255) / 256 : 0;
   if (part != 2) {
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q, w.qh, w.qsc); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh + pack_blocks, t, nwin), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, posp, w.q, w.qh, w.qsc, ctx->batch_stride, ctx->batch_stride2); } PYRE_CHECK_LAUNCH(ctx);
   // pack the positions that fall below the boundary of the longest view of this call
-  int pbn = (int)pyre_packed_boundary((size_t)start + t, a.kv_bits, a.kv_recent);
+  int pbn = (int)pyre_packed_boundary((size_t)start + (size_t)nwin * t, a.kv_bits, a.kv_recent);
   if (posp) {   // one 64-position packing step at most; the kernel decides from the device-side position
     if (a.kv_bits == 4 && !pack_rides) { size_t thr = (size_t)64 * (a.nkv * a.hd / 32) * 2; hipLaunchKernelGGL((k_kv_pack<256>), dim3((unsigned)((thr + 127) / 128)), dim3(128), 0, ctx->stream, a, kv, 0, 0, posp); PYRE_CHECK_LAUNCH(ctx); }
   } else if (pbn > *packed_done) {
@@ -780,7 +786,7 @@ int pyre_attn_launch_sel(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const
 int pyre_attn_append_launch(pyre_ctx* ctx, const AttnDev& a, const KvDev& kv, const AttnWork& w, const float* qkv, int stride, int start, int t) {
   if (a.hd != 256 || a.kv_bits != 0) return pyre_fail(ctx, PYRE_E_SHAPE, "attention append: head dim %d, %d-bit cache (256, f32 only)", a.hd, a.kv_bits);
   if (t < 1 || t > 8 || start < 0 || start + t > kv.cap) return pyre_fail(ctx, PYRE_E_STATE, "attention append: positions %d..%d outside the cache (%d)", start, start + t, kv.cap);
-  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, (const int*)nullptr, w.q, w.qh, w.qsc); } PYRE_CHECK_LAUNCH(ctx);
+  { ProfScope ps(ctx, "attn_prep", 8.0 * t * (a.nh + 2.0 * a.nkv) * a.hd); hipLaunchKernelGGL((k_attn_prep<256>), dim3(a.nkv + a.nh, t), dim3(256), 0, ctx->stream, a, kv, qkv, stride, start, (const int*)nullptr, w.q, w.qh, w.qsc, (size_t)0, (size_t)0); } PYRE_CHECK_LAUNCH(ctx);
   return PYRE_OK;
 }
 

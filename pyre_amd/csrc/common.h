@@ -42,7 +42,7 @@ struct pyre_ctx {
   bool prof_on = false; std::vector<ProfPending> prof_pending; std::map<std::string, ProfAcc> prof_acc; std::vector<hipEvent_t> prof_pool;
   std::string prof_text;
   void* aop_buf = nullptr; size_t aop_bytes = 0;       // split activations of the operator's matrix-core GEMM (grow-only)
-  int batch_n = 1; size_t batch_stride = 0;            // the matrix-core hyper-connection launches (hc.hip) for batch_n windows at once: window z's own buffers batch_stride bytes further on per window (a long prompt's blocks; 1 / 0 otherwise)
+  int batch_n = 1; size_t batch_stride = 0, batch_stride2 = 0;            // the matrix-core hyper-connection launches (hc.hip) for batch_n windows at once: window z's own buffers batch_stride bytes further on per window (a long prompt's blocks; 1 / 0 otherwise)
   void* aop_static = nullptr;                          // device address of this GPU's copy of the file-scope operand array (gemm_m.hip), resolved at creation
   uint32_t* d_iq2xs_sgn = nullptr;                     // IQ2_XS likewise: two tables of 8192 x four signed bytes (weights 0..3 / 4..7 of an entry)
   uint32_t* d_iq3s_sgn = nullptr;                      // IQ3_S codebook with the signs folded in: 8192 x four signed bytes (gemv_n.hip), made at first use

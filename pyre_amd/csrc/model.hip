@@ -715,6 +715,14 @@ struct WinRun {
     const float* prev = first ? s->conv[b][li] : m->proj - o.win_stride / 4 + (size_t)(t - K1) * m->pw_lin;
     return pyre_gdn_conv_block_launch(ctx, L.gdn, m->proj, m->pw_lin, t, n, o.win_stride / 4, prev, first ? m->ch : m->pw_lin, last ? s->conv[b ^ (flips & 1)][li] : nullptr, m->co);
   }
+  // (proj_early, attn_split) the cache write of this window and the n - 1 after it, an attention layer, in one launch (and one packing step)
+  int front_mid_attn(int il, int n, size_t q_stride) {
+    const Layer& L = m->layers[il]; const int ai = L.mix_index;
+    ctx->batch_n = n; ctx->batch_stride = n > 1 ? o.win_stride : 0; ctx->batch_stride2 = n > 1 ? q_stride : 0;
+    const int rc = pyre_attn_launch_sel(ctx, L.attn, s->kv[ai], o.aw_own, m->proj, m->pw_attn, start, t, &s->packed[ai], m->core, nullptr, nullptr, 1);
+    ctx->batch_n = 1; ctx->batch_stride = 0; ctx->batch_stride2 = 0;
+    return rc;
+  }
   // (proj_early) the recurrence of this window and the n - 1 after it in one launch: the state stays in registers from window to window
   bool gdn_group_ok(int il) const { const Layer& L = m->layers[il]; return !L.full && gdn_q_on(m, L); }
   int front_mid_gdn(int il, int n) {
@@ -936,6 +944,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
           const bool gg = early && b.runs[j0].gdn_group_ok(il);          // the group's recurrences in one launch
           if (early && (r = b.runs[j0].front_mid_conv(il, j1 - j0, j0 == 0, j1 == b.NB, gg ? 1 : j1 - j0))) return r;
           if (gg) { if ((r = b.runs[j0].front_mid_gdn(il, j1 - j0))) return r; }
+          else if (early && asplit && m->layers[il].full) { if ((r = b.runs[j0].front_mid_attn(il, j1 - j0, P->q_stride))) return r; }          // the group's cache writes in one launch
           else for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_mid(il))) return r;
           if (hipEventRecord(P->ev[k][il], cx->stream) != hipSuccess) return pyre_fail(cx, PYRE_E_HIP, "hipEventRecord failed");
           for (int j = j0; j < j1; ++j) if ((r = b.runs[j].front_post_attn(il))) return r;
