@@ -323,7 +323,7 @@ bool   pyre_moe_block_ok(const MoeDev& m);
 size_t pyre_moe_block_bytes(const MoeDev& m, int T);
 void   pyre_moe_block_carve(const MoeDev& m, int T, void* base, MoeBlk* b);
 int    pyre_moe_block_zero_rows(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T);
-int    pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64);
+int    pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64, bool router_here = false);      // router_here: the router's sums are formed by this call (k_moe_router_blk), not left by the mixes
 // K parts the gate/up dot products are summed in (1 or 2; k_moe_gu)
 int pyre_moe_gu_parts(const MoeDev& m);
 

@@ -598,6 +598,7 @@ struct WinOpt {
   int start = -1;               // the window's first position when the caller keeps the count (a block of windows taken layer by layer); -1: the state's length
   bool no_len = false;          // ... and the state's length is then advanced by the caller
   size_t win_stride = 0;        // bytes between this window's workspace and the next window's of its block (0: it stands alone)
+  bool router_apart = false;    // a block's window: the router's K-slice sums come from the block's FFN launch, not from this window's FFN mix
   bool proj_early = false;      // a block's window: the layer's projection is launched with the mix in front of it (front_pre_proj), a Gated DeltaNet layer's convolution once for the group (front_mid_conv): neither needs the layer's state
   bool attn_split = false; AttnWork aw_own{};      // a block's window: the attention pass over the cache leaves the chain through the layer's state (front_post_proj runs it); aw_own: the stream's attention workspace with q buffers of this window's own
 };
@@ -783,7 +784,7 @@ struct WinRun {
     const pyre_model_cfg& c = m->c; const int d = c.d; int rc;
     const Layer& L = m->layers[il];
     const int o_parts = outp_in_parts(L, d) ? PYRE_GEMV_PARTS : 1;
-    ride = route_rides && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
+    ride = route_rides && !o.router_apart && pyre_hc_route_ok(L.hcf, L.moe.router);       // the router GEMV rides on the mix's second launch
     HcRoute hr{L.moe.router, m->rpart, m->mw.dgx};          // (the matrix-core mix leaves the digits of its output; after another mix the expert launch makes them)
     if (nz > 0) {
       ctx->batch_n = nz; ctx->batch_stride = nz > 1 ? o.win_stride : 0;
@@ -895,6 +896,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
     const bool batch = [&] { const char* e = getenv("PYRE_PROMPT_BATCH"); if (e && *e && atoi(e) == 0) return false; for (const Layer& L : m->layers) if (!pyre_hc_aop_ok(L.hca) || !pyre_hc_aop_ok(L.hcf)) return false; return true; }();      // a group's mixes in one launch each (the matrix-core mixes; PYRE_PROMPT_BATCH=0: a launch a window)
     const bool early = batch && m->c.conv_k >= 2 && m->c.conv_k <= 9 && !(getenv("PYRE_PROMPT_PROJ_EARLY") && atoi(getenv("PYRE_PROMPT_PROJ_EARLY")) == 0);      // the projections in front of the chain through the layer's state, the convolution once a group (PYRE_PROMPT_PROJ_EARLY=0: both in the chain, a window at a time)
     const bool asplit = P->qmem && !(getenv("PYRE_PROMPT_ATTN_SPLIT") && atoi(getenv("PYRE_PROMPT_ATTN_SPLIT")) == 0);      // an attention layer's pass over the cache outside the chain (PYRE_PROMPT_ATTN_SPLIT=0: in it)
+    const bool rapart = batch && !(getenv("PYRE_PROMPT_ROUTER_APART") && atoi(getenv("PYRE_PROMPT_ROUTER_APART")) == 0);      // the router's sums with the block's FFN launches (beside the other block's windows) instead of riding on every window's FFN mix (PYRE_PROMPT_ROUTER_APART=0: riding)
     const bool pairs = [] { const char* e = getenv("PYRE_PROMPT_PAIRS"); return !(e && *e && atoi(e) == 0); }();      // PYRE_PROMPT_PAIRS=0: one block at a time
     auto cxk = [&](int k) { return k ? P->ctx[k - 1] : ctx; };
     auto bail = [&](int code, pyre_ctx* cx) { s->broken = true; if (cx != ctx) pyre_fail(ctx, code, "%s", cx->err.c_str()); for (auto* c2 : P->ctx) (void)hipStreamSynchronize(c2->stream); (void)hipStreamSynchronize(P->moe_ctx->stream); (void)hipStreamSynchronize(ctx->stream); return code; };
@@ -919,7 +921,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
         for (int j = 0; j < b.NB; ++j) {
           const int set = (j / G) % K; WinOpt o; o.head_tokens = 0; o.keep_from = 8; o.start = pos + 8 * j; o.no_len = true;
           o.ids_dev = P->ids + i0 + 8 * j; if (set) { o.aw = &s->aw_more[set - 1]; o.qw = &s->qw_more[set - 1]; }
-          o.win_stride = P->win_stride; o.proj_early = early;
+          o.win_stride = P->win_stride; o.proj_early = early; o.router_apart = rapart;
           if (asplit) {          // q buffers of the window's own; the partial sums stay the stream's
             o.attn_split = true; o.aw_own = set ? s->aw_more[set - 1] : s->aw;
             uint8_t* qb = (uint8_t*)P->qmem + (size_t)(w * NBMAX + j) * P->q_stride;
@@ -956,7 +958,7 @@ int pyre_forward(pyre_ctx* ctx, const pyre_model* m, pyre_state* s, const uint32
       auto ffn = [&](Blk& b, int il) -> int {
         pyre_ctx* mx = P->moe_ctx;
         for (int k = 0; k < K && k < b.NG; ++k) { if (hipEventRecord(P->front_done[b.which][k], cxk(k)->stream) != hipSuccess || hipStreamWaitEvent(mx->stream, P->front_done[b.which][k], 0) != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "event failed"); }
-        int r = pyre_moe_block_launch(mx, m->layers[il].moe, P->blk[b.which], b.NB * 8, NBMAX * 8, P->blk_nsl, P->blk_r64);
+        int r = pyre_moe_block_launch(mx, m->layers[il].moe, P->blk[b.which], b.NB * 8, NBMAX * 8, P->blk_nsl, P->blk_r64, rapart);
         if (r) return pyre_fail(ctx, r, "%s", mx->err.c_str());
         if (hipEventRecord(P->moe_done[b.which], mx->stream) != hipSuccess) return pyre_fail(ctx, PYRE_E_HIP, "hipEventRecord failed");
         for (int j = 0; j < b.NB; ++j) b.runs[j].moe_from_block();

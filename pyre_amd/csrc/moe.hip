@@ -554,6 +554,29 @@ __global__ __launch_bounds__(1024) void k_moe_route_blk(MoeDev m, MoeBlk b, int 
   route_weights(top_k, rl);
   if ((int)threadIdx.x < top_k) { b.sel_idx[ti * top_k + threadIdx.x] = rl.s_idx[threadIdx.x]; b.sel_w[ti * top_k + threadIdx.x] = rl.s_w[threadIdx.x]; }
 }
+// The router's K-slice sums of a block when they do not ride on the windows' FFN mixes: grid (d / 64, T / 8), 4 waves.  The
+// workgroup stages its window's eight tokens' 64 columns of x and forms, tile of 64 experts by tile, the partial dot products
+// the riding code of k_hc_up_mix_m forms (unit_fma over the same 64 values in the same order): the same bits, where the
+// windows' path has them.
+template <int RF>
+__global__ __launch_bounds__(256) void k_moe_router_blk(MoeDev m, MoeBlk b, int r64) {
+  __shared__ float xs[8][64];
+  const uint2* lds2 = nullptr;
+  const int sl = blockIdx.x, w = blockIdx.y, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const float* xw = b.x + (size_t)w * b.ws;
+  for (int i = threadIdx.x; i < 8 * 64; i += 256) xs[i >> 6][i & 63] = xw[(size_t)(i >> 6) * m.d + sl * 64 + (i & 63)];
+  lds_barrier();
+  float* rp = const_cast<float*>(b.rpart) + (size_t)w * b.ws;
+  for (int tile = wave; tile < m.router.tiles; tile += 4) {
+    const UnitRaw<RF> rraw = unit_load<RF>(m.router, tile, sl, lane);
+#pragma unroll 1
+    for (int t2 = 0; t2 < 8; ++t2) {
+      float ra[1] = {0.0f};
+      unit_fma<RF, 1>(m.router, rraw, sl, lds2, lane, xs[t2], 0, ra);
+      rp[((size_t)sl * 8 + t2) * r64 + (size_t)tile * 64 + lane] = ra[0];
+    }
+  }
+}
 // the (token, choice) pairs of the block by expert: eoff[e] .. eoff[e + 1] of elist hold expert e's entries token * (k + 1) + j
 // (in no particular order: a token's sums do not depend on its neighbours).  One workgroup of 1024 threads.
 __global__ __launch_bounds__(1024) void k_moe_lists(MoeDev m, MoeBlk b, int T) {
@@ -723,10 +746,17 @@ int pyre_moe_block_zero_rows(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, in
 }
 // T = 8 * windows tokens (T_max: the T the scratch was carved and its zero rows were set for); the router's K-slice sums (nsl
 // slices of r64 rows a token) come from the mixes
-int pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64) {
+int pyre_moe_block_launch(pyre_ctx* ctx, const MoeDev& m, const MoeBlk& b, int T, int T_max, int nsl, int r64, bool router_here) {
   if (!pyre_moe_block_ok(m) || T < 8 || T % 8 || T > T_max || nsl < 1 || nsl > 64 || r64 < m.n_exp) return pyre_fail(ctx, PYRE_E_ARG, "moe block: unsupported shape (T = %d, %d router slices)", T, nsl);
   const int hs = m.ff, ny = m.n_exp + (T + 7) / 8, ne = T * (m.top_k + 1), ne_max = T_max * (m.top_k + 1);
   const bool fix = m.n_exp == 512 && m.top_k == 10 && nsl == 32;
+  if (router_here) {          // the router's K-slice sums were not left by the mixes: form them now
+    if (nsl != m.d / 64 || (m.router.fmt != FMT_BF16 && m.router.fmt != FMT_F32)) return pyre_fail(ctx, PYRE_E_ARG, "moe block: the router's sums by %d slices, router format %d", nsl, m.router.fmt);
+    ProfScope ps(ctx, "moe_block_router", qmat_gguf_bytes(m.router, m.router.rows) + 4.0 * T * (m.d + (double)nsl * r64));
+    if (m.router.fmt == FMT_BF16) hipLaunchKernelGGL(k_moe_router_blk<FMT_BF16>, dim3(nsl, T / 8), dim3(256), 0, ctx->stream, m, b, r64);
+    else hipLaunchKernelGGL(k_moe_router_blk<FMT_F32>, dim3(nsl, T / 8), dim3(256), 0, ctx->stream, m, b, r64);
+    PYRE_CHECK_LAUNCH(ctx);
+  }
   { ProfScope ps(ctx, "moe_block_route", 4.0 * T * nsl * m.n_exp);
     if (fix) hipLaunchKernelGGL(k_moe_route_blk<true>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64); else hipLaunchKernelGGL(k_moe_route_blk<false>, dim3(T), dim3(1024), 0, ctx->stream, m, b, nsl, r64);
     hipLaunchKernelGGL(k_moe_lists, dim3(1), dim3(1024), 0, ctx->stream, m, b, T);

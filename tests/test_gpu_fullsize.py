@@ -120,7 +120,7 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
     prompt = g.integers(0, cfg.vocab, 2 * 256 + 45, dtype=np.uint32)
     more = g.integers(0, cfg.vocab, 256 + 100 + 9, dtype=np.uint32)          # a full block and a shorter one
     out = {}
-    modes = ("0", "1", "1 one block at a time", "1 groups of 5", "1 a launch a window", "1 projection in the chain", "1 attention in the chain")
+    modes = ("0", "1", "1 one block at a time", "1 groups of 5", "1 a launch a window", "1 projection in the chain", "1 attention in the chain", "1 router riding")
     for mode in modes:
         monkeypatch.setenv("PYRE_PROMPT_WINDOWS", "1" if mode == "0" else "0")
         monkeypatch.setenv("PYRE_PROMPT_PAIRS", "0" if mode == "1 one block at a time" else "1")     # two blocks in flight, one's FFN beside the other's windows
@@ -128,6 +128,7 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
         monkeypatch.setenv("PYRE_PROMPT_BATCH", "0" if mode == "1 a launch a window" else "1")        # a group's mixes, projections, convolution and recurrences in one launch each
         monkeypatch.setenv("PYRE_PROMPT_PROJ_EARLY", "0" if mode == "1 projection in the chain" else "1")     # projection (and convolution) outside the chain through the layer's state
         monkeypatch.setenv("PYRE_PROMPT_ATTN_SPLIT", "0" if mode == "1 attention in the chain" else "1")      # the pass over the cache outside it
+        monkeypatch.setenv("PYRE_PROMPT_ROUTER_APART", "0" if mode == "1 router riding" else "1")           # the router's sums with the block's FFN launches, not on every window's FFN mix
         st = gm.new_state(1024)
         n0 = gm.prompt_blocks()
         lg = gm.forward(prompt, st)
