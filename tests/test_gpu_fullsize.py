@@ -147,6 +147,22 @@ def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows
     assert relerr(b[2], a[2]) <= 1e-4 and np.array_equal(a[3], b[3])
 
 
+def test_prompt_in_blocks_at_a_long_context_agrees_with_the_windows_path(model4, monkeypatch):
+    """20 000 tokens (the 4-bit boundary of the caches moves some three hundred times, the attention passes cover many chunks,
+    twenty blocks in ten calls' worth of pairs): logits within 1e-4 of the windows' path, the same tokens after it."""
+    cfg, gm = model4
+    prompt = np.random.Generator(np.random.PCG64(27)).integers(0, cfg.vocab, 20000, dtype=np.uint32)
+    out = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("PYRE_PROMPT_WINDOWS", mode)
+        st = gm.new_state(20000 + 32); n0 = gm.prompt_blocks()
+        lg = gm.forward(prompt, st)
+        out[mode] = (lg.copy(), gm.decode_greedy_dev(st, int(np.argmax(lg)), 8).copy(), gm.prompt_blocks() - n0)
+        st.close()
+    assert out["1"][2] == 0 and out["0"][2] == 20
+    assert relerr(out["0"][0], out["1"][0]) <= 1e-4 and np.array_equal(out["0"][1], out["1"][1])
+
+
 def test_prompt_in_blocks_matches_the_oracle_at_full_width(ctx):
     """One block of 256 tokens plus a tail through the two-layer slice against the oracle's token-by-token prompt."""
     cfg = mg.a3b_config(n_layers=2, full_every=2)
