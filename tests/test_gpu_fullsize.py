@@ -111,8 +111,8 @@ def test_drafter_matches_the_oracle_at_full_width(ctx):
 
 
 def test_prompt_in_blocks_with_the_ffn_grouped_by_expert_agrees_with_the_windows_path(ctx, model4, monkeypatch):
-    """A long prompt takes blocks of 32 windows layer by layer, the FFN of a block's 256 tokens grouped by expert on the
-    matrix cores: logits agree with the windows' path (PYRE_PROMPT_BLOCK=0 at run time) to rounding, the tokens that follow
+    """A long prompt takes blocks of up to 128 windows layer by layer, the FFN of a block's tokens grouped by expert on the
+    matrix cores: logits agree with the windows' path (PYRE_PROMPT_WINDOWS=1 at run time) to rounding, the tokens that follow
     and the state's length are the same, for a call that is whole blocks plus a ragged tail, and for a state that continues
     with a second long call."""
     cfg, gm = model4
@@ -164,7 +164,7 @@ def test_prompt_in_blocks_at_a_long_context_agrees_with_the_windows_path(model4,
 
 
 def test_prompt_in_blocks_matches_the_oracle_at_full_width(ctx):
-    """One block of 256 tokens plus a tail through the two-layer slice against the oracle's token-by-token prompt."""
+    """256 tokens in a pair of blocks plus a tail through the two-layer slice against the oracle's token-by-token prompt."""
     cfg = mg.a3b_config(n_layers=2, full_every=2)
     hw = mg.build_host(cfg, seed=8)
     gm = lib.Model(ctx, cfg, hw.layers, hw.globals_); om = orc_model(hw, threads=min(os.cpu_count() or 1, 16))
